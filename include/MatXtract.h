@@ -1,0 +1,219 @@
+/*
+ * MatXtract.h -- the reference's C++ surface, served by libmatxtract_hip.so.
+ *
+ * Source-compatible with the reference's include/MatXtract.h:3-34 (kernel entry points),
+ * include/csr2csc.h:9-13 (transposes) and include/mmio.h:165-179 (Matrix-Market ingest,
+ * exclusive_scan), together with the pieces of include/common.h a driver needs (valT, indT,
+ * fragM/fragK, half, initVec, divup).  A driver written against the reference compiles
+ * against this header unchanged and links with -lmatxtract_hip instead of the CUDA library.
+ *
+ * Same conventions as the reference: precision is chosen at compile time (-Dfp64 -> double,
+ * otherwise IEEE binary16 `half`); every pointer is HOST memory; arrays a function returns
+ * are malloc()ed and released by the caller with free(); device errors print to stderr and
+ * exit(EXIT_FAILURE) (include/common.h:81-90); calls are synchronous.
+ *
+ * Each function is an inline wrapper over one C-ABI entry point of matxtract_hip.h.  The
+ * timing loops run MATXTRACT_WARM (default 200) warm-ups and MATXTRACT_ITERS (default 4000)
+ * timed launches, the reference's counts (src/spmv_kernel/cdSpMV.cu:454-455).
+ *
+ * New here (the reference has it inlined in main(), test/test_autotc_spmv.cpp:1106-1427):
+ * matxtract_preprocess(), the cascaded extraction as a callable.
+ */
+#ifndef MATXTRACT_H
+#define MATXTRACT_H
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "matxtract_hip.h"
+
+#define indT int
+
+#ifdef fp64
+#define valT double
+#define MX_VALT_DTYPE MX_F64
+const int fragM = 8;
+const int fragK = 4;
+const int fragN = 8;
+#else
+/* IEEE binary16 held as its bit pattern; arithmetic converts through float and rounds back
+ * after every operation, which is how CUDA's host-side `half` behaves. */
+extern "C" uint16_t mx_f32_to_f16(float f);
+extern "C" float mx_f16_to_f32(uint16_t h);
+struct half {
+    uint16_t bits;
+    half() : bits(0) {}
+    half(float f) : bits(mx_f32_to_f16(f)) {}
+    half(double d) : bits(mx_f32_to_f16((float)d)) {}
+    half(int i) : bits(mx_f32_to_f16((float)i)) {}
+    operator float() const { return mx_f16_to_f32(bits); }
+};
+inline half operator+(half a, half b) { return half((float)a + (float)b); }
+inline half operator*(half a, half b) { return half((float)a * (float)b); }
+#define valT half
+#define MX_VALT_DTYPE MX_F16
+const int fragM = 8;
+const int fragK = 8;
+#endif
+
+template <typename T>
+inline T divup(T a, T b)
+{
+    return (a + b - 1) / b;
+}
+
+/* include/common.h:237-245 */
+inline void initVec(valT *vec, int length) { mx_init_vec(MX_VALT_DTYPE, vec, length); }
+
+namespace matxtract_detail {
+inline int env_int(const char *name, int dflt)
+{
+    const char *s = std::getenv(name);
+    return (s && *s) ? std::atoi(s) : dflt;
+}
+inline void check(int rc, const char *what)
+{
+    if (rc != MX_OK) {
+        std::fprintf(stderr, "MatXtract HIP error in %s: %s (code %d)\n", what, mx_last_error(), rc);
+        std::exit(EXIT_FAILURE);
+    }
+}
+inline int warm() { return env_int("MATXTRACT_WARM", 200); }
+inline int iters() { return env_int("MATXTRACT_ITERS", 4000); }
+}  // namespace matxtract_detail
+
+/* include/MatXtract.h:3-5.  Y is IN/OUT: Y += A*X.  cdTime, cdPre in ms. */
+inline void cdspmv(valT *csrVal, indT *csrRowPtr, indT *csrColInd, valT *X_val, valT *Y_val, int rowA, int colA,
+                   indT nnzA, double *cdTime, double *cdPre)
+{
+    using namespace matxtract_detail;
+#ifdef fp64
+    check(mx_cdspmv_f64(csrVal, csrRowPtr, csrColInd, X_val, Y_val, rowA, colA, nnzA, warm(), iters(), cdTime, cdPre),
+          "cdspmv");
+#else
+    check(mx_cdspmv_f16((const uint16_t *)csrVal, csrRowPtr, csrColInd, (const uint16_t *)X_val, (uint16_t *)Y_val, rowA,
+                        colA, nnzA, warm(), iters(), cdTime, cdPre),
+          "cdspmv");
+#endif
+}
+
+#ifdef fp64
+/* include/MatXtract.h:7-9.  rowA = dRows, colA = dCols; row_order is unused, as in the
+ * reference; Y is uploaded and added to. */
+inline void du_tcspmv_fp64(indT *chunkPtr, std::vector<int> fragPtr, std::vector<uint32_t> fragBit,
+                           std::vector<double> tcVal, indT *sparse_AToX_index, valT *X_val, valT *Y_val, int rowA,
+                           int colA, int *row_order, double *tcTime)
+{
+    using namespace matxtract_detail;
+    (void)row_order;
+    check(mx_du_tcspmv_f64(chunkPtr, fragPtr.data(), fragBit.data(), tcVal.data(), sparse_AToX_index, X_val, Y_val, rowA,
+                           colA, warm(), iters(), tcTime),
+          "du_tcspmv_fp64");
+}
+#else
+/* include/MatXtract.h:27-29.  Y is overwritten. */
+inline void du_tcspmv_fp16_v2(indT *chunkPtr, std::vector<int> fragPtr, std::vector<uint64_t> fragBit,
+                              std::vector<half> tcVal, indT *sparse_AToX_index, half *X_val, half *Y_val, int rowA,
+                              int colA, int *row_order, double *tcTime)
+{
+    using namespace matxtract_detail;
+    (void)row_order;
+    check(mx_du_tcspmv_f16(chunkPtr, fragPtr.data(), fragBit.data(), (const uint16_t *)tcVal.data(), sparse_AToX_index,
+                           (const uint16_t *)X_val, (uint16_t *)Y_val, rowA, colA, warm(), iters(), tcTime),
+          "du_tcspmv_fp16_v2");
+}
+#endif
+
+/* include/MatXtract.h:14-15 (fp64) / 31-32 (fp16): the "sparse encode" executor of the
+ * extracted block, given as CSR.  Contract kept: Y_val[i] = (A*X)[order_rid[i]] with
+ * order_rid a permutation of [0,rowA).  Here the block runs through the CSR kernel in its
+ * given row order, so order_rid is the identity; NUM, threshold and block_longest steered the
+ * reference's row classification and have no effect. */
+inline void
+#ifdef fp64
+se_tcspmv_fp64
+#else
+se_tcspmv_fp16
+#endif
+    (valT *csrValA, indT *csrRowPtrA, int *csrColIdxA, valT *X_val, valT *Y_val, int *order_rid, int rowA, int colA,
+     indT nnzA, int NUM, double threshold, int block_longest, double *tcTime)
+{
+    (void)NUM;
+    (void)threshold;
+    (void)block_longest;
+    for (int i = 0; i < rowA; ++i) order_rid[i] = i;
+    for (int i = 0; i < rowA; ++i) Y_val[i] = static_cast<valT>(0.0);
+    double pre = 0.0;
+    cdspmv(csrValA, csrRowPtrA, csrColIdxA, X_val, Y_val, rowA, colA, nnzA, tcTime, &pre);
+}
+
+/* include/csr2csc.h:9-13 */
+inline void csr2csc(valT *csrVal, indT *csrRowPtr, indT *csrColInd, int rowA, int colA, indT nnzA, valT **cscVal,
+                    indT **cscColPtr, indT **cscRowInd)
+{
+    matxtract_detail::check(mx_transpose(MX_VALT_DTYPE, rowA, colA, nnzA, csrRowPtr, csrColInd, csrVal, cscColPtr,
+                                         cscRowInd, (void **)cscVal),
+                            "csr2csc");
+}
+inline void csc2csr(valT *cscVal, indT *cscColPtr, indT *cscRowInd, int rowA, int colA, indT nnzA, valT **csrVal,
+                    indT **csrRowPtr, indT **csrColInd)
+{
+    matxtract_detail::check(mx_transpose(MX_VALT_DTYPE, colA, rowA, nnzA, cscColPtr, cscRowInd, cscVal, csrRowPtr,
+                                         csrColInd, (void **)csrVal),
+                            "csc2csr");
+}
+
+/* include/mmio.h:165-179.  Returns 0, or a negative code the reference's callers ignore. */
+inline int mmio_allinone(int *m, int *n, indT *nnz, int *isSymmetric, indT **csrRowPtr, int **csrColIdx, valT **csrVal,
+                         char *filename)
+{
+    int rc = mx_mmio_read(filename, MX_VALT_DTYPE, m, n, nnz, isSymmetric, csrRowPtr, csrColIdx, (void **)csrVal);
+    return rc == MX_OK ? 0 : -1;
+}
+
+/* utilities/mmio.cpp:949-964 */
+inline void exclusive_scan(indT *input, int length)
+{
+    indT run = 0;
+    for (int i = 0; i < length; ++i) {
+        indT v = input[i];
+        input[i] = run;
+        run += v;
+    }
+}
+
+/* The cascaded extraction as one call (test/test_autotc_spmv.cpp:1106-1427, 1486-1492):
+ * column pass with colProp (global_col), row pass with rowProp (local_row), tile format,
+ * residual.  Returns NULL after printing the reason when the arguments are rejected
+ * (colProp < rowProp, as at :1064-1069).  Inspect with mx_partition_get(); release with
+ * mx_partition_destroy(). */
+inline mx_partition *matxtract_preprocess(valT *csrVal, indT *csrRowPtr, indT *csrColInd, int rowA, int colA, indT nnzA,
+                                          float colProp, float rowProp)
+{
+    mx_csr A;
+    A.rows = rowA;
+    A.cols = colA;
+    A.nnz = nnzA;
+    A.dtype = MX_VALT_DTYPE;
+    A.rowPtr = csrRowPtr;
+    A.colInd = csrColInd;
+    A.val = csrVal;
+    mx_partition *p = nullptr;
+    if (mx_partition_create(&A, colProp, rowProp, &p) != MX_OK) {
+        std::fprintf(stderr, "matxtract_preprocess: %s\n", mx_last_error());
+        return nullptr;
+    }
+    return p;
+}
+
+/* y = A*x through a persistent plan built from a partition: the compute entry point.
+ * Host pointers; see mx_spmv() for device pointers. */
+inline void matxtract_compute(mx_plan *plan, valT *X_val, valT *Y_val)
+{
+    matxtract_detail::check(mx_spmv_host(plan, X_val, Y_val), "matxtract_compute");
+}
+
+#endif /* MATXTRACT_H */

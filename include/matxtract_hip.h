@@ -1,0 +1,218 @@
+/*
+ * matxtract_hip.h -- C ABI of libmatxtract_hip.so, the MI355X (gfx950) implementation of
+ * MatXtract's hybrid SpMV path.
+ *
+ * Plain C: opaque handles, plain pointers and sizes, int status codes (0 = MX_OK), no C++
+ * or torch types.  Every entry point names the reference interface it stands in for
+ * (paths relative to the reference repository).  binary16 values cross this boundary as
+ * their uint16_t bit pattern.
+ *
+ * Two groups:
+ *   1. host-only: partition (the cascaded extraction), Matrix-Market ingest, transposes,
+ *      synthetic workload generators.  Usable on a machine without a GPU.
+ *   2. device: plans (persistent device copies of a partition) and the SpMV itself.
+ *      These fail with MX_ERR_DEVICE when no HIP device is present; there is no CPU
+ *      fallback.
+ */
+#ifndef MATXTRACT_HIP_H
+#define MATXTRACT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MX_OK 0
+#define MX_ERR_ARG 1     /* bad argument (null pointer, negative size, tau_c < tau_r ...) */
+#define MX_ERR_ALLOC 2   /* host or device allocation failed */
+#define MX_ERR_DEVICE 3  /* HIP runtime error or no device */
+#define MX_ERR_IO 4      /* file could not be opened / parsed */
+
+typedef enum mx_dtype {
+    MX_F64 = 0, /* binary64 values, binary64 accumulation, 8x4 tiles, 32-bit bitmaps */
+    MX_F16 = 1  /* binary16 values, binary32 accumulation, 8x8 tiles, 64-bit bitmaps */
+} mx_dtype;
+
+/* The CSR triple of the reference (`valT *csrVal, indT *csrRowPtr, indT *csrColInd`,
+ * include/common.h:53-79; produced by mmio_allinone, utilities/mmio.cpp:1547-1713). */
+typedef struct mx_csr {
+    int rows, cols, nnz;
+    mx_dtype dtype;
+    const int *rowPtr;  /* [rows+1] */
+    const int *colInd;  /* [nnz], any order inside a row, duplicates allowed */
+    const void *val;    /* [nnz] double | uint16_t(binary16) */
+} mx_csr;
+
+typedef struct mx_partition mx_partition; /* host result of the cascaded extraction */
+typedef struct mx_plan mx_plan;           /* device-resident executable form */
+
+/* Read-only view of the canonical partition arrays; names are the reference driver's
+ * (test/test_autotc_spmv.cpp:1106-1492).  Pointers stay valid until the partition is
+ * destroyed. */
+typedef struct mx_partition_view {
+    mx_dtype dtype;
+    int rows, cols, nnz;
+    int fragM, fragK;
+    int dCols, sCols, nnzColD, nnzColS;
+    int dRows, sRows, nnzRowD, nnzRowS;
+    float cols_ratio;     /* dCols / cols, printed as "cols_ratio" (:1142) */
+    double tc_nnz_ratio;  /* nnzRowD / (totalTcFrags*fragM*fragK), "TC_nnz_ratio" (:1376) */
+    const int *descColId; /* [cols]  columns by nnz desc (ties: ascending id); NULL at tau=(0,0) */
+    const int *newArray;  /* [sCols] columns not extracted, ascending */
+    const int *rId;       /* [dRows] extracted rows, rank order */
+    const int *newArray_; /* [sRows] rows not extracted, ascending */
+    const int *ddRowPtr;  /* A_dd (dRows x dCols) as CSR */
+    const int *ddColInd;
+    const void *ddVal;
+    int chunkNum, totalTcFrags, tcValCount;
+    const int *chunkPtr;          /* [chunkNum+1] */
+    const int *sparse_AToX_index; /* [totalTcFrags*fragK] */
+    const int *fragPtr;           /* [totalTcFrags+1] */
+    const void *fragBit;          /* [totalTcFrags] uint32_t (F64) | uint64_t (F16) */
+    const void *tcVal;            /* [tcValCount] */
+    int nnzCD;
+    const int *cdRowPtr;  /* residual A_CD (rows x cols): columns [0,dCols) = dense-column */
+    const int *cdColInd;  /* ranks, [dCols,cols) = dCols + index into newArray             */
+    const void *cdVal;
+} mx_partition_view;
+
+/* ---------------------------------------------------------------------------------- */
+/* 1. host-only                                                                        */
+
+/* Last error text of the calling thread ("" if none). */
+const char *mx_last_error(void);
+
+/* Cascaded compute-density extraction: column pass with tau_c (`global_col`), then row
+ * pass with tau_r (`local_row`), tile format over A_dd, residual A_CD.  Stands in for the
+ * code inlined in the reference driver's main(), test/test_autotc_spmv.cpp:1106-1427 and
+ * merge2CSR_opt (:129-250), ecrPreprocess_opt1 (:502-585), generateFormat_opt[_fp16]
+ * (:718-978).  tau_c < tau_r is rejected as the driver does (:1064-1069); tau=(0,0)
+ * yields an empty tile part and A itself as residual (:1638-1658). */
+int mx_partition_create(const mx_csr *A, float tau_c, float tau_r, mx_partition **out);
+void mx_partition_destroy(mx_partition *p);
+int mx_partition_get(const mx_partition *p, mx_partition_view *view);
+/* 64-bit FNV-1a over the canonical arrays (dCols, dRows, descColId[0..dCols), newArray, rId,
+ * newArray_, chunkPtr, sparse_AToX_index, fragPtr, fragBit, tcVal, cdRowPtr, cdColInd,
+ * cdVal), little-endian, in that order. */
+uint64_t mx_partition_hash(const mx_partition *p);
+
+/* csr2csc / csc2csr of utilities/csr2csc.cpp:4-203 as a host transpose: each output line
+ * lists its entries by ascending source line, equal pairs in source order.  Outputs are
+ * malloc()ed by the callee and released by the caller with free() or mx_free(), as in
+ * the reference (csr2csc.cpp:15-17). `outer` = number of source lines (rows for csr2csc),
+ * `inner` = number of output lines. */
+int mx_transpose(mx_dtype dtype, int outer, int inner, int nnz, const int *ptr, const int *ind,
+                 const void *val, int **tPtr, int **tInd, void **tVal);
+void mx_free(void *p);
+
+/* mmio_allinone (utilities/mmio.cpp:1547-1713): Matrix-Market coordinate file -> CSR with
+ * entries kept in file order inside each row, symmetric/hermitian/skew files expanded,
+ * pattern files given value 1.  Outputs malloc()ed; returns MX_ERR_IO on failure. */
+int mx_mmio_read(const char *path, mx_dtype dtype, int *rows, int *cols, int *nnz, int *isSymmetric,
+                 int **rowPtr, int **colInd, void **val);
+
+/* initVec (include/common.h:237-245): v[i] = (valT)(float)(i % 15). */
+void mx_init_vec(mx_dtype dtype, void *v, int n);
+
+/* binary16 <-> binary32, round to nearest even: the conversions behind CUDA's host-side
+ * `half` that the reference's valT relies on (include/common.h:60). */
+uint16_t mx_f32_to_f16(float f);
+float mx_f16_to_f32(uint16_t h);
+
+/* Synthetic workloads 1..5 (seeded; see mx_gen.cpp for the exact recipes).  `scale`
+ * in (0,1] shrinks the row count (1 = full size).  Outputs malloc()ed: the matrix and
+ * the input vector x.  The reference has no generators; these define the benchmark. */
+int mx_gen_config(int config_id, uint64_t seed, double scale, int *rows, int *cols, int *nnz,
+                  mx_dtype *dtype, int **rowPtr, int **colInd, void **val, void **x);
+
+/* Algorithmic bytes of one SpMV: nnz*(sizeof(valT)+4) + (rows+1)*4 + cols*sizeof(valT) +
+ * rows*sizeof(valT) (`data_origin1`, test/test_cdspmv.cpp:214). */
+double mx_algorithmic_bytes(mx_dtype dtype, int rows, int cols, int nnz);
+
+/* ---------------------------------------------------------------------------------- */
+/* 2. device                                                                           */
+
+/* Plan flags */
+#define MX_PLAN_DEFAULT 0
+#define MX_PLAN_NO_TILES 1   /* run the extracted block A_dd through the CSR kernel too */
+#define MX_PLAN_ALL_TILES 2  /* run every extracted chunk through the MFMA tile kernel */
+
+/* Uploads a partition once and keeps it on the device: the persistent counterpart of the
+ * per-call cudaMalloc/cudaMemcpy blocks in cdspmv (src/spmv_kernel/cdSpMV.cu:407-418) and
+ * du_tcspmv_fp64 (src/spmv_kernel/du_tcSpMV_fp64.cu:271-300), plus the x_d/x_s/x_CD
+ * permutation of test/test_autotc_spmv.cpp:1454-1463 folded into the column indices so that
+ * x and y are used in the caller's own ordering. */
+int mx_plan_create(const mx_partition *p, int flags, mx_plan **out);
+void mx_plan_destroy(mx_plan *plan);
+
+/* y = A*x on the device.  x [cols] and y [rows] are DEVICE pointers of the plan's value
+ * type; `stream` is a hipStream_t (NULL = default stream).  Asynchronous.  The hybrid
+ * sequence of test/test_autotc_spmv.cpp:1507-1559 (tile part, scatter through rId,
+ * residual accumulated on top) without host round trips. */
+int mx_spmv(mx_plan *plan, const void *x_dev, void *y_dev, void *stream);
+
+/* Same with HOST pointers (allocates nothing persistent; copies x in and y out). */
+int mx_spmv_host(mx_plan *plan, const void *x_host, void *y_host);
+
+/* The reference's timing protocol (200 warm-ups + 4000 timed back-to-back launches,
+ * src/spmv_kernel/cdSpMV.cu:454-479, du_tcSpMV_fp64.cu:311-333) on the plan's own stream.
+ * ms_total: mean per SpMV of the whole sequence (hipEvents around the loop);
+ * ms_tile / ms_csr: mean per launch of each kernel timed on its own (the two numbers the
+ * reference adds up, test/test_autotc_spmv.cpp:1561-1572); any may be NULL. */
+int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters,
+            double *ms_total, double *ms_tile, double *ms_csr);
+
+/* Facts about a plan, for reporting. */
+typedef struct mx_plan_info {
+    mx_dtype dtype;
+    int rows, cols, nnz;
+    int tile_chunks;     /* chunks executed by the MFMA tile kernel */
+    int tile_frags;      /* fragments executed by the MFMA tile kernel */
+    int tile_nnz;        /* matrix entries held in those fragments */
+    int csr_nnz;         /* entries executed by the CSR kernel */
+    int csr_blocks;      /* workgroups of the CSR kernel */
+    double tile_bytes;   /* bytes the tile kernel must read+write per launch */
+    double csr_bytes;    /* bytes the CSR kernel must read+write per launch */
+} mx_plan_info;
+int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
+
+/* Reference surface, host pointers in / host pointers out, one-shot (allocate, upload,
+ * `warm` + `iters` timed launches into a scratch y, one real launch, download, free).
+ * The C++ functions of include/MatXtract.h are inline wrappers over these.
+ *
+ * mx_cdspmv_*: cdspmv(), include/MatXtract.h:3-5, src/spmv_kernel/cdSpMV.cu:395-491.
+ *   y is IN/OUT: y += A*x.  cdTime = mean ms per launch, cdPre = ms spent building the
+ *   workgroup row map (the reference's pre_startRowPerBlock). */
+int mx_cdspmv_f64(const double *csrVal, const int *csrRowPtr, const int *csrColInd, const double *x,
+                  double *y, int rows, int cols, int nnz, int warm, int iters, double *cdTime,
+                  double *cdPre);
+int mx_cdspmv_f16(const uint16_t *csrVal, const int *csrRowPtr, const int *csrColInd,
+                  const uint16_t *x, uint16_t *y, int rows, int cols, int nnz, int warm, int iters,
+                  double *cdTime, double *cdPre);
+/* mx_du_tcspmv_f64: du_tcspmv_fp64(), include/MatXtract.h:7-9,
+ *   src/spmv_kernel/du_tcSpMV_fp64.cu:258-350.  y is IN/OUT (y += A_dd*x_d).
+ * mx_du_tcspmv_f16: du_tcspmv_fp16_v2(), include/MatXtract.h:27-29,
+ *   src/spmv_kernel/du_tcSpMV_fp16_v2.cu:112-203.  y is overwritten. */
+int mx_du_tcspmv_f64(const int *chunkPtr, const int *fragPtr, const uint32_t *fragBit,
+                     const double *tcVal, const int *sparse_AToX_index, const double *x_d, double *y_d,
+                     int dRows, int dCols, int warm, int iters, double *tcTime);
+int mx_du_tcspmv_f16(const int *chunkPtr, const int *fragPtr, const uint64_t *fragBit,
+                     const uint16_t *tcVal, const int *sparse_AToX_index, const uint16_t *x_d,
+                     uint16_t *y_d, int dRows, int dCols, int warm, int iters, double *tcTime);
+
+/* Number of HIP devices visible (0 when none; never fails). */
+int mx_device_count(void);
+
+/* Diagnostics: D(16x16) = A*B on one wave through the MFMA instruction the tile kernels use,
+ * operands moved with the lane mapping those kernels assume (A 16x4, B 4x16 binary64;
+ * A 16x32, B 32x16 binary16 with a binary32 result), all row-major HOST arrays.  No
+ * counterpart in the reference; the test-suite uses them to pin the operand layout. */
+int mx_probe_mfma_f64(const double *A, const double *B, double *D);
+int mx_probe_mfma_f16(const uint16_t *A, const uint16_t *B, float *D);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MATXTRACT_HIP_H */

@@ -1,0 +1,109 @@
+"""ctypes loader for libmatxtract_hip.so (the C ABI declared in include/matxtract_hip.h).
+
+The library is built in-tree by ``matxtract_amd/csrc/Makefile``.  Loading fails loudly when it
+is missing: there is no Python or CPU fallback for the device entry points.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmatxtract_hip.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+MX_OK, MX_ERR_ARG, MX_ERR_ALLOC, MX_ERR_DEVICE, MX_ERR_IO = 0, 1, 2, 3, 4
+MX_F64, MX_F16 = 0, 1
+MX_PLAN_DEFAULT, MX_PLAN_NO_TILES, MX_PLAN_ALL_TILES = 0, 1, 2
+
+
+class MxError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("matxtract_hip error %d: %s" % (code, msg))
+        self.code = code
+
+
+class CsrStruct(C.Structure):
+    _fields_ = [("rows", C.c_int), ("cols", C.c_int), ("nnz", C.c_int), ("dtype", C.c_int),
+                ("rowPtr", C.c_void_p), ("colInd", C.c_void_p), ("val", C.c_void_p)]
+
+
+class PartitionView(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int), ("rows", C.c_int), ("cols", C.c_int), ("nnz", C.c_int),
+        ("fragM", C.c_int), ("fragK", C.c_int),
+        ("dCols", C.c_int), ("sCols", C.c_int), ("nnzColD", C.c_int), ("nnzColS", C.c_int),
+        ("dRows", C.c_int), ("sRows", C.c_int), ("nnzRowD", C.c_int), ("nnzRowS", C.c_int),
+        ("cols_ratio", C.c_float), ("tc_nnz_ratio", C.c_double),
+        ("descColId", C.c_void_p), ("newArray", C.c_void_p), ("rId", C.c_void_p),
+        ("newArray_", C.c_void_p),
+        ("ddRowPtr", C.c_void_p), ("ddColInd", C.c_void_p), ("ddVal", C.c_void_p),
+        ("chunkNum", C.c_int), ("totalTcFrags", C.c_int), ("tcValCount", C.c_int),
+        ("chunkPtr", C.c_void_p), ("sparse_AToX_index", C.c_void_p), ("fragPtr", C.c_void_p),
+        ("fragBit", C.c_void_p), ("tcVal", C.c_void_p),
+        ("nnzCD", C.c_int),
+        ("cdRowPtr", C.c_void_p), ("cdColInd", C.c_void_p), ("cdVal", C.c_void_p),
+    ]
+
+
+class PlanInfo(C.Structure):
+    _fields_ = [("dtype", C.c_int), ("rows", C.c_int), ("cols", C.c_int), ("nnz", C.c_int),
+                ("tile_chunks", C.c_int), ("tile_frags", C.c_int), ("tile_nnz", C.c_int),
+                ("csr_nnz", C.c_int), ("csr_blocks", C.c_int),
+                ("tile_bytes", C.c_double), ("csr_bytes", C.c_double)]
+
+
+# Every symbol include/matxtract_hip.h declares: name -> (restype, argtypes)
+_vp, _i, _d = C.c_void_p, C.c_int, C.c_double
+_pp = C.POINTER(C.c_void_p)
+_pi = C.POINTER(C.c_int)
+_pd = C.POINTER(C.c_double)
+SIGNATURES = {
+    "mx_last_error": (C.c_char_p, []),
+    "mx_partition_create": (_i, [C.POINTER(CsrStruct), C.c_float, C.c_float, _pp]),
+    "mx_partition_destroy": (None, [_vp]),
+    "mx_partition_get": (_i, [_vp, C.POINTER(PartitionView)]),
+    "mx_partition_hash": (C.c_uint64, [_vp]),
+    "mx_transpose": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _pp, _pp, _pp]),
+    "mx_free": (None, [_vp]),
+    "mx_mmio_read": (_i, [C.c_char_p, _i, _pi, _pi, _pi, _pi, _pp, _pp, _pp]),
+    "mx_init_vec": (None, [_i, _vp, _i]),
+    "mx_f32_to_f16": (C.c_uint16, [C.c_float]),
+    "mx_f16_to_f32": (C.c_float, [C.c_uint16]),
+    "mx_gen_config": (_i, [_i, C.c_uint64, _d, _pi, _pi, _pi, _pi, _pp, _pp, _pp, _pp]),
+    "mx_algorithmic_bytes": (_d, [_i, _i, _i, _i]),
+    "mx_plan_create": (_i, [_vp, _i, _pp]),
+    "mx_plan_destroy": (None, [_vp]),
+    "mx_spmv": (_i, [_vp, _vp, _vp, _vp]),
+    "mx_spmv_host": (_i, [_vp, _vp, _vp]),
+    "mx_time": (_i, [_vp, _vp, _vp, _i, _i, _pd, _pd, _pd]),
+    "mx_plan_get_info": (_i, [_vp, C.POINTER(PlanInfo)]),
+    "mx_cdspmv_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _pd, _pd]),
+    "mx_cdspmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _pd, _pd]),
+    "mx_du_tcspmv_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _pd]),
+    "mx_du_tcspmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _pd]),
+    "mx_device_count": (_i, []),
+    "mx_probe_mfma_f64": (_i, [_vp, _vp, _vp]),
+    "mx_probe_mfma_f16": (_i, [_vp, _vp, _vp]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library (raises if it has not been built)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "%s not found: build it with `make -C %s` (or __graft_entry__.build())" % (LIB_PATH, CSRC))
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != MX_OK:
+        raise MxError(rc, load().mx_last_error().decode("utf-8", "replace"))

@@ -1,0 +1,254 @@
+"""Python face of libmatxtract_hip.so: numpy in/out for the host calls, torch tensors (device
+memory and streams only) for the device calls.  Every function forwards to one C-ABI entry
+point; nothing is computed in Python.
+
+Names follow the reference driver (test/test_autotc_spmv.cpp): a ``Partition`` is what its
+main() derives from (A, col_frac, hot_frac); a ``Plan`` is that partition resident on the GPU.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_DEFAULT, MX_PLAN_NO_TILES, MxError,
+                   check)
+
+__all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "cdspmv",
+           "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "MxError",
+           "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES"]
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _np_dtype(dt):
+    return np.float64 if dt == MX_F64 else np.float16
+
+
+def _take(addr, n, dtype, free=True):
+    """Copy n items from a malloc()ed C array into numpy, then release it."""
+    dtype = np.dtype(dtype)
+    if n > 0 and addr:
+        buf = (C.c_char * (n * dtype.itemsize)).from_address(addr)
+        out = np.frombuffer(buf, dtype=dtype, count=n).copy()
+    else:
+        out = np.zeros(0, dtype)
+    if free and addr:
+        _lib.load().mx_free(addr)
+    return out
+
+
+def _view(addr, n, dtype):
+    return _take(addr, n, dtype, free=False)
+
+
+def device_count():
+    return _lib.load().mx_device_count()
+
+
+def algorithmic_bytes(dtype, rows, cols, nnz):
+    return _lib.load().mx_algorithmic_bytes(dtype, rows, cols, nnz)
+
+
+class Csr:
+    """The reference's CSR triple (csrVal, csrRowPtr, csrColInd) plus its shape."""
+
+    def __init__(self, rows, cols, rowPtr, colInd, val):
+        self.rows, self.cols = int(rows), int(cols)
+        self.rowPtr = np.ascontiguousarray(rowPtr, dtype=np.int32)
+        self.colInd = np.ascontiguousarray(colInd, dtype=np.int32)
+        val = np.ascontiguousarray(val)
+        if val.dtype == np.uint16:
+            val = val.view(np.float16)
+        if val.dtype not in (np.float64, np.float16):
+            raise TypeError("values must be float64 or float16")
+        self.val = val
+        self.nnz = int(len(self.colInd))
+        self.dtype = MX_F64 if val.dtype == np.float64 else MX_F16
+
+    def struct(self):
+        return _lib.CsrStruct(self.rows, self.cols, self.nnz, self.dtype, _p(self.rowPtr).value,
+                              _p(self.colInd).value, _p(self.val).value)
+
+    @property
+    def algorithmic_bytes(self):
+        return algorithmic_bytes(self.dtype, self.rows, self.cols, self.nnz)
+
+
+def gen_config(config_id, seed=0, scale=1.0):
+    """Synthetic workload 1..5 -> (Csr, x)."""
+    L = _lib.load()
+    rows, cols, nnz, dt = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+    rp, ci, va, xv = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
+    check(L.mx_gen_config(config_id, seed, scale, C.byref(rows), C.byref(cols), C.byref(nnz), C.byref(dt),
+                          C.byref(rp), C.byref(ci), C.byref(va), C.byref(xv)))
+    vt = _np_dtype(dt.value)
+    A = Csr(rows.value, cols.value, _take(rp.value, rows.value + 1, np.int32),
+            _take(ci.value, nnz.value, np.int32), _take(va.value, nnz.value, vt))
+    return A, _take(xv.value, cols.value, vt)
+
+
+def mmio_read(path, dtype=MX_F64):
+    L = _lib.load()
+    rows, cols, nnz, sym = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+    rp, ci, va = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    check(L.mx_mmio_read(str(path).encode(), dtype, C.byref(rows), C.byref(cols), C.byref(nnz), C.byref(sym),
+                         C.byref(rp), C.byref(ci), C.byref(va)))
+    A = Csr(rows.value, cols.value, _take(rp.value, rows.value + 1, np.int32),
+            _take(ci.value, nnz.value, np.int32), _take(va.value, nnz.value, _np_dtype(dtype)))
+    return A, bool(sym.value)
+
+
+def init_vec(n, dtype=MX_F64):
+    v = np.zeros(n, _np_dtype(dtype))
+    _lib.load().mx_init_vec(dtype, _p(v), n)
+    return v
+
+
+def transpose(ptr, ind, val, inner):
+    """csr2csc / csc2csr: stable counting-sort transpose."""
+    ptr = np.ascontiguousarray(ptr, dtype=np.int32)
+    ind = np.ascontiguousarray(ind, dtype=np.int32)
+    val = np.ascontiguousarray(val)
+    dt = MX_F64 if val.dtype == np.float64 else MX_F16
+    tp, ti, tv = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    check(_lib.load().mx_transpose(dt, len(ptr) - 1, inner, len(ind), _p(ptr), _p(ind), _p(val),
+                                   C.byref(tp), C.byref(ti), C.byref(tv)))
+    return (_take(tp.value, inner + 1, np.int32), _take(ti.value, len(ind), np.int32),
+            _take(tv.value, len(ind), val.dtype))
+
+
+class Partition:
+    """Result of the cascaded extraction (column pass tau_c, then row pass tau_r)."""
+
+    ARRAYS = ("descColId", "newArray", "rId", "newArray_", "ddRowPtr", "ddColInd", "ddVal", "chunkPtr",
+              "sparse_AToX_index", "fragPtr", "fragBit", "tcVal", "cdRowPtr", "cdColInd", "cdVal")
+
+    def __init__(self, A, tau_c, tau_r):
+        self._h = C.c_void_p()
+        self._A = A  # keep the input arrays alive during the call
+        st = A.struct()
+        check(_lib.load().mx_partition_create(C.byref(st), float(tau_c), float(tau_r), C.byref(self._h)))
+        v = _lib.PartitionView()
+        check(_lib.load().mx_partition_get(self._h, C.byref(v)))
+        for name, _ in _lib.PartitionView._fields_:
+            if name not in self.ARRAYS:
+                setattr(self, name, getattr(v, name))
+        vt = _np_dtype(v.dtype)
+        bt = np.uint32 if v.dtype == MX_F64 else np.uint64
+        self.descColId = _view(v.descColId, v.cols if v.descColId else 0, np.int32)
+        self.newArray = _view(v.newArray, v.sCols, np.int32)
+        self.rId = _view(v.rId, v.dRows, np.int32)
+        self.newArray_ = _view(v.newArray_, v.sRows, np.int32)
+        self.ddRowPtr = _view(v.ddRowPtr, v.dRows + 1, np.int32)
+        self.ddColInd = _view(v.ddColInd, v.nnzRowD, np.int32)
+        self.ddVal = _view(v.ddVal, v.nnzRowD, vt)
+        self.chunkPtr = _view(v.chunkPtr, v.chunkNum + 1, np.int32)
+        self.sparse_AToX_index = _view(v.sparse_AToX_index, v.totalTcFrags * v.fragK, np.int32)
+        self.fragPtr = _view(v.fragPtr, v.totalTcFrags + 1, np.int32)
+        self.fragBit = _view(v.fragBit, v.totalTcFrags, bt)
+        self.tcVal = _view(v.tcVal, v.tcValCount, vt)
+        self.cdRowPtr = _view(v.cdRowPtr, v.rows + 1, np.int32)
+        self.cdColInd = _view(v.cdColInd, v.nnzCD, np.int32)
+        self.cdVal = _view(v.cdVal, v.nnzCD, vt)
+
+    @property
+    def hash(self):
+        return _lib.load().mx_partition_hash(self._h)
+
+    def close(self):
+        if self._h:
+            _lib.load().mx_partition_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _torch_dtype(dt):
+    import torch
+    return torch.float64 if dt == MX_F64 else torch.float16
+
+
+class Plan:
+    """A partition resident on the GPU; ``spmv`` computes y = A x there."""
+
+    def __init__(self, partition, flags=MX_PLAN_DEFAULT):
+        self._h = C.c_void_p()
+        check(_lib.load().mx_plan_create(partition._h, int(flags), C.byref(self._h)))
+        info = _lib.PlanInfo()
+        check(_lib.load().mx_plan_get_info(self._h, C.byref(info)))
+        self.info = {k: getattr(info, k) for k, _ in _lib.PlanInfo._fields_}
+        self.dtype, self.rows, self.cols, self.nnz = info.dtype, info.rows, info.cols, info.nnz
+
+    def _check_vec(self, t, n, name):
+        if (not t.is_cuda) or t.dtype != _torch_dtype(self.dtype) or t.numel() != n or not t.is_contiguous():
+            raise ValueError("%s must be a contiguous device tensor of %d %s" % (name, n, _torch_dtype(self.dtype)))
+
+    def spmv(self, x, y=None, stream=None):
+        """y = A x; x, y torch device tensors.  Launches on `stream` (default: torch's current)."""
+        import torch
+        if y is None:
+            y = torch.empty(self.rows, dtype=x.dtype, device=x.device)
+        self._check_vec(x, self.cols, "x")
+        self._check_vec(y, self.rows, "y")
+        s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+        check(_lib.load().mx_spmv(self._h, x.data_ptr(), y.data_ptr(), s))
+        return y
+
+    def spmv_host(self, x):
+        x = np.ascontiguousarray(x, dtype=_np_dtype(self.dtype))
+        if x.size != self.cols:
+            raise ValueError("x must have %d entries" % self.cols)
+        y = np.zeros(self.rows, x.dtype)
+        check(_lib.load().mx_spmv_host(self._h, _p(x), _p(y)))
+        return y
+
+    def time(self, x, y, warm=200, iters=4000, parts=True):
+        """Mean ms per SpMV by HIP events on the plan's stream -> (total, tile, csr)."""
+        self._check_vec(x, self.cols, "x")
+        self._check_vec(y, self.rows, "y")
+        t, tt, tc = C.c_double(), C.c_double(), C.c_double()
+        check(_lib.load().mx_time(self._h, x.data_ptr(), y.data_ptr(), warm, iters, C.byref(t),
+                                  C.byref(tt) if parts else None, C.byref(tc) if parts else None))
+        return t.value, tt.value, tc.value
+
+    def close(self):
+        if self._h:
+            _lib.load().mx_plan_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def cdspmv(A, x, y, warm=0, iters=0):
+    """Reference cdspmv(): y += A x, host arrays in and out -> (y, cdTime_ms, cdPre_ms)."""
+    vt = _np_dtype(A.dtype)
+    x = np.ascontiguousarray(x, dtype=vt)
+    y = np.array(y, dtype=vt)
+    t, pre = C.c_double(), C.c_double()
+    fn = _lib.load().mx_cdspmv_f64 if A.dtype == MX_F64 else _lib.load().mx_cdspmv_f16
+    check(fn(_p(A.val), _p(A.rowPtr), _p(A.colInd), _p(x), _p(y), A.rows, A.cols, A.nnz, warm, iters,
+             C.byref(t), C.byref(pre)))
+    return y, t.value, pre.value
+
+
+def du_tcspmv(part, x_d, y_d=None, warm=0, iters=0):
+    """Reference du_tcspmv_fp64 / du_tcspmv_fp16_v2 on a partition's canonical tile arrays."""
+    dt = part.dtype
+    vt = _np_dtype(dt)
+    x_d = np.ascontiguousarray(x_d, dtype=vt)
+    y = np.zeros(part.dRows, vt) if y_d is None else np.array(y_d, dtype=vt)
+    t = C.c_double()
+    fn = _lib.load().mx_du_tcspmv_f64 if dt == MX_F64 else _lib.load().mx_du_tcspmv_f16
+    check(fn(_p(part.chunkPtr), _p(part.fragPtr), _p(part.fragBit), _p(part.tcVal), _p(part.sparse_AToX_index),
+             _p(x_d), _p(y), part.dRows, part.dCols, warm, iters, C.byref(t)))
+    return y, t.value

@@ -1,0 +1,40 @@
+// Device-side views shared by the plan code and the kernel launchers.
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include "matxtract_hip.h"
+
+namespace mx {
+
+// CSR matrix resident on the device, plus the row ranges of the CSR kernel's workgroups.
+// col/val carry kCsrPad extra zero entries so that aligned 128-bit loads may overrun.
+struct DeviceCsr {
+    int rows = 0, nnz = 0;
+    int *rowPtr = nullptr;    // [rows+1]
+    int *col = nullptr;       // [nnz + kCsrPad]
+    void *val = nullptr;      // [nnz + kCsrPad]
+    int *blockRow = nullptr;  // [nBlocks+1] first row of each workgroup
+    int nBlocks = 0;
+};
+constexpr int kCsrPad = 16;
+
+// Bitmap tiles resident on the device (the reference's chunkPtr / fragPtr / fragBit / tcVal /
+// sparse_AToX_index, restricted to the chunks the tile kernel executes).
+struct DeviceTiles {
+    int chunkNum = 0;  // executed chunks
+    int dRows = 0;     // 8*chunkNum, or fewer when the last chunk is ragged
+    int frags = 0, vals = 0;
+    int *chunkPtr = nullptr;  // [chunkNum+1]
+    int *fragPtr = nullptr;   // [frags+1]
+    void *fragBit = nullptr;  // [frags] u32 | u64
+    void *tcVal = nullptr;    // [vals]
+    int *atox = nullptr;      // [frags*fragK] indices into the x handed to the kernel
+    int *rowIdx = nullptr;    // [dRows] output row of each tile row; nullptr = identity
+};
+
+hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s);
+hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s);
+hipError_t launch_probe_f64(const double *A, const double *B, double *D, hipStream_t s);
+hipError_t launch_probe_f16(const void *A, const void *B, float *D, hipStream_t s);
+
+}  // namespace mx

@@ -1,0 +1,55 @@
+// Internal declarations shared by the translation units of libmatxtract_hip.so.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "matxtract_hip.h"
+
+namespace mx {
+
+inline int elem_size(mx_dtype d) { return d == MX_F64 ? 8 : 2; }
+inline int frag_k(mx_dtype d) { return d == MX_F64 ? 4 : 8; }
+constexpr int kFragM = 8;
+
+void set_error(const std::string &msg);
+
+// double -> binary16 bits, round to nearest even, straight from the double (no
+// intermediate float rounding); binary16 bits -> float.
+uint16_t f64_to_f16_bits(double v);
+float f16_bits_to_f32(uint16_t h);
+
+// Raw byte buffer holding matrix values of either type.
+struct ValBuf {
+    std::vector<unsigned char> bytes;
+    void resize(size_t n, int elem) { bytes.assign(n * (size_t)elem, 0); }
+    void *data() { return bytes.data(); }
+    const void *data() const { return bytes.data(); }
+};
+
+}  // namespace mx
+
+// Host result of the cascaded extraction; arrays named as in the reference driver.
+struct mx_partition {
+    mx_dtype dtype = MX_F64;
+    int rows = 0, cols = 0, nnz = 0;
+    int fragM = 8, fragK = 4;
+    float tau_c = 0.f, tau_r = 0.f;
+    int dCols = 0, sCols = 0, nnzColD = 0, nnzColS = 0;
+    int dRows = 0, sRows = 0, nnzRowD = 0, nnzRowS = 0;
+    float cols_ratio = 0.f;
+    double tc_nnz_ratio = 0.0;
+    bool extracted = false;  // false at tau = (0,0)
+    std::vector<int> descColId, newArray, rId, newArray_;
+    std::vector<int> ddRowPtr, ddColInd;
+    mx::ValBuf ddVal;
+    int chunkNum = 0, totalTcFrags = 0, tcValCount = 0;
+    std::vector<int> chunkPtr, sparse_AToX_index, fragPtr;
+    std::vector<uint64_t> fragBit64;  // F16
+    std::vector<uint32_t> fragBit32;  // F64
+    mx::ValBuf tcVal;
+    int nnzCD = 0;
+    std::vector<int> cdRowPtr, cdColInd;
+    mx::ValBuf cdVal;
+};

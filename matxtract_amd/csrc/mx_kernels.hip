@@ -1,0 +1,364 @@
+// gfx950 kernels of the hybrid SpMV and their launchers.
+//
+//   csr_rows_kernel   residual / plain CSR part (stands in for cdspmv_kernel,
+//                     src/spmv_kernel/cdSpMV.cu:244-392).  HBM-bound.
+//   tile_f64_kernel   8x4 bitmap tiles through v_mfma_f64_16x16x4_f64 (stands in for
+//                     tcspmv_kernel_fp64, src/spmv_kernel/du_tcSpMV_fp64.cu:81-160).
+//   tile_f16_kernel   8x8 bitmap tiles through v_mfma_f32_16x16x32_f16, f32 accumulation
+//                     (stands in for tcspmv_kernel_fp16_v2, du_tcSpMV_fp16_v2.cu:4-110).
+//
+// Row ownership: every output row is written by exactly one lane of one workgroup in each
+// kernel, so there are no atomics anywhere; the tile kernel runs after the CSR kernel on the
+// same stream and adds its rows on top with a plain read-modify-write.
+#include <hip/hip_runtime.h>
+
+#include "mx_device.h"
+
+namespace mxk {
+
+typedef double v4f64 __attribute__((ext_vector_type(4)));
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef double v2f64 __attribute__((ext_vector_type(2)));
+
+constexpr int kBlock = 256;  // 4 wave64 per workgroup
+
+// Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
+// Re-map so that every XCD walks one contiguous range of logical blocks: neighbouring rows
+// (and the x entries they share) then live in a single L2 instead of all eight.
+__device__ __forceinline__ int xcd_contiguous_block(int bid, int nb)
+{
+    const int q = nb >> 3, rem = nb & 7;
+    const int xcd = bid & 7, idx = bid >> 3;
+    return xcd * q + (xcd < rem ? xcd : rem) + idx;
+}
+
+// ---- cross-lane moves -------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp(double v)
+{
+    const long long b = __builtin_bit_cast(long long, v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)b, CTRL, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, 0xf, 0xf, false);
+    return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)(unsigned)lo);
+}
+__device__ __forceinline__ float swizzle_x16(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+}
+__device__ __forceinline__ double swizzle_x16(double v)
+{
+    const long long b = __builtin_bit_cast(long long, v);
+    const int lo = __builtin_amdgcn_ds_swizzle((int)b, 0x401F);
+    const int hi = __builtin_amdgcn_ds_swizzle((int)(b >> 32), 0x401F);
+    return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)(unsigned)lo);
+}
+
+// Sum over aligned groups of W lanes (W a power of two <= 64); every lane of the group ends
+// up with the total.  Steps 1,2 are quad permutes, 4 and 8 row mirrors (DPP), 16 a
+// ds_swizzle lane-xor, 32 a bpermute.
+template <int W, typename T>
+__device__ __forceinline__ T group_sum(T v)
+{
+    if (W >= 2) v += dpp<0xB1>(v);   // quad_perm [1,0,3,2]
+    if (W >= 4) v += dpp<0x4E>(v);   // quad_perm [2,3,0,1]
+    if (W >= 8) v += dpp<0x141>(v);  // row_half_mirror
+    if (W >= 16) v += dpp<0x140>(v); // row_mirror
+    if (W >= 32) v += swizzle_x16(v);
+    if (W >= 64) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+// ---- CSR part ---------------------------------------------------------------------------
+template <typename VT>
+struct Traits;
+template <>
+struct Traits<double> {
+    typedef double acc_t;
+    static constexpr int NPT = 4;  // entries per lane per tile: one 128-bit index load
+};
+template <>
+struct Traits<_Float16> {
+    typedef float acc_t;
+    static constexpr int NPT = 8;  // one 128-bit value load
+};
+
+template <typename VT, int W>
+__device__ __forceinline__ void reduce_rows(const typename Traits<VT>::acc_t *prod, const int *__restrict__ rowPtr,
+                                            int r0, int nrows, int base, VT *__restrict__ y, int accumulate, int tid)
+{
+    typedef typename Traits<VT>::acc_t AT;
+    constexpr int rowsPerPass = kBlock / W;
+    const int g = tid / W, l = tid % W;
+    for (int rr = g; rr < nrows; rr += rowsPerPass) {
+        const int r = r0 + rr;
+        const int a = rowPtr[r] - base, b = rowPtr[r + 1] - base;
+        AT s = 0;
+        for (int i = a + l; i < b; i += W) s += prod[i];
+        s = group_sum<W>(s);
+        if (l == 0) {
+            if (accumulate) s += (AT)y[r];
+            y[r] = (VT)s;
+        }
+    }
+}
+
+// One workgroup owns the whole rows [blockRow[b], blockRow[b+1]).  The host packs rows so
+// that their entries fit one tile of kBlock*NPT products (a single longer row gets a
+// workgroup of its own).  Phase 1 streams the tile with 128-bit loads, gathers x and parks
+// the products in LDS; phase 2 sums each row from LDS with W lanes per row, W picked from the
+// mean row length of the tile.  col/val are padded by the host so that aligned 128-bit loads
+// may run past the last entry.
+template <typename VT>
+__global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict__ rowPtr, const int *__restrict__ col,
+                                                          const VT *__restrict__ val, const VT *__restrict__ x,
+                                                          VT *__restrict__ y, const int *__restrict__ blockRow,
+                                                          int accumulate)
+{
+    typedef typename Traits<VT>::acc_t AT;
+    constexpr int NPT = Traits<VT>::NPT;
+    constexpr int TILE = kBlock * NPT;
+    __shared__ AT prod[TILE];
+    __shared__ AT wsum[kBlock / 64];
+
+    const int b = xcd_contiguous_block(blockIdx.x, gridDim.x);
+    const int tid = threadIdx.x;
+    const int r0 = blockRow[b], r1 = blockRow[b + 1];
+    if (r1 <= r0) return;
+    const int p0 = rowPtr[r0], p1 = rowPtr[r1];
+    const int base = p0 & ~(NPT - 1);
+
+    if (p1 - base <= TILE) {
+        const int i = base + tid * NPT;
+        if (i < p1) {
+            int c[NPT];
+            AT v[NPT];
+            if constexpr (sizeof(VT) == 8) {
+                const v4i32 c4 = __builtin_nontemporal_load((const v4i32 *)(col + i));
+                const v2f64 v0 = __builtin_nontemporal_load((const v2f64 *)(val + i));
+                const v2f64 v1 = __builtin_nontemporal_load((const v2f64 *)(val + i + 2));
+                c[0] = c4.x; c[1] = c4.y; c[2] = c4.z; c[3] = c4.w;
+                v[0] = v0.x; v[1] = v0.y; v[2] = v1.x; v[3] = v1.y;
+            } else {
+                const v4i32 ca = __builtin_nontemporal_load((const v4i32 *)(col + i));
+                const v4i32 cb = __builtin_nontemporal_load((const v4i32 *)(col + i + 4));
+                const v8f16 hv = __builtin_nontemporal_load((const v8f16 *)(val + i));
+                c[0] = ca.x; c[1] = ca.y; c[2] = ca.z; c[3] = ca.w;
+                c[4] = cb.x; c[5] = cb.y; c[6] = cb.z; c[7] = cb.w;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = (float)hv[j];
+            }
+            AT xv[NPT];
+#pragma unroll
+            for (int j = 0; j < NPT; ++j) xv[j] = (AT)x[c[j]];
+#pragma unroll
+            for (int j = 0; j < NPT; ++j) prod[tid * NPT + j] = v[j] * xv[j];
+        }
+        __syncthreads();
+        const int nrows = r1 - r0;
+        const int mean = (p1 - p0) / nrows;
+        if (mean <= 2) reduce_rows<VT, 1>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
+        else if (mean <= 4) reduce_rows<VT, 2>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
+        else if (mean <= 8) reduce_rows<VT, 4>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
+        else if (mean <= 16) reduce_rows<VT, 8>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
+        else if (mean <= 32) reduce_rows<VT, 16>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
+        else if (mean <= 64) reduce_rows<VT, 32>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
+        else reduce_rows<VT, 64>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
+    } else {
+        // a single row longer than one tile: strided sweep by the whole workgroup
+        AT s = 0;
+        for (int i = p0 + tid; i < p1; i += kBlock) s += (AT)val[i] * (AT)x[col[i]];
+        s = group_sum<64>(s);
+        if ((tid & 63) == 0) wsum[tid >> 6] = s;
+        __syncthreads();
+        if (tid == 0) {
+            AT t = 0;
+#pragma unroll
+            for (int w = 0; w < kBlock / 64; ++w) t += wsum[w];
+            if (accumulate) t += (AT)y[r0];
+            y[r0] = (VT)t;
+        }
+    }
+}
+
+// ---- tile part --------------------------------------------------------------------------
+// One wave per 8-row chunk, 4 chunks per workgroup.
+//
+// v_mfma_f64_16x16x4_f64 operand layout (wave64): lane L holds A[L%16][L/16], B[L/16][L%16] and
+// D[4*(L/16)+i][L%16] in accumulator register i.  A step feeds two fragments: A rows 0..7 =
+// fragment f, rows 8..15 = fragment f+1; B column 0 = the 4 gathered x of fragment f, column
+// 1 = those of fragment f+1, other columns 0.  The chunk's result is D[0..7][0] + D[8..15][1],
+// accumulated across all steps inside the matrix core, so no cross-lane reduction is needed
+// until the single combine at the end.
+__global__ __launch_bounds__(kBlock) void tile_f64_kernel(const int *__restrict__ chunkPtr, const int *__restrict__ fragPtr,
+                                                         const uint32_t *__restrict__ fragBit,
+                                                         const double *__restrict__ tcVal, const int *__restrict__ atox,
+                                                         const int *__restrict__ rowIdx, const double *__restrict__ x,
+                                                         double *__restrict__ y, int chunkNum, int dRows, int accumulate)
+{
+    const int lane = threadIdx.x & 63;
+    const int w = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (w >= chunkNum) return;
+    const int f0 = chunkPtr[w], f1 = chunkPtr[w + 1];
+    const int m = lane & 15, k = lane >> 4;
+    const int t = m >> 3;                // which of the step's two fragments this lane decodes
+    const int bitpos = (m & 7) * 4 + k;  // (local row, local column) -> bitmap bit
+    v4f64 acc = {0.0, 0.0, 0.0, 0.0};
+    for (int f = f0; f < f1; f += 2) {
+        const int fa = f + t;
+        double a = 0.0;
+        if (fa < f1) {
+            const uint32_t bm = fragBit[fa];
+            if ((bm >> bitpos) & 1u) a = tcVal[fragPtr[fa] + __popc(bm & ((1u << bitpos) - 1u))];
+        }
+        double bv = 0.0;
+        if (m < 2 && f + m < f1) bv = x[atox[(f + m) * 4 + k]];
+        acc = __builtin_amdgcn_mfma_f64_16x16x4f64(a, bv, acc, 0, 0, 0);
+    }
+    // rows 0..3: lane 0 (+ lane 33), rows 4..7: lane 16 (+ lane 49)
+    double o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = acc[i] + __shfl(acc[i], lane + 33, 64);
+    if (lane == 0 || lane == 16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int local = w * 8 + (lane >> 2) + i;  // lane 16 -> +4
+            if (local < dRows) {
+                const int row = rowIdx ? rowIdx[local] : local;
+                y[row] = accumulate ? y[row] + o[i] : o[i];
+            }
+        }
+    }
+}
+
+// v_mfma_f32_16x16x32_f16 operand layout (wave64): lane L holds A[L%16][8*(L/16) .. +7],
+// B[8*(L/16) .. +7][L%16] and D[4*(L/16)+i][L%16].  A step feeds eight 8x8 fragments of the
+// chunk: A rows 0..7 = fragments f..f+3 side by side along K, rows 8..15 = fragments f+4..f+7;
+// B column 0 = the 32 gathered x of f..f+3, column 1 = those of f+4..f+7.  A lane's eight A
+// elements are one byte of its fragment's 64-bit bitmap (one tile row), whose values sit
+// consecutively in tcVal.
+__global__ __launch_bounds__(kBlock) void tile_f16_kernel(const int *__restrict__ chunkPtr, const int *__restrict__ fragPtr,
+                                                         const uint64_t *__restrict__ fragBit,
+                                                         const _Float16 *__restrict__ tcVal, const int *__restrict__ atox,
+                                                         const int *__restrict__ rowIdx, const _Float16 *__restrict__ x,
+                                                         _Float16 *__restrict__ y, int chunkNum, int dRows, int accumulate)
+{
+    const int lane = threadIdx.x & 63;
+    const int w = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (w >= chunkNum) return;
+    const int f0 = chunkPtr[w], f1 = chunkPtr[w + 1];
+    const int m = lane & 15, g = lane >> 4;
+    const int r = m & 7;
+    v4f32 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int f = f0; f < f1; f += 8) {
+        const int fa = f + 4 * (m >> 3) + g;
+        v8f16 a = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (fa < f1) {
+            const uint64_t bm = fragBit[fa];
+            const unsigned byte = (unsigned)(bm >> (8 * r)) & 0xffu;
+            if (byte) {
+                const _Float16 *v = tcVal + fragPtr[fa] + __popcll(bm & ((1ull << (8 * r)) - 1ull));
+                int used = 0;
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if ((byte >> j) & 1u) a[j] = v[used++];
+            }
+        }
+        v8f16 bv = {0, 0, 0, 0, 0, 0, 0, 0};
+        const int fb = f + 4 * m + g;
+        if (m < 2 && fb < f1) {
+            const int4 i0 = *(const int4 *)(atox + fb * 8);
+            const int4 i1 = *(const int4 *)(atox + fb * 8 + 4);
+            bv[0] = x[i0.x]; bv[1] = x[i0.y]; bv[2] = x[i0.z]; bv[3] = x[i0.w];
+            bv[4] = x[i1.x]; bv[5] = x[i1.y]; bv[6] = x[i1.z]; bv[7] = x[i1.w];
+        }
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bv, acc, 0, 0, 0);
+    }
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = acc[i] + __shfl(acc[i], lane + 33, 64);
+    if (lane == 0 || lane == 16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int local = w * 8 + (lane >> 2) + i;
+            if (local < dRows) {
+                const int row = rowIdx ? rowIdx[local] : local;
+                const float s = accumulate ? (float)y[row] + o[i] : o[i];
+                y[row] = (_Float16)s;
+            }
+        }
+    }
+}
+
+// MFMA operand-layout probes: D = A*B for one wave, operands and result in row-major
+// global memory, loaded/stored with exactly the lane mapping the tile kernels assume.
+__global__ void probe_mfma_f64_kernel(const double *A /*16x4*/, const double *B /*4x16*/, double *D /*16x16*/)
+{
+    const int lane = threadIdx.x & 63;
+    v4f64 acc = {0.0, 0.0, 0.0, 0.0};
+    acc = __builtin_amdgcn_mfma_f64_16x16x4f64(A[(lane & 15) * 4 + (lane >> 4)], B[(lane >> 4) * 16 + (lane & 15)], acc, 0, 0, 0);
+    for (int i = 0; i < 4; ++i) D[(4 * (lane >> 4) + i) * 16 + (lane & 15)] = acc[i];
+}
+__global__ void probe_mfma_f16_kernel(const _Float16 *A /*16x32*/, const _Float16 *B /*32x16*/, float *D /*16x16*/)
+{
+    const int lane = threadIdx.x & 63;
+    v8f16 a, b;
+    for (int j = 0; j < 8; ++j) {
+        a[j] = A[(lane & 15) * 32 + 8 * (lane >> 4) + j];
+        b[j] = B[(8 * (lane >> 4) + j) * 16 + (lane & 15)];
+    }
+    v4f32 acc = {0.f, 0.f, 0.f, 0.f};
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+    for (int i = 0; i < 4; ++i) D[(4 * (lane >> 4) + i) * 16 + (lane & 15)] = acc[i];
+}
+
+}  // namespace mxk
+
+// ---- launchers (called from mx_plan.cpp; plain functions so that file needs no HIP syntax)
+namespace mx {
+
+hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
+{
+    if (A.nBlocks <= 0) return hipSuccess;
+    if (dtype == MX_F64)
+        hipLaunchKernelGGL(mxk::csr_rows_kernel<double>, dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr, A.col,
+                           (const double *)A.val, (const double *)x, (double *)y, A.blockRow, accumulate);
+    else
+        hipLaunchKernelGGL(mxk::csr_rows_kernel<_Float16>, dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr, A.col,
+                           (const _Float16 *)A.val, (const _Float16 *)x, (_Float16 *)y, A.blockRow, accumulate);
+    return hipGetLastError();
+}
+
+hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s)
+{
+    if (T.chunkNum <= 0) return hipSuccess;
+    const int grid = (T.chunkNum + 3) / 4;
+    if (dtype == MX_F64)
+        hipLaunchKernelGGL(mxk::tile_f64_kernel, dim3(grid), dim3(mxk::kBlock), 0, s, T.chunkPtr, T.fragPtr,
+                           (const uint32_t *)T.fragBit, (const double *)T.tcVal, T.atox, T.rowIdx, (const double *)x,
+                           (double *)y, T.chunkNum, T.dRows, accumulate);
+    else
+        hipLaunchKernelGGL(mxk::tile_f16_kernel, dim3(grid), dim3(mxk::kBlock), 0, s, T.chunkPtr, T.fragPtr,
+                           (const uint64_t *)T.fragBit, (const _Float16 *)T.tcVal, T.atox, T.rowIdx, (const _Float16 *)x,
+                           (_Float16 *)y, T.chunkNum, T.dRows, accumulate);
+    return hipGetLastError();
+}
+
+hipError_t launch_probe_f64(const double *A, const double *B, double *D, hipStream_t s)
+{
+    hipLaunchKernelGGL(mxk::probe_mfma_f64_kernel, dim3(1), dim3(64), 0, s, A, B, D);
+    return hipGetLastError();
+}
+hipError_t launch_probe_f16(const void *A, const void *B, float *D, hipStream_t s)
+{
+    hipLaunchKernelGGL(mxk::probe_mfma_f16_kernel, dim3(1), dim3(64), 0, s, (const _Float16 *)A, (const _Float16 *)B, D);
+    return hipGetLastError();
+}
+
+}  // namespace mx

@@ -1,0 +1,628 @@
+// Device plans: persistent device copies of a partition and the launch sequence of one
+// hybrid SpMV; plus the reference's one-shot host-pointer entry points built on top.
+#include <algorithm>
+#include <chrono>
+#include <cstring>
+#include <numeric>
+#include <vector>
+
+#include "mx_device.h"
+#include "mx_internal.h"
+
+namespace {
+
+using mx::set_error;
+
+#define MX_HIP(call)                                                                                  \
+    do {                                                                                              \
+        hipError_t e_ = (call);                                                                       \
+        if (e_ != hipSuccess) {                                                                       \
+            set_error(std::string(#call) + ": " + hipGetErrorString(e_));                             \
+            return MX_ERR_DEVICE;                                                                     \
+        }                                                                                             \
+    } while (0)
+
+int need_device()
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        set_error("no HIP device available (this library has no CPU fallback)");
+        return MX_ERR_DEVICE;
+    }
+    return MX_OK;
+}
+
+template <typename T>
+int upload(T **dst, const T *src, size_t n, size_t pad = 0)
+{
+    *dst = nullptr;
+    const size_t total = std::max<size_t>(n + pad, 1);
+    MX_HIP(hipMalloc((void **)dst, total * sizeof(T)));
+    if (pad || n == 0) MX_HIP(hipMemset(*dst, 0, total * sizeof(T)));
+    if (n) MX_HIP(hipMemcpy(*dst, src, n * sizeof(T), hipMemcpyHostToDevice));
+    return MX_OK;
+}
+
+int upload_bytes(void **dst, const void *src, size_t n, size_t pad = 0)
+{
+    return upload<unsigned char>((unsigned char **)dst, (const unsigned char *)src, n, pad);
+}
+
+// Rows of each CSR-kernel workgroup (the role of pre_startRowPerBlock,
+// src/spmv_kernel/cdSpMV.cu:4-27, but row-aligned): greedily pack whole rows while their
+// entries, counted from the tile's aligned start, fit one tile; a longer row stands alone.
+void pack_rows(const int *rowPtr, int rows, int npt, std::vector<int> &blockRow)
+{
+    const int tile = 256 * npt;
+    blockRow.clear();
+    blockRow.push_back(0);
+    int r = 0;
+    while (r < rows) {
+        const int base = rowPtr[r] & ~(npt - 1);
+        int r1 = r + 1;
+        while (r1 < rows && rowPtr[r1 + 1] - base <= tile && r1 - r < tile) ++r1;
+        blockRow.push_back(r1);
+        r = r1;
+    }
+}
+
+void free_csr(mx::DeviceCsr &A)
+{
+    (void)hipFree(A.rowPtr);
+    (void)hipFree(A.col);
+    (void)hipFree(A.val);
+    (void)hipFree(A.blockRow);
+    A = mx::DeviceCsr();
+}
+
+void free_tiles(mx::DeviceTiles &T)
+{
+    (void)hipFree(T.chunkPtr);
+    (void)hipFree(T.fragPtr);
+    (void)hipFree(T.fragBit);
+    (void)hipFree(T.tcVal);
+    (void)hipFree(T.atox);
+    (void)hipFree(T.rowIdx);
+    T = mx::DeviceTiles();
+}
+
+int upload_csr(mx_dtype dtype, int rows, int nnz, const int *rowPtr, const int *col, const void *val,
+               mx::DeviceCsr &A, double *pack_ms)
+{
+    const int es = mx::elem_size(dtype), npt = dtype == MX_F64 ? 4 : 8;
+    A.rows = rows;
+    A.nnz = nnz;
+    int rc;
+    if ((rc = upload(&A.rowPtr, rowPtr, (size_t)rows + 1))) return rc;
+    if ((rc = upload(&A.col, col, (size_t)nnz, mx::kCsrPad))) return rc;
+    if ((rc = upload_bytes(&A.val, val, (size_t)nnz * es, (size_t)mx::kCsrPad * es))) return rc;
+    std::vector<int> blockRow;
+    auto t0 = std::chrono::steady_clock::now();
+    pack_rows(rowPtr, rows, npt, blockRow);
+    auto t1 = std::chrono::steady_clock::now();
+    if (pack_ms) *pack_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    A.nBlocks = (int)blockRow.size() - 1;
+    if ((rc = upload(&A.blockRow, blockRow.data(), blockRow.size()))) return rc;
+    return MX_OK;
+}
+
+}  // namespace
+
+struct mx_plan {
+    mx_dtype dtype = MX_F64;
+    int rows = 0, cols = 0, nnz = 0;
+    mx::DeviceCsr csr;
+    mx::DeviceTiles tiles;
+    int tile_nnz = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+};
+
+extern "C" int mx_device_count(void)
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+extern "C" void mx_plan_destroy(mx_plan *plan)
+{
+    if (!plan) return;
+    free_csr(plan->csr);
+    free_tiles(plan->tiles);
+    if (plan->ev0) (void)hipEventDestroy(plan->ev0);
+    if (plan->ev1) (void)hipEventDestroy(plan->ev1);
+    if (plan->stream) (void)hipStreamDestroy(plan->stream);
+    delete plan;
+}
+
+// Minimum fill of a chunk's fragments for the MFMA tile kernel to take it (default plans).
+// Below it the chunk's entries cost fewer bytes as CSR: a fragment costs 8 bytes of bitmap and
+// pointer plus fragK indices, an entry in CSR costs 4 bytes of index.
+static double tile_gate(mx_dtype dtype) { return dtype == MX_F64 ? 0.25 : 0.20; }
+
+extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
+{
+    if (!P || !out) {
+        set_error("mx_plan_create: null argument");
+        return MX_ERR_ARG;
+    }
+    *out = nullptr;
+    int rc = need_device();
+    if (rc) return rc;
+    mx_plan *plan = new (std::nothrow) mx_plan();
+    if (!plan) {
+        set_error("mx_plan_create: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    plan->dtype = P->dtype;
+    plan->rows = P->rows;
+    plan->cols = P->cols;
+    plan->nnz = P->nnz;
+    const int es = mx::elem_size(P->dtype), fragK = P->fragK, fragM = P->fragM;
+    const int rows = P->rows, cols = P->cols;
+    auto fail = [&](int code) {
+        mx_plan_destroy(plan);
+        return code;
+    };
+    try {
+        if (!P->extracted) {
+            rc = upload_csr(P->dtype, rows, P->nnzCD, P->cdRowPtr.data(), P->cdColInd.data(), P->cdVal.data(), plan->csr,
+                            nullptr);
+            if (rc) return fail(rc);
+        } else {
+            // residual column space -> the caller's column ids, so x needs no permutation
+            std::vector<int> colOrig(cols);
+            for (int c = 0; c < P->dCols; ++c) colOrig[c] = P->descColId[c];
+            for (int c = P->dCols; c < cols; ++c) colOrig[c] = P->newArray[c - P->dCols];
+            // which chunks go to the tile kernel
+            const int chunkNum = P->chunkNum;
+            std::vector<char> sel(chunkNum, 0);
+            const double gate = tile_gate(P->dtype);
+            for (int w = 0; w < chunkNum; ++w) {
+                const int nf = P->chunkPtr[w + 1] - P->chunkPtr[w];
+                if (nf == 0) continue;
+                const int vals = P->fragPtr[P->chunkPtr[w + 1]] - P->fragPtr[P->chunkPtr[w]];
+                const double fill = (double)vals / ((double)nf * fragM * fragK);
+                if (flags & MX_PLAN_NO_TILES) sel[w] = 0;
+                else if (flags & MX_PLAN_ALL_TILES) sel[w] = 1;
+                else sel[w] = fill >= gate;
+            }
+            // CSR part = residual rows (+ the A_dd rows of chunks left out of the tile kernel)
+            std::vector<int> rowPtr((size_t)rows + 1, 0);
+            for (int r = 0; r < rows; ++r) rowPtr[r + 1] = P->cdRowPtr[r + 1] - P->cdRowPtr[r];
+            for (int i = 0; i < P->dRows; ++i)
+                if (!sel[i / fragM]) rowPtr[P->rId[i] + 1] += P->ddRowPtr[i + 1] - P->ddRowPtr[i];
+            for (int r = 0; r < rows; ++r) rowPtr[r + 1] += rowPtr[r];
+            const int csrNnz = rowPtr[rows];
+            std::vector<int> col((size_t)csrNnz);
+            std::vector<unsigned char> val((size_t)csrNnz * es);
+            const unsigned char *cdv = (const unsigned char *)P->cdVal.data();
+            const unsigned char *ddv = (const unsigned char *)P->ddVal.data();
+#pragma omp parallel for schedule(static)
+            for (int r = 0; r < rows; ++r) {
+                int q = rowPtr[r];
+                for (int p = P->cdRowPtr[r]; p < P->cdRowPtr[r + 1]; ++p, ++q) {
+                    col[q] = colOrig[P->cdColInd[p]];
+                    std::memcpy(&val[(size_t)q * es], cdv + (size_t)p * es, es);
+                }
+            }
+#pragma omp parallel for schedule(static)
+            for (int i = 0; i < P->dRows; ++i) {
+                if (sel[i / fragM]) continue;
+                const int r = P->rId[i];
+                int q = rowPtr[r] + (P->cdRowPtr[r + 1] - P->cdRowPtr[r]);
+                for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p, ++q) {
+                    col[q] = P->descColId[P->ddColInd[p]];
+                    std::memcpy(&val[(size_t)q * es], ddv + (size_t)p * es, es);
+                }
+            }
+            rc = upload_csr(P->dtype, rows, csrNnz, rowPtr.data(), col.data(), val.data(), plan->csr, nullptr);
+            if (rc) return fail(rc);
+
+            // tile part: the selected chunks, re-packed contiguously
+            int nsel = 0;
+            for (int w = 0; w < chunkNum; ++w) nsel += sel[w];
+            if (nsel > 0) {
+                std::vector<int> chunkPtr(1, 0), fragPtr(1, 0), atox, rowIdx;
+                std::vector<unsigned char> fragBit, tcVal;
+                const int bitBytes = P->dtype == MX_F64 ? 4 : 8;
+                const unsigned char *bits = P->dtype == MX_F64 ? (const unsigned char *)P->fragBit32.data()
+                                                               : (const unsigned char *)P->fragBit64.data();
+                const unsigned char *tv = (const unsigned char *)P->tcVal.data();
+                for (int w = 0; w < chunkNum; ++w) {
+                    if (!sel[w]) continue;
+                    const int f0 = P->chunkPtr[w], f1 = P->chunkPtr[w + 1];
+                    for (int f = f0; f < f1; ++f) {
+                        fragPtr.push_back(fragPtr.back() + (P->fragPtr[f + 1] - P->fragPtr[f]));
+                        for (int k = 0; k < fragK; ++k)
+                            atox.push_back(P->descColId[P->sparse_AToX_index[(size_t)f * fragK + k]]);
+                    }
+                    fragBit.insert(fragBit.end(), bits + (size_t)f0 * bitBytes, bits + (size_t)f1 * bitBytes);
+                    tcVal.insert(tcVal.end(), tv + (size_t)P->fragPtr[f0] * es, tv + (size_t)P->fragPtr[f1] * es);
+                    chunkPtr.push_back(chunkPtr.back() + (f1 - f0));
+                    for (int i = 0; i < fragM; ++i) {
+                        const int local = w * fragM + i;
+                        rowIdx.push_back(local < P->dRows ? P->rId[local] : -1);
+                    }
+                }
+                mx::DeviceTiles &T = plan->tiles;
+                T.chunkNum = nsel;
+                T.frags = chunkPtr.back();
+                T.vals = fragPtr.back();
+                // ragged last chunk: rows past dRows carry -1 and are skipped through dRows
+                T.dRows = nsel * fragM;
+                while (T.dRows > 0 && rowIdx[T.dRows - 1] < 0) --T.dRows;
+                plan->tile_nnz = T.vals;
+                if ((rc = upload(&T.chunkPtr, chunkPtr.data(), chunkPtr.size()))) return fail(rc);
+                if ((rc = upload(&T.fragPtr, fragPtr.data(), fragPtr.size()))) return fail(rc);
+                if ((rc = upload_bytes(&T.fragBit, fragBit.data(), fragBit.size()))) return fail(rc);
+                if ((rc = upload_bytes(&T.tcVal, tcVal.data(), tcVal.size(), 64))) return fail(rc);
+                if ((rc = upload(&T.atox, atox.data(), atox.size(), 16))) return fail(rc);
+                if ((rc = upload(&T.rowIdx, rowIdx.data(), rowIdx.size()))) return fail(rc);
+            }
+        }
+    } catch (const std::bad_alloc &) {
+        set_error("mx_plan_create: out of memory");
+        return fail(MX_ERR_ALLOC);
+    }
+    if (hipStreamCreate(&plan->stream) != hipSuccess || hipEventCreate(&plan->ev0) != hipSuccess ||
+        hipEventCreate(&plan->ev1) != hipSuccess) {
+        set_error("mx_plan_create: could not create stream/events");
+        return fail(MX_ERR_DEVICE);
+    }
+    *out = plan;
+    return MX_OK;
+}
+
+extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
+{
+    if (!plan || !info) {
+        set_error("mx_plan_get_info: null argument");
+        return MX_ERR_ARG;
+    }
+    const double es = mx::elem_size(plan->dtype);
+    const int fragK = mx::frag_k(plan->dtype);
+    const double bitBytes = plan->dtype == MX_F64 ? 4 : 8;
+    info->dtype = plan->dtype;
+    info->rows = plan->rows;
+    info->cols = plan->cols;
+    info->nnz = plan->nnz;
+    info->tile_chunks = plan->tiles.chunkNum;
+    info->tile_frags = plan->tiles.frags;
+    info->tile_nnz = plan->tile_nnz;
+    info->csr_nnz = plan->csr.nnz;
+    info->csr_blocks = plan->csr.nBlocks;
+    // what each kernel has to move at least once: its arrays, x once, its y rows
+    info->csr_bytes = (double)plan->csr.nnz * (es + 4) + ((double)plan->rows + 1) * 4 + (double)plan->cols * es +
+                      (double)plan->rows * es;
+    info->tile_bytes = plan->tiles.chunkNum
+                           ? (double)plan->tiles.frags * (bitBytes + 4 + 4.0 * fragK) + (double)plan->tiles.vals * es +
+                                 ((double)plan->tiles.chunkNum + 1) * 4 + (double)plan->tiles.dRows * (4 + 2 * es)
+                           : 0.0;
+    return MX_OK;
+}
+
+static int spmv_on(mx_plan *plan, const void *x, void *y, hipStream_t s)
+{
+    MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, 0, s));
+    MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x, y, 1, s));
+    return MX_OK;
+}
+
+extern "C" int mx_spmv(mx_plan *plan, const void *x_dev, void *y_dev, void *stream)
+{
+    if (!plan || !x_dev || !y_dev) {
+        set_error("mx_spmv: null argument");
+        return MX_ERR_ARG;
+    }
+    return spmv_on(plan, x_dev, y_dev, (hipStream_t)stream);
+}
+
+extern "C" int mx_spmv_host(mx_plan *plan, const void *x_host, void *y_host)
+{
+    if (!plan || !x_host || !y_host) {
+        set_error("mx_spmv_host: null argument");
+        return MX_ERR_ARG;
+    }
+    const size_t es = (size_t)mx::elem_size(plan->dtype);
+    void *dx = nullptr, *dy = nullptr;
+    MX_HIP(hipMalloc(&dx, std::max<size_t>(plan->cols * es, 1)));
+    if (hipMalloc(&dy, std::max<size_t>(plan->rows * es, 1)) != hipSuccess) {
+        (void)hipFree(dx);
+        set_error("mx_spmv_host: hipMalloc failed");
+        return MX_ERR_DEVICE;
+    }
+    int rc = MX_OK;
+    auto body = [&]() -> int {
+        MX_HIP(hipMemcpyAsync(dx, x_host, plan->cols * es, hipMemcpyHostToDevice, plan->stream));
+        int r = spmv_on(plan, dx, dy, plan->stream);
+        if (r) return r;
+        MX_HIP(hipMemcpyAsync(y_host, dy, plan->rows * es, hipMemcpyDeviceToHost, plan->stream));
+        MX_HIP(hipStreamSynchronize(plan->stream));
+        return MX_OK;
+    };
+    rc = body();
+    (void)hipFree(dx);
+    (void)hipFree(dy);
+    return rc;
+}
+
+// Mean milliseconds per iteration of `body` over `iters` back-to-back runs after `warm`
+// untimed ones, by events on the stream the kernels run on.
+template <typename F>
+static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
+{
+    for (int i = 0; i < warm; ++i) {
+        int rc = body();
+        if (rc) return rc;
+    }
+    MX_HIP(hipStreamSynchronize(plan->stream));
+    MX_HIP(hipEventRecord(plan->ev0, plan->stream));
+    for (int i = 0; i < iters; ++i) {
+        int rc = body();
+        if (rc) return rc;
+    }
+    MX_HIP(hipEventRecord(plan->ev1, plan->stream));
+    MX_HIP(hipEventSynchronize(plan->ev1));
+    float t = 0.f;
+    MX_HIP(hipEventElapsedTime(&t, plan->ev0, plan->ev1));
+    *ms = (double)t / (double)std::max(iters, 1);
+    return MX_OK;
+}
+
+extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters, double *ms_total,
+                       double *ms_tile, double *ms_csr)
+{
+    if (!plan || !x_dev || !y_dev || warm < 0 || iters <= 0) {
+        set_error("mx_time: bad argument");
+        return MX_ERR_ARG;
+    }
+    hipStream_t s = plan->stream;
+    int rc;
+    double t = 0.0;
+    if (ms_total) {
+        rc = time_loop(plan, warm, iters, [&]() { return spmv_on(plan, x_dev, y_dev, s); }, &t);
+        if (rc) return rc;
+        *ms_total = t;
+    }
+    if (ms_csr) {
+        rc = time_loop(plan, warm, iters, [&]() -> int {
+            MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x_dev, y_dev, 0, s));
+            return MX_OK;
+        }, &t);
+        if (rc) return rc;
+        *ms_csr = t;
+    }
+    if (ms_tile) {
+        *ms_tile = 0.0;
+        if (plan->tiles.chunkNum > 0) {
+            // overwrite mode: the timed loop must not grow y without bound
+            rc = time_loop(plan, warm, iters, [&]() -> int {
+                MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x_dev, y_dev, 0, s));
+                return MX_OK;
+            }, &t);
+            if (rc) return rc;
+            *ms_tile = t;
+        }
+    }
+    // leave y holding the product
+    rc = spmv_on(plan, x_dev, y_dev, s);
+    if (rc) return rc;
+    MX_HIP(hipStreamSynchronize(s));
+    return MX_OK;
+}
+
+// ---- reference surface: host pointers in, host pointers out ------------------------------
+
+static int cdspmv_any(mx_dtype dtype, const void *csrVal, const int *csrRowPtr, const int *csrColInd, const void *x,
+                      void *y, int rows, int cols, int nnz, int warm, int iters, double *cdTime, double *cdPre)
+{
+    if (!csrRowPtr || !x || !y || rows < 0 || cols < 0 || nnz < 0 || (nnz > 0 && (!csrVal || !csrColInd))) {
+        set_error("cdspmv: bad argument");
+        return MX_ERR_ARG;
+    }
+    int rc = need_device();
+    if (rc) return rc;
+    for (int p = 0; p < nnz; ++p)
+        if ((unsigned)csrColInd[p] >= (unsigned)cols) {
+            set_error("cdspmv: column index out of range");
+            return MX_ERR_ARG;
+        }
+    if (csrRowPtr[0] != 0 || csrRowPtr[rows] != nnz) {
+        set_error("cdspmv: rowPtr does not span [0, nnz]");
+        return MX_ERR_ARG;
+    }
+    mx_plan plan;
+    plan.dtype = dtype;
+    plan.rows = rows;
+    plan.cols = cols;
+    plan.nnz = nnz;
+    const size_t es = (size_t)mx::elem_size(dtype);
+    void *dx = nullptr, *dy = nullptr, *dscratch = nullptr;
+    auto body = [&]() -> int {
+        double pre = 0.0;
+        int r = upload_csr(dtype, rows, nnz, csrRowPtr, csrColInd, csrVal, plan.csr, &pre);
+        if (r) return r;
+        if (cdPre) *cdPre = pre;
+        if ((r = upload_bytes(&dx, x, cols * es))) return r;
+        if ((r = upload_bytes(&dy, y, rows * es))) return r;
+        if ((r = upload_bytes(&dscratch, nullptr, 0, rows * es))) return r;
+        MX_HIP(hipStreamCreate(&plan.stream));
+        MX_HIP(hipEventCreate(&plan.ev0));
+        MX_HIP(hipEventCreate(&plan.ev1));
+        double ms = 0.0;
+        if (iters > 0) {
+            r = time_loop(&plan, warm, iters, [&]() -> int {
+                MX_HIP(mx::launch_csr(dtype, plan.csr, dx, dscratch, 0, plan.stream));
+                return MX_OK;
+            }, &ms);
+            if (r) return r;
+        }
+        if (cdTime) *cdTime = ms;
+        MX_HIP(mx::launch_csr(dtype, plan.csr, dx, dy, 1, plan.stream));  // y += A*x
+        MX_HIP(hipStreamSynchronize(plan.stream));
+        MX_HIP(hipMemcpy(y, dy, rows * es, hipMemcpyDeviceToHost));
+        return MX_OK;
+    };
+    rc = body();
+    free_csr(plan.csr);
+    (void)hipFree(dx);
+    (void)hipFree(dy);
+    (void)hipFree(dscratch);
+    if (plan.ev0) (void)hipEventDestroy(plan.ev0);
+    if (plan.ev1) (void)hipEventDestroy(plan.ev1);
+    if (plan.stream) (void)hipStreamDestroy(plan.stream);
+    return rc;
+}
+
+extern "C" int mx_cdspmv_f64(const double *csrVal, const int *csrRowPtr, const int *csrColInd, const double *x, double *y,
+                             int rows, int cols, int nnz, int warm, int iters, double *cdTime, double *cdPre)
+{
+    return cdspmv_any(MX_F64, csrVal, csrRowPtr, csrColInd, x, y, rows, cols, nnz, warm, iters, cdTime, cdPre);
+}
+
+extern "C" int mx_cdspmv_f16(const uint16_t *csrVal, const int *csrRowPtr, const int *csrColInd, const uint16_t *x,
+                             uint16_t *y, int rows, int cols, int nnz, int warm, int iters, double *cdTime, double *cdPre)
+{
+    return cdspmv_any(MX_F16, csrVal, csrRowPtr, csrColInd, x, y, rows, cols, nnz, warm, iters, cdTime, cdPre);
+}
+
+static int du_any(mx_dtype dtype, const int *chunkPtr, const int *fragPtr, const void *fragBit, const void *tcVal,
+                  const int *atox, const void *x_d, void *y_d, int dRows, int dCols, int warm, int iters, double *tcTime)
+{
+    if (!chunkPtr || !fragPtr || !x_d || !y_d || dRows < 0 || dCols < 0) {
+        set_error("du_tcspmv: bad argument");
+        return MX_ERR_ARG;
+    }
+    int rc = need_device();
+    if (rc) return rc;
+    const int fragK = mx::frag_k(dtype), fragM = mx::kFragM;
+    const size_t es = (size_t)mx::elem_size(dtype), bitBytes = dtype == MX_F64 ? 4 : 8;
+    const int chunkNum = (dRows + fragM - 1) / fragM;
+    const int frags = chunkPtr[chunkNum];
+    const int vals = fragPtr[frags];
+    if (frags > 0 && (!fragBit || !atox || (vals > 0 && !tcVal))) {
+        set_error("du_tcspmv: missing tile arrays");
+        return MX_ERR_ARG;
+    }
+    for (size_t i = 0; i < (size_t)frags * fragK; ++i)
+        if ((unsigned)atox[i] >= (unsigned)std::max(dCols, 1)) {
+            set_error("du_tcspmv: sparse_AToX_index out of range");
+            return MX_ERR_ARG;
+        }
+    mx_plan plan;
+    plan.dtype = dtype;
+    mx::DeviceTiles &T = plan.tiles;
+    void *dx = nullptr, *dy = nullptr, *dscratch = nullptr;
+    auto body = [&]() -> int {
+        int r;
+        T.chunkNum = chunkNum;
+        T.dRows = dRows;
+        T.frags = frags;
+        T.vals = vals;
+        if ((r = upload(&T.chunkPtr, chunkPtr, (size_t)chunkNum + 1))) return r;
+        if ((r = upload(&T.fragPtr, fragPtr, (size_t)frags + 1))) return r;
+        if ((r = upload_bytes(&T.fragBit, fragBit, frags * bitBytes))) return r;
+        if ((r = upload_bytes(&T.tcVal, tcVal, vals * es, 64))) return r;
+        if ((r = upload(&T.atox, atox, (size_t)frags * fragK, 16))) return r;
+        if ((r = upload_bytes(&dx, x_d, dCols * es))) return r;
+        // FP64 uploads the caller's y and adds to it; FP16 starts from zero
+        // (du_tcSpMV_fp64.cu:296-297 vs du_tcSpMV_fp16_v2.cu:146-147)
+        if (dtype == MX_F64) {
+            if ((r = upload_bytes(&dy, y_d, dRows * es))) return r;
+        } else {
+            if ((r = upload_bytes(&dy, nullptr, 0, dRows * es))) return r;
+        }
+        if ((r = upload_bytes(&dscratch, nullptr, 0, dRows * es))) return r;
+        MX_HIP(hipStreamCreate(&plan.stream));
+        MX_HIP(hipEventCreate(&plan.ev0));
+        MX_HIP(hipEventCreate(&plan.ev1));
+        double ms = 0.0;
+        if (iters > 0 && chunkNum > 0) {
+            r = time_loop(&plan, warm, iters, [&]() -> int {
+                MX_HIP(mx::launch_tiles(dtype, T, dx, dscratch, 0, plan.stream));
+                return MX_OK;
+            }, &ms);
+            if (r) return r;
+        }
+        if (tcTime) *tcTime = ms;
+        MX_HIP(mx::launch_tiles(dtype, T, dx, dy, dtype == MX_F64 ? 1 : 0, plan.stream));
+        MX_HIP(hipStreamSynchronize(plan.stream));
+        MX_HIP(hipMemcpy(y_d, dy, dRows * es, hipMemcpyDeviceToHost));
+        return MX_OK;
+    };
+    rc = body();
+    free_tiles(T);
+    (void)hipFree(dx);
+    (void)hipFree(dy);
+    (void)hipFree(dscratch);
+    if (plan.ev0) (void)hipEventDestroy(plan.ev0);
+    if (plan.ev1) (void)hipEventDestroy(plan.ev1);
+    if (plan.stream) (void)hipStreamDestroy(plan.stream);
+    return rc;
+}
+
+extern "C" int mx_du_tcspmv_f64(const int *chunkPtr, const int *fragPtr, const uint32_t *fragBit, const double *tcVal,
+                                const int *sparse_AToX_index, const double *x_d, double *y_d, int dRows, int dCols,
+                                int warm, int iters, double *tcTime)
+{
+    return du_any(MX_F64, chunkPtr, fragPtr, fragBit, tcVal, sparse_AToX_index, x_d, y_d, dRows, dCols, warm, iters, tcTime);
+}
+
+extern "C" int mx_du_tcspmv_f16(const int *chunkPtr, const int *fragPtr, const uint64_t *fragBit, const uint16_t *tcVal,
+                                const int *sparse_AToX_index, const uint16_t *x_d, uint16_t *y_d, int dRows, int dCols,
+                                int warm, int iters, double *tcTime)
+{
+    return du_any(MX_F16, chunkPtr, fragPtr, fragBit, tcVal, sparse_AToX_index, x_d, y_d, dRows, dCols, warm, iters, tcTime);
+}
+
+// MFMA layout probes (used by the GPU tests): D(16x16) = A*B on one wave.
+extern "C" int mx_probe_mfma_f64(const double *A, const double *B, double *D)
+{
+    int rc = need_device();
+    if (rc) return rc;
+    double *dA = nullptr, *dB = nullptr, *dD = nullptr;
+    auto body = [&]() -> int {
+        int r;
+        if ((r = upload(&dA, A, 64))) return r;
+        if ((r = upload(&dB, B, 64))) return r;
+        if ((r = upload<double>(&dD, nullptr, 0, 256))) return r;
+        MX_HIP(mx::launch_probe_f64(dA, dB, dD, nullptr));
+        MX_HIP(hipDeviceSynchronize());
+        MX_HIP(hipMemcpy(D, dD, 256 * sizeof(double), hipMemcpyDeviceToHost));
+        return MX_OK;
+    };
+    rc = body();
+    (void)hipFree(dA);
+    (void)hipFree(dB);
+    (void)hipFree(dD);
+    return rc;
+}
+
+extern "C" int mx_probe_mfma_f16(const uint16_t *A, const uint16_t *B, float *D)
+{
+    int rc = need_device();
+    if (rc) return rc;
+    uint16_t *dA = nullptr, *dB = nullptr;
+    float *dD = nullptr;
+    auto body = [&]() -> int {
+        int r;
+        if ((r = upload(&dA, A, 512))) return r;
+        if ((r = upload(&dB, B, 512))) return r;
+        if ((r = upload<float>(&dD, nullptr, 0, 256))) return r;
+        MX_HIP(mx::launch_probe_f16(dA, dB, dD, nullptr));
+        MX_HIP(hipDeviceSynchronize());
+        MX_HIP(hipMemcpy(D, dD, 256 * sizeof(float), hipMemcpyDeviceToHost));
+        return MX_OK;
+    };
+    rc = body();
+    (void)hipFree(dA);
+    (void)hipFree(dB);
+    (void)hipFree(dD);
+    return rc;
+}
