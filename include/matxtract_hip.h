@@ -108,7 +108,7 @@ int mx_transpose(mx_dtype dtype, int outer, int inner, int nnz, const int *ptr, 
 void mx_free(void *p);
 
 /* mmio_allinone (utilities/mmio.cpp:1547-1713): Matrix-Market coordinate file -> CSR with
- * entries kept in file order inside each row, symmetric/hermitian/skew files expanded,
+ * entries kept in file order inside each row, symmetric/hermitian files expanded,
  * pattern files given value 1.  Outputs malloc()ed; returns MX_ERR_IO on failure. */
 int mx_mmio_read(const char *path, mx_dtype dtype, int *rows, int *cols, int *nnz, int *isSymmetric,
                  int **rowPtr, int **colInd, void **val);
@@ -205,10 +205,11 @@ int mx_du_tcspmv_f16(const int *chunkPtr, const int *fragPtr, const uint64_t *fr
 /* Number of HIP devices visible (0 when none; never fails). */
 int mx_device_count(void);
 
-/* Diagnostics: D(16x16) = A*B on one wave through the MFMA instruction the tile kernels use,
- * operands moved with the lane mapping those kernels assume (A 16x4, B 4x16 binary64;
- * A 16x32, B 32x16 binary16 with a binary32 result), all row-major HOST arrays.  No
- * counterpart in the reference; the test-suite uses them to pin the operand layout. */
+/* Diagnostics: one MFMA on one wave with raw per-lane operands, so a test can pin the
+ * operand layout the tile kernels assume.  f64 (v_mfma_f64_16x16x4_f64): A[64], B[64] one
+ * value per lane, D[64][4] the four accumulator registers of each lane.  f16
+ * (v_mfma_f32_16x16x32_f16): A[64][8], B[64][8] binary16, D[64][4] binary32.  HOST arrays.
+ * No counterpart in the reference. */
 int mx_probe_mfma_f64(const double *A, const double *B, double *D);
 int mx_probe_mfma_f16(const uint16_t *A, const uint16_t *B, float *D);
 

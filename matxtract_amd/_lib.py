@@ -95,6 +95,13 @@ def load():
         if not os.path.exists(LIB_PATH):
             raise ImportError(
                 "%s not found: build it with `make -C %s` (or __graft_entry__.build())" % (LIB_PATH, CSRC))
+        # PyTorch ships its own copy of the HIP runtime under the same soname; whichever copy
+        # is loaded first serves the whole process.  Import torch first so that device memory
+        # and streams handed over by torch belong to the runtime this library talks to.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)

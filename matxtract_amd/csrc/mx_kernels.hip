@@ -190,12 +190,12 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
 // ---- tile part --------------------------------------------------------------------------
 // One wave per 8-row chunk, 4 chunks per workgroup.
 //
-// v_mfma_f64_16x16x4_f64 operand layout (wave64): lane L holds A[L%16][L/16], B[L/16][L%16] and
-// D[4*(L/16)+i][L%16] in accumulator register i.  A step feeds two fragments: A rows 0..7 =
-// fragment f, rows 8..15 = fragment f+1; B column 0 = the 4 gathered x of fragment f, column
-// 1 = those of fragment f+1, other columns 0.  The chunk's result is D[0..7][0] + D[8..15][1],
-// accumulated across all steps inside the matrix core, so no cross-lane reduction is needed
-// until the single combine at the end.
+// v_mfma_f64_16x16x4_f64 operand layout (wave64): lane L holds A[L%16][L/16] and
+// B[L/16][L%16]; accumulator register g of lane L holds D[4*g + L/16][L%16].  A step feeds two
+// fragments: A rows 0..7 = fragment f, rows 8..15 = fragment f+1; B column 0 = the 4 gathered
+// x of fragment f, column 1 = those of fragment f+1, other columns 0.  The chunk's result is
+// D[0..7][0] + D[8..15][1], accumulated across all steps inside the matrix core, so no
+// cross-lane reduction is needed until the single combine at the end.
 __global__ __launch_bounds__(kBlock) void tile_f64_kernel(const int *__restrict__ chunkPtr, const int *__restrict__ fragPtr,
                                                          const uint32_t *__restrict__ fragBit,
                                                          const double *__restrict__ tcVal, const int *__restrict__ atox,
@@ -221,24 +221,26 @@ __global__ __launch_bounds__(kBlock) void tile_f64_kernel(const int *__restrict_
         if (m < 2 && f + m < f1) bv = x[atox[(f + m) * 4 + k]];
         acc = __builtin_amdgcn_mfma_f64_16x16x4f64(a, bv, acc, 0, 0, 0);
     }
-    // rows 0..3: lane 0 (+ lane 33), rows 4..7: lane 16 (+ lane 49)
-    double o[4];
+    // row q and row q+4 of the chunk end up in lane 16q: D[q][0] = reg 0, D[q+4][0] = reg 1 there,
+    // D[8+q][1] = reg 2 and D[12+q][1] = reg 3 of lane 16q+1.
+    const double o0 = acc[0] + __shfl_down(acc[2], 1, 64);
+    const double o1 = acc[1] + __shfl_down(acc[3], 1, 64);
+    if ((lane & 15) == 0) {
+        const int q = lane >> 4;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = acc[i] + __shfl(acc[i], lane + 33, 64);
-    if (lane == 0 || lane == 16) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int local = w * 8 + (lane >> 2) + i;  // lane 16 -> +4
+        for (int h = 0; h < 2; ++h) {
+            const int local = w * 8 + q + 4 * h;
             if (local < dRows) {
                 const int row = rowIdx ? rowIdx[local] : local;
-                y[row] = accumulate ? y[row] + o[i] : o[i];
+                const double o = h ? o1 : o0;
+                y[row] = accumulate ? y[row] + o : o;
             }
         }
     }
 }
 
 // v_mfma_f32_16x16x32_f16 operand layout (wave64): lane L holds A[L%16][8*(L/16) .. +7],
-// B[8*(L/16) .. +7][L%16] and D[4*(L/16)+i][L%16].  A step feeds eight 8x8 fragments of the
+// B[8*(L/16) .. +7][L%16]; accumulator register g of lane L holds D[4*(L/16)+g][L%16].  A step feeds eight 8x8 fragments of the
 // chunk: A rows 0..7 = fragments f..f+3 side by side along K, rows 8..15 = fragments f+4..f+7;
 // B column 0 = the 32 gathered x of f..f+3, column 1 = those of f+4..f+7.  A lane's eight A
 // elements are one byte of its fragment's 64-bit bitmap (one tile row), whose values sit
@@ -296,26 +298,26 @@ __global__ __launch_bounds__(kBlock) void tile_f16_kernel(const int *__restrict_
     }
 }
 
-// MFMA operand-layout probes: D = A*B for one wave, operands and result in row-major
-// global memory, loaded/stored with exactly the lane mapping the tile kernels assume.
-__global__ void probe_mfma_f64_kernel(const double *A /*16x4*/, const double *B /*4x16*/, double *D /*16x16*/)
+// MFMA probes: one wave, operands and accumulators exchanged lane by lane (raw register
+// contents), so a host test can check the operand layout the tile kernels rely on.
+__global__ void probe_mfma_f64_kernel(const double *A /*[64]*/, const double *B /*[64]*/, double *D /*[64][4]*/)
 {
     const int lane = threadIdx.x & 63;
     v4f64 acc = {0.0, 0.0, 0.0, 0.0};
-    acc = __builtin_amdgcn_mfma_f64_16x16x4f64(A[(lane & 15) * 4 + (lane >> 4)], B[(lane >> 4) * 16 + (lane & 15)], acc, 0, 0, 0);
-    for (int i = 0; i < 4; ++i) D[(4 * (lane >> 4) + i) * 16 + (lane & 15)] = acc[i];
+    acc = __builtin_amdgcn_mfma_f64_16x16x4f64(A[lane], B[lane], acc, 0, 0, 0);
+    for (int i = 0; i < 4; ++i) D[lane * 4 + i] = acc[i];
 }
-__global__ void probe_mfma_f16_kernel(const _Float16 *A /*16x32*/, const _Float16 *B /*32x16*/, float *D /*16x16*/)
+__global__ void probe_mfma_f16_kernel(const _Float16 *A /*[64][8]*/, const _Float16 *B /*[64][8]*/, float *D /*[64][4]*/)
 {
     const int lane = threadIdx.x & 63;
     v8f16 a, b;
     for (int j = 0; j < 8; ++j) {
-        a[j] = A[(lane & 15) * 32 + 8 * (lane >> 4) + j];
-        b[j] = B[(8 * (lane >> 4) + j) * 16 + (lane & 15)];
+        a[j] = A[lane * 8 + j];
+        b[j] = B[lane * 8 + j];
     }
     v4f32 acc = {0.f, 0.f, 0.f, 0.f};
     acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
-    for (int i = 0; i < 4; ++i) D[(4 * (lane >> 4) + i) * 16 + (lane & 15)] = acc[i];
+    for (int i = 0; i < 4; ++i) D[lane * 4 + i] = acc[i];
 }
 
 }  // namespace mxk

@@ -1,0 +1,31 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def mx():
+    """The product package; builds the library first if it is not there."""
+    from matxtract_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    import matxtract_amd
+    return matxtract_amd
+
+
+@pytest.fixture(scope="session")
+def ora():
+    """The CPU oracle (test infrastructure)."""
+    from oracle import mx_oracle
+    mx_oracle.build()
+    return mx_oracle
