@@ -153,7 +153,13 @@ void mx_plan_destroy(mx_plan *plan);
  * residual accumulated on top) without host round trips. */
 int mx_spmv(mx_plan *plan, const void *x_dev, void *y_dev, void *stream);
 
-/* Same with HOST pointers (allocates nothing persistent; copies x in and y out). */
+/* n back-to-back SpMVs y = A*x on `stream`, queued from C without returning to the caller in
+ * between: the reference's timed loops (src/spmv_kernel/cdSpMV.cu:464-469) as an entry point,
+ * for callers whose per-call overhead (an interpreter, an FFI hop) would otherwise sit
+ * between launches.  Asynchronous. */
+int mx_spmv_repeat(mx_plan *plan, const void *x_dev, void *y_dev, int n, void *stream);
+
+/* Same as mx_spmv with HOST pointers (allocates nothing persistent; copies x in and y out). */
 int mx_spmv_host(mx_plan *plan, const void *x_host, void *y_host);
 
 /* The reference's timing protocol (200 warm-ups + 4000 timed back-to-back launches,

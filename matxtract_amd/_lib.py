@@ -73,6 +73,7 @@ SIGNATURES = {
     "mx_plan_create": (_i, [_vp, _i, _pp]),
     "mx_plan_destroy": (None, [_vp]),
     "mx_spmv": (_i, [_vp, _vp, _vp, _vp]),
+    "mx_spmv_repeat": (_i, [_vp, _vp, _vp, _i, _vp]),
     "mx_spmv_host": (_i, [_vp, _vp, _vp]),
     "mx_time": (_i, [_vp, _vp, _vp, _i, _i, _pd, _pd, _pd]),
     "mx_plan_get_info": (_i, [_vp, C.POINTER(PlanInfo)]),

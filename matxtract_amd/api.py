@@ -200,6 +200,15 @@ class Plan:
         check(_lib.load().mx_spmv(self._h, x.data_ptr(), y.data_ptr(), s))
         return y
 
+    def spmv_repeat(self, x, y, n, stream=None):
+        """n back-to-back y = A x, queued from C (no Python between launches)."""
+        import torch
+        self._check_vec(x, self.cols, "x")
+        self._check_vec(y, self.rows, "y")
+        s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+        check(_lib.load().mx_spmv_repeat(self._h, x.data_ptr(), y.data_ptr(), int(n), s))
+        return y
+
     def spmv_host(self, x):
         x = np.ascontiguousarray(x, dtype=_np_dtype(self.dtype))
         if x.size != self.cols:

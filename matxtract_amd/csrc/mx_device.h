@@ -7,16 +7,20 @@
 namespace mx {
 
 // CSR matrix resident on the device, plus the row ranges of the CSR kernel's workgroups.
-// col/val carry kCsrPad extra zero entries so that aligned 128-bit loads may overrun.
+// col/val carry kCsrPad extra zero entries so that a wave's aligned 128-bit loads may overrun.
 struct DeviceCsr {
     int rows = 0, nnz = 0;
     int *rowPtr = nullptr;    // [rows+1]
     int *col = nullptr;       // [nnz + kCsrPad]
     void *val = nullptr;      // [nnz + kCsrPad]
-    int *blockRow = nullptr;  // [nBlocks+1] first row of each workgroup
+    int *blockDesc = nullptr; // [nBlocks][4] {first row, end row, first entry, end entry} per workgroup
     int nBlocks = 0;
+    int npt = 0;              // entries per lane per tile the rows were packed for
 };
-constexpr int kCsrPad = 16;
+constexpr int kCsrPad = 1088;  // a wave may read one whole wave tile (64*16 entries) past the end
+
+// Entries per lane per tile of the CSR kernel (a tile is 256 lanes wide).
+int csr_entries_per_lane(mx_dtype dtype);
 
 // Bitmap tiles resident on the device (the reference's chunkPtr / fragPtr / fragBit / tcVal /
 // sparse_AToX_index, restricted to the chunks the tile kernel executes).

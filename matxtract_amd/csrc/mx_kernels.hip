@@ -77,105 +77,165 @@ __device__ __forceinline__ T group_sum(T v)
 
 // ---- CSR part ---------------------------------------------------------------------------
 template <typename VT>
-struct Traits;
+struct Acc;
 template <>
-struct Traits<double> {
-    typedef double acc_t;
-    static constexpr int NPT = 4;  // entries per lane per tile: one 128-bit index load
+struct Acc<double> {
+    typedef double type;
 };
 template <>
-struct Traits<_Float16> {
-    typedef float acc_t;
-    static constexpr int NPT = 8;  // one 128-bit value load
+struct Acc<_Float16> {
+    typedef float type;
 };
 
-template <typename VT, int W>
-__device__ __forceinline__ void reduce_rows(const typename Traits<VT>::acc_t *prod, const int *__restrict__ rowPtr,
-                                            int r0, int nrows, int base, VT *__restrict__ y, int accumulate, int tid)
+// One wave's share of a tile: 64*NPT consecutive entries starting at the 16-byte aligned
+// position `pos` (wave-uniform).  Indices and values are streamed with 128-bit loads (lane l
+// gets entries 4l..4l+3 of each 256-entry group), then transposed through the wave's own LDS
+// region so that in every x gather lane l holds entry 64j+l: neighbouring lanes then ask for
+// neighbouring entries of a row, whose sorted columns share cache lines, and the address
+// unit serves them together instead of one lane per cycle.  Returns the products
+// p[j] = val[pos+64j+l] * x[col[pos+64j+l]].
+//   cs, vs : this wave's LDS regions, 64*NPT ints / accumulators.
+template <typename VT, int NPT>
+__device__ __forceinline__ void wave_products(const int *__restrict__ col, const VT *__restrict__ val,
+                                              const VT *__restrict__ x, int pos, int lane, int *cs,
+                                              typename Acc<VT>::type *vs, typename Acc<VT>::type (&p)[NPT])
 {
-    typedef typename Traits<VT>::acc_t AT;
+    typedef typename Acc<VT>::type AT;
+    if constexpr (sizeof(VT) == 8) {
+#pragma unroll
+        for (int q = 0; q < NPT / 4; ++q) {
+            const int e = 256 * q + 4 * lane;
+            const v4i32 c4 = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
+            const v2f64 va = __builtin_nontemporal_load((const v2f64 *)(val + pos + e));
+            const v2f64 vb = __builtin_nontemporal_load((const v2f64 *)(val + pos + e + 2));
+            *(v4i32 *)(cs + e) = c4;
+            *(v2f64 *)(vs + e) = va;
+            *(v2f64 *)(vs + e + 2) = vb;
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < NPT / 8; ++q) {
+            const int e = 512 * q + 8 * lane;
+            const v4i32 ca = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
+            const v4i32 cb = __builtin_nontemporal_load((const v4i32 *)(col + pos + e + 4));
+            const v8f16 hv = __builtin_nontemporal_load((const v8f16 *)(val + pos + e));
+            *(v4i32 *)(cs + e) = ca;
+            *(v4i32 *)(cs + e + 4) = cb;
+            v4f32 fa, fb;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                fa[j] = (float)hv[j];
+                fb[j] = (float)hv[4 + j];
+            }
+            *(v4f32 *)(vs + e) = fa;
+            *(v4f32 *)(vs + e + 4) = fb;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    AT xv[NPT];
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) xv[j] = (AT)x[cs[64 * j + lane]];
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) p[j] = vs[64 * j + lane] * xv[j];
+}
+
+// Sums the rows of one tile out of LDS: W lanes per row, `rowOff` holds the rows' start
+// offsets inside the tile (nrows+1 entries).
+template <typename VT, int W>
+__device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, const unsigned short *rowOff, int r0, int nrows,
+                                            VT *__restrict__ y, int accumulate, int tid)
+{
+    typedef typename Acc<VT>::type AT;
     constexpr int rowsPerPass = kBlock / W;
     const int g = tid / W, l = tid % W;
     for (int rr = g; rr < nrows; rr += rowsPerPass) {
-        const int r = r0 + rr;
-        const int a = rowPtr[r] - base, b = rowPtr[r + 1] - base;
+        const int a = rowOff[rr], b = rowOff[rr + 1];
         AT s = 0;
         for (int i = a + l; i < b; i += W) s += prod[i];
         s = group_sum<W>(s);
         if (l == 0) {
-            if (accumulate) s += (AT)y[r];
-            y[r] = (VT)s;
+            if (accumulate) s += (AT)y[r0 + rr];
+            y[r0 + rr] = (VT)s;
         }
     }
 }
 
-// One workgroup owns the whole rows [blockRow[b], blockRow[b+1]).  The host packs rows so
-// that their entries fit one tile of kBlock*NPT products (a single longer row gets a
-// workgroup of its own).  Phase 1 streams the tile with 128-bit loads, gathers x and parks
-// the products in LDS; phase 2 sums each row from LDS with W lanes per row, W picked from the
-// mean row length of the tile.  col/val are padded by the host so that aligned 128-bit loads
-// may run past the last entry.
-template <typename VT>
+// One workgroup owns the whole rows [r0, r1) named by its descriptor {r0, r1, p0, p1}
+// (p = positions of the first and one-past-last entry).  The host packs rows so that their
+// entries fit one tile of kBlock*NPT products and at most kBlock*NPT rows (a single longer
+// row gets a workgroup of its own).  Phase 1 issues the loads of the rows' start offsets and
+// lets each wave form the products of its quarter of the tile (wave_products), parked in
+// LDS.  Phase 2 sums each row from LDS with W lanes per row, W picked from the mean row length
+// of the tile; it touches global memory only to store y.  A row longer than a tile is swept
+// tile by tile with the same loads, each lane keeping a running sum.  col/val are padded by
+// the host so that aligned 128-bit loads may run past the end.
+template <typename VT, int NPT, bool XCD>
 __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict__ rowPtr, const int *__restrict__ col,
                                                           const VT *__restrict__ val, const VT *__restrict__ x,
-                                                          VT *__restrict__ y, const int *__restrict__ blockRow,
+                                                          VT *__restrict__ y, const int4 *__restrict__ blockDesc,
                                                           int accumulate)
 {
-    typedef typename Traits<VT>::acc_t AT;
-    constexpr int NPT = Traits<VT>::NPT;
+    typedef typename Acc<VT>::type AT;
     constexpr int TILE = kBlock * NPT;
-    __shared__ AT prod[TILE];
+    constexpr int WTILE = 64 * NPT;
+    __shared__ __attribute__((aligned(16))) AT prod[TILE];
+    __shared__ __attribute__((aligned(16))) int cols[TILE];
+    __shared__ unsigned short rowOff[TILE + 2];  // offsets inside the tile fit 16 bits
     __shared__ AT wsum[kBlock / 64];
 
-    const int b = xcd_contiguous_block(blockIdx.x, gridDim.x);
-    const int tid = threadIdx.x;
-    const int r0 = blockRow[b], r1 = blockRow[b + 1];
-    if (r1 <= r0) return;
-    const int p0 = rowPtr[r0], p1 = rowPtr[r1];
+    const int b = XCD ? xcd_contiguous_block(blockIdx.x, gridDim.x) : (int)blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int4 d = blockDesc[b];
+    const int r0 = d.x, r1 = d.y, p0 = d.z, p1 = d.w;
+    const int nrows = r1 - r0;
+    if (nrows <= 0) return;
     const int base = p0 & ~(NPT - 1);
+    int *cs = cols + wave * WTILE;
+    AT *vs = prod + wave * WTILE;
 
     if (p1 - base <= TILE) {
-        const int i = base + tid * NPT;
-        if (i < p1) {
-            int c[NPT];
-            AT v[NPT];
-            if constexpr (sizeof(VT) == 8) {
-                const v4i32 c4 = __builtin_nontemporal_load((const v4i32 *)(col + i));
-                const v2f64 v0 = __builtin_nontemporal_load((const v2f64 *)(val + i));
-                const v2f64 v1 = __builtin_nontemporal_load((const v2f64 *)(val + i + 2));
-                c[0] = c4.x; c[1] = c4.y; c[2] = c4.z; c[3] = c4.w;
-                v[0] = v0.x; v[1] = v0.y; v[2] = v1.x; v[3] = v1.y;
-            } else {
-                const v4i32 ca = __builtin_nontemporal_load((const v4i32 *)(col + i));
-                const v4i32 cb = __builtin_nontemporal_load((const v4i32 *)(col + i + 4));
-                const v8f16 hv = __builtin_nontemporal_load((const v8f16 *)(val + i));
-                c[0] = ca.x; c[1] = ca.y; c[2] = ca.z; c[3] = ca.w;
-                c[4] = cb.x; c[5] = cb.y; c[6] = cb.z; c[7] = cb.w;
+        // row offsets: lane t takes rows t, t+256, ... (at most NPT+1 of them)
+        int ro[NPT + 1];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) v[j] = (float)hv[j];
-            }
-            AT xv[NPT];
+        for (int k = 0; k <= NPT; ++k) {
+            const int rr = tid + k * kBlock;
+            ro[k] = rr <= nrows ? rowPtr[r0 + rr] : 0;
+        }
+        if (base + wave * WTILE < p1) {
+            AT p[NPT];
+            wave_products<VT, NPT>(col, val, x, base + wave * WTILE, lane, cs, vs, p);
 #pragma unroll
-            for (int j = 0; j < NPT; ++j) xv[j] = (AT)x[c[j]];
+            for (int j = 0; j < NPT; ++j) vs[64 * j + lane] = p[j];
+        }
 #pragma unroll
-            for (int j = 0; j < NPT; ++j) prod[tid * NPT + j] = v[j] * xv[j];
+        for (int k = 0; k <= NPT; ++k) {
+            const int rr = tid + k * kBlock;
+            if (rr <= nrows) rowOff[rr] = (unsigned short)(ro[k] - base);
         }
         __syncthreads();
-        const int nrows = r1 - r0;
         const int mean = (p1 - p0) / nrows;
-        if (mean <= 2) reduce_rows<VT, 1>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
-        else if (mean <= 4) reduce_rows<VT, 2>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
-        else if (mean <= 8) reduce_rows<VT, 4>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
-        else if (mean <= 16) reduce_rows<VT, 8>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
-        else if (mean <= 32) reduce_rows<VT, 16>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
-        else if (mean <= 64) reduce_rows<VT, 32>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
-        else reduce_rows<VT, 64>(prod, rowPtr, r0, nrows, base, y, accumulate, tid);
+        if (mean <= 2) reduce_rows<VT, 1>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 4) reduce_rows<VT, 2>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 8) reduce_rows<VT, 4>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 16) reduce_rows<VT, 8>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 32) reduce_rows<VT, 16>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 64) reduce_rows<VT, 32>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else reduce_rows<VT, 64>(prod, rowOff, r0, nrows, y, accumulate, tid);
     } else {
-        // a single row longer than one tile: strided sweep by the whole workgroup
+        // a single row longer than one tile
         AT s = 0;
-        for (int i = p0 + tid; i < p1; i += kBlock) s += (AT)val[i] * (AT)x[col[i]];
+        for (int t0 = base + wave * WTILE; t0 < p1; t0 += TILE) {
+            AT p[NPT];
+            wave_products<VT, NPT>(col, val, x, t0, lane, cs, vs, p);
+#pragma unroll
+            for (int j = 0; j < NPT; ++j) {
+                const int e = t0 + 64 * j + lane;
+                if (e >= p0 && e < p1) s += p[j];
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
         s = group_sum<64>(s);
-        if ((tid & 63) == 0) wsum[tid >> 6] = s;
+        if (lane == 0) wsum[wave] = s;
         __syncthreads();
         if (tid == 0) {
             AT t = 0;
@@ -325,15 +385,25 @@ __global__ void probe_mfma_f16_kernel(const _Float16 *A /*[64][8]*/, const _Floa
 // ---- launchers (called from mx_plan.cpp; plain functions so that file needs no HIP syntax)
 namespace mx {
 
+template <typename VT, int NPT>
+static void launch_csr_t(const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
+{
+    hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr, A.col,
+                       (const VT *)A.val, (const VT *)x, (VT *)y, (const int4 *)A.blockDesc, accumulate);
+}
+
 hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
 {
     if (A.nBlocks <= 0) return hipSuccess;
-    if (dtype == MX_F64)
-        hipLaunchKernelGGL(mxk::csr_rows_kernel<double>, dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr, A.col,
-                           (const double *)A.val, (const double *)x, (double *)y, A.blockRow, accumulate);
-    else
-        hipLaunchKernelGGL(mxk::csr_rows_kernel<_Float16>, dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr, A.col,
-                           (const _Float16 *)A.val, (const _Float16 *)x, (_Float16 *)y, A.blockRow, accumulate);
+    if (dtype == MX_F64) {
+        if (A.npt == 8) launch_csr_t<double, 8>(A, x, y, accumulate, s);
+        else if (A.npt == 4) launch_csr_t<double, 4>(A, x, y, accumulate, s);
+        else return hipErrorInvalidValue;
+    } else {
+        if (A.npt == 16) launch_csr_t<_Float16, 16>(A, x, y, accumulate, s);
+        else if (A.npt == 8) launch_csr_t<_Float16, 8>(A, x, y, accumulate, s);
+        else return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

@@ -2,6 +2,7 @@
 // hybrid SpMV; plus the reference's one-shot host-pointer entry points built on top.
 #include <algorithm>
 #include <chrono>
+#include <cstdlib>
 #include <cstring>
 #include <numeric>
 #include <vector>
@@ -52,17 +53,20 @@ int upload_bytes(void **dst, const void *src, size_t n, size_t pad = 0)
 // Rows of each CSR-kernel workgroup (the role of pre_startRowPerBlock,
 // src/spmv_kernel/cdSpMV.cu:4-27, but row-aligned): greedily pack whole rows while their
 // entries, counted from the tile's aligned start, fit one tile; a longer row stands alone.
-void pack_rows(const int *rowPtr, int rows, int npt, std::vector<int> &blockRow)
+// One descriptor {first row, end row, first entry, end entry} per workgroup.
+void pack_rows(const int *rowPtr, int rows, int npt, std::vector<int> &desc)
 {
     const int tile = 256 * npt;
-    blockRow.clear();
-    blockRow.push_back(0);
+    desc.clear();
     int r = 0;
     while (r < rows) {
         const int base = rowPtr[r] & ~(npt - 1);
         int r1 = r + 1;
         while (r1 < rows && rowPtr[r1 + 1] - base <= tile && r1 - r < tile) ++r1;
-        blockRow.push_back(r1);
+        desc.push_back(r);
+        desc.push_back(r1);
+        desc.push_back(rowPtr[r]);
+        desc.push_back(rowPtr[r1]);
         r = r1;
     }
 }
@@ -72,7 +76,7 @@ void free_csr(mx::DeviceCsr &A)
     (void)hipFree(A.rowPtr);
     (void)hipFree(A.col);
     (void)hipFree(A.val);
-    (void)hipFree(A.blockRow);
+    (void)hipFree(A.blockDesc);
     A = mx::DeviceCsr();
 }
 
@@ -90,24 +94,34 @@ void free_tiles(mx::DeviceTiles &T)
 int upload_csr(mx_dtype dtype, int rows, int nnz, const int *rowPtr, const int *col, const void *val,
                mx::DeviceCsr &A, double *pack_ms)
 {
-    const int es = mx::elem_size(dtype), npt = dtype == MX_F64 ? 4 : 8;
+    const int es = mx::elem_size(dtype), npt = mx::csr_entries_per_lane(dtype);
     A.rows = rows;
+    A.npt = npt;
     A.nnz = nnz;
     int rc;
     if ((rc = upload(&A.rowPtr, rowPtr, (size_t)rows + 1))) return rc;
     if ((rc = upload(&A.col, col, (size_t)nnz, mx::kCsrPad))) return rc;
     if ((rc = upload_bytes(&A.val, val, (size_t)nnz * es, (size_t)mx::kCsrPad * es))) return rc;
-    std::vector<int> blockRow;
+    std::vector<int> desc;
     auto t0 = std::chrono::steady_clock::now();
-    pack_rows(rowPtr, rows, npt, blockRow);
+    pack_rows(rowPtr, rows, npt, desc);
     auto t1 = std::chrono::steady_clock::now();
     if (pack_ms) *pack_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
-    A.nBlocks = (int)blockRow.size() - 1;
-    if ((rc = upload(&A.blockRow, blockRow.data(), blockRow.size()))) return rc;
+    A.nBlocks = (int)desc.size() / 4;
+    if ((rc = upload(&A.blockDesc, desc.data(), desc.size()))) return rc;
     return MX_OK;
 }
 
 }  // namespace
+
+// MX_CSR_NPT overrides the default (for tuning runs); only values with a compiled kernel count.
+int mx::csr_entries_per_lane(mx_dtype dtype)
+{
+    const char *e = std::getenv("MX_CSR_NPT");
+    const int v = e ? std::atoi(e) : 0;
+    if (dtype == MX_F64) return (v == 4 || v == 8) ? v : 4;
+    return (v == 8 || v == 16) ? v : 8;
+}
 
 struct mx_plan {
     mx_dtype dtype = MX_F64;
@@ -321,6 +335,19 @@ extern "C" int mx_spmv(mx_plan *plan, const void *x_dev, void *y_dev, void *stre
         return MX_ERR_ARG;
     }
     return spmv_on(plan, x_dev, y_dev, (hipStream_t)stream);
+}
+
+extern "C" int mx_spmv_repeat(mx_plan *plan, const void *x_dev, void *y_dev, int n, void *stream)
+{
+    if (!plan || !x_dev || !y_dev || n < 0) {
+        set_error("mx_spmv_repeat: bad argument");
+        return MX_ERR_ARG;
+    }
+    for (int i = 0; i < n; ++i) {
+        int rc = spmv_on(plan, x_dev, y_dev, (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    return MX_OK;
 }
 
 extern "C" int mx_spmv_host(mx_plan *plan, const void *x_host, void *y_host)
