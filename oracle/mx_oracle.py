@@ -92,7 +92,7 @@ def _i32(a):
 
 
 def _val_dtype(elem):
-    return np.float64 if elem == 8 else np.uint16
+    return np.float64 if elem == 8 else np.float16
 
 
 def as_bits16(a):

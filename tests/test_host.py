@@ -1,0 +1,283 @@
+"""Host side of the product (no GPU): the partitioner against the oracle, bit for bit; the
+generators; Matrix-Market ingest; the C ABI's symbols and error behaviour."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+INT_ARRAYS = ("newArray", "rId", "newArray_", "ddRowPtr", "ddColInd", "chunkPtr", "sparse_AToX_index",
+              "fragPtr", "fragBit", "cdRowPtr", "cdColInd")
+VAL_ARRAYS = ("ddVal", "tcVal", "cdVal")
+SCALARS = ("dCols", "sCols", "nnzColD", "nnzColS", "dRows", "sRows", "nnzRowD", "nnzRowS", "chunkNum",
+           "totalTcFrags", "tcValCount", "nnzCD", "fragM", "fragK")
+
+
+def assert_same_partition(P, O):
+    """P: product partition, O: oracle partition; every canonical array must be identical."""
+    for name in SCALARS:
+        assert getattr(P, name) == getattr(O, name), name
+    for name in INT_ARRAYS:
+        assert np.array_equal(getattr(P, name), getattr(O, name)), name
+    for name in VAL_ARRAYS:  # compare bit patterns, not values
+        a, b = getattr(P, name), getattr(O, name)
+        assert a.dtype.itemsize == b.dtype.itemsize and np.array_equal(a.view(np.uint8), b.view(np.uint8)), name
+    if P.dCols or P.dRows:
+        assert np.array_equal(P.descColId, O.descColId), "descColId"
+        assert P.cols_ratio == O.cols_ratio
+        # 0 extracted entries over 0 fragments is 0/0 = NaN on both sides, as in the reference
+        assert P.tc_nnz_ratio == O.tc_nnz_ratio or (np.isnan(P.tc_nnz_ratio) and np.isnan(O.tc_nnz_ratio))
+
+
+TAUS = [(0.0, 0.0), (0.25, 0.0), (0.25, 0.25), (0.5, 0.25), (0.5, 0.5), (0.75, 0.5), (1.0, 0.0), (1.0, 0.75),
+        (1.0, 1.0), (0.37, 0.11)]
+
+
+@pytest.mark.parametrize("cfg,scale", [(1, 0.25), (2, 1 / 32), (3, 0.004), (4, 1 / 128), (5, 1 / 512)])
+def test_partition_bit_exact_on_synthetic_workloads(mx, ora, cfg, scale):
+    A, _ = mx.gen_config(cfg, scale=scale)
+    for tau in TAUS:
+        P = mx.Partition(A, *tau)
+        O = ora.partition(A.rowPtr, A.colInd, A.val, A.cols, *tau)
+        assert_same_partition(P, O)
+        h = P.hash
+        assert h == mx.Partition(A, *tau).hash  # deterministic (the partitioner is multi-threaded)
+        P.close()
+
+
+@pytest.mark.parametrize("seed", range(8))
+@pytest.mark.parametrize("dtype", [np.float64, np.float16])
+def test_partition_bit_exact_on_hostile_inputs(mx, ora, seed, dtype):
+    """Unsorted rows, repeated (row, col) pairs, empty rows and columns, non-square shapes, a
+    ragged last chunk."""
+    rng = np.random.default_rng(1000 + seed)
+    rows, cols = int(rng.integers(1, 90)), int(rng.integers(1, 90))
+    lens = rng.integers(0, min(cols, 12) + 1, rows)
+    lens[rng.random(rows) < 0.2] = 0
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = rng.integers(0, cols, rp[-1]).astype(np.int32)      # with replacement: duplicates, any order
+    va = (rng.integers(-8, 9, rp[-1]) / 8.0).astype(dtype)
+    A = mx.Csr(rows, cols, rp, ci, va)
+    for tau in TAUS:
+        P = mx.Partition(A, *tau)
+        O = ora.partition(rp, ci, va, cols, *tau)
+        assert_same_partition(P, O)
+        P.close()
+
+
+def test_partition_rejects_bad_arguments(mx):
+    A, _ = mx.gen_config(1, scale=0.05)
+    with pytest.raises(mx.MxError) as e:
+        mx.Partition(A, 0.25, 0.5)  # col_frac < hot_frac, as the reference CLI refuses
+    assert e.value.code == 1 and "col_frac must be greater than hot_frac" in str(e.value)
+    with pytest.raises(mx.MxError):
+        mx.Partition(A, 1.5, 0.5)
+    bad = mx.Csr(A.rows, A.cols, A.rowPtr, A.colInd.copy(), A.val)
+    bad.colInd[3] = A.cols  # out of range
+    with pytest.raises(mx.MxError):
+        mx.Partition(bad, 0.5, 0.25)
+    bad = mx.Csr(A.rows, A.cols, A.rowPtr.copy(), A.colInd, A.val)
+    bad.rowPtr[2] = bad.rowPtr[3] + 1  # not monotone
+    with pytest.raises(mx.MxError):
+        mx.Partition(bad, 0.5, 0.25)
+
+
+def test_empty_matrix(mx, ora):
+    A = mx.Csr(5, 7, np.zeros(6, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float64))
+    for tau in [(0.0, 0.0), (1.0, 1.0)]:
+        P = mx.Partition(A, *tau)
+        O = ora.partition(A.rowPtr, A.colInd, A.val, 7, *tau)
+        assert P.nnzCD == 0 and P.totalTcFrags == 0
+        assert_same_partition(P, O)
+
+
+def test_transpose_matches_oracle_and_scipy(mx, ora):
+    rng = np.random.default_rng(4)
+    A = sp.random(80, 60, 0.1, format="csr", random_state=rng)
+    A.sort_indices()
+    for dtype in (np.float64, np.float16):
+        val = A.data.astype(dtype)
+        got = mx.transpose(A.indptr, A.indices, val, 60)
+        ref = ora.transpose(A.indptr, A.indices, val, 60)
+        for g, r in zip(got, ref):
+            assert np.array_equal(g.view(np.uint8), r.view(np.uint8))
+    C_ = A.tocsc()
+    C_.sort_indices()
+    tp, ti, tv = mx.transpose(A.indptr, A.indices, A.data, 60)
+    assert np.array_equal(tp, C_.indptr) and np.array_equal(ti, C_.indices) and np.array_equal(tv, C_.data)
+
+
+# ---------------------------------------------------------------- generators
+def test_generators_are_seeded_and_well_formed(mx):
+    for cfg, scale in [(1, 0.5), (2, 1 / 16), (3, 0.008), (4, 1 / 64), (5, 1 / 256)]:
+        A, x = mx.gen_config(cfg, scale=scale)
+        B, x2 = mx.gen_config(cfg, scale=scale)
+        assert np.array_equal(A.colInd, B.colInd) and np.array_equal(A.val.view(np.uint8), B.val.view(np.uint8))
+        assert np.array_equal(x.view(np.uint8), x2.view(np.uint8))
+        C_, _ = mx.gen_config(cfg, seed=12345, scale=scale)
+        if cfg != 3:  # the stencil has no random part in the matrix
+            assert not np.array_equal(A.colInd, C_.colInd)
+        assert A.rows == A.cols and A.rowPtr[0] == 0 and A.rowPtr[-1] == A.nnz
+        for r in range(0, A.rows, max(1, A.rows // 200)):  # sorted, distinct columns in each row
+            c = A.colInd[A.rowPtr[r]:A.rowPtr[r + 1]]
+            assert np.all(np.diff(c) > 0) and (len(c) == 0 or (c[0] >= 0 and c[-1] < A.cols))
+        assert A.val.dtype == (np.float64 if cfg <= 3 else np.float16)
+        v = A.val.astype(np.float64)
+        assert np.all(np.abs(v) <= 26.0) and np.all(np.isfinite(v))
+
+
+def test_generator_shapes(mx):
+    A, _ = mx.gen_config(1)
+    assert A.rows == 4096 and A.nnz == 65536 and np.all(np.diff(A.rowPtr) == 16)
+    A, _ = mx.gen_config(2, scale=1 / 8)
+    assert A.rows == 8192 and np.all(np.diff(A.rowPtr) == 64)
+    # 40% of the entries sit in dense, 8-aligned 8x8 blocks
+    dense = 0
+    for br in range(0, A.rows, 8):
+        cols = [set(A.colInd[A.rowPtr[r]:A.rowPtr[r + 1]] // 8 * 8) for r in range(br, br + 8)]
+        for c0 in set.intersection(*cols):
+            if all(np.isin(np.arange(c0, c0 + 8), A.colInd[A.rowPtr[r]:A.rowPtr[r + 1]]).all() for r in range(br, br + 8)):
+                dense += 64
+    assert 0.38 <= dense / A.nnz <= 0.45
+    A, x = mx.gen_config(3, scale=0.008)  # 20^3
+    assert A.rows == 8000 and A.nnz == (3 * 20 - 2) ** 3 and x.min() >= 0 and x.max() <= 1
+    A, _ = mx.gen_config(4, scale=1 / 16)
+    lens = np.diff(A.rowPtr)
+    assert lens.min() == 1 and lens.max() <= 4096 and 6 <= lens.mean() <= 16 and (lens == 1).mean() > 0.8
+    A, _ = mx.gen_config(5, scale=1 / 64)
+    lens = np.diff(A.rowPtr)
+    strip = [r for r in range(0, A.rows, 8) if np.all(lens[r:r + 8] == 32) and
+             np.all(np.diff(A.colInd[A.rowPtr[r]:A.rowPtr[r + 1]]) == 1)]
+    assert 0.12 <= 8 * len(strip) / A.rows <= 0.28
+
+
+# ---------------------------------------------------------------- Matrix-Market ingest
+def write_mtx(path, header, size, lines):
+    with open(path, "w") as f:
+        f.write("%%MatrixMarket matrix coordinate " + header + "\n% a comment\n" + size + "\n" + "\n".join(lines) + "\n")
+
+
+def test_mmio_general_keeps_file_order(mx, tmp_path):
+    p = tmp_path / "g.mtx"
+    write_mtx(p, "real general", "3 4 5", ["2 3 1.5", "1 4 -2", "2 1 3", "1 1 4", "2 3 7"])
+    A, sym = mx.mmio_read(p)
+    assert not sym and (A.rows, A.cols, A.nnz) == (3, 4, 5)
+    assert A.rowPtr.tolist() == [0, 2, 5, 5]
+    assert A.colInd.tolist() == [3, 0, 2, 0, 2]           # file order inside each row, duplicates kept
+    assert A.val.tolist() == [-2.0, 4.0, 1.5, 3.0, 7.0]
+
+
+def test_mmio_symmetric_expansion_and_pattern(mx, tmp_path):
+    p = tmp_path / "s.mtx"
+    write_mtx(p, "pattern symmetric", "3 3 3", ["2 1", "3 3", "3 1"])
+    A, sym = mx.mmio_read(p)
+    assert sym and A.nnz == 5
+    D = sp.csr_matrix((A.val, A.colInd, A.rowPtr), shape=(3, 3)).toarray()
+    assert np.array_equal(D, np.array([[0, 1, 1], [1, 0, 0], [1, 0, 1.0]]))
+    # the mirrored entry directly follows the stored one: row 0 gets (0,1) from "2 1" then (0,2) from "3 1"
+    assert A.colInd[A.rowPtr[0]:A.rowPtr[1]].tolist() == [1, 2]
+    p = tmp_path / "k.mtx"
+    write_mtx(p, "real skew-symmetric", "2 2 1", ["2 1 5"])
+    A, sym = mx.mmio_read(p)
+    assert not sym and A.nnz == 1                          # not expanded, as in the reference
+    p = tmp_path / "i.mtx"
+    write_mtx(p, "integer general", "2 2 2", ["1 1 3", "2 2 -4"])
+    A, _ = mx.mmio_read(p, mx.MX_F16)
+    assert A.val.dtype == np.float16 and A.val.tolist() == [3.0, -4.0]
+    with pytest.raises(mx.MxError) as e:
+        mx.mmio_read(tmp_path / "missing.mtx")
+    assert e.value.code == 4
+
+
+def test_init_vec(mx):
+    v = mx.init_vec(40)
+    assert np.array_equal(v, np.arange(40) % 15)
+    h = mx.init_vec(40, mx.MX_F16)
+    assert h.dtype == np.float16 and np.array_equal(h.astype(np.float64), np.arange(40) % 15)
+
+
+def test_f16_conversions_match_numpy(mx):
+    from matxtract_amd import _lib
+    L = _lib.load()
+    rng = np.random.default_rng(2)
+    vals = np.concatenate([rng.uniform(-70000, 70000, 3000), rng.uniform(-1e-4, 1e-4, 3000),
+                           [0.0, 65504.0, 65520.0, 2.9802322e-08, 1e-9, np.inf]]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        ref = vals.astype(np.float16).view(np.uint16)
+    got = np.array([L.mx_f32_to_f16(float(v)) for v in vals], np.uint16)
+    assert np.array_equal(got, ref)
+    h = np.arange(0, 65536, 7, dtype=np.uint16)
+    back = np.array([L.mx_f16_to_f32(int(b)) for b in h], np.float32)
+    ref = h.view(np.float16).astype(np.float32)
+    ok = ~np.isnan(ref)
+    assert np.array_equal(back[ok], ref[ok])
+
+
+def test_algorithmic_bytes(mx):
+    # nnz*(sizeof(valT)+4) + (rows+1)*4 + cols*sizeof(valT) + rows*sizeof(valT)
+    assert mx.algorithmic_bytes(mx.MX_F64, 4096, 4096, 65536) == 868356
+    assert mx.algorithmic_bytes(mx.MX_F64, 1000000, 1000000, 26463592) == 337563108
+    assert mx.algorithmic_bytes(mx.MX_F16, 10, 20, 100) == 100 * 6 + 11 * 4 + 20 * 2 + 10 * 2
+
+
+# ---------------------------------------------------------------- ABI
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "matxtract_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(mx):
+    from matxtract_amd import _lib
+    L = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(L, n), "libmatxtract_hip.so does not export " + n
+    assert sorted(_lib.SIGNATURES) == names  # the Python binding covers exactly the header
+
+
+def test_device_entry_points_fail_loudly_without_a_gpu(mx):
+    if mx.device_count() > 0:
+        pytest.skip("a GPU is present")
+    A, x = mx.gen_config(1, scale=0.05)
+    P = mx.Partition(A, 0.5, 0.25)
+    with pytest.raises(mx.MxError) as e:
+        mx.Plan(P)
+    assert e.value.code == 3 and "no CPU fallback" in str(e.value)
+    with pytest.raises(mx.MxError):
+        mx.cdspmv(A, x, np.zeros(A.rows))
+
+
+def test_product_does_not_reach_into_the_oracle():
+    """Nothing under the package, the headers or bench-independent entry points names the oracle."""
+    pkg = os.path.join(ROOT, "matxtract_amd")
+    for base, _, files in os.walk(pkg):
+        if os.path.basename(base) == "build":
+            continue
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h", "Makefile")):
+                text = open(os.path.join(base, f), errors="replace").read()
+                assert "mx_oracle" not in text and "oracle/" not in text, os.path.join(base, f)
+
+
+# ---------------------------------------------------------------- CLI argument handling (no GPU needed)
+def cli(*args):
+    exe = os.path.join(ROOT, "matxtract_amd", "bin", "matxtract_perftest")
+    if not os.path.exists(exe):
+        pytest.skip("CLI not built")
+    return subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
+
+
+def test_cli_argument_errors_match_the_reference():
+    r = cli()
+    assert r.returncode == 1 and "Run the code by './matxtract_perftest (col_frac) (hot_frac) matrix.mtx'." in r.stdout
+    r = cli("0.2", "0.5", "x.mtx")
+    assert r.returncode == 1 and "Error: col_frac must be greater than hot_frac." in r.stdout
+    r = cli("0.5", "0.2", "0.1", "x.mtx")
+    assert r.returncode == 1 and "Error: Too many arguments provided." in r.stdout
