@@ -94,3 +94,182 @@ def test_hybrid_spmv_matches_oracle(mx, ora, cfg, scale, flags):
         assert rel_l2(y2.cpu().numpy(), ref) <= tol
         plan.close()
         part.close()
+
+
+# ---------------------------------------------------------------- full BASELINE sizes
+FULL = [
+    # (workload, taus)
+    (2, [(0.0, 0.0), (0.5, 0.25), (1.0, 1.0)]),
+    (3, [(0.0, 0.0), (0.5, 0.5)]),
+    (4, [(0.0, 0.0), (0.5, 0.25)]),
+    (5, [(0.0, 0.0), (0.5, 0.5)]),
+]
+
+
+@pytest.mark.parametrize("cfg,taus", FULL)
+def test_full_size_workloads_match_oracle(mx, ora, cfg, taus):
+    """The oracle is a plain C loop: it handles the full-size matrices in well under a second."""
+    import torch
+    A, x = mx.gen_config(cfg)
+    ref = oracle_y(ora, mx, A, x)
+    tol = F64_TOL if A.dtype == mx.MX_F64 else F16_TOL
+    xd = torch.from_numpy(x).cuda()
+    for tau in taus:
+        for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES):
+            print("full-size workload=%d tau=%s flags=%d" % (cfg, tau, fl), flush=True)
+            part = mx.Partition(A, *tau)
+            plan = mx.Plan(part, fl)
+            y = plan.spmv(xd)
+            torch.cuda.synchronize()
+            err = rel_l2(y.cpu().numpy(), ref)
+            assert err <= tol, (cfg, tau, fl, err)
+            plan.close()
+            part.close()
+
+
+def test_full_size_stencil_closed_form(mx):
+    """100^3 27-point stencil times the all-ones vector: 26 - #neighbours, exactly."""
+    import torch
+    A, _ = mx.gen_config(3)
+    g = 100
+    xd = torch.ones(A.cols, dtype=torch.float64, device="cuda")
+    z, yy, xx = np.meshgrid(np.arange(g), np.arange(g), np.arange(g), indexing="ij")
+    border = lambda i: (i == 0) | (i == g - 1)
+    expect = np.choose(border(z).astype(int) + border(yy) + border(xx), [0.0, 9.0, 15.0, 19.0]).ravel()
+    for tau, fl in (((0.0, 0.0), mx.MX_PLAN_DEFAULT), ((0.5, 0.25), mx.MX_PLAN_ALL_TILES)):
+        part = mx.Partition(A, *tau)
+        plan = mx.Plan(part, fl)
+        y = plan.spmv(xd)
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy(), expect)
+        plan.close()
+        part.close()
+
+
+def test_linearity_at_full_size(mx):
+    import torch
+    A, x = mx.gen_config(2)
+    part = mx.Partition(A, 0.5, 0.25)
+    plan = mx.Plan(part, mx.MX_PLAN_ALL_TILES)
+    x1 = torch.from_numpy(x).cuda()
+    x2 = torch.flip(x1, [0]).contiguous()
+    y1 = plan.spmv(x1).clone()
+    y2 = plan.spmv(x2).clone()
+    y12 = plan.spmv((2.0 * x1 - 0.5 * x2).contiguous())
+    torch.cuda.synchronize()
+    d = (y12 - (2.0 * y1 - 0.5 * y2)).norm() / y12.norm()
+    assert float(d) <= 1e-13
+
+
+# ---------------------------------------------------------------- reference surface
+def test_cdspmv_accumulates_into_y(mx, ora):
+    """cdspmv(): y is IN/OUT (y += A x).  Small-integer data makes FP64 sums exact, so any
+    summation order must agree bit for bit, as in the reference's own self-check."""
+    A, _ = mx.gen_config(2, scale=1 / 32)
+    A = mx.Csr(A.rows, A.cols, A.rowPtr, A.colInd, mx.init_vec(A.nnz))
+    x = mx.init_vec(A.cols)
+    y0 = np.arange(A.rows, dtype=np.float64) % 7
+    y, t, pre = mx.cdspmv(A, x, y0, warm=1, iters=3)
+    assert np.array_equal(y, ora.spmv_f64(A.val, A.rowPtr, A.colInd, x, y0=y0))
+    assert t > 0 and pre >= 0
+    # FP16, uniform data, tolerance of the FP16 path
+    A, x = mx.gen_config(4, scale=1 / 64)
+    y, _, _ = mx.cdspmv(A, x, np.zeros(A.rows, np.float16))
+    assert rel_l2(y, ora.spmv_f16_f32acc(A.val, A.rowPtr, A.colInd, x)[0]) <= F16_TOL
+
+
+def test_du_tcspmv_on_canonical_tile_arrays(mx, ora):
+    """du_tcspmv_fp64 adds A_dd x_d to the y it is given; du_tcspmv_fp16_v2 overwrites y."""
+    A, x = mx.gen_config(2, scale=1 / 32)
+    O = ora.partition(A.rowPtr, A.colInd, A.val, A.cols, 0.5, 0.25)
+    P = mx.Partition(A, 0.5, 0.25)
+    x_d = x[P.descColId[:P.dCols]]
+    y0 = np.linspace(-1, 1, P.dRows)
+    y, t = mx.du_tcspmv(P, x_d, y0, warm=1, iters=3)
+    assert rel_l2(y - y0, ora.tcspmv(O, x_d)) <= F64_TOL and t > 0
+    A, x = mx.gen_config(5, scale=1 / 256)
+    O = ora.partition(A.rowPtr, A.colInd, A.val, A.cols, 0.5, 0.5)
+    P = mx.Partition(A, 0.5, 0.5)
+    x_d = x[P.descColId[:P.dCols]]
+    y, _ = mx.du_tcspmv(P, x_d, np.full(P.dRows, 3.0, np.float16))
+    assert rel_l2(y, ora.tcspmv(O, x_d)) <= F16_TOL
+
+
+def test_spmv_host_and_argument_checks(mx, ora):
+    import torch
+    A, x = mx.gen_config(1)
+    part = mx.Partition(A, 0.5, 0.25)
+    plan = mx.Plan(part)
+    assert rel_l2(plan.spmv_host(x), oracle_y(ora, mx, A, x)) <= F64_TOL
+    with pytest.raises(ValueError):
+        plan.spmv(torch.zeros(A.cols - 1, dtype=torch.float64, device="cuda"))
+    with pytest.raises(ValueError):
+        plan.spmv(torch.zeros(A.cols, dtype=torch.float32, device="cuda"))
+
+
+def test_ragged_and_degenerate_shapes(mx, ora):
+    import torch
+    rng = np.random.default_rng(77)
+    for rows, cols in ((1, 1), (3, 50), (50, 3), (9, 9), (257, 131)):
+        lens = rng.integers(0, min(cols, 9) + 1, rows)
+        rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        ci = np.concatenate([np.sort(rng.choice(cols, l, replace=False)) for l in lens] + [np.zeros(0, int)]).astype(np.int32)
+        for dtype, tol in ((np.float64, F64_TOL), (np.float16, F16_TOL)):
+            va = rng.uniform(-1, 1, rp[-1]).astype(dtype)
+            x = rng.uniform(-1, 1, cols).astype(dtype)
+            A = mx.Csr(rows, cols, rp, ci, va)
+            ref = oracle_y(ora, mx, A, x)
+            for tau in ((0.0, 0.0), (0.6, 0.3), (1.0, 1.0)):
+                print("ragged rows=%d cols=%d dtype=%s tau=%s" % (rows, cols, dtype.__name__, tau), flush=True)
+                part = mx.Partition(A, *tau)
+                plan = mx.Plan(part, mx.MX_PLAN_ALL_TILES)
+                y = plan.spmv(torch.from_numpy(x).cuda())
+                torch.cuda.synchronize()
+                got = y.cpu().numpy().astype(np.float64)
+                assert np.linalg.norm(got - ref) <= tol * max(np.linalg.norm(ref), 1e-30) + 1e-300
+                plan.close()
+                part.close()
+
+
+def test_long_rows_take_the_multi_tile_path(mx, ora):
+    """One row far longer than a workgroup tile, next to short ones."""
+    import torch
+    rng = np.random.default_rng(8)
+    cols = 30000
+    lens = np.array([3, 20000, 0, 5, 9000, 1])
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = np.concatenate([np.sort(rng.choice(cols, l, replace=False)) for l in lens]).astype(np.int32)
+    for dtype, tol in ((np.float64, F64_TOL), (np.float16, F16_TOL)):
+        A = mx.Csr(len(lens), cols, rp, ci, rng.uniform(-1, 1, rp[-1]).astype(dtype))
+        x = rng.uniform(-1, 1, cols).astype(dtype)
+        part = mx.Partition(A, 0.0, 0.0)
+        plan = mx.Plan(part)
+        y = plan.spmv(torch.from_numpy(x).cuda())
+        torch.cuda.synchronize()
+        assert rel_l2(y.cpu().numpy(), oracle_y(ora, mx, A, x)) <= tol
+        plan.close()
+
+
+def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
+    """matxtract_perftest's stdout keeps the forms the reference's scripts grep for."""
+    import re
+    import subprocess
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "matxtract_amd", "bin", "matxtract_perftest")
+    A, _ = mx.gen_config(2, scale=1 / 64)
+    p = tmp_path / "m.mtx"
+    with open(p, "w") as f:
+        f.write("%%MatrixMarket matrix coordinate real general\n")
+        f.write("%d %d %d\n" % (A.rows, A.cols, A.nnz))
+        for r in range(A.rows):
+            for q in range(A.rowPtr[r], A.rowPtr[r + 1]):
+                f.write("%d %d %.17g\n" % (r + 1, A.colInd[q] + 1, A.val[q]))
+    for args in (["0.5", "0.25", str(p)], [str(p)]):
+        out = subprocess.run([exe, "--warm", "2", "--iters", "5", *args], capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        assert re.search(r"MatXtract time\s*=\s*([\d\.Ee+-]+)\s*ms", out.stdout)      # ML/bayes_opt.py:64
+        assert "Success! All values match within the tolerance for %d elements." % A.rows in out.stdout
+        assert re.search(r"MatXtract GFLOPS= \d+\.\d\d", out.stdout)
+        if len(args) == 3:
+            assert re.search(r"cols_ratio = \d\.\d+", out.stdout) and re.search(r"TC_nnz_ratio = \d\.\d+", out.stdout)
