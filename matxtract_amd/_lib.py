@@ -13,6 +13,7 @@ CSRC = os.path.join(_HERE, "csrc")
 MX_OK, MX_ERR_ARG, MX_ERR_ALLOC, MX_ERR_DEVICE, MX_ERR_IO = 0, 1, 2, 3, 4
 MX_F64, MX_F16 = 0, 1
 MX_PLAN_DEFAULT, MX_PLAN_NO_TILES, MX_PLAN_ALL_TILES = 0, 1, 2
+MX_PLAN_CSR_ROWS, MX_PLAN_CSR_PANELS = 4, 8
 
 
 class MxError(RuntimeError):
@@ -47,7 +48,7 @@ class PartitionView(C.Structure):
 class PlanInfo(C.Structure):
     _fields_ = [("dtype", C.c_int), ("rows", C.c_int), ("cols", C.c_int), ("nnz", C.c_int),
                 ("tile_chunks", C.c_int), ("tile_frags", C.c_int), ("tile_nnz", C.c_int),
-                ("csr_nnz", C.c_int), ("csr_blocks", C.c_int),
+                ("csr_nnz", C.c_int), ("csr_blocks", C.c_int), ("csr_variant", C.c_int),
                 ("tile_bytes", C.c_double), ("csr_bytes", C.c_double)]
 
 

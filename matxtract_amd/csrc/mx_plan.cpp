@@ -91,6 +91,110 @@ void free_tiles(mx::DeviceTiles &T)
     T = mx::DeviceTiles();
 }
 
+void free_panels(mx::DevicePanels &P)
+{
+    (void)hipFree(P.blockRow);
+    (void)hipFree(P.listPtr);
+    (void)hipFree(P.list);
+    (void)hipFree(P.erow);
+    (void)hipFree(P.ecol);
+    (void)hipFree(P.eval);
+    P = mx::DevicePanels();
+}
+
+// Re-lays a CSR matrix for csr_panel_kernel: row blocks balanced by entries (at most
+// `maxRows` rows each, about one block per CU), column panels of panel_cols(dtype) columns;
+// the entries of each (block, panel) group keep their row-major order and are padded with
+// zero entries to a multiple of 8 so every group starts on a 16-byte boundary.
+int upload_panels(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU,
+                  mx::DevicePanels &D)
+{
+    const int es = mx::elem_size(dtype);
+    const int PW = mx::panel_cols(dtype), maxRows = mx::panel_max_block_rows(dtype);
+    const size_t depth = (size_t)mx::kPanelListPad;
+    const int nnz = rowPtr[rows];
+    const int nPanels = std::max(1, (cols + PW - 1) / PW);
+    const long long target = std::max<long long>(1, ((long long)nnz + nCU - 1) / std::max(nCU, 1));
+    std::vector<int> blockRow(1, 0);
+    for (int r = 0; r < rows;) {
+        const int start = r;
+        long long cnt = 0;
+        while (r < rows && r - start < maxRows && (cnt < target || r == start)) {
+            cnt += rowPtr[r + 1] - rowPtr[r];
+            ++r;
+        }
+        blockRow.push_back(r);
+    }
+    const int nBlocks = (int)blockRow.size() - 1;
+    std::vector<long long> grp((size_t)nBlocks * nPanels + 1, 0);
+#pragma omp parallel for schedule(dynamic, 4)
+    for (int b = 0; b < nBlocks; ++b) {
+        long long *g = grp.data() + (size_t)b * nPanels + 1;
+        for (int p = rowPtr[blockRow[b]]; p < rowPtr[blockRow[b + 1]]; ++p) g[col[p] / PW]++;
+        for (int q = 0; q < nPanels; ++q) g[q] = (g[q] + 7) / 8 * 8;
+    }
+    for (size_t i = 1; i < grp.size(); ++i) grp[i] += grp[i - 1];
+    const long long total = grp.back();
+    if (total > 2000000000LL) {
+        set_error("panel layout: too many entries for 32-bit offsets");
+        return MX_ERR_ARG;
+    }
+    std::vector<int> grpPtr(grp.begin(), grp.end());
+    // per block, the list of its non-empty groups
+    std::vector<int> listPtr((size_t)nBlocks + 1, 0), list;
+    for (int b = 0; b < nBlocks; ++b) {
+        for (int q = 0; q < nPanels; ++q) {
+            const int e0 = grpPtr[(size_t)b * nPanels + q], e1 = grpPtr[(size_t)b * nPanels + q + 1];
+            if (e1 > e0) {
+                list.push_back(q);
+                list.push_back(e0);
+                list.push_back(e1);
+                list.push_back(0);
+            }
+        }
+        while ((list.size() / 4 - (size_t)listPtr[b]) % depth) {  // pad with empty groups
+            list.push_back(0);
+            list.push_back(0);
+            list.push_back(0);
+            list.push_back(1);
+        }
+        listPtr[b + 1] = (int)(list.size() / 4);
+    }
+    std::vector<unsigned short> erow((size_t)total + 8, 0), ecol((size_t)total + 8, 0);
+    std::vector<unsigned char> ev(((size_t)total + 8) * es, 0);
+    const unsigned char *sv = (const unsigned char *)val;
+#pragma omp parallel
+    {
+        std::vector<int> cursor(nPanels);
+#pragma omp for schedule(dynamic, 4)
+        for (int b = 0; b < nBlocks; ++b) {
+            std::copy(grpPtr.begin() + (size_t)b * nPanels, grpPtr.begin() + (size_t)(b + 1) * nPanels, cursor.begin());
+            for (int r = blockRow[b]; r < blockRow[b + 1]; ++r)
+                for (int p = rowPtr[r]; p < rowPtr[r + 1]; ++p) {
+                    const int q = col[p] / PW;
+                    const int e = cursor[q]++;
+                    erow[e] = (unsigned short)(r - blockRow[b]);
+                    ecol[e] = (unsigned short)(col[p] - q * PW);
+                    std::memcpy(&ev[(size_t)e * es], sv + (size_t)p * es, es);
+                }
+        }
+    }
+    D.nBlocks = nBlocks;
+    D.nPanels = nPanels;
+    D.panelCols = PW;
+    D.maxBlockRows = 0;
+    for (int b = 0; b < nBlocks; ++b) D.maxBlockRows = std::max(D.maxBlockRows, blockRow[b + 1] - blockRow[b]);
+    D.entries = total;
+    int rc;
+    if ((rc = upload(&D.blockRow, blockRow.data(), blockRow.size()))) return rc;
+    if ((rc = upload(&D.listPtr, listPtr.data(), listPtr.size()))) return rc;
+    if ((rc = upload(&D.list, list.data(), list.size(), 16))) return rc;
+    if ((rc = upload(&D.erow, erow.data(), erow.size()))) return rc;
+    if ((rc = upload(&D.ecol, ecol.data(), ecol.size()))) return rc;
+    if ((rc = upload_bytes(&D.eval, ev.data(), ev.size()))) return rc;
+    return MX_OK;
+}
+
 int upload_csr(mx_dtype dtype, int rows, int nnz, const int *rowPtr, const int *col, const void *val,
                mx::DeviceCsr &A, double *pack_ms)
 {
@@ -126,7 +230,10 @@ int mx::csr_entries_per_lane(mx_dtype dtype)
 struct mx_plan {
     mx_dtype dtype = MX_F64;
     int rows = 0, cols = 0, nnz = 0;
-    mx::DeviceCsr csr;
+    mx::DeviceCsr csr;        // CSR part, row-tile form (csr_rows_kernel)
+    mx::DevicePanels panels;  // CSR part, LDS-staged-x form (csr_panel_kernel)
+    bool use_panels = false;  // which of the two runs
+    int csr_nnz = 0;
     mx::DeviceTiles tiles;
     int tile_nnz = 0;
     hipStream_t stream = nullptr;
@@ -147,11 +254,102 @@ extern "C" void mx_plan_destroy(mx_plan *plan)
 {
     if (!plan) return;
     free_csr(plan->csr);
+    free_panels(plan->panels);
     free_tiles(plan->tiles);
     if (plan->ev0) (void)hipEventDestroy(plan->ev0);
     if (plan->ev1) (void)hipEventDestroy(plan->ev1);
     if (plan->stream) (void)hipStreamDestroy(plan->stream);
     delete plan;
+}
+
+// Mean milliseconds per iteration of `body` over `iters` back-to-back runs after `warm`
+// untimed ones, by events on the stream the kernels run on.
+template <typename F>
+static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
+{
+    for (int i = 0; i < warm; ++i) {
+        int rc = body();
+        if (rc) return rc;
+    }
+    MX_HIP(hipStreamSynchronize(plan->stream));
+    MX_HIP(hipEventRecord(plan->ev0, plan->stream));
+    for (int i = 0; i < iters; ++i) {
+        int rc = body();
+        if (rc) return rc;
+    }
+    MX_HIP(hipEventRecord(plan->ev1, plan->stream));
+    MX_HIP(hipEventSynchronize(plan->ev1));
+    float t = 0.f;
+    MX_HIP(hipEventElapsedTime(&t, plan->ev0, plan->ev1));
+    *ms = (double)t / (double)std::max(iters, 1);
+    return MX_OK;
+}
+
+static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate, hipStream_t s)
+{
+    if (plan->use_panels)
+        MX_HIP(mx::launch_panels(plan->dtype, plan->panels, x, y, plan->cols, accumulate, s));
+    else
+        MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s));
+    return MX_OK;
+}
+
+// Puts the CSR part on the device.  Two executable forms exist (row tiles with direct x
+// gathers; column panels with x staged in LDS); unless a flag forces one, both are built,
+// timed on the spot with a few launches each, and the slower one is released.
+static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags)
+{
+    const int rows = plan->rows, cols = plan->cols;
+    const int nnz = rowPtr[rows];
+    plan->csr_nnz = nnz;
+    const char *env = std::getenv("MX_CSR_KERNEL");
+    bool want_rows = true, want_panels = true;
+    if (flags & MX_PLAN_CSR_ROWS) want_panels = false;
+    if (flags & MX_PLAN_CSR_PANELS) want_rows = false;
+    if (env && !std::strcmp(env, "rows")) want_rows = true, want_panels = false;
+    if (env && !std::strcmp(env, "panels")) want_rows = false, want_panels = true;
+    hipDeviceProp_t prop;
+    int dev = 0;
+    MX_HIP(hipGetDevice(&dev));
+    MX_HIP(hipGetDeviceProperties(&prop, dev));
+    const int nCU = std::max(1, prop.multiProcessorCount);
+    if (want_rows && want_panels) {
+        // every workgroup copies each panel it touches; do not even try when that sweep would
+        // dwarf the matrix itself
+        const double sweep = (double)std::max(nCU, rows / mx::panel_max_block_rows(plan->dtype)) * (double)cols *
+                             mx::elem_size(plan->dtype);
+        const double matrix = (double)nnz * (mx::elem_size(plan->dtype) + 4);
+        if (nnz < 4096 || sweep > 64.0 * matrix) want_panels = false;
+    }
+    if (!mx::panels_possible(plan->dtype, cols)) {  // shape the panel kernel cannot take: row tiles
+        want_panels = false;
+        want_rows = true;
+    }
+    int rc;
+    if (want_rows && (rc = upload_csr(plan->dtype, rows, nnz, rowPtr, col, val, plan->csr, nullptr))) return rc;
+    if (want_panels && (rc = upload_panels(plan->dtype, rows, cols, rowPtr, col, val, nCU, plan->panels))) return rc;
+    plan->use_panels = want_panels && !want_rows;
+    if (want_rows && want_panels) {
+        const size_t es = (size_t)mx::elem_size(plan->dtype);
+        void *tx = nullptr, *ty = nullptr;
+        if ((rc = upload_bytes(&tx, nullptr, 0, std::max<size_t>(cols * es, 16)))) return rc;
+        if ((rc = upload_bytes(&ty, nullptr, 0, std::max<size_t>(rows * es, 16)))) {
+            (void)hipFree(tx);
+            return rc;
+        }
+        double ms[2] = {0.0, 0.0};
+        for (int v = 0; v < 2 && !rc; ++v) {
+            plan->use_panels = v == 1;
+            rc = time_loop(plan, 3, 10, [&]() { return launch_csr_part(plan, tx, ty, 0, plan->stream); }, &ms[v]);
+        }
+        (void)hipFree(tx);
+        (void)hipFree(ty);
+        if (rc) return rc;
+        plan->use_panels = ms[1] < ms[0];
+        if (plan->use_panels) free_csr(plan->csr);
+        else free_panels(plan->panels);
+    }
+    return MX_OK;
 }
 
 // Minimum fill of a chunk's fragments for the MFMA tile kernel to take it (default plans).
@@ -183,10 +381,14 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
         mx_plan_destroy(plan);
         return code;
     };
+    if (hipStreamCreate(&plan->stream) != hipSuccess || hipEventCreate(&plan->ev0) != hipSuccess ||
+        hipEventCreate(&plan->ev1) != hipSuccess) {
+        set_error("mx_plan_create: could not create stream/events");
+        return fail(MX_ERR_DEVICE);
+    }
     try {
         if (!P->extracted) {
-            rc = upload_csr(P->dtype, rows, P->nnzCD, P->cdRowPtr.data(), P->cdColInd.data(), P->cdVal.data(), plan->csr,
-                            nullptr);
+            rc = setup_csr_part(plan, P->cdRowPtr.data(), P->cdColInd.data(), P->cdVal.data(), flags);
             if (rc) return fail(rc);
         } else {
             // residual column space -> the caller's column ids, so x needs no permutation
@@ -235,7 +437,7 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                     std::memcpy(&val[(size_t)q * es], ddv + (size_t)p * es, es);
                 }
             }
-            rc = upload_csr(P->dtype, rows, csrNnz, rowPtr.data(), col.data(), val.data(), plan->csr, nullptr);
+            rc = setup_csr_part(plan, rowPtr.data(), col.data(), val.data(), flags);
             if (rc) return fail(rc);
 
             // tile part: the selected chunks, re-packed contiguously
@@ -284,11 +486,6 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
         set_error("mx_plan_create: out of memory");
         return fail(MX_ERR_ALLOC);
     }
-    if (hipStreamCreate(&plan->stream) != hipSuccess || hipEventCreate(&plan->ev0) != hipSuccess ||
-        hipEventCreate(&plan->ev1) != hipSuccess) {
-        set_error("mx_plan_create: could not create stream/events");
-        return fail(MX_ERR_DEVICE);
-    }
     *out = plan;
     return MX_OK;
 }
@@ -309,10 +506,11 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     info->tile_chunks = plan->tiles.chunkNum;
     info->tile_frags = plan->tiles.frags;
     info->tile_nnz = plan->tile_nnz;
-    info->csr_nnz = plan->csr.nnz;
-    info->csr_blocks = plan->csr.nBlocks;
+    info->csr_nnz = plan->csr_nnz;
+    info->csr_blocks = plan->use_panels ? plan->panels.nBlocks : plan->csr.nBlocks;
+    info->csr_variant = plan->use_panels ? 1 : 0;
     // what each kernel has to move at least once: its arrays, x once, its y rows
-    info->csr_bytes = (double)plan->csr.nnz * (es + 4) + ((double)plan->rows + 1) * 4 + (double)plan->cols * es +
+    info->csr_bytes = (double)plan->csr_nnz * (es + 4) + ((double)plan->rows + 1) * 4 + (double)plan->cols * es +
                       (double)plan->rows * es;
     info->tile_bytes = plan->tiles.chunkNum
                            ? (double)plan->tiles.frags * (bitBytes + 4 + 4.0 * fragK) + (double)plan->tiles.vals * es +
@@ -323,7 +521,8 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
 
 static int spmv_on(mx_plan *plan, const void *x, void *y, hipStream_t s)
 {
-    MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, 0, s));
+    int rc = launch_csr_part(plan, x, y, 0, s);
+    if (rc) return rc;
     MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x, y, 1, s));
     return MX_OK;
 }
@@ -379,29 +578,6 @@ extern "C" int mx_spmv_host(mx_plan *plan, const void *x_host, void *y_host)
     return rc;
 }
 
-// Mean milliseconds per iteration of `body` over `iters` back-to-back runs after `warm`
-// untimed ones, by events on the stream the kernels run on.
-template <typename F>
-static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
-{
-    for (int i = 0; i < warm; ++i) {
-        int rc = body();
-        if (rc) return rc;
-    }
-    MX_HIP(hipStreamSynchronize(plan->stream));
-    MX_HIP(hipEventRecord(plan->ev0, plan->stream));
-    for (int i = 0; i < iters; ++i) {
-        int rc = body();
-        if (rc) return rc;
-    }
-    MX_HIP(hipEventRecord(plan->ev1, plan->stream));
-    MX_HIP(hipEventSynchronize(plan->ev1));
-    float t = 0.f;
-    MX_HIP(hipEventElapsedTime(&t, plan->ev0, plan->ev1));
-    *ms = (double)t / (double)std::max(iters, 1);
-    return MX_OK;
-}
-
 extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters, double *ms_total,
                        double *ms_tile, double *ms_csr)
 {
@@ -418,10 +594,7 @@ extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, 
         *ms_total = t;
     }
     if (ms_csr) {
-        rc = time_loop(plan, warm, iters, [&]() -> int {
-            MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x_dev, y_dev, 0, s));
-            return MX_OK;
-        }, &t);
+        rc = time_loop(plan, warm, iters, [&]() { return launch_csr_part(plan, x_dev, y_dev, 0, s); }, &t);
         if (rc) return rc;
         *ms_csr = t;
     }

@@ -72,13 +72,18 @@ TAUS = [(0.0, 0.0), (0.5, 0.25), (1.0, 1.0), (0.75, 0.0), (0.25, 0.25), (1.0, 0.
 
 
 @pytest.mark.parametrize("cfg,scale", CASES)
-@pytest.mark.parametrize("flags", ["default", "no_tiles", "all_tiles"])
+@pytest.mark.parametrize("flags", ["default", "no_tiles", "all_tiles", "all_tiles+csr_rows", "all_tiles+csr_panels",
+                                   "no_tiles+csr_panels"])
 def test_hybrid_spmv_matches_oracle(mx, ora, cfg, scale, flags):
     import torch
     A, x = mx.gen_config(cfg, scale=scale)
     ref = oracle_y(ora, mx, A, x)
     tol = F64_TOL if A.dtype == mx.MX_F64 else F16_TOL
-    fl = {"default": mx.MX_PLAN_DEFAULT, "no_tiles": mx.MX_PLAN_NO_TILES, "all_tiles": mx.MX_PLAN_ALL_TILES}[flags]
+    bits = {"default": mx.MX_PLAN_DEFAULT, "no_tiles": mx.MX_PLAN_NO_TILES, "all_tiles": mx.MX_PLAN_ALL_TILES,
+            "csr_rows": mx.MX_PLAN_CSR_ROWS, "csr_panels": mx.MX_PLAN_CSR_PANELS}
+    fl = 0
+    for name in flags.split("+"):
+        fl |= bits[name]
     xd = torch.from_numpy(x).cuda()
     for tau in TAUS:
         print("case workload=%d scale=%g flags=%s tau=%s" % (cfg, scale, flags, tau), flush=True)
@@ -115,7 +120,8 @@ def test_full_size_workloads_match_oracle(mx, ora, cfg, taus):
     tol = F64_TOL if A.dtype == mx.MX_F64 else F16_TOL
     xd = torch.from_numpy(x).cuda()
     for tau in taus:
-        for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES):
+        for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_ROWS,
+                   mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_PANELS):
             print("full-size workload=%d tau=%s flags=%d" % (cfg, tau, fl), flush=True)
             part = mx.Partition(A, *tau)
             plan = mx.Plan(part, fl)
