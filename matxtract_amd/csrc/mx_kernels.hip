@@ -460,113 +460,233 @@ __global__ __launch_bounds__(kPanelThreads) void csr_panel_kernel(const int *__r
 }
 
 // ---- tile part --------------------------------------------------------------------------
-// One wave per 8-row chunk, 4 chunks per workgroup.
+// A wave works on U 8-row chunks at once, 4 waves per workgroup.  The address unit spends
+// about 16 cycles on every wave-level load whatever the number of active lanes, so all
+// global loads are "one lane, one element": a step's bitmaps and value pointers in one load,
+// its 64 column ids in one, the 64 x values they name in one gather, and its packed values as
+// one contiguous run.  They are parked in the wave's own LDS region, and every lane then
+// picks what the MFMA operand layout asks of it with LDS reads.  The loads of all U chunks are
+// issued before any is used.  The host lays the values out so that the run of every step
+// starts on a 16-byte boundary (fragPtr holds those padded offsets).
 //
 // v_mfma_f64_16x16x4_f64 operand layout (wave64): lane L holds A[L%16][L/16] and
-// B[L/16][L%16]; accumulator register g of lane L holds D[4*g + L/16][L%16].  A step feeds two
-// fragments: A rows 0..7 = fragment f, rows 8..15 = fragment f+1; B column 0 = the 4 gathered
-// x of fragment f, column 1 = those of fragment f+1, other columns 0.  The chunk's result is
-// D[0..7][0] + D[8..15][1], accumulated across all steps inside the matrix core, so no
-// cross-lane reduction is needed until the single combine at the end.
+// B[L/16][L%16]; accumulator register g of lane L holds D[4*g + L/16][L%16].  One MFMA feeds
+// two 8x4 fragments: A rows 0..7 = fragment f, rows 8..15 = fragment f+1; B column 0 = the 4
+// gathered x of fragment f, column 1 = those of fragment f+1, other columns 0.  The chunk's
+// result is D[0..7][0] + D[8..15][1], accumulated across all steps inside the matrix core, so
+// there is no cross-lane reduction until the single combine at the end.  A step is 16
+// fragments = 8 MFMAs.
+constexpr int kTileStepF64 = 16, kTileStepF16 = 8;  // fragments per step
+constexpr int kTileUF64 = 2, kTileUF16 = 4;         // chunks in flight per wave
+
 __global__ __launch_bounds__(kBlock) void tile_f64_kernel(const int *__restrict__ chunkPtr, const int *__restrict__ fragPtr,
                                                          const uint32_t *__restrict__ fragBit,
                                                          const double *__restrict__ tcVal, const int *__restrict__ atox,
                                                          const int *__restrict__ rowIdx, const double *__restrict__ x,
                                                          double *__restrict__ y, int chunkNum, int dRows, int accumulate)
 {
-    const int lane = threadIdx.x & 63;
-    const int w = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-    if (w >= chunkNum) return;
-    const int f0 = chunkPtr[w], f1 = chunkPtr[w + 1];
+    constexpr int U = kTileUF64, SF = kTileStepF64;
+    struct Unit {
+        unsigned hdr[64];  // [0,16) bitmaps, [16,33) value offsets of the step's fragments
+        double xv[64];     // x of the step's 16*4 columns
+        double val[512];   // the step's packed values
+    };
+    __shared__ Unit lds[kBlock / 64][U];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int w0 = (blockIdx.x * (kBlock / 64) + wave) * U;
+    if (w0 >= chunkNum) return;
     const int m = lane & 15, k = lane >> 4;
-    const int t = m >> 3;                // which of the step's two fragments this lane decodes
+    const int t = m >> 3;                // which of an MFMA's two fragments this lane decodes
     const int bitpos = (m & 7) * 4 + k;  // (local row, local column) -> bitmap bit
-    v4f64 acc = {0.0, 0.0, 0.0, 0.0};
-    for (int f = f0; f < f1; f += 2) {
-        const int fa = f + t;
-        double a = 0.0;
-        if (fa < f1) {
-            const uint32_t bm = fragBit[fa];
-            if ((bm >> bitpos) & 1u) a = tcVal[fragPtr[fa] + __popc(bm & ((1u << bitpos) - 1u))];
-        }
-        double bv = 0.0;
-        if (m < 2 && f + m < f1) bv = x[atox[(f + m) * 4 + k]];
-        acc = __builtin_amdgcn_mfma_f64_16x16x4f64(a, bv, acc, 0, 0, 0);
-    }
-    // row q and row q+4 of the chunk end up in lane 16q: D[q][0] = reg 0, D[q+4][0] = reg 1 there,
-    // D[8+q][1] = reg 2 and D[12+q][1] = reg 3 of lane 16q+1.
-    const double o0 = acc[0] + __shfl_down(acc[2], 1, 64);
-    const double o1 = acc[1] + __shfl_down(acc[3], 1, 64);
-    if ((lane & 15) == 0) {
-        const int q = lane >> 4;
+
+    // chunk bounds: lanes 0..U hold chunkPtr[w0 + lane]
+    const int cp = chunkPtr[min(w0 + lane, chunkNum)];
+    int f0[U], f1[U], steps = 0;
+    // output rows: lane r < 8 holds row r of each chunk and its old y
+    int row[U];
+    double yold[U];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int local = w * 8 + q + 4 * h;
-            if (local < dRows) {
-                const int row = rowIdx ? rowIdx[local] : local;
-                const double o = h ? o1 : o0;
-                y[row] = accumulate ? y[row] + o : o;
+    for (int u = 0; u < U; ++u) {
+        f0[u] = __builtin_amdgcn_readlane(cp, u);
+        f1[u] = w0 + u < chunkNum ? __builtin_amdgcn_readlane(cp, u + 1) : f0[u];
+        steps = max(steps, (f1[u] - f0[u] + SF - 1) / SF);
+        const int local = (w0 + u) * 8 + lane;
+        row[u] = (lane < 8 && w0 + u < chunkNum && local < dRows) ? (rowIdx ? rowIdx[local] : local) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) yold[u] = (accumulate && row[u] >= 0) ? y[row[u]] : 0.0;
+
+    v4f64 acc[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc[u] = v4f64{0.0, 0.0, 0.0, 0.0};
+    for (int s = 0; s < steps; ++s) {
+        unsigned hdr[U];
+        int ax[U], nf[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int fs = f0[u] + s * SF;
+            nf[u] = max(0, min(SF, f1[u] - fs));
+            const unsigned *hp = lane < 16 ? fragBit + fs + lane : (const unsigned *)fragPtr + fs + (lane - 16);
+            hdr[u] = (lane < 16 ? lane < nf[u] : (lane - 16 <= nf[u] && nf[u] > 0)) ? *hp : 0u;
+            ax[u] = lane < 4 * nf[u] ? atox[fs * 4 + lane] : -1;
+        }
+        double xg[U];
+        v2f64 vv[U][4];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            xg[u] = ax[u] >= 0 ? x[ax[u]] : 0.0;
+            const int vb = __builtin_amdgcn_readlane((int)hdr[u], 16);
+            const int ve = __builtin_amdgcn_readlane((int)hdr[u], 16 + nf[u]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int o = vb + q * 128 + lane * 2;
+                vv[u][q] = o < ve ? __builtin_nontemporal_load((const v2f64 *)(tcVal + o)) : v2f64{0.0, 0.0};
             }
         }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            Unit &L = lds[wave][u];
+            L.hdr[lane] = hdr[u];
+            L.xv[lane] = xg[u];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *(v2f64 *)(L.val + q * 128 + lane * 2) = vv[u][q];
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const Unit &L = lds[wave][u];
+            const int vb = (int)L.hdr[16];
+#pragma unroll
+            for (int j = 0; j < SF / 2; ++j) {
+                const unsigned bm = L.hdr[2 * j + t];
+                const int fp = (int)L.hdr[16 + 2 * j + t] - vb;
+                const double a = ((bm >> bitpos) & 1u) ? L.val[fp + __popc(bm & ((1u << bitpos) - 1u))] : 0.0;
+                const double bv = m < 2 ? L.xv[(2 * j + m) * 4 + k] : 0.0;
+                acc[u] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, bv, acc[u], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    // row q and row q+4 of a chunk end up in lane 16q: D[q][0] = reg 0, D[q+4][0] = reg 1 there,
+    // D[8+q][1] = reg 2 and D[12+q][1] = reg 3 of lane 16q+1.  Hand them to lanes 0..7 through LDS.
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const double o0 = acc[u][0] + __shfl_down(acc[u][2], 1, 64);
+        const double o1 = acc[u][1] + __shfl_down(acc[u][3], 1, 64);
+        double *out = lds[wave][u].xv;
+        if ((lane & 15) == 0) {
+            out[lane >> 4] = o0;
+            out[(lane >> 4) + 4] = o1;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (row[u] >= 0) y[row[u]] = yold[u] + out[lane];
     }
 }
 
 // v_mfma_f32_16x16x32_f16 operand layout (wave64): lane L holds A[L%16][8*(L/16) .. +7],
-// B[8*(L/16) .. +7][L%16]; accumulator register g of lane L holds D[4*(L/16)+g][L%16].  A step feeds eight 8x8 fragments of the
-// chunk: A rows 0..7 = fragments f..f+3 side by side along K, rows 8..15 = fragments f+4..f+7;
-// B column 0 = the 32 gathered x of f..f+3, column 1 = those of f+4..f+7.  A lane's eight A
-// elements are one byte of its fragment's 64-bit bitmap (one tile row), whose values sit
-// consecutively in tcVal.
+// B[8*(L/16) .. +7][L%16]; accumulator register g of lane L holds D[4*(L/16)+g][L%16].  One MFMA
+// (= one step) feeds eight 8x8 fragments of the chunk: A rows 0..7 = fragments f..f+3 side by
+// side along K, rows 8..15 = fragments f+4..f+7; B column 0 = the 32 gathered x of f..f+3,
+// column 1 = those of f+4..f+7.  A lane's eight A elements are one byte of its fragment's
+// 64-bit bitmap (one tile row), whose values sit consecutively in the step's run in LDS; bit j
+// reads the element at the popcount of the lower bits.
 __global__ __launch_bounds__(kBlock) void tile_f16_kernel(const int *__restrict__ chunkPtr, const int *__restrict__ fragPtr,
                                                          const uint64_t *__restrict__ fragBit,
                                                          const _Float16 *__restrict__ tcVal, const int *__restrict__ atox,
                                                          const int *__restrict__ rowIdx, const _Float16 *__restrict__ x,
                                                          _Float16 *__restrict__ y, int chunkNum, int dRows, int accumulate)
 {
-    const int lane = threadIdx.x & 63;
-    const int w = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-    if (w >= chunkNum) return;
-    const int f0 = chunkPtr[w], f1 = chunkPtr[w + 1];
+    constexpr int U = kTileUF16, SF = kTileStepF16;
+    struct Unit {
+        unsigned hdr[32];    // [0,16) the 8 bitmaps as dwords, [16,25) value offsets
+        _Float16 xv[64];     // x of the step's 8*8 columns
+        unsigned val[264];   // the step's packed values (512 halves) + slack
+    };
+    __shared__ __attribute__((aligned(16))) Unit lds[kBlock / 64][U];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int w0 = (blockIdx.x * (kBlock / 64) + wave) * U;
+    if (w0 >= chunkNum) return;
     const int m = lane & 15, g = lane >> 4;
     const int r = m & 7;
-    v4f32 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int f = f0; f < f1; f += 8) {
-        const int fa = f + 4 * (m >> 3) + g;
-        v8f16 a = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (fa < f1) {
-            const uint64_t bm = fragBit[fa];
-            const unsigned byte = (unsigned)(bm >> (8 * r)) & 0xffu;
-            if (byte) {
-                const _Float16 *v = tcVal + fragPtr[fa] + __popcll(bm & ((1ull << (8 * r)) - 1ull));
-                int used = 0;
+
+    const int cp = chunkPtr[min(w0 + lane, chunkNum)];
+    int f0[U], f1[U], steps = 0;
+    int row[U];
+    float yold[U];
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if ((byte >> j) & 1u) a[j] = v[used++];
-            }
-        }
-        v8f16 bv = {0, 0, 0, 0, 0, 0, 0, 0};
-        const int fb = f + 4 * m + g;
-        if (m < 2 && fb < f1) {
-            const int4 i0 = *(const int4 *)(atox + fb * 8);
-            const int4 i1 = *(const int4 *)(atox + fb * 8 + 4);
-            bv[0] = x[i0.x]; bv[1] = x[i0.y]; bv[2] = x[i0.z]; bv[3] = x[i0.w];
-            bv[4] = x[i1.x]; bv[5] = x[i1.y]; bv[6] = x[i1.z]; bv[7] = x[i1.w];
-        }
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bv, acc, 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+        f0[u] = __builtin_amdgcn_readlane(cp, u);
+        f1[u] = w0 + u < chunkNum ? __builtin_amdgcn_readlane(cp, u + 1) : f0[u];
+        steps = max(steps, (f1[u] - f0[u] + SF - 1) / SF);
+        const int local = (w0 + u) * 8 + lane;
+        row[u] = (lane < 8 && w0 + u < chunkNum && local < dRows) ? (rowIdx ? rowIdx[local] : local) : -1;
     }
-    float o[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = acc[i] + __shfl(acc[i], lane + 33, 64);
-    if (lane == 0 || lane == 16) {
+    for (int u = 0; u < U; ++u) yold[u] = (accumulate && row[u] >= 0) ? (float)y[row[u]] : 0.f;
+
+    v4f32 acc[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc[u] = v4f32{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < steps; ++s) {
+        unsigned hdr[U];
+        int ax[U], nf[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int fs = f0[u] + s * SF;
+            nf[u] = max(0, min(SF, f1[u] - fs));
+            const unsigned *hp = lane < 16 ? (const unsigned *)fragBit + 2 * fs + lane : (const unsigned *)fragPtr + fs + (lane - 16);
+            hdr[u] = (lane < 16 ? lane < 2 * nf[u] : (lane - 16 <= nf[u] && nf[u] > 0 && lane < 32)) ? *hp : 0u;
+            ax[u] = lane < 8 * nf[u] ? atox[fs * 8 + lane] : -1;
+        }
+        _Float16 xg[U];
+        v4i32 vv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            xg[u] = ax[u] >= 0 ? x[ax[u]] : (_Float16)0;
+            const int vb = __builtin_amdgcn_readlane((int)hdr[u], 16);
+            const int ve = __builtin_amdgcn_readlane((int)hdr[u], 16 + nf[u]);
+            const int o = vb + lane * 8;
+            vv[u] = o < ve ? __builtin_nontemporal_load((const v4i32 *)(tcVal + o)) : v4i32{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            Unit &L = lds[wave][u];
+            if (lane < 32) L.hdr[lane] = hdr[u];
+            L.xv[lane] = xg[u];
+            *(v4i32 *)(L.val + lane * 4) = vv[u];
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const Unit &L = lds[wave][u];
+            const int fa = 4 * (m >> 3) + g;  // this lane's fragment within the step
+            const unsigned lo = L.hdr[2 * fa], hi = L.hdr[2 * fa + 1];
+            const uint64_t bm = ((uint64_t)hi << 32) | lo;
+            const unsigned byte = (unsigned)(bm >> (8 * r)) & 0xffu;
+            const int v0 = (int)L.hdr[16 + fa] - (int)L.hdr[16] + __popcll(bm & ((1ull << (8 * r)) - 1ull));
+            // bit j of the byte takes the next value of the run: its index is v0 + popcount of the lower bits
+            const _Float16 *run = (const _Float16 *)L.val + v0;
+            v8f16 a;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                a[j] = ((byte >> j) & 1u) ? run[__popc(byte & ((1u << j) - 1u))] : (_Float16)0;
+            v8f16 bv = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (m < 2) bv = *(const v8f16 *)(L.xv + (4 * m + g) * 8);
+            acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bv, acc[u], 0, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    // rows 0..3 of a chunk: lane 0 (+ lane 33), rows 4..7: lane 16 (+ lane 49); to lanes 0..7 through LDS
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        float *out = (float *)lds[wave][u].val;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int local = w * 8 + (lane >> 2) + i;
-            if (local < dRows) {
-                const int row = rowIdx ? rowIdx[local] : local;
-                const float s = accumulate ? (float)y[row] + o[i] : o[i];
-                y[row] = (_Float16)s;
-            }
+            const float o = acc[u][i] + __shfl(acc[u][i], lane + 33, 64);
+            if (lane == 0 || lane == 16) out[(lane >> 2) + i] = o;
         }
+        __builtin_amdgcn_wave_barrier();
+        if (row[u] >= 0) y[row[u]] = (_Float16)(yold[u] + out[lane]);
     }
 }
 
@@ -649,7 +769,8 @@ hipError_t launch_panels(mx_dtype dtype, const DevicePanels &P, const void *x, v
 hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s)
 {
     if (T.chunkNum <= 0) return hipSuccess;
-    const int grid = (T.chunkNum + 3) / 4;
+    const int perBlock = 4 * (dtype == MX_F64 ? mxk::kTileUF64 : mxk::kTileUF16);  // chunks per workgroup
+    const int grid = (T.chunkNum + perBlock - 1) / perBlock;
     if (dtype == MX_F64)
         hipLaunchKernelGGL(mxk::tile_f64_kernel, dim3(grid), dim3(mxk::kBlock), 0, s, T.chunkPtr, T.fragPtr,
                            (const uint32_t *)T.fragBit, (const double *)T.tcVal, T.atox, T.rowIdx, (const double *)x,

@@ -195,6 +195,70 @@ int upload_panels(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
     return MX_OK;
 }
 
+// Puts bitmap tiles on the device for the tile kernels: the chunks named by `sel` (all when
+// null), re-packed contiguously.  Column ids go through `colMap` and output rows through
+// `rowMap` when given.  Values keep their order, but the run of every kernel step (8 fragments
+// for binary16, 16 for binary64, counted from the chunk's first fragment) is moved up to a
+// 16-byte boundary, and the device fragPtr holds those padded offsets.
+int upload_tiles(mx_dtype dtype, int chunkNum, const char *sel, int dRows, const int *chunkPtr, const int *fragPtr,
+                 const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap,
+                 mx::DeviceTiles &T, int *tile_nnz)
+{
+    const int es = mx::elem_size(dtype), fragK = mx::frag_k(dtype), fragM = mx::kFragM;
+    const int bitBytes = dtype == MX_F64 ? 4 : 8;
+    const int stepFrags = dtype == MX_F64 ? 16 : 8, align = 16 / es;
+    std::vector<int> dChunkPtr(1, 0), dFragPtr, dAtox, rowIdx;
+    std::vector<unsigned char> dBits, dVal;
+    const unsigned char *bits = (const unsigned char *)fragBit, *tv = (const unsigned char *)tcVal;
+    int nsel = 0, nnz = 0;
+    size_t voff = 0;  // in elements
+    for (int w = 0; w < chunkNum; ++w) {
+        if (sel && !sel[w]) continue;
+        ++nsel;
+        const int f0 = chunkPtr[w], f1 = chunkPtr[w + 1];
+        for (int f = f0; f < f1; ++f) {
+            if ((f - f0) % stepFrags == 0) voff = (voff + align - 1) / align * align;
+            dFragPtr.push_back((int)voff);
+            const int cnt = fragPtr[f + 1] - fragPtr[f];
+            dVal.resize((voff + cnt) * es, 0);
+            if (cnt) std::memcpy(&dVal[voff * es], tv + (size_t)fragPtr[f] * es, (size_t)cnt * es);
+            voff += cnt;
+            nnz += cnt;
+            for (int k = 0; k < fragK; ++k) {
+                const int c = atox[(size_t)f * fragK + k];
+                dAtox.push_back(colMap ? colMap[c] : c);
+            }
+        }
+        dBits.insert(dBits.end(), bits + (size_t)f0 * bitBytes, bits + (size_t)f1 * bitBytes);
+        dChunkPtr.push_back(dChunkPtr.back() + (f1 - f0));
+        for (int i = 0; i < fragM; ++i) {
+            const int local = w * fragM + i;
+            rowIdx.push_back(local < dRows ? (rowMap ? rowMap[local] : local) : -1);
+        }
+        if (voff > 2000000000u) {
+            set_error("tile layout: too many values for 32-bit offsets");
+            return MX_ERR_ARG;
+        }
+    }
+    dFragPtr.push_back((int)voff);
+    T.chunkNum = nsel;
+    T.frags = dChunkPtr.back();
+    T.vals = nnz;
+    // ragged last chunk: rows past dRows carry -1 and are cut off through dRows
+    T.dRows = nsel * fragM;
+    while (T.dRows > 0 && rowIdx[T.dRows - 1] < 0) --T.dRows;
+    if (tile_nnz) *tile_nnz = nnz;
+    if (nsel == 0) return MX_OK;
+    int rc;
+    if ((rc = upload(&T.chunkPtr, dChunkPtr.data(), dChunkPtr.size(), 64))) return rc;
+    if ((rc = upload(&T.fragPtr, dFragPtr.data(), dFragPtr.size(), 64))) return rc;
+    if ((rc = upload_bytes(&T.fragBit, dBits.data(), dBits.size(), 256))) return rc;
+    if ((rc = upload_bytes(&T.tcVal, dVal.data(), dVal.size(), 8192))) return rc;
+    if ((rc = upload(&T.atox, dAtox.data(), dAtox.size(), 64))) return rc;
+    if ((rc = upload(&T.rowIdx, rowIdx.data(), rowIdx.size(), 64))) return rc;
+    return MX_OK;
+}
+
 int upload_csr(mx_dtype dtype, int rows, int nnz, const int *rowPtr, const int *col, const void *val,
                mx::DeviceCsr &A, double *pack_ms)
 {
@@ -440,47 +504,12 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             rc = setup_csr_part(plan, rowPtr.data(), col.data(), val.data(), flags);
             if (rc) return fail(rc);
 
-            // tile part: the selected chunks, re-packed contiguously
-            int nsel = 0;
-            for (int w = 0; w < chunkNum; ++w) nsel += sel[w];
-            if (nsel > 0) {
-                std::vector<int> chunkPtr(1, 0), fragPtr(1, 0), atox, rowIdx;
-                std::vector<unsigned char> fragBit, tcVal;
-                const int bitBytes = P->dtype == MX_F64 ? 4 : 8;
-                const unsigned char *bits = P->dtype == MX_F64 ? (const unsigned char *)P->fragBit32.data()
-                                                               : (const unsigned char *)P->fragBit64.data();
-                const unsigned char *tv = (const unsigned char *)P->tcVal.data();
-                for (int w = 0; w < chunkNum; ++w) {
-                    if (!sel[w]) continue;
-                    const int f0 = P->chunkPtr[w], f1 = P->chunkPtr[w + 1];
-                    for (int f = f0; f < f1; ++f) {
-                        fragPtr.push_back(fragPtr.back() + (P->fragPtr[f + 1] - P->fragPtr[f]));
-                        for (int k = 0; k < fragK; ++k)
-                            atox.push_back(P->descColId[P->sparse_AToX_index[(size_t)f * fragK + k]]);
-                    }
-                    fragBit.insert(fragBit.end(), bits + (size_t)f0 * bitBytes, bits + (size_t)f1 * bitBytes);
-                    tcVal.insert(tcVal.end(), tv + (size_t)P->fragPtr[f0] * es, tv + (size_t)P->fragPtr[f1] * es);
-                    chunkPtr.push_back(chunkPtr.back() + (f1 - f0));
-                    for (int i = 0; i < fragM; ++i) {
-                        const int local = w * fragM + i;
-                        rowIdx.push_back(local < P->dRows ? P->rId[local] : -1);
-                    }
-                }
-                mx::DeviceTiles &T = plan->tiles;
-                T.chunkNum = nsel;
-                T.frags = chunkPtr.back();
-                T.vals = fragPtr.back();
-                // ragged last chunk: rows past dRows carry -1 and are skipped through dRows
-                T.dRows = nsel * fragM;
-                while (T.dRows > 0 && rowIdx[T.dRows - 1] < 0) --T.dRows;
-                plan->tile_nnz = T.vals;
-                if ((rc = upload(&T.chunkPtr, chunkPtr.data(), chunkPtr.size()))) return fail(rc);
-                if ((rc = upload(&T.fragPtr, fragPtr.data(), fragPtr.size()))) return fail(rc);
-                if ((rc = upload_bytes(&T.fragBit, fragBit.data(), fragBit.size()))) return fail(rc);
-                if ((rc = upload_bytes(&T.tcVal, tcVal.data(), tcVal.size(), 64))) return fail(rc);
-                if ((rc = upload(&T.atox, atox.data(), atox.size(), 16))) return fail(rc);
-                if ((rc = upload(&T.rowIdx, rowIdx.data(), rowIdx.size()))) return fail(rc);
-            }
+            // tile part: the selected chunks; columns and rows back in the caller's numbering
+            rc = upload_tiles(P->dtype, chunkNum, sel.data(), P->dRows, P->chunkPtr.data(), P->fragPtr.data(),
+                              P->dtype == MX_F64 ? (const void *)P->fragBit32.data() : (const void *)P->fragBit64.data(),
+                              P->tcVal.data(), P->sparse_AToX_index.data(), P->descColId.data(), P->rId.data(),
+                              plan->tiles, &plan->tile_nnz);
+            if (rc) return fail(rc);
         }
     } catch (const std::bad_alloc &) {
         set_error("mx_plan_create: out of memory");
@@ -702,7 +731,7 @@ static int du_any(mx_dtype dtype, const int *chunkPtr, const int *fragPtr, const
     int rc = need_device();
     if (rc) return rc;
     const int fragK = mx::frag_k(dtype), fragM = mx::kFragM;
-    const size_t es = (size_t)mx::elem_size(dtype), bitBytes = dtype == MX_F64 ? 4 : 8;
+    const size_t es = (size_t)mx::elem_size(dtype);
     const int chunkNum = (dRows + fragM - 1) / fragM;
     const int frags = chunkPtr[chunkNum];
     const int vals = fragPtr[frags];
@@ -721,15 +750,10 @@ static int du_any(mx_dtype dtype, const int *chunkPtr, const int *fragPtr, const
     void *dx = nullptr, *dy = nullptr, *dscratch = nullptr;
     auto body = [&]() -> int {
         int r;
-        T.chunkNum = chunkNum;
+        if ((r = upload_tiles(dtype, chunkNum, nullptr, dRows, chunkPtr, fragPtr, fragBit, tcVal, atox, nullptr, nullptr, T,
+                              nullptr)))
+            return r;
         T.dRows = dRows;
-        T.frags = frags;
-        T.vals = vals;
-        if ((r = upload(&T.chunkPtr, chunkPtr, (size_t)chunkNum + 1))) return r;
-        if ((r = upload(&T.fragPtr, fragPtr, (size_t)frags + 1))) return r;
-        if ((r = upload_bytes(&T.fragBit, fragBit, frags * bitBytes))) return r;
-        if ((r = upload_bytes(&T.tcVal, tcVal, vals * es, 64))) return r;
-        if ((r = upload(&T.atox, atox, (size_t)frags * fragK, 16))) return r;
         if ((r = upload_bytes(&dx, x_d, dCols * es))) return r;
         // FP64 uploads the caller's y and adds to it; FP16 starts from zero
         // (du_tcSpMV_fp64.cu:296-297 vs du_tcSpMV_fp16_v2.cu:146-147)
