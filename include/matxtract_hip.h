@@ -139,7 +139,7 @@ double mx_algorithmic_bytes(mx_dtype dtype, int rows, int cols, int nnz);
 #define MX_PLAN_NO_TILES 1   /* run the extracted block A_dd through the CSR kernel too */
 #define MX_PLAN_ALL_TILES 2  /* run every extracted chunk through the MFMA tile kernel */
 #define MX_PLAN_CSR_ROWS 4   /* CSR part: force the row-tile kernel (direct x gathers) */
-#define MX_PLAN_CSR_PANELS 8 /* CSR part: force the column-panel kernel (x staged in LDS) */
+#define MX_PLAN_CSR_SLICES 8 /* CSR part: prefer the column-slice kernel (x resident in LDS) when the matrix suits it */
 
 /* Uploads a partition once and keeps it on the device: the persistent counterpart of the
  * per-call cudaMalloc/cudaMemcpy blocks in cdspmv (src/spmv_kernel/cdSpMV.cu:407-418) and
@@ -181,7 +181,7 @@ typedef struct mx_plan_info {
     int tile_nnz;        /* matrix entries held in those fragments */
     int csr_nnz;         /* entries executed by the CSR kernel */
     int csr_blocks;      /* workgroups of the CSR kernel */
-    int csr_variant;     /* 0 = row tiles (csr_rows_kernel), 1 = column panels (csr_panel_kernel) */
+    int csr_variant;     /* 0 = row tiles (csr_rows_kernel), 1 = column slices (csr_slice_kernel) */
     double tile_bytes;   /* bytes the tile kernel must read+write per launch */
     double csr_bytes;    /* bytes the CSR kernel must read+write per launch */
 } mx_plan_info;

@@ -10,13 +10,13 @@ import ctypes as C
 import numpy as np
 
 from . import _lib
-from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_PANELS, MX_PLAN_CSR_ROWS, MX_PLAN_DEFAULT,
+from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLAN_CSR_ROWS, MX_PLAN_DEFAULT,
                    MX_PLAN_NO_TILES, MxError, check)
 
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
-           "MX_PLAN_CSR_PANELS"]
+           "MX_PLAN_CSR_SLICES"]
 
 
 def _p(a):

@@ -36,34 +36,28 @@ struct DeviceTiles {
     int *rowIdx = nullptr;    // [dRows] output row of each tile row; nullptr = identity
 };
 
-// The CSR part re-laid for LDS-staged x: rows cut into blocks (one workgroup each), columns
-// into panels of kPanelBytes of x; the entries of every (block, panel) group are contiguous and
-// carry 16-bit row and column offsets inside their block / panel.
-struct DevicePanels {
-    int nBlocks = 0, nPanels = 0, panelCols = 0, maxBlockRows = 0;
-    long long entries = 0;             // stored entries including the zero padding of groups
-    int *blockRow = nullptr;           // [nBlocks+1]
-    int *listPtr = nullptr;            // [nBlocks+1] range of each block's groups in `list`
-    int *list = nullptr;               // [groups][4] {panel, first entry, end entry, 0}; entry offsets are multiples of 8
-    unsigned short *erow = nullptr;    // [entries] row - blockRow[b]
-    unsigned short *ecol = nullptr;    // [entries] col - panel*panelCols
-    void *eval = nullptr;              // [entries]
+// The CSR part re-laid for x resident in LDS: columns cut into S slices of kSliceBytes of x,
+// rows into groups; workgroup (group, slice) handles its rows in sub-blocks whose accumulators
+// fit LDS.  Entries carry 16-bit row offsets inside their sub-block and column offsets inside
+// their slice; the entries of each (workgroup, sub-block) are contiguous, row-major, padded
+// with zero entries to a multiple of 8.
+struct DeviceSlices {
+    int nWG = 0, S = 0, rows = 0, cols = 0, maxSubRows = 0;
+    long long entries = 0;
+    int *wgSubPtr = nullptr;         // [nWG+1] range of each workgroup's sub-blocks in `subs`
+    int *subs = nullptr;             // [subBlocks][4] {first row, rows, first entry, end entry}
+    unsigned short *erow = nullptr;  // [entries] row - sub-block's first row
+    unsigned short *ecol = nullptr;  // [entries] col - slice * slice_cols
+    void *eval = nullptr;            // [entries]
+    void *partial = nullptr;         // [S][rows] accumulators (only when S > 1)
 };
-constexpr int kPanelBytes = 65536;     // one panel of x held in LDS
-constexpr int kPanelThreads = 1024;    // one workgroup per CU
-constexpr int kPanelListMax = 512;     // most panels one matrix may have for the panel kernel
-constexpr int kPanelListPad = 6;       // a block's group list is padded to a multiple of this (the entry ring depth)
-// The panel kernel copies x in 16-byte vectors: the column count must be a whole number of them.
-inline bool panels_possible(mx_dtype d, int cols)
-{
-    const int epv = d == MX_F64 ? 2 : 8, pw = kPanelBytes / (d == MX_F64 ? 8 : 2);
-    return cols >= epv && cols % epv == 0 && (cols + pw - 1) / pw <= kPanelListMax;
-}
-inline int panel_cols(mx_dtype d) { return kPanelBytes / (d == MX_F64 ? 8 : 2); }
-inline int panel_max_block_rows(mx_dtype d) { return d == MX_F64 ? 4096 : 16384; }  // LDS accumulators
+constexpr int kSliceBytes = 131072;   // the slice of x a workgroup keeps in LDS
+constexpr int kSliceThreads = 1024;   // one workgroup per CU
+constexpr int kSliceAccBytes = 24576; // LDS left for the row accumulators of a sub-block
+inline int slice_cols(mx_dtype d) { return kSliceBytes / (d == MX_F64 ? 8 : 2); }
+inline int slice_sub_rows(mx_dtype d) { return kSliceAccBytes / (d == MX_F64 ? 8 : 4); }
 
-hipError_t launch_panels(mx_dtype dtype, const DevicePanels &P, const void *x, void *y, int cols, int accumulate,
-                         hipStream_t s);
+hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s);
 hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s);
 hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s);
 hipError_t launch_probe_f64(const double *A, const double *B, double *D, hipStream_t s);

@@ -11,8 +11,8 @@
 // kernel, so there are no atomics anywhere; the tile kernel runs after the CSR kernel on the
 // same stream and adds its rows on top with a plain read-modify-write.
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <cstdlib>
-#include <type_traits>
 
 #include "mx_device.h"
 
@@ -26,9 +26,8 @@ typedef double v2f64 __attribute__((ext_vector_type(2)));
 typedef int v2i32 __attribute__((ext_vector_type(2)));
 
 constexpr int kBlock = 256;  // 4 wave64 per workgroup
-using mx::kPanelBytes;
-using mx::kPanelThreads;
-using mx::kPanelListMax;
+using mx::kSliceBytes;
+using mx::kSliceThreads;
 
 // Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
 // Re-map so that every XCD walks one contiguous range of logical blocks: neighbouring rows
@@ -94,8 +93,8 @@ struct Acc<_Float16> {
 };
 
 // One wave's share of a tile: 64*NPT consecutive entries starting at the 16-byte aligned
-// position `pos` (wave-uniform).  Indices and values are streamed with 128-bit loads (lane l
-// gets entries 4l..4l+3 of each 256-entry group), then transposed through the wave's own LDS
+// position `pos` (wave-uniform).  Indices and values are streamed with 128-bit loads into the
+// wave's own LDS region (in entry order), then read back transposed
 // region so that in every x gather lane l holds entry 64j+l: neighbouring lanes then ask for
 // neighbouring entries of a row, whose sorted columns share cache lines, and the address
 // unit serves them together instead of one lane per cycle.  Returns the products
@@ -107,26 +106,29 @@ __device__ __forceinline__ void wave_products(const int *__restrict__ col, const
                                               typename Acc<VT>::type *vs, typename Acc<VT>::type (&p)[NPT])
 {
     typedef typename Acc<VT>::type AT;
+    // every load instruction reads one contiguous stretch (lane l right after lane l-1): a
+    // streamed line is then asked for once, not once per instruction that touches a piece of it
     if constexpr (sizeof(VT) == 8) {
 #pragma unroll
         for (int q = 0; q < NPT / 4; ++q) {
             const int e = 256 * q + 4 * lane;
-            const v4i32 c4 = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
-            const v2f64 va = __builtin_nontemporal_load((const v2f64 *)(val + pos + e));
-            const v2f64 vb = __builtin_nontemporal_load((const v2f64 *)(val + pos + e + 2));
-            *(v4i32 *)(cs + e) = c4;
-            *(v2f64 *)(vs + e) = va;
-            *(v2f64 *)(vs + e + 2) = vb;
+            *(v4i32 *)(cs + e) = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
+        }
+#pragma unroll
+        for (int q = 0; q < NPT / 2; ++q) {
+            const int e = 128 * q + 2 * lane;
+            *(v2f64 *)(vs + e) = __builtin_nontemporal_load((const v2f64 *)(val + pos + e));
         }
     } else {
 #pragma unroll
+        for (int q = 0; q < NPT / 4; ++q) {
+            const int e = 256 * q + 4 * lane;
+            *(v4i32 *)(cs + e) = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
+        }
+#pragma unroll
         for (int q = 0; q < NPT / 8; ++q) {
             const int e = 512 * q + 8 * lane;
-            const v4i32 ca = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
-            const v4i32 cb = __builtin_nontemporal_load((const v4i32 *)(col + pos + e + 4));
             const v8f16 hv = __builtin_nontemporal_load((const v8f16 *)(val + pos + e));
-            *(v4i32 *)(cs + e) = ca;
-            *(v4i32 *)(cs + e + 4) = cb;
             v4f32 fa, fb;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -253,209 +255,159 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
     }
 }
 
-// ---- CSR part, LDS-staged x ---------------------------------------------------------------
+// ---- CSR part, x resident in LDS ----------------------------------------------------------
 // For matrices whose x gathers are scattered, a gather from L2 moves a whole 128-byte line
-// for one value and the kernel is bound by that, not by HBM.  Here one workgroup per CU owns a
-// block of rows and sweeps the column panels that hold entries of its rows: the panel's slice
-// of x is copied, fully coalesced, into LDS, then the group's entries -- 16-bit row and
-// column offsets plus the value, read with wide loads -- gather x from LDS and add their
-// products to per-row accumulators in LDS (ds_add_f64 / ds_add_f32; consecutive entries of
-// one row are summed in registers first).  Every y row has one owner workgroup, which stores
-// it once at the end; no global atomics.
-//
-// The 16 waves split the work by kind so that each wave's loads are of one kind only (loads
-// of a wave retire in issue order, and an x slice must never queue behind an entry load
-// that takes several times longer): waves 0..7 move x -- they keep the slices of the next DX
-// panels in flight in registers (an L2-resident sweep, bound by the ~35 B/clk a CU can pull
-// from L2) and store the current one to LDS; waves 8..15 own the entries -- they keep the
-// first EPT entries per lane of the next DE groups in flight (streamed from HBM) and do the
-// gathers and accumulator updates.  Two workgroup barriers per panel hand the LDS slice over.
-// Every step issues the same loads whatever the data, so the waits the compiler derives name
-// only loads that are already old.
-struct PanelRef {  // one (block, panel) group; pad = 1 marks list padding (no entries, no x needed)
-    int panel, e0, e1, pad;
+// for one value, a CU can keep only ~64 KB of such requests in flight, and the kernel is bound
+// by that instead of HBM.  When x is small enough, the gathers can be served from LDS instead:
+// the columns are cut into S slices of kSliceBytes of x, the rows into G groups, and workgroup
+// (g, s) -- one per CU -- copies slice s into LDS once, then streams the entries of its rows
+// that fall into the slice (16-bit row and column offsets plus the value, 128-bit loads, the
+// next pass already in flight), gathers x from LDS and adds the products to per-row
+// accumulators in LDS (ds_add_f64 / ds_add_f32; consecutive entries of one row are summed in
+// registers first).  The rows of a group are handled in sub-blocks that fit the accumulators.
+// With S > 1 every workgroup owns one column of a [S][rows] array of partial sums, written
+// once, coalesced, and a second small kernel adds the S partials of each row; with S = 1 the
+// workgroup stores y itself.  No global atomics in either case.
+struct SubBlock {  // rows [row0, row0+nrows) of the matrix, entries [e0, e1) of this workgroup
+    int row0, nrows, e0, e1;
 };
 
+// Eight entries of one lane: row offsets, column offsets (16 bit each, packed) and values.
 template <typename VT>
-struct PanelCfg;
-template <>
-struct PanelCfg<double> {
-    static constexpr int EPT = 4;  // entries per lane per prefetched pass
-};
-template <>
-struct PanelCfg<_Float16> {
-    static constexpr int EPT = 8;
-};
-constexpr int kPanelDX = 2;  // x slices in flight (mover waves)
-constexpr int kPanelDE = 6;  // entry passes in flight (entry waves); the host pads lists to a multiple
-
-// EPT entries of one lane: row offsets, column offsets (16 bit each, packed) and values.
-template <typename VT, int EPT>
 struct EntryRegs {
-    unsigned r[EPT / 2], c[EPT / 2];
-    typename std::conditional<sizeof(VT) == 8, double, unsigned>::type v[sizeof(VT) == 8 ? EPT : EPT / 2];
+    v4i32 r, c;
+    v4i32 v[sizeof(VT) == 8 ? 4 : 1];
 };
 
 template <typename VT>
-__global__ __launch_bounds__(kPanelThreads) void csr_panel_kernel(const int *__restrict__ blockRow,
-                                                                  const int *__restrict__ listPtr,
-                                                                  const PanelRef *__restrict__ list,
+__device__ __forceinline__ void load_entries(EntryRegs<VT> &en, const unsigned short *__restrict__ erow,
+                                             const unsigned short *__restrict__ ecol, const VT *__restrict__ eval, int e)
+{
+    en.r = __builtin_nontemporal_load((const v4i32 *)(erow + e));
+    en.c = __builtin_nontemporal_load((const v4i32 *)(ecol + e));
+    if constexpr (sizeof(VT) == 8) {
+        // binary64 values are stored permuted inside every 512-entry block of a group so that
+        // each of the four loads is contiguous across the wave: piece q of lane l (entries
+        // 8l+2q, 8l+2q+1 of the block) sits at block + 128q + 2l
+        const int lane = threadIdx.x & 63;
+        const VT *blk = eval + (e - 8 * lane);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) en.v[q] = __builtin_nontemporal_load((const v4i32 *)(blk + 128 * q + 2 * lane));
+    } else {
+        en.v[0] = __builtin_nontemporal_load((const v4i32 *)(eval + e));
+    }
+}
+
+// gather x from LDS, sum runs of equal rows in registers, add to the accumulators
+template <typename VT>
+__device__ __forceinline__ void consume_entries(const EntryRegs<VT> &en, const VT *xs, typename Acc<VT>::type *acc)
+{
+    typedef typename Acc<VT>::type AT;
+    unsigned r[8];
+    AT prod[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const unsigned rw = (unsigned)en.r[j >> 1], cw = (unsigned)en.c[j >> 1];
+        r[j] = (j & 1) ? rw >> 16 : rw & 0xffffu;
+        const unsigned c = (j & 1) ? cw >> 16 : cw & 0xffffu;
+        AT v;
+        if constexpr (sizeof(VT) == 8) {
+            const v2f64 t = __builtin_bit_cast(v2f64, en.v[j >> 1]);
+            v = (j & 1) ? t.y : t.x;
+        } else {
+            const unsigned w = (unsigned)en.v[0][j >> 1];
+            v = (float)__builtin_bit_cast(_Float16, (unsigned short)((j & 1) ? w >> 16 : w & 0xffffu));
+        }
+        prod[j] = v * (AT)xs[c];
+    }
+    AT run = prod[0];
+    unsigned cur = r[0];
+#pragma unroll
+    for (int j = 1; j < 8; ++j) {
+        if (r[j] == cur) {
+            run += prod[j];
+        } else {
+            __hip_atomic_fetch_add(&acc[cur], run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            cur = r[j];
+            run = prod[j];
+        }
+    }
+    __hip_atomic_fetch_add(&acc[cur], run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+template <typename VT>
+__global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int *__restrict__ wgSubPtr,
+                                                                  const SubBlock *__restrict__ subs,
                                                                   const unsigned short *__restrict__ erow,
                                                                   const unsigned short *__restrict__ ecol,
                                                                   const VT *__restrict__ eval, const VT *__restrict__ x,
-                                                                  VT *__restrict__ y, int cols, int accumulate)
+                                                                  typename Acc<VT>::type *__restrict__ partial,
+                                                                  VT *__restrict__ y, int rows, int cols, int S,
+                                                                  int accumulate)
 {
     typedef typename Acc<VT>::type AT;
-    constexpr int DX = kPanelDX, DE = kPanelDE, EPT = PanelCfg<VT>::EPT;
-    constexpr int MOVERS = kPanelThreads / 2;              // lanes that move x; the rest own entries
-    constexpr int VPT = kPanelBytes / 16 / MOVERS;         // 16-byte vectors per mover lane per panel
-    constexpr int PW = kPanelBytes / (int)sizeof(VT);      // columns per panel
-    constexpr int EPV = 16 / (int)sizeof(VT);              // x entries per vector
-    constexpr int PASS = (kPanelThreads - MOVERS) * EPT;   // entries covered by one prefetched pass
-    typedef EntryRegs<VT, EPT> Entries;
+    constexpr int SW = kSliceBytes / (int)sizeof(VT);      // columns per slice
+    constexpr int VPT = kSliceBytes / 16 / kSliceThreads;  // 16-byte vectors per lane for the slice copy
+    constexpr int EPV = 16 / (int)sizeof(VT);
+    constexpr int PASS = kSliceThreads * 8;                // entries per pass of the workgroup
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     VT *xs = (VT *)smem;
-    AT *acc = (AT *)(smem + kPanelBytes);
+    AT *acc = (AT *)(smem + kSliceBytes);
 
     const int b = blockIdx.x, tid = threadIdx.x;
-    const int r0 = blockRow[b], nrows = blockRow[b + 1] - r0;
-    for (int i = tid; i < nrows; i += kPanelThreads) acc[i] = 0;
-    const PanelRef *gl = list + listPtr[b];
-    const int n = listPtr[b + 1] - listPtr[b];  // a multiple of DE and DX (the host pads the list)
-    // the block's group list, copied to LDS once: reading it from memory at every panel would
-    // put a dependent load in front of every fetch
-    __shared__ PanelRef pl[kPanelListMax + 8];
-    for (int i = tid; i < n; i += kPanelThreads) pl[i] = gl[i];
-    __syncthreads();
-
-    auto load_entries = [&](Entries &en, int e) {
-        if constexpr (EPT == 8) {
-            const v4i32 rr = __builtin_nontemporal_load((const v4i32 *)(erow + e));
-            const v4i32 cc = __builtin_nontemporal_load((const v4i32 *)(ecol + e));
+    const int slice = b % S;
+    // the slice of x, once
+    {
+        v4i32 xv[VPT];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                en.r[j] = (unsigned)rr[j];
-                en.c[j] = (unsigned)cc[j];
-            }
-        } else {
-            const v2i32 rr = __builtin_nontemporal_load((const v2i32 *)(erow + e));
-            const v2i32 cc = __builtin_nontemporal_load((const v2i32 *)(ecol + e));
-            en.r[0] = (unsigned)rr.x; en.r[1] = (unsigned)rr.y;
-            en.c[0] = (unsigned)cc.x; en.c[1] = (unsigned)cc.y;
+        for (int q = 0; q < VPT; ++q) {
+            const int c = slice * SW + (q * kSliceThreads + tid) * EPV;
+            xv[q] = c + EPV <= cols ? *(const v4i32 *)(x + c) : v4i32{0, 0, 0, 0};
         }
-        if constexpr (sizeof(VT) == 8) {
 #pragma unroll
-            for (int q = 0; q < EPT / 2; ++q) {
-                const v2f64 t = __builtin_nontemporal_load((const v2f64 *)(eval + e + 2 * q));
-                en.v[2 * q] = t.x;
-                en.v[2 * q + 1] = t.y;
-            }
-        } else {
-            const v4i32 t = __builtin_nontemporal_load((const v4i32 *)(eval + e));
-#pragma unroll
-            for (int j = 0; j < 4; ++j) en.v[j] = (unsigned)t[j];
-        }
-    };
-    // EPT entries: gather x from LDS, sum runs of equal rows in registers, add to the accumulators
-    auto consume = [&](const Entries &en) {
-        unsigned r[EPT];
-        AT prod[EPT];
-#pragma unroll
-        for (int j = 0; j < EPT; ++j) {
-            r[j] = (j & 1) ? en.r[j >> 1] >> 16 : en.r[j >> 1] & 0xffffu;
-            const unsigned c = (j & 1) ? en.c[j >> 1] >> 16 : en.c[j >> 1] & 0xffffu;
-            AT v;
-            if constexpr (sizeof(VT) == 8) {
-                v = en.v[j];
-            } else {
-                const unsigned short h = (j & 1) ? (unsigned short)(en.v[j >> 1] >> 16) : (unsigned short)(en.v[j >> 1] & 0xffffu);
-                v = (float)__builtin_bit_cast(_Float16, h);
-            }
-            prod[j] = v * (AT)xs[c];
-        }
-        AT run = prod[0];
-        unsigned cur = r[0];
-#pragma unroll
-        for (int j = 1; j < EPT; ++j) {
-            if (r[j] == cur) {
-                run += prod[j];
-            } else {
-                __hip_atomic_fetch_add(&acc[cur], run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                cur = r[j];
-                run = prod[j];
-            }
-        }
-        __hip_atomic_fetch_add(&acc[cur], run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    };
-    // entries of a group beyond the prefetched pass: all 16 waves, plain loads
-    auto remainder = [&](const PanelRef g) {
-        for (int e = g.e0 + PASS + tid * EPT; e < g.e1; e += kPanelThreads * EPT) {
-            Entries en;
-            load_entries(en, e);
-            consume(en);
-        }
-    };
-
-    if (tid < MOVERS) {
-        v4f32 X[DX][VPT];
-        auto fetch_x = [&](int slot, const PanelRef g) {
-#pragma unroll
-            for (int q = 0; q < VPT; ++q) {
-                int c = g.panel * PW + (q * MOVERS + tid) * EPV;  // first column of this vector
-                if (g.pad || c + EPV > cols) c = 0;                 // never used: any valid address
-                X[slot][q] = *(const v4f32 *)(x + c);
-            }
-        };
-        if (n > 0) {
-#pragma unroll
-            for (int sl = 0; sl < DX; ++sl) fetch_x(sl, pl[sl]);
-        }
-        for (int base = 0; base < n; base += DX) {
-#pragma unroll
-            for (int sl = 0; sl < DX; ++sl) {
-                const int i = base + sl;
-                const PanelRef g = pl[i];
-                __syncthreads();  // the previous panel is no longer read
-#pragma unroll
-                for (int q = 0; q < VPT; ++q) *(v4f32 *)(xs + (q * MOVERS + tid) * EPV) = X[sl][q];
-                __syncthreads();
-                fetch_x(sl, pl[i + DX < n ? i + DX : n - 1]);
-                remainder(g);
-            }
-        }
-    } else {
-        const int t = tid - MOVERS;
-        Entries E[DE];
-        // entry loads only in waves that have entries (a wave-uniform test)
-        auto fetch_e = [&](int slot, const PanelRef g) {
-            if (g.e0 + (t & ~63) * EPT < g.e1) {
-                int e = g.e0 + t * EPT;
-                if (e >= g.e1) e = g.e0;
-                load_entries(E[slot], e);
-            }
-        };
-        if (n > 0) {
-#pragma unroll
-            for (int sl = 0; sl < DE; ++sl) fetch_e(sl, pl[sl]);
-        }
-        for (int base = 0; base < n; base += DE) {
-#pragma unroll
-            for (int sl = 0; sl < DE; ++sl) {
-                const int i = base + sl;
-                const PanelRef g = pl[i];
-                __syncthreads();
-                __syncthreads();  // the panel's slice of x is in LDS
-                if (g.e0 + t * EPT < g.e1) consume(E[sl]);
-                fetch_e(sl, pl[i + DE < n ? i + DE : n - 1]);
-                remainder(g);
-            }
-        }
+        for (int q = 0; q < VPT; ++q) *(v4i32 *)(xs + (q * kSliceThreads + tid) * EPV) = xv[q];
     }
-    __syncthreads();
-    for (int i = tid; i < nrows; i += kPanelThreads) {
-        AT sum = acc[i];
-        if (accumulate) sum += (AT)y[r0 + i];
-        y[r0 + i] = (VT)sum;
+    const int s0 = wgSubPtr[b], s1 = wgSubPtr[b + 1];
+    for (int sb = s0; sb < s1; ++sb) {
+        const SubBlock d = subs[sb];
+        for (int i = tid; i < d.nrows; i += kSliceThreads) acc[i] = 0;
+        __syncthreads();  // accumulators cleared (and, the first time, the slice in place)
+        // lanes are never moved to another entry: load_entries derives the wave's block from
+        // "entry - 8*lane"; a lane past the end simply does not load
+        EntryRegs<VT> cur, nxt;
+        int e = d.e0 + tid * 8;
+        if (e < d.e1) load_entries(cur, erow, ecol, eval, e);
+        for (; e < d.e1; e += PASS) {
+            const bool more = e + PASS < d.e1;
+            if (more) load_entries(nxt, erow, ecol, eval, e + PASS);
+            consume_entries<VT>(cur, xs, acc);
+            if (more) cur = nxt;
+        }
+        __syncthreads();
+        if (S > 1) {
+            AT *out = partial + (size_t)slice * rows + d.row0;
+            for (int i = tid; i < d.nrows; i += kSliceThreads) out[i] = acc[i];
+        } else {
+            for (int i = tid; i < d.nrows; i += kSliceThreads) {
+                AT sum = acc[i];
+                if (accumulate) sum += (AT)y[d.row0 + i];
+                y[d.row0 + i] = (VT)sum;
+            }
+        }
+        __syncthreads();  // accumulators free for the next sub-block
+    }
+}
+
+// y[r] = sum over the S slices of partial[s][r] (+ y[r])
+template <typename VT>
+__global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Acc<VT>::type *__restrict__ partial,
+                                                              VT *__restrict__ y, int rows, int S, int accumulate)
+{
+    typedef typename Acc<VT>::type AT;
+    for (int r = blockIdx.x * kBlock + threadIdx.x; r < rows; r += gridDim.x * kBlock) {
+        AT sum = accumulate ? (AT)y[r] : (AT)0;
+        for (int s = 0; s < S; ++s) sum += partial[(size_t)s * rows + r];
+        y[r] = (VT)sum;
     }
 }
 
@@ -740,30 +692,34 @@ hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y
 }
 
 template <typename VT>
-static hipError_t launch_panels_t(const DevicePanels &P, const void *x, void *y, int cols, int accumulate, hipStream_t s)
+static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s)
 {
-    const size_t lds = (size_t)kPanelBytes + (size_t)P.maxBlockRows * sizeof(typename mxk::Acc<VT>::type);
-    if (P.nPanels > kPanelListMax) return hipErrorInvalidValue;
+    typedef typename mxk::Acc<VT>::type AT;
+    const size_t lds = (size_t)kSliceBytes + (size_t)P.maxSubRows * sizeof(AT);
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)mxk::csr_panel_kernel<VT>,
+        hipError_t e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           160 * 1024 - 16 * (kPanelListMax + 8) - 1024);
+                                           mx::kSliceBytes + mx::kSliceAccBytes);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL((mxk::csr_panel_kernel<VT>), dim3(P.nBlocks), dim3(kPanelThreads), lds, s, P.blockRow, P.listPtr,
-                       (const mxk::PanelRef *)P.list, P.erow, P.ecol, (const VT *)P.eval, (const VT *)x, (VT *)y, cols,
-                       accumulate);
+    hipLaunchKernelGGL((mxk::csr_slice_kernel<VT>), dim3(P.nWG), dim3(kSliceThreads), lds, s, P.wgSubPtr,
+                       (const mxk::SubBlock *)P.subs, P.erow, P.ecol, (const VT *)P.eval, (const VT *)x, (AT *)P.partial,
+                       (VT *)y, P.rows, P.cols, P.S, accumulate);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || P.S <= 1) return e;
+    const int grid = std::min(2048, (P.rows + mxk::kBlock - 1) / mxk::kBlock);
+    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(grid), dim3(mxk::kBlock), 0, s, (const AT *)P.partial, (VT *)y,
+                       P.rows, P.S, accumulate);
     return hipGetLastError();
 }
 
-hipError_t launch_panels(mx_dtype dtype, const DevicePanels &P, const void *x, void *y, int cols, int accumulate,
-                         hipStream_t s)
+hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s)
 {
-    if (P.nBlocks <= 0) return hipSuccess;
-    if (dtype == MX_F64) return launch_panels_t<double>(P, x, y, cols, accumulate, s);
-    return launch_panels_t<_Float16>(P, x, y, cols, accumulate, s);
+    if (P.nWG <= 0) return hipSuccess;
+    if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s);
+    return launch_slices_t<_Float16>(P, x, y, accumulate, s);
 }
 
 hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s)

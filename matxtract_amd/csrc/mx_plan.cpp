@@ -91,107 +91,133 @@ void free_tiles(mx::DeviceTiles &T)
     T = mx::DeviceTiles();
 }
 
-void free_panels(mx::DevicePanels &P)
+void free_slices(mx::DeviceSlices &P)
 {
-    (void)hipFree(P.blockRow);
-    (void)hipFree(P.listPtr);
-    (void)hipFree(P.list);
+    (void)hipFree(P.wgSubPtr);
+    (void)hipFree(P.subs);
     (void)hipFree(P.erow);
     (void)hipFree(P.ecol);
     (void)hipFree(P.eval);
-    P = mx::DevicePanels();
+    (void)hipFree(P.partial);
+    P = mx::DeviceSlices();
 }
 
-// Re-lays a CSR matrix for csr_panel_kernel: row blocks balanced by entries (at most
-// `maxRows` rows each, about one block per CU), column panels of panel_cols(dtype) columns;
-// the entries of each (block, panel) group keep their row-major order and are padded with
-// zero entries to a multiple of 8 so every group starts on a 16-byte boundary.
-int upload_panels(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU,
-                  mx::DevicePanels &D)
+// Number of column slices csr_slice_kernel would need, or 0 when the matrix does not suit it:
+// x is copied in 16-byte vectors (cols must be a whole number of them), and with S slices the
+// kernel writes and re-reads S partial sums per row, which must stay small next to the matrix.
+int slice_count(mx_dtype dtype, int rows, int cols, int nnz, int nCU)
+{
+    const int es = mx::elem_size(dtype), epv = 16 / es;
+    if (cols < epv || cols % epv || nnz < 4096) return 0;
+    const int S = (cols + mx::slice_cols(dtype) - 1) / mx::slice_cols(dtype);
+    if (S > nCU) return 0;
+    const double accBytes = dtype == MX_F64 ? 8 : 4;
+    const double extra = S > 1 ? 2.0 * S * (double)rows * accBytes : 0.0;
+    if (extra > 2.0 * (double)nnz * (es + 4)) return 0;
+    return S;
+}
+
+// Re-lays a CSR matrix for csr_slice_kernel (see DeviceSlices).  Row groups are balanced by
+// entries; workgroup g*S+s gets group g and slice s.
+int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
+                  mx::DeviceSlices &D)
 {
     const int es = mx::elem_size(dtype);
-    const int PW = mx::panel_cols(dtype), maxRows = mx::panel_max_block_rows(dtype);
-    const size_t depth = (size_t)mx::kPanelListPad;
+    const int SW = mx::slice_cols(dtype), subMax = mx::slice_sub_rows(dtype);
+    // groups are padded with zero entries to whole 8-entry lanes; binary64 groups to whole
+    // 512-entry wave blocks, inside which the values are stored permuted (see load_entries)
+    const int gpad = dtype == MX_F64 ? 512 : 8;
     const int nnz = rowPtr[rows];
-    const int nPanels = std::max(1, (cols + PW - 1) / PW);
-    const long long target = std::max<long long>(1, ((long long)nnz + nCU - 1) / std::max(nCU, 1));
-    std::vector<int> blockRow(1, 0);
-    for (int r = 0; r < rows;) {
-        const int start = r;
-        long long cnt = 0;
-        while (r < rows && r - start < maxRows && (cnt < target || r == start)) {
-            cnt += rowPtr[r + 1] - rowPtr[r];
-            ++r;
+    const int G = std::max(1, nCU / S);
+    // row groups with about nnz/G entries each
+    std::vector<int> groupRow(1, 0);
+    for (int g = 1; g < G; ++g) {
+        const long long target = (long long)nnz * g / G;
+        int r = (int)(std::lower_bound(rowPtr, rowPtr + rows + 1, (int)target) - rowPtr);
+        r = std::min(std::max(r, groupRow.back()), rows);
+        groupRow.push_back(r);
+    }
+    groupRow.push_back(rows);
+    // sub-blocks of each group (shared by its S workgroups)
+    std::vector<int> gSubPtr(1, 0), subRow0, subRows;
+    for (int g = 0; g < G; ++g) {
+        for (int r = groupRow[g]; r < groupRow[g + 1]; r += subMax) {
+            subRow0.push_back(r);
+            subRows.push_back(std::min(subMax, groupRow[g + 1] - r));
         }
-        blockRow.push_back(r);
+        gSubPtr.push_back((int)subRow0.size());
     }
-    const int nBlocks = (int)blockRow.size() - 1;
-    std::vector<long long> grp((size_t)nBlocks * nPanels + 1, 0);
-#pragma omp parallel for schedule(dynamic, 4)
-    for (int b = 0; b < nBlocks; ++b) {
-        long long *g = grp.data() + (size_t)b * nPanels + 1;
-        for (int p = rowPtr[blockRow[b]]; p < rowPtr[blockRow[b + 1]]; ++p) g[col[p] / PW]++;
-        for (int q = 0; q < nPanels; ++q) g[q] = (g[q] + 7) / 8 * 8;
+    const int nSubG = (int)subRow0.size();
+    // entry counts per (sub-block, slice), padded to multiples of 8
+    std::vector<long long> cnt((size_t)nSubG * S, 0);
+#pragma omp parallel for schedule(dynamic, 16)
+    for (int i = 0; i < nSubG; ++i) {
+        long long *c = cnt.data() + (size_t)i * S;
+        for (int p = rowPtr[subRow0[i]]; p < rowPtr[subRow0[i] + subRows[i]]; ++p) c[col[p] / SW]++;
+        for (int q = 0; q < S; ++q) c[q] = (c[q] + gpad - 1) / gpad * gpad;
     }
-    for (size_t i = 1; i < grp.size(); ++i) grp[i] += grp[i - 1];
-    const long long total = grp.back();
+    // layout order: workgroup (g, s), then its sub-blocks
+    const int nWG = G * S;
+    std::vector<int> wgSubPtr(1, 0), subs;
+    std::vector<long long> start((size_t)nSubG * S, 0);
+    long long total = 0;
+    int maxSub = 0;
+    for (int g = 0; g < G; ++g)
+        for (int q = 0; q < S; ++q) {
+            for (int i = gSubPtr[g]; i < gSubPtr[g + 1]; ++i) {
+                start[(size_t)i * S + q] = total;
+                subs.push_back(subRow0[i]);
+                subs.push_back(subRows[i]);
+                subs.push_back((int)total);
+                total += cnt[(size_t)i * S + q];
+                subs.push_back((int)total);
+                maxSub = std::max(maxSub, subRows[i]);
+            }
+            wgSubPtr.push_back((int)(subs.size() / 4));
+        }
     if (total > 2000000000LL) {
-        set_error("panel layout: too many entries for 32-bit offsets");
+        set_error("slice layout: too many entries for 32-bit offsets");
         return MX_ERR_ARG;
     }
-    std::vector<int> grpPtr(grp.begin(), grp.end());
-    // per block, the list of its non-empty groups
-    std::vector<int> listPtr((size_t)nBlocks + 1, 0), list;
-    for (int b = 0; b < nBlocks; ++b) {
-        for (int q = 0; q < nPanels; ++q) {
-            const int e0 = grpPtr[(size_t)b * nPanels + q], e1 = grpPtr[(size_t)b * nPanels + q + 1];
-            if (e1 > e0) {
-                list.push_back(q);
-                list.push_back(e0);
-                list.push_back(e1);
-                list.push_back(0);
-            }
-        }
-        while ((list.size() / 4 - (size_t)listPtr[b]) % depth) {  // pad with empty groups
-            list.push_back(0);
-            list.push_back(0);
-            list.push_back(0);
-            list.push_back(1);
-        }
-        listPtr[b + 1] = (int)(list.size() / 4);
-    }
-    std::vector<unsigned short> erow((size_t)total + 8, 0), ecol((size_t)total + 8, 0);
-    std::vector<unsigned char> ev(((size_t)total + 8) * es, 0);
+    // 1024 spare zero entries: a wave may read one whole 512-entry block starting at any entry
+    std::vector<unsigned short> erow((size_t)total + 1024, 0), ecol((size_t)total + 1024, 0);
+    std::vector<unsigned char> ev(((size_t)total + 1024) * es, 0);
     const unsigned char *sv = (const unsigned char *)val;
 #pragma omp parallel
     {
-        std::vector<int> cursor(nPanels);
-#pragma omp for schedule(dynamic, 4)
-        for (int b = 0; b < nBlocks; ++b) {
-            std::copy(grpPtr.begin() + (size_t)b * nPanels, grpPtr.begin() + (size_t)(b + 1) * nPanels, cursor.begin());
-            for (int r = blockRow[b]; r < blockRow[b + 1]; ++r)
+        std::vector<long long> cursor(S);
+#pragma omp for schedule(dynamic, 16)
+        for (int i = 0; i < nSubG; ++i) {
+            std::copy(start.begin() + (size_t)i * S, start.begin() + (size_t)(i + 1) * S, cursor.begin());
+            for (int r = subRow0[i]; r < subRow0[i] + subRows[i]; ++r)
                 for (int p = rowPtr[r]; p < rowPtr[r + 1]; ++p) {
-                    const int q = col[p] / PW;
-                    const int e = cursor[q]++;
-                    erow[e] = (unsigned short)(r - blockRow[b]);
-                    ecol[e] = (unsigned short)(col[p] - q * PW);
-                    std::memcpy(&ev[(size_t)e * es], sv + (size_t)p * es, es);
+                    const int q = col[p] / SW;
+                    const long long e = cursor[q]++;
+                    erow[e] = (unsigned short)(r - subRow0[i]);
+                    ecol[e] = (unsigned short)(col[p] - q * SW);
+                    long long ve = e;
+                    if (dtype == MX_F64) {  // position inside the group's 512-entry block
+                        const long long g0 = start[(size_t)i * S + q], rel = e - g0;
+                        const long long within = rel % 512, l = within / 8, j8 = within % 8;
+                        ve = g0 + rel / 512 * 512 + (j8 / 2) * 128 + 2 * l + (j8 % 2);
+                    }
+                    std::memcpy(&ev[(size_t)ve * es], sv + (size_t)p * es, es);
                 }
         }
     }
-    D.nBlocks = nBlocks;
-    D.nPanels = nPanels;
-    D.panelCols = PW;
-    D.maxBlockRows = 0;
-    for (int b = 0; b < nBlocks; ++b) D.maxBlockRows = std::max(D.maxBlockRows, blockRow[b + 1] - blockRow[b]);
+    D.nWG = nWG;
+    D.S = S;
+    D.rows = rows;
+    D.cols = cols;
+    D.maxSubRows = maxSub;
     D.entries = total;
     int rc;
-    if ((rc = upload(&D.blockRow, blockRow.data(), blockRow.size()))) return rc;
-    if ((rc = upload(&D.listPtr, listPtr.data(), listPtr.size()))) return rc;
-    if ((rc = upload(&D.list, list.data(), list.size(), 16))) return rc;
+    if ((rc = upload(&D.wgSubPtr, wgSubPtr.data(), wgSubPtr.size()))) return rc;
+    if ((rc = upload(&D.subs, subs.data(), subs.size(), 16))) return rc;
     if ((rc = upload(&D.erow, erow.data(), erow.size()))) return rc;
     if ((rc = upload(&D.ecol, ecol.data(), ecol.size()))) return rc;
     if ((rc = upload_bytes(&D.eval, ev.data(), ev.size()))) return rc;
+    if (S > 1 && (rc = upload_bytes(&D.partial, nullptr, 0, (size_t)S * rows * (dtype == MX_F64 ? 8 : 4)))) return rc;
     return MX_OK;
 }
 
@@ -295,8 +321,8 @@ struct mx_plan {
     mx_dtype dtype = MX_F64;
     int rows = 0, cols = 0, nnz = 0;
     mx::DeviceCsr csr;        // CSR part, row-tile form (csr_rows_kernel)
-    mx::DevicePanels panels;  // CSR part, LDS-staged-x form (csr_panel_kernel)
-    bool use_panels = false;  // which of the two runs
+    mx::DeviceSlices slices;  // CSR part, x-resident-in-LDS form (csr_slice_kernel)
+    bool use_slices = false;  // which of the two runs
     int csr_nnz = 0;
     mx::DeviceTiles tiles;
     int tile_nnz = 0;
@@ -318,7 +344,7 @@ extern "C" void mx_plan_destroy(mx_plan *plan)
 {
     if (!plan) return;
     free_csr(plan->csr);
-    free_panels(plan->panels);
+    free_slices(plan->slices);
     free_tiles(plan->tiles);
     if (plan->ev0) (void)hipEventDestroy(plan->ev0);
     if (plan->ev1) (void)hipEventDestroy(plan->ev1);
@@ -351,49 +377,43 @@ static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
 
 static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate, hipStream_t s)
 {
-    if (plan->use_panels)
-        MX_HIP(mx::launch_panels(plan->dtype, plan->panels, x, y, plan->cols, accumulate, s));
+    if (plan->use_slices)
+        MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s));
     else
         MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s));
     return MX_OK;
 }
 
 // Puts the CSR part on the device.  Two executable forms exist (row tiles with direct x
-// gathers; column panels with x staged in LDS); unless a flag forces one, both are built,
-// timed on the spot with a few launches each, and the slower one is released.
+// gathers; column slices with x resident in LDS); unless a flag forces one, both are built
+// when the matrix suits the second, timed on the spot with a few launches each, and the
+// slower one is released.
 static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags)
 {
     const int rows = plan->rows, cols = plan->cols;
     const int nnz = rowPtr[rows];
     plan->csr_nnz = nnz;
     const char *env = std::getenv("MX_CSR_KERNEL");
-    bool want_rows = true, want_panels = true;
-    if (flags & MX_PLAN_CSR_ROWS) want_panels = false;
-    if (flags & MX_PLAN_CSR_PANELS) want_rows = false;
-    if (env && !std::strcmp(env, "rows")) want_rows = true, want_panels = false;
-    if (env && !std::strcmp(env, "panels")) want_rows = false, want_panels = true;
+    bool want_rows = true, want_slices = true;
+    if (flags & MX_PLAN_CSR_ROWS) want_slices = false;
+    if (flags & MX_PLAN_CSR_SLICES) want_rows = false;
+    if (env && !std::strcmp(env, "rows")) want_rows = true, want_slices = false;
+    if (env && !std::strcmp(env, "slices")) want_rows = false, want_slices = true;
     hipDeviceProp_t prop;
     int dev = 0;
     MX_HIP(hipGetDevice(&dev));
     MX_HIP(hipGetDeviceProperties(&prop, dev));
     const int nCU = std::max(1, prop.multiProcessorCount);
-    if (want_rows && want_panels) {
-        // every workgroup copies each panel it touches; do not even try when that sweep would
-        // dwarf the matrix itself
-        const double sweep = (double)std::max(nCU, rows / mx::panel_max_block_rows(plan->dtype)) * (double)cols *
-                             mx::elem_size(plan->dtype);
-        const double matrix = (double)nnz * (mx::elem_size(plan->dtype) + 4);
-        if (nnz < 4096 || sweep > 64.0 * matrix) want_panels = false;
-    }
-    if (!mx::panels_possible(plan->dtype, cols)) {  // shape the panel kernel cannot take: row tiles
-        want_panels = false;
+    const int S = slice_count(plan->dtype, rows, cols, nnz, nCU);
+    if (S == 0) {  // a matrix the slice kernel cannot take runs on row tiles whatever was asked
+        want_slices = false;
         want_rows = true;
     }
     int rc;
     if (want_rows && (rc = upload_csr(plan->dtype, rows, nnz, rowPtr, col, val, plan->csr, nullptr))) return rc;
-    if (want_panels && (rc = upload_panels(plan->dtype, rows, cols, rowPtr, col, val, nCU, plan->panels))) return rc;
-    plan->use_panels = want_panels && !want_rows;
-    if (want_rows && want_panels) {
+    if (want_slices && (rc = upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, plan->slices))) return rc;
+    plan->use_slices = want_slices && !want_rows;
+    if (want_rows && want_slices) {
         const size_t es = (size_t)mx::elem_size(plan->dtype);
         void *tx = nullptr, *ty = nullptr;
         if ((rc = upload_bytes(&tx, nullptr, 0, std::max<size_t>(cols * es, 16)))) return rc;
@@ -403,15 +423,15 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
         }
         double ms[2] = {0.0, 0.0};
         for (int v = 0; v < 2 && !rc; ++v) {
-            plan->use_panels = v == 1;
+            plan->use_slices = v == 1;
             rc = time_loop(plan, 3, 10, [&]() { return launch_csr_part(plan, tx, ty, 0, plan->stream); }, &ms[v]);
         }
         (void)hipFree(tx);
         (void)hipFree(ty);
         if (rc) return rc;
-        plan->use_panels = ms[1] < ms[0];
-        if (plan->use_panels) free_csr(plan->csr);
-        else free_panels(plan->panels);
+        plan->use_slices = ms[1] < ms[0];
+        if (plan->use_slices) free_csr(plan->csr);
+        else free_slices(plan->slices);
     }
     return MX_OK;
 }
@@ -536,8 +556,8 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     info->tile_frags = plan->tiles.frags;
     info->tile_nnz = plan->tile_nnz;
     info->csr_nnz = plan->csr_nnz;
-    info->csr_blocks = plan->use_panels ? plan->panels.nBlocks : plan->csr.nBlocks;
-    info->csr_variant = plan->use_panels ? 1 : 0;
+    info->csr_blocks = plan->use_slices ? plan->slices.nWG : plan->csr.nBlocks;
+    info->csr_variant = plan->use_slices ? 1 : 0;
     // what each kernel has to move at least once: its arrays, x once, its y rows
     info->csr_bytes = (double)plan->csr_nnz * (es + 4) + ((double)plan->rows + 1) * 4 + (double)plan->cols * es +
                       (double)plan->rows * es;

@@ -72,15 +72,15 @@ TAUS = [(0.0, 0.0), (0.5, 0.25), (1.0, 1.0), (0.75, 0.0), (0.25, 0.25), (1.0, 0.
 
 
 @pytest.mark.parametrize("cfg,scale", CASES)
-@pytest.mark.parametrize("flags", ["default", "no_tiles", "all_tiles", "all_tiles+csr_rows", "all_tiles+csr_panels",
-                                   "no_tiles+csr_panels"])
+@pytest.mark.parametrize("flags", ["default", "no_tiles", "all_tiles", "all_tiles+csr_rows", "all_tiles+csr_slices",
+                                   "no_tiles+csr_slices"])
 def test_hybrid_spmv_matches_oracle(mx, ora, cfg, scale, flags):
     import torch
     A, x = mx.gen_config(cfg, scale=scale)
     ref = oracle_y(ora, mx, A, x)
     tol = F64_TOL if A.dtype == mx.MX_F64 else F16_TOL
     bits = {"default": mx.MX_PLAN_DEFAULT, "no_tiles": mx.MX_PLAN_NO_TILES, "all_tiles": mx.MX_PLAN_ALL_TILES,
-            "csr_rows": mx.MX_PLAN_CSR_ROWS, "csr_panels": mx.MX_PLAN_CSR_PANELS}
+            "csr_rows": mx.MX_PLAN_CSR_ROWS, "csr_slices": mx.MX_PLAN_CSR_SLICES}
     fl = 0
     for name in flags.split("+"):
         fl |= bits[name]
@@ -121,7 +121,7 @@ def test_full_size_workloads_match_oracle(mx, ora, cfg, taus):
     xd = torch.from_numpy(x).cuda()
     for tau in taus:
         for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_ROWS,
-                   mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_PANELS):
+                   mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_SLICES):
             print("full-size workload=%d tau=%s flags=%d" % (cfg, tau, fl), flush=True)
             part = mx.Partition(A, *tau)
             plan = mx.Plan(part, fl)
