@@ -172,6 +172,10 @@ int mx_spmv_host(mx_plan *plan, const void *x_host, void *y_host);
 int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters,
             double *ms_total, double *ms_tile, double *ms_csr);
 
+/* Mean ms per launch of the CSR part's main kernel alone (csr_rows_kernel, or csr_slice_kernel
+ * without its combine kernel), same protocol as mx_time: the figure a roofline is priced on. */
+int mx_time_csr_main(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters, double *ms);
+
 /* Facts about a plan, for reporting. */
 typedef struct mx_plan_info {
     mx_dtype dtype;

@@ -77,6 +77,7 @@ SIGNATURES = {
     "mx_spmv_repeat": (_i, [_vp, _vp, _vp, _i, _vp]),
     "mx_spmv_host": (_i, [_vp, _vp, _vp]),
     "mx_time": (_i, [_vp, _vp, _vp, _i, _i, _pd, _pd, _pd]),
+    "mx_time_csr_main": (_i, [_vp, _vp, _vp, _i, _i, _pd]),
     "mx_plan_get_info": (_i, [_vp, C.POINTER(PlanInfo)]),
     "mx_cdspmv_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _pd, _pd]),
     "mx_cdspmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _pd, _pd]),

@@ -227,6 +227,14 @@ class Plan:
                                   C.byref(tt) if parts else None, C.byref(tc) if parts else None))
         return t.value, tt.value, tc.value
 
+    def time_csr_main(self, x, y, warm=200, iters=4000):
+        """Mean ms per launch of the CSR part's main kernel alone."""
+        self._check_vec(x, self.cols, "x")
+        self._check_vec(y, self.rows, "y")
+        t = C.c_double()
+        check(_lib.load().mx_time_csr_main(self._h, x.data_ptr(), y.data_ptr(), warm, iters, C.byref(t)))
+        return t.value
+
     def close(self):
         if self._h:
             _lib.load().mx_plan_destroy(self._h)

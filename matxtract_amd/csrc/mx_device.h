@@ -57,7 +57,9 @@ constexpr int kSliceAccBytes = 24576; // LDS left for the row accumulators of a 
 inline int slice_cols(mx_dtype d) { return kSliceBytes / (d == MX_F64 ? 8 : 2); }
 inline int slice_sub_rows(mx_dtype d) { return kSliceAccBytes / (d == MX_F64 ? 8 : 4); }
 
-hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s);
+// `what`: 0 = slice kernel then combine kernel, 1 = slice kernel only, 2 = combine kernel only
+hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
+                         int what = 0);
 hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s);
 hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s);
 hipError_t launch_probe_f64(const double *A, const double *B, double *D, hipStream_t s);

@@ -356,7 +356,13 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int *__r
 
     const int b = blockIdx.x, tid = threadIdx.x;
     const int slice = b % S;
-    // the slice of x, once
+    const int s0 = wgSubPtr[b], s1 = wgSubPtr[b + 1];
+    // lanes are never moved to another entry: load_entries derives the wave's block from
+    // "entry - 8*lane"; a lane past the end simply does not load
+    EntryRegs<VT> cur, nxt;
+    SubBlock d = s0 < s1 ? subs[s0] : SubBlock{0, 0, 0, 0};
+    int e = d.e0 + tid * 8;
+    if (e < d.e1) load_entries(cur, erow, ecol, eval, e);  // the first pass travels while the slice is copied
     {
         v4i32 xv[VPT];
 #pragma unroll
@@ -367,16 +373,14 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int *__r
 #pragma unroll
         for (int q = 0; q < VPT; ++q) *(v4i32 *)(xs + (q * kSliceThreads + tid) * EPV) = xv[q];
     }
-    const int s0 = wgSubPtr[b], s1 = wgSubPtr[b + 1];
     for (int sb = s0; sb < s1; ++sb) {
-        const SubBlock d = subs[sb];
+        if (sb > s0) {
+            d = subs[sb];
+            e = d.e0 + tid * 8;
+            if (e < d.e1) load_entries(cur, erow, ecol, eval, e);
+        }
         for (int i = tid; i < d.nrows; i += kSliceThreads) acc[i] = 0;
         __syncthreads();  // accumulators cleared (and, the first time, the slice in place)
-        // lanes are never moved to another entry: load_entries derives the wave's block from
-        // "entry - 8*lane"; a lane past the end simply does not load
-        EntryRegs<VT> cur, nxt;
-        int e = d.e0 + tid * 8;
-        if (e < d.e1) load_entries(cur, erow, ecol, eval, e);
         for (; e < d.e1; e += PASS) {
             const bool more = e + PASS < d.e1;
             if (more) load_entries(nxt, erow, ecol, eval, e + PASS);
@@ -692,7 +696,7 @@ hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y
 }
 
 template <typename VT>
-static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s)
+static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, int what)
 {
     typedef typename mxk::Acc<VT>::type AT;
     const size_t lds = (size_t)kSliceBytes + (size_t)P.maxSubRows * sizeof(AT);
@@ -704,22 +708,24 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL((mxk::csr_slice_kernel<VT>), dim3(P.nWG), dim3(kSliceThreads), lds, s, P.wgSubPtr,
-                       (const mxk::SubBlock *)P.subs, P.erow, P.ecol, (const VT *)P.eval, (const VT *)x, (AT *)P.partial,
-                       (VT *)y, P.rows, P.cols, P.S, accumulate);
+    if (what != 2)
+        hipLaunchKernelGGL((mxk::csr_slice_kernel<VT>), dim3(P.nWG), dim3(kSliceThreads), lds, s, P.wgSubPtr,
+                           (const mxk::SubBlock *)P.subs, P.erow, P.ecol, (const VT *)P.eval, (const VT *)x,
+                           (AT *)P.partial, (VT *)y, P.rows, P.cols, P.S, accumulate);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || P.S <= 1) return e;
+    if (e != hipSuccess || P.S <= 1 || what == 1) return e;
     const int grid = std::min(2048, (P.rows + mxk::kBlock - 1) / mxk::kBlock);
     hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(grid), dim3(mxk::kBlock), 0, s, (const AT *)P.partial, (VT *)y,
                        P.rows, P.S, accumulate);
     return hipGetLastError();
 }
 
-hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s)
+hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
+                         int what)
 {
     if (P.nWG <= 0) return hipSuccess;
-    if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s);
-    return launch_slices_t<_Float16>(P, x, y, accumulate, s);
+    if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s, what);
+    return launch_slices_t<_Float16>(P, x, y, accumulate, s, what);
 }
 
 hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s)

@@ -627,6 +627,27 @@ extern "C" int mx_spmv_host(mx_plan *plan, const void *x_host, void *y_host)
     return rc;
 }
 
+extern "C" int mx_time_csr_main(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters, double *ms)
+{
+    if (!plan || !x_dev || !y_dev || warm < 0 || iters <= 0 || !ms) {
+        set_error("mx_time_csr_main: bad argument");
+        return MX_ERR_ARG;
+    }
+    hipStream_t s = plan->stream;
+    int rc = time_loop(plan, warm, iters, [&]() -> int {
+        if (plan->use_slices)
+            MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x_dev, y_dev, 0, s, 1));
+        else
+            MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x_dev, y_dev, 0, s));
+        return MX_OK;
+    }, ms);
+    if (rc) return rc;
+    rc = spmv_on(plan, x_dev, y_dev, s);  // leave y holding the product
+    if (rc) return rc;
+    MX_HIP(hipStreamSynchronize(s));
+    return MX_OK;
+}
+
 extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters, double *ms_total,
                        double *ms_tile, double *ms_csr)
 {
