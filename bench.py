@@ -150,6 +150,9 @@ def main():
     ap.add_argument("--workload", type=int, default=2, choices=sorted(WORKLOADS))
     ap.add_argument("--all", action="store_true", help="also run workloads 3, 4, 5 (reported under 'others')")
     ap.add_argument("--no-sweep", action="store_true", help="tau=(0,0) only")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="also launch one elementwise kernel that reads and writes MIB MiB (a known size to "
+                         "scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on exactly one GPU (the hybrid SpMV path has no multi-GPU part); "
@@ -180,6 +183,14 @@ def main():
         "best_hybrid": main_rec["best_hybrid"],
         "sweep": main_rec["sweep"],
     }
+    if args.calibrate_copy:
+        n = args.calibrate_copy * (1 << 20) // 4
+        src = torch.ones(n, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)  # reads 4n bytes, writes 4n bytes
+        torch.cuda.synchronize()
+        out["calibrate_copy_bytes_each_way"] = 4 * n
     if args.all:
         others = {}
         for cfg in (3, 4, 5):

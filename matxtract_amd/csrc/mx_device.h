@@ -9,9 +9,11 @@ namespace mx {
 // CSR matrix resident on the device, plus the row ranges of the CSR kernel's workgroups.
 // col/val carry kCsrPad extra zero entries so that a wave's aligned 128-bit loads may overrun.
 struct DeviceCsr {
-    int rows = 0, nnz = 0;
+    int rows = 0, cols = 0, nnz = 0;
     int *rowPtr = nullptr;    // [rows+1]
-    int *col = nullptr;       // [nnz + kCsrPad]
+    int *col = nullptr;       // [nnz + kCsrPad], or nullptr when the 16-bit form below is used
+    unsigned short *col16 = nullptr;  // [nnz + kCsrPad] column ids as offsets from colBase[workgroup]
+    int *colBase = nullptr;           // [nBlocks] lowest column of each workgroup's entries
     void *val = nullptr;      // [nnz + kCsrPad]
     int *blockDesc = nullptr; // [nBlocks][4] {first row, end row, first entry, end entry} per workgroup
     int nBlocks = 0;

@@ -100,31 +100,44 @@ struct Acc<_Float16> {
 // unit serves them together instead of one lane per cycle.  Returns the products
 // p[j] = val[pos+64j+l] * x[col[pos+64j+l]].
 //   cs, vs : this wave's LDS regions, 64*NPT ints / accumulators.
-template <typename VT, int NPT>
-__device__ __forceinline__ void wave_products(const int *__restrict__ col, const VT *__restrict__ val,
+//   C16   : the column ids are stored as 16-bit offsets from x (the caller has moved x to the
+//           workgroup's lowest column); lim = the largest offset that is still inside x
+template <typename VT, int NPT, bool C16>
+__device__ __forceinline__ void wave_products(const void *__restrict__ colv, const VT *__restrict__ val,
                                               const VT *__restrict__ x, int pos, int lane, int *cs,
-                                              typename Acc<VT>::type *vs, typename Acc<VT>::type (&p)[NPT])
+                                              typename Acc<VT>::type *vs, typename Acc<VT>::type (&p)[NPT],
+                                              int lim = 0)
 {
     typedef typename Acc<VT>::type AT;
     // every load instruction reads one contiguous stretch (lane l right after lane l-1): a
     // streamed line is then asked for once, not once per instruction that touches a piece of it
-    if constexpr (sizeof(VT) == 8) {
+    if constexpr (C16) {
+        const unsigned short *col = (const unsigned short *)colv;
+        unsigned short *c16 = (unsigned short *)cs;
+        if constexpr (NPT == 4) {
+            *(v2i32 *)(c16 + 4 * lane) = __builtin_nontemporal_load((const v2i32 *)(col + pos + 4 * lane));
+        } else {
+#pragma unroll
+            for (int q = 0; q < NPT / 8; ++q) {
+                const int e = 512 * q + 8 * lane;
+                *(v4i32 *)(c16 + e) = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
+            }
+        }
+    } else {
+        const int *col = (const int *)colv;
 #pragma unroll
         for (int q = 0; q < NPT / 4; ++q) {
             const int e = 256 * q + 4 * lane;
             *(v4i32 *)(cs + e) = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
         }
+    }
+    if constexpr (sizeof(VT) == 8) {
 #pragma unroll
         for (int q = 0; q < NPT / 2; ++q) {
             const int e = 128 * q + 2 * lane;
             *(v2f64 *)(vs + e) = __builtin_nontemporal_load((const v2f64 *)(val + pos + e));
         }
     } else {
-#pragma unroll
-        for (int q = 0; q < NPT / 4; ++q) {
-            const int e = 256 * q + 4 * lane;
-            *(v4i32 *)(cs + e) = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
-        }
 #pragma unroll
         for (int q = 0; q < NPT / 8; ++q) {
             const int e = 512 * q + 8 * lane;
@@ -141,8 +154,16 @@ __device__ __forceinline__ void wave_products(const int *__restrict__ col, const
     }
     __builtin_amdgcn_wave_barrier();
     AT xv[NPT];
+    if constexpr (C16) {
+        const unsigned short *c16 = (const unsigned short *)cs;
 #pragma unroll
-    for (int j = 0; j < NPT; ++j) xv[j] = (AT)x[cs[64 * j + lane]];
+        // entries of the neighbouring workgroups share the wave's aligned loads; their offsets
+        // belong to another base, so keep them inside x (their products are dropped later)
+        for (int j = 0; j < NPT; ++j) xv[j] = (AT)x[min((int)c16[64 * j + lane], lim)];
+    } else {
+#pragma unroll
+        for (int j = 0; j < NPT; ++j) xv[j] = (AT)x[cs[64 * j + lane]];
+    }
 #pragma unroll
     for (int j = 0; j < NPT; ++j) p[j] = vs[64 * j + lane] * xv[j];
 }
@@ -176,12 +197,15 @@ __device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, 
 // LDS.  Phase 2 sums each row from LDS with W lanes per row, W picked from the mean row length
 // of the tile; it touches global memory only to store y.  A row longer than a tile is swept
 // tile by tile with the same loads, each lane keeping a running sum.  col/val are padded by
-// the host so that aligned 128-bit loads may run past the end.
-template <typename VT, int NPT, bool XCD>
-__global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict__ rowPtr, const int *__restrict__ col,
-                                                          const VT *__restrict__ val, const VT *__restrict__ x,
+// the host so that aligned 128-bit loads may run past the end.  With C16 the column ids are
+// 16-bit offsets from colBase[workgroup] (the host uses this form when the columns of every
+// workgroup span fewer than 65536), which takes a third off the bytes of an FP16 entry and
+// a sixth off an FP64 one.
+template <typename VT, int NPT, bool XCD, bool C16>
+__global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict__ rowPtr, const void *__restrict__ col,
+                                                          const VT *__restrict__ val, const VT *__restrict__ xfull,
                                                           VT *__restrict__ y, const int4 *__restrict__ blockDesc,
-                                                          int accumulate)
+                                                          const int *__restrict__ colBase, int xcols, int accumulate)
 {
     typedef typename Acc<VT>::type AT;
     constexpr int TILE = kBlock * NPT;
@@ -197,6 +221,9 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
     const int r0 = d.x, r1 = d.y, p0 = d.z, p1 = d.w;
     const int nrows = r1 - r0;
     if (nrows <= 0) return;
+    const int cb = C16 ? colBase[b] : 0;
+    const VT *x = xfull + cb;
+    const int lim = xcols - 1 - cb;
     const int base = p0 & ~(NPT - 1);
     int *cs = cols + wave * WTILE;
     AT *vs = prod + wave * WTILE;
@@ -211,7 +238,7 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
         }
         if (base + wave * WTILE < p1) {
             AT p[NPT];
-            wave_products<VT, NPT>(col, val, x, base + wave * WTILE, lane, cs, vs, p);
+            wave_products<VT, NPT, C16>(col, val, x, base + wave * WTILE, lane, cs, vs, p, lim);
 #pragma unroll
             for (int j = 0; j < NPT; ++j) vs[64 * j + lane] = p[j];
         }
@@ -234,7 +261,7 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
         AT s = 0;
         for (int t0 = base + wave * WTILE; t0 < p1; t0 += TILE) {
             AT p[NPT];
-            wave_products<VT, NPT>(col, val, x, t0, lane, cs, vs, p);
+            wave_products<VT, NPT, C16>(col, val, x, t0, lane, cs, vs, p, lim);
 #pragma unroll
             for (int j = 0; j < NPT; ++j) {
                 const int e = t0 + 64 * j + lane;
@@ -676,8 +703,14 @@ namespace mx {
 template <typename VT, int NPT>
 static void launch_csr_t(const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
 {
-    hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr, A.col,
-                       (const VT *)A.val, (const VT *)x, (VT *)y, (const int4 *)A.blockDesc, accumulate);
+    if (A.col16)
+        hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, true>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr,
+                           (const void *)A.col16, (const VT *)A.val, (const VT *)x, (VT *)y, (const int4 *)A.blockDesc,
+                           A.colBase, A.cols, accumulate);
+    else
+        hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, false>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr,
+                           (const void *)A.col, (const VT *)A.val, (const VT *)x, (VT *)y, (const int4 *)A.blockDesc,
+                           (const int *)nullptr, A.cols, accumulate);
 }
 
 hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)

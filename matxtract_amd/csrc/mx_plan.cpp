@@ -2,6 +2,7 @@
 // hybrid SpMV; plus the reference's one-shot host-pointer entry points built on top.
 #include <algorithm>
 #include <chrono>
+#include <climits>
 #include <cstdlib>
 #include <cstring>
 #include <numeric>
@@ -75,6 +76,8 @@ void free_csr(mx::DeviceCsr &A)
 {
     (void)hipFree(A.rowPtr);
     (void)hipFree(A.col);
+    (void)hipFree(A.col16);
+    (void)hipFree(A.colBase);
     (void)hipFree(A.val);
     (void)hipFree(A.blockDesc);
     A = mx::DeviceCsr();
@@ -285,24 +288,59 @@ int upload_tiles(mx_dtype dtype, int chunkNum, const char *sel, int dRows, const
     return MX_OK;
 }
 
-int upload_csr(mx_dtype dtype, int rows, int nnz, const int *rowPtr, const int *col, const void *val,
+int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, const int *col, const void *val,
                mx::DeviceCsr &A, double *pack_ms)
 {
     const int es = mx::elem_size(dtype), npt = mx::csr_entries_per_lane(dtype);
     A.rows = rows;
+    A.cols = cols;
     A.npt = npt;
     A.nnz = nnz;
     int rc;
     if ((rc = upload(&A.rowPtr, rowPtr, (size_t)rows + 1))) return rc;
-    if ((rc = upload(&A.col, col, (size_t)nnz, mx::kCsrPad))) return rc;
     if ((rc = upload_bytes(&A.val, val, (size_t)nnz * es, (size_t)mx::kCsrPad * es))) return rc;
     std::vector<int> desc;
     auto t0 = std::chrono::steady_clock::now();
     pack_rows(rowPtr, rows, npt, desc);
-    auto t1 = std::chrono::steady_clock::now();
-    if (pack_ms) *pack_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
     A.nBlocks = (int)desc.size() / 4;
     if ((rc = upload(&A.blockDesc, desc.data(), desc.size()))) return rc;
+    // 16-bit column offsets when every workgroup's columns span fewer than 65536
+    // (MX_CSR_COL16=0 keeps 32-bit ids)
+    const char *env16 = std::getenv("MX_CSR_COL16");
+    bool narrow = !(env16 && std::atoi(env16) == 0) && nnz > 0;
+    std::vector<int> cbase((size_t)A.nBlocks, 0);
+    if (narrow) {
+        int wide = 0;
+#pragma omp parallel for schedule(static) reduction(+ : wide)
+        for (int b = 0; b < A.nBlocks; ++b) {
+            const int p0 = desc[4 * (size_t)b + 2], p1 = desc[4 * (size_t)b + 3];
+            int lo = INT_MAX, hi = 0;
+            for (int p = p0; p < p1; ++p) {
+                lo = std::min(lo, col[p]);
+                hi = std::max(hi, col[p]);
+            }
+            if (p1 > p0) {
+                cbase[b] = lo;
+                wide += hi - lo > 65535;
+            }
+        }
+        narrow = wide == 0;
+    }
+    if (narrow) {
+        std::vector<unsigned short> c16((size_t)nnz);
+#pragma omp parallel for schedule(static)
+        for (int b = 0; b < A.nBlocks; ++b)
+            for (int p = desc[4 * (size_t)b + 2]; p < desc[4 * (size_t)b + 3]; ++p)
+                c16[p] = (unsigned short)(col[p] - cbase[b]);
+        void *d16 = nullptr;
+        if ((rc = upload_bytes(&d16, c16.data(), (size_t)nnz * 2, (size_t)mx::kCsrPad * 2))) return rc;
+        A.col16 = (unsigned short *)d16;
+        if ((rc = upload(&A.colBase, cbase.data(), cbase.size()))) return rc;
+    } else {
+        if ((rc = upload(&A.col, col, (size_t)nnz, mx::kCsrPad))) return rc;
+    }
+    auto t1 = std::chrono::steady_clock::now();
+    if (pack_ms) *pack_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
     return MX_OK;
 }
 
@@ -410,7 +448,7 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
         want_rows = true;
     }
     int rc;
-    if (want_rows && (rc = upload_csr(plan->dtype, rows, nnz, rowPtr, col, val, plan->csr, nullptr))) return rc;
+    if (want_rows && (rc = upload_csr(plan->dtype, rows, plan->cols, nnz, rowPtr, col, val, plan->csr, nullptr))) return rc;
     if (want_slices && (rc = upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, plan->slices))) return rc;
     plan->use_slices = want_slices && !want_rows;
     if (want_rows && want_slices) {
@@ -716,7 +754,7 @@ static int cdspmv_any(mx_dtype dtype, const void *csrVal, const int *csrRowPtr, 
     void *dx = nullptr, *dy = nullptr, *dscratch = nullptr;
     auto body = [&]() -> int {
         double pre = 0.0;
-        int r = upload_csr(dtype, rows, nnz, csrRowPtr, csrColInd, csrVal, plan.csr, &pre);
+        int r = upload_csr(dtype, rows, cols, nnz, csrRowPtr, csrColInd, csrVal, plan.csr, &pre);
         if (r) return r;
         if (cdPre) *cdPre = pre;
         if ((r = upload_bytes(&dx, x, cols * es))) return r;
