@@ -237,6 +237,42 @@ def test_ragged_and_degenerate_shapes(mx, ora):
                 part.close()
 
 
+@pytest.mark.parametrize("span", [65535, 65536, 200])
+def test_row_kernel_column_widths(mx, ora, span, monkeypatch):
+    """The row kernel stores columns as 16-bit offsets when every workgroup's span allows it and
+    as 32-bit ids otherwise; both forms, with columns reaching the last element of x."""
+    import torch
+    rng = np.random.default_rng(span)
+    rows, cols = 700, 70000
+    lens = rng.integers(1, 12, rows)
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    chunks = []
+    for r, l in enumerate(lens):
+        # wide spans: every row reaches the last column; span 200: a band, so that workgroups
+        # have different bases
+        lo = cols - 1 - span if span > 60000 else min(r * 99, cols - 1 - span)
+        c = np.sort(rng.choice(np.arange(lo, lo + span + 1), l, replace=False))
+        if r == 0:
+            c[0], c[-1] = lo, lo + span  # the first workgroup's span is exactly `span`
+        chunks.append(c)
+    chunks[-1][-1] = cols - 1
+    ci = np.concatenate(chunks).astype(np.int32)
+    for dtype, tol in ((np.float64, F64_TOL), (np.float16, F16_TOL)):
+        A = mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, rp[-1]).astype(dtype))
+        x = rng.uniform(-1, 1, cols).astype(dtype)
+        ref = oracle_y(ora, mx, A, x)
+        for env in ("1", "0"):
+            print("column width span=%d dtype=%s MX_CSR_COL16=%s" % (span, dtype.__name__, env), flush=True)
+            monkeypatch.setenv("MX_CSR_COL16", env)
+            part = mx.Partition(A, 0.0, 0.0)
+            plan = mx.Plan(part, mx.MX_PLAN_CSR_ROWS)
+            y = plan.spmv(torch.from_numpy(x).cuda())
+            torch.cuda.synchronize()
+            assert rel_l2(y.cpu().numpy(), ref) <= tol
+            plan.close()
+            part.close()
+
+
 def test_long_rows_take_the_multi_tile_path(mx, ora):
     """One row far longer than a workgroup tile, next to short ones."""
     import torch
