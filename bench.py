@@ -24,6 +24,15 @@ sys.path.insert(0, ROOT)
 METRIC = "SpMV GFLOP/s (2·nnz/t) + % of HBM roofline, FP64 and FP16, 1 GPU"
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 GRID = (0.0, 0.25, 0.5, 0.75, 1.0)
+# HBM-side bytes per launch (read + written) of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE runs of this script, each counter scaled by what it reads for an elementwise kernel of
+# known size (--calibrate-copy): FETCH_SIZE x 2.000, WRITE_SIZE x 1.000.  The text files under profiles/
+# hold the counter values.  (workload, kernel) -> bytes
+TRAFFIC = {
+    (2, "csr_rows_kernel<f64>"): 47183402,
+    (2, "csr_slice_kernel<f64>"): 54402556,
+    (3, "csr_rows_kernel<f64>"): 287447594,
+}
 WORKLOADS = {
     1: "configs[0]: FP64 random 4096x4096, 16 nnz/row",
     2: "configs[1]: FP64 block-clustered 65536x65536, ~64 nnz/row, 40% of nnz in dense 8x8 blocks in a 2048-wide band",
@@ -136,7 +145,8 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline):
         "csr_only_ms": csr_only["ms_total"],
         "best_hybrid": best_hybrid and {k: best_hybrid[k] for k in ("tau_c", "tau_r", "ms_total", "tile_nnz", "csr_nnz")},
         "roofline": {"bound": "hbm", "kernel": dom["kernel"], "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": None,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK,
+                     "traffic": TRAFFIC.get((cfg, dom["kernel"])) if (tau == (0.0, 0.0) or info["tile_nnz"] == 0) else None,
                      "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"]},
         "sweep": [{k: r[k] for k in ("tau_c", "tau_r", "ms_total", "ms_tile", "ms_csr", "tile_nnz")} for r in table],
     }
