@@ -28,6 +28,7 @@ typedef int v2i32 __attribute__((ext_vector_type(2)));
 constexpr int kBlock = 256;  // 4 wave64 per workgroup
 using mx::kSliceBytes;
 using mx::kSliceThreads;
+using mx::kSliceWaves;
 
 // Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
 // Re-map so that every XCD walks one contiguous range of logical blocks: neighbouring rows
@@ -170,9 +171,11 @@ __device__ __forceinline__ void wave_products(const void *__restrict__ colv, con
 
 // Sums the rows of one tile out of LDS: W lanes per row, `rowOff` holds the rows' start
 // offsets inside the tile (nrows+1 entries).
+// rowOut (LDS, may be null) names the output row of each of the tile's rows.
 template <typename VT, int W>
-__device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, const unsigned short *rowOff, int r0, int nrows,
-                                            VT *__restrict__ y, int accumulate, int tid)
+__device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, const unsigned short *rowOff,
+                                            const int *rowOut, int r0, int nrows, VT *__restrict__ y, int accumulate,
+                                            int tid)
 {
     typedef typename Acc<VT>::type AT;
     constexpr int rowsPerPass = kBlock / W;
@@ -183,8 +186,9 @@ __device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, 
         for (int i = a + l; i < b; i += W) s += prod[i];
         s = group_sum<W>(s);
         if (l == 0) {
-            if (accumulate) s += (AT)y[r0 + rr];
-            y[r0 + rr] = (VT)s;
+            const int o = rowOut ? rowOut[rr] : r0 + rr;
+            if (accumulate) s += (AT)y[o];
+            y[o] = (VT)s;
         }
     }
 }
@@ -201,11 +205,14 @@ __device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, 
 // 16-bit offsets from colBase[workgroup] (the host uses this form when the columns of every
 // workgroup span fewer than 65536), which takes a third off the bytes of an FP16 entry and
 // a sixth off an FP64 one.
-template <typename VT, int NPT, bool XCD, bool C16>
+// With PERM the rows are walked in an order of the host's choosing and rowIdx names the output
+// row of each.
+template <typename VT, int NPT, bool XCD, bool C16, bool PERM>
 __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict__ rowPtr, const void *__restrict__ col,
                                                           const VT *__restrict__ val, const VT *__restrict__ xfull,
                                                           VT *__restrict__ y, const int4 *__restrict__ blockDesc,
-                                                          const int *__restrict__ colBase, int xcols, int accumulate)
+                                                          const int *__restrict__ colBase,
+                                                          const int *__restrict__ rowIdx, int xcols, int accumulate)
 {
     typedef typename Acc<VT>::type AT;
     constexpr int TILE = kBlock * NPT;
@@ -213,7 +220,9 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
     __shared__ __attribute__((aligned(16))) AT prod[TILE];
     __shared__ __attribute__((aligned(16))) int cols[TILE];
     __shared__ unsigned short rowOff[TILE + 2];  // offsets inside the tile fit 16 bits
+    __shared__ int rowOutS[PERM ? TILE : 1];
     __shared__ AT wsum[kBlock / 64];
+    const int *rowOut = PERM ? rowOutS : nullptr;
 
     const int b = XCD ? xcd_contiguous_block(blockIdx.x, gridDim.x) : (int)blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -230,11 +239,12 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
 
     if (p1 - base <= TILE) {
         // row offsets: lane t takes rows t, t+256, ... (at most NPT+1 of them)
-        int ro[NPT + 1];
+        int ro[NPT + 1], rx[PERM ? NPT : 1];
 #pragma unroll
         for (int k = 0; k <= NPT; ++k) {
             const int rr = tid + k * kBlock;
             ro[k] = rr <= nrows ? rowPtr[r0 + rr] : 0;
+            if (PERM && k < NPT) rx[k] = rr < nrows ? rowIdx[r0 + rr] : 0;
         }
         if (base + wave * WTILE < p1) {
             AT p[NPT];
@@ -246,16 +256,17 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
         for (int k = 0; k <= NPT; ++k) {
             const int rr = tid + k * kBlock;
             if (rr <= nrows) rowOff[rr] = (unsigned short)(ro[k] - base);
+            if (PERM && k < NPT && rr < nrows) rowOutS[rr] = rx[k];
         }
         __syncthreads();
         const int mean = (p1 - p0) / nrows;
-        if (mean <= 2) reduce_rows<VT, 1>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 4) reduce_rows<VT, 2>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 8) reduce_rows<VT, 4>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 16) reduce_rows<VT, 8>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 32) reduce_rows<VT, 16>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 64) reduce_rows<VT, 32>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else reduce_rows<VT, 64>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        if (mean <= 2) reduce_rows<VT, 1>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
+        else if (mean <= 4) reduce_rows<VT, 2>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
+        else if (mean <= 8) reduce_rows<VT, 4>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
+        else if (mean <= 16) reduce_rows<VT, 8>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
+        else if (mean <= 32) reduce_rows<VT, 16>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
+        else if (mean <= 64) reduce_rows<VT, 32>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
+        else reduce_rows<VT, 64>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
     } else {
         // a single row longer than one tile
         AT s = 0;
@@ -276,156 +287,188 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
             AT t = 0;
 #pragma unroll
             for (int w = 0; w < kBlock / 64; ++w) t += wsum[w];
-            if (accumulate) t += (AT)y[r0];
-            y[r0] = (VT)t;
+            const int o = PERM ? rowIdx[r0] : r0;
+            if (accumulate) t += (AT)y[o];
+            y[o] = (VT)t;
         }
     }
 }
 
 // ---- CSR part, x resident in LDS ----------------------------------------------------------
-// For matrices whose x gathers are scattered, a gather from L2 moves a whole 128-byte line
-// for one value, a CU can keep only ~64 KB of such requests in flight, and the kernel is bound
-// by that instead of HBM.  When x is small enough, the gathers can be served from LDS instead:
-// the columns are cut into S slices of kSliceBytes of x, the rows into G groups, and workgroup
-// (g, s) -- one per CU -- copies slice s into LDS once, then streams the entries of its rows
-// that fall into the slice (16-bit row and column offsets plus the value, 128-bit loads, the
-// next pass already in flight), gathers x from LDS and adds the products to per-row
-// accumulators in LDS (ds_add_f64 / ds_add_f32; consecutive entries of one row are summed in
-// registers first).  The rows of a group are handled in sub-blocks that fit the accumulators.
-// With S > 1 every workgroup owns one column of a [S][rows] array of partial sums, written
-// once, coalesced, and a second small kernel adds the S partials of each row; with S = 1 the
-// workgroup stores y itself.  No global atomics in either case.
-struct SubBlock {  // rows [row0, row0+nrows) of the matrix, entries [e0, e1) of this workgroup
-    int row0, nrows, e0, e1;
+// For matrices whose x gathers are scattered, every gather from L2 moves a whole 128-byte line
+// for one value and a CU can keep only so many of those in flight: the kernel is bound by that
+// instead of HBM.  When x is small enough the gathers can be served from LDS instead.  The
+// columns are cut into S slices (a slice of x fits LDS), the rows into G groups, and workgroup
+// (g, s) -- one per CU -- copies slice s into LDS once and then streams the entries of its
+// rows that fall into the slice.  Those are laid out as sliced ELL (see DeviceSlices): one row
+// per lane, E entries per lane per step, steps contiguous across the wave, so a lane sums its
+// row in a register with no cross-lane traffic at all, and at the end of a chunk of 64 rows
+// every lane stores one sum.  With S > 1 the sums go to one column of a [S][rows] array of
+// partial sums and a second small kernel adds the S partials of each row; with S = 1 the
+// workgroup stores y itself.  No atomics in either case.
+template <typename VT>
+struct SliceBatch;  // what one lane reads per batch: 8 column offsets, 8 values
+template <>
+struct SliceBatch<double> {
+    static constexpr int E = 2, SPB = 4;  // entries per step, steps per batch
+    v4i32 c;
+    v2f64 v[4];
+    __device__ __forceinline__ void load(const unsigned short *ecol, const double *eval, size_t batch, int lane)
+    {
+        c = __builtin_nontemporal_load((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            v[j] = __builtin_nontemporal_load((const v2f64 *)(eval + batch * 512 + j * 128 + lane * 2));
+    }
+    __device__ __forceinline__ double dot(const double *xs, int j) const
+    {
+        const unsigned w = (unsigned)c[j];
+        return v[j].x * xs[w & 0xffffu] + v[j].y * xs[w >> 16];
+    }
 };
-
-// Eight entries of one lane: row offsets, column offsets (16 bit each, packed) and values.
-template <typename VT>
-struct EntryRegs {
-    v4i32 r, c;
-    v4i32 v[sizeof(VT) == 8 ? 4 : 1];
+template <>
+struct SliceBatch<_Float16> {
+    static constexpr int E = 4, SPB = 2;
+    v4i32 c, v;
+    __device__ __forceinline__ void load(const unsigned short *ecol, const _Float16 *eval, size_t batch, int lane)
+    {
+        c = __builtin_nontemporal_load((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
+        v = __builtin_nontemporal_load((const v4i32 *)(eval + (batch * 64 + lane) * 8));
+    }
+    __device__ __forceinline__ float dot(const _Float16 *xs, int j) const
+    {
+        const unsigned c0 = (unsigned)c[2 * j], c1 = (unsigned)c[2 * j + 1];
+        const unsigned v0 = (unsigned)v[2 * j], v1 = (unsigned)v[2 * j + 1];
+        auto h = [](unsigned bits) { return (float)__builtin_bit_cast(_Float16, (unsigned short)bits); };
+        return h(v0 & 0xffffu) * (float)xs[c0 & 0xffffu] + h(v0 >> 16) * (float)xs[c0 >> 16] +
+               h(v1 & 0xffffu) * (float)xs[c1 & 0xffffu] + h(v1 >> 16) * (float)xs[c1 >> 16];
+    }
 };
+static_assert(mx::kSliceBatchEntries == 8, "SliceBatch holds 8 entries per lane");
+
+// What a CU can take in from L2 or beyond is bounded in bytes (about 32 per cycle, whatever
+// the width of the loads), so nothing is loaded that is not needed: a lane keeps up to kSliceRing
+// batches in flight, streams no longer than the ring are loaded whole before anything else
+// happens; longer ones run a loop in which every consumed batch is reloaded with the batch one
+// ring length ahead (those reloads are unconditional inside the loop, so the number of loads
+// in flight is known at compile time and no wait is longer than it has to be), and a tail.
+// The sums of finished chunks are parked in LDS and leave the workgroup in one coalesced sweep.
+constexpr int kSliceRing = 6;
 
 template <typename VT>
-__device__ __forceinline__ void load_entries(EntryRegs<VT> &en, const unsigned short *__restrict__ erow,
-                                             const unsigned short *__restrict__ ecol, const VT *__restrict__ eval, int e)
-{
-    en.r = __builtin_nontemporal_load((const v4i32 *)(erow + e));
-    en.c = __builtin_nontemporal_load((const v4i32 *)(ecol + e));
-    if constexpr (sizeof(VT) == 8) {
-        // binary64 values are stored permuted inside every 512-entry block of a group so that
-        // each of the four loads is contiguous across the wave: piece q of lane l (entries
-        // 8l+2q, 8l+2q+1 of the block) sits at block + 128q + 2l
-        const int lane = threadIdx.x & 63;
-        const VT *blk = eval + (e - 8 * lane);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) en.v[q] = __builtin_nontemporal_load((const v4i32 *)(blk + 128 * q + 2 * lane));
-    } else {
-        en.v[0] = __builtin_nontemporal_load((const v4i32 *)(eval + e));
-    }
-}
-
-// gather x from LDS, sum runs of equal rows in registers, add to the accumulators
-template <typename VT>
-__device__ __forceinline__ void consume_entries(const EntryRegs<VT> &en, const VT *xs, typename Acc<VT>::type *acc)
-{
-    typedef typename Acc<VT>::type AT;
-    unsigned r[8];
-    AT prod[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const unsigned rw = (unsigned)en.r[j >> 1], cw = (unsigned)en.c[j >> 1];
-        r[j] = (j & 1) ? rw >> 16 : rw & 0xffffu;
-        const unsigned c = (j & 1) ? cw >> 16 : cw & 0xffffu;
-        AT v;
-        if constexpr (sizeof(VT) == 8) {
-            const v2f64 t = __builtin_bit_cast(v2f64, en.v[j >> 1]);
-            v = (j & 1) ? t.y : t.x;
-        } else {
-            const unsigned w = (unsigned)en.v[0][j >> 1];
-            v = (float)__builtin_bit_cast(_Float16, (unsigned short)((j & 1) ? w >> 16 : w & 0xffffu));
-        }
-        prod[j] = v * (AT)xs[c];
-    }
-    AT run = prod[0];
-    unsigned cur = r[0];
-#pragma unroll
-    for (int j = 1; j < 8; ++j) {
-        if (r[j] == cur) {
-            run += prod[j];
-        } else {
-            __hip_atomic_fetch_add(&acc[cur], run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            cur = r[j];
-            run = prod[j];
-        }
-    }
-    __hip_atomic_fetch_add(&acc[cur], run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-}
-
-template <typename VT>
-__global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int *__restrict__ wgSubPtr,
-                                                                  const SubBlock *__restrict__ subs,
-                                                                  const unsigned short *__restrict__ erow,
+__global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__restrict__ wgDesc,
+                                                                  const int4 *__restrict__ waveDesc,
+                                                                  const int *__restrict__ chunkEnd,
+                                                                  const unsigned short *__restrict__ chunkRows,
                                                                   const unsigned short *__restrict__ ecol,
                                                                   const VT *__restrict__ eval, const VT *__restrict__ x,
                                                                   typename Acc<VT>::type *__restrict__ partial,
                                                                   VT *__restrict__ y, int rows, int cols, int S,
-                                                                  int accumulate)
+                                                                  int sliceCols, int maxGroupRows, int accumulate)
 {
     typedef typename Acc<VT>::type AT;
-    constexpr int SW = kSliceBytes / (int)sizeof(VT);      // columns per slice
-    constexpr int VPT = kSliceBytes / 16 / kSliceThreads;  // 16-byte vectors per lane for the slice copy
+    typedef SliceBatch<VT> Batch;
+    constexpr int SPB = Batch::SPB, NB = kSliceRing;
     constexpr int EPV = 16 / (int)sizeof(VT);
-    constexpr int PASS = kSliceThreads * 8;                // entries per pass of the workgroup
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    VT *xs = (VT *)smem;
-    AT *acc = (AT *)(smem + kSliceBytes);
+    VT *xs = (VT *)smem;                                                   // [sliceCols]
+    AT *ybuf = (AT *)(smem + (size_t)sliceCols * sizeof(VT));              // [maxGroupRows] sums by group row
+    unsigned short *rowsL = (unsigned short *)(ybuf + maxGroupRows);       // [chunks of the workgroup][64]
+    int *endsL = (int *)(rowsL + ((maxGroupRows + 63) / 64) * 64);         // [chunks of the workgroup]
 
-    const int b = blockIdx.x, tid = threadIdx.x;
-    const int slice = b % S;
-    const int s0 = wgSubPtr[b], s1 = wgSubPtr[b + 1];
-    // lanes are never moved to another entry: load_entries derives the wave's block from
-    // "entry - 8*lane"; a lane past the end simply does not load
-    EntryRegs<VT> cur, nxt;
-    SubBlock d = s0 < s1 ? subs[s0] : SubBlock{0, 0, 0, 0};
-    int e = d.e0 + tid * 8;
-    if (e < d.e1) load_entries(cur, erow, ecol, eval, e);  // the first pass travels while the slice is copied
-    {
-        v4i32 xv[VPT];
+    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int4 gd = wgDesc[b];
+    const int4 d = waveDesc[b * kSliceWaves + wave];
+    const int row0 = gd.x, nr = gd.y, slice = gd.z, wgChunk0 = gd.w;
+    const int batch0 = __builtin_amdgcn_readfirstlane(d.x), nb = __builtin_amdgcn_readfirstlane(d.y);
+    const int chunk0 = __builtin_amdgcn_readfirstlane(d.z), nChunks = __builtin_amdgcn_readfirstlane(d.w);
+    const int wgChunks = (nr + 63) / 64;
+    // row ids and chunk ends of the workgroup, and the slice (all of it at once, one 16-byte
+    // vector per lane and round)
+    unsigned short rl[2];
+    const int ridx = 2 * tid;  // 512 lanes * 2 = 1024 ... more rows go round again below
+    *(unsigned *)rl = ridx < wgChunks * 64 ? *(const unsigned *)(chunkRows + (size_t)wgChunk0 * 64 + ridx) : 0xffffffffu;
+    const int ce = tid < wgChunks ? chunkEnd[wgChunk0 + tid] : 0;
+    constexpr int CB = kSliceBytes / 16 / kSliceThreads;  // rounds of a full slice
+    const int nvec = sliceCols / EPV;
+    v4i32 xv[CB];
 #pragma unroll
-        for (int q = 0; q < VPT; ++q) {
-            const int c = slice * SW + (q * kSliceThreads + tid) * EPV;
-            xv[q] = c + EPV <= cols ? *(const v4i32 *)(x + c) : v4i32{0, 0, 0, 0};
-        }
-#pragma unroll
-        for (int q = 0; q < VPT; ++q) *(v4i32 *)(xs + (q * kSliceThreads + tid) * EPV) = xv[q];
+    for (int q = 0; q < CB; ++q) {
+        const int i = tid + q * kSliceThreads;
+        const int c = slice * sliceCols + i * EPV;
+        xv[q] = v4i32{0, 0, 0, 0};
+        if (i < nvec && c + EPV <= cols) xv[q] = *(const v4i32 *)(x + c);
     }
-    for (int sb = s0; sb < s1; ++sb) {
-        if (sb > s0) {
-            d = subs[sb];
-            e = d.e0 + tid * 8;
-            if (e < d.e1) load_entries(cur, erow, ecol, eval, e);
+    {
+        if (ridx < wgChunks * 64) *(unsigned *)(rowsL + ridx) = *(unsigned *)rl;
+        if (tid < wgChunks) endsL[tid] = ce;
+        for (int i = 2 * kSliceThreads + 2 * tid; i < wgChunks * 64; i += 2 * kSliceThreads)
+            *(unsigned *)(rowsL + i) = *(const unsigned *)(chunkRows + (size_t)wgChunk0 * 64 + i);
+        for (int i = kSliceThreads + tid; i < wgChunks; i += kSliceThreads) endsL[i] = chunkEnd[wgChunk0 + i];
+#pragma unroll
+        for (int q = 0; q < CB; ++q) {
+            const int i = tid + q * kSliceThreads;
+            if (i < nvec) *(v4i32 *)(xs + i * EPV) = xv[q];
         }
-        for (int i = tid; i < d.nrows; i += kSliceThreads) acc[i] = 0;
-        __syncthreads();  // accumulators cleared (and, the first time, the slice in place)
-        for (; e < d.e1; e += PASS) {
-            const bool more = e + PASS < d.e1;
-            if (more) load_entries(nxt, erow, ecol, eval, e + PASS);
-            consume_entries<VT>(cur, xs, acc);
-            if (more) cur = nxt;
+        // ragged end of x: the last, partial vector is filled element by element
+        if (cols % EPV) {
+            const int c = cols - cols % EPV, i = (c - slice * sliceCols) / EPV;
+            if (c >= slice * sliceCols && i < nvec && tid < EPV) xs[i * EPV + tid] = tid < cols % EPV ? x[c + tid] : (VT)0;
         }
-        __syncthreads();
-        if (S > 1) {
-            AT *out = partial + (size_t)slice * rows + d.row0;
-            for (int i = tid; i < d.nrows; i += kSliceThreads) out[i] = acc[i];
-        } else {
-            for (int i = tid; i < d.nrows; i += kSliceThreads) {
-                AT sum = acc[i];
-                if (accumulate) sum += (AT)y[d.row0 + i];
-                y[d.row0 + i] = (VT)sum;
-            }
+    }
+    // the ring is issued only now: a wave that is busy issuing loads cannot store the slice, and
+    // the address unit takes the loads no faster than their data moves
+    Batch buf[NB];
+#pragma unroll
+    for (int k = 0; k < NB; ++k)
+        if (k < nb) buf[k].load(ecol, eval, (size_t)(batch0 + k), lane);
+    __syncthreads();
+    int ci = 0;
+    int nextEnd = nChunks > 0 ? endsL[chunk0] : -1;
+    AT acc = 0;
+    auto flush = [&]() {
+        const int r = rowsL[(chunk0 + ci) * 64 + lane];
+        if (r != 0xffff) ybuf[r] = acc;
+        acc = 0;
+        ++ci;
+        nextEnd = ci < nChunks ? endsL[chunk0 + ci] : -1;
+    };
+    auto consume = [&](const Batch &B, int t) {  // t = number of the batch in the wave's stream
+#pragma unroll
+        for (int j = 0; j < SPB; ++j) {
+            acc += B.dot(xs, j);
+            if (t * SPB + j + 1 == nextEnd) flush();
         }
-        __syncthreads();  // accumulators free for the next sub-block
+    };
+    int t = 0;
+    // while a whole ring beyond the one in flight remains: consume and reload, no conditions
+    for (; t + 2 * NB <= nb; t += NB) {
+#pragma unroll
+        for (int k = 0; k < NB; ++k) {
+            consume(buf[k], t + k);
+            buf[k].load(ecol, eval, (size_t)(batch0 + t + NB + k), lane);
+        }
+    }
+    // tail: what is in flight, reloading while batches remain, then those
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+        if (t + k < nb) consume(buf[k], t + k);
+        if (t + NB + k < nb) buf[k].load(ecol, eval, (size_t)(batch0 + t + NB + k), lane);
+    }
+#pragma unroll
+    for (int k = 0; k < NB; ++k)
+        if (t + NB + k < nb) consume(buf[k], t + NB + k);
+    while (ci < nChunks) flush();  // chunks of empty rows
+    __syncthreads();
+    if (S <= 1) {
+        for (int i = tid; i < nr; i += kSliceThreads) {
+            AT sum = ybuf[i];
+            if (accumulate) sum += (AT)y[row0 + i];
+            y[row0 + i] = (VT)sum;
+        }
+    } else {
+        for (int i = tid; i < nr; i += kSliceThreads) partial[(size_t)slice * rows + row0 + i] = ybuf[i];
     }
 }
 
@@ -703,14 +746,15 @@ namespace mx {
 template <typename VT, int NPT>
 static void launch_csr_t(const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
 {
-    if (A.col16)
-        hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, true>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr,
-                           (const void *)A.col16, (const VT *)A.val, (const VT *)x, (VT *)y, (const int4 *)A.blockDesc,
-                           A.colBase, A.cols, accumulate);
-    else
-        hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, false>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s, A.rowPtr,
-                           (const void *)A.col, (const VT *)A.val, (const VT *)x, (VT *)y, (const int4 *)A.blockDesc,
-                           (const int *)nullptr, A.cols, accumulate);
+#define MX_LAUNCH_ROWS(C16, PERM, COLS, BASE)                                                                       \
+    hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, C16, PERM>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s,      \
+                       A.rowPtr, (const void *)(COLS), (const VT *)A.val, (const VT *)x, (VT *)y,                      \
+                       (const int4 *)A.blockDesc, (const int *)(BASE), (const int *)A.rowIdx, A.cols, accumulate)
+    if (A.col16 && A.rowIdx) MX_LAUNCH_ROWS(true, true, A.col16, A.colBase);
+    else if (A.col16) MX_LAUNCH_ROWS(true, false, A.col16, A.colBase);
+    else if (A.rowIdx) MX_LAUNCH_ROWS(false, true, A.col, nullptr);
+    else MX_LAUNCH_ROWS(false, false, A.col, nullptr);
+#undef MX_LAUNCH_ROWS
 }
 
 hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
@@ -732,19 +776,22 @@ template <typename VT>
 static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, int what)
 {
     typedef typename mxk::Acc<VT>::type AT;
-    const size_t lds = (size_t)kSliceBytes + (size_t)P.maxSubRows * sizeof(AT);
+    const int chunkCap = (P.maxGroupRows + 63) / 64;
+    const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)P.maxGroupRows * sizeof(AT) +
+                       (size_t)chunkCap * 64 * 2 + (size_t)chunkCap * 4 + 64;  // + room for the combine flags
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           mx::kSliceBytes + mx::kSliceAccBytes);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
+    if (lds > (size_t)mx::kSliceLdsMax) return hipErrorInvalidValue;
     if (what != 2)
-        hipLaunchKernelGGL((mxk::csr_slice_kernel<VT>), dim3(P.nWG), dim3(kSliceThreads), lds, s, P.wgSubPtr,
-                           (const mxk::SubBlock *)P.subs, P.erow, P.ecol, (const VT *)P.eval, (const VT *)x,
-                           (AT *)P.partial, (VT *)y, P.rows, P.cols, P.S, accumulate);
+        hipLaunchKernelGGL((mxk::csr_slice_kernel<VT>), dim3(P.nWG), dim3(kSliceThreads), lds, s,
+                           (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.chunkRows, P.ecol,
+                           (const VT *)P.eval, (const VT *)x, (AT *)P.partial, (VT *)y, P.rows, P.cols, P.S, P.sliceCols,
+                           P.maxGroupRows, accumulate);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || P.S <= 1 || what == 1) return e;
     const int grid = std::min(2048, (P.rows + mxk::kBlock - 1) / mxk::kBlock);

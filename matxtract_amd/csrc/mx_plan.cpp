@@ -4,6 +4,7 @@
 #include <chrono>
 #include <climits>
 #include <cstdlib>
+#include <cstdio>
 #include <cstring>
 #include <numeric>
 #include <vector>
@@ -75,6 +76,7 @@ void pack_rows(const int *rowPtr, int rows, int npt, std::vector<int> &desc)
 void free_csr(mx::DeviceCsr &A)
 {
     (void)hipFree(A.rowPtr);
+    (void)hipFree(A.rowIdx);
     (void)hipFree(A.col);
     (void)hipFree(A.col16);
     (void)hipFree(A.colBase);
@@ -96,128 +98,219 @@ void free_tiles(mx::DeviceTiles &T)
 
 void free_slices(mx::DeviceSlices &P)
 {
-    (void)hipFree(P.wgSubPtr);
-    (void)hipFree(P.subs);
-    (void)hipFree(P.erow);
+    (void)hipFree(P.waveDesc);
+    (void)hipFree(P.chunkEnd);
+    (void)hipFree(P.chunkRows);
+    (void)hipFree(P.wgDesc);
     (void)hipFree(P.ecol);
     (void)hipFree(P.eval);
     (void)hipFree(P.partial);
     P = mx::DeviceSlices();
 }
 
-// Number of column slices csr_slice_kernel would need, or 0 when the matrix does not suit it:
-// x is copied in 16-byte vectors (cols must be a whole number of them), and with S slices the
-// kernel writes and re-reads S partial sums per row, which must stay small next to the matrix.
+// Number of column slices csr_slice_kernel would need, or 0 when the matrix does not suit it.
+// With S slices the kernel writes and re-reads S partial sums per row, which must stay small
+// next to the matrix, and its one-row-per-lane layout wants rows that still have a few entries
+// each inside a slice.
 int slice_count(mx_dtype dtype, int rows, int cols, int nnz, int nCU)
 {
-    const int es = mx::elem_size(dtype), epv = 16 / es;
-    if (cols < epv || cols % epv || nnz < 4096) return 0;
+    const int es = mx::elem_size(dtype);
+    if (cols < 1 || rows < 1 || nnz < 4096) return 0;
     const int S = (cols + mx::slice_cols(dtype) - 1) / mx::slice_cols(dtype);
     if (S > nCU) return 0;
     const double accBytes = dtype == MX_F64 ? 8 : 4;
     const double extra = S > 1 ? 2.0 * S * (double)rows * accBytes : 0.0;
-    if (extra > 2.0 * (double)nnz * (es + 4)) return 0;
+    if (extra > 0.5 * (double)nnz * (es + 2)) return 0;
+    if ((double)nnz < 4.0 * (double)rows * S) return 0;
     return S;
 }
 
-// Re-lays a CSR matrix for csr_slice_kernel (see DeviceSlices).  Row groups are balanced by
-// entries; workgroup g*S+s gets group g and slice s.
+// Re-lays a CSR matrix for csr_slice_kernel (see DeviceSlices).
 int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
                   mx::DeviceSlices &D)
 {
-    const int es = mx::elem_size(dtype);
-    const int SW = mx::slice_cols(dtype), subMax = mx::slice_sub_rows(dtype);
-    // groups are padded with zero entries to whole 8-entry lanes; binary64 groups to whole
-    // 512-entry wave blocks, inside which the values are stored permuted (see load_entries)
-    const int gpad = dtype == MX_F64 ? 512 : 8;
+    const int es = mx::elem_size(dtype), E = mx::slice_step_entries(dtype);
+    const int BE = mx::kSliceBatchEntries, SPB = BE / E;  // steps per batch
+    const int SW = mx::slice_cols(dtype), W = mx::kSliceWaves, GR = mx::kSliceGroupRows;
     const int nnz = rowPtr[rows];
-    const int G = std::max(1, nCU / S);
-    // row groups with about nnz/G entries each
-    std::vector<int> groupRow(1, 0);
-    for (int g = 1; g < G; ++g) {
-        const long long target = (long long)nnz * g / G;
-        int r = (int)(std::lower_bound(rowPtr, rowPtr + rows + 1, (int)target) - rowPtr);
-        r = std::min(std::max(r, groupRow.back()), rows);
-        groupRow.push_back(r);
+    // entries sorted by (slice, row), order inside a row kept: seg[q*rows + r] = first entry of
+    // row r in slice q
+    std::vector<int> seg((size_t)S * rows + 1, 0), perm((size_t)nnz);
+    for (int r = 0; r < rows; ++r)
+        for (int p = rowPtr[r]; p < rowPtr[r + 1]; ++p) seg[(size_t)(col[p] / SW) * rows + r + 1]++;
+    for (size_t k = 0; k < (size_t)S * rows; ++k) seg[k + 1] += seg[k];
+    {
+        std::vector<int> cur(seg.begin(), seg.end() - 1);
+        for (int r = 0; r < rows; ++r)
+            for (int p = rowPtr[r]; p < rowPtr[r + 1]; ++p) perm[cur[(size_t)(col[p] / SW) * rows + r]++] = p;
     }
-    groupRow.push_back(rows);
-    // sub-blocks of each group (shared by its S workgroups)
-    std::vector<int> gSubPtr(1, 0), subRow0, subRows;
-    for (int g = 0; g < G; ++g) {
-        for (int r = groupRow[g]; r < groupRow[g + 1]; r += subMax) {
-            subRow0.push_back(r);
-            subRows.push_back(std::min(subMax, groupRow[g + 1] - r));
-        }
-        gSubPtr.push_back((int)subRow0.size());
-    }
-    const int nSubG = (int)subRow0.size();
-    // entry counts per (sub-block, slice), padded to multiples of 8
-    std::vector<long long> cnt((size_t)nSubG * S, 0);
-#pragma omp parallel for schedule(dynamic, 16)
-    for (int i = 0; i < nSubG; ++i) {
-        long long *c = cnt.data() + (size_t)i * S;
-        for (int p = rowPtr[subRow0[i]]; p < rowPtr[subRow0[i] + subRows[i]]; ++p) c[col[p] / SW]++;
-        for (int q = 0; q < S; ++q) c[q] = (c[q] + gpad - 1) / gpad * gpad;
-    }
-    // layout order: workgroup (g, s), then its sub-blocks
-    const int nWG = G * S;
-    std::vector<int> wgSubPtr(1, 0), subs;
-    std::vector<long long> start((size_t)nSubG * S, 0);
-    long long total = 0;
-    int maxSub = 0;
-    for (int g = 0; g < G; ++g)
+    // Workgroups: every slice gets a share of the CUs in proportion to its entries (largest
+    // remainders, at least one each), and cuts the rows into that many groups of about equal
+    // entries *of that slice* -- a slice that holds the diagonal band of some rows would
+    // otherwise give their workgroup several times the work of the others.  No group is longer
+    // than kSliceGroupRows rows.
+    const int minG = (rows + GR - 1) / GR;
+    std::vector<int> Gq(S, 1);
+    {
+        const int budget = std::max(nCU, S);
+        std::vector<double> want(S);
+        int used = 0;
         for (int q = 0; q < S; ++q) {
-            for (int i = gSubPtr[g]; i < gSubPtr[g + 1]; ++i) {
-                start[(size_t)i * S + q] = total;
-                subs.push_back(subRow0[i]);
-                subs.push_back(subRows[i]);
-                subs.push_back((int)total);
-                total += cnt[(size_t)i * S + q];
-                subs.push_back((int)total);
-                maxSub = std::max(maxSub, subRows[i]);
-            }
-            wgSubPtr.push_back((int)(subs.size() / 4));
+            const double nq = (double)(seg[(size_t)(q + 1) * rows] - seg[(size_t)q * rows]);
+            want[q] = nnz > 0 ? nq * budget / nnz : 1.0;
+            Gq[q] = std::max(1, (int)want[q]);
+            used += Gq[q];
         }
-    if (total > 2000000000LL) {
+        while (used < budget) {  // hand out what rounding down left over
+            int best = 0;
+            for (int q = 1; q < S; ++q)
+                if (want[q] - Gq[q] > want[best] - Gq[best]) best = q;
+            ++Gq[best];
+            ++used;
+        }
+        for (int q = 0; q < S; ++q) Gq[q] = std::max(Gq[q], minG);
+    }
+    struct Wg {
+        int slice, row0, nr;
+    };
+    std::vector<Wg> wgs;
+    for (int q = 0; q < S; ++q) {
+        const int *sp = &seg[(size_t)q * rows];
+        const long long nq = sp[rows] - sp[0];
+        int r0 = 0;
+        for (int g = 1; g <= Gq[q] && r0 < rows; ++g) {
+            int r1 = rows;
+            if (g < Gq[q]) {
+                const long long target = sp[0] + nq * g / Gq[q];
+                r1 = (int)(std::lower_bound(sp, sp + rows + 1, (int)target) - sp);
+                r1 = std::min(std::max(r1, r0 + 1), rows);
+            }
+            r1 = std::min(r1, r0 + GR);
+            r1 = std::max(r1, rows - (Gq[q] - g) * GR);  // leave no more than GR rows to each later group
+            wgs.push_back({q, r0, r1 - r0});
+            r0 = r1;
+        }
+        while (r0 < rows) {  // rows the limits above left over
+            const int r1 = std::min(rows, r0 + GR);
+            wgs.push_back({q, r0, r1 - r0});
+            r0 = r1;
+        }
+    }
+    const int nWG = (int)wgs.size();
+    // per workgroup: the sorted rows, their chunks and the chunks' places in the waves' streams
+    struct WgLayout {
+        std::vector<int> sortedRow;   // group-local rows, by entries in the slice, descending
+        std::vector<int> chunkOrder;  // chunks in stream order (wave by wave)
+        std::vector<int> chunkSteps;  // steps of each chunk (indexed by chunk)
+        int waveSteps[mx::kSliceWaves], waveChunks[mx::kSliceWaves];
+        long long steps = 0;
+    };
+    std::vector<WgLayout> lay((size_t)nWG);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int b = 0; b < nWG; ++b) {
+        const int nr = wgs[b].nr;
+        const int *cnt0 = &seg[(size_t)wgs[b].slice * rows + wgs[b].row0];
+        WgLayout &L = lay[b];
+        L.sortedRow.resize(nr);
+        std::iota(L.sortedRow.begin(), L.sortedRow.end(), 0);
+        std::stable_sort(L.sortedRow.begin(), L.sortedRow.end(),
+                         [&](int a, int c) { return cnt0[a + 1] - cnt0[a] > cnt0[c + 1] - cnt0[c]; });
+        const int nc = (nr + 63) / 64;
+        L.chunkSteps.resize(nc);
+        for (int c = 0; c < nc; ++c) {
+            const int lead = L.sortedRow[(size_t)c * 64];
+            L.chunkSteps[c] = (cnt0[lead + 1] - cnt0[lead] + E - 1) / E;
+        }
+        // longest chunk first, each to the wave with the fewest steps so far
+        std::vector<std::vector<int>> mine(W);
+        for (int w = 0; w < W; ++w) L.waveSteps[w] = 0;
+        for (int c = 0; c < nc; ++c) {
+            int best = 0;
+            for (int w = 1; w < W; ++w)
+                if (L.waveSteps[w] < L.waveSteps[best]) best = w;
+            mine[best].push_back(c);
+            L.waveSteps[best] += L.chunkSteps[c];
+        }
+        L.steps = 0;
+        for (int w = 0; w < W; ++w) {
+            L.waveChunks[w] = (int)mine[w].size();
+            L.chunkOrder.insert(L.chunkOrder.end(), mine[w].begin(), mine[w].end());
+            L.steps += (L.waveSteps[w] + SPB - 1) / SPB * SPB;  // a wave's stream is whole batches
+        }
+    }
+    long long totalSteps = 0, totalChunks = 0;
+    std::vector<long long> wgStep((size_t)nWG + 1, 0), wgChunk((size_t)nWG + 1, 0);
+    int maxGroupRows = 0;
+    for (int b = 0; b < nWG; ++b) {
+        wgStep[b] = totalSteps;
+        wgChunk[b] = totalChunks;
+        totalSteps += lay[b].steps;
+        totalChunks += (long long)lay[b].chunkOrder.size();
+        maxGroupRows = std::max(maxGroupRows, wgs[b].nr);
+    }
+    if (totalSteps * 64 * E > 2000000000LL) {
         set_error("slice layout: too many entries for 32-bit offsets");
         return MX_ERR_ARG;
     }
-    // 1024 spare zero entries: a wave may read one whole 512-entry block starting at any entry
-    std::vector<unsigned short> erow((size_t)total + 1024, 0), ecol((size_t)total + 1024, 0);
-    std::vector<unsigned char> ev(((size_t)total + 1024) * es, 0);
+    const size_t padSteps = 16;  // spare zero steps after the last
+    std::vector<unsigned short> ecol(((size_t)totalSteps + padSteps) * 64 * E, 0);
+    std::vector<unsigned char> ev(((size_t)totalSteps + padSteps) * 64 * E * es, 0);
+    std::vector<int> wgDesc((size_t)nWG * 4, 0), waveDesc((size_t)nWG * W * 4, 0), chunkEnd((size_t)totalChunks + 64, 0);
+    std::vector<unsigned short> chunkRows(((size_t)totalChunks + 1) * 64, 0xffff);
     const unsigned char *sv = (const unsigned char *)val;
-#pragma omp parallel
-    {
-        std::vector<long long> cursor(S);
-#pragma omp for schedule(dynamic, 16)
-        for (int i = 0; i < nSubG; ++i) {
-            std::copy(start.begin() + (size_t)i * S, start.begin() + (size_t)(i + 1) * S, cursor.begin());
-            for (int r = subRow0[i]; r < subRow0[i] + subRows[i]; ++r)
-                for (int p = rowPtr[r]; p < rowPtr[r + 1]; ++p) {
-                    const int q = col[p] / SW;
-                    const long long e = cursor[q]++;
-                    erow[e] = (unsigned short)(r - subRow0[i]);
-                    ecol[e] = (unsigned short)(col[p] - q * SW);
-                    long long ve = e;
-                    if (dtype == MX_F64) {  // position inside the group's 512-entry block
-                        const long long g0 = start[(size_t)i * S + q], rel = e - g0;
-                        const long long within = rel % 512, l = within / 8, j8 = within % 8;
-                        ve = g0 + rel / 512 * 512 + (j8 / 2) * 128 + 2 * l + (j8 % 2);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int b = 0; b < nWG; ++b) {
+        const int q = wgs[b].slice, nr = wgs[b].nr;
+        const WgLayout &L = lay[b];
+        const int *sp = &seg[(size_t)q * rows + wgs[b].row0];
+        long long step = wgStep[b], chunk = wgChunk[b];
+        wgDesc[(size_t)b * 4 + 0] = wgs[b].row0;
+        wgDesc[(size_t)b * 4 + 1] = nr;
+        wgDesc[(size_t)b * 4 + 2] = q;
+        wgDesc[(size_t)b * 4 + 3] = (int)chunk;
+        size_t k = 0;
+        for (int w = 0; w < W; ++w) {
+            int *d = &waveDesc[((size_t)b * W + w) * 4];
+            d[0] = (int)(step / SPB);                        // first batch
+            d[1] = (L.waveSteps[w] + SPB - 1) / SPB;         // batches
+            d[2] = (int)(chunk - wgChunk[b]);                // first chunk, counted inside the workgroup
+            d[3] = L.waveChunks[w];
+            int rel = 0;
+            for (int j = 0; j < L.waveChunks[w]; ++j, ++k, ++chunk) {
+                const int c = L.chunkOrder[k], cs = L.chunkSteps[c];
+                for (int l = 0; l < 64 && c * 64 + l < nr; ++l) {
+                    const int i = L.sortedRow[(size_t)c * 64 + l];
+                    chunkRows[(size_t)chunk * 64 + l] = (unsigned short)i;
+                    for (int e = sp[i]; e < sp[i + 1]; ++e) {
+                        const int n = e - sp[i], p = perm[e];
+                        const size_t st = (size_t)step + n / E, batch = st / SPB, sub = st % SPB;
+                        // a lane's column offsets of a batch are contiguous; so are its binary16
+                        // values; binary64 values go step by step, two per lane
+                        const size_t atc = (batch * 64 + l) * BE + sub * E + n % E;
+                        const size_t atv = dtype == MX_F64 ? batch * 64 * BE + sub * 128 + (size_t)l * 2 + n % E : atc;
+                        ecol[atc] = (unsigned short)(col[p] - q * SW);
+                        std::memcpy(&ev[atv * es], sv + (size_t)p * es, es);
                     }
-                    std::memcpy(&ev[(size_t)ve * es], sv + (size_t)p * es, es);
                 }
+                step += cs;
+                rel += cs;
+                chunkEnd[chunk] = rel;
+            }
+            step = (step + SPB - 1) / SPB * SPB;
         }
     }
     D.nWG = nWG;
     D.S = S;
     D.rows = rows;
     D.cols = cols;
-    D.maxSubRows = maxSub;
-    D.entries = total;
+    D.sliceCols = SW;
+    D.maxGroupRows = maxGroupRows;
+    D.steps = totalSteps;
     int rc;
-    if ((rc = upload(&D.wgSubPtr, wgSubPtr.data(), wgSubPtr.size()))) return rc;
-    if ((rc = upload(&D.subs, subs.data(), subs.size(), 16))) return rc;
-    if ((rc = upload(&D.erow, erow.data(), erow.size()))) return rc;
+    if ((rc = upload(&D.wgDesc, wgDesc.data(), wgDesc.size()))) return rc;
+    if ((rc = upload(&D.waveDesc, waveDesc.data(), waveDesc.size()))) return rc;
+    if ((rc = upload(&D.chunkEnd, chunkEnd.data(), chunkEnd.size()))) return rc;
+    if ((rc = upload(&D.chunkRows, chunkRows.data(), chunkRows.size()))) return rc;
     if ((rc = upload(&D.ecol, ecol.data(), ecol.size()))) return rc;
     if ((rc = upload_bytes(&D.eval, ev.data(), ev.size()))) return rc;
     if (S > 1 && (rc = upload_bytes(&D.partial, nullptr, 0, (size_t)S * rows * (dtype == MX_F64 ? 8 : 4)))) return rc;
@@ -288,6 +381,60 @@ int upload_tiles(mx_dtype dtype, int chunkNum, const char *sel, int dRows, const
     return MX_OK;
 }
 
+// Number of (workgroup, 128-byte line of x) pairs the row kernel would touch when it walks the
+// rows in the order given (identity when null), with `tile` entries per workgroup: the x lines
+// a workgroup's gathers have to bring into its CU at least once.
+long long x_lines_touched(int rows, int cols, const int *rowPtr, const int *col, const int *order, int tile, int es)
+{
+    const int perLine = 128 / es;
+    std::vector<int> stamp((size_t)cols / perLine + 2, -1);
+    long long lines = 0, filled = 0;
+    int wg = 0;
+    for (int i = 0; i < rows; ++i) {
+        const int r = order ? order[i] : i;
+        for (int p = rowPtr[r]; p < rowPtr[r + 1]; ++p) {
+            const int l = col[p] / perLine;
+            if (stamp[l] != wg) {
+                stamp[l] = wg;
+                ++lines;
+            }
+        }
+        filled += rowPtr[r + 1] - rowPtr[r];
+        if (filled >= tile) {
+            filled = 0;
+            ++wg;
+        }
+    }
+    return lines;
+}
+
+// Rows ordered by the median of their column ids (ties and empty rows keep their natural
+// position): rows that gather from the same stretch of x end up in the same workgroup.
+void order_rows_by_median(int rows, int cols, const int *rowPtr, const int *col, std::vector<int> &order)
+{
+    std::vector<long long> key((size_t)rows);
+#pragma omp parallel
+    {
+        std::vector<int> tmp;
+#pragma omp for schedule(dynamic, 1024)
+        for (int r = 0; r < rows; ++r) {
+            const int n = rowPtr[r + 1] - rowPtr[r];
+            int med;
+            if (n == 0) {
+                med = (int)((long long)r * cols / std::max(rows, 1));
+            } else {
+                tmp.assign(col + rowPtr[r], col + rowPtr[r + 1]);
+                std::nth_element(tmp.begin(), tmp.begin() + n / 2, tmp.end());
+                med = tmp[n / 2];
+            }
+            key[r] = ((long long)med << 32) | (unsigned)r;
+        }
+    }
+    std::sort(key.begin(), key.end());
+    order.resize((size_t)rows);
+    for (int i = 0; i < rows; ++i) order[i] = (int)(key[i] & 0xffffffffll);
+}
+
 int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, const int *col, const void *val,
                mx::DeviceCsr &A, double *pack_ms)
 {
@@ -297,10 +444,46 @@ int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, c
     A.npt = npt;
     A.nnz = nnz;
     int rc;
+    auto t0 = std::chrono::steady_clock::now();
+    // Row order.  The kernel may walk the rows in any order (it stores y through rowIdx then).
+    // Rows sorted by median column are taken when that cuts the x lines the workgroups touch
+    // by more than a third; MX_CSR_ROWORDER=natural|sorted overrides.
+    std::vector<int> order, pRowPtr, pCol;
+    std::vector<unsigned char> pVal;
+    {
+        const char *envo = std::getenv("MX_CSR_ROWORDER");
+        bool sorted = false;
+        if (rows > 1 && nnz > 0 && !(envo && !std::strcmp(envo, "natural"))) {
+            order_rows_by_median(rows, cols, rowPtr, col, order);
+            if (envo && !std::strcmp(envo, "sorted")) {
+                sorted = true;
+            } else {
+                const long long nat = x_lines_touched(rows, cols, rowPtr, col, nullptr, 256 * npt, es);
+                const long long srt = x_lines_touched(rows, cols, rowPtr, col, order.data(), 256 * npt, es);
+                sorted = (double)srt < 0.667 * (double)nat;
+            }
+        }
+        if (sorted) {
+            pRowPtr.assign((size_t)rows + 1, 0);
+            for (int i = 0; i < rows; ++i) pRowPtr[i + 1] = pRowPtr[i] + (rowPtr[order[i] + 1] - rowPtr[order[i]]);
+            pCol.resize((size_t)nnz);
+            pVal.resize((size_t)nnz * es);
+            const unsigned char *sv = (const unsigned char *)val;
+#pragma omp parallel for schedule(static)
+            for (int i = 0; i < rows; ++i) {
+                const int r = order[i], n = rowPtr[r + 1] - rowPtr[r];
+                std::copy(col + rowPtr[r], col + rowPtr[r] + n, pCol.begin() + pRowPtr[i]);
+                std::memcpy(&pVal[(size_t)pRowPtr[i] * es], sv + (size_t)rowPtr[r] * es, (size_t)n * es);
+            }
+            rowPtr = pRowPtr.data();
+            col = pCol.data();
+            val = pVal.data();
+            if ((rc = upload(&A.rowIdx, order.data(), (size_t)rows))) return rc;
+        }
+    }
     if ((rc = upload(&A.rowPtr, rowPtr, (size_t)rows + 1))) return rc;
     if ((rc = upload_bytes(&A.val, val, (size_t)nnz * es, (size_t)mx::kCsrPad * es))) return rc;
     std::vector<int> desc;
-    auto t0 = std::chrono::steady_clock::now();
     pack_rows(rowPtr, rows, npt, desc);
     A.nBlocks = (int)desc.size() / 4;
     if ((rc = upload(&A.blockDesc, desc.data(), desc.size()))) return rc;
@@ -415,6 +598,10 @@ static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
 
 static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate, hipStream_t s)
 {
+    if (plan->use_slices && ((uintptr_t)x & 15)) {
+        set_error("mx_spmv: x must be 16-byte aligned for this plan");
+        return MX_ERR_ARG;
+    }
     if (plan->use_slices)
         MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s));
     else
