@@ -10,8 +10,7 @@ namespace mx {
 // col/val carry kCsrPad extra zero entries so that a wave's aligned 128-bit loads may overrun.
 struct DeviceCsr {
     int rows = 0, cols = 0, nnz = 0;
-    int *rowPtr = nullptr;    // [rows+1], rows in the order the kernel walks them
-    int *rowIdx = nullptr;    // [rows] output row of each walked row; nullptr = natural order
+    int *rowPtr = nullptr;    // [rows+1]
     int *col = nullptr;       // [nnz + kCsrPad], or nullptr when the 16-bit form below is used
     unsigned short *col16 = nullptr;  // [nnz + kCsrPad] column ids as offsets from colBase[workgroup]
     int *colBase = nullptr;           // [nBlocks] lowest column of each workgroup's entries
@@ -19,6 +18,7 @@ struct DeviceCsr {
     int *blockDesc = nullptr; // [nBlocks][4] {first row, end row, first entry, end entry} per workgroup
     int nBlocks = 0;
     int npt = 0;              // entries per lane per tile the rows were packed for
+    bool scan = false;        // sum the rows of a tile by a segmented scan (row lengths vary a lot)
 };
 constexpr int kCsrPad = 1088;  // a wave may read one whole wave tile (64*16 entries) past the end
 

@@ -94,22 +94,19 @@ struct Acc<_Float16> {
 };
 
 // One wave's share of a tile: 64*NPT consecutive entries starting at the 16-byte aligned
-// position `pos` (wave-uniform).  Indices and values are streamed with 128-bit loads into the
-// wave's own LDS region (in entry order), then read back transposed
-// region so that in every x gather lane l holds entry 64j+l: neighbouring lanes then ask for
-// neighbouring entries of a row, whose sorted columns share cache lines, and the address
-// unit serves them together instead of one lane per cycle.  Returns the products
+// position `pos` (wave-uniform).  wave_stream moves indices and values with 128-bit loads into
+// the wave's own LDS region (in entry order); wave_gather reads them back transposed, so that
+// in every x gather lane l holds entry 64j+l: neighbouring lanes then ask for neighbouring
+// entries of a row, whose sorted columns share cache lines, and the address unit serves them
+// together instead of one lane per cycle.  It returns the products
 // p[j] = val[pos+64j+l] * x[col[pos+64j+l]].
 //   cs, vs : this wave's LDS regions, 64*NPT ints / accumulators.
 //   C16   : the column ids are stored as 16-bit offsets from x (the caller has moved x to the
 //           workgroup's lowest column); lim = the largest offset that is still inside x
 template <typename VT, int NPT, bool C16>
-__device__ __forceinline__ void wave_products(const void *__restrict__ colv, const VT *__restrict__ val,
-                                              const VT *__restrict__ x, int pos, int lane, int *cs,
-                                              typename Acc<VT>::type *vs, typename Acc<VT>::type (&p)[NPT],
-                                              int lim = 0)
+__device__ __forceinline__ void wave_stream(const void *__restrict__ colv, const VT *__restrict__ val, int pos, int lane,
+                                            int *cs, typename Acc<VT>::type *vs)
 {
-    typedef typename Acc<VT>::type AT;
     // every load instruction reads one contiguous stretch (lane l right after lane l-1): a
     // streamed line is then asked for once, not once per instruction that touches a piece of it
     if constexpr (C16) {
@@ -153,6 +150,13 @@ __device__ __forceinline__ void wave_products(const void *__restrict__ colv, con
             *(v4f32 *)(vs + e + 4) = fb;
         }
     }
+}
+
+template <typename VT, int NPT, bool C16>
+__device__ __forceinline__ void wave_gather(const VT *__restrict__ x, int lane, const int *cs,
+                                            const typename Acc<VT>::type *vs, typename Acc<VT>::type (&p)[NPT], int lim)
+{
+    typedef typename Acc<VT>::type AT;
     __builtin_amdgcn_wave_barrier();
     AT xv[NPT];
     if constexpr (C16) {
@@ -171,11 +175,9 @@ __device__ __forceinline__ void wave_products(const void *__restrict__ colv, con
 
 // Sums the rows of one tile out of LDS: W lanes per row, `rowOff` holds the rows' start
 // offsets inside the tile (nrows+1 entries).
-// rowOut (LDS, may be null) names the output row of each of the tile's rows.
 template <typename VT, int W>
-__device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, const unsigned short *rowOff,
-                                            const int *rowOut, int r0, int nrows, VT *__restrict__ y, int accumulate,
-                                            int tid)
+__device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, const unsigned short *rowOff, int r0,
+                                            int nrows, VT *__restrict__ y, int accumulate, int tid)
 {
     typedef typename Acc<VT>::type AT;
     constexpr int rowsPerPass = kBlock / W;
@@ -186,11 +188,118 @@ __device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, 
         for (int i = a + l; i < b; i += W) s += prod[i];
         s = group_sum<W>(s);
         if (l == 0) {
-            const int o = rowOut ? rowOut[rr] : r0 + rr;
-            if (accumulate) s += (AT)y[o];
-            y[o] = (VT)s;
+            if (accumulate) s += (AT)y[r0 + rr];
+            y[r0 + rr] = (VT)s;
         }
     }
+}
+
+// The same sums for tiles whose rows differ a lot in length (a few long rows would keep their
+// W lanes busy while all others wait).  Every lane owns NPT consecutive products and walks
+// them once: `head` (LDS, one int per entry) holds row+1 where a row starts and 0 elsewhere.
+// A row that starts and ends inside a lane's stretch is stored right away; what is left is,
+// per lane, the sum before its first row start (it belongs to a row opened by an earlier lane)
+// and the sum after its last one (a row that goes on in later lanes).  Those are stitched
+// together by a segmented scan over the 256 lanes (shuffles inside a wave, one LDS exchange
+// between the waves), and the lane in which a row starts closes the row that was open before.
+struct ScanItem {
+    int f;  // a row starts in this lane (or in one that the item has absorbed)
+    int r;  // row open at the end
+};
+template <typename VT, int NPT>
+__device__ __forceinline__ void reduce_scan(const typename Acc<VT>::type *prod, const int *head, const unsigned short *rowOff,
+                                            int r0, int nrows, VT *__restrict__ y, int accumulate, int tid,
+                                            typename Acc<VT>::type *carryV, int *carryF, int *carryR)
+{
+    typedef typename Acc<VT>::type AT;
+    const int lane = tid & 63, wave = tid >> 6;
+    auto store = [&](int row, AT v) {
+        if (accumulate) v += (AT)y[r0 + row];
+        y[r0 + row] = (VT)v;
+    };
+    AT v[NPT];
+    int h[NPT];
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) {
+        v[j] = prod[NPT * tid + j];
+        h[j] = head[NPT * tid + j];
+    }
+    AT before = 0, run = 0;  // before: sum ahead of the first row start
+    int cur = -1;            // row open right now, -1 = the one inherited from earlier lanes
+    int f = 0;
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) {
+        if (h[j] != 0) {
+            if (f) store(cur, run);
+            else before = run;
+            f = 1;
+            cur = h[j] - 1;
+            run = 0;
+        }
+        run += v[j];
+    }
+    if (!f) before = run;
+    // inclusive segmented scan of (f, value, row): value = sum since the last row start
+    AT sv = run;  // with no start in the lane, run == before == the lane's whole sum
+    int sf = f, sr = cur;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const AT pv = __shfl_up(sv, d, 64);
+        const int pf = __shfl_up(sf, d, 64), pr = __shfl_up(sr, d, 64);
+        if (lane >= d) {
+            if (!sf) {
+                sv += pv;
+                sr = pr;
+            }
+            sf |= pf;
+        }
+    }
+    if (lane == 63) {
+        carryV[wave] = sv;
+        carryF[wave] = sf;
+        carryR[wave] = sr;
+    }
+    // what the lane before this one ends with, inside the wave
+    AT ev = __shfl_up(sv, 1, 64);
+    int ef = __shfl_up(sf, 1, 64), er = __shfl_up(sr, 1, 64);
+    if (lane == 0) {
+        ev = 0;
+        ef = 0;
+        er = -1;
+    }
+    __syncthreads();
+    // fold in the waves before this one
+    AT cv = 0;
+    int cf = 0, cr = -1;
+    for (int w = 0; w < wave; ++w) {
+        if (carryF[w]) {
+            cv = carryV[w];
+            cr = carryR[w];
+            cf = 1;
+        } else {
+            cv += carryV[w];
+        }
+    }
+    if (!ef) {
+        ev += cv;
+        er = cr;
+    }
+    (void)cf;
+    // a lane in which a row starts closes the row that was open before it
+    if (f && er >= 0) store(er, ev + before);
+    // the last lane closes the row that is still open at the end of the tile
+    if (tid == kBlock - 1) {
+        AT tv = sv;
+        int tr = sr;
+        if (!sf) {
+            tv += cv;
+            tr = cr;
+        }
+        if (tr >= 0) store(tr, tv);
+    }
+    // rows without entries
+    for (int rr = tid; rr < nrows; rr += kBlock)
+        if (rowOff[rr] == rowOff[rr + 1]) store(rr, (AT)0);
 }
 
 // One workgroup owns the whole rows [r0, r1) named by its descriptor {r0, r1, p0, p1}
@@ -205,14 +314,13 @@ __device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, 
 // 16-bit offsets from colBase[workgroup] (the host uses this form when the columns of every
 // workgroup span fewer than 65536), which takes a third off the bytes of an FP16 entry and
 // a sixth off an FP64 one.
-// With PERM the rows are walked in an order of the host's choosing and rowIdx names the output
-// row of each.
-template <typename VT, int NPT, bool XCD, bool C16, bool PERM>
+// With SCAN the rows of a tile are summed by reduce_scan instead of reduce_rows (the host asks
+// for it when row lengths vary a lot).
+template <typename VT, int NPT, bool XCD, bool C16, bool SCAN>
 __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict__ rowPtr, const void *__restrict__ col,
                                                           const VT *__restrict__ val, const VT *__restrict__ xfull,
                                                           VT *__restrict__ y, const int4 *__restrict__ blockDesc,
-                                                          const int *__restrict__ colBase,
-                                                          const int *__restrict__ rowIdx, int xcols, int accumulate)
+                                                          const int *__restrict__ colBase, int xcols, int accumulate)
 {
     typedef typename Acc<VT>::type AT;
     constexpr int TILE = kBlock * NPT;
@@ -220,9 +328,8 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
     __shared__ __attribute__((aligned(16))) AT prod[TILE];
     __shared__ __attribute__((aligned(16))) int cols[TILE];
     __shared__ unsigned short rowOff[TILE + 2];  // offsets inside the tile fit 16 bits
-    __shared__ int rowOutS[PERM ? TILE : 1];
     __shared__ AT wsum[kBlock / 64];
-    const int *rowOut = PERM ? rowOutS : nullptr;
+    __shared__ int wflag[kBlock / 64], wrow[kBlock / 64];
 
     const int b = XCD ? xcd_contiguous_block(blockIdx.x, gridDim.x) : (int)blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -236,43 +343,68 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
     const int base = p0 & ~(NPT - 1);
     int *cs = cols + wave * WTILE;
     AT *vs = prod + wave * WTILE;
-
     if (p1 - base <= TILE) {
         // row offsets: lane t takes rows t, t+256, ... (at most NPT+1 of them)
-        int ro[NPT + 1], rx[PERM ? NPT : 1];
+        int ro[NPT + 1];
 #pragma unroll
         for (int k = 0; k <= NPT; ++k) {
             const int rr = tid + k * kBlock;
             ro[k] = rr <= nrows ? rowPtr[r0 + rr] : 0;
-            if (PERM && k < NPT) rx[k] = rr < nrows ? rowIdx[r0 + rr] : 0;
         }
-        if (base + wave * WTILE < p1) {
+        const bool active = base + wave * WTILE < p1;
+        if (active) wave_stream<VT, NPT, C16>(col, val, base + wave * WTILE, lane, cs, vs);
+        if (active) {
             AT p[NPT];
-            wave_products<VT, NPT, C16>(col, val, x, base + wave * WTILE, lane, cs, vs, p, lim);
+            wave_gather<VT, NPT, C16>(x, lane, cs, vs, p, lim);
 #pragma unroll
-            for (int j = 0; j < NPT; ++j) vs[64 * j + lane] = p[j];
+            for (int j = 0; j < NPT; ++j) {
+                // reduce_scan walks the whole tile: what is not this workgroup's must be zero
+                const int e = base + wave * WTILE + 64 * j + lane;
+                vs[64 * j + lane] = (!SCAN || (e >= p0 && e < p1)) ? p[j] : (AT)0;
+            }
+        } else if (SCAN) {
+#pragma unroll
+            for (int j = 0; j < NPT; ++j) vs[64 * j + lane] = 0;
+        }
+        if constexpr (SCAN) {  // the wave's column ids are spent: its region becomes row-start marks
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int j = 0; j < NPT; ++j) cs[64 * j + lane] = 0;
         }
 #pragma unroll
         for (int k = 0; k <= NPT; ++k) {
             const int rr = tid + k * kBlock;
             if (rr <= nrows) rowOff[rr] = (unsigned short)(ro[k] - base);
-            if (PERM && k < NPT && rr < nrows) rowOutS[rr] = rx[k];
+        }
+        if constexpr (SCAN) {
+            __syncthreads();
+            // rows that start at the same entry are empty except the last of them: the highest wins
+#pragma unroll
+            for (int k = 0; k < NPT; ++k) {
+                const int rr = tid + k * kBlock, pos = ro[k] - base;
+                if (rr < nrows && pos < TILE) atomicMax(&cols[pos], rr + 1);
+            }
         }
         __syncthreads();
+        if constexpr (SCAN) {
+            reduce_scan<VT, NPT>(prod, cols, rowOff, r0, nrows, y, accumulate, tid, wsum, wflag, wrow);
+            return;
+        }
         const int mean = (p1 - p0) / nrows;
-        if (mean <= 2) reduce_rows<VT, 1>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
-        else if (mean <= 4) reduce_rows<VT, 2>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
-        else if (mean <= 8) reduce_rows<VT, 4>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
-        else if (mean <= 16) reduce_rows<VT, 8>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
-        else if (mean <= 32) reduce_rows<VT, 16>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
-        else if (mean <= 64) reduce_rows<VT, 32>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
-        else reduce_rows<VT, 64>(prod, rowOff, rowOut, r0, nrows, y, accumulate, tid);
+        if (mean <= 2) reduce_rows<VT, 1>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 4) reduce_rows<VT, 2>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 8) reduce_rows<VT, 4>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 16) reduce_rows<VT, 8>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 32) reduce_rows<VT, 16>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else if (mean <= 64) reduce_rows<VT, 32>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        else reduce_rows<VT, 64>(prod, rowOff, r0, nrows, y, accumulate, tid);
     } else {
         // a single row longer than one tile
         AT s = 0;
         for (int t0 = base + wave * WTILE; t0 < p1; t0 += TILE) {
             AT p[NPT];
-            wave_products<VT, NPT, C16>(col, val, x, t0, lane, cs, vs, p, lim);
+            wave_stream<VT, NPT, C16>(col, val, t0, lane, cs, vs);
+            wave_gather<VT, NPT, C16>(x, lane, cs, vs, p, lim);
 #pragma unroll
             for (int j = 0; j < NPT; ++j) {
                 const int e = t0 + 64 * j + lane;
@@ -287,9 +419,8 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
             AT t = 0;
 #pragma unroll
             for (int w = 0; w < kBlock / 64; ++w) t += wsum[w];
-            const int o = PERM ? rowIdx[r0] : r0;
-            if (accumulate) t += (AT)y[o];
-            y[o] = (VT)t;
+            if (accumulate) t += (AT)y[r0];
+            y[r0] = (VT)t;
         }
     }
 }
@@ -746,13 +877,13 @@ namespace mx {
 template <typename VT, int NPT>
 static void launch_csr_t(const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
 {
-#define MX_LAUNCH_ROWS(C16, PERM, COLS, BASE)                                                                       \
-    hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, C16, PERM>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s,      \
+#define MX_LAUNCH_ROWS(C16, SCAN, COLS, BASE)                                                                       \
+    hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, C16, SCAN>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s,      \
                        A.rowPtr, (const void *)(COLS), (const VT *)A.val, (const VT *)x, (VT *)y,                      \
-                       (const int4 *)A.blockDesc, (const int *)(BASE), (const int *)A.rowIdx, A.cols, accumulate)
-    if (A.col16 && A.rowIdx) MX_LAUNCH_ROWS(true, true, A.col16, A.colBase);
+                       (const int4 *)A.blockDesc, (const int *)(BASE), A.cols, accumulate)
+    if (A.col16 && A.scan) MX_LAUNCH_ROWS(true, true, A.col16, A.colBase);
     else if (A.col16) MX_LAUNCH_ROWS(true, false, A.col16, A.colBase);
-    else if (A.rowIdx) MX_LAUNCH_ROWS(false, true, A.col, nullptr);
+    else if (A.scan) MX_LAUNCH_ROWS(false, true, A.col, nullptr);
     else MX_LAUNCH_ROWS(false, false, A.col, nullptr);
 #undef MX_LAUNCH_ROWS
 }

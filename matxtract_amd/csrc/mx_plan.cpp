@@ -76,7 +76,6 @@ void pack_rows(const int *rowPtr, int rows, int npt, std::vector<int> &desc)
 void free_csr(mx::DeviceCsr &A)
 {
     (void)hipFree(A.rowPtr);
-    (void)hipFree(A.rowIdx);
     (void)hipFree(A.col);
     (void)hipFree(A.col16);
     (void)hipFree(A.colBase);
@@ -381,60 +380,6 @@ int upload_tiles(mx_dtype dtype, int chunkNum, const char *sel, int dRows, const
     return MX_OK;
 }
 
-// Number of (workgroup, 128-byte line of x) pairs the row kernel would touch when it walks the
-// rows in the order given (identity when null), with `tile` entries per workgroup: the x lines
-// a workgroup's gathers have to bring into its CU at least once.
-long long x_lines_touched(int rows, int cols, const int *rowPtr, const int *col, const int *order, int tile, int es)
-{
-    const int perLine = 128 / es;
-    std::vector<int> stamp((size_t)cols / perLine + 2, -1);
-    long long lines = 0, filled = 0;
-    int wg = 0;
-    for (int i = 0; i < rows; ++i) {
-        const int r = order ? order[i] : i;
-        for (int p = rowPtr[r]; p < rowPtr[r + 1]; ++p) {
-            const int l = col[p] / perLine;
-            if (stamp[l] != wg) {
-                stamp[l] = wg;
-                ++lines;
-            }
-        }
-        filled += rowPtr[r + 1] - rowPtr[r];
-        if (filled >= tile) {
-            filled = 0;
-            ++wg;
-        }
-    }
-    return lines;
-}
-
-// Rows ordered by the median of their column ids (ties and empty rows keep their natural
-// position): rows that gather from the same stretch of x end up in the same workgroup.
-void order_rows_by_median(int rows, int cols, const int *rowPtr, const int *col, std::vector<int> &order)
-{
-    std::vector<long long> key((size_t)rows);
-#pragma omp parallel
-    {
-        std::vector<int> tmp;
-#pragma omp for schedule(dynamic, 1024)
-        for (int r = 0; r < rows; ++r) {
-            const int n = rowPtr[r + 1] - rowPtr[r];
-            int med;
-            if (n == 0) {
-                med = (int)((long long)r * cols / std::max(rows, 1));
-            } else {
-                tmp.assign(col + rowPtr[r], col + rowPtr[r + 1]);
-                std::nth_element(tmp.begin(), tmp.begin() + n / 2, tmp.end());
-                med = tmp[n / 2];
-            }
-            key[r] = ((long long)med << 32) | (unsigned)r;
-        }
-    }
-    std::sort(key.begin(), key.end());
-    order.resize((size_t)rows);
-    for (int i = 0; i < rows; ++i) order[i] = (int)(key[i] & 0xffffffffll);
-}
-
 int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, const int *col, const void *val,
                mx::DeviceCsr &A, double *pack_ms)
 {
@@ -445,48 +390,26 @@ int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, c
     A.nnz = nnz;
     int rc;
     auto t0 = std::chrono::steady_clock::now();
-    // Row order.  The kernel may walk the rows in any order (it stores y through rowIdx then).
-    // Rows sorted by median column are taken when that cuts the x lines the workgroups touch
-    // by more than a third; MX_CSR_ROWORDER=natural|sorted overrides.
-    std::vector<int> order, pRowPtr, pCol;
-    std::vector<unsigned char> pVal;
-    {
-        const char *envo = std::getenv("MX_CSR_ROWORDER");
-        bool sorted = false;
-        if (rows > 1 && nnz > 0 && !(envo && !std::strcmp(envo, "natural"))) {
-            order_rows_by_median(rows, cols, rowPtr, col, order);
-            if (envo && !std::strcmp(envo, "sorted")) {
-                sorted = true;
-            } else {
-                const long long nat = x_lines_touched(rows, cols, rowPtr, col, nullptr, 256 * npt, es);
-                const long long srt = x_lines_touched(rows, cols, rowPtr, col, order.data(), 256 * npt, es);
-                sorted = (double)srt < 0.667 * (double)nat;
-            }
-        }
-        if (sorted) {
-            pRowPtr.assign((size_t)rows + 1, 0);
-            for (int i = 0; i < rows; ++i) pRowPtr[i + 1] = pRowPtr[i] + (rowPtr[order[i] + 1] - rowPtr[order[i]]);
-            pCol.resize((size_t)nnz);
-            pVal.resize((size_t)nnz * es);
-            const unsigned char *sv = (const unsigned char *)val;
-#pragma omp parallel for schedule(static)
-            for (int i = 0; i < rows; ++i) {
-                const int r = order[i], n = rowPtr[r + 1] - rowPtr[r];
-                std::copy(col + rowPtr[r], col + rowPtr[r] + n, pCol.begin() + pRowPtr[i]);
-                std::memcpy(&pVal[(size_t)pRowPtr[i] * es], sv + (size_t)rowPtr[r] * es, (size_t)n * es);
-            }
-            rowPtr = pRowPtr.data();
-            col = pCol.data();
-            val = pVal.data();
-            if ((rc = upload(&A.rowIdx, order.data(), (size_t)rows))) return rc;
-        }
-    }
-    if ((rc = upload(&A.rowPtr, rowPtr, (size_t)rows + 1))) return rc;
-    if ((rc = upload_bytes(&A.val, val, (size_t)nnz * es, (size_t)mx::kCsrPad * es))) return rc;
     std::vector<int> desc;
     pack_rows(rowPtr, rows, npt, desc);
+    if ((rc = upload(&A.rowPtr, rowPtr, (size_t)rows + 1))) return rc;
+    if ((rc = upload_bytes(&A.val, val, (size_t)nnz * es, (size_t)mx::kCsrPad * es))) return rc;
     A.nBlocks = (int)desc.size() / 4;
     if ((rc = upload(&A.blockDesc, desc.data(), desc.size()))) return rc;
+    {
+        // rows of very different lengths: sum tiles by a segmented scan (MX_CSR_REDUCE=rows|scan overrides)
+        double sum = 0.0, sq = 0.0;
+        for (int r = 0; r < rows; ++r) {
+            const double n = rowPtr[r + 1] - rowPtr[r];
+            sum += n;
+            sq += n * n;
+        }
+        const double mean = rows > 0 ? sum / rows : 0.0, var = rows > 0 ? sq / rows - mean * mean : 0.0;
+        A.scan = mean > 0.0 && var > 0.25 * mean * mean;
+        const char *envr = std::getenv("MX_CSR_REDUCE");
+        if (envr && !std::strcmp(envr, "rows")) A.scan = false;
+        if (envr && !std::strcmp(envr, "scan")) A.scan = true;
+    }
     // 16-bit column offsets when every workgroup's columns span fewer than 65536
     // (MX_CSR_COL16=0 keeps 32-bit ids)
     const char *env16 = std::getenv("MX_CSR_COL16");
