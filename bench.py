@@ -207,7 +207,7 @@ def main():
         sys.exit(2)
 
     import torch
-    import matxtract_amd as mx
+    import matxtractt_amd as mx
     from oracle import mx_oracle as ora
     if not torch.cuda.is_available() or mx.device_count() < 1:
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)

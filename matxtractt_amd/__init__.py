@@ -1,4 +1,4 @@
-"""matxtract_amd -- MI355X (gfx950) implementation of MatXtract's hybrid SpMV path.
+"""matxtractt_amd -- MI355X (gfx950) implementation of MatXtract's hybrid SpMV path.
 
 The product is ``libmatxtract_hip.so`` (C ABI in ``include/matxtract_hip.h``, the reference's
 C++ surface in ``include/MatXtract.h``, the ``matxtract_perftest`` CLI in ``bin/``).  This

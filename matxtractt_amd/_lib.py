@@ -1,6 +1,6 @@
 """ctypes loader for libmatxtract_hip.so (the C ABI declared in include/matxtract_hip.h).
 
-The library is built in-tree by ``matxtract_amd/csrc/Makefile``.  Loading fails loudly when it
+The library is built in-tree by ``matxtractt_amd/csrc/Makefile``.  Loading fails loudly when it
 is missing: there is no Python or CPU fallback for the device entry points.
 """
 import ctypes as C

@@ -15,12 +15,12 @@ def pytest_configure(config):
 @pytest.fixture(scope="session")
 def mx():
     """The product package; builds the library first if it is not there."""
-    from matxtract_amd import _lib
+    from matxtractt_amd import _lib
     if not os.path.exists(_lib.LIB_PATH):
         import __graft_entry__
         __graft_entry__.build()
-    import matxtract_amd
-    return matxtract_amd
+    import matxtractt_amd
+    return matxtractt_amd
 
 
 @pytest.fixture(scope="session")

@@ -24,7 +24,7 @@ def oracle_y(ora, mx, A, x):
 def test_mfma_operand_layout_f64(mx):
     """v_mfma_f64_16x16x4_f64: A[i][k] in lane 16k+i, B[k][j] in lane 16k+j, D[i][j] in
     accumulator register i//4 of lane 16*(i%4)+j -- the mapping tile_f64_kernel relies on."""
-    from matxtract_amd import _lib
+    from matxtractt_amd import _lib
     rng = np.random.default_rng(5)
     A = rng.integers(-4, 5, (16, 4)).astype(np.float64)
     B = rng.integers(-4, 5, (4, 16)).astype(np.float64)
@@ -45,7 +45,7 @@ def test_mfma_operand_layout_f64(mx):
 def test_mfma_operand_layout_f16(mx):
     """v_mfma_f32_16x16x32_f16: A[i][8g+e] is element e of lane 16g+i, B[8g+e][j] element e of
     lane 16g+j, D[i][j] accumulator register i%4 of lane 16*(i//4)+j (tile_f16_kernel)."""
-    from matxtract_amd import _lib
+    from matxtractt_amd import _lib
     rng = np.random.default_rng(6)
     A = rng.integers(-4, 5, (16, 32)).astype(np.float16)
     B = rng.integers(-4, 5, (32, 16)).astype(np.float16)
@@ -298,7 +298,7 @@ def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
     import subprocess
     import os
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    exe = os.path.join(root, "matxtract_amd", "bin", "matxtract_perftest")
+    exe = os.path.join(root, "matxtractt_amd", "bin", "matxtract_perftest")
     A, _ = mx.gen_config(2, scale=1 / 64)
     p = tmp_path / "m.mtx"
     with open(p, "w") as f:

@@ -202,7 +202,7 @@ def test_init_vec(mx):
 
 
 def test_f16_conversions_match_numpy(mx):
-    from matxtract_amd import _lib
+    from matxtractt_amd import _lib
     L = _lib.load()
     rng = np.random.default_rng(2)
     vals = np.concatenate([rng.uniform(-70000, 70000, 3000), rng.uniform(-1e-4, 1e-4, 3000),
@@ -233,7 +233,7 @@ def declared_symbols():
 
 
 def test_library_exports_every_declared_symbol(mx):
-    from matxtract_amd import _lib
+    from matxtractt_amd import _lib
     L = _lib.load()
     names = declared_symbols()
     assert len(names) >= 25
@@ -256,7 +256,7 @@ def test_device_entry_points_fail_loudly_without_a_gpu(mx):
 
 def test_product_does_not_reach_into_the_oracle():
     """Nothing under the package, the headers or bench-independent entry points names the oracle."""
-    pkg = os.path.join(ROOT, "matxtract_amd")
+    pkg = os.path.join(ROOT, "matxtractt_amd")
     for base, _, files in os.walk(pkg):
         if os.path.basename(base) == "build":
             continue
@@ -268,7 +268,7 @@ def test_product_does_not_reach_into_the_oracle():
 
 # ---------------------------------------------------------------- CLI argument handling (no GPU needed)
 def cli(*args):
-    exe = os.path.join(ROOT, "matxtract_amd", "bin", "matxtract_perftest")
+    exe = os.path.join(ROOT, "matxtractt_amd", "bin", "matxtract_perftest")
     if not os.path.exists(exe):
         pytest.skip("CLI not built")
     return subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
