@@ -25,19 +25,37 @@ constexpr int kCsrPad = 1088;  // a wave may read one whole wave tile (64*16 ent
 // Entries per lane per tile of the CSR kernel (a tile is 256 lanes wide).
 int csr_entries_per_lane(mx_dtype dtype);
 
-// Bitmap tiles resident on the device (the reference's chunkPtr / fragPtr / fragBit / tcVal /
-// sparse_AToX_index, restricted to the chunks the tile kernel executes).
+// Tiles resident on the device, re-packed for the tile kernels.  The fragments the plan
+// selects are expanded from the reference's encoding (bitmap + packed values) into full
+// fragM x fragK blocks, zeros included (row-major inside a block), so that a lane can load
+// exactly what the matrix core wants from it with no decoding; the plan only selects fragments
+// that are mostly full.  The blocks are grouped into "steps" -- what one wave feeds to the
+// matrix core at a time: two halves of up to kTileSlots(dtype)/2 blocks.  A chunk with more
+// selected fragments than half a step takes whole steps of its own (filling half 0 first; its
+// two halves are added at the end); smaller chunks share a step, one per half.  Per step:
+//   hdr    kTileHdr dwords: [0,16) output row of each of the 8 rows of half 0 and half 1
+//          (-1 = none); [16] flags (1 = store the sums after this step, 2 = the halves are
+//          different chunks); [17],[18] blocks in half 0 and half 1; [19],[20] first value
+//          and blocks in half 0 of the step four further on (a wave learns where to prefetch
+//          from there; its own last step when it has no such step).
+//   atox   64 column ids (slot-major), -1 for unused ones
+//   values the blocks of half 0, then those of half 1; nothing for absent blocks.
+// Waves take whole chunks: waveDesc = {first step, end step, first value of the wave's first
+// four steps, blocks in half 0 of each of them (one byte each), 0}.
 struct DeviceTiles {
-    int chunkNum = 0;  // executed chunks
-    int dRows = 0;     // 8*chunkNum, or fewer when the last chunk is ragged
-    int frags = 0, vals = 0;
-    int *chunkPtr = nullptr;  // [chunkNum+1]
-    int *fragPtr = nullptr;   // [frags+1]
-    void *fragBit = nullptr;  // [frags] u32 | u64
-    void *tcVal = nullptr;    // [vals]
-    int *atox = nullptr;      // [frags*fragK] indices into the x handed to the kernel
-    int *rowIdx = nullptr;    // [dRows] output row of each tile row; nullptr = identity
+    int chunkNum = 0;  // chunks with at least one selected fragment
+    int frags = 0, vals = 0;   // selected fragments, entries they hold
+    long long stored = 0;      // values stored (zeros included)
+    int steps = 0, nWaves = 0;
+    int *waveDesc = nullptr;   // [nWaves][8]
+    int *hdr = nullptr;        // [steps][kTileHdr]
+    int *atox = nullptr;       // [steps][64]
+    void *tcVal = nullptr;     // blocks
 };
+constexpr int kTileHdr = 32;
+inline int tile_slots(mx_dtype d) { return d == MX_F64 ? 16 : 8; }  // fragment slots per step
+// slot of block i of half h: binary64 MFMA j takes slots 2j and 2j+1, binary16 slots 0..3 and 4..7
+inline int tile_slot(mx_dtype d, int half, int i) { return d == MX_F64 ? 2 * i + half : 4 * half + i; }
 
 // The CSR part re-laid for x resident in LDS.  The columns are cut into S slices of sliceCols
 // columns (a slice of x fits LDS); every slice cuts the rows into groups of about equal entries of

@@ -13,6 +13,7 @@
 #include <hip/hip_runtime.h>
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 #include "mx_device.h"
 
@@ -617,233 +618,173 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
 }
 
 // ---- tile part --------------------------------------------------------------------------
-// A wave works on U 8-row chunks at once, 4 waves per workgroup.  The address unit spends
-// about 16 cycles on every wave-level load whatever the number of active lanes, so all
-// global loads are "one lane, one element": a step's bitmaps and value pointers in one load,
-// its 64 column ids in one, the 64 x values they name in one gather, and its packed values as
-// one contiguous run.  They are parked in the wave's own LDS region, and every lane then
-// picks what the MFMA operand layout asks of it with LDS reads.  The loads of all U chunks are
-// issued before any is used.  The host lays the values out so that the run of every step
-// starts on a 16-byte boundary (fragPtr holds those padded offsets).
+// The selected fragments arrive expanded to full blocks and regrouped into steps (see
+// DeviceTiles): what one wave hands to the matrix core at a time.  A wave owns a run of steps
+// made of whole chunks and walks it with everything prefetched: while step s is multiplied, the
+// header, column ids and values of steps s+1 .. s+4 and the x values and old y of steps s+1 and
+// s+2 are already on their way, so the dependent accesses of a step (column ids -> x, header ->
+// rows -> y) never stall the wave.  Every lane loads the values it feeds to the matrix core
+// itself, straight from the block, so only the gathered x goes through LDS.
 //
-// v_mfma_f64_16x16x4_f64 operand layout (wave64): lane L holds A[L%16][L/16] and
-// B[L/16][L%16]; accumulator register g of lane L holds D[4*g + L/16][L%16].  One MFMA feeds
-// two 8x4 fragments: A rows 0..7 = fragment f, rows 8..15 = fragment f+1; B column 0 = the 4
-// gathered x of fragment f, column 1 = those of fragment f+1, other columns 0.  The chunk's
-// result is D[0..7][0] + D[8..15][1], accumulated across all steps inside the matrix core, so
-// there is no cross-lane reduction until the single combine at the end.  A step is 16
-// fragments = 8 MFMAs.
-constexpr int kTileStepF64 = 16, kTileStepF16 = 8;  // fragments per step
-constexpr int kTileUF64 = 2, kTileUF16 = 4;         // chunks in flight per wave
+// v_mfma_f64_16x16x4_f64 (wave64): lane L holds A[L%16][L/16] and B[L/16][L%16]; accumulator
+// register g of lane L holds D[4*g + L/16][L%16].  One MFMA feeds two 8x4 blocks: A rows 0..7 =
+// block j of half 0, rows 8..15 = block j of half 1; B column 0 = the 4 gathered x of the
+// former, column 1 = those of the latter, other columns 0.  D[0..7][0] collects half 0 and
+// D[8..15][1] half 1 over the 8 MFMAs of a step and all steps of a chunk, inside the matrix core.
+//
+// v_mfma_f32_16x16x32_f16 (wave64): lane L holds A[L%16][8*(L/16) .. +7], B[8*(L/16) .. +7][L%16];
+// accumulator register g of lane L holds D[4*(L/16)+g][L%16].  One MFMA is a whole step: A rows
+// 0..7 = the 4 blocks of half 0 side by side along K, rows 8..15 = those of half 1; B column 0 =
+// the 32 gathered x of half 0, column 1 = those of half 1.  A lane's eight A elements are one
+// row of one 8x8 block: 16 contiguous bytes.
+using mx::kTileHdr;
 
-__global__ __launch_bounds__(kBlock) void tile_f64_kernel(const int *__restrict__ chunkPtr, const int *__restrict__ fragPtr,
-                                                         const uint32_t *__restrict__ fragBit,
-                                                         const double *__restrict__ tcVal, const int *__restrict__ atox,
-                                                         const int *__restrict__ rowIdx, const double *__restrict__ x,
-                                                         double *__restrict__ y, int chunkNum, int dRows, int accumulate)
+// The MFMA calls of tile_kernel sit in code shared by both precisions; overloads pick the
+// instruction.
+__device__ __forceinline__ v4f64 tile_mma(double a, double b, v4f64 c)
 {
-    constexpr int U = kTileUF64, SF = kTileStepF64;
-    struct Unit {
-        unsigned hdr[64];  // [0,16) bitmaps, [16,33) value offsets of the step's fragments
-        double xv[64];     // x of the step's 16*4 columns
-        double val[512];   // the step's packed values
-    };
-    __shared__ Unit lds[kBlock / 64][U];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int w0 = (blockIdx.x * (kBlock / 64) + wave) * U;
-    if (w0 >= chunkNum) return;
-    const int m = lane & 15, k = lane >> 4;
-    const int t = m >> 3;                // which of an MFMA's two fragments this lane decodes
-    const int bitpos = (m & 7) * 4 + k;  // (local row, local column) -> bitmap bit
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ v4f32 tile_mma(v8f16 a, v8f16 b, v4f32 c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
 
-    // chunk bounds: lanes 0..U hold chunkPtr[w0 + lane]
-    const int cp = chunkPtr[min(w0 + lane, chunkNum)];
-    int f0[U], f1[U], steps = 0;
-    // output rows: lane r < 8 holds row r of each chunk and its old y
-    int row[U];
-    double yold[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        f0[u] = __builtin_amdgcn_readlane(cp, u);
-        f1[u] = w0 + u < chunkNum ? __builtin_amdgcn_readlane(cp, u + 1) : f0[u];
-        steps = max(steps, (f1[u] - f0[u] + SF - 1) / SF);
-        const int local = (w0 + u) * 8 + lane;
-        row[u] = (lane < 8 && w0 + u < chunkNum && local < dRows) ? (rowIdx ? rowIdx[local] : local) : -1;
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) yold[u] = (accumulate && row[u] >= 0) ? y[row[u]] : 0.0;
+template <typename VT>
+struct TileStep {  // one step's loads, as one lane holds them
+    int hdr;       // header dword lane%32: lanes 0..15 hold the output rows
+    int ax;        // column id
+    typename std::conditional<sizeof(VT) == 8, double[8], v4i32>::type v;  // A operands
+    VT xr, yr;     // gathered x and old y, as loaded (looked at only when the step is multiplied)
+};
 
-    v4f64 acc[U];
+// All loads of a step are unconditional: the count of loads in flight is then known at compile
+// time and the wave can wait for one step while the next ones are still on their way.  A lane
+// whose block is absent reads what follows the step's values (the host leaves slack at the end)
+// and ignores it.  vo = first value of the step, na = blocks in its half 0.
+template <typename VT>
+__device__ __forceinline__ void tile_issue(TileStep<VT> &R, const int *__restrict__ hdr, const int *__restrict__ atox,
+                                           const VT *__restrict__ tcVal, int step, int vo, int na, int lane)
+{
+    R.ax = atox[(size_t)step * 64 + lane];
+    R.hdr = hdr[(size_t)step * kTileHdr + (lane & 31)];
+    const int m = lane & 15, g = lane >> 4, h = m >> 3;
+    if constexpr (sizeof(VT) == 8) {
+        const VT *p = tcVal + vo + (h ? na : 0) * 32 + (m & 7) * 4 + g;
 #pragma unroll
-    for (int u = 0; u < U; ++u) acc[u] = v4f64{0.0, 0.0, 0.0, 0.0};
-    for (int s = 0; s < steps; ++s) {
-        unsigned hdr[U];
-        int ax[U], nf[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int fs = f0[u] + s * SF;
-            nf[u] = max(0, min(SF, f1[u] - fs));
-            const unsigned *hp = lane < 16 ? fragBit + fs + lane : (const unsigned *)fragPtr + fs + (lane - 16);
-            hdr[u] = (lane < 16 ? lane < nf[u] : (lane - 16 <= nf[u] && nf[u] > 0)) ? *hp : 0u;
-            ax[u] = lane < 4 * nf[u] ? atox[fs * 4 + lane] : -1;
-        }
-        double xg[U];
-        v2f64 vv[U][4];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            xg[u] = ax[u] >= 0 ? x[ax[u]] : 0.0;
-            const int vb = __builtin_amdgcn_readlane((int)hdr[u], 16);
-            const int ve = __builtin_amdgcn_readlane((int)hdr[u], 16 + nf[u]);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int o = vb + q * 128 + lane * 2;
-                vv[u][q] = o < ve ? __builtin_nontemporal_load((const v2f64 *)(tcVal + o)) : v2f64{0.0, 0.0};
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            Unit &L = lds[wave][u];
-            L.hdr[lane] = hdr[u];
-            L.xv[lane] = xg[u];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) *(v2f64 *)(L.val + q * 128 + lane * 2) = vv[u][q];
-        }
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const Unit &L = lds[wave][u];
-            const int vb = (int)L.hdr[16];
-#pragma unroll
-            for (int j = 0; j < SF / 2; ++j) {
-                const unsigned bm = L.hdr[2 * j + t];
-                const int fp = (int)L.hdr[16 + 2 * j + t] - vb;
-                const double a = ((bm >> bitpos) & 1u) ? L.val[fp + __popc(bm & ((1u << bitpos) - 1u))] : 0.0;
-                const double bv = m < 2 ? L.xv[(2 * j + m) * 4 + k] : 0.0;
-                acc[u] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, bv, acc[u], 0, 0, 0);
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-    }
-    // row q and row q+4 of a chunk end up in lane 16q: D[q][0] = reg 0, D[q+4][0] = reg 1 there,
-    // D[8+q][1] = reg 2 and D[12+q][1] = reg 3 of lane 16q+1.  Hand them to lanes 0..7 through LDS.
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const double o0 = acc[u][0] + __shfl_down(acc[u][2], 1, 64);
-        const double o1 = acc[u][1] + __shfl_down(acc[u][3], 1, 64);
-        double *out = lds[wave][u].xv;
-        if ((lane & 15) == 0) {
-            out[lane >> 4] = o0;
-            out[(lane >> 4) + 4] = o1;
-        }
-        __builtin_amdgcn_wave_barrier();
-        if (row[u] >= 0) y[row[u]] = yold[u] + out[lane];
+        for (int j = 0; j < 8; ++j) R.v[j] = __builtin_nontemporal_load(p + j * 32);
+    } else {
+        R.v = __builtin_nontemporal_load((const v4i32 *)(tcVal + vo + ((h ? na : 0) + g) * 64 + (m & 7) * 8));
     }
 }
 
-// v_mfma_f32_16x16x32_f16 operand layout (wave64): lane L holds A[L%16][8*(L/16) .. +7],
-// B[8*(L/16) .. +7][L%16]; accumulator register g of lane L holds D[4*(L/16)+g][L%16].  One MFMA
-// (= one step) feeds eight 8x8 fragments of the chunk: A rows 0..7 = fragments f..f+3 side by
-// side along K, rows 8..15 = fragments f+4..f+7; B column 0 = the 32 gathered x of f..f+3,
-// column 1 = those of f+4..f+7.  A lane's eight A elements are one byte of its fragment's
-// 64-bit bitmap (one tile row), whose values sit consecutively in the step's run in LDS; bit j
-// reads the element at the popcount of the lower bits.
-__global__ __launch_bounds__(kBlock) void tile_f16_kernel(const int *__restrict__ chunkPtr, const int *__restrict__ fragPtr,
-                                                         const uint64_t *__restrict__ fragBit,
-                                                         const _Float16 *__restrict__ tcVal, const int *__restrict__ atox,
-                                                         const int *__restrict__ rowIdx, const _Float16 *__restrict__ x,
-                                                         _Float16 *__restrict__ y, int chunkNum, int dRows, int accumulate)
+template <typename VT>
+__global__ __launch_bounds__(kBlock) void tile_kernel(const int4 *__restrict__ waveDesc, const int *__restrict__ hdr,
+                                                     const int *__restrict__ atox, const VT *__restrict__ tcVal,
+                                                     const VT *__restrict__ x, VT *__restrict__ y, int nWaves,
+                                                     int accumulate)
 {
-    constexpr int U = kTileUF16, SF = kTileStepF16;
-    struct Unit {
-        unsigned hdr[32];    // [0,16) the 8 bitmaps as dwords, [16,25) value offsets
-        _Float16 xv[64];     // x of the step's 8*8 columns
-        unsigned val[264];   // the step's packed values (512 halves) + slack
+    typedef typename Acc<VT>::type AT;
+    constexpr bool F64 = sizeof(VT) == 8;
+    struct Park {
+        VT xv[64];
+        AT out[16];
     };
-    __shared__ __attribute__((aligned(16))) Unit lds[kBlock / 64][U];
+    __shared__ __attribute__((aligned(16))) Park park[kBlock / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int w0 = (blockIdx.x * (kBlock / 64) + wave) * U;
-    if (w0 >= chunkNum) return;
-    const int m = lane & 15, g = lane >> 4;
-    const int r = m & 7;
+    const int gw = blockIdx.x * (kBlock / 64) + wave;
+    if (gw >= nWaves) return;
+    Park &P = park[wave];
+    const int4 d0 = waveDesc[2 * gw], d1 = waveDesc[2 * gw + 1];
+    const int s0 = __builtin_amdgcn_readfirstlane(d0.x), s1 = __builtin_amdgcn_readfirstlane(d0.y);
+    if (s0 >= s1) return;
+    const int last = s1 - 1;
+    const int m = lane & 15, g = lane >> 4, h = m >> 3;
 
-    const int cp = chunkPtr[min(w0 + lane, chunkNum)];
-    int f0[U], f1[U], steps = 0;
-    int row[U];
-    float yold[U];
+    // Five register sets take turns: the step being multiplied, the two after it (their gathers
+    // are in flight or about to be issued) and two more whose header, column ids and values are
+    // on their way.  Everything a step waits for was asked for two steps earlier.  The loop
+    // below is unrolled five times so that no set is ever copied into another (a copy would have
+    // to wait for the loads that fill it).
+    typedef TileStep<VT> Regs;
+    Regs R0, R1, R2, R3, R4;
+    // x and old y of a step, once its column ids and header are there (lanes without a column
+    // or a row read element 0 and ignore it)
+    auto gather = [&](Regs &R) {
+        R.xr = x[max(R.ax, 0)];
+        R.yr = y[lane < 16 ? max(R.hdr, 0) : 0];
+    };
+    typedef typename std::conditional<F64, v4f64, v4f32>::type AccV;
+    AccV acc;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        f0[u] = __builtin_amdgcn_readlane(cp, u);
-        f1[u] = w0 + u < chunkNum ? __builtin_amdgcn_readlane(cp, u + 1) : f0[u];
-        steps = max(steps, (f1[u] - f0[u] + SF - 1) / SF);
-        const int local = (w0 + u) * 8 + lane;
-        row[u] = (lane < 8 && w0 + u < chunkNum && local < dRows) ? (rowIdx ? rowIdx[local] : local) : -1;
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) yold[u] = (accumulate && row[u] >= 0) ? (float)y[row[u]] : 0.f;
-
-    v4f32 acc[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) acc[u] = v4f32{0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < steps; ++s) {
-        unsigned hdr[U];
-        int ax[U], nf[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int fs = f0[u] + s * SF;
-            nf[u] = max(0, min(SF, f1[u] - fs));
-            const unsigned *hp = lane < 16 ? (const unsigned *)fragBit + 2 * fs + lane : (const unsigned *)fragPtr + fs + (lane - 16);
-            hdr[u] = (lane < 16 ? lane < 2 * nf[u] : (lane - 16 <= nf[u] && nf[u] > 0 && lane < 32)) ? *hp : 0u;
-            ax[u] = lane < 8 * nf[u] ? atox[fs * 8 + lane] : -1;
-        }
-        _Float16 xg[U];
-        v4i32 vv[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            xg[u] = ax[u] >= 0 ? x[ax[u]] : (_Float16)0;
-            const int vb = __builtin_amdgcn_readlane((int)hdr[u], 16);
-            const int ve = __builtin_amdgcn_readlane((int)hdr[u], 16 + nf[u]);
-            const int o = vb + lane * 8;
-            vv[u] = o < ve ? __builtin_nontemporal_load((const v4i32 *)(tcVal + o)) : v4i32{0, 0, 0, 0};
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            Unit &L = lds[wave][u];
-            if (lane < 32) L.hdr[lane] = hdr[u];
-            L.xv[lane] = xg[u];
-            *(v4i32 *)(L.val + lane * 4) = vv[u];
-        }
+    for (int i = 0; i < 4; ++i) acc[i] = 0;
+    // one step: Ra is multiplied, Rg (two steps on) gets its gathers, Ri (four steps on) is issued
+    auto step = [&](int s, Regs &Ra, Regs &Rg, Regs &Ri) {
+        // where the values of step s+4 start is written in the header of step s
+        tile_issue<VT>(Ri, hdr, atox, tcVal, min(s + 4, last), __builtin_amdgcn_readlane(Ra.hdr, 19),
+                       __builtin_amdgcn_readlane(Ra.hdr, 20), lane);
+        gather(Rg);
+        P.xv[lane] = Ra.ax >= 0 ? Ra.xr : (VT)0;
         __builtin_amdgcn_wave_barrier();
+        const int flags = __builtin_amdgcn_readlane(Ra.hdr, 16);
+        const int nblk = h ? __builtin_amdgcn_readlane(Ra.hdr, 18) : __builtin_amdgcn_readlane(Ra.hdr, 17);
+        if constexpr (F64) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const Unit &L = lds[wave][u];
-            const int fa = 4 * (m >> 3) + g;  // this lane's fragment within the step
-            const unsigned lo = L.hdr[2 * fa], hi = L.hdr[2 * fa + 1];
-            const uint64_t bm = ((uint64_t)hi << 32) | lo;
-            const unsigned byte = (unsigned)(bm >> (8 * r)) & 0xffu;
-            const int v0 = (int)L.hdr[16 + fa] - (int)L.hdr[16] + __popcll(bm & ((1ull << (8 * r)) - 1ull));
-            // bit j of the byte takes the next value of the run: its index is v0 + popcount of the lower bits
-            const _Float16 *run = (const _Float16 *)L.val + v0;
-            v8f16 a;
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                a[j] = ((byte >> j) & 1u) ? run[__popc(byte & ((1u << j) - 1u))] : (_Float16)0;
+            for (int j = 0; j < 8; ++j) {
+                const double a = j < nblk ? Ra.v[j] : 0.0;
+                const double bv = m < 2 ? P.xv[(2 * j + m) * 4 + g] : 0.0;
+                acc = tile_mma(a, bv, acc);
+            }
+        } else {
+            const v4i32 z = {0, 0, 0, 0};
+            const v8f16 a = __builtin_bit_cast(v8f16, g < nblk ? Ra.v : z);
             v8f16 bv = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (m < 2) bv = *(const v8f16 *)(L.xv + (4 * m + g) * 8);
-            acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bv, acc[u], 0, 0, 0);
+            if (m < 2) bv = *(const v8f16 *)(P.xv + (4 * m + g) * 8);
+            acc = tile_mma(a, bv, acc);
+        }
+        if (flags & 1) {
+            // half 0 = D[0..7][0], half 1 = D[8..15][1]; hand them to lanes 0..15 through LDS
+            if constexpr (F64) {
+                // D[q][0] = reg 0 and D[q+4][0] = reg 1 of lane 16q; D[8+q][1] = reg 2, D[12+q][1] = reg 3 of lane 16q+1
+                if (m == 0) {
+                    P.out[g] = acc[0];
+                    P.out[g + 4] = acc[1];
+                }
+                if (m == 1) {
+                    P.out[8 + g] = acc[2];
+                    P.out[12 + g] = acc[3];
+                }
+            } else {
+                // D[0..3][0] in lane 0, D[4..7][0] in lane 16, D[8..11][1] in lane 33, D[12..15][1] in lane 49
+                if (lane == 0 || lane == 16 || lane == 33 || lane == 49) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) P.out[4 * g + i] = acc[i];
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (lane < 16 && Ra.hdr >= 0) {
+                AT o = P.out[lane];
+                if (!(flags & 2)) o += P.out[lane + 8];  // one chunk in both halves (only lanes 0..7 have rows)
+                y[Ra.hdr] = (VT)((accumulate ? (AT)Ra.yr : (AT)0) + o);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = 0;
         }
         __builtin_amdgcn_wave_barrier();
-    }
-    // rows 0..3 of a chunk: lane 0 (+ lane 33), rows 4..7: lane 16 (+ lane 49); to lanes 0..7 through LDS
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        float *out = (float *)lds[wave][u].val;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float o = acc[u][i] + __shfl(acc[u][i], lane + 33, 64);
-            if (lane == 0 || lane == 16) out[(lane >> 2) + i] = o;
-        }
-        __builtin_amdgcn_wave_barrier();
-        if (row[u] >= 0) y[row[u]] = (_Float16)(yold[u] + out[lane]);
+    };
+    const int na = __builtin_amdgcn_readfirstlane(d1.z);
+    tile_issue<VT>(R0, hdr, atox, tcVal, s0, __builtin_amdgcn_readfirstlane(d0.z), na & 255, lane);
+    tile_issue<VT>(R1, hdr, atox, tcVal, min(s0 + 1, last), __builtin_amdgcn_readfirstlane(d0.w), (na >> 8) & 255, lane);
+    tile_issue<VT>(R2, hdr, atox, tcVal, min(s0 + 2, last), __builtin_amdgcn_readfirstlane(d1.x), (na >> 16) & 255, lane);
+    tile_issue<VT>(R3, hdr, atox, tcVal, min(s0 + 3, last), __builtin_amdgcn_readfirstlane(d1.y), (na >> 24) & 255, lane);
+    gather(R0);
+    gather(R1);
+    for (int s = s0; s < s1; s += 5) {
+        step(s, R0, R2, R4);
+        if (s + 1 < s1) step(s + 1, R1, R3, R0);
+        if (s + 2 < s1) step(s + 2, R2, R4, R1);
+        if (s + 3 < s1) step(s + 3, R3, R0, R2);
+        if (s + 4 < s1) step(s + 4, R4, R1, R3);
     }
 }
 
@@ -941,17 +882,14 @@ hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, v
 
 hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s)
 {
-    if (T.chunkNum <= 0) return hipSuccess;
-    const int perBlock = 4 * (dtype == MX_F64 ? mxk::kTileUF64 : mxk::kTileUF16);  // chunks per workgroup
-    const int grid = (T.chunkNum + perBlock - 1) / perBlock;
+    if (T.nWaves <= 0) return hipSuccess;
+    const int grid = (T.nWaves + 3) / 4;
     if (dtype == MX_F64)
-        hipLaunchKernelGGL(mxk::tile_f64_kernel, dim3(grid), dim3(mxk::kBlock), 0, s, T.chunkPtr, T.fragPtr,
-                           (const uint32_t *)T.fragBit, (const double *)T.tcVal, T.atox, T.rowIdx, (const double *)x,
-                           (double *)y, T.chunkNum, T.dRows, accumulate);
+        hipLaunchKernelGGL((mxk::tile_kernel<double>), dim3(grid), dim3(mxk::kBlock), 0, s, (const int4 *)T.waveDesc, T.hdr,
+                           T.atox, (const double *)T.tcVal, (const double *)x, (double *)y, T.nWaves, accumulate);
     else
-        hipLaunchKernelGGL(mxk::tile_f16_kernel, dim3(grid), dim3(mxk::kBlock), 0, s, T.chunkPtr, T.fragPtr,
-                           (const uint64_t *)T.fragBit, (const _Float16 *)T.tcVal, T.atox, T.rowIdx, (const _Float16 *)x,
-                           (_Float16 *)y, T.chunkNum, T.dRows, accumulate);
+        hipLaunchKernelGGL((mxk::tile_kernel<_Float16>), dim3(grid), dim3(mxk::kBlock), 0, s, (const int4 *)T.waveDesc, T.hdr,
+                           T.atox, (const _Float16 *)T.tcVal, (const _Float16 *)x, (_Float16 *)y, T.nWaves, accumulate);
     return hipGetLastError();
 }
 

@@ -86,12 +86,10 @@ void free_csr(mx::DeviceCsr &A)
 
 void free_tiles(mx::DeviceTiles &T)
 {
-    (void)hipFree(T.chunkPtr);
-    (void)hipFree(T.fragPtr);
-    (void)hipFree(T.fragBit);
-    (void)hipFree(T.tcVal);
+    (void)hipFree(T.waveDesc);
+    (void)hipFree(T.hdr);
     (void)hipFree(T.atox);
-    (void)hipFree(T.rowIdx);
+    (void)hipFree(T.tcVal);
     T = mx::DeviceTiles();
 }
 
@@ -316,67 +314,136 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
     return MX_OK;
 }
 
-// Puts bitmap tiles on the device for the tile kernels: the chunks named by `sel` (all when
-// null), re-packed contiguously.  Column ids go through `colMap` and output rows through
-// `rowMap` when given.  Values keep their order, but the run of every kernel step (8 fragments
-// for binary16, 16 for binary64, counted from the chunk's first fragment) is moved up to a
-// 16-byte boundary, and the device fragPtr holds those padded offsets.
-int upload_tiles(mx_dtype dtype, int chunkNum, const char *sel, int dRows, const int *chunkPtr, const int *fragPtr,
+// Puts tiles on the device for the tile kernels (see DeviceTiles): the fragments named by
+// `selFrag` (all when null), expanded to full blocks.  Column ids go through `colMap` and
+// output rows through `rowMap` when given.
+int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, const int *chunkPtr, const int *fragPtr,
                  const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap,
                  mx::DeviceTiles &T, int *tile_nnz)
 {
     const int es = mx::elem_size(dtype), fragK = mx::frag_k(dtype), fragM = mx::kFragM;
-    const int bitBytes = dtype == MX_F64 ? 4 : 8;
-    const int stepFrags = dtype == MX_F64 ? 16 : 8, align = 16 / es;
-    std::vector<int> dChunkPtr(1, 0), dFragPtr, dAtox, rowIdx;
-    std::vector<unsigned char> dBits, dVal;
-    const unsigned char *bits = (const unsigned char *)fragBit, *tv = (const unsigned char *)tcVal;
-    int nsel = 0, nnz = 0;
-    size_t voff = 0;  // in elements
-    for (int w = 0; w < chunkNum; ++w) {
-        if (sel && !sel[w]) continue;
-        ++nsel;
-        const int f0 = chunkPtr[w], f1 = chunkPtr[w + 1];
-        for (int f = f0; f < f1; ++f) {
-            if ((f - f0) % stepFrags == 0) voff = (voff + align - 1) / align * align;
-            dFragPtr.push_back((int)voff);
-            const int cnt = fragPtr[f + 1] - fragPtr[f];
-            dVal.resize((voff + cnt) * es, 0);
-            if (cnt) std::memcpy(&dVal[voff * es], tv + (size_t)fragPtr[f] * es, (size_t)cnt * es);
-            voff += cnt;
-            nnz += cnt;
-            for (int k = 0; k < fragK; ++k) {
-                const int c = atox[(size_t)f * fragK + k];
-                dAtox.push_back(colMap ? colMap[c] : c);
+    const int SF = mx::tile_slots(dtype), HF = SF / 2, H = mx::kTileHdr, BS = fragM * fragK;  // BS: values per block
+    const bool f64 = dtype == MX_F64;
+    const uint32_t *bit32 = (const uint32_t *)fragBit;
+    const uint64_t *bit64 = (const uint64_t *)fragBit;
+    const unsigned char *tv = (const unsigned char *)tcVal;
+    std::vector<int> hdr, dAtox, stepVo, stepA, stepChunkEnd;  // stepChunkEnd: 1 when a wave may end after the step
+    std::vector<unsigned char> dVal;
+    size_t voff = 0;  // values stored so far; always a multiple of BS, so every block is 16-byte aligned
+    int nsel = 0, nnz = 0, nfr = 0;
+    auto put_block = [&](size_t s, int slot, int f) {  // fragment f, expanded, as the next block of step s
+        const int cnt = fragPtr[f + 1] - fragPtr[f];
+        dVal.resize((voff + BS) * es, 0);
+        const uint64_t bm = f64 ? (uint64_t)bit32[f] : bit64[f];
+        int k = 0;
+        for (int bit = 0; bit < BS; ++bit)
+            if ((bm >> bit) & 1ull) {
+                std::memcpy(&dVal[(voff + bit) * es], tv + (size_t)(fragPtr[f] + k) * es, es);
+                ++k;
+            }
+        voff += BS;
+        nnz += cnt;
+        ++nfr;
+        for (int c = 0; c < fragK; ++c) {
+            const int col = atox[(size_t)f * fragK + c];
+            dAtox[s * 64 + (size_t)slot * fragK + c] = colMap ? colMap[col] : col;
+        }
+    };
+    // a step with the fragments a0 (half 0) and a1 (half 1) of the chunks w0 and w1 (w1 < 0: none)
+    auto emit = [&](const int *a0, int n0, int w0, const int *a1, int n1, int w1, int flags) {
+        const size_t s = stepVo.size();
+        hdr.resize((s + 1) * H, 0);
+        dAtox.resize((s + 1) * 64, -1);
+        stepVo.push_back((int)voff);
+        stepA.push_back(n0);
+        stepChunkEnd.push_back(flags & 1);
+        for (int i = 0; i < 16; ++i) hdr[s * H + i] = -1;
+        for (int half = 0; half < 2; ++half) {
+            const int w = half ? w1 : w0;
+            if (w < 0 || (half && !(flags & 2))) continue;
+            for (int i = 0; i < fragM; ++i) {
+                const int local = w * fragM + i;
+                hdr[s * H + half * 8 + i] = local < dRows ? (rowMap ? rowMap[local] : local) : -1;
             }
         }
-        dBits.insert(dBits.end(), bits + (size_t)f0 * bitBytes, bits + (size_t)f1 * bitBytes);
-        dChunkPtr.push_back(dChunkPtr.back() + (f1 - f0));
-        for (int i = 0; i < fragM; ++i) {
-            const int local = w * fragM + i;
-            rowIdx.push_back(local < dRows ? (rowMap ? rowMap[local] : local) : -1);
+        hdr[s * H + 16] = flags;
+        hdr[s * H + 17] = n0;
+        hdr[s * H + 18] = n1;
+        for (int i = 0; i < n0; ++i) put_block(s, mx::tile_slot(dtype, 0, i), a0[i]);
+        for (int i = 0; i < n1; ++i) put_block(s, mx::tile_slot(dtype, 1, i), a1[i]);
+    };
+    std::vector<int> fsel, pending;
+    int pendingChunk = -1;  // a small chunk waiting for a partner
+    for (int w = 0; w < chunkNum; ++w) {
+        fsel.clear();
+        for (int f = chunkPtr[w]; f < chunkPtr[w + 1]; ++f)
+            if (fragPtr[f + 1] > fragPtr[f] && (!selFrag || selFrag[f])) fsel.push_back(f);
+        if (fsel.empty()) continue;
+        ++nsel;
+        if ((int)fsel.size() <= HF) {
+            if (pendingChunk >= 0) {
+                emit(pending.data(), (int)pending.size(), pendingChunk, fsel.data(), (int)fsel.size(), w, 3);
+                pendingChunk = -1;
+            } else {
+                pendingChunk = w;
+                pending = fsel;
+            }
+        } else {
+            for (size_t i0 = 0; i0 < fsel.size(); i0 += SF) {
+                const int n = (int)std::min(fsel.size() - i0, (size_t)SF), n0 = std::min(n, HF);
+                emit(&fsel[i0], n0, w, &fsel[i0 + n0], n - n0, w, i0 + SF >= fsel.size() ? 1 : 0);
+            }
         }
         if (voff > 2000000000u) {
             set_error("tile layout: too many values for 32-bit offsets");
             return MX_ERR_ARG;
         }
     }
-    dFragPtr.push_back((int)voff);
+    if (pendingChunk >= 0) emit(pending.data(), (int)pending.size(), pendingChunk, nullptr, 0, -1, 3);
+    const int steps = (int)stepVo.size();
     T.chunkNum = nsel;
-    T.frags = dChunkPtr.back();
+    T.frags = nfr;
     T.vals = nnz;
-    // ragged last chunk: rows past dRows carry -1 and are cut off through dRows
-    T.dRows = nsel * fragM;
-    while (T.dRows > 0 && rowIdx[T.dRows - 1] < 0) --T.dRows;
+    T.stored = (long long)voff;
+    T.steps = steps;
     if (tile_nnz) *tile_nnz = nnz;
-    if (nsel == 0) return MX_OK;
+    if (steps == 0) return MX_OK;
+    // waves: whole chunks, about `per` steps each; few enough waves that all of them are resident
+    // at once (24 per CU), so that none has to wait for a second round
+    int nCU = 256;
+    {
+        hipDeviceProp_t prop;
+        int dev = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            nCU = std::max(1, prop.multiProcessorCount);
+    }
+    const int tper = std::getenv("MX_TILE_PER") ? std::atoi(std::getenv("MX_TILE_PER")) : 0;
+    const int per = tper > 0 ? tper : std::max(2, (steps + nCU * 24 - 1) / (nCU * 24));
+    std::vector<int> waveDesc;
+    for (int s0 = 0; s0 < steps;) {
+        int s1 = std::min(steps, s0 + per);
+        while (s1 < steps && !stepChunkEnd[s1 - 1]) ++s1;
+        int d[8] = {s0, s1, 0, 0, 0, 0, 0, 0};
+        for (int k = 0; k < 4; ++k) {
+            const int sk = std::min(s0 + k, s1 - 1);
+            d[2 + k] = stepVo[sk];
+            d[6] |= stepA[sk] << (8 * k);
+        }
+        waveDesc.insert(waveDesc.end(), d, d + 8);
+        for (int s = s0; s < s1; ++s) {  // the step four further on (the wave's last when past it)
+            const int s4 = std::min(s + 4, s1 - 1);
+            hdr[(size_t)s * H + 19] = stepVo[s4];
+            hdr[(size_t)s * H + 20] = stepA[s4];
+        }
+        s0 = s1;
+    }
+    T.nWaves = (int)waveDesc.size() / 8;
     int rc;
-    if ((rc = upload(&T.chunkPtr, dChunkPtr.data(), dChunkPtr.size(), 64))) return rc;
-    if ((rc = upload(&T.fragPtr, dFragPtr.data(), dFragPtr.size(), 64))) return rc;
-    if ((rc = upload_bytes(&T.fragBit, dBits.data(), dBits.size(), 256))) return rc;
+    if ((rc = upload(&T.waveDesc, waveDesc.data(), waveDesc.size(), 64))) return rc;
+    if ((rc = upload(&T.hdr, hdr.data(), hdr.size(), 256))) return rc;
+    if ((rc = upload(&T.atox, dAtox.data(), dAtox.size(), 256))) return rc;
+    // a lane of a step with few blocks reads where an absent block would be: 4 KB of slack
     if ((rc = upload_bytes(&T.tcVal, dVal.data(), dVal.size(), 8192))) return rc;
-    if ((rc = upload(&T.atox, dAtox.data(), dAtox.size(), 64))) return rc;
-    if ((rc = upload(&T.rowIdx, rowIdx.data(), rowIdx.size(), 64))) return rc;
     return MX_OK;
 }
 
@@ -584,10 +651,19 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
     return MX_OK;
 }
 
-// Minimum fill of a chunk's fragments for the MFMA tile kernel to take it (default plans).
-// Below it the chunk's entries cost fewer bytes as CSR: a fragment costs 8 bytes of bitmap and
-// pointer plus fragK indices, an entry in CSR costs 4 bytes of index.
-static double tile_gate(mx_dtype dtype) { return dtype == MX_F64 ? 0.25 : 0.20; }
+// Minimum fill of a fragment for the MFMA tile kernel to take it (default plans;
+// MX_TILE_GATE=<fraction> overrides).  A fragment costs its bitmap, its value offset and fragK
+// column ids whatever it holds, and the decode work of a whole tile; below about half full the
+// same entries are cheaper in the CSR part.
+static double tile_gate(mx_dtype)
+{
+    const char *e = std::getenv("MX_TILE_GATE");
+    if (e) {
+        const double v = std::atof(e);
+        if (v >= 0.0 && v <= 1.0) return v;
+    }
+    return 0.5;
+}
 
 extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
 {
@@ -627,24 +703,39 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             std::vector<int> colOrig(cols);
             for (int c = 0; c < P->dCols; ++c) colOrig[c] = P->descColId[c];
             for (int c = P->dCols; c < cols; ++c) colOrig[c] = P->newArray[c - P->dCols];
-            // which chunks go to the tile kernel
-            const int chunkNum = P->chunkNum;
-            std::vector<char> sel(chunkNum, 0);
+            // which fragments go to the tile kernel
+            const int chunkNum = P->chunkNum, nFrags = P->chunkPtr[chunkNum];
+            std::vector<char> sel((size_t)nFrags, 0);
             const double gate = tile_gate(P->dtype);
-            for (int w = 0; w < chunkNum; ++w) {
-                const int nf = P->chunkPtr[w + 1] - P->chunkPtr[w];
-                if (nf == 0) continue;
-                const int vals = P->fragPtr[P->chunkPtr[w + 1]] - P->fragPtr[P->chunkPtr[w]];
-                const double fill = (double)vals / ((double)nf * fragM * fragK);
-                if (flags & MX_PLAN_NO_TILES) sel[w] = 0;
-                else if (flags & MX_PLAN_ALL_TILES) sel[w] = 1;
-                else sel[w] = fill >= gate;
+            if (!(flags & MX_PLAN_NO_TILES)) {
+                for (int f = 0; f < nFrags; ++f) {
+                    const int vals = P->fragPtr[f + 1] - P->fragPtr[f];
+                    sel[f] = (flags & MX_PLAN_ALL_TILES) ? vals > 0 : (vals > 0 && (double)vals >= gate * fragM * fragK);
+                }
             }
-            // CSR part = residual rows (+ the A_dd rows of chunks left out of the tile kernel)
+            // fragment of every A_dd entry: the rank of its column among the chunk's columns, / fragK
+            auto frag_of = [&](int w, int ddcol) {
+                const int f0 = P->chunkPtr[w], f1 = P->chunkPtr[w + 1];
+                const int *a = &P->sparse_AToX_index[(size_t)f0 * fragK];
+                // the used prefix of the chunk's list is ascending; the zero padding after it is not
+                int n = (f1 - f0) * fragK;
+                while (n > 1 && a[n - 1] == 0) --n;
+                const int rank = (int)(std::lower_bound(a, a + n, ddcol) - a);
+                return f0 + rank / fragK;
+            };
+            // CSR part = residual rows + the A_dd entries whose fragment stays out of the tile kernel
             std::vector<int> rowPtr((size_t)rows + 1, 0);
             for (int r = 0; r < rows; ++r) rowPtr[r + 1] = P->cdRowPtr[r + 1] - P->cdRowPtr[r];
-            for (int i = 0; i < P->dRows; ++i)
-                if (!sel[i / fragM]) rowPtr[P->rId[i] + 1] += P->ddRowPtr[i + 1] - P->ddRowPtr[i];
+            std::vector<char> keep((size_t)P->ddRowPtr[P->dRows], 0);  // A_dd entry goes to the CSR part
+#pragma omp parallel for schedule(static)
+            for (int i = 0; i < P->dRows; ++i) {
+                int n = 0;
+                for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
+                    keep[p] = !sel[frag_of(i / fragM, P->ddColInd[p])];
+                    n += keep[p];
+                }
+                rowPtr[P->rId[i] + 1] += n;
+            }
             for (int r = 0; r < rows; ++r) rowPtr[r + 1] += rowPtr[r];
             const int csrNnz = rowPtr[rows];
             std::vector<int> col((size_t)csrNnz);
@@ -661,12 +752,13 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             }
 #pragma omp parallel for schedule(static)
             for (int i = 0; i < P->dRows; ++i) {
-                if (sel[i / fragM]) continue;
                 const int r = P->rId[i];
                 int q = rowPtr[r] + (P->cdRowPtr[r + 1] - P->cdRowPtr[r]);
-                for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p, ++q) {
+                for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
+                    if (!keep[p]) continue;
                     col[q] = P->descColId[P->ddColInd[p]];
                     std::memcpy(&val[(size_t)q * es], ddv + (size_t)p * es, es);
+                    ++q;
                 }
             }
             rc = setup_csr_part(plan, rowPtr.data(), col.data(), val.data(), flags);
@@ -709,10 +801,13 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     // what each kernel has to move at least once: its arrays, x once, its y rows
     info->csr_bytes = (double)plan->csr_nnz * (es + 4) + ((double)plan->rows + 1) * 4 + (double)plan->cols * es +
                       (double)plan->rows * es;
-    info->tile_bytes = plan->tiles.chunkNum
-                           ? (double)plan->tiles.frags * (bitBytes + 4 + 4.0 * fragK) + (double)plan->tiles.vals * es +
-                                 ((double)plan->tiles.chunkNum + 1) * 4 + (double)plan->tiles.dRows * (4 + 2 * es)
+    // what the tile kernel reads and writes per launch: headers, column ids, values, x once per
+    // column id, y once per row
+    info->tile_bytes = plan->tiles.steps
+                           ? (double)plan->tiles.steps * (mx::kTileHdr * 4.0 + 64 * 4.0) + (double)plan->tiles.stored * es +
+                                 (double)plan->tiles.frags * fragK * es + (double)plan->tiles.chunkNum * 8 * 2 * es
                            : 0.0;
+    (void)bitBytes;
     return MX_OK;
 }
 
@@ -942,7 +1037,6 @@ static int du_any(mx_dtype dtype, const int *chunkPtr, const int *fragPtr, const
         if ((r = upload_tiles(dtype, chunkNum, nullptr, dRows, chunkPtr, fragPtr, fragBit, tcVal, atox, nullptr, nullptr, T,
                               nullptr)))
             return r;
-        T.dRows = dRows;
         if ((r = upload_bytes(&dx, x_d, dCols * es))) return r;
         // FP64 uploads the caller's y and adds to it; FP16 starts from zero
         // (du_tcSpMV_fp64.cu:296-297 vs du_tcSpMV_fp16_v2.cu:146-147)
