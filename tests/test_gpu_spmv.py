@@ -292,6 +292,129 @@ def test_long_rows_take_the_multi_tile_path(mx, ora):
         plan.close()
 
 
+def _random_csr(mx, rng, rows, cols, lens, dtype):
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = np.concatenate([np.sort(rng.choice(cols, int(l), replace=False)) for l in lens] + [np.zeros(0, int)]).astype(np.int32)
+    return mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, rp[-1]).astype(dtype))
+
+
+@pytest.mark.parametrize("reduce", ["rows", "scan"])
+def test_row_kernel_reductions_on_uneven_rows(mx, ora, reduce, monkeypatch):
+    """Both ways the row kernel sums a tile (lanes per row; segmented scan): rows of length 0, 1,
+    a few and several hundred in one tile, empty rows first and last, whole tiles of empty rows,
+    and y accumulated into (cdspmv adds A*x to the y it is given)."""
+    import torch
+    monkeypatch.setenv("MX_CSR_REDUCE", reduce)
+    rng = np.random.default_rng(5)
+    cols = 5000
+    for dtype, tol in ((np.float64, F64_TOL), (np.float16, F16_TOL)):
+        for trial in range(3):
+            lens = np.minimum(np.floor(1.0 / rng.uniform(1e-3, 1.0, 4000) ** 0.9).astype(int), 900)
+            lens[rng.uniform(size=lens.size) < 0.3] = 0
+            lens[:5] = 0
+            lens[-3:] = 0
+            lens[1000:1300] = 0  # more empty rows than one tile holds products
+            A = _random_csr(mx, rng, lens.size, cols, lens, dtype)
+            x = rng.uniform(-1, 1, cols).astype(dtype)
+            ref = oracle_y(ora, mx, A, x)
+            print("uneven rows reduce=%s dtype=%s trial=%d nnz=%d" % (reduce, dtype.__name__, trial, A.nnz), flush=True)
+            part = mx.Partition(A, 0.0, 0.0)
+            plan = mx.Plan(part, mx.MX_PLAN_CSR_ROWS)
+            y = plan.spmv(torch.from_numpy(x).cuda())
+            torch.cuda.synchronize()
+            assert rel_l2(y.cpu().numpy(), ref) <= tol
+            plan.close()
+            part.close()
+            y0 = rng.uniform(-1, 1, lens.size).astype(dtype)
+            got = mx.cdspmv(A, x, y0.copy())[0]
+            want = y0.astype(np.float64) + np.asarray(ref, np.float64)
+            assert rel_l2(got, want) <= (tol if dtype == np.float64 else 2e-2)
+
+
+def test_slice_kernel_layouts(mx, ora):
+    """The column-slice kernel on shapes that stress its layout: a ragged end of x (columns not a
+    multiple of a 16-byte vector), one slice only, several slices of which one is empty, row
+    groups at their size limit, rows without entries, rows much longer than the others."""
+    import torch
+    rng = np.random.default_rng(11)
+    shapes = [
+        # rows, cols, mean row length, dtype
+        (900, 16001, 40, np.float64),     # one slice, ragged x
+        (3000, 40003, 60, np.float64),    # three slices, ragged x
+        (20000, 33001, 14, np.float64),   # more rows than 256 groups of the smallest size would hold evenly
+        (1500, 70001, 90, np.float16),    # two binary16 slices, ragged x
+        (9000, 8000, 30, np.float16),     # one binary16 slice
+    ]
+    for rows, cols, mean, dtype in shapes:
+        lens = rng.poisson(mean, rows)
+        lens[rng.uniform(size=rows) < 0.05] = 0
+        lens[rows // 2] = min(cols, 40 * mean)
+        A = _random_csr(mx, rng, rows, cols, lens, dtype)
+        if dtype == np.float64 and cols > 40000:
+            # empty the middle slice: columns 16384..32767 are moved elsewhere
+            ci = A.colInd.copy()
+            mid = (ci >= 16384) & (ci < 32768)
+            ci[mid] = ci[mid] % 16384
+            A = mx.Csr(rows, cols, A.rowPtr, ci, A.val)  # duplicates inside a row are summed
+        x = rng.uniform(-1, 1, cols).astype(dtype)
+        ref = oracle_y(ora, mx, A, x)
+        tol = F64_TOL if dtype == np.float64 else F16_TOL
+        print("slice layout rows=%d cols=%d mean=%d dtype=%s" % (rows, cols, mean, dtype.__name__), flush=True)
+        part = mx.Partition(A, 0.0, 0.0)
+        plan = mx.Plan(part, mx.MX_PLAN_CSR_SLICES)
+        assert plan.info["csr_variant"] == 1, "the matrix was meant to take the slice kernel"
+        xd = torch.from_numpy(x).cuda()
+        y = plan.spmv(xd)
+        torch.cuda.synchronize()
+        assert rel_l2(y.cpu().numpy(), ref) <= tol
+        y2 = plan.spmv(xd, y)  # the partial sums of the first call must not leak into the second
+        torch.cuda.synchronize()
+        assert rel_l2(y2.cpu().numpy(), ref) <= tol
+        plan.close()
+        part.close()
+
+
+def test_tile_kernel_step_packing(mx, ora):
+    """Chunks with one fragment, with exactly half a step, a whole step, more than a step and a
+    ragged last chunk; every fill from almost empty to full, through the fragment gate and
+    with every fragment forced into the tile kernel."""
+    import torch
+    rng = np.random.default_rng(21)
+    for dtype, fragK, tol in ((np.float64, 4, F64_TOL), (np.float16, 8, F16_TOL)):
+        rows, cols = 8 * 37 + 3, 4096
+        rp = [0]
+        ci, va = [], []
+        for r in range(rows):
+            chunk = r // 8
+            nfr = [1, 4, 8, 9, 16, 17, 40][chunk % 7]       # fragments of the chunk
+            fill = [1.0, 0.75, 0.5, 0.2, 0.05][chunk % 5]    # density inside them
+            base = (chunk * 131) % (cols - nfr * fragK)
+            c = np.arange(base, base + nfr * fragK)
+            keep = rng.uniform(size=c.size) < fill
+            if not keep.any():
+                keep[rng.integers(c.size)] = True
+            c = c[keep]
+            ci.append(c)
+            va.append(rng.uniform(-1, 1, c.size))
+            rp.append(rp[-1] + c.size)
+        A = mx.Csr(rows, cols, np.array(rp, np.int32), np.concatenate(ci).astype(np.int32), np.concatenate(va).astype(dtype))
+        x = rng.uniform(-1, 1, cols).astype(dtype)
+        ref = oracle_y(ora, mx, A, x)
+        xd = torch.from_numpy(x).cuda()
+        for tau in ((1.0, 1.0), (1.0, 0.5), (0.5, 0.5)):
+            for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES):
+                print("tile packing dtype=%s tau=%s flags=%d" % (dtype.__name__, tau, fl), flush=True)
+                part = mx.Partition(A, *tau)
+                plan = mx.Plan(part, fl)
+                y = plan.spmv(xd)
+                torch.cuda.synchronize()
+                assert rel_l2(y.cpu().numpy(), ref) <= tol, (tau, fl, plan.info)
+                if fl == mx.MX_PLAN_ALL_TILES and tau == (1.0, 1.0):
+                    assert plan.info["tile_nnz"] == A.nnz and plan.info["csr_nnz"] == 0
+                plan.close()
+                part.close()
+
+
 def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
     """matxtract_perftest's stdout keeps the forms the reference's scripts grep for."""
     import re
