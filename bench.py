@@ -29,9 +29,10 @@ GRID = (0.0, 0.25, 0.5, 0.75, 1.0)
 # known size (--calibrate-copy): FETCH_SIZE x 2.000, WRITE_SIZE x 1.000.  The text files under profiles/
 # hold the counter values.  (workload, kernel) -> bytes
 TRAFFIC = {
-    (2, "csr_rows_kernel<f64>"): 47183402,
-    (2, "csr_slice_kernel<f64>"): 54402556,
-    (3, "csr_rows_kernel<f64>"): 287447594,
+    (2, "csr_rows_kernel<f64>"): 47165962,
+    (2, "csr_slice_kernel<f64>"): 59259567,
+    (3, "csr_rows_kernel<f64>"): 287435306,
+    (4, "csr_rows_kernel<f16>"): 97439082,
 }
 WORKLOADS = {
     1: "configs[0]: FP64 random 4096x4096, 16 nnz/row",
