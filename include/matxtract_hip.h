@@ -150,9 +150,11 @@ int mx_plan_create(const mx_partition *p, int flags, mx_plan **out);
 void mx_plan_destroy(mx_plan *plan);
 
 /* y = A*x on the device.  x [cols] and y [rows] are DEVICE pointers of the plan's value
- * type; `stream` is a hipStream_t (NULL = default stream).  Asynchronous.  The hybrid
- * sequence of test/test_autotc_spmv.cpp:1507-1559 (tile part, scatter through rId,
- * residual accumulated on top) without host round trips. */
+ * type, x 16-byte aligned (the kernels copy it in 16-byte vectors; a plan whose CSR part keeps
+ * x in LDS returns MX_ERR_ARG otherwise); `stream` is a hipStream_t (NULL = default stream).
+ * Asynchronous.  The hybrid sequence of test/test_autotc_spmv.cpp:1507-1559 (tile part, scatter
+ * through rId, residual accumulated on top) without host round trips.  A plan holds device
+ * buffers of partial sums: calls on the same plan must not overlap in time. */
 int mx_spmv(mx_plan *plan, const void *x_dev, void *y_dev, void *stream);
 
 /* n back-to-back SpMVs y = A*x on `stream`, queued from C without returning to the caller in

@@ -1,11 +1,13 @@
 // gfx950 kernels of the hybrid SpMV and their launchers.
 //
-//   csr_rows_kernel   residual / plain CSR part (stands in for cdspmv_kernel,
-//                     src/spmv_kernel/cdSpMV.cu:244-392).  HBM-bound.
-//   tile_f64_kernel   8x4 bitmap tiles through v_mfma_f64_16x16x4_f64 (stands in for
-//                     tcspmv_kernel_fp64, src/spmv_kernel/du_tcSpMV_fp64.cu:81-160).
-//   tile_f16_kernel   8x8 bitmap tiles through v_mfma_f32_16x16x32_f16, f32 accumulation
-//                     (stands in for tcspmv_kernel_fp16_v2, du_tcSpMV_fp16_v2.cu:4-110).
+//   csr_rows_kernel    residual / plain CSR part, x gathered from memory (stands in for
+//                      cdspmv_kernel, src/spmv_kernel/cdSpMV.cu:244-392).
+//   csr_slice_kernel   the same part with x resident in LDS, for matrices with a small x and
+//   slice_combine_kernel   scattered columns; the second adds the per-slice partial sums.
+//   tile_kernel<double>    8x4 tiles through v_mfma_f64_16x16x4_f64 (stands in for
+//                      tcspmv_kernel_fp64, src/spmv_kernel/du_tcSpMV_fp64.cu:81-160).
+//   tile_kernel<_Float16>  8x8 tiles through v_mfma_f32_16x16x32_f16, f32 accumulation
+//                      (stands in for tcspmv_kernel_fp16_v2, du_tcSpMV_fp16_v2.cu:4-110).
 //
 // Row ownership: every output row is written by exactly one lane of one workgroup in each
 // kernel, so there are no atomics anywhere; the tile kernel runs after the CSR kernel on the

@@ -23,7 +23,7 @@ def oracle_y(ora, mx, A, x):
 
 def test_mfma_operand_layout_f64(mx):
     """v_mfma_f64_16x16x4_f64: A[i][k] in lane 16k+i, B[k][j] in lane 16k+j, D[i][j] in
-    accumulator register i//4 of lane 16*(i%4)+j -- the mapping tile_f64_kernel relies on."""
+    accumulator register i//4 of lane 16*(i%4)+j -- the mapping tile_kernel<double> relies on."""
     from matxtractt_amd import _lib
     rng = np.random.default_rng(5)
     A = rng.integers(-4, 5, (16, 4)).astype(np.float64)
@@ -44,7 +44,7 @@ def test_mfma_operand_layout_f64(mx):
 
 def test_mfma_operand_layout_f16(mx):
     """v_mfma_f32_16x16x32_f16: A[i][8g+e] is element e of lane 16g+i, B[8g+e][j] element e of
-    lane 16g+j, D[i][j] accumulator register i%4 of lane 16*(i//4)+j (tile_f16_kernel)."""
+    lane 16g+j, D[i][j] accumulator register i%4 of lane 16*(i//4)+j (tile_kernel<_Float16>)."""
     from matxtractt_amd import _lib
     rng = np.random.default_rng(6)
     A = rng.integers(-4, 5, (16, 32)).astype(np.float16)
