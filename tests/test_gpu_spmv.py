@@ -101,7 +101,7 @@ def test_hybrid_spmv_matches_oracle(mx, ora, cfg, scale, flags):
         part.close()
 
 
-# ---------------------------------------------------------------- full BASELINE sizes
+# ---------------------------------------------------------------- full benchmark sizes
 FULL = [
     # (workload, taus)
     (2, [(0.0, 0.0), (0.5, 0.25), (1.0, 1.0)]),
