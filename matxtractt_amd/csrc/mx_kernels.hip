@@ -540,15 +540,20 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         for (int i = 2 * kSliceThreads + 2 * tid; i < wgChunks * 64; i += 2 * kSliceThreads)
             *(unsigned *)(rowsL + i) = *(const unsigned *)(chunkRows + (size_t)wgChunk0 * 64 + i);
         for (int i = kSliceThreads + tid; i < wgChunks; i += kSliceThreads) endsL[i] = chunkEnd[wgChunk0 + i];
+        // ragged end of x: the last, partial vector is filled element by element, and left out
+        // of the sweep below (whose lane for it is in another wave and holds zeros)
+        int ragged = -1;
+        if (cols % EPV) {
+            const int c = cols - cols % EPV, i = (c - slice * sliceCols) / EPV;
+            if (c >= slice * sliceCols && i < nvec) {
+                ragged = i;
+                if (tid < EPV) xs[i * EPV + tid] = tid < cols % EPV ? x[c + tid] : (VT)0;
+            }
+        }
 #pragma unroll
         for (int q = 0; q < CB; ++q) {
             const int i = tid + q * kSliceThreads;
-            if (i < nvec) *(v4i32 *)(xs + i * EPV) = xv[q];
-        }
-        // ragged end of x: the last, partial vector is filled element by element
-        if (cols % EPV) {
-            const int c = cols - cols % EPV, i = (c - slice * sliceCols) / EPV;
-            if (c >= slice * sliceCols && i < nvec && tid < EPV) xs[i * EPV + tid] = tid < cols % EPV ? x[c + tid] : (VT)0;
+            if (i < nvec && i != ragged) *(v4i32 *)(xs + i * EPV) = xv[q];
         }
     }
     // the ring is issued only now: a wave that is busy issuing loads cannot store the slice, and
