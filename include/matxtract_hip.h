@@ -76,6 +76,7 @@ typedef struct mx_partition_view {
     const int *cdRowPtr;  /* residual A_CD (rows x cols): columns [0,dCols) = dense-column */
     const int *cdColInd;  /* ranks, [dCols,cols) = dCols + index into newArray             */
     const void *cdVal;
+    float tau_c, tau_r;   /* the fractions the partition was made with */
 } mx_partition_view;
 
 /* ---------------------------------------------------------------------------------- */
@@ -97,6 +98,16 @@ int mx_partition_get(const mx_partition *p, mx_partition_view *view);
  * newArray_, chunkPtr, sparse_AToX_index, fragPtr, fragBit, tcVal, cdRowPtr, cdColInd,
  * cdVal), little-endian, in that order. */
 uint64_t mx_partition_hash(const mx_partition *p);
+
+/* A partition on disk.  The file starts with the reference's "_preprocessed.dat" fields in its
+ * own byte layout (written by test/tcpreprocess.cpp:1208-1255, read by test/tckernel.cpp:586-638:
+ * chunkPtr, sparse_AToX_index, fragPtr, fragBit, tcVal -- so that tool reads the tile part of a
+ * binary64 file unchanged) and goes on with what the reference does not store: sizes,
+ * thresholds, the index maps, A_dd, the residual A_CD and a checksum.  mx_partition_load checks
+ * the precision, every size and index range and the checksum; a file written by the reference
+ * tool (tile part only) is refused with MX_ERR_IO and a message that says so. */
+int mx_partition_save(const mx_partition *p, const char *path);
+int mx_partition_load(const char *path, mx_dtype dtype, mx_partition **out);
 
 /* csr2csc / csc2csr of utilities/csr2csc.cpp:4-203 as a host transpose: each output line
  * lists its entries by ascending source line, equal pairs in source order.  Outputs are

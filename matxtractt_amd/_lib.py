@@ -42,6 +42,7 @@ class PartitionView(C.Structure):
         ("fragBit", C.c_void_p), ("tcVal", C.c_void_p),
         ("nnzCD", C.c_int),
         ("cdRowPtr", C.c_void_p), ("cdColInd", C.c_void_p), ("cdVal", C.c_void_p),
+        ("tau_c", C.c_float), ("tau_r", C.c_float),
     ]
 
 
@@ -63,6 +64,8 @@ SIGNATURES = {
     "mx_partition_destroy": (None, [_vp]),
     "mx_partition_get": (_i, [_vp, C.POINTER(PartitionView)]),
     "mx_partition_hash": (C.c_uint64, [_vp]),
+    "mx_partition_save": (_i, [_vp, C.c_char_p]),
+    "mx_partition_load": (_i, [C.c_char_p, _i, _pp]),
     "mx_transpose": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _pp, _pp, _pp]),
     "mx_free": (None, [_vp]),
     "mx_mmio_read": (_i, [C.c_char_p, _i, _pi, _pi, _pi, _pi, _pp, _pp, _pp]),

@@ -6,6 +6,7 @@ Names follow the reference driver (test/test_autotc_spmv.cpp): a ``Partition`` i
 main() derives from (A, col_frac, hot_frac); a ``Plan`` is that partition resident on the GPU.
 """
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -131,6 +132,23 @@ class Partition:
         self._A = A  # keep the input arrays alive during the call
         st = A.struct()
         check(_lib.load().mx_partition_create(C.byref(st), float(tau_c), float(tau_r), C.byref(self._h)))
+        self._bind()
+
+    @classmethod
+    def load(cls, path, dtype=MX_F64):
+        """A partition written by save() (mx_partition_load)."""
+        self = cls.__new__(cls)
+        self._h = C.c_void_p()
+        self._A = None
+        check(_lib.load().mx_partition_load(os.fsencode(path), int(dtype), C.byref(self._h)))
+        self._bind()
+        return self
+
+    def save(self, path):
+        """Write the partition to `path`: the reference's _preprocessed.dat fields, then the rest."""
+        check(_lib.load().mx_partition_save(self._h, os.fsencode(path)))
+
+    def _bind(self):
         v = _lib.PartitionView()
         check(_lib.load().mx_partition_get(self._h, C.byref(v)))
         for name, _ in _lib.PartitionView._fields_:
@@ -153,6 +171,7 @@ class Partition:
         self.cdRowPtr = _view(v.cdRowPtr, v.rows + 1, np.int32)
         self.cdColInd = _view(v.cdColInd, v.nnzCD, np.int32)
         self.cdVal = _view(v.cdVal, v.nnzCD, vt)
+        self.tau_c, self.tau_r = float(v.tau_c), float(v.tau_r)
 
     @property
     def hash(self):

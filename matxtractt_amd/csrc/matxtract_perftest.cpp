@@ -7,7 +7,8 @@
 // Additive options: --scale S (shrink a synthetic workload), --seed S, --keep-values (do not
 // overwrite the file's values with i%15 as the reference does at :1091), --warm W --iters K
 // (default 200 / 4000), --no-tiles / --all-tiles (plan flags), --json (one JSON record on the
-// last line).  Precision is the build's: -Dfp64 -> FP64 binary, otherwise FP16.
+// last line), --partition-cache FILE (read the partition from FILE when it was made for a
+// matrix of this shape with these fractions, otherwise compute it and write FILE).  Precision is the build's: -Dfp64 -> FP64 binary, otherwise FP16.
 //
 // Lines other tools parse (ML/bayes_opt.py:64, script/duse.sh:35-38) keep their form:
 //   cols_ratio = %f / TC_nnz_ratio = %lf / MatXtract time = %lf ms / Success! ... |
@@ -92,6 +93,7 @@ int main(int argc, char **argv)
     double scale = 1.0;
     unsigned long long seed = 0;
     bool keepValues = false, json = false;
+    std::string cachePath;
     for (int i = 1; i < argc; ++i) {
         std::string a = argv[i];
         auto next = [&](const char *name) -> const char * {
@@ -110,6 +112,7 @@ int main(int argc, char **argv)
         else if (a == "--no-tiles") planFlags = MX_PLAN_NO_TILES;
         else if (a == "--all-tiles") planFlags = MX_PLAN_ALL_TILES;
         else if (a == "--json") json = true;
+        else if (a == "--partition-cache") cachePath = next("--partition-cache");
         else pos.push_back(a);
     }
     const size_t npos = pos.size() + (config ? 1 : 0);  // a --config stands for the file name
@@ -179,9 +182,26 @@ int main(int argc, char **argv)
         std::cout << "---------------------Compression Info--------------------" << std::endl;
     }
     auto t0 = std::chrono::steady_clock::now();
-    mx_partition *part = matxtract_preprocess(csrVal, csrRowPtr, csrColInd, rowA, colA, nnzA, colProp, rowProp);
+    mx_partition *part = nullptr;
+    bool fromCache = false;
+    if (!cachePath.empty() && mx_partition_load(cachePath.c_str(), MX_VALT_DTYPE, &part) == MX_OK) {
+        // The file is used only if it was made from a matrix of this shape with these fractions.
+        mx_partition_view cv;
+        mx_partition_get(part, &cv);
+        fromCache = cv.rows == rowA && cv.cols == colA && cv.nnz == (long long)nnzA && cv.tau_c == colProp && cv.tau_r == rowProp;
+        if (!fromCache) {
+            mx_partition_destroy(part);
+            part = nullptr;
+        }
+    }
+    if (!part) part = matxtract_preprocess(csrVal, csrRowPtr, csrColInd, rowA, colA, nnzA, colProp, rowProp);
     auto t1 = std::chrono::steady_clock::now();
     if (!part) return 1;
+    if (!cachePath.empty()) {
+        if (fromCache) printf("partition read from %s\n", cachePath.c_str());
+        else if (mx_partition_save(part, cachePath.c_str()) != MX_OK) printf("Warning: %s\n", mx_last_error());
+        else printf("partition written to %s\n", cachePath.c_str());
+    }
     const double preprocess_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
     mx_partition_view pv;
     mx_partition_get(part, &pv);

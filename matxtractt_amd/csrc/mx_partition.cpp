@@ -12,6 +12,7 @@
 //   * tiles are built per 8-row chunk from those sorted rows (:502-585, :718-978).
 // Rows are independent, so steps run under OpenMP.
 #include <algorithm>
+#include <cstdio>
 #include <cstring>
 #include <numeric>
 #include <utility>
@@ -418,6 +419,8 @@ extern "C" int mx_partition_get(const mx_partition *p, mx_partition_view *v)
     v->cdRowPtr = p->cdRowPtr.data();
     v->cdColInd = p->cdColInd.data();
     v->cdVal = p->cdVal.data();
+    v->tau_c = p->tau_c;
+    v->tau_r = p->tau_r;
     return MX_OK;
 }
 
@@ -444,6 +447,251 @@ extern "C" uint64_t mx_partition_hash(const mx_partition *p)
     h = fnv(p->cdColInd.data(), p->cdColInd.size() * 4, h);
     h = fnv(p->cdVal.data(), (size_t)p->nnzCD * es, h);
     return h;
+}
+
+// ---- partition file -------------------------------------------------------------------
+// The head of the file is the reference's "_preprocessed.dat" (written by
+// test/tcpreprocess.cpp:1208-1255, read back by test/tckernel.cpp:586-638), field for field:
+//   int chunkNum; int chunkPtr[chunkNum+1]; int totalTcFrags; int fragK;
+//   int sparse_AToX_index[totalTcFrags*fragK]; size_t n; int fragPtr[n];
+//   size_t n; bitmap fragBit[n]; size_t n; valT tcVal[n]
+// (bitmaps are uint32_t for binary64 as there, uint64_t for binary16), so that tool's reader
+// takes the tile part of a binary64 file as it is.  The reference stores nothing else; the
+// rest of the partition (sizes, thresholds, the four index maps, A_dd and the residual A_CD)
+// follows in an extension that starts with a magic word.
+namespace {
+
+const uint64_t kFileMagic = 0x3154524150584d00ull;  // "\0MXPART1", little-endian
+
+struct Writer {
+    FILE *f;
+    bool ok = true;
+    void raw(const void *p, size_t n)
+    {
+        if (n && fwrite(p, 1, n, f) != n) ok = false;
+    }
+    template <typename T>
+    void pod(const T &v) { raw(&v, sizeof(T)); }
+    template <typename T>
+    void vec(const std::vector<T> &v)
+    {
+        pod<uint64_t>((uint64_t)v.size());
+        raw(v.data(), v.size() * sizeof(T));
+    }
+};
+
+struct Reader {
+    FILE *f;
+    bool ok = true;
+    void raw(void *p, size_t n)
+    {
+        if (n && fread(p, 1, n, f) != n) ok = false;
+    }
+    template <typename T>
+    void pod(T &v) { raw(&v, sizeof(T)); }
+    template <typename T>
+    void vec(std::vector<T> &v, uint64_t limit)
+    {
+        uint64_t n = 0;
+        pod(n);
+        if (!ok || n > limit) {
+            ok = false;
+            return;
+        }
+        v.resize((size_t)n);
+        raw(v.data(), (size_t)n * sizeof(T));
+    }
+};
+
+}  // namespace
+
+extern "C" int mx_partition_save(const mx_partition *p, const char *path)
+{
+    if (!p || !path) {
+        set_error("mx_partition_save: null argument");
+        return MX_ERR_ARG;
+    }
+    FILE *f = fopen(path, "wb");
+    if (!f) {
+        set_error(std::string("mx_partition_save: cannot open ") + path);
+        return MX_ERR_IO;
+    }
+    Writer w{f};
+    const int es = mx::elem_size(p->dtype);
+    // the reference's fields
+    w.pod<int>(p->chunkNum);
+    std::vector<int> cp(p->chunkPtr);
+    cp.resize((size_t)p->chunkNum + 1, 0);
+    w.raw(cp.data(), cp.size() * sizeof(int));
+    w.pod<int>(p->totalTcFrags);
+    w.pod<int>(p->fragK);
+    w.raw(p->sparse_AToX_index.data(), (size_t)p->totalTcFrags * p->fragK * sizeof(int));
+    std::vector<int> fp(p->fragPtr);
+    fp.resize((size_t)p->totalTcFrags + 1, 0);
+    w.pod<size_t>(fp.size());
+    w.raw(fp.data(), fp.size() * sizeof(int));
+    w.pod<size_t>((size_t)p->totalTcFrags);
+    if (p->dtype == MX_F64) w.raw(p->fragBit32.data(), (size_t)p->totalTcFrags * 4);
+    else w.raw(p->fragBit64.data(), (size_t)p->totalTcFrags * 8);
+    w.pod<size_t>((size_t)p->tcValCount);
+    w.raw(p->tcVal.data(), (size_t)p->tcValCount * es);
+    // the extension
+    w.pod(kFileMagic);
+    const int head[8] = {(int)p->dtype, p->rows, p->cols, p->nnz, p->fragM, p->fragK, p->extracted ? 1 : 0, 0};
+    w.raw(head, sizeof(head));
+    w.pod(p->tau_c);
+    w.pod(p->tau_r);
+    const int counts[10] = {p->dCols, p->sCols, p->nnzColD, p->nnzColS, p->dRows, p->sRows, p->nnzRowD, p->nnzRowS,
+                            p->nnzCD, p->tcValCount};
+    w.raw(counts, sizeof(counts));
+    w.pod(p->cols_ratio);
+    w.pod(p->tc_nnz_ratio);
+    w.vec(p->descColId);
+    w.vec(p->newArray);
+    w.vec(p->rId);
+    w.vec(p->newArray_);
+    w.vec(p->ddRowPtr);
+    w.vec(p->ddColInd);
+    w.vec(p->ddVal.bytes);
+    w.vec(p->cdRowPtr);
+    w.vec(p->cdColInd);
+    w.vec(p->cdVal.bytes);
+    w.pod<uint64_t>(mx_partition_hash(p));
+    const bool ok = w.ok && fclose(f) == 0;
+    if (!ok) {
+        set_error(std::string("mx_partition_save: write failed: ") + path);
+        return MX_ERR_IO;
+    }
+    return MX_OK;
+}
+
+extern "C" int mx_partition_load(const char *path, mx_dtype dtype, mx_partition **out)
+{
+    if (!path || !out) {
+        set_error("mx_partition_load: null argument");
+        return MX_ERR_ARG;
+    }
+    *out = nullptr;
+    FILE *f = fopen(path, "rb");
+    if (!f) {
+        set_error(std::string("mx_partition_load: cannot open ") + path);
+        return MX_ERR_IO;
+    }
+    fseek(f, 0, SEEK_END);
+    const uint64_t fileSize = (uint64_t)ftell(f);  // no array can be longer than the file
+    fseek(f, 0, SEEK_SET);
+    mx_partition *p = new (std::nothrow) mx_partition();
+    if (!p) {
+        fclose(f);
+        set_error("mx_partition_load: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    auto fail = [&](const char *what) {
+        fclose(f);
+        delete p;
+        set_error(std::string("mx_partition_load: ") + what + ": " + path);
+        return MX_ERR_IO;
+    };
+    try {
+        Reader r{f};
+        const int es = mx::elem_size(dtype);
+        r.pod(p->chunkNum);
+        if (!r.ok || p->chunkNum < 0 || (uint64_t)p->chunkNum * 4 > fileSize) return fail("bad chunk count");
+        p->chunkPtr.resize((size_t)p->chunkNum + 1);
+        r.raw(p->chunkPtr.data(), p->chunkPtr.size() * sizeof(int));
+        r.pod(p->totalTcFrags);
+        r.pod(p->fragK);
+        if (!r.ok || p->totalTcFrags < 0 || p->fragK != mx::frag_k(dtype) ||
+            (uint64_t)p->totalTcFrags * p->fragK * 4 > fileSize)
+            return fail("tile header does not fit the requested precision");
+        p->sparse_AToX_index.resize((size_t)p->totalTcFrags * p->fragK);
+        r.raw(p->sparse_AToX_index.data(), p->sparse_AToX_index.size() * sizeof(int));
+        size_t n = 0;
+        r.pod(n);
+        if (!r.ok || n != (size_t)p->totalTcFrags + 1) return fail("bad fragPtr length");
+        p->fragPtr.resize(n);
+        r.raw(p->fragPtr.data(), n * sizeof(int));
+        r.pod(n);
+        if (!r.ok || n != (size_t)p->totalTcFrags) return fail("bad fragBit length");
+        if (dtype == MX_F64) {
+            p->fragBit32.resize(n);
+            r.raw(p->fragBit32.data(), n * 4);
+        } else {
+            p->fragBit64.resize(n);
+            r.raw(p->fragBit64.data(), n * 8);
+        }
+        r.pod(n);
+        if (!r.ok || (uint64_t)n * es > fileSize) return fail("bad tcVal length");
+        p->tcValCount = (int)n;
+        p->tcVal.resize(n, es);
+        r.raw(p->tcVal.data(), n * es);
+        uint64_t magic = 0;
+        r.pod(magic);
+        if (!r.ok || magic != kFileMagic)
+            return fail("the file holds the tile part only (written by the reference tool): the residual is missing");
+        int head[8], counts[10];
+        r.raw(head, sizeof(head));
+        r.pod(p->tau_c);
+        r.pod(p->tau_r);
+        r.raw(counts, sizeof(counts));
+        r.pod(p->cols_ratio);
+        r.pod(p->tc_nnz_ratio);
+        if (!r.ok || head[0] != (int)dtype || head[4] != mx::kFragM || head[5] != p->fragK)
+            return fail("written for the other precision");
+        p->dtype = dtype;
+        p->rows = head[1];
+        p->cols = head[2];
+        p->nnz = head[3];
+        p->fragM = head[4];
+        p->extracted = head[6] != 0;
+        p->dCols = counts[0];
+        p->sCols = counts[1];
+        p->nnzColD = counts[2];
+        p->nnzColS = counts[3];
+        p->dRows = counts[4];
+        p->sRows = counts[5];
+        p->nnzRowD = counts[6];
+        p->nnzRowS = counts[7];
+        p->nnzCD = counts[8];
+        if (counts[9] != p->tcValCount) return fail("inconsistent value count");
+        r.vec(p->descColId, fileSize);
+        r.vec(p->newArray, fileSize);
+        r.vec(p->rId, fileSize);
+        r.vec(p->newArray_, fileSize);
+        r.vec(p->ddRowPtr, fileSize);
+        r.vec(p->ddColInd, fileSize);
+        r.vec(p->ddVal.bytes, fileSize);
+        r.vec(p->cdRowPtr, fileSize);
+        r.vec(p->cdColInd, fileSize);
+        r.vec(p->cdVal.bytes, fileSize);
+        uint64_t hash = 0;
+        r.pod(hash);
+        if (!r.ok) return fail("truncated");
+        // sizes the rest of the library relies on
+        if (p->rows < 0 || p->cols < 0 || p->dRows < 0 || p->dCols < 0 || p->dCols > p->cols || p->dRows > p->rows ||
+            (int)p->cdRowPtr.size() != p->rows + 1 || (int)p->cdColInd.size() != p->nnzCD ||
+            p->cdVal.bytes.size() != (size_t)p->nnzCD * es || (int)p->rId.size() != p->dRows ||
+            (int)p->ddRowPtr.size() != (p->extracted ? p->dRows + 1 : (int)p->ddRowPtr.size()) ||
+            (p->extracted && (int)p->descColId.size() != p->cols) ||
+            p->chunkNum != (p->extracted ? (p->dRows + p->fragM - 1) / p->fragM : p->chunkNum) ||
+            p->chunkPtr.back() != p->totalTcFrags || p->fragPtr.back() != p->tcValCount)
+            return fail("inconsistent sizes");
+        for (int c : p->cdColInd)
+            if ((unsigned)c >= (unsigned)std::max(p->cols, 1)) return fail("column index out of range");
+        for (int c : p->sparse_AToX_index)
+            if ((unsigned)c >= (unsigned)std::max(p->dCols, 1)) return fail("tile column out of range");
+        for (int c : p->rId)
+            if ((unsigned)c >= (unsigned)std::max(p->rows, 1)) return fail("row index out of range");
+        if (hash != mx_partition_hash(p)) return fail("checksum mismatch");
+    } catch (const std::bad_alloc &) {
+        fclose(f);
+        delete p;
+        set_error("mx_partition_load: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    fclose(f);
+    *out = p;
+    return MX_OK;
 }
 
 // csr2csc / csc2csr (utilities/csr2csc.cpp:4-203) as a stable counting-sort transpose.

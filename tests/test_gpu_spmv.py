@@ -415,6 +415,28 @@ def test_tile_kernel_step_packing(mx, ora):
                 part.close()
 
 
+def test_plan_from_a_saved_partition(mx, ora, tmp_path):
+    """A partition that went through a file gives the same plan (and the same y, bit for bit)."""
+    import torch
+    for cfg, scale in ((2, 1 / 16), (5, 1 / 128)):
+        A, x = mx.gen_config(cfg, scale=scale)
+        P = mx.Partition(A, 0.75, 0.5)
+        path = str(tmp_path / ("w%d.dat" % cfg))
+        P.save(path)
+        Q = mx.Partition.load(path, A.dtype)
+        xd = torch.from_numpy(x).cuda()
+        ys = []
+        for part in (P, Q):
+            plan = mx.Plan(part, mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_ROWS)
+            ys.append(plan.spmv(xd).cpu().numpy())
+            plan.close()
+        assert np.array_equal(ys[0].view(np.uint8), ys[1].view(np.uint8))
+        tol = F64_TOL if A.dtype == mx.MX_F64 else F16_TOL
+        assert rel_l2(ys[1], oracle_y(ora, mx, A, x)) <= tol
+        P.close()
+        Q.close()
+
+
 def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
     """matxtract_perftest's stdout keeps the forms the reference's scripts grep for."""
     import re
@@ -438,3 +460,17 @@ def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
         assert re.search(r"MatXtract GFLOPS= \d+\.\d\d", out.stdout)
         if len(args) == 3:
             assert re.search(r"cols_ratio = \d\.\d+", out.stdout) and re.search(r"TC_nnz_ratio = \d\.\d+", out.stdout)
+    # --partition-cache: written by the first run, read by the second, recomputed when the fractions change
+    cache = str(tmp_path / "m_preprocessed.dat")
+    seen = []
+    for fr in (("0.5", "0.25"), ("0.5", "0.25"), ("0.75", "0.25")):
+        out = subprocess.run([exe, "--warm", "2", "--iters", "5", "--partition-cache", cache, *fr, str(p)],
+                             capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        assert "Success! All values match" in out.stdout
+        seen.append("read" if "partition read from" in out.stdout else
+                    "written" if "partition written to" in out.stdout else "neither")
+    assert seen == ["written", "read", "written"]
+    Q = mx.Partition.load(cache)
+    assert (Q.tau_c, Q.tau_r) == (0.75, 0.25) and (Q.rows, Q.cols, Q.nnz) == (A.rows, A.cols, A.nnz)
+    Q.close()

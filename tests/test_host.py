@@ -194,6 +194,89 @@ def test_mmio_symmetric_expansion_and_pattern(mx, tmp_path):
     assert e.value.code == 4
 
 
+def _read_reference_head(path, fragbit_dtype, val_dtype):
+    """The read sequence of the reference's tile-file reader (test/tckernel.cpp:586-638)."""
+    with open(path, "rb") as f:
+        def arr(dtype, n):
+            return np.frombuffer(f.read(np.dtype(dtype).itemsize * n), dtype=dtype)
+        chunkNum = int(arr(np.int32, 1)[0])
+        chunkPtr = arr(np.int32, chunkNum + 1)
+        totalTcFrags, fragK = (int(v) for v in arr(np.int32, 2))
+        atox = arr(np.int32, totalTcFrags * fragK)
+        fragPtr = arr(np.int32, int(arr(np.uint64, 1)[0]))
+        fragBit = arr(fragbit_dtype, int(arr(np.uint64, 1)[0]))
+        tcVal = arr(val_dtype, int(arr(np.uint64, 1)[0]))
+        return chunkPtr, fragK, atox, fragPtr, fragBit, tcVal, f.tell()
+
+
+@pytest.mark.parametrize("cfg,scale", [(1, 1.0), (2, 1 / 16), (5, 1 / 256)])
+def test_partition_file_round_trip(mx, cfg, scale, tmp_path):
+    """save -> load gives the same partition, array for array; the head of the file is laid out
+    as the reference's tile file, so a reader written after the reference's finds its arrays."""
+    A, _ = mx.gen_config(cfg, scale=scale)
+    f64 = A.dtype == mx.MX_F64
+    for tau in ((0.0, 0.0), (0.5, 0.25), (1.0, 1.0)):
+        P = mx.Partition(A, *tau)
+        path = str(tmp_path / ("p_%d_%g_%g.dat" % (cfg, tau[0], tau[1])))
+        P.save(path)
+        Q = mx.Partition.load(path, A.dtype)
+        assert Q.hash == P.hash
+        assert (Q.tau_c, Q.tau_r) == (P.tau_c, P.tau_r) == (np.float32(tau[0]), np.float32(tau[1]))
+        for name in mx.Partition.ARRAYS:
+            assert np.array_equal(getattr(P, name), getattr(Q, name)), name
+        for name in ("rows", "cols", "nnz", "dCols", "sCols", "dRows", "sRows", "nnzRowD", "nnzCD", "chunkNum",
+                     "totalTcFrags", "tcValCount", "cols_ratio", "tc_nnz_ratio"):
+            assert getattr(P, name) == getattr(Q, name), name
+        chunkPtr, fragK, atox, fragPtr, fragBit, tcVal, _ = _read_reference_head(
+            path, np.uint32 if f64 else np.uint64, np.float64 if f64 else np.float16)
+        assert fragK == P.fragK
+        assert np.array_equal(chunkPtr, P.chunkPtr) and np.array_equal(atox, P.sparse_AToX_index)
+        assert np.array_equal(fragPtr, P.fragPtr) and np.array_equal(fragBit, P.fragBit)
+        assert np.array_equal(tcVal.view(np.uint8), np.asarray(P.tcVal).view(np.uint8))
+        P.close()
+        Q.close()
+
+
+def test_partition_file_is_checked_on_load(mx, tmp_path):
+    A, _ = mx.gen_config(2, scale=1 / 32)
+    P = mx.Partition(A, 0.5, 0.25)
+    good = str(tmp_path / "good.dat")
+    P.save(good)
+    blob = open(good, "rb").read()
+    _, _, _, _, _, _, head_end = _read_reference_head(good, np.uint32, np.float64)
+
+    def load(data, dtype=mx.MX_F64):
+        path = str(tmp_path / "case.dat")
+        with open(path, "wb") as f:
+            f.write(data)
+        return mx.Partition.load(path, dtype)
+
+    # a value changed in the residual: the checksum catches it
+    bad = bytearray(blob)
+    bad[-64] ^= 0x40
+    with pytest.raises(mx.MxError, match="checksum|range|inconsistent"):
+        load(bytes(bad))
+    # cut short, in the head and in the extension
+    for n in (10, head_end - 3, head_end + 40, len(blob) - 1):
+        with pytest.raises(mx.MxError):
+            load(blob[:n])
+    # the tile part alone is what the reference's tool writes: refused, with a message that says why
+    with pytest.raises(mx.MxError, match="tile part only"):
+        load(blob[:head_end])
+    # read with the other precision
+    with pytest.raises(mx.MxError):
+        load(blob, mx.MX_F16)
+    # a column index pushed out of range (inside the reference's part of the file)
+    bad = bytearray(blob)
+    off = 4 + 4 * (P.chunkNum + 1) + 8  # first entry of sparse_AToX_index
+    bad[off:off + 4] = np.int32(P.dCols + 5).tobytes()
+    with pytest.raises(mx.MxError):
+        load(bytes(bad))
+    with pytest.raises(mx.MxError):
+        mx.Partition.load(str(tmp_path / "missing.dat"))
+    P.close()
+
+
 def test_init_vec(mx):
     v = mx.init_vec(40)
     assert np.array_equal(v, np.arange(40) % 15)
