@@ -198,11 +198,34 @@ typedef struct mx_plan_info {
     int tile_nnz;        /* matrix entries held in those fragments */
     int csr_nnz;         /* entries executed by the CSR kernel */
     int csr_blocks;      /* workgroups of the CSR kernel */
-    int csr_variant;     /* 0 = row tiles (csr_rows_kernel), 1 = column slices (csr_slice_kernel) */
+    int csr_variant;     /* 0 = row tiles (csr_rows_kernel), 1 = column slices (csr_slice_kernel),
+                            2 = row tiles for the short rows, then column slices for the long ones */
     double tile_bytes;   /* bytes the tile kernel must read+write per launch */
     double csr_bytes;    /* bytes the CSR kernel must read+write per launch */
 } mx_plan_info;
 int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
+
+/* The layout csr_slice_kernel runs on, built on the host for a machine with `nCU` compute units,
+ * for inspection (tests walk it the way the kernel does; nothing here touches a device).  `sel`
+ * marks the rows to include (NULL = all).  No counterpart in the reference, whose CSR kernel
+ * (src/spmv_kernel/cdSpMV.cu:29-393) gathers x from global memory.
+ *   wgDesc    [nWG][4]  {slice, first chunk, chunks, 0}
+ *   waveDesc  [nWG*waves][4] {first batch, batches, first chunk inside the workgroup, chunks}
+ *   chunkEnd  [chunks]  step, counted from the wave's first, at which the chunk ends
+ *   ecol      [batches][64][batchEntries] column - slice*sliceCols
+ *   eval      per batch: binary16 [64][batchEntries]; binary64 [batchEntries/stepEntries][64][stepEntries]
+ *   virtual row v = 64*chunk + lane; matrix row r owns segIdx[segPtr[r] .. segPtr[r+1])
+ *   heavy     rows with more than lightSegs virtual rows
+ * Release with mx_slice_layout_free. */
+typedef struct mx_slice_layout_view {
+    int nWG, S, sliceCols, waves, stepEntries, batchEntries, cap, chunks, batches, vrows, nHeavy, lightSegs;
+    long long nEcol;
+    int *wgDesc, *waveDesc, *chunkEnd, *segPtr, *segIdx, *heavy;
+    unsigned short *ecol;
+    unsigned char *eval;
+} mx_slice_layout_view;
+int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *sel, mx_slice_layout_view *out);
+void mx_slice_layout_free(mx_slice_layout_view *v);
 
 /* Reference surface, host pointers in / host pointers out, one-shot (allocate, upload,
  * `warm` + `iters` timed launches into a scratch y, one real launch, download, free).

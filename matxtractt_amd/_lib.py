@@ -53,6 +53,13 @@ class PlanInfo(C.Structure):
                 ("tile_bytes", C.c_double), ("csr_bytes", C.c_double)]
 
 
+class SliceLayoutView(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("nWG", "S", "sliceCols", "waves", "stepEntries", "batchEntries", "cap", "chunks",
+                                       "batches", "vrows", "nHeavy", "lightSegs")] + \
+               [("nEcol", C.c_longlong)] + \
+               [(n, C.c_void_p) for n in ("wgDesc", "waveDesc", "chunkEnd", "segPtr", "segIdx", "heavy", "ecol", "eval")]
+
+
 # Every symbol include/matxtract_hip.h declares: name -> (restype, argtypes)
 _vp, _i, _d = C.c_void_p, C.c_int, C.c_double
 _pp = C.POINTER(C.c_void_p)
@@ -82,6 +89,8 @@ SIGNATURES = {
     "mx_time": (_i, [_vp, _vp, _vp, _i, _i, _pd, _pd, _pd]),
     "mx_time_csr_main": (_i, [_vp, _vp, _vp, _i, _i, _pd]),
     "mx_plan_get_info": (_i, [_vp, C.POINTER(PlanInfo)]),
+    "mx_slice_layout": (_i, [C.POINTER(CsrStruct), _i, _vp, C.POINTER(SliceLayoutView)]),
+    "mx_slice_layout_free": (None, [C.POINTER(SliceLayoutView)]),
     "mx_cdspmv_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _pd, _pd]),
     "mx_cdspmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _pd, _pd]),
     "mx_du_tcspmv_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _pd]),

@@ -15,7 +15,7 @@ from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLA
                    MX_PLAN_NO_TILES, MxError, check)
 
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "cdspmv",
-           "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "MxError",
+           "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
            "MX_PLAN_CSR_SLICES"]
 
@@ -187,6 +187,35 @@ class Partition:
             self.close()
         except Exception:
             pass
+
+
+def slice_layout(A, nCU=256, sel=None):
+    """The host-side layout of the column-slice kernel for matrix A as a dict of numpy arrays
+    and sizes (see mx_slice_layout in include/matxtract_hip.h).  `sel`: optional mask of the rows
+    to include."""
+    v = _lib.SliceLayoutView()
+    st = A.struct()
+    selp = None
+    if sel is not None:
+        sel = np.ascontiguousarray(sel, dtype=np.uint8)
+        assert sel.shape == (A.rows,)
+        selp = sel.ctypes.data
+    check(_lib.load().mx_slice_layout(C.byref(st), int(nCU), selp, C.byref(v)))
+    try:
+        out = {n: int(getattr(v, n)) for n in ("nWG", "S", "sliceCols", "waves", "stepEntries", "batchEntries", "cap",
+                                               "chunks", "batches", "vrows", "nHeavy", "lightSegs")}
+        vt = _np_dtype(A.dtype)
+        out["wgDesc"] = _view(v.wgDesc, v.nWG * 4, np.int32).reshape(-1, 4).copy()
+        out["waveDesc"] = _view(v.waveDesc, v.nWG * v.waves * 4, np.int32).reshape(-1, 4).copy()
+        out["chunkEnd"] = _view(v.chunkEnd, v.chunks, np.int32).copy()
+        out["segPtr"] = _view(v.segPtr, A.rows + 1, np.int32).copy()
+        out["segIdx"] = _view(v.segIdx, v.vrows, np.int32).copy()
+        out["heavy"] = _view(v.heavy, v.nHeavy, np.int32).copy()
+        out["ecol"] = _view(v.ecol, v.nEcol, np.uint16).copy()
+        out["eval"] = _view(v.eval, v.nEcol, vt).copy()
+    finally:
+        _lib.load().mx_slice_layout_free(C.byref(v))
+    return out
 
 
 def _torch_dtype(dt):

@@ -57,40 +57,51 @@ inline int tile_slots(mx_dtype d) { return d == MX_F64 ? 16 : 8; }  // fragment 
 // slot of block i of half h: binary64 MFMA j takes slots 2j and 2j+1, binary16 slots 0..3 and 4..7
 inline int tile_slot(mx_dtype d, int half, int i) { return d == MX_F64 ? 2 * i + half : 4 * half + i; }
 
-// The CSR part re-laid for x resident in LDS.  The columns are cut into S slices of sliceCols
-// columns (a slice of x fits LDS); every slice cuts the rows into groups of about equal entries of
-// that slice, and a workgroup owns the entries of one group of one slice.  Inside a workgroup the group's rows are
-// sorted by their number of entries in the slice and cut into chunks of 64 rows, one row per
-// lane (a sliced-ELL layout: every row of a chunk is padded to the chunk's longest row, and the
-// sort keeps that padding small).  A lane walks its row E entries -- one "step" -- at a time
-// (E = 2 binary64, 4 binary16); chunks end on step boundaries.  The chunks of a workgroup are
-// dealt to its waves so that the waves' step counts are about equal, a wave's chunks follow
-// each other in the wave's stream, and the stream is stored in batches of kSliceBatchEntries
-// entries per lane (zero-padded to a whole batch at the end): per batch the lanes' column
-// offsets (lanes contiguous), then their values -- binary16: lanes contiguous; binary64: one
-// sub-block of 16 bytes per lane for every step -- so that every load of a wave is one
-// contiguous stretch.
+// The CSR part (or the rows of it that the plan selects) re-laid for x resident in LDS.  The
+// columns are cut into S slices of sliceCols columns (a slice of x fits LDS).  The entries of
+// a row that fall into one slice form a "virtual row"; one longer than the plan's cap is cut
+// into several, so a matrix row owns one or more virtual rows and its result is the sum of
+// theirs.  Per slice the virtual rows are sorted by length and cut into chunks of 64, one
+// virtual row per lane (a sliced-ELL layout: every row of a chunk is padded to the chunk's
+// longest, and the sort keeps that padding small).  A slice gets workgroups in proportion to
+// its entries, its chunks are dealt to them longest first, and inside a workgroup to its waves
+// the same way.  A lane walks its virtual row E entries -- one "step" -- at a time (E = 2
+// binary64, 4 binary16); chunks end on step boundaries; a wave's chunks follow each other in
+// the wave's stream, which is stored in batches of kSliceBatchEntries entries per lane
+// (zero-padded to a whole batch at the end): per batch the lanes' column offsets (lanes
+// contiguous), then their values -- binary16: lanes contiguous; binary64: one sub-block of 16
+// bytes per lane for every step -- so that every load of a wave is one contiguous stretch.
+// Chunks are numbered workgroup by workgroup, wave by wave; virtual row v = 64 * chunk + lane
+// puts its sum into partial[v], and a second kernel adds up the virtual rows of every matrix
+// row: those of row r are segIdx[segPtr[r] .. segPtr[r+1]).
 struct DeviceSlices {
     int nWG = 0, S = 0, rows = 0, cols = 0, sliceCols = 0;
-    int maxGroupRows = 0;             // rows of the largest group (their sums are parked in LDS)
+    int maxWgChunks = 0;              // chunks of the largest workgroup (their ends are kept in LDS)
     long long steps = 0;              // total steps stored (64 lanes * E entries each)
-    int *wgDesc = nullptr;            // [nWG][4] {first row, rows, slice, first chunk}
+    long long chunks = 0;             // total chunks
+    int nnz = 0;                      // entries held
+    int vrows = 0;                    // virtual rows
+    bool subset = false;              // only some rows are held: their sums are added to y, the others left alone
+    int *wgDesc = nullptr;            // [nWG][4] {slice, first chunk, chunks, 0}
     int *waveDesc = nullptr;          // [nWG*kSliceWaves][4] {first batch, batches, first chunk inside the workgroup, chunks}
     int *chunkEnd = nullptr;          // [chunks] step, counted from the wave's first, at which the chunk ends
-    unsigned short *chunkRows = nullptr;  // [chunks][64] row - first row of the group; 0xffff = no row.
-                                          // A group's chunks are padded to whole multiples of 64 rows.
     unsigned short *ecol = nullptr;   // [batches][64][kSliceBatchEntries] col - slice * sliceCols
     void *eval = nullptr;             // [batches] values, laid out as described above
-    void *partial = nullptr;          // [S][rows] accumulators (only when S > 1)
+    void *partial = nullptr;          // [chunks*64] accumulators
+    int *segPtr = nullptr;            // [rows+1]
+    int *segIdx = nullptr;            // [vrows]
+    int *heavy = nullptr;             // [nHeavy] rows with more than kSliceLightSegs virtual rows
+    int nHeavy = 0;
 };
 constexpr int kSliceBytes = 131072;   // the slice of x a workgroup keeps in LDS
 constexpr int kSliceLdsMax = 163840;  // LDS of a CU
-constexpr int kSliceGroupRows = 3072; // most rows a group may have: their sums and row ids share the rest of LDS
+constexpr int kSliceWgChunks = 4096;  // most chunks a workgroup may have
 constexpr int kSliceWaves = 8;        // waves per workgroup; one workgroup per CU
 constexpr int kSliceThreads = 64 * kSliceWaves;
 inline int slice_cols(mx_dtype d) { return kSliceBytes / (d == MX_F64 ? 8 : 2); }
 constexpr int kSliceBatchEntries = 8;  // entries a lane loads at a time
 inline int slice_step_entries(mx_dtype d) { return d == MX_F64 ? 2 : 4; }  // kSliceE
+constexpr int kSliceLightSegs = 8;     // rows with at most this many virtual rows are summed by one lane
 
 // `what`: 0 = slice kernel then combine kernel, 1 = slice kernel only, 2 = combine kernel only
 hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,

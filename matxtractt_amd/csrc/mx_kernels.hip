@@ -429,17 +429,16 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
 }
 
 // ---- CSR part, x resident in LDS ----------------------------------------------------------
-// For matrices whose x gathers are scattered, every gather from L2 moves a whole 128-byte line
-// for one value and a CU can keep only so many of those in flight: the kernel is bound by that
-// instead of HBM.  When x is small enough the gathers can be served from LDS instead.  The
-// columns are cut into S slices (a slice of x fits LDS), the rows into G groups, and workgroup
-// (g, s) -- one per CU -- copies slice s into LDS once and then streams the entries of its
-// rows that fall into the slice.  Those are laid out as sliced ELL (see DeviceSlices): one row
-// per lane, E entries per lane per step, steps contiguous across the wave, so a lane sums its
-// row in a register with no cross-lane traffic at all, and at the end of a chunk of 64 rows
-// every lane stores one sum.  With S > 1 the sums go to one column of a [S][rows] array of
-// partial sums and a second small kernel adds the S partials of each row; with S = 1 the
-// workgroup stores y itself.  No atomics in either case.
+// For matrices whose x gathers are scattered, every gather from L2 moves a whole cache line
+// for one value and a CU can take in only so many bytes per cycle: the kernel is bound by that
+// instead of HBM.  Gathers from LDS cost next to nothing.  The columns are cut into S slices
+// (a slice of x fits LDS); a workgroup -- one per CU -- copies one slice into LDS once and then
+// streams entries whose columns fall into it.  Those are laid out as sliced ELL over "virtual
+// rows" (see DeviceSlices): one virtual row per lane, E entries per lane per step, steps
+// contiguous across the wave, so a lane sums its virtual row in a register with no cross-lane
+// traffic at all, and at the end of a chunk of 64 virtual rows every lane stores one sum,
+// the wave 64 consecutive ones.  A second kernel adds up the virtual rows of every matrix row.
+// No atomics anywhere: every sum and every y has one owner.
 template <typename VT>
 struct SliceBatch;  // what one lane reads per batch: 8 column offsets, 8 values
 template <>
@@ -486,43 +485,34 @@ static_assert(mx::kSliceBatchEntries == 8, "SliceBatch holds 8 entries per lane"
 // happens; longer ones run a loop in which every consumed batch is reloaded with the batch one
 // ring length ahead (those reloads are unconditional inside the loop, so the number of loads
 // in flight is known at compile time and no wait is longer than it has to be), and a tail.
-// The sums of finished chunks are parked in LDS and leave the workgroup in one coalesced sweep.
 constexpr int kSliceRing = 6;
 
 template <typename VT>
 __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__restrict__ wgDesc,
                                                                   const int4 *__restrict__ waveDesc,
                                                                   const int *__restrict__ chunkEnd,
-                                                                  const unsigned short *__restrict__ chunkRows,
                                                                   const unsigned short *__restrict__ ecol,
                                                                   const VT *__restrict__ eval, const VT *__restrict__ x,
-                                                                  typename Acc<VT>::type *__restrict__ partial,
-                                                                  VT *__restrict__ y, int rows, int cols, int S,
-                                                                  int sliceCols, int maxGroupRows, int accumulate)
+                                                                  typename Acc<VT>::type *__restrict__ partial, int cols,
+                                                                  int sliceCols)
 {
     typedef typename Acc<VT>::type AT;
     typedef SliceBatch<VT> Batch;
     constexpr int SPB = Batch::SPB, NB = kSliceRing;
     constexpr int EPV = 16 / (int)sizeof(VT);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    VT *xs = (VT *)smem;                                                   // [sliceCols]
-    AT *ybuf = (AT *)(smem + (size_t)sliceCols * sizeof(VT));              // [maxGroupRows] sums by group row
-    unsigned short *rowsL = (unsigned short *)(ybuf + maxGroupRows);       // [chunks of the workgroup][64]
-    int *endsL = (int *)(rowsL + ((maxGroupRows + 63) / 64) * 64);         // [chunks of the workgroup]
+    VT *xs = (VT *)smem;                                           // [sliceCols]
+    int *endsL = (int *)(smem + (size_t)sliceCols * sizeof(VT));   // [chunks of the workgroup]
 
     const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int4 gd = wgDesc[b];
     const int4 d = waveDesc[b * kSliceWaves + wave];
-    const int row0 = gd.x, nr = gd.y, slice = gd.z, wgChunk0 = gd.w;
+    const int slice = gd.x, wgChunk0 = gd.y, wgChunks = gd.z;
     const int batch0 = __builtin_amdgcn_readfirstlane(d.x), nb = __builtin_amdgcn_readfirstlane(d.y);
     const int chunk0 = __builtin_amdgcn_readfirstlane(d.z), nChunks = __builtin_amdgcn_readfirstlane(d.w);
-    const int wgChunks = (nr + 63) / 64;
-    // row ids and chunk ends of the workgroup, and the slice (all of it at once, one 16-byte
-    // vector per lane and round)
-    unsigned short rl[2];
-    const int ridx = 2 * tid;  // 512 lanes * 2 = 1024 ... more rows go round again below
-    *(unsigned *)rl = ridx < wgChunks * 64 ? *(const unsigned *)(chunkRows + (size_t)wgChunk0 * 64 + ridx) : 0xffffffffu;
+    // chunk ends of the workgroup, and the slice (all of it at once, one 16-byte vector per
+    // lane and round)
     const int ce = tid < wgChunks ? chunkEnd[wgChunk0 + tid] : 0;
     constexpr int CB = kSliceBytes / 16 / kSliceThreads;  // rounds of a full slice
     const int nvec = sliceCols / EPV;
@@ -535,10 +525,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         if (i < nvec && c + EPV <= cols) xv[q] = *(const v4i32 *)(x + c);
     }
     {
-        if (ridx < wgChunks * 64) *(unsigned *)(rowsL + ridx) = *(unsigned *)rl;
         if (tid < wgChunks) endsL[tid] = ce;
-        for (int i = 2 * kSliceThreads + 2 * tid; i < wgChunks * 64; i += 2 * kSliceThreads)
-            *(unsigned *)(rowsL + i) = *(const unsigned *)(chunkRows + (size_t)wgChunk0 * 64 + i);
         for (int i = kSliceThreads + tid; i < wgChunks; i += kSliceThreads) endsL[i] = chunkEnd[wgChunk0 + i];
         // ragged end of x: the last, partial vector is filled element by element, and left out
         // of the sweep below (whose lane for it is in another wave and holds zeros)
@@ -566,9 +553,9 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     int ci = 0;
     int nextEnd = nChunks > 0 ? endsL[chunk0] : -1;
     AT acc = 0;
+    AT *out = partial + (size_t)(wgChunk0 + chunk0) * 64 + lane;
     auto flush = [&]() {
-        const int r = rowsL[(chunk0 + ci) * 64 + lane];
-        if (r != 0xffff) ybuf[r] = acc;
+        out[(size_t)ci * 64] = acc;
         acc = 0;
         ++ci;
         nextEnd = ci < nChunks ? endsL[chunk0 + ci] : -1;
@@ -598,29 +585,43 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 #pragma unroll
     for (int k = 0; k < NB; ++k)
         if (t + NB + k < nb) consume(buf[k], t + NB + k);
-    while (ci < nChunks) flush();  // chunks of empty rows
-    __syncthreads();
-    if (S <= 1) {
-        for (int i = tid; i < nr; i += kSliceThreads) {
-            AT sum = ybuf[i];
-            if (accumulate) sum += (AT)y[row0 + i];
-            y[row0 + i] = (VT)sum;
-        }
-    } else {
-        for (int i = tid; i < nr; i += kSliceThreads) partial[(size_t)slice * rows + row0 + i] = ybuf[i];
-    }
 }
 
-// y[r] = sum over the S slices of partial[s][r] (+ y[r])
+// y[r] = sum of the virtual rows of matrix row r (+ y[r]).  Rows with few virtual rows take one
+// lane each (the first `lightBlocks` workgroups walk all rows and skip the others); a row with
+// many takes a wave (the remaining workgroups walk the list `heavy`).  With `subset` the rows
+// that own no virtual row are left as they are.
 template <typename VT>
 __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Acc<VT>::type *__restrict__ partial,
-                                                              VT *__restrict__ y, int rows, int S, int accumulate)
+                                                              const int *__restrict__ segPtr,
+                                                              const int *__restrict__ segIdx,
+                                                              const int *__restrict__ heavy, int nHeavy, int lightBlocks,
+                                                              VT *__restrict__ y, int rows, int accumulate, int subset)
 {
     typedef typename Acc<VT>::type AT;
-    for (int r = blockIdx.x * kBlock + threadIdx.x; r < rows; r += gridDim.x * kBlock) {
+    const int tid = threadIdx.x;
+    if ((int)blockIdx.x < lightBlocks) {
+        const int r = blockIdx.x * kBlock + tid;
+        if (r >= rows) return;
+        const int a = segPtr[r], n = segPtr[r + 1] - a;
+        if (n > mx::kSliceLightSegs || (subset && n == 0)) return;
+        int id[mx::kSliceLightSegs];
+#pragma unroll
+        for (int k = 0; k < mx::kSliceLightSegs; ++k) id[k] = k < n ? segIdx[a + k] : -1;
         AT sum = accumulate ? (AT)y[r] : (AT)0;
-        for (int s = 0; s < S; ++s) sum += partial[(size_t)s * rows + r];
+#pragma unroll
+        for (int k = 0; k < mx::kSliceLightSegs; ++k)
+            if (id[k] >= 0) sum += partial[id[k]];
         y[r] = (VT)sum;
+    } else {
+        const int w = ((int)blockIdx.x - lightBlocks) * (kBlock / 64) + (tid >> 6), lane = tid & 63;
+        if (w >= nHeavy) return;
+        const int r = heavy[w];
+        const int a = segPtr[r], e = segPtr[r + 1];
+        AT sum = 0;
+        for (int k = a + lane; k < e; k += 64) sum += partial[segIdx[k]];
+        sum = group_sum<64>(sum);
+        if (lane == 0) y[r] = (VT)(sum + (accumulate ? (AT)y[r] : (AT)0));
     }
 }
 
@@ -855,9 +856,7 @@ template <typename VT>
 static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, int what)
 {
     typedef typename mxk::Acc<VT>::type AT;
-    const int chunkCap = (P.maxGroupRows + 63) / 64;
-    const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)P.maxGroupRows * sizeof(AT) +
-                       (size_t)chunkCap * 64 * 2 + (size_t)chunkCap * 4 + 64;  // + room for the combine flags
+    const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)P.maxWgChunks * 4 + 64;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT>,
@@ -865,24 +864,26 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    if (lds > (size_t)mx::kSliceLdsMax) return hipErrorInvalidValue;
-    if (what != 2)
+    if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16))
+        return hipErrorInvalidValue;
+    if (what != 2 && P.nWG > 0)
         hipLaunchKernelGGL((mxk::csr_slice_kernel<VT>), dim3(P.nWG), dim3(kSliceThreads), lds, s,
-                           (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.chunkRows, P.ecol,
-                           (const VT *)P.eval, (const VT *)x, (AT *)P.partial, (VT *)y, P.rows, P.cols, P.S, P.sliceCols,
-                           P.maxGroupRows, accumulate);
+                           (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.eval,
+                           (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || P.S <= 1 || what == 1) return e;
-    const int grid = std::min(2048, (P.rows + mxk::kBlock - 1) / mxk::kBlock);
-    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(grid), dim3(mxk::kBlock), 0, s, (const AT *)P.partial, (VT *)y,
-                       P.rows, P.S, accumulate);
+    if (e != hipSuccess || what == 1) return e;
+    const int light = (P.rows + mxk::kBlock - 1) / mxk::kBlock;
+    const int heavy = (P.nHeavy + mxk::kBlock / 64 - 1) / (mxk::kBlock / 64);
+    if (light + heavy == 0) return hipSuccess;
+    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(light + heavy), dim3(mxk::kBlock), 0, s, (const AT *)P.partial,
+                       P.segPtr, P.segIdx, P.heavy, P.nHeavy, light, (VT *)y, P.rows, (accumulate || P.subset) ? 1 : 0,
+                       P.subset ? 1 : 0);
     return hipGetLastError();
 }
-
 hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
                          int what)
 {
-    if (P.nWG <= 0) return hipSuccess;
+    if (P.rows <= 0) return hipSuccess;
     if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s, what);
     return launch_slices_t<_Float16>(P, x, y, accumulate, s, what);
 }

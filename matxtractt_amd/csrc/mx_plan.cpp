@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstring>
 #include <numeric>
+#include <queue>
 #include <vector>
 
 #include "mx_device.h"
@@ -97,189 +98,232 @@ void free_slices(mx::DeviceSlices &P)
 {
     (void)hipFree(P.waveDesc);
     (void)hipFree(P.chunkEnd);
-    (void)hipFree(P.chunkRows);
     (void)hipFree(P.wgDesc);
     (void)hipFree(P.ecol);
     (void)hipFree(P.eval);
     (void)hipFree(P.partial);
+    (void)hipFree(P.segPtr);
+    (void)hipFree(P.segIdx);
+    (void)hipFree(P.heavy);
     P = mx::DeviceSlices();
 }
 
-// Number of column slices csr_slice_kernel would need, or 0 when the matrix does not suit it.
-// With S slices the kernel writes and re-reads S partial sums per row, which must stay small
-// next to the matrix, and its one-row-per-lane layout wants rows that still have a few entries
-// each inside a slice.
+// Number of column slices csr_slice_kernel would cut x into, or 0 when the matrix does not suit
+// it: every slice costs at least one workgroup that copies 128 KB of x, which has to stay small
+// next to the matrix itself.
 int slice_count(mx_dtype dtype, int rows, int cols, int nnz, int nCU)
 {
-    const int es = mx::elem_size(dtype);
     if (cols < 1 || rows < 1 || nnz < 4096) return 0;
     const int S = (cols + mx::slice_cols(dtype) - 1) / mx::slice_cols(dtype);
-    if (S > nCU) return 0;
-    const double accBytes = dtype == MX_F64 ? 8 : 4;
-    const double extra = S > 1 ? 2.0 * S * (double)rows * accBytes : 0.0;
-    if (extra > 0.5 * (double)nnz * (es + 2)) return 0;
-    if ((double)nnz < 4.0 * (double)rows * S) return 0;
+    if (S > 2 * nCU) return 0;
+    if ((double)S * mx::kSliceBytes > 2.0 * (double)nnz * (mx::elem_size(dtype) + 2)) return 0;
     return S;
 }
 
-// Re-lays a CSR matrix for csr_slice_kernel (see DeviceSlices).
-int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
-                  mx::DeviceSlices &D)
+// Re-lays the rows `sel` marks (all rows when null) of a CSR matrix for csr_slice_kernel (see
+// DeviceSlices).
+struct HostSlices {
+    int nWG = 0, S = 0, rows = 0, cols = 0, sliceCols = 0, maxWgChunks = 0, nnz = 0, vrows = 0, cap = 0;
+    long long steps = 0, chunks = 0;
+    bool subset = false;
+    std::vector<int> wgDesc, waveDesc, chunkEnd, segPtr, segIdx, heavy;
+    std::vector<unsigned short> ecol;
+    std::vector<unsigned char> eval;
+};
+
+int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
+                 const char *sel, HostSlices &D)
 {
     const int es = mx::elem_size(dtype), E = mx::slice_step_entries(dtype);
     const int BE = mx::kSliceBatchEntries, SPB = BE / E;  // steps per batch
-    const int SW = mx::slice_cols(dtype), W = mx::kSliceWaves, GR = mx::kSliceGroupRows;
-    const int nnz = rowPtr[rows];
-    // entries sorted by (slice, row), order inside a row kept: seg[q*rows + r] = first entry of
-    // row r in slice q
-    std::vector<int> seg((size_t)S * rows + 1, 0), perm((size_t)nnz);
-    for (int r = 0; r < rows; ++r)
-        for (int p = rowPtr[r]; p < rowPtr[r + 1]; ++p) seg[(size_t)(col[p] / SW) * rows + r + 1]++;
-    for (size_t k = 0; k < (size_t)S * rows; ++k) seg[k + 1] += seg[k];
-    {
-        std::vector<int> cur(seg.begin(), seg.end() - 1);
-        for (int r = 0; r < rows; ++r)
-            for (int p = rowPtr[r]; p < rowPtr[r + 1]; ++p) perm[cur[(size_t)(col[p] / SW) * rows + r]++] = p;
+    const int SW = mx::slice_cols(dtype), W = mx::kSliceWaves;
+    // entries of the selected rows, row by row, ascending by column (stable)
+    std::vector<int> selPtr((size_t)rows + 1, 0);
+    for (int r = 0; r < rows; ++r) selPtr[r + 1] = selPtr[r] + ((!sel || sel[r]) ? rowPtr[r + 1] - rowPtr[r] : 0);
+    const int nnz = selPtr[rows];
+    std::vector<int> ord((size_t)nnz);
+    // a lane's fair share of the entries; virtual rows are cut to half of it so that the chunks
+    // can be dealt evenly
+    const int budget = std::max(nCU, 1);
+    const long long fair = (long long)nnz / ((long long)budget * W * 64);
+    const int cap = (int)std::min<long long>(512, std::max<long long>(16, (fair / 2 + BE - 1) / BE * BE));
+    std::vector<int> segPtr((size_t)rows + 1, 0);
+#pragma omp parallel for schedule(dynamic, 1024)
+    for (int r = 0; r < rows; ++r) {
+        const int n = selPtr[r + 1] - selPtr[r];
+        if (n == 0) continue;
+        int *o = &ord[selPtr[r]];
+        std::iota(o, o + n, rowPtr[r]);
+        bool sorted = true;
+        for (int k = 1; k < n && sorted; ++k) sorted = col[o[k - 1]] <= col[o[k]];
+        if (!sorted) std::stable_sort(o, o + n, [&](int a, int b) { return col[a] < col[b]; });
+        int nv = 0;
+        for (int k = 0; k < n;) {
+            const int q = col[o[k]] / SW;
+            int e = k;
+            while (e < n && e - k < cap && col[o[e]] / SW == q) ++e;
+            ++nv;
+            k = e;
+        }
+        segPtr[r + 1] = nv;
     }
-    // Workgroups: every slice gets a share of the CUs in proportion to its entries (largest
-    // remainders, at least one each), and cuts the rows into that many groups of about equal
-    // entries *of that slice* -- a slice that holds the diagonal band of some rows would
-    // otherwise give their workgroup several times the work of the others.  No group is longer
-    // than kSliceGroupRows rows.
-    const int minG = (rows + GR - 1) / GR;
-    std::vector<int> Gq(S, 1);
+    for (int r = 0; r < rows; ++r) segPtr[r + 1] += segPtr[r];
+    const int nV = segPtr[rows];
+    struct VRow {
+        int start, len, slice;  // start: into ord
+    };
+    std::vector<VRow> vr((size_t)nV);
+#pragma omp parallel for schedule(dynamic, 1024)
+    for (int r = 0; r < rows; ++r) {
+        const int n = selPtr[r + 1] - selPtr[r];
+        const int *o = n ? &ord[selPtr[r]] : nullptr;
+        int t = segPtr[r];
+        for (int k = 0; k < n;) {
+            const int q = col[o[k]] / SW;
+            int e = k;
+            while (e < n && e - k < cap && col[o[e]] / SW == q) ++e;
+            vr[t++] = {selPtr[r] + k, e - k, q};
+            k = e;
+        }
+    }
+    // virtual rows by (slice, length descending), row order kept among equals: a counting sort
+    const size_t nKeys = (size_t)S * (cap + 1);
+    std::vector<int> keyStart(nKeys + 1, 0), sorted((size_t)nV);
+    auto key_of = [&](const VRow &v) { return (size_t)v.slice * (cap + 1) + (size_t)(cap - v.len); };
+    for (int t = 0; t < nV; ++t) keyStart[key_of(vr[t]) + 1]++;
+    for (size_t k = 0; k < nKeys; ++k) keyStart[k + 1] += keyStart[k];
     {
-        const int budget = std::max(nCU, S);
-        std::vector<double> want(S);
+        std::vector<int> cur(keyStart.begin(), keyStart.end() - 1);
+        for (int t = 0; t < nV; ++t) sorted[cur[key_of(vr[t])]++] = t;
+    }
+    // chunks of every slice, and the slice's share of the workgroups (in proportion to its
+    // steps, largest remainders, at least one when it holds anything)
+    struct Chunk {
+        int first, n, steps;  // first: into sorted
+    };
+    std::vector<std::vector<Chunk>> sliceChunks(S);
+    std::vector<long long> sliceSteps(S, 0);
+    long long allSteps = 0;
+    int busy = 0;
+    for (int q = 0; q < S; ++q) {
+        const int a = keyStart[(size_t)q * (cap + 1)], b = keyStart[(size_t)(q + 1) * (cap + 1)];
+        for (int f = a; f < b; f += 64) {
+            const int n = std::min(64, b - f), steps = (vr[sorted[f]].len + E - 1) / E;
+            sliceChunks[q].push_back({f, n, steps});
+            sliceSteps[q] += steps;
+        }
+        allSteps += sliceSteps[q];
+        busy += b > a;
+    }
+    std::vector<int> Gq(S, 0);
+    {
+        const int total = std::max(budget, busy);
+        std::vector<double> want(S, 0.0);
         int used = 0;
         for (int q = 0; q < S; ++q) {
-            const double nq = (double)(seg[(size_t)(q + 1) * rows] - seg[(size_t)q * rows]);
-            want[q] = nnz > 0 ? nq * budget / nnz : 1.0;
+            if (sliceChunks[q].empty()) continue;
+            want[q] = allSteps > 0 ? (double)sliceSteps[q] * total / (double)allSteps : 1.0;
             Gq[q] = std::max(1, (int)want[q]);
             used += Gq[q];
         }
-        while (used < budget) {  // hand out what rounding down left over
-            int best = 0;
-            for (int q = 1; q < S; ++q)
-                if (want[q] - Gq[q] > want[best] - Gq[best]) best = q;
+        while (used < total && busy > 0) {  // hand out what rounding down left over
+            int best = -1;
+            for (int q = 0; q < S; ++q)
+                if (!sliceChunks[q].empty() && (best < 0 || want[q] - Gq[q] > want[best] - Gq[best])) best = q;
             ++Gq[best];
             ++used;
         }
-        for (int q = 0; q < S; ++q) Gq[q] = std::max(Gq[q], minG);
+        for (int q = 0; q < S; ++q) {
+            const int nc = (int)sliceChunks[q].size();
+            Gq[q] = std::min(std::max(Gq[q], (nc + mx::kSliceWgChunks - 1) / mx::kSliceWgChunks), std::max(nc, 1));
+            if (nc == 0) Gq[q] = 0;
+        }
     }
+    // workgroups: a slice's chunks, longest first, each to the workgroup of the slice with the
+    // fewest steps so far; then the same inside the workgroup for its waves
     struct Wg {
-        int slice, row0, nr;
+        int slice;
+        std::vector<int> chunk[mx::kSliceWaves];  // per wave: indices into sliceChunks[slice]
+        int waveSteps[mx::kSliceWaves];
+        long long steps = 0;   // stored steps (every wave's stream rounded up to whole batches)
+        int chunks = 0;
     };
     std::vector<Wg> wgs;
     for (int q = 0; q < S; ++q) {
-        const int *sp = &seg[(size_t)q * rows];
-        const long long nq = sp[rows] - sp[0];
-        int r0 = 0;
-        for (int g = 1; g <= Gq[q] && r0 < rows; ++g) {
-            int r1 = rows;
-            if (g < Gq[q]) {
-                const long long target = sp[0] + nq * g / Gq[q];
-                r1 = (int)(std::lower_bound(sp, sp + rows + 1, (int)target) - sp);
-                r1 = std::min(std::max(r1, r0 + 1), rows);
-            }
-            r1 = std::min(r1, r0 + GR);
-            r1 = std::max(r1, rows - (Gq[q] - g) * GR);  // leave no more than GR rows to each later group
-            wgs.push_back({q, r0, r1 - r0});
-            r0 = r1;
+        const int g0 = (int)wgs.size(), G = Gq[q];
+        if (G == 0) continue;
+        wgs.resize(wgs.size() + G);
+        std::vector<std::vector<int>> mine(G);
+        typedef std::pair<long long, int> Load;
+        std::priority_queue<Load, std::vector<Load>, std::greater<Load>> heap;
+        for (int g = 0; g < G; ++g) heap.push({0, g});
+        const auto &ch = sliceChunks[q];
+        for (int c = 0; c < (int)ch.size(); ++c) {
+            Load top = heap.top();
+            heap.pop();
+            mine[top.second].push_back(c);
+            top.first += ch[c].steps;
+            if ((int)mine[top.second].size() < mx::kSliceWgChunks) heap.push(top);
         }
-        while (r0 < rows) {  // rows the limits above left over
-            const int r1 = std::min(rows, r0 + GR);
-            wgs.push_back({q, r0, r1 - r0});
-            r0 = r1;
+        for (int g = 0; g < G; ++g) {
+            Wg &w = wgs[g0 + g];
+            w.slice = q;
+            for (int k = 0; k < W; ++k) w.waveSteps[k] = 0;
+            for (int c : mine[g]) {
+                int best = 0;
+                for (int k = 1; k < W; ++k)
+                    if (w.waveSteps[k] < w.waveSteps[best]) best = k;
+                w.chunk[best].push_back(c);
+                w.waveSteps[best] += ch[c].steps;
+            }
+            w.chunks = (int)mine[g].size();
+            for (int k = 0; k < W; ++k) w.steps += (w.waveSteps[k] + SPB - 1) / SPB * SPB;
         }
     }
     const int nWG = (int)wgs.size();
-    // per workgroup: the sorted rows, their chunks and the chunks' places in the waves' streams
-    struct WgLayout {
-        std::vector<int> sortedRow;   // group-local rows, by entries in the slice, descending
-        std::vector<int> chunkOrder;  // chunks in stream order (wave by wave)
-        std::vector<int> chunkSteps;  // steps of each chunk (indexed by chunk)
-        int waveSteps[mx::kSliceWaves], waveChunks[mx::kSliceWaves];
-        long long steps = 0;
-    };
-    std::vector<WgLayout> lay((size_t)nWG);
-#pragma omp parallel for schedule(dynamic, 1)
-    for (int b = 0; b < nWG; ++b) {
-        const int nr = wgs[b].nr;
-        const int *cnt0 = &seg[(size_t)wgs[b].slice * rows + wgs[b].row0];
-        WgLayout &L = lay[b];
-        L.sortedRow.resize(nr);
-        std::iota(L.sortedRow.begin(), L.sortedRow.end(), 0);
-        std::stable_sort(L.sortedRow.begin(), L.sortedRow.end(),
-                         [&](int a, int c) { return cnt0[a + 1] - cnt0[a] > cnt0[c + 1] - cnt0[c]; });
-        const int nc = (nr + 63) / 64;
-        L.chunkSteps.resize(nc);
-        for (int c = 0; c < nc; ++c) {
-            const int lead = L.sortedRow[(size_t)c * 64];
-            L.chunkSteps[c] = (cnt0[lead + 1] - cnt0[lead] + E - 1) / E;
-        }
-        // longest chunk first, each to the wave with the fewest steps so far
-        std::vector<std::vector<int>> mine(W);
-        for (int w = 0; w < W; ++w) L.waveSteps[w] = 0;
-        for (int c = 0; c < nc; ++c) {
-            int best = 0;
-            for (int w = 1; w < W; ++w)
-                if (L.waveSteps[w] < L.waveSteps[best]) best = w;
-            mine[best].push_back(c);
-            L.waveSteps[best] += L.chunkSteps[c];
-        }
-        L.steps = 0;
-        for (int w = 0; w < W; ++w) {
-            L.waveChunks[w] = (int)mine[w].size();
-            L.chunkOrder.insert(L.chunkOrder.end(), mine[w].begin(), mine[w].end());
-            L.steps += (L.waveSteps[w] + SPB - 1) / SPB * SPB;  // a wave's stream is whole batches
-        }
-    }
     long long totalSteps = 0, totalChunks = 0;
     std::vector<long long> wgStep((size_t)nWG + 1, 0), wgChunk((size_t)nWG + 1, 0);
-    int maxGroupRows = 0;
+    int maxWgChunks = 0;
     for (int b = 0; b < nWG; ++b) {
         wgStep[b] = totalSteps;
         wgChunk[b] = totalChunks;
-        totalSteps += lay[b].steps;
-        totalChunks += (long long)lay[b].chunkOrder.size();
-        maxGroupRows = std::max(maxGroupRows, wgs[b].nr);
+        totalSteps += wgs[b].steps;
+        totalChunks += wgs[b].chunks;
+        maxWgChunks = std::max(maxWgChunks, wgs[b].chunks);
     }
-    if (totalSteps * 64 * E > 2000000000LL) {
+    if (totalSteps * 64 * E > 2000000000LL || totalChunks * 64 > 2000000000LL) {
         set_error("slice layout: too many entries for 32-bit offsets");
         return MX_ERR_ARG;
     }
     const size_t padSteps = 16;  // spare zero steps after the last
     std::vector<unsigned short> ecol(((size_t)totalSteps + padSteps) * 64 * E, 0);
     std::vector<unsigned char> ev(((size_t)totalSteps + padSteps) * 64 * E * es, 0);
-    std::vector<int> wgDesc((size_t)nWG * 4, 0), waveDesc((size_t)nWG * W * 4, 0), chunkEnd((size_t)totalChunks + 64, 0);
-    std::vector<unsigned short> chunkRows(((size_t)totalChunks + 1) * 64, 0xffff);
+    std::vector<int> wgDesc((size_t)nWG * 4 + 4, 0), waveDesc((size_t)nWG * W * 4 + 4, 0), chunkEnd((size_t)totalChunks + 64, 0);
+    std::vector<int> segIdx((size_t)nV + 1, 0);
     const unsigned char *sv = (const unsigned char *)val;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int b = 0; b < nWG; ++b) {
-        const int q = wgs[b].slice, nr = wgs[b].nr;
-        const WgLayout &L = lay[b];
-        const int *sp = &seg[(size_t)q * rows + wgs[b].row0];
+        const Wg &G = wgs[b];
+        const int q = G.slice;
+        const auto &ch = sliceChunks[q];
         long long step = wgStep[b], chunk = wgChunk[b];
-        wgDesc[(size_t)b * 4 + 0] = wgs[b].row0;
-        wgDesc[(size_t)b * 4 + 1] = nr;
-        wgDesc[(size_t)b * 4 + 2] = q;
-        wgDesc[(size_t)b * 4 + 3] = (int)chunk;
-        size_t k = 0;
+        wgDesc[(size_t)b * 4 + 0] = q;
+        wgDesc[(size_t)b * 4 + 1] = (int)chunk;
+        wgDesc[(size_t)b * 4 + 2] = G.chunks;
         for (int w = 0; w < W; ++w) {
             int *d = &waveDesc[((size_t)b * W + w) * 4];
-            d[0] = (int)(step / SPB);                        // first batch
-            d[1] = (L.waveSteps[w] + SPB - 1) / SPB;         // batches
-            d[2] = (int)(chunk - wgChunk[b]);                // first chunk, counted inside the workgroup
-            d[3] = L.waveChunks[w];
+            d[0] = (int)(step / SPB);                   // first batch
+            d[1] = (G.waveSteps[w] + SPB - 1) / SPB;    // batches
+            d[2] = (int)(chunk - wgChunk[b]);           // first chunk, counted inside the workgroup
+            d[3] = (int)G.chunk[w].size();
             int rel = 0;
-            for (int j = 0; j < L.waveChunks[w]; ++j, ++k, ++chunk) {
-                const int c = L.chunkOrder[k], cs = L.chunkSteps[c];
-                for (int l = 0; l < 64 && c * 64 + l < nr; ++l) {
-                    const int i = L.sortedRow[(size_t)c * 64 + l];
-                    chunkRows[(size_t)chunk * 64 + l] = (unsigned short)i;
-                    for (int e = sp[i]; e < sp[i + 1]; ++e) {
-                        const int n = e - sp[i], p = perm[e];
+            for (int c : G.chunk[w]) {
+                for (int l = 0; l < ch[c].n; ++l) {
+                    const int t = sorted[ch[c].first + l];
+                    const VRow &v = vr[t];
+                    segIdx[t] = (int)(chunk * 64 + l);
+                    for (int n = 0; n < v.len; ++n) {
+                        const int p = ord[v.start + n];
                         const size_t st = (size_t)step + n / E, batch = st / SPB, sub = st % SPB;
                         // a lane's column offsets of a batch are contiguous; so are its binary16
                         // values; binary64 values go step by step, two per lane
@@ -289,28 +333,66 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
                         std::memcpy(&ev[atv * es], sv + (size_t)p * es, es);
                     }
                 }
-                step += cs;
-                rel += cs;
-                chunkEnd[chunk] = rel;
+                step += ch[c].steps;
+                rel += ch[c].steps;
+                chunkEnd[chunk++] = rel;
             }
             step = (step + SPB - 1) / SPB * SPB;
         }
     }
+    std::vector<int> heavy;
+    for (int r = 0; r < rows; ++r)
+        if (segPtr[r + 1] - segPtr[r] > mx::kSliceLightSegs) heavy.push_back(r);
     D.nWG = nWG;
     D.S = S;
     D.rows = rows;
     D.cols = cols;
     D.sliceCols = SW;
-    D.maxGroupRows = maxGroupRows;
+    D.maxWgChunks = maxWgChunks;
     D.steps = totalSteps;
-    int rc;
-    if ((rc = upload(&D.wgDesc, wgDesc.data(), wgDesc.size()))) return rc;
-    if ((rc = upload(&D.waveDesc, waveDesc.data(), waveDesc.size()))) return rc;
-    if ((rc = upload(&D.chunkEnd, chunkEnd.data(), chunkEnd.size()))) return rc;
-    if ((rc = upload(&D.chunkRows, chunkRows.data(), chunkRows.size()))) return rc;
-    if ((rc = upload(&D.ecol, ecol.data(), ecol.size()))) return rc;
-    if ((rc = upload_bytes(&D.eval, ev.data(), ev.size()))) return rc;
-    if (S > 1 && (rc = upload_bytes(&D.partial, nullptr, 0, (size_t)S * rows * (dtype == MX_F64 ? 8 : 4)))) return rc;
+    D.chunks = totalChunks;
+    D.nnz = nnz;
+    D.vrows = nV;
+    D.cap = cap;
+    D.subset = sel != nullptr;
+    D.wgDesc.swap(wgDesc);
+    D.waveDesc.swap(waveDesc);
+    D.chunkEnd.swap(chunkEnd);
+    D.segPtr.swap(segPtr);
+    D.segIdx.swap(segIdx);
+    D.heavy.swap(heavy);
+    D.ecol.swap(ecol);
+    D.eval.swap(ev);
+    return MX_OK;
+}
+
+int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
+                  const char *sel, mx::DeviceSlices &D)
+{
+    HostSlices H;
+    int rc = build_slices(dtype, rows, cols, rowPtr, col, val, nCU, S, sel, H);
+    if (rc) return rc;
+    D.nWG = H.nWG;
+    D.S = H.S;
+    D.rows = H.rows;
+    D.cols = H.cols;
+    D.sliceCols = H.sliceCols;
+    D.maxWgChunks = H.maxWgChunks;
+    D.steps = H.steps;
+    D.chunks = H.chunks;
+    D.nnz = H.nnz;
+    D.vrows = H.vrows;
+    D.subset = H.subset;
+    D.nHeavy = (int)H.heavy.size();
+    if ((rc = upload(&D.wgDesc, H.wgDesc.data(), H.wgDesc.size()))) return rc;
+    if ((rc = upload(&D.waveDesc, H.waveDesc.data(), H.waveDesc.size()))) return rc;
+    if ((rc = upload(&D.chunkEnd, H.chunkEnd.data(), H.chunkEnd.size()))) return rc;
+    if ((rc = upload(&D.ecol, H.ecol.data(), H.ecol.size()))) return rc;
+    if ((rc = upload_bytes(&D.eval, H.eval.data(), H.eval.size()))) return rc;
+    if ((rc = upload_bytes(&D.partial, nullptr, 0, ((size_t)H.chunks * 64 + 64) * (dtype == MX_F64 ? 8 : 4)))) return rc;
+    if ((rc = upload(&D.segPtr, H.segPtr.data(), H.segPtr.size()))) return rc;
+    if ((rc = upload(&D.segIdx, H.segIdx.data(), H.segIdx.size()))) return rc;
+    if ((rc = upload(&D.heavy, H.heavy.data(), H.heavy.size(), 1))) return rc;
     return MX_OK;
 }
 
@@ -519,6 +601,72 @@ int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, c
 
 }  // namespace
 
+extern "C" int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *sel, mx_slice_layout_view *out)
+{
+    if (!A || !out || nCU < 1 || A->rows < 0 || A->cols < 1 || !A->rowPtr || (A->nnz > 0 && (!A->colInd || !A->val))) {
+        set_error("mx_slice_layout: bad argument");
+        return MX_ERR_ARG;
+    }
+    std::memset(out, 0, sizeof(*out));
+    const int S = (A->cols + mx::slice_cols(A->dtype) - 1) / mx::slice_cols(A->dtype);
+    HostSlices H;
+    try {
+        int rc = build_slices(A->dtype, A->rows, A->cols, A->rowPtr, A->colInd, A->val, nCU, S, (const char *)sel, H);
+        if (rc) return rc;
+    } catch (const std::bad_alloc &) {
+        set_error("mx_slice_layout: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    auto give = [](const auto &v) {
+        typedef typename std::decay<decltype(v)>::type::value_type T;
+        T *p = (T *)malloc(std::max<size_t>(v.size(), 1) * sizeof(T));
+        if (p && !v.empty()) std::memcpy(p, v.data(), v.size() * sizeof(T));
+        return p;
+    };
+    out->nWG = H.nWG;
+    out->S = H.S;
+    out->sliceCols = H.sliceCols;
+    out->waves = mx::kSliceWaves;
+    out->stepEntries = mx::slice_step_entries(A->dtype);
+    out->batchEntries = mx::kSliceBatchEntries;
+    out->cap = H.cap;
+    out->chunks = (int)H.chunks;
+    out->batches = (int)(H.steps / (mx::kSliceBatchEntries / mx::slice_step_entries(A->dtype)));
+    out->vrows = H.vrows;
+    out->nHeavy = (int)H.heavy.size();
+    out->lightSegs = mx::kSliceLightSegs;
+    out->nEcol = (long long)H.ecol.size();
+    out->wgDesc = give(H.wgDesc);
+    out->waveDesc = give(H.waveDesc);
+    out->chunkEnd = give(H.chunkEnd);
+    out->segPtr = give(H.segPtr);
+    out->segIdx = give(H.segIdx);
+    out->heavy = give(H.heavy);
+    out->ecol = give(H.ecol);
+    out->eval = give(H.eval);
+    if (!out->wgDesc || !out->waveDesc || !out->chunkEnd || !out->segPtr || !out->segIdx || !out->heavy || !out->ecol ||
+        !out->eval) {
+        mx_slice_layout_free(out);
+        set_error("mx_slice_layout: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    return MX_OK;
+}
+
+extern "C" void mx_slice_layout_free(mx_slice_layout_view *v)
+{
+    if (!v) return;
+    free(v->wgDesc);
+    free(v->waveDesc);
+    free(v->chunkEnd);
+    free(v->segPtr);
+    free(v->segIdx);
+    free(v->heavy);
+    free(v->ecol);
+    free(v->eval);
+    std::memset(v, 0, sizeof(*v));
+}
+
 // MX_CSR_NPT overrides the default (for tuning runs); only values with a compiled kernel count.
 int mx::csr_entries_per_lane(mx_dtype dtype)
 {
@@ -531,9 +679,9 @@ int mx::csr_entries_per_lane(mx_dtype dtype)
 struct mx_plan {
     mx_dtype dtype = MX_F64;
     int rows = 0, cols = 0, nnz = 0;
-    mx::DeviceCsr csr;        // CSR part, row-tile form (csr_rows_kernel)
-    mx::DeviceSlices slices;  // CSR part, x-resident-in-LDS form (csr_slice_kernel)
-    bool use_slices = false;  // which of the two runs
+    mx::DeviceCsr csr;        // CSR part (or its short rows), row-tile form (csr_rows_kernel)
+    mx::DeviceSlices slices;  // CSR part (or its long rows), x-resident-in-LDS form (csr_slice_kernel)
+    int csr_variant = 0;      // 0 = row tiles, 1 = slices, 2 = row tiles for the short rows, then slices for the long ones
     int csr_nnz = 0;
     mx::DeviceTiles tiles;
     int tile_nnz = 0;
@@ -588,67 +736,126 @@ static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
 
 static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate, hipStream_t s)
 {
-    if (plan->use_slices && ((uintptr_t)x & 15)) {
+    if (plan->csr_variant != 0 && ((uintptr_t)x & 15)) {
         set_error("mx_spmv: x must be 16-byte aligned for this plan");
         return MX_ERR_ARG;
     }
-    if (plan->use_slices)
-        MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s));
-    else
-        MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s));
+    if (plan->csr_variant != 1) MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s));
+    if (plan->csr_variant != 0) MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s));
     return MX_OK;
 }
 
-// Puts the CSR part on the device.  Two executable forms exist (row tiles with direct x
-// gathers; column slices with x resident in LDS); unless a flag forces one, both are built
-// when the matrix suits the second, timed on the spot with a few launches each, and the
-// slower one is released.
+// Row length from which a row of a split plan goes to the slice kernel (MX_SPLIT_LEN overrides).
+static int split_length()
+{
+    const char *e = std::getenv("MX_SPLIT_LEN");
+    const int v = e ? std::atoi(e) : 0;
+    return v > 0 ? v : 32;
+}
+
+// Puts the CSR part on the device.  Three executable forms exist: row tiles with direct x
+// gathers; column slices with x resident in LDS; and a split in which the long rows (most of
+// the entries of a matrix with a heavy tail of row lengths) take the slices and the many short
+// ones the row tiles.  Unless a flag or MX_CSR_KERNEL=rows|slices|split forces one, every form
+// the matrix suits is built in turn and timed on the spot with a few launches, and the fastest
+// is kept.
 static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags)
 {
     const int rows = plan->rows, cols = plan->cols;
     const int nnz = rowPtr[rows];
+    const size_t es = (size_t)mx::elem_size(plan->dtype);
     plan->csr_nnz = nnz;
     const char *env = std::getenv("MX_CSR_KERNEL");
-    bool want_rows = true, want_slices = true;
-    if (flags & MX_PLAN_CSR_ROWS) want_slices = false;
-    if (flags & MX_PLAN_CSR_SLICES) want_rows = false;
-    if (env && !std::strcmp(env, "rows")) want_rows = true, want_slices = false;
-    if (env && !std::strcmp(env, "slices")) want_rows = false, want_slices = true;
+    bool want[3] = {true, true, true};
+    if (flags & MX_PLAN_CSR_ROWS) want[1] = want[2] = false;
+    if (flags & MX_PLAN_CSR_SLICES) want[0] = want[2] = false;
+    if (env && !std::strcmp(env, "rows")) want[0] = true, want[1] = want[2] = false;
+    if (env && !std::strcmp(env, "slices")) want[1] = true, want[0] = want[2] = false;
+    if (env && !std::strcmp(env, "split")) want[2] = true, want[0] = want[1] = false;
     hipDeviceProp_t prop;
     int dev = 0;
     MX_HIP(hipGetDevice(&dev));
     MX_HIP(hipGetDeviceProperties(&prop, dev));
     const int nCU = std::max(1, prop.multiProcessorCount);
     const int S = slice_count(plan->dtype, rows, cols, nnz, nCU);
-    if (S == 0) {  // a matrix the slice kernel cannot take runs on row tiles whatever was asked
-        want_slices = false;
-        want_rows = true;
+    // the split: rows of at least split_length() entries, when they hold a good part of the matrix
+    std::vector<char> longRow;
+    int longNnz = 0, longRows = 0;
+    if (S > 0 && want[2]) {
+        const int T = split_length();
+        longRow.assign((size_t)rows, 0);
+        for (int r = 0; r < rows; ++r)
+            if (rowPtr[r + 1] - rowPtr[r] >= T) {
+                longRow[r] = 1;
+                longNnz += rowPtr[r + 1] - rowPtr[r];
+                ++longRows;
+            }
+        if (longNnz < 4096 || longRows == rows || (double)longNnz < 0.1 * (double)nnz) want[2] = false;
     }
+    if (S == 0) want[1] = want[2] = false;
+    if (!want[0] && !want[1] && !want[2]) want[0] = true;  // a matrix the slice kernel cannot take runs on row tiles whatever was asked
+    const int nWant = (int)want[0] + (int)want[1] + (int)want[2];
     int rc;
-    if (want_rows && (rc = upload_csr(plan->dtype, rows, plan->cols, nnz, rowPtr, col, val, plan->csr, nullptr))) return rc;
-    if (want_slices && (rc = upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, plan->slices))) return rc;
-    plan->use_slices = want_slices && !want_rows;
-    if (want_rows && want_slices) {
-        const size_t es = (size_t)mx::elem_size(plan->dtype);
-        void *tx = nullptr, *ty = nullptr;
+    void *tx = nullptr, *ty = nullptr;
+    if (nWant > 1) {
         if ((rc = upload_bytes(&tx, nullptr, 0, std::max<size_t>(cols * es, 16)))) return rc;
         if ((rc = upload_bytes(&ty, nullptr, 0, std::max<size_t>(rows * es, 16)))) {
             (void)hipFree(tx);
             return rc;
         }
-        double ms[2] = {0.0, 0.0};
-        for (int v = 0; v < 2 && !rc; ++v) {
-            plan->use_slices = v == 1;
-            rc = time_loop(plan, 3, 10, [&]() { return launch_csr_part(plan, tx, ty, 0, plan->stream); }, &ms[v]);
-        }
-        (void)hipFree(tx);
-        (void)hipFree(ty);
-        if (rc) return rc;
-        plan->use_slices = ms[1] < ms[0];
-        if (plan->use_slices) free_csr(plan->csr);
-        else free_slices(plan->slices);
     }
-    return MX_OK;
+    auto build = [&](int v, mx::DeviceCsr &C, mx::DeviceSlices &L) -> int {
+        if (v == 0) return upload_csr(plan->dtype, rows, cols, nnz, rowPtr, col, val, C, nullptr);
+        if (v == 1) return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, nullptr, L);
+        // the short rows as a CSR matrix of their own (the long rows empty), the long ones as slices
+        std::vector<int> rp((size_t)rows + 1, 0);
+        for (int r = 0; r < rows; ++r) rp[r + 1] = rp[r] + (longRow[r] ? 0 : rowPtr[r + 1] - rowPtr[r]);
+        std::vector<int> c2((size_t)rp[rows]);
+        std::vector<unsigned char> v2((size_t)rp[rows] * es);
+#pragma omp parallel for schedule(static)
+        for (int r = 0; r < rows; ++r) {
+            if (longRow[r]) continue;
+            const int n = rowPtr[r + 1] - rowPtr[r];
+            if (n == 0) continue;
+            std::memcpy(&c2[rp[r]], col + rowPtr[r], (size_t)n * sizeof(int));
+            std::memcpy(&v2[(size_t)rp[r] * es], (const unsigned char *)val + (size_t)rowPtr[r] * es, (size_t)n * es);
+        }
+        int r1 = upload_csr(plan->dtype, rows, cols, rp[rows], rp.data(), c2.data(), v2.data(), C, nullptr);
+        if (r1) return r1;
+        return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, longRow.data(), L);
+    };
+    double best = 0.0;
+    bool have = false;
+    rc = MX_OK;
+    for (int v = 0; v < 3 && !rc; ++v) {
+        if (!want[v]) continue;
+        mx::DeviceCsr C;
+        mx::DeviceSlices L;
+        rc = build(v, C, L);
+        double ms = 0.0;
+        if (!rc && nWant > 1) {
+            std::swap(plan->csr, C);
+            std::swap(plan->slices, L);
+            const int keepVariant = plan->csr_variant;
+            plan->csr_variant = v;
+            rc = time_loop(plan, 3, 10, [&]() { return launch_csr_part(plan, tx, ty, 0, plan->stream); }, &ms);
+            plan->csr_variant = keepVariant;
+            std::swap(plan->csr, C);
+            std::swap(plan->slices, L);
+        }
+        if (!rc && (!have || ms < best)) {
+            std::swap(plan->csr, C);
+            std::swap(plan->slices, L);
+            plan->csr_variant = v;
+            best = ms;
+            have = true;
+        }
+        free_csr(C);
+        free_slices(L);
+    }
+    (void)hipFree(tx);
+    (void)hipFree(ty);
+    return rc;
 }
 
 // Minimum fill of a fragment for the MFMA tile kernel to take it (default plans;
@@ -796,8 +1003,8 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     info->tile_frags = plan->tiles.frags;
     info->tile_nnz = plan->tile_nnz;
     info->csr_nnz = plan->csr_nnz;
-    info->csr_blocks = plan->use_slices ? plan->slices.nWG : plan->csr.nBlocks;
-    info->csr_variant = plan->use_slices ? 1 : 0;
+    info->csr_blocks = plan->csr_variant == 1 ? plan->slices.nWG : plan->csr.nBlocks;
+    info->csr_variant = plan->csr_variant;
     // what each kernel has to move at least once: its arrays, x once, its y rows
     info->csr_bytes = (double)plan->csr_nnz * (es + 4) + ((double)plan->rows + 1) * 4 + (double)plan->cols * es +
                       (double)plan->rows * es;
@@ -878,7 +1085,8 @@ extern "C" int mx_time_csr_main(mx_plan *plan, const void *x_dev, void *y_dev, i
     }
     hipStream_t s = plan->stream;
     int rc = time_loop(plan, warm, iters, [&]() -> int {
-        if (plan->use_slices)
+        // the kernel that holds most of the entries
+        if (plan->csr_variant == 1 || (plan->csr_variant == 2 && plan->slices.nnz > plan->csr.nnz))
             MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x_dev, y_dev, 0, s, 1));
         else
             MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x_dev, y_dev, 0, s));

@@ -277,6 +277,118 @@ def test_partition_file_is_checked_on_load(mx, tmp_path):
     P.close()
 
 
+def _walk_slice_layout(L, x, f64):
+    """y from the slice kernel's layout, walked the way the kernel walks it (workgroup, wave,
+    batch, step, lane), every index checked on the way.  Accumulates in float64."""
+    E, BE, W = L["stepEntries"], L["batchEntries"], L["waves"]
+    SPB, SW = BE // E, L["sliceCols"]
+    ecol, ev = L["ecol"], L["eval"].astype(np.float64)
+    partial = np.full(L["chunks"] * 64, np.nan)
+    assert len(ecol) >= L["batches"] * 64 * BE
+    lane = np.arange(64)
+    seen_chunks = 0
+    for b in range(L["nWG"]):
+        q, wgChunk0, wgChunks, _ = L["wgDesc"][b]
+        assert 0 <= q < L["S"] and wgChunk0 == seen_chunks and 0 < wgChunks <= 4096
+        xs = np.zeros(SW)
+        n = max(0, min(SW, len(x) - q * SW))
+        xs[:n] = x[q * SW:q * SW + n]
+        inside = 0
+        for w in range(W):
+            batch0, nb, chunk0, nChunks = L["waveDesc"][b * W + w]
+            assert chunk0 == inside and 0 <= batch0 and batch0 + nb <= L["batches"]
+            inside += nChunks
+            ends = L["chunkEnd"][wgChunk0 + chunk0:wgChunk0 + chunk0 + nChunks]
+            assert np.all(np.diff(np.concatenate(([0], ends))) > 0) and (nChunks == 0 or ends[-1] <= nb * SPB)
+            assert nChunks == 0 or ends[-1] > (nb - 1) * SPB, "a wave's stream has no spare batch"
+            acc, ci = np.zeros(64), 0
+            for t in range(nb):
+                bt = batch0 + t
+                c = ecol[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(64, BE)
+                if f64:
+                    v = ev[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(SPB, 64, E)
+                else:
+                    v = ev[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(64, SPB, E).transpose(1, 0, 2)
+                for j in range(SPB):
+                    cj = c[:, j * E:(j + 1) * E].astype(np.int64)
+                    assert cj.max() < SW
+                    acc += (v[j] * xs[cj]).sum(axis=1)
+                    if ci < nChunks and t * SPB + j + 1 == ends[ci]:
+                        partial[(wgChunk0 + chunk0 + ci) * 64 + lane] = acc
+                        acc, ci = np.zeros(64), ci + 1
+            assert ci == nChunks
+        assert inside == wgChunks
+        seen_chunks += wgChunks
+    assert seen_chunks == L["chunks"] and not np.isnan(partial).any()
+    segPtr, segIdx = L["segPtr"], L["segIdx"]
+    assert segPtr[0] == 0 and segPtr[-1] == L["vrows"] == len(segIdx) and np.all(np.diff(segPtr) >= 0)
+    assert len(np.unique(segIdx)) == len(segIdx) and (len(segIdx) == 0 or (segIdx.min() >= 0 and segIdx.max() < len(partial)))
+    heavy = np.flatnonzero(np.diff(segPtr) > L["lightSegs"])
+    assert np.array_equal(heavy, L["heavy"])
+    y = np.zeros(len(segPtr) - 1)
+    np.add.at(y, np.repeat(np.arange(len(y)), np.diff(segPtr)), partial[segIdx])
+    return y, partial
+
+
+@pytest.mark.parametrize("case", ["block", "powerlaw", "mixed", "unsorted", "tiny", "wide_f64", "subset"])
+def test_slice_layout_walk(mx, ora, case):
+    """The column-slice layout, walked on the CPU exactly as the kernel reads it, gives A x; the
+    padding it stores is zero; rows cut into several virtual rows add up; a subset of the rows
+    leaves the others without virtual rows."""
+    rng = np.random.default_rng(5)
+    sel = None
+    nCU = 8
+    if case == "block":
+        A, x = mx.gen_config(2, scale=1 / 32)
+    elif case == "powerlaw":
+        A, x = mx.gen_config(4, scale=1 / 64)
+    elif case == "mixed":
+        A, x = mx.gen_config(5, scale=1 / 128)
+        nCU = 3
+    elif case == "wide_f64":   # five binary64 slices, one of them empty, ragged last slice
+        rows, cols = 700, 4 * 16384 + 77
+        lens = rng.integers(0, 90, rows)
+        lens[5] = 3000
+        rp = np.zeros(rows + 1, np.int32)
+        rp[1:] = np.cumsum(lens)
+        ci = np.concatenate([np.sort(rng.choice(cols, n, replace=False)) for n in lens]).astype(np.int32)
+        ci[(ci >= 16384) & (ci < 32768)] += 16384
+        A = mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, len(ci)))
+        x = rng.uniform(-1, 1, cols)
+    elif case == "unsorted":   # columns in any order inside a row, duplicates allowed
+        rows, cols = 300, 70000
+        lens = rng.integers(0, 200, rows)
+        rp = np.zeros(rows + 1, np.int32)
+        rp[1:] = np.cumsum(lens)
+        ci = rng.integers(0, cols, rp[-1]).astype(np.int32)
+        A = mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, len(ci)).astype(np.float16))
+        x = rng.uniform(-1, 1, cols).astype(np.float16)
+    elif case == "tiny":
+        A = mx.Csr(3, 5, np.array([0, 2, 2, 3], np.int32), np.array([4, 0, 2], np.int32), np.array([1.0, 2.0, 3.0]))
+        x = np.arange(1.0, 6.0)
+    else:
+        A, x = mx.gen_config(4, scale=1 / 64)
+        sel = (np.diff(A.rowPtr) >= 32).astype(np.uint8)
+    f64 = A.dtype == mx.MX_F64
+    L = mx.slice_layout(A, nCU=nCU, sel=sel)
+    assert L["S"] == -(-A.cols // L["sliceCols"])
+    y, _ = _walk_slice_layout(L, np.asarray(x, np.float64), f64)
+    lens = np.diff(A.rowPtr)
+    keep = np.ones(A.rows, bool) if sel is None else sel.astype(bool)
+    ref = np.zeros(A.rows)
+    rowOf = np.repeat(np.arange(A.rows), lens)
+    np.add.at(ref, rowOf, A.val.astype(np.float64) * np.asarray(x, np.float64)[A.colInd])
+    ref[~keep] = 0.0
+    assert np.allclose(y, ref, rtol=1e-12, atol=1e-12 * max(1.0, np.abs(ref).max()))
+    # every stored value is an entry of the matrix or a zero: the sums of absolute values agree
+    held = np.abs(A.val.astype(np.float64))[np.repeat(keep, lens)].sum()
+    assert np.isclose(np.abs(L["eval"].astype(np.float64)).sum(), held, rtol=1e-12)
+    # rows outside the subset own nothing; no virtual row is longer than the cap
+    nv = np.diff(L["segPtr"])
+    assert np.all(nv[~keep] == 0) and np.all(nv[keep & (lens > 0)] >= 1) and np.all(nv[lens == 0] == 0)
+    assert np.all(nv <= -(-lens // 1) ) and L["cap"] % L["batchEntries"] == 0
+
+
 def test_init_vec(mx):
     v = mx.init_vec(40)
     assert np.array_equal(v, np.arange(40) % 15)
