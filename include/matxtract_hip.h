@@ -215,12 +215,14 @@ int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
  *   ecol      [batches][64][batchEntries] column - slice*sliceCols
  *   eval      per batch: binary16 [64][batchEntries]; binary64 [batchEntries/stepEntries][64][stepEntries]
  *   virtual row v = 64*chunk + lane; matrix row r owns segIdx[segPtr[r] .. segPtr[r+1])
- *   heavy     rows with more than lightSegs virtual rows
+ *   rowInfo   [rows] the virtual row of a row that owns exactly one; -1 for none, -2 for several
+ *   lightInfo [nLight][4] {row, segPtr[row], count, 0} of the rows with 2..lightSegs virtual rows
+ *   heavyInfo [nHeavy][4] the same for the rows with more
  * Release with mx_slice_layout_free. */
 typedef struct mx_slice_layout_view {
-    int nWG, S, sliceCols, waves, stepEntries, batchEntries, cap, chunks, batches, vrows, nHeavy, lightSegs;
+    int nWG, S, sliceCols, waves, stepEntries, batchEntries, cap, chunks, batches, vrows, nLight, nHeavy, lightSegs;
     long long nEcol;
-    int *wgDesc, *waveDesc, *chunkEnd, *segPtr, *segIdx, *heavy;
+    int *wgDesc, *waveDesc, *chunkEnd, *segPtr, *segIdx, *rowInfo, *lightInfo, *heavyInfo;
     unsigned short *ecol;
     unsigned char *eval;
 } mx_slice_layout_view;

@@ -55,9 +55,10 @@ class PlanInfo(C.Structure):
 
 class SliceLayoutView(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("nWG", "S", "sliceCols", "waves", "stepEntries", "batchEntries", "cap", "chunks",
-                                       "batches", "vrows", "nHeavy", "lightSegs")] + \
+                                       "batches", "vrows", "nLight", "nHeavy", "lightSegs")] + \
                [("nEcol", C.c_longlong)] + \
-               [(n, C.c_void_p) for n in ("wgDesc", "waveDesc", "chunkEnd", "segPtr", "segIdx", "heavy", "ecol", "eval")]
+               [(n, C.c_void_p) for n in ("wgDesc", "waveDesc", "chunkEnd", "segPtr", "segIdx", "rowInfo", "lightInfo",
+                                        "heavyInfo", "ecol", "eval")]
 
 
 # Every symbol include/matxtract_hip.h declares: name -> (restype, argtypes)

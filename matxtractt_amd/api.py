@@ -203,14 +203,16 @@ def slice_layout(A, nCU=256, sel=None):
     check(_lib.load().mx_slice_layout(C.byref(st), int(nCU), selp, C.byref(v)))
     try:
         out = {n: int(getattr(v, n)) for n in ("nWG", "S", "sliceCols", "waves", "stepEntries", "batchEntries", "cap",
-                                               "chunks", "batches", "vrows", "nHeavy", "lightSegs")}
+                                               "chunks", "batches", "vrows", "nLight", "nHeavy", "lightSegs")}
         vt = _np_dtype(A.dtype)
         out["wgDesc"] = _view(v.wgDesc, v.nWG * 4, np.int32).reshape(-1, 4).copy()
         out["waveDesc"] = _view(v.waveDesc, v.nWG * v.waves * 4, np.int32).reshape(-1, 4).copy()
         out["chunkEnd"] = _view(v.chunkEnd, v.chunks, np.int32).copy()
         out["segPtr"] = _view(v.segPtr, A.rows + 1, np.int32).copy()
         out["segIdx"] = _view(v.segIdx, v.vrows, np.int32).copy()
-        out["heavy"] = _view(v.heavy, v.nHeavy, np.int32).copy()
+        out["rowInfo"] = _view(v.rowInfo, A.rows, np.int32).copy()
+        out["lightInfo"] = _view(v.lightInfo, v.nLight * 4, np.int32).reshape(-1, 4).copy()
+        out["heavyInfo"] = _view(v.heavyInfo, v.nHeavy * 4, np.int32).reshape(-1, 4).copy()
         out["ecol"] = _view(v.ecol, v.nEcol, np.uint16).copy()
         out["eval"] = _view(v.eval, v.nEcol, vt).copy()
     finally:

@@ -72,8 +72,11 @@ inline int tile_slot(mx_dtype d, int half, int i) { return d == MX_F64 ? 2 * i +
 // contiguous), then their values -- binary16: lanes contiguous; binary64: one sub-block of 16
 // bytes per lane for every step -- so that every load of a wave is one contiguous stretch.
 // Chunks are numbered workgroup by workgroup, wave by wave; virtual row v = 64 * chunk + lane
-// puts its sum into partial[v], and a second kernel adds up the virtual rows of every matrix
-// row: those of row r are segIdx[segPtr[r] .. segPtr[r+1]).
+// puts its sum into partial[v], and a second kernel turns those into y: rowInfo[r] is the
+// virtual row of a matrix row that owns exactly one, -1 for a row that owns none, -2 for a row
+// that owns several; those list theirs in segIdx -- lightInfo / heavyInfo hold {row, first index
+// into segIdx, count, 0} for the rows with up to kSliceLightSegs virtual rows and for those with
+// more.
 struct DeviceSlices {
     int nWG = 0, S = 0, rows = 0, cols = 0, sliceCols = 0;
     int maxWgChunks = 0;              // chunks of the largest workgroup (their ends are kept in LDS)
@@ -88,10 +91,11 @@ struct DeviceSlices {
     unsigned short *ecol = nullptr;   // [batches][64][kSliceBatchEntries] col - slice * sliceCols
     void *eval = nullptr;             // [batches] values, laid out as described above
     void *partial = nullptr;          // [chunks*64] accumulators
-    int *segPtr = nullptr;            // [rows+1]
-    int *segIdx = nullptr;            // [vrows]
-    int *heavy = nullptr;             // [nHeavy] rows with more than kSliceLightSegs virtual rows
-    int nHeavy = 0;
+    int *rowInfo = nullptr;           // [rows, padded to a multiple of 4 with -2]
+    int *segIdx = nullptr;            // [vrows of rows with several]
+    int *lightInfo = nullptr;         // [nLight][4]
+    int *heavyInfo = nullptr;         // [nHeavy][4]
+    int nLight = 0, nHeavy = 0;
 };
 constexpr int kSliceBytes = 131072;   // the slice of x a workgroup keeps in LDS
 constexpr int kSliceLdsMax = 163840;  // LDS of a CU

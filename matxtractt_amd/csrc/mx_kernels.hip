@@ -587,42 +587,70 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         if (t + NB + k < nb) consume(buf[k], t + NB + k);
 }
 
-// y[r] = sum of the virtual rows of matrix row r (+ y[r]).  Rows with few virtual rows take one
-// lane each (the first `lightBlocks` workgroups walk all rows and skip the others); a row with
-// many takes a wave (the remaining workgroups walk the list `heavy`).  With `subset` the rows
-// that own no virtual row are left as they are.
+// The sums of the virtual rows become y in one launch of three kinds of workgroups:
+//  * the first `nRowWG` walk the matrix rows, four per lane: rowInfo[r] >= 0 names the one virtual
+//    row of row r, whose sum is the row's result; -1 is a row without entries (zero, or left
+//    alone when `skipEmpty`); anything else a row that the lists below cover;
+//  * the next `nLightWG` take the rows with 2..kSliceLightSegs virtual rows, one lane each:
+//    {row, first index into segIdx, count};
+//  * the rest take the rows with more, sixteen lanes each.
 template <typename VT>
 __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Acc<VT>::type *__restrict__ partial,
-                                                              const int *__restrict__ segPtr,
-                                                              const int *__restrict__ segIdx,
-                                                              const int *__restrict__ heavy, int nHeavy, int lightBlocks,
-                                                              VT *__restrict__ y, int rows, int accumulate, int subset)
+                                                              const int *__restrict__ rowInfo, int rows, int nRowWG,
+                                                              const int4 *__restrict__ lightInfo, int nLight, int nLightWG,
+                                                              const int4 *__restrict__ heavyInfo, int nHeavy,
+                                                              const int *__restrict__ segIdx, VT *__restrict__ y,
+                                                              int accumulate, int skipEmpty)
 {
     typedef typename Acc<VT>::type AT;
     const int tid = threadIdx.x;
-    if ((int)blockIdx.x < lightBlocks) {
-        const int r = blockIdx.x * kBlock + tid;
-        if (r >= rows) return;
-        const int a = segPtr[r], n = segPtr[r + 1] - a;
-        if (n > mx::kSliceLightSegs || (subset && n == 0)) return;
+    int b = blockIdx.x;
+    if (b < nRowWG) {
+        const int r0 = 4 * (b * kBlock + tid);
+        if (r0 >= rows) return;
+        const int4 d = ((const int4 *)rowInfo)[r0 >> 2];  // padded to a multiple of four with -2
+        const int dd[4] = {d.x, d.y, d.z, d.w};
+        AT sum[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sum[j] = dd[j] >= 0 ? partial[dd[j]] : (AT)0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool mine = dd[j] >= 0 || (dd[j] == -1 && !skipEmpty);
+            if (mine && accumulate) sum[j] += (AT)y[r0 + j];
+            if (mine) y[r0 + j] = (VT)sum[j];
+        }
+        return;
+    }
+    b -= nRowWG;
+    if (b < nLightWG) {
+        const int i = b * kBlock + tid;
+        if (i >= nLight) return;
+        const int4 h = lightInfo[i];
         int id[mx::kSliceLightSegs];
 #pragma unroll
-        for (int k = 0; k < mx::kSliceLightSegs; ++k) id[k] = k < n ? segIdx[a + k] : -1;
-        AT sum = accumulate ? (AT)y[r] : (AT)0;
+        for (int k = 0; k < mx::kSliceLightSegs; ++k) id[k] = k < h.z ? segIdx[h.y + k] : -1;
+        AT sum = accumulate ? (AT)y[h.x] : (AT)0;
 #pragma unroll
         for (int k = 0; k < mx::kSliceLightSegs; ++k)
             if (id[k] >= 0) sum += partial[id[k]];
-        y[r] = (VT)sum;
-    } else {
-        const int w = ((int)blockIdx.x - lightBlocks) * (kBlock / 64) + (tid >> 6), lane = tid & 63;
-        if (w >= nHeavy) return;
-        const int r = heavy[w];
-        const int a = segPtr[r], e = segPtr[r + 1];
-        AT sum = 0;
-        for (int k = a + lane; k < e; k += 64) sum += partial[segIdx[k]];
-        sum = group_sum<64>(sum);
-        if (lane == 0) y[r] = (VT)(sum + (accumulate ? (AT)y[r] : (AT)0));
+        y[h.x] = (VT)sum;
+        return;
     }
+    b -= nLightWG;
+    const int g = b * (kBlock / 16) + (tid >> 4), sub = tid & 15;
+    const bool live = g < nHeavy;
+    const int4 h = live ? heavyInfo[g] : int4{0, 0, 0, 0};
+    AT sum = 0;
+    for (int k = sub; k < h.z; k += 64) {
+        int id[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) id[j] = k + 16 * j < h.z ? segIdx[h.y + k + 16 * j] : -1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (id[j] >= 0) sum += partial[id[j]];
+    }
+    sum = group_sum<16>(sum);
+    if (live && sub == 0) y[h.x] = (VT)(sum + (accumulate ? (AT)y[h.x] : (AT)0));
 }
 
 // ---- tile part --------------------------------------------------------------------------
@@ -872,11 +900,13 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
                            (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || what == 1) return e;
-    const int light = (P.rows + mxk::kBlock - 1) / mxk::kBlock;
-    const int heavy = (P.nHeavy + mxk::kBlock / 64 - 1) / (mxk::kBlock / 64);
-    if (light + heavy == 0) return hipSuccess;
-    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(light + heavy), dim3(mxk::kBlock), 0, s, (const AT *)P.partial,
-                       P.segPtr, P.segIdx, P.heavy, P.nHeavy, light, (VT *)y, P.rows, (accumulate || P.subset) ? 1 : 0,
+    const int nRowWG = ((P.rows + 3) / 4 + mxk::kBlock - 1) / mxk::kBlock;
+    const int nLightWG = (P.nLight + mxk::kBlock - 1) / mxk::kBlock;
+    const int nHeavyWG = (P.nHeavy + mxk::kBlock / 16 - 1) / (mxk::kBlock / 16);
+    if (nRowWG + nLightWG + nHeavyWG == 0) return hipSuccess;
+    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(nRowWG + nLightWG + nHeavyWG), dim3(mxk::kBlock), 0, s,
+                       (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, (const int4 *)P.lightInfo, P.nLight, nLightWG,
+                       (const int4 *)P.heavyInfo, P.nHeavy, P.segIdx, (VT *)y, (accumulate || P.subset) ? 1 : 0,
                        P.subset ? 1 : 0);
     return hipGetLastError();
 }

@@ -102,9 +102,10 @@ void free_slices(mx::DeviceSlices &P)
     (void)hipFree(P.ecol);
     (void)hipFree(P.eval);
     (void)hipFree(P.partial);
-    (void)hipFree(P.segPtr);
+    (void)hipFree(P.rowInfo);
+    (void)hipFree(P.lightInfo);
+    (void)hipFree(P.heavyInfo);
     (void)hipFree(P.segIdx);
-    (void)hipFree(P.heavy);
     P = mx::DeviceSlices();
 }
 
@@ -126,7 +127,7 @@ struct HostSlices {
     int nWG = 0, S = 0, rows = 0, cols = 0, sliceCols = 0, maxWgChunks = 0, nnz = 0, vrows = 0, cap = 0;
     long long steps = 0, chunks = 0;
     bool subset = false;
-    std::vector<int> wgDesc, waveDesc, chunkEnd, segPtr, segIdx, heavy;
+    std::vector<int> wgDesc, waveDesc, chunkEnd, segPtr, segIdx, rowInfo, lightInfo, heavyInfo;
     std::vector<unsigned short> ecol;
     std::vector<unsigned char> eval;
 };
@@ -340,9 +341,17 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
             step = (step + SPB - 1) / SPB * SPB;
         }
     }
-    std::vector<int> heavy;
-    for (int r = 0; r < rows; ++r)
-        if (segPtr[r + 1] - segPtr[r] > mx::kSliceLightSegs) heavy.push_back(r);
+    // how the sums become y: rows with one virtual row are named at that virtual row, the others
+    // are listed
+    std::vector<int> rowInfo(((size_t)rows + 3) / 4 * 4 + 4, -2), lightInfo, heavyInfo;
+    for (int r = 0; r < rows; ++r) {
+        const int a = segPtr[r], n = segPtr[r + 1] - a;
+        rowInfo[r] = n == 0 ? -1 : n == 1 ? segIdx[a] : -2;
+        if (n > 1) {
+            std::vector<int> &L = n > mx::kSliceLightSegs ? heavyInfo : lightInfo;
+            L.insert(L.end(), {r, a, n, 0});
+        }
+    }
     D.nWG = nWG;
     D.S = S;
     D.rows = rows;
@@ -360,7 +369,9 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     D.chunkEnd.swap(chunkEnd);
     D.segPtr.swap(segPtr);
     D.segIdx.swap(segIdx);
-    D.heavy.swap(heavy);
+    D.rowInfo.swap(rowInfo);
+    D.lightInfo.swap(lightInfo);
+    D.heavyInfo.swap(heavyInfo);
     D.ecol.swap(ecol);
     D.eval.swap(ev);
     return MX_OK;
@@ -383,16 +394,18 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
     D.nnz = H.nnz;
     D.vrows = H.vrows;
     D.subset = H.subset;
-    D.nHeavy = (int)H.heavy.size();
+    D.nLight = (int)H.lightInfo.size() / 4;
+    D.nHeavy = (int)H.heavyInfo.size() / 4;
     if ((rc = upload(&D.wgDesc, H.wgDesc.data(), H.wgDesc.size()))) return rc;
     if ((rc = upload(&D.waveDesc, H.waveDesc.data(), H.waveDesc.size()))) return rc;
     if ((rc = upload(&D.chunkEnd, H.chunkEnd.data(), H.chunkEnd.size()))) return rc;
     if ((rc = upload(&D.ecol, H.ecol.data(), H.ecol.size()))) return rc;
     if ((rc = upload_bytes(&D.eval, H.eval.data(), H.eval.size()))) return rc;
     if ((rc = upload_bytes(&D.partial, nullptr, 0, ((size_t)H.chunks * 64 + 64) * (dtype == MX_F64 ? 8 : 4)))) return rc;
-    if ((rc = upload(&D.segPtr, H.segPtr.data(), H.segPtr.size()))) return rc;
+    if ((rc = upload(&D.rowInfo, H.rowInfo.data(), H.rowInfo.size()))) return rc;
     if ((rc = upload(&D.segIdx, H.segIdx.data(), H.segIdx.size()))) return rc;
-    if ((rc = upload(&D.heavy, H.heavy.data(), H.heavy.size(), 1))) return rc;
+    if ((rc = upload(&D.lightInfo, H.lightInfo.data(), H.lightInfo.size(), 4))) return rc;
+    if ((rc = upload(&D.heavyInfo, H.heavyInfo.data(), H.heavyInfo.size(), 4))) return rc;
     return MX_OK;
 }
 
@@ -633,7 +646,8 @@ extern "C" int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *se
     out->chunks = (int)H.chunks;
     out->batches = (int)(H.steps / (mx::kSliceBatchEntries / mx::slice_step_entries(A->dtype)));
     out->vrows = H.vrows;
-    out->nHeavy = (int)H.heavy.size();
+    out->nLight = (int)H.lightInfo.size() / 4;
+    out->nHeavy = (int)H.heavyInfo.size() / 4;
     out->lightSegs = mx::kSliceLightSegs;
     out->nEcol = (long long)H.ecol.size();
     out->wgDesc = give(H.wgDesc);
@@ -641,10 +655,13 @@ extern "C" int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *se
     out->chunkEnd = give(H.chunkEnd);
     out->segPtr = give(H.segPtr);
     out->segIdx = give(H.segIdx);
-    out->heavy = give(H.heavy);
+    out->rowInfo = give(H.rowInfo);
+    out->lightInfo = give(H.lightInfo);
+    out->heavyInfo = give(H.heavyInfo);
     out->ecol = give(H.ecol);
     out->eval = give(H.eval);
-    if (!out->wgDesc || !out->waveDesc || !out->chunkEnd || !out->segPtr || !out->segIdx || !out->heavy || !out->ecol ||
+    if (!out->wgDesc || !out->waveDesc || !out->chunkEnd || !out->segPtr || !out->segIdx || !out->rowInfo || !out->lightInfo ||
+        !out->heavyInfo || !out->ecol ||
         !out->eval) {
         mx_slice_layout_free(out);
         set_error("mx_slice_layout: out of memory");
@@ -661,7 +678,9 @@ extern "C" void mx_slice_layout_free(mx_slice_layout_view *v)
     free(v->chunkEnd);
     free(v->segPtr);
     free(v->segIdx);
-    free(v->heavy);
+    free(v->rowInfo);
+    free(v->lightInfo);
+    free(v->heavyInfo);
     free(v->ecol);
     free(v->eval);
     std::memset(v, 0, sizeof(*v));

@@ -277,7 +277,7 @@ def test_partition_file_is_checked_on_load(mx, tmp_path):
     P.close()
 
 
-def _walk_slice_layout(L, x, f64):
+def _walk_slice_layout(L, x, f64, subset=False):
     """y from the slice kernel's layout, walked the way the kernel walks it (workgroup, wave,
     batch, step, lane), every index checked on the way.  Accumulates in float64."""
     E, BE, W = L["stepEntries"], L["batchEntries"], L["waves"]
@@ -323,10 +323,20 @@ def _walk_slice_layout(L, x, f64):
     segPtr, segIdx = L["segPtr"], L["segIdx"]
     assert segPtr[0] == 0 and segPtr[-1] == L["vrows"] == len(segIdx) and np.all(np.diff(segPtr) >= 0)
     assert len(np.unique(segIdx)) == len(segIdx) and (len(segIdx) == 0 or (segIdx.min() >= 0 and segIdx.max() < len(partial)))
-    heavy = np.flatnonzero(np.diff(segPtr) > L["lightSegs"])
-    assert np.array_equal(heavy, L["heavy"])
-    y = np.zeros(len(segPtr) - 1)
-    np.add.at(y, np.repeat(np.arange(len(y)), np.diff(segPtr)), partial[segIdx])
+    # y as the combine kernel forms it: rows with one virtual row through rowInfo, the others through the lists
+    nv = np.diff(segPtr)
+    info = L["rowInfo"]
+    assert np.array_equal(info[nv == 0], np.full((nv == 0).sum(), -1)) and np.all(info[nv > 1] == -2)
+    single = nv == 1
+    assert np.array_equal(info[single], segIdx[segPtr[:-1][single]])
+    y = np.zeros(len(nv))      # rows without entries: zero (all rows) or not written (subset)
+    y[single] = partial[info[single]]
+    y[nv > 1] = np.nan
+    for lst, lo, hi in ((L["lightInfo"], 2, L["lightSegs"]), (L["heavyInfo"], L["lightSegs"] + 1, 1 << 30)):
+        for r, a, n, _ in lst:
+            assert n == nv[r] and a == segPtr[r] and lo <= n <= hi and np.isnan(y[r])
+            y[r] = partial[segIdx[a:a + n]].sum()
+    assert not np.isnan(y).any()
     return y, partial
 
 
@@ -372,7 +382,7 @@ def test_slice_layout_walk(mx, ora, case):
     f64 = A.dtype == mx.MX_F64
     L = mx.slice_layout(A, nCU=nCU, sel=sel)
     assert L["S"] == -(-A.cols // L["sliceCols"])
-    y, _ = _walk_slice_layout(L, np.asarray(x, np.float64), f64)
+    y, _ = _walk_slice_layout(L, np.asarray(x, np.float64), f64, subset=sel is not None)
     lens = np.diff(A.rowPtr)
     keep = np.ones(A.rows, bool) if sel is None else sel.astype(bool)
     ref = np.zeros(A.rows)
