@@ -213,7 +213,8 @@ int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
  *   waveDesc  [nWG*waves][4] {first batch, batches, first chunk inside the workgroup, chunks}
  *   chunkEnd  [chunks]  step, counted from the wave's first, at which the chunk ends
  *   ecol      [batches][64][batchEntries] column - slice*sliceCols
- *   eval      per batch: binary16 [64][batchEntries]; binary64 [batchEntries/stepEntries][64][stepEntries]
+ *   eval      per batch: binary16 [64][batchEntries]; binary64 [batchEntries/2][64][2]
+ *   a lane takes stepEntries (= 1) entries per step; chunkEnd counts steps
  *   virtual row v = 64*chunk + lane; matrix row r owns segIdx[segPtr[r] .. segPtr[r+1])
  *   rowInfo   [rows] the virtual row of a row that owns exactly one; -1 for none, -2 for several
  *   lightInfo [nLight][4] {row, segPtr[row], count, 0} of the rows with 2..lightSegs virtual rows

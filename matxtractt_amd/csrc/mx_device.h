@@ -65,12 +65,11 @@ inline int tile_slot(mx_dtype d, int half, int i) { return d == MX_F64 ? 2 * i +
 // virtual row per lane (a sliced-ELL layout: every row of a chunk is padded to the chunk's
 // longest, and the sort keeps that padding small).  A slice gets workgroups in proportion to
 // its entries, its chunks are dealt to them longest first, and inside a workgroup to its waves
-// the same way.  A lane walks its virtual row E entries -- one "step" -- at a time (E = 2
-// binary64, 4 binary16); chunks end on step boundaries; a wave's chunks follow each other in
+// the same way.  A lane walks its virtual row one entry -- one "step" -- at a time; a wave's chunks follow each other in
 // the wave's stream, which is stored in batches of kSliceBatchEntries entries per lane
 // (zero-padded to a whole batch at the end): per batch the lanes' column offsets (lanes
 // contiguous), then their values -- binary16: lanes contiguous; binary64: one sub-block of 16
-// bytes per lane for every step -- so that every load of a wave is one contiguous stretch.
+// bytes (two values) per lane -- so that every load of a wave is one contiguous stretch.
 // Chunks are numbered workgroup by workgroup, wave by wave; virtual row v = 64 * chunk + lane
 // puts its sum into partial[v], and a second kernel turns those into y: rowInfo[r] is the
 // virtual row of a matrix row that owns exactly one, -1 for a row that owns none, -2 for a row
@@ -80,7 +79,7 @@ inline int tile_slot(mx_dtype d, int half, int i) { return d == MX_F64 ? 2 * i +
 struct DeviceSlices {
     int nWG = 0, S = 0, rows = 0, cols = 0, sliceCols = 0;
     int maxWgChunks = 0;              // chunks of the largest workgroup (their ends are kept in LDS)
-    long long steps = 0;              // total steps stored (64 lanes * E entries each)
+    long long steps = 0;              // total steps stored (64 lanes, one entry each)
     long long chunks = 0;             // total chunks
     int nnz = 0;                      // entries held
     int vrows = 0;                    // virtual rows
@@ -104,7 +103,7 @@ constexpr int kSliceWaves = 8;        // waves per workgroup; one workgroup per 
 constexpr int kSliceThreads = 64 * kSliceWaves;
 inline int slice_cols(mx_dtype d) { return kSliceBytes / (d == MX_F64 ? 8 : 2); }
 constexpr int kSliceBatchEntries = 8;  // entries a lane loads at a time
-inline int slice_step_entries(mx_dtype d) { return d == MX_F64 ? 2 : 4; }  // kSliceE
+inline int slice_step_entries(mx_dtype) { return 1; }  // entries a lane takes per step; chunks end between steps
 constexpr int kSliceLightSegs = 8;     // rows with at most this many virtual rows are summed by one lane
 
 // `what`: 0 = slice kernel then combine kernel, 1 = slice kernel only, 2 = combine kernel only

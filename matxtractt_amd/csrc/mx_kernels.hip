@@ -434,7 +434,7 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
 // instead of HBM.  Gathers from LDS cost next to nothing.  The columns are cut into S slices
 // (a slice of x fits LDS); a workgroup -- one per CU -- copies one slice into LDS once and then
 // streams entries whose columns fall into it.  Those are laid out as sliced ELL over "virtual
-// rows" (see DeviceSlices): one virtual row per lane, E entries per lane per step, steps
+// rows" (see DeviceSlices): one virtual row per lane, one entry per lane per step, steps
 // contiguous across the wave, so a lane sums its virtual row in a register with no cross-lane
 // traffic at all, and at the end of a chunk of 64 virtual rows every lane stores one sum,
 // the wave 64 consecutive ones.  A second kernel adds up the virtual rows of every matrix row.
@@ -443,7 +443,6 @@ template <typename VT>
 struct SliceBatch;  // what one lane reads per batch: 8 column offsets, 8 values
 template <>
 struct SliceBatch<double> {
-    static constexpr int E = 2, SPB = 4;  // entries per step, steps per batch
     v4i32 c;
     v2f64 v[4];
     __device__ __forceinline__ void load(const unsigned short *ecol, const double *eval, size_t batch, int lane)
@@ -453,28 +452,26 @@ struct SliceBatch<double> {
         for (int j = 0; j < 4; ++j)
             v[j] = __builtin_nontemporal_load((const v2f64 *)(eval + batch * 512 + j * 128 + lane * 2));
     }
-    __device__ __forceinline__ double dot(const double *xs, int j) const
+    // value * x of entry k of the batch
+    __device__ __forceinline__ double term(const double *xs, int k) const
     {
-        const unsigned w = (unsigned)c[j];
-        return v[j].x * xs[w & 0xffffu] + v[j].y * xs[w >> 16];
+        const unsigned w = (unsigned)c[k >> 1];
+        return (k & 1) ? v[k >> 1].y * xs[w >> 16] : v[k >> 1].x * xs[w & 0xffffu];
     }
 };
 template <>
 struct SliceBatch<_Float16> {
-    static constexpr int E = 4, SPB = 2;
     v4i32 c, v;
     __device__ __forceinline__ void load(const unsigned short *ecol, const _Float16 *eval, size_t batch, int lane)
     {
         c = __builtin_nontemporal_load((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
         v = __builtin_nontemporal_load((const v4i32 *)(eval + (batch * 64 + lane) * 8));
     }
-    __device__ __forceinline__ float dot(const _Float16 *xs, int j) const
+    __device__ __forceinline__ float term(const _Float16 *xs, int k) const
     {
-        const unsigned c0 = (unsigned)c[2 * j], c1 = (unsigned)c[2 * j + 1];
-        const unsigned v0 = (unsigned)v[2 * j], v1 = (unsigned)v[2 * j + 1];
-        auto h = [](unsigned bits) { return (float)__builtin_bit_cast(_Float16, (unsigned short)bits); };
-        return h(v0 & 0xffffu) * (float)xs[c0 & 0xffffu] + h(v0 >> 16) * (float)xs[c0 >> 16] +
-               h(v1 & 0xffffu) * (float)xs[c1 & 0xffffu] + h(v1 >> 16) * (float)xs[c1 >> 16];
+        const unsigned cw = (unsigned)c[k >> 1], vw = (unsigned)v[k >> 1];
+        const unsigned ci = (k & 1) ? cw >> 16 : cw & 0xffffu, vi = (k & 1) ? vw >> 16 : vw & 0xffffu;
+        return (float)__builtin_bit_cast(_Float16, (unsigned short)vi) * (float)xs[ci];
     }
 };
 static_assert(mx::kSliceBatchEntries == 8, "SliceBatch holds 8 entries per lane");
@@ -498,7 +495,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 {
     typedef typename Acc<VT>::type AT;
     typedef SliceBatch<VT> Batch;
-    constexpr int SPB = Batch::SPB, NB = kSliceRing;
+    constexpr int SPB = mx::kSliceBatchEntries, NB = kSliceRing;  // a step is one entry per lane
     constexpr int EPV = 16 / (int)sizeof(VT);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     VT *xs = (VT *)smem;                                           // [sliceCols]
@@ -563,7 +560,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     auto consume = [&](const Batch &B, int t) {  // t = number of the batch in the wave's stream
 #pragma unroll
         for (int j = 0; j < SPB; ++j) {
-            acc += B.dot(xs, j);
+            acc += B.term(xs, j);
             if (t * SPB + j + 1 == nextEnd) flush();
         }
     };
@@ -903,6 +900,18 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     const int nRowWG = ((P.rows + 3) / 4 + mxk::kBlock - 1) / mxk::kBlock;
     const int nLightWG = (P.nLight + mxk::kBlock - 1) / mxk::kBlock;
     const int nHeavyWG = (P.nHeavy + mxk::kBlock / 16 - 1) / (mxk::kBlock / 16);
+    static int dbg = -1;
+    if (dbg < 0) dbg = getenv("MX_DBG_COMBINE") ? atoi(getenv("MX_DBG_COMBINE")) : 0;
+    const int xr = (dbg & 1) ? 0 : P.rows, xl = (dbg & 2) ? 0 : P.nLight, xh = (dbg & 4) ? 0 : P.nHeavy;
+    if (dbg) {
+        const int a = (dbg & 1) ? 0 : nRowWG, b = (dbg & 2) ? 0 : nLightWG, c = (dbg & 4) ? 0 : nHeavyWG;
+        if (a + b + c == 0) return hipSuccess;
+        hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(a + b + c), dim3(mxk::kBlock), 0, s,
+                       (const AT *)P.partial, P.rowInfo, xr, a, (const int4 *)P.lightInfo, xl, b,
+                       (const int4 *)P.heavyInfo, xh, P.segIdx, (VT *)y, (accumulate || P.subset) ? 1 : 0,
+                       P.subset ? 1 : 0);
+        return hipGetLastError();
+    }
     if (nRowWG + nLightWG + nHeavyWG == 0) return hipSuccess;
     hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(nRowWG + nLightWG + nHeavyWG), dim3(mxk::kBlock), 0, s,
                        (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, (const int4 *)P.lightInfo, P.nLight, nLightWG,

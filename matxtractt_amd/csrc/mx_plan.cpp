@@ -325,11 +325,11 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
                     segIdx[t] = (int)(chunk * 64 + l);
                     for (int n = 0; n < v.len; ++n) {
                         const int p = ord[v.start + n];
-                        const size_t st = (size_t)step + n / E, batch = st / SPB, sub = st % SPB;
+                        const size_t st = (size_t)step + n, batch = st / BE, k = st % BE;
                         // a lane's column offsets of a batch are contiguous; so are its binary16
-                        // values; binary64 values go step by step, two per lane
-                        const size_t atc = (batch * 64 + l) * BE + sub * E + n % E;
-                        const size_t atv = dtype == MX_F64 ? batch * 64 * BE + sub * 128 + (size_t)l * 2 + n % E : atc;
+                        // values; binary64 values go in sub-blocks of two per lane
+                        const size_t atc = (batch * 64 + l) * BE + k;
+                        const size_t atv = dtype == MX_F64 ? batch * 64 * BE + (k / 2) * 128 + (size_t)l * 2 + k % 2 : atc;
                         ecol[atc] = (unsigned short)(col[p] - q * SW);
                         std::memcpy(&ev[atv * es], sv + (size_t)p * es, es);
                     }

@@ -280,8 +280,8 @@ def test_partition_file_is_checked_on_load(mx, tmp_path):
 def _walk_slice_layout(L, x, f64, subset=False):
     """y from the slice kernel's layout, walked the way the kernel walks it (workgroup, wave,
     batch, step, lane), every index checked on the way.  Accumulates in float64."""
-    E, BE, W = L["stepEntries"], L["batchEntries"], L["waves"]
-    SPB, SW = BE // E, L["sliceCols"]
+    BE, W, SW = L["batchEntries"], L["waves"], L["sliceCols"]
+    assert L["stepEntries"] == 1   # chunks may end after any entry
     ecol, ev = L["ecol"], L["eval"].astype(np.float64)
     partial = np.full(L["chunks"] * 64, np.nan)
     assert len(ecol) >= L["batches"] * 64 * BE
@@ -299,21 +299,20 @@ def _walk_slice_layout(L, x, f64, subset=False):
             assert chunk0 == inside and 0 <= batch0 and batch0 + nb <= L["batches"]
             inside += nChunks
             ends = L["chunkEnd"][wgChunk0 + chunk0:wgChunk0 + chunk0 + nChunks]
-            assert np.all(np.diff(np.concatenate(([0], ends))) > 0) and (nChunks == 0 or ends[-1] <= nb * SPB)
-            assert nChunks == 0 or ends[-1] > (nb - 1) * SPB, "a wave's stream has no spare batch"
+            assert np.all(np.diff(np.concatenate(([0], ends))) > 0) and (nChunks == 0 or ends[-1] <= nb * BE)
+            assert nChunks == 0 or ends[-1] > (nb - 1) * BE, "a wave's stream has no spare batch"
             acc, ci = np.zeros(64), 0
             for t in range(nb):
                 bt = batch0 + t
-                c = ecol[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(64, BE)
-                if f64:
-                    v = ev[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(SPB, 64, E)
+                c = ecol[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(64, BE).astype(np.int64)
+                if f64:   # sub-blocks of two values per lane
+                    v = ev[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(BE // 2, 64, 2).transpose(1, 0, 2).reshape(64, BE)
                 else:
-                    v = ev[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(64, SPB, E).transpose(1, 0, 2)
-                for j in range(SPB):
-                    cj = c[:, j * E:(j + 1) * E].astype(np.int64)
-                    assert cj.max() < SW
-                    acc += (v[j] * xs[cj]).sum(axis=1)
-                    if ci < nChunks and t * SPB + j + 1 == ends[ci]:
+                    v = ev[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(64, BE)
+                assert c.max() < SW
+                for k in range(BE):
+                    acc += v[:, k] * xs[c[:, k]]
+                    if ci < nChunks and t * BE + k + 1 == ends[ci]:
                         partial[(wgChunk0 + chunk0 + ci) * 64 + lane] = acc
                         acc, ci = np.zeros(64), ci + 1
             assert ci == nChunks
