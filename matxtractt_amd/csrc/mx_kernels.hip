@@ -543,12 +543,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     // the ring is issued only now: a wave that is busy issuing loads cannot store the slice, and
     // the address unit takes the loads no faster than their data moves
     Batch buf[NB];
-#pragma unroll
-    for (int k = 0; k < NB; ++k)
-        if (k < nb) buf[k].load(ecol, eval, (size_t)(batch0 + k), lane);
-    __syncthreads();
-    int ci = 0;
-    int nextEnd = nChunks > 0 ? endsL[chunk0] : -1;
+    int ci = 0, nextEnd = -1, t = 0;
     AT acc = 0;
     AT *out = partial + (size_t)(wgChunk0 + chunk0) * 64 + lane;
     auto flush = [&]() {
@@ -564,14 +559,29 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
             if (t * SPB + j + 1 == nextEnd) flush();
         }
     };
-    int t = 0;
-    // while a whole ring beyond the one in flight remains: consume and reload, no conditions
-    for (; t + 2 * NB <= nb; t += NB) {
+    // A stream of at least two ring lengths runs a loop in which every consumed batch is
+    // reloaded at once, with no condition anywhere on the way from the first load to the loop: the
+    // compiler then knows how many loads are in flight at every use and waits for exactly the
+    // one it needs.  (With the conditional loads of the short path in front of it the loop would
+    // wait for all of them at every turn.)  Both paths meet the workgroup's one barrier.
+    if (nb >= 2 * NB) {
 #pragma unroll
-        for (int k = 0; k < NB; ++k) {
-            consume(buf[k], t + k);
-            buf[k].load(ecol, eval, (size_t)(batch0 + t + NB + k), lane);
+        for (int k = 0; k < NB; ++k) buf[k].load(ecol, eval, (size_t)(batch0 + k), lane);
+        __syncthreads();
+        nextEnd = endsL[chunk0];
+        for (; t + 2 * NB <= nb; t += NB) {
+#pragma unroll
+            for (int k = 0; k < NB; ++k) {
+                consume(buf[k], t + k);
+                buf[k].load(ecol, eval, (size_t)(batch0 + t + NB + k), lane);
+            }
         }
+    } else {
+#pragma unroll
+        for (int k = 0; k < NB; ++k)
+            if (k < nb) buf[k].load(ecol, eval, (size_t)(batch0 + k), lane);
+        __syncthreads();
+        nextEnd = nChunks > 0 ? endsL[chunk0] : -1;
     }
     // tail: what is in flight, reloading while batches remain, then those
 #pragma unroll
@@ -585,12 +595,13 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 }
 
 // The sums of the virtual rows become y in one launch of three kinds of workgroups:
-//  * the first `nRowWG` walk the matrix rows, four per lane: rowInfo[r] >= 0 names the one virtual
+//  * the first `nRowWG` walk the matrix rows, kCombineRows per lane: rowInfo[r] >= 0 names the one virtual
 //    row of row r, whose sum is the row's result; -1 is a row without entries (zero, or left
 //    alone when `skipEmpty`); anything else a row that the lists below cover;
 //  * the next `nLightWG` take the rows with 2..kSliceLightSegs virtual rows, one lane each:
 //    {row, first index into segIdx, count};
 //  * the rest take the rows with more, sixteen lanes each.
+constexpr int kCombineRows = 16;  // rows a lane of the first kind takes
 template <typename VT>
 __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Acc<VT>::type *__restrict__ partial,
                                                               const int *__restrict__ rowInfo, int rows, int nRowWG,
@@ -603,18 +614,23 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
     const int tid = threadIdx.x;
     int b = blockIdx.x;
     if (b < nRowWG) {
-        const int r0 = 4 * (b * kBlock + tid);
-        if (r0 >= rows) return;
-        const int4 d = ((const int4 *)rowInfo)[r0 >> 2];  // padded to a multiple of four with -2
-        const int dd[4] = {d.x, d.y, d.z, d.w};
-        AT sum[4];
+        // kCombineRows rows per lane, as quads a wave apart so that its loads and stores stay contiguous
+        int dd[kCombineRows];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) sum[j] = dd[j] >= 0 ? partial[dd[j]] : (AT)0;
+        for (int q = 0; q < kCombineRows / 4; ++q) {
+            const int r0 = 4 * ((b * (kCombineRows / 4) + q) * kBlock + tid);
+            const int4 d = r0 < rows ? ((const int4 *)rowInfo)[r0 >> 2] : int4{-2, -2, -2, -2};  // padded with -2
+            dd[4 * q] = d.x, dd[4 * q + 1] = d.y, dd[4 * q + 2] = d.z, dd[4 * q + 3] = d.w;
+        }
+        AT sum[kCombineRows];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kCombineRows; ++j) sum[j] = dd[j] >= 0 ? partial[dd[j]] : (AT)0;
+#pragma unroll
+        for (int j = 0; j < kCombineRows; ++j) {
+            const int r = 4 * ((b * (kCombineRows / 4) + j / 4) * kBlock + tid) + j % 4;
             const bool mine = dd[j] >= 0 || (dd[j] == -1 && !skipEmpty);
-            if (mine && accumulate) sum[j] += (AT)y[r0 + j];
-            if (mine) y[r0 + j] = (VT)sum[j];
+            if (mine && accumulate) sum[j] += (AT)y[r];
+            if (mine) y[r] = (VT)sum[j];
         }
         return;
     }
@@ -897,7 +913,7 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
                            (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || what == 1) return e;
-    const int nRowWG = ((P.rows + 3) / 4 + mxk::kBlock - 1) / mxk::kBlock;
+    const int nRowWG = (P.rows + mxk::kCombineRows * mxk::kBlock - 1) / (mxk::kCombineRows * mxk::kBlock);
     const int nLightWG = (P.nLight + mxk::kBlock - 1) / mxk::kBlock;
     const int nHeavyWG = (P.nHeavy + mxk::kBlock / 16 - 1) / (mxk::kBlock / 16);
     static int dbg = -1;

@@ -143,11 +143,16 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     for (int r = 0; r < rows; ++r) selPtr[r + 1] = selPtr[r] + ((!sel || sel[r]) ? rowPtr[r + 1] - rowPtr[r] : 0);
     const int nnz = selPtr[rows];
     std::vector<int> ord((size_t)nnz);
-    // a lane's fair share of the entries; virtual rows are cut to half of it so that the chunks
-    // can be dealt evenly
+    // a lane's fair share of the entries; virtual rows are cut to that, so that no chunk is more
+    // than a wave's share and the chunks can be dealt evenly (measured: half of it costs more
+    // in extra virtual rows than it gains in balance)
     const int budget = std::max(nCU, 1);
     const long long fair = (long long)nnz / ((long long)budget * W * 64);
-    const int cap = (int)std::min<long long>(512, std::max<long long>(16, (fair / 2 + BE - 1) / BE * BE));
+    int cap = (int)std::min<long long>(512, std::max<long long>(16, (fair + BE - 1) / BE * BE));
+    if (const char *e = std::getenv("MX_SLICE_CAP")) {  // for tuning runs
+        const int v = std::atoi(e);
+        if (v >= BE && v <= 4096) cap = v / BE * BE;
+    }
     std::vector<int> segPtr((size_t)rows + 1, 0);
 #pragma omp parallel for schedule(dynamic, 1024)
     for (int r = 0; r < rows; ++r) {
