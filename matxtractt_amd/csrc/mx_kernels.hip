@@ -477,11 +477,9 @@ struct SliceBatch<_Float16> {
 static_assert(mx::kSliceBatchEntries == 8, "SliceBatch holds 8 entries per lane");
 
 // What a CU can take in from L2 or beyond is bounded in bytes (about 32 per cycle, whatever
-// the width of the loads), so nothing is loaded that is not needed: a lane keeps up to kSliceRing
-// batches in flight, streams no longer than the ring are loaded whole before anything else
-// happens; longer ones run a loop in which every consumed batch is reloaded with the batch one
-// ring length ahead (those reloads are unconditional inside the loop, so the number of loads
-// in flight is known at compile time and no wait is longer than it has to be), and a tail.
+// the width of the loads).  A lane keeps kSliceRing batches in flight: a stream no longer than
+// the ring is loaded whole before anything else happens; a longer one runs a loop in which
+// every consumed batch is reloaded with the batch one ring length ahead.
 constexpr int kSliceRing = 6;
 
 template <typename VT>
@@ -508,42 +506,55 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     const int slice = gd.x, wgChunk0 = gd.y, wgChunks = gd.z;
     const int batch0 = __builtin_amdgcn_readfirstlane(d.x), nb = __builtin_amdgcn_readfirstlane(d.y);
     const int chunk0 = __builtin_amdgcn_readfirstlane(d.z), nChunks = __builtin_amdgcn_readfirstlane(d.w);
+    // Every load below is unconditional -- indices are clamped instead, and what a clamped load
+    // brings is masked or never used -- because the compiler can count the loads in flight, and so
+    // wait for exactly the one it needs, only along paths on which the loads are certain.  After
+    // a conditional load it waits for all of them at every use, and the pipeline is gone.
+    //
     // chunk ends of the workgroup, and the slice (all of it at once, one 16-byte vector per
-    // lane and round)
-    const int ce = tid < wgChunks ? chunkEnd[wgChunk0 + tid] : 0;
+    // lane and round).  The last vector of x may be partial: it is read whole (an aligned 16-byte
+    // read cannot leave the page its first byte is on) and the elements beyond x are zeroed.
+    const int ce = chunkEnd[wgChunk0 + min(tid, wgChunks - 1)];
     constexpr int CB = kSliceBytes / 16 / kSliceThreads;  // rounds of a full slice
-    const int nvec = sliceCols / EPV;
+    const int lastVec = (cols + EPV - 1) / EPV - 1;
     v4i32 xv[CB];
 #pragma unroll
     for (int q = 0; q < CB; ++q) {
-        const int i = tid + q * kSliceThreads;
-        const int c = slice * sliceCols + i * EPV;
-        xv[q] = v4i32{0, 0, 0, 0};
-        if (i < nvec && c + EPV <= cols) xv[q] = *(const v4i32 *)(x + c);
+        const int gi = slice * (sliceCols / EPV) + tid + q * kSliceThreads;
+        xv[q] = ((const v4i32 *)x)[min(gi, lastVec)];
     }
-    {
-        if (tid < wgChunks) endsL[tid] = ce;
-        for (int i = kSliceThreads + tid; i < wgChunks; i += kSliceThreads) endsL[i] = chunkEnd[wgChunk0 + i];
-        // ragged end of x: the last, partial vector is filled element by element, and left out
-        // of the sweep below (whose lane for it is in another wave and holds zeros)
-        int ragged = -1;
-        if (cols % EPV) {
-            const int c = cols - cols % EPV, i = (c - slice * sliceCols) / EPV;
-            if (c >= slice * sliceCols && i < nvec) {
-                ragged = i;
-                if (tid < EPV) xs[i * EPV + tid] = tid < cols % EPV ? x[c + tid] : (VT)0;
-            }
-        }
+    // the ring: the first batches of the wave's stream (the last one again and again when the
+    // stream is shorter than the ring)
+    Batch buf[NB];
+    const int lastBatch = batch0 + max(nb - 1, 0);
+#pragma unroll
+    for (int k = 0; k < NB; ++k) buf[k].load(ecol, eval, (size_t)min(batch0 + k, lastBatch), lane);
+    endsL[min(tid, wgChunks - 1)] = ce;
+    if ((slice + 1) * sliceCols <= cols) {  // the whole slice lies inside x
+#pragma unroll
+        for (int q = 0; q < CB; ++q) *(v4i32 *)(xs + (tid + q * kSliceThreads) * EPV) = xv[q];
+    } else {
 #pragma unroll
         for (int q = 0; q < CB; ++q) {
             const int i = tid + q * kSliceThreads;
-            if (i < nvec && i != ragged) *(v4i32 *)(xs + i * EPV) = xv[q];
+            const int have = cols - (slice * sliceCols + i * EPV);  // elements of this vector inside x
+            v4i32 v = xv[q];
+            if (sizeof(VT) == 8) {
+                if (have < 1) v[0] = v[1] = 0;
+                if (have < 2) v[2] = v[3] = 0;
+            } else {
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    if (have < 2 * d + 1) v[d] = 0;
+                    else if (have < 2 * d + 2) v[d] &= 0xffff;
+                }
+            }
+            *(v4i32 *)(xs + i * EPV) = v;
         }
     }
-    // the ring is issued only now: a wave that is busy issuing loads cannot store the slice, and
-    // the address unit takes the loads no faster than their data moves
-    Batch buf[NB];
-    int ci = 0, nextEnd = -1, t = 0;
+    for (int i = kSliceThreads + tid; i < wgChunks; i += kSliceThreads) endsL[i] = chunkEnd[wgChunk0 + i];
+    __syncthreads();
+    int ci = 0, nextEnd = nChunks > 0 ? endsL[chunk0] : -1;
     AT acc = 0;
     AT *out = partial + (size_t)(wgChunk0 + chunk0) * 64 + lane;
     auto flush = [&]() {
@@ -559,35 +570,27 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
             if (t * SPB + j + 1 == nextEnd) flush();
         }
     };
-    // A stream of at least two ring lengths runs a loop in which every consumed batch is
-    // reloaded at once, with no condition anywhere on the way from the first load to the loop: the
-    // compiler then knows how many loads are in flight at every use and waits for exactly the
-    // one it needs.  (With the conditional loads of the short path in front of it the loop would
-    // wait for all of them at every turn.)  Both paths meet the workgroup's one barrier.
-    if (nb >= 2 * NB) {
-#pragma unroll
-        for (int k = 0; k < NB; ++k) buf[k].load(ecol, eval, (size_t)(batch0 + k), lane);
-        __syncthreads();
-        nextEnd = endsL[chunk0];
-        for (; t + 2 * NB <= nb; t += NB) {
-#pragma unroll
-            for (int k = 0; k < NB; ++k) {
-                consume(buf[k], t + k);
-                buf[k].load(ecol, eval, (size_t)(batch0 + t + NB + k), lane);
-            }
-        }
-    } else {
+    if (nb <= NB) {  // everything is in the ring already
 #pragma unroll
         for (int k = 0; k < NB; ++k)
-            if (k < nb) buf[k].load(ecol, eval, (size_t)(batch0 + k), lane);
-        __syncthreads();
-        nextEnd = nChunks > 0 ? endsL[chunk0] : -1;
+            if (k < nb) consume(buf[k], k);
+        return;
     }
-    // tail: what is in flight, reloading while batches remain, then those
+    int t = 0;
+    // while a whole ring beyond the one in flight remains: consume and reload
+    for (; t + 2 * NB <= nb; t += NB) {
+#pragma unroll
+        for (int k = 0; k < NB; ++k) {
+            consume(buf[k], t + k);
+            buf[k].load(ecol, eval, (size_t)(batch0 + t + NB + k), lane);
+        }
+    }
+    // one ring in flight and less than one more to come: consume and reload while batches
+    // remain (the last one again after that), then those
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
-        if (t + k < nb) consume(buf[k], t + k);
-        if (t + NB + k < nb) buf[k].load(ecol, eval, (size_t)(batch0 + t + NB + k), lane);
+        consume(buf[k], t + k);
+        buf[k].load(ecol, eval, (size_t)min(batch0 + t + NB + k, lastBatch), lane);
     }
 #pragma unroll
     for (int k = 0; k < NB; ++k)
