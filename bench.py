@@ -127,13 +127,13 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline):
     else:
         # the CSR part's main kernel alone (the slice variant has a small combine kernel after it)
         ms_main = plan.time_csr_main(xd, yd, warm=warmup, iters=steps)
-        name = "csr_slice_kernel<%s>" if info["csr_variant"] == 1 else "csr_rows_kernel<%s>"
+        name = "csr_slice_kernel<%s>" if info["csr_main_kernel"] == 1 else "csr_rows_kernel<%s>"
         dom = {"kernel": name % dtype, "ms": ms_main,
-               "bytes": kernel_bytes(mx, A.dtype, A.rows, A.cols, info["csr_nnz"])}
+               "bytes": kernel_bytes(mx, A.dtype, A.rows, A.cols, info["csr_main_nnz"])}
     achieved = dom["bytes"] / (dom["ms"] * 1e-3)
     rec = {
         "workload": WORKLOADS[cfg], "dtype": dtype, "rows": A.rows, "nnz": A.nnz,
-        "tau_c": tau[0], "tau_r": tau[1], "csr_variant": "slices" if info["csr_variant"] == 1 else "rows",
+        "tau_c": tau[0], "tau_r": tau[1], "csr_variant": ("rows", "slices", "split")[info["csr_variant"]],
         "ms_per_step": wall_ms, "ms_per_step_events": ev_total,
         "gflops": 2.0 * A.nnz / (wall_ms * 1e-3) / 1e9,
         "algorithmic_bytes": B,

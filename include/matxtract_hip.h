@@ -202,6 +202,9 @@ typedef struct mx_plan_info {
                             2 = row tiles for the short rows, then column slices for the long ones */
     double tile_bytes;   /* bytes the tile kernel must read+write per launch */
     double csr_bytes;    /* bytes the CSR kernel must read+write per launch */
+    int csr_main_kernel; /* the CSR-part kernel that holds most entries (the one mx_time_csr_main times):
+                            0 = csr_rows_kernel, 1 = csr_slice_kernel */
+    int csr_main_nnz;    /* entries that kernel holds */
 } mx_plan_info;
 int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
 

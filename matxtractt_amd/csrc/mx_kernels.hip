@@ -539,29 +539,25 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
             const int i = tid + q * kSliceThreads;
             const int have = cols - (slice * sliceCols + i * EPV);  // elements of this vector inside x
             v4i32 v = xv[q];
-            if (sizeof(VT) == 8) {
-                if (have < 1) v[0] = v[1] = 0;
-                if (have < 2) v[2] = v[3] = 0;
-            } else {
 #pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    if (have < 2 * d + 1) v[d] = 0;
-                    else if (have < 2 * d + 2) v[d] &= 0xffff;
-                }
+            for (int d = 0; d < 4; ++d) {  // dword d holds half an element, or two
+                const int lo = sizeof(VT) == 8 ? d / 2 : 2 * d, hi = sizeof(VT) == 8 ? d / 2 : 2 * d + 1;
+                v[d] &= (have > lo ? 0xffff : 0) | (have > hi ? 0xffff0000 : 0);
             }
             *(v4i32 *)(xs + i * EPV) = v;
         }
     }
     for (int i = kSliceThreads + tid; i < wgChunks; i += kSliceThreads) endsL[i] = chunkEnd[wgChunk0 + i];
     __syncthreads();
-    int ci = 0, nextEnd = nChunks > 0 ? endsL[chunk0] : -1;
+    // (the chunk ends are the same for all lanes of the wave: kept in scalar registers)
+    int ci = 0, nextEnd = nChunks > 0 ? __builtin_amdgcn_readfirstlane(endsL[chunk0]) : -1;
     AT acc = 0;
     AT *out = partial + (size_t)(wgChunk0 + chunk0) * 64 + lane;
     auto flush = [&]() {
         out[(size_t)ci * 64] = acc;
         acc = 0;
         ++ci;
-        nextEnd = ci < nChunks ? endsL[chunk0 + ci] : -1;
+        nextEnd = ci < nChunks ? __builtin_amdgcn_readfirstlane(endsL[chunk0 + ci]) : -1;
     };
     auto consume = [&](const Batch &B, int t) {  // t = number of the batch in the wave's stream
 #pragma unroll

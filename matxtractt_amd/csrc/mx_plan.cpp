@@ -1039,6 +1039,9 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
                                  (double)plan->tiles.frags * fragK * es + (double)plan->tiles.chunkNum * 8 * 2 * es
                            : 0.0;
     (void)bitBytes;
+    const bool sliceMain = plan->csr_variant == 1 || (plan->csr_variant == 2 && plan->slices.nnz > plan->csr.nnz);
+    info->csr_main_kernel = sliceMain ? 1 : 0;
+    info->csr_main_nnz = plan->csr_variant == 2 ? (sliceMain ? plan->slices.nnz : plan->csr.nnz) : plan->csr_nnz;
     return MX_OK;
 }
 
