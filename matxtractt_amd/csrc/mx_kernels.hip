@@ -915,18 +915,6 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     const int nRowWG = (P.rows + mxk::kCombineRows * mxk::kBlock - 1) / (mxk::kCombineRows * mxk::kBlock);
     const int nLightWG = (P.nLight + mxk::kBlock - 1) / mxk::kBlock;
     const int nHeavyWG = (P.nHeavy + mxk::kBlock / 16 - 1) / (mxk::kBlock / 16);
-    static int dbg = -1;
-    if (dbg < 0) dbg = getenv("MX_DBG_COMBINE") ? atoi(getenv("MX_DBG_COMBINE")) : 0;
-    const int xr = (dbg & 1) ? 0 : P.rows, xl = (dbg & 2) ? 0 : P.nLight, xh = (dbg & 4) ? 0 : P.nHeavy;
-    if (dbg) {
-        const int a = (dbg & 1) ? 0 : nRowWG, b = (dbg & 2) ? 0 : nLightWG, c = (dbg & 4) ? 0 : nHeavyWG;
-        if (a + b + c == 0) return hipSuccess;
-        hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(a + b + c), dim3(mxk::kBlock), 0, s,
-                       (const AT *)P.partial, P.rowInfo, xr, a, (const int4 *)P.lightInfo, xl, b,
-                       (const int4 *)P.heavyInfo, xh, P.segIdx, (VT *)y, (accumulate || P.subset) ? 1 : 0,
-                       P.subset ? 1 : 0);
-        return hipGetLastError();
-    }
     if (nRowWG + nLightWG + nHeavyWG == 0) return hipSuccess;
     hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(nRowWG + nLightWG + nHeavyWG), dim3(mxk::kBlock), 0, s,
                        (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, (const int4 *)P.lightInfo, P.nLight, nLightWG,
