@@ -374,6 +374,48 @@ def test_slice_kernel_layouts(mx, ora):
         part.close()
 
 
+@pytest.mark.parametrize("variant", ["slices", "split"])
+def test_slice_kernel_virtual_rows(mx, ora, variant, monkeypatch):
+    """Rows of very different lengths through the slice kernel: mostly single entries (their sums
+    are fetched one per row), some rows without entries, a few rows so long that they are cut at
+    the cap and spread over every slice (summed by sixteen lanes), rows in between (one lane).
+    `split` keeps the short rows on row tiles and adds the long rows' sums to what those wrote."""
+    import torch
+    monkeypatch.setenv("MX_CSR_KERNEL", variant)
+    monkeypatch.setenv("MX_SPLIT_LEN", "24")
+    rng = np.random.default_rng(23)
+    for rows, cols, dtype in ((6000, 300001, np.float16), (5000, 120003, np.float64), (4100, 70000, np.float16)):
+        lens = np.ones(rows, np.int64)
+        lens[rng.uniform(size=rows) < 0.1] = 0
+        mid = rng.choice(rows, rows // 20, replace=False)
+        lens[mid] = rng.integers(2, 200, mid.size)
+        longr = rng.choice(rows, 24, replace=False)
+        lens[longr] = rng.integers(3000, 9000, longr.size)
+        lens[-1] = 5000   # the last row is long, the first is empty
+        lens[0] = 0
+        A = _random_csr(mx, rng, rows, cols, lens, dtype)
+        x = rng.uniform(-1, 1, cols).astype(dtype)
+        ref = oracle_y(ora, mx, A, x)
+        tol = F64_TOL if dtype == np.float64 else F16_TOL
+        print("virtual rows %s rows=%d cols=%d dtype=%s" % (variant, rows, cols, dtype.__name__), flush=True)
+        part = mx.Partition(A, 0.0, 0.0)
+        plan = mx.Plan(part)
+        assert plan.info["csr_variant"] == (1 if variant == "slices" else 2)
+        assert plan.info["csr_main_kernel"] == 1 and plan.info["csr_main_nnz"] <= A.nnz
+        xd = torch.from_numpy(x).cuda()
+        y = torch.full((rows,), 7.0, dtype=xd.dtype, device="cuda")   # what y held before must not matter
+        plan.spmv(xd, y)
+        torch.cuda.synchronize()
+        assert rel_l2(y.cpu().numpy(), ref) <= tol
+        got = y.cpu().numpy().astype(np.float64)
+        assert np.all(got[lens == 0] == 0.0)
+        y2 = plan.spmv(xd, y)
+        torch.cuda.synchronize()
+        assert np.array_equal(y2.cpu().numpy().view(np.uint8), got.astype(dtype).view(np.uint8)), "not reproducible"
+        plan.close()
+        part.close()
+
+
 def test_tile_kernel_step_packing(mx, ora):
     """Chunks with one fragment, with exactly half a step, a whole step, more than a step and a
     ragged last chunk; every fill from almost empty to full, through the fragment gate and
