@@ -73,9 +73,10 @@ inline int tile_slot(mx_dtype d, int half, int i) { return d == MX_F64 ? 2 * i +
 // Chunks are numbered workgroup by workgroup, wave by wave; virtual row v = 64 * chunk + lane
 // puts its sum into partial[v], and a second kernel turns those into y: rowInfo[r] is the
 // virtual row of a matrix row that owns exactly one, -1 for a row that owns none, -2 for a row
-// that owns several; those list theirs in segIdx -- lightInfo / heavyInfo hold {row, first index
-// into segIdx, count, 0} for the rows with up to kSliceLightSegs virtual rows and for those with
-// more.
+// that owns several.  Of those, the rows with up to kSliceLightSegs virtual rows are lightRow[i]
+// with their virtual rows in lightIdx[i][kSliceLightSegs] (-1 = none); the rows with more are
+// heavyInfo[i] = {row, first index into segIdx, count, 0} with their virtual rows listed in
+// segIdx.
 struct DeviceSlices {
     int nWG = 0, S = 0, rows = 0, cols = 0, sliceCols = 0;
     int maxWgChunks = 0;              // chunks of the largest workgroup (their ends are kept in LDS)
@@ -92,7 +93,8 @@ struct DeviceSlices {
     void *partial = nullptr;          // [chunks*64] accumulators
     int *rowInfo = nullptr;           // [rows, padded to a multiple of 4 with -2]
     int *segIdx = nullptr;            // [vrows of rows with several]
-    int *lightInfo = nullptr;         // [nLight][4]
+    int *lightRow = nullptr;          // [nLight]
+    int *lightIdx = nullptr;          // [nLight][kSliceLightSegs]
     int *heavyInfo = nullptr;         // [nHeavy][4]
     int nLight = 0, nHeavy = 0;
 };

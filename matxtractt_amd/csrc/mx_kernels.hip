@@ -597,14 +597,16 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 //  * the first `nRowWG` walk the matrix rows, kCombineRows per lane: rowInfo[r] >= 0 names the one virtual
 //    row of row r, whose sum is the row's result; -1 is a row without entries (zero, or left
 //    alone when `skipEmpty`); anything else a row that the lists below cover;
-//  * the next `nLightWG` take the rows with 2..kSliceLightSegs virtual rows, one lane each:
-//    {row, first index into segIdx, count};
+//  * the next `nLightWG` take the rows with 2..kSliceLightSegs virtual rows, one lane each: the
+//    row and its kSliceLightSegs indices into `partial` (-1 = none) lie at the lane's own place in
+//    two arrays, so nothing the lane loads depends on another load but the sums themselves;
 //  * the rest take the rows with more, sixteen lanes each.
 constexpr int kCombineRows = 16;  // rows a lane of the first kind takes
 template <typename VT>
 __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Acc<VT>::type *__restrict__ partial,
                                                               const int *__restrict__ rowInfo, int rows, int nRowWG,
-                                                              const int4 *__restrict__ lightInfo, int nLight, int nLightWG,
+                                                              const int *__restrict__ lightRow,
+                                                              const int4 *__restrict__ lightIdx, int nLight, int nLightWG,
                                                               const int4 *__restrict__ heavyInfo, int nHeavy,
                                                               const int *__restrict__ segIdx, VT *__restrict__ y,
                                                               int accumulate, int skipEmpty)
@@ -637,15 +639,15 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
     if (b < nLightWG) {
         const int i = b * kBlock + tid;
         if (i >= nLight) return;
-        const int4 h = lightInfo[i];
-        int id[mx::kSliceLightSegs];
+        static_assert(mx::kSliceLightSegs == 8, "two int4 of indices per light row");
+        const int r = lightRow[i];
+        const int4 i0 = lightIdx[2 * i], i1 = lightIdx[2 * i + 1];
+        const int id[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
+        AT sum = accumulate ? (AT)y[r] : (AT)0;
 #pragma unroll
-        for (int k = 0; k < mx::kSliceLightSegs; ++k) id[k] = k < h.z ? segIdx[h.y + k] : -1;
-        AT sum = accumulate ? (AT)y[h.x] : (AT)0;
-#pragma unroll
-        for (int k = 0; k < mx::kSliceLightSegs; ++k)
+        for (int k = 0; k < 8; ++k)
             if (id[k] >= 0) sum += partial[id[k]];
-        y[h.x] = (VT)sum;
+        y[r] = (VT)sum;
         return;
     }
     b -= nLightWG;
@@ -917,7 +919,7 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     const int nHeavyWG = (P.nHeavy + mxk::kBlock / 16 - 1) / (mxk::kBlock / 16);
     if (nRowWG + nLightWG + nHeavyWG == 0) return hipSuccess;
     hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(nRowWG + nLightWG + nHeavyWG), dim3(mxk::kBlock), 0, s,
-                       (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, (const int4 *)P.lightInfo, P.nLight, nLightWG,
+                       (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, P.lightRow, (const int4 *)P.lightIdx, P.nLight, nLightWG,
                        (const int4 *)P.heavyInfo, P.nHeavy, P.segIdx, (VT *)y, (accumulate || P.subset) ? 1 : 0,
                        P.subset ? 1 : 0);
     return hipGetLastError();

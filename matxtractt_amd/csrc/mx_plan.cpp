@@ -103,7 +103,8 @@ void free_slices(mx::DeviceSlices &P)
     (void)hipFree(P.eval);
     (void)hipFree(P.partial);
     (void)hipFree(P.rowInfo);
-    (void)hipFree(P.lightInfo);
+    (void)hipFree(P.lightRow);
+    (void)hipFree(P.lightIdx);
     (void)hipFree(P.heavyInfo);
     (void)hipFree(P.segIdx);
     P = mx::DeviceSlices();
@@ -409,7 +410,18 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
     if ((rc = upload_bytes(&D.partial, nullptr, 0, ((size_t)H.chunks * 64 + 64) * (dtype == MX_F64 ? 8 : 4)))) return rc;
     if ((rc = upload(&D.rowInfo, H.rowInfo.data(), H.rowInfo.size()))) return rc;
     if ((rc = upload(&D.segIdx, H.segIdx.data(), H.segIdx.size()))) return rc;
-    if ((rc = upload(&D.lightInfo, H.lightInfo.data(), H.lightInfo.size(), 4))) return rc;
+    {
+        // the light rows' virtual rows, eight places per row
+        const int nL = (int)H.lightInfo.size() / 4;
+        std::vector<int> lr((size_t)nL), li((size_t)nL * mx::kSliceLightSegs, -1);
+        for (int i = 0; i < nL; ++i) {
+            lr[i] = H.lightInfo[4 * (size_t)i];
+            const int a = H.lightInfo[4 * (size_t)i + 1], n = H.lightInfo[4 * (size_t)i + 2];
+            for (int k = 0; k < n; ++k) li[(size_t)i * mx::kSliceLightSegs + k] = H.segIdx[a + k];
+        }
+        if ((rc = upload(&D.lightRow, lr.data(), lr.size(), 1))) return rc;
+        if ((rc = upload(&D.lightIdx, li.data(), li.size(), 8))) return rc;
+    }
     if ((rc = upload(&D.heavyInfo, H.heavyInfo.data(), H.heavyInfo.size(), 4))) return rc;
     return MX_OK;
 }
