@@ -792,9 +792,10 @@ static int split_length()
 // Puts the CSR part on the device.  Three executable forms exist: row tiles with direct x
 // gathers; column slices with x resident in LDS; and a split in which the long rows (most of
 // the entries of a matrix with a heavy tail of row lengths) take the slices and the many short
-// ones the row tiles.  Unless a flag or MX_CSR_KERNEL=rows|slices|split forces one, every form
-// the matrix suits is built in turn and timed on the spot with a few launches, and the fastest
-// is kept.
+// ones the row tiles.  Unless a flag or MX_CSR_KERNEL=rows|slices|split forces one, the first
+// two are built in turn (the second when the matrix suits it) and timed on the spot with a few
+// launches, and the faster is kept.  The split runs only when asked for: it has not won on any
+// matrix measured so far and building it makes a plan half as slow again.
 static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags)
 {
     const int rows = plan->rows, cols = plan->cols;
@@ -802,7 +803,7 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
     const size_t es = (size_t)mx::elem_size(plan->dtype);
     plan->csr_nnz = nnz;
     const char *env = std::getenv("MX_CSR_KERNEL");
-    bool want[3] = {true, true, true};
+    bool want[3] = {true, true, false};
     if (flags & MX_PLAN_CSR_ROWS) want[1] = want[2] = false;
     if (flags & MX_PLAN_CSR_SLICES) want[0] = want[2] = false;
     if (env && !std::strcmp(env, "rows")) want[0] = true, want[1] = want[2] = false;

@@ -398,6 +398,38 @@ def test_slice_layout_walk(mx, ora, case):
     assert np.all(nv <= -(-lens // 1) ) and L["cap"] % L["batchEntries"] == 0
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_slice_layout_walk_random_shapes(mx, seed):
+    """Random shapes, precisions, machine sizes and row subsets through the same walk."""
+    rng = np.random.default_rng(100 + seed)
+    f64 = bool(seed % 2)
+    rows = int(rng.integers(1, 3000))
+    cols = int(rng.integers(1, 5 * (16384 if f64 else 65536)))
+    kind = seed % 3
+    if kind == 0:
+        lens = rng.integers(0, 60, rows)
+    elif kind == 1:
+        lens = np.minimum(cols, np.floor(1.5 * rng.uniform(1e-4, 1, rows) ** (-1 / 0.6)).astype(np.int64))
+    else:
+        lens = (rng.uniform(size=rows) < 0.3).astype(np.int64)
+        lens[rng.integers(0, rows)] = min(cols, 20000)
+    lens = np.minimum(lens, cols)
+    rp = np.zeros(rows + 1, np.int32)
+    rp[1:] = np.cumsum(lens)
+    ci = np.concatenate([rng.choice(cols, n, replace=False) for n in lens] + [np.zeros(0, np.int64)]).astype(np.int32)
+    dt = np.float64 if f64 else np.float16
+    A = mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, len(ci)).astype(dt))
+    x = rng.uniform(-1, 1, cols).astype(dt).astype(np.float64)
+    sel = (rng.uniform(size=rows) < 0.5).astype(np.uint8) if seed >= 3 else None
+    L = mx.slice_layout(A, nCU=int(rng.integers(1, 40)), sel=sel)
+    y, _ = _walk_slice_layout(L, x, f64, subset=sel is not None)
+    keep = np.ones(rows, bool) if sel is None else sel.astype(bool)
+    ref = np.zeros(rows)
+    np.add.at(ref, np.repeat(np.arange(rows), lens), A.val.astype(np.float64) * x[A.colInd])
+    ref[~keep] = 0.0
+    assert np.allclose(y, ref, rtol=1e-12, atol=1e-12 * max(1.0, np.abs(ref).max(initial=0.0)))
+
+
 def test_init_vec(mx):
     v = mx.init_vec(40)
     assert np.array_equal(v, np.arange(40) % 15)
