@@ -189,6 +189,23 @@ int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters,
  * without its combine kernel), same protocol as mx_time: the figure a roofline is priced on. */
 int mx_time_csr_main(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters, double *ms);
 
+/* Choice of (tau_c, tau_r) for a matrix on this device.  The reference tunes the two fractions
+ * per matrix by running its CLI once per candidate and reading "MatXtract time" back
+ * (ML/bayes_opt.py:22-84: candidates with hot_frac > col_frac are rejected, :37-38); here the
+ * candidates are the `levels` x `levels` grid {0, 1/(levels-1), .. 1}^2 with tau_c >= tau_r, each
+ * one partitioned, planned (with `flags`) and timed on the device with the protocol of mx_time
+ * (`warm` untimed and `iters` timed back-to-back products of a seeded x).  Candidates that send
+ * nothing to the tile kernel are one and the same plan and are timed once, as (0, 0).
+ * Returns the fastest in tau_c/tau_r; when `table` is given, up to `cap` candidates are written
+ * to it in grid order (tau_c outer, ascending) and *n_points is set to their number. */
+typedef struct mx_tau_point {
+    float tau_c, tau_r;
+    double ms_total;  /* mean ms per product */
+    int tile_nnz;     /* entries the tile kernel holds at this point */
+} mx_tau_point;
+int mx_tune_tau(const mx_csr *A, int levels, int flags, int warm, int iters, float *tau_c, float *tau_r,
+                mx_tau_point *table, int cap, int *n_points);
+
 /* Facts about a plan, for reporting. */
 typedef struct mx_plan_info {
     mx_dtype dtype;

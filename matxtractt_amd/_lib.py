@@ -62,6 +62,10 @@ class SliceLayoutView(C.Structure):
                                         "heavyInfo", "ecol", "eval")]
 
 
+class TauPoint(C.Structure):
+    _fields_ = [("tau_c", C.c_float), ("tau_r", C.c_float), ("ms_total", C.c_double), ("tile_nnz", C.c_int)]
+
+
 # Every symbol include/matxtract_hip.h declares: name -> (restype, argtypes)
 _vp, _i, _d = C.c_void_p, C.c_int, C.c_double
 _pp = C.POINTER(C.c_void_p)
@@ -91,6 +95,8 @@ SIGNATURES = {
     "mx_time": (_i, [_vp, _vp, _vp, _i, _i, _pd, _pd, _pd]),
     "mx_time_csr_main": (_i, [_vp, _vp, _vp, _i, _i, _pd]),
     "mx_plan_get_info": (_i, [_vp, C.POINTER(PlanInfo)]),
+    "mx_tune_tau": (_i, [C.POINTER(CsrStruct), _i, _i, _i, _i, C.POINTER(C.c_float), C.POINTER(C.c_float),
+                         C.POINTER(TauPoint), _i, _pi]),
     "mx_slice_layout": (_i, [C.POINTER(CsrStruct), _i, _vp, C.POINTER(SliceLayoutView)]),
     "mx_slice_layout_free": (None, [C.POINTER(SliceLayoutView)]),
     "mx_cdspmv_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _pd, _pd]),

@@ -15,7 +15,7 @@ from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLA
                    MX_PLAN_NO_TILES, MxError, check)
 
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "cdspmv",
-           "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "MxError",
+           "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
            "MX_PLAN_CSR_SLICES"]
 
@@ -218,6 +218,18 @@ def slice_layout(A, nCU=256, sel=None):
     finally:
         _lib.load().mx_slice_layout_free(C.byref(v))
     return out
+
+
+def tune_tau(A, levels=5, flags=MX_PLAN_DEFAULT, warm=20, iters=200):
+    """(tau_c, tau_r, table) for matrix A on this device: every grid point with tau_c >= tau_r is
+    partitioned, planned and timed (mx_tune_tau); table = [(tau_c, tau_r, ms, tile_nnz), ...]."""
+    st = A.struct()
+    cap = levels * (levels + 1) // 2
+    table = (_lib.TauPoint * cap)()
+    c, r, n = C.c_float(), C.c_float(), C.c_int()
+    check(_lib.load().mx_tune_tau(C.byref(st), int(levels), int(flags), int(warm), int(iters), C.byref(c), C.byref(r),
+                                  table, cap, C.byref(n)))
+    return c.value, r.value, [(t.tau_c, t.tau_r, t.ms_total, t.tile_nnz) for t in table[:n.value]]
 
 
 def _torch_dtype(dt):

@@ -7,7 +7,8 @@
 // Additive options: --scale S (shrink a synthetic workload), --seed S, --keep-values (do not
 // overwrite the file's values with i%15 as the reference does at :1091), --warm W --iters K
 // (default 200 / 4000), --no-tiles / --all-tiles (plan flags), --json (one JSON record on the
-// last line), --partition-cache FILE (read the partition from FILE when it was made for a
+// last line), --tune (pick the two fractions from the 5x5 grid by timing each on the device,
+// then run with them), --partition-cache FILE (read the partition from FILE when it was made for a
 // matrix of this shape with these fractions, otherwise compute it and write FILE).  Precision is the build's: -Dfp64 -> FP64 binary, otherwise FP16.
 //
 // Lines other tools parse (ML/bayes_opt.py:64, script/duse.sh:35-38) keep their form:
@@ -92,7 +93,7 @@ int main(int argc, char **argv)
     int config = 0, warm = 200, iters = 4000, planFlags = MX_PLAN_DEFAULT;
     double scale = 1.0;
     unsigned long long seed = 0;
-    bool keepValues = false, json = false;
+    bool keepValues = false, json = false, tune = false;
     std::string cachePath;
     for (int i = 1; i < argc; ++i) {
         std::string a = argv[i];
@@ -113,6 +114,7 @@ int main(int argc, char **argv)
         else if (a == "--all-tiles") planFlags = MX_PLAN_ALL_TILES;
         else if (a == "--json") json = true;
         else if (a == "--partition-cache") cachePath = next("--partition-cache");
+        else if (a == "--tune") tune = true;
         else pos.push_back(a);
     }
     const size_t npos = pos.size() + (config ? 1 : 0);  // a --config stands for the file name
@@ -172,6 +174,23 @@ int main(int argc, char **argv)
         initVec(X_val, colA);  // :1433-1434
     }
 
+    if (tune) {
+        // the two fractions chosen on the device instead of given (what ML/bayes_opt.py does around this program)
+        mx_csr A{rowA, colA, (int)nnzA, MX_VALT_DTYPE, csrRowPtr, csrColInd, csrVal};
+        mx_tau_point table[15];
+        float tc = 0.f, tr = 0.f;
+        int n = 0;
+        if (mx_tune_tau(&A, 5, planFlags, 20, 200, &tc, &tr, table, 15, &n) != MX_OK) {
+            printf("Error: %s\n", mx_last_error());
+            return 1;
+        }
+        for (int i = 0; i < n && i < 15; ++i)
+            printf("tune: col_frac = %.2f hot_frac = %.2f time = %lf ms tile_nnz = %d\n", table[i].tau_c, table[i].tau_r,
+                   table[i].ms_total, table[i].tile_nnz);
+        printf("tuned: col_frac = %.2f hot_frac = %.2f\n", tc, tr);
+        col_frac = tc;
+        hot_frac = tr;
+    }
     const float colProp = (float)col_frac, rowProp = (float)hot_frac;
     const bool extracting = !((rowProp == 0.0) && (colProp == 0.0));
     if (extracting) {

@@ -1178,6 +1178,78 @@ extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, 
     return MX_OK;
 }
 
+extern "C" int mx_tune_tau(const mx_csr *A, int levels, int flags, int warm, int iters, float *tau_c, float *tau_r,
+                           mx_tau_point *table, int cap, int *n_points)
+{
+    if (!A || levels < 2 || levels > 65 || warm < 0 || iters <= 0 || !tau_c || !tau_r || (table && cap < 0)) {
+        set_error("mx_tune_tau: bad argument");
+        return MX_ERR_ARG;
+    }
+    int rc = need_device();
+    if (rc) return rc;
+    const size_t es = (size_t)mx::elem_size(A->dtype);
+    void *dx = nullptr, *dy = nullptr;
+    {
+        // x as the reference's driver fills it (initVec, include/common.h:237-245)
+        std::vector<unsigned char> hx(std::max<size_t>((size_t)A->cols * es, 16));
+        mx_init_vec(A->dtype, hx.data(), A->cols);
+        if ((rc = upload_bytes(&dx, hx.data(), hx.size()))) return rc;
+        if ((rc = upload_bytes(&dy, nullptr, 0, std::max<size_t>((size_t)A->rows * es, 16)))) {
+            (void)hipFree(dx);
+            return rc;
+        }
+    }
+    double best = 0.0, csrOnly = -1.0;
+    bool have = false;
+    int n = 0;
+    rc = MX_OK;
+    for (int ic = 0; ic < levels && !rc; ++ic)
+        for (int ir = 0; ir <= ic && !rc; ++ir) {
+            const float c = (float)ic / (float)(levels - 1), r = (float)ir / (float)(levels - 1);
+            mx_partition *P = nullptr;
+            mx_plan *plan = nullptr;
+            double ms = 0.0;
+            int tileNnz = 0;
+            if ((rc = mx_partition_create(A, c, r, &P))) break;
+            // entries the plan would hand to the tile kernel
+            bool anyTile = false;
+            if (P->extracted && !(flags & MX_PLAN_NO_TILES)) {
+                const double gate = tile_gate(P->dtype) * P->fragM * P->fragK;
+                const int nFrags = P->chunkPtr[P->chunkNum];
+                for (int f = 0; f < nFrags && !anyTile; ++f) {
+                    const int vals = P->fragPtr[f + 1] - P->fragPtr[f];
+                    anyTile = (flags & MX_PLAN_ALL_TILES) ? vals > 0 : (vals > 0 && (double)vals >= gate);
+                }
+            }
+            if (!anyTile && csrOnly >= 0.0) {
+                ms = csrOnly;  // the same plan as an earlier candidate
+            } else {
+                rc = mx_plan_create(P, flags, &plan);
+                if (!rc) rc = mx_time(plan, dx, dy, warm, iters, &ms, nullptr, nullptr);
+                if (!rc) {
+                    tileNnz = plan->tile_nnz;
+                    if (!anyTile) csrOnly = ms;
+                }
+                mx_plan_destroy(plan);
+            }
+            mx_partition_destroy(P);
+            if (rc) break;
+            if (table && n < cap) table[n] = mx_tau_point{c, r, ms, tileNnz};
+            ++n;
+            // a candidate without tiles never displaces an equally fast earlier one: ties go to (0, 0)
+            if (!have || ms < best) {
+                best = ms;
+                *tau_c = anyTile ? c : 0.0f;
+                *tau_r = anyTile ? r : 0.0f;
+                have = true;
+            }
+        }
+    (void)hipFree(dx);
+    (void)hipFree(dy);
+    if (n_points) *n_points = n;
+    return rc;
+}
+
 // ---- reference surface: host pointers in, host pointers out ------------------------------
 
 static int cdspmv_any(mx_dtype dtype, const void *csrVal, const int *csrRowPtr, const int *csrColInd, const void *x,

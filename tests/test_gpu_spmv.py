@@ -479,6 +479,29 @@ def test_plan_from_a_saved_partition(mx, ora, tmp_path):
         Q.close()
 
 
+def test_tau_tuner(mx, ora):
+    """mx_tune_tau walks the grid with tau_c >= tau_r, reports every candidate, returns the fastest;
+    candidates without tiles share one timing and are reported as (0, 0)."""
+    import torch
+    A, x = mx.gen_config(5, scale=1 / 128)
+    tc, tr, table = mx.tune_tau(A, levels=3, warm=2, iters=10)
+    assert [(c, r) for c, r, _, _ in table] == [(0.0, 0.0), (0.5, 0.0), (0.5, 0.5), (1.0, 0.0), (1.0, 0.5), (1.0, 1.0)]
+    assert all(ms > 0 for _, _, ms, _ in table)
+    no_tiles = [ms for _, _, ms, n in table if n == 0]
+    assert len(set(no_tiles)) == 1, "candidates without tiles are one plan"
+    best = min(table, key=lambda t: t[2])
+    assert (tc, tr) == ((best[0], best[1]) if best[3] > 0 else (0.0, 0.0))
+    assert any(n > 0 for _, _, _, n in table), "the strips of this workload fill whole fragments"
+    P = mx.Partition(A, tc, tr)
+    plan = mx.Plan(P)
+    y = plan.spmv(torch.from_numpy(x).cuda()).cpu().numpy()
+    assert rel_l2(y, oracle_y(ora, mx, A, x)) <= F16_TOL
+    plan.close()
+    P.close()
+    with pytest.raises(mx.MxError):
+        mx.tune_tau(A, levels=1)
+
+
 def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
     """matxtract_perftest's stdout keeps the forms the reference's scripts grep for."""
     import re
@@ -494,6 +517,10 @@ def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
         for r in range(A.rows):
             for q in range(A.rowPtr[r], A.rowPtr[r + 1]):
                 f.write("%d %d %.17g\n" % (r + 1, A.colInd[q] + 1, A.val[q]))
+    out = subprocess.run([exe, "--warm", "2", "--iters", "5", "--tune", str(p)], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert len(re.findall(r"tune: col_frac = ", out.stdout)) == 15 and re.search(r"tuned: col_frac = \d\.\d\d hot_frac = \d\.\d\d", out.stdout)
+    assert "Success! All values match" in out.stdout
     for args in (["0.5", "0.25", str(p)], [str(p)]):
         out = subprocess.run([exe, "--warm", "2", "--iters", "5", *args], capture_output=True, text=True, timeout=120)
         assert out.returncode == 0, out.stderr
