@@ -2,8 +2,9 @@
 //
 //   csr_rows_kernel    residual / plain CSR part, x gathered from memory (stands in for
 //                      cdspmv_kernel, src/spmv_kernel/cdSpMV.cu:244-392).
-//   csr_slice_kernel   the same part with x resident in LDS, for matrices with a small x and
-//   slice_combine_kernel   scattered columns; the second adds the per-slice partial sums.
+//   csr_slice_kernel   the same part with a slice of x resident in LDS, for matrices with
+//   slice_combine_kernel   scattered columns: rows are cut at the slice borders into "virtual
+//                      rows", the first kernel sums those, the second adds up each row's.
 //   tile_kernel<double>    8x4 tiles through v_mfma_f64_16x16x4_f64 (stands in for
 //                      tcspmv_kernel_fp64, src/spmv_kernel/du_tcSpMV_fp64.cu:81-160).
 //   tile_kernel<_Float16>  8x8 tiles through v_mfma_f32_16x16x32_f16, f32 accumulation
