@@ -500,7 +500,9 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     VT *xs = (VT *)smem;                                           // [sliceCols]
     int *endsL = (int *)(smem + (size_t)sliceCols * sizeof(VT));   // [chunks of the workgroup]
 
-    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    // the workgroups of a slice are numbered consecutively: with every XCD on one contiguous range
+    // of them a slice of x is fetched into one L2, not into all eight
+    const int b = xcd_contiguous_block(blockIdx.x, gridDim.x), tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int4 gd = wgDesc[b];
     const int4 d = waveDesc[b * kSliceWaves + wave];
@@ -614,7 +616,14 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
 {
     typedef typename Acc<VT>::type AT;
     const int tid = threadIdx.x;
+    // Every kind of workgroup walks its rows in ascending order, and the sums of neighbouring rows
+    // lie close together wherever their virtual rows fall into the same slice and length class:
+    // one XCD per contiguous range of rows keeps those sectors in a single L2.
     int b = blockIdx.x;
+    const int nHeavyWG = (int)gridDim.x - nRowWG - nLightWG;
+    if (b < nRowWG) b = xcd_contiguous_block(b, nRowWG);
+    else if (b < nRowWG + nLightWG) b = nRowWG + xcd_contiguous_block(b - nRowWG, nLightWG);
+    else b = nRowWG + nLightWG + xcd_contiguous_block(b - nRowWG - nLightWG, nHeavyWG);
     if (b < nRowWG) {
         // kCombineRows rows per lane, as quads a wave apart so that its loads and stores stay contiguous
         int dd[kCombineRows];
