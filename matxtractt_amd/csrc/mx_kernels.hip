@@ -752,7 +752,9 @@ __global__ __launch_bounds__(kBlock) void tile_kernel(const int4 *__restrict__ w
     };
     __shared__ __attribute__((aligned(16))) Park park[kBlock / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int gw = blockIdx.x * (kBlock / 64) + wave;
+    // waves follow the chunks in order, and neighbouring chunks share columns of x and lines of
+    // y: every XCD takes one contiguous range of them
+    const int gw = xcd_contiguous_block(blockIdx.x, gridDim.x) * (kBlock / 64) + wave;
     if (gw >= nWaves) return;
     Park &P = park[wave];
     const int4 d0 = waveDesc[2 * gw], d1 = waveDesc[2 * gw + 1];
