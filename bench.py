@@ -30,10 +30,10 @@ GRID = (0.0, 0.25, 0.5, 0.75, 1.0)
 # hold the counter values.  (workload, kernel) -> bytes
 TRAFFIC = {
     (2, "csr_rows_kernel<f64>"): 47165962,
-    (2, "csr_slice_kernel<f64>"): 52090074,
+    (2, "csr_slice_kernel<f64>"): 48810843,
     (3, "csr_rows_kernel<f64>"): 287435306,
-    (4, "csr_slice_kernel<f16>"): 70527078,
-    (5, "csr_slice_kernel<f16>"): 326496189,
+    (4, "csr_slice_kernel<f16>"): 55698523,
+    (5, "csr_slice_kernel<f16>"): 301473538,
 }
 WORKLOADS = {
     1: "configs[0]: FP64 random 4096x4096, 16 nnz/row",
