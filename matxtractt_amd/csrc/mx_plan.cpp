@@ -638,6 +638,20 @@ extern "C" int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *se
         return MX_ERR_ARG;
     }
     std::memset(out, 0, sizeof(*out));
+    if (A->rowPtr[0] != 0 || A->rowPtr[A->rows] != A->nnz) {
+        set_error("mx_slice_layout: rowPtr does not span [0, nnz]");
+        return MX_ERR_ARG;
+    }
+    for (int r = 0; r < A->rows; ++r)
+        if (A->rowPtr[r + 1] < A->rowPtr[r]) {
+            set_error("mx_slice_layout: rowPtr is not ascending");
+            return MX_ERR_ARG;
+        }
+    for (int p = 0; p < A->nnz; ++p)
+        if ((unsigned)A->colInd[p] >= (unsigned)A->cols) {
+            set_error("mx_slice_layout: column index out of range");
+            return MX_ERR_ARG;
+        }
     const int S = (A->cols + mx::slice_cols(A->dtype) - 1) / mx::slice_cols(A->dtype);
     HostSlices H;
     try {

@@ -398,6 +398,25 @@ def test_slice_layout_walk(mx, ora, case):
     assert np.all(nv <= -(-lens // 1) ) and L["cap"] % L["batchEntries"] == 0
 
 
+def test_slice_layout_rejects_bad_matrices(mx):
+    rp = np.array([0, 2, 3], np.int32)
+    good = mx.Csr(2, 4, rp, np.array([0, 3, 1], np.int32), np.ones(3))
+    assert mx.slice_layout(good, nCU=4)["vrows"] == 2          # both rows lie in one slice: one virtual row each
+    for bad_cols in (np.array([0, 4, 1], np.int32), np.array([0, -1, 1], np.int32)):
+        A = mx.Csr.__new__(mx.Csr)
+        A.__dict__.update(good.__dict__)
+        A.colInd = bad_cols
+        with pytest.raises(mx.MxError, match="column index"):
+            mx.slice_layout(A, nCU=4)
+    A = mx.Csr.__new__(mx.Csr)
+    A.__dict__.update(good.__dict__)
+    A.rowPtr = np.array([0, 3, 2], np.int32)
+    with pytest.raises(mx.MxError, match="rowPtr"):
+        mx.slice_layout(A, nCU=4)
+    with pytest.raises(mx.MxError):
+        mx.slice_layout(good, nCU=0)
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_slice_layout_walk_random_shapes(mx, seed):
     """Random shapes, precisions, machine sizes and row subsets through the same walk."""
