@@ -162,7 +162,9 @@ void mx_plan_destroy(mx_plan *plan);
 
 /* y = A*x on the device.  x [cols] and y [rows] are DEVICE pointers of the plan's value
  * type, x 16-byte aligned (the kernels copy it in 16-byte vectors; a plan whose CSR part keeps
- * x in LDS returns MX_ERR_ARG otherwise); `stream` is a hipStream_t (NULL = default stream).
+ * x in LDS returns MX_ERR_ARG otherwise, and reads the last 16-byte block of x whole when cols is
+ * not a multiple of the vector -- the bytes past x[cols-1] in that block are read, never used);
+ * `stream` is a hipStream_t (NULL = default stream).
  * Asynchronous.  The hybrid sequence of test/test_autotc_spmv.cpp:1507-1559 (tile part, scatter
  * through rId, residual accumulated on top) without host round trips.  A plan holds device
  * buffers of partial sums: calls on the same plan must not overlap in time. */
