@@ -65,8 +65,9 @@ inline int tile_slot(mx_dtype d, int half, int i) { return d == MX_F64 ? 2 * i +
 // virtual row per lane (a sliced-ELL layout: every row of a chunk is padded to the chunk's
 // longest, and the sort keeps that padding small).  A slice gets workgroups in proportion to
 // its entries, its chunks are dealt to them longest first, and inside a workgroup to its waves
-// the same way.  A lane walks its virtual row one entry -- one "step" -- at a time; a wave's chunks follow each other in
-// the wave's stream, which is stored in batches of kSliceBatchEntries entries per lane
+// the same way.  A lane walks its virtual row one entry -- one "step" -- at a time; a wave's
+// chunks follow each other in the wave's stream, which is stored in batches of
+// kSliceBatchEntries entries per lane
 // (zero-padded to a whole batch at the end): per batch the lanes' column offsets (lanes
 // contiguous), then their values -- binary16: lanes contiguous; binary64: one sub-block of 16
 // bytes (two values) per lane -- so that every load of a wave is one contiguous stretch.
@@ -92,7 +93,7 @@ struct DeviceSlices {
     void *eval = nullptr;             // [batches] values, laid out as described above
     void *partial = nullptr;          // [chunks*64] accumulators
     int *rowInfo = nullptr;           // [rows, padded to a multiple of 4 with -2]
-    int *segIdx = nullptr;            // [vrows of rows with several]
+    int *segIdx = nullptr;            // [vrows] virtual rows listed matrix row by matrix row
     int *lightRow = nullptr;          // [nLight]
     int *lightIdx = nullptr;          // [nLight][kSliceLightSegs]
     int *heavyInfo = nullptr;         // [nHeavy][4]
