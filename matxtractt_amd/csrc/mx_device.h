@@ -29,7 +29,10 @@ int csr_entries_per_lane(mx_dtype dtype);
 // selects are expanded from the reference's encoding (bitmap + packed values) into full
 // fragM x fragK blocks, zeros included (row-major inside a block), so that a lane can load
 // exactly what the matrix core wants from it with no decoding; the plan only selects fragments
-// that are mostly full.  The blocks are grouped into "steps" -- what one wave feeds to the
+// that are mostly full.  The columns of a chunk's selected fragments are first put in ascending
+// order of the caller's column ids and cut into blocks anew (the reference orders them by their
+// rank among the dense columns, which scatters neighbours): gathers touch fewer lines, and dense
+// strips become blocks of consecutive columns.  The blocks are grouped into "steps" -- what one wave feeds to the
 // matrix core at a time: two halves of up to kTileSlots(dtype)/2 blocks.  A chunk with more
 // selected fragments than half a step takes whole steps of its own (filling half 0 first; its
 // two halves are added at the end); smaller chunks share a step, one per half.  Per step:
@@ -37,7 +40,8 @@ int csr_entries_per_lane(mx_dtype dtype);
 //          (-1 = none); [16] flags (1 = store the sums after this step, 2 = the halves are
 //          different chunks); [17],[18] blocks in half 0 and half 1; [19],[20] first value
 //          and blocks in half 0 of the step four further on (a wave learns where to prefetch
-//          from there; its own last step when it has no such step).
+//          from there; its own last step when it has no such step); [21,29) first column of
+//          the block in each slot (-1 = none), used by the strip form of the binary16 kernel.
 //   atox   64 column ids (slot-major), -1 for unused ones
 //   values the blocks of half 0, then those of half 1; nothing for absent blocks.
 // Waves take whole chunks: waveDesc = {first step, end step, first value of the wave's first
@@ -47,6 +51,10 @@ struct DeviceTiles {
     int frags = 0, vals = 0;   // selected fragments, entries they hold
     long long stored = 0;      // values stored (zeros included)
     int steps = 0, nWaves = 0;
+    bool dense = false;        // binary16 chunks the plan formed from rows of dense strips: every block's eight
+                               // columns are consecutive from a multiple of eight and every chunk fits one step
+                               // (two share a step when both fit a half): tile_dense_kernel can run it
+    bool ownedRows = false;    // set by the plan: no row of these tiles gets anything from the CSR part
     int *waveDesc = nullptr;   // [nWaves][8]
     int *hdr = nullptr;        // [steps][kTileHdr]
     int *atox = nullptr;       // [steps][64]

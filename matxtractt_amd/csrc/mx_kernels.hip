@@ -850,6 +850,82 @@ __global__ __launch_bounds__(kBlock) void tile_kernel(const int4 *__restrict__ w
     }
 }
 
+// The binary16 tile kernel for blocks whose eight columns are consecutive and start at a multiple
+// of eight (dense strips), for chunks of at most one step whose rows receive nothing from the CSR
+// part.  A lane's B operand -- the eight x of one block -- is
+// then one aligned 16-byte read of x, so the column ids, the gather, the trip through LDS and the
+// old y all fall away: per step a header, the blocks and 16 bytes of x per block.  The results
+// leave from the four lanes that hold them.  Same step stream, headers and wave ranges as
+// tile_kernel; the header carries the first column of every block slot in dwords 21..28.
+struct DenseStep {
+    int hdr;      // header dword lane%32
+    v4i32 v, b;   // A operand (one block row), B operand (the eight x of the lane's block)
+};
+__global__ __launch_bounds__(kBlock) void tile_dense_kernel(const int4 *__restrict__ waveDesc, const int *__restrict__ hdr,
+                                                           const _Float16 *__restrict__ tcVal,
+                                                           const _Float16 *__restrict__ x, _Float16 *__restrict__ y,
+                                                           int nWaves)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gw = xcd_contiguous_block(blockIdx.x, gridDim.x) * (kBlock / 64) + wave;
+    if (gw >= nWaves) return;
+    const int4 d0 = waveDesc[2 * gw], d1 = waveDesc[2 * gw + 1];
+    const int s0 = __builtin_amdgcn_readfirstlane(d0.x), s1 = __builtin_amdgcn_readfirstlane(d0.y);
+    if (s0 >= s1) return;
+    const int last = s1 - 1;
+    const int m = lane & 15, g = lane >> 4, h = m >> 3;
+    auto issue = [&](DenseStep &R, int step, int vo, int na) {
+        R.hdr = hdr[(size_t)step * kTileHdr + (lane & 31)];
+        R.v = __builtin_nontemporal_load((const v4i32 *)(tcVal + vo + ((h ? na : 0) + g) * 64 + (m & 7) * 8));
+    };
+    // the x of the lane's block, once the header is there: B column m (0 = half 0, 1 = half 1),
+    // rows 8g..8g+7 = slot 4m+g; the other lanes read what lane m&1 of their group reads
+    auto fetch = [&](DenseStep &R) {
+        const int base = __shfl(R.hdr, 21 + 4 * (m & 1) + g);
+        R.b = *(const v4i32 *)(x + max(base, 0));
+    };
+    auto step = [&](int s, DenseStep &Ra, DenseStep &Rg, DenseStep &Ri) {
+        issue(Ri, min(s + 4, last), __builtin_amdgcn_readlane(Ra.hdr, 19), __builtin_amdgcn_readlane(Ra.hdr, 20));
+        fetch(Rg);
+        const int n0 = __builtin_amdgcn_readlane(Ra.hdr, 17), n1 = __builtin_amdgcn_readlane(Ra.hdr, 18);
+        const v4i32 z = {0, 0, 0, 0};
+        const v8f16 a = __builtin_bit_cast(v8f16, g < (h ? n1 : n0) ? Ra.v : z);
+        const v8f16 bv = __builtin_bit_cast(v8f16, (m < 2 && g < (m ? n1 : n0)) ? Ra.b : z);
+        const v4f32 zero = {0.f, 0.f, 0.f, 0.f};
+        v4f32 acc = tile_mma(a, bv, zero);
+        // D[0..3][0] in lane 0, D[4..7][0] in lane 16, D[8..11][1] in lane 33, D[12..15][1] in lane 49:
+        // register i of those lanes is output row 4g+i of the step.  A chunk that fills both
+        // halves has its rows in the first two only: they add what the other two hold.
+        if (!(__builtin_amdgcn_readlane(Ra.hdr, 16) & 2)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += __shfl(acc[i], (lane + 33) & 63);
+        }
+        int row[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) row[i] = __shfl(Ra.hdr, 4 * g + i);
+        if (lane == 0 || lane == 16 || lane == 33 || lane == 49) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (row[i] >= 0) y[row[i]] = (_Float16)acc[i];
+        }
+    };
+    DenseStep R0, R1, R2, R3, R4;
+    const int na = __builtin_amdgcn_readfirstlane(d1.z);
+    issue(R0, s0, __builtin_amdgcn_readfirstlane(d0.z), na & 255);
+    issue(R1, min(s0 + 1, last), __builtin_amdgcn_readfirstlane(d0.w), (na >> 8) & 255);
+    issue(R2, min(s0 + 2, last), __builtin_amdgcn_readfirstlane(d1.x), (na >> 16) & 255);
+    issue(R3, min(s0 + 3, last), __builtin_amdgcn_readfirstlane(d1.y), (na >> 24) & 255);
+    fetch(R0);
+    fetch(R1);
+    for (int s = s0; s < s1; s += 5) {
+        step(s, R0, R2, R4);
+        if (s + 1 < s1) step(s + 1, R1, R3, R0);
+        if (s + 2 < s1) step(s + 2, R2, R4, R1);
+        if (s + 3 < s1) step(s + 3, R3, R0, R2);
+        if (s + 4 < s1) step(s + 4, R4, R1, R3);
+    }
+}
+
 // MFMA probes: one wave, operands and accumulators exchanged lane by lane (raw register
 // contents), so a host test can check the operand layout the tile kernels rely on.
 __global__ void probe_mfma_f64_kernel(const double *A /*[64]*/, const double *B /*[64]*/, double *D /*[64][4]*/)
@@ -948,6 +1024,13 @@ hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, voi
 {
     if (T.nWaves <= 0) return hipSuccess;
     const int grid = (T.nWaves + 3) / 4;
+    // the strip form overwrites its rows: it runs when the caller overwrites, or adds to rows that
+    // the plan knows hold zero at that point; and it reads x in aligned 16-byte pieces
+    if (dtype == MX_F16 && T.dense && (!accumulate || T.ownedRows) && !((uintptr_t)x & 15)) {
+        hipLaunchKernelGGL(mxk::tile_dense_kernel, dim3(grid), dim3(mxk::kBlock), 0, s, (const int4 *)T.waveDesc, T.hdr,
+                           (const _Float16 *)T.tcVal, (const _Float16 *)x, (_Float16 *)y, T.nWaves);
+        return hipGetLastError();
+    }
     if (dtype == MX_F64)
         hipLaunchKernelGGL((mxk::tile_kernel<double>), dim3(grid), dim3(mxk::kBlock), 0, s, (const int4 *)T.waveDesc, T.hdr,
                            T.atox, (const double *)T.tcVal, (const double *)x, (double *)y, T.nWaves, accumulate);

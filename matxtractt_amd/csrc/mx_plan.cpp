@@ -429,9 +429,28 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
 // Puts tiles on the device for the tile kernels (see DeviceTiles): the fragments named by
 // `selFrag` (all when null), expanded to full blocks.  Column ids go through `colMap` and
 // output rows through `rowMap` when given.
+// One block of the tile kernels: fragM x fragK values, row-major, zeros included, and the column
+// of each of its fragK positions (-1 = unused).
+struct TileBlock {
+    std::vector<unsigned char> vals;
+    int cols[8];
+};
+// A chunk the plan forms itself for tile_dense_kernel: up to fragM rows (caller's numbering, -1 =
+// none) with one and the same set of columns -- whole runs of fragK from a multiple of fragK --
+// and that set as blocks.
+struct StripChunk {
+    int rows[8];
+    std::vector<TileBlock> blocks;
+    int nnz;
+};
+
+// `rowTaken` (optional, per row of A_dd) marks rows whose entries the plan has put into strip
+// chunks: they are left out of the fragments here.  With `stripChunks` the canonical chunks are
+// not used at all: the given chunks are laid out, for tile_dense_kernel.
 int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, const int *chunkPtr, const int *fragPtr,
                  const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap,
-                 mx::DeviceTiles &T, int *tile_nnz)
+                 mx::DeviceTiles &T, int *tile_nnz, const char *rowTaken = nullptr,
+                 const std::vector<StripChunk> *stripChunks = nullptr)
 {
     const int es = mx::elem_size(dtype), fragK = mx::frag_k(dtype), fragM = mx::kFragM;
     const int SF = mx::tile_slots(dtype), HF = SF / 2, H = mx::kTileHdr, BS = fragM * fragK;  // BS: values per block
@@ -443,26 +462,81 @@ int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, c
     std::vector<unsigned char> dVal;
     size_t voff = 0;  // values stored so far; always a multiple of BS, so every block is 16-byte aligned
     int nsel = 0, nnz = 0, nfr = 0;
-    auto put_block = [&](size_t s, int slot, int f) {  // fragment f, expanded, as the next block of step s
-        const int cnt = fragPtr[f + 1] - fragPtr[f];
-        dVal.resize((voff + BS) * es, 0);
-        const uint64_t bm = f64 ? (uint64_t)bit32[f] : bit64[f];
-        int k = 0;
-        for (int bit = 0; bit < BS; ++bit)
-            if ((bm >> bit) & 1ull) {
-                std::memcpy(&dVal[(voff + bit) * es], tv + (size_t)(fragPtr[f] + k) * es, es);
-                ++k;
+
+    // The blocks of a chunk, rebuilt from its selected fragments: their columns (in the caller's
+    // numbering) in ascending order, fragK per block.  The reference orders a chunk's columns by
+    // their rank among the dense columns, which scatters neighbouring columns over the fragments;
+    // in ascending order a dense strip becomes blocks of consecutive columns, and the gathers of
+    // any chunk touch fewer lines.
+    typedef TileBlock Block;
+    std::vector<Block> blocks;
+    struct ColRef {
+        int col, f, pos;
+    };
+    std::vector<ColRef> refs;
+    int chunkVals = 0;  // entries build_blocks put into `blocks`
+    std::vector<int> chunkOfFrag;  // only needed to find a fragment's rows
+    if (rowTaken) {
+        chunkOfFrag.resize((size_t)chunkPtr[chunkNum]);
+        for (int w = 0; w < chunkNum; ++w)
+            for (int f = chunkPtr[w]; f < chunkPtr[w + 1]; ++f) chunkOfFrag[f] = w;
+    }
+    auto gone = [&](int f, int r) {  // row r of fragment f was taken into a strip chunk
+        if (!rowTaken) return false;
+        const int i = chunkOfFrag[f] * fragM + r;
+        return i < dRows && rowTaken[i] != 0;
+    };
+    auto build_blocks = [&](const std::vector<int> &fsel) {
+        refs.clear();
+        for (int f : fsel) {
+            const uint64_t bm = f64 ? (uint64_t)bit32[f] : bit64[f];
+            for (int c = 0; c < fragK; ++c) {
+                bool used = false;
+                for (int r = 0; r < fragM && !used; ++r) used = ((bm >> (r * fragK + c)) & 1ull) && !gone(f, r);
+                if (!used) continue;  // a padding position of the chunk's last fragment, or only rows that went elsewhere
+                const int col = atox[(size_t)f * fragK + c];
+                refs.push_back({colMap ? colMap[col] : col, f, c});
             }
-        voff += BS;
-        nnz += cnt;
-        ++nfr;
-        for (int c = 0; c < fragK; ++c) {
-            const int col = atox[(size_t)f * fragK + c];
-            dAtox[s * 64 + (size_t)slot * fragK + c] = colMap ? colMap[col] : col;
+        }
+        std::sort(refs.begin(), refs.end(), [](const ColRef &a, const ColRef &b) { return a.col < b.col; });
+        chunkVals = 0;
+        const int nb = ((int)refs.size() + fragK - 1) / fragK;
+        blocks.assign(nb, Block());
+        for (Block &B : blocks) {
+            B.vals.assign((size_t)BS * es, 0);
+            for (int c = 0; c < 8; ++c) B.cols[c] = -1;
+        }
+        // where each fragment's values start for every (row, position): walk its bits in order
+        for (int i = 0; i < (int)refs.size(); ++i) blocks[i / fragK].cols[i % fragK] = refs[i].col;
+        std::vector<int> where((size_t)fsel.size() * fragK, -1);  // (fragment in fsel, pos) -> index in refs
+        for (int i = 0; i < (int)refs.size(); ++i) {
+            const int fi = (int)(std::find(fsel.begin(), fsel.end(), refs[i].f) - fsel.begin());
+            where[(size_t)fi * fragK + refs[i].pos] = i;
+        }
+        for (int fi = 0; fi < (int)fsel.size(); ++fi) {
+            const int f = fsel[fi];
+            const uint64_t bm = f64 ? (uint64_t)bit32[f] : bit64[f];
+            int k = 0;
+            for (int bit = 0; bit < BS; ++bit)
+                if ((bm >> bit) & 1ull) {
+                    const int r = bit / fragK, i = where[(size_t)fi * fragK + bit % fragK];
+                    if (!gone(f, r)) {
+                        std::memcpy(&blocks[i / fragK].vals[((size_t)r * fragK + i % fragK) * es], tv + (size_t)(fragPtr[f] + k) * es, es);
+                        ++chunkVals;
+                    }
+                    ++k;
+                }
         }
     };
-    // a step with the fragments a0 (half 0) and a1 (half 1) of the chunks w0 and w1 (w1 < 0: none)
-    auto emit = [&](const int *a0, int n0, int w0, const int *a1, int n1, int w1, int flags) {
+    auto put_block = [&](size_t s, int slot, const Block &B) {  // the next block of step s
+        dVal.insert(dVal.end(), B.vals.begin(), B.vals.end());
+        voff += BS;
+        for (int c = 0; c < fragK; ++c) dAtox[s * 64 + (size_t)slot * fragK + c] = B.cols[c];
+        if (!f64) hdr[s * H + 21 + slot] = B.cols[0];
+    };
+    // a step with the blocks a0[0..n0) (half 0) and a1[0..n1) (half 1) of two chunks, given by
+    // their fragM output rows r0 and r1 (r1 null: none; with flags & 2 clear both halves are r0's)
+    auto emit = [&](const Block *a0, int n0, const int *r0, const Block *a1, int n1, const int *r1, int flags) {
         const size_t s = stepVo.size();
         hdr.resize((s + 1) * H, 0);
         dAtox.resize((s + 1) * 64, -1);
@@ -471,53 +545,81 @@ int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, c
         stepChunkEnd.push_back(flags & 1);
         for (int i = 0; i < 16; ++i) hdr[s * H + i] = -1;
         for (int half = 0; half < 2; ++half) {
-            const int w = half ? w1 : w0;
-            if (w < 0 || (half && !(flags & 2))) continue;
-            for (int i = 0; i < fragM; ++i) {
-                const int local = w * fragM + i;
-                hdr[s * H + half * 8 + i] = local < dRows ? (rowMap ? rowMap[local] : local) : -1;
-            }
+            const int *rr = half ? r1 : r0;
+            if (!rr || (half && !(flags & 2))) continue;
+            for (int i = 0; i < fragM; ++i) hdr[s * H + half * 8 + i] = rr[i];
         }
         hdr[s * H + 16] = flags;
         hdr[s * H + 17] = n0;
         hdr[s * H + 18] = n1;
+        for (int i = 21; i < 29; ++i) hdr[s * H + i] = -1;
         for (int i = 0; i < n0; ++i) put_block(s, mx::tile_slot(dtype, 0, i), a0[i]);
         for (int i = 0; i < n1; ++i) put_block(s, mx::tile_slot(dtype, 1, i), a1[i]);
     };
-    std::vector<int> fsel, pending;
-    int pendingChunk = -1;  // a small chunk waiting for a partner
-    for (int w = 0; w < chunkNum; ++w) {
-        fsel.clear();
-        for (int f = chunkPtr[w]; f < chunkPtr[w + 1]; ++f)
-            if (fragPtr[f + 1] > fragPtr[f] && (!selFrag || selFrag[f])) fsel.push_back(f);
-        if (fsel.empty()) continue;
-        ++nsel;
-        if ((int)fsel.size() <= HF) {
-            if (pendingChunk >= 0) {
-                emit(pending.data(), (int)pending.size(), pendingChunk, fsel.data(), (int)fsel.size(), w, 3);
-                pendingChunk = -1;
+    std::vector<int> fsel;
+    std::vector<Block> pending;
+    int pendingRows[8], curRows[8];
+    bool havePending = false;  // a small chunk waiting for a partner
+    // a chunk's blocks into steps: up to half a step shares one with the next such chunk, more
+    // takes whole steps of its own
+    auto place = [&](const std::vector<Block> &bl, const int *rows) {
+        if ((int)bl.size() <= HF) {
+            if (havePending) {
+                emit(pending.data(), (int)pending.size(), pendingRows, bl.data(), (int)bl.size(), rows, 3);
+                havePending = false;
             } else {
-                pendingChunk = w;
-                pending = fsel;
+                havePending = true;
+                pending = bl;
+                std::copy(rows, rows + 8, pendingRows);
             }
         } else {
-            for (size_t i0 = 0; i0 < fsel.size(); i0 += SF) {
-                const int n = (int)std::min(fsel.size() - i0, (size_t)SF), n0 = std::min(n, HF);
-                emit(&fsel[i0], n0, w, &fsel[i0 + n0], n - n0, w, i0 + SF >= fsel.size() ? 1 : 0);
+            for (size_t i0 = 0; i0 < bl.size(); i0 += SF) {
+                const int n = (int)std::min(bl.size() - i0, (size_t)SF), n0 = std::min(n, HF);
+                emit(&bl[i0], n0, rows, &bl[i0 + n0], n - n0, rows, i0 + SF >= bl.size() ? 1 : 0);
             }
         }
-        if (voff > 2000000000u) {
-            set_error("tile layout: too many values for 32-bit offsets");
-            return MX_ERR_ARG;
+    };
+    if (stripChunks) {
+        for (const StripChunk &C : *stripChunks) {
+            ++nsel;
+            nnz += C.nnz;
+            nfr += (int)C.blocks.size();
+            place(C.blocks, C.rows);
+            if (voff > 2000000000u) {
+                set_error("tile layout: too many values for 32-bit offsets");
+                return MX_ERR_ARG;
+            }
+        }
+    } else {
+        for (int w = 0; w < chunkNum; ++w) {
+            fsel.clear();
+            for (int f = chunkPtr[w]; f < chunkPtr[w + 1]; ++f)
+                if (fragPtr[f + 1] > fragPtr[f] && (!selFrag || selFrag[f])) fsel.push_back(f);
+            if (fsel.empty()) continue;
+            build_blocks(fsel);
+            if (blocks.empty()) continue;  // all its rows went into strip chunks
+            ++nsel;
+            nnz += chunkVals;
+            nfr += (int)fsel.size();
+            for (int i = 0; i < 8; ++i) {
+                const int local = w * fragM + i;
+                curRows[i] = (i < fragM && local < dRows) ? (rowMap ? rowMap[local] : local) : -1;
+            }
+            place(blocks, curRows);
+            if (voff > 2000000000u) {
+                set_error("tile layout: too many values for 32-bit offsets");
+                return MX_ERR_ARG;
+            }
         }
     }
-    if (pendingChunk >= 0) emit(pending.data(), (int)pending.size(), pendingChunk, nullptr, 0, -1, 3);
+    if (havePending) emit(pending.data(), (int)pending.size(), pendingRows, nullptr, 0, nullptr, 3);
     const int steps = (int)stepVo.size();
     T.chunkNum = nsel;
     T.frags = nfr;
     T.vals = nnz;
     T.stored = (long long)voff;
     T.steps = steps;
+    T.dense = stripChunks != nullptr && steps > 0;
     if (tile_nnz) *tile_nnz = nnz;
     if (steps == 0) return MX_OK;
     // waves: whole chunks, about `per` steps each; few enough waves that all of them are resident
@@ -733,7 +835,8 @@ struct mx_plan {
     mx::DeviceSlices slices;  // CSR part (or its long rows), x-resident-in-LDS form (csr_slice_kernel)
     int csr_variant = 0;      // 0 = row tiles, 1 = slices, 2 = row tiles for the short rows, then slices for the long ones
     int csr_nnz = 0;
-    mx::DeviceTiles tiles;
+    mx::DeviceTiles tiles;    // tile part, general form (tile_kernel)
+    mx::DeviceTiles strips;   // tile part, binary16 strips on rows of their own (tile_dense_kernel)
     int tile_nnz = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -755,6 +858,7 @@ extern "C" void mx_plan_destroy(mx_plan *plan)
     free_csr(plan->csr);
     free_slices(plan->slices);
     free_tiles(plan->tiles);
+    free_tiles(plan->strips);
     if (plan->ev0) (void)hipEventDestroy(plan->ev0);
     if (plan->ev1) (void)hipEventDestroy(plan->ev1);
     if (plan->stream) (void)hipStreamDestroy(plan->stream);
@@ -971,6 +1075,83 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                     sel[f] = (flags & MX_PLAN_ALL_TILES) ? vals > 0 : (vals > 0 && (double)vals >= gate * fragM * fragK);
                 }
             }
+            // binary16 rows of A_dd whose columns, in the caller's numbering, are one run of a
+            // multiple of fragK columns from a multiple of fragK (a row of a dense strip), with
+            // nothing in the residual: rows with the same run are put together, fragM at a time,
+            // into chunks of the plan's own (the canonical chunks follow the row order, where
+            // rows of other shapes fall between them and one chunk straddles two strips).  A
+            // chunk at least half full goes to tile_dense_kernel; its rows leave the fragments.
+            std::vector<char> taken;
+            std::vector<StripChunk> stripChunks;
+            if (P->dtype == MX_F16 && fragM == 8 && fragK == 8 && !(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES)) &&
+                !(std::getenv("MX_NO_STRIPS") && std::atoi(std::getenv("MX_NO_STRIPS")))) {
+                const int maxRun = mx::tile_slots(P->dtype) * fragK;
+                struct Cand {
+                    int c0, n, i;
+                };
+                std::vector<Cand> cand;
+                for (int i = 0; i < P->dRows; ++i) {
+                    const int p0 = P->ddRowPtr[i], n = P->ddRowPtr[i + 1] - p0, r = P->rId[i];
+                    if (n < fragK || n > maxRun || n % fragK || P->cdRowPtr[r + 1] != P->cdRowPtr[r]) continue;
+                    int lo = INT_MAX, hi = -1;
+                    for (int p = p0; p < p0 + n; ++p) {
+                        const int c = P->descColId[P->ddColInd[p]];
+                        lo = std::min(lo, c);
+                        hi = std::max(hi, c);
+                    }
+                    // n distinct columns within [lo, lo + n) are exactly that run
+                    if (lo % fragK == 0 && hi - lo + 1 == n) cand.push_back({lo, n, i});
+                }
+                std::sort(cand.begin(), cand.end(), [](const Cand &a, const Cand &b) {
+                    return a.c0 != b.c0 ? a.c0 < b.c0 : a.n != b.n ? a.n < b.n : a.i < b.i;
+                });
+                taken.assign((size_t)P->dRows, 0);
+                const uint16_t *ddv16 = (const uint16_t *)P->ddVal.data();  // binary16 bit patterns
+                for (size_t a = 0; a < cand.size();) {
+                    size_t b = a;
+                    while (b < cand.size() && cand[b].c0 == cand[a].c0 && cand[b].n == cand[a].n) ++b;
+                    for (size_t g = a; g < b; g += fragM) {
+                        const int nr = (int)std::min(b - g, (size_t)fragM);
+                        if (2 * nr < fragM) break;
+                        StripChunk C;
+                        const int c0 = cand[a].c0, n = cand[a].n, nb = n / fragK;
+                        C.nnz = nr * n;
+                        C.blocks.resize(nb);
+                        for (int k = 0; k < nb; ++k) {
+                            C.blocks[k].vals.assign((size_t)fragM * fragK * es, 0);
+                            for (int c = 0; c < fragK; ++c) C.blocks[k].cols[c] = c0 + k * fragK + c;
+                        }
+                        for (int j = 0; j < 8; ++j) C.rows[j] = -1;
+                        for (int j = 0; j < nr; ++j) {
+                            const int i = cand[g + j].i;
+                            taken[i] = 1;
+                            C.rows[j] = P->rId[i];
+                            for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
+                                const int c = P->descColId[P->ddColInd[p]] - c0;
+                                ((uint16_t *)C.blocks[c / fragK].vals.data())[j * fragK + c % fragK] = ddv16[p];
+                            }
+                        }
+                        stripChunks.push_back(std::move(C));
+                    }
+                    a = b;
+                }
+                if (stripChunks.empty()) taken.clear();
+            }
+            if (!taken.empty()) {
+                // the gate again, on what the taken rows leave of each fragment
+#pragma omp parallel for schedule(static)
+                for (int w = 0; w < chunkNum; ++w) {
+                    uint64_t rowsLeft = 0;  // bits of the rows that stay
+                    for (int r = 0; r < fragM; ++r) {
+                        const int i = w * fragM + r;
+                        if (i < P->dRows && !taken[i]) rowsLeft |= 0xffull << (r * fragK);
+                    }
+                    for (int f = P->chunkPtr[w]; f < P->chunkPtr[w + 1]; ++f) {
+                        const int vals = __builtin_popcountll(P->fragBit64[f] & rowsLeft);
+                        sel[f] = sel[f] && vals > 0 && (double)vals >= gate * fragM * fragK;
+                    }
+                }
+            }
             // fragment of every A_dd entry: the rank of its column among the chunk's columns, / fragK
             auto frag_of = [&](int w, int ddcol) {
                 const int f0 = P->chunkPtr[w], f1 = P->chunkPtr[w + 1];
@@ -989,7 +1170,7 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             for (int i = 0; i < P->dRows; ++i) {
                 int n = 0;
                 for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
-                    keep[p] = !sel[frag_of(i / fragM, P->ddColInd[p])];
+                    keep[p] = (!taken.empty() && taken[i]) ? 0 : !sel[frag_of(i / fragM, P->ddColInd[p])];
                     n += keep[p];
                 }
                 rowPtr[P->rId[i] + 1] += n;
@@ -1023,11 +1204,22 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             if (rc) return fail(rc);
 
             // tile part: the selected chunks; columns and rows back in the caller's numbering
-            rc = upload_tiles(P->dtype, chunkNum, sel.data(), P->dRows, P->chunkPtr.data(), P->fragPtr.data(),
-                              P->dtype == MX_F64 ? (const void *)P->fragBit32.data() : (const void *)P->fragBit64.data(),
+            const void *bits = P->dtype == MX_F64 ? (const void *)P->fragBit32.data() : (const void *)P->fragBit64.data();
+            int nnzGeneral = 0, nnzStrips = 0;
+            rc = upload_tiles(P->dtype, chunkNum, sel.data(), P->dRows, P->chunkPtr.data(), P->fragPtr.data(), bits,
                               P->tcVal.data(), P->sparse_AToX_index.data(), P->descColId.data(), P->rId.data(),
-                              plan->tiles, &plan->tile_nnz);
+                              plan->tiles, &nnzGeneral, taken.empty() ? nullptr : taken.data());
             if (rc) return fail(rc);
+            if (!stripChunks.empty()) {
+                rc = upload_tiles(P->dtype, chunkNum, sel.data(), P->dRows, P->chunkPtr.data(), P->fragPtr.data(), bits,
+                                  P->tcVal.data(), P->sparse_AToX_index.data(), P->descColId.data(), P->rId.data(),
+                                  plan->strips, &nnzStrips, nullptr, &stripChunks);
+                if (rc) return fail(rc);
+                // strip rows have nothing in the residual and left the fragments: the CSR part,
+                // which runs first, writes zeros there and the strip kernel may overwrite
+                plan->strips.ownedRows = true;
+            }
+            plan->tile_nnz = nnzGeneral + nnzStrips;
         }
     } catch (const std::bad_alloc &) {
         set_error("mx_plan_create: out of memory");
@@ -1050,8 +1242,8 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     info->rows = plan->rows;
     info->cols = plan->cols;
     info->nnz = plan->nnz;
-    info->tile_chunks = plan->tiles.chunkNum;
-    info->tile_frags = plan->tiles.frags;
+    info->tile_chunks = plan->tiles.chunkNum + plan->strips.chunkNum;
+    info->tile_frags = plan->tiles.frags + plan->strips.frags;
     info->tile_nnz = plan->tile_nnz;
     info->csr_nnz = plan->csr_nnz;
     info->csr_blocks = plan->csr_variant == 1 ? plan->slices.nWG : plan->csr.nBlocks;
@@ -1061,14 +1253,19 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
                       (double)plan->rows * es;
     // what the tile kernel reads and writes per launch: headers, column ids, values, x once per
     // column id, y once per row
-    info->tile_bytes = plan->tiles.steps
-                           ? (double)plan->tiles.steps * (mx::kTileHdr * 4.0 + 64 * 4.0) + (double)plan->tiles.stored * es +
-                                 (double)plan->tiles.frags * fragK * es + (double)plan->tiles.chunkNum * 8 * 2 * es
-                           : 0.0;
+    info->tile_bytes = 0.0;
+    if (plan->tiles.steps)
+        info->tile_bytes += (double)plan->tiles.steps * (mx::kTileHdr * 4.0 + 64 * 4.0) + (double)plan->tiles.stored * es +
+                            (double)plan->tiles.frags * fragK * es + (double)plan->tiles.chunkNum * 8 * 2 * es;
+    if (plan->strips.steps)  // no column ids, no old y
+        info->tile_bytes += (double)plan->strips.steps * (mx::kTileHdr * 4.0) + (double)plan->strips.stored * es +
+                            (double)plan->strips.frags * fragK * es + (double)plan->strips.chunkNum * 8 * es;
     (void)bitBytes;
     const bool sliceMain = plan->csr_variant == 1 || (plan->csr_variant == 2 && plan->slices.nnz > plan->csr.nnz);
     info->csr_main_kernel = sliceMain ? 1 : 0;
     info->csr_main_nnz = plan->csr_variant == 2 ? (sliceMain ? plan->slices.nnz : plan->csr.nnz) : plan->csr_nnz;
+    info->tile_variant = plan->strips.steps > 0 ? 1 : 0;
+    info->tile_strip_nnz = plan->strips.vals;
     return MX_OK;
 }
 
@@ -1077,6 +1274,7 @@ static int spmv_on(mx_plan *plan, const void *x, void *y, hipStream_t s)
     int rc = launch_csr_part(plan, x, y, 0, s);
     if (rc) return rc;
     MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x, y, 1, s));
+    MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x, y, 1, s));
     return MX_OK;
 }
 
@@ -1175,10 +1373,11 @@ extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, 
     }
     if (ms_tile) {
         *ms_tile = 0.0;
-        if (plan->tiles.chunkNum > 0) {
+        if (plan->tiles.chunkNum + plan->strips.chunkNum > 0) {
             // overwrite mode: the timed loop must not grow y without bound
             rc = time_loop(plan, warm, iters, [&]() -> int {
                 MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x_dev, y_dev, 0, s));
+                MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x_dev, y_dev, 0, s));
                 return MX_OK;
             }, &t);
             if (rc) return rc;

@@ -479,6 +479,65 @@ def test_plan_from_a_saved_partition(mx, ora, tmp_path):
         Q.close()
 
 
+def test_strip_form_of_the_fp16_tile_kernel(mx, ora, monkeypatch):
+    """Rows of dense strips (one run of 8k consecutive columns from a multiple of eight, nothing
+    else in the row) are grouped by the plan into chunks for the strip form of the binary16 tile
+    kernel, wherever they sit in the row order; rows that break the conditions -- a run off the
+    grid of eight, a further entry -- stay with the general kernel, and so does everything when x
+    is not 16-byte aligned.  Same result every time."""
+    import torch
+    rng = np.random.default_rng(31)
+    rows, cols = 4096, 50000
+
+    def strips(shift=0, extra=False, interloper=False):
+        rp, ci = [0], []
+        for r in range(rows):
+            if interloper and r == 130:       # as long as a strip row: shifts the reference's chunks against the strips
+                ci += sorted(rng.choice(cols, 32, replace=False).tolist())
+                rp.append(len(ci))
+                continue
+            if (r // 128) % 3 == 0:           # a strip row: 32 consecutive columns from a multiple of 8
+                base = 8 * ((r // 8) % 4000) + shift
+                c = list(range(base, base + 32))
+                if extra and r % 64 == 0:
+                    c.append(base + 40000)    # an entry the tiles do not take
+            else:
+                c = sorted(rng.choice(cols, 1 + int(rng.integers(0, 3)), replace=False).tolist())
+            ci += c
+            rp.append(len(ci))
+        return mx.Csr(rows, cols, np.array(rp, np.int32), np.array(ci, np.int32),
+                      rng.uniform(-1, 1, len(ci)).astype(np.float16))
+
+    x = rng.uniform(-1, 1, cols + 8).astype(np.float16)
+    xd_all = torch.from_numpy(x).cuda()
+    # want: the share of the tile entries that the strip form takes (all, none, some)
+    for name, A, xoff, want in (("strips", strips(), 0, "all"), ("off the grid", strips(shift=3), 0, "none"),
+                                ("rows with more", strips(extra=True), 0, "some"), ("x not aligned", strips(), 1, "all"),
+                                ("a row of another shape among them", strips(interloper=True), 0, "all")):
+        xv = x[xoff:xoff + cols]
+        ref = oracle_y(ora, mx, A, xv)
+        P = mx.Partition(A, 1.0, 1.0)
+        for variant in ("rows", "slices"):
+            monkeypatch.setenv("MX_CSR_KERNEL", variant)
+            plan = mx.Plan(P)
+            print("strip form:", name, variant, "tile_nnz", plan.info["tile_nnz"], "in strips", plan.info["tile_strip_nnz"], flush=True)
+            assert plan.info["tile_nnz"] > 0.5 * A.nnz
+            sn, tn = plan.info["tile_strip_nnz"], plan.info["tile_nnz"]
+            assert plan.info["tile_variant"] == (sn > 0)
+            assert (want == "all" and sn == tn) or (want == "none" and sn == 0) or (want == "some" and 0 < sn <= tn)
+            xd = xd_all[xoff:xoff + cols]
+            if xoff and plan.info["csr_variant"] != 0:
+                with pytest.raises(mx.MxError):      # the slice kernel itself needs an aligned x
+                    plan.spmv(xd)
+            else:
+                y = torch.full((rows,), 3.0, dtype=torch.float16, device="cuda")
+                plan.spmv(xd, y)
+                torch.cuda.synchronize()
+                assert rel_l2(y.cpu().numpy(), ref) <= F16_TOL
+            plan.close()
+        P.close()
+
+
 def test_tau_tuner(mx, ora):
     """mx_tune_tau walks the grid with tau_c >= tau_r, reports every candidate, returns the fastest;
     candidates without tiles share one timing and are reported as (0, 0)."""
