@@ -27,13 +27,13 @@ GRID = (0.0, 0.25, 0.5, 0.75, 1.0)
 # HBM-side bytes per launch (read + written) of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE runs of this script, each counter scaled by what it reads for an elementwise kernel of
 # known size (--calibrate-copy): FETCH_SIZE x 2.000, WRITE_SIZE x 1.000.  The text files under profiles/
-# hold the counter values.  (workload, kernel) -> bytes
+# hold the counter values.  (workload, kernel, plan has tiles) -> bytes
 TRAFFIC = {
-    (2, "csr_rows_kernel<f64>"): 47165962,
-    (2, "csr_slice_kernel<f64>"): 48810843,
-    (3, "csr_rows_kernel<f64>"): 287435306,
-    (4, "csr_slice_kernel<f16>"): 55698523,
-    (5, "csr_slice_kernel<f16>"): 301473538,
+    (2, "csr_rows_kernel<f64>", False): 47165962,
+    (2, "csr_slice_kernel<f64>", False): 48810843,
+    (3, "csr_rows_kernel<f64>", False): 287435306,
+    (4, "csr_slice_kernel<f16>", False): 55698523,
+    (5, "csr_slice_kernel<f16>", False): 301473538,
 }
 WORKLOADS = {
     1: "configs[0]: FP64 random 4096x4096, 16 nnz/row",
@@ -64,7 +64,7 @@ def measure(mx, torch, A, xd, yd, tau, warm, iters, flags=None):
     return part, plan, rec
 
 
-def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline):
+def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_tau=None):
     import numpy as np
     t0 = time.time()
     A, x = mx.gen_config(cfg)
@@ -77,6 +77,8 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline):
 
     # tau sweep with short timing loops
     points = [(c, r) for c in GRID for r in GRID if c >= r] if sweep else [(0.0, 0.0)]
+    if only_tau is not None:
+        points = [tuple(only_tau)]  # nothing else: a profile of this run then shows one plan's kernels only
     table = []
     for tau in points:
         part, plan, rec = measure(mx, torch, A, xd, yd, tau, 20, 200)
@@ -85,13 +87,13 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline):
             (tau[0], tau[1], rec["ms_total"] * 1e3, rec["ms_tile"] * 1e3, rec["ms_csr"] * 1e3, rec["tile_nnz"]))
         plan.close()
         part.close()
-    best = min(table, key=lambda r: r["ms_total"])
-    if best["tile_nnz"] == 0:
+    best = min(table, key=lambda r: r["ms_total"]) if only_tau is None else table[-1]
+    if best["tile_nnz"] == 0 and only_tau is None:
         # every point that sends nothing to the tile kernel is the same CSR-only plan: call it (0, 0)
         best = next(r for r in table if (r["tau_c"], r["tau_r"]) == (0.0, 0.0))
     hybrid = [r for r in table if r["tile_nnz"] > 0]
     best_hybrid = min(hybrid, key=lambda r: r["ms_total"]) if hybrid else None
-    csr_only = next(r for r in table if (r["tau_c"], r["tau_r"]) == (0.0, 0.0))
+    csr_only = next((r for r in table if (r["tau_c"], r["tau_r"]) == (0.0, 0.0)), None)
 
     # the timed run on the best point: W warm-up steps, then exactly K steps between syncs
     tau = (best["tau_c"], best["tau_r"])
@@ -147,11 +149,11 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline):
                        "how": "median of 15 single launches, each after a 1 GiB buffer sweep and a sync; "
                               "the quoted value is the back-to-back (warm) one"},
         "rel_l2_vs_oracle": rel_l2,
-        "csr_only_ms": csr_only["ms_total"],
+        "csr_only_ms": csr_only and csr_only["ms_total"],
         "best_hybrid": best_hybrid and {k: best_hybrid[k] for k in ("tau_c", "tau_r", "ms_total", "tile_nnz", "csr_nnz")},
         "roofline": {"bound": "hbm", "kernel": dom["kernel"], "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK,
-                     "traffic": TRAFFIC.get((cfg, dom["kernel"])) if (tau == (0.0, 0.0) or info["tile_nnz"] == 0) else None,
+                     "traffic": TRAFFIC.get((cfg, dom["kernel"], info["tile_nnz"] > 0)),
                      "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"]},
         "sweep": [{k: r[k] for k in ("tau_c", "tau_r", "ms_total", "ms_tile", "ms_csr", "tile_nnz")} for r in table],
     }
@@ -202,6 +204,8 @@ def main():
     ap.add_argument("--workload", type=int, default=2, choices=sorted(WORKLOADS))
     ap.add_argument("--all", action="store_true", help="also run workloads 3, 4, 5 (reported under 'others')")
     ap.add_argument("--no-sweep", action="store_true", help="tau=(0,0) only")
+    ap.add_argument("--tau", type=float, nargs=2, metavar=("TAU_C", "TAU_R"), default=None,
+                    help="no sweep: run this point (a profile of a fixed plan)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also launch one elementwise kernel that reads and writes MIB MiB (a known size to "
                          "scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -218,7 +222,7 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(1)
 
-    main_rec = run_workload(mx, torch, ora, args.workload, args.steps, args.warmup, not args.no_sweep, True)
+    main_rec = run_workload(mx, torch, ora, args.workload, args.steps, args.warmup, not args.no_sweep, True, args.tau)
     out = {
         "metric": METRIC, "value": main_rec["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_rec["ms_per_step"],
@@ -226,7 +230,8 @@ def main():
         "dtype": main_rec["dtype"], "data": "synthetic",
         "config": {"workload": main_rec["workload"], "rows": main_rec["rows"], "nnz": main_rec["nnz"],
                    "tau_c": main_rec["tau_c"], "tau_r": main_rec["tau_r"], "csr_variant": main_rec["csr_variant"],
-                   "tau_grid": "5x5 {0,.25,.5,.75,1}^2, tau_c>=tau_r, best of sweep"},
+                   "tau_grid": "5x5 {0,.25,.5,.75,1}^2, tau_c>=tau_r, best of sweep" if args.tau is None and not args.no_sweep
+                   else "no sweep: point fixed on the command line"},
         "roofline": main_rec["roofline"],
         "cpu_baseline": main_rec.pop("cpu_baseline"),
         "cpu_all_cores": main_rec.pop("cpu_all_cores"),

@@ -178,6 +178,7 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     const int nV = segPtr[rows];
     struct VRow {
         int start, len, slice;  // start: into ord
+        int kind;               // of its row: 0 = this is its only virtual row, 1 = light, 2 = heavy
     };
     std::vector<VRow> vr((size_t)nV);
 #pragma omp parallel for schedule(dynamic, 1024)
@@ -185,18 +186,22 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
         const int n = selPtr[r + 1] - selPtr[r];
         const int *o = n ? &ord[selPtr[r]] : nullptr;
         int t = segPtr[r];
+        const int nv = segPtr[r + 1] - segPtr[r], kind = nv <= 1 ? 0 : nv <= mx::kSliceLightSegs ? 1 : 2;
         for (int k = 0; k < n;) {
             const int q = col[o[k]] / SW;
             int e = k;
             while (e < n && e - k < cap && col[o[e]] / SW == q) ++e;
-            vr[t++] = {selPtr[r] + k, e - k, q};
+            vr[t++] = {selPtr[r] + k, e - k, q, kind};
             k = e;
         }
     }
-    // virtual rows by (slice, length descending), row order kept among equals: a counting sort
-    const size_t nKeys = (size_t)S * (cap + 1);
+    // virtual rows by (slice, length descending, kind of row), row order kept among equals: a
+    // counting sort.  The kind keeps the sums that one workgroup of the combine kernel gathers
+    // close together: consecutive heavy rows have virtual rows of the same slice and length more
+    // often than a heavy row and its neighbours of other kinds do.
+    const size_t perSlice = (size_t)(cap + 1) * 3, nKeys = (size_t)S * perSlice;
     std::vector<int> keyStart(nKeys + 1, 0), sorted((size_t)nV);
-    auto key_of = [&](const VRow &v) { return (size_t)v.slice * (cap + 1) + (size_t)(cap - v.len); };
+    auto key_of = [&](const VRow &v) { return (size_t)v.slice * perSlice + (size_t)(cap - v.len) * 3 + (size_t)v.kind; };
     for (int t = 0; t < nV; ++t) keyStart[key_of(vr[t]) + 1]++;
     for (size_t k = 0; k < nKeys; ++k) keyStart[k + 1] += keyStart[k];
     {
@@ -213,7 +218,7 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     long long allSteps = 0;
     int busy = 0;
     for (int q = 0; q < S; ++q) {
-        const int a = keyStart[(size_t)q * (cap + 1)], b = keyStart[(size_t)(q + 1) * (cap + 1)];
+        const int a = keyStart[(size_t)q * perSlice], b = keyStart[(size_t)(q + 1) * perSlice];
         for (int f = a; f < b; f += 64) {
             const int n = std::min(64, b - f), steps = (vr[sorted[f]].len + E - 1) / E;
             sliceChunks[q].push_back({f, n, steps});
