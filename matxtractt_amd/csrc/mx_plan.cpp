@@ -1104,8 +1104,12 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                         lo = std::min(lo, c);
                         hi = std::max(hi, c);
                     }
-                    // n distinct columns within [lo, lo + n) are exactly that run
-                    if (lo % fragK == 0 && hi - lo + 1 == n) cand.push_back({lo, n, i});
+                    if (lo % fragK || hi - lo + 1 != n) continue;
+                    // n entries within [lo, lo + n): that run exactly, unless a column comes twice
+                    // (such a row stays with the fragments, where the last of the two counts)
+                    uint64_t seen = 0;
+                    for (int p = p0; p < p0 + n; ++p) seen |= 1ull << (P->descColId[P->ddColInd[p]] - lo);
+                    if (__builtin_popcountll(seen) == n) cand.push_back({lo, n, i});
                 }
                 std::sort(cand.begin(), cand.end(), [](const Cand &a, const Cand &b) {
                     return a.c0 != b.c0 ? a.c0 < b.c0 : a.n != b.n ? a.n < b.n : a.i < b.i;
@@ -1175,7 +1179,11 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             for (int i = 0; i < P->dRows; ++i) {
                 int n = 0;
                 for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
-                    keep[p] = (!taken.empty() && taken[i]) ? 0 : !sel[frag_of(i / fragM, P->ddColInd[p])];
+                    // Of entries that name the same column twice the tile format holds the last
+                    // (generateFormat_opt overwrites, test/test_autotc_spmv.cpp:718-847); the
+                    // earlier ones go to the CSR part, so that y is the sum of all of them.
+                    const bool earlierTwin = p + 1 < P->ddRowPtr[i + 1] && P->ddColInd[p + 1] == P->ddColInd[p];
+                    keep[p] = (!taken.empty() && taken[i]) ? 0 : (earlierTwin || !sel[frag_of(i / fragM, P->ddColInd[p])]);
                     n += keep[p];
                 }
                 rowPtr[P->rId[i] + 1] += n;

@@ -457,6 +457,42 @@ def test_tile_kernel_step_packing(mx, ora):
                 part.close()
 
 
+def test_columns_named_twice_in_a_row_are_summed(mx, ora):
+    """The tile format keeps one value per (row, column) -- the last, as the reference's does; the
+    plan sends the earlier ones to the CSR part, so y is the sum over all entries, as in
+    spmv_serial.  Rows in any column order, a column up to four times in a row, a strip row with
+    one column twice."""
+    import torch
+    rng = np.random.default_rng(77)
+    for dtype, tol in ((np.float64, F64_TOL), (np.float16, F16_TOL)):
+        rows, cols = 700, 96
+        lens = rng.integers(0, 60, rows)
+        lens[8:16] = 32
+        rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        ci = rng.integers(0, cols, rp[-1]).astype(np.int32)     # with replacement
+        # rows 8..15: columns 32..63 once each, except that 33 is named as 32 (a strip row but for that)
+        for r in range(8, 16):
+            c = np.arange(32, 64)
+            c[1] = 32
+            ci[rp[r]:rp[r + 1]] = c
+        # small integers: every sum is exact in both precisions, whatever the order
+        va = rng.integers(-3, 4, rp[-1]).astype(dtype)
+        A = mx.Csr(rows, cols, rp, ci, va)
+        x = rng.integers(-2, 3, cols).astype(dtype)
+        ref = oracle_y(ora, mx, A, x)
+        xd = torch.from_numpy(x).cuda()
+        for tau in ((1.0, 1.0), (0.75, 0.5)):
+            for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES):
+                print("twice-named columns dtype=%s tau=%s flags=%d" % (dtype.__name__, tau, fl), flush=True)
+                part = mx.Partition(A, *tau)
+                plan = mx.Plan(part, fl)
+                y = plan.spmv(xd)
+                torch.cuda.synchronize()
+                assert np.array_equal(y.cpu().numpy().astype(np.float64), ref.astype(np.float64)), (tau, fl, plan.info)
+                plan.close()
+                part.close()
+
+
 def test_plan_from_a_saved_partition(mx, ora, tmp_path):
     """A partition that went through a file gives the same plan (and the same y, bit for bit)."""
     import torch
