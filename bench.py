@@ -243,6 +243,25 @@ def main():
         "best_hybrid": main_rec["best_hybrid"],
         "sweep": main_rec["sweep"],
     }
+    # what a plain device copy reaches on this GPU, next to the 8 TB/s the roofline is priced at:
+    # read + written bytes over the time of back-to-back copies, at this workload's algorithmic
+    # size and at 1 GiB
+    copy = {}
+    for label, nbytes in (("workload_sized", int(main_rec["roofline"]["bytes_per_launch"]) // 2), ("1GiB", 1 << 29)):
+        src = torch.ones(nbytes // 4, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 200 if nbytes < (1 << 27) else 20
+        e0.record()
+        for _ in range(reps):
+            dst.copy_(src)
+        e1.record()
+        torch.cuda.synchronize()
+        copy[label] = {"bytes_read_plus_written": 2 * (nbytes // 4) * 4, "GBs": 2 * (nbytes // 4) * 4 / (e0.elapsed_time(e1) / reps * 1e-3) / 1e9}
+        del src, dst
+    out["device_copy"] = copy
     if args.calibrate_copy:
         n = args.calibrate_copy * (1 << 20) // 4
         src = torch.ones(n, dtype=torch.float32, device="cuda:0")
