@@ -133,6 +133,26 @@ def test_full_size_workloads_match_oracle(mx, ora, cfg, taus):
             part.close()
 
 
+def test_full_size_mixed_workload_with_its_strips(mx, ora):
+    """Workload 5 at the point the benchmark picks, tau = (1, 1): the 20 % strip rows run through
+    the strip form of the binary16 tile kernel (26.8 M entries), everything else through the CSR
+    part; y against the oracle."""
+    import torch
+    A, x = mx.gen_config(5)
+    ref = oracle_y(ora, mx, A, x)
+    part = mx.Partition(A, 1.0, 1.0)
+    plan = mx.Plan(part)
+    info = plan.info
+    print("workload 5 tau=(1,1):", info, flush=True)
+    assert info["tile_variant"] == 1 and info["tile_strip_nnz"] > 0.4 * A.nnz
+    assert info["tile_nnz"] + info["csr_nnz"] == A.nnz
+    y = plan.spmv(torch.from_numpy(x).cuda())
+    torch.cuda.synchronize()
+    assert rel_l2(y.cpu().numpy(), ref) <= F16_TOL
+    plan.close()
+    part.close()
+
+
 def test_full_size_stencil_closed_form(mx):
     """100^3 27-point stencil times the all-ones vector: 26 - #neighbours, exactly."""
     import torch
