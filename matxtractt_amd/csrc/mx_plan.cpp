@@ -1032,6 +1032,19 @@ static double tile_gate(mx_dtype)
     return 0.5;
 }
 
+// MX_PLAN_LOG=1: the phases of mx_plan_create with their host time, on stderr
+struct PhaseLog {
+    bool on = std::getenv("MX_PLAN_LOG") && std::atoi(std::getenv("MX_PLAN_LOG"));
+    std::chrono::steady_clock::time_point t = std::chrono::steady_clock::now();
+    void operator()(const char *what)
+    {
+        if (!on) return;
+        const auto now = std::chrono::steady_clock::now();
+        std::fprintf(stderr, "mx_plan_create: %-28s %8.1f ms\n", what, std::chrono::duration<double, std::milli>(now - t).count());
+        t = now;
+    }
+};
+
 extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
 {
     if (!P || !out) {
@@ -1061,10 +1074,12 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
         set_error("mx_plan_create: could not create stream/events");
         return fail(MX_ERR_DEVICE);
     }
+    PhaseLog phase;
     try {
         if (!P->extracted) {
             rc = setup_csr_part(plan, P->cdRowPtr.data(), P->cdColInd.data(), P->cdVal.data(), flags);
             if (rc) return fail(rc);
+            phase("CSR part (layouts, trial)");
         } else {
             // residual column space -> the caller's column ids, so x needs no permutation
             std::vector<int> colOrig(cols);
@@ -1146,6 +1161,7 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                 }
                 if (stripChunks.empty()) taken.clear();
             }
+            phase("fragment gate, strip rows");
             if (!taken.empty()) {
                 // the gate again, on what the taken rows leave of each fragment
 #pragma omp parallel for schedule(static)
@@ -1161,29 +1177,38 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                     }
                 }
             }
-            // fragment of every A_dd entry: the rank of its column among the chunk's columns, / fragK
-            auto frag_of = [&](int w, int ddcol) {
+            // fragment of every A_dd entry: the rank of its column among the chunk's columns, / fragK.
+            // The used prefix of a chunk's column list is ascending (the zero padding after it is
+            // not), and so are the columns of a row of A_dd: one walk over both.
+            std::vector<int> usedCols((size_t)chunkNum, 0);
+#pragma omp parallel for schedule(static)
+            for (int w = 0; w < chunkNum; ++w) {
                 const int f0 = P->chunkPtr[w], f1 = P->chunkPtr[w + 1];
                 const int *a = &P->sparse_AToX_index[(size_t)f0 * fragK];
-                // the used prefix of the chunk's list is ascending; the zero padding after it is not
                 int n = (f1 - f0) * fragK;
                 while (n > 1 && a[n - 1] == 0) --n;
-                const int rank = (int)(std::lower_bound(a, a + n, ddcol) - a);
-                return f0 + rank / fragK;
-            };
+                usedCols[w] = n;
+            }
             // CSR part = residual rows + the A_dd entries whose fragment stays out of the tile kernel
             std::vector<int> rowPtr((size_t)rows + 1, 0);
             for (int r = 0; r < rows; ++r) rowPtr[r + 1] = P->cdRowPtr[r + 1] - P->cdRowPtr[r];
             std::vector<char> keep((size_t)P->ddRowPtr[P->dRows], 0);  // A_dd entry goes to the CSR part
-#pragma omp parallel for schedule(static)
+            // (rows of A_dd come longest first: small dynamic pieces, not one static range per thread)
+#pragma omp parallel for schedule(dynamic, 512)
             for (int i = 0; i < P->dRows; ++i) {
-                int n = 0;
+                const int w = i / fragM, f0 = P->chunkPtr[w];
+                const int *a = &P->sparse_AToX_index[(size_t)f0 * fragK];
+                const int na = usedCols[w];
+                const bool rowTaken = !taken.empty() && taken[i];
+                int n = 0, rank = 0;
                 for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
+                    const int c = P->ddColInd[p];
+                    while (rank < na && a[rank] < c) ++rank;
                     // Of entries that name the same column twice the tile format holds the last
                     // (generateFormat_opt overwrites, test/test_autotc_spmv.cpp:718-847); the
                     // earlier ones go to the CSR part, so that y is the sum of all of them.
-                    const bool earlierTwin = p + 1 < P->ddRowPtr[i + 1] && P->ddColInd[p + 1] == P->ddColInd[p];
-                    keep[p] = (!taken.empty() && taken[i]) ? 0 : (earlierTwin || !sel[frag_of(i / fragM, P->ddColInd[p])]);
+                    const bool earlierTwin = p + 1 < P->ddRowPtr[i + 1] && P->ddColInd[p + 1] == c;
+                    keep[p] = rowTaken ? 0 : (earlierTwin || !sel[f0 + rank / fragK]);
                     n += keep[p];
                 }
                 rowPtr[P->rId[i] + 1] += n;
@@ -1202,7 +1227,7 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                     std::memcpy(&val[(size_t)q * es], cdv + (size_t)p * es, es);
                 }
             }
-#pragma omp parallel for schedule(static)
+#pragma omp parallel for schedule(dynamic, 512)
             for (int i = 0; i < P->dRows; ++i) {
                 const int r = P->rId[i];
                 int q = rowPtr[r] + (P->cdRowPtr[r + 1] - P->cdRowPtr[r]);
@@ -1213,8 +1238,10 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                     ++q;
                 }
             }
+            phase("CSR part assembled");
             rc = setup_csr_part(plan, rowPtr.data(), col.data(), val.data(), flags);
             if (rc) return fail(rc);
+            phase("CSR part (layouts, trial)");
 
             // tile part: the selected chunks; columns and rows back in the caller's numbering
             const void *bits = P->dtype == MX_F64 ? (const void *)P->fragBit32.data() : (const void *)P->fragBit64.data();
@@ -1233,6 +1260,7 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                 plan->strips.ownedRows = true;
             }
             plan->tile_nnz = nnzGeneral + nnzStrips;
+            phase("tile layouts");
         }
     } catch (const std::bad_alloc &) {
         set_error("mx_plan_create: out of memory");
