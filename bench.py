@@ -81,8 +81,10 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
     if only_tau is not None:
         points = [tuple(only_tau)]  # nothing else: a profile of this run then shows one plan's kernels only
     table = []
+    # (MX_PLAN_KEEP_TILES: every point runs the hybrid its fragments give, also where the plan's own
+    # estimate would send everything through the CSR part; what that estimate says is recorded below)
     for tau in points:
-        part, plan, rec = measure(mx, torch, A, xd, yd, tau, 20, 200)
+        part, plan, rec = measure(mx, torch, A, xd, yd, tau, 20, 200, mx.MX_PLAN_KEEP_TILES)
         table.append(rec)
         log("  tau=(%.2f,%.2f) total %.2f us (tile %.2f + csr %.2f) tile_nnz=%d" %
             (tau[0], tau[1], rec["ms_total"] * 1e3, rec["ms_tile"] * 1e3, rec["ms_csr"] * 1e3, rec["tile_nnz"]))
@@ -98,7 +100,13 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
 
     # the timed run on the best point: W warm-up steps, then exactly K steps between syncs
     tau = (best["tau_c"], best["tau_r"])
-    part, plan, _ = measure(mx, torch, A, xd, yd, tau, 5, 20)
+    if best_hybrid:
+        p2 = mx.Partition(A, best_hybrid["tau_c"], best_hybrid["tau_r"])
+        q2 = mx.Plan(p2)  # default flags: the plan's own decision at the best hybrid point
+        best_hybrid["default_plan_keeps_tiles"] = q2.info["tile_nnz"] > 0
+        q2.close()
+        p2.close()
+    part, plan, _ = measure(mx, torch, A, xd, yd, tau, 5, 20, mx.MX_PLAN_KEEP_TILES)
     plan.spmv_repeat(xd, yd, warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -151,7 +159,7 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
                               "the quoted value is the back-to-back (warm) one"},
         "rel_l2_vs_oracle": rel_l2,
         "csr_only_ms": csr_only and csr_only["ms_total"],
-        "best_hybrid": best_hybrid and {k: best_hybrid[k] for k in ("tau_c", "tau_r", "ms_total", "tile_nnz", "csr_nnz")},
+        "best_hybrid": best_hybrid and {k: best_hybrid[k] for k in ("tau_c", "tau_r", "ms_total", "tile_nnz", "csr_nnz", "default_plan_keeps_tiles")},
         "roofline": {"bound": "hbm", "kernel": dom["kernel"], "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK,
                      "traffic": TRAFFIC.get((cfg, dom["kernel"], info["tile_nnz"] > 0)),

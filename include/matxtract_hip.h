@@ -151,6 +151,12 @@ double mx_algorithmic_bytes(mx_dtype dtype, int rows, int cols, int nnz);
 #define MX_PLAN_ALL_TILES 2  /* run every extracted chunk through the MFMA tile kernel */
 #define MX_PLAN_CSR_ROWS 4   /* CSR part: force the row-tile kernel (direct x gathers) */
 #define MX_PLAN_CSR_SLICES 8 /* CSR part: prefer the column-slice kernel (x resident in LDS) when the matrix suits it */
+#define MX_PLAN_KEEP_TILES 16 /* keep the tiles that the per-fragment fill gate selects.  Without this flag (and
+                                 without MX_PLAN_ALL_TILES) a plan also asks whether the tiles pay for their
+                                 own launch -- the entries they take off the CSR part against the bytes they
+                                 stream themselves, at rates measured on MI355X -- and runs everything through
+                                 the CSR part when they do not (the reference gates its tile kernel on matrix
+                                 size and fill, test/test_autotc_spmv.cpp:1507,1518) */
 
 /* Uploads a partition once and keeps it on the device: the persistent counterpart of the
  * per-call cudaMalloc/cudaMemcpy blocks in cdspmv (src/spmv_kernel/cdSpMV.cu:407-418) and

@@ -13,7 +13,7 @@ CSRC = os.path.join(_HERE, "csrc")
 MX_OK, MX_ERR_ARG, MX_ERR_ALLOC, MX_ERR_DEVICE, MX_ERR_IO = 0, 1, 2, 3, 4
 MX_F64, MX_F16 = 0, 1
 MX_PLAN_DEFAULT, MX_PLAN_NO_TILES, MX_PLAN_ALL_TILES = 0, 1, 2
-MX_PLAN_CSR_ROWS, MX_PLAN_CSR_SLICES = 4, 8
+MX_PLAN_CSR_ROWS, MX_PLAN_CSR_SLICES, MX_PLAN_KEEP_TILES = 4, 8, 16
 
 
 class MxError(RuntimeError):

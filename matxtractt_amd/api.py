@@ -12,12 +12,12 @@ import numpy as np
 
 from . import _lib
 from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLAN_CSR_ROWS, MX_PLAN_DEFAULT,
-                   MX_PLAN_NO_TILES, MxError, check)
+                   MX_PLAN_KEEP_TILES, MX_PLAN_NO_TILES, MxError, check)
 
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
-           "MX_PLAN_CSR_SLICES"]
+           "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES"]
 
 
 def _p(a):

@@ -112,6 +112,7 @@ int main(int argc, char **argv)
         else if (a == "--keep-values") keepValues = true;
         else if (a == "--no-tiles") planFlags = MX_PLAN_NO_TILES;
         else if (a == "--all-tiles") planFlags = MX_PLAN_ALL_TILES;
+        else if (a == "--keep-tiles") planFlags = MX_PLAN_KEEP_TILES;
         else if (a == "--json") json = true;
         else if (a == "--partition-cache") cachePath = next("--partition-cache");
         else if (a == "--tune") tune = true;

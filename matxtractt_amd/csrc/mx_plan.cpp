@@ -1177,6 +1177,46 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                     }
                 }
             }
+            // Do the tiles pay for their launch?  (The reference gates its tile kernel on the size
+            // of the matrix and its fill, test/test_autotc_spmv.cpp:1507,1518.)  What they take off
+            // the CSR part saves es + 2 bytes per entry of its stream; what they cost is a launch
+            // and their own stream.  Rates as measured on MI355X: the CSR part and the strip
+            // form of the tile kernel move about 5 bytes per ns, the general tile kernel, bound
+            // by instruction issue, about 2.2.  MX_PLAN_KEEP_TILES skips the question.
+            if (!(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES | MX_PLAN_KEEP_TILES))) {
+                double generalEntries = 0, generalFrags = 0, stripEntries = 0, stripBlocks = 0;
+                for (int w = 0; w < chunkNum; ++w) {
+                    uint64_t rowsLeft = ~0ull;
+                    if (!taken.empty())
+                        for (int r = 0; r < fragM; ++r) {
+                            const int i = w * fragM + r;
+                            if (i < P->dRows && taken[i]) rowsLeft &= ~(0xffull << (r * fragK));
+                        }
+                    for (int f = P->chunkPtr[w]; f < P->chunkPtr[w + 1]; ++f) {
+                        if (!sel[f]) continue;
+                        generalFrags += 1;
+                        generalEntries += taken.empty() ? P->fragPtr[f + 1] - P->fragPtr[f]
+                                                        : __builtin_popcountll(P->fragBit64[f] & rowsLeft);
+                    }
+                }
+                for (const StripChunk &C : stripChunks) {
+                    stripEntries += C.nnz;
+                    stripBlocks += (double)C.blocks.size();
+                }
+                const double blockBytes = (double)fragM * fragK * es, slots = mx::tile_slots(P->dtype);
+                const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
+                const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
+                const double launchNs = 2500.0;
+                const double savedNs = (generalEntries + stripEntries) * (es + 2) / 5.0;
+                const double costNs = (generalFrags > 0 ? launchNs + generalBytes / 2.2 : 0.0) + (stripBlocks > 0 ? launchNs + stripBytes / 5.0 : 0.0);
+                if (savedNs <= costNs) {
+                    std::fill(sel.begin(), sel.end(), 0);
+                    stripChunks.clear();
+                    taken.clear();
+                } else if (generalFrags > 0 && generalEntries * (es + 2) / 5.0 <= launchNs + generalBytes / 2.2) {
+                    std::fill(sel.begin(), sel.end(), 0);  // the strips pay, the general tiles do not
+                }
+            }
             // fragment of every A_dd entry: the rank of its column among the chunk's columns, / fragK.
             // The used prefix of a chunk's column list is ascending (the zero padding after it is
             // not), and so are the columns of a row of A_dd: one walk over both.

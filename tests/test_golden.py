@@ -91,7 +91,7 @@ def test_plans_give_the_fixtures_y(mx, dtype):
                    np.array(fx["val"], dtype))
         xd = torch.from_numpy(np.array(fx["x"], dtype)).cuda()
         for tau in ((fx["tau_c"], fx["tau_r"]), (0.0, 0.0)):
-            for flags in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES):
+            for flags in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_ALL_TILES):
                 print("golden", fx["name"], np.dtype(dtype).name, tau, flags, flush=True)
                 P = mx.Partition(A, *tau)
                 plan = mx.Plan(P, flags)

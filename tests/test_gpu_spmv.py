@@ -72,14 +72,15 @@ TAUS = [(0.0, 0.0), (0.5, 0.25), (1.0, 1.0), (0.75, 0.0), (0.25, 0.25), (1.0, 0.
 
 
 @pytest.mark.parametrize("cfg,scale", CASES)
-@pytest.mark.parametrize("flags", ["default", "no_tiles", "all_tiles", "all_tiles+csr_rows", "all_tiles+csr_slices",
-                                   "no_tiles+csr_slices"])
+@pytest.mark.parametrize("flags", ["default", "keep_tiles", "no_tiles", "all_tiles", "all_tiles+csr_rows",
+                                   "all_tiles+csr_slices", "no_tiles+csr_slices"])
 def test_hybrid_spmv_matches_oracle(mx, ora, cfg, scale, flags):
     import torch
     A, x = mx.gen_config(cfg, scale=scale)
     ref = oracle_y(ora, mx, A, x)
     tol = F64_TOL if A.dtype == mx.MX_F64 else F16_TOL
-    bits = {"default": mx.MX_PLAN_DEFAULT, "no_tiles": mx.MX_PLAN_NO_TILES, "all_tiles": mx.MX_PLAN_ALL_TILES,
+    bits = {"default": mx.MX_PLAN_DEFAULT, "keep_tiles": mx.MX_PLAN_KEEP_TILES, "no_tiles": mx.MX_PLAN_NO_TILES,
+            "all_tiles": mx.MX_PLAN_ALL_TILES,
             "csr_rows": mx.MX_PLAN_CSR_ROWS, "csr_slices": mx.MX_PLAN_CSR_SLICES}
     fl = 0
     for name in flags.split("+"):
@@ -151,6 +152,28 @@ def test_full_size_mixed_workload_with_its_strips(mx, ora):
     assert rel_l2(y.cpu().numpy(), ref) <= F16_TOL
     plan.close()
     part.close()
+
+
+def test_plan_asks_whether_tiles_pay(mx, ora):
+    """Default flags: the plan keeps the selected tiles only when what they take off the CSR part
+    outweighs their own launch and stream.  On the small block-clustered matrix they do not (one
+    launch less, same y); MX_PLAN_KEEP_TILES keeps them."""
+    import torch
+    A, x = mx.gen_config(2, scale=1 / 16)
+    ref = oracle_y(ora, mx, A, x)
+    xd = torch.from_numpy(x).cuda()
+    part = mx.Partition(A, 1.0, 1.0)
+    seen = {}
+    for name, fl in (("default", mx.MX_PLAN_DEFAULT), ("keep", mx.MX_PLAN_KEEP_TILES)):
+        plan = mx.Plan(part, fl)
+        seen[name] = plan.info["tile_nnz"]
+        assert plan.info["tile_nnz"] + plan.info["csr_nnz"] == A.nnz
+        y = plan.spmv(xd)
+        torch.cuda.synchronize()
+        assert rel_l2(y.cpu().numpy(), ref) <= F64_TOL
+        plan.close()
+    part.close()
+    assert seen["default"] == 0 and seen["keep"] > 0, seen
 
 
 def test_full_size_stencil_closed_form(mx):
@@ -464,7 +487,7 @@ def test_tile_kernel_step_packing(mx, ora):
         ref = oracle_y(ora, mx, A, x)
         xd = torch.from_numpy(x).cuda()
         for tau in ((1.0, 1.0), (1.0, 0.5), (0.5, 0.5)):
-            for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES):
+            for fl in (mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_ALL_TILES):
                 print("tile packing dtype=%s tau=%s flags=%d" % (dtype.__name__, tau, fl), flush=True)
                 part = mx.Partition(A, *tau)
                 plan = mx.Plan(part, fl)
@@ -502,7 +525,7 @@ def test_columns_named_twice_in_a_row_are_summed(mx, ora):
         ref = oracle_y(ora, mx, A, x)
         xd = torch.from_numpy(x).cuda()
         for tau in ((1.0, 1.0), (0.75, 0.5)):
-            for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES):
+            for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_ALL_TILES):
                 print("twice-named columns dtype=%s tau=%s flags=%d" % (dtype.__name__, tau, fl), flush=True)
                 part = mx.Partition(A, *tau)
                 plan = mx.Plan(part, fl)
@@ -575,7 +598,7 @@ def test_strip_form_of_the_fp16_tile_kernel(mx, ora, monkeypatch):
         P = mx.Partition(A, 1.0, 1.0)
         for variant in ("rows", "slices"):
             monkeypatch.setenv("MX_CSR_KERNEL", variant)
-            plan = mx.Plan(P)
+            plan = mx.Plan(P, mx.MX_PLAN_KEEP_TILES)   # a matrix this small would otherwise go without tiles
             print("strip form:", name, variant, "tile_nnz", plan.info["tile_nnz"], "in strips", plan.info["tile_strip_nnz"], flush=True)
             assert plan.info["tile_nnz"] > 0.5 * A.nnz
             sn, tn = plan.info["tile_strip_nnz"], plan.info["tile_nnz"]
@@ -599,7 +622,7 @@ def test_tau_tuner(mx, ora):
     candidates without tiles share one timing and are reported as (0, 0)."""
     import torch
     A, x = mx.gen_config(5, scale=1 / 128)
-    tc, tr, table = mx.tune_tau(A, levels=3, warm=2, iters=10)
+    tc, tr, table = mx.tune_tau(A, levels=3, flags=mx.MX_PLAN_KEEP_TILES, warm=2, iters=10)
     assert [(c, r) for c, r, _, _ in table] == [(0.0, 0.0), (0.5, 0.0), (0.5, 0.5), (1.0, 0.0), (1.0, 0.5), (1.0, 1.0)]
     assert all(ms > 0 for _, _, ms, _ in table)
     no_tiles = [ms for _, _, ms, n in table if n == 0]
@@ -608,7 +631,7 @@ def test_tau_tuner(mx, ora):
     assert (tc, tr) == ((best[0], best[1]) if best[3] > 0 else (0.0, 0.0))
     assert any(n > 0 for _, _, _, n in table), "the strips of this workload fill whole fragments"
     P = mx.Partition(A, tc, tr)
-    plan = mx.Plan(P)
+    plan = mx.Plan(P, mx.MX_PLAN_KEEP_TILES)
     y = plan.spmv(torch.from_numpy(x).cuda()).cpu().numpy()
     assert rel_l2(y, oracle_y(ora, mx, A, x)) <= F16_TOL
     plan.close()
