@@ -617,6 +617,42 @@ def test_strip_form_of_the_fp16_tile_kernel(mx, ora, monkeypatch):
         P.close()
 
 
+def test_spmv_in_a_hip_graph(mx, ora):
+    """mx_spmv only queues kernels on the stream it is given (no allocation, no memset, no
+    synchronisation), so a caller can capture it into a HIP graph.  The captured hybrid (CSR part
+    in slice form + both tile kernels) is replayed on new contents of x, with eager work and
+    synchronisations between the replays, and every replay is checked."""
+    import torch
+    A, x = mx.gen_config(5, scale=1 / 32)
+    P = mx.Partition(A, 1.0, 1.0)
+    plan = mx.Plan(P, mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_SLICES)
+    assert plan.info["tile_nnz"] > 0 and plan.info["csr_variant"] == 1
+    xs = torch.from_numpy(x).cuda()
+    ys = torch.zeros(A.rows, dtype=xs.dtype, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        plan.spmv(xs, ys)                     # once outside the capture (lazy initialisation inside the runtime)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        plan.spmv(xs, ys)                     # launches on torch's current stream: the capturing one
+    rng = np.random.default_rng(3)
+    for rep in range(4):
+        xn = rng.uniform(-1, 1, A.cols).astype(np.float16)
+        xs.copy_(torch.from_numpy(xn).cuda())
+        ys.fill_(7.0)
+        g.replay()
+        torch.cuda.synchronize()
+        got = ys.cpu().numpy()
+        eager = plan.spmv(xs).cpu().numpy()
+        assert np.array_equal(got.view(np.uint16), eager.view(np.uint16)), rep
+        assert rel_l2(got, oracle_y(ora, mx, A, xn)) <= F16_TOL
+    plan.close()
+    P.close()
+
+
 def test_tau_tuner(mx, ora):
     """mx_tune_tau walks the grid with tau_c >= tau_r, reports every candidate, returns the fastest;
     candidates without tiles share one timing and are reported as (0, 0)."""
