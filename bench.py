@@ -175,7 +175,14 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
             runner()
             reps.append(time.perf_counter() - t0)
         t_cpu = min(reps[2:])
+        cpu_model = "unknown"
+        try:
+            with open("/proc/cpuinfo") as f:
+                cpu_model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "unknown")
+        except OSError:
+            pass
         rec["cpu_baseline"] = {"value": 2.0 * A.nnz / t_cpu / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+                               "cpu": cpu_model, "cpus_visible": len(os.sched_getaffinity(0)),
                                "sample": "the full matrix of this workload, best of 10 after 2 warm-ups "
                                          "(%.1f ms per SpMV), single thread as the reference's spmv_serial" % (t_cpu * 1e3)}
         # not the reference's: the same oracle routine over nnz-balanced row ranges, one thread per
