@@ -118,8 +118,13 @@ inline int slice_step_entries(mx_dtype) { return 1; }  // entries a lane takes p
 constexpr int kSliceLightSegs = 8;     // rows with at most this many virtual rows are summed by one lane
 
 // `what`: 0 = slice kernel then combine kernel, 1 = slice kernel only, 2 = combine kernel only
+// `strips` (optional): a tile layout in the dense binary16 form whose steps workgroups of the
+// combine kernel's launch run as well (strips_can_ride says whether a layout may); the rows of
+// those strips must be marked in the slice layout (rowInfo -2) so that the combine kernel leaves
+// them alone.
 hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
-                         int what = 0);
+                         int what = 0, const DeviceTiles *strips = nullptr);
+bool strips_can_ride(mx_dtype dtype, const DeviceTiles &T, const void *x);
 hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s);
 hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s);
 hipError_t launch_probe_f64(const double *A, const double *B, double *D, hipStream_t s);

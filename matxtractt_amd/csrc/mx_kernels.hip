@@ -596,87 +596,6 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         if (t + NB + k < nb) consume(buf[k], t + NB + k);
 }
 
-// The sums of the virtual rows become y in one launch of three kinds of workgroups:
-//  * the first `nRowWG` walk the matrix rows, kCombineRows per lane: rowInfo[r] >= 0 names the one virtual
-//    row of row r, whose sum is the row's result; -1 is a row without entries (zero, or left
-//    alone when `skipEmpty`); anything else a row that the lists below cover;
-//  * the next `nLightWG` take the rows with 2..kSliceLightSegs virtual rows, one lane each: the
-//    row and its kSliceLightSegs indices into `partial` (-1 = none) lie at the lane's own place in
-//    two arrays, so nothing the lane loads depends on another load but the sums themselves;
-//  * the rest take the rows with more, sixteen lanes each.
-constexpr int kCombineRows = 16;  // rows a lane of the first kind takes
-template <typename VT>
-__global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Acc<VT>::type *__restrict__ partial,
-                                                              const int *__restrict__ rowInfo, int rows, int nRowWG,
-                                                              const int *__restrict__ lightRow,
-                                                              const int4 *__restrict__ lightIdx, int nLight, int nLightWG,
-                                                              const int4 *__restrict__ heavyInfo, int nHeavy,
-                                                              const int *__restrict__ segIdx, VT *__restrict__ y,
-                                                              int accumulate, int skipEmpty)
-{
-    typedef typename Acc<VT>::type AT;
-    const int tid = threadIdx.x;
-    // Every kind of workgroup walks its rows in ascending order, and the sums of neighbouring rows
-    // lie close together wherever their virtual rows fall into the same slice and length class:
-    // one XCD per contiguous range of rows keeps those sectors in a single L2.
-    int b = blockIdx.x;
-    const int nHeavyWG = (int)gridDim.x - nRowWG - nLightWG;
-    if (b < nRowWG) b = xcd_contiguous_block(b, nRowWG);
-    else if (b < nRowWG + nLightWG) b = nRowWG + xcd_contiguous_block(b - nRowWG, nLightWG);
-    else b = nRowWG + nLightWG + xcd_contiguous_block(b - nRowWG - nLightWG, nHeavyWG);
-    if (b < nRowWG) {
-        // kCombineRows rows per lane, as quads a wave apart so that its loads and stores stay contiguous
-        int dd[kCombineRows];
-#pragma unroll
-        for (int q = 0; q < kCombineRows / 4; ++q) {
-            const int r0 = 4 * ((b * (kCombineRows / 4) + q) * kBlock + tid);
-            const int4 d = r0 < rows ? ((const int4 *)rowInfo)[r0 >> 2] : int4{-2, -2, -2, -2};  // padded with -2
-            dd[4 * q] = d.x, dd[4 * q + 1] = d.y, dd[4 * q + 2] = d.z, dd[4 * q + 3] = d.w;
-        }
-        AT sum[kCombineRows];
-#pragma unroll
-        for (int j = 0; j < kCombineRows; ++j) sum[j] = dd[j] >= 0 ? partial[dd[j]] : (AT)0;
-#pragma unroll
-        for (int j = 0; j < kCombineRows; ++j) {
-            const int r = 4 * ((b * (kCombineRows / 4) + j / 4) * kBlock + tid) + j % 4;
-            const bool mine = dd[j] >= 0 || (dd[j] == -1 && !skipEmpty);
-            if (mine && accumulate) sum[j] += (AT)y[r];
-            if (mine) y[r] = (VT)sum[j];
-        }
-        return;
-    }
-    b -= nRowWG;
-    if (b < nLightWG) {
-        const int i = b * kBlock + tid;
-        if (i >= nLight) return;
-        static_assert(mx::kSliceLightSegs == 8, "two int4 of indices per light row");
-        const int r = lightRow[i];
-        const int4 i0 = lightIdx[2 * i], i1 = lightIdx[2 * i + 1];
-        const int id[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
-        AT sum = accumulate ? (AT)y[r] : (AT)0;
-#pragma unroll
-        for (int k = 0; k < 8; ++k)
-            if (id[k] >= 0) sum += partial[id[k]];
-        y[r] = (VT)sum;
-        return;
-    }
-    b -= nLightWG;
-    const int g = b * (kBlock / 16) + (tid >> 4), sub = tid & 15;
-    const bool live = g < nHeavy;
-    const int4 h = live ? heavyInfo[g] : int4{0, 0, 0, 0};
-    AT sum = 0;
-    for (int k = sub; k < h.z; k += 64) {
-        int id[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) id[j] = k + 16 * j < h.z ? segIdx[h.y + k + 16 * j] : -1;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (id[j] >= 0) sum += partial[id[j]];
-    }
-    sum = group_sum<16>(sum);
-    if (live && sub == 0) y[h.x] = (VT)(sum + (accumulate ? (AT)y[h.x] : (AT)0));
-}
-
 // ---- tile part --------------------------------------------------------------------------
 // The selected fragments arrive expanded to full blocks and regrouped into steps (see
 // DeviceTiles): what one wave hands to the matrix core at a time.  A wave owns a run of steps
@@ -861,14 +780,11 @@ struct DenseStep {
     int hdr;      // header dword lane%32
     v4i32 v, b;   // A operand (one block row), B operand (the eight x of the lane's block)
 };
-__global__ __launch_bounds__(kBlock) void tile_dense_kernel(const int4 *__restrict__ waveDesc, const int *__restrict__ hdr,
-                                                           const _Float16 *__restrict__ tcVal,
-                                                           const _Float16 *__restrict__ x, _Float16 *__restrict__ y,
-                                                           int nWaves)
+// One wave's range of steps (wave `gw` of the layout).
+__device__ __forceinline__ void tile_dense_wave(const int4 *__restrict__ waveDesc, const int *__restrict__ hdr,
+                                                const _Float16 *__restrict__ tcVal, const _Float16 *__restrict__ x,
+                                                _Float16 *__restrict__ y, int gw, int lane)
 {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int gw = xcd_contiguous_block(blockIdx.x, gridDim.x) * (kBlock / 64) + wave;
-    if (gw >= nWaves) return;
     const int4 d0 = waveDesc[2 * gw], d1 = waveDesc[2 * gw + 1];
     const int s0 = __builtin_amdgcn_readfirstlane(d0.x), s1 = __builtin_amdgcn_readfirstlane(d0.y);
     if (s0 >= s1) return;
@@ -924,6 +840,112 @@ __global__ __launch_bounds__(kBlock) void tile_dense_kernel(const int4 *__restri
         if (s + 3 < s1) step(s + 3, R3, R0, R2);
         if (s + 4 < s1) step(s + 4, R4, R1, R3);
     }
+}
+
+__global__ __launch_bounds__(kBlock) void tile_dense_kernel(const int4 *__restrict__ waveDesc, const int *__restrict__ hdr,
+                                                           const _Float16 *__restrict__ tcVal,
+                                                           const _Float16 *__restrict__ x, _Float16 *__restrict__ y,
+                                                           int nWaves)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gw = xcd_contiguous_block(blockIdx.x, gridDim.x) * (kBlock / 64) + wave;
+    if (gw < nWaves) tile_dense_wave(waveDesc, hdr, tcVal, x, y, gw, lane);
+}
+
+// The sums of the virtual rows become y in one launch of three kinds of workgroups:
+//  * the first `nRowWG` walk the matrix rows, kCombineRows per lane: rowInfo[r] >= 0 names the one virtual
+//    row of row r, whose sum is the row's result; -1 is a row without entries (zero, or left
+//    alone when `skipEmpty`); anything else a row that the lists below cover;
+//  * the next `nLightWG` take the rows with 2..kSliceLightSegs virtual rows, one lane each: the
+//    row and its kSliceLightSegs indices into `partial` (-1 = none) lie at the lane's own place in
+//    two arrays, so nothing the lane loads depends on another load but the sums themselves;
+//  * the rest take the rows with more, sixteen lanes each.
+constexpr int kCombineRows = 16;  // rows a lane of the first kind takes
+template <typename VT>
+__global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Acc<VT>::type *__restrict__ partial,
+                                                              const int *__restrict__ rowInfo, int rows, int nRowWG,
+                                                              const int *__restrict__ lightRow,
+                                                              const int4 *__restrict__ lightIdx, int nLight, int nLightWG,
+                                                              const int4 *__restrict__ heavyInfo, int nHeavy,
+                                                              const int *__restrict__ segIdx, VT *__restrict__ y,
+                                                              int accumulate, int skipEmpty,
+                                                              const int4 *__restrict__ stripWaveDesc,
+                                                              const int *__restrict__ stripHdr,
+                                                              const VT *__restrict__ stripVal, const VT *__restrict__ x,
+                                                              int nStripWaves, int nStripWG, int nHeavyWG)
+{
+    typedef typename Acc<VT>::type AT;
+    const int tid = threadIdx.x;
+    // A fourth kind of workgroup, first in the grid: the strips of a binary16 plan (the work of
+    // tile_dense_kernel), which need nothing from the sums and write rows that the other kinds
+    // leave alone (rowInfo -2).  In one launch they cost no dependent launch of their own.  (Spread
+    // evenly among the other kinds instead of ahead of them they cost more than a launch: 80 us
+    // against 73 us on the mixed workload.)
+    if ((int)blockIdx.x < nStripWG) {
+        if constexpr (sizeof(VT) == 2) {
+            const int gw = xcd_contiguous_block(blockIdx.x, nStripWG) * (kBlock / 64) + (tid >> 6);
+            if (gw < nStripWaves) tile_dense_wave(stripWaveDesc, stripHdr, stripVal, x, y, gw, tid & 63);
+        }
+        return;
+    }
+    // Every kind of workgroup walks its rows in ascending order, and the sums of neighbouring rows
+    // lie close together wherever their virtual rows fall into the same slice and length class:
+    // one XCD per contiguous range of rows keeps those sectors in a single L2.
+    int b = (int)blockIdx.x - nStripWG;
+    if (b < nRowWG) b = xcd_contiguous_block(b, nRowWG);
+    else if (b < nRowWG + nLightWG) b = nRowWG + xcd_contiguous_block(b - nRowWG, nLightWG);
+    else b = nRowWG + nLightWG + xcd_contiguous_block(b - nRowWG - nLightWG, nHeavyWG);
+    if (b < nRowWG) {
+        // kCombineRows rows per lane, as quads a wave apart so that its loads and stores stay contiguous
+        int dd[kCombineRows];
+#pragma unroll
+        for (int q = 0; q < kCombineRows / 4; ++q) {
+            const int r0 = 4 * ((b * (kCombineRows / 4) + q) * kBlock + tid);
+            const int4 d = r0 < rows ? ((const int4 *)rowInfo)[r0 >> 2] : int4{-2, -2, -2, -2};  // padded with -2
+            dd[4 * q] = d.x, dd[4 * q + 1] = d.y, dd[4 * q + 2] = d.z, dd[4 * q + 3] = d.w;
+        }
+        AT sum[kCombineRows];
+#pragma unroll
+        for (int j = 0; j < kCombineRows; ++j) sum[j] = dd[j] >= 0 ? partial[dd[j]] : (AT)0;
+#pragma unroll
+        for (int j = 0; j < kCombineRows; ++j) {
+            const int r = 4 * ((b * (kCombineRows / 4) + j / 4) * kBlock + tid) + j % 4;
+            const bool mine = dd[j] >= 0 || (dd[j] == -1 && !skipEmpty);
+            if (mine && accumulate) sum[j] += (AT)y[r];
+            if (mine) y[r] = (VT)sum[j];
+        }
+        return;
+    }
+    b -= nRowWG;
+    if (b < nLightWG) {
+        const int i = b * kBlock + tid;
+        if (i >= nLight) return;
+        static_assert(mx::kSliceLightSegs == 8, "two int4 of indices per light row");
+        const int r = lightRow[i];
+        const int4 i0 = lightIdx[2 * i], i1 = lightIdx[2 * i + 1];
+        const int id[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
+        AT sum = accumulate ? (AT)y[r] : (AT)0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (id[k] >= 0) sum += partial[id[k]];
+        y[r] = (VT)sum;
+        return;
+    }
+    b -= nLightWG;
+    const int g = b * (kBlock / 16) + (tid >> 4), sub = tid & 15;
+    const bool live = g < nHeavy;
+    const int4 h = live ? heavyInfo[g] : int4{0, 0, 0, 0};
+    AT sum = 0;
+    for (int k = sub; k < h.z; k += 64) {
+        int id[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) id[j] = k + 16 * j < h.z ? segIdx[h.y + k + 16 * j] : -1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (id[j] >= 0) sum += partial[id[j]];
+    }
+    sum = group_sum<16>(sum);
+    if (live && sub == 0) y[h.x] = (VT)(sum + (accumulate ? (AT)y[h.x] : (AT)0));
 }
 
 // MFMA probes: one wave, operands and accumulators exchanged lane by lane (raw register
@@ -983,7 +1005,8 @@ hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y
 }
 
 template <typename VT>
-static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, int what)
+static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, int what,
+                                  const DeviceTiles *strips)
 {
     typedef typename mxk::Acc<VT>::type AT;
     const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)P.maxWgChunks * 4 + 64;
@@ -1005,19 +1028,28 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     const int nRowWG = (P.rows + mxk::kCombineRows * mxk::kBlock - 1) / (mxk::kCombineRows * mxk::kBlock);
     const int nLightWG = (P.nLight + mxk::kBlock - 1) / mxk::kBlock;
     const int nHeavyWG = (P.nHeavy + mxk::kBlock / 16 - 1) / (mxk::kBlock / 16);
-    if (nRowWG + nLightWG + nHeavyWG == 0) return hipSuccess;
-    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(nRowWG + nLightWG + nHeavyWG), dim3(mxk::kBlock), 0, s,
+    // strips that ride along (binary16 only; the caller has checked that they may: dense form,
+    // rows of their own, x aligned)
+    const bool ride = strips && sizeof(VT) == 2 && strips->nWaves > 0;
+    const int nStripWG = ride ? (strips->nWaves + 3) / 4 : 0;
+    if (nStripWG + nRowWG + nLightWG + nHeavyWG == 0) return hipSuccess;
+    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(nStripWG + nRowWG + nLightWG + nHeavyWG), dim3(mxk::kBlock), 0, s,
                        (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, P.lightRow, (const int4 *)P.lightIdx, P.nLight, nLightWG,
                        (const int4 *)P.heavyInfo, P.nHeavy, P.segIdx, (VT *)y, (accumulate || P.subset) ? 1 : 0,
-                       P.subset ? 1 : 0);
+                       P.subset ? 1 : 0, ride ? (const int4 *)strips->waveDesc : nullptr, ride ? strips->hdr : nullptr,
+                       ride ? (const VT *)strips->tcVal : nullptr, (const VT *)x, ride ? strips->nWaves : 0, nStripWG, nHeavyWG);
     return hipGetLastError();
 }
 hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
-                         int what)
+                         int what, const DeviceTiles *strips)
 {
     if (P.rows <= 0) return hipSuccess;
-    if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s, what);
-    return launch_slices_t<_Float16>(P, x, y, accumulate, s, what);
+    if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s, what, nullptr);
+    return launch_slices_t<_Float16>(P, x, y, accumulate, s, what, strips);
+}
+bool strips_can_ride(mx_dtype dtype, const DeviceTiles &T, const void *x)
+{
+    return dtype == MX_F16 && T.nWaves > 0 && T.dense && T.ownedRows && !((uintptr_t)x & 15);
 }
 
 hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s)

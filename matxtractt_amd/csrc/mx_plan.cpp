@@ -133,8 +133,10 @@ struct HostSlices {
     std::vector<unsigned char> eval;
 };
 
+// `elsewhere` (optional) marks rows whose result another kernel writes (the strips of a binary16
+// plan): rowInfo -2, so that the combine kernel neither zeroes nor adds to them.
 int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
-                 const char *sel, HostSlices &D)
+                 const char *sel, HostSlices &D, const char *elsewhere = nullptr)
 {
     const int es = mx::elem_size(dtype), E = mx::slice_step_entries(dtype);
     const int BE = mx::kSliceBatchEntries, SPB = BE / E;  // steps per batch
@@ -357,7 +359,7 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     std::vector<int> rowInfo(((size_t)rows + 3) / 4 * 4 + 4, -2), lightInfo, heavyInfo;
     for (int r = 0; r < rows; ++r) {
         const int a = segPtr[r], n = segPtr[r + 1] - a;
-        rowInfo[r] = n == 0 ? -1 : n == 1 ? segIdx[a] : -2;
+        rowInfo[r] = n == 0 ? ((elsewhere && elsewhere[r]) ? -2 : -1) : n == 1 ? segIdx[a] : -2;
         if (n > 1) {
             std::vector<int> &L = n > mx::kSliceLightSegs ? heavyInfo : lightInfo;
             L.insert(L.end(), {r, a, n, 0});
@@ -389,10 +391,10 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
 }
 
 int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
-                  const char *sel, mx::DeviceSlices &D)
+                  const char *sel, mx::DeviceSlices &D, const char *elsewhere = nullptr)
 {
     HostSlices H;
-    int rc = build_slices(dtype, rows, cols, rowPtr, col, val, nCU, S, sel, H);
+    int rc = build_slices(dtype, rows, cols, rowPtr, col, val, nCU, S, sel, H, elsewhere);
     if (rc) return rc;
     D.nWG = H.nWG;
     D.S = H.S;
@@ -893,14 +895,15 @@ static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
     return MX_OK;
 }
 
-static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate, hipStream_t s)
+static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate, hipStream_t s,
+                           const mx::DeviceTiles *strips = nullptr)
 {
     if (plan->csr_variant != 0 && ((uintptr_t)x & 15)) {
         set_error("mx_spmv: x must be 16-byte aligned for this plan");
         return MX_ERR_ARG;
     }
     if (plan->csr_variant != 1) MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s));
-    if (plan->csr_variant != 0) MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s));
+    if (plan->csr_variant != 0) MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s, 0, strips));
     return MX_OK;
 }
 
@@ -919,7 +922,10 @@ static int split_length()
 // two are built in turn (the second when the matrix suits it) and timed on the spot with a few
 // launches, and the faster is kept.  The split runs only when asked for: it has not won on any
 // matrix measured so far and building it makes a plan half as slow again.
-static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags)
+// `stripRows` (optional): rows that the strip form of the tile kernel writes (and the CSR part has
+// nothing for).
+static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags,
+                          const char *stripRows = nullptr)
 {
     const int rows = plan->rows, cols = plan->cols;
     const int nnz = rowPtr[rows];
@@ -966,7 +972,7 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
     }
     auto build = [&](int v, mx::DeviceCsr &C, mx::DeviceSlices &L) -> int {
         if (v == 0) return upload_csr(plan->dtype, rows, cols, nnz, rowPtr, col, val, C, nullptr);
-        if (v == 1) return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, nullptr, L);
+        if (v == 1) return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, nullptr, L, stripRows);
         // the short rows as a CSR matrix of their own (the long rows empty), the long ones as slices
         std::vector<int> rp((size_t)rows + 1, 0);
         for (int r = 0; r < rows; ++r) rp[r + 1] = rp[r] + (longRow[r] ? 0 : rowPtr[r + 1] - rowPtr[r]);
@@ -982,7 +988,7 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
         }
         int r1 = upload_csr(plan->dtype, rows, cols, rp[rows], rp.data(), c2.data(), v2.data(), C, nullptr);
         if (r1) return r1;
-        return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, longRow.data(), L);
+        return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, longRow.data(), L, stripRows);
     };
     double best = 0.0;
     bool have = false;
@@ -1179,10 +1185,14 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             }
             // Do the tiles pay for their launch?  (The reference gates its tile kernel on the size
             // of the matrix and its fill, test/test_autotc_spmv.cpp:1507,1518.)  What they take off
-            // the CSR part saves es + 2 bytes per entry of its stream; what they cost is a launch
-            // and their own stream.  Rates as measured on MI355X: the CSR part and the strip
-            // form of the tile kernel move about 5 bytes per ns, the general tile kernel, bound
-            // by instruction issue, about 2.2.  MX_PLAN_KEEP_TILES skips the question.
+            // the CSR part saves es + 2 bytes per entry of its stream; what they cost is one more
+            // dependent launch and their own stream.  Rates as measured on MI355X: the CSR part and
+            // the strip form of the tile kernel move about 5000 bytes per ns (5 TB/s), the general
+            // tile kernel, bound by instruction issue, about 2200; a further launch in the sequence
+            // costs about 5 us with its ramp and tail (the strips of the mixed workload break even at
+            // about 15 M entries when launched apart); strips usually ride in the launch of the
+            // combine kernel, where they came out ahead at every size tried (1.7 M entries and up):
+            // they are charged little.  MX_PLAN_KEEP_TILES skips the question.
             if (!(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES | MX_PLAN_KEEP_TILES))) {
                 double generalEntries = 0, generalFrags = 0, stripEntries = 0, stripBlocks = 0;
                 for (int w = 0; w < chunkNum; ++w) {
@@ -1206,14 +1216,15 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                 const double blockBytes = (double)fragM * fragK * es, slots = mx::tile_slots(P->dtype);
                 const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
                 const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
-                const double launchNs = 2500.0;
-                const double savedNs = (generalEntries + stripEntries) * (es + 2) / 5.0;
-                const double costNs = (generalFrags > 0 ? launchNs + generalBytes / 2.2 : 0.0) + (stripBlocks > 0 ? launchNs + stripBytes / 5.0 : 0.0);
+                const double launchNs = 5000.0, stripLaunchNs = 1000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
+                const double savedNs = (generalEntries + stripEntries) * (es + 2) / fastRate;
+                const double costNs = (generalFrags > 0 ? launchNs + generalBytes / generalRate : 0.0) +
+                                      (stripBlocks > 0 ? stripLaunchNs + stripBytes / fastRate : 0.0);
                 if (savedNs <= costNs) {
                     std::fill(sel.begin(), sel.end(), 0);
                     stripChunks.clear();
                     taken.clear();
-                } else if (generalFrags > 0 && generalEntries * (es + 2) / 5.0 <= launchNs + generalBytes / 2.2) {
+                } else if (generalFrags > 0 && generalEntries * (es + 2) / fastRate <= launchNs + generalBytes / generalRate) {
                     std::fill(sel.begin(), sel.end(), 0);  // the strips pay, the general tiles do not
                 }
             }
@@ -1278,8 +1289,14 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                     ++q;
                 }
             }
+            std::vector<char> stripRows;
+            if (!taken.empty()) {
+                stripRows.assign((size_t)rows, 0);
+                for (int i = 0; i < P->dRows; ++i)
+                    if (taken[i]) stripRows[P->rId[i]] = 1;
+            }
             phase("CSR part assembled");
-            rc = setup_csr_part(plan, rowPtr.data(), col.data(), val.data(), flags);
+            rc = setup_csr_part(plan, rowPtr.data(), col.data(), val.data(), flags, stripRows.empty() ? nullptr : stripRows.data());
             if (rc) return fail(rc);
             phase("CSR part (layouts, trial)");
 
@@ -1352,10 +1369,14 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
 
 static int spmv_on(mx_plan *plan, const void *x, void *y, hipStream_t s)
 {
-    int rc = launch_csr_part(plan, x, y, 0, s);
+    // the strips ride in the launch of the combine kernel when the CSR part has one (MX_STRIPS_APART=1:
+    // a launch of their own, as with the row-tile form of the CSR part)
+    static const bool apart = std::getenv("MX_STRIPS_APART") && std::atoi(std::getenv("MX_STRIPS_APART"));
+    const bool ride = !apart && plan->csr_variant == 1 && mx::strips_can_ride(plan->dtype, plan->strips, x);
+    int rc = launch_csr_part(plan, x, y, 0, s, ride ? &plan->strips : nullptr);
     if (rc) return rc;
     MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x, y, 1, s));
-    MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x, y, 1, s));
+    if (!ride) MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x, y, 1, s));
     return MX_OK;
 }
 
