@@ -861,7 +861,7 @@ __global__ __launch_bounds__(kBlock) void tile_dense_kernel(const int4 *__restri
 //    two arrays, so nothing the lane loads depends on another load but the sums themselves;
 //  * the rest take the rows with more, sixteen lanes each.
 constexpr int kCombineRows = 16;  // rows a lane of the first kind takes
-template <typename VT>
+template <typename VT, bool STRIPS>  // STRIPS: an instance of its own, so that the plain one keeps its few registers
 __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Acc<VT>::type *__restrict__ partial,
                                                               const int *__restrict__ rowInfo, int rows, int nRowWG,
                                                               const int *__restrict__ lightRow,
@@ -881,8 +881,8 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
     // leave alone (rowInfo -2).  In one launch they cost no dependent launch of their own.  (Spread
     // evenly among the other kinds instead of ahead of them they cost more than a launch: 80 us
     // against 73 us on the mixed workload.)
-    if ((int)blockIdx.x < nStripWG) {
-        if constexpr (sizeof(VT) == 2) {
+    if (STRIPS && (int)blockIdx.x < nStripWG) {
+        if constexpr (STRIPS && sizeof(VT) == 2) {
             const int gw = xcd_contiguous_block(blockIdx.x, nStripWG) * (kBlock / 64) + (tid >> 6);
             if (gw < nStripWaves) tile_dense_wave(stripWaveDesc, stripHdr, stripVal, x, y, gw, tid & 63);
         }
@@ -1033,11 +1033,16 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     const bool ride = strips && sizeof(VT) == 2 && strips->nWaves > 0;
     const int nStripWG = ride ? (strips->nWaves + 3) / 4 : 0;
     if (nStripWG + nRowWG + nLightWG + nHeavyWG == 0) return hipSuccess;
-    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT>), dim3(nStripWG + nRowWG + nLightWG + nHeavyWG), dim3(mxk::kBlock), 0, s,
-                       (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, P.lightRow, (const int4 *)P.lightIdx, P.nLight, nLightWG,
-                       (const int4 *)P.heavyInfo, P.nHeavy, P.segIdx, (VT *)y, (accumulate || P.subset) ? 1 : 0,
-                       P.subset ? 1 : 0, ride ? (const int4 *)strips->waveDesc : nullptr, ride ? strips->hdr : nullptr,
-                       ride ? (const VT *)strips->tcVal : nullptr, (const VT *)x, ride ? strips->nWaves : 0, nStripWG, nHeavyWG);
+#define MX_LAUNCH_COMBINE(STRIPS)                                                                                          \
+    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT, STRIPS>), dim3(nStripWG + nRowWG + nLightWG + nHeavyWG),                 \
+                       dim3(mxk::kBlock), 0, s, (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, P.lightRow,                    \
+                       (const int4 *)P.lightIdx, P.nLight, nLightWG, (const int4 *)P.heavyInfo, P.nHeavy, P.segIdx, (VT *)y,    \
+                       (accumulate || P.subset) ? 1 : 0, P.subset ? 1 : 0, ride ? (const int4 *)strips->waveDesc : nullptr,   \
+                       ride ? strips->hdr : nullptr, ride ? (const VT *)strips->tcVal : nullptr, (const VT *)x,              \
+                       ride ? strips->nWaves : 0, nStripWG, nHeavyWG)
+    if (ride) MX_LAUNCH_COMBINE(true);
+    else MX_LAUNCH_COMBINE(false);
+#undef MX_LAUNCH_COMBINE
     return hipGetLastError();
 }
 hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
