@@ -265,6 +265,35 @@ typedef struct mx_slice_layout_view {
 int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *sel, mx_slice_layout_view *out);
 void mx_slice_layout_free(mx_slice_layout_view *v);
 
+/* The host half of a plan for a partition, for inspection and tests on a machine without a GPU
+ * (no counterpart in the reference, where these decisions are inline in main(),
+ * test/test_autotc_spmv.cpp:1486-1559): the CSR part in the caller's numbering (the residual plus
+ * every entry of the extracted block that the tile kernels do not take; for a partition with
+ * tau = (0,0) the matrix itself), and up to two tile layouts as the kernels read them -- [0] for
+ * tile_kernel, [1] the strip chunks for tile_dense_kernel.  Per step: hdr[32] ints (output rows
+ * [0,16) of the two halves, -1 = none; [16] flags: 1 = the sums are stored after this step, 2 = the
+ * halves belong to two chunks; [17],[18] blocks in half 0 and 1; [21,29) first column per slot in
+ * the strip layout), atox[64] column ids (slot-major, -1 = unused; block i of half h sits in
+ * slot 2i+h of a binary64 step and in slot 4h+i of a binary16 step), and the blocks' values in
+ * `val` from valOffset[step] on (elements): the blocks of half 0, then of half 1, each
+ * fragM x fragK row-major.  `nCU` sizes the waves (waveDesc[nWaves][8] = {first step, end step,
+ * ...}).  Release with mx_plan_layout_free. */
+typedef struct mx_tile_layout_view {
+    int steps, nWaves, chunks, nnz, dense;
+    long long nVal; /* elements in val */
+    int *hdr, *atox, *waveDesc, *valOffset;
+    unsigned char *val;
+} mx_tile_layout_view;
+typedef struct mx_plan_layout_view {
+    int rows, cols, csr_nnz, fragM, fragK, slots; /* slots: block slots of a step (two halves of slots/2) */
+    int *csrRowPtr, *csrColInd;
+    unsigned char *csrVal;
+    unsigned char *stripRows; /* [rows] 1 = the row is written by the strip layout alone */
+    mx_tile_layout_view tiles[2];
+} mx_plan_layout_view;
+int mx_plan_layout(const mx_partition *P, int flags, int nCU, mx_plan_layout_view *out);
+void mx_plan_layout_free(mx_plan_layout_view *v);
+
 /* Reference surface, host pointers in / host pointers out, one-shot (allocate, upload,
  * `warm` + `iters` timed launches into a scratch y, one real launch, download, free).
  * The C++ functions of include/MatXtract.h are inline wrappers over these.

@@ -62,6 +62,17 @@ class SliceLayoutView(C.Structure):
                                         "heavyInfo", "ecol", "eval")]
 
 
+class TileLayoutView(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("steps", "nWaves", "chunks", "nnz", "dense")] + [("nVal", C.c_longlong)] + \
+               [(n, C.c_void_p) for n in ("hdr", "atox", "waveDesc", "valOffset", "val")]
+
+
+class PlanLayoutView(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("rows", "cols", "csr_nnz", "fragM", "fragK", "slots")] + \
+               [(n, C.c_void_p) for n in ("csrRowPtr", "csrColInd", "csrVal", "stripRows")] + \
+               [("tiles", TileLayoutView * 2)]
+
+
 class TauPoint(C.Structure):
     _fields_ = [("tau_c", C.c_float), ("tau_r", C.c_float), ("ms_total", C.c_double), ("tile_nnz", C.c_int)]
 
@@ -99,6 +110,8 @@ SIGNATURES = {
                          C.POINTER(TauPoint), _i, _pi]),
     "mx_slice_layout": (_i, [C.POINTER(CsrStruct), _i, _vp, C.POINTER(SliceLayoutView)]),
     "mx_slice_layout_free": (None, [C.POINTER(SliceLayoutView)]),
+    "mx_plan_layout": (_i, [_vp, _i, _i, C.POINTER(PlanLayoutView)]),
+    "mx_plan_layout_free": (None, [C.POINTER(PlanLayoutView)]),
     "mx_cdspmv_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _pd, _pd]),
     "mx_cdspmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _pd, _pd]),
     "mx_du_tcspmv_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _pd]),

@@ -17,7 +17,7 @@ from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLA
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
-           "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES"]
+           "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "plan_layout"]
 
 
 def _p(a):
@@ -217,6 +217,35 @@ def slice_layout(A, nCU=256, sel=None):
         out["eval"] = _view(v.eval, v.nEcol, vt).copy()
     finally:
         _lib.load().mx_slice_layout_free(C.byref(v))
+    return out
+
+
+def plan_layout(part, flags=MX_PLAN_DEFAULT, nCU=256):
+    """The host half of a plan for partition `part` (no GPU needed): the CSR part in the caller's
+    numbering and the two tile layouts as the kernels read them, as a dict of numpy arrays (see
+    mx_plan_layout in include/matxtract_hip.h)."""
+    v = _lib.PlanLayoutView()
+    check(_lib.load().mx_plan_layout(part._h, int(flags), int(nCU), C.byref(v)))
+    try:
+        vt = _np_dtype(part.dtype)
+        out = {n: int(getattr(v, n)) for n in ("rows", "cols", "csr_nnz", "fragM", "fragK", "slots")}
+        out["csrRowPtr"] = _view(v.csrRowPtr, v.rows + 1, np.int32).copy()
+        out["csrColInd"] = _view(v.csrColInd, v.csr_nnz, np.int32).copy()
+        out["csrVal"] = _view(v.csrVal, v.csr_nnz, vt).copy()
+        out["stripRows"] = _view(v.stripRows, v.rows, np.uint8).copy()
+        out["tiles"] = []
+        for t in v.tiles:
+            out["tiles"].append({
+                "steps": int(t.steps), "nWaves": int(t.nWaves), "chunks": int(t.chunks), "nnz": int(t.nnz),
+                "dense": bool(t.dense),
+                "hdr": _view(t.hdr, t.steps * 32, np.int32).reshape(-1, 32).copy(),
+                "atox": _view(t.atox, t.steps * 64, np.int32).reshape(-1, 64).copy(),
+                "waveDesc": _view(t.waveDesc, t.nWaves * 8, np.int32).reshape(-1, 8).copy(),
+                "valOffset": _view(t.valOffset, t.steps, np.int32).copy(),
+                "val": _view(t.val, t.nVal, vt).copy(),
+            })
+    finally:
+        _lib.load().mx_plan_layout_free(C.byref(v))
     return out
 
 

@@ -454,10 +454,19 @@ struct StripChunk {
 // `rowTaken` (optional, per row of A_dd) marks rows whose entries the plan has put into strip
 // chunks: they are left out of the fragments here.  With `stripChunks` the canonical chunks are
 // not used at all: the given chunks are laid out, for tile_dense_kernel.
-int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, const int *chunkPtr, const int *fragPtr,
-                 const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap,
-                 mx::DeviceTiles &T, int *tile_nnz, const char *rowTaken = nullptr,
-                 const std::vector<StripChunk> *stripChunks = nullptr)
+// (The layout is made on the host alone -- build_tiles; `nCU` only sizes the waves -- and
+// upload_tiles puts it on the device.)
+struct HostTiles {
+    int chunkNum = 0, frags = 0, vals = 0, steps = 0, nWaves = 0;
+    long long stored = 0;
+    bool dense = false;
+    std::vector<int> waveDesc, hdr, atox, valOffset;  // valOffset: first value of every step (the kernels get it from the headers)
+    std::vector<unsigned char> val;
+};
+
+int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, const int *chunkPtr, const int *fragPtr,
+                const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap, int nCU,
+                HostTiles &T, const char *rowTaken = nullptr, const std::vector<StripChunk> *stripChunks = nullptr)
 {
     const int es = mx::elem_size(dtype), fragK = mx::frag_k(dtype), fragM = mx::kFragM;
     const int SF = mx::tile_slots(dtype), HF = SF / 2, H = mx::kTileHdr, BS = fragM * fragK;  // BS: values per block
@@ -627,17 +636,10 @@ int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, c
     T.stored = (long long)voff;
     T.steps = steps;
     T.dense = stripChunks != nullptr && steps > 0;
-    if (tile_nnz) *tile_nnz = nnz;
     if (steps == 0) return MX_OK;
     // waves: whole chunks, about `per` steps each; few enough waves that all of them are resident
     // at once (24 per CU), so that none has to wait for a second round
-    int nCU = 256;
-    {
-        hipDeviceProp_t prop;
-        int dev = 0;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            nCU = std::max(1, prop.multiProcessorCount);
-    }
+    nCU = std::max(1, nCU);
     const int tper = std::getenv("MX_TILE_PER") ? std::atoi(std::getenv("MX_TILE_PER")) : 0;
     const int per = tper > 0 ? tper : std::max(2, (steps + nCU * 24 - 1) / (nCU * 24));
     std::vector<int> waveDesc;
@@ -659,12 +661,44 @@ int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, c
         s0 = s1;
     }
     T.nWaves = (int)waveDesc.size() / 8;
-    int rc;
-    if ((rc = upload(&T.waveDesc, waveDesc.data(), waveDesc.size(), 64))) return rc;
-    if ((rc = upload(&T.hdr, hdr.data(), hdr.size(), 256))) return rc;
-    if ((rc = upload(&T.atox, dAtox.data(), dAtox.size(), 256))) return rc;
+    T.waveDesc.swap(waveDesc);
+    T.hdr.swap(hdr);
+    T.atox.swap(dAtox);
+    T.valOffset.swap(stepVo);
+    T.val.swap(dVal);
+    return MX_OK;
+}
+
+int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, const int *chunkPtr, const int *fragPtr,
+                 const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap,
+                 mx::DeviceTiles &T, int *tile_nnz, const char *rowTaken = nullptr,
+                 const std::vector<StripChunk> *stripChunks = nullptr)
+{
+    int nCU = 256;
+    {
+        hipDeviceProp_t prop;
+        int dev = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            nCU = std::max(1, prop.multiProcessorCount);
+    }
+    HostTiles H;
+    int rc = build_tiles(dtype, chunkNum, selFrag, dRows, chunkPtr, fragPtr, fragBit, tcVal, atox, colMap, rowMap, nCU, H,
+                         rowTaken, stripChunks);
+    if (rc) return rc;
+    T.chunkNum = H.chunkNum;
+    T.frags = H.frags;
+    T.vals = H.vals;
+    T.stored = H.stored;
+    T.steps = H.steps;
+    T.dense = H.dense;
+    T.nWaves = H.nWaves;
+    if (tile_nnz) *tile_nnz = H.vals;
+    if (H.steps == 0) return MX_OK;
+    if ((rc = upload(&T.waveDesc, H.waveDesc.data(), H.waveDesc.size(), 64))) return rc;
+    if ((rc = upload(&T.hdr, H.hdr.data(), H.hdr.size(), 256))) return rc;
+    if ((rc = upload(&T.atox, H.atox.data(), H.atox.size(), 256))) return rc;
     // a lane of a step with few blocks reads where an absent block would be: 4 KB of slack
-    if ((rc = upload_bytes(&T.tcVal, dVal.data(), dVal.size(), 8192))) return rc;
+    if ((rc = upload_bytes(&T.tcVal, H.val.data(), H.val.size(), 8192))) return rc;
     return MX_OK;
 }
 
@@ -1051,6 +1085,239 @@ struct PhaseLog {
     }
 };
 
+// The host half of a plan for an extracted partition: which fragments the tile kernels take
+// (`sel`), which rows of A_dd go into strip chunks of the plan's own (`taken`, `stripChunks`,
+// `stripRows` = the same rows in the caller's numbering), and the CSR part -- the residual plus
+// every entry of A_dd that the tiles leave -- in the caller's numbering.
+struct HostPlanParts {
+    std::vector<char> sel, taken, stripRows;
+    std::vector<StripChunk> stripChunks;
+    std::vector<int> rowPtr, col;
+    std::vector<unsigned char> val;
+};
+
+static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, PhaseLog &phase)
+{
+    const int es = mx::elem_size(P->dtype), fragK = P->fragK, fragM = P->fragM;
+    const int rows = P->rows, cols = P->cols;
+    // residual column space -> the caller's column ids, so x needs no permutation
+    std::vector<int> colOrig(cols);
+    for (int c = 0; c < P->dCols; ++c) colOrig[c] = P->descColId[c];
+    for (int c = P->dCols; c < cols; ++c) colOrig[c] = P->newArray[c - P->dCols];
+    // which fragments go to the tile kernel
+    const int chunkNum = P->chunkNum, nFrags = P->chunkPtr[chunkNum];
+    std::vector<char> &sel = H.sel;
+    sel.assign((size_t)nFrags, 0);
+    const double gate = tile_gate(P->dtype);
+    if (!(flags & MX_PLAN_NO_TILES)) {
+        for (int f = 0; f < nFrags; ++f) {
+            const int vals = P->fragPtr[f + 1] - P->fragPtr[f];
+            sel[f] = (flags & MX_PLAN_ALL_TILES) ? vals > 0 : (vals > 0 && (double)vals >= gate * fragM * fragK);
+        }
+    }
+    // binary16 rows of A_dd whose columns, in the caller's numbering, are one run of a
+    // multiple of fragK columns from a multiple of fragK (a row of a dense strip), with
+    // nothing in the residual: rows with the same run are put together, fragM at a time,
+    // into chunks of the plan's own (the canonical chunks follow the row order, where
+    // rows of other shapes fall between them and one chunk straddles two strips).  A
+    // chunk at least half full goes to tile_dense_kernel; its rows leave the fragments.
+    std::vector<char> &taken = H.taken;
+    std::vector<StripChunk> &stripChunks = H.stripChunks;
+    taken.clear();
+    stripChunks.clear();
+    if (P->dtype == MX_F16 && fragM == 8 && fragK == 8 && !(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES)) &&
+        !(std::getenv("MX_NO_STRIPS") && std::atoi(std::getenv("MX_NO_STRIPS")))) {
+        const int maxRun = mx::tile_slots(P->dtype) * fragK;
+        struct Cand {
+            int c0, n, i;
+        };
+        std::vector<Cand> cand;
+        for (int i = 0; i < P->dRows; ++i) {
+            const int p0 = P->ddRowPtr[i], n = P->ddRowPtr[i + 1] - p0, r = P->rId[i];
+            if (n < fragK || n > maxRun || n % fragK || P->cdRowPtr[r + 1] != P->cdRowPtr[r]) continue;
+            int lo = INT_MAX, hi = -1;
+            for (int p = p0; p < p0 + n; ++p) {
+                const int c = P->descColId[P->ddColInd[p]];
+                lo = std::min(lo, c);
+                hi = std::max(hi, c);
+            }
+            if (lo % fragK || hi - lo + 1 != n) continue;
+            // n entries within [lo, lo + n): that run exactly, unless a column comes twice
+            // (such a row stays with the fragments, where the last of the two counts)
+            uint64_t seen = 0;
+            for (int p = p0; p < p0 + n; ++p) seen |= 1ull << (P->descColId[P->ddColInd[p]] - lo);
+            if (__builtin_popcountll(seen) == n) cand.push_back({lo, n, i});
+        }
+        std::sort(cand.begin(), cand.end(), [](const Cand &a, const Cand &b) {
+            return a.c0 != b.c0 ? a.c0 < b.c0 : a.n != b.n ? a.n < b.n : a.i < b.i;
+        });
+        taken.assign((size_t)P->dRows, 0);
+        const uint16_t *ddv16 = (const uint16_t *)P->ddVal.data();  // binary16 bit patterns
+        for (size_t a = 0; a < cand.size();) {
+            size_t b = a;
+            while (b < cand.size() && cand[b].c0 == cand[a].c0 && cand[b].n == cand[a].n) ++b;
+            for (size_t g = a; g < b; g += fragM) {
+                const int nr = (int)std::min(b - g, (size_t)fragM);
+                if (2 * nr < fragM) break;
+                StripChunk C;
+                const int c0 = cand[a].c0, n = cand[a].n, nb = n / fragK;
+                C.nnz = nr * n;
+                C.blocks.resize(nb);
+                for (int k = 0; k < nb; ++k) {
+                    C.blocks[k].vals.assign((size_t)fragM * fragK * es, 0);
+                    for (int c = 0; c < fragK; ++c) C.blocks[k].cols[c] = c0 + k * fragK + c;
+                }
+                for (int j = 0; j < 8; ++j) C.rows[j] = -1;
+                for (int j = 0; j < nr; ++j) {
+                    const int i = cand[g + j].i;
+                    taken[i] = 1;
+                    C.rows[j] = P->rId[i];
+                    for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
+                        const int c = P->descColId[P->ddColInd[p]] - c0;
+                        ((uint16_t *)C.blocks[c / fragK].vals.data())[j * fragK + c % fragK] = ddv16[p];
+                    }
+                }
+                stripChunks.push_back(std::move(C));
+            }
+            a = b;
+        }
+        if (stripChunks.empty()) taken.clear();
+    }
+    phase("fragment gate, strip rows");
+    if (!taken.empty()) {
+        // the gate again, on what the taken rows leave of each fragment
+#pragma omp parallel for schedule(static)
+        for (int w = 0; w < chunkNum; ++w) {
+            uint64_t rowsLeft = 0;  // bits of the rows that stay
+            for (int r = 0; r < fragM; ++r) {
+                const int i = w * fragM + r;
+                if (i < P->dRows && !taken[i]) rowsLeft |= 0xffull << (r * fragK);
+            }
+            for (int f = P->chunkPtr[w]; f < P->chunkPtr[w + 1]; ++f) {
+                const int vals = __builtin_popcountll(P->fragBit64[f] & rowsLeft);
+                sel[f] = sel[f] && vals > 0 && (double)vals >= gate * fragM * fragK;
+            }
+        }
+    }
+    // Do the tiles pay for their launch?  (The reference gates its tile kernel on the size
+    // of the matrix and its fill, test/test_autotc_spmv.cpp:1507,1518.)  What they take off
+    // the CSR part saves es + 2 bytes per entry of its stream; what they cost is one more
+    // dependent launch and their own stream.  Rates as measured on MI355X: the CSR part and
+    // the strip form of the tile kernel move about 5000 bytes per ns (5 TB/s), the general
+    // tile kernel, bound by instruction issue, about 2200; a further launch in the sequence
+    // costs about 5 us with its ramp and tail (the strips of the mixed workload break even at
+    // about 15 M entries when launched apart); strips usually ride in the launch of the
+    // combine kernel, where they came out ahead at every size tried (1.7 M entries and up):
+    // they are charged little.  MX_PLAN_KEEP_TILES skips the question.
+    if (!(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES | MX_PLAN_KEEP_TILES))) {
+        double generalEntries = 0, generalFrags = 0, stripEntries = 0, stripBlocks = 0;
+        for (int w = 0; w < chunkNum; ++w) {
+            uint64_t rowsLeft = ~0ull;
+            if (!taken.empty())
+                for (int r = 0; r < fragM; ++r) {
+                    const int i = w * fragM + r;
+                    if (i < P->dRows && taken[i]) rowsLeft &= ~(0xffull << (r * fragK));
+                }
+            for (int f = P->chunkPtr[w]; f < P->chunkPtr[w + 1]; ++f) {
+                if (!sel[f]) continue;
+                generalFrags += 1;
+                generalEntries += taken.empty() ? P->fragPtr[f + 1] - P->fragPtr[f]
+                                                : __builtin_popcountll(P->fragBit64[f] & rowsLeft);
+            }
+        }
+        for (const StripChunk &C : stripChunks) {
+            stripEntries += C.nnz;
+            stripBlocks += (double)C.blocks.size();
+        }
+        const double blockBytes = (double)fragM * fragK * es, slots = mx::tile_slots(P->dtype);
+        const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
+        const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
+        const double launchNs = 5000.0, stripLaunchNs = 1000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
+        const double savedNs = (generalEntries + stripEntries) * (es + 2) / fastRate;
+        const double costNs = (generalFrags > 0 ? launchNs + generalBytes / generalRate : 0.0) +
+                              (stripBlocks > 0 ? stripLaunchNs + stripBytes / fastRate : 0.0);
+        if (savedNs <= costNs) {
+            std::fill(sel.begin(), sel.end(), 0);
+            stripChunks.clear();
+            taken.clear();
+        } else if (generalFrags > 0 && generalEntries * (es + 2) / fastRate <= launchNs + generalBytes / generalRate) {
+            std::fill(sel.begin(), sel.end(), 0);  // the strips pay, the general tiles do not
+        }
+    }
+    // fragment of every A_dd entry: the rank of its column among the chunk's columns, / fragK.
+    // The used prefix of a chunk's column list is ascending (the zero padding after it is
+    // not), and so are the columns of a row of A_dd: one walk over both.
+    std::vector<int> usedCols((size_t)chunkNum, 0);
+#pragma omp parallel for schedule(static)
+    for (int w = 0; w < chunkNum; ++w) {
+        const int f0 = P->chunkPtr[w], f1 = P->chunkPtr[w + 1];
+        const int *a = &P->sparse_AToX_index[(size_t)f0 * fragK];
+        int n = (f1 - f0) * fragK;
+        while (n > 1 && a[n - 1] == 0) --n;
+        usedCols[w] = n;
+    }
+    // CSR part = residual rows + the A_dd entries whose fragment stays out of the tile kernel
+    std::vector<int> &rowPtr = H.rowPtr;
+    rowPtr.assign((size_t)rows + 1, 0);
+    for (int r = 0; r < rows; ++r) rowPtr[r + 1] = P->cdRowPtr[r + 1] - P->cdRowPtr[r];
+    std::vector<char> keep((size_t)P->ddRowPtr[P->dRows], 0);  // A_dd entry goes to the CSR part
+    // (rows of A_dd come longest first: small dynamic pieces, not one static range per thread)
+#pragma omp parallel for schedule(dynamic, 512)
+    for (int i = 0; i < P->dRows; ++i) {
+        const int w = i / fragM, f0 = P->chunkPtr[w];
+        const int *a = &P->sparse_AToX_index[(size_t)f0 * fragK];
+        const int na = usedCols[w];
+        const bool rowTaken = !taken.empty() && taken[i];
+        int n = 0, rank = 0;
+        for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
+            const int c = P->ddColInd[p];
+            while (rank < na && a[rank] < c) ++rank;
+            // Of entries that name the same column twice the tile format holds the last
+            // (generateFormat_opt overwrites, test/test_autotc_spmv.cpp:718-847); the
+            // earlier ones go to the CSR part, so that y is the sum of all of them.
+            const bool earlierTwin = p + 1 < P->ddRowPtr[i + 1] && P->ddColInd[p + 1] == c;
+            keep[p] = rowTaken ? 0 : (earlierTwin || !sel[f0 + rank / fragK]);
+            n += keep[p];
+        }
+        rowPtr[P->rId[i] + 1] += n;
+    }
+    for (int r = 0; r < rows; ++r) rowPtr[r + 1] += rowPtr[r];
+    const int csrNnz = rowPtr[rows];
+    std::vector<int> &col = H.col;
+    std::vector<unsigned char> &val = H.val;
+    col.assign((size_t)csrNnz, 0);
+    val.assign((size_t)csrNnz * es, 0);
+    const unsigned char *cdv = (const unsigned char *)P->cdVal.data();
+    const unsigned char *ddv = (const unsigned char *)P->ddVal.data();
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; ++r) {
+        int q = rowPtr[r];
+        for (int p = P->cdRowPtr[r]; p < P->cdRowPtr[r + 1]; ++p, ++q) {
+            col[q] = colOrig[P->cdColInd[p]];
+            std::memcpy(&val[(size_t)q * es], cdv + (size_t)p * es, es);
+        }
+    }
+#pragma omp parallel for schedule(dynamic, 512)
+    for (int i = 0; i < P->dRows; ++i) {
+        const int r = P->rId[i];
+        int q = rowPtr[r] + (P->cdRowPtr[r + 1] - P->cdRowPtr[r]);
+        for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
+            if (!keep[p]) continue;
+            col[q] = P->descColId[P->ddColInd[p]];
+            std::memcpy(&val[(size_t)q * es], ddv + (size_t)p * es, es);
+            ++q;
+        }
+    }
+    std::vector<char> &stripRows = H.stripRows;
+    stripRows.clear();
+    if (!taken.empty()) {
+        stripRows.assign((size_t)rows, 0);
+        for (int i = 0; i < P->dRows; ++i)
+            if (taken[i]) stripRows[P->rId[i]] = 1;
+    }
+    return MX_OK;
+}
+
 extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
 {
     if (!P || !out) {
@@ -1069,8 +1336,6 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
     plan->rows = P->rows;
     plan->cols = P->cols;
     plan->nnz = P->nnz;
-    const int es = mx::elem_size(P->dtype), fragK = P->fragK, fragM = P->fragM;
-    const int rows = P->rows, cols = P->cols;
     auto fail = [&](int code) {
         mx_plan_destroy(plan);
         return code;
@@ -1087,214 +1352,14 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             if (rc) return fail(rc);
             phase("CSR part (layouts, trial)");
         } else {
-            // residual column space -> the caller's column ids, so x needs no permutation
-            std::vector<int> colOrig(cols);
-            for (int c = 0; c < P->dCols; ++c) colOrig[c] = P->descColId[c];
-            for (int c = P->dCols; c < cols; ++c) colOrig[c] = P->newArray[c - P->dCols];
-            // which fragments go to the tile kernel
-            const int chunkNum = P->chunkNum, nFrags = P->chunkPtr[chunkNum];
-            std::vector<char> sel((size_t)nFrags, 0);
-            const double gate = tile_gate(P->dtype);
-            if (!(flags & MX_PLAN_NO_TILES)) {
-                for (int f = 0; f < nFrags; ++f) {
-                    const int vals = P->fragPtr[f + 1] - P->fragPtr[f];
-                    sel[f] = (flags & MX_PLAN_ALL_TILES) ? vals > 0 : (vals > 0 && (double)vals >= gate * fragM * fragK);
-                }
-            }
-            // binary16 rows of A_dd whose columns, in the caller's numbering, are one run of a
-            // multiple of fragK columns from a multiple of fragK (a row of a dense strip), with
-            // nothing in the residual: rows with the same run are put together, fragM at a time,
-            // into chunks of the plan's own (the canonical chunks follow the row order, where
-            // rows of other shapes fall between them and one chunk straddles two strips).  A
-            // chunk at least half full goes to tile_dense_kernel; its rows leave the fragments.
-            std::vector<char> taken;
-            std::vector<StripChunk> stripChunks;
-            if (P->dtype == MX_F16 && fragM == 8 && fragK == 8 && !(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES)) &&
-                !(std::getenv("MX_NO_STRIPS") && std::atoi(std::getenv("MX_NO_STRIPS")))) {
-                const int maxRun = mx::tile_slots(P->dtype) * fragK;
-                struct Cand {
-                    int c0, n, i;
-                };
-                std::vector<Cand> cand;
-                for (int i = 0; i < P->dRows; ++i) {
-                    const int p0 = P->ddRowPtr[i], n = P->ddRowPtr[i + 1] - p0, r = P->rId[i];
-                    if (n < fragK || n > maxRun || n % fragK || P->cdRowPtr[r + 1] != P->cdRowPtr[r]) continue;
-                    int lo = INT_MAX, hi = -1;
-                    for (int p = p0; p < p0 + n; ++p) {
-                        const int c = P->descColId[P->ddColInd[p]];
-                        lo = std::min(lo, c);
-                        hi = std::max(hi, c);
-                    }
-                    if (lo % fragK || hi - lo + 1 != n) continue;
-                    // n entries within [lo, lo + n): that run exactly, unless a column comes twice
-                    // (such a row stays with the fragments, where the last of the two counts)
-                    uint64_t seen = 0;
-                    for (int p = p0; p < p0 + n; ++p) seen |= 1ull << (P->descColId[P->ddColInd[p]] - lo);
-                    if (__builtin_popcountll(seen) == n) cand.push_back({lo, n, i});
-                }
-                std::sort(cand.begin(), cand.end(), [](const Cand &a, const Cand &b) {
-                    return a.c0 != b.c0 ? a.c0 < b.c0 : a.n != b.n ? a.n < b.n : a.i < b.i;
-                });
-                taken.assign((size_t)P->dRows, 0);
-                const uint16_t *ddv16 = (const uint16_t *)P->ddVal.data();  // binary16 bit patterns
-                for (size_t a = 0; a < cand.size();) {
-                    size_t b = a;
-                    while (b < cand.size() && cand[b].c0 == cand[a].c0 && cand[b].n == cand[a].n) ++b;
-                    for (size_t g = a; g < b; g += fragM) {
-                        const int nr = (int)std::min(b - g, (size_t)fragM);
-                        if (2 * nr < fragM) break;
-                        StripChunk C;
-                        const int c0 = cand[a].c0, n = cand[a].n, nb = n / fragK;
-                        C.nnz = nr * n;
-                        C.blocks.resize(nb);
-                        for (int k = 0; k < nb; ++k) {
-                            C.blocks[k].vals.assign((size_t)fragM * fragK * es, 0);
-                            for (int c = 0; c < fragK; ++c) C.blocks[k].cols[c] = c0 + k * fragK + c;
-                        }
-                        for (int j = 0; j < 8; ++j) C.rows[j] = -1;
-                        for (int j = 0; j < nr; ++j) {
-                            const int i = cand[g + j].i;
-                            taken[i] = 1;
-                            C.rows[j] = P->rId[i];
-                            for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
-                                const int c = P->descColId[P->ddColInd[p]] - c0;
-                                ((uint16_t *)C.blocks[c / fragK].vals.data())[j * fragK + c % fragK] = ddv16[p];
-                            }
-                        }
-                        stripChunks.push_back(std::move(C));
-                    }
-                    a = b;
-                }
-                if (stripChunks.empty()) taken.clear();
-            }
-            phase("fragment gate, strip rows");
-            if (!taken.empty()) {
-                // the gate again, on what the taken rows leave of each fragment
-#pragma omp parallel for schedule(static)
-                for (int w = 0; w < chunkNum; ++w) {
-                    uint64_t rowsLeft = 0;  // bits of the rows that stay
-                    for (int r = 0; r < fragM; ++r) {
-                        const int i = w * fragM + r;
-                        if (i < P->dRows && !taken[i]) rowsLeft |= 0xffull << (r * fragK);
-                    }
-                    for (int f = P->chunkPtr[w]; f < P->chunkPtr[w + 1]; ++f) {
-                        const int vals = __builtin_popcountll(P->fragBit64[f] & rowsLeft);
-                        sel[f] = sel[f] && vals > 0 && (double)vals >= gate * fragM * fragK;
-                    }
-                }
-            }
-            // Do the tiles pay for their launch?  (The reference gates its tile kernel on the size
-            // of the matrix and its fill, test/test_autotc_spmv.cpp:1507,1518.)  What they take off
-            // the CSR part saves es + 2 bytes per entry of its stream; what they cost is one more
-            // dependent launch and their own stream.  Rates as measured on MI355X: the CSR part and
-            // the strip form of the tile kernel move about 5000 bytes per ns (5 TB/s), the general
-            // tile kernel, bound by instruction issue, about 2200; a further launch in the sequence
-            // costs about 5 us with its ramp and tail (the strips of the mixed workload break even at
-            // about 15 M entries when launched apart); strips usually ride in the launch of the
-            // combine kernel, where they came out ahead at every size tried (1.7 M entries and up):
-            // they are charged little.  MX_PLAN_KEEP_TILES skips the question.
-            if (!(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES | MX_PLAN_KEEP_TILES))) {
-                double generalEntries = 0, generalFrags = 0, stripEntries = 0, stripBlocks = 0;
-                for (int w = 0; w < chunkNum; ++w) {
-                    uint64_t rowsLeft = ~0ull;
-                    if (!taken.empty())
-                        for (int r = 0; r < fragM; ++r) {
-                            const int i = w * fragM + r;
-                            if (i < P->dRows && taken[i]) rowsLeft &= ~(0xffull << (r * fragK));
-                        }
-                    for (int f = P->chunkPtr[w]; f < P->chunkPtr[w + 1]; ++f) {
-                        if (!sel[f]) continue;
-                        generalFrags += 1;
-                        generalEntries += taken.empty() ? P->fragPtr[f + 1] - P->fragPtr[f]
-                                                        : __builtin_popcountll(P->fragBit64[f] & rowsLeft);
-                    }
-                }
-                for (const StripChunk &C : stripChunks) {
-                    stripEntries += C.nnz;
-                    stripBlocks += (double)C.blocks.size();
-                }
-                const double blockBytes = (double)fragM * fragK * es, slots = mx::tile_slots(P->dtype);
-                const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
-                const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
-                const double launchNs = 5000.0, stripLaunchNs = 1000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
-                const double savedNs = (generalEntries + stripEntries) * (es + 2) / fastRate;
-                const double costNs = (generalFrags > 0 ? launchNs + generalBytes / generalRate : 0.0) +
-                                      (stripBlocks > 0 ? stripLaunchNs + stripBytes / fastRate : 0.0);
-                if (savedNs <= costNs) {
-                    std::fill(sel.begin(), sel.end(), 0);
-                    stripChunks.clear();
-                    taken.clear();
-                } else if (generalFrags > 0 && generalEntries * (es + 2) / fastRate <= launchNs + generalBytes / generalRate) {
-                    std::fill(sel.begin(), sel.end(), 0);  // the strips pay, the general tiles do not
-                }
-            }
-            // fragment of every A_dd entry: the rank of its column among the chunk's columns, / fragK.
-            // The used prefix of a chunk's column list is ascending (the zero padding after it is
-            // not), and so are the columns of a row of A_dd: one walk over both.
-            std::vector<int> usedCols((size_t)chunkNum, 0);
-#pragma omp parallel for schedule(static)
-            for (int w = 0; w < chunkNum; ++w) {
-                const int f0 = P->chunkPtr[w], f1 = P->chunkPtr[w + 1];
-                const int *a = &P->sparse_AToX_index[(size_t)f0 * fragK];
-                int n = (f1 - f0) * fragK;
-                while (n > 1 && a[n - 1] == 0) --n;
-                usedCols[w] = n;
-            }
-            // CSR part = residual rows + the A_dd entries whose fragment stays out of the tile kernel
-            std::vector<int> rowPtr((size_t)rows + 1, 0);
-            for (int r = 0; r < rows; ++r) rowPtr[r + 1] = P->cdRowPtr[r + 1] - P->cdRowPtr[r];
-            std::vector<char> keep((size_t)P->ddRowPtr[P->dRows], 0);  // A_dd entry goes to the CSR part
-            // (rows of A_dd come longest first: small dynamic pieces, not one static range per thread)
-#pragma omp parallel for schedule(dynamic, 512)
-            for (int i = 0; i < P->dRows; ++i) {
-                const int w = i / fragM, f0 = P->chunkPtr[w];
-                const int *a = &P->sparse_AToX_index[(size_t)f0 * fragK];
-                const int na = usedCols[w];
-                const bool rowTaken = !taken.empty() && taken[i];
-                int n = 0, rank = 0;
-                for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
-                    const int c = P->ddColInd[p];
-                    while (rank < na && a[rank] < c) ++rank;
-                    // Of entries that name the same column twice the tile format holds the last
-                    // (generateFormat_opt overwrites, test/test_autotc_spmv.cpp:718-847); the
-                    // earlier ones go to the CSR part, so that y is the sum of all of them.
-                    const bool earlierTwin = p + 1 < P->ddRowPtr[i + 1] && P->ddColInd[p + 1] == c;
-                    keep[p] = rowTaken ? 0 : (earlierTwin || !sel[f0 + rank / fragK]);
-                    n += keep[p];
-                }
-                rowPtr[P->rId[i] + 1] += n;
-            }
-            for (int r = 0; r < rows; ++r) rowPtr[r + 1] += rowPtr[r];
-            const int csrNnz = rowPtr[rows];
-            std::vector<int> col((size_t)csrNnz);
-            std::vector<unsigned char> val((size_t)csrNnz * es);
-            const unsigned char *cdv = (const unsigned char *)P->cdVal.data();
-            const unsigned char *ddv = (const unsigned char *)P->ddVal.data();
-#pragma omp parallel for schedule(static)
-            for (int r = 0; r < rows; ++r) {
-                int q = rowPtr[r];
-                for (int p = P->cdRowPtr[r]; p < P->cdRowPtr[r + 1]; ++p, ++q) {
-                    col[q] = colOrig[P->cdColInd[p]];
-                    std::memcpy(&val[(size_t)q * es], cdv + (size_t)p * es, es);
-                }
-            }
-#pragma omp parallel for schedule(dynamic, 512)
-            for (int i = 0; i < P->dRows; ++i) {
-                const int r = P->rId[i];
-                int q = rowPtr[r] + (P->cdRowPtr[r + 1] - P->cdRowPtr[r]);
-                for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
-                    if (!keep[p]) continue;
-                    col[q] = P->descColId[P->ddColInd[p]];
-                    std::memcpy(&val[(size_t)q * es], ddv + (size_t)p * es, es);
-                    ++q;
-                }
-            }
-            std::vector<char> stripRows;
-            if (!taken.empty()) {
-                stripRows.assign((size_t)rows, 0);
-                for (int i = 0; i < P->dRows; ++i)
-                    if (taken[i]) stripRows[P->rId[i]] = 1;
-            }
+            HostPlanParts H;
+            rc = plan_host_parts(P, flags, H, phase);
+            if (rc) return fail(rc);
+            const int chunkNum = P->chunkNum;
+            std::vector<char> &sel = H.sel, &taken = H.taken, &stripRows = H.stripRows;
+            std::vector<StripChunk> &stripChunks = H.stripChunks;
+            std::vector<int> &rowPtr = H.rowPtr, &col = H.col;
+            std::vector<unsigned char> &val = H.val;
             phase("CSR part assembled");
             rc = setup_csr_part(plan, rowPtr.data(), col.data(), val.data(), flags, stripRows.empty() ? nullptr : stripRows.data());
             if (rc) return fail(rc);
@@ -1324,6 +1389,103 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
         return fail(MX_ERR_ALLOC);
     }
     *out = plan;
+    return MX_OK;
+}
+
+extern "C" void mx_plan_layout_free(mx_plan_layout_view *v)
+{
+    if (!v) return;
+    free(v->csrRowPtr);
+    free(v->csrColInd);
+    free(v->csrVal);
+    free(v->stripRows);
+    for (int t = 0; t < 2; ++t) {
+        free(v->tiles[t].hdr);
+        free(v->tiles[t].atox);
+        free(v->tiles[t].waveDesc);
+        free(v->tiles[t].valOffset);
+        free(v->tiles[t].val);
+    }
+    std::memset(v, 0, sizeof(*v));
+}
+
+extern "C" int mx_plan_layout(const mx_partition *P, int flags, int nCU, mx_plan_layout_view *out)
+{
+    if (!P || !out || nCU < 1) {
+        set_error("mx_plan_layout: bad argument");
+        return MX_ERR_ARG;
+    }
+    std::memset(out, 0, sizeof(*out));
+    const int es = mx::elem_size(P->dtype);
+    auto give = [](const auto *p, size_t n) {
+        typedef typename std::remove_cv<typename std::remove_pointer<decltype(p)>::type>::type T;
+        T *q = (T *)malloc(std::max<size_t>(n, 1) * sizeof(T));
+        if (q && n) std::memcpy(q, p, n * sizeof(T));
+        return q;
+    };
+    try {
+        out->rows = P->rows;
+        out->cols = P->cols;
+        out->fragM = P->fragM;
+        out->fragK = P->fragK;
+        out->slots = mx::tile_slots(P->dtype);
+        HostPlanParts H;
+        HostTiles T[2];
+        if (!P->extracted) {
+            out->csr_nnz = P->cdRowPtr[P->rows];
+            out->csrRowPtr = give(P->cdRowPtr.data(), (size_t)P->rows + 1);
+            out->csrColInd = give(P->cdColInd.data(), (size_t)out->csr_nnz);
+            out->csrVal = give((const unsigned char *)P->cdVal.data(), (size_t)out->csr_nnz * es);
+        } else {
+            PhaseLog quiet;
+            quiet.on = false;
+            int rc = plan_host_parts(P, flags, H, quiet);
+            if (rc) return rc;
+            out->csr_nnz = H.rowPtr[P->rows];
+            out->csrRowPtr = give(H.rowPtr.data(), H.rowPtr.size());
+            out->csrColInd = give(H.col.data(), H.col.size());
+            out->csrVal = give(H.val.data(), H.val.size());
+            const void *bits = P->dtype == MX_F64 ? (const void *)P->fragBit32.data() : (const void *)P->fragBit64.data();
+            rc = build_tiles(P->dtype, P->chunkNum, H.sel.data(), P->dRows, P->chunkPtr.data(), P->fragPtr.data(), bits,
+                             P->tcVal.data(), P->sparse_AToX_index.data(), P->descColId.data(), P->rId.data(), nCU, T[0],
+                             H.taken.empty() ? nullptr : H.taken.data());
+            if (rc) return rc;
+            if (!H.stripChunks.empty()) {
+                rc = build_tiles(P->dtype, P->chunkNum, H.sel.data(), P->dRows, P->chunkPtr.data(), P->fragPtr.data(), bits,
+                                 P->tcVal.data(), P->sparse_AToX_index.data(), P->descColId.data(), P->rId.data(), nCU, T[1],
+                                 nullptr, &H.stripChunks);
+                if (rc) return rc;
+            }
+        }
+        std::vector<unsigned char> sr((size_t)P->rows, 0);
+        if (!H.stripRows.empty()) std::memcpy(sr.data(), H.stripRows.data(), sr.size());
+        out->stripRows = give(sr.data(), sr.size());
+        bool ok = out->csrRowPtr && out->csrColInd && out->csrVal && out->stripRows;
+        for (int t = 0; t < 2; ++t) {
+            mx_tile_layout_view &V = out->tiles[t];
+            V.steps = T[t].steps;
+            V.nWaves = T[t].nWaves;
+            V.chunks = T[t].chunkNum;
+            V.nnz = T[t].vals;
+            V.dense = T[t].dense ? 1 : 0;
+            V.nVal = (long long)(T[t].val.size() / (size_t)es);
+            V.hdr = give(T[t].hdr.data(), T[t].hdr.size());
+            V.atox = give(T[t].atox.data(), T[t].atox.size());
+            V.waveDesc = give(T[t].waveDesc.data(), T[t].waveDesc.size());
+            V.valOffset = give(T[t].valOffset.data(), T[t].valOffset.size());
+            V.val = give(T[t].val.data(), T[t].val.size());
+            ok = ok && V.hdr && V.atox && V.waveDesc && V.valOffset && V.val;
+        }
+        if (!ok) {
+            mx_plan_layout_free(out);
+            set_error("mx_plan_layout: out of memory");
+            return MX_ERR_ALLOC;
+        }
+    } catch (const std::bad_alloc &) {
+        mx_plan_layout_free(out);
+        set_error("mx_plan_layout: out of memory");
+        return MX_ERR_ALLOC;
+    }
     return MX_OK;
 }
 

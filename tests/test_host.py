@@ -536,3 +536,125 @@ def test_cli_argument_errors_match_the_reference():
     assert r.returncode == 1 and "Error: col_frac must be greater than hot_frac." in r.stdout
     r = cli("0.5", "0.2", "0.1", "x.mtx")
     assert r.returncode == 1 and "Error: Too many arguments provided." in r.stdout
+
+
+# ---------------------------------------------------------------- the host half of a plan, walked on the CPU
+def _walk_plan_layout(L, x, dtype):
+    """y as the kernels would compute it from a plan's host layout: the CSR part row by row, the
+    tile layouts step by step -- slot j of half h multiplies its fragM x fragK block with the x at
+    the step's column ids (general layout) or at first column + 0..fragK-1 (strip layout); a
+    half's rows collect until a step with flag 1, then the sums go to y (added in the general
+    layout, stored in the strip layout, whose rows nothing else may write)."""
+    fragM, fragK, slots = L["fragM"], L["fragK"], L["slots"]
+    half = slots // 2
+    x = np.asarray(x, np.float64)
+    y = np.zeros(L["rows"])
+    rp, ci, va = L["csrRowPtr"], L["csrColInd"], L["csrVal"].astype(np.float64)
+    for r in range(L["rows"]):
+        y[r] = np.dot(va[rp[r]:rp[r + 1]], x[ci[rp[r]:rp[r + 1]]])
+    touched = np.zeros(L["rows"], bool)
+    entries = 0
+    for t, T in enumerate(L["tiles"]):
+        val = T["val"].astype(np.float64)
+        seen_steps = 0
+        for w in range(T["nWaves"]):
+            s0, s1 = T["waveDesc"][w][:2]
+            assert s0 == seen_steps and s1 > s0, "waves cover the steps in order"
+            seen_steps = s1
+            acc = np.zeros((2, fragM))
+            for s in range(s0, s1):
+                hdr = T["hdr"][s]
+                flags, n = hdr[16], (hdr[17], hdr[18])
+                assert 0 <= n[0] <= half and 0 <= n[1] <= half and n[0] + n[1] > 0
+                vo = T["valOffset"][s]
+                for h in range(2):
+                    for j in range(n[h]):
+                        slot = 2 * j + h if fragK == 4 else half * h + j   # the binary64 step interleaves its halves
+                        blk = val[vo + ((n[0] if h else 0) + j) * fragM * fragK:][:fragM * fragK].reshape(fragM, fragK)
+                        if t == 1:
+                            c0 = hdr[21 + slot]
+                            assert c0 >= 0 and c0 % fragK == 0 and c0 + fragK <= L["cols"]
+                            cols = np.arange(c0, c0 + fragK)
+                            assert np.array_equal(T["atox"][s][slot * fragK:(slot + 1) * fragK], cols), "both forms of a strip step agree"
+                        else:
+                            cols = T["atox"][s][slot * fragK:(slot + 1) * fragK]
+                        used = cols >= 0
+                        assert np.all(blk[:, ~used] == 0) and np.all(cols[used] < L["cols"])
+                        acc[h] += blk[:, used] @ x[cols[used]]
+                        entries += int(np.count_nonzero(blk))
+                if flags & 1:
+                    for h in range(2):
+                        rows = hdr[8 * h:8 * h + fragM] if (flags & 2) or h == 0 else None
+                        if rows is None:
+                            continue
+                        sums = acc[h] if (flags & 2) else acc[0] + acc[1]
+                        for i, r in enumerate(rows):
+                            if r < 0:
+                                assert sums[i] == 0
+                                continue
+                            if t == 1:
+                                assert L["stripRows"][r] == 1 and not touched[r] and y[r] == 0, "a strip row is written once, by the strips alone"
+                                touched[r] = True
+                                y[r] = sums[i]
+                            else:
+                                assert L["stripRows"][r] == 0
+                                y[r] += sums[i]
+                    acc[:] = 0
+            assert not acc.any(), "a wave ends on a stored step"
+        assert seen_steps == T["steps"]
+    assert np.array_equal(touched, L["stripRows"].astype(bool)), "every strip row is written"
+    return y, entries
+
+
+def _strip_matrix(mx, rng, rows=1024, cols=6000):
+    """binary16: runs of rows that are one aligned run of 32 columns, among short random rows, one of
+    them as long as a strip row."""
+    rp, ci = [0], []
+    for r in range(rows):
+        if r == 70:
+            c = sorted(rng.choice(cols, 32, replace=False).tolist())
+        elif (r // 64) % 3 == 0:
+            base = 8 * ((r // 8) % 600)
+            c = list(range(base, base + 32))
+        else:
+            c = sorted(rng.choice(cols, 1 + int(rng.integers(0, 3)), replace=False).tolist())
+        ci += c
+        rp.append(len(ci))
+    va = rng.integers(-3, 4, len(ci)).astype(np.float16)
+    return mx.Csr(rows, cols, np.array(rp, np.int32), np.array(ci, np.int32), va)
+
+
+@pytest.mark.parametrize("case", ["block_f64", "mixed_f16", "strips_f16", "twice_f64", "twice_f16", "stencil_f64"])
+def test_plan_layout_walk(mx, ora, case):
+    """The host half of a plan -- fragment gate, strip rows, the CSR part, both tile layouts --
+    reproduces A x exactly (integer data) for every combination of plan flags, without a GPU."""
+    rng = np.random.default_rng(sum(map(ord, case)))
+    if case == "strips_f16":
+        A = _strip_matrix(mx, rng)
+    elif case.startswith("twice"):
+        dtype = np.float64 if case.endswith("f64") else np.float16
+        lens = rng.integers(0, 50, 300)
+        rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        A = mx.Csr(300, 80, rp, rng.integers(0, 80, rp[-1]).astype(np.int32), rng.integers(-3, 4, rp[-1]).astype(dtype))
+    else:
+        cfg, scale = {"block_f64": (2, 1 / 64), "mixed_f16": (5, 1 / 512), "stencil_f64": (3, 1 / 512)}[case]
+        A, _ = mx.gen_config(cfg, scale=scale)
+        A = mx.Csr(A.rows, A.cols, A.rowPtr, A.colInd, rng.integers(-3, 4, A.nnz).astype(A.val.dtype))
+    x = rng.integers(-2, 3, A.cols).astype(A.val.dtype)
+    ref = (ora.spmv_f64(A.val, A.rowPtr, A.colInd, x) if A.dtype == mx.MX_F64
+           else ora.spmv_f16_f32acc(A.val, A.rowPtr, A.colInd, x)[0]).astype(np.float64)
+    strips_seen = 0
+    for tau in ((1.0, 1.0), (0.75, 0.5), (0.5, 0.0), (0.0, 0.0)):
+        P = mx.Partition(A, *tau)
+        for flags in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_ALL_TILES, mx.MX_PLAN_NO_TILES):
+            L = mx.plan_layout(P, flags, nCU=4)
+            y, entries = _walk_plan_layout(L, x, A.val.dtype)
+            assert np.array_equal(y, ref), (case, tau, flags)
+            if flags == mx.MX_PLAN_NO_TILES or tau == (0.0, 0.0):
+                assert L["tiles"][0]["steps"] == 0 and L["tiles"][1]["steps"] == 0 and L["csr_nnz"] == A.nnz
+            if flags == mx.MX_PLAN_ALL_TILES:
+                assert L["tiles"][1]["steps"] == 0, "strip chunks are a matter of the default selection"
+            strips_seen += L["tiles"][1]["steps"]
+        P.close()
+    assert (strips_seen > 0) == (case in ("strips_f16", "mixed_f16")), strips_seen
+
