@@ -658,3 +658,28 @@ def test_plan_layout_walk(mx, ora, case):
         P.close()
     assert (strips_seen > 0) == (case in ("strips_f16", "mixed_f16")), strips_seen
 
+
+
+def test_host_code_under_sanitizers(tmp_path):
+    """The library's host code (generators, partition, slice layout, the host half of a plan) built
+    with -fsanitize=address,undefined and run on the five workloads at small scale: no report."""
+    import shutil
+    import subprocess
+    if shutil.which("g++") is None:
+        pytest.skip("no g++")
+    src = os.path.join(ROOT, "matxtractt_amd", "csrc")
+    exe = str(tmp_path / "host_driver")
+    cmd = ["g++", "-O1", "-g", "-std=c++17", "-fopenmp", "-fsanitize=address,undefined", "-fno-omit-frame-pointer",
+           "-fno-sanitize-recover=undefined", "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(ROOT, "include"), "-I" + src,
+           "-I/opt/rocm/include", os.path.join(ROOT, "tests", "sanitize", "host_driver.cpp"),
+           os.path.join(ROOT, "tests", "sanitize", "launch_stubs.cpp")] + \
+          [os.path.join(src, f) for f in ("mx_util.cpp", "mx_partition.cpp", "mx_gen.cpp", "mx_mmio.cpp", "mx_plan.cpp")] + \
+          ["-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib", "-o", exe]
+    b = subprocess.run(cmd, capture_output=True, text=True)
+    if b.returncode != 0 and ("asan" in b.stderr or "ubsan" in b.stderr) and "cannot find" in b.stderr:
+        pytest.skip("sanitizer runtimes not installed")
+    assert b.returncode == 0, b.stderr[-2000:]
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", OMP_NUM_THREADS="4")
+    r = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=600)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), (r.stdout[-500:], r.stderr[-3000:])
+    assert "ERROR: AddressSanitizer" not in r.stderr and "runtime error" not in r.stderr, r.stderr[-3000:]
