@@ -121,7 +121,7 @@ def test_full_size_workloads_match_oracle(mx, ora, cfg, taus):
     tol = F64_TOL if A.dtype == mx.MX_F64 else F16_TOL
     xd = torch.from_numpy(x).cuda()
     for tau in taus:
-        for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_ROWS,
+        for fl in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_ROWS,
                    mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_SLICES):
             print("full-size workload=%d tau=%s flags=%d" % (cfg, tau, fl), flush=True)
             part = mx.Partition(A, *tau)
