@@ -30,11 +30,11 @@ GRID = (0.0, 0.25, 0.5, 0.75, 1.0)
 # hold the counter values.  (workload, kernel, plan has tiles) -> bytes
 TRAFFIC = {
     (2, "csr_rows_kernel<f64>", False): 47165962,
-    (2, "csr_slice_kernel<f64>", False): 48771514,
-    (3, "csr_rows_kernel<f64>", False): 287435306,
-    (4, "csr_slice_kernel<f16>", False): 55549356,
-    (5, "csr_slice_kernel<f16>", False): 301452548,
-    (5, "csr_slice_kernel<f16>", True): 190230169,   # tau=(1,1): the strips run through tile_dense_kernel
+    (2, "csr_slice_kernel<f64>", False): 48823291,
+    (3, "csr_rows_kernel<f64>", False): 287431623,
+    (4, "csr_slice_kernel<f16>", False): 55821536,
+    (5, "csr_slice_kernel<f16>", False): 301417778,
+    (5, "csr_slice_kernel<f16>", True): 190181456,   # tau=(1,1): the strips run through tile_dense_kernel
 }
 WORKLOADS = {
     1: "configs[0]: FP64 random 4096x4096, 16 nnz/row",
