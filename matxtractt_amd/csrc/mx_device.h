@@ -32,8 +32,10 @@ int csr_entries_per_lane(mx_dtype dtype);
 // that are mostly full.  The columns of a chunk's selected fragments are first put in ascending
 // order of the caller's column ids and cut into blocks anew (the reference orders them by their
 // rank among the dense columns, which scatters neighbours): gathers touch fewer lines, and dense
-// strips become blocks of consecutive columns.  The blocks are grouped into "steps" -- what one wave feeds to the
-// matrix core at a time: two halves of up to kTileSlots(dtype)/2 blocks.  A chunk with more
+// strips become blocks of consecutive columns.  (Rows of binary16 strips do not come from the
+// reference's chunks at all: the plan groups them into chunks of its own, see `dense`.)  The
+// blocks are grouped into "steps" -- what one wave feeds to the matrix core at a time: two
+// halves of up to tile_slots(dtype)/2 blocks.  A chunk with more
 // selected fragments than half a step takes whole steps of its own (filling half 0 first; its
 // two halves are added at the end); smaller chunks share a step, one per half.  Per step:
 //   hdr    kTileHdr dwords: [0,16) output row of each of the 8 rows of half 0 and half 1
@@ -69,7 +71,8 @@ inline int tile_slot(mx_dtype d, int half, int i) { return d == MX_F64 ? 2 * i +
 // columns are cut into S slices of sliceCols columns (a slice of x fits LDS).  The entries of
 // a row that fall into one slice form a "virtual row"; one longer than the plan's cap is cut
 // into several, so a matrix row owns one or more virtual rows and its result is the sum of
-// theirs.  Per slice the virtual rows are sorted by length and cut into chunks of 64, one
+// theirs.  Per slice the virtual rows are sorted by length (among equals by the kind of their
+// row -- sole virtual row, a few, many -- then by row) and cut into chunks of 64, one
 // virtual row per lane (a sliced-ELL layout: every row of a chunk is padded to the chunk's
 // longest, and the sort keeps that padding small).  A slice gets workgroups in proportion to
 // its entries, its chunks are dealt to them longest first, and inside a workgroup to its waves
