@@ -170,10 +170,22 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
         reps = []
         runner = (lambda: ora.spmv_f64(A.val, A.rowPtr, A.colInd, x)) if A.dtype == mx.MX_F64 else \
                  (lambda: ora.spmv_f16_f32acc(A.val, A.rowPtr, A.colInd, x))
-        for i in range(12):
-            t0 = time.perf_counter()
-            runner()
-            reps.append(time.perf_counter() - t0)
+        # one thread on one core, as the reference's spmv_serial: pinned for the duration
+        affinity = os.sched_getaffinity(0)
+        pinned = None
+        try:
+            pinned = min(affinity)
+            os.sched_setaffinity(0, {pinned})
+        except OSError:
+            pinned = None
+        try:
+            for i in range(12):
+                t0 = time.perf_counter()
+                runner()
+                reps.append(time.perf_counter() - t0)
+        finally:
+            if pinned is not None:
+                os.sched_setaffinity(0, affinity)
         t_cpu = min(reps[2:])
         cpu_model = "unknown"
         try:
@@ -182,7 +194,7 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
         except OSError:
             pass
         rec["cpu_baseline"] = {"value": 2.0 * A.nnz / t_cpu / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
-                               "cpu": cpu_model, "cpus_visible": len(os.sched_getaffinity(0)),
+                               "cpu": cpu_model, "cpus_visible": len(os.sched_getaffinity(0)), "pinned_to_cpu": pinned,
                                "sample": "the full matrix of this workload, best of 10 after 2 warm-ups "
                                          "(%.1f ms per SpMV), single thread as the reference's spmv_serial" % (t_cpu * 1e3)}
         # not the reference's: the same oracle routine over nnz-balanced row ranges, one thread per
