@@ -231,11 +231,12 @@ typedef struct mx_plan_info {
                             0 = csr_rows_kernel, 1 = csr_slice_kernel */
     int csr_main_nnz;    /* entries that kernel holds */
     int tile_variant;    /* 1 when part of the tiles runs through tile_dense_kernel: binary16 rows whose columns
-                            are one run of 8, 16, .. 64 consecutive columns from a multiple of 8, with nothing
-                            in the residual; the plan groups rows with the same run, 8 at a time, into chunks
-                            of its own (at least 4 rows each) and takes them out of the reference's fragments.
-                            MX_NO_STRIPS=1 in the environment switches this off; with an x that is not
-                            16-byte aligned these chunks run through tile_kernel */
+                            fill at most 8 aligned blocks of 8 columns at least half (a row of a dense strip in
+                            the simplest case), with nothing in the residual and no column named twice; the plan
+                            groups rows with the same blocks, 8 at a time, into chunks of its own (at least 4
+                            rows each) and takes them out of the reference's fragments.  MX_NO_STRIPS=1 in the
+                            environment switches this off; with an x that is not 16-byte aligned these chunks
+                            run through tile_kernel */
     int tile_strip_nnz;  /* entries held by those chunks */
 } mx_plan_info;
 int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);

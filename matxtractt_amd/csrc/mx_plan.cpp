@@ -619,7 +619,9 @@ int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, co
             nfr += (int)fsel.size();
             for (int i = 0; i < 8; ++i) {
                 const int local = w * fragM + i;
-                curRows[i] = (i < fragM && local < dRows) ? (rowMap ? rowMap[local] : local) : -1;
+                // (a row that went into a strip chunk has nothing here and is not written from here)
+                const bool here = i < fragM && local < dRows && !(rowTaken && rowTaken[local]);
+                curRows[i] = here ? (rowMap ? rowMap[local] : local) : -1;
             }
             place(blocks, curRows);
             if (voff > 2000000000u) {
@@ -1115,66 +1117,81 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
             sel[f] = (flags & MX_PLAN_ALL_TILES) ? vals > 0 : (vals > 0 && (double)vals >= gate * fragM * fragK);
         }
     }
-    // binary16 rows of A_dd whose columns, in the caller's numbering, are one run of a
-    // multiple of fragK columns from a multiple of fragK (a row of a dense strip), with
-    // nothing in the residual: rows with the same run are put together, fragM at a time,
-    // into chunks of the plan's own (the canonical chunks follow the row order, where
-    // rows of other shapes fall between them and one chunk straddles two strips).  A
-    // chunk at least half full goes to tile_dense_kernel; its rows leave the fragments.
+    // binary16 rows of A_dd whose columns, in the caller's numbering, fall into at most a
+    // step's worth of aligned blocks of fragK columns (multiples of fragK) and fill them at
+    // least half -- a row of a dense strip in the simplest case -- with nothing in the
+    // residual and no column named twice: rows with the same set of blocks are put together,
+    // fragM at a time, into chunks of the plan's own (the canonical chunks follow the row
+    // order, where rows of other shapes fall between them and one chunk straddles two
+    // strips).  A chunk of at least fragM/2 rows goes to tile_dense_kernel; its rows leave the
+    // fragments.
     std::vector<char> &taken = H.taken;
     std::vector<StripChunk> &stripChunks = H.stripChunks;
     taken.clear();
     stripChunks.clear();
     if (P->dtype == MX_F16 && fragM == 8 && fragK == 8 && !(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES)) &&
         !(std::getenv("MX_NO_STRIPS") && std::atoi(std::getenv("MX_NO_STRIPS")))) {
-        const int maxRun = mx::tile_slots(P->dtype) * fragK;
+        constexpr int kMaxBlocks = 8;  // block slots of a binary16 step
         struct Cand {
-            int c0, n, i;
+            int nb, b[kMaxBlocks], n, i;  // blocks (column / fragK, ascending), entries, row of A_dd
         };
         std::vector<Cand> cand;
+        std::vector<int> cols;
         for (int i = 0; i < P->dRows; ++i) {
             const int p0 = P->ddRowPtr[i], n = P->ddRowPtr[i + 1] - p0, r = P->rId[i];
-            if (n < fragK || n > maxRun || n % fragK || P->cdRowPtr[r + 1] != P->cdRowPtr[r]) continue;
-            int lo = INT_MAX, hi = -1;
-            for (int p = p0; p < p0 + n; ++p) {
-                const int c = P->descColId[P->ddColInd[p]];
-                lo = std::min(lo, c);
-                hi = std::max(hi, c);
+            if (n < fragK / 2 || n > kMaxBlocks * fragK || P->cdRowPtr[r + 1] != P->cdRowPtr[r]) continue;
+            cols.resize((size_t)n);
+            for (int k = 0; k < n; ++k) cols[k] = P->descColId[P->ddColInd[p0 + k]];
+            std::sort(cols.begin(), cols.end());
+            Cand c;
+            c.nb = 0;
+            c.n = n;
+            c.i = i;
+            bool ok = true;
+            for (int k = 0; k < n && ok; ++k) {
+                if (k && cols[k] == cols[k - 1]) ok = false;  // named twice: stays with the fragments, where the last counts
+                const int blk = cols[k] / fragK;
+                if ((blk + 1) * fragK > P->cols) ok = false;  // the block would reach past the end of x
+                if (c.nb == 0 || c.b[c.nb - 1] != blk) {
+                    if (c.nb == kMaxBlocks) ok = false;
+                    else c.b[c.nb++] = blk;
+                }
             }
-            if (lo % fragK || hi - lo + 1 != n) continue;
-            // n entries within [lo, lo + n): that run exactly, unless a column comes twice
-            // (such a row stays with the fragments, where the last of the two counts)
-            uint64_t seen = 0;
-            for (int p = p0; p < p0 + n; ++p) seen |= 1ull << (P->descColId[P->ddColInd[p]] - lo);
-            if (__builtin_popcountll(seen) == n) cand.push_back({lo, n, i});
+            if (!ok || 2 * n < c.nb * fragK) continue;
+            for (int k = c.nb; k < kMaxBlocks; ++k) c.b[k] = -1;
+            cand.push_back(c);
         }
-        std::sort(cand.begin(), cand.end(), [](const Cand &a, const Cand &b) {
-            return a.c0 != b.c0 ? a.c0 < b.c0 : a.n != b.n ? a.n < b.n : a.i < b.i;
+        auto same = [](const Cand &x, const Cand &y) { return x.nb == y.nb && std::equal(x.b, x.b + kMaxBlocks, y.b); };
+        std::sort(cand.begin(), cand.end(), [](const Cand &x, const Cand &y) {
+            if (!std::equal(x.b, x.b + kMaxBlocks, y.b)) return std::lexicographical_compare(x.b, x.b + kMaxBlocks, y.b, y.b + kMaxBlocks);
+            return x.i < y.i;
         });
         taken.assign((size_t)P->dRows, 0);
         const uint16_t *ddv16 = (const uint16_t *)P->ddVal.data();  // binary16 bit patterns
         for (size_t a = 0; a < cand.size();) {
             size_t b = a;
-            while (b < cand.size() && cand[b].c0 == cand[a].c0 && cand[b].n == cand[a].n) ++b;
+            while (b < cand.size() && same(cand[b], cand[a])) ++b;
             for (size_t g = a; g < b; g += fragM) {
                 const int nr = (int)std::min(b - g, (size_t)fragM);
                 if (2 * nr < fragM) break;
                 StripChunk C;
-                const int c0 = cand[a].c0, n = cand[a].n, nb = n / fragK;
-                C.nnz = nr * n;
+                const int nb = cand[a].nb;
+                C.nnz = 0;
                 C.blocks.resize(nb);
                 for (int k = 0; k < nb; ++k) {
                     C.blocks[k].vals.assign((size_t)fragM * fragK * es, 0);
-                    for (int c = 0; c < fragK; ++c) C.blocks[k].cols[c] = c0 + k * fragK + c;
+                    for (int c = 0; c < fragK; ++c) C.blocks[k].cols[c] = cand[a].b[k] * fragK + c;
                 }
                 for (int j = 0; j < 8; ++j) C.rows[j] = -1;
                 for (int j = 0; j < nr; ++j) {
                     const int i = cand[g + j].i;
                     taken[i] = 1;
                     C.rows[j] = P->rId[i];
+                    C.nnz += cand[g + j].n;
                     for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
-                        const int c = P->descColId[P->ddColInd[p]] - c0;
-                        ((uint16_t *)C.blocks[c / fragK].vals.data())[j * fragK + c % fragK] = ddv16[p];
+                        const int c = P->descColId[P->ddColInd[p]];
+                        const int k = (int)(std::lower_bound(cand[a].b, cand[a].b + nb, c / fragK) - cand[a].b);
+                        ((uint16_t *)C.blocks[k].vals.data())[j * fragK + c % fragK] = ddv16[p];
                     }
                 }
                 stripChunks.push_back(std::move(C));

@@ -624,13 +624,38 @@ def _strip_matrix(mx, rng, rows=1024, cols=6000):
     return mx.Csr(rows, cols, np.array(rp, np.int32), np.array(ci, np.int32), va)
 
 
-@pytest.mark.parametrize("case", ["block_f64", "mixed_f16", "strips_f16", "twice_f64", "twice_f16", "stencil_f64"])
+def _block_rows_matrix(mx, rng, rows=768, cols=4003):
+    """binary16: groups of rows that share two or three aligned blocks of eight columns, far apart,
+    each row holding five to eight of a block's columns; runs of 20 columns off the grid of eight;
+    short random rows between."""
+    rp, ci = [0], []
+    for r in range(rows):
+        grp = r // 16
+        if grp % 3 == 0:
+            blocks = [(7 * grp) % 400, 100 + (11 * grp) % 300, 450 + grp % 40][:2 + grp % 2]
+            c = sorted(int(8 * b + k) for b in set(blocks) for k in rng.choice(8, int(rng.integers(5, 9)), replace=False))
+        elif grp % 3 == 1:
+            base = 8 * ((5 * grp) % 450) + 3
+            c = list(range(base, base + 20))
+        elif grp == 5:
+            c = list(range(3992, 4003))    # reaches into the last, partial block of x: never a strip row
+        else:
+            c = sorted(rng.choice(cols, 1 + int(rng.integers(0, 3)), replace=False).tolist())
+        ci += c
+        rp.append(len(ci))
+    va = rng.integers(-3, 4, len(ci)).astype(np.float16)
+    return mx.Csr(rows, cols, np.array(rp, np.int32), np.array(ci, np.int32), va)
+
+
+@pytest.mark.parametrize("case", ["block_f64", "mixed_f16", "strips_f16", "blocks_f16", "twice_f64", "twice_f16", "stencil_f64"])
 def test_plan_layout_walk(mx, ora, case):
     """The host half of a plan -- fragment gate, strip rows, the CSR part, both tile layouts --
     reproduces A x exactly (integer data) for every combination of plan flags, without a GPU."""
     rng = np.random.default_rng(sum(map(ord, case)))
     if case == "strips_f16":
         A = _strip_matrix(mx, rng)
+    elif case == "blocks_f16":
+        A = _block_rows_matrix(mx, rng)
     elif case.startswith("twice"):
         dtype = np.float64 if case.endswith("f64") else np.float16
         lens = rng.integers(0, 50, 300)
@@ -656,7 +681,7 @@ def test_plan_layout_walk(mx, ora, case):
                 assert L["tiles"][1]["steps"] == 0, "strip chunks are a matter of the default selection"
             strips_seen += L["tiles"][1]["steps"]
         P.close()
-    assert (strips_seen > 0) == (case in ("strips_f16", "mixed_f16")), strips_seen
+    assert (strips_seen > 0) == (case in ("strips_f16", "blocks_f16", "mixed_f16")), strips_seen
 
 
 
