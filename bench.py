@@ -32,6 +32,7 @@ TRAFFIC = {
     (2, "csr_rows_kernel<f64>", False): 47165962,
     (2, "csr_slice_kernel<f64>", False): 48823291,
     (3, "csr_rows_kernel<f64>", False): 287431623,
+    (3, "csr_rows_kernel<f64,dict>", False): 101747762,   # one byte per value: the stencil has two distinct values
     (4, "csr_slice_kernel<f16>", False): 55821536,
     (5, "csr_slice_kernel<f16>", False): 301417778,
     (5, "csr_slice_kernel<f16>", True): 190181456,   # tau=(1,1): the strips run through tile_dense_kernel
@@ -143,6 +144,8 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
         # the CSR part's main kernel alone (the slice variant has a small combine kernel after it)
         ms_main = plan.time_csr_main(xd, yd, warm=warmup, iters=steps)
         name = "csr_slice_kernel<%s>" if info["csr_main_kernel"] == 1 else "csr_rows_kernel<%s>"
+        if info["csr_main_kernel"] == 0 and info["csr_value_dict"]:
+            name = "csr_rows_kernel<%s,dict>"
         dom = {"kernel": name % dtype, "ms": ms_main,
                "bytes": kernel_bytes(mx, A.dtype, A.rows, A.cols, info["csr_main_nnz"])}
     achieved = dom["bytes"] / (dom["ms"] * 1e-3)

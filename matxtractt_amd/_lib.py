@@ -51,7 +51,8 @@ class PlanInfo(C.Structure):
                 ("tile_chunks", C.c_int), ("tile_frags", C.c_int), ("tile_nnz", C.c_int),
                 ("csr_nnz", C.c_int), ("csr_blocks", C.c_int), ("csr_variant", C.c_int),
                 ("tile_bytes", C.c_double), ("csr_bytes", C.c_double),
-                ("csr_main_kernel", C.c_int), ("csr_main_nnz", C.c_int), ("tile_variant", C.c_int), ("tile_strip_nnz", C.c_int)]
+                ("csr_main_kernel", C.c_int), ("csr_main_nnz", C.c_int), ("tile_variant", C.c_int), ("tile_strip_nnz", C.c_int),
+                ("csr_value_dict", C.c_int)]
 
 
 class SliceLayoutView(C.Structure):

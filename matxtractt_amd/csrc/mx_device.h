@@ -19,6 +19,12 @@ struct DeviceCsr {
     int nBlocks = 0;
     int npt = 0;              // entries per lane per tile the rows were packed for
     bool scan = false;        // sum the rows of a tile by a segmented scan (row lengths vary a lot)
+    // a matrix with at most 256 distinct values (a stencil, a graph): one byte per entry that
+    // names the value, and the values themselves (padded to 256); used with col16 only
+    unsigned char *codes = nullptr;  // [nnz + kCsrPad]
+    void *dict = nullptr;            // [256]
+    int nDict = 0;
+    bool useDict = false;            // the plan found this form the faster one
 };
 constexpr int kCsrPad = 1088;  // a wave may read one whole wave tile (64*16 entries) past the end
 

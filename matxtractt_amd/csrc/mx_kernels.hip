@@ -107,9 +107,12 @@ struct Acc<_Float16> {
 //   cs, vs : this wave's LDS regions, 64*NPT ints / accumulators.
 //   C16   : the column ids are stored as 16-bit offsets from x (the caller has moved x to the
 //           workgroup's lowest column); lim = the largest offset that is still inside x
-template <typename VT, int NPT, bool C16>
+//   DICT  : the matrix has at most 256 distinct values; `val` then points at one byte per entry,
+//           an index into `dict` (the distinct values as accumulators, in LDS)
+template <typename VT, int NPT, bool C16, bool DICT = false>
 __device__ __forceinline__ void wave_stream(const void *__restrict__ colv, const VT *__restrict__ val, int pos, int lane,
-                                            int *cs, typename Acc<VT>::type *vs)
+                                            int *cs, typename Acc<VT>::type *vs,
+                                            const typename Acc<VT>::type *dict = nullptr)
 {
     // every load instruction reads one contiguous stretch (lane l right after lane l-1): a
     // streamed line is then asked for once, not once per instruction that touches a piece of it
@@ -133,7 +136,23 @@ __device__ __forceinline__ void wave_stream(const void *__restrict__ colv, const
             *(v4i32 *)(cs + e) = __builtin_nontemporal_load((const v4i32 *)(col + pos + e));
         }
     }
-    if constexpr (sizeof(VT) == 8) {
+    if constexpr (DICT) {
+        // lane l takes the NPT codes NPT*l .. NPT*l+NPT-1 of the wave's stretch: one load of NPT bytes
+        static_assert(NPT == 4 || NPT == 8 || NPT == 16, "codes come in 4, 8 or 16 bytes per lane");
+        const unsigned char *codes = (const unsigned char *)val + pos + NPT * lane;
+        unsigned w[NPT / 4];
+        if constexpr (NPT == 4) {
+            w[0] = __builtin_nontemporal_load((const unsigned *)codes);
+        } else if constexpr (NPT == 8) {
+            const v2i32 t = __builtin_nontemporal_load((const v2i32 *)codes);
+            w[0] = (unsigned)t.x, w[1] = (unsigned)t.y;
+        } else {
+            const v4i32 t = __builtin_nontemporal_load((const v4i32 *)codes);
+            w[0] = (unsigned)t.x, w[1] = (unsigned)t.y, w[2] = (unsigned)t.z, w[3] = (unsigned)t.w;
+        }
+#pragma unroll
+        for (int k = 0; k < NPT; ++k) vs[NPT * lane + k] = dict[(w[k / 4] >> (8 * (k % 4))) & 255u];
+    } else if constexpr (sizeof(VT) == 8) {
 #pragma unroll
         for (int q = 0; q < NPT / 2; ++q) {
             const int e = 128 * q + 2 * lane;
@@ -320,13 +339,18 @@ __device__ __forceinline__ void reduce_scan(const typename Acc<VT>::type *prod, 
 // a sixth off an FP64 one.
 // With SCAN the rows of a tile are summed by reduce_scan instead of reduce_rows (the host asks
 // for it when row lengths vary a lot).
-template <typename VT, int NPT, bool XCD, bool C16, bool SCAN>
+// With DICT the values are one byte per entry, indices into the matrix's at most 256 distinct
+// values (`dictG`, copied to LDS first): a stencil or a graph matrix then streams 3 bytes per
+// entry instead of 10.
+template <typename VT, int NPT, bool XCD, bool C16, bool SCAN, bool DICT = false>
 __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict__ rowPtr, const void *__restrict__ col,
                                                           const VT *__restrict__ val, const VT *__restrict__ xfull,
                                                           VT *__restrict__ y, const int4 *__restrict__ blockDesc,
-                                                          const int *__restrict__ colBase, int xcols, int accumulate)
+                                                          const int *__restrict__ colBase, int xcols, int accumulate,
+                                                          const VT *__restrict__ dictG)
 {
     typedef typename Acc<VT>::type AT;
+    __shared__ AT dictL[DICT ? 256 : 1];
     constexpr int TILE = kBlock * NPT;
     constexpr int WTILE = 64 * NPT;
     __shared__ __attribute__((aligned(16))) AT prod[TILE];
@@ -341,6 +365,10 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
     const int r0 = d.x, r1 = d.y, p0 = d.z, p1 = d.w;
     const int nrows = r1 - r0;
     if (nrows <= 0) return;
+    if constexpr (DICT) {
+        dictL[tid] = (AT)dictG[tid];  // kBlock == 256 entries (the host pads the dictionary)
+        __syncthreads();
+    }
     const int cb = C16 ? colBase[b] : 0;
     const VT *x = xfull + cb;
     const int lim = xcols - 1 - cb;
@@ -356,7 +384,7 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
             ro[k] = rr <= nrows ? rowPtr[r0 + rr] : 0;
         }
         const bool active = base + wave * WTILE < p1;
-        if (active) wave_stream<VT, NPT, C16>(col, val, base + wave * WTILE, lane, cs, vs);
+        if (active) wave_stream<VT, NPT, C16, DICT>(col, val, base + wave * WTILE, lane, cs, vs, dictL);
         if (active) {
             AT p[NPT];
             wave_gather<VT, NPT, C16>(x, lane, cs, vs, p, lim);
@@ -407,7 +435,7 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
         AT s = 0;
         for (int t0 = base + wave * WTILE; t0 < p1; t0 += TILE) {
             AT p[NPT];
-            wave_stream<VT, NPT, C16>(col, val, t0, lane, cs, vs);
+            wave_stream<VT, NPT, C16, DICT>(col, val, t0, lane, cs, vs, dictL);
             wave_gather<VT, NPT, C16>(x, lane, cs, vs, p, lim);
 #pragma unroll
             for (int j = 0; j < NPT; ++j) {
@@ -981,12 +1009,21 @@ static void launch_csr_t(const DeviceCsr &A, const void *x, void *y, int accumul
 #define MX_LAUNCH_ROWS(C16, SCAN, COLS, BASE)                                                                       \
     hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, C16, SCAN>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s,      \
                        A.rowPtr, (const void *)(COLS), (const VT *)A.val, (const VT *)x, (VT *)y,                      \
-                       (const int4 *)A.blockDesc, (const int *)(BASE), A.cols, accumulate)
-    if (A.col16 && A.scan) MX_LAUNCH_ROWS(true, true, A.col16, A.colBase);
+                       (const int4 *)A.blockDesc, (const int *)(BASE), A.cols, accumulate, (const VT *)nullptr)
+#define MX_LAUNCH_ROWS_DICT(SCAN)                                                                                    \
+    hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, true, SCAN, true>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, \
+                       s, A.rowPtr, (const void *)A.col16, (const VT *)A.codes, (const VT *)x, (VT *)y,                  \
+                       (const int4 *)A.blockDesc, (const int *)A.colBase, A.cols, accumulate, (const VT *)A.dict)
+    static_assert(mxk::kBlock == 256, "a workgroup copies the 256 dictionary entries, one per lane");
+    if (A.useDict && A.col16 && A.codes && A.dict) {
+        if (A.scan) MX_LAUNCH_ROWS_DICT(true);
+        else MX_LAUNCH_ROWS_DICT(false);
+    } else if (A.col16 && A.scan) MX_LAUNCH_ROWS(true, true, A.col16, A.colBase);
     else if (A.col16) MX_LAUNCH_ROWS(true, false, A.col16, A.colBase);
     else if (A.scan) MX_LAUNCH_ROWS(false, true, A.col, nullptr);
     else MX_LAUNCH_ROWS(false, false, A.col, nullptr);
 #undef MX_LAUNCH_ROWS
+#undef MX_LAUNCH_ROWS_DICT
 }
 
 hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)

@@ -81,6 +81,8 @@ void free_csr(mx::DeviceCsr &A)
     (void)hipFree(A.col16);
     (void)hipFree(A.colBase);
     (void)hipFree(A.val);
+    (void)hipFree(A.codes);
+    (void)hipFree(A.dict);
     (void)hipFree(A.blockDesc);
     A = mx::DeviceCsr();
 }
@@ -766,6 +768,53 @@ int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, c
         if ((rc = upload_bytes(&d16, c16.data(), (size_t)nnz * 2, (size_t)mx::kCsrPad * 2))) return rc;
         A.col16 = (unsigned short *)d16;
         if ((rc = upload(&A.colBase, cbase.data(), cbase.size()))) return rc;
+        // at most 256 distinct values (bit patterns): a byte per entry and a dictionary beside the
+        // values; the plan times both forms (MX_CSR_DICT=0: never)
+        const char *ed = std::getenv("MX_CSR_DICT");
+        if (nnz >= 65536 && !(ed && !std::atoi(ed))) {
+            std::vector<unsigned char> codes((size_t)nnz);
+            std::vector<unsigned char> dict((size_t)256 * es, 0);
+            int nd = 0;
+            bool few = true;
+            if (es == 8) {
+                const uint64_t *v = (const uint64_t *)val;
+                uint64_t seen[256];
+                for (int p = 0; p < nnz && few; ++p) {
+                    int k = 0;
+                    while (k < nd && seen[k] != v[p]) ++k;  // few values: a short scan, most hits early
+                    if (k == nd) {
+                        if (nd == 256) few = false;
+                        else seen[nd++] = v[p];
+                    }
+                    codes[p] = (unsigned char)k;
+                }
+                if (few) std::memcpy(dict.data(), seen, (size_t)nd * 8);
+            } else {
+                const uint16_t *v = (const uint16_t *)val;
+                std::vector<int> codeOf(65536, -1);
+                uint16_t seen[256];
+                for (int p = 0; p < nnz && few; ++p) {
+                    int k = codeOf[v[p]];
+                    if (k < 0) {
+                        if (nd == 256) few = false;
+                        else {
+                            k = nd;
+                            codeOf[v[p]] = nd;
+                            seen[nd++] = v[p];
+                        }
+                    }
+                    codes[p] = (unsigned char)k;
+                }
+                if (few) std::memcpy(dict.data(), seen, (size_t)nd * 2);
+            }
+            if (few) {
+                void *dc = nullptr;
+                if ((rc = upload_bytes(&dc, codes.data(), (size_t)nnz, (size_t)mx::kCsrPad))) return rc;
+                A.codes = (unsigned char *)dc;
+                if ((rc = upload_bytes(&A.dict, dict.data(), dict.size()))) return rc;
+                A.nDict = nd;
+            }
+        }
     } else {
         if ((rc = upload(&A.col, col, (size_t)nnz, mx::kCsrPad))) return rc;
     }
@@ -998,14 +1047,17 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
     if (!want[0] && !want[1] && !want[2]) want[0] = true;  // a matrix the slice kernel cannot take runs on row tiles whatever was asked
     const int nWant = (int)want[0] + (int)want[1] + (int)want[2];
     int rc;
-    void *tx = nullptr, *ty = nullptr;
-    if (nWant > 1) {
-        if ((rc = upload_bytes(&tx, nullptr, 0, std::max<size_t>(cols * es, 16)))) return rc;
-        if ((rc = upload_bytes(&ty, nullptr, 0, std::max<size_t>(rows * es, 16)))) {
+    void *tx = nullptr, *ty = nullptr;  // an x and a y to time candidates with, when there is a choice
+    auto scratch = [&]() -> int {
+        if (tx) return MX_OK;
+        int e = upload_bytes(&tx, nullptr, 0, std::max<size_t>(cols * es, 16));
+        if (e) return e;
+        if ((e = upload_bytes(&ty, nullptr, 0, std::max<size_t>(rows * es, 16)))) {
             (void)hipFree(tx);
-            return rc;
+            tx = nullptr;
         }
-    }
+        return e;
+    };
     auto build = [&](int v, mx::DeviceCsr &C, mx::DeviceSlices &L) -> int {
         if (v == 0) return upload_csr(plan->dtype, rows, cols, nnz, rowPtr, col, val, C, nullptr);
         if (v == 1) return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, nullptr, L, stripRows);
@@ -1035,12 +1087,21 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
         mx::DeviceSlices L;
         rc = build(v, C, L);
         double ms = 0.0;
-        if (!rc && nWant > 1) {
+        if (!rc && (nWant > 1 || (v == 0 && C.codes))) rc = scratch();
+        if (!rc && (nWant > 1 || (v == 0 && C.codes))) {
             std::swap(plan->csr, C);
             std::swap(plan->slices, L);
             const int keepVariant = plan->csr_variant;
             plan->csr_variant = v;
             rc = time_loop(plan, 3, 10, [&]() { return launch_csr_part(plan, tx, ty, 0, plan->stream); }, &ms);
+            if (!rc && v == 0 && plan->csr.codes) {  // the same rows with one byte per value (MX_CSR_DICT=2: whatever the timing)
+                double msDict = 0.0;
+                plan->csr.useDict = true;
+                rc = time_loop(plan, 3, 10, [&]() { return launch_csr_part(plan, tx, ty, 0, plan->stream); }, &msDict);
+                const char *ed = std::getenv("MX_CSR_DICT");
+                if (!rc && (msDict < ms || (ed && std::atoi(ed) == 2))) ms = msDict;
+                else plan->csr.useDict = false;
+            }
             plan->csr_variant = keepVariant;
             std::swap(plan->csr, C);
             std::swap(plan->slices, L);
@@ -1543,6 +1604,7 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     info->csr_main_nnz = plan->csr_variant == 2 ? (sliceMain ? plan->slices.nnz : plan->csr.nnz) : plan->csr_nnz;
     info->tile_variant = plan->strips.steps > 0 ? 1 : 0;
     info->tile_strip_nnz = plan->strips.vals;
+    info->csr_value_dict = (plan->csr_variant != 1 && plan->csr.useDict) ? plan->csr.nDict : 0;
     return MX_OK;
 }
 

@@ -374,6 +374,41 @@ def test_row_kernel_reductions_on_uneven_rows(mx, ora, reduce, monkeypatch):
             assert rel_l2(got, want) <= (tol if dtype == np.float64 else 2e-2)
 
 
+@pytest.mark.parametrize("dtype", [np.float64, np.float16])
+def test_row_kernel_with_a_value_dictionary(mx, ora, dtype, monkeypatch):
+    """A matrix with few distinct values (here five) may run the row-tile kernel on one byte per
+    entry and a dictionary: rows of every length in one tile, rows longer than a tile, both
+    reductions, y exact on integer data.  More than 256 distinct values: no dictionary."""
+    import torch
+    rng = np.random.default_rng(41)
+    rows, cols = 30000, 20000
+    for reduce in ("rows", "scan"):
+        monkeypatch.setenv("MX_CSR_REDUCE", reduce)
+        monkeypatch.setenv("MX_CSR_DICT", "2")     # use it wherever it exists, whatever the timing says
+        lens = rng.poisson(6, rows)
+        lens[rng.uniform(size=rows) < 0.1] = 0
+        lens[[5, 17000, rows - 1]] = [5000, 9000, 300]
+        A = _random_csr(mx, rng, rows, cols, lens, dtype)
+        vals = rng.choice(np.array([-2, -1, 1, 2, 3]), A.nnz).astype(dtype)
+        A = mx.Csr(rows, cols, A.rowPtr, A.colInd, vals)
+        x = rng.integers(-1, 2, cols).astype(dtype)
+        ref = oracle_y(ora, mx, A, x).astype(np.float64)
+        part = mx.Partition(A, 0.0, 0.0)
+        plan = mx.Plan(part, mx.MX_PLAN_CSR_ROWS)
+        assert plan.info["csr_variant"] == 0 and plan.info["csr_value_dict"] == 5, plan.info
+        y = plan.spmv(torch.from_numpy(x).cuda())
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy().astype(np.float64), ref), reduce
+        plan.close()
+        part.close()
+    many = mx.Csr(rows, cols, A.rowPtr, A.colInd, rng.uniform(-1, 1, A.nnz).astype(dtype))
+    part = mx.Partition(many, 0.0, 0.0)
+    plan = mx.Plan(part, mx.MX_PLAN_CSR_ROWS)
+    assert plan.info["csr_value_dict"] == 0
+    plan.close()
+    part.close()
+
+
 def test_slice_kernel_layouts(mx, ora):
     """The column-slice kernel on shapes that stress its layout: a ragged end of x (columns not a
     multiple of a 16-byte vector), one slice only, several slices of which one is empty, row
