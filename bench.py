@@ -33,6 +33,7 @@ TRAFFIC = {
     (2, "csr_slice_kernel<f64>", False): 48823291,
     (3, "csr_rows_kernel<f64>", False): 287431623,
     (3, "csr_rows_kernel<f64,dict>", False): 101747762,   # one byte per value: the stencil has two distinct values
+    (3, "csr_slice_kernel<f64,dict>", False): 109970561,
     (4, "csr_slice_kernel<f16>", False): 55821536,
     (5, "csr_slice_kernel<f16>", False): 301417778,
     (5, "csr_slice_kernel<f16>", True): 190181456,   # tau=(1,1): the strips run through tile_dense_kernel
@@ -144,8 +145,8 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
         # the CSR part's main kernel alone (the slice variant has a small combine kernel after it)
         ms_main = plan.time_csr_main(xd, yd, warm=warmup, iters=steps)
         name = "csr_slice_kernel<%s>" if info["csr_main_kernel"] == 1 else "csr_rows_kernel<%s>"
-        if info["csr_main_kernel"] == 0 and info["csr_value_dict"]:
-            name = "csr_rows_kernel<%s,dict>"
+        if info["csr_value_dict"]:
+            name = name.replace("<%s>", "<%s,dict>")
         dom = {"kernel": name % dtype, "ms": ms_main,
                "bytes": kernel_bytes(mx, A.dtype, A.rows, A.cols, info["csr_main_nnz"])}
     achieved = dom["bytes"] / (dom["ms"] * 1e-3)
@@ -166,7 +167,10 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
         "roofline": {"bound": "hbm", "kernel": dom["kernel"], "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK,
                      "traffic": TRAFFIC.get((cfg, dom["kernel"], info["tile_nnz"] > 0)),
-                     "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"]},
+                     "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"],
+                     **({"note": "the matrix has %d distinct values and the kernel reads one byte per entry for them: the "
+                                 "algorithmic bytes still count sizeof(valT) per entry, so frac can exceed 1; `traffic` is "
+                                 "what the kernel really moves" % info["csr_value_dict"]} if info["csr_value_dict"] else {})},
         "sweep": [{k: r[k] for k in ("tau_c", "tau_r", "ms_total", "ms_tile", "ms_csr", "tile_nnz")} for r in table],
     }
     if cpu_baseline:

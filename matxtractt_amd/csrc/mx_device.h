@@ -108,6 +108,12 @@ struct DeviceSlices {
     int *chunkEnd = nullptr;          // [chunks] step, counted from the wave's first, at which the chunk ends
     unsigned short *ecol = nullptr;   // [batches][64][kSliceBatchEntries] col - slice * sliceCols
     void *eval = nullptr;             // [batches] values, laid out as described above
+    // a matrix with at most 256 distinct values: a byte per entry (at the place of its column
+    // offset) that names the value, and the values (padded to 256)
+    unsigned char *ecode = nullptr;   // [batches][64][kSliceBatchEntries]
+    void *dict = nullptr;             // [256]
+    int nDict = 0;
+    bool useDict = false;             // the plan found this form the faster one
     void *partial = nullptr;          // [chunks*64] accumulators
     int *rowInfo = nullptr;           // [rows, padded to a multiple of 4 with -2]
     int *segIdx = nullptr;            // [vrows] virtual rows listed matrix row by matrix row

@@ -503,6 +503,26 @@ struct SliceBatch<_Float16> {
         return (float)__builtin_bit_cast(_Float16, (unsigned short)vi) * (float)xs[ci];
     }
 };
+// The same with a value dictionary: a byte per entry that names one of at most 256 distinct
+// values (kept as accumulators in LDS) in place of the value itself.
+template <typename VT>
+struct SliceBatchDict {
+    typedef typename Acc<VT>::type AT;
+    v4i32 c;
+    v2i32 k;
+    __device__ __forceinline__ void load(const unsigned short *ecol, const unsigned char *ecode, size_t batch, int lane)
+    {
+        c = __builtin_nontemporal_load((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
+        k = __builtin_nontemporal_load((const v2i32 *)(ecode + (batch * 64 + lane) * 8));
+    }
+    __device__ __forceinline__ AT term(const VT *xs, int j, const AT *dict) const
+    {
+        const unsigned cw = (unsigned)c[j >> 1];
+        const unsigned ci = (j & 1) ? cw >> 16 : cw & 0xffffu;
+        const unsigned code = ((unsigned)k[j >> 2] >> (8 * (j & 3))) & 255u;
+        return dict[code] * (AT)xs[ci];
+    }
+};
 static_assert(mx::kSliceBatchEntries == 8, "SliceBatch holds 8 entries per lane");
 
 // What a CU can take in from L2 or beyond is bounded in bytes (about 32 per cycle, whatever
@@ -511,22 +531,31 @@ static_assert(mx::kSliceBatchEntries == 8, "SliceBatch holds 8 entries per lane"
 // every consumed batch is reloaded with the batch one ring length ahead.
 constexpr int kSliceRing = 6;
 
-template <typename VT>
+// DICT: `eval` points at one byte per entry (same places as the column offsets) and `dictG` at the
+// 256 values they name; a workgroup keeps those in LDS behind the chunk ends.
+template <typename VT, bool DICT = false>
 __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__restrict__ wgDesc,
                                                                   const int4 *__restrict__ waveDesc,
                                                                   const int *__restrict__ chunkEnd,
                                                                   const unsigned short *__restrict__ ecol,
                                                                   const VT *__restrict__ eval, const VT *__restrict__ x,
                                                                   typename Acc<VT>::type *__restrict__ partial, int cols,
-                                                                  int sliceCols)
+                                                                  int sliceCols, const VT *__restrict__ dictG,
+                                                                  int maxWgChunks)
 {
     typedef typename Acc<VT>::type AT;
-    typedef SliceBatch<VT> Batch;
+    typedef typename std::conditional<DICT, SliceBatchDict<VT>, SliceBatch<VT>>::type Batch;
+    typedef typename std::conditional<DICT, unsigned char, VT>::type StreamT;
+    const StreamT *estream = (const StreamT *)eval;
     constexpr int SPB = mx::kSliceBatchEntries, NB = kSliceRing;  // a step is one entry per lane
     constexpr int EPV = 16 / (int)sizeof(VT);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     VT *xs = (VT *)smem;                                           // [sliceCols]
     int *endsL = (int *)(smem + (size_t)sliceCols * sizeof(VT));   // [chunks of the workgroup]
+    AT *dictL = (AT *)(endsL + ((maxWgChunks + 3) & ~3));            // [256] with DICT
+    if constexpr (DICT) {
+        if (threadIdx.x < 256) dictL[threadIdx.x] = (AT)dictG[threadIdx.x];  // visible after the barrier below
+    }
 
     // the workgroups of a slice are numbered consecutively: with every XCD on one contiguous range
     // of them a slice of x is fetched into one L2, not into all eight
@@ -559,7 +588,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     Batch buf[NB];
     const int lastBatch = batch0 + max(nb - 1, 0);
 #pragma unroll
-    for (int k = 0; k < NB; ++k) buf[k].load(ecol, eval, (size_t)min(batch0 + k, lastBatch), lane);
+    for (int k = 0; k < NB; ++k) buf[k].load(ecol, estream, (size_t)min(batch0 + k, lastBatch), lane);
     endsL[min(tid, wgChunks - 1)] = ce;
     if ((slice + 1) * sliceCols <= cols) {  // the whole slice lies inside x
 #pragma unroll
@@ -593,7 +622,8 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     auto consume = [&](const Batch &B, int t) {  // t = number of the batch in the wave's stream
 #pragma unroll
         for (int j = 0; j < SPB; ++j) {
-            acc += B.term(xs, j);
+            if constexpr (DICT) acc += B.term(xs, j, dictL);
+            else acc += B.term(xs, j);
             if (t * SPB + j + 1 == nextEnd) flush();
         }
     };
@@ -609,7 +639,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 #pragma unroll
         for (int k = 0; k < NB; ++k) {
             consume(buf[k], t + k);
-            buf[k].load(ecol, eval, (size_t)(batch0 + t + NB + k), lane);
+            buf[k].load(ecol, estream, (size_t)(batch0 + t + NB + k), lane);
         }
     }
     // one ring in flight and less than one more to come: consume and reload while batches
@@ -617,7 +647,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
         consume(buf[k], t + k);
-        buf[k].load(ecol, eval, (size_t)min(batch0 + t + NB + k, lastBatch), lane);
+        buf[k].load(ecol, estream, (size_t)min(batch0 + t + NB + k, lastBatch), lane);
     }
 #pragma unroll
     for (int k = 0; k < NB; ++k)
@@ -1046,20 +1076,30 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
                                   const DeviceTiles *strips)
 {
     typedef typename mxk::Acc<VT>::type AT;
-    const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)P.maxWgChunks * 4 + 64;
+    const bool dict = P.useDict && P.ecode && P.dict;
+    const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)((P.maxWgChunks + 3) & ~3) * 4 + 64 + (dict ? 256 * sizeof(AT) : 0);
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT>,
+        hipError_t e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT, false>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT, true>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
     if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16))
         return hipErrorInvalidValue;
-    if (what != 2 && P.nWG > 0)
-        hipLaunchKernelGGL((mxk::csr_slice_kernel<VT>), dim3(P.nWG), dim3(kSliceThreads), lds, s,
-                           (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.eval,
-                           (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols);
+    if (what != 2 && P.nWG > 0) {
+        if (dict)
+            hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, true>), dim3(P.nWG), dim3(kSliceThreads), lds, s,
+                               (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.ecode,
+                               (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols, (const VT *)P.dict, P.maxWgChunks);
+        else
+            hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, false>), dim3(P.nWG), dim3(kSliceThreads), lds, s,
+                               (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.eval,
+                               (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols, (const VT *)nullptr, P.maxWgChunks);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || what == 1) return e;
     const int nRowWG = (P.rows + mxk::kCombineRows * mxk::kBlock - 1) / (mxk::kCombineRows * mxk::kBlock);

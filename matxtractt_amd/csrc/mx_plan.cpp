@@ -103,6 +103,8 @@ void free_slices(mx::DeviceSlices &P)
     (void)hipFree(P.wgDesc);
     (void)hipFree(P.ecol);
     (void)hipFree(P.eval);
+    (void)hipFree(P.ecode);
+    (void)hipFree(P.dict);
     (void)hipFree(P.partial);
     (void)hipFree(P.rowInfo);
     (void)hipFree(P.lightRow);
@@ -124,6 +126,48 @@ int slice_count(mx_dtype dtype, int rows, int cols, int nnz, int nCU)
     return S;
 }
 
+// The distinct values (bit patterns) of a matrix, when there are at most `most` (<= 256):
+// codes[p] names the value of entry p, dict holds the values padded with zeros to 256.  False when
+// there are more.
+bool make_value_dict(int es, const void *val, int nnz, std::vector<unsigned char> &codes, std::vector<unsigned char> &dict,
+                     int *nDict, int most = 256)
+{
+    codes.assign((size_t)nnz, 0);
+    dict.assign((size_t)256 * es, 0);
+    int nd = 0;
+    if (es == 8) {
+        const uint64_t *v = (const uint64_t *)val;
+        uint64_t seen[256];
+        for (int p = 0; p < nnz; ++p) {
+            int k = 0;
+            while (k < nd && seen[k] != v[p]) ++k;  // few values: a short scan, most hits early
+            if (k == nd) {
+                if (nd == most) return false;
+                seen[nd++] = v[p];
+            }
+            codes[p] = (unsigned char)k;
+        }
+        std::memcpy(dict.data(), seen, (size_t)nd * 8);
+    } else {
+        const uint16_t *v = (const uint16_t *)val;
+        std::vector<int> codeOf(65536, -1);
+        uint16_t seen[256];
+        for (int p = 0; p < nnz; ++p) {
+            int k = codeOf[v[p]];
+            if (k < 0) {
+                if (nd == most) return false;
+                k = nd;
+                codeOf[v[p]] = nd;
+                seen[nd++] = v[p];
+            }
+            codes[p] = (unsigned char)k;
+        }
+        std::memcpy(dict.data(), seen, (size_t)nd * 2);
+    }
+    *nDict = nd;
+    return true;
+}
+
 // Re-lays the rows `sel` marks (all rows when null) of a CSR matrix for csr_slice_kernel (see
 // DeviceSlices).
 struct HostSlices {
@@ -133,6 +177,8 @@ struct HostSlices {
     std::vector<int> wgDesc, waveDesc, chunkEnd, segPtr, segIdx, rowInfo, lightInfo, heavyInfo;
     std::vector<unsigned short> ecol;
     std::vector<unsigned char> eval;
+    std::vector<unsigned char> ecode, dict;  // value dictionary form (empty when the rows hold more than 256 values)
+    int nDict = 0;
 };
 
 // `elsewhere` (optional) marks rows whose result another kernel writes (the strips of a binary16
@@ -314,6 +360,18 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     const size_t padSteps = 16;  // spare zero steps after the last
     std::vector<unsigned short> ecol(((size_t)totalSteps + padSteps) * 64 * E, 0);
     std::vector<unsigned char> ev(((size_t)totalSteps + padSteps) * 64 * E * es, 0);
+    // one byte per entry instead of its value when the selected rows hold at most 256 distinct
+    // values (MX_CSR_DICT=0: never)
+    std::vector<unsigned char> codeOfEntry, dictv, ecode;
+    int nDict = 0;
+    bool haveDict = false;
+    {
+        const char *ed = std::getenv("MX_CSR_DICT");
+        // (255 values at most: code 255 names the zero that the padding of the layout multiplies x with)
+        if (!sel && nnz >= 65536 && !(ed && !std::atoi(ed)))
+            haveDict = make_value_dict(es, val, rowPtr[rows], codeOfEntry, dictv, &nDict, 255);
+        if (haveDict) ecode.assign(ecol.size(), 255);
+    }
     std::vector<int> wgDesc((size_t)nWG * 4 + 4, 0), waveDesc((size_t)nWG * W * 4 + 4, 0), chunkEnd((size_t)totalChunks + 64, 0);
     std::vector<int> segIdx((size_t)nV + 1, 0);
     const unsigned char *sv = (const unsigned char *)val;
@@ -346,6 +404,7 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
                         const size_t atc = (batch * 64 + l) * BE + k;
                         const size_t atv = dtype == MX_F64 ? batch * 64 * BE + (k / 2) * 128 + (size_t)l * 2 + k % 2 : atc;
                         ecol[atc] = (unsigned short)(col[p] - q * SW);
+                        if (haveDict) ecode[atc] = codeOfEntry[p];
                         std::memcpy(&ev[atv * es], sv + (size_t)p * es, es);
                     }
                 }
@@ -389,6 +448,11 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     D.heavyInfo.swap(heavyInfo);
     D.ecol.swap(ecol);
     D.eval.swap(ev);
+    if (haveDict) {
+        D.ecode.swap(ecode);
+        D.dict.swap(dictv);
+        D.nDict = nDict;
+    }
     return MX_OK;
 }
 
@@ -416,6 +480,13 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
     if ((rc = upload(&D.chunkEnd, H.chunkEnd.data(), H.chunkEnd.size()))) return rc;
     if ((rc = upload(&D.ecol, H.ecol.data(), H.ecol.size()))) return rc;
     if ((rc = upload_bytes(&D.eval, H.eval.data(), H.eval.size()))) return rc;
+    if (!H.ecode.empty()) {
+        void *dc = nullptr;
+        if ((rc = upload_bytes(&dc, H.ecode.data(), H.ecode.size()))) return rc;
+        D.ecode = (unsigned char *)dc;
+        if ((rc = upload_bytes(&D.dict, H.dict.data(), H.dict.size()))) return rc;
+        D.nDict = H.nDict;
+    }
     if ((rc = upload_bytes(&D.partial, nullptr, 0, ((size_t)H.chunks * 64 + 64) * (dtype == MX_F64 ? 8 : 4)))) return rc;
     if ((rc = upload(&D.rowInfo, H.rowInfo.data(), H.rowInfo.size()))) return rc;
     if ((rc = upload(&D.segIdx, H.segIdx.data(), H.segIdx.size()))) return rc;
@@ -772,41 +843,9 @@ int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, c
         // values; the plan times both forms (MX_CSR_DICT=0: never)
         const char *ed = std::getenv("MX_CSR_DICT");
         if (nnz >= 65536 && !(ed && !std::atoi(ed))) {
-            std::vector<unsigned char> codes((size_t)nnz);
-            std::vector<unsigned char> dict((size_t)256 * es, 0);
+            std::vector<unsigned char> codes, dict;
             int nd = 0;
-            bool few = true;
-            if (es == 8) {
-                const uint64_t *v = (const uint64_t *)val;
-                uint64_t seen[256];
-                for (int p = 0; p < nnz && few; ++p) {
-                    int k = 0;
-                    while (k < nd && seen[k] != v[p]) ++k;  // few values: a short scan, most hits early
-                    if (k == nd) {
-                        if (nd == 256) few = false;
-                        else seen[nd++] = v[p];
-                    }
-                    codes[p] = (unsigned char)k;
-                }
-                if (few) std::memcpy(dict.data(), seen, (size_t)nd * 8);
-            } else {
-                const uint16_t *v = (const uint16_t *)val;
-                std::vector<int> codeOf(65536, -1);
-                uint16_t seen[256];
-                for (int p = 0; p < nnz && few; ++p) {
-                    int k = codeOf[v[p]];
-                    if (k < 0) {
-                        if (nd == 256) few = false;
-                        else {
-                            k = nd;
-                            codeOf[v[p]] = nd;
-                            seen[nd++] = v[p];
-                        }
-                    }
-                    codes[p] = (unsigned char)k;
-                }
-                if (few) std::memcpy(dict.data(), seen, (size_t)nd * 2);
-            }
+            const bool few = make_value_dict(es, val, nnz, codes, dict, &nd);
             if (few) {
                 void *dc = nullptr;
                 if ((rc = upload_bytes(&dc, codes.data(), (size_t)nnz, (size_t)mx::kCsrPad))) return rc;
@@ -1087,13 +1126,22 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
         mx::DeviceSlices L;
         rc = build(v, C, L);
         double ms = 0.0;
-        if (!rc && (nWant > 1 || (v == 0 && C.codes))) rc = scratch();
-        if (!rc && (nWant > 1 || (v == 0 && C.codes))) {
+        const bool choice = nWant > 1 || (v == 0 && C.codes) || (v == 1 && L.ecode);
+        if (!rc && choice) rc = scratch();
+        if (!rc && choice) {
             std::swap(plan->csr, C);
             std::swap(plan->slices, L);
             const int keepVariant = plan->csr_variant;
             plan->csr_variant = v;
             rc = time_loop(plan, 3, 10, [&]() { return launch_csr_part(plan, tx, ty, 0, plan->stream); }, &ms);
+            if (!rc && v == 1 && plan->slices.ecode) {  // the same slices with one byte per value
+                double msDict = 0.0;
+                plan->slices.useDict = true;
+                rc = time_loop(plan, 3, 10, [&]() { return launch_csr_part(plan, tx, ty, 0, plan->stream); }, &msDict);
+                const char *ed = std::getenv("MX_CSR_DICT");
+                if (!rc && (msDict < ms || (ed && std::atoi(ed) == 2))) ms = msDict;
+                else plan->slices.useDict = false;
+            }
             if (!rc && v == 0 && plan->csr.codes) {  // the same rows with one byte per value (MX_CSR_DICT=2: whatever the timing)
                 double msDict = 0.0;
                 plan->csr.useDict = true;
@@ -1604,7 +1652,8 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     info->csr_main_nnz = plan->csr_variant == 2 ? (sliceMain ? plan->slices.nnz : plan->csr.nnz) : plan->csr_nnz;
     info->tile_variant = plan->strips.steps > 0 ? 1 : 0;
     info->tile_strip_nnz = plan->strips.vals;
-    info->csr_value_dict = (plan->csr_variant != 1 && plan->csr.useDict) ? plan->csr.nDict : 0;
+    info->csr_value_dict = plan->csr_variant == 1 ? (plan->slices.useDict ? plan->slices.nDict : 0)
+                                                  : (plan->csr.useDict ? plan->csr.nDict : 0);
     return MX_OK;
 }
 

@@ -409,6 +409,33 @@ def test_row_kernel_with_a_value_dictionary(mx, ora, dtype, monkeypatch):
     part.close()
 
 
+@pytest.mark.parametrize("dtype", [np.float64, np.float16])
+def test_slice_kernel_with_a_value_dictionary(mx, ora, dtype, monkeypatch):
+    """The column-slice kernel on one byte per entry and a dictionary (a matrix with five distinct
+    values): several slices, a ragged last one, rows of every length, y exact on integer data."""
+    import torch
+    rng = np.random.default_rng(43)
+    monkeypatch.setenv("MX_CSR_DICT", "2")
+    rows, cols = (9000, 40001) if dtype == np.float64 else (9000, 150001)
+    lens = rng.poisson(20, rows)
+    lens[rng.uniform(size=rows) < 0.05] = 0
+    lens[[3, rows // 2]] = [6000, 2500]
+    A = _random_csr(mx, rng, rows, cols, lens, dtype)
+    A = mx.Csr(rows, cols, A.rowPtr, A.colInd, rng.choice(np.array([-2, -1, 1, 2, 3]), A.nnz).astype(dtype))
+    x = rng.integers(-1, 2, cols).astype(dtype)
+    ref = oracle_y(ora, mx, A, x).astype(np.float64)
+    part = mx.Partition(A, 0.0, 0.0)
+    plan = mx.Plan(part, mx.MX_PLAN_CSR_SLICES)
+    assert plan.info["csr_variant"] == 1 and plan.info["csr_value_dict"] == 5, plan.info
+    xd = torch.from_numpy(x).cuda()
+    for _ in range(2):
+        y = plan.spmv(xd)
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy().astype(np.float64), ref)
+    plan.close()
+    part.close()
+
+
 def test_slice_kernel_layouts(mx, ora):
     """The column-slice kernel on shapes that stress its layout: a ragged end of x (columns not a
     multiple of a 16-byte vector), one slice only, several slices of which one is empty, row
