@@ -118,7 +118,8 @@ struct DeviceSlices {
     int *rowInfo = nullptr;           // [rows, padded to a multiple of 4 with -2]
     int *segIdx = nullptr;            // [vrows] virtual rows listed matrix row by matrix row
     int *lightRow = nullptr;          // [nLight]
-    int *lightIdx = nullptr;          // [nLight][kSliceLightSegs]
+    int *lightIdx = nullptr;          // [nLight][4 * lightQuads]
+    int lightQuads = 2;               // 1 when no light row has more than four virtual rows
     int *heavyInfo = nullptr;         // [nHeavy][4]
     int nLight = 0, nHeavy = 0;
 };

@@ -930,7 +930,7 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
                                                               const int4 *__restrict__ stripWaveDesc,
                                                               const int *__restrict__ stripHdr,
                                                               const VT *__restrict__ stripVal, const VT *__restrict__ x,
-                                                              int nStripWaves, int nStripWG, int nHeavyWG)
+                                                              int nStripWaves, int nStripWG, int nHeavyWG, int lightQuads)
 {
     typedef typename Acc<VT>::type AT;
     const int tid = threadIdx.x;
@@ -980,7 +980,9 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
         if (i >= nLight) return;
         static_assert(mx::kSliceLightSegs == 8, "two int4 of indices per light row");
         const int r = lightRow[i];
-        const int4 i0 = lightIdx[2 * i], i1 = lightIdx[2 * i + 1];
+        // (a layout whose light rows all have at most four virtual rows keeps four places per row)
+        const int4 none = {-1, -1, -1, -1};
+        const int4 i0 = lightQuads == 1 ? lightIdx[i] : lightIdx[2 * i], i1 = lightQuads == 1 ? none : lightIdx[2 * i + 1];
         const int id[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
         AT sum = accumulate ? (AT)y[r] : (AT)0;
 #pragma unroll
@@ -1116,7 +1118,7 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
                        (const int4 *)P.lightIdx, P.nLight, nLightWG, (const int4 *)P.heavyInfo, P.nHeavy, P.segIdx, (VT *)y,    \
                        (accumulate || P.subset) ? 1 : 0, P.subset ? 1 : 0, ride ? (const int4 *)strips->waveDesc : nullptr,   \
                        ride ? strips->hdr : nullptr, ride ? (const VT *)strips->tcVal : nullptr, (const VT *)x,              \
-                       ride ? strips->nWaves : 0, nStripWG, nHeavyWG)
+                       ride ? strips->nWaves : 0, nStripWG, nHeavyWG, P.lightQuads)
     if (ride) MX_LAUNCH_COMBINE(true);
     else MX_LAUNCH_COMBINE(false);
 #undef MX_LAUNCH_COMBINE

@@ -493,11 +493,15 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
     {
         // the light rows' virtual rows, eight places per row
         const int nL = (int)H.lightInfo.size() / 4;
-        std::vector<int> lr((size_t)nL), li((size_t)nL * mx::kSliceLightSegs, -1);
+        int most = 0;
+        for (int i = 0; i < nL; ++i) most = std::max(most, H.lightInfo[4 * (size_t)i + 2]);
+        const int places = most <= 4 ? 4 : mx::kSliceLightSegs;  // four places per row where that is enough
+        D.lightQuads = places / 4;
+        std::vector<int> lr((size_t)nL), li((size_t)nL * places, -1);
         for (int i = 0; i < nL; ++i) {
             lr[i] = H.lightInfo[4 * (size_t)i];
             const int a = H.lightInfo[4 * (size_t)i + 1], n = H.lightInfo[4 * (size_t)i + 2];
-            for (int k = 0; k < n; ++k) li[(size_t)i * mx::kSliceLightSegs + k] = H.segIdx[a + k];
+            for (int k = 0; k < n; ++k) li[(size_t)i * places + k] = H.segIdx[a + k];
         }
         if ((rc = upload(&D.lightRow, lr.data(), lr.size(), 1))) return rc;
         if ((rc = upload(&D.lightIdx, li.data(), li.size(), 8))) return rc;
