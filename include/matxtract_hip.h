@@ -238,9 +238,10 @@ typedef struct mx_plan_info {
                             environment switches this off; with an x that is not 16-byte aligned these chunks
                             run through tile_kernel */
     int tile_strip_nnz;  /* entries held by those chunks */
-    int csr_value_dict;  /* > 0: the row-tile kernel reads one byte per entry, an index into this many distinct
-                            values (matrices with at most 256 of them: stencils, graphs), because the plan
-                            found that faster; 0: values as they are.  MX_CSR_DICT=0 switches it off */
+    int csr_value_dict;  /* > 0: the main kernel of the CSR part reads one byte per entry, an index into this many
+                            distinct values (matrices with at most 255 of them: stencils, graphs), because the
+                            plan found that faster; 0: values as they are.  MX_CSR_DICT=0 switches it off, =2
+                            takes it wherever it exists */
 } mx_plan_info;
 int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
 
