@@ -266,6 +266,9 @@ typedef struct mx_slice_layout_view {
     int *wgDesc, *waveDesc, *chunkEnd, *segPtr, *segIdx, *rowInfo, *lightInfo, *heavyInfo;
     unsigned short *ecol;
     unsigned char *eval;
+    int nDict;            /* > 0: the value dictionary form exists beside the values (at most 255 distinct values) */
+    unsigned char *ecode; /* [nEcol] one byte per entry, at the place of its column offset; 255 = the padding's zero */
+    unsigned char *dict;  /* [256] values (binary64 or binary16), zeros beyond nDict */
 } mx_slice_layout_view;
 int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *sel, mx_slice_layout_view *out);
 void mx_slice_layout_free(mx_slice_layout_view *v);

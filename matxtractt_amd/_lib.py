@@ -60,7 +60,8 @@ class SliceLayoutView(C.Structure):
                                        "batches", "vrows", "nLight", "nHeavy", "lightSegs")] + \
                [("nEcol", C.c_longlong)] + \
                [(n, C.c_void_p) for n in ("wgDesc", "waveDesc", "chunkEnd", "segPtr", "segIdx", "rowInfo", "lightInfo",
-                                        "heavyInfo", "ecol", "eval")]
+                                        "heavyInfo", "ecol", "eval")] + \
+               [("nDict", C.c_int), ("ecode", C.c_void_p), ("dict", C.c_void_p)]
 
 
 class TileLayoutView(C.Structure):

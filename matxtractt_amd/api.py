@@ -215,6 +215,9 @@ def slice_layout(A, nCU=256, sel=None):
         out["heavyInfo"] = _view(v.heavyInfo, v.nHeavy * 4, np.int32).reshape(-1, 4).copy()
         out["ecol"] = _view(v.ecol, v.nEcol, np.uint16).copy()
         out["eval"] = _view(v.eval, v.nEcol, vt).copy()
+        out["nDict"] = int(v.nDict)
+        out["ecode"] = _view(v.ecode, v.nEcol if v.nDict else 0, np.uint8).copy()
+        out["dict"] = _view(v.dict, 256 if v.nDict else 0, vt).copy()
     finally:
         _lib.load().mx_slice_layout_free(C.byref(v))
     return out

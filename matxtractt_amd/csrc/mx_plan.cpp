@@ -928,8 +928,11 @@ extern "C" int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *se
     out->heavyInfo = give(H.heavyInfo);
     out->ecol = give(H.ecol);
     out->eval = give(H.eval);
+    out->nDict = H.ecode.empty() ? 0 : H.nDict;
+    out->ecode = give(H.ecode);
+    out->dict = give(H.dict);
     if (!out->wgDesc || !out->waveDesc || !out->chunkEnd || !out->segPtr || !out->segIdx || !out->rowInfo || !out->lightInfo ||
-        !out->heavyInfo || !out->ecol ||
+        !out->heavyInfo || !out->ecol || !out->ecode || !out->dict ||
         !out->eval) {
         mx_slice_layout_free(out);
         set_error("mx_slice_layout: out of memory");
@@ -951,6 +954,8 @@ extern "C" void mx_slice_layout_free(mx_slice_layout_view *v)
     free(v->heavyInfo);
     free(v->ecol);
     free(v->eval);
+    free(v->ecode);
+    free(v->dict);
     std::memset(v, 0, sizeof(*v));
 }
 

@@ -283,6 +283,10 @@ def _walk_slice_layout(L, x, f64, subset=False):
     BE, W, SW = L["batchEntries"], L["waves"], L["sliceCols"]
     assert L["stepEntries"] == 1   # chunks may end after any entry
     ecol, ev = L["ecol"], L["eval"].astype(np.float64)
+    if L.get("use_dict"):
+        # the value dictionary form: a byte per entry at the place of its column offset names the value
+        assert 0 < L["nDict"] <= 255 and len(L["ecode"]) == len(ecol) and np.all(L["dict"][L["nDict"]:] == 0)
+        assert np.all((L["ecode"] < L["nDict"]) | (L["ecode"] == 255))
     partial = np.full(L["chunks"] * 64, np.nan)
     assert len(ecol) >= L["batches"] * 64 * BE
     lane = np.arange(64)
@@ -305,7 +309,9 @@ def _walk_slice_layout(L, x, f64, subset=False):
             for t in range(nb):
                 bt = batch0 + t
                 c = ecol[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(64, BE).astype(np.int64)
-                if f64:   # sub-blocks of two values per lane
+                if L.get("use_dict"):
+                    v = L["dict"].astype(np.float64)[L["ecode"][bt * 64 * BE:(bt + 1) * 64 * BE]].reshape(64, BE)
+                elif f64:   # sub-blocks of two values per lane
                     v = ev[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(BE // 2, 64, 2).transpose(1, 0, 2).reshape(64, BE)
                 else:
                     v = ev[bt * 64 * BE:(bt + 1) * 64 * BE].reshape(64, BE)
@@ -337,6 +343,27 @@ def _walk_slice_layout(L, x, f64, subset=False):
             y[r] = partial[segIdx[a:a + n]].sum()
     assert not np.isnan(y).any()
     return y, partial
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float16])
+def test_slice_layout_walk_with_a_value_dictionary(mx, ora, dtype):
+    """A matrix with few distinct values: the layout also holds one byte per entry and the values
+    they name; walked through those instead of the values it gives the same sums, bit for bit, and
+    its padding names the zero.  A matrix with more than 255 values has no such form."""
+    rng = np.random.default_rng(12)
+    A, _ = mx.gen_config(5 if dtype == np.float16 else 2, scale=1 / 256 if dtype == np.float16 else 1 / 32)
+    assert A.nnz >= 65536
+    few = mx.Csr(A.rows, A.cols, A.rowPtr, A.colInd, rng.choice(np.array([-2.0, -0.5, 0.25, 1.0, 3.0]), A.nnz).astype(dtype))
+    x = rng.integers(-2, 3, A.cols).astype(np.float64)
+    L = mx.slice_layout(few, nCU=8)
+    assert L["nDict"] == 5
+    y_plain, p_plain = _walk_slice_layout(L, x, dtype == np.float64)
+    L["use_dict"] = True
+    y_dict, p_dict = _walk_slice_layout(L, x, dtype == np.float64)
+    assert np.array_equal(p_plain, p_dict) and np.array_equal(y_plain, y_dict)
+    M = sp.csr_matrix((few.val.astype(np.float64), few.colInd, few.rowPtr), shape=(few.rows, few.cols))
+    assert np.array_equal(y_dict, M @ x)
+    assert mx.slice_layout(A, nCU=8)["nDict"] == 0   # the generator's values: thousands of them
 
 
 @pytest.mark.parametrize("case", ["block", "powerlaw", "mixed", "unsorted", "tiny", "wide_f64", "subset"])
