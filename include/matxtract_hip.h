@@ -118,6 +118,18 @@ int mx_transpose(mx_dtype dtype, int outer, int inner, int nnz, const int *ptr, 
                  const void *val, int **tPtr, int **tInd, void **tVal);
 void mx_free(void *p);
 
+/* The same transpose on the device, as the reference runs it (csr2csc / csc2csr upload the
+ * matrix, call cusparseCsr2cscEx2 and download the result, utilities/csr2csc.cpp:4-203) -- but
+ * on arrays that already live in device memory and stay there.  Every pointer is a device
+ * pointer; the caller provides tPtr_dev[inner + 1], tInd_dev[nnz] and tVal_dev[nnz].  The order
+ * inside every output line is mx_transpose's (ascending source line, equal pairs in source
+ * order), so both give the same arrays.  Scratch memory (about 16 bytes per entry plus the
+ * sort's own) is allocated and released inside the call, which returns after `stream` (a
+ * hipStream_t, or NULL) has finished the work.  MX_ERR_ARG when an index lies outside
+ * [0, inner), MX_ERR_ALLOC / MX_ERR_DEVICE as elsewhere. */
+int mx_transpose_device(mx_dtype dtype, int outer, int inner, int nnz, const int *ptr_dev, const int *ind_dev,
+                        const void *val_dev, int *tPtr_dev, int *tInd_dev, void *tVal_dev, void *stream);
+
 /* mmio_allinone (utilities/mmio.cpp:1547-1713): Matrix-Market coordinate file -> CSR with
  * entries kept in file order inside each row, symmetric/hermitian files expanded,
  * pattern files given value 1.  Outputs malloc()ed; returns MX_ERR_IO on failure. */

@@ -14,7 +14,7 @@ from . import _lib
 from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLAN_CSR_ROWS, MX_PLAN_DEFAULT,
                    MX_PLAN_KEEP_TILES, MX_PLAN_NO_TILES, MxError, check)
 
-__all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "cdspmv",
+__all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
            "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "plan_layout"]
@@ -119,6 +119,27 @@ def transpose(ptr, ind, val, inner):
                                    C.byref(tp), C.byref(ti), C.byref(tv)))
     return (_take(tp.value, inner + 1, np.int32), _take(ti.value, len(ind), np.int32),
             _take(tv.value, len(ind), val.dtype))
+
+
+def transpose_device(ptr, ind, val, inner, stream=None):
+    """csr2csc / csc2csr on the device: torch device tensors in (int32 ptr and ind, float64 or
+    float16 val), torch device tensors out, same arrays as transpose()."""
+    import torch
+    for name, t, dt in (("ptr", ptr, torch.int32), ("ind", ind, torch.int32)):
+        if (not t.is_cuda) or t.dtype != dt or not t.is_contiguous():
+            raise ValueError("%s must be a contiguous int32 device tensor" % name)
+    if (not val.is_cuda) or val.dtype not in (torch.float64, torch.float16) or not val.is_contiguous() \
+            or val.numel() != ind.numel():
+        raise ValueError("val must be a contiguous float64 or float16 device tensor as long as ind")
+    dt = MX_F64 if val.dtype == torch.float64 else MX_F16
+    nnz = ind.numel()
+    tp = torch.empty(inner + 1, dtype=torch.int32, device=ptr.device)
+    ti = torch.empty(nnz, dtype=torch.int32, device=ptr.device)
+    tv = torch.empty(nnz, dtype=val.dtype, device=ptr.device)
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    check(_lib.load().mx_transpose_device(dt, ptr.numel() - 1, inner, nnz, ptr.data_ptr(), ind.data_ptr(),
+                                          val.data_ptr(), tp.data_ptr(), ti.data_ptr(), tv.data_ptr(), s))
+    return tp, ti, tv
 
 
 class Partition:

@@ -779,3 +779,50 @@ def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
     Q = mx.Partition.load(cache)
     assert (Q.tau_c, Q.tau_r) == (0.75, 0.25) and (Q.rows, Q.cols, Q.nnz) == (A.rows, A.cols, A.nnz)
     Q.close()
+
+
+@pytest.mark.gpu
+def test_device_transpose_equals_the_host_transpose(mx, ora):
+    """mx_transpose_device (csr2csc / csc2csr on arrays that stay in device memory) against
+    mx_transpose and the oracle's transpose: same pointers, same order inside every output line
+    (ascending source line, equal pairs in source order), same value bits -- on sorted rows, on
+    unsorted rows that name columns twice, with empty lines on both sides, on one line, on an
+    empty matrix, wide and tall, both precisions, and at a size where the sort takes several
+    passes; csr -> csc -> csr brings back the matrix with its rows sorted (stably)."""
+    import torch
+    rng = np.random.default_rng(11)
+
+    def check(ptr, ind, val, inner):
+        ptr, ind = np.asarray(ptr, np.int32), np.asarray(ind, np.int32)
+        ref = ora.transpose(ptr, ind, val, inner)
+        host = mx.transpose(ptr, ind, val, inner)
+        got = mx.transpose_device(torch.from_numpy(ptr).cuda(), torch.from_numpy(ind).cuda(),
+                                  torch.from_numpy(val).cuda(), inner)
+        got = [g.cpu().numpy() for g in got]
+        for g, h, r in zip(got, host, ref):
+            assert np.array_equal(g.view(np.uint8), r.view(np.uint8))
+            assert np.array_equal(h.view(np.uint8), r.view(np.uint8))
+        return got
+
+    for dtype in (np.float64, np.float16):
+        for outer, inner, lo, hi in [(80, 60, 0, 12), (7, 3000, 0, 40), (3000, 7, 0, 5), (1, 50, 50, 50), (50, 1, 0, 1),
+                                     (4096, 70000, 0, 48)]:
+            lens = rng.integers(lo, hi + 1, outer)
+            ptr = np.concatenate([[0], np.cumsum(lens)])
+            ind = rng.integers(0, inner, ptr[-1])  # unsorted, columns named twice
+            val = rng.uniform(-1, 1, ptr[-1]).astype(dtype)
+            tp, ti, tv = check(ptr, ind, val, inner)
+            bp, bi, bv = check(tp, ti, tv, outer)  # back again: rows sorted by column, stably
+            assert np.array_equal(bp, ptr)
+            for r in range(0, outer, max(1, outer // 16)):
+                o = np.argsort(ind[ptr[r]:ptr[r + 1]], kind="stable")
+                assert np.array_equal(bi[ptr[r]:ptr[r + 1]], ind[ptr[r]:ptr[r + 1]][o])
+                assert np.array_equal(bv[ptr[r]:ptr[r + 1]].view(np.uint8), val[ptr[r]:ptr[r + 1]][o].view(np.uint8))
+        check(np.zeros(6, np.int32), np.zeros(0, np.int32), np.zeros(0, dtype), 9)  # no entries
+    # a workload at full size: workload 2 (4.2 M entries, 17 key bits)
+    A, _ = mx.gen_config(2)
+    check(A.rowPtr, A.colInd, A.val, A.cols)
+    # an index outside [0, inner) is refused, not followed
+    with pytest.raises(mx.MxError):
+        mx.transpose_device(torch.tensor([0, 2], dtype=torch.int32).cuda(), torch.tensor([1, 5], dtype=torch.int32).cuda(),
+                            torch.tensor([1.0, 2.0], dtype=torch.float64).cuda(), 5)
