@@ -130,6 +130,23 @@ void mx_free(void *p);
 int mx_transpose_device(mx_dtype dtype, int outer, int inner, int nnz, const int *ptr_dev, const int *ind_dev,
                         const void *val_dev, int *tPtr_dev, int *tInd_dev, void *tVal_dev, void *stream);
 
+/* The two selections of the cascaded extraction, on a matrix that lives in device memory
+ * (test/test_autotc_spmv.cpp:1122-1141 for the columns, :1240-1267 for the rows; the reference
+ * counts through its transposes and sorts with qsort on the host):
+ *   descColId_dev[cols] = the columns by entry count descending, ties by ascending column;
+ *   dCols = the shortest prefix whose counts sum to >= (int)((float)nnz * tau_c), nnzColD its sum;
+ *   descRowId_dev[rows] = the rows by their number of entries in those dCols columns, descending,
+ *   ties by ascending row; dRows, nnzRowD likewise with tau_r (the first dRows are rId).
+ * These are the values mx_partition_create derives on the host (a target out of reach selects
+ * every line with a count above zero, as there).  rowPtr_dev, colInd_dev and both outputs are
+ * device pointers; `out` is host memory.  Scratch is allocated and released inside; the call
+ * returns after `stream` has finished. */
+typedef struct mx_selection {
+    int dCols, nnzColD, dRows, nnzRowD;
+} mx_selection;
+int mx_select_device(int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev, float tau_c,
+                     float tau_r, int *descColId_dev, int *descRowId_dev, mx_selection *out, void *stream);
+
 /* mmio_allinone (utilities/mmio.cpp:1547-1713): Matrix-Market coordinate file -> CSR with
  * entries kept in file order inside each row, symmetric/hermitian files expanded,
  * pattern files given value 1.  Outputs malloc()ed; returns MX_ERR_IO on failure. */

@@ -14,7 +14,7 @@ from . import _lib
 from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLAN_CSR_ROWS, MX_PLAN_DEFAULT,
                    MX_PLAN_KEEP_TILES, MX_PLAN_NO_TILES, MxError, check)
 
-__all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "cdspmv",
+__all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
            "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "plan_layout"]
@@ -140,6 +140,23 @@ def transpose_device(ptr, ind, val, inner, stream=None):
     check(_lib.load().mx_transpose_device(dt, ptr.numel() - 1, inner, nnz, ptr.data_ptr(), ind.data_ptr(),
                                           val.data_ptr(), tp.data_ptr(), ti.data_ptr(), tv.data_ptr(), s))
     return tp, ti, tv
+
+
+def select_device(rowPtr, colInd, cols, tau_c, tau_r, stream=None):
+    """The column and row selections of the cascaded extraction on a device-resident CSR matrix:
+    returns (descColId, descRowId, {dCols, nnzColD, dRows, nnzRowD}); the orders are device tensors."""
+    import torch
+    for name, t in (("rowPtr", rowPtr), ("colInd", colInd)):
+        if (not t.is_cuda) or t.dtype != torch.int32 or not t.is_contiguous():
+            raise ValueError("%s must be a contiguous int32 device tensor" % name)
+    rows = rowPtr.numel() - 1
+    dc = torch.empty(cols, dtype=torch.int32, device=rowPtr.device)
+    dr = torch.empty(rows, dtype=torch.int32, device=rowPtr.device)
+    out = (C.c_int * 4)()
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    check(_lib.load().mx_select_device(rows, cols, colInd.numel(), rowPtr.data_ptr(), colInd.data_ptr(), tau_c, tau_r,
+                                       dc.data_ptr(), dr.data_ptr(), C.cast(out, C.c_void_p), s))
+    return dc, dr, dict(zip(("dCols", "nnzColD", "dRows", "nnzRowD"), out))
 
 
 class Partition:

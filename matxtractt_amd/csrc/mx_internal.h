@@ -15,6 +15,15 @@ constexpr int kFragM = 8;
 
 void set_error(const std::string &msg);
 
+// `int dColsNnz = nnzA * colProp;` (test/test_autotc_spmv.cpp:1131, :1249): int * float is a float
+// product, truncated.
+inline int threshold(int nnz, float frac)
+{
+    float t = (float)nnz * frac;
+    if (t >= 2147483648.0f) return 2147483647;
+    return (int)t;
+}
+
 // double -> binary16 bits, round to nearest even, straight from the double (no
 // intermediate float rounding); binary16 bits -> float.
 uint16_t f64_to_f16_bits(double v);

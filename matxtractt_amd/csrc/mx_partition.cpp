@@ -42,13 +42,7 @@ void order_by_count_desc(const std::vector<int> &cnt, std::vector<int> &order)
     for (int i = 0; i < n; ++i) order[start[cnt[i]]++] = i;
 }
 
-// `int dColsNnz = nnzA * colProp;` (:1131, :1249): int * float is a float product, truncated.
-int threshold(int nnz, float frac)
-{
-    float t = (float)nnz * frac;
-    if (t >= 2147483648.0f) return 2147483647;
-    return (int)t;
-}
+using mx::threshold;
 
 // Shortest prefix of `order` whose counts sum to >= target (:1133-1141, :1251-1259).  An
 // unreachable target (possible only through float rounding of nnz) selects every line with

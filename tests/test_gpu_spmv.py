@@ -826,3 +826,40 @@ def test_device_transpose_equals_the_host_transpose(mx, ora):
     with pytest.raises(mx.MxError):
         mx.transpose_device(torch.tensor([0, 2], dtype=torch.int32).cuda(), torch.tensor([1, 5], dtype=torch.int32).cuda(),
                             torch.tensor([1.0, 2.0], dtype=torch.float64).cuda(), 5)
+
+
+@pytest.mark.gpu
+def test_device_selection_equals_the_host_partition(mx, ora):
+    """mx_select_device (column counts, order by count with ties by id, shortest prefix that
+    reaches (int)((float)nnz*tau); then the same on the rows' counts inside the chosen columns)
+    against what mx_partition_create derives on the host and the oracle: descColId whole, rId,
+    dCols, dRows and both sums -- on all five workloads at reduced size over a tau grid that
+    includes tau_r = 0 (one row) and tau = 1 (every line with an entry), on a matrix whose
+    columns all have the same count (ties only), on one with empty rows and columns, and on
+    workload 2 at full size."""
+    import torch
+    cases = [mx.gen_config(c, scale=s)[0] for c, s in [(1, 0.5), (2, 1 / 16), (3, 0.008), (4, 1 / 64), (5, 1 / 256)]]
+    n = 48  # circulant: every row and column holds 5 entries
+    ptr = np.arange(0, 5 * n + 1, 5, dtype=np.int32)
+    ind = ((np.arange(n)[:, None] * 7 + np.array([0, 3, 11, 20, 33])[None, :]) % n).astype(np.int32).ravel()
+    cases.append(mx.Csr(n, n, ptr, ind, np.ones(5 * n)))
+    rng = np.random.default_rng(5)
+    lens = rng.integers(0, 4, 300) * (rng.random(300) < 0.5)
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cases.append(mx.Csr(300, 900, ptr, rng.integers(0, 450, ptr[-1]).astype(np.int32), np.ones(ptr[-1])))
+    cases.append(mx.gen_config(2)[0])
+    for A in cases:
+        rp, ci = torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda()
+        for tau in [(0.25, 0.0), (0.5, 0.25), (0.75, 0.75), (1.0, 0.5), (1.0, 1.0), (0.01, 0.01)]:
+            P = mx.Partition(A, *tau)
+            dc, dr, sel = mx.select_device(rp, ci, A.cols, *tau)
+            assert sel == {"dCols": P.dCols, "nnzColD": P.nnzColD, "dRows": P.dRows, "nnzRowD": P.nnzRowD}, (tau, sel)
+            assert np.array_equal(dc.cpu().numpy(), P.descColId)
+            assert np.array_equal(dr.cpu().numpy()[:P.dRows], P.rId)
+            if A.rows <= 70000:
+                O = ora.partition(A.rowPtr, A.colInd, A.val, A.cols, *tau)
+                assert np.array_equal(dc.cpu().numpy(), O.descColId) and np.array_equal(dr.cpu().numpy()[:P.dRows], O.rId)
+                assert (O.dCols, O.nnzColD, O.dRows, O.nnzRowD) == (sel["dCols"], sel["nnzColD"], sel["dRows"], sel["nnzRowD"])
+            P.close()
+    with pytest.raises(mx.MxError):  # tau_c < tau_r
+        mx.select_device(rp, ci, A.cols, 0.25, 0.5)
