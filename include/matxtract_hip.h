@@ -147,6 +147,23 @@ typedef struct mx_selection {
 int mx_select_device(int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev, float tau_c,
                      float tau_r, int *descColId_dev, int *descRowId_dev, mx_selection *out, void *stream);
 
+/* The split that follows the selections (test/test_autotc_spmv.cpp:1286-1300 for A_dd,
+ * :129-250 merge2CSR_opt for the residual), device arrays in and out.  With `sel`, descColId_dev
+ * and descRowId_dev as mx_select_device left them:
+ *   A_dd  = the dRows selected rows in rank order, their entries in selected columns, column =
+ *           rank of the column, ascending (ddRowPtr_dev[dRows + 1], ddColInd_dev / ddVal_dev[nnzRowD]);
+ *   A_CD  = every row in place: first its entries in unselected columns (column = dCols + position
+ *           of the column among the unselected, ascending), then, for a row that was not selected,
+ *           its entries in selected columns (cdRowPtr_dev[rows + 1], cdColInd_dev / cdVal_dev[nnz - nnzRowD]).
+ * Entries that name the same row and column twice keep their source order.  The arrays equal
+ * mx_partition_create's ddRowPtr .. cdVal.  The caller sizes the outputs from `sel`; a selection that
+ * does not belong to the matrix is reported (MX_ERR_ARG) when its totals differ, but its index arrays
+ * are trusted.  Scratch (about 28 bytes per entry) is allocated and released inside. */
+int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
+                    const void *val_dev, const mx_selection *sel, const int *descColId_dev, const int *descRowId_dev,
+                    int *ddRowPtr_dev, int *ddColInd_dev, void *ddVal_dev, int *cdRowPtr_dev, int *cdColInd_dev,
+                    void *cdVal_dev, void *stream);
+
 /* mmio_allinone (utilities/mmio.cpp:1547-1713): Matrix-Market coordinate file -> CSR with
  * entries kept in file order inside each row, symmetric/hermitian files expanded,
  * pattern files given value 1.  Outputs malloc()ed; returns MX_ERR_IO on failure. */

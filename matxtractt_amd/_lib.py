@@ -95,6 +95,7 @@ SIGNATURES = {
     "mx_transpose": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _pp, _pp, _pp]),
     "mx_transpose_device": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mx_select_device": (_i, [_i, _i, _i, _vp, _vp, C.c_float, C.c_float, _vp, _vp, _vp, _vp]),
+    "mx_split_device": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mx_free": (None, [_vp]),
     "mx_mmio_read": (_i, [C.c_char_p, _i, _pi, _pi, _pi, _pi, _pp, _pp, _pp]),
     "mx_init_vec": (None, [_i, _vp, _i]),

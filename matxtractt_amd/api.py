@@ -14,7 +14,7 @@ from . import _lib
 from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLAN_CSR_ROWS, MX_PLAN_DEFAULT,
                    MX_PLAN_KEEP_TILES, MX_PLAN_NO_TILES, MxError, check)
 
-__all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "cdspmv",
+__all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "split_device", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
            "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "plan_layout"]
@@ -157,6 +157,25 @@ def select_device(rowPtr, colInd, cols, tau_c, tau_r, stream=None):
     check(_lib.load().mx_select_device(rows, cols, colInd.numel(), rowPtr.data_ptr(), colInd.data_ptr(), tau_c, tau_r,
                                        dc.data_ptr(), dr.data_ptr(), C.cast(out, C.c_void_p), s))
     return dc, dr, dict(zip(("dCols", "nnzColD", "dRows", "nnzRowD"), out))
+
+
+def split_device(rowPtr, colInd, val, cols, sel, descColId, descRowId, stream=None):
+    """A_dd and the residual A_CD from the selections of select_device(), all device tensors:
+    returns (ddRowPtr, ddColInd, ddVal, cdRowPtr, cdColInd, cdVal)."""
+    import torch
+    rows, nnz = rowPtr.numel() - 1, colInd.numel()
+    dt = MX_F64 if val.dtype == torch.float64 else MX_F16
+    dev, i32 = rowPtr.device, torch.int32
+    nDD = sel["nnzRowD"]
+    out = (torch.empty(sel["dRows"] + 1, dtype=i32, device=dev), torch.empty(nDD, dtype=i32, device=dev),
+           torch.empty(nDD, dtype=val.dtype, device=dev), torch.empty(rows + 1, dtype=i32, device=dev),
+           torch.empty(nnz - nDD, dtype=i32, device=dev), torch.empty(nnz - nDD, dtype=val.dtype, device=dev))
+    csel = (C.c_int * 4)(sel["dCols"], sel["nnzColD"], sel["dRows"], sel["nnzRowD"])
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    check(_lib.load().mx_split_device(dt, rows, cols, nnz, rowPtr.data_ptr(), colInd.data_ptr(), val.data_ptr(),
+                                      C.cast(csel, C.c_void_p), descColId.data_ptr(), descRowId.data_ptr(),
+                                      *[t.data_ptr() for t in out], s))
+    return out
 
 
 class Partition:

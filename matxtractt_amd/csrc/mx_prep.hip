@@ -142,6 +142,81 @@ __global__ __launch_bounds__(kBlock) void dense_row_counts_kernel(const int *__r
     if (dense[col[e]]) atomicAdd(&rcnt[line_of(rowPtr, rows, e)], 1);
 }
 
+// ---- split --------------------------------------------------------------------------------
+// rank[order[i]] = i for the first k lines of the order
+__global__ __launch_bounds__(kBlock) void scatter_rank_kernel(const int *__restrict__ order, int k, int *__restrict__ rank)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < k) rank[order[i]] = i;
+}
+
+// notSel[c] = 1 where the column was not selected (input of the running count that numbers them)
+__global__ __launch_bounds__(kBlock) void not_selected_kernel(const unsigned char *__restrict__ dense, int cols, int *__restrict__ notSel)
+{
+    const int c = blockIdx.x * kBlock + threadIdx.x;
+    if (c <= cols) notSel[c] = c < cols ? !dense[c] : 0;
+}
+
+// new column id of an unselected column: dCols + its position among the unselected, ascending
+__global__ __launch_bounds__(kBlock) void sparse_columns_kernel(const unsigned char *__restrict__ dense, const int *__restrict__ pos,
+                                                                int cols, int dCols, int *__restrict__ newCol)
+{
+    const int c = blockIdx.x * kBlock + threadIdx.x;
+    if (c < cols && !dense[c]) newCol[c] = dCols + pos[c];
+}
+
+// lengths of the residual's rows (entries in unselected columns, plus those in selected columns
+// when the row itself was not selected) and of A_dd's rows (rank order); one more element, zero,
+// so that a running count over n + 1 elements ends with the total
+__global__ __launch_bounds__(kBlock) void split_lengths_kernel(const int *__restrict__ rowPtr, const int *__restrict__ rcnt,
+                                                               const int *__restrict__ rowRank, const int *__restrict__ rowOrder,
+                                                               int rows, int dRows, int *__restrict__ cdLen, int *__restrict__ ddLen)
+{
+    const int r = blockIdx.x * kBlock + threadIdx.x;
+    if (r <= rows) cdLen[r] = r < rows ? (rowPtr[r + 1] - rowPtr[r] - rcnt[r]) + (rowRank[r] < 0 ? rcnt[r] : 0) : 0;
+    if (r <= dRows) ddLen[r] = r < dRows ? rcnt[rowOrder[r]] : 0;
+}
+
+// Sort key of an entry: [which matrix][its row there][residual only: selected column?][new column].
+// A_dd (matrix 0) sorts in front of the residual (matrix 1); inside a residual row the entries in
+// unselected columns come first, then those in selected ones; equal keys keep source order.
+__global__ __launch_bounds__(kBlock) void split_keys_kernel(const int *__restrict__ rowPtr, const int *__restrict__ col,
+                                                            const int *__restrict__ newCol, const int *__restrict__ rowRank,
+                                                            int rows, int nnz, int dCols, int colBits, int rowBits,
+                                                            unsigned long long *__restrict__ key, int *__restrict__ payload)
+{
+    const int e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= nnz) return;
+    const int r = line_of(rowPtr, rows, e), nc = newCol[col[e]], rank = rowRank[r];
+    const bool sel = nc < dCols;
+    unsigned long long k;
+    if (sel && rank >= 0) k = ((unsigned long long)rank << (colBits + 1)) | (unsigned long long)nc;
+    else
+        k = (1ull << (rowBits + colBits + 1)) | ((unsigned long long)r << (colBits + 1)) |
+            ((unsigned long long)sel << colBits) | (unsigned long long)nc;
+    key[e] = k;
+    payload[e] = e;
+}
+
+template <typename V>
+__global__ __launch_bounds__(kBlock) void split_gather_kernel(const unsigned long long *__restrict__ key, const int *__restrict__ payload,
+                                                              const V *__restrict__ val, int nnz, int nDD, int colBits,
+                                                              int *__restrict__ ddInd, V *__restrict__ ddVal,
+                                                              int *__restrict__ cdInd, V *__restrict__ cdVal)
+{
+    const int k = blockIdx.x * kBlock + threadIdx.x;
+    if (k >= nnz) return;
+    const int nc = (int)(key[k] & ((1ull << colBits) - 1));
+    const V v = val[payload[k]];
+    if (k < nDD) {
+        ddInd[k] = nc;
+        ddVal[k] = v;
+    } else {
+        cdInd[k - nDD] = nc;
+        cdVal[k - nDD] = v;
+    }
+}
+
 struct Scratch {
     void *p = nullptr;
     ~Scratch()
@@ -324,4 +399,113 @@ extern "C" int mx_select_device(int rows, int cols, int nnz, const int *rowPtr_d
     rc = order_and_reach(cnt, rows, mx::threshold(nnz, tau_r), descRowId_dev, work, sortTmp, sortBytes, scanTmp, scanBytes, s,
                          &out->dRows, &out->nnzRowD);
     return rc;
+}
+
+#undef MXP_TRY
+#define MXP_TRY(call)                                                                                   \
+    do {                                                                                                \
+        hipError_t e_ = (call);                                                                         \
+        if (e_ != hipSuccess) {                                                                         \
+            mx::set_error(std::string("mx_split_device: ") + #call + ": " + hipGetErrorString(e_));    \
+            return e_ == hipErrorOutOfMemory ? MX_ERR_ALLOC : MX_ERR_DEVICE;                            \
+        }                                                                                               \
+    } while (0)
+
+extern "C" int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
+                               const void *val_dev, const mx_selection *sel, const int *descColId_dev,
+                               const int *descRowId_dev, int *ddRowPtr_dev, int *ddColInd_dev, void *ddVal_dev,
+                               int *cdRowPtr_dev, int *cdColInd_dev, void *cdVal_dev, void *stream)
+{
+    using namespace mxp;
+    if ((dtype != MX_F64 && dtype != MX_F16) || rows < 0 || cols < 0 || nnz < 0 || !sel || !rowPtr_dev || !ddRowPtr_dev ||
+        !cdRowPtr_dev || sel->dCols < 0 || sel->dCols > cols || sel->dRows < 0 || sel->dRows > rows || sel->nnzRowD < 0 ||
+        sel->nnzRowD > nnz || (sel->dCols > 0 && !descColId_dev) || (sel->dRows > 0 && !descRowId_dev) ||
+        (nnz > 0 && (!colInd_dev || !val_dev || rows == 0 || cols == 0)) || (sel->nnzRowD > 0 && (!ddColInd_dev || !ddVal_dev)) ||
+        (nnz - sel->nnzRowD > 0 && (!cdColInd_dev || !cdVal_dev))) {
+        mx::set_error("mx_split_device: bad argument");
+        return MX_ERR_ARG;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    const int dCols = sel->dCols, dRows = sel->dRows, nDD = sel->nnzRowD;
+    int colBits = 1, rowBits = 1;
+    while (colBits < 31 && (1ll << colBits) < (long long)cols) ++colBits;
+    while (rowBits < 31 && (1ll << rowBits) < (long long)rows) ++rowBits;
+    const unsigned keyBits = (unsigned)(colBits + rowBits + 2);
+    const size_t nScan = (size_t)std::max(rows, cols) + 1;
+    size_t sortBytes = 0, scanBytes = 0;
+    if (nnz > 0)
+        MXP_TRY(rocprim::radix_sort_pairs(nullptr, sortBytes, (const unsigned long long *)nullptr, (unsigned long long *)nullptr,
+                                          (const int *)nullptr, (int *)nullptr, (size_t)nnz, 0u, keyBits, s));
+    MXP_TRY(rocprim::exclusive_scan(nullptr, scanBytes, (const int *)nullptr, (int *)nullptr, 0, nScan, rocprim::plus<int>(), s));
+    sortBytes = (sortBytes + 255) & ~(size_t)255;
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const size_t colB = al(((size_t)cols + 1) * sizeof(int)), rowB = al(((size_t)rows + 1) * sizeof(int));
+    const size_t denseB = al((size_t)cols + 1), keyB = al((size_t)nnz * 8), payB = al((size_t)nnz * 4);
+    // newCol, notSel, pos [cols+1]; rowRank, rcnt, cdLen, ddLen [rows+1]; dense; keys and payloads in and out
+    Scratch scratch;
+    MXP_TRY(hipMalloc(&scratch.p, 3 * colB + 4 * rowB + denseB + 2 * keyB + 2 * payB + sortBytes + scanBytes + 256));
+    unsigned char *b = (unsigned char *)scratch.p;
+    int *newCol = (int *)b, *notSel = (int *)(b + colB), *pos = (int *)(b + 2 * colB);
+    b += 3 * colB;
+    int *rowRank = (int *)b, *rcnt = (int *)(b + rowB), *cdLen = (int *)(b + 2 * rowB), *ddLen = (int *)(b + 3 * rowB);
+    b += 4 * rowB;
+    unsigned char *dense = b;
+    b += denseB;
+    unsigned long long *keyIn = (unsigned long long *)b, *keyOut = (unsigned long long *)(b + keyB);
+    b += 2 * keyB;
+    int *payIn = (int *)b, *payOut = (int *)(b + payB);
+    b += 2 * payB;
+    void *sortTmp = b, *scanTmp = b + sortBytes;
+    auto grid = [](long long n) { return dim3((unsigned)((n + kBlock - 1) / kBlock)); };
+
+    // new column ids: rank for a selected column, dCols + position among the others otherwise
+    MXP_TRY(hipMemsetAsync(dense, 0, denseB, s));
+    MXP_TRY(hipMemsetAsync(rowRank, 0xff, rowB, s));  // -1
+    MXP_TRY(hipMemsetAsync(rcnt, 0, rowB, s));
+    if (dCols > 0) {
+        hipLaunchKernelGGL(mark_selected_kernel, grid(dCols), dim3(kBlock), 0, s, descColId_dev, dCols, dense);
+        hipLaunchKernelGGL(scatter_rank_kernel, grid(dCols), dim3(kBlock), 0, s, descColId_dev, dCols, newCol);
+    }
+    hipLaunchKernelGGL(not_selected_kernel, grid((long long)cols + 1), dim3(kBlock), 0, s, (const unsigned char *)dense, cols, notSel);
+    MXP_TRY(hipGetLastError());
+    MXP_TRY(rocprim::exclusive_scan(scanTmp, scanBytes, (const int *)notSel, pos, 0, (size_t)cols + 1, rocprim::plus<int>(), s));
+    if (cols > 0)
+        hipLaunchKernelGGL(sparse_columns_kernel, grid(cols), dim3(kBlock), 0, s, (const unsigned char *)dense, (const int *)pos, cols,
+                           dCols, newCol);
+    // rows: rank of the selected ones, counts inside the selected columns, lengths, pointers
+    if (dRows > 0) hipLaunchKernelGGL(scatter_rank_kernel, grid(dRows), dim3(kBlock), 0, s, descRowId_dev, dRows, rowRank);
+    if (nnz > 0)
+        hipLaunchKernelGGL(dense_row_counts_kernel, grid(nnz), dim3(kBlock), 0, s, rowPtr_dev, colInd_dev,
+                           (const unsigned char *)dense, rows, nnz, rcnt);
+    hipLaunchKernelGGL(split_lengths_kernel, grid((long long)rows + 1), dim3(kBlock), 0, s, rowPtr_dev, (const int *)rcnt,
+                       (const int *)rowRank, descRowId_dev, rows, dRows, cdLen, ddLen);
+    MXP_TRY(hipGetLastError());
+    MXP_TRY(rocprim::exclusive_scan(scanTmp, scanBytes, (const int *)cdLen, cdRowPtr_dev, 0, (size_t)rows + 1, rocprim::plus<int>(), s));
+    MXP_TRY(rocprim::exclusive_scan(scanTmp, scanBytes, (const int *)ddLen, ddRowPtr_dev, 0, (size_t)dRows + 1, rocprim::plus<int>(), s));
+    if (nnz > 0) {
+        hipLaunchKernelGGL(split_keys_kernel, grid(nnz), dim3(kBlock), 0, s, rowPtr_dev, colInd_dev, (const int *)newCol,
+                           (const int *)rowRank, rows, nnz, dCols, colBits, rowBits, keyIn, payIn);
+        MXP_TRY(hipGetLastError());
+        MXP_TRY(rocprim::radix_sort_pairs(sortTmp, sortBytes, (const unsigned long long *)keyIn, keyOut, (const int *)payIn, payOut,
+                                          (size_t)nnz, 0u, keyBits, s));
+        if (dtype == MX_F64)
+            hipLaunchKernelGGL(split_gather_kernel<double>, grid(nnz), dim3(kBlock), 0, s, (const unsigned long long *)keyOut,
+                               (const int *)payOut, (const double *)val_dev, nnz, nDD, colBits, ddColInd_dev, (double *)ddVal_dev,
+                               cdColInd_dev, (double *)cdVal_dev);
+        else
+            hipLaunchKernelGGL(split_gather_kernel<uint16_t>, grid(nnz), dim3(kBlock), 0, s, (const unsigned long long *)keyOut,
+                               (const int *)payOut, (const uint16_t *)val_dev, nnz, nDD, colBits, ddColInd_dev,
+                               (uint16_t *)ddVal_dev, cdColInd_dev, (uint16_t *)cdVal_dev);
+        MXP_TRY(hipGetLastError());
+    }
+    // the totals must be what the caller sized the outputs for
+    int totals[2] = {0, 0};
+    MXP_TRY(hipMemcpyAsync(&totals[0], ddRowPtr_dev + dRows, sizeof(int), hipMemcpyDeviceToHost, s));
+    MXP_TRY(hipMemcpyAsync(&totals[1], cdRowPtr_dev + rows, sizeof(int), hipMemcpyDeviceToHost, s));
+    MXP_TRY(hipStreamSynchronize(s));
+    if (totals[0] != nDD || totals[1] != nnz - nDD) {
+        mx::set_error("mx_split_device: the selection does not belong to this matrix (entry totals differ)");
+        return MX_ERR_ARG;
+    }
+    return MX_OK;
 }

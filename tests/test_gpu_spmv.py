@@ -829,8 +829,9 @@ def test_device_transpose_equals_the_host_transpose(mx, ora):
 
 
 @pytest.mark.gpu
-def test_device_selection_equals_the_host_partition(mx, ora):
-    """mx_select_device (column counts, order by count with ties by id, shortest prefix that
+def test_device_selection_and_split_equal_the_host_partition(mx, ora):
+    """mx_split_device gives A_dd and the residual A_CD of mx_partition_create from those selections,
+    in both precisions (workloads 4 and 5 are binary16), with rows that name a column twice.  mx_select_device (column counts, order by count with ties by id, shortest prefix that
     reaches (int)((float)nnz*tau); then the same on the rows' counts inside the chosen columns)
     against what mx_partition_create derives on the host and the oracle: descColId whole, rId,
     dCols, dRows and both sums -- on all five workloads at reduced size over a tau grid that
@@ -847,6 +848,11 @@ def test_device_selection_equals_the_host_partition(mx, ora):
     lens = rng.integers(0, 4, 300) * (rng.random(300) < 0.5)
     ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     cases.append(mx.Csr(300, 900, ptr, rng.integers(0, 450, ptr[-1]).astype(np.int32), np.ones(ptr[-1])))
+    lens = rng.integers(0, 31, 64)  # unsorted rows that name columns twice, distinct values
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cases.append(mx.Csr(64, 40, ptr, rng.integers(0, 40, ptr[-1]).astype(np.int32), rng.uniform(-1, 1, ptr[-1])))
+    cases.append(mx.Csr(5, 7, np.zeros(6, np.int32), np.zeros(0, np.int32), np.zeros(0)))  # no entries
+    cases.append(mx.Csr(1, 1, np.array([0, 1], np.int32), np.zeros(1, np.int32), np.ones(1)))
     cases.append(mx.gen_config(2)[0])
     for A in cases:
         rp, ci = torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda()
@@ -856,6 +862,11 @@ def test_device_selection_equals_the_host_partition(mx, ora):
             assert sel == {"dCols": P.dCols, "nnzColD": P.nnzColD, "dRows": P.dRows, "nnzRowD": P.nnzRowD}, (tau, sel)
             assert np.array_equal(dc.cpu().numpy(), P.descColId)
             assert np.array_equal(dr.cpu().numpy()[:P.dRows], P.rId)
+            # the split that follows: A_dd and the residual, bit for bit the host partition's
+            got = mx.split_device(rp, ci, torch.from_numpy(A.val).cuda(), A.cols, sel, dc, dr)
+            for g, name in zip(got, ("ddRowPtr", "ddColInd", "ddVal", "cdRowPtr", "cdColInd", "cdVal")):
+                want = getattr(P, name)
+                assert np.array_equal(g.cpu().numpy().view(np.uint8), np.ascontiguousarray(want).view(np.uint8)), (tau, name)
             if A.rows <= 70000:
                 O = ora.partition(A.rowPtr, A.colInd, A.val, A.cols, *tau)
                 assert np.array_equal(dc.cpu().numpy(), O.descColId) and np.array_equal(dr.cpu().numpy()[:P.dRows], O.rId)
