@@ -189,9 +189,10 @@ inline void exclusive_scan(indT *input, int length)
  * column pass with colProp (global_col), row pass with rowProp (local_row), tile format,
  * residual.  Returns NULL after printing the reason when the arguments are rejected
  * (colProp < rowProp, as at :1064-1069).  Inspect with mx_partition_get(); release with
- * mx_partition_destroy(). */
+ * mx_partition_destroy().  onDevice: the extraction runs on the GPU (mx_partition_create_device); the
+ * partition is the same. */
 inline mx_partition *matxtract_preprocess(valT *csrVal, indT *csrRowPtr, indT *csrColInd, int rowA, int colA, indT nnzA,
-                                          float colProp, float rowProp)
+                                          float colProp, float rowProp, bool onDevice = false)
 {
     mx_csr A;
     A.rows = rowA;
@@ -202,7 +203,7 @@ inline mx_partition *matxtract_preprocess(valT *csrVal, indT *csrRowPtr, indT *c
     A.colInd = csrColInd;
     A.val = csrVal;
     mx_partition *p = nullptr;
-    if (mx_partition_create(&A, colProp, rowProp, &p) != MX_OK) {
+    if ((onDevice ? mx_partition_create_device(&A, colProp, rowProp, &p) : mx_partition_create(&A, colProp, rowProp, &p)) != MX_OK) {
         std::fprintf(stderr, "matxtract_preprocess: %s\n", mx_last_error());
         return nullptr;
     }

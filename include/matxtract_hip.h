@@ -164,6 +164,35 @@ int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowP
                     int *ddRowPtr_dev, int *ddColInd_dev, void *ddVal_dev, int *cdRowPtr_dev, int *cdColInd_dev,
                     void *cdVal_dev, void *stream);
 
+/* The tile encoding of A_dd on the device (ecrPreprocess_opt1 test/test_autotc_spmv.cpp:502-585,
+ * chunkPtr and sparse_AToX_index :1369-1404, generateFormat_opt :718-847 / _fp16 :849-978):
+ * from A_dd as mx_split_device left it (rows sorted by column) to the arrays the tile kernels
+ * read.  Per chunk of 8 rows: its distinct columns ascending (sparse_AToX_index, padded with
+ * zeros to whole fragments of fragK = 4 (binary64) or 8 (binary16) columns); per fragment a
+ * bitmap with bit r * fragK + c for an entry in local row r and compacted column c; tcVal in
+ * ascending bit order, of entries naming the same place the last.  The arrays equal
+ * mx_partition_create's.  The library allocates them in one block (device memory) and fills
+ * in `out`; mx_tiles_device_free releases the block. */
+typedef struct mx_device_tiles {
+    int chunkNum, totalTcFrags, fragK, tcValCount;
+    int *chunkPtr;          /* [chunkNum + 1] */
+    int *sparse_AToX_index; /* [totalTcFrags * fragK] */
+    int *fragPtr;           /* [totalTcFrags + 1] */
+    void *fragBit;          /* [totalTcFrags] uint32_t (binary64) or uint64_t (binary16) */
+    void *tcVal;            /* [tcValCount] */
+    void *base;             /* the block that holds them */
+} mx_device_tiles;
+int mx_tiles_device(mx_dtype dtype, int dRows, int dCols, int nnzRowD, const int *ddRowPtr_dev, const int *ddColInd_dev,
+                    const void *ddVal_dev, mx_device_tiles *out, void *stream);
+void mx_tiles_device_free(mx_device_tiles *t);
+
+/* mx_partition_create by the device route: A (host arrays, as there) is uploaded, the three
+ * steps above run on the device and the arrays are copied back into the same kind of handle --
+ * every array, count and the checksum (mx_partition_hash) equal mx_partition_create's, so plans,
+ * files and callers cannot tell the routes apart.  tau = (0, 0) extracts nothing and is handed to
+ * the host routine.  MX_ERR_DEVICE without a HIP device: there is no silent fallback. */
+int mx_partition_create_device(const mx_csr *A, float tau_c, float tau_r, mx_partition **out);
+
 /* mmio_allinone (utilities/mmio.cpp:1547-1713): Matrix-Market coordinate file -> CSR with
  * entries kept in file order inside each row, symmetric/hermitian files expanded,
  * pattern files given value 1.  Outputs malloc()ed; returns MX_ERR_IO on failure. */

@@ -84,9 +84,15 @@ _vp, _i, _d = C.c_void_p, C.c_int, C.c_double
 _pp = C.POINTER(C.c_void_p)
 _pi = C.POINTER(C.c_int)
 _pd = C.POINTER(C.c_double)
+class DeviceTiles(C.Structure):
+    _fields_ = [("chunkNum", _i), ("totalTcFrags", _i), ("fragK", _i), ("tcValCount", _i), ("chunkPtr", _vp),
+                ("sparse_AToX_index", _vp), ("fragPtr", _vp), ("fragBit", _vp), ("tcVal", _vp), ("base", _vp)]
+
+
 SIGNATURES = {
     "mx_last_error": (C.c_char_p, []),
     "mx_partition_create": (_i, [C.POINTER(CsrStruct), C.c_float, C.c_float, _pp]),
+    "mx_partition_create_device": (_i, [C.POINTER(CsrStruct), C.c_float, C.c_float, _pp]),
     "mx_partition_destroy": (None, [_vp]),
     "mx_partition_get": (_i, [_vp, C.POINTER(PartitionView)]),
     "mx_partition_hash": (C.c_uint64, [_vp]),
@@ -96,6 +102,8 @@ SIGNATURES = {
     "mx_transpose_device": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mx_select_device": (_i, [_i, _i, _i, _vp, _vp, C.c_float, C.c_float, _vp, _vp, _vp, _vp]),
     "mx_split_device": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "mx_tiles_device": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, C.POINTER(DeviceTiles), _vp]),
+    "mx_tiles_device_free": (None, [C.POINTER(DeviceTiles)]),
     "mx_free": (None, [_vp]),
     "mx_mmio_read": (_i, [C.c_char_p, _i, _pi, _pi, _pi, _pi, _pp, _pp, _pp]),
     "mx_init_vec": (None, [_i, _vp, _i]),

@@ -14,7 +14,7 @@ from . import _lib
 from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLAN_CSR_ROWS, MX_PLAN_DEFAULT,
                    MX_PLAN_KEEP_TILES, MX_PLAN_NO_TILES, MxError, check)
 
-__all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "split_device", "cdspmv",
+__all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "split_device", "tiles_device", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
            "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "plan_layout"]
@@ -178,17 +178,49 @@ def split_device(rowPtr, colInd, val, cols, sel, descColId, descRowId, stream=No
     return out
 
 
+def tiles_device(ddRowPtr, ddColInd, ddVal, dCols, stream=None):
+    """The tile arrays of A_dd (device tensors as split_device() returns them), built on the device;
+    returned as a dict of device tensors (copies; the library's block is released before returning)."""
+    import torch
+    dt = MX_F64 if ddVal.dtype == torch.float64 else MX_F16
+    t = _lib.DeviceTiles()
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    lib = _lib.load()
+    check(lib.mx_tiles_device(dt, ddRowPtr.numel() - 1, dCols, ddColInd.numel(), ddRowPtr.data_ptr(), ddColInd.data_ptr(),
+                              ddVal.data_ptr(), C.byref(t), s))
+    try:
+        def take(ptr, n, dtype):
+            out = torch.empty(n, dtype=dtype, device=ddRowPtr.device)
+            if n:
+                hip = C.CDLL("libamdhip64.so")
+                hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+                if hip.hipMemcpy(out.data_ptr(), ptr, n * out.element_size(), 3) != 0:  # device to device
+                    raise MxError("hipMemcpy failed")
+            return out
+        bit_t = torch.int32 if dt == MX_F64 else torch.int64
+        return {"chunkNum": t.chunkNum, "totalTcFrags": t.totalTcFrags, "fragK": t.fragK, "tcValCount": t.tcValCount,
+                "chunkPtr": take(t.chunkPtr, t.chunkNum + 1, torch.int32),
+                "sparse_AToX_index": take(t.sparse_AToX_index, t.totalTcFrags * t.fragK, torch.int32),
+                "fragPtr": take(t.fragPtr, t.totalTcFrags + 1, torch.int32),
+                "fragBit": take(t.fragBit, t.totalTcFrags, bit_t),
+                "tcVal": take(t.tcVal, t.tcValCount, ddVal.dtype)}
+    finally:
+        lib.mx_tiles_device_free(C.byref(t))
+
+
 class Partition:
     """Result of the cascaded extraction (column pass tau_c, then row pass tau_r)."""
 
     ARRAYS = ("descColId", "newArray", "rId", "newArray_", "ddRowPtr", "ddColInd", "ddVal", "chunkPtr",
               "sparse_AToX_index", "fragPtr", "fragBit", "tcVal", "cdRowPtr", "cdColInd", "cdVal")
 
-    def __init__(self, A, tau_c, tau_r):
+    def __init__(self, A, tau_c, tau_r, device=False):
+        """device=True: the extraction runs on the GPU (mx_partition_create_device); same result."""
         self._h = C.c_void_p()
         self._A = A  # keep the input arrays alive during the call
         st = A.struct()
-        check(_lib.load().mx_partition_create(C.byref(st), float(tau_c), float(tau_r), C.byref(self._h)))
+        create = _lib.load().mx_partition_create_device if device else _lib.load().mx_partition_create
+        check(create(C.byref(st), float(tau_c), float(tau_r), C.byref(self._h)))
         self._bind()
 
     @classmethod

@@ -9,7 +9,8 @@
 // (default 200 / 4000), --no-tiles / --all-tiles (plan flags), --json (one JSON record on the
 // last line), --tune (pick the two fractions from the 5x5 grid by timing each on the device,
 // then run with them), --partition-cache FILE (read the partition from FILE when it was made for a
-// matrix of this shape with these fractions, otherwise compute it and write FILE).  Precision is the build's: -Dfp64 -> FP64 binary, otherwise FP16.
+// matrix of this shape with these fractions, otherwise compute it and write FILE), --device-prep (the extraction runs on the GPU instead of the
+// host cores; same partition).  Precision is the build's: -Dfp64 -> FP64 binary, otherwise FP16.
 //
 // Lines other tools parse (ML/bayes_opt.py:64, script/duse.sh:35-38) keep their form:
 //   cols_ratio = %f / TC_nnz_ratio = %lf / MatXtract time = %lf ms / Success! ... |
@@ -93,7 +94,7 @@ int main(int argc, char **argv)
     int config = 0, warm = 200, iters = 4000, planFlags = MX_PLAN_DEFAULT;
     double scale = 1.0;
     unsigned long long seed = 0;
-    bool keepValues = false, json = false, tune = false;
+    bool keepValues = false, json = false, tune = false, devicePrep = false;
     std::string cachePath;
     for (int i = 1; i < argc; ++i) {
         std::string a = argv[i];
@@ -116,6 +117,7 @@ int main(int argc, char **argv)
         else if (a == "--json") json = true;
         else if (a == "--partition-cache") cachePath = next("--partition-cache");
         else if (a == "--tune") tune = true;
+        else if (a == "--device-prep") devicePrep = true;
         else pos.push_back(a);
     }
     const size_t npos = pos.size() + (config ? 1 : 0);  // a --config stands for the file name
@@ -214,7 +216,7 @@ int main(int argc, char **argv)
             part = nullptr;
         }
     }
-    if (!part) part = matxtract_preprocess(csrVal, csrRowPtr, csrColInd, rowA, colA, nnzA, colProp, rowProp);
+    if (!part) part = matxtract_preprocess(csrVal, csrRowPtr, csrColInd, rowA, colA, nnzA, colProp, rowProp, devicePrep);
     auto t1 = std::chrono::steady_clock::now();
     if (!part) return 1;
     if (!cachePath.empty()) {

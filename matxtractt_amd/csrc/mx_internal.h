@@ -62,3 +62,9 @@ struct mx_partition {
     std::vector<int> cdRowPtr, cdColInd;
     mx::ValBuf cdVal;
 };
+
+namespace mx {
+// The argument checks of mx_partition_create (null pointers, shape, tau range and order, rowPtr
+// monotone over [0, nnz], column range); *out is cleared.
+int check_partition_args(const mx_csr *A, float tau_c, float tau_r, mx_partition **out);
+}  // namespace mx

@@ -305,7 +305,8 @@ uint64_t fnv(const void *p, size_t n, uint64_t h)
 
 }  // namespace
 
-extern "C" int mx_partition_create(const mx_csr *A, float tau_c, float tau_r, mx_partition **out)
+// The argument checks of mx_partition_create, shared with the device route.
+int mx::check_partition_args(const mx_csr *A, float tau_c, float tau_r, mx_partition **out)
 {
     if (!A || !out) {
         set_error("mx_partition_create: null argument");
@@ -342,6 +343,13 @@ extern "C" int mx_partition_create(const mx_csr *A, float tau_c, float tau_r, mx
             set_error("mx_partition_create: column index out of range");
             return MX_ERR_ARG;
         }
+    return MX_OK;
+}
+
+extern "C" int mx_partition_create(const mx_csr *A, float tau_c, float tau_r, mx_partition **out)
+{
+    const int ok = mx::check_partition_args(A, tau_c, tau_r, out);
+    if (ok != MX_OK) return ok;
     mx_partition *P = new (std::nothrow) mx_partition();
     if (!P) {
         set_error("mx_partition_create: out of memory");

@@ -22,6 +22,7 @@
 #include <cstdint>
 #include <cstring>
 #include <string>
+#include <vector>
 
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_scan.hpp>
@@ -215,6 +216,94 @@ __global__ __launch_bounds__(kBlock) void split_gather_kernel(const unsigned lon
         cdInd[k - nDD] = nc;
         cdVal[k - nDD] = v;
     }
+}
+
+// ---- tile encoding ------------------------------------------------------------------------
+// key = [chunk of the entry's row][column] for every entry of A_dd; payload = the entry
+__global__ __launch_bounds__(kBlock) void tile_keys_kernel(const int *__restrict__ ddRowPtr, const int *__restrict__ ddCol,
+                                                           int dRows, int n, int colBits, unsigned long long *__restrict__ key,
+                                                           int *__restrict__ payload)
+{
+    const int e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= n) return;
+    const int w = line_of(ddRowPtr, dRows, e) / mx::kFragM;
+    key[e] = ((unsigned long long)w << colBits) | (unsigned long long)ddCol[e];
+    payload[e] = e;
+}
+
+// head[k] = 1 where sorted position k holds the first occurrence of its (chunk, column)
+__global__ __launch_bounds__(kBlock) void tile_heads_kernel(const unsigned long long *__restrict__ key, int n, int *__restrict__ head)
+{
+    const int k = blockIdx.x * kBlock + threadIdx.x;
+    if (k < n) head[k] = k == 0 || key[k] != key[k - 1];
+}
+
+// frags[w] = ceil(distinct columns of chunk w / fragK); one more element, zero.  The entries of
+// chunk w sit at sorted positions [a, b) = ddRowPtr[8w] .. ddRowPtr[min(8w + 8, dRows)], and `run`
+// is the inclusive running count of the heads.
+__global__ __launch_bounds__(kBlock) void tile_chunk_frags_kernel(const int *__restrict__ ddRowPtr, const int *__restrict__ run,
+                                                                  int dRows, int chunkNum, int fragK, int *__restrict__ frags)
+{
+    const int w = blockIdx.x * kBlock + threadIdx.x;
+    if (w > chunkNum) return;
+    int f = 0;
+    if (w < chunkNum) {
+        const int a = ddRowPtr[w * mx::kFragM], b = ddRowPtr[min(w * mx::kFragM + mx::kFragM, dRows)];
+        if (b > a) f = (run[b - 1] - run[a] + 1 + fragK - 1) / fragK;
+    }
+    frags[w] = f;
+}
+
+// Per sorted position: the rank of its column inside its chunk (ecr) goes back to the entry; a
+// head also writes its column into the chunk's list; every entry sets its bit.
+__global__ __launch_bounds__(kBlock) void tile_rank_kernel(const unsigned long long *__restrict__ key, const int *__restrict__ payload,
+                                                           const int *__restrict__ head, const int *__restrict__ run,
+                                                           const int *__restrict__ ddRowPtr, const int *__restrict__ chunkPtr, int dRows,
+                                                           int n, int colBits, int fragK, int *__restrict__ ecr, int *__restrict__ atox,
+                                                           unsigned long long *__restrict__ bits)
+{
+    const int k = blockIdx.x * kBlock + threadIdx.x;
+    if (k >= n) return;
+    const int w = (int)(key[k] >> colBits), c = (int)(key[k] & ((1ull << colBits) - 1));
+    const int rank = run[k] - run[ddRowPtr[w * mx::kFragM]];
+    const int e = payload[k];
+    ecr[e] = rank;
+    const int f0 = chunkPtr[w];
+    if (head[k]) atox[(size_t)f0 * fragK + rank] = c;
+    const int r = line_of(ddRowPtr, dRows, e) - w * mx::kFragM;
+    atomicOr(&bits[f0 + rank / fragK], 1ull << (r * fragK + rank % fragK));
+}
+
+// count[f] = set bits of fragment f; one more element, zero
+__global__ __launch_bounds__(kBlock) void tile_popcount_kernel(const unsigned long long *__restrict__ bits, int nf, int *__restrict__ count)
+{
+    const int f = blockIdx.x * kBlock + threadIdx.x;
+    if (f <= nf) count[f] = f < nf ? __popcll(bits[f]) : 0;
+}
+
+// Values of a fragment in ascending bit order: an entry's place is the number of set bits below
+// its own.  Of entries that name the same row and column (neighbours in the sorted row) the last
+// one is kept.
+template <typename V>
+__global__ __launch_bounds__(kBlock) void tile_values_kernel(const int *__restrict__ ddRowPtr, const int *__restrict__ ddCol,
+                                                             const V *__restrict__ ddVal, const int *__restrict__ ecr,
+                                                             const int *__restrict__ chunkPtr, const int *__restrict__ fragPtr,
+                                                             const unsigned long long *__restrict__ bits, int dRows, int n, int fragK,
+                                                             V *__restrict__ tcVal)
+{
+    const int e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= n) return;
+    const int i = line_of(ddRowPtr, dRows, e);
+    if (e + 1 < ddRowPtr[i + 1] && ddCol[e + 1] == ddCol[e]) return;  // a later twin wins
+    const int w = i / mx::kFragM, rank = ecr[e], f = chunkPtr[w] + rank / fragK;
+    const int bit = (i - w * mx::kFragM) * fragK + rank % fragK;
+    tcVal[fragPtr[f] + __popcll(bits[f] & ((1ull << bit) - 1))] = ddVal[e];
+}
+
+__global__ __launch_bounds__(kBlock) void narrow_bits_kernel(const unsigned long long *__restrict__ bits, int nf, unsigned *__restrict__ out)
+{
+    const int f = blockIdx.x * kBlock + threadIdx.x;
+    if (f < nf) out[f] = (unsigned)bits[f];
 }
 
 struct Scratch {
@@ -507,5 +596,300 @@ extern "C" int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, cons
         mx::set_error("mx_split_device: the selection does not belong to this matrix (entry totals differ)");
         return MX_ERR_ARG;
     }
+    return MX_OK;
+}
+
+#undef MXP_TRY
+#define MXP_TRY(call)                                                                                   \
+    do {                                                                                                \
+        hipError_t e_ = (call);                                                                         \
+        if (e_ != hipSuccess) {                                                                         \
+            mx::set_error(std::string("mx_tiles_device: ") + #call + ": " + hipGetErrorString(e_));    \
+            return e_ == hipErrorOutOfMemory ? MX_ERR_ALLOC : MX_ERR_DEVICE;                            \
+        }                                                                                               \
+    } while (0)
+
+extern "C" void mx_tiles_device_free(mx_device_tiles *t)
+{
+    if (!t) return;
+    if (t->base) (void)hipFree(t->base);
+    *t = mx_device_tiles{};
+}
+
+extern "C" int mx_tiles_device(mx_dtype dtype, int dRows, int dCols, int nnzRowD, const int *ddRowPtr_dev,
+                               const int *ddColInd_dev, const void *ddVal_dev, mx_device_tiles *out, void *stream)
+{
+    using namespace mxp;
+    if ((dtype != MX_F64 && dtype != MX_F16) || dRows < 0 || dCols < 0 || nnzRowD < 0 || !out || !ddRowPtr_dev ||
+        (nnzRowD > 0 && (!ddColInd_dev || !ddVal_dev || dRows == 0 || dCols == 0))) {
+        mx::set_error("mx_tiles_device: bad argument");
+        return MX_ERR_ARG;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    *out = mx_device_tiles{};
+    const int fragK = mx::frag_k(dtype), n = nnzRowD, chunkNum = (dRows + mx::kFragM - 1) / mx::kFragM;
+    const size_t es = (size_t)mx::elem_size(dtype);
+    int colBits = 1, chunkBits = 1;
+    while (colBits < 31 && (1ll << colBits) < (long long)dCols) ++colBits;
+    while (chunkBits < 31 && (1ll << chunkBits) < (long long)chunkNum) ++chunkBits;
+    const unsigned keyBits = (unsigned)(colBits + chunkBits);
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    auto grid = [](long long m) { return dim3((unsigned)((m + kBlock - 1) / kBlock)); };
+    size_t sortBytes = 0, scanBytes = 0;
+    if (n > 0)
+        MXP_TRY(rocprim::radix_sort_pairs(nullptr, sortBytes, (const unsigned long long *)nullptr, (unsigned long long *)nullptr,
+                                          (const int *)nullptr, (int *)nullptr, (size_t)n, 0u, keyBits, s));
+    MXP_TRY(rocprim::inclusive_scan(nullptr, scanBytes, (const int *)nullptr, (int *)nullptr,
+                                    (size_t)std::max(n, chunkNum) + 1, rocprim::plus<int>(), s));
+    {   // the exclusive form may ask for a different amount: take the larger
+        size_t b2 = 0;
+        MXP_TRY(rocprim::exclusive_scan(nullptr, b2, (const int *)nullptr, (int *)nullptr, 0, (size_t)std::max(n, chunkNum) + 1,
+                                        rocprim::plus<int>(), s));
+        scanBytes = std::max(scanBytes, b2);
+    }
+    sortBytes = al(sortBytes);
+    scanBytes = al(scanBytes);
+    // scratch: keys and payloads in and out, heads, their running count, ecr, per-chunk fragments
+    const size_t keyB = al((size_t)n * 8), intB = al(((size_t)n + 1) * 4), chB = al(((size_t)chunkNum + 1) * 4);
+    Scratch scratch;
+    MXP_TRY(hipMalloc(&scratch.p, 2 * keyB + 5 * intB + 2 * chB + sortBytes + scanBytes + 256));
+    unsigned char *b = (unsigned char *)scratch.p;
+    unsigned long long *keyIn = (unsigned long long *)b, *keyOut = (unsigned long long *)(b + keyB);
+    b += 2 * keyB;
+    int *payIn = (int *)b, *payOut = (int *)(b + intB), *head = (int *)(b + 2 * intB), *run = (int *)(b + 3 * intB),
+        *ecr = (int *)(b + 4 * intB);
+    b += 5 * intB;
+    int *frags = (int *)b, *chunkPtrTmp = (int *)(b + chB);
+    b += 2 * chB;
+    void *sortTmp = b, *scanTmp = b + sortBytes;
+
+    // distinct columns per chunk: sort by (chunk, column), mark first occurrences, count them
+    if (n > 0) {
+        hipLaunchKernelGGL(tile_keys_kernel, grid(n), dim3(kBlock), 0, s, ddRowPtr_dev, ddColInd_dev, dRows, n, colBits, keyIn, payIn);
+        MXP_TRY(hipGetLastError());
+        MXP_TRY(rocprim::radix_sort_pairs(sortTmp, sortBytes, (const unsigned long long *)keyIn, keyOut, (const int *)payIn, payOut,
+                                          (size_t)n, 0u, keyBits, s));
+        hipLaunchKernelGGL(tile_heads_kernel, grid(n), dim3(kBlock), 0, s, (const unsigned long long *)keyOut, n, head);
+        MXP_TRY(hipGetLastError());
+        MXP_TRY(rocprim::inclusive_scan(scanTmp, scanBytes, (const int *)head, run, (size_t)n, rocprim::plus<int>(), s));
+    }
+    hipLaunchKernelGGL(tile_chunk_frags_kernel, grid((long long)chunkNum + 1), dim3(kBlock), 0, s, ddRowPtr_dev, (const int *)run,
+                       dRows, chunkNum, fragK, frags);
+    MXP_TRY(hipGetLastError());
+    // chunkPtr lives in the output block, whose size needs the total first
+    MXP_TRY(rocprim::exclusive_scan(scanTmp, scanBytes, (const int *)frags, chunkPtrTmp, 0, (size_t)chunkNum + 1, rocprim::plus<int>(), s));
+    int totalTcFrags = 0;
+    MXP_TRY(hipMemcpyAsync(&totalTcFrags, chunkPtrTmp + chunkNum, sizeof(int), hipMemcpyDeviceToHost, s));
+    MXP_TRY(hipStreamSynchronize(s));
+
+    // output block: chunkPtr, sparse_AToX_index, fragPtr, fragBit (64-bit while it is built), tcVal (at most n)
+    const size_t cpB = al(((size_t)chunkNum + 1) * 4), axB = al((size_t)totalTcFrags * fragK * 4 + 4),
+                 fpB = al(((size_t)totalTcFrags + 1) * 4), fbB = al((size_t)totalTcFrags * 8 + 8), tvB = al((size_t)n * es + 8);
+    Scratch outBlock;
+    MXP_TRY(hipMalloc(&outBlock.p, cpB + axB + fpB + fbB + tvB));
+    unsigned char *o = (unsigned char *)outBlock.p;
+    int *chunkPtr = (int *)o, *atox = (int *)(o + cpB), *fragPtr = (int *)(o + cpB + axB);
+    unsigned long long *bits = (unsigned long long *)(o + cpB + axB + fpB);
+    void *tcVal = o + cpB + axB + fpB + fbB;
+    MXP_TRY(hipMemcpyAsync(chunkPtr, chunkPtrTmp, ((size_t)chunkNum + 1) * 4, hipMemcpyDeviceToDevice, s));
+    MXP_TRY(hipMemsetAsync(atox, 0, axB + fpB + fbB, s));  // padding of the column lists is zero (:1380-1404)
+    if (n > 0) {
+        hipLaunchKernelGGL(tile_rank_kernel, grid(n), dim3(kBlock), 0, s, (const unsigned long long *)keyOut, (const int *)payOut,
+                           (const int *)head, (const int *)run, ddRowPtr_dev, (const int *)chunkPtr, dRows, n, colBits, fragK, ecr,
+                           atox, bits);
+        MXP_TRY(hipGetLastError());
+    }
+    // fragPtr: running count of the set bits.  head[] is free again and long enough only when
+    // totalTcFrags <= n, which holds (every fragment has an entry) -- but take no chances:
+    if (totalTcFrags > n) {
+        mx::set_error("mx_tiles_device: more fragments than entries (ddRowPtr is not A_dd's)");
+        return MX_ERR_ARG;
+    }
+    hipLaunchKernelGGL(tile_popcount_kernel, grid((long long)totalTcFrags + 1), dim3(kBlock), 0, s, (const unsigned long long *)bits,
+                       totalTcFrags, head);
+    MXP_TRY(hipGetLastError());
+    MXP_TRY(rocprim::exclusive_scan(scanTmp, scanBytes, (const int *)head, fragPtr, 0, (size_t)totalTcFrags + 1, rocprim::plus<int>(), s));
+    if (n > 0) {
+        if (dtype == MX_F64)
+            hipLaunchKernelGGL(tile_values_kernel<double>, grid(n), dim3(kBlock), 0, s, ddRowPtr_dev, ddColInd_dev,
+                               (const double *)ddVal_dev, (const int *)ecr, (const int *)chunkPtr, (const int *)fragPtr,
+                               (const unsigned long long *)bits, dRows, n, fragK, (double *)tcVal);
+        else
+            hipLaunchKernelGGL(tile_values_kernel<uint16_t>, grid(n), dim3(kBlock), 0, s, ddRowPtr_dev, ddColInd_dev,
+                               (const uint16_t *)ddVal_dev, (const int *)ecr, (const int *)chunkPtr, (const int *)fragPtr,
+                               (const unsigned long long *)bits, dRows, n, fragK, (uint16_t *)tcVal);
+        MXP_TRY(hipGetLastError());
+    }
+    if (dtype == MX_F64 && totalTcFrags > 0) {  // 8 x 4 bits: the reference keeps them in 32-bit words
+        // narrowed in place, front to back: word f of the narrow form lies below word f of the wide one,
+        // but another thread may still need it -- go through the free scratch instead
+        hipLaunchKernelGGL(narrow_bits_kernel, grid(totalTcFrags), dim3(kBlock), 0, s, (const unsigned long long *)bits, totalTcFrags,
+                           (unsigned *)run);
+        MXP_TRY(hipGetLastError());
+        MXP_TRY(hipMemcpyAsync(bits, run, (size_t)totalTcFrags * 4, hipMemcpyDeviceToDevice, s));
+    }
+    int tcValCount = 0;
+    MXP_TRY(hipMemcpyAsync(&tcValCount, fragPtr + totalTcFrags, sizeof(int), hipMemcpyDeviceToHost, s));
+    MXP_TRY(hipStreamSynchronize(s));
+    out->chunkNum = chunkNum;
+    out->totalTcFrags = totalTcFrags;
+    out->fragK = fragK;
+    out->tcValCount = tcValCount;
+    out->chunkPtr = chunkPtr;
+    out->sparse_AToX_index = atox;
+    out->fragPtr = fragPtr;
+    out->fragBit = bits;
+    out->tcVal = tcVal;
+    out->base = outBlock.p;
+    outBlock.p = nullptr;  // the caller's now
+    return MX_OK;
+}
+
+#undef MXP_TRY
+#define MXP_TRY(call)                                                                                            \
+    do {                                                                                                         \
+        hipError_t e_ = (call);                                                                                  \
+        if (e_ != hipSuccess) {                                                                                  \
+            mx::set_error(std::string("mx_partition_create_device: ") + #call + ": " + hipGetErrorString(e_));  \
+            return e_ == hipErrorOutOfMemory ? MX_ERR_ALLOC : MX_ERR_DEVICE;                                     \
+        }                                                                                                        \
+    } while (0)
+
+// mx_partition_create with the extraction done on the device: the matrix is uploaded, selected,
+// split and encoded there (mx_select_device, mx_split_device, mx_tiles_device) and the arrays come
+// back into the same host structure, so that everything downstream (plans, files, the checksum)
+// cannot tell the two routes apart.
+extern "C" int mx_partition_create_device(const mx_csr *A, float tau_c, float tau_r, mx_partition **out)
+{
+    using namespace mxp;
+    const int ok = mx::check_partition_args(A, tau_c, tau_r, out);
+    if (ok != MX_OK) return ok;
+    if (tau_c == 0.0f && tau_r == 0.0f) return mx_partition_create(A, tau_c, tau_r, out);  // nothing to extract
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) {
+        mx::set_error("mx_partition_create_device: no HIP device");
+        return MX_ERR_DEVICE;
+    }
+    const int rows = A->rows, cols = A->cols, nnz = A->nnz;
+    const size_t es = (size_t)mx::elem_size(A->dtype);
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    // the matrix and the two orders
+    const size_t rpB = al(((size_t)rows + 1) * 4), ciB = al((size_t)nnz * 4 + 4), vaB = al((size_t)nnz * es + 8),
+                 dcB = al((size_t)cols * 4 + 4), drB = al((size_t)rows * 4 + 4);
+    Scratch in;
+    MXP_TRY(hipMalloc(&in.p, rpB + ciB + vaB + dcB + drB));
+    unsigned char *b = (unsigned char *)in.p;
+    int *rp = (int *)b, *ci = (int *)(b + rpB);
+    void *va = b + rpB + ciB;
+    int *dc = (int *)(b + rpB + ciB + vaB), *dr = (int *)(b + rpB + ciB + vaB + dcB);
+    MXP_TRY(hipMemcpy(rp, A->rowPtr, ((size_t)rows + 1) * 4, hipMemcpyHostToDevice));
+    if (nnz > 0) {
+        MXP_TRY(hipMemcpy(ci, A->colInd, (size_t)nnz * 4, hipMemcpyHostToDevice));
+        MXP_TRY(hipMemcpy(va, A->val, (size_t)nnz * es, hipMemcpyHostToDevice));
+    }
+    mx_selection sel{};
+    int rc = mx_select_device(rows, cols, nnz, rp, ci, tau_c, tau_r, dc, dr, &sel, nullptr);
+    if (rc != MX_OK) return rc;
+    const int nDD = sel.nnzRowD, nCD = nnz - nDD;
+    const size_t ddpB = al(((size_t)sel.dRows + 1) * 4), ddcB = al((size_t)nDD * 4 + 4), ddvB = al((size_t)nDD * es + 8),
+                 cdpB = al(((size_t)rows + 1) * 4), cdcB = al((size_t)nCD * 4 + 4), cdvB = al((size_t)nCD * es + 8);
+    Scratch mid;
+    MXP_TRY(hipMalloc(&mid.p, ddpB + ddcB + ddvB + cdpB + cdcB + cdvB));
+    b = (unsigned char *)mid.p;
+    int *ddp = (int *)b, *ddc = (int *)(b + ddpB);
+    void *ddv = b + ddpB + ddcB;
+    int *cdp = (int *)(b + ddpB + ddcB + ddvB), *cdc = (int *)(b + ddpB + ddcB + ddvB + cdpB);
+    void *cdv = b + ddpB + ddcB + ddvB + cdpB + cdcB;
+    rc = mx_split_device(A->dtype, rows, cols, nnz, rp, ci, va, &sel, dc, dr, ddp, ddc, ddv, cdp, cdc, cdv, nullptr);
+    if (rc != MX_OK) return rc;
+    mx_device_tiles T{};
+    rc = mx_tiles_device(A->dtype, sel.dRows, sel.dCols, nDD, ddp, ddc, ddv, &T, nullptr);
+    if (rc != MX_OK) return rc;
+    struct TilesGuard {
+        mx_device_tiles *t;
+        ~TilesGuard() { mx_tiles_device_free(t); }
+    } guard{&T};
+
+    mx_partition *P = new (std::nothrow) mx_partition();
+    if (!P) {
+        mx::set_error("mx_partition_create_device: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    struct PartGuard {
+        mx_partition *p;
+        ~PartGuard() { delete p; }
+    } pg{P};
+    try {
+        P->dtype = A->dtype;
+        P->rows = rows;
+        P->cols = cols;
+        P->nnz = nnz;
+        P->fragM = mx::kFragM;
+        P->fragK = mx::frag_k(A->dtype);
+        P->tau_c = tau_c;
+        P->tau_r = tau_r;
+        P->extracted = true;
+        P->dCols = sel.dCols;
+        P->sCols = cols - sel.dCols;
+        P->nnzColD = sel.nnzColD;
+        P->nnzColS = nnz - sel.nnzColD;
+        P->cols_ratio = (float)sel.dCols / (float)cols;
+        P->dRows = sel.dRows;
+        P->sRows = rows - sel.dRows;
+        P->nnzRowD = nDD;
+        P->nnzRowS = sel.nnzColD - nDD;
+        P->nnzCD = nCD;
+        P->descColId.resize(cols);
+        P->rId.resize(sel.dRows);
+        P->ddRowPtr.resize((size_t)sel.dRows + 1);
+        P->ddColInd.resize(nDD);
+        P->ddVal.resize(nDD, (int)es);
+        P->cdRowPtr.resize((size_t)rows + 1);
+        P->cdColInd.resize(nCD);
+        P->cdVal.resize(nCD, (int)es);
+        P->chunkNum = T.chunkNum;
+        P->totalTcFrags = T.totalTcFrags;
+        P->tcValCount = T.tcValCount;
+        P->tc_nnz_ratio = (double)nDD / ((double)T.totalTcFrags * mx::kFragM * P->fragK);
+        P->chunkPtr.resize((size_t)T.chunkNum + 1);
+        P->sparse_AToX_index.resize((size_t)T.totalTcFrags * T.fragK);
+        P->fragPtr.resize((size_t)T.totalTcFrags + 1);
+        if (A->dtype == MX_F64) P->fragBit32.resize(T.totalTcFrags);
+        else P->fragBit64.resize(T.totalTcFrags);
+        P->tcVal.resize(T.tcValCount, (int)es);
+    } catch (const std::bad_alloc &) {
+        mx::set_error("mx_partition_create_device: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    auto down = [](void *dst, const void *src, size_t bytes) {
+        return bytes ? hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost) : hipSuccess;
+    };
+    MXP_TRY(down(P->descColId.data(), dc, (size_t)cols * 4));
+    MXP_TRY(down(P->rId.data(), dr, (size_t)sel.dRows * 4));
+    MXP_TRY(down(P->ddRowPtr.data(), ddp, ((size_t)sel.dRows + 1) * 4));
+    MXP_TRY(down(P->ddColInd.data(), ddc, (size_t)nDD * 4));
+    MXP_TRY(down(P->ddVal.data(), ddv, (size_t)nDD * es));
+    MXP_TRY(down(P->cdRowPtr.data(), cdp, ((size_t)rows + 1) * 4));
+    MXP_TRY(down(P->cdColInd.data(), cdc, (size_t)nCD * 4));
+    MXP_TRY(down(P->cdVal.data(), cdv, (size_t)nCD * es));
+    MXP_TRY(down(P->chunkPtr.data(), T.chunkPtr, ((size_t)T.chunkNum + 1) * 4));
+    MXP_TRY(down(P->sparse_AToX_index.data(), T.sparse_AToX_index, (size_t)T.totalTcFrags * T.fragK * 4));
+    MXP_TRY(down(P->fragPtr.data(), T.fragPtr, ((size_t)T.totalTcFrags + 1) * 4));
+    if (A->dtype == MX_F64) MXP_TRY(down(P->fragBit32.data(), T.fragBit, (size_t)T.totalTcFrags * 4));
+    else MXP_TRY(down(P->fragBit64.data(), T.fragBit, (size_t)T.totalTcFrags * 8));
+    MXP_TRY(down(P->tcVal.data(), T.tcVal, (size_t)T.tcValCount * es));
+    // the lists of what was not selected, ascending (test/test_autotc_spmv.cpp:1143-1160, :1261-1277)
+    std::vector<unsigned char> taken((size_t)std::max(rows, cols), 0);
+    for (int i = 0; i < sel.dCols; ++i) taken[P->descColId[i]] = 1;
+    P->newArray.reserve(P->sCols);
+    for (int c = 0; c < cols; ++c)
+        if (!taken[c]) P->newArray.push_back(c);
+    std::fill(taken.begin(), taken.end(), 0);
+    for (int i = 0; i < sel.dRows; ++i) taken[P->rId[i]] = 1;
+    P->newArray_.reserve(P->sRows);
+    for (int r = 0; r < rows; ++r)
+        if (!taken[r]) P->newArray_.push_back(r);
+    pg.p = nullptr;
+    *out = P;
     return MX_OK;
 }

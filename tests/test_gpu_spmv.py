@@ -765,6 +765,16 @@ def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
         assert re.search(r"MatXtract GFLOPS= \d+\.\d\d", out.stdout)
         if len(args) == 3:
             assert re.search(r"cols_ratio = \d\.\d+", out.stdout) and re.search(r"TC_nnz_ratio = \d\.\d+", out.stdout)
+    # --device-prep: the extraction on the GPU gives the same partition (checksum in the JSON record)
+    import json
+    hashes = []
+    for extra in ([], ["--device-prep"]):
+        out = subprocess.run([exe, "--warm", "2", "--iters", "5", "--json", *extra, "0.5", "0.25", str(p)],
+                             capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        assert "Success! All values match" in out.stdout
+        hashes.append(json.loads(out.stdout.strip().splitlines()[-1])["partition_hash"])
+    assert hashes[0] == hashes[1]
     # --partition-cache: written by the first run, read by the second, recomputed when the fractions change
     cache = str(tmp_path / "m_preprocessed.dat")
     seen = []
@@ -867,6 +877,13 @@ def test_device_selection_and_split_equal_the_host_partition(mx, ora):
             for g, name in zip(got, ("ddRowPtr", "ddColInd", "ddVal", "cdRowPtr", "cdColInd", "cdVal")):
                 want = getattr(P, name)
                 assert np.array_equal(g.cpu().numpy().view(np.uint8), np.ascontiguousarray(want).view(np.uint8)), (tau, name)
+            # and the tile encoding of that A_dd
+            T = mx.tiles_device(got[0], got[1], got[2], sel["dCols"])
+            assert (T["chunkNum"], T["totalTcFrags"], T["fragK"], T["tcValCount"]) == \
+                (P.chunkNum, P.totalTcFrags, P.fragK, P.tcValCount), (tau, T)
+            for name in ("chunkPtr", "sparse_AToX_index", "fragPtr", "fragBit", "tcVal"):
+                assert np.array_equal(T[name].cpu().numpy().view(np.uint8),
+                                      np.ascontiguousarray(getattr(P, name)).view(np.uint8)), (tau, name)
             if A.rows <= 70000:
                 O = ora.partition(A.rowPtr, A.colInd, A.val, A.cols, *tau)
                 assert np.array_equal(dc.cpu().numpy(), O.descColId) and np.array_equal(dr.cpu().numpy()[:P.dRows], O.rId)
@@ -874,3 +891,52 @@ def test_device_selection_and_split_equal_the_host_partition(mx, ora):
             P.close()
     with pytest.raises(mx.MxError):  # tau_c < tau_r
         mx.select_device(rp, ci, A.cols, 0.25, 0.5)
+
+
+@pytest.mark.gpu
+def test_partition_by_the_device_route_is_the_same_partition(mx, ora):
+    """mx_partition_create_device: every scalar, every array and the checksum of the partition
+    built on the GPU equal the host-built one (and with it the oracle's and the golden vectors',
+    which the host route is held to) -- five workloads at reduced size over a tau grid, the golden
+    matrices, workload 5 at full size -- and a plan made from it multiplies like any other."""
+    import glob
+    import json
+    import torch
+    import os
+    SCALARS = ("dCols", "sCols", "nnzColD", "nnzColS", "dRows", "sRows", "nnzRowD", "nnzRowS", "chunkNum", "totalTcFrags",
+               "tcValCount", "nnzCD", "fragM", "fragK", "cols_ratio", "tc_nnz_ratio")
+    INT_ARRAYS = ("ddRowPtr", "ddColInd", "chunkPtr", "sparse_AToX_index", "fragPtr", "fragBit", "cdRowPtr", "cdColInd")
+    VAL_ARRAYS = ("ddVal", "tcVal", "cdVal")
+
+    def same(A, tau):
+        H, D = mx.Partition(A, *tau), mx.Partition(A, *tau, device=True)
+        for name in SCALARS:
+            a, b = getattr(H, name), getattr(D, name)
+            assert a == b or (a != a and b != b), (tau, name, a, b)
+        for name in INT_ARRAYS + VAL_ARRAYS + ("descColId", "newArray", "newArray_", "rId"):
+            a, b = np.ascontiguousarray(getattr(H, name)), np.ascontiguousarray(getattr(D, name))
+            assert a.dtype == b.dtype and np.array_equal(a.view(np.uint8), b.view(np.uint8)), (tau, name)
+        assert H.hash == D.hash
+        H.close()
+        return D
+
+    for cfg, scale in [(1, 0.5), (2, 1 / 16), (3, 0.008), (4, 1 / 64), (5, 1 / 256)]:
+        A, x = mx.gen_config(cfg, scale=scale)
+        for tau in [(0.0, 0.0), (0.25, 0.0), (0.5, 0.25), (0.75, 0.75), (1.0, 0.5), (1.0, 1.0)]:
+            same(A, tau).close()
+    for path in sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "partition_*.json"))):
+        fx = json.load(open(path))
+        if not {"rowPtr", "colInd", "val", "cols"} <= set(fx):
+            continue
+        for dtype in (np.float64, np.float16):
+            A = mx.Csr(len(fx["rowPtr"]) - 1, fx["cols"], np.array(fx["rowPtr"], np.int32), np.array(fx["colInd"], np.int32),
+                       np.array(fx["val"], dtype))
+            same(A, (fx["tau_c"], fx["tau_r"])).close()
+    A, x = mx.gen_config(5)
+    D = same(A, (1.0, 1.0))
+    plan = mx.Plan(D)
+    y = plan.spmv(torch.from_numpy(x).cuda())
+    torch.cuda.synchronize()
+    assert rel_l2(y.cpu().numpy().astype(np.float64), oracle_y(ora, mx, A, x)) <= F16_TOL
+    plan.close()
+    D.close()
