@@ -138,9 +138,22 @@ __global__ __launch_bounds__(kBlock) void dense_row_counts_kernel(const int *__r
                                                                   const unsigned char *__restrict__ dense, int rows, int nnz,
                                                                   int *__restrict__ rcnt)
 {
+    // The lanes of a wave hold consecutive entries, so their rows ascend: the first lane of every run
+    // of equal rows adds the run's count in one atomic (a row of thousands of entries would otherwise
+    // take thousands of atomics on one address).
     const int e = blockIdx.x * kBlock + threadIdx.x;
-    if (e >= nnz) return;
-    if (dense[col[e]]) atomicAdd(&rcnt[line_of(rowPtr, rows, e)], 1);
+    const bool in = e < nnz;
+    const int r = in ? line_of(rowPtr, rows, e) : -1;
+    const bool d = in && dense[col[e]];
+    const int lane = threadIdx.x & 63;
+    const int rPrev = __shfl_up(r, 1);
+    const unsigned long long heads = __ballot(lane == 0 || r != rPrev), hits = __ballot(d);
+    if (!in || !((heads >> lane) & 1)) return;
+    const unsigned long long above = lane == 63 ? 0ull : heads >> (lane + 1);
+    const int next = above ? lane + 1 + __builtin_ctzll(above) : 64;
+    const unsigned long long run = (next == 64 ? ~0ull : (1ull << next) - 1) & ~((1ull << lane) - 1);
+    const int c = __popcll(hits & run);
+    if (c) atomicAdd(&rcnt[r], c);
 }
 
 // ---- split --------------------------------------------------------------------------------
@@ -262,16 +275,30 @@ __global__ __launch_bounds__(kBlock) void tile_rank_kernel(const unsigned long l
                                                            int n, int colBits, int fragK, int *__restrict__ ecr, int *__restrict__ atox,
                                                            unsigned long long *__restrict__ bits)
 {
-    const int k = blockIdx.x * kBlock + threadIdx.x;
-    if (k >= n) return;
-    const int w = (int)(key[k] >> colBits), c = (int)(key[k] & ((1ull << colBits) - 1));
-    const int rank = run[k] - run[ddRowPtr[w * mx::kFragM]];
-    const int e = payload[k];
-    ecr[e] = rank;
-    const int f0 = chunkPtr[w];
-    if (head[k]) atox[(size_t)f0 * fragK + rank] = c;
-    const int r = line_of(ddRowPtr, dRows, e) - w * mx::kFragM;
-    atomicOr(&bits[f0 + rank / fragK], 1ull << (r * fragK + rank % fragK));
+    const int k = blockIdx.x * kBlock + threadIdx.x, lane = threadIdx.x & 63;
+    int f = -1;
+    unsigned long long v = 0;
+    if (k < n) {
+        const int w = (int)(key[k] >> colBits), c = (int)(key[k] & ((1ull << colBits) - 1));
+        const int rank = run[k] - run[ddRowPtr[w * mx::kFragM]];
+        const int e = payload[k];
+        ecr[e] = rank;
+        const int f0 = chunkPtr[w];
+        if (head[k]) atox[(size_t)f0 * fragK + rank] = c;
+        const int r = line_of(ddRowPtr, dRows, e) - w * mx::kFragM;
+        f = f0 + rank / fragK;
+        v = 1ull << (r * fragK + rank % fragK);
+    }
+    // Sorted positions ascend by (chunk, column), so the fragments of a wave's lanes ascend too: the
+    // bits of every run of equal fragments are gathered at its first lane, which issues one atomic.
+    const int fPrev = __shfl_up(f, 1);
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long o = __shfl_down(v, off);
+        const int fo = __shfl_down(f, off);
+        if (lane + off < 64 && fo == f) v |= o;
+    }
+    if (f >= 0 && (lane == 0 || f != fPrev)) atomicOr(&bits[f], v);
 }
 
 // count[f] = set bits of fragment f; one more element, zero
