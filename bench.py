@@ -226,6 +226,20 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
         rec["cpu_all_cores"] = {"value": 2.0 * A.nnz / t_all / 1e9, "unit": "GFLOP/s", "cores": ncore, "kind": "port",
                                 "sample": "not the reference's (its CPU path is serial): the oracle routine on %d "
                                           "nnz-balanced row ranges in parallel threads, best of 5 (%.2f ms)" % (ncore, t_all * 1e3)}
+        # the extraction itself (not part of `value`): host route against the device route, same partition
+        pt = (0.5, 0.25)
+        mx.Partition(A, *pt, device=True).close()  # first use of the device code
+        t0 = time.perf_counter()
+        ph = mx.Partition(A, *pt)
+        t1 = time.perf_counter()
+        pd = mx.Partition(A, *pt, device=True)
+        t2 = time.perf_counter()
+        rec["preprocess"] = {"tau_c": pt[0], "tau_r": pt[1], "host_ms": (t1 - t0) * 1e3, "device_route_ms": (t2 - t1) * 1e3,
+                             "same_partition": ph.hash == pd.hash,
+                             "note": "mx_partition_create on the host cores against mx_partition_create_device "
+                                     "(upload, extraction on the GPU, download)"}
+        ph.close()
+        pd.close()
     plan.close()
     part.close()
     return rec
@@ -270,6 +284,7 @@ def main():
         "roofline": main_rec["roofline"],
         "cpu_baseline": main_rec.pop("cpu_baseline"),
         "cpu_all_cores": main_rec.pop("cpu_all_cores"),
+        "preprocess": main_rec.pop("preprocess"),
         "hbm_frac_whole_spmv": main_rec["hbm_frac_whole_spmv"],
         "cold_cache": main_rec["cold_cache"],
         "rel_l2_vs_oracle": main_rec["rel_l2_vs_oracle"],
