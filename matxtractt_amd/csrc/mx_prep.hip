@@ -32,6 +32,8 @@
 namespace mxp {
 
 constexpr int kBlock = 256;
+// Entry numbers are formed as blockIdx.x * kBlock + threadIdx.x in 32 bits: the last block must not pass 2^31.
+constexpr int kMaxCount = 2147483647 - 2 * kBlock;
 
 // line[e] = r with ptr[r] <= e < ptr[r+1]; bad |= 1 where ind[e] lies outside [0, inner).
 __global__ __launch_bounds__(kBlock) void entry_lines_kernel(const int *__restrict__ ptr, const int *__restrict__ ind,
@@ -361,6 +363,10 @@ extern "C" int mx_transpose_device(mx_dtype dtype, int outer, int inner, int nnz
         mx::set_error("mx_transpose_device: bad argument");
         return MX_ERR_ARG;
     }
+    if (nnz > kMaxCount || inner > kMaxCount || outer > kMaxCount) {
+        mx::set_error("mx_transpose_device: more than 2^31 - 513 entries or lines");
+        return MX_ERR_ARG;
+    }
     hipStream_t s = (hipStream_t)stream;
     const int pblocks = (int)(((long long)nnz + 1 + kBlock - 1) / kBlock);
     if (nnz == 0) {
@@ -462,6 +468,10 @@ extern "C" int mx_select_device(int rows, int cols, int nnz, const int *rowPtr_d
         mx::set_error("mx_select_device: bad argument");
         return MX_ERR_ARG;
     }
+    if (nnz > kMaxCount || rows > kMaxCount || cols > kMaxCount) {
+        mx::set_error("mx_select_device: more than 2^31 - 513 entries, rows or columns");
+        return MX_ERR_ARG;
+    }
     hipStream_t s = (hipStream_t)stream;
     *out = mx_selection{0, 0, 0, 0};
     const size_t n = (size_t)std::max(rows, cols);
@@ -539,6 +549,10 @@ extern "C" int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, cons
         (nnz > 0 && (!colInd_dev || !val_dev || rows == 0 || cols == 0)) || (sel->nnzRowD > 0 && (!ddColInd_dev || !ddVal_dev)) ||
         (nnz - sel->nnzRowD > 0 && (!cdColInd_dev || !cdVal_dev))) {
         mx::set_error("mx_split_device: bad argument");
+        return MX_ERR_ARG;
+    }
+    if (nnz > kMaxCount || rows > kMaxCount || cols > kMaxCount) {
+        mx::set_error("mx_split_device: more than 2^31 - 513 entries, rows or columns");
         return MX_ERR_ARG;
     }
     hipStream_t s = (hipStream_t)stream;
@@ -650,6 +664,10 @@ extern "C" int mx_tiles_device(mx_dtype dtype, int dRows, int dCols, int nnzRowD
     if ((dtype != MX_F64 && dtype != MX_F16) || dRows < 0 || dCols < 0 || nnzRowD < 0 || !out || !ddRowPtr_dev ||
         (nnzRowD > 0 && (!ddColInd_dev || !ddVal_dev || dRows == 0 || dCols == 0))) {
         mx::set_error("mx_tiles_device: bad argument");
+        return MX_ERR_ARG;
+    }
+    if (nnzRowD > kMaxCount || dRows > kMaxCount || dCols > kMaxCount) {
+        mx::set_error("mx_tiles_device: more than 2^31 - 513 entries, rows or columns");
         return MX_ERR_ARG;
     }
     hipStream_t s = (hipStream_t)stream;

@@ -534,6 +534,15 @@ def test_device_entry_points_fail_loudly_without_a_gpu(mx):
     assert e.value.code == 3 and "no CPU fallback" in str(e.value)
     with pytest.raises(mx.MxError):
         mx.cdspmv(A, x, np.zeros(A.rows))
+    # the device route of the extraction has no host fallback either
+    with pytest.raises(mx.MxError) as e:
+        mx.Partition(A, 0.5, 0.25, device=True)
+    assert e.value.code == 3 and "no HIP device" in str(e.value)
+    with pytest.raises(mx.MxError) as e:  # arguments are checked before anything touches the device
+        mx.Partition(A, 0.25, 0.5, device=True)
+    assert e.value.code == 1
+    # tau = (0, 0) extracts nothing: handed to the host routine, device or not
+    mx.Partition(A, 0.0, 0.0, device=True).close()
 
 
 def test_product_does_not_reach_into_the_oracle():
