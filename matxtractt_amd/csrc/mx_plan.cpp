@@ -1824,7 +1824,9 @@ extern "C" int mx_tune_tau(const mx_csr *A, int levels, int flags, int warm, int
             mx_plan *plan = nullptr;
             double ms = 0.0;
             int tileNnz = 0;
-            if ((rc = mx_partition_create(A, c, r, &P))) break;
+            // the tuner needs the device anyway: large matrices are also extracted there (same partition,
+            // a fraction of the time; below about two million entries the copies cost more than they save)
+            if ((rc = (A->nnz >= (1 << 21) ? mx_partition_create_device(A, c, r, &P) : mx_partition_create(A, c, r, &P)))) break;
             // entries the plan would hand to the tile kernel
             bool anyTile = false;
             if (P->extracted && !(flags & MX_PLAN_NO_TILES)) {

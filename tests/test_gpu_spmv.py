@@ -736,6 +736,17 @@ def test_tau_tuner(mx, ora):
     P.close()
     with pytest.raises(mx.MxError):
         mx.tune_tau(A, levels=1)
+    # a matrix large enough for the tuner to extract on the device: same candidates, same tile entries
+    # as plans made from host-built partitions
+    A, x = mx.gen_config(2)
+    tc, tr, table = mx.tune_tau(A, levels=3, flags=mx.MX_PLAN_KEEP_TILES, warm=2, iters=10)
+    assert [(c, r) for c, r, _, _ in table] == [(0.0, 0.0), (0.5, 0.0), (0.5, 0.5), (1.0, 0.0), (1.0, 0.5), (1.0, 1.0)]
+    for c, r, ms, n in table:
+        P = mx.Partition(A, c, r)
+        plan = mx.Plan(P, mx.MX_PLAN_KEEP_TILES)
+        assert plan.info["tile_nnz"] == n and ms > 0, (c, r)
+        plan.close()
+        P.close()
 
 
 def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
