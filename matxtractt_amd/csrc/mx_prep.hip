@@ -345,18 +345,20 @@ struct Scratch {
 
 }  // namespace mxp
 
-#define MXP_TRY(call)                                                                                      \
-    do {                                                                                                   \
-        hipError_t e_ = (call);                                                                            \
-        if (e_ != hipSuccess) {                                                                            \
-            mx::set_error(std::string("mx_transpose_device: ") + #call + ": " + hipGetErrorString(e_));   \
-            return e_ == hipErrorOutOfMemory ? MX_ERR_ALLOC : MX_ERR_DEVICE;                                  \
-        }                                                                                                  \
+// `who` is the name of the entry point the enclosing function works for
+#define MXP_TRY(call)                                                                       \
+    do {                                                                                    \
+        hipError_t e_ = (call);                                                             \
+        if (e_ != hipSuccess) {                                                             \
+            mx::set_error(std::string(who) + ": " + #call + ": " + hipGetErrorString(e_)); \
+            return e_ == hipErrorOutOfMemory ? MX_ERR_ALLOC : MX_ERR_DEVICE;                \
+        }                                                                                   \
     } while (0)
 
 extern "C" int mx_transpose_device(mx_dtype dtype, int outer, int inner, int nnz, const int *ptr_dev, const int *ind_dev,
                                    const void *val_dev, int *tPtr_dev, int *tInd_dev, void *tVal_dev, void *stream)
 {
+    static const char who[] = "mx_transpose_device";
     using namespace mxp;
     if ((dtype != MX_F64 && dtype != MX_F16) || outer < 0 || inner < 0 || nnz < 0 || !ptr_dev || !tPtr_dev ||
         (nnz > 0 && (!ind_dev || !val_dev || !tInd_dev || !tVal_dev || outer == 0))) {
@@ -416,15 +418,6 @@ extern "C" int mx_transpose_device(mx_dtype dtype, int outer, int inner, int nnz
     return MX_OK;
 }
 
-#undef MXP_TRY
-#define MXP_TRY(call)                                                                                    \
-    do {                                                                                                 \
-        hipError_t e_ = (call);                                                                          \
-        if (e_ != hipSuccess) {                                                                          \
-            mx::set_error(std::string("mx_select_device: ") + #call + ": " + hipGetErrorString(e_));    \
-            return e_ == hipErrorOutOfMemory ? MX_ERR_ALLOC : MX_ERR_DEVICE;                             \
-        }                                                                                                \
-    } while (0)
 
 namespace mxp {
 
@@ -434,6 +427,7 @@ namespace mxp {
 static int order_and_reach(const int *cnt, int n, int target, int *order, int *work, void *sortTmp, size_t sortBytes,
                            void *scanTmp, size_t scanBytes, hipStream_t s, int *len, int *sum)
 {
+    static const char who[] = "mx_select_device";
     *len = 0;
     *sum = 0;
     if (n == 0) return MX_OK;
@@ -461,6 +455,7 @@ static int order_and_reach(const int *cnt, int n, int target, int *order, int *w
 extern "C" int mx_select_device(int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev, float tau_c,
                                 float tau_r, int *descColId_dev, int *descRowId_dev, mx_selection *out, void *stream)
 {
+    static const char who[] = "mx_select_device";
     using namespace mxp;
     if (rows < 0 || cols < 0 || nnz < 0 || !rowPtr_dev || !out || (cols > 0 && !descColId_dev) ||
         (rows > 0 && !descRowId_dev) || (nnz > 0 && (!colInd_dev || rows == 0 || cols == 0)) || !(tau_c >= 0.f) ||
@@ -527,21 +522,13 @@ extern "C" int mx_select_device(int rows, int cols, int nnz, const int *rowPtr_d
     return rc;
 }
 
-#undef MXP_TRY
-#define MXP_TRY(call)                                                                                   \
-    do {                                                                                                \
-        hipError_t e_ = (call);                                                                         \
-        if (e_ != hipSuccess) {                                                                         \
-            mx::set_error(std::string("mx_split_device: ") + #call + ": " + hipGetErrorString(e_));    \
-            return e_ == hipErrorOutOfMemory ? MX_ERR_ALLOC : MX_ERR_DEVICE;                            \
-        }                                                                                               \
-    } while (0)
 
 extern "C" int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
                                const void *val_dev, const mx_selection *sel, const int *descColId_dev,
                                const int *descRowId_dev, int *ddRowPtr_dev, int *ddColInd_dev, void *ddVal_dev,
                                int *cdRowPtr_dev, int *cdColInd_dev, void *cdVal_dev, void *stream)
 {
+    static const char who[] = "mx_split_device";
     using namespace mxp;
     if ((dtype != MX_F64 && dtype != MX_F16) || rows < 0 || cols < 0 || nnz < 0 || !sel || !rowPtr_dev || !ddRowPtr_dev ||
         !cdRowPtr_dev || sel->dCols < 0 || sel->dCols > cols || sel->dRows < 0 || sel->dRows > rows || sel->nnzRowD < 0 ||
@@ -640,15 +627,6 @@ extern "C" int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, cons
     return MX_OK;
 }
 
-#undef MXP_TRY
-#define MXP_TRY(call)                                                                                   \
-    do {                                                                                                \
-        hipError_t e_ = (call);                                                                         \
-        if (e_ != hipSuccess) {                                                                         \
-            mx::set_error(std::string("mx_tiles_device: ") + #call + ": " + hipGetErrorString(e_));    \
-            return e_ == hipErrorOutOfMemory ? MX_ERR_ALLOC : MX_ERR_DEVICE;                            \
-        }                                                                                               \
-    } while (0)
 
 extern "C" void mx_tiles_device_free(mx_device_tiles *t)
 {
@@ -660,6 +638,7 @@ extern "C" void mx_tiles_device_free(mx_device_tiles *t)
 extern "C" int mx_tiles_device(mx_dtype dtype, int dRows, int dCols, int nnzRowD, const int *ddRowPtr_dev,
                                const int *ddColInd_dev, const void *ddVal_dev, mx_device_tiles *out, void *stream)
 {
+    static const char who[] = "mx_tiles_device";
     using namespace mxp;
     if ((dtype != MX_F64 && dtype != MX_F16) || dRows < 0 || dCols < 0 || nnzRowD < 0 || !out || !ddRowPtr_dev ||
         (nnzRowD > 0 && (!ddColInd_dev || !ddVal_dev || dRows == 0 || dCols == 0))) {
@@ -790,15 +769,6 @@ extern "C" int mx_tiles_device(mx_dtype dtype, int dRows, int dCols, int nnzRowD
     return MX_OK;
 }
 
-#undef MXP_TRY
-#define MXP_TRY(call)                                                                                            \
-    do {                                                                                                         \
-        hipError_t e_ = (call);                                                                                  \
-        if (e_ != hipSuccess) {                                                                                  \
-            mx::set_error(std::string("mx_partition_create_device: ") + #call + ": " + hipGetErrorString(e_));  \
-            return e_ == hipErrorOutOfMemory ? MX_ERR_ALLOC : MX_ERR_DEVICE;                                     \
-        }                                                                                                        \
-    } while (0)
 
 // mx_partition_create with the extraction done on the device: the matrix is uploaded, selected,
 // split and encoded there (mx_select_device, mx_split_device, mx_tiles_device) and the arrays come
@@ -806,6 +776,7 @@ extern "C" int mx_tiles_device(mx_dtype dtype, int dRows, int dCols, int nnzRowD
 // cannot tell the two routes apart.
 extern "C" int mx_partition_create_device(const mx_csr *A, float tau_c, float tau_r, mx_partition **out)
 {
+    static const char who[] = "mx_partition_create_device";
     using namespace mxp;
     const int ok = mx::check_partition_args(A, tau_c, tau_r, out);
     if (ok != MX_OK) return ok;
