@@ -9,3 +9,5 @@ bool strips_can_ride(mx_dtype, const DeviceTiles &, const void *) { return false
 hipError_t launch_probe_f64(const double *, const double *, double *, hipStream_t) { return hipErrorUnknown; }
 hipError_t launch_probe_f16(const void *, const void *, float *, hipStream_t) { return hipErrorUnknown; }
 }
+// The device route of the extraction lives in a HIP source as well; the tuner names it.
+extern "C" int mx_partition_create_device(const mx_csr *, float, float, mx_partition **) { return MX_ERR_DEVICE; }
