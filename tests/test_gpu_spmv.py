@@ -909,7 +909,7 @@ def test_partition_by_the_device_route_is_the_same_partition(mx, ora):
     """mx_partition_create_device: every scalar, every array and the checksum of the partition
     built on the GPU equal the host-built one (and with it the oracle's and the golden vectors',
     which the host route is held to) -- five workloads at reduced size over a tau grid, the golden
-    matrices, workload 5 at full size -- and a plan made from it multiplies like any other."""
+    matrices, workloads 3, 4 and 5 at full size -- and a plan made from it multiplies like any other."""
     import glob
     import json
     import torch
@@ -943,6 +943,9 @@ def test_partition_by_the_device_route_is_the_same_partition(mx, ora):
             A = mx.Csr(len(fx["rowPtr"]) - 1, fx["cols"], np.array(fx["rowPtr"], np.int32), np.array(fx["colInd"], np.int32),
                        np.array(fx["val"], dtype))
             same(A, (fx["tau_c"], fx["tau_r"])).close()
+    for cfg in (3, 4):  # the other two large workloads at full size (binary64 stencil, binary16 power law)
+        A, x = mx.gen_config(cfg)
+        same(A, (0.5, 0.25)).close()
     A, x = mx.gen_config(5)
     D = same(A, (1.0, 1.0))
     plan = mx.Plan(D)
