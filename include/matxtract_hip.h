@@ -251,6 +251,22 @@ void mx_plan_destroy(mx_plan *plan);
  * buffers of partial sums: calls on the same plan must not overlap in time. */
 int mx_spmv(mx_plan *plan, const void *x_dev, void *y_dev, void *stream);
 
+/* mx_spmv for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * compute calls allocate on every call (src/spmv_kernel/cdSpMV.cu:407-418).  Same arguments,
+ * same kernels and bit-for-bit the same y as mx_spmv; the one buffer the kernels need beyond
+ * the plan's arrays, x and y -- the sums of the virtual rows that csr_slice_kernel hands to
+ * slice_combine_kernel -- lives in a fixed array of mx_static_scratch_bytes() (16 MiB) that is
+ * part of the library's code object on every GPU it runs on (held until the process ends) and
+ * is addressed through hipGetSymbolAddress once per device.  The call itself allocates
+ * nothing, frees nothing and calls no allocating routine.  A plan whose sums need more than
+ * the array holds is refused with MX_ERR_ARG and a message that says so (the mixed workload at
+ * full size: 27 MB).  Every call on one GPU shares that GPU's array: calls that overlap in time
+ * on one GPU -- also through different plans or streams -- race.  Nothing in the array has to
+ * start at zero: every sum the second kernel reads is written by the first in the same call. */
+int mx_spmv_static(mx_plan *plan, const void *x_dev, void *y_dev, void *stream);
+int mx_static_scratch_bytes(void);
+
 /* n back-to-back SpMVs y = A*x on `stream`, queued from C without returning to the caller in
  * between: the reference's timed loops (src/spmv_kernel/cdSpMV.cu:464-469) as an entry point,
  * for callers whose per-call overhead (an interpreter, an FFI hop) would otherwise sit

@@ -114,6 +114,8 @@ SIGNATURES = {
     "mx_plan_create": (_i, [_vp, _i, _pp]),
     "mx_plan_destroy": (None, [_vp]),
     "mx_spmv": (_i, [_vp, _vp, _vp, _vp]),
+    "mx_spmv_static": (_i, [_vp, _vp, _vp, _vp]),
+    "mx_static_scratch_bytes": (_i, []),
     "mx_spmv_repeat": (_i, [_vp, _vp, _vp, _i, _vp]),
     "mx_spmv_host": (_i, [_vp, _vp, _vp]),
     "mx_time": (_i, [_vp, _vp, _vp, _i, _i, _pd, _pd, _pd]),

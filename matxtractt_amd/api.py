@@ -384,6 +384,16 @@ class Plan:
         check(_lib.load().mx_spmv(self._h, x.data_ptr(), y.data_ptr(), s))
         return y
 
+    def spmv_static(self, x, y, stream=None):
+        """y = A x without any allocation: the kernels' partial sums go to the library's fixed
+        device array (mx_spmv_static).  y must be given."""
+        import torch
+        self._check_vec(x, self.cols, "x")
+        self._check_vec(y, self.rows, "y")
+        s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+        check(_lib.load().mx_spmv_static(self._h, x.data_ptr(), y.data_ptr(), s))
+        return y
+
     def spmv_repeat(self, x, y, n, stream=None):
         """n back-to-back y = A x, queued from C (no Python between launches)."""
         import torch

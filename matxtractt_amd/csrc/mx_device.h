@@ -133,6 +133,12 @@ constexpr int kSliceBatchEntries = 8;  // entries a lane loads at a time
 inline int slice_step_entries(mx_dtype) { return 1; }  // entries a lane takes per step; chunks end between steps
 constexpr int kSliceLightSegs = 8;     // rows with at most this many virtual rows are summed by one lane
 
+// The sums of the virtual rows (DeviceSlices::partial) of mx_spmv_static live in a fixed array
+// in device memory instead of the plan's own buffer: static_scratch gives the address of the
+// current device's copy (looked up once per device, no allocation).
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+hipError_t static_scratch(void **ptr);
+
 // `what`: 0 = slice kernel then combine kernel, 1 = slice kernel only, 2 = combine kernel only
 // `strips` (optional): a tile layout in the dense binary16 form whose steps workgroups of the
 // combine kernel's launch run as well (strips_can_ride says whether a layout may); the rows of

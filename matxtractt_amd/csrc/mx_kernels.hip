@@ -16,6 +16,7 @@
 #include <hip/hip_runtime.h>
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 #include "mx_device.h"
@@ -1035,6 +1036,35 @@ __global__ void probe_mfma_f16_kernel(const _Float16 *A /*[64][8]*/, const _Floa
 // ---- launchers (called from mx_plan.cpp; plain functions so that file needs no HIP syntax)
 namespace mx {
 
+constexpr int kMaxDevices = 64;
+
+// Device memory that exists without any allocation call: one array per GPU, part of the
+// library's code object, held from the moment the library is loaded on that GPU until the
+// process ends.  Host code must not use the array's name as an address (it is a host-side
+// stand-in): the device address is asked for once per device and kept.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+hipError_t static_scratch(void **ptr)
+{
+    static std::mutex lock;
+    static void *addr[kMaxDevices] = {};
+    *ptr = nullptr;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> hold(lock);
+    if (!addr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        addr[dev] = p;
+    }
+    *ptr = addr[dev];
+    return hipSuccess;
+}
+
 template <typename VT, int NPT>
 static void launch_csr_t(const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
 {
@@ -1080,15 +1110,24 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     typedef typename mxk::Acc<VT>::type AT;
     const bool dict = P.useDict && P.ecode && P.dict;
     const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)((P.maxWgChunks + 3) & ~3) * 4 + 64 + (dict ? 256 * sizeof(AT) : 0);
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT, false>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT, true>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
+    // (a function attribute belongs to the device that is current when it is set: once per device)
+    {
+        static std::mutex attrLock;
+        static bool attrSet[kMaxDevices] = {};
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
         if (e != hipSuccess) return e;
-        attr_set = true;
+        if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+        std::lock_guard<std::mutex> hold(attrLock);
+        if (!attrSet[dev]) {
+            e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT, false>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
+            if (e == hipSuccess)
+                e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT, true>,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
+            if (e != hipSuccess) return e;
+            attrSet[dev] = true;
+        }
     }
     if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16))
         return hipErrorInvalidValue;

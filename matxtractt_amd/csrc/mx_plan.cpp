@@ -1028,16 +1028,33 @@ static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
     return MX_OK;
 }
 
+// `partial` (optional): where the slice kernel puts the sums of the virtual rows, in place of the
+// plan's own buffer.
 static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate, hipStream_t s,
-                           const mx::DeviceTiles *strips = nullptr)
+                           const mx::DeviceTiles *strips = nullptr, void *partial = nullptr)
 {
     if (plan->csr_variant != 0 && ((uintptr_t)x & 15)) {
         set_error("mx_spmv: x must be 16-byte aligned for this plan");
         return MX_ERR_ARG;
     }
     if (plan->csr_variant != 1) MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s));
-    if (plan->csr_variant != 0) MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s, 0, strips));
+    if (plan->csr_variant != 0) {
+        if (partial) {
+            mx::DeviceSlices L = plan->slices;  // a view: same arrays, other sums
+            L.partial = partial;
+            MX_HIP(mx::launch_slices(plan->dtype, L, x, y, accumulate, s, 0, strips));
+        } else {
+            MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s, 0, strips));
+        }
+    }
     return MX_OK;
+}
+
+// Bytes of the sums of a plan's virtual rows (what upload_slices allocates for them).
+static size_t partial_bytes(const mx_plan *plan)
+{
+    if (plan->csr_variant == 0) return 0;
+    return ((size_t)plan->slices.chunks * 64 + 64) * (plan->dtype == MX_F64 ? 8 : 4);
 }
 
 // Row length from which a row of a split plan goes to the slice kernel (MX_SPLIT_LEN overrides).
@@ -1480,6 +1497,15 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
         set_error("mx_plan_create: could not create stream/events");
         return fail(MX_ERR_DEVICE);
     }
+    {
+        // set-up: the address of the fixed array of mx_spmv_static on this device (kept per device)
+        void *fixed = nullptr;
+        if (mx::static_scratch(&fixed) != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("mx_plan_create: hipGetSymbolAddress failed for the fixed array of sums");
+            return fail(MX_ERR_DEVICE);
+        }
+    }
     PhaseLog phase;
     try {
         if (!P->extracted) {
@@ -1666,13 +1692,13 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     return MX_OK;
 }
 
-static int spmv_on(mx_plan *plan, const void *x, void *y, hipStream_t s)
+static int spmv_on(mx_plan *plan, const void *x, void *y, hipStream_t s, void *partial = nullptr)
 {
     // the strips ride in the launch of the combine kernel when the CSR part has one (MX_STRIPS_APART=1:
     // a launch of their own, as with the row-tile form of the CSR part)
     static const bool apart = std::getenv("MX_STRIPS_APART") && std::atoi(std::getenv("MX_STRIPS_APART"));
     const bool ride = !apart && plan->csr_variant == 1 && mx::strips_can_ride(plan->dtype, plan->strips, x);
-    int rc = launch_csr_part(plan, x, y, 0, s, ride ? &plan->strips : nullptr);
+    int rc = launch_csr_part(plan, x, y, 0, s, ride ? &plan->strips : nullptr, partial);
     if (rc) return rc;
     MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x, y, 1, s));
     if (!ride) MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x, y, 1, s));
@@ -1687,6 +1713,26 @@ extern "C" int mx_spmv(mx_plan *plan, const void *x_dev, void *y_dev, void *stre
     }
     return spmv_on(plan, x_dev, y_dev, (hipStream_t)stream);
 }
+
+extern "C" int mx_spmv_static(mx_plan *plan, const void *x_dev, void *y_dev, void *stream)
+{
+    if (!plan || !x_dev || !y_dev) {
+        set_error("mx_spmv_static: null argument");
+        return MX_ERR_ARG;
+    }
+    const size_t need = partial_bytes(plan);
+    if (need > mx::kStaticScratchBytes) {
+        set_error("mx_spmv_static: the plan's virtual rows need " + std::to_string(need) +
+                  " bytes of sums, the fixed array holds " + std::to_string(mx::kStaticScratchBytes) +
+                  " (use mx_spmv, which keeps them in the plan's own buffer)");
+        return MX_ERR_ARG;
+    }
+    void *fixed = nullptr;
+    MX_HIP(mx::static_scratch(&fixed));  // the address on the current device; looked up once per device
+    return spmv_on(plan, x_dev, y_dev, (hipStream_t)stream, need ? fixed : nullptr);
+}
+
+extern "C" int mx_static_scratch_bytes(void) { return (int)mx::kStaticScratchBytes; }
 
 extern "C" int mx_spmv_repeat(mx_plan *plan, const void *x_dev, void *y_dev, int n, void *stream)
 {
