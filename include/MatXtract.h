@@ -4,8 +4,14 @@
  * Source-compatible with the reference's include/MatXtract.h:3-34 (kernel entry points),
  * include/csr2csc.h:9-13 (transposes) and include/mmio.h:165-179 (Matrix-Market ingest,
  * exclusive_scan), together with the pieces of include/common.h a driver needs (valT, indT,
- * fragM/fragK, half, initVec, divup).  A driver written against the reference compiles
- * against this header unchanged and links with -lmatxtract_hip instead of the CUDA library.
+ * fragM/fragK, half, initVec, divup) and the standard headers that common.h:3-35 pulls in for
+ * its includers (<iostream>, <map>, <algorithm>, <parallel/algorithm>, <omp.h>, <sys/time.h>,
+ * <math.h> ...; the CUDA, thrust, cuSPARSE and cuBLAS ones have no counterpart).  mmio.h and
+ * csr2csc.h beside this file forward here.  The reference's driver,
+ * test/test_autotc_spmv.cpp, compiles against this directory in both precisions once its one
+ * direct CUDA call, cudaDeviceSynchronize() (:1529), is deleted (every wrapper here returns
+ * after its work is done), and links with -lmatxtract_hip instead of the CUDA libraries;
+ * tests/test_cxx_surface.py checks exactly that when the reference's source is at hand.
  *
  * Same conventions as the reference: precision is chosen at compile time (-Dfp64 -> double,
  * otherwise IEEE binary16 `half`); every pointer is HOST memory; arrays a function returns
@@ -22,11 +28,28 @@
 #ifndef MATXTRACT_H
 #define MATXTRACT_H
 
+/* what include/common.h:3-35 hands to every file that includes it */
+#include <algorithm>
+#include <array>
+#include <cassert>
+#include <cstddef>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <filesystem>
+#include <fstream>
+#include <iostream>
+#include <map>
 #include <vector>
+#include <parallel/algorithm>
+#include <math.h>
+#include <omp.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <sys/time.h>
+#include <time.h>
 
 #include "matxtract_hip.h"
 

@@ -144,11 +144,17 @@ hipError_t static_scratch(void **ptr);
 // combine kernel's launch run as well (strips_can_ride says whether a layout may); the rows of
 // those strips must be marked in the slice layout (rowInfo -2) so that the combine kernel leaves
 // them alone.
+// `ywide` (optional, all three launchers): an array of accumulators (binary32 for binary16
+// plans), one per row.  The CSR launchers also store every sum they write to y there,
+// unrounded; the tile launcher reads the old y of its rows from there instead of y, so that a
+// row which gets sums from both parts is rounded to the value type once.
 hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
-                         int what = 0, const DeviceTiles *strips = nullptr);
+                         int what = 0, const DeviceTiles *strips = nullptr, void *ywide = nullptr);
 bool strips_can_ride(mx_dtype dtype, const DeviceTiles &T, const void *x);
-hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s);
-hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s);
+hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s,
+                      void *ywide = nullptr);
+hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s,
+                        const void *ywide = nullptr);
 hipError_t launch_probe_f64(const double *A, const double *B, double *D, hipStream_t s);
 hipError_t launch_probe_f16(const void *A, const void *B, float *D, hipStream_t s);
 

@@ -201,7 +201,8 @@ __device__ __forceinline__ void wave_gather(const VT *__restrict__ x, int lane, 
 // offsets inside the tile (nrows+1 entries).
 template <typename VT, int W>
 __device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, const unsigned short *rowOff, int r0,
-                                            int nrows, VT *__restrict__ y, int accumulate, int tid)
+                                            int nrows, VT *__restrict__ y, int accumulate, int tid,
+                                            typename Acc<VT>::type *__restrict__ ywide)
 {
     typedef typename Acc<VT>::type AT;
     constexpr int rowsPerPass = kBlock / W;
@@ -214,6 +215,7 @@ __device__ __forceinline__ void reduce_rows(const typename Acc<VT>::type *prod, 
         if (l == 0) {
             if (accumulate) s += (AT)y[r0 + rr];
             y[r0 + rr] = (VT)s;
+            if (ywide) ywide[r0 + rr] = s;
         }
     }
 }
@@ -233,13 +235,15 @@ struct ScanItem {
 template <typename VT, int NPT>
 __device__ __forceinline__ void reduce_scan(const typename Acc<VT>::type *prod, const int *head, const unsigned short *rowOff,
                                             int r0, int nrows, VT *__restrict__ y, int accumulate, int tid,
-                                            typename Acc<VT>::type *carryV, int *carryF, int *carryR)
+                                            typename Acc<VT>::type *carryV, int *carryF, int *carryR,
+                                            typename Acc<VT>::type *__restrict__ ywide)
 {
     typedef typename Acc<VT>::type AT;
     const int lane = tid & 63, wave = tid >> 6;
     auto store = [&](int row, AT v) {
         if (accumulate) v += (AT)y[r0 + row];
         y[r0 + row] = (VT)v;
+        if (ywide) ywide[r0 + row] = v;
     };
     AT v[NPT];
     int h[NPT];
@@ -343,12 +347,15 @@ __device__ __forceinline__ void reduce_scan(const typename Acc<VT>::type *prod, 
 // With DICT the values are one byte per entry, indices into the matrix's at most 256 distinct
 // values (`dictG`, copied to LDS first): a stencil or a graph matrix then streams 3 bytes per
 // entry instead of 10.
+// `ywide` (optional): the sums as accumulators, unrounded, for a kernel that adds to these rows
+// afterwards (binary16 plans with tiles on shared rows: y is then rounded once, at the end).
 template <typename VT, int NPT, bool XCD, bool C16, bool SCAN, bool DICT = false>
 __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict__ rowPtr, const void *__restrict__ col,
                                                           const VT *__restrict__ val, const VT *__restrict__ xfull,
                                                           VT *__restrict__ y, const int4 *__restrict__ blockDesc,
                                                           const int *__restrict__ colBase, int xcols, int accumulate,
-                                                          const VT *__restrict__ dictG)
+                                                          const VT *__restrict__ dictG,
+                                                          typename Acc<VT>::type *__restrict__ ywide)
 {
     typedef typename Acc<VT>::type AT;
     __shared__ AT dictL[DICT ? 256 : 1];
@@ -420,17 +427,17 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
         }
         __syncthreads();
         if constexpr (SCAN) {
-            reduce_scan<VT, NPT>(prod, cols, rowOff, r0, nrows, y, accumulate, tid, wsum, wflag, wrow);
+            reduce_scan<VT, NPT>(prod, cols, rowOff, r0, nrows, y, accumulate, tid, wsum, wflag, wrow, ywide);
             return;
         }
         const int mean = (p1 - p0) / nrows;
-        if (mean <= 2) reduce_rows<VT, 1>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 4) reduce_rows<VT, 2>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 8) reduce_rows<VT, 4>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 16) reduce_rows<VT, 8>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 32) reduce_rows<VT, 16>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else if (mean <= 64) reduce_rows<VT, 32>(prod, rowOff, r0, nrows, y, accumulate, tid);
-        else reduce_rows<VT, 64>(prod, rowOff, r0, nrows, y, accumulate, tid);
+        if (mean <= 2) reduce_rows<VT, 1>(prod, rowOff, r0, nrows, y, accumulate, tid, ywide);
+        else if (mean <= 4) reduce_rows<VT, 2>(prod, rowOff, r0, nrows, y, accumulate, tid, ywide);
+        else if (mean <= 8) reduce_rows<VT, 4>(prod, rowOff, r0, nrows, y, accumulate, tid, ywide);
+        else if (mean <= 16) reduce_rows<VT, 8>(prod, rowOff, r0, nrows, y, accumulate, tid, ywide);
+        else if (mean <= 32) reduce_rows<VT, 16>(prod, rowOff, r0, nrows, y, accumulate, tid, ywide);
+        else if (mean <= 64) reduce_rows<VT, 32>(prod, rowOff, r0, nrows, y, accumulate, tid, ywide);
+        else reduce_rows<VT, 64>(prod, rowOff, r0, nrows, y, accumulate, tid, ywide);
     } else {
         // a single row longer than one tile
         AT s = 0;
@@ -454,6 +461,7 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
             for (int w = 0; w < kBlock / 64; ++w) t += wsum[w];
             if (accumulate) t += (AT)y[r0];
             y[r0] = (VT)t;
+            if (ywide) ywide[r0] = t;
         }
     }
 }
@@ -693,7 +701,8 @@ struct TileStep {  // one step's loads, as one lane holds them
     int hdr;       // header dword lane%32: lanes 0..15 hold the output rows
     int ax;        // column id
     typename std::conditional<sizeof(VT) == 8, double[8], v4i32>::type v;  // A operands
-    VT xr, yr;     // gathered x and old y, as loaded (looked at only when the step is multiplied)
+    VT xr;         // gathered x, as loaded (looked at only when the step is multiplied)
+    typename Acc<VT>::type yr;  // old y
 };
 
 // All loads of a step are unconditional: the count of loads in flight is then known at compile
@@ -720,7 +729,7 @@ template <typename VT>
 __global__ __launch_bounds__(kBlock) void tile_kernel(const int4 *__restrict__ waveDesc, const int *__restrict__ hdr,
                                                      const int *__restrict__ atox, const VT *__restrict__ tcVal,
                                                      const VT *__restrict__ x, VT *__restrict__ y, int nWaves,
-                                                     int accumulate)
+                                                     int accumulate, const typename Acc<VT>::type *__restrict__ ywide)
 {
     typedef typename Acc<VT>::type AT;
     constexpr bool F64 = sizeof(VT) == 8;
@@ -752,7 +761,9 @@ __global__ __launch_bounds__(kBlock) void tile_kernel(const int4 *__restrict__ w
     // or a row read element 0 and ignore it)
     auto gather = [&](Regs &R) {
         R.xr = x[max(R.ax, 0)];
-        R.yr = y[lane < 16 ? max(R.hdr, 0) : 0];
+        // (old y: as the kernel before this one left it, unrounded where that kernel kept it so)
+        const int yi = lane < 16 ? max(R.hdr, 0) : 0;
+        R.yr = ywide ? ywide[yi] : (AT)y[yi];
     };
     typedef typename std::conditional<F64, v4f64, v4f32>::type AccV;
     AccV acc;
@@ -805,7 +816,7 @@ __global__ __launch_bounds__(kBlock) void tile_kernel(const int4 *__restrict__ w
             if (lane < 16 && Ra.hdr >= 0) {
                 AT o = P.out[lane];
                 if (!(flags & 2)) o += P.out[lane + 8];  // one chunk in both halves (only lanes 0..7 have rows)
-                y[Ra.hdr] = (VT)((accumulate ? (AT)Ra.yr : (AT)0) + o);
+                y[Ra.hdr] = (VT)((accumulate ? Ra.yr : (AT)0) + o);
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[i] = 0;
@@ -928,6 +939,7 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
                                                               const int4 *__restrict__ heavyInfo, int nHeavy,
                                                               const int *__restrict__ segIdx, VT *__restrict__ y,
                                                               int accumulate, int skipEmpty,
+                                                              typename Acc<VT>::type *__restrict__ ywide,
                                                               const int4 *__restrict__ stripWaveDesc,
                                                               const int *__restrict__ stripHdr,
                                                               const VT *__restrict__ stripVal, const VT *__restrict__ x,
@@ -972,6 +984,7 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
             const bool mine = dd[j] >= 0 || (dd[j] == -1 && !skipEmpty);
             if (mine && accumulate) sum[j] += (AT)y[r];
             if (mine) y[r] = (VT)sum[j];
+            if (mine && ywide) ywide[r] = sum[j];
         }
         return;
     }
@@ -990,6 +1003,7 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
         for (int k = 0; k < 8; ++k)
             if (id[k] >= 0) sum += partial[id[k]];
         y[r] = (VT)sum;
+        if (ywide) ywide[r] = sum;
         return;
     }
     b -= nLightWG;
@@ -1006,7 +1020,11 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
             if (id[j] >= 0) sum += partial[id[j]];
     }
     sum = group_sum<16>(sum);
-    if (live && sub == 0) y[h.x] = (VT)(sum + (accumulate ? (AT)y[h.x] : (AT)0));
+    if (live && sub == 0) {
+        sum += accumulate ? (AT)y[h.x] : (AT)0;
+        y[h.x] = (VT)sum;
+        if (ywide) ywide[h.x] = sum;
+    }
 }
 
 // MFMA probes: one wave, operands and accumulators exchanged lane by lane (raw register
@@ -1066,16 +1084,17 @@ hipError_t static_scratch(void **ptr)
 }
 
 template <typename VT, int NPT>
-static void launch_csr_t(const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
+static void launch_csr_t(const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s, void *ywide)
 {
+    typedef typename mxk::Acc<VT>::type AT;
 #define MX_LAUNCH_ROWS(C16, SCAN, COLS, BASE)                                                                       \
     hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, C16, SCAN>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, s,      \
                        A.rowPtr, (const void *)(COLS), (const VT *)A.val, (const VT *)x, (VT *)y,                      \
-                       (const int4 *)A.blockDesc, (const int *)(BASE), A.cols, accumulate, (const VT *)nullptr)
+                       (const int4 *)A.blockDesc, (const int *)(BASE), A.cols, accumulate, (const VT *)nullptr, (AT *)ywide)
 #define MX_LAUNCH_ROWS_DICT(SCAN)                                                                                    \
     hipLaunchKernelGGL((mxk::csr_rows_kernel<VT, NPT, true, true, SCAN, true>), dim3(A.nBlocks), dim3(mxk::kBlock), 0, \
                        s, A.rowPtr, (const void *)A.col16, (const VT *)A.codes, (const VT *)x, (VT *)y,                  \
-                       (const int4 *)A.blockDesc, (const int *)A.colBase, A.cols, accumulate, (const VT *)A.dict)
+                       (const int4 *)A.blockDesc, (const int *)A.colBase, A.cols, accumulate, (const VT *)A.dict, (AT *)ywide)
     static_assert(mxk::kBlock == 256, "a workgroup copies the 256 dictionary entries, one per lane");
     if (A.useDict && A.col16 && A.codes && A.dict) {
         if (A.scan) MX_LAUNCH_ROWS_DICT(true);
@@ -1088,16 +1107,16 @@ static void launch_csr_t(const DeviceCsr &A, const void *x, void *y, int accumul
 #undef MX_LAUNCH_ROWS_DICT
 }
 
-hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s)
+hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s, void *ywide)
 {
     if (A.nBlocks <= 0) return hipSuccess;
     if (dtype == MX_F64) {
-        if (A.npt == 8) launch_csr_t<double, 8>(A, x, y, accumulate, s);
-        else if (A.npt == 4) launch_csr_t<double, 4>(A, x, y, accumulate, s);
+        if (A.npt == 8) launch_csr_t<double, 8>(A, x, y, accumulate, s, ywide);
+        else if (A.npt == 4) launch_csr_t<double, 4>(A, x, y, accumulate, s, ywide);
         else return hipErrorInvalidValue;
     } else {
-        if (A.npt == 16) launch_csr_t<_Float16, 16>(A, x, y, accumulate, s);
-        else if (A.npt == 8) launch_csr_t<_Float16, 8>(A, x, y, accumulate, s);
+        if (A.npt == 16) launch_csr_t<_Float16, 16>(A, x, y, accumulate, s, ywide);
+        else if (A.npt == 8) launch_csr_t<_Float16, 8>(A, x, y, accumulate, s, ywide);
         else return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -1105,7 +1124,7 @@ hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y
 
 template <typename VT>
 static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, int what,
-                                  const DeviceTiles *strips)
+                                  const DeviceTiles *strips, void *ywide)
 {
     typedef typename mxk::Acc<VT>::type AT;
     const bool dict = P.useDict && P.ecode && P.dict;
@@ -1155,7 +1174,7 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     hipLaunchKernelGGL((mxk::slice_combine_kernel<VT, STRIPS>), dim3(nStripWG + nRowWG + nLightWG + nHeavyWG),                 \
                        dim3(mxk::kBlock), 0, s, (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, P.lightRow,                    \
                        (const int4 *)P.lightIdx, P.nLight, nLightWG, (const int4 *)P.heavyInfo, P.nHeavy, P.segIdx, (VT *)y,    \
-                       (accumulate || P.subset) ? 1 : 0, P.subset ? 1 : 0, ride ? (const int4 *)strips->waveDesc : nullptr,   \
+                       (accumulate || P.subset) ? 1 : 0, P.subset ? 1 : 0, (AT *)ywide, ride ? (const int4 *)strips->waveDesc : nullptr,   \
                        ride ? strips->hdr : nullptr, ride ? (const VT *)strips->tcVal : nullptr, (const VT *)x,              \
                        ride ? strips->nWaves : 0, nStripWG, nHeavyWG, P.lightQuads)
     if (ride) MX_LAUNCH_COMBINE(true);
@@ -1164,18 +1183,19 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     return hipGetLastError();
 }
 hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
-                         int what, const DeviceTiles *strips)
+                         int what, const DeviceTiles *strips, void *ywide)
 {
     if (P.rows <= 0) return hipSuccess;
-    if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s, what, nullptr);
-    return launch_slices_t<_Float16>(P, x, y, accumulate, s, what, strips);
+    if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s, what, nullptr, ywide);
+    return launch_slices_t<_Float16>(P, x, y, accumulate, s, what, strips, ywide);
 }
 bool strips_can_ride(mx_dtype dtype, const DeviceTiles &T, const void *x)
 {
     return dtype == MX_F16 && T.nWaves > 0 && T.dense && T.ownedRows && !((uintptr_t)x & 15);
 }
 
-hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s)
+hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s,
+                        const void *ywide)
 {
     if (T.nWaves <= 0) return hipSuccess;
     const int grid = (T.nWaves + 3) / 4;
@@ -1188,10 +1208,10 @@ hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, voi
     }
     if (dtype == MX_F64)
         hipLaunchKernelGGL((mxk::tile_kernel<double>), dim3(grid), dim3(mxk::kBlock), 0, s, (const int4 *)T.waveDesc, T.hdr,
-                           T.atox, (const double *)T.tcVal, (const double *)x, (double *)y, T.nWaves, accumulate);
+                           T.atox, (const double *)T.tcVal, (const double *)x, (double *)y, T.nWaves, accumulate, (const double *)ywide);
     else
         hipLaunchKernelGGL((mxk::tile_kernel<_Float16>), dim3(grid), dim3(mxk::kBlock), 0, s, (const int4 *)T.waveDesc, T.hdr,
-                           T.atox, (const _Float16 *)T.tcVal, (const _Float16 *)x, (_Float16 *)y, T.nWaves, accumulate);
+                           T.atox, (const _Float16 *)T.tcVal, (const _Float16 *)x, (_Float16 *)y, T.nWaves, accumulate, (const float *)ywide);
     return hipGetLastError();
 }
 

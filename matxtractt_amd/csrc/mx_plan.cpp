@@ -978,6 +978,9 @@ struct mx_plan {
     mx::DeviceTiles tiles;    // tile part, general form (tile_kernel)
     mx::DeviceTiles strips;   // tile part, binary16 strips on rows of their own (tile_dense_kernel)
     int tile_nnz = 0;
+    // binary16 plans whose general tiles share rows with the CSR part: the CSR part's sums as
+    // binary32, one per row, which the tile kernel adds to (y is then rounded once)
+    void *ywide = nullptr;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 };
@@ -999,6 +1002,7 @@ extern "C" void mx_plan_destroy(mx_plan *plan)
     free_slices(plan->slices);
     free_tiles(plan->tiles);
     free_tiles(plan->strips);
+    (void)hipFree(plan->ywide);
     if (plan->ev0) (void)hipEventDestroy(plan->ev0);
     if (plan->ev1) (void)hipEventDestroy(plan->ev1);
     if (plan->stream) (void)hipStreamDestroy(plan->stream);
@@ -1031,20 +1035,20 @@ static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
 // `partial` (optional): where the slice kernel puts the sums of the virtual rows, in place of the
 // plan's own buffer.
 static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate, hipStream_t s,
-                           const mx::DeviceTiles *strips = nullptr, void *partial = nullptr)
+                           const mx::DeviceTiles *strips = nullptr, void *partial = nullptr, void *ywide = nullptr)
 {
     if (plan->csr_variant != 0 && ((uintptr_t)x & 15)) {
         set_error("mx_spmv: x must be 16-byte aligned for this plan");
         return MX_ERR_ARG;
     }
-    if (plan->csr_variant != 1) MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s));
+    if (plan->csr_variant != 1) MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s, ywide));
     if (plan->csr_variant != 0) {
         if (partial) {
             mx::DeviceSlices L = plan->slices;  // a view: same arrays, other sums
             L.partial = partial;
-            MX_HIP(mx::launch_slices(plan->dtype, L, x, y, accumulate, s, 0, strips));
+            MX_HIP(mx::launch_slices(plan->dtype, L, x, y, accumulate, s, 0, strips, ywide));
         } else {
-            MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s, 0, strips));
+            MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x, y, accumulate, s, 0, strips, ywide));
         }
     }
     return MX_OK;
@@ -1543,6 +1547,10 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                 plan->strips.ownedRows = true;
             }
             plan->tile_nnz = nnzGeneral + nnzStrips;
+            if (P->dtype == MX_F16 && plan->tiles.nWaves > 0) {
+                rc = upload_bytes(&plan->ywide, nullptr, 0, (size_t)std::max(P->rows, 1) * sizeof(float));
+                if (rc) return fail(rc);
+            }
             phase("tile layouts");
         }
     } catch (const std::bad_alloc &) {
@@ -1698,9 +1706,12 @@ static int spmv_on(mx_plan *plan, const void *x, void *y, hipStream_t s, void *p
     // a launch of their own, as with the row-tile form of the CSR part)
     static const bool apart = std::getenv("MX_STRIPS_APART") && std::atoi(std::getenv("MX_STRIPS_APART"));
     const bool ride = !apart && plan->csr_variant == 1 && mx::strips_can_ride(plan->dtype, plan->strips, x);
-    int rc = launch_csr_part(plan, x, y, 0, s, ride ? &plan->strips : nullptr, partial);
+    // (a binary16 row that gets sums from both parts: the CSR part leaves its sum in binary32 as
+    // well and the tile kernel adds to that, so that y is rounded once, not twice)
+    void *wide = plan->tiles.nWaves > 0 ? plan->ywide : nullptr;
+    int rc = launch_csr_part(plan, x, y, 0, s, ride ? &plan->strips : nullptr, partial, wide);
     if (rc) return rc;
-    MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x, y, 1, s));
+    MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x, y, 1, s, wide));
     if (!ride) MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x, y, 1, s));
     return MX_OK;
 }

@@ -2,9 +2,9 @@
 // their names.  The sanitizer driver never reaches them.
 #include "mx_device.h"
 namespace mx {
-hipError_t launch_tiles(mx_dtype, const DeviceTiles &, const void *, void *, int, hipStream_t) { return hipErrorUnknown; }
-hipError_t launch_csr(mx_dtype, const DeviceCsr &, const void *, void *, int, hipStream_t) { return hipErrorUnknown; }
-hipError_t launch_slices(mx_dtype, const DeviceSlices &, const void *, void *, int, hipStream_t, int, const DeviceTiles *) { return hipErrorUnknown; }
+hipError_t launch_tiles(mx_dtype, const DeviceTiles &, const void *, void *, int, hipStream_t, const void *) { return hipErrorUnknown; }
+hipError_t launch_csr(mx_dtype, const DeviceCsr &, const void *, void *, int, hipStream_t, void *) { return hipErrorUnknown; }
+hipError_t launch_slices(mx_dtype, const DeviceSlices &, const void *, void *, int, hipStream_t, int, const DeviceTiles *, void *) { return hipErrorUnknown; }
 hipError_t static_scratch(void **p) { *p = nullptr; return hipErrorUnknown; }
 bool strips_can_ride(mx_dtype, const DeviceTiles &, const void *) { return false; }
 hipError_t launch_probe_f64(const double *, const double *, double *, hipStream_t) { return hipErrorUnknown; }

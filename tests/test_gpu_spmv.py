@@ -802,6 +802,87 @@ def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
     Q.close()
 
 
+def test_fp16_cli_passes_its_own_element_check(mx, tmp_path):
+    """matxtract_perftest_fp16 (the reference's USE_FP64=OFF build, CMakeLists.txt:17-36) on the
+    seeded binary16 workloads and on a Matrix-Market file with the reference's i % 15 data: the
+    reference-style element check (eQcheck, relative 1e-1 per element, test/test_autotc_spmv.cpp:
+    257-293) must print `Success!`, the line the reference's scripts look for
+    (script/duse.sh:35-38).  Hybrid plans put sums from the CSR part and from the tiles on the
+    same rows: those are rounded to binary16 once, so a row whose parts cancel still passes."""
+    import os
+    import re
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "matxtractt_amd", "bin", "matxtract_perftest_fp16")
+    base = [exe, "--warm", "2", "--iters", "5"]
+    for cfg, scale in ((4, 1 / 16), (5, 1 / 32)):
+        for tau in (("0", "0"), ("0.5", "0.25"), ("1", "1")):
+            for extra in ([], ["--keep-tiles"], ["--all-tiles"]):
+                cmd = base + extra + [tau[0], tau[1], "--config", str(cfg), "--scale", repr(scale)]
+                print("fp16 cli:", " ".join(cmd[1:]), flush=True)
+                out = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+                assert out.returncode == 0, out.stderr[-2000:]
+                assert "Processing the synthetic workload %d graph in FP16" % cfg in out.stdout
+                assert "Success! All values match within the tolerance" in out.stdout, out.stdout[-1500:]
+                assert "Error at index (" not in out.stdout
+                assert re.search(r"MatXtract time\s*=\s*([\d\.Ee+-]+)\s*ms", out.stdout)
+                assert re.search(r"MatXtract GFLOPS= \d+\.\d\d", out.stdout)
+    # a .mtx file; the values are overwritten with i % 15 as the reference does (:1091)
+    A, _ = mx.gen_config(5, scale=1 / 256)
+    p = tmp_path / "m.mtx"
+    with open(p, "w") as f:
+        f.write("%%MatrixMarket matrix coordinate real general\n")
+        f.write("%d %d %d\n" % (A.rows, A.cols, A.nnz))
+        for r in range(A.rows):
+            for q in range(A.rowPtr[r], A.rowPtr[r + 1]):
+                f.write("%d %d 1.0\n" % (r + 1, A.colInd[q] + 1))
+    for args in (["0.5", "0.25", str(p)], ["1", "1", str(p)], ["--all-tiles", "0.75", "0.5", str(p)], [str(p)]):
+        out = subprocess.run(base + args, capture_output=True, text=True, timeout=300)
+        assert out.returncode == 0, out.stderr[-2000:]
+        assert "Success! All values match within the tolerance for %d elements." % A.rows in out.stdout, out.stdout[-1500:]
+
+
+def test_binary16_rows_shared_by_both_parts_are_rounded_once(mx, ora):
+    """Rows built so that the CSR part's sum and the tiles' sum cancel almost entirely: with y
+    rounded to binary16 between the two parts the small remainder would be lost in the
+    rounding of the large partial sum; rounded once it is exact."""
+    import torch
+    rng = np.random.default_rng(11)
+    rows, cols = 512, 1024
+    rp, ci, va = [0], [], []
+    for r in range(rows):
+        # a dense run of 8 columns (the tiles take it) whose sum is s, and scattered entries
+        # (the CSR part) whose sum is -s + a small remainder
+        c0 = 8 * int(rng.integers(0, 16))
+        run = rng.integers(1, 60, 8).astype(np.float64) / 64.0          # exact in binary16
+        s = run.sum()
+        far = np.sort(rng.choice(np.arange(256, cols), 3, replace=False))
+        rem = float(rng.integers(1, 8)) / 1024.0                          # small, exact
+        sc = np.array([-(s // 2), -(s - s // 2), rem])                    # exact in binary16 (|.| < 32, step 1/64)
+        ci += list(range(c0, c0 + 8)) + far.tolist()
+        va += run.tolist() + sc.tolist()
+        rp.append(len(ci))
+    A = mx.Csr(rows, cols, np.array(rp, np.int32), np.array(ci, np.int32), np.array(va, np.float16))
+    assert np.array_equal(A.val.astype(np.float64), np.array(va))        # nothing was rounded
+    x = np.ones(cols, np.float16)
+    ref = ora.spmv_f16_f32acc(A.val, A.rowPtr, A.colInd, x)[0].astype(np.float64)
+    assert np.all(ref > 0) and ref.max() < 0.01                           # only the remainders are left
+    xd = torch.from_numpy(x).cuda()
+    seen_tiles = 0
+    for tau in ((0.5, 0.5), (0.25, 0.25), (1.0, 0.5)):
+        for flags in (mx.MX_PLAN_ALL_TILES, mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_SLICES, mx.MX_PLAN_KEEP_TILES):
+            part = mx.Partition(A, *tau)
+            plan = mx.Plan(part, flags)
+            y = plan.spmv(xd)
+            torch.cuda.synchronize()
+            if plan.info["tile_nnz"] > 0 and plan.info["csr_nnz"] > 0:
+                seen_tiles += 1
+                assert np.array_equal(y.cpu().numpy().astype(np.float64), ref), (tau, flags)
+            plan.close()
+            part.close()
+    assert seen_tiles >= 3
+
+
 @pytest.mark.gpu
 def test_device_transpose_equals_the_host_transpose(mx, ora):
     """mx_transpose_device (csr2csc / csc2csr on arrays that stay in device memory) against
