@@ -1,20 +1,29 @@
 #!/usr/bin/env python3
 """Benchmark of the hybrid SpMV hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 2] [--all] [--no-sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload N ...] [--no-sweep | --tau C R]
 
-A step is one y = A*x over the whole matrix, inputs resident in HBM.  The default workload is
-the FP64 block-clustered 65536x65536 matrix (synthetic workload 2) with (tau_c, tau_r) picked
-by a sweep of the 5x5 grid {0,.25,.5,.75,1}^2 restricted to tau_c >= tau_r; `--all` adds the
-other workloads (3: FP64 stencil, 4/5: FP16) as extra records in the same JSON line.
+A step is one y = A*x over the whole matrix, inputs resident in HBM.  With no flags the four
+GPU workloads of the benchmark run: the headline is the largest one, workload 5 (FP16 mixed,
+4.2 M rows, 63 M entries; (tau_c, tau_r) = best of the 5x5 grid {0,.25,.5,.75,1}^2 with
+tau_c >= tau_r), and workloads 2 (FP64 block-clustered, same sweep), 3 (FP64 stencil) and 4
+(FP16 power-law) follow under "others", each with its own roofline record, parity figure and
+cold-cache time.
 
-Prints ONE JSON line: whole-job GFLOP/s = 2*nnz/t, the roofline record of the dominant kernel
-(algorithmic bytes of that kernel / its mean launch time by HIP events on the launch stream,
-against 8 TB/s), and the CPU baseline (the oracle's single-thread CSR SpMV on the same matrix).
+Prints ONE JSON line.  `value` = 2*nnz/t of the headline workload (GFLOP/s).  `roofline` prices
+the WHOLE product: the reference's algorithmic bytes of the matrix (nnz*(sizeof(valT)+4) +
+(rows+1)*4 + cols*sizeof(valT) + rows*sizeof(valT), test/test_cdspmv.cpp:214) over the time of
+one product -- HIP events on the plan's own stream around K back-to-back products -- against
+8 TB/s.  `roofline.kernels` lists every kernel launch of the product timed alone, each with its
+share of those bytes (the shares add up to the whole) and, where profiles/ holds a rocprofv3
+counter run of that kernel on that workload and plan, its measured HBM traffic.  `cpu_baseline`
+is the oracle's single-thread CSR loop on the same matrix, on this box's host cores.
 """
 import argparse
+import glob
 import json
 import os
+import re
 import sys
 import time
 
@@ -24,20 +33,6 @@ sys.path.insert(0, ROOT)
 METRIC = "SpMV GFLOP/s (2·nnz/t) + % of HBM roofline, FP64 and FP16, 1 GPU"
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 GRID = (0.0, 0.25, 0.5, 0.75, 1.0)
-# HBM-side bytes per launch (read + written) of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE runs of this script, each counter scaled by what it reads for an elementwise kernel of
-# known size (--calibrate-copy): FETCH_SIZE x 2.000, WRITE_SIZE x 1.000.  The text files under profiles/
-# hold the counter values.  (workload, kernel, plan has tiles) -> bytes
-TRAFFIC = {
-    (2, "csr_rows_kernel<f64>", False): 47165962,
-    (2, "csr_slice_kernel<f64>", False): 48823291,
-    (3, "csr_rows_kernel<f64>", False): 287431623,
-    (3, "csr_rows_kernel<f64,dict>", False): 101747762,   # one byte per value: the stencil has two distinct values
-    (3, "csr_slice_kernel<f64,dict>", False): 109970561,
-    (4, "csr_slice_kernel<f16>", False): 55821536,
-    (5, "csr_slice_kernel<f16>", False): 301417778,
-    (5, "csr_slice_kernel<f16>", True): 190181456,   # tau=(1,1): the strips run through tile_dense_kernel
-}
 WORKLOADS = {
     1: "configs[0]: FP64 random 4096x4096, 16 nnz/row",
     2: "configs[1]: FP64 block-clustered 65536x65536, ~64 nnz/row, 40% of nnz in dense 8x8 blocks in a 2048-wide band",
@@ -45,29 +40,88 @@ WORKLOADS = {
     4: "configs[3]: FP16 power-law 1048576x1048576, Zipf(1.6) row lengths in [1,4096], mean ~10",
     5: "configs[4]: FP16 mixed 4194304x4194304, 20% of rows in dense 32-column strips + power-law rows",
 }
+SWEPT = (2, 5)  # the workloads BASELINE.json sweeps; 3 and 4 run CSR-only and at two hybrid points for the record
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def kernel_bytes(mx, dtype, rows, cols, nnz):
-    """Algorithmic bytes of a CSR-form SpMV over `nnz` entries (data_origin1 of the reference)."""
-    return mx.algorithmic_bytes(dtype, rows, cols, nnz)
+def read_traffic():
+    """HBM bytes per launch from the rocprofv3 counter runs under profiles/: lines of the form
+    `TRAFFIC workload=<n> plan=<csr_only|hybrid> kernel=<name> read=<bytes> written=<bytes>` (FETCH_SIZE and
+    WRITE_SIZE per dispatch, scaled by what the same counters read for a copy kernel of known size;
+    the files say how).  Nothing is hard-coded here: a kernel without such a line reports null."""
+    table = {}
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.txt"))):
+        with open(path) as f:
+            for line in f:
+                m = re.match(r"TRAFFIC workload=(\d+) plan=(\w+) kernel=(\S+) read=(\d+) written=(\d+)", line.strip())
+                if m:
+                    table[(int(m.group(1)), m.group(2), m.group(3))] = {
+                        "read": int(m.group(4)), "written": int(m.group(5)), "file": os.path.relpath(path, ROOT)}
+    return table
 
 
-def measure(mx, torch, A, xd, yd, tau, warm, iters, flags=None):
-    part = mx.Partition(A, *tau)
-    plan = mx.Plan(part, mx.MX_PLAN_DEFAULT if flags is None else flags)
-    tot, tile, csr = plan.time(xd, yd, warm=warm, iters=iters)
-    rec = {"tau_c": tau[0], "tau_r": tau[1], "ms_total": tot, "ms_tile": tile, "ms_csr": csr,
-           "tile_nnz": plan.info["tile_nnz"], "csr_nnz": plan.info["csr_nnz"],
-           "tile_chunks": plan.info["tile_chunks"], "tile_bytes": plan.info["tile_bytes"],
-           "csr_bytes": plan.info["csr_bytes"], "tc_nnz_ratio": part.tc_nnz_ratio if tau != (0.0, 0.0) else 0.0}
-    return part, plan, rec
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            return next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "unknown")
+    except OSError:
+        return "unknown"
 
 
-def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_tau=None):
+def cpu_baseline(mx, ora, A, x):
+    """The oracle's CSR loop on the same matrix: one thread pinned to one core, as the reference's
+    spmv_serial; and (labelled as not the reference's) the same routine on all cores."""
+    import numpy as np
+    f16 = A.dtype != mx.MX_F64
+    run = (lambda rp: ora.spmv_f16_f32acc(A.val, rp, A.colInd, x)) if f16 else (lambda rp: ora.spmv_f64(A.val, rp, A.colInd, x))
+    affinity = os.sched_getaffinity(0)
+    pinned = None
+    try:
+        pinned = min(affinity)
+        os.sched_setaffinity(0, {pinned})
+    except OSError:
+        pinned = None
+    reps = []
+    try:
+        for _ in range(12):
+            t0 = time.perf_counter()
+            run(A.rowPtr)
+            reps.append(time.perf_counter() - t0)
+    finally:
+        if pinned is not None:
+            os.sched_setaffinity(0, affinity)
+    t_cpu = min(reps[2:])
+    base = {"value": 2.0 * A.nnz / t_cpu / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+            "cpu": cpu_model(), "cpus_visible": len(affinity), "pinned_to_cpu": pinned,
+            "sample": "the full matrix of the headline workload, best of 10 after 2 warm-ups (%.1f ms per SpMV, %.1f s of "
+                      "CPU work in all), single thread as the reference's spmv_serial" % (t_cpu * 1e3, sum(reps))}
+    from concurrent.futures import ThreadPoolExecutor
+    ncore = max(1, min(16, len(affinity)))
+    cuts = np.searchsorted(A.rowPtr, np.linspace(0, A.nnz, ncore + 1)).astype(int)
+    cuts[0], cuts[-1] = 0, A.rows
+
+    def part_run(k):
+        r0, r1 = int(cuts[k]), int(cuts[k + 1])
+        if r1 > r0:
+            run(A.rowPtr[r0:r1 + 1])
+    reps = []
+    with ThreadPoolExecutor(ncore) as ex:
+        for _ in range(7):
+            t0 = time.perf_counter()
+            list(ex.map(part_run, range(ncore)))
+            reps.append(time.perf_counter() - t0)
+    t_all = min(reps[2:])
+    allc = {"value": 2.0 * A.nnz / t_all / 1e9, "unit": "GFLOP/s", "cores": ncore, "kind": "port",
+            "sample": "not the reference's (its CPU path is serial): the oracle routine on %d nnz-balanced row ranges in "
+                      "parallel threads, best of 5 (%.2f ms)" % (ncore, t_all * 1e3)}
+    return base, allc
+
+
+def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=None):
+    """mode: 'sweep' (the 5x5 grid), 'points' (CSR-only and two hybrid points) or 'csr' ((0,0) only)."""
     import numpy as np
     t0 = time.time()
     A, x = mx.gen_config(cfg)
@@ -78,56 +132,88 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
     B = A.algorithmic_bytes
     dtype = "f64" if A.dtype == mx.MX_F64 else "f16"
 
-    # tau sweep with short timing loops
-    points = [(c, r) for c in GRID for r in GRID if c >= r] if sweep else [(0.0, 0.0)]
+    # ---- which (tau_c, tau_r): every candidate is partitioned (on the device for large matrices),
+    # planned and timed by mx_tune_tau with short loops; candidates that send nothing to the tile
+    # kernels are one and the same CSR-only plan and are timed once.  MX_PLAN_KEEP_TILES: every
+    # candidate runs the hybrid its fragments give, also where the plan's own estimate would send
+    # everything through the CSR part (what that estimate says is recorded below).
+    t0 = time.time()
     if only_tau is not None:
-        points = [tuple(only_tau)]  # nothing else: a profile of this run then shows one plan's kernels only
+        points = [tuple(only_tau)]
+    elif mode == "sweep":
+        points = None
+    elif mode == "points":
+        points = [(0.0, 0.0), (0.5, 0.25), (1.0, 1.0)]
+    else:
+        points = [(0.0, 0.0)]
     table = []
-    # (MX_PLAN_KEEP_TILES: every point runs the hybrid its fragments give, also where the plan's own
-    # estimate would send everything through the CSR part; what that estimate says is recorded below)
-    for tau in points:
-        part, plan, rec = measure(mx, torch, A, xd, yd, tau, 20, 200, mx.MX_PLAN_KEEP_TILES)
-        table.append(rec)
-        log("  tau=(%.2f,%.2f) total %.2f us (tile %.2f + csr %.2f) tile_nnz=%d" %
-            (tau[0], tau[1], rec["ms_total"] * 1e3, rec["ms_tile"] * 1e3, rec["ms_csr"] * 1e3, rec["tile_nnz"]))
-        plan.close()
-        part.close()
-    best = min(table, key=lambda r: r["ms_total"]) if only_tau is None else table[-1]
-    if best["tile_nnz"] == 0 and only_tau is None:
-        # every point that sends nothing to the tile kernel is the same CSR-only plan: call it (0, 0)
-        best = next(r for r in table if (r["tau_c"], r["tau_r"]) == (0.0, 0.0))
+    if points is None:
+        _, _, tt = mx.tune_tau(A, levels=5, flags=mx.MX_PLAN_KEEP_TILES, warm=10, iters=100)
+        table = [{"tau_c": c, "tau_r": r, "ms_total": ms, "tile_nnz": tn} for c, r, ms, tn in tt]
+    else:
+        for tau in points:
+            part = mx.Partition(A, *tau, device=A.nnz >= (1 << 21) and tau != (0.0, 0.0))
+            plan = mx.Plan(part, mx.MX_PLAN_KEEP_TILES)
+            ms = plan.time(xd, yd, warm=10, iters=100, parts=False)[0]
+            table.append({"tau_c": tau[0], "tau_r": tau[1], "ms_total": ms, "tile_nnz": plan.info["tile_nnz"]})
+            plan.close()
+            part.close()
+    for r in table:
+        log("  tau=(%.2f,%.2f) %.2f us tile_nnz=%d" % (r["tau_c"], r["tau_r"], r["ms_total"] * 1e3, r["tile_nnz"]))
+    sweep_s = time.time() - t0
+    csr_only = next((r for r in table if r["tile_nnz"] == 0), None)
     hybrid = [r for r in table if r["tile_nnz"] > 0]
     best_hybrid = min(hybrid, key=lambda r: r["ms_total"]) if hybrid else None
-    csr_only = next((r for r in table if (r["tau_c"], r["tau_r"]) == (0.0, 0.0)), None)
-
-    # the timed run on the best point: W warm-up steps, then exactly K steps between syncs
+    best = min(table, key=lambda r: r["ms_total"])
+    if best["tile_nnz"] == 0:
+        best = dict(csr_only, tau_c=0.0, tau_r=0.0)  # every point without tiles is the CSR-only plan: call it (0, 0)
     tau = (best["tau_c"], best["tau_r"])
-    if best_hybrid:
-        p2 = mx.Partition(A, best_hybrid["tau_c"], best_hybrid["tau_r"])
-        q2 = mx.Plan(p2)  # default flags: the plan's own decision at the best hybrid point
-        best_hybrid["default_plan_keeps_tiles"] = q2.info["tile_nnz"] > 0
+
+    # ---- the plan of the best point, from the matrix to the first y: host route and device route
+    def first_y(device):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        part = mx.Partition(A, *tau, device=device)
+        t1 = time.perf_counter()
+        plan = mx.Plan(part, mx.MX_PLAN_KEEP_TILES)
+        t2 = time.perf_counter()
+        plan.spmv(xd, yd)
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        return part, plan, {"partition_ms": (t1 - t0) * 1e3, "plan_create_ms": (t2 - t1) * 1e3,
+                            "first_spmv_ms": (t3 - t2) * 1e3, "total_ms": (t3 - t0) * 1e3}
+    part, plan, host_route = first_y(False)
+    route = {"host": host_route}
+    if tau != (0.0, 0.0):
+        mx.Partition(A, 0.25, 0.25, device=True).close()  # first use of the device code, not timed
+        p2, q2, route["device"] = first_y(True)
+        route["same_partition"] = part.hash == p2.hash
         q2.close()
         p2.close()
-    part, plan, _ = measure(mx, torch, A, xd, yd, tau, 5, 20, mx.MX_PLAN_KEEP_TILES)
+    info = plan.info
+
+    # ---- the timed run: W warm-up products, then exactly K products between synchronisations
     plan.spmv_repeat(xd, yd, warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     plan.spmv_repeat(xd, yd, steps)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    # per-kernel launch durations by HIP events on the plan's own stream
-    ev_total, ev_tile, ev_csr = plan.time(xd, yd, warm=warmup, iters=steps)
+    # the same by HIP events on the plan's own stream, over enough launches to average the launch jitter
+    n_ev = max(steps, 1000)
+    ev_total = plan.time(xd, yd, warm=max(warmup, 100), iters=n_ev, parts=False)[0]
+    kernels = plan.time_kernels(xd, yd, warm=max(warmup, 100), iters=n_ev)
     y = yd.cpu().numpy().astype(np.float64)
 
-    # parity of the timed configuration against the oracle
+    # ---- parity of the timed configuration against the oracle
     if A.dtype == mx.MX_F64:
         ref = ora.spmv_f64(A.val, A.rowPtr, A.colInd, x)
     else:
         ref = ora.spmv_f16_f32acc(A.val, A.rowPtr, A.colInd, x)[0].astype(np.float64)
     rel_l2 = float(np.linalg.norm(y - ref) / np.linalg.norm(ref))
 
-    # the same SpMV with cold caches: a 1 GiB buffer is swept between launches, so neither the
-    # L2s (8 x 4 MB) nor the 256 MB memory-side cache hold the matrix when the launch starts
+    # ---- cold caches: a 1 GiB buffer is swept between launches, so neither the L2s (8 x 4 MB) nor
+    # the 256 MB memory-side cache hold the matrix when the product starts
     flush = torch.empty(1 << 28, dtype=torch.float32, device=dev)
     cold = []
     for _ in range(15):
@@ -137,124 +223,76 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, sweep, cpu_baseline, only_t
     del flush
     cold_ms = float(np.median(cold))
 
-    info = plan.info
-    if ev_tile > ev_csr:
-        dom = {"kernel": "tile_%s_kernel" % dtype, "ms": ev_tile,
-               "bytes": kernel_bytes(mx, A.dtype, min(A.rows, 8 * info["tile_chunks"]), 0, info["tile_nnz"])}
-    else:
-        # the CSR part's main kernel alone (the slice variant has a small combine kernel after it)
-        ms_main = plan.time_csr_main(xd, yd, warm=warmup, iters=steps)
-        name = "csr_slice_kernel<%s>" if info["csr_main_kernel"] == 1 else "csr_rows_kernel<%s>"
-        if info["csr_value_dict"]:
-            name = name.replace("<%s>", "<%s,dict>")
-        dom = {"kernel": name % dtype, "ms": ms_main,
-               "bytes": kernel_bytes(mx, A.dtype, A.rows, A.cols, info["csr_main_nnz"])}
-    achieved = dom["bytes"] / (dom["ms"] * 1e-3)
+    # ---- what the plan's own estimate decides at the best hybrid point (default flags)
+    if best_hybrid:
+        p2 = mx.Partition(A, best_hybrid["tau_c"], best_hybrid["tau_r"], device=A.nnz >= (1 << 21))
+        q2 = mx.Plan(p2)
+        best_hybrid = dict(best_hybrid, default_plan_keeps_tiles=q2.info["tile_nnz"] > 0)
+        q2.close()
+        p2.close()
+
+    plan_kind = "hybrid" if info["tile_nnz"] > 0 else "csr_only"
+    krecs, tr_sum, tr_all = [], 0, True
+    for k in kernels:
+        t = traffic.get((cfg, plan_kind, k["name"]))
+        if t is None:
+            tr_all = False
+        else:
+            tr_sum += t["read"] + t["written"]
+        krecs.append({"kernel": k["name"], "ms_per_launch": k["ms"], "nnz": k["nnz"],
+                      "algorithmic_bytes": k["algorithmic_bytes"],
+                      "achieved": k["algorithmic_bytes"] / (k["ms"] * 1e-3) / 1e9,
+                      "frac": k["algorithmic_bytes"] / (k["ms"] * 1e-3) / HBM_PEAK,
+                      "traffic": (t["read"] + t["written"]) if t else None,
+                      "traffic_from": t["file"] if t else None})
+    achieved = B / (ev_total * 1e-3)
+    roofline = {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": achieved / HBM_PEAK,
+                "traffic": tr_sum if (tr_all and krecs) else None,
+                "what": "the whole product (%s): algorithmic bytes of the matrix over the mean time of one product in a "
+                        "train of %d back-to-back products, HIP events on the plan's stream" %
+                        (" + ".join(k["kernel"] for k in krecs), n_ev),
+                "bytes_per_launch": B, "ms_per_launch": ev_total, "kernels": krecs}
+    if info["csr_value_dict"]:
+        roofline["note"] = ("the matrix has %d distinct values and the main kernel reads one byte per entry for them: the "
+                            "algorithmic bytes still count sizeof(valT) per entry, so frac can exceed what the traffic "
+                            "would give; `traffic` is what the kernels really move" % info["csr_value_dict"])
     rec = {
         "workload": WORKLOADS[cfg], "dtype": dtype, "rows": A.rows, "nnz": A.nnz,
-        "tau_c": tau[0], "tau_r": tau[1], "csr_variant": ("rows", "slices", "split")[info["csr_variant"]],
+        "tau_c": tau[0], "tau_r": tau[1], "plan": plan_kind, "csr_variant": ("rows", "slices", "split")[info["csr_variant"]],
+        "tile_nnz": info["tile_nnz"], "csr_nnz": info["csr_nnz"],
         "ms_per_step": wall_ms, "ms_per_step_events": ev_total,
         "gflops": 2.0 * A.nnz / (wall_ms * 1e-3) / 1e9,
         "algorithmic_bytes": B,
         "hbm_frac_whole_spmv": B / (wall_ms * 1e-3) / HBM_PEAK,
         "cold_cache": {"ms_per_step": cold_ms, "gflops": 2.0 * A.nnz / (cold_ms * 1e-3) / 1e9,
                        "hbm_frac_whole_spmv": B / (cold_ms * 1e-3) / HBM_PEAK,
-                       "how": "median of 15 single launches, each after a 1 GiB buffer sweep and a sync; "
-                              "the quoted value is the back-to-back (warm) one"},
+                       "how": "median of 15 single products, each after a 1 GiB buffer sweep and a sync; the quoted value "
+                              "is the back-to-back (warm) one"},
         "rel_l2_vs_oracle": rel_l2,
+        "plan_create_ms": host_route["plan_create_ms"],
+        "matrix_to_first_y": route,
+        "plan_estimates_us": {"rows": info["est_rows_us"], "slices": info["est_slices_us"]},
         "csr_only_ms": csr_only and csr_only["ms_total"],
-        "best_hybrid": best_hybrid and {k: best_hybrid[k] for k in ("tau_c", "tau_r", "ms_total", "tile_nnz", "csr_nnz", "default_plan_keeps_tiles")},
-        "roofline": {"bound": "hbm", "kernel": dom["kernel"], "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK,
-                     "traffic": TRAFFIC.get((cfg, dom["kernel"], info["tile_nnz"] > 0)),
-                     "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"],
-                     **({"note": "the matrix has %d distinct values and the kernel reads one byte per entry for them: the "
-                                 "algorithmic bytes still count sizeof(valT) per entry, so frac can exceed 1; `traffic` is "
-                                 "what the kernel really moves" % info["csr_value_dict"]} if info["csr_value_dict"] else {})},
-        "sweep": [{k: r[k] for k in ("tau_c", "tau_r", "ms_total", "ms_tile", "ms_csr", "tile_nnz")} for r in table],
+        "best_hybrid": best_hybrid,
+        "roofline": roofline,
+        "sweep": table, "sweep_seconds": sweep_s,
     }
-    if cpu_baseline:
-        reps = []
-        runner = (lambda: ora.spmv_f64(A.val, A.rowPtr, A.colInd, x)) if A.dtype == mx.MX_F64 else \
-                 (lambda: ora.spmv_f16_f32acc(A.val, A.rowPtr, A.colInd, x))
-        # one thread on one core, as the reference's spmv_serial: pinned for the duration
-        affinity = os.sched_getaffinity(0)
-        pinned = None
-        try:
-            pinned = min(affinity)
-            os.sched_setaffinity(0, {pinned})
-        except OSError:
-            pinned = None
-        try:
-            for i in range(12):
-                t0 = time.perf_counter()
-                runner()
-                reps.append(time.perf_counter() - t0)
-        finally:
-            if pinned is not None:
-                os.sched_setaffinity(0, affinity)
-        t_cpu = min(reps[2:])
-        cpu_model = "unknown"
-        try:
-            with open("/proc/cpuinfo") as f:
-                cpu_model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "unknown")
-        except OSError:
-            pass
-        rec["cpu_baseline"] = {"value": 2.0 * A.nnz / t_cpu / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
-                               "cpu": cpu_model, "cpus_visible": len(os.sched_getaffinity(0)), "pinned_to_cpu": pinned,
-                               "sample": "the full matrix of this workload, best of 10 after 2 warm-ups "
-                                         "(%.1f ms per SpMV), single thread as the reference's spmv_serial" % (t_cpu * 1e3)}
-        # not the reference's: the same oracle routine over nnz-balanced row ranges, one thread per
-        # core (the C call releases the interpreter lock)
-        from concurrent.futures import ThreadPoolExecutor
-        ncore = max(1, min(16, len(os.sched_getaffinity(0))))
-        cuts = np.searchsorted(A.rowPtr, np.linspace(0, A.nnz, ncore + 1)).astype(int)
-        cuts[0], cuts[-1] = 0, A.rows
-        f16 = A.dtype != mx.MX_F64
-
-        def part_run(k):
-            r0, r1 = int(cuts[k]), int(cuts[k + 1])
-            if r1 > r0:
-                (ora.spmv_f16_f32acc if f16 else ora.spmv_f64)(A.val, A.rowPtr[r0:r1 + 1], A.colInd, x)
-        reps = []
-        with ThreadPoolExecutor(ncore) as ex:
-            for i in range(7):
-                t0 = time.perf_counter()
-                list(ex.map(part_run, range(ncore)))
-                reps.append(time.perf_counter() - t0)
-        t_all = min(reps[2:])
-        rec["cpu_all_cores"] = {"value": 2.0 * A.nnz / t_all / 1e9, "unit": "GFLOP/s", "cores": ncore, "kind": "port",
-                                "sample": "not the reference's (its CPU path is serial): the oracle routine on %d "
-                                          "nnz-balanced row ranges in parallel threads, best of 5 (%.2f ms)" % (ncore, t_all * 1e3)}
-        # the extraction itself (not part of `value`): host route against the device route, same partition
-        pt = (0.5, 0.25)
-        mx.Partition(A, *pt, device=True).close()  # first use of the device code
-        t0 = time.perf_counter()
-        ph = mx.Partition(A, *pt)
-        t1 = time.perf_counter()
-        pd = mx.Partition(A, *pt, device=True)
-        t2 = time.perf_counter()
-        rec["preprocess"] = {"tau_c": pt[0], "tau_r": pt[1], "host_ms": (t1 - t0) * 1e3, "device_route_ms": (t2 - t1) * 1e3,
-                             "same_partition": ph.hash == pd.hash,
-                             "note": "mx_partition_create on the host cores against mx_partition_create_device "
-                                     "(upload, extraction on the GPU, download)"}
-        ph.close()
-        pd.close()
     plan.close()
     part.close()
-    return rec
+    return rec, (A, x)
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", type=int, default=2, choices=sorted(WORKLOADS))
-    ap.add_argument("--all", action="store_true", help="also run workloads 3, 4, 5 (reported under 'others')")
+    ap.add_argument("--workload", type=int, nargs="+", default=None, choices=sorted(WORKLOADS),
+                    help="the first is the headline, the others go under 'others' (default: 5 2 3 4)")
     ap.add_argument("--no-sweep", action="store_true", help="tau=(0,0) only")
     ap.add_argument("--tau", type=float, nargs=2, metavar=("TAU_C", "TAU_R"), default=None,
                     help="no sweep: run this point (a profile of a fixed plan)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profile runs)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also launch one elementwise kernel that reads and writes MIB MiB (a known size to "
                          "scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -270,33 +308,39 @@ def main():
     if not torch.cuda.is_available() or mx.device_count() < 1:
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(1)
+    t_start = time.time()
+    traffic = read_traffic()
+    cfgs = args.workload or [5, 2, 3, 4]
 
-    main_rec = run_workload(mx, torch, ora, args.workload, args.steps, args.warmup, not args.no_sweep, True, args.tau)
+    def mode_of(cfg):
+        if args.no_sweep:
+            return "csr"
+        return "sweep" if cfg in SWEPT else "points"
+    main_rec, (A, x) = run_workload(mx, torch, ora, cfgs[0], args.steps, args.warmup, mode_of(cfgs[0]), traffic, args.tau)
     out = {
         "metric": METRIC, "value": main_rec["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_rec["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": main_rec["dtype"], "data": "synthetic",
         "config": {"workload": main_rec["workload"], "rows": main_rec["rows"], "nnz": main_rec["nnz"],
-                   "tau_c": main_rec["tau_c"], "tau_r": main_rec["tau_r"], "csr_variant": main_rec["csr_variant"],
-                   "tau_grid": "5x5 {0,.25,.5,.75,1}^2, tau_c>=tau_r, best of sweep" if args.tau is None and not args.no_sweep
-                   else "no sweep: point fixed on the command line"},
-        "roofline": main_rec["roofline"],
-        "cpu_baseline": main_rec.pop("cpu_baseline"),
-        "cpu_all_cores": main_rec.pop("cpu_all_cores"),
-        "preprocess": main_rec.pop("preprocess"),
-        "hbm_frac_whole_spmv": main_rec["hbm_frac_whole_spmv"],
-        "cold_cache": main_rec["cold_cache"],
-        "rel_l2_vs_oracle": main_rec["rel_l2_vs_oracle"],
-        "csr_only_ms": main_rec["csr_only_ms"],
-        "best_hybrid": main_rec["best_hybrid"],
-        "sweep": main_rec["sweep"],
+                   "tau_c": main_rec["tau_c"], "tau_r": main_rec["tau_r"], "plan": main_rec["plan"],
+                   "csr_variant": main_rec["csr_variant"],
+                   "tau_grid": "5x5 {0,.25,.5,.75,1}^2, tau_c>=tau_r, best of sweep" if mode_of(cfgs[0]) == "sweep" and args.tau is None
+                   else "no sweep: point(s) fixed"},
+        "roofline": main_rec.pop("roofline"),
     }
+    if not args.no_cpu:
+        out["cpu_baseline"], out["cpu_all_cores"] = cpu_baseline(mx, ora, A, x)
+    del A, x
+    for k in ("hbm_frac_whole_spmv", "cold_cache", "rel_l2_vs_oracle", "plan_create_ms", "matrix_to_first_y",
+              "plan_estimates_us", "csr_only_ms", "best_hybrid", "tile_nnz", "csr_nnz", "ms_per_step_events",
+              "algorithmic_bytes", "sweep", "sweep_seconds"):
+        out[k] = main_rec[k]
+
     # what a plain device copy reaches on this GPU, next to the 8 TB/s the roofline is priced at:
-    # read + written bytes over the time of back-to-back copies, at this workload's algorithmic
-    # size and at 1 GiB
+    # read + written bytes over the time of back-to-back copies, at 64 MB and at 1 GiB
     copy = {}
-    for label, nbytes in (("workload_sized", int(main_rec["roofline"]["bytes_per_launch"]) // 2), ("1GiB", 1 << 29)):
+    for label, nbytes in (("64MB", 32 << 20), ("1GiB", 1 << 29)):
         src = torch.ones(nbytes // 4, dtype=torch.float32, device="cuda:0")
         dst = torch.empty_like(src)
         for _ in range(5):
@@ -308,7 +352,7 @@ def main():
             dst.copy_(src)
         e1.record()
         torch.cuda.synchronize()
-        copy[label] = {"bytes_read_plus_written": 2 * (nbytes // 4) * 4, "GBs": 2 * (nbytes // 4) * 4 / (e0.elapsed_time(e1) / reps * 1e-3) / 1e9}
+        copy[label] = {"bytes_read_plus_written": 2 * nbytes, "GBs": 2 * nbytes / (e0.elapsed_time(e1) / reps * 1e-3) / 1e9}
         del src, dst
     out["device_copy"] = copy
     if args.calibrate_copy:
@@ -319,16 +363,14 @@ def main():
             torch.add(src, 1.0, out=dst)  # reads 4n bytes, writes 4n bytes
         torch.cuda.synchronize()
         out["calibrate_copy_bytes_each_way"] = 4 * n
-    if args.all:
-        others = {}
-        for cfg in (3, 4, 5):
-            if cfg == args.workload:
-                continue
-            r = run_workload(mx, torch, ora, cfg, max(200, args.steps // 4), args.warmup, not args.no_sweep, False)
-            others["workload_%d" % cfg] = {k: r[k] for k in (
-                "workload", "dtype", "rows", "nnz", "tau_c", "tau_r", "csr_variant", "ms_per_step", "gflops", "hbm_frac_whole_spmv",
-                "cold_cache", "rel_l2_vs_oracle", "csr_only_ms", "best_hybrid", "roofline")}
+        del src, dst
+    others = {}
+    for cfg in cfgs[1:]:
+        r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, mode_of(cfg), traffic, None)
+        others["workload_%d" % cfg] = r
+    if others:
         out["others"] = others
+    out["bench_seconds"] = time.time() - t_start
     print(json.dumps(out))
 
 

@@ -288,6 +288,21 @@ int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters,
  * without its combine kernel), same protocol as mx_time: the figure a roofline is priced on. */
 int mx_time_csr_main(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters, double *ms);
 
+/* Every kernel launch of one product, timed alone with the protocol of mx_time, in launch order,
+ * each with its share of the algorithmic bytes (the shares add up to mx_algorithmic_bytes of the
+ * matrix: entries go to the kernel that multiplies them, x to the first kernel that reads it, the
+ * row structure and y to the kernel that writes y).  The reference times its two kernels apart
+ * in the same way (test/test_autotc_spmv.cpp:1561-1572).  Up to `cap` records; *n_kernels = how many. */
+typedef struct mx_kernel_time {
+    char name[64];            /* e.g. "csr_slice_kernel<f16>", "slice_combine_kernel<f16,strips>" */
+    double ms;                /* mean per launch */
+    double algorithmic_bytes; /* this kernel's share */
+    int nnz;                  /* matrix entries this kernel multiplies */
+    int reserved;
+} mx_kernel_time;
+int mx_time_kernels(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters, mx_kernel_time *out, int cap,
+                    int *n_kernels);
+
 /* Choice of (tau_c, tau_r) for a matrix on this device.  The reference tunes the two fractions
  * per matrix by running its CLI once per candidate and reading "MatXtract time" back
  * (ML/bayes_opt.py:22-84: candidates with hot_frac > col_frac are rejected, :37-38); here the
@@ -330,9 +345,13 @@ typedef struct mx_plan_info {
                             run through tile_kernel */
     int tile_strip_nnz;  /* entries held by those chunks */
     int csr_value_dict;  /* > 0: the main kernel of the CSR part reads one byte per entry, an index into this many
-                            distinct values (matrices with at most 255 of them: stencils, graphs), because the
-                            plan found that faster; 0: values as they are.  MX_CSR_DICT=0 switches it off, =2
-                            takes it wherever it exists */
+                            distinct values (matrices with at most 255 of them: stencils, graphs); 0: values as
+                            they are.  MX_CSR_DICT=0 switches the form off */
+    double est_rows_us;  /* what the choice between row tiles and slices was made from: the estimated microseconds */
+    double est_slices_us;/* per product through either form, from counts over the matrix and rates measured on
+                            MI355X (both 0 when a flag, MX_CSR_KERNEL or the shape of the matrix left no choice).
+                            Nothing is timed unless MX_PLAN_AUTOTUNE=1 is set, so a matrix gets the same plan on
+                            every run */
 } mx_plan_info;
 int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
 
@@ -389,6 +408,9 @@ typedef struct mx_plan_layout_view {
     unsigned char *csrVal;
     unsigned char *stripRows; /* [rows] 1 = the row is written by the strip layout alone */
     mx_tile_layout_view tiles[2];
+    int csr_variant;     /* the form mx_plan_create would give the CSR part on a device with nCU compute units:
+                            0 row tiles, 1 slices, 2 split; -1 when MX_PLAN_AUTOTUNE=1 leaves it to a timed trial */
+    double est_rows_us, est_slices_us; /* the estimates behind that choice (mx_plan_info) */
 } mx_plan_layout_view;
 int mx_plan_layout(const mx_partition *P, int flags, int nCU, mx_plan_layout_view *out);
 void mx_plan_layout_free(mx_plan_layout_view *v);

@@ -52,7 +52,7 @@ class PlanInfo(C.Structure):
                 ("csr_nnz", C.c_int), ("csr_blocks", C.c_int), ("csr_variant", C.c_int),
                 ("tile_bytes", C.c_double), ("csr_bytes", C.c_double),
                 ("csr_main_kernel", C.c_int), ("csr_main_nnz", C.c_int), ("tile_variant", C.c_int), ("tile_strip_nnz", C.c_int),
-                ("csr_value_dict", C.c_int)]
+                ("csr_value_dict", C.c_int), ("est_rows_us", C.c_double), ("est_slices_us", C.c_double)]
 
 
 class SliceLayoutView(C.Structure):
@@ -72,7 +72,13 @@ class TileLayoutView(C.Structure):
 class PlanLayoutView(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("rows", "cols", "csr_nnz", "fragM", "fragK", "slots")] + \
                [(n, C.c_void_p) for n in ("csrRowPtr", "csrColInd", "csrVal", "stripRows")] + \
-               [("tiles", TileLayoutView * 2)]
+               [("tiles", TileLayoutView * 2), ("csr_variant", C.c_int), ("est_rows_us", C.c_double),
+                ("est_slices_us", C.c_double)]
+
+
+class KernelTime(C.Structure):
+    _fields_ = [("name", C.c_char * 64), ("ms", C.c_double), ("algorithmic_bytes", C.c_double), ("nnz", C.c_int),
+                ("reserved", C.c_int)]
 
 
 class TauPoint(C.Structure):
@@ -119,6 +125,7 @@ SIGNATURES = {
     "mx_spmv_repeat": (_i, [_vp, _vp, _vp, _i, _vp]),
     "mx_spmv_host": (_i, [_vp, _vp, _vp]),
     "mx_time": (_i, [_vp, _vp, _vp, _i, _i, _pd, _pd, _pd]),
+    "mx_time_kernels": (_i, [_vp, _vp, _vp, _i, _i, C.POINTER(KernelTime), _i, _pi]),
     "mx_time_csr_main": (_i, [_vp, _vp, _vp, _i, _i, _pd]),
     "mx_plan_get_info": (_i, [_vp, C.POINTER(PlanInfo)]),
     "mx_tune_tau": (_i, [C.POINTER(CsrStruct), _i, _i, _i, _i, C.POINTER(C.c_float), C.POINTER(C.c_float),

@@ -320,7 +320,8 @@ def plan_layout(part, flags=MX_PLAN_DEFAULT, nCU=256):
     check(_lib.load().mx_plan_layout(part._h, int(flags), int(nCU), C.byref(v)))
     try:
         vt = _np_dtype(part.dtype)
-        out = {n: int(getattr(v, n)) for n in ("rows", "cols", "csr_nnz", "fragM", "fragK", "slots")}
+        out = {n: int(getattr(v, n)) for n in ("rows", "cols", "csr_nnz", "fragM", "fragK", "slots", "csr_variant")}
+        out["est_rows_us"], out["est_slices_us"] = float(v.est_rows_us), float(v.est_slices_us)
         out["csrRowPtr"] = _view(v.csrRowPtr, v.rows + 1, np.int32).copy()
         out["csrColInd"] = _view(v.csrColInd, v.csr_nnz, np.int32).copy()
         out["csrVal"] = _view(v.csrVal, v.csr_nnz, vt).copy()
@@ -419,6 +420,17 @@ class Plan:
         check(_lib.load().mx_time(self._h, x.data_ptr(), y.data_ptr(), warm, iters, C.byref(t),
                                   C.byref(tt) if parts else None, C.byref(tc) if parts else None))
         return t.value, tt.value, tc.value
+
+    def time_kernels(self, x, y, warm=200, iters=4000):
+        """Every kernel launch of one product timed alone (mx_time_kernels) ->
+        [{"name", "ms", "algorithmic_bytes", "nnz"}, ...] in launch order."""
+        self._check_vec(x, self.cols, "x")
+        self._check_vec(y, self.rows, "y")
+        recs = (_lib.KernelTime * 8)()
+        n = C.c_int()
+        check(_lib.load().mx_time_kernels(self._h, x.data_ptr(), y.data_ptr(), warm, iters, recs, 8, C.byref(n)))
+        return [{"name": r.name.decode(), "ms": r.ms, "algorithmic_bytes": r.algorithmic_bytes, "nnz": r.nnz}
+                for r in recs[:n.value]]
 
     def time_csr_main(self, x, y, warm=200, iters=4000):
         """Mean ms per launch of the CSR part's main kernel alone."""

@@ -975,6 +975,7 @@ struct mx_plan {
     mx::DeviceSlices slices;  // CSR part (or its long rows), x-resident-in-LDS form (csr_slice_kernel)
     int csr_variant = 0;      // 0 = row tiles, 1 = slices, 2 = row tiles for the short rows, then slices for the long ones
     int csr_nnz = 0;
+    double est_rows_us = 0, est_slices_us = 0;  // what the choice of the form was made from (0: no choice was made)
     mx::DeviceTiles tiles;    // tile part, general form (tile_kernel)
     mx::DeviceTiles strips;   // tile part, binary16 strips on rows of their own (tile_dense_kernel)
     int tile_nnz = 0;
@@ -1069,13 +1070,131 @@ static int split_length()
     return v > 0 ? v : 32;
 }
 
+// What the choice between the forms of the CSR part looks at: all of it is counted from the
+// matrix, none of it is timed, so the same matrix gets the same plan on every run.
+struct CsrStats {
+    double linesPerGather = 0;  // mean number of distinct 64-byte lines of x that 64 consecutive entries name
+    double vrows = 0;           // virtual rows the slice layout would have (distinct slices per row, long ones cut)
+    bool fewValues = false;     // at most 255 distinct values: the one-byte-per-value forms exist
+};
+
+static CsrStats csr_stats(mx_dtype dtype, int rows, const int *rowPtr, const int *col, const void *val, int nCU)
+{
+    CsrStats st;
+    const int nnz = rowPtr[rows], es = mx::elem_size(dtype), perLine = 64 / es, SW = mx::slice_cols(dtype);
+    // (a mean: every stride-th window of 64 entries is enough, at most 65536 of them)
+    const long long windows = nnz / 64, stride = std::max<long long>(1, windows / 65536);
+    const long long sampled = windows / stride;
+    double lines = 0;
+#pragma omp parallel for schedule(static) reduction(+ : lines)
+    for (long long i = 0; i < sampled; ++i) {
+        const long long w = i * stride;
+        int l[64];
+        for (int k = 0; k < 64; ++k) l[k] = col[w * 64 + k] / perLine;
+        std::sort(l, l + 64);
+        int d = 1;
+        for (int k = 1; k < 64; ++k) d += l[k] != l[k - 1];
+        lines += d;
+    }
+    st.linesPerGather = sampled > 0 ? lines / (double)sampled : 1.0;
+    const long long fair = (long long)nnz / ((long long)std::max(nCU, 1) * mx::kSliceWaves * 64);
+    const int BE = mx::kSliceBatchEntries;
+    const int cap = (int)std::min<long long>(512, std::max<long long>(16, (fair + BE - 1) / BE * BE));
+    double vrows = 0;
+#pragma omp parallel for schedule(dynamic, 4096) reduction(+ : vrows)
+    for (int r = 0; r < rows; ++r) {
+        const int a = rowPtr[r], b = rowPtr[r + 1];
+        if (b <= a) continue;
+        // distinct slices of the row (its columns are ascending in all but hostile input, where this
+        // overcounts a little), and what the cap adds for a long run inside one slice
+        int n = 0, run = 0, last = -1;
+        for (int p = a; p < b; ++p) {
+            const int q = col[p] / SW;
+            if (q != last || run == cap) {
+                ++n;
+                run = 0;
+                last = q;
+            }
+            ++run;
+        }
+        vrows += n;
+    }
+    st.vrows = vrows;
+    const char *ed = std::getenv("MX_CSR_DICT");
+    if (nnz >= 65536 && !(ed && !std::atoi(ed))) {
+        std::vector<unsigned char> codes, dict;
+        int nd = 0;
+        st.fewValues = make_value_dict(es, val, nnz, codes, dict, &nd, 255);
+    }
+    return st;
+}
+
+// Estimated time of a product through the row-tile form and through the slice form, in
+// microseconds, from rates measured on MI355X (back-to-back products, five synthetic workloads at
+// three sizes each; the estimates are within 20 % of every one of them):
+//  * row tiles: one launch (2.5), then the entries at a cost that grows with the number of
+//    distinct lines of x a wave-wide gather names -- 1.4 + 0.05 * lines microseconds per million
+//    entries -- times up to 1.6 when x does not fit one L2 (4 MB) and the gathers are scattered,
+//    times 0.85 with one byte per value;
+//  * slices: two dependent launches and the copy of x into LDS (9.5), the stream of stored
+//    bytes (column offset 2 + value sizeof(valT) or 1, padded by about 8 %) at 9 bytes per ns
+//    while it stays inside the memory-side cache from one product to the next (up to 64 MB),
+//    5.8 beyond, and 2 microseconds per million virtual rows in the combine kernel.
+static void csr_estimates(mx_dtype dtype, int cols, int nnz, const CsrStats &st, double *usRows, double *usSlices)
+{
+    const double es = mx::elem_size(dtype), M = 1e-6 * (double)nnz;
+    double perM = 1.4 + 0.05 * st.linesPerGather;
+    // (scattered gathers that miss the L2: nothing for a stencil's dozen lines, all of it from two dozen on)
+    if ((double)cols * es > 4.0e6) perM *= 1.0 + 0.6 * std::min(1.0, std::max(0.0, (st.linesPerGather - 12.0) / 12.0));
+    if (st.fewValues) perM *= 0.85;
+    *usRows = 2.5 + M * perM;
+    const double bytes = (double)nnz * 1.08 * (2.0 + (st.fewValues ? 1.0 : es));
+    *usSlices = 9.5 + bytes / (bytes <= 64.0e6 ? 9.0e6 : 5.8e6) + 2.0e-6 * st.vrows;
+}
+
+// Which forms of the CSR part a plan may take (want[0] row tiles, [1] slices, [2] split) after the
+// caller's flags, MX_CSR_KERNEL and -- when both of the first two are still open and nothing is to be
+// timed -- the estimates.  S = slice_count() of the matrix.
+struct CsrChoice {
+    bool want[3] = {true, true, false};
+    double usRows = 0, usSlices = 0;  // the estimates, when they decided
+    bool fewValues = false;
+};
+static bool plan_autotune()
+{
+    static const bool on = std::getenv("MX_PLAN_AUTOTUNE") && std::atoi(std::getenv("MX_PLAN_AUTOTUNE"));
+    return on;
+}
+static CsrChoice choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val,
+                                 int flags, int nCU, int S)
+{
+    CsrChoice c;
+    const char *env = std::getenv("MX_CSR_KERNEL");
+    if (flags & MX_PLAN_CSR_ROWS) c.want[1] = c.want[2] = false;
+    if (flags & MX_PLAN_CSR_SLICES) c.want[0] = c.want[2] = false;
+    if (env && !std::strcmp(env, "rows")) c.want[0] = true, c.want[1] = c.want[2] = false;
+    if (env && !std::strcmp(env, "slices")) c.want[1] = true, c.want[0] = c.want[2] = false;
+    if (env && !std::strcmp(env, "split")) c.want[2] = true, c.want[0] = c.want[1] = false;
+    if (S == 0) c.want[1] = c.want[2] = false;
+    if (c.want[0] && c.want[1] && !plan_autotune()) {
+        const CsrStats st = csr_stats(dtype, rows, rowPtr, col, val, nCU);
+        csr_estimates(dtype, cols, rowPtr[rows], st, &c.usRows, &c.usSlices);
+        c.fewValues = st.fewValues;
+        c.want[c.usSlices < c.usRows ? 0 : 1] = false;
+    }
+    return c;
+}
+
 // Puts the CSR part on the device.  Three executable forms exist: row tiles with direct x
 // gathers; column slices with x resident in LDS; and a split in which the long rows (most of
 // the entries of a matrix with a heavy tail of row lengths) take the slices and the many short
-// ones the row tiles.  Unless a flag or MX_CSR_KERNEL=rows|slices|split forces one, the first
-// two are built in turn (the second when the matrix suits it) and timed on the spot with a few
-// launches, and the faster is kept.  The split runs only when asked for: it has not won on any
-// matrix measured so far and building it makes a plan half as slow again.
+// ones the row tiles.  Unless a flag or MX_CSR_KERNEL=rows|slices|split forces one, the choice
+// between the first two is made from counts over the matrix (csr_stats, csr_estimates): the form
+// with the lower estimate is built, and the one-byte-per-value form of it wherever the matrix has
+// at most 255 distinct values.  Nothing is timed, so a matrix gets the same plan on every run, with
+// or without a profiler attached.  MX_PLAN_AUTOTUNE=1 brings the timed choice back: both forms
+// (and both value forms) are built and run a few times on the spot and the fastest is kept.
+// The split runs only when asked for: it has not won on any matrix measured so far.
 // `stripRows` (optional): rows that the strip form of the tile kernel writes (and the CSR part has
 // nothing for).
 static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags,
@@ -1085,19 +1204,17 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
     const int nnz = rowPtr[rows];
     const size_t es = (size_t)mx::elem_size(plan->dtype);
     plan->csr_nnz = nnz;
-    const char *env = std::getenv("MX_CSR_KERNEL");
-    bool want[3] = {true, true, false};
-    if (flags & MX_PLAN_CSR_ROWS) want[1] = want[2] = false;
-    if (flags & MX_PLAN_CSR_SLICES) want[0] = want[2] = false;
-    if (env && !std::strcmp(env, "rows")) want[0] = true, want[1] = want[2] = false;
-    if (env && !std::strcmp(env, "slices")) want[1] = true, want[0] = want[2] = false;
-    if (env && !std::strcmp(env, "split")) want[2] = true, want[0] = want[1] = false;
     hipDeviceProp_t prop;
     int dev = 0;
     MX_HIP(hipGetDevice(&dev));
     MX_HIP(hipGetDeviceProperties(&prop, dev));
     const int nCU = std::max(1, prop.multiProcessorCount);
     const int S = slice_count(plan->dtype, rows, cols, nnz, nCU);
+    CsrChoice pick = choose_csr_form(plan->dtype, rows, cols, rowPtr, col, val, flags, nCU, S);
+    bool(&want)[3] = pick.want;
+    plan->est_rows_us = pick.usRows;
+    plan->est_slices_us = pick.usSlices;
+    const bool autotune = plan_autotune();
     // the split: rows of at least split_length() entries, when they hold a good part of the matrix
     std::vector<char> longRow;
     int longNnz = 0, longRows = 0;
@@ -1112,7 +1229,6 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
             }
         if (longNnz < 4096 || longRows == rows || (double)longNnz < 0.1 * (double)nnz) want[2] = false;
     }
-    if (S == 0) want[1] = want[2] = false;
     if (!want[0] && !want[1] && !want[2]) want[0] = true;  // a matrix the slice kernel cannot take runs on row tiles whatever was asked
     const int nWant = (int)want[0] + (int)want[1] + (int)want[2];
     int rc;
@@ -1156,7 +1272,12 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
         mx::DeviceSlices L;
         rc = build(v, C, L);
         double ms = 0.0;
-        const bool choice = nWant > 1 || (v == 0 && C.codes) || (v == 1 && L.ecode);
+        // (the one-byte-per-value form is taken wherever it exists; MX_CSR_DICT=0 keeps it from being built)
+        if (!rc && !autotune) {
+            if (v == 0 && C.codes) C.useDict = true;
+            if (v != 0 && L.ecode) L.useDict = true;
+        }
+        const bool choice = autotune && (nWant > 1 || (v == 0 && C.codes) || (v == 1 && L.ecode));
         if (!rc && choice) rc = scratch();
         if (!rc && choice) {
             std::swap(plan->csr, C);
@@ -1626,6 +1747,17 @@ extern "C" int mx_plan_layout(const mx_partition *P, int flags, int nCU, mx_plan
                 if (rc) return rc;
             }
         }
+        {
+            // the form of the CSR part a plan on a device with nCU compute units takes for it
+            const int *rp = P->extracted ? H.rowPtr.data() : P->cdRowPtr.data();
+            const int *ci = P->extracted ? H.col.data() : P->cdColInd.data();
+            const void *va = P->extracted ? (const void *)H.val.data() : P->cdVal.data();
+            const int S = slice_count(P->dtype, P->rows, P->cols, rp[P->rows], nCU);
+            const CsrChoice pick = choose_csr_form(P->dtype, P->rows, P->cols, rp, ci, va, flags, nCU, S);
+            out->csr_variant = pick.want[2] ? 2 : pick.want[0] && pick.want[1] ? -1 : pick.want[1] ? 1 : 0;
+            out->est_rows_us = pick.usRows;
+            out->est_slices_us = pick.usSlices;
+        }
         std::vector<unsigned char> sr((size_t)P->rows, 0);
         if (!H.stripRows.empty()) std::memcpy(sr.data(), H.stripRows.data(), sr.size());
         out->stripRows = give(sr.data(), sr.size());
@@ -1697,6 +1829,8 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     info->tile_strip_nnz = plan->strips.vals;
     info->csr_value_dict = plan->csr_variant == 1 ? (plan->slices.useDict ? plan->slices.nDict : 0)
                                                   : (plan->csr.useDict ? plan->csr.nDict : 0);
+    info->est_rows_us = plan->est_rows_us;
+    info->est_slices_us = plan->est_slices_us;
     return MX_OK;
 }
 
@@ -1844,6 +1978,81 @@ extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, 
     }
     // leave y holding the product
     rc = spmv_on(plan, x_dev, y_dev, s);
+    if (rc) return rc;
+    MX_HIP(hipStreamSynchronize(s));
+    return MX_OK;
+}
+
+// One record per kernel launch of a product, in launch order: its mean time alone (same protocol as
+// mx_time) and its share of the algorithmic bytes -- entries at sizeof(valT) + 4 each go to the
+// kernel that multiplies them, x to the first kernel that reads it, the row structure
+// ((rows + 1) * 4) and y to the kernel that writes y -- so that the shares add up to
+// mx_algorithmic_bytes of the whole matrix.
+extern "C" int mx_time_kernels(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters, mx_kernel_time *out,
+                               int cap, int *n_kernels)
+{
+    if (!plan || !x_dev || !y_dev || warm < 0 || iters <= 0 || !out || cap < 1 || !n_kernels) {
+        set_error("mx_time_kernels: bad argument");
+        return MX_ERR_ARG;
+    }
+    hipStream_t s = plan->stream;
+    const double es = mx::elem_size(plan->dtype);
+    const char *vt = plan->dtype == MX_F64 ? "f64" : "f16";
+    const double xBytes = (double)plan->cols * es, yBytes = ((double)plan->rows + 1) * 4 + (double)plan->rows * es;
+    static const bool apart = std::getenv("MX_STRIPS_APART") && std::atoi(std::getenv("MX_STRIPS_APART"));
+    const bool ride = !apart && plan->csr_variant == 1 && mx::strips_can_ride(plan->dtype, plan->strips, x_dev);
+    void *wide = plan->tiles.nWaves > 0 ? plan->ywide : nullptr;
+    int n = 0, rc = MX_OK;
+    auto add = [&](const std::string &name, double bytes, int nnz, auto body) {
+        if (rc || n >= cap) return;
+        mx_kernel_time &K = out[n];
+        std::memset(&K, 0, sizeof(K));
+        std::snprintf(K.name, sizeof(K.name), "%s", name.c_str());
+        K.algorithmic_bytes = bytes;
+        K.nnz = nnz;
+        rc = time_loop(plan, warm, iters, body, &K.ms);
+        ++n;
+    };
+    if (plan->csr_variant != 0 && ((uintptr_t)x_dev & 15)) {
+        set_error("mx_time_kernels: x must be 16-byte aligned for this plan");
+        return MX_ERR_ARG;
+    }
+    bool xCounted = false;
+    if (plan->csr_variant != 1 && plan->csr.nBlocks > 0) {
+        const bool last = plan->csr_variant == 0;  // writes y for good
+        add(std::string("csr_rows_kernel<") + vt + (plan->csr.useDict ? ",dict>" : ">"),
+            (double)plan->csr.nnz * (es + 4) + xBytes + (last ? yBytes : 0.0), plan->csr.nnz, [&]() -> int {
+                MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x_dev, y_dev, 0, s, wide));
+                return MX_OK;
+            });
+        xCounted = true;
+    }
+    if (plan->csr_variant != 0) {
+        add(std::string("csr_slice_kernel<") + vt + (plan->slices.useDict ? ",dict>" : ">"),
+            (double)plan->slices.nnz * (es + 4) + (xCounted ? 0.0 : xBytes), plan->slices.nnz, [&]() -> int {
+                MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x_dev, y_dev, 0, s, 1));
+                return MX_OK;
+            });
+        const int stripNnz = ride ? plan->strips.vals : 0;
+        add(std::string("slice_combine_kernel<") + vt + (ride ? ",strips>" : ">"), (double)stripNnz * (es + 4) + yBytes, stripNnz,
+            [&]() -> int {
+                MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x_dev, y_dev, 0, s, 2, ride ? &plan->strips : nullptr, wide));
+                return MX_OK;
+            });
+    }
+    if (plan->tiles.nWaves > 0)
+        add(std::string("tile_kernel<") + vt + ">", (double)plan->tiles.vals * (es + 4), plan->tiles.vals, [&]() -> int {
+            MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x_dev, y_dev, 1, s, wide));
+            return MX_OK;
+        });
+    if (!ride && plan->strips.nWaves > 0)
+        add("tile_dense_kernel<f16>", (double)plan->strips.vals * (es + 4), plan->strips.vals, [&]() -> int {
+            MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x_dev, y_dev, 1, s));
+            return MX_OK;
+        });
+    if (rc) return rc;
+    *n_kernels = n;
+    rc = spmv_on(plan, x_dev, y_dev, s);  // leave y holding the product
     if (rc) return rc;
     MX_HIP(hipStreamSynchronize(s));
     return MX_OK;
