@@ -156,9 +156,11 @@ int mx_select_device(int rows, int cols, int nnz, const int *rowPtr_dev, const i
  *           of the column among the unselected, ascending), then, for a row that was not selected,
  *           its entries in selected columns (cdRowPtr_dev[rows + 1], cdColInd_dev / cdVal_dev[nnz - nnzRowD]).
  * Entries that name the same row and column twice keep their source order.  The arrays equal
- * mx_partition_create's ddRowPtr .. cdVal.  The caller sizes the outputs from `sel`; a selection that
- * does not belong to the matrix is reported (MX_ERR_ARG) when its totals differ, but its index arrays
- * are trusted.  Scratch (about 28 bytes per entry) is allocated and released inside. */
+ * mx_partition_create's ddRowPtr .. cdVal.  The caller sizes the outputs from `sel`.  Everything
+ * that is used as an address is looked at first: a rowPtr that does not rise from 0 to nnz, a
+ * column id outside [0, cols), an entry of descColId[0, dCols) outside [0, cols) or of
+ * descRowId[0, dRows) outside [0, rows), and a selection whose totals differ from the matrix's
+ * are refused with MX_ERR_ARG.  Scratch (about 28 bytes per entry) is allocated and released inside. */
 int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
                     const void *val_dev, const mx_selection *sel, const int *descColId_dev, const int *descRowId_dev,
                     int *ddRowPtr_dev, int *ddColInd_dev, void *ddVal_dev, int *cdRowPtr_dev, int *cdColInd_dev,
@@ -171,8 +173,9 @@ int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowP
  * zeros to whole fragments of fragK = 4 (binary64) or 8 (binary16) columns); per fragment a
  * bitmap with bit r * fragK + c for an entry in local row r and compacted column c; tcVal in
  * ascending bit order, of entries naming the same place the last.  The arrays equal
- * mx_partition_create's.  The library allocates them in one block (device memory) and fills
- * in `out`; mx_tiles_device_free releases the block. */
+ * mx_partition_create's.  A ddRowPtr that does not rise from 0 to nnzRowD or a column id outside
+ * [0, dCols) is refused with MX_ERR_ARG before it is used.  The library allocates the outputs in
+ * one block (device memory) and fills in `out`; mx_tiles_device_free releases the block. */
 typedef struct mx_device_tiles {
     int chunkNum, totalTcFrags, fragK, tcValCount;
     int *chunkPtr;          /* [chunkNum + 1] */

@@ -429,7 +429,7 @@ extern "C" int mx_partition_get(const mx_partition *p, mx_partition_view *v)
 extern "C" uint64_t mx_partition_hash(const mx_partition *p)
 {
     if (!p) return 0;
-    uint64_t h = 1469598103934665603ull;
+    uint64_t h = 14695981039346656037ull;
     const int es = mx::elem_size(p->dtype);
     h = fnv(&p->dCols, 4, h);
     h = fnv(&p->dRows, 4, h);

@@ -103,6 +103,24 @@ __global__ __launch_bounds__(kBlock) void index_histogram_kernel(const int *__re
     else atomicAdd(&cnt[c], 1);
 }
 
+// bad |= bit where v[i] lies outside [0, lim): the index arrays of a caller are looked at before a
+// kernel uses them as addresses.
+__global__ __launch_bounds__(kBlock) void range_check_kernel(const int *__restrict__ v, int n, int lim, int bit,
+                                                             int *__restrict__ bad)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < n && (unsigned)v[i] >= (unsigned)lim) atomicOr(bad, bit);
+}
+// bad |= bit unless ptr[0] == 0, ptr[n] == total and ptr never falls.
+__global__ __launch_bounds__(kBlock) void pointer_check_kernel(const int *__restrict__ ptr, int n, int total, int bit,
+                                                               int *__restrict__ bad)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i > n) return;
+    const int p = ptr[i];
+    if ((i == 0 && p != 0) || (i == n && p != total) || (i < n && ptr[i + 1] < p) || p < 0 || p > total) atomicOr(bad, bit);
+}
+
 __global__ __launch_bounds__(kBlock) void iota_kernel(int *__restrict__ v, int n)
 {
     const int i = blockIdx.x * kBlock + threadIdx.x;
@@ -573,7 +591,28 @@ extern "C" int mx_split_device(mx_dtype dtype, int rows, int cols, int nnz, cons
     int *payIn = (int *)b, *payOut = (int *)(b + payB);
     b += 2 * payB;
     void *sortTmp = b, *scanTmp = b + sortBytes;
+    int *bad = (int *)((unsigned char *)sortTmp + sortBytes + scanBytes);  // in the 256 spare bytes at the end
     auto grid = [](long long n) { return dim3((unsigned)((n + kBlock - 1) / kBlock)); };
+
+    // the caller's arrays become addresses below: row pointers, column ids and both orders are
+    // looked at first (1 = rowPtr, 2 = colInd, 4 = descColId, 8 = descRowId)
+    MXP_TRY(hipMemsetAsync(bad, 0, sizeof(int), s));
+    hipLaunchKernelGGL(pointer_check_kernel, grid((long long)rows + 1), dim3(kBlock), 0, s, rowPtr_dev, rows, nnz, 1, bad);
+    if (nnz > 0) hipLaunchKernelGGL(range_check_kernel, grid(nnz), dim3(kBlock), 0, s, colInd_dev, nnz, cols, 2, bad);
+    if (dCols > 0) hipLaunchKernelGGL(range_check_kernel, grid(dCols), dim3(kBlock), 0, s, descColId_dev, dCols, cols, 4, bad);
+    if (dRows > 0) hipLaunchKernelGGL(range_check_kernel, grid(dRows), dim3(kBlock), 0, s, descRowId_dev, dRows, rows, 8, bad);
+    MXP_TRY(hipGetLastError());
+    {
+        int badHost = 0;
+        MXP_TRY(hipMemcpyAsync(&badHost, bad, sizeof(int), hipMemcpyDeviceToHost, s));
+        MXP_TRY(hipStreamSynchronize(s));
+        if (badHost) {
+            mx::set_error(std::string("mx_split_device: ") + ((badHost & 1) ? "rowPtr does not rise from 0 to nnz" :
+                          (badHost & 2) ? "column index out of range" : (badHost & 4) ? "descColId entry out of range" :
+                          "descRowId entry out of range"));
+            return MX_ERR_ARG;
+        }
+    }
 
     // new column ids: rank for a selected column, dCols + position among the others otherwise
     MXP_TRY(hipMemsetAsync(dense, 0, denseB, s));
@@ -686,6 +725,22 @@ extern "C" int mx_tiles_device(mx_dtype dtype, int dRows, int dCols, int nnzRowD
     int *frags = (int *)b, *chunkPtrTmp = (int *)(b + chB);
     b += 2 * chB;
     void *sortTmp = b, *scanTmp = b + sortBytes;
+    {
+        // the caller's A_dd is about to be used for addressing: pointers and column ids are looked at first
+        int *bad = (int *)((unsigned char *)sortTmp + sortBytes + scanBytes);  // in the 256 spare bytes at the end
+        MXP_TRY(hipMemsetAsync(bad, 0, sizeof(int), s));
+        hipLaunchKernelGGL(pointer_check_kernel, grid((long long)dRows + 1), dim3(kBlock), 0, s, ddRowPtr_dev, dRows, n, 1, bad);
+        if (n > 0) hipLaunchKernelGGL(range_check_kernel, grid(n), dim3(kBlock), 0, s, ddColInd_dev, n, dCols, 2, bad);
+        MXP_TRY(hipGetLastError());
+        int badHost = 0;
+        MXP_TRY(hipMemcpyAsync(&badHost, bad, sizeof(int), hipMemcpyDeviceToHost, s));
+        MXP_TRY(hipStreamSynchronize(s));
+        if (badHost) {
+            mx::set_error((badHost & 1) ? "mx_tiles_device: ddRowPtr does not rise from 0 to nnzRowD"
+                                        : "mx_tiles_device: column index out of range");
+            return MX_ERR_ARG;
+        }
+    }
 
     // distinct columns per chunk: sort by (chunk, column), mark first occurrences, count them
     if (n > 0) {

@@ -687,7 +687,7 @@ void ora_hybrid_f16(const ora_partition *P, const uint16_t *x, float *y)
 uint64_t ora_hash(const void *p, size_t n, uint64_t h)
 {
     const unsigned char *b = (const unsigned char *)p;
-    if (h == 0) h = 1469598103934665603ull;
+    if (h == 0) h = 14695981039346656037ull;
     for (size_t i = 0; i < n; ++i) {
         h ^= b[i];
         h *= 1099511628211ull;

@@ -983,6 +983,33 @@ def test_device_selection_and_split_equal_the_host_partition(mx, ora):
             P.close()
     with pytest.raises(mx.MxError):  # tau_c < tau_r
         mx.select_device(rp, ci, A.cols, 0.25, 0.5)
+    # arrays that would be used as addresses are looked at first: an index out of range is refused
+    # by the split and by the tile encoding, not followed
+    A = mx.gen_config(2, scale=1 / 64)[0]
+    rp, ci, va = torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda()
+    dc, dr, sel = mx.select_device(rp, ci, A.cols, 0.5, 0.25)
+    for what in ("colInd", "descColId", "descRowId", "rowPtr"):
+        rp2, ci2, dc2, dr2 = rp.clone(), ci.clone(), dc.clone(), dr.clone()
+        if what == "colInd":
+            ci2[7] = A.cols + 5
+        elif what == "descColId":
+            dc2[0] = -3
+        elif what == "descRowId":
+            dr2[sel["dRows"] - 1] = A.rows
+        else:
+            rp2[3] = rp2[4] + 1
+        with pytest.raises(mx.MxError) as e:
+            mx.split_device(rp2, ci2, va, A.cols, sel, dc2, dr2)
+        assert e.value.code == 1, what
+    got = mx.split_device(rp, ci, va, A.cols, sel, dc, dr)
+    bad_col = got[1].clone()
+    bad_col[0] = sel["dCols"]
+    with pytest.raises(mx.MxError):
+        mx.tiles_device(got[0], bad_col, got[2], sel["dCols"])
+    bad_ptr = got[0].clone()
+    bad_ptr[-1] += 1
+    with pytest.raises(mx.MxError):
+        mx.tiles_device(bad_ptr, got[1], got[2], sel["dCols"])
 
 
 @pytest.mark.gpu

@@ -308,3 +308,41 @@ def test_hybrid_equals_plain_spmv(ora, tau):
     y = P.hybrid(x)
     ref = A @ x
     assert np.linalg.norm(y - ref) <= 1e-13 * np.linalg.norm(ref)
+
+
+def test_eqcheck_binary16(ora):
+    """ora_eqcheck_f16 (the reference's FP16 eQcheck, test/test_autotc_spmv.cpp:276-292: values
+    widened to float, relative to the larger magnitude, 0/0 passes) against a numpy restatement on
+    hand-picked pairs."""
+    a = np.array([0.0, 1.0, 1.0, -2.0, 100.0, 1e-4, 0.5, 65504.0, 6e-8], np.float16)
+    b = np.array([0.0, 1.0, 1.125, -2.25, 89.0, 1.2e-4, -0.5, 60000.0, 0.0], np.float16)
+    af, bf = a.astype(np.float32), b.astype(np.float32)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        rel = np.abs(af - bf) / np.maximum(np.abs(af), np.abs(bf))
+    for tol in (1e-1, 0.12, 1e-3, 0.5, 2.5):
+        bad = np.nonzero(rel > np.float32(tol))[0]  # NaN (0/0) compares false: passes
+        assert ora.eqcheck(a, b, tol) == (int(bad[0]) if len(bad) else -1), tol
+    assert ora.eqcheck(a, a.copy(), 1e-1) == -1
+    # known answers: |1 - 1.125| / 1.125 = 1/9 is the first failure at 0.1; 11/100 passes 0.12, 0.2/1.2 does not; a sign flip is 2
+    assert ora.eqcheck(a, b, 1e-1) == 2 and ora.eqcheck(a, b, 0.12) == 5 and ora.eqcheck(a, b, 0.5) == 6
+    assert ora.eqcheck(a[:2], b[:2], 0.0) == -1
+
+
+def test_hash_is_fnv1a_64(ora, mx):
+    """ora_hash against the published FNV-1a 64-bit test vectors, chained calls against one call,
+    and the library's mx_partition_hash (same function over the canonical arrays in the
+    documented order)."""
+    vec = {b"": 0xcbf29ce484222325, b"a": 0xaf63dc4c8601ec8c, b"b": 0xaf63df4c8601f1a5, b"foobar": 0x85944171f73967e8,
+           b"chongo was here!\n": 0x46810940eff5f915}
+    for s, h in vec.items():
+        assert ora.hash_arrays(np.frombuffer(s, np.uint8)) == h, s
+    parts = [np.frombuffer(b"foo", np.uint8), np.frombuffer(b"bar", np.uint8)]
+    assert ora.hash_arrays(*parts) == vec[b"foobar"]
+    A, _ = mx.gen_config(2, scale=1 / 64)
+    for tau in ((0.5, 0.25), (1.0, 1.0)):
+        P = mx.Partition(A, *tau)
+        Q = ora.partition(A.rowPtr, A.colInd, A.val, A.cols, *tau)
+        arrays = [np.array([Q.dCols], np.int32), np.array([Q.dRows], np.int32), Q.descColId[:Q.dCols], Q.newArray, Q.rId,
+                  Q.newArray_, Q.chunkPtr, Q.sparse_AToX_index, Q.fragPtr, Q.fragBit, Q.tcVal, Q.cdRowPtr, Q.cdColInd, Q.cdVal]
+        assert ora.hash_arrays(*arrays) == P.hash
+        P.close()
