@@ -407,6 +407,16 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
                         if (haveDict) ecode[atc] = codeOfEntry[p];
                         std::memcpy(&ev[atv * es], sv + (size_t)p * es, es);
                     }
+                    // the padding up to the chunk's longest member multiplies zero with the x of the
+                    // virtual row's own last column: a non-finite x then reaches the rows that name its
+                    // column, as in a plain CSR product, and no others
+                    if (v.len > 0) {
+                        const unsigned short lastCol = (unsigned short)(col[ord[v.start + v.len - 1]] - q * SW);
+                        for (int n = v.len; n < ch[c].steps * E; ++n) {
+                            const size_t st = (size_t)step + n, batch = st / BE, k = st % BE;
+                            ecol[(batch * 64 + l) * BE + k] = lastCol;
+                        }
+                    }
                 }
                 step += ch[c].steps;
                 rel += ch[c].steps;

@@ -521,6 +521,46 @@ def test_slice_kernel_virtual_rows(mx, ora, variant, monkeypatch):
         part.close()
 
 
+def test_a_non_finite_x_reaches_only_the_rows_that_name_its_column(mx, ora):
+    """Inf and NaN in x, at the first column of a slice among others (where the padding of the
+    sliced layout once pointed): y is non-finite exactly on the rows that have an entry in such
+    a column, as in a plain CSR product, in every form of the CSR part and in both precisions."""
+    import torch
+    rng = np.random.default_rng(21)
+    for vt, cols in ((np.float64, 40000), (np.float16, 150000)):
+        rows = 3000
+        lens = rng.integers(1, 40, rows)
+        lens[::97] = 300   # a few long rows, so that chunks are padded to very different lengths
+        ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        ci = np.concatenate([np.sort(rng.choice(cols, n, replace=False)) for n in lens]).astype(np.int32)
+        A = mx.Csr(rows, cols, ptr, ci, rng.uniform(0.5, 1.0, ptr[-1]).astype(vt))
+        x = rng.uniform(0.5, 1.0, cols).astype(vt)
+        sw = 16384 if vt == np.float64 else 65536
+        hot = [0, sw, 2 * sw, 7, cols - 1]
+        x[hot[0]] = np.inf
+        x[hot[1]] = np.nan
+        x[hot[2]] = -np.inf
+        x[hot[3]] = np.nan
+        x[hot[4]] = np.inf
+        touched = np.zeros(rows, bool)
+        for r in range(rows):
+            touched[r] = np.isin(ci[ptr[r]:ptr[r + 1]], hot).any()
+        assert 0 < touched.sum() < rows // 4
+        ref = oracle_y(ora, mx, A, x).astype(np.float64)
+        assert np.array_equal(~np.isfinite(ref), touched)
+        xd = torch.from_numpy(x).cuda()
+        part = mx.Partition(A, 0.0, 0.0)
+        for fl in (mx.MX_PLAN_CSR_SLICES, mx.MX_PLAN_CSR_ROWS):
+            plan = mx.Plan(part, fl)
+            assert plan.info["csr_variant"] == (1 if fl == mx.MX_PLAN_CSR_SLICES else 0)
+            y = plan.spmv(xd).cpu().numpy().astype(np.float64)
+            assert np.array_equal(~np.isfinite(y), touched), (vt, fl, int((~np.isfinite(y)).sum()), int(touched.sum()))
+            ok = ~touched
+            assert rel_l2(y[ok], ref[ok]) <= (F64_TOL if vt == np.float64 else F16_TOL)
+            plan.close()
+        part.close()
+
+
 def test_tile_kernel_step_packing(mx, ora):
     """Chunks with one fragment, with exactly half a step, a whole step, more than a step and a
     ragged last chunk; every fill from almost empty to full, through the fragment gate and
