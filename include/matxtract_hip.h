@@ -345,7 +345,13 @@ typedef struct mx_plan_info {
                             groups rows with the same blocks, 8 at a time, into chunks of its own (at least 4
                             rows each) and takes them out of the reference's fragments.  MX_NO_STRIPS=1 in the
                             environment switches this off; with an x that is not 16-byte aligned these chunks
-                            run through tile_kernel */
+                            run through tile_kernel.
+                            2: a binary64 plan whose tiles are aligned blocks of 8 x 8 (eight consecutive rows
+                            from a multiple of eight, eight consecutive columns from a multiple of eight, in the
+                            caller's numbering, at least three quarters full) found in the extracted block and
+                            run through v_mfma_f64_16x16x4_f64 with x read in aligned 16-byte pieces; their rows
+                            keep their other entries in the CSR part, and with the slice form of that part the
+                            blocks ride in the combine kernel's launch (MX_NO_BLOCKS=1 switches the form off) */
     int tile_strip_nnz;  /* entries held by those chunks */
     int csr_value_dict;  /* > 0: the main kernel of the CSR part reads one byte per entry, an index into this many
                             distinct values (matrices with at most 255 of them: stencils, graphs); 0: values as
@@ -391,7 +397,8 @@ void mx_slice_layout_free(mx_slice_layout_view *v);
  * test/test_autotc_spmv.cpp:1486-1559): the CSR part in the caller's numbering (the residual plus
  * every entry of the extracted block that the tile kernels do not take; for a partition with
  * tau = (0,0) the matrix itself), and up to two tile layouts as the kernels read them -- [0] for
- * tile_kernel, [1] the strip chunks for tile_dense_kernel.  Per step: hdr[32] ints (output rows
+ * tile_kernel, [1] the plan's own chunks of 8-column blocks (binary16 strips for tile_dense_kernel,
+ * binary64 8 x 8 blocks for tile_block_wave: four block slots per half, slot 4h+i, blocks 8 x 8).  Per step: hdr[32] ints (output rows
  * [0,16) of the two halves, -1 = none; [16] flags: 1 = the sums are stored after this step, 2 = the
  * halves belong to two chunks; [17],[18] blocks in half 0 and 1; [21,29) first column per slot in
  * the strip layout), atox[64] column ids (slot-major, -1 = unused; block i of half h sits in
@@ -409,7 +416,8 @@ typedef struct mx_plan_layout_view {
     int rows, cols, csr_nnz, fragM, fragK, slots; /* slots: block slots of a step (two halves of slots/2) */
     int *csrRowPtr, *csrColInd;
     unsigned char *csrVal;
-    unsigned char *stripRows; /* [rows] 1 = the row is written by the strip layout alone */
+    unsigned char *stripRows; /* [rows] 1 = the row is written by the strip layout alone (binary16); 2 = the row's sums from
+                                 the CSR part and from the 8 x 8 blocks of tiles[1] are added (binary64) */
     mx_tile_layout_view tiles[2];
     int csr_variant;     /* the form mx_plan_create would give the CSR part on a device with nCU compute units:
                             0 row tiles, 1 slices, 2 split; -1 when MX_PLAN_AUTOTUNE=1 leaves it to a timed trial */

@@ -63,6 +63,10 @@ struct DeviceTiles {
                                // columns are consecutive from a multiple of eight and every chunk fits one step
                                // (two share a step when both fit a half): tile_dense_kernel can run it
     bool ownedRows = false;    // set by the plan: no row of these tiles gets anything from the CSR part
+    // binary64 `dense` layouts (blocks of 8 x 8 on rows that the CSR part shares) when they ride in the
+    // combine kernel's launch: per step 128 indices into the slice layout's sums -- half h, row i,
+    // place j at [64h + 8i + j], -1 = none -- set on the step after which the half's sums are stored
+    int *vidx = nullptr;
     int *waveDesc = nullptr;   // [nWaves][8]
     int *hdr = nullptr;        // [steps][kTileHdr]
     int *atox = nullptr;       // [steps][64]

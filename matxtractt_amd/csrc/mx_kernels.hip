@@ -922,6 +922,122 @@ __global__ __launch_bounds__(kBlock) void tile_dense_kernel(const int4 *__restri
     if (gw < nWaves) tile_dense_wave(waveDesc, hdr, tcVal, x, y, gw, lane);
 }
 
+// The binary64 counterpart: aligned blocks of 8 x 8 (eight consecutive columns from a multiple of
+// eight, on eight consecutive rows) that the plan finds in the extracted block -- the dense
+// blocks of a block-structured matrix -- on rows that also have other entries.  Same step stream
+// as the strips (two halves of up to four blocks, headers with the first column of every block
+// slot, blocks stored whole and row-major, waves over whole chunks, four steps prefetched), with
+// eight v_mfma_f64_16x16x4_f64 per step: MFMA 2p and 2p+1 take block p of both halves, the first
+// the even columns of the block (k-th A column = block column 2k), the second the odd ones, so that
+// a lane's two A values (row m%8, columns 2k and 2k+1) and its two B values (x[first + 2k],
+// x[first + 2k + 1]) are each one aligned 16-byte load.  No column ids, nothing through LDS.
+// The rows get the rest of their sum from the CSR part.  RIDE: the wave runs inside the combine
+// kernel's launch and fetches the sums of the rows' virtual rows itself (vidx: per step and half,
+// eight places per row, -1 = none), so that y is written once, here, and the combine kernel's own
+// kinds leave these rows alone.  Otherwise y holds the CSR part's sum already and is added to.
+// Waves are many and short -- the host gives each one step, more only to a chunk of more than
+// eight blocks -- and keep nothing in flight beyond the step at hand: a step is two dependent
+// rounds of loads (header, values and places; then x and the sums the places name), and what
+// hides them is the number of waves a CU holds, so the wave is written for few registers.
+template <bool RIDE>
+__device__ __forceinline__ void tile_block_wave(const int4 *__restrict__ waveDesc, const int *__restrict__ hdr,
+                                                const int *__restrict__ vidx, const double *__restrict__ tcVal,
+                                                const double *__restrict__ x, const double *__restrict__ partial,
+                                                double *__restrict__ y, int gw, int lane)
+{
+    const int4 d0 = waveDesc[2 * gw], d1 = waveDesc[2 * gw + 1];
+    const int s0 = __builtin_amdgcn_readfirstlane(d0.x), s1 = __builtin_amdgcn_readfirstlane(d0.y);
+    if (s0 >= s1) return;
+    const int m = lane & 15, k = lane >> 4, h = m >> 3;
+    // where the values of the next four steps start and how many blocks their first halves hold:
+    // from the wave's descriptor at first, then from the header of the step four back
+    int vo0 = __builtin_amdgcn_readfirstlane(d0.z), vo1 = __builtin_amdgcn_readfirstlane(d0.w);
+    int vo2 = __builtin_amdgcn_readfirstlane(d1.x), vo3 = __builtin_amdgcn_readfirstlane(d1.y);
+    const int na4 = __builtin_amdgcn_readfirstlane(d1.z);
+    int na0 = na4 & 255, na1 = (na4 >> 8) & 255, na2 = (na4 >> 16) & 255, na3 = (na4 >> 24) & 255;
+    v4f64 acc = {0.0, 0.0, 0.0, 0.0};
+    for (int s = s0; s < s1; ++s) {
+        // round one: header, the lane's A operands (block q of its half, row m%8, columns 2k and 2k+1:
+        // a lane whose block is absent reads what follows the step's values and ignores it) and places
+        const int hd = hdr[(size_t)s * kTileHdr + (lane & 31)];
+        const double *p = tcVal + vo0 + (size_t)(h ? na0 : 0) * 64 + (m & 7) * 8 + 2 * k;
+        v2f64 v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = __builtin_nontemporal_load((const v2f64 *)(p + q * 64));
+        int vi0 = -1, vi1 = -1;
+        if constexpr (RIDE) {
+            vi0 = vidx[(size_t)s * 128 + lane];
+            vi1 = vidx[(size_t)s * 128 + 64 + lane];
+        }
+        // round two: the B operands (lanes 0 and 1 of each 16: the x of block q of half 0 / half 1, one
+        // aligned 16-byte read) and the other part of the rows' sums
+        v2f64 bx[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int base = __shfl(hd, 21 + 4 * (m & 1) + q);
+            bx[q] = *(const v2f64 *)(x + max(base, 0) + 2 * k);
+        }
+        double ps0, ps1;
+        if constexpr (RIDE) {
+            const double a = partial[max(vi0, 0)], b = partial[max(vi1, 0)];
+            ps0 = vi0 >= 0 ? a : 0.0;
+            ps1 = vi1 >= 0 ? b : 0.0;
+        } else {
+            const int r0 = __shfl(hd, lane >> 3), r1 = __shfl(hd, 8 + (lane >> 3));
+            const double a = y[max(r0, 0)], b = y[max(r1, 0)];
+            ps0 = ((lane & 7) == 0 && r0 >= 0) ? a : 0.0;
+            ps1 = ((lane & 7) == 0 && r1 >= 0) ? b : 0.0;
+        }
+        const int n0 = __builtin_amdgcn_readlane(hd, 17), n1 = __builtin_amdgcn_readlane(hd, 18);
+        const int na = h ? n1 : n0, nb = m ? n1 : n0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const double a0 = q < na ? v[q].x : 0.0, a1 = q < na ? v[q].y : 0.0;
+            const double b0 = (m < 2 && q < nb) ? bx[q].x : 0.0, b1 = (m < 2 && q < nb) ? bx[q].y : 0.0;
+            acc = tile_mma(a0, b0, acc);
+            acc = tile_mma(a1, b1, acc);
+        }
+        const int flags = __builtin_amdgcn_readlane(hd, 16);
+        if (flags & 1) {
+            // the other part of every row's sum: eight places per row, summed inside groups of 8 lanes
+            const double c0 = group_sum<8>(ps0), c1 = group_sum<8>(ps1);
+            // D[j][0] and D[4+j][0] are registers 0 and 1 of lane 16j; D[8+j][1] and D[12+j][1] are
+            // registers 2 and 3 of lane 16j+1.  A chunk that fills both halves has its rows in the
+            // first only: lane 16j adds what lane 16j+1 holds.
+            const double u2 = __shfl(acc[2], (lane + 1) & 63), u3 = __shfl(acc[3], (lane + 1) & 63);
+            // row j's other part sits in lanes 8j..8j+7, row 4+j's in lanes 32+8j..: lanes 16j and 16j+1 both want lane>>1
+            const double t0 = __shfl(c0, lane >> 1), t1 = __shfl(c0, (lane >> 1) + 32);
+            const double w0 = __shfl(c1, lane >> 1), w1 = __shfl(c1, (lane >> 1) + 32);
+            const int ra = __shfl(hd, k), rb = __shfl(hd, 4 + k), rc = __shfl(hd, 8 + k), rd = __shfl(hd, 12 + k);
+            if (m == 0) {
+                const double e0 = (flags & 2) ? 0.0 : u2, e1 = (flags & 2) ? 0.0 : u3;
+                if (ra >= 0) y[ra] = acc[0] + e0 + t0;
+                if (rb >= 0) y[rb] = acc[1] + e1 + t1;
+            }
+            if (m == 1 && (flags & 2)) {
+                if (rc >= 0) y[rc] = acc[2] + w0;
+                if (rd >= 0) y[rd] = acc[3] + w1;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = 0.0;
+        }
+        // the ring moves on: step s leaves, step s+4 comes in from the header of step s
+        vo0 = vo1, vo1 = vo2, vo2 = vo3, na0 = na1, na1 = na2, na2 = na3;
+        vo3 = __builtin_amdgcn_readlane(hd, 19);
+        na3 = __builtin_amdgcn_readlane(hd, 20);
+    }
+}
+
+// The blocks in a launch of their own, after the CSR part: y is added to.
+__global__ __launch_bounds__(kBlock) void tile_block_kernel(const int4 *__restrict__ waveDesc, const int *__restrict__ hdr,
+                                                           const double *__restrict__ tcVal, const double *__restrict__ x,
+                                                           double *__restrict__ y, int nWaves)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gw = xcd_contiguous_block(blockIdx.x, gridDim.x) * (kBlock / 64) + wave;
+    if (gw < nWaves) tile_block_wave<false>(waveDesc, hdr, nullptr, tcVal, x, nullptr, y, gw, lane);
+}
+
 // The sums of the virtual rows become y in one launch of three kinds of workgroups:
 //  * the first `nRowWG` walk the matrix rows, kCombineRows per lane: rowInfo[r] >= 0 names the one virtual
 //    row of row r, whose sum is the row's result; -1 is a row without entries (zero, or left
@@ -943,7 +1059,8 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
                                                               const int4 *__restrict__ stripWaveDesc,
                                                               const int *__restrict__ stripHdr,
                                                               const VT *__restrict__ stripVal, const VT *__restrict__ x,
-                                                              int nStripWaves, int nStripWG, int nHeavyWG, int lightQuads)
+                                                              int nStripWaves, int nStripWG, int nHeavyWG, int lightQuads,
+                                                              const int *__restrict__ stripVidx)
 {
     typedef typename Acc<VT>::type AT;
     const int tid = threadIdx.x;
@@ -956,6 +1073,14 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
         if constexpr (STRIPS && sizeof(VT) == 2) {
             const int gw = xcd_contiguous_block(blockIdx.x, nStripWG) * (kBlock / 64) + (tid >> 6);
             if (gw < nStripWaves) tile_dense_wave(stripWaveDesc, stripHdr, stripVal, x, y, gw, tid & 63);
+        }
+        // binary64: the 8 x 8 blocks, whose waves also fetch the sums of their rows' virtual rows
+        // (those rows are marked -2 in rowInfo and appear in none of the lists below)
+        if constexpr (STRIPS && sizeof(VT) == 8) {
+            const int gw = xcd_contiguous_block(blockIdx.x, nStripWG) * (kBlock / 64) + (tid >> 6);
+            if (gw < nStripWaves)
+                tile_block_wave<true>(stripWaveDesc, stripHdr, stripVidx, (const double *)stripVal, (const double *)x,
+                                      (const double *)partial, (double *)y, gw, tid & 63);
         }
         return;
     }
@@ -1167,7 +1292,7 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     const int nHeavyWG = (P.nHeavy + mxk::kBlock / 16 - 1) / (mxk::kBlock / 16);
     // strips that ride along (binary16 only; the caller has checked that they may: dense form,
     // rows of their own, x aligned)
-    const bool ride = strips && sizeof(VT) == 2 && strips->nWaves > 0;
+    const bool ride = strips && strips->nWaves > 0 && (sizeof(VT) == 2 || strips->vidx);
     const int nStripWG = ride ? (strips->nWaves + 3) / 4 : 0;
     if (nStripWG + nRowWG + nLightWG + nHeavyWG == 0) return hipSuccess;
 #define MX_LAUNCH_COMBINE(STRIPS)                                                                                          \
@@ -1176,7 +1301,7 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
                        (const int4 *)P.lightIdx, P.nLight, nLightWG, (const int4 *)P.heavyInfo, P.nHeavy, P.segIdx, (VT *)y,    \
                        (accumulate || P.subset) ? 1 : 0, P.subset ? 1 : 0, (AT *)ywide, ride ? (const int4 *)strips->waveDesc : nullptr,   \
                        ride ? strips->hdr : nullptr, ride ? (const VT *)strips->tcVal : nullptr, (const VT *)x,              \
-                       ride ? strips->nWaves : 0, nStripWG, nHeavyWG, P.lightQuads)
+                       ride ? strips->nWaves : 0, nStripWG, nHeavyWG, P.lightQuads, ride ? strips->vidx : nullptr)
     if (ride) MX_LAUNCH_COMBINE(true);
     else MX_LAUNCH_COMBINE(false);
 #undef MX_LAUNCH_COMBINE
@@ -1186,7 +1311,7 @@ hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, v
                          int what, const DeviceTiles *strips, void *ywide)
 {
     if (P.rows <= 0) return hipSuccess;
-    if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s, what, nullptr, ywide);
+    if (dtype == MX_F64) return launch_slices_t<double>(P, x, y, accumulate, s, what, strips, ywide);
     return launch_slices_t<_Float16>(P, x, y, accumulate, s, what, strips, ywide);
 }
 bool strips_can_ride(mx_dtype dtype, const DeviceTiles &T, const void *x)
@@ -1204,6 +1329,13 @@ hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, voi
     if (dtype == MX_F16 && T.dense && (!accumulate || T.ownedRows) && !((uintptr_t)x & 15)) {
         hipLaunchKernelGGL(mxk::tile_dense_kernel, dim3(grid), dim3(mxk::kBlock), 0, s, (const int4 *)T.waveDesc, T.hdr,
                            (const _Float16 *)T.tcVal, (const _Float16 *)x, (_Float16 *)y, T.nWaves);
+        return hipGetLastError();
+    }
+    if (dtype == MX_F64 && T.dense) {
+        // the 8 x 8 blocks in a launch of their own: they add to the y the CSR part has written
+        if (!accumulate || ((uintptr_t)x & 15)) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(mxk::tile_block_kernel, dim3(grid), dim3(mxk::kBlock), 0, s, (const int4 *)T.waveDesc, T.hdr,
+                           (const double *)T.tcVal, (const double *)x, (double *)y, T.nWaves);
         return hipGetLastError();
     }
     if (dtype == MX_F64)

@@ -93,6 +93,7 @@ void free_tiles(mx::DeviceTiles &T)
     (void)hipFree(T.hdr);
     (void)hipFree(T.atox);
     (void)hipFree(T.tcVal);
+    (void)hipFree(T.vidx);
     T = mx::DeviceTiles();
 }
 
@@ -181,8 +182,10 @@ struct HostSlices {
     int nDict = 0;
 };
 
-// `elsewhere` (optional) marks rows whose result another kernel writes (the strips of a binary16
-// plan): rowInfo -2, so that the combine kernel neither zeroes nor adds to them.
+// `elsewhere` (optional) marks rows whose result another kernel writes: 1 = the strips of a binary16
+// plan (the row has nothing here), 2 = the 8 x 8 blocks of a binary64 plan, whose waves fetch the sums
+// of the row's virtual rows themselves.  Such rows get rowInfo -2 and appear in no list, so that the
+// combine kernel's own kinds neither zero them nor add to them.
 int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
                  const char *sel, HostSlices &D, const char *elsewhere = nullptr)
 {
@@ -430,8 +433,10 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     std::vector<int> rowInfo(((size_t)rows + 3) / 4 * 4 + 4, -2), lightInfo, heavyInfo;
     for (int r = 0; r < rows; ++r) {
         const int a = segPtr[r], n = segPtr[r + 1] - a;
-        rowInfo[r] = n == 0 ? ((elsewhere && elsewhere[r]) ? -2 : -1) : n == 1 ? segIdx[a] : -2;
-        if (n > 1) {
+        // (elsewhere 2: the row's sums are fetched by the block layout of a binary64 plan, which writes its y)
+        const bool fetched = elsewhere && elsewhere[r] == 2;
+        rowInfo[r] = fetched ? -2 : n == 0 ? ((elsewhere && elsewhere[r]) ? -2 : -1) : n == 1 ? segIdx[a] : -2;
+        if (n > 1 && !fetched) {
             std::vector<int> &L = n > mx::kSliceLightSegs ? heavyInfo : lightInfo;
             L.insert(L.end(), {r, a, n, 0});
         }
@@ -466,12 +471,18 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     return MX_OK;
 }
 
+// `segOut` (optional): receives segPtr and segIdx (the virtual rows of every matrix row).
 int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
-                  const char *sel, mx::DeviceSlices &D, const char *elsewhere = nullptr)
+                  const char *sel, mx::DeviceSlices &D, const char *elsewhere = nullptr,
+                  std::pair<std::vector<int>, std::vector<int>> *segOut = nullptr)
 {
     HostSlices H;
     int rc = build_slices(dtype, rows, cols, rowPtr, col, val, nCU, S, sel, H, elsewhere);
     if (rc) return rc;
+    if (segOut) {
+        segOut->first = H.segPtr;
+        segOut->second = H.segIdx;
+    }
     D.nWG = H.nWG;
     D.S = H.S;
     D.rows = H.rows;
@@ -555,9 +566,13 @@ int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, co
                 const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap, int nCU,
                 HostTiles &T, const char *rowTaken = nullptr, const std::vector<StripChunk> *stripChunks = nullptr)
 {
-    const int es = mx::elem_size(dtype), fragK = mx::frag_k(dtype), fragM = mx::kFragM;
-    const int SF = mx::tile_slots(dtype), HF = SF / 2, H = mx::kTileHdr, BS = fragM * fragK;  // BS: values per block
+    const int es = mx::elem_size(dtype), fragM = mx::kFragM;
+    // (the plan's own chunks -- binary16 strips, binary64 blocks -- are made of blocks of 8 columns, four
+    // to a half, in both precisions; the reference's fragments are fragK wide)
+    const int fragK = stripChunks ? 8 : mx::frag_k(dtype);
+    const int SF = stripChunks ? 8 : mx::tile_slots(dtype), HF = SF / 2, H = mx::kTileHdr, BS = fragM * fragK;  // BS: values per block
     const bool f64 = dtype == MX_F64;
+    auto slot_of = [&](int half, int i) { return stripChunks ? 4 * half + i : mx::tile_slot(dtype, half, i); };
     const uint32_t *bit32 = (const uint32_t *)fragBit;
     const uint64_t *bit64 = (const uint64_t *)fragBit;
     const unsigned char *tv = (const unsigned char *)tcVal;
@@ -635,7 +650,7 @@ int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, co
         dVal.insert(dVal.end(), B.vals.begin(), B.vals.end());
         voff += BS;
         for (int c = 0; c < fragK; ++c) dAtox[s * 64 + (size_t)slot * fragK + c] = B.cols[c];
-        if (!f64) hdr[s * H + 21 + slot] = B.cols[0];
+        if (SF == 8) hdr[s * H + 21 + slot] = B.cols[0];
     };
     // a step with the blocks a0[0..n0) (half 0) and a1[0..n1) (half 1) of two chunks, given by
     // their fragM output rows r0 and r1 (r1 null: none; with flags & 2 clear both halves are r0's)
@@ -656,8 +671,8 @@ int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, co
         hdr[s * H + 17] = n0;
         hdr[s * H + 18] = n1;
         for (int i = 21; i < 29; ++i) hdr[s * H + i] = -1;
-        for (int i = 0; i < n0; ++i) put_block(s, mx::tile_slot(dtype, 0, i), a0[i]);
-        for (int i = 0; i < n1; ++i) put_block(s, mx::tile_slot(dtype, 1, i), a1[i]);
+        for (int i = 0; i < n0; ++i) put_block(s, slot_of(0, i), a0[i]);
+        for (int i = 0; i < n1; ++i) put_block(s, slot_of(1, i), a1[i]);
     };
     std::vector<int> fsel;
     std::vector<Block> pending;
@@ -730,7 +745,9 @@ int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, co
     // at once (24 per CU), so that none has to wait for a second round
     nCU = std::max(1, nCU);
     const int tper = std::getenv("MX_TILE_PER") ? std::atoi(std::getenv("MX_TILE_PER")) : 0;
-    const int per = tper > 0 ? tper : std::max(2, (steps + nCU * 24 - 1) / (nCU * 24));
+    // (binary64 block waves keep two steps in registers and live on the number of waves: a step each)
+    const int perMin = (stripChunks && f64) ? 1 : 2;
+    const int per = tper > 0 ? tper : std::max(perMin, (steps + nCU * 24 - 1) / (nCU * 24));
     std::vector<int> waveDesc;
     for (int s0 = 0; s0 < steps;) {
         int s1 = std::min(steps, s0 + per);
@@ -761,7 +778,7 @@ int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, co
 int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, const int *chunkPtr, const int *fragPtr,
                  const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap,
                  mx::DeviceTiles &T, int *tile_nnz, const char *rowTaken = nullptr,
-                 const std::vector<StripChunk> *stripChunks = nullptr)
+                 const std::vector<StripChunk> *stripChunks = nullptr, std::vector<int> *hdrOut = nullptr)
 {
     int nCU = 256;
     {
@@ -782,6 +799,7 @@ int upload_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, c
     T.dense = H.dense;
     T.nWaves = H.nWaves;
     if (tile_nnz) *tile_nnz = H.vals;
+    if (hdrOut) *hdrOut = H.hdr;
     if (H.steps == 0) return MX_OK;
     if ((rc = upload(&T.waveDesc, H.waveDesc.data(), H.waveDesc.size(), 64))) return rc;
     if ((rc = upload(&T.hdr, H.hdr.data(), H.hdr.size(), 256))) return rc;
@@ -1115,17 +1133,39 @@ static CsrStats csr_stats(mx_dtype dtype, int rows, const int *rowPtr, const int
     for (int r = 0; r < rows; ++r) {
         const int a = rowPtr[r], b = rowPtr[r + 1];
         if (b <= a) continue;
-        // distinct slices of the row (its columns are ascending in all but hostile input, where this
-        // overcounts a little), and what the cap adds for a long run inside one slice
+        // distinct slices of the row, and what the cap adds for a long run inside one slice (rows come
+        // sorted by column from most callers; the residual of an extracted partition does not)
         int n = 0, run = 0, last = -1;
-        for (int p = a; p < b; ++p) {
+        bool ascending = true;
+        for (int p = a; p < b && ascending; ++p) {
             const int q = col[p] / SW;
+            ascending = q >= last;
             if (q != last || run == cap) {
                 ++n;
                 run = 0;
                 last = q;
             }
             ++run;
+        }
+        if (!ascending) {
+            int local[64];
+            std::vector<int> big;
+            int *sl = local;
+            if (b - a > 64) {
+                big.resize((size_t)(b - a));
+                sl = big.data();
+            }
+            for (int p = a; p < b; ++p) sl[p - a] = col[p] / SW;
+            std::sort(sl, sl + (b - a));
+            n = 0, run = 0, last = -1;
+            for (int p = 0; p < b - a; ++p) {
+                if (sl[p] != last || run == cap) {
+                    ++n;
+                    run = 0;
+                    last = sl[p];
+                }
+                ++run;
+            }
         }
         vrows += n;
     }
@@ -1143,7 +1183,7 @@ static CsrStats csr_stats(mx_dtype dtype, int rows, const int *rowPtr, const int
 // microseconds, from rates measured on MI355X (back-to-back products, five synthetic workloads at
 // three sizes each; the estimates are within 20 % of every one of them):
 //  * row tiles: one launch (2.5), then the entries at a cost that grows with the number of
-//    distinct lines of x a wave-wide gather names -- 1.4 + 0.05 * lines microseconds per million
+//    distinct lines of x a wave-wide gather names -- 1.2 + 0.065 * lines microseconds per million
 //    entries -- times up to 1.6 when x does not fit one L2 (4 MB) and the gathers are scattered,
 //    times 0.85 with one byte per value;
 //  * slices: two dependent launches and the copy of x into LDS (9.5), the stream of stored
@@ -1153,7 +1193,7 @@ static CsrStats csr_stats(mx_dtype dtype, int rows, const int *rowPtr, const int
 static void csr_estimates(mx_dtype dtype, int cols, int nnz, const CsrStats &st, double *usRows, double *usSlices)
 {
     const double es = mx::elem_size(dtype), M = 1e-6 * (double)nnz;
-    double perM = 1.4 + 0.05 * st.linesPerGather;
+    double perM = 1.2 + 0.065 * st.linesPerGather;
     // (scattered gathers that miss the L2: nothing for a stencil's dozen lines, all of it from two dozen on)
     if ((double)cols * es > 4.0e6) perM *= 1.0 + 0.6 * std::min(1.0, std::max(0.0, (st.linesPerGather - 12.0) / 12.0));
     if (st.fewValues) perM *= 0.85;
@@ -1207,8 +1247,10 @@ static CsrChoice choose_csr_form(mx_dtype dtype, int rows, int cols, const int *
 // The split runs only when asked for: it has not won on any matrix measured so far.
 // `stripRows` (optional): rows that the strip form of the tile kernel writes (and the CSR part has
 // nothing for).
+// `segOut` (optional): receives the virtual rows of every matrix row when the slice form is taken.
 static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags,
-                          const char *stripRows = nullptr)
+                          const char *stripRows = nullptr,
+                          std::pair<std::vector<int>, std::vector<int>> *segOut = nullptr)
 {
     const int rows = plan->rows, cols = plan->cols;
     const int nnz = rowPtr[rows];
@@ -1255,7 +1297,7 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
     };
     auto build = [&](int v, mx::DeviceCsr &C, mx::DeviceSlices &L) -> int {
         if (v == 0) return upload_csr(plan->dtype, rows, cols, nnz, rowPtr, col, val, C, nullptr);
-        if (v == 1) return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, nullptr, L, stripRows);
+        if (v == 1) return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, nullptr, L, stripRows, segOut);
         // the short rows as a CSR matrix of their own (the long rows empty), the long ones as slices
         std::vector<int> rp((size_t)rows + 1, 0);
         for (int r = 0; r < rows; ++r) rp[r + 1] = rp[r] + (longRow[r] ? 0 : rowPtr[r + 1] - rowPtr[r]);
@@ -1271,7 +1313,10 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
         }
         int r1 = upload_csr(plan->dtype, rows, cols, rp[rows], rp.data(), c2.data(), v2.data(), C, nullptr);
         if (r1) return r1;
-        return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, longRow.data(), L, stripRows);
+        // (binary64 blocks do not ride with the split form: their rows stay with the combine kernel's own
+        // kinds and the blocks add to y afterwards)
+        return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, longRow.data(), L,
+                             plan->dtype == MX_F64 ? nullptr : stripRows);
     };
     double best = 0.0;
     bool have = false;
@@ -1362,13 +1407,14 @@ struct PhaseLog {
 // `stripRows` = the same rows in the caller's numbering), and the CSR part -- the residual plus
 // every entry of A_dd that the tiles leave -- in the caller's numbering.
 struct HostPlanParts {
-    std::vector<char> sel, taken, stripRows;
+    std::vector<char> sel, taken, stripRows;  // stripRows: 1 = written by the strips alone, 2 = shared with binary64 blocks
+    std::vector<char> inBlock;                // binary64: A_dd entries that went into 8 x 8 blocks
     std::vector<StripChunk> stripChunks;
     std::vector<int> rowPtr, col;
     std::vector<unsigned char> val;
 };
 
-static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, PhaseLog &phase)
+static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, PhaseLog &phase, bool noBlocks = false)
 {
     const int es = mx::elem_size(P->dtype), fragK = P->fragK, fragM = P->fragM;
     const int rows = P->rows, cols = P->cols;
@@ -1470,6 +1516,91 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
         }
         if (stripChunks.empty()) taken.clear();
     }
+    // binary64: aligned 8 x 8 blocks (eight consecutive rows from a multiple of eight, eight consecutive
+    // columns from a multiple of eight, both in the caller's numbering) that the extracted block fills
+    // at least three quarters -- the dense blocks of a block-structured matrix.  Their entries leave the
+    // CSR part (and the reference's fragments, which are not used beside them: the general tile kernel
+    // is bound by instruction issue and has not paid on any matrix measured); each row of eight rows with
+    // such blocks becomes one chunk for tile_block_wave.  A column named twice keeps its last value in
+    // the block; the earlier ones stay in the CSR part, so that y is the sum of all of them.
+    std::vector<char> &inBlock = H.inBlock;
+    inBlock.clear();
+    const char *envNoBlocks = std::getenv("MX_NO_BLOCKS");
+    if (P->dtype == MX_F64 && !noBlocks && !(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES)) &&
+        !(envNoBlocks && std::atoi(envNoBlocks)) && P->dRows > 0) {
+        const int need = 48;  // of 64
+        std::vector<int> ddRowOf((size_t)rows, -1);
+        for (int i = 0; i < P->dRows; ++i) ddRowOf[P->rId[i]] = i;
+        const int nbr = (rows + 7) / 8;
+        std::vector<std::vector<int>> blocksOf((size_t)nbr);  // block columns taken, ascending, per block row
+#pragma omp parallel
+        {
+            std::vector<int> bc;
+#pragma omp for schedule(dynamic, 64)
+            for (int br = 0; br < nbr; ++br) {
+                bc.clear();
+                for (int r = 8 * br; r < std::min(rows, 8 * br + 8); ++r) {
+                    const int i = ddRowOf[r];
+                    if (i < 0) continue;
+                    for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
+                        if (p + 1 < P->ddRowPtr[i + 1] && P->ddColInd[p + 1] == P->ddColInd[p]) continue;  // an earlier twin
+                        bc.push_back(P->descColId[P->ddColInd[p]] / 8);
+                    }
+                }
+                if ((int)bc.size() < need) continue;
+                std::sort(bc.begin(), bc.end());
+                for (size_t a = 0; a < bc.size();) {
+                    size_t b = a;
+                    while (b < bc.size() && bc[b] == bc[a]) ++b;
+                    if ((int)(b - a) >= need && (bc[a] + 1) * 8 <= cols) blocksOf[br].push_back(bc[a]);
+                    a = b;
+                }
+            }
+        }
+        size_t nChunks = 0;
+        for (int br = 0; br < nbr; ++br) nChunks += !blocksOf[br].empty();
+        if (nChunks > 0) {
+            inBlock.assign((size_t)P->ddRowPtr[P->dRows], 0);
+            H.stripRows.assign((size_t)rows, 0);
+            std::vector<int> chunkOf((size_t)nbr, -1);
+            for (int br = 0; br < nbr; ++br)
+                if (!blocksOf[br].empty()) {
+                    chunkOf[br] = (int)stripChunks.size();
+                    stripChunks.emplace_back();
+                }
+            const double *ddv = (const double *)P->ddVal.data();
+#pragma omp parallel for schedule(dynamic, 64)
+            for (int br = 0; br < nbr; ++br) {
+                if (chunkOf[br] < 0) continue;
+                const std::vector<int> &bcs = blocksOf[br];
+                StripChunk &C = stripChunks[chunkOf[br]];
+                C.nnz = 0;
+                C.blocks.resize(bcs.size());
+                for (size_t b = 0; b < bcs.size(); ++b) {
+                    C.blocks[b].vals.assign((size_t)64 * es, 0);
+                    for (int c = 0; c < 8; ++c) C.blocks[b].cols[c] = bcs[b] * 8 + c;
+                }
+                for (int j = 0; j < 8; ++j) {
+                    const int r = 8 * br + j;
+                    C.rows[j] = r < rows ? r : -1;
+                    if (r >= rows) continue;
+                    H.stripRows[r] = 2;
+                    const int i = ddRowOf[r];
+                    if (i < 0) continue;
+                    for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
+                        if (p + 1 < P->ddRowPtr[i + 1] && P->ddColInd[p + 1] == P->ddColInd[p]) continue;
+                        const int c = P->descColId[P->ddColInd[p]];
+                        const auto it = std::lower_bound(bcs.begin(), bcs.end(), c / 8);
+                        if (it == bcs.end() || *it != c / 8) continue;
+                        ((double *)C.blocks[it - bcs.begin()].vals.data())[j * 8 + c % 8] = ddv[p];
+                        inBlock[p] = 1;
+                        ++C.nnz;
+                    }
+                }
+            }
+            std::fill(sel.begin(), sel.end(), 0);
+        }
+    }
     phase("fragment gate, strip rows");
     if (!taken.empty()) {
         // the gate again, on what the taken rows leave of each fragment
@@ -1516,7 +1647,7 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
             stripEntries += C.nnz;
             stripBlocks += (double)C.blocks.size();
         }
-        const double blockBytes = (double)fragM * fragK * es, slots = mx::tile_slots(P->dtype);
+        const double blockBytes = (double)fragM * (inBlock.empty() ? fragK : 8) * es, slots = mx::tile_slots(P->dtype);
         const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
         const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
         const double launchNs = 5000.0, stripLaunchNs = 1000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
@@ -1527,6 +1658,8 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
             std::fill(sel.begin(), sel.end(), 0);
             stripChunks.clear();
             taken.clear();
+            inBlock.clear();
+            H.stripRows.clear();
         } else if (generalFrags > 0 && generalEntries * (es + 2) / fastRate <= launchNs + generalBytes / generalRate) {
             std::fill(sel.begin(), sel.end(), 0);  // the strips pay, the general tiles do not
         }
@@ -1563,7 +1696,7 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
             // (generateFormat_opt overwrites, test/test_autotc_spmv.cpp:718-847); the
             // earlier ones go to the CSR part, so that y is the sum of all of them.
             const bool earlierTwin = p + 1 < P->ddRowPtr[i + 1] && P->ddColInd[p + 1] == c;
-            keep[p] = rowTaken ? 0 : (earlierTwin || !sel[f0 + rank / fragK]);
+            keep[p] = rowTaken ? 0 : (!inBlock.empty() && inBlock[p]) ? 0 : (earlierTwin || !sel[f0 + rank / fragK]);
             n += keep[p];
         }
         rowPtr[P->rId[i] + 1] += n;
@@ -1596,7 +1729,7 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
         }
     }
     std::vector<char> &stripRows = H.stripRows;
-    stripRows.clear();
+    if (inBlock.empty()) stripRows.clear();
     if (!taken.empty()) {
         stripRows.assign((size_t)rows, 0);
         for (int i = 0; i < P->dRows; ++i)
@@ -1605,7 +1738,15 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
     return MX_OK;
 }
 
+static int create_plan(const mx_partition *P, int flags, mx_plan **out, bool noBlocks);
 extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
+{
+    return create_plan(P, flags, out, false);
+}
+
+// `noBlocks`: a binary64 plan without the 8 x 8 block form (the second attempt, when a row of a block
+// chunk turned out to have more virtual rows than the block layout has places for).
+static int create_plan(const mx_partition *P, int flags, mx_plan **out, bool noBlocks)
 {
     if (!P || !out) {
         set_error("mx_plan_create: null argument");
@@ -1649,7 +1790,7 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             phase("CSR part (layouts, trial)");
         } else {
             HostPlanParts H;
-            rc = plan_host_parts(P, flags, H, phase);
+            rc = plan_host_parts(P, flags, H, phase, noBlocks);
             if (rc) return fail(rc);
             const int chunkNum = P->chunkNum;
             std::vector<char> &sel = H.sel, &taken = H.taken, &stripRows = H.stripRows;
@@ -1657,7 +1798,10 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
             std::vector<int> &rowPtr = H.rowPtr, &col = H.col;
             std::vector<unsigned char> &val = H.val;
             phase("CSR part assembled");
-            rc = setup_csr_part(plan, rowPtr.data(), col.data(), val.data(), flags, stripRows.empty() ? nullptr : stripRows.data());
+            const bool blocks64 = P->dtype == MX_F64 && !stripChunks.empty();
+            std::pair<std::vector<int>, std::vector<int>> seg;  // virtual rows of every row (slice form)
+            rc = setup_csr_part(plan, rowPtr.data(), col.data(), val.data(), flags, stripRows.empty() ? nullptr : stripRows.data(),
+                                blocks64 ? &seg : nullptr);
             if (rc) return fail(rc);
             phase("CSR part (layouts, trial)");
 
@@ -1669,13 +1813,40 @@ extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
                               plan->tiles, &nnzGeneral, taken.empty() ? nullptr : taken.data());
             if (rc) return fail(rc);
             if (!stripChunks.empty()) {
+                std::vector<int> stepHdr;  // the layout's headers, for the places of the virtual-row sums
                 rc = upload_tiles(P->dtype, chunkNum, sel.data(), P->dRows, P->chunkPtr.data(), P->fragPtr.data(), bits,
                                   P->tcVal.data(), P->sparse_AToX_index.data(), P->descColId.data(), P->rId.data(),
-                                  plan->strips, &nnzStrips, nullptr, &stripChunks);
+                                  plan->strips, &nnzStrips, nullptr, &stripChunks, blocks64 ? &stepHdr : nullptr);
                 if (rc) return fail(rc);
-                // strip rows have nothing in the residual and left the fragments: the CSR part,
-                // which runs first, writes zeros there and the strip kernel may overwrite
-                plan->strips.ownedRows = true;
+                if (!blocks64) {
+                    // strip rows have nothing in the residual and left the fragments: the CSR part,
+                    // which runs first, writes zeros there and the strip kernel may overwrite
+                    plan->strips.ownedRows = true;
+                } else if (plan->csr_variant == 1) {
+                    // the blocks ride in the combine kernel's launch: where each of their rows finds the
+                    // sums of its virtual rows (eight places per row; a row with more sends the whole plan
+                    // back to be made without blocks)
+                    const int steps = plan->strips.steps;
+                    std::vector<int> vidx((size_t)steps * 128, -1);
+                    bool fits = true;
+                    for (int st = 0; st < steps && fits; ++st) {
+                        const int *h = &stepHdr[(size_t)st * mx::kTileHdr];
+                        if (!(h[16] & 1)) continue;
+                        for (int half = 0; half < 2; ++half)
+                            for (int i = 0; i < 8; ++i) {
+                                const int r = h[half * 8 + i];
+                                if (r < 0) continue;
+                                const int a = seg.first[r], n = seg.first[r + 1] - a;
+                                if (n > 8) fits = false;
+                                for (int j = 0; j < std::min(n, 8); ++j) vidx[(size_t)st * 128 + half * 64 + i * 8 + j] = seg.second[a + j];
+                            }
+                    }
+                    if (!fits) {
+                        mx_plan_destroy(plan);
+                        return create_plan(P, flags, out, true);
+                    }
+                    if ((rc = upload(&plan->strips.vidx, vidx.data(), vidx.size(), 128))) return fail(rc);
+                }
             }
             plan->tile_nnz = nnzGeneral + nnzStrips;
             if (P->dtype == MX_F16 && plan->tiles.nWaves > 0) {
@@ -1830,12 +2001,12 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
                             (double)plan->tiles.frags * fragK * es + (double)plan->tiles.chunkNum * 8 * 2 * es;
     if (plan->strips.steps)  // no column ids, no old y
         info->tile_bytes += (double)plan->strips.steps * (mx::kTileHdr * 4.0) + (double)plan->strips.stored * es +
-                            (double)plan->strips.frags * fragK * es + (double)plan->strips.chunkNum * 8 * es;
+                            (double)plan->strips.frags * 8 * es + (double)plan->strips.chunkNum * 8 * es;
     (void)bitBytes;
     const bool sliceMain = plan->csr_variant == 1 || (plan->csr_variant == 2 && plan->slices.nnz > plan->csr.nnz);
     info->csr_main_kernel = sliceMain ? 1 : 0;
     info->csr_main_nnz = plan->csr_variant == 2 ? (sliceMain ? plan->slices.nnz : plan->csr.nnz) : plan->csr_nnz;
-    info->tile_variant = plan->strips.steps > 0 ? 1 : 0;
+    info->tile_variant = plan->strips.steps > 0 ? (plan->dtype == MX_F64 ? 2 : 1) : 0;
     info->tile_strip_nnz = plan->strips.vals;
     info->csr_value_dict = plan->csr_variant == 1 ? (plan->slices.useDict ? plan->slices.nDict : 0)
                                                   : (plan->csr.useDict ? plan->csr.nDict : 0);
@@ -1849,7 +2020,8 @@ static int spmv_on(mx_plan *plan, const void *x, void *y, hipStream_t s, void *p
     // the strips ride in the launch of the combine kernel when the CSR part has one (MX_STRIPS_APART=1:
     // a launch of their own, as with the row-tile form of the CSR part)
     static const bool apart = std::getenv("MX_STRIPS_APART") && std::atoi(std::getenv("MX_STRIPS_APART"));
-    const bool ride = !apart && plan->csr_variant == 1 && mx::strips_can_ride(plan->dtype, plan->strips, x);
+    const bool ride = plan->dtype == MX_F64 ? (plan->csr_variant == 1 && plan->strips.vidx != nullptr)
+                                            : (!apart && plan->csr_variant == 1 && mx::strips_can_ride(plan->dtype, plan->strips, x));
     // (a binary16 row that gets sums from both parts: the CSR part leaves its sum in binary32 as
     // well and the tile kernel adds to that, so that y is rounded once, not twice)
     void *wide = plan->tiles.nWaves > 0 ? plan->ywide : nullptr;
@@ -1979,7 +2151,8 @@ extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, 
             // overwrite mode: the timed loop must not grow y without bound
             rc = time_loop(plan, warm, iters, [&]() -> int {
                 MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x_dev, y_dev, 0, s));
-                MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x_dev, y_dev, 0, s));
+                // (binary64 blocks always add to y: a few thousand additions stay far from overflow)
+                MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x_dev, y_dev, plan->dtype == MX_F64 ? 1 : 0, s));
                 return MX_OK;
             }, &t);
             if (rc) return rc;
@@ -2010,7 +2183,8 @@ extern "C" int mx_time_kernels(mx_plan *plan, const void *x_dev, void *y_dev, in
     const char *vt = plan->dtype == MX_F64 ? "f64" : "f16";
     const double xBytes = (double)plan->cols * es, yBytes = ((double)plan->rows + 1) * 4 + (double)plan->rows * es;
     static const bool apart = std::getenv("MX_STRIPS_APART") && std::atoi(std::getenv("MX_STRIPS_APART"));
-    const bool ride = !apart && plan->csr_variant == 1 && mx::strips_can_ride(plan->dtype, plan->strips, x_dev);
+    const bool ride = plan->dtype == MX_F64 ? (plan->csr_variant == 1 && plan->strips.vidx != nullptr)
+                                            : (!apart && plan->csr_variant == 1 && mx::strips_can_ride(plan->dtype, plan->strips, x_dev));
     void *wide = plan->tiles.nWaves > 0 ? plan->ywide : nullptr;
     int n = 0, rc = MX_OK;
     auto add = [&](const std::string &name, double bytes, int nnz, auto body) {
@@ -2044,7 +2218,8 @@ extern "C" int mx_time_kernels(mx_plan *plan, const void *x_dev, void *y_dev, in
                 return MX_OK;
             });
         const int stripNnz = ride ? plan->strips.vals : 0;
-        add(std::string("slice_combine_kernel<") + vt + (ride ? ",strips>" : ">"), (double)stripNnz * (es + 4) + yBytes, stripNnz,
+        add(std::string("slice_combine_kernel<") + vt + (!ride ? ">" : plan->dtype == MX_F64 ? ",blocks>" : ",strips>"),
+            (double)stripNnz * (es + 4) + yBytes, stripNnz,
             [&]() -> int {
                 MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x_dev, y_dev, 0, s, 2, ride ? &plan->strips : nullptr, wide));
                 return MX_OK;
@@ -2056,7 +2231,8 @@ extern "C" int mx_time_kernels(mx_plan *plan, const void *x_dev, void *y_dev, in
             return MX_OK;
         });
     if (!ride && plan->strips.nWaves > 0)
-        add("tile_dense_kernel<f16>", (double)plan->strips.vals * (es + 4), plan->strips.vals, [&]() -> int {
+        add(plan->dtype == MX_F64 ? "tile_block_kernel<f64>" : "tile_dense_kernel<f16>", (double)plan->strips.vals * (es + 4),
+            plan->strips.vals, [&]() -> int {
             MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x_dev, y_dev, 1, s));
             return MX_OK;
         });

@@ -521,6 +521,64 @@ def test_slice_kernel_virtual_rows(mx, ora, variant, monkeypatch):
         part.close()
 
 
+def test_binary64_block_form(mx, ora, monkeypatch):
+    """Aligned 8 x 8 blocks of a binary64 matrix through v_mfma_f64_16x16x4_f64 (tile_block_wave):
+    riding in the combine kernel's launch when the CSR part is in slice form (the block waves fetch
+    the sums of their rows' virtual rows and write y once), in a launch of their own after the row
+    kernel otherwise; blocks of every fill from three quarters up, chunks of one to eleven blocks,
+    a ragged last block row, rows with nothing but blocks and rows with nothing in blocks, columns
+    named twice.  Integer data: y must equal the oracle's exactly."""
+    import torch
+    rng = np.random.default_rng(64)
+    rows, cols = 8 * 300 + 5, 40000
+    rp, ci, va = [0], [], []
+    for r in range(rows):
+        br = r // 8
+        nblk = [0, 1, 2, 4, 5, 8, 11][br % 7]
+        brng = np.random.default_rng(1000 + br)            # the same block columns for the 8 rows of a block row
+        bcs = np.sort(brng.choice(cols // 8 - 1, nblk, replace=False))
+        c = []
+        for bc in bcs:
+            keep = rng.random(8) < (1.0 if br % 3 else 0.85)
+            c += [8 * bc + k for k in range(8) if keep[k]]
+        extra = [] if br % 5 == 0 else rng.choice(cols, rng.integers(0, 30), replace=False).tolist()
+        c = sorted(set(c) | set(extra))
+        if br % 11 == 3 and c:
+            c.append(c[len(c) // 2])                       # a column named twice, out of order
+        ci += c
+        va += rng.integers(-3, 4, len(c)).tolist()
+        rp.append(len(ci))
+    A = mx.Csr(rows, cols, np.array(rp, np.int32), np.array(ci, np.int32), np.array(va, np.float64))
+    x = rng.integers(-2, 3, cols).astype(np.float64)
+    ref = ora.spmv_f64(A.val, A.rowPtr, A.colInd, x)
+    xd = torch.from_numpy(x).cuda()
+    seen = set()
+    for tau in ((1.0, 1.0), (0.75, 0.5), (0.5, 0.25)):
+        part = mx.Partition(A, *tau)
+        for flags in (mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_SLICES, mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_ROWS,
+                      mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_DEFAULT):
+            plan = mx.Plan(part, flags)
+            y = plan.spmv(xd).cpu().numpy()
+            assert np.array_equal(y, ref), (tau, flags, plan.info)
+            y2 = torch.full((rows,), float("nan"), dtype=torch.float64, device="cuda")
+            plan.spmv_static(xd, y2)
+            assert np.array_equal(y2.cpu().numpy(), ref), (tau, flags)
+            if flags & mx.MX_PLAN_KEEP_TILES:
+                seen.add((plan.info["tile_variant"], plan.info["csr_variant"]))
+                if tau == (1.0, 1.0):
+                    assert plan.info["tile_variant"] == 2 and plan.info["tile_strip_nnz"] > 0.5 * A.nnz
+            plan.close()
+        part.close()
+    assert (2, 1) in seen and (2, 0) in seen, seen
+    # switched off: the same product without the form
+    monkeypatch.setenv("MX_NO_BLOCKS", "1")
+    part = mx.Partition(A, 1.0, 1.0)
+    plan = mx.Plan(part, mx.MX_PLAN_KEEP_TILES)
+    assert plan.info["tile_variant"] == 0 and np.array_equal(plan.spmv(xd).cpu().numpy(), ref)
+    plan.close()
+    part.close()
+
+
 def test_a_non_finite_x_reaches_only_the_rows_that_name_its_column(mx, ora):
     """Inf and NaN in x, at the first column of a slice among others (where the padding of the
     sliced layout once pointed): y is non-finite exactly on the rows that have an entry in such

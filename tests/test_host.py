@@ -580,9 +580,10 @@ def _walk_plan_layout(L, x, dtype):
     tile layouts step by step -- slot j of half h multiplies its fragM x fragK block with the x at
     the step's column ids (general layout) or at first column + 0..fragK-1 (strip layout); a
     half's rows collect until a step with flag 1, then the sums go to y (added in the general
-    layout, stored in the strip layout, whose rows nothing else may write)."""
-    fragM, fragK, slots = L["fragM"], L["fragK"], L["slots"]
-    half = slots // 2
+    layout, stored in the strip layout, whose rows nothing else may write; the binary64 form of the
+    second layout -- blocks of 8 x 8, four slots per half -- shares its rows with the CSR part and is
+    added once)."""
+    fragM, slots = L["fragM"], L["slots"]
     x = np.asarray(x, np.float64)
     y = np.zeros(L["rows"])
     rp, ci, va = L["csrRowPtr"], L["csrColInd"], L["csrVal"].astype(np.float64)
@@ -591,6 +592,8 @@ def _walk_plan_layout(L, x, dtype):
     touched = np.zeros(L["rows"], bool)
     entries = 0
     for t, T in enumerate(L["tiles"]):
+        fragK = 8 if t == 1 else L["fragK"]        # the plan's own chunks are made of 8-column blocks
+        half = 4 if t == 1 else slots // 2
         val = T["val"].astype(np.float64)
         seen_steps = 0
         for w in range(T["nWaves"]):
@@ -605,7 +608,7 @@ def _walk_plan_layout(L, x, dtype):
                 vo = T["valOffset"][s]
                 for h in range(2):
                     for j in range(n[h]):
-                        slot = 2 * j + h if fragK == 4 else half * h + j   # the binary64 step interleaves its halves
+                        slot = 2 * j + h if (t == 0 and fragK == 4) else half * h + j   # the general binary64 step interleaves its halves
                         blk = val[vo + ((n[0] if h else 0) + j) * fragM * fragK:][:fragM * fragK].reshape(fragM, fragK)
                         if t == 1:
                             c0 = hdr[21 + slot]
@@ -628,7 +631,11 @@ def _walk_plan_layout(L, x, dtype):
                             if r < 0:
                                 assert sums[i] == 0
                                 continue
-                            if t == 1:
+                            if t == 1 and L["fragK"] == 4:
+                                assert L["stripRows"][r] == 2 and not touched[r], "a row of a block chunk is finished once"
+                                touched[r] = True
+                                y[r] += sums[i]
+                            elif t == 1:
                                 assert L["stripRows"][r] == 1 and not touched[r] and y[r] == 0, "a strip row is written once, by the strips alone"
                                 touched[r] = True
                                 y[r] = sums[i]
@@ -717,7 +724,7 @@ def test_plan_layout_walk(mx, ora, case):
                 assert L["tiles"][1]["steps"] == 0, "strip chunks are a matter of the default selection"
             strips_seen += L["tiles"][1]["steps"]
         P.close()
-    assert (strips_seen > 0) == (case in ("strips_f16", "blocks_f16", "mixed_f16")), strips_seen
+    assert (strips_seen > 0) == (case in ("strips_f16", "blocks_f16", "mixed_f16", "block_f64")), strips_seen
 
 
 
