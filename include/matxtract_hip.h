@@ -390,6 +390,12 @@ typedef struct mx_slice_layout_view {
     unsigned char *dict;  /* [256] values (binary64 or binary16), zeros beyond nDict */
 } mx_slice_layout_view;
 int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *sel, mx_slice_layout_view *out);
+/* The same view by the route plans take for a whole matrix: A goes up, the layout is built on the
+ * device from the device arrays (sorts, running sums and placement kernels; only the assignment of
+ * chunks to workgroups and waves, a few values per thousand entries, is decided on the host, by the
+ * routine both routes share) and comes down.  Every array equals mx_slice_layout's (sel = NULL) byte
+ * for byte.  MX_ERR_DEVICE without a HIP device. */
+int mx_slice_layout_device(const mx_csr *A, int nCU, mx_slice_layout_view *out);
 void mx_slice_layout_free(mx_slice_layout_view *v);
 
 /* The host half of a plan for a partition, for inspection and tests on a machine without a GPU

@@ -131,6 +131,7 @@ SIGNATURES = {
     "mx_tune_tau": (_i, [C.POINTER(CsrStruct), _i, _i, _i, _i, C.POINTER(C.c_float), C.POINTER(C.c_float),
                          C.POINTER(TauPoint), _i, _pi]),
     "mx_slice_layout": (_i, [C.POINTER(CsrStruct), _i, _vp, C.POINTER(SliceLayoutView)]),
+    "mx_slice_layout_device": (_i, [C.POINTER(CsrStruct), _i, C.POINTER(SliceLayoutView)]),
     "mx_slice_layout_free": (None, [C.POINTER(SliceLayoutView)]),
     "mx_plan_layout": (_i, [_vp, _i, _i, C.POINTER(PlanLayoutView)]),
     "mx_plan_layout_free": (None, [C.POINTER(PlanLayoutView)]),

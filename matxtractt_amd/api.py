@@ -278,18 +278,22 @@ class Partition:
             pass
 
 
-def slice_layout(A, nCU=256, sel=None):
-    """The host-side layout of the column-slice kernel for matrix A as a dict of numpy arrays
-    and sizes (see mx_slice_layout in include/matxtract_hip.h).  `sel`: optional mask of the rows
-    to include."""
+def slice_layout(A, nCU=256, sel=None, device=False):
+    """The layout of the column-slice kernel for matrix A as a dict of numpy arrays and sizes (see
+    mx_slice_layout in include/matxtract_hip.h), built on the host, or with device=True on the GPU
+    (mx_slice_layout_device: the same arrays).  `sel`: optional mask of the rows to include (host
+    route only)."""
     v = _lib.SliceLayoutView()
     st = A.struct()
     selp = None
     if sel is not None:
         sel = np.ascontiguousarray(sel, dtype=np.uint8)
-        assert sel.shape == (A.rows,)
+        assert sel.shape == (A.rows,) and not device
         selp = sel.ctypes.data
-    check(_lib.load().mx_slice_layout(C.byref(st), int(nCU), selp, C.byref(v)))
+    if device:
+        check(_lib.load().mx_slice_layout_device(C.byref(st), int(nCU), C.byref(v)))
+    else:
+        check(_lib.load().mx_slice_layout(C.byref(st), int(nCU), selp, C.byref(v)))
     try:
         out = {n: int(getattr(v, n)) for n in ("nWG", "S", "sliceCols", "waves", "stepEntries", "batchEntries", "cap",
                                                "chunks", "batches", "vrows", "nLight", "nHeavy", "lightSegs")}

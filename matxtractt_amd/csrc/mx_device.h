@@ -143,6 +143,35 @@ constexpr int kSliceLightSegs = 8;     // rows with at most this many virtual ro
 constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
 hipError_t static_scratch(void **ptr);
 
+}  // namespace mx
+#include <vector>
+namespace mx {
+// One chunk of a slice on its way into the layout: `first` = index of its first virtual row in
+// the sorted order of virtual rows, n = how many it has (64 but for the last of a slice), steps
+// = the length of its longest (first) member.
+struct SliceChunk {
+    int first, n, steps;
+};
+// What plan_slice_chunks decides: the descriptors the kernels read (DeviceSlices) and, for every
+// chunk in its final numbering (workgroup by workgroup, wave by wave), where it comes from and at
+// which step of the streams it starts.
+struct SlicePlan {
+    int nWG = 0, maxWgChunks = 0;
+    long long totalSteps = 0, totalChunks = 0;
+    std::vector<int> wgDesc, waveDesc, chunkEnd;
+    std::vector<int> chunkSlice, chunkFirst, chunkN, chunkSteps;
+    std::vector<long long> chunkStep0;
+};
+int plan_slice_chunks(mx_dtype dtype, int budget, int S, const std::vector<std::vector<SliceChunk>> &sliceChunks, SlicePlan &P);
+constexpr int kSlicePadSteps = 16;  // spare zero steps after the last of the streams
+// The slice layout built on the device from a CSR matrix in device memory (mx_layout.hip): the
+// arrays of `D` equal those of the host route byte for byte.  `elsewhere_dev`: optional marks per
+// row (device memory) as in the host route.  segPtrOut / segIdxOut (optional): host copies of the
+// virtual rows of every row.
+int build_slices_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, const void *val_dev,
+                        int nCU, int S, const char *elsewhere_dev, DeviceSlices &D, hipStream_t s, std::vector<int> *segPtrOut = nullptr,
+                        std::vector<int> *segIdxOut = nullptr);
+
 // `what`: 0 = slice kernel then combine kernel, 1 = slice kernel only, 2 = combine kernel only
 // `strips` (optional): a tile layout in the dense binary16 form whose steps workgroups of the
 // combine kernel's launch run as well (strips_can_ride says whether a layout may); the rows of

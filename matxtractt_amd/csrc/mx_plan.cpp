@@ -190,7 +190,7 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
                  const char *sel, HostSlices &D, const char *elsewhere = nullptr)
 {
     const int es = mx::elem_size(dtype), E = mx::slice_step_entries(dtype);
-    const int BE = mx::kSliceBatchEntries, SPB = BE / E;  // steps per batch
+    const int BE = mx::kSliceBatchEntries;
     const int SW = mx::slice_cols(dtype), W = mx::kSliceWaves;
     // entries of the selected rows, row by row, ascending by column (stable)
     std::vector<int> selPtr((size_t)rows + 1, 0);
@@ -261,106 +261,20 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
         std::vector<int> cur(keyStart.begin(), keyStart.end() - 1);
         for (int t = 0; t < nV; ++t) sorted[cur[key_of(vr[t])]++] = t;
     }
-    // chunks of every slice, and the slice's share of the workgroups (in proportion to its
-    // steps, largest remainders, at least one when it holds anything)
-    struct Chunk {
-        int first, n, steps;  // first: into sorted
-    };
-    std::vector<std::vector<Chunk>> sliceChunks(S);
-    std::vector<long long> sliceSteps(S, 0);
-    long long allSteps = 0;
-    int busy = 0;
+    // chunks of every slice: 64 virtual rows of the sorted order each, as long as their first member
+    std::vector<std::vector<mx::SliceChunk>> sliceChunks(S);
     for (int q = 0; q < S; ++q) {
         const int a = keyStart[(size_t)q * perSlice], b = keyStart[(size_t)(q + 1) * perSlice];
-        for (int f = a; f < b; f += 64) {
-            const int n = std::min(64, b - f), steps = (vr[sorted[f]].len + E - 1) / E;
-            sliceChunks[q].push_back({f, n, steps});
-            sliceSteps[q] += steps;
-        }
-        allSteps += sliceSteps[q];
-        busy += b > a;
+        for (int f = a; f < b; f += 64) sliceChunks[q].push_back({f, std::min(64, b - f), (vr[sorted[f]].len + E - 1) / E});
     }
-    std::vector<int> Gq(S, 0);
+    mx::SlicePlan SP;
     {
-        const int total = std::max(budget, busy);
-        std::vector<double> want(S, 0.0);
-        int used = 0;
-        for (int q = 0; q < S; ++q) {
-            if (sliceChunks[q].empty()) continue;
-            want[q] = allSteps > 0 ? (double)sliceSteps[q] * total / (double)allSteps : 1.0;
-            Gq[q] = std::max(1, (int)want[q]);
-            used += Gq[q];
-        }
-        while (used < total && busy > 0) {  // hand out what rounding down left over
-            int best = -1;
-            for (int q = 0; q < S; ++q)
-                if (!sliceChunks[q].empty() && (best < 0 || want[q] - Gq[q] > want[best] - Gq[best])) best = q;
-            ++Gq[best];
-            ++used;
-        }
-        for (int q = 0; q < S; ++q) {
-            const int nc = (int)sliceChunks[q].size();
-            Gq[q] = std::min(std::max(Gq[q], (nc + mx::kSliceWgChunks - 1) / mx::kSliceWgChunks), std::max(nc, 1));
-            if (nc == 0) Gq[q] = 0;
-        }
+        const int rc = mx::plan_slice_chunks(dtype, budget, S, sliceChunks, SP);
+        if (rc) return rc;
     }
-    // workgroups: a slice's chunks, longest first, each to the workgroup of the slice with the
-    // fewest steps so far; then the same inside the workgroup for its waves
-    struct Wg {
-        int slice;
-        std::vector<int> chunk[mx::kSliceWaves];  // per wave: indices into sliceChunks[slice]
-        int waveSteps[mx::kSliceWaves];
-        long long steps = 0;   // stored steps (every wave's stream rounded up to whole batches)
-        int chunks = 0;
-    };
-    std::vector<Wg> wgs;
-    for (int q = 0; q < S; ++q) {
-        const int g0 = (int)wgs.size(), G = Gq[q];
-        if (G == 0) continue;
-        wgs.resize(wgs.size() + G);
-        std::vector<std::vector<int>> mine(G);
-        typedef std::pair<long long, int> Load;
-        std::priority_queue<Load, std::vector<Load>, std::greater<Load>> heap;
-        for (int g = 0; g < G; ++g) heap.push({0, g});
-        const auto &ch = sliceChunks[q];
-        for (int c = 0; c < (int)ch.size(); ++c) {
-            Load top = heap.top();
-            heap.pop();
-            mine[top.second].push_back(c);
-            top.first += ch[c].steps;
-            if ((int)mine[top.second].size() < mx::kSliceWgChunks) heap.push(top);
-        }
-        for (int g = 0; g < G; ++g) {
-            Wg &w = wgs[g0 + g];
-            w.slice = q;
-            for (int k = 0; k < W; ++k) w.waveSteps[k] = 0;
-            for (int c : mine[g]) {
-                int best = 0;
-                for (int k = 1; k < W; ++k)
-                    if (w.waveSteps[k] < w.waveSteps[best]) best = k;
-                w.chunk[best].push_back(c);
-                w.waveSteps[best] += ch[c].steps;
-            }
-            w.chunks = (int)mine[g].size();
-            for (int k = 0; k < W; ++k) w.steps += (w.waveSteps[k] + SPB - 1) / SPB * SPB;
-        }
-    }
-    const int nWG = (int)wgs.size();
-    long long totalSteps = 0, totalChunks = 0;
-    std::vector<long long> wgStep((size_t)nWG + 1, 0), wgChunk((size_t)nWG + 1, 0);
-    int maxWgChunks = 0;
-    for (int b = 0; b < nWG; ++b) {
-        wgStep[b] = totalSteps;
-        wgChunk[b] = totalChunks;
-        totalSteps += wgs[b].steps;
-        totalChunks += wgs[b].chunks;
-        maxWgChunks = std::max(maxWgChunks, wgs[b].chunks);
-    }
-    if (totalSteps * 64 * E > 2000000000LL || totalChunks * 64 > 2000000000LL) {
-        set_error("slice layout: too many entries for 32-bit offsets");
-        return MX_ERR_ARG;
-    }
-    const size_t padSteps = 16;  // spare zero steps after the last
+    const int nWG = SP.nWG, maxWgChunks = SP.maxWgChunks;
+    const long long totalSteps = SP.totalSteps, totalChunks = SP.totalChunks;
+    const size_t padSteps = mx::kSlicePadSteps;  // spare zero steps after the last
     std::vector<unsigned short> ecol(((size_t)totalSteps + padSteps) * 64 * E, 0);
     std::vector<unsigned char> ev(((size_t)totalSteps + padSteps) * 64 * E * es, 0);
     // one byte per entry instead of its value when the selected rows hold at most 256 distinct
@@ -375,57 +289,38 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
             haveDict = make_value_dict(es, val, rowPtr[rows], codeOfEntry, dictv, &nDict, 255);
         if (haveDict) ecode.assign(ecol.size(), 255);
     }
-    std::vector<int> wgDesc((size_t)nWG * 4 + 4, 0), waveDesc((size_t)nWG * W * 4 + 4, 0), chunkEnd((size_t)totalChunks + 64, 0);
+    std::vector<int> &wgDesc = SP.wgDesc, &waveDesc = SP.waveDesc, &chunkEnd = SP.chunkEnd;
     std::vector<int> segIdx((size_t)nV + 1, 0);
     const unsigned char *sv = (const unsigned char *)val;
-#pragma omp parallel for schedule(dynamic, 1)
-    for (int b = 0; b < nWG; ++b) {
-        const Wg &G = wgs[b];
-        const int q = G.slice;
-        const auto &ch = sliceChunks[q];
-        long long step = wgStep[b], chunk = wgChunk[b];
-        wgDesc[(size_t)b * 4 + 0] = q;
-        wgDesc[(size_t)b * 4 + 1] = (int)chunk;
-        wgDesc[(size_t)b * 4 + 2] = G.chunks;
-        for (int w = 0; w < W; ++w) {
-            int *d = &waveDesc[((size_t)b * W + w) * 4];
-            d[0] = (int)(step / SPB);                   // first batch
-            d[1] = (G.waveSteps[w] + SPB - 1) / SPB;    // batches
-            d[2] = (int)(chunk - wgChunk[b]);           // first chunk, counted inside the workgroup
-            d[3] = (int)G.chunk[w].size();
-            int rel = 0;
-            for (int c : G.chunk[w]) {
-                for (int l = 0; l < ch[c].n; ++l) {
-                    const int t = sorted[ch[c].first + l];
-                    const VRow &v = vr[t];
-                    segIdx[t] = (int)(chunk * 64 + l);
-                    for (int n = 0; n < v.len; ++n) {
-                        const int p = ord[v.start + n];
-                        const size_t st = (size_t)step + n, batch = st / BE, k = st % BE;
-                        // a lane's column offsets of a batch are contiguous; so are its binary16
-                        // values; binary64 values go in sub-blocks of two per lane
-                        const size_t atc = (batch * 64 + l) * BE + k;
-                        const size_t atv = dtype == MX_F64 ? batch * 64 * BE + (k / 2) * 128 + (size_t)l * 2 + k % 2 : atc;
-                        ecol[atc] = (unsigned short)(col[p] - q * SW);
-                        if (haveDict) ecode[atc] = codeOfEntry[p];
-                        std::memcpy(&ev[atv * es], sv + (size_t)p * es, es);
-                    }
-                    // the padding up to the chunk's longest member multiplies zero with the x of the
-                    // virtual row's own last column: a non-finite x then reaches the rows that name its
-                    // column, as in a plain CSR product, and no others
-                    if (v.len > 0) {
-                        const unsigned short lastCol = (unsigned short)(col[ord[v.start + v.len - 1]] - q * SW);
-                        for (int n = v.len; n < ch[c].steps * E; ++n) {
-                            const size_t st = (size_t)step + n, batch = st / BE, k = st % BE;
-                            ecol[(batch * 64 + l) * BE + k] = lastCol;
-                        }
-                    }
-                }
-                step += ch[c].steps;
-                rel += ch[c].steps;
-                chunkEnd[chunk++] = rel;
+#pragma omp parallel for schedule(dynamic, 64)
+    for (long long c = 0; c < totalChunks; ++c) {
+        const int q = SP.chunkSlice[c], steps = SP.chunkSteps[c];
+        const long long step = SP.chunkStep0[c];
+        for (int l = 0; l < SP.chunkN[c]; ++l) {
+            const int t = sorted[SP.chunkFirst[c] + l];
+            const VRow &v = vr[t];
+            segIdx[t] = (int)(c * 64 + l);
+            for (int n = 0; n < v.len; ++n) {
+                const int p = ord[v.start + n];
+                const size_t st = (size_t)step + n, batch = st / BE, k = st % BE;
+                // a lane's column offsets of a batch are contiguous; so are its binary16
+                // values; binary64 values go in sub-blocks of two per lane
+                const size_t atc = (batch * 64 + l) * BE + k;
+                const size_t atv = dtype == MX_F64 ? batch * 64 * BE + (k / 2) * 128 + (size_t)l * 2 + k % 2 : atc;
+                ecol[atc] = (unsigned short)(col[p] - q * SW);
+                if (haveDict) ecode[atc] = codeOfEntry[p];
+                std::memcpy(&ev[atv * es], sv + (size_t)p * es, es);
             }
-            step = (step + SPB - 1) / SPB * SPB;
+            // the padding up to the chunk's longest member multiplies zero with the x of the
+            // virtual row's own last column: a non-finite x then reaches the rows that name its
+            // column, as in a plain CSR product, and no others
+            if (v.len > 0) {
+                const unsigned short lastCol = (unsigned short)(col[ord[v.start + v.len - 1]] - q * SW);
+                for (int n = v.len; n < steps * E; ++n) {
+                    const size_t st = (size_t)step + n, batch = st / BE, k = st % BE;
+                    ecol[(batch * 64 + l) * BE + k] = lastCol;
+                }
+            }
         }
     }
     // how the sums become y: rows with one virtual row are named at that virtual row, the others
@@ -476,6 +371,27 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
                   const char *sel, mx::DeviceSlices &D, const char *elsewhere = nullptr,
                   std::pair<std::vector<int>, std::vector<int>> *segOut = nullptr)
 {
+    // The whole matrix: the layout is made on the device (the same arrays, in a fraction of the
+    // time for a large matrix); MX_LAYOUT=host keeps the host route, which also serves row subsets.
+    const char *lay = std::getenv("MX_LAYOUT");
+    if (!sel && !(lay && !std::strcmp(lay, "host"))) {
+        const size_t es = (size_t)mx::elem_size(dtype);
+        const int nnz = rowPtr[rows];
+        int *dRowPtr = nullptr, *dCol = nullptr;
+        void *dVal = nullptr, *dElse = nullptr;
+        int rc = upload(&dRowPtr, rowPtr, (size_t)rows + 1);
+        if (!rc) rc = upload(&dCol, col, (size_t)nnz);
+        if (!rc) rc = upload_bytes(&dVal, val, (size_t)nnz * es);
+        if (!rc && elsewhere) rc = upload_bytes(&dElse, elsewhere, (size_t)rows);
+        if (!rc)
+            rc = mx::build_slices_device(dtype, rows, cols, nnz, dRowPtr, dCol, dVal, nCU, S, (const char *)dElse, D, nullptr,
+                                         segOut ? &segOut->first : nullptr, segOut ? &segOut->second : nullptr);
+        (void)hipFree(dRowPtr);
+        (void)hipFree(dCol);
+        (void)hipFree(dVal);
+        (void)hipFree(dElse);
+        return rc;
+    }
     HostSlices H;
     int rc = build_slices(dtype, rows, cols, rowPtr, col, val, nCU, S, sel, H, elsewhere);
     if (rc) return rc;
@@ -896,6 +812,147 @@ int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, c
 
 }  // namespace
 
+// The part of the slice layout that looks at chunks only (64 virtual rows each; a few per thousand
+// entries): which workgroup and wave streams which chunk, and where.  Shared by the host route and
+// the device route of the layout, which hand in the chunks of every slice (longest first, as the
+// sort leaves them) and fill the streams from what comes back.
+int mx::plan_slice_chunks(mx_dtype dtype, int budget, int S, const std::vector<std::vector<mx::SliceChunk>> &sliceChunks,
+                          mx::SlicePlan &P)
+{
+    const int E = mx::slice_step_entries(dtype), SPB = mx::kSliceBatchEntries / E, W = mx::kSliceWaves;
+    // the slice's share of the workgroups (in proportion to its steps, largest remainders, at
+    // least one when it holds anything)
+    std::vector<long long> sliceSteps(S, 0);
+    long long allSteps = 0;
+    int busy = 0;
+    for (int q = 0; q < S; ++q) {
+        for (const mx::SliceChunk &c : sliceChunks[q]) sliceSteps[q] += c.steps;
+        allSteps += sliceSteps[q];
+        busy += !sliceChunks[q].empty();
+    }
+    std::vector<int> Gq(S, 0);
+    {
+        const int total = std::max(budget, busy);
+        std::vector<double> want(S, 0.0);
+        int used = 0;
+        for (int q = 0; q < S; ++q) {
+            if (sliceChunks[q].empty()) continue;
+            want[q] = allSteps > 0 ? (double)sliceSteps[q] * total / (double)allSteps : 1.0;
+            Gq[q] = std::max(1, (int)want[q]);
+            used += Gq[q];
+        }
+        while (used < total && busy > 0) {  // hand out what rounding down left over
+            int best = -1;
+            for (int q = 0; q < S; ++q)
+                if (!sliceChunks[q].empty() && (best < 0 || want[q] - Gq[q] > want[best] - Gq[best])) best = q;
+            ++Gq[best];
+            ++used;
+        }
+        for (int q = 0; q < S; ++q) {
+            const int nc = (int)sliceChunks[q].size();
+            Gq[q] = std::min(std::max(Gq[q], (nc + mx::kSliceWgChunks - 1) / mx::kSliceWgChunks), std::max(nc, 1));
+            if (nc == 0) Gq[q] = 0;
+        }
+    }
+    // workgroups: a slice's chunks, longest first, each to the workgroup of the slice with the
+    // fewest steps so far; then the same inside the workgroup for its waves
+    struct Wg {
+        int slice;
+        std::vector<int> chunk[mx::kSliceWaves];  // per wave: indices into sliceChunks[slice]
+        int waveSteps[mx::kSliceWaves];
+        long long steps = 0;   // stored steps (every wave's stream rounded up to whole batches)
+        int chunks = 0;
+    };
+    std::vector<Wg> wgs;
+    for (int q = 0; q < S; ++q) {
+        const int g0 = (int)wgs.size(), G = Gq[q];
+        if (G == 0) continue;
+        wgs.resize(wgs.size() + G);
+        std::vector<std::vector<int>> mine(G);
+        typedef std::pair<long long, int> Load;
+        std::priority_queue<Load, std::vector<Load>, std::greater<Load>> heap;
+        for (int g = 0; g < G; ++g) heap.push({0, g});
+        const auto &ch = sliceChunks[q];
+        for (int c = 0; c < (int)ch.size(); ++c) {
+            Load top = heap.top();
+            heap.pop();
+            mine[top.second].push_back(c);
+            top.first += ch[c].steps;
+            if ((int)mine[top.second].size() < mx::kSliceWgChunks) heap.push(top);
+        }
+        for (int g = 0; g < G; ++g) {
+            Wg &w = wgs[g0 + g];
+            w.slice = q;
+            for (int k = 0; k < W; ++k) w.waveSteps[k] = 0;
+            for (int c : mine[g]) {
+                int best = 0;
+                for (int k = 1; k < W; ++k)
+                    if (w.waveSteps[k] < w.waveSteps[best]) best = k;
+                w.chunk[best].push_back(c);
+                w.waveSteps[best] += ch[c].steps;
+            }
+            w.chunks = (int)mine[g].size();
+            for (int k = 0; k < W; ++k) w.steps += (w.waveSteps[k] + SPB - 1) / SPB * SPB;
+        }
+    }
+    const int nWG = (int)wgs.size();
+    long long totalSteps = 0, totalChunks = 0;
+    std::vector<long long> wgStep((size_t)nWG + 1, 0), wgChunk((size_t)nWG + 1, 0);
+    int maxWgChunks = 0;
+    for (int b = 0; b < nWG; ++b) {
+        wgStep[b] = totalSteps;
+        wgChunk[b] = totalChunks;
+        totalSteps += wgs[b].steps;
+        totalChunks += wgs[b].chunks;
+        maxWgChunks = std::max(maxWgChunks, wgs[b].chunks);
+    }
+    if (totalSteps * 64 * E > 2000000000LL || totalChunks * 64 > 2000000000LL) {
+        set_error("slice layout: too many entries for 32-bit offsets");
+        return MX_ERR_ARG;
+    }
+    P.nWG = nWG;
+    P.maxWgChunks = maxWgChunks;
+    P.totalSteps = totalSteps;
+    P.totalChunks = totalChunks;
+    P.wgDesc.assign((size_t)nWG * 4 + 4, 0);
+    P.waveDesc.assign((size_t)nWG * W * 4 + 4, 0);
+    P.chunkEnd.assign((size_t)totalChunks + 64, 0);
+    P.chunkSlice.assign((size_t)totalChunks, 0);
+    P.chunkFirst.assign((size_t)totalChunks, 0);
+    P.chunkN.assign((size_t)totalChunks, 0);
+    P.chunkSteps.assign((size_t)totalChunks, 0);
+    P.chunkStep0.assign((size_t)totalChunks, 0);
+    for (int b = 0; b < nWG; ++b) {
+        const Wg &G = wgs[b];
+        const int q = G.slice;
+        const auto &ch = sliceChunks[q];
+        long long step = wgStep[b], chunk = wgChunk[b];
+        P.wgDesc[(size_t)b * 4 + 0] = q;
+        P.wgDesc[(size_t)b * 4 + 1] = (int)chunk;
+        P.wgDesc[(size_t)b * 4 + 2] = G.chunks;
+        for (int w = 0; w < W; ++w) {
+            int *d = &P.waveDesc[((size_t)b * W + w) * 4];
+            d[0] = (int)(step / SPB);                   // first batch
+            d[1] = (G.waveSteps[w] + SPB - 1) / SPB;    // batches
+            d[2] = (int)(chunk - wgChunk[b]);           // first chunk, counted inside the workgroup
+            d[3] = (int)G.chunk[w].size();
+            int rel = 0;
+            for (int c : G.chunk[w]) {
+                P.chunkSlice[chunk] = q;
+                P.chunkFirst[chunk] = ch[c].first;
+                P.chunkN[chunk] = ch[c].n;
+                P.chunkSteps[chunk] = ch[c].steps;
+                P.chunkStep0[chunk] = step;
+                step += ch[c].steps;
+                rel += ch[c].steps;
+                P.chunkEnd[chunk++] = rel;
+            }
+            step = (step + SPB - 1) / SPB * SPB;
+        }
+    }
+    return MX_OK;
+}
+
 extern "C" int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *sel, mx_slice_layout_view *out)
 {
     if (!A || !out || nCU < 1 || A->rows < 0 || A->cols < 1 || !A->rowPtr || (A->nnz > 0 && (!A->colInd || !A->val))) {
@@ -985,6 +1042,112 @@ extern "C" void mx_slice_layout_free(mx_slice_layout_view *v)
     free(v->ecode);
     free(v->dict);
     std::memset(v, 0, sizeof(*v));
+}
+
+// The same view from the device route of the layout: the matrix goes up, the layout is built
+// there (mx_layout.hip) and comes down.  For tests: every array must equal mx_slice_layout's.
+extern "C" int mx_slice_layout_device(const mx_csr *A, int nCU, mx_slice_layout_view *out)
+{
+    if (!A || !out || nCU < 1 || A->rows < 1 || A->cols < 1 || !A->rowPtr || (A->nnz > 0 && (!A->colInd || !A->val))) {
+        set_error("mx_slice_layout_device: bad argument");
+        return MX_ERR_ARG;
+    }
+    std::memset(out, 0, sizeof(*out));
+    int rc = need_device();
+    if (rc) return rc;
+    if (A->rowPtr[0] != 0 || A->rowPtr[A->rows] != A->nnz) {
+        set_error("mx_slice_layout_device: rowPtr does not span [0, nnz]");
+        return MX_ERR_ARG;
+    }
+    for (int p = 0; p < A->nnz; ++p)
+        if ((unsigned)A->colInd[p] >= (unsigned)A->cols) {
+            set_error("mx_slice_layout_device: column index out of range");
+            return MX_ERR_ARG;
+        }
+    const int S = (A->cols + mx::slice_cols(A->dtype) - 1) / mx::slice_cols(A->dtype);
+    const size_t es = (size_t)mx::elem_size(A->dtype);
+    int *dRowPtr = nullptr, *dCol = nullptr;
+    void *dVal = nullptr;
+    mx::DeviceSlices D;
+    std::vector<int> segPtr, segIdx;
+    rc = upload(&dRowPtr, A->rowPtr, (size_t)A->rows + 1);
+    if (!rc) rc = upload(&dCol, A->colInd, (size_t)A->nnz);
+    if (!rc) rc = upload_bytes(&dVal, A->val, (size_t)A->nnz * es);
+    if (!rc) rc = mx::build_slices_device(A->dtype, A->rows, A->cols, A->nnz, dRowPtr, dCol, dVal, nCU, S, nullptr, D, nullptr, &segPtr, &segIdx);
+    (void)hipFree(dRowPtr);
+    (void)hipFree(dCol);
+    (void)hipFree(dVal);
+    if (rc) {
+        free_slices(D);
+        return rc;
+    }
+    auto down = [&](const void *src, size_t bytes) -> void * {
+        void *p = malloc(std::max<size_t>(bytes, 1));
+        if (p && bytes && hipMemcpy(p, src, bytes, hipMemcpyDeviceToHost) != hipSuccess) {
+            free(p);
+            p = nullptr;
+        }
+        return p;
+    };
+    const int E = mx::slice_step_entries(A->dtype);
+    out->nWG = D.nWG;
+    out->S = D.S;
+    out->sliceCols = D.sliceCols;
+    out->waves = mx::kSliceWaves;
+    out->stepEntries = E;
+    out->batchEntries = mx::kSliceBatchEntries;
+    out->chunks = (int)D.chunks;
+    out->batches = (int)(D.steps / (mx::kSliceBatchEntries / E));
+    out->vrows = D.vrows;
+    out->nLight = D.nLight;
+    out->nHeavy = D.nHeavy;
+    out->lightSegs = mx::kSliceLightSegs;
+    out->nEcol = (long long)(((size_t)D.steps + mx::kSlicePadSteps) * 64 * E);
+    {
+        // (the cap is a function of the size alone, as in the host route)
+        const long long fair = (long long)A->nnz / ((long long)nCU * mx::kSliceWaves * 64);
+        const int BE = mx::kSliceBatchEntries;
+        out->cap = (int)std::min<long long>(512, std::max<long long>(16, (fair + BE - 1) / BE * BE));
+        if (const char *e = std::getenv("MX_SLICE_CAP")) {
+            const int v = std::atoi(e);
+            if (v >= BE && v <= 4096) out->cap = v / BE * BE;
+        }
+    }
+    out->wgDesc = (int *)down(D.wgDesc, ((size_t)D.nWG * 4 + 4) * 4);
+    out->waveDesc = (int *)down(D.waveDesc, ((size_t)D.nWG * mx::kSliceWaves * 4 + 4) * 4);
+    out->chunkEnd = (int *)down(D.chunkEnd, ((size_t)D.chunks + 64) * 4);
+    out->segPtr = (int *)malloc(std::max<size_t>(segPtr.size(), 1) * 4);
+    if (out->segPtr) std::memcpy(out->segPtr, segPtr.data(), segPtr.size() * 4);
+    out->segIdx = (int *)down(D.segIdx, ((size_t)D.vrows + 1) * 4);
+    out->rowInfo = (int *)down(D.rowInfo, (((size_t)A->rows + 3) / 4 * 4 + 4) * 4);
+    out->heavyInfo = (int *)down(D.heavyInfo, ((size_t)D.nHeavy * 4 + 4) * 4);
+    out->ecol = (unsigned short *)down(D.ecol, (size_t)out->nEcol * 2);
+    out->eval = (unsigned char *)down(D.eval, (size_t)out->nEcol * es);
+    out->nDict = D.ecode ? D.nDict : 0;
+    out->ecode = (unsigned char *)(D.ecode ? down(D.ecode, (size_t)out->nEcol) : malloc(1));
+    out->dict = (unsigned char *)(D.ecode ? down(D.dict, 256 * es) : malloc(1));
+    // the light rows in the form of the host view: {row, first virtual row in segIdx, count, 0}
+    {
+        std::vector<int> lr((size_t)D.nLight + 1, 0);
+        bool ok = D.nLight == 0 || hipMemcpy(lr.data(), D.lightRow, (size_t)D.nLight * 4, hipMemcpyDeviceToHost) == hipSuccess;
+        out->lightInfo = ok ? (int *)malloc(std::max<size_t>((size_t)D.nLight * 16, 1)) : nullptr;
+        if (out->lightInfo)
+            for (int i = 0; i < D.nLight; ++i) {
+                const int r = lr[i];
+                out->lightInfo[4 * i] = r;
+                out->lightInfo[4 * i + 1] = segPtr[r];
+                out->lightInfo[4 * i + 2] = segPtr[r + 1] - segPtr[r];
+                out->lightInfo[4 * i + 3] = 0;
+            }
+    }
+    free_slices(D);
+    if (!out->wgDesc || !out->waveDesc || !out->chunkEnd || !out->segPtr || !out->segIdx || !out->rowInfo || !out->lightInfo ||
+        !out->heavyInfo || !out->ecol || !out->ecode || !out->dict || !out->eval) {
+        mx_slice_layout_free(out);
+        set_error("mx_slice_layout_device: out of memory or copy failed");
+        return MX_ERR_ALLOC;
+    }
+    return MX_OK;
 }
 
 // MX_CSR_NPT overrides the default (for tuning runs); only values with a compiled kernel count.

@@ -6,6 +6,8 @@ hipError_t launch_tiles(mx_dtype, const DeviceTiles &, const void *, void *, int
 hipError_t launch_csr(mx_dtype, const DeviceCsr &, const void *, void *, int, hipStream_t, void *) { return hipErrorUnknown; }
 hipError_t launch_slices(mx_dtype, const DeviceSlices &, const void *, void *, int, hipStream_t, int, const DeviceTiles *, void *) { return hipErrorUnknown; }
 hipError_t static_scratch(void **p) { *p = nullptr; return hipErrorUnknown; }
+int build_slices_device(mx_dtype, int, int, int, const int *, const int *, const void *, int, int, const char *, DeviceSlices &, hipStream_t,
+                        std::vector<int> *, std::vector<int> *) { return MX_ERR_DEVICE; }
 bool strips_can_ride(mx_dtype, const DeviceTiles &, const void *) { return false; }
 hipError_t launch_probe_f64(const double *, const double *, double *, hipStream_t) { return hipErrorUnknown; }
 hipError_t launch_probe_f16(const void *, const void *, float *, hipStream_t) { return hipErrorUnknown; }

@@ -1160,3 +1160,35 @@ def test_partition_by_the_device_route_is_the_same_partition(mx, ora):
     assert rel_l2(y.cpu().numpy().astype(np.float64), oracle_y(ora, mx, A, x)) <= F16_TOL
     plan.close()
     D.close()
+
+
+@pytest.mark.gpu
+def test_slice_layout_by_the_device_route_is_the_same_layout(mx, monkeypatch):
+    """mx_slice_layout_device -- the route plans take -- against mx_slice_layout: every array of the
+    layout byte for byte, on the five workloads at reduced size, on workloads 2 and 4 at full size,
+    on a matrix with at most 255 distinct values (the one-byte form), and on rows in any order that
+    name columns twice."""
+    rng = np.random.default_rng(77)
+    cases = [mx.gen_config(c, scale=sc)[0] for c, sc in ((1, 1.0), (2, 1 / 8), (3, 0.05), (4, 1 / 16), (5, 1 / 64), (2, 1.0), (4, 1.0))]
+    A = cases[2]
+    cases.append(mx.Csr(A.rows, A.cols, A.rowPtr, A.colInd, A.val.astype(np.float16)))          # a binary16 stencil: two values
+    lens = rng.integers(0, 90, 4000)
+    lens[::50] = 1500
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cases.append(mx.Csr(4000, 70000, ptr, rng.integers(0, 70000, ptr[-1]).astype(np.int32), rng.integers(-9, 10, ptr[-1]).astype(np.float64)))
+    cases.append(mx.Csr(4000, 300000, ptr, rng.integers(0, 300000, ptr[-1]).astype(np.int32), rng.uniform(-1, 1, ptr[-1]).astype(np.float16)))
+    names = ("wgDesc", "waveDesc", "chunkEnd", "segPtr", "segIdx", "rowInfo", "lightInfo", "heavyInfo", "ecol", "eval", "ecode", "dict")
+    scalars = ("nWG", "S", "sliceCols", "waves", "stepEntries", "batchEntries", "cap", "chunks", "batches", "vrows", "nLight", "nHeavy",
+               "lightSegs", "nDict")
+    dicts = 0
+    for i, A in enumerate(cases):
+        for ncu in ((256,) if A.nnz > 3000000 else (256, 7)):
+            print("layout case %d: rows=%d nnz=%d nCU=%d" % (i, A.rows, A.nnz, ncu), flush=True)
+            H = mx.slice_layout(A, nCU=ncu)
+            D = mx.slice_layout(A, nCU=ncu, device=True)
+            for k in scalars:
+                assert H[k] == D[k], (i, ncu, k, H[k], D[k])
+            for k in names:
+                assert H[k].shape == D[k].shape and np.array_equal(H[k].view(np.uint8), D[k].view(np.uint8)), (i, ncu, k)
+            dicts += H["nDict"] > 0
+    assert dicts >= 2
