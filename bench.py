@@ -120,9 +120,10 @@ def cpu_baseline(mx, ora, A, x):
     return base, allc
 
 
-def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=None):
+def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=None, keep=None):
     """mode: 'sweep' (the 5x5 grid), 'points' (CSR-only and two hybrid points) or 'csr' ((0,0) only)."""
     import numpy as np
+    keep = mx.MX_PLAN_KEEP_TILES if keep is None else keep
     t0 = time.time()
     A, x = mx.gen_config(cfg)
     log("workload %d: rows=%d nnz=%d generated in %.1fs" % (cfg, A.rows, A.nnz, time.time() - t0))
@@ -148,12 +149,12 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
         points = [(0.0, 0.0)]
     table = []
     if points is None:
-        _, _, tt = mx.tune_tau(A, levels=5, flags=mx.MX_PLAN_KEEP_TILES, warm=10, iters=100)
+        _, _, tt = mx.tune_tau(A, levels=5, flags=keep, warm=10, iters=100)
         table = [{"tau_c": c, "tau_r": r, "ms_total": ms, "tile_nnz": tn} for c, r, ms, tn in tt]
     else:
         for tau in points:
             part = mx.Partition(A, *tau, device=A.nnz >= (1 << 21) and tau != (0.0, 0.0))
-            plan = mx.Plan(part, mx.MX_PLAN_KEEP_TILES)
+            plan = mx.Plan(part, keep)
             ms = plan.time(xd, yd, warm=10, iters=100, parts=False)[0]
             table.append({"tau_c": tau[0], "tau_r": tau[1], "ms_total": ms, "tile_nnz": plan.info["tile_nnz"]})
             plan.close()
@@ -177,7 +178,7 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
         t0 = time.perf_counter()
         part = mx.Partition(A, *tau, device=device)
         t1 = time.perf_counter()
-        plan = mx.Plan(part, mx.MX_PLAN_KEEP_TILES)
+        plan = mx.Plan(part, keep)
         t2 = time.perf_counter()
         plan.spmv(xd, yd)
         torch.cuda.synchronize()
@@ -295,6 +296,8 @@ def main():
     ap.add_argument("--tau", type=float, nargs=2, metavar=("TAU_C", "TAU_R"), default=None,
                     help="no sweep: run this point (a profile of a fixed plan)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profile runs)")
+    ap.add_argument("--all-tiles", action="store_true",
+                    help="plans with MX_PLAN_ALL_TILES: every extracted chunk through the general MFMA tile kernel (profile runs)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also launch one elementwise kernel that reads and writes MIB MiB (a known size to "
                          "scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -318,7 +321,8 @@ def main():
         if args.no_sweep:
             return "csr"
         return "sweep" if cfg in SWEPT else "points"
-    main_rec, (A, x) = run_workload(mx, torch, ora, cfgs[0], args.steps, args.warmup, mode_of(cfgs[0]), traffic, args.tau)
+    keep = mx.MX_PLAN_ALL_TILES if args.all_tiles else None
+    main_rec, (A, x) = run_workload(mx, torch, ora, cfgs[0], args.steps, args.warmup, mode_of(cfgs[0]), traffic, args.tau, keep)
     out = {
         "metric": METRIC, "value": main_rec["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_rec["ms_per_step"],
@@ -368,7 +372,7 @@ def main():
         del src, dst
     others = {}
     for cfg in cfgs[1:]:
-        r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, mode_of(cfg), traffic, None)
+        r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, mode_of(cfg), traffic, None, keep)
         others["workload_%d" % cfg] = r
     if others:
         out["others"] = others

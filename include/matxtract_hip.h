@@ -244,6 +244,19 @@ double mx_algorithmic_bytes(mx_dtype dtype, int rows, int cols, int nnz);
 int mx_plan_create(const mx_partition *p, int flags, mx_plan **out);
 void mx_plan_destroy(mx_plan *plan);
 
+/* A plan for y = A x from a CSR matrix that already lives in device memory (the counterpart of
+ * mx_plan_create for the reference's tau = (0, 0) branch, test/test_autotc_spmv.cpp:1638-1658, where
+ * the whole matrix is the CSR part; the reference always starts from host arrays and uploads them
+ * on every call, src/spmv_kernel/cdSpMV.cu:407-418).  Every pointer is a device pointer; the arrays
+ * are read during the call and may be released after it.  The layouts are built on the device from
+ * the device arrays; of the matrix only the row pointers (row-tile form) or the lengths of its chunks
+ * (slice form) cross to the host.  The form is chosen as in mx_plan_create, from the same counts taken
+ * on the device: the plan, and with it every y, equals the one mx_plan_create makes from a partition
+ * of the same matrix with tau = (0, 0).  rowPtr_dev and colInd_dev are checked on the device before
+ * they are used as addresses (MX_ERR_ARG).  flags: MX_PLAN_CSR_ROWS, MX_PLAN_CSR_SLICES or 0. */
+int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
+                              const void *val_dev, int flags, mx_plan **out);
+
 /* y = A*x on the device.  x [cols] and y [rows] are DEVICE pointers of the plan's value
  * type, x 16-byte aligned (the kernels copy it in 16-byte vectors; a plan whose CSR part keeps
  * x in LDS returns MX_ERR_ARG otherwise, and reads the last 16-byte block of x whole when cols is

@@ -118,6 +118,7 @@ SIGNATURES = {
     "mx_gen_config": (_i, [_i, C.c_uint64, _d, _pi, _pi, _pi, _pi, _pp, _pp, _pp, _pp]),
     "mx_algorithmic_bytes": (_d, [_i, _i, _i, _i]),
     "mx_plan_create": (_i, [_vp, _i, _pp]),
+    "mx_plan_create_device_csr": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _i, _pp]),
     "mx_plan_destroy": (None, [_vp]),
     "mx_spmv": (_i, [_vp, _vp, _vp, _vp]),
     "mx_spmv_static": (_i, [_vp, _vp, _vp, _vp]),

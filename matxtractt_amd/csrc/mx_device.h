@@ -172,6 +172,14 @@ int build_slices_device(mx_dtype dtype, int rows, int cols, int nnz, const int *
                         int nCU, int S, const char *elsewhere_dev, DeviceSlices &D, hipStream_t s, std::vector<int> *segPtrOut = nullptr,
                         std::vector<int> *segIdxOut = nullptr);
 
+// For plans made from a matrix that lives in device memory: the caller's arrays looked at before
+// they are used as addresses; the mean number of distinct lines of x per wave-wide gather (sampled
+// as on the host); the row-tile form from device arrays (`desc` = pack_rows of the row pointers).
+int check_csr_device(int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, hipStream_t s, const char *who);
+int lines_per_gather_device(mx_dtype dtype, int nnz, const int *col_dev, hipStream_t s, double *out);
+int upload_csr_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, const void *val_dev,
+                      const std::vector<int> &desc, bool scan, DeviceCsr &A, hipStream_t s);
+
 // `what`: 0 = slice kernel then combine kernel, 1 = slice kernel only, 2 = combine kernel only
 // `strips` (optional): a tile layout in the dense binary16 form whose steps workgroups of the
 // combine kernel's launch run as well (strips_can_ride says whether a layout may); the rows of

@@ -124,11 +124,11 @@ __global__ __launch_bounds__(kBlock) void seg_ptr_kernel(const int *__restrict__
     segPtr[r] = p < nnz ? vid[p] : nV;
 }
 
-// the sort key of every virtual row -- (slice, cap - length, kind of its row) -- and the number of virtual rows per slice
+// the sort key of every virtual row: (slice, cap - length, kind of its row)
 __global__ __launch_bounds__(kBlock) void vrow_keys_kernel(const int *__restrict__ vStart, const int *__restrict__ vRow,
                                                            const int *__restrict__ vSlice, const int *__restrict__ segPtr, int nV,
                                                            int nnz, int cap, int lightSegs, unsigned *__restrict__ key,
-                                                           int *__restrict__ pay, int *__restrict__ vLen, int *__restrict__ sliceCount)
+                                                           int *__restrict__ pay, int *__restrict__ vLen)
 {
     const int t = blockIdx.x * kBlock + threadIdx.x;
     if (t >= nV) return;
@@ -138,7 +138,22 @@ __global__ __launch_bounds__(kBlock) void vrow_keys_kernel(const int *__restrict
     key[t] = ((unsigned)vSlice[t] * (unsigned)(cap + 1) + (unsigned)(cap - len)) * 3u + (unsigned)kind;
     pay[t] = t;
     vLen[t] = len;
-    atomicAdd(&sliceCount[vSlice[t]], 1);  // integer counts: the order does not matter
+}
+
+// sliceStart[q] = number of sorted keys that belong to slices before q, for q in [0, S]
+__global__ __launch_bounds__(kBlock) void slice_starts_kernel(const unsigned *__restrict__ sortedKey, int nV, int S, unsigned perSlice,
+                                                              int *__restrict__ sliceStart)
+{
+    const int q = blockIdx.x * kBlock + threadIdx.x;
+    if (q > S) return;
+    const unsigned long long want = (unsigned long long)q * perSlice;
+    int lo = 0, hi = nV;
+    while (lo < hi) {  // first position whose key is not below `want`
+        const int mid = (lo + hi) >> 1;
+        if ((unsigned long long)sortedKey[mid] < want) lo = mid + 1;
+        else hi = mid;
+    }
+    sliceStart[q] = lo;
 }
 
 __global__ __launch_bounds__(kBlock) void gather_len_kernel(const int *__restrict__ sorted, const int *__restrict__ vLen,
@@ -298,6 +313,65 @@ __global__ __launch_bounds__(kBlock) void value_codes_kernel(const V *__restrict
     code[k] = codeOf[lo];
 }
 
+// ---- statistics and the row-tile form from device arrays ----
+// bad |= 1 unless rowPtr rises from 0 to nnz; bad |= 2 for a column outside [0, cols)
+__global__ __launch_bounds__(kBlock) void check_csr_kernel(const int *__restrict__ rowPtr, const int *__restrict__ col, int rows, int cols,
+                                                           int nnz, int *__restrict__ bad)
+{
+    const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
+    if (i <= rows) {
+        const int p = rowPtr[i];
+        if ((i == 0 && p != 0) || (i == rows && p != nnz) || (i < rows && rowPtr[i + 1] < p) || p < 0 || p > nnz) atomicOr(bad, 1);
+    }
+    if (i < nnz && (unsigned)col[i] >= (unsigned)cols) atomicOr(bad, 2);
+}
+// sum += distinct 64-byte lines of x that the 64 entries of every stride-th window name (one thread per window)
+__global__ __launch_bounds__(kBlock) void window_lines_kernel(const int *__restrict__ col, long long sampled, long long stride, int perLine,
+                                                              unsigned long long *__restrict__ sum)
+{
+    const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= sampled) return;
+    const int *c = col + i * stride * 64;
+    int d = 0;
+    for (int a = 0; a < 64; ++a) {
+        const int la = c[a] / perLine;
+        bool seen = false;
+        for (int b = 0; b < a && !seen; ++b) seen = c[b] / perLine == la;
+        d += !seen;
+    }
+    atomicAdd(sum, (unsigned long long)d);
+}
+// one wave per workgroup of the row kernel: the lowest and the highest column of its entries
+__global__ __launch_bounds__(kBlock) void block_ranges_kernel(const int4 *__restrict__ desc, const int *__restrict__ col, int nBlocks,
+                                                              int *__restrict__ lo, int *__restrict__ wide)
+{
+    const int b = (blockIdx.x * kBlock + threadIdx.x) >> 6, lane = threadIdx.x & 63;
+    if (b >= nBlocks) return;
+    const int4 d = desc[b];
+    int mn = 0x7fffffff, mx_ = 0;
+    for (int p = d.z + lane; p < d.w; p += 64) {
+        mn = min(mn, col[p]);
+        mx_ = max(mx_, col[p]);
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        mn = min(mn, __shfl_xor(mn, o, 64));
+        mx_ = max(mx_, __shfl_xor(mx_, o, 64));
+    }
+    if (lane == 0) {
+        lo[b] = d.w > d.z ? mn : 0;
+        if (d.w > d.z && mx_ - mn > 65535) atomicOr(wide, 1);
+    }
+}
+__global__ __launch_bounds__(kBlock) void narrow_columns_kernel(const int4 *__restrict__ desc, const int *__restrict__ col,
+                                                                const int *__restrict__ lo, int nBlocks, unsigned short *__restrict__ c16)
+{
+    const int b = (blockIdx.x * kBlock + threadIdx.x) >> 6, lane = threadIdx.x & 63;
+    if (b >= nBlocks) return;
+    const int4 d = desc[b];
+    const int base = lo[b];
+    for (int p = d.z + lane; p < d.w; p += 64) c16[p] = (unsigned short)(col[p] - base);
+}
+
 inline dim3 grid(long long n) { return dim3((unsigned)((std::max<long long>(n, 1) + kBlock - 1) / kBlock)); }
 
 }  // namespace mxl
@@ -317,10 +391,10 @@ namespace mx {
 // most 255 distinct bit patterns, numbered in the order of their first entry; codes[nnz] (device)
 // and dict (256 values, host, zero-padded).  *nDict = 0 when the matrix has more.
 template <typename V>
-static int device_value_dict(const V *val, int nnz, mxl::Buf &codes, std::vector<unsigned char> &dict, int *nDict, hipStream_t s)
+static int device_value_dict(const V *val, int nnz, mxl::Buf &codes, std::vector<unsigned char> &dict, int *nDict, hipStream_t s,
+                             int most = 255, size_t codePad = 0)
 {
     using namespace mxl;
-    const int most = 255;
     *nDict = 0;
     {
         // most matrices have thousands of distinct values among their first entries: look there first
@@ -389,7 +463,8 @@ static int device_value_dict(const V *val, int nnz, mxl::Buf &codes, std::vector
     Buf dCodeOf;
     MXL_TRY(hipMalloc(&dCodeOf.p, 256));
     MXL_TRY(hipMemcpyAsync(dCodeOf.p, codeOf.data(), 256, hipMemcpyHostToDevice, s));
-    MXL_TRY(hipMalloc(&codes.p, (size_t)nnz));
+    MXL_TRY(hipMalloc(&codes.p, (size_t)nnz + codePad));
+    if (codePad) MXL_TRY(hipMemsetAsync((unsigned char *)codes.p + nnz, 0, codePad, s));
     hipLaunchKernelGGL(value_codes_kernel<V>, grid(nnz), dim3(kBlock), 0, s, val, nnz, (const unsigned long long *)tabVal.p,
                        (const unsigned char *)dCodeOf.p, nd, codes.as<unsigned char>());
     MXL_TRY(hipGetLastError());
@@ -494,8 +569,7 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
     MXL_TRY(hipMalloc(&keyOut.p, nv1 * 4));
     MXL_TRY(hipMalloc(&pay.p, nv1 * 4));
     MXL_TRY(hipMalloc(&sorted.p, nv1 * 4));
-    MXL_TRY(hipMalloc(&sliceCount.p, ((size_t)S + 1) * 4));
-    MXL_TRY(hipMemsetAsync(sliceCount.p, 0, ((size_t)S + 1) * 4, s));
+    MXL_TRY(hipMalloc(&sliceCount.p, ((size_t)S + 2) * 4));
     if (nnz > 0) {
         hipLaunchKernelGGL(vrow_records_kernel, grid(nnz), dim3(kBlock), 0, s, (const int *)start.p, (const int *)vid.p, (const int *)row.p,
                            col, (const int *)ord.p, nnz, SW, vStart.as<int>(), vRow.as<int>(), vSlice.as<int>());
@@ -507,8 +581,7 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
     std::vector<int> sliceCnt((size_t)S, 0);
     if (nV > 0) {
         hipLaunchKernelGGL(vrow_keys_kernel, grid(nV), dim3(kBlock), 0, s, (const int *)vStart.p, (const int *)vRow.p, (const int *)vSlice.p,
-                           (const int *)segPtr.p, nV, nnz, cap, kSliceLightSegs, key.as<unsigned>(), pay.as<int>(), vLen.as<int>(),
-                           sliceCount.as<int>());
+                           (const int *)segPtr.p, nV, nnz, cap, kSliceLightSegs, key.as<unsigned>(), pay.as<int>(), vLen.as<int>());
         MXL_TRY(hipGetLastError());
         unsigned keyBits = 1;
         while (keyBits < 32 && (1ull << keyBits) < (unsigned long long)S * (unsigned long long)(cap + 1) * 3ull) ++keyBits;
@@ -519,8 +592,13 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
         MXL_TRY(hipMalloc(&sortTmp.p, sortBytes + 256));
         MXL_TRY(rocprim::radix_sort_pairs(sortTmp.p, sortBytes, (const unsigned *)key.p, keyOut.as<unsigned>(), (const int *)pay.p,
                                           sorted.as<int>(), (size_t)nV, 0u, keyBits, s));
-        MXL_TRY(hipMemcpyAsync(sliceCnt.data(), sliceCount.p, (size_t)S * 4, hipMemcpyDeviceToHost, s));
+        hipLaunchKernelGGL(slice_starts_kernel, grid((long long)S + 1), dim3(kBlock), 0, s, (const unsigned *)keyOut.p, nV, S,
+                           (unsigned)(cap + 1) * 3u, sliceCount.as<int>());
+        MXL_TRY(hipGetLastError());
+        std::vector<int> sliceStart((size_t)S + 1, 0);
+        MXL_TRY(hipMemcpyAsync(sliceStart.data(), sliceCount.p, ((size_t)S + 1) * 4, hipMemcpyDeviceToHost, s));
         MXL_TRY(hipStreamSynchronize(s));
+        for (int q = 0; q < S; ++q) sliceCnt[q] = sliceStart[q + 1] - sliceStart[q];
     }
     // ---- chunks: their lengths come down, the plan of the streams goes up
     std::vector<std::vector<SliceChunk>> sliceChunks((size_t)S);
@@ -663,6 +741,112 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
     if (segIdxOut) {
         segIdxOut->assign(nv1, 0);
         MXL_TRY(hipMemcpyAsync(segIdxOut->data(), D.segIdx, nv1 * 4, hipMemcpyDeviceToHost, s));
+    }
+    MXL_TRY(hipStreamSynchronize(s));
+    return MX_OK;
+}
+
+int check_csr_device(int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, hipStream_t s, const char *who)
+{
+    using namespace mxl;
+    Buf bad;
+    MXL_TRY(hipMalloc(&bad.p, 256));
+    MXL_TRY(hipMemsetAsync(bad.p, 0, 256, s));
+    hipLaunchKernelGGL(check_csr_kernel, grid(std::max<long long>((long long)rows + 1, nnz)), dim3(kBlock), 0, s, rowPtr_dev, col_dev, rows,
+                       cols, nnz, bad.as<int>());
+    MXL_TRY(hipGetLastError());
+    int h = 0;
+    MXL_TRY(hipMemcpyAsync(&h, bad.p, 4, hipMemcpyDeviceToHost, s));
+    MXL_TRY(hipStreamSynchronize(s));
+    if (h) {
+        set_error(std::string(who) + ((h & 1) ? ": rowPtr does not rise from 0 to nnz" : ": column index out of range"));
+        return MX_ERR_ARG;
+    }
+    return MX_OK;
+}
+
+int lines_per_gather_device(mx_dtype dtype, int nnz, const int *col_dev, hipStream_t s, double *out)
+{
+    using namespace mxl;
+    const long long windows = nnz / 64, stride = std::max<long long>(1, windows / 65536), sampled = windows / stride;
+    *out = 1.0;
+    if (sampled <= 0) return MX_OK;
+    Buf sum;
+    MXL_TRY(hipMalloc(&sum.p, 256));
+    MXL_TRY(hipMemsetAsync(sum.p, 0, 256, s));
+    hipLaunchKernelGGL(window_lines_kernel, grid(sampled), dim3(kBlock), 0, s, col_dev, sampled, stride, 64 / elem_size(dtype),
+                       sum.as<unsigned long long>());
+    MXL_TRY(hipGetLastError());
+    unsigned long long h = 0;
+    MXL_TRY(hipMemcpyAsync(&h, sum.p, 8, hipMemcpyDeviceToHost, s));
+    MXL_TRY(hipStreamSynchronize(s));
+    *out = (double)h / (double)sampled;
+    return MX_OK;
+}
+
+// The row-tile form (DeviceCsr) of a CSR matrix in device memory: what upload_csr makes from host
+// arrays.  `desc` = the workgroups' row ranges (pack_rows, made on the host from the row pointers).
+int upload_csr_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, const void *val_dev,
+                      const std::vector<int> &desc, bool scan, DeviceCsr &A, hipStream_t s)
+{
+    using namespace mxl;
+    const size_t es = (size_t)elem_size(dtype);
+    A = DeviceCsr();
+    A.rows = rows;
+    A.cols = cols;
+    A.nnz = nnz;
+    A.npt = csr_entries_per_lane(dtype);
+    A.scan = scan;
+    A.nBlocks = (int)desc.size() / 4;
+    MXL_TRY(hipMalloc((void **)&A.rowPtr, ((size_t)rows + 1) * 4));
+    MXL_TRY(hipMemcpyAsync(A.rowPtr, rowPtr_dev, ((size_t)rows + 1) * 4, hipMemcpyDeviceToDevice, s));
+    MXL_TRY(hipMalloc(&A.val, ((size_t)nnz + kCsrPad) * es));
+    MXL_TRY(hipMemsetAsync((unsigned char *)A.val + (size_t)nnz * es, 0, (size_t)kCsrPad * es, s));
+    if (nnz) MXL_TRY(hipMemcpyAsync(A.val, val_dev, (size_t)nnz * es, hipMemcpyDeviceToDevice, s));
+    MXL_TRY(hipMalloc((void **)&A.blockDesc, std::max<size_t>(desc.size(), 4) * 4));
+    if (!desc.empty()) MXL_TRY(hipMemcpyAsync(A.blockDesc, desc.data(), desc.size() * 4, hipMemcpyHostToDevice, s));
+    const char *env16 = std::getenv("MX_CSR_COL16");
+    bool narrow = !(env16 && std::atoi(env16) == 0) && nnz > 0;
+    Buf lo, wide;
+    if (narrow) {
+        MXL_TRY(hipMalloc(&lo.p, std::max<size_t>((size_t)A.nBlocks, 1) * 4));
+        MXL_TRY(hipMalloc(&wide.p, 256));
+        MXL_TRY(hipMemsetAsync(wide.p, 0, 256, s));
+        hipLaunchKernelGGL(block_ranges_kernel, grid((long long)A.nBlocks * 64), dim3(kBlock), 0, s, (const int4 *)A.blockDesc, col_dev,
+                           A.nBlocks, lo.as<int>(), wide.as<int>());
+        MXL_TRY(hipGetLastError());
+        int w = 0;
+        MXL_TRY(hipMemcpyAsync(&w, wide.p, 4, hipMemcpyDeviceToHost, s));
+        MXL_TRY(hipStreamSynchronize(s));
+        narrow = w == 0;
+    }
+    if (narrow) {
+        MXL_TRY(hipMalloc((void **)&A.col16, ((size_t)nnz + kCsrPad) * 2));
+        MXL_TRY(hipMemsetAsync(A.col16 + nnz, 0, (size_t)kCsrPad * 2, s));
+        hipLaunchKernelGGL(narrow_columns_kernel, grid((long long)A.nBlocks * 64), dim3(kBlock), 0, s, (const int4 *)A.blockDesc, col_dev,
+                           (const int *)lo.p, A.nBlocks, A.col16);
+        MXL_TRY(hipGetLastError());
+        A.colBase = (int *)lo.take();
+        const char *ed = std::getenv("MX_CSR_DICT");
+        if (nnz >= 65536 && !(ed && !std::atoi(ed))) {
+            Buf codes;
+            std::vector<unsigned char> dict;
+            int nd = 0, rc;
+            if (dtype == MX_F64) rc = device_value_dict<double>((const double *)val_dev, nnz, codes, dict, &nd, s, 256, kCsrPad);
+            else rc = device_value_dict<_Float16>((const _Float16 *)val_dev, nnz, codes, dict, &nd, s, 256, kCsrPad);
+            if (rc) return rc;
+            if (nd > 0) {
+                A.codes = (unsigned char *)codes.take();
+                MXL_TRY(hipMalloc(&A.dict, dict.size()));
+                MXL_TRY(hipMemcpyAsync(A.dict, dict.data(), dict.size(), hipMemcpyHostToDevice, s));
+                MXL_TRY(hipStreamSynchronize(s));
+                A.nDict = nd;
+            }
+        }
+    } else {
+        MXL_TRY(hipMalloc((void **)&A.col, ((size_t)nnz + kCsrPad) * 4));
+        MXL_TRY(hipMemsetAsync(A.col + nnz, 0, (size_t)kCsrPad * 4, s));
+        if (nnz) MXL_TRY(hipMemcpyAsync(A.col, col_dev, (size_t)nnz * 4, hipMemcpyDeviceToDevice, s));
     }
     MXL_TRY(hipStreamSynchronize(s));
     return MX_OK;

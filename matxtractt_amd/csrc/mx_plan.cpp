@@ -2026,6 +2026,110 @@ static int create_plan(const mx_partition *P, int flags, mx_plan **out, bool noB
     return MX_OK;
 }
 
+// A plan for y = A x from a CSR matrix that lives in device memory: nothing of the matrix crosses
+// to the host but its row pointers (for the row-tile form) or the lengths of its chunks (for the
+// slice form).  The form is chosen as in mx_plan_create -- the same counts, taken on the device --
+// so the plan equals the one mx_plan_create makes from a partition of the same matrix with
+// tau = (0, 0).
+extern "C" int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
+                                         const void *val_dev, int flags, mx_plan **out)
+{
+    if (!out || (dtype != MX_F64 && dtype != MX_F16) || rows < 0 || cols < 0 || nnz < 0 || !rowPtr_dev ||
+        (nnz > 0 && (!colInd_dev || !val_dev || rows == 0 || cols == 0))) {
+        set_error("mx_plan_create_device_csr: bad argument");
+        return MX_ERR_ARG;
+    }
+    *out = nullptr;
+    int rc = need_device();
+    if (rc) return rc;
+    if ((rc = mx::check_csr_device(rows, cols, nnz, rowPtr_dev, colInd_dev, nullptr, "mx_plan_create_device_csr"))) return rc;
+    mx_plan *plan = new (std::nothrow) mx_plan();
+    if (!plan) {
+        set_error("mx_plan_create_device_csr: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    plan->dtype = dtype;
+    plan->rows = rows;
+    plan->cols = cols;
+    plan->nnz = nnz;
+    plan->csr_nnz = nnz;
+    auto fail = [&](int code) {
+        mx_plan_destroy(plan);
+        return code;
+    };
+    if (hipStreamCreate(&plan->stream) != hipSuccess || hipEventCreate(&plan->ev0) != hipSuccess ||
+        hipEventCreate(&plan->ev1) != hipSuccess) {
+        set_error("mx_plan_create_device_csr: could not create stream/events");
+        return fail(MX_ERR_DEVICE);
+    }
+    {
+        void *fixed = nullptr;
+        if (mx::static_scratch(&fixed) != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("mx_plan_create_device_csr: hipGetSymbolAddress failed for the fixed array of sums");
+            return fail(MX_ERR_DEVICE);
+        }
+    }
+    try {
+        hipDeviceProp_t prop;
+        int dev = 0;
+        MX_HIP(hipGetDevice(&dev));
+        MX_HIP(hipGetDeviceProperties(&prop, dev));
+        const int nCU = std::max(1, prop.multiProcessorCount);
+        const int S = rows > 0 ? slice_count(dtype, rows, cols, nnz, nCU) : 0;
+        bool want[2] = {true, S > 0};
+        const char *env = std::getenv("MX_CSR_KERNEL");
+        if (flags & MX_PLAN_CSR_ROWS) want[1] = false;
+        if ((flags & MX_PLAN_CSR_SLICES) && S > 0) want[0] = false;
+        if (env && !std::strcmp(env, "rows")) want[0] = true, want[1] = false;
+        if (env && !std::strcmp(env, "slices") && S > 0) want[1] = true, want[0] = false;
+        if (want[1]) {
+            rc = mx::build_slices_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, nCU, S, nullptr, plan->slices, nullptr);
+            if (rc) return fail(rc);
+            if (plan->slices.ecode) plan->slices.useDict = true;
+        }
+        if (want[0] && want[1]) {
+            // the estimates of csr_estimates from what the device counted: the virtual rows are those of
+            // the layout just made, the one-byte form exists when the layout has it
+            CsrStats st;
+            st.vrows = plan->slices.vrows;
+            st.fewValues = plan->slices.ecode != nullptr;
+            if ((rc = mx::lines_per_gather_device(dtype, nnz, colInd_dev, nullptr, &st.linesPerGather))) return fail(rc);
+            csr_estimates(dtype, cols, nnz, st, &plan->est_rows_us, &plan->est_slices_us);
+            want[plan->est_slices_us < plan->est_rows_us ? 0 : 1] = false;
+        }
+        if (want[1]) {
+            plan->csr_variant = 1;
+        } else {
+            free_slices(plan->slices);
+            plan->csr_variant = 0;
+            std::vector<int> rp((size_t)rows + 1, 0), desc;
+            MX_HIP(hipMemcpy(rp.data(), rowPtr_dev, ((size_t)rows + 1) * 4, hipMemcpyDeviceToHost));
+            const int npt = mx::csr_entries_per_lane(dtype);
+            pack_rows(rp.data(), rows, npt, desc);
+            double sum = 0.0, sq = 0.0;
+            for (int r = 0; r < rows; ++r) {
+                const double n = rp[r + 1] - rp[r];
+                sum += n;
+                sq += n * n;
+            }
+            const double mean = rows > 0 ? sum / rows : 0.0, var = rows > 0 ? sq / rows - mean * mean : 0.0;
+            bool scan = mean > 0.0 && var > 0.25 * mean * mean;
+            const char *envr = std::getenv("MX_CSR_REDUCE");
+            if (envr && !std::strcmp(envr, "rows")) scan = false;
+            if (envr && !std::strcmp(envr, "scan")) scan = true;
+            rc = mx::upload_csr_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, desc, scan, plan->csr, nullptr);
+            if (rc) return fail(rc);
+            if (plan->csr.codes) plan->csr.useDict = true;
+        }
+    } catch (const std::bad_alloc &) {
+        set_error("mx_plan_create_device_csr: out of memory");
+        return fail(MX_ERR_ALLOC);
+    }
+    *out = plan;
+    return MX_OK;
+}
+
 extern "C" void mx_plan_layout_free(mx_plan_layout_view *v)
 {
     if (!v) return;

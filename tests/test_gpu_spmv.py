@@ -1192,3 +1192,49 @@ def test_slice_layout_by_the_device_route_is_the_same_layout(mx, monkeypatch):
                 assert H[k].shape == D[k].shape and np.array_equal(H[k].view(np.uint8), D[k].view(np.uint8)), (i, ncu, k)
             dicts += H["nDict"] > 0
     assert dicts >= 2
+
+
+@pytest.mark.gpu
+def test_plan_from_a_matrix_in_device_memory(mx, ora):
+    """mx_plan_create_device_csr: the plan made from device arrays alone is the plan mx_plan_create
+    makes from the host matrix -- same form, same estimates behind the choice, same value
+    dictionary, and a y that is equal bit for bit -- in both forms and both precisions, on rows in
+    any order; a bad index is refused before it is used."""
+    import torch
+    rng = np.random.default_rng(5)
+    cases = [mx.gen_config(c, scale=sc)[0] for c, sc in ((1, 1.0), (2, 1.0), (2, 1 / 8), (3, 0.1), (4, 0.25), (5, 0.1))]
+    lens = rng.integers(0, 60, 5000)
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cases.append(mx.Csr(5000, 90000, ptr, rng.integers(0, 90000, ptr[-1]).astype(np.int32), rng.integers(-4, 5, ptr[-1]).astype(np.float64)))
+    seen = set()
+    for i, A in enumerate(cases):
+        x = rng.uniform(-1, 1, A.cols).astype(A.val.dtype)
+        xd = torch.from_numpy(x).cuda()
+        rp, ci, va = torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda()
+        ref = oracle_y(ora, mx, A, x)
+        part = mx.Partition(A, 0.0, 0.0)
+        for flags in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_CSR_ROWS, mx.MX_PLAN_CSR_SLICES):
+            print("device csr plan: case %d rows=%d nnz=%d flags=%d" % (i, A.rows, A.nnz, flags), flush=True)
+            H = mx.Plan(part, flags)
+            D = mx.Plan.from_device_csr(rp, ci, va, A.cols, flags)
+            for k in ("csr_variant", "csr_value_dict", "csr_nnz", "csr_blocks", "tile_nnz"):
+                assert H.info[k] == D.info[k], (i, flags, k, H.info[k], D.info[k])
+            if flags == mx.MX_PLAN_DEFAULT and H.info["est_rows_us"] > 0:
+                assert abs(H.info["est_rows_us"] - D.info["est_rows_us"]) < 1e-9 and abs(H.info["est_slices_us"] - D.info["est_slices_us"]) < 1e-9
+            yh, yd = H.spmv(xd).cpu().numpy(), D.spmv(xd).cpu().numpy()
+            assert np.array_equal(yh.view(np.uint8), yd.view(np.uint8)), (i, flags)
+            assert rel_l2(yd, ref) <= (F64_TOL if A.dtype == mx.MX_F64 else F16_TOL)
+            seen.add((D.info["csr_variant"], D.info["csr_value_dict"] > 0))
+            H.close()
+            D.close()
+        part.close()
+    assert {(0, False), (1, False), (1, True), (0, True)} <= seen, seen
+    bad = ci.clone()
+    bad[11] = A.cols
+    with pytest.raises(mx.MxError) as e:
+        mx.Plan.from_device_csr(rp, bad, va, A.cols)
+    assert e.value.code == 1
+    badp = rp.clone()
+    badp[5] = badp[6] + 1
+    with pytest.raises(mx.MxError):
+        mx.Plan.from_device_csr(badp, ci, va, A.cols)
