@@ -8,6 +8,9 @@ hipError_t launch_slices(mx_dtype, const DeviceSlices &, const void *, void *, i
 hipError_t static_scratch(void **p) { *p = nullptr; return hipErrorUnknown; }
 int build_slices_device(mx_dtype, int, int, int, const int *, const int *, const void *, int, int, const char *, DeviceSlices &, hipStream_t,
                         std::vector<int> *, std::vector<int> *) { return MX_ERR_DEVICE; }
+int check_csr_device(int, int, int, const int *, const int *, hipStream_t, const char *) { return MX_ERR_DEVICE; }
+int lines_per_gather_device(mx_dtype, int, const int *, hipStream_t, double *) { return MX_ERR_DEVICE; }
+int upload_csr_device(mx_dtype, int, int, int, const int *, const int *, const void *, const std::vector<int> &, bool, DeviceCsr &, hipStream_t) { return MX_ERR_DEVICE; }
 bool strips_can_ride(mx_dtype, const DeviceTiles &, const void *) { return false; }
 hipError_t launch_probe_f64(const double *, const double *, double *, hipStream_t) { return hipErrorUnknown; }
 hipError_t launch_probe_f16(const void *, const void *, float *, hipStream_t) { return hipErrorUnknown; }
