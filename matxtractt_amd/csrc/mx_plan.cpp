@@ -7,6 +7,8 @@
 #include <cstdio>
 #include <cstring>
 #include <numeric>
+#include <omp.h>
+#include <parallel/algorithm>
 #include <queue>
 #include <vector>
 
@@ -1615,46 +1617,78 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
             int nb, b[kMaxBlocks], n, i;  // blocks (column / fragK, ascending), entries, row of A_dd
         };
         std::vector<Cand> cand;
-        std::vector<int> cols;
-        for (int i = 0; i < P->dRows; ++i) {
-            const int p0 = P->ddRowPtr[i], n = P->ddRowPtr[i + 1] - p0, r = P->rId[i];
-            if (n < fragK / 2 || n > kMaxBlocks * fragK || P->cdRowPtr[r + 1] != P->cdRowPtr[r]) continue;
-            cols.resize((size_t)n);
-            for (int k = 0; k < n; ++k) cols[k] = P->descColId[P->ddColInd[p0 + k]];
-            std::sort(cols.begin(), cols.end());
-            Cand c;
-            c.nb = 0;
-            c.n = n;
-            c.i = i;
-            bool ok = true;
-            for (int k = 0; k < n && ok; ++k) {
-                if (k && cols[k] == cols[k - 1]) ok = false;  // named twice: stays with the fragments, where the last counts
-                const int blk = cols[k] / fragK;
-                if ((blk + 1) * fragK > P->cols) ok = false;  // the block would reach past the end of x
-                if (c.nb == 0 || c.b[c.nb - 1] != blk) {
-                    if (c.nb == kMaxBlocks) ok = false;
-                    else c.b[c.nb++] = blk;
+        const int nThreads = std::max(1, omp_get_max_threads());
+        std::vector<std::vector<Cand>> found((size_t)nThreads);
+#pragma omp parallel num_threads(nThreads)
+        {
+            std::vector<Cand> &mine = found[(size_t)omp_get_thread_num()];
+            std::vector<int> cols;
+#pragma omp for schedule(static)
+            for (int i = 0; i < P->dRows; ++i) {
+                const int p0 = P->ddRowPtr[i], n = P->ddRowPtr[i + 1] - p0, r = P->rId[i];
+                if (n < fragK / 2 || n > kMaxBlocks * fragK || P->cdRowPtr[r + 1] != P->cdRowPtr[r]) continue;
+                cols.resize((size_t)n);
+                for (int k = 0; k < n; ++k) cols[k] = P->descColId[P->ddColInd[p0 + k]];
+                std::sort(cols.begin(), cols.end());
+                Cand c;
+                c.nb = 0;
+                c.n = n;
+                c.i = i;
+                bool ok = true;
+                for (int k = 0; k < n && ok; ++k) {
+                    if (k && cols[k] == cols[k - 1]) ok = false;  // named twice: stays with the fragments, where the last counts
+                    const int blk = cols[k] / fragK;
+                    if ((blk + 1) * fragK > P->cols) ok = false;  // the block would reach past the end of x
+                    if (c.nb == 0 || c.b[c.nb - 1] != blk) {
+                        if (c.nb == kMaxBlocks) ok = false;
+                        else c.b[c.nb++] = blk;
+                    }
                 }
+                if (!ok || 2 * n < c.nb * fragK) continue;
+                for (int k = c.nb; k < kMaxBlocks; ++k) c.b[k] = -1;
+                mine.push_back(c);
             }
-            if (!ok || 2 * n < c.nb * fragK) continue;
-            for (int k = c.nb; k < kMaxBlocks; ++k) c.b[k] = -1;
-            cand.push_back(c);
         }
+        for (const std::vector<Cand> &f : found) cand.insert(cand.end(), f.begin(), f.end());
+        found.clear();
         auto same = [](const Cand &x, const Cand &y) { return x.nb == y.nb && std::equal(x.b, x.b + kMaxBlocks, y.b); };
-        std::sort(cand.begin(), cand.end(), [](const Cand &x, const Cand &y) {
+        // (a total order -- no two candidates share a row -- so the result does not depend on how the sort splits its work)
+        __gnu_parallel::sort(cand.begin(), cand.end(), [](const Cand &x, const Cand &y) {
             if (!std::equal(x.b, x.b + kMaxBlocks, y.b)) return std::lexicographical_compare(x.b, x.b + kMaxBlocks, y.b, y.b + kMaxBlocks);
             return x.i < y.i;
         });
         taken.assign((size_t)P->dRows, 0);
         const uint16_t *ddv16 = (const uint16_t *)P->ddVal.data();  // binary16 bit patterns
+        // runs of candidates with the same blocks, and the first chunk of each
+        std::vector<size_t> runStart;
+        std::vector<size_t> runChunk0;
+        size_t nStripChunks = 0;
         for (size_t a = 0; a < cand.size();) {
             size_t b = a;
             while (b < cand.size() && same(cand[b], cand[a])) ++b;
-            for (size_t g = a; g < b; g += fragM) {
+            const size_t full = (b - a) / fragM, rest = (b - a) % fragM;
+            const size_t n = full + (2 * rest >= (size_t)fragM ? 1 : 0);
+            if (n) {
+                runStart.push_back(a);
+                runChunk0.push_back(nStripChunks);
+                nStripChunks += n;
+            }
+            a = b;
+        }
+        runStart.push_back(cand.size());
+        runChunk0.push_back(nStripChunks);
+        stripChunks.resize(nStripChunks);
+        const long nRuns = (long)runChunk0.size() - 1;
+#pragma omp parallel for schedule(dynamic, 16)
+        for (long run = 0; run < nRuns; ++run) {
+            const size_t a = runStart[run];
+            const int nb = cand[a].nb;
+            size_t b = a;
+            while (b < cand.size() && same(cand[b], cand[a])) ++b;
+            for (size_t q = 0; q < runChunk0[run + 1] - runChunk0[run]; ++q) {
+                const size_t g = a + q * fragM;
                 const int nr = (int)std::min(b - g, (size_t)fragM);
-                if (2 * nr < fragM) break;
-                StripChunk C;
-                const int nb = cand[a].nb;
+                StripChunk &C = stripChunks[runChunk0[run] + q];
                 C.nnz = 0;
                 C.blocks.resize(nb);
                 for (int k = 0; k < nb; ++k) {
@@ -1673,9 +1707,7 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
                         ((uint16_t *)C.blocks[k].vals.data())[j * fragK + c % fragK] = ddv16[p];
                     }
                 }
-                stripChunks.push_back(std::move(C));
             }
-            a = b;
         }
         if (stripChunks.empty()) taken.clear();
     }
