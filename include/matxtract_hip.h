@@ -257,6 +257,37 @@ void mx_plan_destroy(mx_plan *plan);
 int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
                               const void *val_dev, int flags, mx_plan **out);
 
+/* The whole preparation of the reference's driver on the device, for a CSR matrix that lives in
+ * device memory: the cascaded extraction with tau_c / tau_r (test/test_autotc_spmv.cpp:1099-1300),
+ * the tile encoding (:1352-1421), and what mx_plan_create does with the result -- the fill gate of
+ * the fragments, the search for rows of dense binary16 strips and their chunks, the question whether
+ * the tiles pay, the CSR part in the caller's numbering with its layout, the strips' steps.  Nothing
+ * of the matrix crosses to the host: decisions are made there from counts (fragments and entries
+ * that pass the gate, blocks and entries per strip chunk, lengths of the slice layout's chunks).
+ * The plan equals -- array for array, and so y bit for bit -- the one mx_plan_create makes from
+ * mx_partition_create of the same matrix with the same fractions and flags.  Two tile forms are not
+ * laid out on the device, the general one and the binary64 8 x 8 blocks; they are counted there, and
+ * a matrix on which the plan keeps one of them (with default flags none of the workloads measured;
+ * always with MX_PLAN_ALL_TILES) is copied to the host and goes through mx_partition_create_device
+ * and mx_plan_create -- mx_plan_info.prep_route says which way a plan came.  Every pointer is a
+ * device pointer; the arrays are read during the call and may be released after it; rowPtr_dev and
+ * colInd_dev are checked on the device before they are used as addresses (MX_ERR_ARG).
+ * tau = (0, 0) is mx_plan_create_device_csr. */
+int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
+                          const void *val_dev, float tau_c, float tau_r, int flags, mx_plan **out);
+
+/* Every device array of a plan copied to host memory, each with a name ("slices.ecol",
+ * "strips.hdr", ...) and its size: for tests that hold two routes of making a plan against each
+ * other.  `out` has room for `cap` entries (32 is enough); *n receives their number; the data
+ * pointers are malloc()ed and mx_plan_arrays_free releases them.  No counterpart in the reference. */
+typedef struct mx_plan_array {
+    const char *name;
+    size_t bytes;
+    void *data;
+} mx_plan_array;
+int mx_plan_arrays(const mx_plan *plan, mx_plan_array *out, int cap, int *n);
+void mx_plan_arrays_free(mx_plan_array *a, int n);
+
 /* y = A*x on the device.  x [cols] and y [rows] are DEVICE pointers of the plan's value
  * type, x 16-byte aligned (the kernels copy it in 16-byte vectors; a plan whose CSR part keeps
  * x in LDS returns MX_ERR_ARG otherwise, and reads the last 16-byte block of x whole when cols is
@@ -374,6 +405,12 @@ typedef struct mx_plan_info {
                             MI355X (both 0 when a flag, MX_CSR_KERNEL or the shape of the matrix left no choice).
                             Nothing is timed unless MX_PLAN_AUTOTUNE=1 is set, so a matrix gets the same plan on
                             every run */
+    int prep_route;      /* where the plan's layouts were made: 0 = from host arrays (mx_plan_create), 1 = on the
+                            device from device arrays (mx_plan_create_device, mx_plan_create_device_csr), 2 =
+                            mx_plan_create_device copied the matrix to the host and took the host route */
+    int ext_dCols, ext_dRows, ext_nnzRowD, ext_frags; /* what the extraction behind the plan selected (columns, rows,
+                            entries of A_dd) and the fragments of its tile encoding -- cols_ratio and TC_nnz_ratio of
+                            the reference's driver follow from them; 0 for plans without an extraction */
 } mx_plan_info;
 int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
 

@@ -52,7 +52,13 @@ class PlanInfo(C.Structure):
                 ("csr_nnz", C.c_int), ("csr_blocks", C.c_int), ("csr_variant", C.c_int),
                 ("tile_bytes", C.c_double), ("csr_bytes", C.c_double),
                 ("csr_main_kernel", C.c_int), ("csr_main_nnz", C.c_int), ("tile_variant", C.c_int), ("tile_strip_nnz", C.c_int),
-                ("csr_value_dict", C.c_int), ("est_rows_us", C.c_double), ("est_slices_us", C.c_double)]
+                ("csr_value_dict", C.c_int), ("est_rows_us", C.c_double), ("est_slices_us", C.c_double),
+                ("prep_route", C.c_int), ("ext_dCols", C.c_int), ("ext_dRows", C.c_int), ("ext_nnzRowD", C.c_int),
+                ("ext_frags", C.c_int)]
+
+
+class PlanArray(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("bytes", C.c_size_t), ("data", C.c_void_p)]
 
 
 class SliceLayoutView(C.Structure):
@@ -119,6 +125,9 @@ SIGNATURES = {
     "mx_algorithmic_bytes": (_d, [_i, _i, _i, _i]),
     "mx_plan_create": (_i, [_vp, _i, _pp]),
     "mx_plan_create_device_csr": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _i, _pp]),
+    "mx_plan_create_device": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, C.c_float, C.c_float, _i, _pp]),
+    "mx_plan_arrays": (_i, [_vp, _vp, _i, _vp]),
+    "mx_plan_arrays_free": (None, [_vp, _i]),
     "mx_plan_destroy": (None, [_vp]),
     "mx_spmv": (_i, [_vp, _vp, _vp, _vp]),
     "mx_spmv_static": (_i, [_vp, _vp, _vp, _vp]),

@@ -396,6 +396,41 @@ class Plan:
         self.dtype, self.rows, self.cols, self.nnz = info.dtype, info.rows, info.cols, info.nnz
         return self
 
+    @classmethod
+    def from_device(cls, rowPtr, colInd, val, cols, tau_c, tau_r, flags=MX_PLAN_DEFAULT):
+        """A hybrid plan from a CSR matrix held in torch device tensors and the two extraction
+        fractions: mx_plan_create_device -- extraction, decisions and layouts on the device."""
+        import torch
+        for name, t in (("rowPtr", rowPtr), ("colInd", colInd)):
+            if (not t.is_cuda) or t.dtype != torch.int32 or not t.is_contiguous():
+                raise ValueError("%s must be a contiguous int32 device tensor" % name)
+        if (not val.is_cuda) or val.dtype not in (torch.float64, torch.float16) or not val.is_contiguous() \
+                or val.numel() != colInd.numel():
+            raise ValueError("val must be a contiguous float64 or float16 device tensor as long as colInd")
+        self = cls.__new__(cls)
+        self._h = C.c_void_p()
+        dt = MX_F64 if val.dtype == torch.float64 else MX_F16
+        check(_lib.load().mx_plan_create_device(dt, rowPtr.numel() - 1, int(cols), colInd.numel(), rowPtr.data_ptr(),
+                                                colInd.data_ptr(), val.data_ptr(), float(tau_c), float(tau_r), int(flags),
+                                                C.byref(self._h)))
+        info = _lib.PlanInfo()
+        check(_lib.load().mx_plan_get_info(self._h, C.byref(info)))
+        self.info = {k: getattr(info, k) for k, _ in _lib.PlanInfo._fields_}
+        self.dtype, self.rows, self.cols, self.nnz = info.dtype, info.rows, info.cols, info.nnz
+        return self
+
+    def arrays(self):
+        """{name: bytes} of every device array of the plan (mx_plan_arrays), for tests that compare
+        two routes of making a plan."""
+        cap = 48
+        buf = (_lib.PlanArray * cap)()
+        n = C.c_int(0)
+        check(_lib.load().mx_plan_arrays(self._h, buf, cap, C.byref(n)))
+        try:
+            return {buf[i].name.decode(): C.string_at(buf[i].data, buf[i].bytes) for i in range(n.value)}
+        finally:
+            _lib.load().mx_plan_arrays_free(buf, n.value)
+
     def _check_vec(self, t, n, name):
         if (not t.is_cuda) or t.dtype != _torch_dtype(self.dtype) or t.numel() != n or not t.is_contiguous():
             raise ValueError("%s must be a contiguous device tensor of %d %s" % (name, n, _torch_dtype(self.dtype)))

@@ -10,7 +10,10 @@
 // last line), --tune (pick the two fractions from the 5x5 grid by timing each on the device,
 // then run with them), --partition-cache FILE (read the partition from FILE when it was made for a
 // matrix of this shape with these fractions, otherwise compute it and write FILE), --device-prep (the extraction runs on the GPU instead of the
-// host cores; same partition).  Precision is the build's: -Dfp64 -> FP64 binary, otherwise FP16.
+// host cores; same partition), --device-plan (the matrix is uploaded as it is and everything after
+// that -- extraction, the plan's decisions, its layouts -- happens on the GPU: mx_plan_create_device;
+// same plan, no partition on the host, so no --partition-cache and no checksum in the JSON record).
+// Precision is the build's: -Dfp64 -> FP64 binary, otherwise FP16.
 //
 // Lines other tools parse (ML/bayes_opt.py:64, script/duse.sh:35-38) keep their form:
 //   cols_ratio = %f / TC_nnz_ratio = %lf / MatXtract time = %lf ms / Success! ... |
@@ -94,7 +97,7 @@ int main(int argc, char **argv)
     int config = 0, warm = 200, iters = 4000, planFlags = MX_PLAN_DEFAULT;
     double scale = 1.0;
     unsigned long long seed = 0;
-    bool keepValues = false, json = false, tune = false, devicePrep = false;
+    bool keepValues = false, json = false, tune = false, devicePrep = false, devicePlan = false;
     std::string cachePath;
     for (int i = 1; i < argc; ++i) {
         std::string a = argv[i];
@@ -118,6 +121,7 @@ int main(int argc, char **argv)
         else if (a == "--partition-cache") cachePath = next("--partition-cache");
         else if (a == "--tune") tune = true;
         else if (a == "--device-prep") devicePrep = true;
+        else if (a == "--device-plan") devicePlan = true;
         else pos.push_back(a);
     }
     const size_t npos = pos.size() + (config ? 1 : 0);  // a --config stands for the file name
@@ -205,38 +209,70 @@ int main(int argc, char **argv)
     }
     auto t0 = std::chrono::steady_clock::now();
     mx_partition *part = nullptr;
-    bool fromCache = false;
-    if (!cachePath.empty() && mx_partition_load(cachePath.c_str(), MX_VALT_DTYPE, &part) == MX_OK) {
-        // The file is used only if it was made from a matrix of this shape with these fractions.
-        mx_partition_view cv;
-        mx_partition_get(part, &cv);
-        fromCache = cv.rows == rowA && cv.cols == colA && cv.nnz == (long long)nnzA && cv.tau_c == colProp && cv.tau_r == rowProp;
-        if (!fromCache) {
-            mx_partition_destroy(part);
-            part = nullptr;
+    mx_plan *plan = nullptr;
+    mx_plan_info info;
+    mx_partition_view pv{};
+    double preprocess_ms = 0.0;
+    if (devicePlan) {
+        if (!cachePath.empty()) {
+            printf("Error: --device-plan keeps no partition on the host; it cannot be combined with --partition-cache.\n");
+            return 1;
         }
+        // the matrix goes up as it is; extraction, decisions and layouts are made on the device
+        void *dRowPtr = nullptr, *dColInd = nullptr, *dVal = nullptr;
+        const size_t nz = (size_t)(nnzA > 0 ? nnzA : 1);
+        if (hipMalloc(&dRowPtr, sizeof(indT) * ((size_t)rowA + 1)) != hipSuccess || hipMalloc(&dColInd, sizeof(indT) * nz) != hipSuccess ||
+            hipMalloc(&dVal, sizeof(valT) * nz) != hipSuccess ||
+            hipMemcpy(dRowPtr, csrRowPtr, sizeof(indT) * ((size_t)rowA + 1), hipMemcpyHostToDevice) != hipSuccess ||
+            hipMemcpy(dColInd, csrColInd, sizeof(indT) * (size_t)nnzA, hipMemcpyHostToDevice) != hipSuccess ||
+            hipMemcpy(dVal, csrVal, sizeof(valT) * (size_t)nnzA, hipMemcpyHostToDevice) != hipSuccess) {
+            fprintf(stderr, "MatXtract HIP error: could not put the matrix on the device\n");
+            return EXIT_FAILURE;
+        }
+        matxtract_detail::check(mx_plan_create_device(MX_VALT_DTYPE, rowA, colA, (int)nnzA, (const int *)dRowPtr, (const int *)dColInd, dVal,
+                                                      colProp, rowProp, planFlags, &plan),
+                                "mx_plan_create_device");
+        (void)hipFree(dRowPtr);
+        (void)hipFree(dColInd);
+        (void)hipFree(dVal);
+        preprocess_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        mx_plan_get_info(plan, &info);
+        pv.dCols = info.ext_dCols;
+        pv.dRows = info.ext_dRows;
+        pv.cols_ratio = colA > 0 ? (float)info.ext_dCols / (float)colA : 0.0f;
+        pv.tc_nnz_ratio = info.ext_frags > 0 ? (double)info.ext_nnzRowD / ((double)info.ext_frags * 8.0 * (MX_VALT_DTYPE == MX_F64 ? 4 : 8)) : 0.0;
+    } else {
+        bool fromCache = false;
+        if (!cachePath.empty() && mx_partition_load(cachePath.c_str(), MX_VALT_DTYPE, &part) == MX_OK) {
+            // The file is used only if it was made from a matrix of this shape with these fractions.
+            mx_partition_view cv;
+            mx_partition_get(part, &cv);
+            fromCache = cv.rows == rowA && cv.cols == colA && cv.nnz == (long long)nnzA && cv.tau_c == colProp && cv.tau_r == rowProp;
+            if (!fromCache) {
+                mx_partition_destroy(part);
+                part = nullptr;
+            }
+        }
+        if (!part) part = matxtract_preprocess(csrVal, csrRowPtr, csrColInd, rowA, colA, nnzA, colProp, rowProp, devicePrep);
+        auto t1 = std::chrono::steady_clock::now();
+        if (!part) return 1;
+        if (!cachePath.empty()) {
+            if (fromCache) printf("partition read from %s\n", cachePath.c_str());
+            else if (mx_partition_save(part, cachePath.c_str()) != MX_OK) printf("Warning: %s\n", mx_last_error());
+            else printf("partition written to %s\n", cachePath.c_str());
+        }
+        preprocess_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+        mx_partition_get(part, &pv);
     }
-    if (!part) part = matxtract_preprocess(csrVal, csrRowPtr, csrColInd, rowA, colA, nnzA, colProp, rowProp, devicePrep);
-    auto t1 = std::chrono::steady_clock::now();
-    if (!part) return 1;
-    if (!cachePath.empty()) {
-        if (fromCache) printf("partition read from %s\n", cachePath.c_str());
-        else if (mx_partition_save(part, cachePath.c_str()) != MX_OK) printf("Warning: %s\n", mx_last_error());
-        else printf("partition written to %s\n", cachePath.c_str());
-    }
-    const double preprocess_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
-    mx_partition_view pv;
-    mx_partition_get(part, &pv);
     if (extracting) {
         printf("cols_ratio = %f \n", pv.cols_ratio);
         printf("TC_nnz_ratio = %lf\n", pv.tc_nnz_ratio);
         std::cout << "---------------------Performance Info--------------------" << std::endl;
     }
-
-    mx_plan *plan = nullptr;
-    matxtract_detail::check(mx_plan_create(part, planFlags, &plan), "mx_plan_create");
-    mx_plan_info info;
-    mx_plan_get_info(plan, &info);
+    if (!plan) {
+        matxtract_detail::check(mx_plan_create(part, planFlags, &plan), "mx_plan_create");
+        mx_plan_get_info(plan, &info);
+    }
 
     valT *Y_val = (valT *)malloc(sizeof(valT) * (size_t)(rowA > 0 ? rowA : 1));
     valT *ourY_val = (valT *)malloc(sizeof(valT) * (size_t)(rowA > 0 ? rowA : 1));
@@ -273,7 +309,7 @@ int main(int argc, char **argv)
                "\"dCols\": %d, \"dRows\": %d, \"tc_nnz_ratio\": %.6f, \"tile_chunks\": %d, \"tile_nnz\": %d, "
                "\"csr_nnz\": %d, \"preprocess_ms\": %.3f, \"ms_total\": %.6f, \"ms_tile\": %.6f, \"ms_csr\": %.6f, "
                "\"gflops\": %.3f, \"algorithmic_bytes\": %.0f, \"gbs\": %.3f, \"hbm_frac\": %.5f, \"rel_l2\": %.3e, "
-               "\"pass\": %s, \"partition_hash\": \"%016llx\"}\n",
+               "\"pass\": %s, \"partition_hash\": \"%016llx\", \"prep_route\": %d}\n",
                rowA, colA, nnzA,
 #ifdef fp64
                "f64",
@@ -282,12 +318,13 @@ int main(int argc, char **argv)
 #endif
                col_frac, hot_frac, pv.dCols, pv.dRows, extracting ? pv.tc_nnz_ratio : 0.0, info.tile_chunks, info.tile_nnz,
                info.csr_nnz, preprocess_ms, ms_total, ms_tile, ms_csr, gflops, bytes, gbs, gbs / 8000.0,
-               rel_l2(Y_val, ourY_val, rowA), result == 0 ? "true" : "false", (unsigned long long)mx_partition_hash(part));
+               rel_l2(Y_val, ourY_val, rowA), result == 0 ? "true" : "false", part ? (unsigned long long)mx_partition_hash(part) : 0ull,
+               info.prep_route);
     }
     (void)hipFree(dx);
     (void)hipFree(dy);
     mx_plan_destroy(plan);
-    mx_partition_destroy(part);
+    if (part) mx_partition_destroy(part);
     free(Y_val);
     free(ourY_val);
     free(X_val);

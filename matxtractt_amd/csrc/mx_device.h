@@ -180,6 +180,38 @@ int lines_per_gather_device(mx_dtype dtype, int nnz, const int *col_dev, hipStre
 int upload_csr_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, const void *val_dev,
                       const std::vector<int> &desc, bool scan, DeviceCsr &A, hipStream_t s);
 
+// The host half of a hybrid plan done on the device (mx_hybrid.hip), for a matrix that lives in
+// device memory.  analyse() runs the extraction and counts what the plan's decision needs;
+// csr_part() assembles the CSR part (residual rows, then the entries of A_dd that stay) in the
+// caller's numbering, in new device arrays that pass to the caller; strip_layout() lays the
+// binary16 strip chunks out as steps (the caller plans the steps from the chunks' block counts,
+// as the host route does).  All arrays equal the host route's byte for byte.
+struct HybridCounts {
+    long long generalFrags = 0, generalEntries = 0;  // fragments that pass the fill gate (after the strips took their rows)
+    long long stripEntries = 0, stripBlocks = 0;     // binary16 strip chunks, or binary64 8 x 8 blocks (blocks64)
+    bool blocks64 = false;
+    int dRows = 0, dCols = 0, nnzRowD = 0, frags = 0;  // what the extraction selected; fragments of the tile encoding
+    std::vector<int> stripChunkBlocks, stripChunkEntries;  // per strip chunk, in layout order
+};
+struct HybridDevice {
+    struct Impl;
+    Impl *impl = nullptr;
+    HybridDevice() = default;
+    HybridDevice(const HybridDevice &) = delete;
+    HybridDevice &operator=(const HybridDevice &) = delete;
+    ~HybridDevice();
+    // minVals: entries a fragment needs to pass the gate; want*: which forms the flags allow
+    int analyse(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, const void *val_dev, float tau_c,
+                float tau_r, int minVals, bool wantGeneral, bool wantStrips, bool wantBlocks, HybridCounts *counts, hipStream_t s);
+    // stripRows_dev: marks of the rows the strips write (null when keepStrips is false or there are none)
+    int csr_part(bool keepStrips, int **rowPtr_dev, int **col_dev, void **val_dev, int *nnz, char **stripRows_dev);
+    // stepDesc: 8 ints per step {chunk of half 0, chunk of half 1 (-1 none, -2 the first goes on), flags, blocks in half 0,
+    // blocks in half 1, first value, first value and blocks in half 0 of the step four further on}; chunkBlock0: first block
+    // of every chunk; T receives waveDesc, hdr, atox and tcVal
+    int strip_layout(const std::vector<int> &stepDesc, const std::vector<int> &chunkBlock0, const std::vector<int> &waveDesc,
+                     long long totalBlocks, DeviceTiles &T);
+};
+
 // `what`: 0 = slice kernel then combine kernel, 1 = slice kernel only, 2 = combine kernel only
 // `strips` (optional): a tile layout in the dense binary16 form whose steps workgroups of the
 // combine kernel's launch run as well (strips_can_ride says whether a layout may); the rows of

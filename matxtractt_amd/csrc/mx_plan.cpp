@@ -480,6 +480,39 @@ struct HostTiles {
     std::vector<unsigned char> val;
 };
 
+// The waves of a tile layout: whole chunks, about `per` steps each; few enough waves that all of
+// them are resident at once (24 per CU), so that none has to wait for a second round.
+// stepVo / stepA / stepChunkEnd: first value, blocks in half 0 and "a wave may end here" of every
+// step.  waveDesc: 8 ints per wave (see DeviceTiles); ahead: per step the first value and the
+// blocks in half 0 of the step four further on (the wave's last when past it).
+static void tile_waves(int steps, int nCU, int perMin, const std::vector<int> &stepVo, const std::vector<int> &stepA,
+                       const std::vector<int> &stepChunkEnd, std::vector<int> &waveDesc, std::vector<int> &ahead)
+{
+    nCU = std::max(1, nCU);
+    const int tper = std::getenv("MX_TILE_PER") ? std::atoi(std::getenv("MX_TILE_PER")) : 0;
+    // (binary64 block waves keep two steps in registers and live on the number of waves: a step each)
+    const int per = tper > 0 ? tper : std::max(perMin, (steps + nCU * 24 - 1) / (nCU * 24));
+    waveDesc.clear();
+    ahead.assign((size_t)steps * 2, 0);
+    for (int s0 = 0; s0 < steps;) {
+        int s1 = std::min(steps, s0 + per);
+        while (s1 < steps && !stepChunkEnd[s1 - 1]) ++s1;
+        int d[8] = {s0, s1, 0, 0, 0, 0, 0, 0};
+        for (int k = 0; k < 4; ++k) {
+            const int sk = std::min(s0 + k, s1 - 1);
+            d[2 + k] = stepVo[sk];
+            d[6] |= stepA[sk] << (8 * k);
+        }
+        waveDesc.insert(waveDesc.end(), d, d + 8);
+        for (int s = s0; s < s1; ++s) {
+            const int s4 = std::min(s + 4, s1 - 1);
+            ahead[2 * (size_t)s] = stepVo[s4];
+            ahead[2 * (size_t)s + 1] = stepA[s4];
+        }
+        s0 = s1;
+    }
+}
+
 int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, const int *chunkPtr, const int *fragPtr,
                 const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap, int nCU,
                 HostTiles &T, const char *rowTaken = nullptr, const std::vector<StripChunk> *stripChunks = nullptr)
@@ -659,30 +692,11 @@ int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, co
     T.steps = steps;
     T.dense = stripChunks != nullptr && steps > 0;
     if (steps == 0) return MX_OK;
-    // waves: whole chunks, about `per` steps each; few enough waves that all of them are resident
-    // at once (24 per CU), so that none has to wait for a second round
-    nCU = std::max(1, nCU);
-    const int tper = std::getenv("MX_TILE_PER") ? std::atoi(std::getenv("MX_TILE_PER")) : 0;
-    // (binary64 block waves keep two steps in registers and live on the number of waves: a step each)
-    const int perMin = (stripChunks && f64) ? 1 : 2;
-    const int per = tper > 0 ? tper : std::max(perMin, (steps + nCU * 24 - 1) / (nCU * 24));
-    std::vector<int> waveDesc;
-    for (int s0 = 0; s0 < steps;) {
-        int s1 = std::min(steps, s0 + per);
-        while (s1 < steps && !stepChunkEnd[s1 - 1]) ++s1;
-        int d[8] = {s0, s1, 0, 0, 0, 0, 0, 0};
-        for (int k = 0; k < 4; ++k) {
-            const int sk = std::min(s0 + k, s1 - 1);
-            d[2 + k] = stepVo[sk];
-            d[6] |= stepA[sk] << (8 * k);
-        }
-        waveDesc.insert(waveDesc.end(), d, d + 8);
-        for (int s = s0; s < s1; ++s) {  // the step four further on (the wave's last when past it)
-            const int s4 = std::min(s + 4, s1 - 1);
-            hdr[(size_t)s * H + 19] = stepVo[s4];
-            hdr[(size_t)s * H + 20] = stepA[s4];
-        }
-        s0 = s1;
+    std::vector<int> waveDesc, ahead;
+    tile_waves(steps, nCU, (stripChunks && f64) ? 1 : 2, stepVo, stepA, stepChunkEnd, waveDesc, ahead);
+    for (int s = 0; s < steps; ++s) {
+        hdr[(size_t)s * H + 19] = ahead[2 * (size_t)s];
+        hdr[(size_t)s * H + 20] = ahead[2 * (size_t)s + 1];
     }
     T.nWaves = (int)waveDesc.size() / 8;
     T.waveDesc.swap(waveDesc);
@@ -1175,6 +1189,8 @@ struct mx_plan {
     // binary16 plans whose general tiles share rows with the CSR part: the CSR part's sums as
     // binary32, one per row, which the tile kernel adds to (y is then rounded once)
     void *ywide = nullptr;
+    int ext_dCols = 0, ext_dRows = 0, ext_nnzRowD = 0, ext_frags = 0;  // what the extraction behind the plan selected
+    int prep_route = 0;  // 0 = laid out on the host, 1 = on the device, 2 = mx_plan_create_device sent the matrix to the host route
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 };
@@ -1554,6 +1570,34 @@ static double tile_gate(mx_dtype)
     return 0.5;
 }
 
+// Do the tiles pay for their launch?  (The reference gates its tile kernel on the size of the
+// matrix and its fill, test/test_autotc_spmv.cpp:1507,1518.)  What they take off the CSR part
+// saves es + 2 bytes per entry of its stream; what they cost is one more dependent launch and
+// their own stream.  Rates as measured on MI355X: the CSR part and the strip form of the tile
+// kernel move about 5000 bytes per ns (5 TB/s), the general tile kernel, bound by instruction
+// issue, about 2200; a further launch in the sequence costs about 5 us with its ramp and tail
+// (the strips of the mixed workload break even at about 15 M entries when launched apart);
+// strips usually ride in the launch of the combine kernel, where they came out ahead at every
+// size tried (1.7 M entries and up): they are charged little.
+// general*: the reference's fragments that pass the fill gate; strip*: the chunks of the plan's
+// own (binary16 strips, or binary64 8 x 8 blocks with `blocks64`).
+// 0 = nothing pays, 1 = only the plan's own chunks do, 2 = keep both.
+static int tiles_worth(mx_dtype dtype, int fragM, int fragK, bool blocks64, double generalEntries, double generalFrags,
+                       double stripEntries, double stripBlocks)
+{
+    const int es = mx::elem_size(dtype);
+    const double blockBytes = (double)fragM * (blocks64 ? 8 : fragK) * es, slots = mx::tile_slots(dtype);
+    const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
+    const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
+    const double launchNs = 5000.0, stripLaunchNs = 1000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
+    const double savedNs = (generalEntries + stripEntries) * (es + 2) / fastRate;
+    const double costNs = (generalFrags > 0 ? launchNs + generalBytes / generalRate : 0.0) +
+                          (stripBlocks > 0 ? stripLaunchNs + stripBytes / fastRate : 0.0);
+    if (savedNs <= costNs) return 0;
+    if (generalFrags > 0 && generalEntries * (es + 2) / fastRate <= launchNs + generalBytes / generalRate) return 1;
+    return 2;
+}
+
 // MX_PLAN_LOG=1: the phases of mx_plan_create with their host time, on stderr
 struct PhaseLog {
     bool on = std::getenv("MX_PLAN_LOG") && std::atoi(std::getenv("MX_PLAN_LOG"));
@@ -1812,16 +1856,7 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
             }
         }
     }
-    // Do the tiles pay for their launch?  (The reference gates its tile kernel on the size
-    // of the matrix and its fill, test/test_autotc_spmv.cpp:1507,1518.)  What they take off
-    // the CSR part saves es + 2 bytes per entry of its stream; what they cost is one more
-    // dependent launch and their own stream.  Rates as measured on MI355X: the CSR part and
-    // the strip form of the tile kernel move about 5000 bytes per ns (5 TB/s), the general
-    // tile kernel, bound by instruction issue, about 2200; a further launch in the sequence
-    // costs about 5 us with its ramp and tail (the strips of the mixed workload break even at
-    // about 15 M entries when launched apart); strips usually ride in the launch of the
-    // combine kernel, where they came out ahead at every size tried (1.7 M entries and up):
-    // they are charged little.  MX_PLAN_KEEP_TILES skips the question.
+    // do the tiles pay for their launch (tiles_worth)?  MX_PLAN_KEEP_TILES skips the question.
     if (!(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES | MX_PLAN_KEEP_TILES))) {
         double generalEntries = 0, generalFrags = 0, stripEntries = 0, stripBlocks = 0;
         for (int w = 0; w < chunkNum; ++w) {
@@ -1842,20 +1877,14 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
             stripEntries += C.nnz;
             stripBlocks += (double)C.blocks.size();
         }
-        const double blockBytes = (double)fragM * (inBlock.empty() ? fragK : 8) * es, slots = mx::tile_slots(P->dtype);
-        const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
-        const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
-        const double launchNs = 5000.0, stripLaunchNs = 1000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
-        const double savedNs = (generalEntries + stripEntries) * (es + 2) / fastRate;
-        const double costNs = (generalFrags > 0 ? launchNs + generalBytes / generalRate : 0.0) +
-                              (stripBlocks > 0 ? stripLaunchNs + stripBytes / fastRate : 0.0);
-        if (savedNs <= costNs) {
+        const int worth = tiles_worth(P->dtype, fragM, fragK, !inBlock.empty(), generalEntries, generalFrags, stripEntries, stripBlocks);
+        if (worth == 0) {
             std::fill(sel.begin(), sel.end(), 0);
             stripChunks.clear();
             taken.clear();
             inBlock.clear();
             H.stripRows.clear();
-        } else if (generalFrags > 0 && generalEntries * (es + 2) / fastRate <= launchNs + generalBytes / generalRate) {
+        } else if (worth == 1) {
             std::fill(sel.begin(), sel.end(), 0);  // the strips pay, the general tiles do not
         }
     }
@@ -1959,6 +1988,12 @@ static int create_plan(const mx_partition *P, int flags, mx_plan **out, bool noB
     plan->rows = P->rows;
     plan->cols = P->cols;
     plan->nnz = P->nnz;
+    if (P->extracted) {
+        plan->ext_dCols = P->dCols;
+        plan->ext_dRows = P->dRows;
+        plan->ext_nnzRowD = P->nnzRowD;
+        plan->ext_frags = P->totalTcFrags;
+    }
     auto fail = [&](int code) {
         mx_plan_destroy(plan);
         return code;
@@ -2058,6 +2093,71 @@ static int create_plan(const mx_partition *P, int flags, mx_plan **out, bool noB
     return MX_OK;
 }
 
+// The CSR part of a plan from arrays in device memory: the form is chosen as setup_csr_part chooses
+// it -- the same counts, taken on the device -- and only that form is built, there.  Nothing of the
+// matrix crosses to the host but its row pointers (for the row-tile form) or the lengths of its
+// chunks (for the slice form).  `elsewhere_dev` (optional): marks of rows that another kernel writes.
+static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, const int *colInd_dev, const void *val_dev, int flags,
+                                 const char *elsewhere_dev)
+{
+    const mx_dtype dtype = plan->dtype;
+    const int rows = plan->rows, cols = plan->cols;
+    int rc;
+    plan->csr_nnz = nnz;
+    hipDeviceProp_t prop;
+    int dev = 0;
+    MX_HIP(hipGetDevice(&dev));
+    MX_HIP(hipGetDeviceProperties(&prop, dev));
+    const int nCU = std::max(1, prop.multiProcessorCount);
+    const int S = rows > 0 ? slice_count(dtype, rows, cols, nnz, nCU) : 0;
+    bool want[2] = {true, S > 0};
+    const char *env = std::getenv("MX_CSR_KERNEL");
+    if (flags & MX_PLAN_CSR_ROWS) want[1] = false;
+    if ((flags & MX_PLAN_CSR_SLICES) && S > 0) want[0] = false;
+    if (env && !std::strcmp(env, "rows")) want[0] = true, want[1] = false;
+    if (env && !std::strcmp(env, "slices") && S > 0) want[1] = true, want[0] = false;
+    if (want[1]) {
+        rc = mx::build_slices_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, nCU, S, elsewhere_dev, plan->slices, nullptr);
+        if (rc) return rc;
+        if (plan->slices.ecode) plan->slices.useDict = true;
+    }
+    if (want[0] && want[1]) {
+        // the estimates of csr_estimates from what the device counted: the virtual rows are those of
+        // the layout just made, the one-byte form exists when the layout has it
+        CsrStats st;
+        st.vrows = plan->slices.vrows;
+        st.fewValues = plan->slices.ecode != nullptr;
+        if ((rc = mx::lines_per_gather_device(dtype, nnz, colInd_dev, nullptr, &st.linesPerGather))) return rc;
+        csr_estimates(dtype, cols, nnz, st, &plan->est_rows_us, &plan->est_slices_us);
+        want[plan->est_slices_us < plan->est_rows_us ? 0 : 1] = false;
+    }
+    if (want[1]) {
+        plan->csr_variant = 1;
+        return MX_OK;
+    }
+    free_slices(plan->slices);
+    plan->csr_variant = 0;
+    std::vector<int> rp((size_t)rows + 1, 0), desc;
+    MX_HIP(hipMemcpy(rp.data(), rowPtr_dev, ((size_t)rows + 1) * 4, hipMemcpyDeviceToHost));
+    const int npt = mx::csr_entries_per_lane(dtype);
+    pack_rows(rp.data(), rows, npt, desc);
+    double sum = 0.0, sq = 0.0;
+    for (int r = 0; r < rows; ++r) {
+        const double n = rp[r + 1] - rp[r];
+        sum += n;
+        sq += n * n;
+    }
+    const double mean = rows > 0 ? sum / rows : 0.0, var = rows > 0 ? sq / rows - mean * mean : 0.0;
+    bool scan = mean > 0.0 && var > 0.25 * mean * mean;
+    const char *envr = std::getenv("MX_CSR_REDUCE");
+    if (envr && !std::strcmp(envr, "rows")) scan = false;
+    if (envr && !std::strcmp(envr, "scan")) scan = true;
+    rc = mx::upload_csr_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, desc, scan, plan->csr, nullptr);
+    if (rc) return rc;
+    if (plan->csr.codes) plan->csr.useDict = true;
+    return MX_OK;
+}
+
 // A plan for y = A x from a CSR matrix that lives in device memory: nothing of the matrix crosses
 // to the host but its row pointers (for the row-tile form) or the lengths of its chunks (for the
 // slice form).  The form is chosen as in mx_plan_create -- the same counts, taken on the device --
@@ -2085,6 +2185,7 @@ extern "C" int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int
     plan->cols = cols;
     plan->nnz = nnz;
     plan->csr_nnz = nnz;
+    plan->prep_route = 1;
     auto fail = [&](int code) {
         mx_plan_destroy(plan);
         return code;
@@ -2103,63 +2204,310 @@ extern "C" int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int
         }
     }
     try {
-        hipDeviceProp_t prop;
-        int dev = 0;
-        MX_HIP(hipGetDevice(&dev));
-        MX_HIP(hipGetDeviceProperties(&prop, dev));
-        const int nCU = std::max(1, prop.multiProcessorCount);
-        const int S = rows > 0 ? slice_count(dtype, rows, cols, nnz, nCU) : 0;
-        bool want[2] = {true, S > 0};
-        const char *env = std::getenv("MX_CSR_KERNEL");
-        if (flags & MX_PLAN_CSR_ROWS) want[1] = false;
-        if ((flags & MX_PLAN_CSR_SLICES) && S > 0) want[0] = false;
-        if (env && !std::strcmp(env, "rows")) want[0] = true, want[1] = false;
-        if (env && !std::strcmp(env, "slices") && S > 0) want[1] = true, want[0] = false;
-        if (want[1]) {
-            rc = mx::build_slices_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, nCU, S, nullptr, plan->slices, nullptr);
-            if (rc) return fail(rc);
-            if (plan->slices.ecode) plan->slices.useDict = true;
-        }
-        if (want[0] && want[1]) {
-            // the estimates of csr_estimates from what the device counted: the virtual rows are those of
-            // the layout just made, the one-byte form exists when the layout has it
-            CsrStats st;
-            st.vrows = plan->slices.vrows;
-            st.fewValues = plan->slices.ecode != nullptr;
-            if ((rc = mx::lines_per_gather_device(dtype, nnz, colInd_dev, nullptr, &st.linesPerGather))) return fail(rc);
-            csr_estimates(dtype, cols, nnz, st, &plan->est_rows_us, &plan->est_slices_us);
-            want[plan->est_slices_us < plan->est_rows_us ? 0 : 1] = false;
-        }
-        if (want[1]) {
-            plan->csr_variant = 1;
-        } else {
-            free_slices(plan->slices);
-            plan->csr_variant = 0;
-            std::vector<int> rp((size_t)rows + 1, 0), desc;
-            MX_HIP(hipMemcpy(rp.data(), rowPtr_dev, ((size_t)rows + 1) * 4, hipMemcpyDeviceToHost));
-            const int npt = mx::csr_entries_per_lane(dtype);
-            pack_rows(rp.data(), rows, npt, desc);
-            double sum = 0.0, sq = 0.0;
-            for (int r = 0; r < rows; ++r) {
-                const double n = rp[r + 1] - rp[r];
-                sum += n;
-                sq += n * n;
-            }
-            const double mean = rows > 0 ? sum / rows : 0.0, var = rows > 0 ? sq / rows - mean * mean : 0.0;
-            bool scan = mean > 0.0 && var > 0.25 * mean * mean;
-            const char *envr = std::getenv("MX_CSR_REDUCE");
-            if (envr && !std::strcmp(envr, "rows")) scan = false;
-            if (envr && !std::strcmp(envr, "scan")) scan = true;
-            rc = mx::upload_csr_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, desc, scan, plan->csr, nullptr);
-            if (rc) return fail(rc);
-            if (plan->csr.codes) plan->csr.useDict = true;
-        }
+        rc = setup_csr_part_device(plan, nnz, rowPtr_dev, colInd_dev, val_dev, flags, nullptr);
+        if (rc) return fail(rc);
     } catch (const std::bad_alloc &) {
         set_error("mx_plan_create_device_csr: out of memory");
         return fail(MX_ERR_ALLOC);
     }
     *out = plan;
     return MX_OK;
+}
+
+// The steps of binary16 strip chunks from their block counts alone, as build_tiles lays them out: a
+// chunk of up to four blocks shares a step with the next such chunk (half 0 and half 1), a larger
+// one (up to eight) takes a step of its own with its fifth and further blocks in half 1.
+// stepDesc: 8 ints per step {chunk of half 0, chunk of half 1 (-1 none, -2 the first goes on), flags,
+// blocks in half 0, blocks in half 1, first value, first value and blocks in half 0 of the step four
+// further on}; chunkBlock0: the first block of every chunk in the stored values.
+static int plan_strip_steps(const std::vector<int> &chunkBlocks, int nCU, std::vector<int> &stepDesc, std::vector<int> &chunkBlock0,
+                            std::vector<int> &waveDesc, long long *totalBlocks)
+{
+    const int HF = 4, n = (int)chunkBlocks.size();
+    std::vector<int> stepVo, stepA, stepEnd, who;  // who: {chunk of half 0, of half 1, flags, blocks, blocks} per step
+    chunkBlock0.assign((size_t)n, 0);
+    long long blocks = 0;
+    int pending = -1;
+    auto emit = [&](int a, int b, int flags, int n0, int n1) {
+        const int d[5] = {a, b, flags, n0, n1};
+        who.insert(who.end(), d, d + 5);
+        stepVo.push_back((int)(blocks * 64));
+        stepA.push_back(n0);
+        stepEnd.push_back(flags & 1);
+        blocks += n0 + n1;
+    };
+    for (int k = 0; k < n; ++k) {
+        const int nb = chunkBlocks[k];
+        if (nb < 1 || nb > 2 * HF) {
+            set_error("strip layout: a chunk with an impossible number of blocks");
+            return MX_ERR_DEVICE;
+        }
+        if (nb <= HF) {
+            if (pending >= 0) {
+                chunkBlock0[pending] = (int)blocks;
+                chunkBlock0[k] = (int)blocks + chunkBlocks[pending];
+                emit(pending, k, 3, chunkBlocks[pending], nb);
+                pending = -1;
+            } else {
+                pending = k;
+            }
+        } else {
+            chunkBlock0[k] = (int)blocks;
+            emit(k, -2, 1, HF, nb - HF);
+        }
+        if (blocks * 64 > 2000000000LL) {
+            set_error("tile layout: too many values for 32-bit offsets");
+            return MX_ERR_ARG;
+        }
+    }
+    if (pending >= 0) {
+        chunkBlock0[pending] = (int)blocks;
+        emit(pending, -1, 3, chunkBlocks[pending], 0);
+    }
+    const int steps = (int)stepVo.size();
+    std::vector<int> ahead;
+    tile_waves(steps, nCU, 2, stepVo, stepA, stepEnd, waveDesc, ahead);
+    stepDesc.assign((size_t)steps * 8, 0);
+    for (int st = 0; st < steps; ++st) {
+        int *d = &stepDesc[(size_t)st * 8];
+        for (int k = 0; k < 5; ++k) d[k] = who[(size_t)st * 5 + k];
+        d[5] = stepVo[st];
+        d[6] = ahead[2 * (size_t)st];
+        d[7] = ahead[2 * (size_t)st + 1];
+    }
+    *totalBlocks = blocks;
+    return MX_OK;
+}
+
+// A hybrid plan from a CSR matrix in device memory and the two extraction fractions: the
+// extraction, the plan's decisions, the CSR part with its layout and the strips' layout are all
+// made on the device (mx_hybrid.hip, mx_layout.hip); what a decision needs comes to the host as
+// counts.  The plan equals the one mx_plan_create makes from mx_partition_create(_device) of the
+// same matrix.  Two tile forms are not laid out on the device -- the general one and the binary64
+// blocks; a matrix on which the plan keeps one of them (none of the measured workloads with
+// default flags) is copied to the host and takes the host route.
+extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
+                                     const void *val_dev, float tau_c, float tau_r, int flags, mx_plan **out)
+{
+    static const char who[] = "mx_plan_create_device";
+    if (!out || (dtype != MX_F64 && dtype != MX_F16) || rows < 1 || cols < 1 || nnz < 0 || !rowPtr_dev ||
+        (nnz > 0 && (!colInd_dev || !val_dev)) || !(tau_c >= 0.0f && tau_c <= 1.0f) || !(tau_r >= 0.0f && tau_r <= 1.0f)) {
+        set_error(std::string(who) + ": bad argument");
+        return MX_ERR_ARG;
+    }
+    *out = nullptr;
+    if (tau_c == 0.0f && tau_r == 0.0f)  // nothing to extract
+        return mx_plan_create_device_csr(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, flags, out);
+    int rc = need_device();
+    if (rc) return rc;
+    if ((rc = mx::check_csr_device(rows, cols, nnz, rowPtr_dev, colInd_dev, nullptr, who))) return rc;
+    const size_t es = (size_t)mx::elem_size(dtype);
+    // the host route for this matrix: it comes down once and goes through mx_partition_create_device
+    auto host_route = [&]() -> int {
+        std::vector<int> rp((size_t)rows + 1), ci((size_t)nnz);
+        std::vector<unsigned char> va((size_t)nnz * es);
+        MX_HIP(hipMemcpy(rp.data(), rowPtr_dev, rp.size() * 4, hipMemcpyDeviceToHost));
+        if (nnz > 0) {
+            MX_HIP(hipMemcpy(ci.data(), colInd_dev, ci.size() * 4, hipMemcpyDeviceToHost));
+            MX_HIP(hipMemcpy(va.data(), val_dev, va.size(), hipMemcpyDeviceToHost));
+        }
+        mx_csr A{};
+        A.dtype = dtype;
+        A.rows = rows;
+        A.cols = cols;
+        A.nnz = nnz;
+        A.rowPtr = rp.data();
+        A.colInd = ci.data();
+        A.val = va.data();
+        mx_partition *P = nullptr;
+        int e = mx_partition_create_device(&A, tau_c, tau_r, &P);
+        if (e) return e;
+        e = mx_plan_create(P, flags, out);
+        mx_partition_destroy(P);
+        if (!e) (*out)->prep_route = 2;
+        return e;
+    };
+    if (flags & MX_PLAN_ALL_TILES) return host_route();
+    try {
+        hipDeviceProp_t prop;
+        int dev = 0;
+        MX_HIP(hipGetDevice(&dev));
+        MX_HIP(hipGetDeviceProperties(&prop, dev));
+        const int nCU = std::max(1, prop.multiProcessorCount);
+        const int fragM = mx::kFragM, fragK = mx::frag_k(dtype);
+        const bool noTiles = (flags & MX_PLAN_NO_TILES) != 0;
+        const char *envNoStrips = std::getenv("MX_NO_STRIPS"), *envNoBlocks = std::getenv("MX_NO_BLOCKS");
+        const bool wantStrips = dtype == MX_F16 && !noTiles && !(envNoStrips && std::atoi(envNoStrips));
+        const bool wantBlocks = dtype == MX_F64 && !noTiles && !(envNoBlocks && std::atoi(envNoBlocks));
+        // (the smallest count that passes `(double)vals >= gate * fragM * fragK`)
+        const double need = tile_gate(dtype) * fragM * fragK;
+        int minVals = (int)need;
+        while ((double)minVals < need) ++minVals;
+        mx::HybridDevice H;
+        mx::HybridCounts cnt;
+        rc = H.analyse(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, tau_c, tau_r, minVals, !noTiles, wantStrips, wantBlocks, &cnt,
+                       nullptr);
+        if (rc) return rc;
+        if (cnt.blocks64) cnt.generalFrags = cnt.generalEntries = 0;  // the general tiles are not used beside blocks
+        int worth = 2;
+        if (noTiles) worth = 0;
+        else if (!(flags & MX_PLAN_KEEP_TILES))
+            worth = tiles_worth(dtype, fragM, fragK, cnt.blocks64, (double)cnt.generalEntries, (double)cnt.generalFrags,
+                                (double)cnt.stripEntries, (double)cnt.stripBlocks);
+        if ((worth == 2 && cnt.generalFrags > 0) || (worth >= 1 && cnt.blocks64 && cnt.stripBlocks > 0)) return host_route();
+        const bool keepStrips = worth >= 1 && !cnt.blocks64 && cnt.stripBlocks > 0;
+
+        mx_plan *plan = new (std::nothrow) mx_plan();
+        if (!plan) {
+            set_error(std::string(who) + ": out of memory");
+            return MX_ERR_ALLOC;
+        }
+        plan->dtype = dtype;
+        plan->rows = rows;
+        plan->cols = cols;
+        plan->nnz = nnz;
+        plan->prep_route = 1;
+        plan->ext_dCols = cnt.dCols;
+        plan->ext_dRows = cnt.dRows;
+        plan->ext_nnzRowD = cnt.nnzRowD;
+        plan->ext_frags = cnt.frags;
+        int *partPtr = nullptr, *partCol = nullptr;
+        void *partVal = nullptr;
+        char *stripRows = nullptr;
+        auto fail = [&](int code) {
+            (void)hipFree(partPtr);
+            (void)hipFree(partCol);
+            (void)hipFree(partVal);
+            (void)hipFree(stripRows);
+            mx_plan_destroy(plan);
+            return code;
+        };
+        if (hipStreamCreate(&plan->stream) != hipSuccess || hipEventCreate(&plan->ev0) != hipSuccess ||
+            hipEventCreate(&plan->ev1) != hipSuccess) {
+            set_error(std::string(who) + ": could not create stream/events");
+            return fail(MX_ERR_DEVICE);
+        }
+        {
+            void *fixed = nullptr;
+            if (mx::static_scratch(&fixed) != hipSuccess) {
+                (void)hipGetLastError();
+                set_error(std::string(who) + ": hipGetSymbolAddress failed for the fixed array of sums");
+                return fail(MX_ERR_DEVICE);
+            }
+        }
+        int partNnz = 0;
+        if ((rc = H.csr_part(keepStrips, &partPtr, &partCol, &partVal, &partNnz, &stripRows))) return fail(rc);
+        if ((rc = setup_csr_part_device(plan, partNnz, partPtr, partCol, partVal, flags, stripRows))) return fail(rc);
+        if (keepStrips) {
+            std::vector<int> stepDesc, chunkBlock0, waveDesc;
+            long long totalBlocks = 0;
+            if ((rc = plan_strip_steps(cnt.stripChunkBlocks, nCU, stepDesc, chunkBlock0, waveDesc, &totalBlocks))) return fail(rc);
+            mx::DeviceTiles &T = plan->strips;
+            T.chunkNum = (int)cnt.stripChunkBlocks.size();
+            T.frags = (int)cnt.stripBlocks;
+            T.vals = (int)cnt.stripEntries;
+            T.stored = totalBlocks * 64;
+            T.steps = (int)(stepDesc.size() / 8);
+            T.dense = T.steps > 0;
+            T.nWaves = (int)(waveDesc.size() / 8);
+            if ((rc = H.strip_layout(stepDesc, chunkBlock0, waveDesc, totalBlocks, T))) return fail(rc);
+            T.ownedRows = true;  // strip rows have nothing in the CSR part, which leaves zeros there
+            plan->tile_nnz = T.vals;
+        }
+        (void)hipFree(partPtr);
+        (void)hipFree(partCol);
+        (void)hipFree(partVal);
+        (void)hipFree(stripRows);
+        *out = plan;
+        return MX_OK;
+    } catch (const std::bad_alloc &) {
+        set_error(std::string(who) + ": out of memory");
+        return MX_ERR_ALLOC;
+    }
+}
+
+// Every device array of a plan copied to host memory, with a name: for tests that hold the routes
+// of making a plan against each other.
+extern "C" void mx_plan_arrays_free(mx_plan_array *a, int n)
+{
+    if (!a) return;
+    for (int i = 0; i < n; ++i) {
+        free(a[i].data);
+        a[i].data = nullptr;
+    }
+}
+extern "C" int mx_plan_arrays(const mx_plan *plan, mx_plan_array *out, int cap, int *n)
+{
+    if (!plan || !out || !n || cap < 1) {
+        set_error("mx_plan_arrays: bad argument");
+        return MX_ERR_ARG;
+    }
+    *n = 0;
+    const size_t es = (size_t)mx::elem_size(plan->dtype);
+    int rc = MX_OK;
+    auto add = [&](const char *name, const void *dev, size_t bytes) {
+        if (rc || !dev) return;
+        if (*n >= cap) {
+            set_error("mx_plan_arrays: more arrays than the caller has room for");
+            rc = MX_ERR_ARG;
+            return;
+        }
+        void *p = malloc(std::max<size_t>(bytes, 1));
+        if (!p || (bytes && hipMemcpy(p, dev, bytes, hipMemcpyDeviceToHost) != hipSuccess)) {
+            free(p);
+            set_error("mx_plan_arrays: out of memory or copy failed");
+            rc = MX_ERR_ALLOC;
+            return;
+        }
+        out[*n].name = name;
+        out[*n].bytes = bytes;
+        out[*n].data = p;
+        ++*n;
+    };
+    if (plan->csr_variant != 1) {
+        const mx::DeviceCsr &A = plan->csr;
+        add("csr.rowPtr", A.rowPtr, ((size_t)A.rows + 1) * 4);
+        add("csr.col", A.col, (size_t)A.nnz * 4);
+        add("csr.col16", A.col16, (size_t)A.nnz * 2);
+        add("csr.colBase", A.colBase, (size_t)A.nBlocks * 4);
+        add("csr.val", A.val, (size_t)A.nnz * es);
+        add("csr.blockDesc", A.blockDesc, (size_t)A.nBlocks * 16);
+        add("csr.codes", A.codes, (size_t)A.nnz);
+        add("csr.dict", A.dict, 256 * es);
+    }
+    if (plan->csr_variant != 0) {
+        const mx::DeviceSlices &D = plan->slices;
+        const size_t nEcol = ((size_t)D.steps + mx::kSlicePadSteps) * 64 * mx::slice_step_entries(plan->dtype);
+        add("slices.wgDesc", D.wgDesc, ((size_t)D.nWG * 4 + 4) * 4);
+        add("slices.waveDesc", D.waveDesc, ((size_t)D.nWG * mx::kSliceWaves * 4 + 4) * 4);
+        add("slices.chunkEnd", D.chunkEnd, ((size_t)D.chunks + 64) * 4);
+        add("slices.ecol", D.ecol, nEcol * 2);
+        add("slices.eval", D.eval, nEcol * es);
+        add("slices.ecode", D.ecode, nEcol);
+        add("slices.dict", D.dict, 256 * es);
+        add("slices.rowInfo", D.rowInfo, (((size_t)D.rows + 3) / 4 * 4 + 4) * 4);
+        add("slices.segIdx", D.segIdx, ((size_t)D.vrows + 1) * 4);
+        add("slices.lightRow", D.lightRow, (size_t)D.nLight * 4);
+        add("slices.lightIdx", D.lightIdx, (size_t)D.nLight * 4 * D.lightQuads * 4);
+        add("slices.heavyInfo", D.heavyInfo, ((size_t)D.nHeavy * 4 + 4) * 4);
+    }
+    const mx::DeviceTiles *two[2] = {&plan->tiles, &plan->strips};
+    static const char *const names[2][5] = {{"tiles.waveDesc", "tiles.hdr", "tiles.atox", "tiles.tcVal", "tiles.vidx"},
+                                            {"strips.waveDesc", "strips.hdr", "strips.atox", "strips.tcVal", "strips.vidx"}};
+    for (int t = 0; t < 2; ++t) {
+        const mx::DeviceTiles &T = *two[t];
+        if (T.nWaves <= 0) continue;
+        add(names[t][0], T.waveDesc, (size_t)T.nWaves * 8 * 4);
+        add(names[t][1], T.hdr, (size_t)T.steps * mx::kTileHdr * 4);
+        add(names[t][2], T.atox, (size_t)T.steps * 64 * 4);
+        add(names[t][3], T.tcVal, (size_t)T.stored * es);
+        add(names[t][4], T.vidx, (size_t)T.steps * 128 * 4);
+    }
+    if (rc) {
+        mx_plan_arrays_free(out, *n);
+        *n = 0;
+    }
+    return rc;
 }
 
 extern "C" void mx_plan_layout_free(mx_plan_layout_view *v)
@@ -2311,6 +2659,11 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
                                                   : (plan->csr.useDict ? plan->csr.nDict : 0);
     info->est_rows_us = plan->est_rows_us;
     info->est_slices_us = plan->est_slices_us;
+    info->prep_route = plan->prep_route;
+    info->ext_dCols = plan->ext_dCols;
+    info->ext_dRows = plan->ext_dRows;
+    info->ext_nnzRowD = plan->ext_nnzRowD;
+    info->ext_frags = plan->ext_frags;
     return MX_OK;
 }
 

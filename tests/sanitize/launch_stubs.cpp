@@ -12,6 +12,15 @@ int check_csr_device(int, int, int, const int *, const int *, hipStream_t, const
 int lines_per_gather_device(mx_dtype, int, const int *, hipStream_t, double *) { return MX_ERR_DEVICE; }
 int upload_csr_device(mx_dtype, int, int, int, const int *, const int *, const void *, const std::vector<int> &, bool, DeviceCsr &, hipStream_t) { return MX_ERR_DEVICE; }
 bool strips_can_ride(mx_dtype, const DeviceTiles &, const void *) { return false; }
+struct HybridDevice::Impl {};
+HybridDevice::~HybridDevice() { delete impl; }
+int HybridDevice::analyse(mx_dtype, int, int, int, const int *, const int *, const void *, float, float, int, bool, bool, bool, HybridCounts *,
+                          hipStream_t) { return MX_ERR_DEVICE; }
+int HybridDevice::csr_part(bool, int **, int **, void **, int *, char **) { return MX_ERR_DEVICE; }
+int HybridDevice::strip_layout(const std::vector<int> &, const std::vector<int> &, const std::vector<int> &, long long, DeviceTiles &)
+{
+    return MX_ERR_DEVICE;
+}
 hipError_t launch_probe_f64(const double *, const double *, double *, hipStream_t) { return hipErrorUnknown; }
 hipError_t launch_probe_f16(const void *, const void *, float *, hipStream_t) { return hipErrorUnknown; }
 }

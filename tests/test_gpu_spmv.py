@@ -884,6 +884,19 @@ def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
         assert "Success! All values match" in out.stdout
         hashes.append(json.loads(out.stdout.strip().splitlines()[-1])["partition_hash"])
     assert hashes[0] == hashes[1]
+    # --device-plan: nothing but the upload happens on the host; same plan, same lines
+    recs, ratios = [], []
+    for extra in ([], ["--device-plan"]):
+        out = subprocess.run([exe, "--warm", "2", "--iters", "5", "--json", *extra, "0.5", "0.25", str(p)],
+                             capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        assert "Success! All values match" in out.stdout
+        recs.append(json.loads(out.stdout.strip().splitlines()[-1]))
+        ratios.append((re.search(r"cols_ratio = (\d\.\d+)", out.stdout).group(1), re.search(r"TC_nnz_ratio = (\d\.\d+)", out.stdout).group(1)))
+    assert ratios[0] == ratios[1], ratios
+    for k in ("dCols", "dRows", "tile_chunks", "tile_nnz", "csr_nnz", "tc_nnz_ratio"):
+        assert recs[0][k] == recs[1][k], (k, recs[0][k], recs[1][k])
+    assert recs[0]["prep_route"] == 0 and recs[1]["prep_route"] in (1, 2)
     # --partition-cache: written by the first run, read by the second, recomputed when the fractions change
     cache = str(tmp_path / "m_preprocessed.dat")
     seen = []
@@ -1238,3 +1251,98 @@ def test_plan_from_a_matrix_in_device_memory(mx, ora):
     badp[5] = badp[6] + 1
     with pytest.raises(mx.MxError):
         mx.Plan.from_device_csr(badp, ci, va, A.cols)
+
+
+def _strip_matrix(mx, rng, rows, cols, dtype=np.float16):
+    """Rows of dense strips in many shapes (runs on and off the grid of eight, one to nine blocks,
+    separate blocks, groups of one to twenty rows with the same blocks, a column named twice, a row
+    with something outside the strip) among sparse random rows."""
+    rp, ci = [0], []
+    r = 0
+    while r < rows:
+        kind = rng.integers(0, 10)
+        if kind < 6:
+            n = int(rng.integers(1, 5))
+            ci.extend(np.sort(rng.choice(cols, n, replace=False)).tolist())
+            rp.append(len(ci))
+            r += 1
+            continue
+        group = int(rng.integers(1, 21))
+        start = int(rng.integers(0, cols - 200))
+        if kind < 9:
+            start -= start % 8
+        width = int(rng.choice([8, 16, 24, 32, 40, 64, 72]))
+        far = int(rng.integers(0, cols - 16)) // 8 * 8 if kind == 9 else -1
+        for _ in range(min(group, rows - r)):
+            c = np.arange(start, start + width)
+            c = c[rng.random(width) < 0.9]
+            if far >= 0:
+                c = np.union1d(c, np.arange(far, far + 8))
+            c = c.tolist()
+            if rng.random() < 0.03 and c:
+                c.append(c[-1])                      # a column named twice
+            if rng.random() < 0.03:
+                c.append(int(rng.integers(0, cols)))  # something outside the strip
+            ci.extend(c)
+            rp.append(len(ci))
+            r += 1
+    ci = np.asarray(ci, dtype=np.int32)
+    val = rng.integers(-3, 4, ci.size).astype(dtype)
+    val[val == 0] = 1
+    return mx.Csr(rows, cols, np.asarray(rp, dtype=np.int32), ci, val)
+
+
+@pytest.mark.gpu
+def test_hybrid_plan_made_on_the_device(mx, ora):
+    """mx_plan_create_device: extraction, decisions and layouts made on the device from a matrix
+    in device memory give the plan mx_plan_create makes from mx_partition_create of the same
+    matrix -- every counted fact, every array of the layouts byte for byte, y bit for bit --
+    whether the plan keeps strips, nothing, or a form that sends the matrix to the host route."""
+    import torch
+    rng = np.random.default_rng(12)
+    cases = []
+    for cfg, sc, taus in ((5, 0.25, ((1.0, 1.0), (0.5, 0.25))), (5, 0.03, ((1.0, 1.0), (1.0, 0.5))), (4, 0.25, ((1.0, 1.0),)),
+                          (2, 1.0, ((1.0, 1.0), (0.5, 0.5))), (3, 0.1, ((1.0, 1.0),)), (1, 1.0, ((1.0, 1.0),))):
+        A = mx.gen_config(cfg, scale=sc)[0]
+        cases += [("config %d x %g" % (cfg, sc), A, t) for t in taus]
+    S = _strip_matrix(mx, rng, 60000, 70000)
+    cases += [("strips of many shapes", S, (1.0, 1.0)), ("strips of many shapes", S, (0.75, 0.5))]
+    routes, strip_plans = set(), 0
+    for name, A, (tc, tr) in cases:
+        x = rng.integers(-2, 3, A.cols).astype(A.val.dtype)
+        xd = torch.from_numpy(x).cuda()
+        rp, ci, va = torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda()
+        ref = oracle_y(ora, mx, A, x)
+        part = mx.Partition(A, tc, tr)
+        for flags in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_NO_TILES, mx.MX_PLAN_CSR_ROWS):
+            print("device hybrid plan: %s tau=(%g, %g) flags=%d rows=%d nnz=%d" % (name, tc, tr, flags, A.rows, A.nnz), flush=True)
+            H = mx.Plan(part, flags)
+            D = mx.Plan.from_device(rp, ci, va, A.cols, tc, tr, flags)
+            routes.add(D.info["prep_route"])
+            for k in ("csr_variant", "csr_value_dict", "csr_nnz", "csr_blocks", "tile_nnz", "tile_chunks", "tile_frags", "tile_variant",
+                      "tile_strip_nnz"):
+                assert H.info[k] == D.info[k], (name, tc, tr, flags, k, H.info[k], D.info[k])
+            assert abs(H.info["est_rows_us"] - D.info["est_rows_us"]) < 1e-9 and abs(H.info["est_slices_us"] - D.info["est_slices_us"]) < 1e-9
+            ah, ad = H.arrays(), D.arrays()
+            assert sorted(ah) == sorted(ad), (name, flags, sorted(ah), sorted(ad))
+            for k in ah:
+                assert len(ah[k]) == len(ad[k]), (name, flags, k, len(ah[k]), len(ad[k]))
+                if ah[k] != ad[k]:
+                    a, b = np.frombuffer(ah[k], np.uint8), np.frombuffer(ad[k], np.uint8)
+                    at = int(np.flatnonzero(a != b)[0])
+                    raise AssertionError("%s tau=(%g, %g) flags=%d: %s differs from byte %d of %d" % (name, tc, tr, flags, k, at, a.size))
+            if D.info["prep_route"] == 1 and D.info["tile_strip_nnz"] > 0:
+                strip_plans += 1
+            yh, yd = H.spmv(xd).cpu().numpy(), D.spmv(xd).cpu().numpy()
+            assert np.array_equal(yh.view(np.uint8), yd.view(np.uint8)), (name, flags)
+            assert rel_l2(yd, ref) <= (F64_TOL if A.dtype == mx.MX_F64 else F16_TOL)
+            H.close()
+            D.close()
+        part.close()
+    assert routes == {1, 2}, routes
+    assert strip_plans >= 3, strip_plans
+    bad = ci.clone()
+    bad[7] = A.cols
+    with pytest.raises(mx.MxError) as e:
+        mx.Plan.from_device(rp, bad, va, A.cols, 1.0, 1.0)
+    assert e.value.code == 1
