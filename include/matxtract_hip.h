@@ -356,7 +356,9 @@ int mx_time_kernels(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int
  * candidates are the `levels` x `levels` grid {0, 1/(levels-1), .. 1}^2 with tau_c >= tau_r, each
  * one partitioned, planned (with `flags`) and timed on the device with the protocol of mx_time
  * (`warm` untimed and `iters` timed back-to-back products of a seeded x).  Candidates that send
- * nothing to the tile kernel are one and the same plan and are timed once, as (0, 0).
+ * nothing to the tile kernel are one and the same plan and are timed once, as (0, 0).  A matrix of
+ * two million entries or more is uploaded once and every candidate's extraction and plan are made
+ * on the device (mx_plan_create_device: the same plans).
  * Returns the fastest in tau_c/tau_r; when `table` is given, up to `cap` candidates are written
  * to it in grid order (tau_c outer, ascending) and *n_points is set to their number. */
 typedef struct mx_tau_point {

@@ -2917,6 +2917,28 @@ extern "C" int mx_tune_tau(const mx_csr *A, int levels, int flags, int warm, int
             return rc;
         }
     }
+    // The tuner needs the device anyway: a large matrix goes up once and every candidate's extraction
+    // and plan are made there (mx_plan_create_device: the same plans, a fraction of the time); below
+    // about two million entries the host route is as fast.
+    const bool onDevice = A->nnz >= (1 << 21) && A->rows > 0 && A->cols > 0;
+    int *dRowPtr = nullptr, *dColInd = nullptr;
+    void *dVal = nullptr;
+    auto release = [&]() {
+        (void)hipFree(dx);
+        (void)hipFree(dy);
+        (void)hipFree(dRowPtr);
+        (void)hipFree(dColInd);
+        (void)hipFree(dVal);
+    };
+    if (onDevice) {
+        rc = upload(&dRowPtr, A->rowPtr, (size_t)A->rows + 1);
+        if (!rc) rc = upload(&dColInd, A->colInd, (size_t)A->nnz);
+        if (!rc) rc = upload_bytes(&dVal, A->val, (size_t)A->nnz * es);
+        if (rc) {
+            release();
+            return rc;
+        }
+    }
     double best = 0.0, csrOnly = -1.0;
     bool have = false;
     int n = 0;
@@ -2928,30 +2950,32 @@ extern "C" int mx_tune_tau(const mx_csr *A, int levels, int flags, int warm, int
             mx_plan *plan = nullptr;
             double ms = 0.0;
             int tileNnz = 0;
-            // the tuner needs the device anyway: large matrices are also extracted there (same partition,
-            // a fraction of the time; below about two million entries the copies cost more than they save)
-            if ((rc = (A->nnz >= (1 << 21) ? mx_partition_create_device(A, c, r, &P) : mx_partition_create(A, c, r, &P)))) break;
-            // entries the plan would hand to the tile kernel
-            bool anyTile = false;
-            if (P->extracted && !(flags & MX_PLAN_NO_TILES)) {
-                const double gate = tile_gate(P->dtype) * P->fragM * P->fragK;
-                const int nFrags = P->chunkPtr[P->chunkNum];
-                for (int f = 0; f < nFrags && !anyTile; ++f) {
-                    const int vals = P->fragPtr[f + 1] - P->fragPtr[f];
-                    anyTile = (flags & MX_PLAN_ALL_TILES) ? vals > 0 : (vals > 0 && (double)vals >= gate);
+            bool anyTile = false;  // does the candidate hand anything to a tile kernel?
+            if (onDevice) {
+                if ((rc = mx_plan_create_device(A->dtype, A->rows, A->cols, A->nnz, dRowPtr, dColInd, dVal, c, r, flags, &plan))) break;
+                anyTile = plan->tile_nnz > 0;
+            } else {
+                if ((rc = mx_partition_create(A, c, r, &P))) break;
+                if (P->extracted && !(flags & MX_PLAN_NO_TILES)) {
+                    const double gate = tile_gate(P->dtype) * P->fragM * P->fragK;
+                    const int nFrags = P->chunkPtr[P->chunkNum];
+                    for (int f = 0; f < nFrags && !anyTile; ++f) {
+                        const int vals = P->fragPtr[f + 1] - P->fragPtr[f];
+                        anyTile = (flags & MX_PLAN_ALL_TILES) ? vals > 0 : (vals > 0 && (double)vals >= gate);
+                    }
                 }
             }
             if (!anyTile && csrOnly >= 0.0) {
                 ms = csrOnly;  // the same plan as an earlier candidate
             } else {
-                rc = mx_plan_create(P, flags, &plan);
+                if (!plan) rc = mx_plan_create(P, flags, &plan);
                 if (!rc) rc = mx_time(plan, dx, dy, warm, iters, &ms, nullptr, nullptr);
                 if (!rc) {
                     tileNnz = plan->tile_nnz;
                     if (!anyTile) csrOnly = ms;
                 }
-                mx_plan_destroy(plan);
             }
+            mx_plan_destroy(plan);
             mx_partition_destroy(P);
             if (rc) break;
             if (table && n < cap) table[n] = mx_tau_point{c, r, ms, tileNnz};
@@ -2964,8 +2988,7 @@ extern "C" int mx_tune_tau(const mx_csr *A, int levels, int flags, int warm, int
                 have = true;
             }
         }
-    (void)hipFree(dx);
-    (void)hipFree(dy);
+    release();
     if (n_points) *n_points = n;
     return rc;
 }
