@@ -1606,7 +1606,7 @@ struct PhaseLog {
     {
         if (!on) return;
         const auto now = std::chrono::steady_clock::now();
-        std::fprintf(stderr, "mx_plan_create: %-28s %8.1f ms\n", what, std::chrono::duration<double, std::milli>(now - t).count());
+        std::fprintf(stderr, "mx_plan_create: %-38s %8.1f ms\n", what, std::chrono::duration<double, std::milli>(now - t).count());
         t = now;
     }
 };
@@ -2345,9 +2345,11 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
         while ((double)minVals < need) ++minVals;
         mx::HybridDevice H;
         mx::HybridCounts cnt;
+        PhaseLog phase;
         rc = H.analyse(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, tau_c, tau_r, minVals, !noTiles, wantStrips, wantBlocks, &cnt,
                        nullptr);
         if (rc) return rc;
+        phase("extraction, gate, strip rows (device)");
         if (cnt.blocks64) cnt.generalFrags = cnt.generalEntries = 0;  // the general tiles are not used beside blocks
         int worth = 2;
         if (noTiles) worth = 0;
@@ -2397,7 +2399,9 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
         }
         int partNnz = 0;
         if ((rc = H.csr_part(keepStrips, &partPtr, &partCol, &partVal, &partNnz, &stripRows))) return fail(rc);
+        phase("CSR part assembled (device)");
         if ((rc = setup_csr_part_device(plan, partNnz, partPtr, partCol, partVal, flags, stripRows))) return fail(rc);
+        phase("CSR part layout (device)");
         if (keepStrips) {
             std::vector<int> stepDesc, chunkBlock0, waveDesc;
             long long totalBlocks = 0;
@@ -2413,6 +2417,7 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
             if ((rc = H.strip_layout(stepDesc, chunkBlock0, waveDesc, totalBlocks, T))) return fail(rc);
             T.ownedRows = true;  // strip rows have nothing in the CSR part, which leaves zeros there
             plan->tile_nnz = T.vals;
+            phase("strip steps (device)");
         }
         (void)hipFree(partPtr);
         (void)hipFree(partCol);
