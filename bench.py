@@ -289,7 +289,10 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
                        "how": "median of 15 single products, each after a 1 GiB buffer sweep and a sync; the quoted value "
                               "is the back-to-back (warm) one"},
         "rel_l2_vs_oracle": rel_l2,
+        # mx_plan_create from a partition in host memory; mx_plan_create_device from the matrix in device memory,
+        # extraction included (matrix_to_first_y has both routes whole)
         "plan_create_ms": host_route["plan_create_ms"],
+        "plan_create_device_ms": route["device"]["plan_create_ms"],
         "matrix_to_first_y": route,
         "plan_estimates_us": {"rows": info["est_rows_us"], "slices": info["est_slices_us"]},
         "csr_only_ms": csr_only and csr_only["ms_total"],
@@ -355,7 +358,7 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"], out["cpu_all_cores"] = cpu_baseline(mx, ora, A, x)
     del A, x
-    for k in ("hbm_frac_whole_spmv", "cold_cache", "rel_l2_vs_oracle", "plan_create_ms", "matrix_to_first_y",
+    for k in ("hbm_frac_whole_spmv", "cold_cache", "rel_l2_vs_oracle", "plan_create_ms", "plan_create_device_ms", "matrix_to_first_y",
               "plan_estimates_us", "csr_only_ms", "best_hybrid", "tile_nnz", "csr_nnz", "ms_per_step_events",
               "algorithmic_bytes", "sweep", "sweep_seconds"):
         out[k] = main_rec[k]

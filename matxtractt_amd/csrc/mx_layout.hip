@@ -749,6 +749,12 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
 int check_csr_device(int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, hipStream_t s, const char *who)
 {
     using namespace mxl;
+    // (the kernels number entries and rows with 32-bit thread indices, rounded up to whole workgroups)
+    constexpr int most = 2147483647 - 2 * kBlock;
+    if (rows > most || cols > most || nnz > most) {
+        set_error(std::string(who) + ": more rows, columns or entries than the device route can number");
+        return MX_ERR_ARG;
+    }
     Buf bad;
     MXL_TRY(hipMalloc(&bad.p, 256));
     MXL_TRY(hipMemsetAsync(bad.p, 0, 256, s));

@@ -147,9 +147,20 @@ def test_full_size_mixed_workload_with_its_strips(mx, ora):
     print("workload 5 tau=(1,1):", info, flush=True)
     assert info["tile_variant"] == 1 and info["tile_strip_nnz"] > 0.4 * A.nnz
     assert info["tile_nnz"] + info["csr_nnz"] == A.nnz
-    y = plan.spmv(torch.from_numpy(x).cuda())
+    xd = torch.from_numpy(x).cuda()
+    y = plan.spmv(xd)
     torch.cuda.synchronize()
     assert rel_l2(y.cpu().numpy(), ref) <= F16_TOL
+    # the same plan made on the device from the matrix in device memory: same facts, same y bit for bit
+    dplan = mx.Plan.from_device(torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda(),
+                                A.cols, 1.0, 1.0)
+    assert dplan.info["prep_route"] == 1
+    for k in ("csr_variant", "csr_nnz", "csr_blocks", "tile_nnz", "tile_chunks", "tile_frags", "tile_variant", "tile_strip_nnz"):
+        assert dplan.info[k] == info[k], (k, dplan.info[k], info[k])
+    yd = dplan.spmv(xd)
+    torch.cuda.synchronize()
+    assert torch.equal(y, yd)
+    dplan.close()
     plan.close()
     part.close()
 
