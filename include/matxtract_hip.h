@@ -265,10 +265,12 @@ int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int nnz, const
  * of the matrix crosses to the host: decisions are made there from counts (fragments and entries
  * that pass the gate, blocks and entries per strip chunk, lengths of the slice layout's chunks).
  * The plan equals -- array for array, and so y bit for bit -- the one mx_plan_create makes from
- * mx_partition_create of the same matrix with the same fractions and flags.  Two tile forms are not
- * laid out on the device, the general one and the binary64 8 x 8 blocks; they are counted there, and
- * a matrix on which the plan keeps one of them (with default flags none of the workloads measured;
- * always with MX_PLAN_ALL_TILES) is copied to the host and goes through mx_partition_create_device
+ * mx_partition_create of the same matrix with the same fractions and flags.  The general tile form
+ * is laid out there as well (the columns of a chunk's fragments sorted by the caller's ids with one
+ * radix sort over all chunks, the values placed by the walk over A_dd that assembles the CSR part).
+ * One tile form is not: the binary64 8 x 8 blocks are counted on the device, and a matrix on which
+ * the plan keeps them (none of the workloads measured with default flags: they do not pay below
+ * about 45 000 dense blocks) is copied to the host and goes through mx_partition_create_device
  * and mx_plan_create -- mx_plan_info.prep_route says which way a plan came.  Every pointer is a
  * device pointer; the arrays are read during the call and may be released after it; rowPtr_dev and
  * colInd_dev are checked on the device before they are used as addresses (MX_ERR_ARG).

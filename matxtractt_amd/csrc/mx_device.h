@@ -203,8 +203,16 @@ struct HybridDevice {
     // minVals: entries a fragment needs to pass the gate; want*: which forms the flags allow
     int analyse(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, const void *val_dev, float tau_c,
                 float tau_r, int minVals, bool wantGeneral, bool wantStrips, bool wantBlocks, HybridCounts *counts, hipStream_t s);
-    // stripRows_dev: marks of the rows the strips write (null when keepStrips is false or there are none)
-    int csr_part(bool keepStrips, int **rowPtr_dev, int **col_dev, void **val_dev, int *nnz, char **stripRows_dev);
+    // stripRows_dev: marks of the rows the strips write (null when keepStrips is false or there are none).
+    // keepGeneral: the fragments that pass the gate go to the general tile form -- tile_chunks and tile_layout
+    // come first then, and the values of that layout are filled here.
+    int csr_part(bool keepStrips, bool keepGeneral, int **rowPtr_dev, int **col_dev, void **val_dev, int *nnz, char **stripRows_dev);
+    // the general tile form: blocks per chunk that has any (chunk order); then the layout from the caller's steps --
+    // stepDesc has 10 ints per step: the 8 of strip_layout with chunks numbered as in `blocks`, then the first block
+    // of half 0 inside its chunk (a chunk of more blocks than a step holds takes several), then 0
+    int tile_chunks(bool keepStrips, std::vector<int> &blocks);
+    int tile_layout(bool keepStrips, const std::vector<int> &stepDesc, const std::vector<int> &chunkBlock0, const std::vector<int> &waveDesc,
+                    long long totalBlocks, DeviceTiles &T);
     // stepDesc: 8 ints per step {chunk of half 0, chunk of half 1 (-1 none, -2 the first goes on), flags, blocks in half 0,
     // blocks in half 1, first value, first value and blocks in half 0 of the step four further on}; chunkBlock0: first block
     // of every chunk; T receives waveDesc, hdr, atox and tcVal

@@ -7,9 +7,9 @@
 // the host (a few bytes each), never an entry of the matrix.  The reference does all of this on
 // the host (test/test_autotc_spmv.cpp:1099-1421).
 //
-// What this route does not lay out -- the general tile form and the binary64 block form -- it
-// only counts, so that the caller can decide exactly as the host route does and, when one of
-// those forms is to be kept, take the host route for that matrix.
+// The general tile form is laid out here as well (tile_chunks, tile_layout).  The binary64 block
+// form is only counted, so that the caller can decide exactly as the host route does and, when the
+// blocks are to be kept, take the host route for that matrix.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -416,6 +416,192 @@ __global__ __launch_bounds__(kBlock) void strip_values_kernel(const int *__restr
     }
 }
 
+
+// ---- the general tile form: the reference's fragments that pass the gate, re-blocked.
+// One thread per chunk of the reference's numbering: which of its fragments pass the gate on what the
+// taken rows leave (selFrag), which of their column positions are still in use -- one sort key
+// (chunk, caller's column) each, all ones for a position out of use -- how many there are, and how
+// many of the chunk's column ids are real (the list is padded with zeros to whole fragments).
+template <bool F64>
+__global__ __launch_bounds__(kBlock) void chunk_refs_kernel(const int *__restrict__ chunkPtr, const void *__restrict__ fragBit,
+                                                            const int *__restrict__ atox, const int *__restrict__ descColId,
+                                                            const unsigned char *__restrict__ taken, int chunkNum, int dRows, int minVals,
+                                                            unsigned char *__restrict__ selFrag, unsigned long long *__restrict__ refKey,
+                                                            int *__restrict__ nrefs, int *__restrict__ usedCols)
+{
+    constexpr int K = F64 ? 4 : 8;
+    const int w = blockIdx.x * kBlock + threadIdx.x;
+    if (w >= chunkNum) return;
+    unsigned long long rowsLeft = 0;
+    for (int r = 0; r < 8; ++r) {
+        const int i = w * 8 + r;
+        if (i < dRows && !(taken && taken[i])) rowsLeft |= (F64 ? 0xfull : 0xffull) << (r * K);
+    }
+    const int f0 = chunkPtr[w], f1 = chunkPtr[w + 1];
+    int n = 0;
+    for (int f = f0; f < f1; ++f) {
+        const unsigned long long bm = F64 ? (unsigned long long)((const unsigned *)fragBit)[f] : ((const unsigned long long *)fragBit)[f];
+        const unsigned long long left = bm & rowsLeft;
+        const int vals = __popcll(left);
+        const bool pass = vals > 0 && vals >= minVals;
+        selFrag[f] = pass ? 1 : 0;
+        for (int c = 0; c < K; ++c) {
+            const unsigned long long colBits = (F64 ? 0x11111111ull : 0x0101010101010101ull) << c;
+            const bool used = pass && (left & colBits) != 0;
+            refKey[(size_t)f * K + c] =
+                used ? ((unsigned long long)(unsigned)w << 32) | (unsigned)descColId[atox[(size_t)f * K + c]] : ~0ull;
+            n += used;
+        }
+    }
+    nrefs[w] = n;
+    int u = (f1 - f0) * K;
+    const int *a = atox + (size_t)f0 * K;
+    while (u > 1 && a[u - 1] == 0) --u;
+    usedCols[w] = u;
+}
+// sorted position -> the column there and, for the (fragment, position) it came from, its place in the chunk
+__global__ __launch_bounds__(kBlock) void ref_places_kernel(const unsigned long long *__restrict__ key, const int *__restrict__ pay,
+                                                            const int *__restrict__ refStart, int n, int *__restrict__ sortedCol,
+                                                            int *__restrict__ where)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const unsigned long long k = key[i];
+    const int w = (int)(k >> 32);
+    sortedCol[i] = (int)(unsigned)k;
+    where[pay[i]] = i - refStart[w];
+}
+__global__ __launch_bounds__(kBlock) void chunk_blocks_kernel(const int *__restrict__ nrefs, int chunkNum, int K, int *__restrict__ isSel)
+{
+    const int w = blockIdx.x * kBlock + threadIdx.x;
+    if (w <= chunkNum) isSel[w] = w < chunkNum && nrefs[w] > 0 ? 1 : 0;
+}
+__global__ __launch_bounds__(kBlock) void sel_chunks_kernel(const int *__restrict__ nrefs, const int *__restrict__ isSel,
+                                                            const int *__restrict__ selPos, int chunkNum, int K, int *__restrict__ selW,
+                                                            int *__restrict__ selNb)
+{
+    const int w = blockIdx.x * kBlock + threadIdx.x;
+    if (w >= chunkNum || !isSel[w]) return;
+    selW[selPos[w]] = w;
+    selNb[selPos[w]] = (nrefs[w] + K - 1) / K;
+}
+// stepDesc[s] = {selected chunk of half 0, of half 1 (-1 none, -2 the first goes on), flags, blocks in
+// half 0, blocks in half 1, first value, first value and blocks in half 0 of the step four further on,
+// first block of half 0 inside its chunk}; one wave per step writes header and column ids.
+template <bool F64>
+__global__ __launch_bounds__(64) void tile_steps_kernel(const int *__restrict__ stepDesc, const int *__restrict__ selW,
+                                                        const int *__restrict__ nrefs, const int *__restrict__ refStart,
+                                                        const int *__restrict__ sortedCol, const unsigned char *__restrict__ taken,
+                                                        const int *__restrict__ rId, int dRows, int steps, int *__restrict__ hdr,
+                                                        int *__restrict__ atox)
+{
+    constexpr int K = F64 ? 4 : 8, SLOTS = F64 ? 16 : 8;
+    const int s = blockIdx.x, l = threadIdx.x;
+    if (s >= steps) return;
+    const int *d = stepDesc + (size_t)s * 10;
+    const int A = selW[d[0]], B = d[1] >= 0 ? selW[d[1]] : d[1], n0 = d[3], n1 = d[4], i0 = d[8];
+    // column c of the block in a slot, -1 = none
+    auto column = [&](int slot, int c) {
+        const int half = F64 ? (slot & 1) : (slot >> 2), i = F64 ? (slot >> 1) : (slot & 3);
+        int X, b;
+        if (half == 0) {
+            if (i >= n0) return -1;
+            X = A;
+            b = i0 + i;
+        } else {
+            if (i >= n1) return -1;
+            X = B >= 0 ? B : A;
+            b = B >= 0 ? i : i0 + n0 + i;
+        }
+        const int at = b * K + c;
+        return at < nrefs[X] ? sortedCol[refStart[X] + at] : -1;
+    };
+    auto out_row = [&](int X, int i) {
+        const int local = X * 8 + i;
+        return local < dRows && !(taken && taken[local]) ? rId[local] : -1;
+    };
+    if (l < mx::kTileHdr) {
+        int v = 0;
+        if (l < 8) v = out_row(A, l);
+        else if (l < 16) v = B >= 0 ? out_row(B, l - 8) : -1;
+        else if (l == 16) v = d[2];
+        else if (l == 17) v = n0;
+        else if (l == 18) v = n1;
+        else if (l == 19) v = d[6];
+        else if (l == 20) v = d[7];
+        else if (l < 29) v = SLOTS == 8 ? column(l - 21, 0) : -1;
+        hdr[(size_t)s * mx::kTileHdr + l] = v;
+    }
+    atox[(size_t)s * 64 + l] = column(l / K, l % K);
+}
+// One thread per row of A_dd walks the row beside its chunk's column list (both ascending), which
+// gives every entry its fragment and position.  COUNT: how many entries stay in the CSR part (the row's
+// earlier twins and the entries of fragments that failed the gate; none of a taken row).  Otherwise:
+// those entries written behind the row's residual entries, and the others into the tile values.
+template <typename V, bool COUNT>
+__global__ __launch_bounds__(kBlock) void dd_rows_kernel(const int *__restrict__ ddRowPtr, const int *__restrict__ ddCol,
+                                                         const V *__restrict__ ddVal, const int *__restrict__ descColId,
+                                                         const int *__restrict__ rId, const unsigned char *__restrict__ taken,
+                                                         const int *__restrict__ chunkPtr, const int *__restrict__ atox,
+                                                         const int *__restrict__ usedCols, const unsigned char *__restrict__ selFrag,
+                                                         int dRows, int K, int *__restrict__ kept,
+                                                         // (not COUNT)
+                                                         const int *__restrict__ cdRowPtr, const int *__restrict__ outPtr,
+                                                         int *__restrict__ col, V *__restrict__ val, const int *__restrict__ where,
+                                                         const int *__restrict__ selPos, const int *__restrict__ chunkBlock0,
+                                                         V *__restrict__ tcVal)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= dRows) return;
+    const int p0 = ddRowPtr[i], p1 = ddRowPtr[i + 1];
+    const bool rowTaken = taken && taken[i];
+    if (rowTaken) {
+        if (COUNT) kept[i] = 0;
+        return;
+    }
+    const int w = i >> 3, r8 = i & 7, f0 = chunkPtr[w], na = usedCols[w];
+    const int *a = atox + (size_t)f0 * K;
+    int rank = 0, n = 0, q = 0;
+    size_t base = 0;
+    if (!COUNT) {
+        const int r = rId[i];
+        q = outPtr[r] + (cdRowPtr[r + 1] - cdRowPtr[r]);
+        base = (size_t)chunkBlock0[selPos[w]] * 8 * K;  // (read only when the chunk has selected fragments)
+    }
+    for (int p = p0; p < p1; ++p) {
+        const int c = ddCol[p];
+        while (rank < na && a[rank] < c) ++rank;
+        const bool earlierTwin = p + 1 < p1 && ddCol[p + 1] == c;
+        const int f = f0 + rank / K;
+        const bool keep = earlierTwin || !selFrag[f];
+        if (COUNT) {
+            n += keep;
+        } else if (keep) {
+            col[q] = descColId[c];
+            val[q] = ddVal[p];
+            ++q;
+        } else {
+            const int at = where[(size_t)f * K + rank % K];  // place of the column among the chunk's, ascending by caller's id
+            tcVal[base + (size_t)(at / K) * 8 * K + r8 * K + at % K] = ddVal[p];
+        }
+    }
+    if (COUNT) kept[i] = n;
+}
+__global__ __launch_bounds__(kBlock) void part_lengths_kept_kernel(const int *__restrict__ cdRowPtr, const int *__restrict__ kept,
+                                                                   const int *__restrict__ ddRowOf, const unsigned char *__restrict__ taken,
+                                                                   int rows, int *__restrict__ len, char *__restrict__ stripRows)
+{
+    const int r = blockIdx.x * kBlock + threadIdx.x;
+    if (r > rows) return;
+    if (r == rows) {
+        len[r] = 0;
+        return;
+    }
+    const int i = ddRowOf[r];
+    len[r] = cdRowPtr[r + 1] - cdRowPtr[r] + (i >= 0 ? kept[i] : 0);
+    if (stripRows) stripRows[r] = i >= 0 && taken && taken[i] ? 1 : 0;
+}
+
 }  // namespace mxh
 
 #define MXH_TRY(call)                                                                                 \
@@ -448,6 +634,10 @@ struct HybridDevice::Impl {
     // strip chunks
     int nCand = 0, nChunks = 0;
     Buf perm, candRow, candKey, candNb, runIdIncl, runStart, memberChunk, chunkRows, chunkKey, chunkNb, chunkNnz;
+    // the general tile form (tile_chunks)
+    int minVals = 1, nSel = 0;
+    Buf selFrag, usedCols, nrefs, refStart, sortedCol, where, selPos, selW, tileBlock0;
+    void *tileVal = nullptr;  // the values of the general tile layout (owned by the caller's DeviceTiles): csr_part fills them
     ~Impl() { mx_tiles_device_free(&T); }
 };
 
@@ -466,6 +656,7 @@ int HybridDevice::analyse(mx_dtype dtype, int rows, int cols, int nnz, const int
     I.cols = cols;
     I.nnz = nnz;
     I.s = s;
+    I.minVals = minVals;
     *counts = HybridCounts();
     const size_t es = (size_t)mx::elem_size(dtype);
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
@@ -684,21 +875,39 @@ int HybridDevice::analyse(mx_dtype dtype, int rows, int cols, int nnz, const int
 }
 
 template <typename V>
-static int csr_part_t(HybridDevice::Impl &I, bool keepStrips, int **rowPtrOut, int **colOut, void **valOut, int *nnzOut, char **stripRowsOut)
+static int csr_part_t(HybridDevice::Impl &I, bool keepStrips, bool keepGeneral, int **rowPtrOut, int **colOut, void **valOut, int *nnzOut,
+                      char **stripRowsOut)
 {
     using namespace mxh;
     hipStream_t s = I.s;
-    const int rows = I.rows;
+    const int rows = I.rows, K = mx::frag_k(I.dtype);
     const unsigned char *taken = keepStrips && I.nChunks > 0 ? (const unsigned char *)I.taken.p : nullptr;
-    Buf len, ptr, tmp, col, val, marks;
+    const bool general = keepGeneral && I.nSel > 0 && I.dRows > 0;
+    if (general && !I.tileVal) {
+        mx::set_error("hybrid plan on the device: the tile layout has to be made before the CSR part");
+        return MX_ERR_ARG;
+    }
+    Buf len, ptr, tmp, col, val, marks, kept;
     size_t scanBytes = 0;
     MXH_TRY(rocprim::exclusive_scan(nullptr, scanBytes, (const int *)nullptr, (int *)nullptr, 0, (size_t)rows + 1, rocprim::plus<int>(), s));
     MXH_TRY(hipMalloc(&len.p, ((size_t)rows + 1) * 4));
     MXH_TRY(hipMalloc(&ptr.p, ((size_t)rows + 1) * 4));
     MXH_TRY(hipMalloc(&tmp.p, scanBytes + 256));
     if (taken) MXH_TRY(hipMalloc(&marks.p, (size_t)rows + 4));
-    hipLaunchKernelGGL(part_lengths_kernel, grid((long long)rows + 1), dim3(kBlock), 0, s, (const int *)I.cdp, (const int *)I.ddp,
-                       (const int *)I.ddRowOf.p, taken, rows, len.as<int>(), taken ? marks.as<char>() : nullptr);
+    if (general) {
+        MXH_TRY(hipMalloc(&kept.p, (size_t)I.dRows * 4 + 4));
+        hipLaunchKernelGGL((dd_rows_kernel<V, true>), grid(I.dRows), dim3(kBlock), 0, s, (const int *)I.ddp, (const int *)I.ddc,
+                           (const V *)I.ddv, (const int *)I.dc, (const int *)I.dr, taken, (const int *)I.T.chunkPtr,
+                           (const int *)I.T.sparse_AToX_index, (const int *)I.usedCols.p, (const unsigned char *)I.selFrag.p, I.dRows, K,
+                           kept.as<int>(), (const int *)nullptr, (const int *)nullptr, (int *)nullptr, (V *)nullptr, (const int *)nullptr,
+                           (const int *)nullptr, (const int *)nullptr, (V *)nullptr);
+        MXH_TRY(hipGetLastError());
+        hipLaunchKernelGGL(part_lengths_kept_kernel, grid((long long)rows + 1), dim3(kBlock), 0, s, (const int *)I.cdp, (const int *)kept.p,
+                           (const int *)I.ddRowOf.p, taken, rows, len.as<int>(), taken ? marks.as<char>() : nullptr);
+    } else {
+        hipLaunchKernelGGL(part_lengths_kernel, grid((long long)rows + 1), dim3(kBlock), 0, s, (const int *)I.cdp, (const int *)I.ddp,
+                           (const int *)I.ddRowOf.p, taken, rows, len.as<int>(), taken ? marks.as<char>() : nullptr);
+    }
     MXH_TRY(hipGetLastError());
     MXH_TRY(rocprim::exclusive_scan(tmp.p, scanBytes, (const int *)len.p, ptr.as<int>(), 0, (size_t)rows + 1, rocprim::plus<int>(), s));
     int n = 0;
@@ -711,7 +920,14 @@ static int csr_part_t(HybridDevice::Impl &I, bool keepStrips, int **rowPtrOut, i
                            (const int *)I.colOrig.p, (const int *)ptr.p, rows, I.nCD, col.as<int>(), val.as<V>());
         MXH_TRY(hipGetLastError());
     }
-    if (I.nDD > 0) {
+    if (general) {
+        hipLaunchKernelGGL((dd_rows_kernel<V, false>), grid(I.dRows), dim3(kBlock), 0, s, (const int *)I.ddp, (const int *)I.ddc,
+                           (const V *)I.ddv, (const int *)I.dc, (const int *)I.dr, taken, (const int *)I.T.chunkPtr,
+                           (const int *)I.T.sparse_AToX_index, (const int *)I.usedCols.p, (const unsigned char *)I.selFrag.p, I.dRows, K,
+                           (int *)nullptr, (const int *)I.cdp, (const int *)ptr.p, col.as<int>(), val.as<V>(), (const int *)I.where.p,
+                           (const int *)I.selPos.p, (const int *)I.tileBlock0.p, (V *)I.tileVal);
+        MXH_TRY(hipGetLastError());
+    } else if (I.nDD > 0) {
         hipLaunchKernelGGL(part_dense_kernel<V>, grid(I.nDD), dim3(kBlock), 0, s, (const int *)I.ddp, (const int *)I.ddc, (const V *)I.ddv,
                            (const int *)I.dc, (const int *)I.dr, taken, (const int *)I.cdp, (const int *)ptr.p, I.dRows, I.nDD, col.as<int>(),
                            val.as<V>());
@@ -726,11 +942,130 @@ static int csr_part_t(HybridDevice::Impl &I, bool keepStrips, int **rowPtrOut, i
     return MX_OK;
 }
 
-int HybridDevice::csr_part(bool keepStrips, int **rowPtr_dev, int **col_dev, void **val_dev, int *nnz, char **stripRows_dev)
+int HybridDevice::csr_part(bool keepStrips, bool keepGeneral, int **rowPtr_dev, int **col_dev, void **val_dev, int *nnz, char **stripRows_dev)
 {
     if (!impl) return MX_ERR_ARG;
-    if (impl->dtype == MX_F64) return csr_part_t<double>(*impl, keepStrips, rowPtr_dev, col_dev, val_dev, nnz, stripRows_dev);
-    return csr_part_t<unsigned short>(*impl, keepStrips, rowPtr_dev, col_dev, val_dev, nnz, stripRows_dev);
+    if (impl->dtype == MX_F64) return csr_part_t<double>(*impl, keepStrips, keepGeneral, rowPtr_dev, col_dev, val_dev, nnz, stripRows_dev);
+    return csr_part_t<unsigned short>(*impl, keepStrips, keepGeneral, rowPtr_dev, col_dev, val_dev, nnz, stripRows_dev);
+}
+
+// The chunks of the general tile form: the fragments that pass the gate on what the strips leave,
+// their columns in use sorted by the caller's ids inside every chunk.  blocks: per chunk with at
+// least one such column, in chunk order, the number of blocks of fragK columns it needs.
+int HybridDevice::tile_chunks(bool keepStrips, std::vector<int> &blocks)
+{
+    using namespace mxh;
+    blocks.clear();
+    if (!impl) return MX_ERR_ARG;
+    Impl &I = *impl;
+    hipStream_t s = I.s;
+    const int K = mx::frag_k(I.dtype), chunkNum = I.T.chunkNum, nFrags = I.T.totalTcFrags;
+    I.nSel = 0;
+    if (chunkNum <= 0 || nFrags <= 0) return MX_OK;
+    const unsigned char *taken = keepStrips && I.nChunks > 0 ? (const unsigned char *)I.taken.p : nullptr;
+    const size_t nKey = (size_t)nFrags * K;
+    Buf keyIn, keyOut, payIn, payOut, sortTmp, isSel, scanTmp, selNb;
+    size_t sortBytes = 0, scanBytes = 0;
+    MXH_TRY(rocprim::radix_sort_pairs(nullptr, sortBytes, (const unsigned long long *)nullptr, (unsigned long long *)nullptr,
+                                      (const int *)nullptr, (int *)nullptr, nKey, 0u, 64u, s));
+    MXH_TRY(rocprim::exclusive_scan(nullptr, scanBytes, (const int *)nullptr, (int *)nullptr, 0, (size_t)chunkNum + 1, rocprim::plus<int>(), s));
+    MXH_TRY(hipMalloc(&I.selFrag.p, (size_t)nFrags + 4));
+    MXH_TRY(hipMalloc(&I.usedCols.p, (size_t)chunkNum * 4 + 4));
+    MXH_TRY(hipMalloc(&I.nrefs.p, ((size_t)chunkNum + 1) * 4));
+    MXH_TRY(hipMalloc(&I.refStart.p, ((size_t)chunkNum + 1) * 4));
+    MXH_TRY(hipMalloc(&I.selPos.p, ((size_t)chunkNum + 1) * 4));
+    MXH_TRY(hipMalloc(&I.where.p, nKey * 4 + 4));
+    MXH_TRY(hipMalloc(&keyIn.p, nKey * 8));
+    MXH_TRY(hipMalloc(&keyOut.p, nKey * 8));
+    MXH_TRY(hipMalloc(&payIn.p, nKey * 4));
+    MXH_TRY(hipMalloc(&payOut.p, nKey * 4));
+    MXH_TRY(hipMalloc(&sortTmp.p, sortBytes + 256));
+    MXH_TRY(hipMalloc(&scanTmp.p, scanBytes + 256));
+    MXH_TRY(hipMalloc(&isSel.p, ((size_t)chunkNum + 1) * 4));
+    MXH_TRY(hipMemsetAsync(I.nrefs.p, 0, ((size_t)chunkNum + 1) * 4, s));
+    MXH_TRY(hipMemsetAsync(I.where.p, 0xff, nKey * 4 + 4, s));
+    if (I.dtype == MX_F64)
+        hipLaunchKernelGGL(chunk_refs_kernel<true>, grid(chunkNum), dim3(kBlock), 0, s, (const int *)I.T.chunkPtr, (const void *)I.T.fragBit,
+                           (const int *)I.T.sparse_AToX_index, (const int *)I.dc, taken, chunkNum, I.dRows, I.minVals,
+                           I.selFrag.as<unsigned char>(), keyIn.as<unsigned long long>(), I.nrefs.as<int>(), I.usedCols.as<int>());
+    else
+        hipLaunchKernelGGL(chunk_refs_kernel<false>, grid(chunkNum), dim3(kBlock), 0, s, (const int *)I.T.chunkPtr, (const void *)I.T.fragBit,
+                           (const int *)I.T.sparse_AToX_index, (const int *)I.dc, taken, chunkNum, I.dRows, I.minVals,
+                           I.selFrag.as<unsigned char>(), keyIn.as<unsigned long long>(), I.nrefs.as<int>(), I.usedCols.as<int>());
+    MXH_TRY(hipGetLastError());
+    hipLaunchKernelGGL(iota_kernel, grid((long long)nKey), dim3(kBlock), 0, s, payIn.as<int>(), (int)nKey);
+    MXH_TRY(hipGetLastError());
+    MXH_TRY(rocprim::radix_sort_pairs(sortTmp.p, sortBytes, (const unsigned long long *)keyIn.p, keyOut.as<unsigned long long>(),
+                                      (const int *)payIn.p, payOut.as<int>(), nKey, 0u, 64u, s));
+    MXH_TRY(rocprim::exclusive_scan(scanTmp.p, scanBytes, (const int *)I.nrefs.p, I.refStart.as<int>(), 0, (size_t)chunkNum + 1,
+                                    rocprim::plus<int>(), s));
+    hipLaunchKernelGGL(chunk_blocks_kernel, grid((long long)chunkNum + 1), dim3(kBlock), 0, s, (const int *)I.nrefs.p, chunkNum, K,
+                       isSel.as<int>());
+    MXH_TRY(hipGetLastError());
+    MXH_TRY(rocprim::exclusive_scan(scanTmp.p, scanBytes, (const int *)isSel.p, I.selPos.as<int>(), 0, (size_t)chunkNum + 1,
+                                    rocprim::plus<int>(), s));
+    int nRefs = 0, nSel = 0;
+    MXH_TRY(hipMemcpyAsync(&nRefs, I.refStart.as<int>() + chunkNum, 4, hipMemcpyDeviceToHost, s));
+    MXH_TRY(hipMemcpyAsync(&nSel, I.selPos.as<int>() + chunkNum, 4, hipMemcpyDeviceToHost, s));
+    MXH_TRY(hipStreamSynchronize(s));
+    if (nSel <= 0 || nRefs <= 0) return MX_OK;
+    MXH_TRY(hipMalloc(&I.sortedCol.p, (size_t)nRefs * 4 + 4));
+    MXH_TRY(hipMalloc(&I.selW.p, (size_t)nSel * 4 + 4));
+    MXH_TRY(hipMalloc(&selNb.p, (size_t)nSel * 4 + 4));
+    hipLaunchKernelGGL(ref_places_kernel, grid(nRefs), dim3(kBlock), 0, s, (const unsigned long long *)keyOut.p, (const int *)payOut.p,
+                       (const int *)I.refStart.p, nRefs, I.sortedCol.as<int>(), I.where.as<int>());
+    MXH_TRY(hipGetLastError());
+    hipLaunchKernelGGL(sel_chunks_kernel, grid(chunkNum), dim3(kBlock), 0, s, (const int *)I.nrefs.p, (const int *)isSel.p,
+                       (const int *)I.selPos.p, chunkNum, K, I.selW.as<int>(), selNb.as<int>());
+    MXH_TRY(hipGetLastError());
+    blocks.assign((size_t)nSel, 0);
+    MXH_TRY(hipMemcpyAsync(blocks.data(), selNb.p, (size_t)nSel * 4, hipMemcpyDeviceToHost, s));
+    MXH_TRY(hipStreamSynchronize(s));
+    I.nSel = nSel;
+    return MX_OK;
+}
+
+// The general tile layout: headers and column ids of every step, and the (zeroed) values, which
+// csr_part fills as it walks the rows of A_dd -- so this comes first.
+int HybridDevice::tile_layout(bool keepStrips, const std::vector<int> &stepDesc, const std::vector<int> &chunkBlock0,
+                              const std::vector<int> &waveDesc, long long totalBlocks, DeviceTiles &T)
+{
+    using namespace mxh;
+    if (!impl || impl->nSel <= 0 || (int)chunkBlock0.size() != impl->nSel) return MX_ERR_ARG;
+    Impl &I = *impl;
+    hipStream_t s = I.s;
+    const int steps = (int)(stepDesc.size() / 10), K = mx::frag_k(I.dtype);
+    const size_t es = (size_t)mx::elem_size(I.dtype);
+    const unsigned char *taken = keepStrips && I.nChunks > 0 ? (const unsigned char *)I.taken.p : nullptr;
+    Buf dDesc;
+    MXH_TRY(hipMalloc(&dDesc.p, stepDesc.size() * 4 + 4));
+    MXH_TRY(hipMemcpyAsync(dDesc.p, stepDesc.data(), stepDesc.size() * 4, hipMemcpyHostToDevice, s));
+    MXH_TRY(hipMalloc(&I.tileBlock0.p, ((size_t)I.nSel + 1) * 4));
+    MXH_TRY(hipMemsetAsync(I.tileBlock0.p, 0, ((size_t)I.nSel + 1) * 4, s));
+    MXH_TRY(hipMemcpyAsync(I.tileBlock0.p, chunkBlock0.data(), chunkBlock0.size() * 4, hipMemcpyHostToDevice, s));
+    const size_t nWave = waveDesc.size() + 64, nHdr = (size_t)steps * kTileHdr + 256, nAtox = (size_t)steps * 64 + 256,
+                 valBytes = (size_t)totalBlocks * 8 * K * es + 8192;
+    MXH_TRY(hipMalloc((void **)&T.waveDesc, nWave * 4));
+    MXH_TRY(hipMemsetAsync(T.waveDesc, 0, nWave * 4, s));
+    MXH_TRY(hipMemcpyAsync(T.waveDesc, waveDesc.data(), waveDesc.size() * 4, hipMemcpyHostToDevice, s));
+    MXH_TRY(hipMalloc((void **)&T.hdr, nHdr * 4));
+    MXH_TRY(hipMemsetAsync(T.hdr, 0, nHdr * 4, s));
+    MXH_TRY(hipMalloc((void **)&T.atox, nAtox * 4));
+    MXH_TRY(hipMemsetAsync(T.atox, 0, nAtox * 4, s));
+    MXH_TRY(hipMalloc(&T.tcVal, valBytes));
+    MXH_TRY(hipMemsetAsync(T.tcVal, 0, valBytes, s));
+    if (I.dtype == MX_F64)
+        hipLaunchKernelGGL(tile_steps_kernel<true>, dim3(steps), dim3(64), 0, s, (const int *)dDesc.p, (const int *)I.selW.p,
+                           (const int *)I.nrefs.p, (const int *)I.refStart.p, (const int *)I.sortedCol.p, taken, (const int *)I.dr, I.dRows,
+                           steps, T.hdr, T.atox);
+    else
+        hipLaunchKernelGGL(tile_steps_kernel<false>, dim3(steps), dim3(64), 0, s, (const int *)dDesc.p, (const int *)I.selW.p,
+                           (const int *)I.nrefs.p, (const int *)I.refStart.p, (const int *)I.sortedCol.p, taken, (const int *)I.dr, I.dRows,
+                           steps, T.hdr, T.atox);
+    MXH_TRY(hipGetLastError());
+    MXH_TRY(hipStreamSynchronize(s));
+    I.tileVal = T.tcVal;
+    return MX_OK;
 }
 
 int HybridDevice::strip_layout(const std::vector<int> &stepDesc, const std::vector<int> &chunkBlock0, const std::vector<int> &waveDesc,

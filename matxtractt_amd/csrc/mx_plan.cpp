@@ -2214,66 +2214,71 @@ extern "C" int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int
     return MX_OK;
 }
 
-// The steps of binary16 strip chunks from their block counts alone, as build_tiles lays them out: a
-// chunk of up to four blocks shares a step with the next such chunk (half 0 and half 1), a larger
-// one (up to eight) takes a step of its own with its fifth and further blocks in half 1.
-// stepDesc: 8 ints per step {chunk of half 0, chunk of half 1 (-1 none, -2 the first goes on), flags,
-// blocks in half 0, blocks in half 1, first value, first value and blocks in half 0 of the step four
-// further on}; chunkBlock0: the first block of every chunk in the stored values.
-static int plan_strip_steps(const std::vector<int> &chunkBlocks, int nCU, std::vector<int> &stepDesc, std::vector<int> &chunkBlock0,
-                            std::vector<int> &waveDesc, long long *totalBlocks)
+// The steps of a tile layout from the block counts of its chunks alone, as build_tiles lays them out:
+// a chunk of up to half a step's blocks shares a step with the next such chunk (half 0 and half 1), a
+// larger one takes whole steps of its own, half 0 filled first.  SF: block slots of a step; BS: values
+// per block.  stepDesc: `stride` (8 or 10) ints per step {chunk of half 0, chunk of half 1 (-1 none, -2
+// the first goes on), flags, blocks in half 0, blocks in half 1, first value, first value and blocks in
+// half 0 of the step four further on[, first block of half 0 inside its chunk, 0]}; chunkBlock0: the first
+// block of every chunk in the stored values.
+static int plan_tile_steps(const std::vector<int> &chunkBlocks, int SF, int BS, int perMin, int nCU, int stride, std::vector<int> &stepDesc,
+                           std::vector<int> &chunkBlock0, std::vector<int> &waveDesc, long long *totalBlocks)
 {
-    const int HF = 4, n = (int)chunkBlocks.size();
-    std::vector<int> stepVo, stepA, stepEnd, who;  // who: {chunk of half 0, of half 1, flags, blocks, blocks} per step
+    const int HF = SF / 2, n = (int)chunkBlocks.size();
+    std::vector<int> stepVo, stepA, stepEnd, who;  // who: {chunk of half 0, of half 1, flags, blocks, blocks, first block} per step
     chunkBlock0.assign((size_t)n, 0);
     long long blocks = 0;
     int pending = -1;
-    auto emit = [&](int a, int b, int flags, int n0, int n1) {
-        const int d[5] = {a, b, flags, n0, n1};
-        who.insert(who.end(), d, d + 5);
-        stepVo.push_back((int)(blocks * 64));
+    auto emit = [&](int a, int b, int flags, int n0, int n1, int i0) {
+        const int d[6] = {a, b, flags, n0, n1, i0};
+        who.insert(who.end(), d, d + 6);
+        stepVo.push_back((int)(blocks * BS));
         stepA.push_back(n0);
         stepEnd.push_back(flags & 1);
         blocks += n0 + n1;
     };
     for (int k = 0; k < n; ++k) {
         const int nb = chunkBlocks[k];
-        if (nb < 1 || nb > 2 * HF) {
-            set_error("strip layout: a chunk with an impossible number of blocks");
+        if (nb < 1 || (stride == 8 && nb > SF)) {
+            set_error("tile layout: a chunk with an impossible number of blocks");
             return MX_ERR_DEVICE;
         }
         if (nb <= HF) {
             if (pending >= 0) {
                 chunkBlock0[pending] = (int)blocks;
                 chunkBlock0[k] = (int)blocks + chunkBlocks[pending];
-                emit(pending, k, 3, chunkBlocks[pending], nb);
+                emit(pending, k, 3, chunkBlocks[pending], nb, 0);
                 pending = -1;
             } else {
                 pending = k;
             }
         } else {
             chunkBlock0[k] = (int)blocks;
-            emit(k, -2, 1, HF, nb - HF);
+            for (int i0 = 0; i0 < nb; i0 += SF) {
+                const int m = std::min(nb - i0, SF), n0 = std::min(m, HF);
+                emit(k, -2, i0 + SF >= nb ? 1 : 0, n0, m - n0, i0);
+            }
         }
-        if (blocks * 64 > 2000000000LL) {
+        if (blocks * BS > 2000000000LL) {
             set_error("tile layout: too many values for 32-bit offsets");
             return MX_ERR_ARG;
         }
     }
     if (pending >= 0) {
         chunkBlock0[pending] = (int)blocks;
-        emit(pending, -1, 3, chunkBlocks[pending], 0);
+        emit(pending, -1, 3, chunkBlocks[pending], 0, 0);
     }
     const int steps = (int)stepVo.size();
     std::vector<int> ahead;
-    tile_waves(steps, nCU, 2, stepVo, stepA, stepEnd, waveDesc, ahead);
-    stepDesc.assign((size_t)steps * 8, 0);
+    tile_waves(steps, nCU, perMin, stepVo, stepA, stepEnd, waveDesc, ahead);
+    stepDesc.assign((size_t)steps * stride, 0);
     for (int st = 0; st < steps; ++st) {
-        int *d = &stepDesc[(size_t)st * 8];
-        for (int k = 0; k < 5; ++k) d[k] = who[(size_t)st * 5 + k];
+        int *d = &stepDesc[(size_t)st * stride];
+        for (int k = 0; k < 5; ++k) d[k] = who[(size_t)st * 6 + k];
         d[5] = stepVo[st];
         d[6] = ahead[2 * (size_t)st];
         d[7] = ahead[2 * (size_t)st + 1];
+        if (stride > 8) d[8] = who[(size_t)st * 6 + 5];
     }
     *totalBlocks = blocks;
     return MX_OK;
@@ -2283,9 +2288,9 @@ static int plan_strip_steps(const std::vector<int> &chunkBlocks, int nCU, std::v
 // extraction, the plan's decisions, the CSR part with its layout and the strips' layout are all
 // made on the device (mx_hybrid.hip, mx_layout.hip); what a decision needs comes to the host as
 // counts.  The plan equals the one mx_plan_create makes from mx_partition_create(_device) of the
-// same matrix.  Two tile forms are not laid out on the device -- the general one and the binary64
-// blocks; a matrix on which the plan keeps one of them (none of the measured workloads with
-// default flags) is copied to the host and takes the host route.
+// same matrix.  One tile form is not laid out on the device, the binary64 blocks; a matrix on which
+// the plan keeps them (none of the measured workloads with default flags) is copied to the host and
+// takes the host route.
 extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
                                      const void *val_dev, float tau_c, float tau_r, int flags, mx_plan **out)
 {
@@ -2327,7 +2332,6 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
         if (!e) (*out)->prep_route = 2;
         return e;
     };
-    if (flags & MX_PLAN_ALL_TILES) return host_route();
     try {
         hipDeviceProp_t prop;
         int dev = 0;
@@ -2335,14 +2339,16 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
         MX_HIP(hipGetDeviceProperties(&prop, dev));
         const int nCU = std::max(1, prop.multiProcessorCount);
         const int fragM = mx::kFragM, fragK = mx::frag_k(dtype);
-        const bool noTiles = (flags & MX_PLAN_NO_TILES) != 0;
+        const bool noTiles = (flags & MX_PLAN_NO_TILES) != 0, allTiles = !noTiles && (flags & MX_PLAN_ALL_TILES) != 0;
         const char *envNoStrips = std::getenv("MX_NO_STRIPS"), *envNoBlocks = std::getenv("MX_NO_BLOCKS");
-        const bool wantStrips = dtype == MX_F16 && !noTiles && !(envNoStrips && std::atoi(envNoStrips));
-        const bool wantBlocks = dtype == MX_F64 && !noTiles && !(envNoBlocks && std::atoi(envNoBlocks));
-        // (the smallest count that passes `(double)vals >= gate * fragM * fragK`)
+        const bool wantStrips = dtype == MX_F16 && !noTiles && !allTiles && !(envNoStrips && std::atoi(envNoStrips));
+        const bool wantBlocks = dtype == MX_F64 && !noTiles && !allTiles && !(envNoBlocks && std::atoi(envNoBlocks));
+        // (the smallest count that passes `(double)vals >= gate * fragM * fragK`; every fragment that holds anything
+        // with MX_PLAN_ALL_TILES)
         const double need = tile_gate(dtype) * fragM * fragK;
         int minVals = (int)need;
         while ((double)minVals < need) ++minVals;
+        if (allTiles) minVals = 1;
         mx::HybridDevice H;
         mx::HybridCounts cnt;
         PhaseLog phase;
@@ -2353,11 +2359,12 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
         if (cnt.blocks64) cnt.generalFrags = cnt.generalEntries = 0;  // the general tiles are not used beside blocks
         int worth = 2;
         if (noTiles) worth = 0;
-        else if (!(flags & MX_PLAN_KEEP_TILES))
+        else if (!(flags & (MX_PLAN_KEEP_TILES | MX_PLAN_ALL_TILES)))
             worth = tiles_worth(dtype, fragM, fragK, cnt.blocks64, (double)cnt.generalEntries, (double)cnt.generalFrags,
                                 (double)cnt.stripEntries, (double)cnt.stripBlocks);
-        if ((worth == 2 && cnt.generalFrags > 0) || (worth >= 1 && cnt.blocks64 && cnt.stripBlocks > 0)) return host_route();
+        if (worth >= 1 && cnt.blocks64 && cnt.stripBlocks > 0) return host_route();  // binary64 blocks: laid out on the host
         const bool keepStrips = worth >= 1 && !cnt.blocks64 && cnt.stripBlocks > 0;
+        const bool keepGeneral = worth == 2 && cnt.generalFrags > 0;
 
         mx_plan *plan = new (std::nothrow) mx_plan();
         if (!plan) {
@@ -2397,15 +2404,37 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
                 return fail(MX_ERR_DEVICE);
             }
         }
+        if (keepGeneral) {
+            // the general tile form first: the walk over A_dd that assembles the CSR part also fills its values
+            std::vector<int> chunkBlocks, stepDesc, chunkBlock0, waveDesc;
+            long long totalBlocks = 0;
+            if ((rc = H.tile_chunks(keepStrips, chunkBlocks))) return fail(rc);
+            if (!chunkBlocks.empty()) {
+                const int BS = fragM * fragK;
+                if ((rc = plan_tile_steps(chunkBlocks, mx::tile_slots(dtype), BS, 2, nCU, 10, stepDesc, chunkBlock0, waveDesc, &totalBlocks)))
+                    return fail(rc);
+                mx::DeviceTiles &T = plan->tiles;
+                T.chunkNum = (int)chunkBlocks.size();
+                T.frags = (int)cnt.generalFrags;
+                T.vals = (int)cnt.generalEntries;
+                T.stored = totalBlocks * BS;
+                T.steps = (int)(stepDesc.size() / 10);
+                T.dense = false;
+                T.nWaves = (int)(waveDesc.size() / 8);
+                if ((rc = H.tile_layout(keepStrips, stepDesc, chunkBlock0, waveDesc, totalBlocks, T))) return fail(rc);
+                plan->tile_nnz += T.vals;
+                phase("tile steps (device)");
+            }
+        }
         int partNnz = 0;
-        if ((rc = H.csr_part(keepStrips, &partPtr, &partCol, &partVal, &partNnz, &stripRows))) return fail(rc);
+        if ((rc = H.csr_part(keepStrips, keepGeneral, &partPtr, &partCol, &partVal, &partNnz, &stripRows))) return fail(rc);
         phase("CSR part assembled (device)");
         if ((rc = setup_csr_part_device(plan, partNnz, partPtr, partCol, partVal, flags, stripRows))) return fail(rc);
         phase("CSR part layout (device)");
         if (keepStrips) {
             std::vector<int> stepDesc, chunkBlock0, waveDesc;
             long long totalBlocks = 0;
-            if ((rc = plan_strip_steps(cnt.stripChunkBlocks, nCU, stepDesc, chunkBlock0, waveDesc, &totalBlocks))) return fail(rc);
+            if ((rc = plan_tile_steps(cnt.stripChunkBlocks, 8, 64, 2, nCU, 8, stepDesc, chunkBlock0, waveDesc, &totalBlocks))) return fail(rc);
             mx::DeviceTiles &T = plan->strips;
             T.chunkNum = (int)cnt.stripChunkBlocks.size();
             T.frags = (int)cnt.stripBlocks;
@@ -2416,8 +2445,12 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
             T.nWaves = (int)(waveDesc.size() / 8);
             if ((rc = H.strip_layout(stepDesc, chunkBlock0, waveDesc, totalBlocks, T))) return fail(rc);
             T.ownedRows = true;  // strip rows have nothing in the CSR part, which leaves zeros there
-            plan->tile_nnz = T.vals;
+            plan->tile_nnz += T.vals;
             phase("strip steps (device)");
+        }
+        if (dtype == MX_F16 && plan->tiles.nWaves > 0) {
+            // (general tiles share rows with the CSR part: its sums stay binary32 until the tile kernel has added its own)
+            if ((rc = upload_bytes(&plan->ywide, nullptr, 0, (size_t)std::max(rows, 1) * sizeof(float)))) return fail(rc);
         }
         (void)hipFree(partPtr);
         (void)hipFree(partCol);

@@ -1318,14 +1318,15 @@ def test_hybrid_plan_made_on_the_device(mx, ora):
         cases += [("config %d x %g" % (cfg, sc), A, t) for t in taus]
     S = _strip_matrix(mx, rng, 60000, 70000)
     cases += [("strips of many shapes", S, (1.0, 1.0)), ("strips of many shapes", S, (0.75, 0.5))]
-    routes, strip_plans = set(), 0
+    routes, strip_plans, general_plans = set(), 0, set()
     for name, A, (tc, tr) in cases:
         x = rng.integers(-2, 3, A.cols).astype(A.val.dtype)
         xd = torch.from_numpy(x).cuda()
         rp, ci, va = torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda()
         ref = oracle_y(ora, mx, A, x)
         part = mx.Partition(A, tc, tr)
-        for flags in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_NO_TILES, mx.MX_PLAN_CSR_ROWS):
+        for flags in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_NO_TILES, mx.MX_PLAN_CSR_ROWS, mx.MX_PLAN_ALL_TILES,
+                      mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_ROWS):
             print("device hybrid plan: %s tau=(%g, %g) flags=%d rows=%d nnz=%d" % (name, tc, tr, flags, A.rows, A.nnz), flush=True)
             H = mx.Plan(part, flags)
             D = mx.Plan.from_device(rp, ci, va, A.cols, tc, tr, flags)
@@ -1344,6 +1345,8 @@ def test_hybrid_plan_made_on_the_device(mx, ora):
                     raise AssertionError("%s tau=(%g, %g) flags=%d: %s differs from byte %d of %d" % (name, tc, tr, flags, k, at, a.size))
             if D.info["prep_route"] == 1 and D.info["tile_strip_nnz"] > 0:
                 strip_plans += 1
+            if D.info["prep_route"] == 1 and D.info["tile_nnz"] > D.info["tile_strip_nnz"]:
+                general_plans.add((A.dtype, D.info["tile_strip_nnz"] > 0))
             yh, yd = H.spmv(xd).cpu().numpy(), D.spmv(xd).cpu().numpy()
             assert np.array_equal(yh.view(np.uint8), yd.view(np.uint8)), (name, flags)
             assert rel_l2(yd, ref) <= (F64_TOL if A.dtype == mx.MX_F64 else F16_TOL)
@@ -1352,6 +1355,8 @@ def test_hybrid_plan_made_on_the_device(mx, ora):
         part.close()
     assert routes == {1, 2}, routes
     assert strip_plans >= 3, strip_plans
+    # the general tile form laid out on the device: both precisions, with and without strips beside it
+    assert {(mx.MX_F64, False), (mx.MX_F16, False), (mx.MX_F16, True)} <= general_plans, general_plans
     bad = ci.clone()
     bad[7] = A.cols
     with pytest.raises(mx.MxError) as e:
