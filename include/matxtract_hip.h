@@ -265,13 +265,10 @@ int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int nnz, const
  * of the matrix crosses to the host: decisions are made there from counts (fragments and entries
  * that pass the gate, blocks and entries per strip chunk, lengths of the slice layout's chunks).
  * The plan equals -- array for array, and so y bit for bit -- the one mx_plan_create makes from
- * mx_partition_create of the same matrix with the same fractions and flags.  The general tile form
- * is laid out there as well (the columns of a chunk's fragments sorted by the caller's ids with one
- * radix sort over all chunks, the values placed by the walk over A_dd that assembles the CSR part).
- * One tile form is not: the binary64 8 x 8 blocks are counted on the device, and a matrix on which
- * the plan keeps them (none of the workloads measured with default flags: they do not pay below
- * about 45 000 dense blocks) is copied to the host and goes through mx_partition_create_device
- * and mx_plan_create -- mx_plan_info.prep_route says which way a plan came.  Every pointer is a
+ * mx_partition_create of the same matrix with the same fractions and flags, whatever tile forms it
+ * keeps: the general form (the columns of a chunk's fragments sorted by the caller's ids with one radix
+ * sort over all chunks, the values placed by the walk over A_dd that assembles the CSR part), the
+ * binary16 strips, the binary64 8 x 8 blocks (one sort of (block row, block column) keys).  Every pointer is a
  * device pointer; the arrays are read during the call and may be released after it; rowPtr_dev and
  * colInd_dev are checked on the device before they are used as addresses (MX_ERR_ARG).
  * tau = (0, 0) is mx_plan_create_device_csr. */
@@ -410,8 +407,7 @@ typedef struct mx_plan_info {
                             Nothing is timed unless MX_PLAN_AUTOTUNE=1 is set, so a matrix gets the same plan on
                             every run */
     int prep_route;      /* where the plan's layouts were made: 0 = from host arrays (mx_plan_create), 1 = on the
-                            device from device arrays (mx_plan_create_device, mx_plan_create_device_csr), 2 =
-                            mx_plan_create_device copied the matrix to the host and took the host route */
+                            device from device arrays (mx_plan_create_device, mx_plan_create_device_csr) */
     int ext_dCols, ext_dRows, ext_nnzRowD, ext_frags; /* what the extraction behind the plan selected (columns, rows,
                             entries of A_dd) and the fragments of its tile encoding -- cols_ratio and TC_nnz_ratio of
                             the reference's driver follow from them; 0 for plans without an extraction */

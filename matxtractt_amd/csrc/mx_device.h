@@ -206,7 +206,15 @@ struct HybridDevice {
     // stripRows_dev: marks of the rows the strips write (null when keepStrips is false or there are none).
     // keepGeneral: the fragments that pass the gate go to the general tile form -- tile_chunks and tile_layout
     // come first then, and the values of that layout are filled here.
-    int csr_part(bool keepStrips, bool keepGeneral, int **rowPtr_dev, int **col_dev, void **val_dev, int *nnz, char **stripRows_dev);
+    // keepBlocks (binary64, alone): the entries of the 8 x 8 blocks leave the CSR part and the rows of block chunks are
+    // marked 2 -- block_chunks comes first then.
+    int csr_part(bool keepStrips, bool keepGeneral, bool keepBlocks, int **rowPtr_dev, int **col_dev, void **val_dev, int *nnz,
+                 char **stripRows_dev);
+    // the binary64 block form: blocks per block row that has any and those block rows (ascending); then the layout
+    // from the caller's steps (10 ints per step as for tile_layout)
+    int block_chunks(std::vector<int> &blocks, std::vector<int> &blockRows);
+    int block_layout(const std::vector<int> &stepDesc, const std::vector<int> &chunkBlock0, const std::vector<int> &waveDesc,
+                     long long totalBlocks, DeviceTiles &T);
     // the general tile form: blocks per chunk that has any (chunk order); then the layout from the caller's steps --
     // stepDesc has 10 ints per step: the 8 of strip_layout with chunks numbered as in `blocks`, then the first block
     // of half 0 inside its chunk (a chunk of more blocks than a step holds takes several), then 0

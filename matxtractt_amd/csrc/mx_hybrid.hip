@@ -602,6 +602,160 @@ __global__ __launch_bounds__(kBlock) void part_lengths_kept_kernel(const int *__
     if (stripRows) stripRows[r] = i >= 0 && taken && taken[i] ? 1 : 0;
 }
 
+
+// ---- the binary64 block form: the qualifying runs of the sorted (block row, block column) keys.
+__global__ __launch_bounds__(kBlock) void block_heads_kernel(const unsigned long long *__restrict__ key, int n, int need, int cols,
+                                                             int *__restrict__ selHead)
+{
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p > n) return;
+    int h = 0;
+    if (p < n && key[p] != ~0ull && (p == 0 || key[p - 1] != key[p])) {
+        int e = p + 1;
+        while (e < n && e - p < 64 && key[e] == key[p]) ++e;
+        h = e - p >= need && (int)(unsigned)key[p] + 1 <= cols / 8 ? 1 : 0;
+    }
+    selHead[p] = h;
+}
+// per block (numbered in key order): its block row and column; per entry of A_dd: its block, -1 = none
+__global__ __launch_bounds__(kBlock) void block_records_kernel(const unsigned long long *__restrict__ key, const int *__restrict__ pay,
+                                                               const int *__restrict__ selHead, const int *__restrict__ blockId, int n,
+                                                               int *__restrict__ blkBr, int *__restrict__ blkBc,
+                                                               int *__restrict__ entryBlock)
+{
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= n || !selHead[p]) return;
+    const int g = blockId[p];
+    blkBr[g] = (int)(key[p] >> 32);
+    blkBc[g] = (int)(unsigned)key[p];
+    for (int e = p; e < n && e - p < 64 && key[e] == key[p]; ++e) entryBlock[pay[e]] = g;
+}
+__global__ __launch_bounds__(kBlock) void block_chunk_heads_kernel(const int *__restrict__ blkBr, int nBlocks, int *__restrict__ head)
+{
+    const int g = blockIdx.x * kBlock + threadIdx.x;
+    if (g < nBlocks) head[g] = g == 0 || blkBr[g] != blkBr[g - 1] ? 1 : 0;
+}
+__global__ __launch_bounds__(kBlock) void block_chunk_starts_kernel(const int *__restrict__ head, const int *__restrict__ chunkIdIncl,
+                                                                    const int *__restrict__ blkBr, int nBlocks,
+                                                                    int *__restrict__ chunkStart, int *__restrict__ chunkBr)
+{
+    const int g = blockIdx.x * kBlock + threadIdx.x;
+    if (g >= nBlocks) return;
+    if (head[g]) {
+        chunkStart[chunkIdIncl[g] - 1] = g;
+        chunkBr[chunkIdIncl[g] - 1] = blkBr[g];
+    }
+    if (g == nBlocks - 1) chunkStart[chunkIdIncl[g]] = nBlocks;
+}
+__global__ __launch_bounds__(kBlock) void block_chunk_sizes_kernel(const int *__restrict__ chunkStart, int nChunks, int *__restrict__ nb)
+{
+    const int c = blockIdx.x * kBlock + threadIdx.x;
+    if (c < nChunks) nb[c] = chunkStart[c + 1] - chunkStart[c];
+}
+// marks of the rows of block chunks (2: the block waves fetch the sums of these rows' virtual rows themselves)
+__global__ __launch_bounds__(kBlock) void block_marks_kernel(const int *__restrict__ chunkBr, int nChunks, int rows, char *__restrict__ marks)
+{
+    const int c = blockIdx.x * kBlock + threadIdx.x;
+    if (c >= nChunks) return;
+    for (int j = 0; j < 8; ++j) {
+        const int r = chunkBr[c] * 8 + j;
+        if (r < rows) marks[r] = 2;
+    }
+}
+// stepDesc as for the general form (10 ints per step, chunks numbered in block-row order)
+__global__ __launch_bounds__(64) void block_steps_kernel(const int *__restrict__ stepDesc, const int *__restrict__ chunkStart,
+                                                         const int *__restrict__ chunkBr, const int *__restrict__ blkBc, int rows,
+                                                         int steps, int *__restrict__ hdr, int *__restrict__ atox)
+{
+    const int s = blockIdx.x, l = threadIdx.x;
+    if (s >= steps) return;
+    const int *d = stepDesc + (size_t)s * 10;
+    const int A = d[0], B = d[1], n0 = d[3], n1 = d[4], i0 = d[8];
+    auto first_col = [&](int slot) {
+        const int half = slot >> 2, i = slot & 3;
+        if (half == 0) return i < n0 ? blkBc[chunkStart[A] + i0 + i] * 8 : -1;
+        if (i >= n1) return -1;
+        return (B >= 0 ? blkBc[chunkStart[B] + i] : blkBc[chunkStart[A] + i0 + n0 + i]) * 8;
+    };
+    auto out_row = [&](int X, int j) {
+        const int r = chunkBr[X] * 8 + j;
+        return r < rows ? r : -1;
+    };
+    if (l < mx::kTileHdr) {
+        int v = 0;
+        if (l < 8) v = out_row(A, l);
+        else if (l < 16) v = B >= 0 ? out_row(B, l - 8) : -1;
+        else if (l == 16) v = d[2];
+        else if (l == 17) v = n0;
+        else if (l == 18) v = n1;
+        else if (l == 19) v = d[6];
+        else if (l == 20) v = d[7];
+        else if (l < 29) v = first_col(l - 21);
+        hdr[(size_t)s * mx::kTileHdr + l] = v;
+    }
+    const int c0 = first_col(l >> 3);
+    atox[(size_t)s * 64 + l] = c0 >= 0 ? c0 + (l & 7) : -1;
+}
+__global__ __launch_bounds__(kBlock) void block_values_kernel(const int *__restrict__ entryBlock, const int *__restrict__ chunkIdIncl,
+                                                              const int *__restrict__ chunkStart, const int *__restrict__ chunkBlock0,
+                                                              const int *__restrict__ ddRowPtr, const int *__restrict__ ddCol,
+                                                              const double *__restrict__ ddVal, const int *__restrict__ descColId,
+                                                              const int *__restrict__ rId, int dRows, int nDD, double *__restrict__ tcVal)
+{
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= nDD) return;
+    const int g = entryBlock[p];
+    if (g < 0) return;
+    int lo = 0, hi = dRows - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (ddRowPtr[mid] <= p) lo = mid;
+        else hi = mid - 1;
+    }
+    const int chunk = chunkIdIncl[g] - 1, r = rId[lo], c = descColId[ddCol[p]];
+    tcVal[((size_t)chunkBlock0[chunk] + (g - chunkStart[chunk])) * 64 + (r & 7) * 8 + (c & 7)] = ddVal[p];
+}
+// the CSR part beside blocks: an entry stays unless a block took it
+__global__ __launch_bounds__(kBlock) void block_keep_kernel(const int *__restrict__ entryBlock, int nDD, int *__restrict__ keep)
+{
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p <= nDD) keep[p] = p < nDD && entryBlock[p] < 0 ? 1 : 0;
+}
+__global__ __launch_bounds__(kBlock) void part_lengths_scan_kernel(const int *__restrict__ cdRowPtr, const int *__restrict__ ddRowPtr,
+                                                                   const int *__restrict__ ddRowOf, const int *__restrict__ keptBefore,
+                                                                   int rows, int *__restrict__ len)
+{
+    const int r = blockIdx.x * kBlock + threadIdx.x;
+    if (r > rows) return;
+    if (r == rows) {
+        len[r] = 0;
+        return;
+    }
+    const int i = ddRowOf[r];
+    len[r] = cdRowPtr[r + 1] - cdRowPtr[r] + (i >= 0 ? keptBefore[ddRowPtr[i + 1]] - keptBefore[ddRowPtr[i]] : 0);
+}
+template <typename V>
+__global__ __launch_bounds__(kBlock) void part_dense_scan_kernel(const int *__restrict__ ddRowPtr, const int *__restrict__ ddCol,
+                                                                 const V *__restrict__ ddVal, const int *__restrict__ descColId,
+                                                                 const int *__restrict__ rId, const int *__restrict__ entryBlock,
+                                                                 const int *__restrict__ keptBefore, const int *__restrict__ cdRowPtr,
+                                                                 const int *__restrict__ outPtr, int dRows, int nDD, int *__restrict__ col,
+                                                                 V *__restrict__ val)
+{
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= nDD || entryBlock[p] >= 0) return;
+    int lo = 0, hi = dRows - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (ddRowPtr[mid] <= p) lo = mid;
+        else hi = mid - 1;
+    }
+    const int r = rId[lo];
+    const int q = outPtr[r] + (cdRowPtr[r + 1] - cdRowPtr[r]) + (keptBefore[p] - keptBefore[ddRowPtr[lo]]);
+    col[q] = descColId[ddCol[p]];
+    val[q] = ddVal[p];
+}
+
 }  // namespace mxh
 
 #define MXH_TRY(call)                                                                                 \
@@ -637,6 +791,9 @@ struct HybridDevice::Impl {
     // the general tile form (tile_chunks)
     int minVals = 1, nSel = 0;
     Buf selFrag, usedCols, nrefs, refStart, sortedCol, where, selPos, selW, tileBlock0;
+    // the binary64 block form (analyse keeps the sorted keys; block_chunks, block_layout)
+    int nBlk = 0, nBlkChunks = 0;
+    Buf blkKey, blkPay, blkBr, blkBc, entryBlock, blkChunkIdIncl, blkChunkStart, blkChunkBr;
     void *tileVal = nullptr;  // the values of the general tile layout (owned by the caller's DeviceTiles): csr_part fills them
     ~Impl() { mx_tiles_device_free(&T); }
 };
@@ -830,20 +987,26 @@ int HybridDevice::analyse(mx_dtype dtype, int rows, int cols, int nnz, const int
             }
         }
     }
-    // ---- binary64: aligned 8 x 8 blocks at least three quarters full (counted only)
+    // ---- binary64: aligned 8 x 8 blocks at least three quarters full (counted here; block_chunks lays them out)
     if (wantBlocks && dtype == MX_F64 && I.dRows > 0 && I.nDD > 0) {
-        Buf keyIn, keyOut, sortTmp;
+        Buf keyIn, payIn, sortTmp;
         const size_t n = (size_t)I.nDD;
         size_t sortBytes = 0;
-        MXH_TRY(rocprim::radix_sort_keys(nullptr, sortBytes, (const unsigned long long *)nullptr, (unsigned long long *)nullptr, n, 0u, 64u, s));
+        MXH_TRY(rocprim::radix_sort_pairs(nullptr, sortBytes, (const unsigned long long *)nullptr, (unsigned long long *)nullptr,
+                                          (const int *)nullptr, (int *)nullptr, n, 0u, 64u, s));
         MXH_TRY(hipMalloc(&keyIn.p, n * 8));
-        MXH_TRY(hipMalloc(&keyOut.p, n * 8));
+        MXH_TRY(hipMalloc(&payIn.p, n * 4));
+        MXH_TRY(hipMalloc(&I.blkKey.p, n * 8));
+        MXH_TRY(hipMalloc(&I.blkPay.p, n * 4));
         MXH_TRY(hipMalloc(&sortTmp.p, sortBytes + 256));
         hipLaunchKernelGGL(block_keys_kernel, grid(I.nDD), dim3(kBlock), 0, s, (const int *)I.ddp, (const int *)I.ddc, (const int *)I.dc,
                            (const int *)I.dr, I.dRows, I.nDD, keyIn.as<unsigned long long>());
         MXH_TRY(hipGetLastError());
-        MXH_TRY(rocprim::radix_sort_keys(sortTmp.p, sortBytes, (const unsigned long long *)keyIn.p, keyOut.as<unsigned long long>(), n, 0u, 64u, s));
-        hipLaunchKernelGGL(block_runs_kernel, grid(I.nDD), dim3(kBlock), 0, s, (const unsigned long long *)keyOut.p, I.nDD, 48, cols, tot + 2);
+        hipLaunchKernelGGL(iota_kernel, grid(I.nDD), dim3(kBlock), 0, s, payIn.as<int>(), I.nDD);
+        MXH_TRY(hipGetLastError());
+        MXH_TRY(rocprim::radix_sort_pairs(sortTmp.p, sortBytes, (const unsigned long long *)keyIn.p, I.blkKey.as<unsigned long long>(),
+                                          (const int *)payIn.p, I.blkPay.as<int>(), n, 0u, 64u, s));
+        hipLaunchKernelGGL(block_runs_kernel, grid(I.nDD), dim3(kBlock), 0, s, (const unsigned long long *)I.blkKey.p, I.nDD, 48, cols, tot + 2);
         MXH_TRY(hipGetLastError());
     }
     // ---- the fill gate of the reference's fragments
@@ -875,8 +1038,8 @@ int HybridDevice::analyse(mx_dtype dtype, int rows, int cols, int nnz, const int
 }
 
 template <typename V>
-static int csr_part_t(HybridDevice::Impl &I, bool keepStrips, bool keepGeneral, int **rowPtrOut, int **colOut, void **valOut, int *nnzOut,
-                      char **stripRowsOut)
+static int csr_part_t(HybridDevice::Impl &I, bool keepStrips, bool keepGeneral, bool keepBlocks, int **rowPtrOut, int **colOut, void **valOut,
+                      int *nnzOut, char **stripRowsOut)
 {
     using namespace mxh;
     hipStream_t s = I.s;
@@ -887,14 +1050,35 @@ static int csr_part_t(HybridDevice::Impl &I, bool keepStrips, bool keepGeneral, 
         mx::set_error("hybrid plan on the device: the tile layout has to be made before the CSR part");
         return MX_ERR_ARG;
     }
-    Buf len, ptr, tmp, col, val, marks, kept;
+    const bool blocks = keepBlocks && I.nBlkChunks > 0;
+    if (blocks && (general || taken)) {
+        mx::set_error("hybrid plan on the device: blocks do not go with strips or general tiles");
+        return MX_ERR_ARG;
+    }
+    Buf len, ptr, tmp, col, val, marks, kept, keptBefore;
     size_t scanBytes = 0;
-    MXH_TRY(rocprim::exclusive_scan(nullptr, scanBytes, (const int *)nullptr, (int *)nullptr, 0, (size_t)rows + 1, rocprim::plus<int>(), s));
+    MXH_TRY(rocprim::exclusive_scan(nullptr, scanBytes, (const int *)nullptr, (int *)nullptr, 0, (size_t)std::max(rows, blocks ? I.nDD : 0) + 1,
+                                    rocprim::plus<int>(), s));
     MXH_TRY(hipMalloc(&len.p, ((size_t)rows + 1) * 4));
     MXH_TRY(hipMalloc(&ptr.p, ((size_t)rows + 1) * 4));
     MXH_TRY(hipMalloc(&tmp.p, scanBytes + 256));
     if (taken) MXH_TRY(hipMalloc(&marks.p, (size_t)rows + 4));
-    if (general) {
+    if (blocks) {
+        Buf keep;
+        MXH_TRY(hipMalloc(&keep.p, ((size_t)I.nDD + 1) * 4));
+        MXH_TRY(hipMalloc(&keptBefore.p, ((size_t)I.nDD + 1) * 4));
+        MXH_TRY(hipMalloc(&marks.p, (size_t)rows + 4));
+        MXH_TRY(hipMemsetAsync(marks.p, 0, (size_t)rows + 4, s));
+        hipLaunchKernelGGL(block_keep_kernel, grid((long long)I.nDD + 1), dim3(kBlock), 0, s, (const int *)I.entryBlock.p, I.nDD, keep.as<int>());
+        MXH_TRY(hipGetLastError());
+        MXH_TRY(rocprim::exclusive_scan(tmp.p, scanBytes, (const int *)keep.p, keptBefore.as<int>(), 0, (size_t)I.nDD + 1, rocprim::plus<int>(), s));
+        hipLaunchKernelGGL(part_lengths_scan_kernel, grid((long long)rows + 1), dim3(kBlock), 0, s, (const int *)I.cdp, (const int *)I.ddp,
+                           (const int *)I.ddRowOf.p, (const int *)keptBefore.p, rows, len.as<int>());
+        MXH_TRY(hipGetLastError());
+        hipLaunchKernelGGL(block_marks_kernel, grid(I.nBlkChunks), dim3(kBlock), 0, s, (const int *)I.blkChunkBr.p, I.nBlkChunks, rows,
+                           marks.as<char>());
+        MXH_TRY(hipStreamSynchronize(s));  // (`keep` leaves scope)
+    } else if (general) {
         MXH_TRY(hipMalloc(&kept.p, (size_t)I.dRows * 4 + 4));
         hipLaunchKernelGGL((dd_rows_kernel<V, true>), grid(I.dRows), dim3(kBlock), 0, s, (const int *)I.ddp, (const int *)I.ddc,
                            (const V *)I.ddv, (const int *)I.dc, (const int *)I.dr, taken, (const int *)I.T.chunkPtr,
@@ -920,7 +1104,12 @@ static int csr_part_t(HybridDevice::Impl &I, bool keepStrips, bool keepGeneral, 
                            (const int *)I.colOrig.p, (const int *)ptr.p, rows, I.nCD, col.as<int>(), val.as<V>());
         MXH_TRY(hipGetLastError());
     }
-    if (general) {
+    if (blocks) {
+        hipLaunchKernelGGL(part_dense_scan_kernel<V>, grid(I.nDD), dim3(kBlock), 0, s, (const int *)I.ddp, (const int *)I.ddc, (const V *)I.ddv,
+                           (const int *)I.dc, (const int *)I.dr, (const int *)I.entryBlock.p, (const int *)keptBefore.p, (const int *)I.cdp,
+                           (const int *)ptr.p, I.dRows, I.nDD, col.as<int>(), val.as<V>());
+        MXH_TRY(hipGetLastError());
+    } else if (general) {
         hipLaunchKernelGGL((dd_rows_kernel<V, false>), grid(I.dRows), dim3(kBlock), 0, s, (const int *)I.ddp, (const int *)I.ddc,
                            (const V *)I.ddv, (const int *)I.dc, (const int *)I.dr, taken, (const int *)I.T.chunkPtr,
                            (const int *)I.T.sparse_AToX_index, (const int *)I.usedCols.p, (const unsigned char *)I.selFrag.p, I.dRows, K,
@@ -942,11 +1131,112 @@ static int csr_part_t(HybridDevice::Impl &I, bool keepStrips, bool keepGeneral, 
     return MX_OK;
 }
 
-int HybridDevice::csr_part(bool keepStrips, bool keepGeneral, int **rowPtr_dev, int **col_dev, void **val_dev, int *nnz, char **stripRows_dev)
+int HybridDevice::csr_part(bool keepStrips, bool keepGeneral, bool keepBlocks, int **rowPtr_dev, int **col_dev, void **val_dev, int *nnz,
+                           char **stripRows_dev)
 {
     if (!impl) return MX_ERR_ARG;
-    if (impl->dtype == MX_F64) return csr_part_t<double>(*impl, keepStrips, keepGeneral, rowPtr_dev, col_dev, val_dev, nnz, stripRows_dev);
-    return csr_part_t<unsigned short>(*impl, keepStrips, keepGeneral, rowPtr_dev, col_dev, val_dev, nnz, stripRows_dev);
+    if (impl->dtype == MX_F64)
+        return csr_part_t<double>(*impl, keepStrips, keepGeneral, keepBlocks, rowPtr_dev, col_dev, val_dev, nnz, stripRows_dev);
+    return csr_part_t<unsigned short>(*impl, keepStrips, keepGeneral, keepBlocks, rowPtr_dev, col_dev, val_dev, nnz, stripRows_dev);
+}
+
+// The chunks of the binary64 block form: per block row with at least one block, in ascending order, how
+// many blocks it has (`blocks`) and which block row it is (`blockRows`).
+int HybridDevice::block_chunks(std::vector<int> &blocks, std::vector<int> &blockRows)
+{
+    using namespace mxh;
+    blocks.clear();
+    blockRows.clear();
+    if (!impl || impl->dtype != MX_F64) return MX_ERR_ARG;
+    Impl &I = *impl;
+    hipStream_t s = I.s;
+    I.nBlk = I.nBlkChunks = 0;
+    if (!I.blkKey.p || I.nDD <= 0) return MX_OK;
+    const size_t n = (size_t)I.nDD;
+    Buf selHead, blockId, tmp, head, nb;
+    size_t scanBytes = 0, b2 = 0;
+    MXH_TRY(rocprim::exclusive_scan(nullptr, scanBytes, (const int *)nullptr, (int *)nullptr, 0, n + 1, rocprim::plus<int>(), s));
+    MXH_TRY(rocprim::inclusive_scan(nullptr, b2, (const int *)nullptr, (int *)nullptr, n + 1, rocprim::plus<int>(), s));
+    scanBytes = std::max(scanBytes, b2);
+    MXH_TRY(hipMalloc(&selHead.p, (n + 1) * 4));
+    MXH_TRY(hipMalloc(&blockId.p, (n + 1) * 4));
+    MXH_TRY(hipMalloc(&tmp.p, scanBytes + 256));
+    MXH_TRY(hipMalloc(&I.entryBlock.p, n * 4 + 4));
+    MXH_TRY(hipMemsetAsync(I.entryBlock.p, 0xff, n * 4 + 4, s));
+    hipLaunchKernelGGL(block_heads_kernel, grid((long long)n + 1), dim3(kBlock), 0, s, (const unsigned long long *)I.blkKey.p, I.nDD, 48, I.cols,
+                       selHead.as<int>());
+    MXH_TRY(hipGetLastError());
+    MXH_TRY(rocprim::exclusive_scan(tmp.p, scanBytes, (const int *)selHead.p, blockId.as<int>(), 0, n + 1, rocprim::plus<int>(), s));
+    int nBlk = 0;
+    MXH_TRY(hipMemcpyAsync(&nBlk, blockId.as<int>() + n, 4, hipMemcpyDeviceToHost, s));
+    MXH_TRY(hipStreamSynchronize(s));
+    if (nBlk <= 0) return MX_OK;
+    const size_t nbk = (size_t)nBlk;
+    MXH_TRY(hipMalloc(&I.blkBr.p, nbk * 4 + 4));
+    MXH_TRY(hipMalloc(&I.blkBc.p, nbk * 4 + 4));
+    MXH_TRY(hipMalloc(&head.p, nbk * 4 + 4));
+    MXH_TRY(hipMalloc(&I.blkChunkIdIncl.p, nbk * 4 + 4));
+    hipLaunchKernelGGL(block_records_kernel, grid(I.nDD), dim3(kBlock), 0, s, (const unsigned long long *)I.blkKey.p, (const int *)I.blkPay.p,
+                       (const int *)selHead.p, (const int *)blockId.p, I.nDD, I.blkBr.as<int>(), I.blkBc.as<int>(), I.entryBlock.as<int>());
+    MXH_TRY(hipGetLastError());
+    hipLaunchKernelGGL(block_chunk_heads_kernel, grid(nBlk), dim3(kBlock), 0, s, (const int *)I.blkBr.p, nBlk, head.as<int>());
+    MXH_TRY(hipGetLastError());
+    // (nBlk <= nDD: the scan's temporary storage is large enough)
+    MXH_TRY(rocprim::inclusive_scan(tmp.p, scanBytes, (const int *)head.p, I.blkChunkIdIncl.as<int>(), nbk, rocprim::plus<int>(), s));
+    int nChunks = 0;
+    MXH_TRY(hipMemcpyAsync(&nChunks, I.blkChunkIdIncl.as<int>() + (nbk - 1), 4, hipMemcpyDeviceToHost, s));
+    MXH_TRY(hipStreamSynchronize(s));
+    MXH_TRY(hipMalloc(&I.blkChunkStart.p, ((size_t)nChunks + 1) * 4));
+    MXH_TRY(hipMalloc(&I.blkChunkBr.p, ((size_t)nChunks + 1) * 4));
+    MXH_TRY(hipMalloc(&nb.p, ((size_t)nChunks + 1) * 4));
+    hipLaunchKernelGGL(block_chunk_starts_kernel, grid(nBlk), dim3(kBlock), 0, s, (const int *)head.p, (const int *)I.blkChunkIdIncl.p,
+                       (const int *)I.blkBr.p, nBlk, I.blkChunkStart.as<int>(), I.blkChunkBr.as<int>());
+    MXH_TRY(hipGetLastError());
+    hipLaunchKernelGGL(block_chunk_sizes_kernel, grid(nChunks), dim3(kBlock), 0, s, (const int *)I.blkChunkStart.p, nChunks, nb.as<int>());
+    MXH_TRY(hipGetLastError());
+    blocks.assign((size_t)nChunks, 0);
+    blockRows.assign((size_t)nChunks, 0);
+    MXH_TRY(hipMemcpyAsync(blocks.data(), nb.p, (size_t)nChunks * 4, hipMemcpyDeviceToHost, s));
+    MXH_TRY(hipMemcpyAsync(blockRows.data(), I.blkChunkBr.p, (size_t)nChunks * 4, hipMemcpyDeviceToHost, s));
+    MXH_TRY(hipStreamSynchronize(s));
+    I.nBlk = nBlk;
+    I.nBlkChunks = nChunks;
+    return MX_OK;
+}
+
+int HybridDevice::block_layout(const std::vector<int> &stepDesc, const std::vector<int> &chunkBlock0, const std::vector<int> &waveDesc,
+                               long long totalBlocks, DeviceTiles &T)
+{
+    using namespace mxh;
+    if (!impl || impl->nBlkChunks <= 0 || (int)chunkBlock0.size() != impl->nBlkChunks) return MX_ERR_ARG;
+    Impl &I = *impl;
+    hipStream_t s = I.s;
+    const int steps = (int)(stepDesc.size() / 10);
+    Buf dDesc, dBlock0;
+    MXH_TRY(hipMalloc(&dDesc.p, stepDesc.size() * 4 + 4));
+    MXH_TRY(hipMalloc(&dBlock0.p, chunkBlock0.size() * 4 + 4));
+    MXH_TRY(hipMemcpyAsync(dDesc.p, stepDesc.data(), stepDesc.size() * 4, hipMemcpyHostToDevice, s));
+    MXH_TRY(hipMemcpyAsync(dBlock0.p, chunkBlock0.data(), chunkBlock0.size() * 4, hipMemcpyHostToDevice, s));
+    const size_t nWave = waveDesc.size() + 64, nHdr = (size_t)steps * kTileHdr + 256, nAtox = (size_t)steps * 64 + 256,
+                 valBytes = (size_t)totalBlocks * 64 * 8 + 8192;
+    MXH_TRY(hipMalloc((void **)&T.waveDesc, nWave * 4));
+    MXH_TRY(hipMemsetAsync(T.waveDesc, 0, nWave * 4, s));
+    MXH_TRY(hipMemcpyAsync(T.waveDesc, waveDesc.data(), waveDesc.size() * 4, hipMemcpyHostToDevice, s));
+    MXH_TRY(hipMalloc((void **)&T.hdr, nHdr * 4));
+    MXH_TRY(hipMemsetAsync(T.hdr, 0, nHdr * 4, s));
+    MXH_TRY(hipMalloc((void **)&T.atox, nAtox * 4));
+    MXH_TRY(hipMemsetAsync(T.atox, 0, nAtox * 4, s));
+    MXH_TRY(hipMalloc(&T.tcVal, valBytes));
+    MXH_TRY(hipMemsetAsync(T.tcVal, 0, valBytes, s));
+    hipLaunchKernelGGL(block_steps_kernel, dim3(steps), dim3(64), 0, s, (const int *)dDesc.p, (const int *)I.blkChunkStart.p,
+                       (const int *)I.blkChunkBr.p, (const int *)I.blkBc.p, I.rows, steps, T.hdr, T.atox);
+    MXH_TRY(hipGetLastError());
+    hipLaunchKernelGGL(block_values_kernel, grid(I.nDD), dim3(kBlock), 0, s, (const int *)I.entryBlock.p, (const int *)I.blkChunkIdIncl.p,
+                       (const int *)I.blkChunkStart.p, (const int *)dBlock0.p, (const int *)I.ddp, (const int *)I.ddc, (const double *)I.ddv,
+                       (const int *)I.dc, (const int *)I.dr, I.dRows, I.nDD, (double *)T.tcVal);
+    MXH_TRY(hipGetLastError());
+    MXH_TRY(hipStreamSynchronize(s));
+    return MX_OK;
 }
 
 // The chunks of the general tile form: the fragments that pass the gate on what the strips leave,

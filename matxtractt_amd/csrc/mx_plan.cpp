@@ -1190,7 +1190,7 @@ struct mx_plan {
     // binary32, one per row, which the tile kernel adds to (y is then rounded once)
     void *ywide = nullptr;
     int ext_dCols = 0, ext_dRows = 0, ext_nnzRowD = 0, ext_frags = 0;  // what the extraction behind the plan selected
-    int prep_route = 0;  // 0 = laid out on the host, 1 = on the device, 2 = mx_plan_create_device sent the matrix to the host route
+    int prep_route = 0;  // 0 = laid out on the host from host arrays, 1 = on the device from device arrays
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 };
@@ -2098,7 +2098,7 @@ static int create_plan(const mx_partition *P, int flags, mx_plan **out, bool noB
 // matrix crosses to the host but its row pointers (for the row-tile form) or the lengths of its
 // chunks (for the slice form).  `elsewhere_dev` (optional): marks of rows that another kernel writes.
 static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, const int *colInd_dev, const void *val_dev, int flags,
-                                 const char *elsewhere_dev)
+                                 const char *elsewhere_dev, std::pair<std::vector<int>, std::vector<int>> *segOut = nullptr)
 {
     const mx_dtype dtype = plan->dtype;
     const int rows = plan->rows, cols = plan->cols;
@@ -2117,7 +2117,8 @@ static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, 
     if (env && !std::strcmp(env, "rows")) want[0] = true, want[1] = false;
     if (env && !std::strcmp(env, "slices") && S > 0) want[1] = true, want[0] = false;
     if (want[1]) {
-        rc = mx::build_slices_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, nCU, S, elsewhere_dev, plan->slices, nullptr);
+        rc = mx::build_slices_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, nCU, S, elsewhere_dev, plan->slices, nullptr,
+                                     segOut ? &segOut->first : nullptr, segOut ? &segOut->second : nullptr);
         if (rc) return rc;
         if (plan->slices.ecode) plan->slices.useDict = true;
     }
@@ -2288,11 +2289,19 @@ static int plan_tile_steps(const std::vector<int> &chunkBlocks, int SF, int BS, 
 // extraction, the plan's decisions, the CSR part with its layout and the strips' layout are all
 // made on the device (mx_hybrid.hip, mx_layout.hip); what a decision needs comes to the host as
 // counts.  The plan equals the one mx_plan_create makes from mx_partition_create(_device) of the
-// same matrix.  One tile form is not laid out on the device, the binary64 blocks; a matrix on which
-// the plan keeps them (none of the measured workloads with default flags) is copied to the host and
-// takes the host route.
+// same matrix, whatever tile forms it keeps.
+static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev, const void *val_dev,
+                              float tau_c, float tau_r, int flags, mx_plan **out, bool noBlocks);
 extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
                                      const void *val_dev, float tau_c, float tau_r, int flags, mx_plan **out)
+{
+    return create_plan_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, tau_c, tau_r, flags, out, false);
+}
+
+// `noBlocks`: a binary64 plan without the 8 x 8 block form (the second attempt, when a row of a block
+// chunk turned out to have more virtual rows than the block layout has places for).
+static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev, const void *val_dev,
+                              float tau_c, float tau_r, int flags, mx_plan **out, bool noBlocks)
 {
     static const char who[] = "mx_plan_create_device";
     if (!out || (dtype != MX_F64 && dtype != MX_F16) || rows < 1 || cols < 1 || nnz < 0 || !rowPtr_dev ||
@@ -2306,32 +2315,6 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
     int rc = need_device();
     if (rc) return rc;
     if ((rc = mx::check_csr_device(rows, cols, nnz, rowPtr_dev, colInd_dev, nullptr, who))) return rc;
-    const size_t es = (size_t)mx::elem_size(dtype);
-    // the host route for this matrix: it comes down once and goes through mx_partition_create_device
-    auto host_route = [&]() -> int {
-        std::vector<int> rp((size_t)rows + 1), ci((size_t)nnz);
-        std::vector<unsigned char> va((size_t)nnz * es);
-        MX_HIP(hipMemcpy(rp.data(), rowPtr_dev, rp.size() * 4, hipMemcpyDeviceToHost));
-        if (nnz > 0) {
-            MX_HIP(hipMemcpy(ci.data(), colInd_dev, ci.size() * 4, hipMemcpyDeviceToHost));
-            MX_HIP(hipMemcpy(va.data(), val_dev, va.size(), hipMemcpyDeviceToHost));
-        }
-        mx_csr A{};
-        A.dtype = dtype;
-        A.rows = rows;
-        A.cols = cols;
-        A.nnz = nnz;
-        A.rowPtr = rp.data();
-        A.colInd = ci.data();
-        A.val = va.data();
-        mx_partition *P = nullptr;
-        int e = mx_partition_create_device(&A, tau_c, tau_r, &P);
-        if (e) return e;
-        e = mx_plan_create(P, flags, out);
-        mx_partition_destroy(P);
-        if (!e) (*out)->prep_route = 2;
-        return e;
-    };
     try {
         hipDeviceProp_t prop;
         int dev = 0;
@@ -2342,7 +2325,7 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
         const bool noTiles = (flags & MX_PLAN_NO_TILES) != 0, allTiles = !noTiles && (flags & MX_PLAN_ALL_TILES) != 0;
         const char *envNoStrips = std::getenv("MX_NO_STRIPS"), *envNoBlocks = std::getenv("MX_NO_BLOCKS");
         const bool wantStrips = dtype == MX_F16 && !noTiles && !allTiles && !(envNoStrips && std::atoi(envNoStrips));
-        const bool wantBlocks = dtype == MX_F64 && !noTiles && !allTiles && !(envNoBlocks && std::atoi(envNoBlocks));
+        const bool wantBlocks = dtype == MX_F64 && !noTiles && !allTiles && !noBlocks && !(envNoBlocks && std::atoi(envNoBlocks));
         // (the smallest count that passes `(double)vals >= gate * fragM * fragK`; every fragment that holds anything
         // with MX_PLAN_ALL_TILES)
         const double need = tile_gate(dtype) * fragM * fragK;
@@ -2362,7 +2345,7 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
         else if (!(flags & (MX_PLAN_KEEP_TILES | MX_PLAN_ALL_TILES)))
             worth = tiles_worth(dtype, fragM, fragK, cnt.blocks64, (double)cnt.generalEntries, (double)cnt.generalFrags,
                                 (double)cnt.stripEntries, (double)cnt.stripBlocks);
-        if (worth >= 1 && cnt.blocks64 && cnt.stripBlocks > 0) return host_route();  // binary64 blocks: laid out on the host
+        const bool keepBlocks = worth >= 1 && cnt.blocks64 && cnt.stripBlocks > 0;
         const bool keepStrips = worth >= 1 && !cnt.blocks64 && cnt.stripBlocks > 0;
         const bool keepGeneral = worth == 2 && cnt.generalFrags > 0;
 
@@ -2426,11 +2409,58 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
                 phase("tile steps (device)");
             }
         }
+        std::vector<int> blockStepDesc, blockRows;  // binary64 blocks: their steps and the block row of every chunk
+        if (keepBlocks) {
+            std::vector<int> chunkBlocks, chunkBlock0, waveDesc;
+            long long totalBlocks = 0;
+            if ((rc = H.block_chunks(chunkBlocks, blockRows))) return fail(rc);
+            if ((rc = plan_tile_steps(chunkBlocks, 8, 64, 1, nCU, 10, blockStepDesc, chunkBlock0, waveDesc, &totalBlocks))) return fail(rc);
+            mx::DeviceTiles &T = plan->strips;
+            T.chunkNum = (int)chunkBlocks.size();
+            T.frags = (int)cnt.stripBlocks;
+            T.vals = (int)cnt.stripEntries;
+            T.stored = totalBlocks * 64;
+            T.steps = (int)(blockStepDesc.size() / 10);
+            T.dense = T.steps > 0;
+            T.nWaves = (int)(waveDesc.size() / 8);
+            if ((rc = H.block_layout(blockStepDesc, chunkBlock0, waveDesc, totalBlocks, T))) return fail(rc);
+            plan->tile_nnz += T.vals;
+            phase("block steps (device)");
+        }
         int partNnz = 0;
-        if ((rc = H.csr_part(keepStrips, keepGeneral, &partPtr, &partCol, &partVal, &partNnz, &stripRows))) return fail(rc);
+        if ((rc = H.csr_part(keepStrips, keepGeneral, keepBlocks, &partPtr, &partCol, &partVal, &partNnz, &stripRows))) return fail(rc);
         phase("CSR part assembled (device)");
-        if ((rc = setup_csr_part_device(plan, partNnz, partPtr, partCol, partVal, flags, stripRows))) return fail(rc);
+        std::pair<std::vector<int>, std::vector<int>> seg;  // virtual rows of every row (slice form), for the blocks
+        if ((rc = setup_csr_part_device(plan, partNnz, partPtr, partCol, partVal, flags, stripRows, keepBlocks ? &seg : nullptr)))
+            return fail(rc);
         phase("CSR part layout (device)");
+        if (keepBlocks && plan->csr_variant == 1) {
+            // the blocks ride in the combine kernel's launch: where each of their rows finds the sums of its
+            // virtual rows (eight places per row; a row with more sends the whole plan back to be made without blocks)
+            const int steps = plan->strips.steps;
+            std::vector<int> vidx((size_t)steps * 128, -1);
+            bool fits = true;
+            for (int st = 0; st < steps && fits; ++st) {
+                const int *d = &blockStepDesc[(size_t)st * 10];
+                if (!(d[2] & 1)) continue;
+                for (int half = 0; half < 2; ++half) {
+                    const int chunk = half == 0 ? d[0] : d[1];
+                    if (chunk < 0) continue;
+                    for (int i = 0; i < 8; ++i) {
+                        const int r = blockRows[chunk] * 8 + i;
+                        if (r >= rows) continue;
+                        const int a = seg.first[r], n = seg.first[r + 1] - a;
+                        if (n > 8) fits = false;
+                        for (int j = 0; j < std::min(n, 8); ++j) vidx[(size_t)st * 128 + half * 64 + i * 8 + j] = seg.second[a + j];
+                    }
+                }
+            }
+            if (!fits) {
+                fail(MX_OK);
+                return create_plan_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, tau_c, tau_r, flags, out, true);
+            }
+            if ((rc = upload(&plan->strips.vidx, vidx.data(), vidx.size(), 128))) return fail(rc);
+        }
         if (keepStrips) {
             std::vector<int> stepDesc, chunkBlock0, waveDesc;
             long long totalBlocks = 0;

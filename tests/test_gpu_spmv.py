@@ -563,6 +563,7 @@ def test_binary64_block_form(mx, ora, monkeypatch):
     x = rng.integers(-2, 3, cols).astype(np.float64)
     ref = ora.spmv_f64(A.val, A.rowPtr, A.colInd, x)
     xd = torch.from_numpy(x).cuda()
+    drp, dci, dva = torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda()
     seen = set()
     for tau in ((1.0, 1.0), (0.75, 0.5), (0.5, 0.25)):
         part = mx.Partition(A, *tau)
@@ -578,6 +579,17 @@ def test_binary64_block_form(mx, ora, monkeypatch):
                 seen.add((plan.info["tile_variant"], plan.info["csr_variant"]))
                 if tau == (1.0, 1.0):
                     assert plan.info["tile_variant"] == 2 and plan.info["tile_strip_nnz"] > 0.5 * A.nnz
+            # the same plan made on the device from the matrix in device memory: every array, and y
+            dplan = mx.Plan.from_device(drp, dci, dva, A.cols, tau[0], tau[1], flags)
+            assert dplan.info["prep_route"] == 1
+            for k in ("csr_variant", "csr_nnz", "tile_nnz", "tile_chunks", "tile_frags", "tile_variant", "tile_strip_nnz"):
+                assert dplan.info[k] == plan.info[k], (tau, flags, k, dplan.info[k], plan.info[k])
+            ah, ad = plan.arrays(), dplan.arrays()
+            assert sorted(ah) == sorted(ad), (tau, flags, sorted(ah), sorted(ad))
+            for k in ah:
+                assert ah[k] == ad[k], (tau, flags, k)
+            assert np.array_equal(dplan.spmv(xd).cpu().numpy(), ref), (tau, flags)
+            dplan.close()
             plan.close()
         part.close()
     assert (2, 1) in seen and (2, 0) in seen, seen
@@ -907,7 +919,7 @@ def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
     assert ratios[0] == ratios[1], ratios
     for k in ("dCols", "dRows", "tile_chunks", "tile_nnz", "csr_nnz", "tc_nnz_ratio"):
         assert recs[0][k] == recs[1][k], (k, recs[0][k], recs[1][k])
-    assert recs[0]["prep_route"] == 0 and recs[1]["prep_route"] in (1, 2)
+    assert recs[0]["prep_route"] == 0 and recs[1]["prep_route"] == 1
     # --partition-cache: written by the first run, read by the second, recomputed when the fractions change
     cache = str(tmp_path / "m_preprocessed.dat")
     seen = []
@@ -1308,7 +1320,7 @@ def test_hybrid_plan_made_on_the_device(mx, ora):
     """mx_plan_create_device: extraction, decisions and layouts made on the device from a matrix
     in device memory give the plan mx_plan_create makes from mx_partition_create of the same
     matrix -- every counted fact, every array of the layouts byte for byte, y bit for bit --
-    whether the plan keeps strips, nothing, or a form that sends the matrix to the host route."""
+    whether the plan keeps strips, general tiles, binary64 blocks or nothing."""
     import torch
     rng = np.random.default_rng(12)
     cases = []
@@ -1318,7 +1330,7 @@ def test_hybrid_plan_made_on_the_device(mx, ora):
         cases += [("config %d x %g" % (cfg, sc), A, t) for t in taus]
     S = _strip_matrix(mx, rng, 60000, 70000)
     cases += [("strips of many shapes", S, (1.0, 1.0)), ("strips of many shapes", S, (0.75, 0.5))]
-    routes, strip_plans, general_plans = set(), 0, set()
+    routes, strip_plans, general_plans, block_plans = set(), 0, set(), 0
     for name, A, (tc, tr) in cases:
         x = rng.integers(-2, 3, A.cols).astype(A.val.dtype)
         xd = torch.from_numpy(x).cuda()
@@ -1345,6 +1357,8 @@ def test_hybrid_plan_made_on_the_device(mx, ora):
                     raise AssertionError("%s tau=(%g, %g) flags=%d: %s differs from byte %d of %d" % (name, tc, tr, flags, k, at, a.size))
             if D.info["prep_route"] == 1 and D.info["tile_strip_nnz"] > 0:
                 strip_plans += 1
+            if D.info["prep_route"] == 1 and D.info["tile_variant"] == 2:
+                block_plans += 1
             if D.info["prep_route"] == 1 and D.info["tile_nnz"] > D.info["tile_strip_nnz"]:
                 general_plans.add((A.dtype, D.info["tile_strip_nnz"] > 0))
             yh, yd = H.spmv(xd).cpu().numpy(), D.spmv(xd).cpu().numpy()
@@ -1353,7 +1367,8 @@ def test_hybrid_plan_made_on_the_device(mx, ora):
             H.close()
             D.close()
         part.close()
-    assert routes == {1, 2}, routes
+    assert routes == {1}, routes
+    assert block_plans >= 2, block_plans
     assert strip_plans >= 3, strip_plans
     # the general tile form laid out on the device: both precisions, with and without strips beside it
     assert {(mx.MX_F64, False), (mx.MX_F16, False), (mx.MX_F16, True)} <= general_plans, general_plans
@@ -1362,3 +1377,42 @@ def test_hybrid_plan_made_on_the_device(mx, ora):
     with pytest.raises(mx.MxError) as e:
         mx.Plan.from_device(rp, bad, va, A.cols, 1.0, 1.0)
     assert e.value.code == 1
+
+
+@pytest.mark.gpu
+def test_block_rows_with_many_virtual_rows_fall_back_to_a_plan_without_blocks(mx, ora):
+    """A row of a block chunk has eight places for the sums of its virtual rows.  A matrix in which
+    such a row reaches into more than eight slices gets its plan made again without the block form --
+    by the host route and by the device route alike, with the same arrays and an exact y."""
+    import torch
+    rng = np.random.default_rng(77)
+    rows, cols = 8 * 3000, 16384 * 12
+    rp, ci = [0], []
+    for r in range(rows):
+        br = r // 8
+        c = set(range(8 * (br % 2000), 8 * (br % 2000) + 8))               # a dense aligned block
+        c |= set(rng.choice(cols, 12, replace=False).tolist())
+        if br == 17:
+            c |= {16384 * q + 5 + r % 8 for q in range(12)}                # these rows reach into all twelve slices
+        ci += sorted(c)
+        rp.append(len(ci))
+    ci = np.array(ci, np.int32)
+    A = mx.Csr(rows, cols, np.array(rp, np.int32), ci, rng.integers(-3, 4, ci.size).astype(np.float64))
+    x = rng.integers(-2, 3, cols).astype(np.float64)
+    ref = ora.spmv_f64(A.val, A.rowPtr, A.colInd, x)
+    xd = torch.from_numpy(x).cuda()
+    drp, dci, dva = torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda()
+    part = mx.Partition(A, 1.0, 1.0)
+    for flags, blocks in ((mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_SLICES, False), (mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_ROWS, True)):
+        H = mx.Plan(part, flags)
+        D = mx.Plan.from_device(drp, dci, dva, A.cols, 1.0, 1.0, flags)
+        # (with the row-tile form the blocks add to y in a launch of their own and need no places)
+        assert (H.info["tile_variant"] == 2) == blocks and (D.info["tile_variant"] == 2) == blocks, (flags, H.info, D.info)
+        ah, ad = H.arrays(), D.arrays()
+        assert sorted(ah) == sorted(ad)
+        for k in ah:
+            assert ah[k] == ad[k], (flags, k)
+        assert np.array_equal(H.spmv(xd).cpu().numpy(), ref) and np.array_equal(D.spmv(xd).cpu().numpy(), ref)
+        H.close()
+        D.close()
+    part.close()
