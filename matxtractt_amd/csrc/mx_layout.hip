@@ -47,20 +47,22 @@ struct Buf {  // device memory released at scope exit unless taken
     }
 };
 
-// row[k] = the row of entry k; flag |= 1 when some row's columns are not ascending
-__global__ __launch_bounds__(kBlock) void entry_rows_kernel(const int *__restrict__ rowPtr, const int *__restrict__ col, int rows,
-                                                            int nnz, int *__restrict__ row, int *__restrict__ flag)
+// The row of every entry, in two steps: every row that has entries writes its number at the place of
+// its first entry (all other places hold 0), and a running maximum carries it to the rest of the row.
+__global__ __launch_bounds__(kBlock) void row_heads_kernel(const int *__restrict__ rowPtr, int rows, int *__restrict__ head)
+{
+    const int r = blockIdx.x * kBlock + threadIdx.x;
+    if (r < rows && rowPtr[r + 1] > rowPtr[r]) head[rowPtr[r]] = r;
+}
+// flag |= 1 when some row's columns are not ascending
+__global__ __launch_bounds__(kBlock) void row_order_kernel(const int *__restrict__ rowPtr, const int *__restrict__ col,
+                                                           const int *__restrict__ row, int nnz, int *__restrict__ flag)
 {
     const int k = blockIdx.x * kBlock + threadIdx.x;
-    if (k >= nnz) return;
-    int lo = 0, hi = rows - 1;
-    while (lo < hi) {  // last r with rowPtr[r] <= k
-        const int mid = (lo + hi + 1) >> 1;
-        if (rowPtr[mid] <= k) lo = mid;
-        else hi = mid - 1;
-    }
-    row[k] = lo;
-    if (k > rowPtr[lo] && col[k] < col[k - 1]) atomicOr(flag, 1);
+    const bool descends = k < nnz && k > rowPtr[row[k]] && col[k] < col[k - 1];
+    // (one atomic per wave at most, and none once the flag is up: a matrix whose rows are all out of order would
+    // put one per entry on the same word, and half a million of them take four milliseconds)
+    if (__any(descends) && (threadIdx.x & 63) == 0 && *(volatile int *)flag == 0) atomicOr(flag, 1);
 }
 
 __global__ __launch_bounds__(kBlock) void sort_keys_kernel(const int *__restrict__ row, const int *__restrict__ col, int nnz,
@@ -500,8 +502,20 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
     MXL_TRY(hipMalloc(&flag.p, 256));
     MXL_TRY(hipMemsetAsync(flag.p, 0, 256, s));
     int *over4 = flag.as<int>() + 1;
+    Buf tmp;
+    size_t scanBytes = 0, b2 = 0;
+    const size_t nScan = (size_t)std::max(nnz, rows + 1) + 1;
+    MXL_TRY(rocprim::inclusive_scan(nullptr, scanBytes, (const int *)nullptr, (int *)nullptr, nScan, MaxOp(), s));
+    MXL_TRY(rocprim::exclusive_scan(nullptr, b2, (const int *)nullptr, (int *)nullptr, 0, nScan, rocprim::plus<int>(), s));
+    scanBytes = std::max(scanBytes, b2);
+    MXL_TRY(hipMalloc(&tmp.p, scanBytes + 256));
     if (nnz > 0) {
-        hipLaunchKernelGGL(entry_rows_kernel, grid(nnz), dim3(kBlock), 0, s, rowPtr, col, rows, nnz, row.as<int>(), flag.as<int>());
+        // (`ord` is free until the order of the entries is known: it holds the row heads meanwhile)
+        MXL_TRY(hipMemsetAsync(ord.p, 0, (size_t)nnz * 4, s));
+        hipLaunchKernelGGL(row_heads_kernel, grid(rows), dim3(kBlock), 0, s, rowPtr, rows, ord.as<int>());
+        MXL_TRY(hipGetLastError());
+        MXL_TRY(rocprim::inclusive_scan(tmp.p, scanBytes, (const int *)ord.p, row.as<int>(), (size_t)nnz, MaxOp(), s));
+        hipLaunchKernelGGL(row_order_kernel, grid(nnz), dim3(kBlock), 0, s, rowPtr, col, (const int *)row.p, nnz, flag.as<int>());
         MXL_TRY(hipGetLastError());
     }
     int unsorted = 0;
@@ -530,13 +544,7 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
         MXL_TRY(hipGetLastError());
     }
     // ---- virtual rows
-    Buf runHead, runStart, start, vid, tmp;
-    size_t scanBytes = 0, b2 = 0;
-    const size_t nScan = (size_t)std::max(nnz, rows + 1) + 1;
-    MXL_TRY(rocprim::inclusive_scan(nullptr, scanBytes, (const int *)nullptr, (int *)nullptr, nScan, MaxOp(), s));
-    MXL_TRY(rocprim::exclusive_scan(nullptr, b2, (const int *)nullptr, (int *)nullptr, 0, nScan, rocprim::plus<int>(), s));
-    scanBytes = std::max(scanBytes, b2);
-    MXL_TRY(hipMalloc(&tmp.p, scanBytes + 256));
+    Buf runHead, runStart, start, vid;
     MXL_TRY(hipMalloc(&runHead.p, ((size_t)nnz + 1) * 4));
     MXL_TRY(hipMalloc(&runStart.p, ((size_t)nnz + 1) * 4));
     MXL_TRY(hipMalloc(&start.p, ((size_t)nnz + 1) * 4));
