@@ -40,7 +40,7 @@ WORKLOADS = {
     4: "configs[3]: FP16 power-law 1048576x1048576, Zipf(1.6) row lengths in [1,4096], mean ~10",
     5: "configs[4]: FP16 mixed 4194304x4194304, 20% of rows in dense 32-column strips + power-law rows",
 }
-SWEPT = (2, 5)  # the workloads BASELINE.json sweeps; 3 and 4 run CSR-only and at two hybrid points for the record
+SWEPT = (2, 5)  # the workloads whose 5 x 5 grid of extraction fractions is swept; 3 and 4 run CSR-only and at two hybrid points for the record
 
 
 def log(*a):
