@@ -951,7 +951,7 @@ def test_fp16_cli_passes_its_own_element_check(mx, tmp_path):
     base = [exe, "--warm", "2", "--iters", "5"]
     for cfg, scale in ((4, 1 / 16), (5, 1 / 32)):
         for tau in (("0", "0"), ("0.5", "0.25"), ("1", "1")):
-            for extra in ([], ["--keep-tiles"], ["--all-tiles"]):
+            for extra in ([], ["--keep-tiles"], ["--all-tiles"], ["--device-plan"], ["--device-plan", "--keep-tiles"]):
                 cmd = base + extra + [tau[0], tau[1], "--config", str(cfg), "--scale", repr(scale)]
                 print("fp16 cli:", " ".join(cmd[1:]), flush=True)
                 out = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
