@@ -30,9 +30,14 @@ constexpr int kBlock = 256;
 
 struct Buf {  // device memory released at scope exit unless taken
     void *p = nullptr;
-    ~Buf()
+    Buf() = default;
+    Buf(const Buf &) = delete;
+    Buf &operator=(const Buf &) = delete;
+    ~Buf() { release(); }
+    void release()
     {
         if (p) (void)hipFree(p);
+        p = nullptr;
     }
     template <typename T>
     T *as() const
@@ -564,7 +569,7 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
         MXL_TRY(hipStreamSynchronize(s));
         nV = lastVid + lastStart;
     }
-    runHead = Buf();  // (released)
+    runHead.release();
     D.vrows = nV;
     Buf vStart, vRow, vSlice, vLen, segPtr, key, keyOut, pay, sorted, sliceCount;
     const size_t nv1 = (size_t)nV + 1;
