@@ -1416,3 +1416,35 @@ def test_block_rows_with_many_virtual_rows_fall_back_to_a_plan_without_blocks(mx
         H.close()
         D.close()
     part.close()
+
+
+@pytest.mark.gpu
+def test_plans_release_their_device_memory(mx):
+    """Plans made and destroyed again and again -- by the host route and by the device route, with
+    strips, with general tiles, with blocks, CSR-only -- leave the device memory in use where it was
+    after the first round (temporaries of the layouts included)."""
+    import torch
+
+    def used():
+        torch.cuda.synchronize()
+        free, total = torch.cuda.mem_get_info()
+        return total - free
+
+    for cfg, sc, tau, flags in ((2, 0.5, (1.0, 1.0), mx.MX_PLAN_KEEP_TILES), (5, 0.1, (1.0, 1.0), mx.MX_PLAN_DEFAULT),
+                                (5, 0.1, (1.0, 1.0), mx.MX_PLAN_ALL_TILES), (4, 0.5, (0.0, 0.0), mx.MX_PLAN_DEFAULT)):
+        A, x = mx.gen_config(cfg, scale=sc)
+        rp, ci, va = torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda()
+        xd = torch.from_numpy(x).cuda()
+        part = mx.Partition(A, *tau)
+        seq = []
+        for rep in range(5):
+            D = mx.Plan.from_device(rp, ci, va, A.cols, tau[0], tau[1], flags)
+            D.spmv(xd)
+            D.close()
+            H = mx.Plan(part, flags)
+            H.spmv(xd)
+            H.close()
+            seq.append(used())
+        part.close()
+        print("memory in use, workload %d flags %d:" % (cfg, flags), [u >> 20 for u in seq], flush=True)
+        assert max(seq[1:]) - seq[0] <= (8 << 20), (cfg, flags, seq)
