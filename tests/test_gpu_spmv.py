@@ -1448,3 +1448,67 @@ def test_plans_release_their_device_memory(mx):
         part.close()
         print("memory in use, workload %d flags %d:" % (cfg, flags), [u >> 20 for u in seq], flush=True)
         assert max(seq[1:]) - seq[0] <= (8 << 20), (cfg, flags, seq)
+
+
+@pytest.mark.gpu
+def test_device_route_on_random_small_matrices(mx):
+    """Host route against device route of plan creation on seeded random matrices of awkward shapes
+    (one row, seven columns, empty rows, rows out of order that name columns twice, a few very long
+    rows, strips and blocks along the diagonal): every array of the plans and y equal, in both
+    precisions and under five sets of flags."""
+    import torch
+    rng = np.random.default_rng(2024)
+    compared = 0
+    for case in range(40):
+        dt = np.float64 if case % 2 else np.float16
+        rows = int(rng.choice([1, 3, 7, 8, 9, 40, 300, 2500, 9000]))
+        cols = int(rng.choice([1, 5, 8, 9, 64, 1000, 20000, 70000, 200000]))
+        kind = case % 4
+        rp, ci = [0], []
+        for r in range(rows):
+            c = []
+            if kind == 0:
+                c = rng.choice(cols, int(rng.integers(0, min(cols, 12) + 1)), replace=False).tolist()
+            elif kind == 1:
+                if cols >= 64:
+                    b0 = (r // 8 * 8) % (cols - 40)
+                    b0 -= b0 % 8
+                    w = int(rng.choice([8, 16, 32, 40]))
+                    c = [b0 + k for k in range(w) if rng.random() < 0.92]
+                if rng.random() < 0.3:
+                    c += rng.choice(cols, min(cols, 3), replace=False).tolist()
+            elif kind == 2:
+                n = int(min(cols, rng.choice([0, 1, 2, 500]) if rng.random() < 0.9 else 5000))
+                c = rng.choice(cols, n, replace=False).tolist()
+            else:
+                c = rng.integers(0, cols, int(rng.integers(0, 20))).tolist()
+            if rng.random() < 0.5:
+                c = sorted(set(c))
+            ci += c
+            rp.append(len(ci))
+        ci = np.asarray(ci, np.int32)
+        if ci.size == 0:
+            continue
+        A = mx.Csr(rows, cols, np.asarray(rp, np.int32), ci, rng.integers(-3, 4, ci.size).astype(dt))
+        xd = torch.from_numpy(rng.integers(-2, 3, cols).astype(dt)).cuda()
+        d = [torch.from_numpy(a).cuda() for a in (A.rowPtr, A.colInd, A.val)]
+        for tc, tr in ((1.0, 1.0), (0.5, 0.25), (0.75, 0.0)):
+            part = mx.Partition(A, tc, tr)
+            for flags in (mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_ALL_TILES, mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_SLICES,
+                          mx.MX_PLAN_NO_TILES | mx.MX_PLAN_CSR_ROWS):
+                print("case %d %s rows=%d cols=%d nnz=%d kind=%d tau=(%g, %g) flags=%d" % (case, dt.__name__, rows, cols, ci.size, kind, tc, tr,
+                                                                                       flags), flush=True)
+                H = mx.Plan(part, flags)
+                D = mx.Plan.from_device(d[0], d[1], d[2], cols, tc, tr, flags)
+                for k in ("csr_variant", "csr_nnz", "tile_nnz", "tile_chunks", "tile_frags", "tile_variant", "tile_strip_nnz"):
+                    assert H.info[k] == D.info[k], (case, tc, tr, flags, k, H.info[k], D.info[k])
+                ah, ad = H.arrays(), D.arrays()
+                assert sorted(ah) == sorted(ad), (case, tc, tr, flags)
+                for k in ah:
+                    assert ah[k] == ad[k], (case, tc, tr, flags, k)
+                assert torch.equal(H.spmv(xd), D.spmv(xd)), (case, tc, tr, flags)
+                compared += 1
+                H.close()
+                D.close()
+            part.close()
+    assert compared >= 400, compared
