@@ -368,6 +368,21 @@ typedef struct mx_tau_point {
 int mx_tune_tau(const mx_csr *A, int levels, int flags, int warm, int iters, float *tau_c, float *tau_r,
                 mx_tau_point *table, int cap, int *n_points);
 
+/* The same choice from counts alone, nothing planned or timed: for every point of that grid the
+ * extraction runs on the device and the estimate a plan makes of its own tiles -- the entries they
+ * take off the CSR part against their launch and their own stream, at rates measured on MI355X -- is
+ * read off; the point whose tiles save most wins, (0, 0) when none saves anything.  The reference's
+ * counterpart is the regression model of ML/train_*.py over the count features of
+ * ML/extract_features.cpp:31-95, queried through ML/bayes_opt.py; here the features are the counts the
+ * plan itself decides from (fragments and entries that pass the fill gate, strip chunks, 8 x 8
+ * blocks).  A host matrix is uploaded once.  `table` as in mx_tune_tau. */
+typedef struct mx_tau_estimate {
+    float tau_c, tau_r;
+    double saved_us;         /* estimated microseconds per product that the kept tile forms save (0: none kept) */
+    long long tile_entries;  /* entries those forms would hold */
+} mx_tau_estimate;
+int mx_estimate_tau(const mx_csr *A, int levels, float *tau_c, float *tau_r, mx_tau_estimate *table, int cap, int *n_points);
+
 /* Facts about a plan, for reporting. */
 typedef struct mx_plan_info {
     mx_dtype dtype;

@@ -57,6 +57,10 @@ class PlanInfo(C.Structure):
                 ("ext_frags", C.c_int)]
 
 
+class TauEstimate(C.Structure):
+    _fields_ = [("tau_c", C.c_float), ("tau_r", C.c_float), ("saved_us", C.c_double), ("tile_entries", C.c_longlong)]
+
+
 class PlanArray(C.Structure):
     _fields_ = [("name", C.c_char_p), ("bytes", C.c_size_t), ("data", C.c_void_p)]
 
@@ -126,6 +130,7 @@ SIGNATURES = {
     "mx_plan_create": (_i, [_vp, _i, _pp]),
     "mx_plan_create_device_csr": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _i, _pp]),
     "mx_plan_create_device": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, C.c_float, C.c_float, _i, _pp]),
+    "mx_estimate_tau": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp]),
     "mx_plan_arrays": (_i, [_vp, _vp, _i, _vp]),
     "mx_plan_arrays_free": (None, [_vp, _i]),
     "mx_plan_destroy": (None, [_vp]),

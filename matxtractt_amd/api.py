@@ -15,7 +15,7 @@ from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLA
                    MX_PLAN_KEEP_TILES, MX_PLAN_NO_TILES, MxError, check)
 
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "split_device", "tiles_device", "cdspmv",
-           "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "MxError",
+           "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "estimate_tau", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
            "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "plan_layout"]
 
@@ -356,6 +356,17 @@ def tune_tau(A, levels=5, flags=MX_PLAN_DEFAULT, warm=20, iters=200):
     check(_lib.load().mx_tune_tau(C.byref(st), int(levels), int(flags), int(warm), int(iters), C.byref(c), C.byref(r),
                                   table, cap, C.byref(n)))
     return c.value, r.value, [(t.tau_c, t.tau_r, t.ms_total, t.tile_nnz) for t in table[:n.value]]
+
+
+def estimate_tau(A, levels=5):
+    """(tau_c, tau_r, table) for matrix A from counts alone (mx_estimate_tau): nothing is planned or
+    timed; table = [(tau_c, tau_r, saved_us, tile_entries), ...]."""
+    st = A.struct()
+    cap = levels * (levels + 1) // 2
+    table = (_lib.TauEstimate * cap)()
+    c, r, n = C.c_float(), C.c_float(), C.c_int()
+    check(_lib.load().mx_estimate_tau(C.byref(st), int(levels), C.byref(c), C.byref(r), table, cap, C.byref(n)))
+    return c.value, r.value, [(t.tau_c, t.tau_r, t.saved_us, t.tile_entries) for t in table[:n.value]]
 
 
 def _torch_dtype(dt):

@@ -8,7 +8,7 @@
 // overwrite the file's values with i%15 as the reference does at :1091), --warm W --iters K
 // (default 200 / 4000), --no-tiles / --all-tiles (plan flags), --json (one JSON record on the
 // last line), --tune (pick the two fractions from the 5x5 grid by timing each on the device,
-// then run with them), --partition-cache FILE (read the partition from FILE when it was made for a
+// then run with them), --estimate-tau (pick them from counts over the same grid, nothing timed), --partition-cache FILE (read the partition from FILE when it was made for a
 // matrix of this shape with these fractions, otherwise compute it and write FILE), --device-prep (the extraction runs on the GPU instead of the
 // host cores; same partition), --device-plan (the matrix is uploaded as it is and everything after
 // that -- extraction, the plan's decisions, its layouts -- happens on the GPU: mx_plan_create_device;
@@ -97,7 +97,7 @@ int main(int argc, char **argv)
     int config = 0, warm = 200, iters = 4000, planFlags = MX_PLAN_DEFAULT;
     double scale = 1.0;
     unsigned long long seed = 0;
-    bool keepValues = false, json = false, tune = false, devicePrep = false, devicePlan = false;
+    bool keepValues = false, json = false, tune = false, estimate = false, devicePrep = false, devicePlan = false;
     std::string cachePath;
     for (int i = 1; i < argc; ++i) {
         std::string a = argv[i];
@@ -120,6 +120,7 @@ int main(int argc, char **argv)
         else if (a == "--json") json = true;
         else if (a == "--partition-cache") cachePath = next("--partition-cache");
         else if (a == "--tune") tune = true;
+        else if (a == "--estimate-tau") estimate = true;
         else if (a == "--device-prep") devicePrep = true;
         else if (a == "--device-plan") devicePlan = true;
         else pos.push_back(a);
@@ -195,6 +196,23 @@ int main(int argc, char **argv)
             printf("tune: col_frac = %.2f hot_frac = %.2f time = %lf ms tile_nnz = %d\n", table[i].tau_c, table[i].tau_r,
                    table[i].ms_total, table[i].tile_nnz);
         printf("tuned: col_frac = %.2f hot_frac = %.2f\n", tc, tr);
+        col_frac = tc;
+        hot_frac = tr;
+    }
+    if (estimate) {
+        // the two fractions from counts over the grid (the plan's own estimate of what its tiles save), nothing timed
+        mx_csr A{rowA, colA, (int)nnzA, MX_VALT_DTYPE, csrRowPtr, csrColInd, csrVal};
+        mx_tau_estimate table[15];
+        float tc = 0.f, tr = 0.f;
+        int n = 0;
+        if (mx_estimate_tau(&A, 5, &tc, &tr, table, 15, &n) != MX_OK) {
+            printf("Error: %s\n", mx_last_error());
+            return 1;
+        }
+        for (int i = 0; i < n && i < 15; ++i)
+            printf("estimate: col_frac = %.2f hot_frac = %.2f saved = %lf us tile_nnz = %lld\n", table[i].tau_c, table[i].tau_r,
+                   table[i].saved_us, table[i].tile_entries);
+        printf("estimated: col_frac = %.2f hot_frac = %.2f\n", tc, tr);
         col_frac = tc;
         hot_frac = tr;
     }

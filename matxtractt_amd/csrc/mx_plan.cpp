@@ -1582,8 +1582,9 @@ static double tile_gate(mx_dtype)
 // general*: the reference's fragments that pass the fill gate; strip*: the chunks of the plan's
 // own (binary16 strips, or binary64 8 x 8 blocks with `blocks64`).
 // 0 = nothing pays, 1 = only the plan's own chunks do, 2 = keep both.
+// `netNs` (optional): what the forms that are kept save per product by this estimate, in ns.
 static int tiles_worth(mx_dtype dtype, int fragM, int fragK, bool blocks64, double generalEntries, double generalFrags,
-                       double stripEntries, double stripBlocks)
+                       double stripEntries, double stripBlocks, double *netNs = nullptr)
 {
     const int es = mx::elem_size(dtype);
     const double blockBytes = (double)fragM * (blocks64 ? 8 : fragK) * es, slots = mx::tile_slots(dtype);
@@ -1591,10 +1592,15 @@ static int tiles_worth(mx_dtype dtype, int fragM, int fragK, bool blocks64, doub
     const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
     const double launchNs = 5000.0, stripLaunchNs = 1000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
     const double savedNs = (generalEntries + stripEntries) * (es + 2) / fastRate;
-    const double costNs = (generalFrags > 0 ? launchNs + generalBytes / generalRate : 0.0) +
-                          (stripBlocks > 0 ? stripLaunchNs + stripBytes / fastRate : 0.0);
-    if (savedNs <= costNs) return 0;
-    if (generalFrags > 0 && generalEntries * (es + 2) / fastRate <= launchNs + generalBytes / generalRate) return 1;
+    const double generalCost = generalFrags > 0 ? launchNs + generalBytes / generalRate : 0.0;
+    const double stripCost = stripBlocks > 0 ? stripLaunchNs + stripBytes / fastRate : 0.0;
+    if (netNs) *netNs = 0.0;
+    if (savedNs <= generalCost + stripCost) return 0;
+    if (generalFrags > 0 && generalEntries * (es + 2) / fastRate <= generalCost) {
+        if (netNs) *netNs = stripEntries * (es + 2) / fastRate - stripCost;
+        return 1;
+    }
+    if (netNs) *netNs = savedNs - generalCost - stripCost;
     return 2;
 }
 
@@ -3056,6 +3062,81 @@ extern "C" int mx_tune_tau(const mx_csr *A, int levels, int flags, int warm, int
                 have = true;
             }
         }
+    release();
+    if (n_points) *n_points = n;
+    return rc;
+}
+
+// The two fractions from counts alone: for every point of the grid the extraction runs on the device
+// (HybridDevice::analyse) and the plan's own estimate of what its tiles save per product is read off;
+// the point with the largest saving wins, (0, 0) when none saves anything.  Nothing is planned or
+// timed.  (The reference's counterpart is the regression model of ML/train_*.py over the count
+// features of ML/extract_features.cpp:31-95, queried through ML/bayes_opt.py.)
+extern "C" int mx_estimate_tau(const mx_csr *A, int levels, float *tau_c, float *tau_r, mx_tau_estimate *table, int cap, int *n_points)
+{
+    if (!A || levels < 2 || levels > 65 || !tau_c || !tau_r || (table && cap < 0) || A->rows < 1 || A->cols < 1 || A->nnz < 0 ||
+        !A->rowPtr || (A->nnz > 0 && (!A->colInd || !A->val)) || (A->dtype != MX_F64 && A->dtype != MX_F16)) {
+        set_error("mx_estimate_tau: bad argument");
+        return MX_ERR_ARG;
+    }
+    int rc = need_device();
+    if (rc) return rc;
+    const size_t es = (size_t)mx::elem_size(A->dtype);
+    int *dRowPtr = nullptr, *dColInd = nullptr;
+    void *dVal = nullptr;
+    auto release = [&]() {
+        (void)hipFree(dRowPtr);
+        (void)hipFree(dColInd);
+        (void)hipFree(dVal);
+    };
+    rc = upload(&dRowPtr, A->rowPtr, (size_t)A->rows + 1);
+    if (!rc) rc = upload(&dColInd, A->colInd, (size_t)A->nnz);
+    if (!rc) rc = upload_bytes(&dVal, A->val, (size_t)A->nnz * es);
+    if (!rc) rc = mx::check_csr_device(A->rows, A->cols, A->nnz, dRowPtr, dColInd, nullptr, "mx_estimate_tau");
+    if (rc) {
+        release();
+        return rc;
+    }
+    const int fragM = mx::kFragM, fragK = mx::frag_k(A->dtype);
+    const double need = tile_gate(A->dtype) * fragM * fragK;
+    int minVals = (int)need;
+    while ((double)minVals < need) ++minVals;
+    const char *envNoStrips = std::getenv("MX_NO_STRIPS"), *envNoBlocks = std::getenv("MX_NO_BLOCKS");
+    const bool wantStrips = A->dtype == MX_F16 && !(envNoStrips && std::atoi(envNoStrips));
+    const bool wantBlocks = A->dtype == MX_F64 && !(envNoBlocks && std::atoi(envNoBlocks));
+    double best = 0.0;
+    *tau_c = *tau_r = 0.0f;
+    int n = 0;
+    try {
+        for (int ic = 0; ic < levels && !rc; ++ic)
+            for (int ir = 0; ir <= ic && !rc; ++ir) {
+                const float c = (float)ic / (float)(levels - 1), r = (float)ir / (float)(levels - 1);
+                mx_tau_estimate e{c, r, 0.0, 0};
+                if (ic > 0 && A->nnz > 0) {  // (tau_c = 0 selects nothing)
+                    mx::HybridDevice H;
+                    mx::HybridCounts cnt;
+                    if ((rc = H.analyse(A->dtype, A->rows, A->cols, A->nnz, dRowPtr, dColInd, dVal, c, r, minVals, true, wantStrips, wantBlocks,
+                                        &cnt, nullptr)))
+                        break;
+                    if (cnt.blocks64) cnt.generalFrags = cnt.generalEntries = 0;
+                    double netNs = 0.0;
+                    const int worth = tiles_worth(A->dtype, fragM, fragK, cnt.blocks64, (double)cnt.generalEntries, (double)cnt.generalFrags,
+                                                  (double)cnt.stripEntries, (double)cnt.stripBlocks, &netNs);
+                    e.saved_us = netNs * 1e-3;
+                    e.tile_entries = worth == 0 ? 0 : (worth == 2 ? cnt.generalEntries : 0) + cnt.stripEntries;
+                }
+                if (table && n < cap) table[n] = e;
+                ++n;
+                if (e.saved_us > best) {
+                    best = e.saved_us;
+                    *tau_c = c;
+                    *tau_r = r;
+                }
+            }
+    } catch (const std::bad_alloc &) {
+        set_error("mx_estimate_tau: out of memory");
+        rc = MX_ERR_ALLOC;
+    }
     release();
     if (n_points) *n_points = n;
     return rc;

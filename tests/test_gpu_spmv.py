@@ -870,6 +870,34 @@ def test_tau_tuner(mx, ora):
         P.close()
 
 
+def test_tau_from_counts_alone(mx, ora):
+    """mx_estimate_tau: the grid of mx_tune_tau walked without planning or timing anything -- per
+    point the extraction on the device and the plan's own estimate of what its tiles save.  On the
+    mixed workload it names a point whose default plan keeps exactly the strip entries it counted
+    and multiplies to the oracle's y; on the others, where no default plan keeps tiles, (0, 0)."""
+    import torch
+    A, x = mx.gen_config(5, scale=1 / 4)
+    tc, tr, table = mx.estimate_tau(A, levels=3)
+    assert [(c, r) for c, r, _, _ in table] == [(0.0, 0.0), (0.5, 0.0), (0.5, 0.5), (1.0, 0.0), (1.0, 0.5), (1.0, 1.0)]
+    best = max(table, key=lambda t: t[2])
+    assert best[2] > 0 and (tc, tr) == (best[0], best[1]), table
+    for c, r, saved, entries in table:
+        P = mx.Partition(A, c, r)
+        plan = mx.Plan(P)                      # default flags: the plan asks the same question
+        assert plan.info["tile_nnz"] == entries and (saved > 0) == (entries > 0), (c, r, saved, entries, plan.info["tile_nnz"])
+        if (c, r) == (tc, tr):
+            y = plan.spmv(torch.from_numpy(x).cuda()).cpu().numpy()
+            assert rel_l2(y, oracle_y(ora, mx, A, x)) <= F16_TOL
+        plan.close()
+        P.close()
+    for cfg, scale in ((2, 1.0), (4, 0.25), (1, 1.0)):
+        A, _ = mx.gen_config(cfg, scale=scale)
+        tc, tr, table = mx.estimate_tau(A, levels=3)
+        assert (tc, tr) == (0.0, 0.0) and all(saved == 0 and entries == 0 for _, _, saved, entries in table), (cfg, table)
+    with pytest.raises(mx.MxError):
+        mx.estimate_tau(A, levels=1)
+
+
 def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
     """matxtract_perftest's stdout keeps the forms the reference's scripts grep for."""
     import re
@@ -888,6 +916,10 @@ def test_cli_prints_the_lines_other_tools_parse(mx, tmp_path):
     out = subprocess.run([exe, "--warm", "2", "--iters", "5", "--tune", str(p)], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stderr
     assert len(re.findall(r"tune: col_frac = ", out.stdout)) == 15 and re.search(r"tuned: col_frac = \d\.\d\d hot_frac = \d\.\d\d", out.stdout)
+    assert "Success! All values match" in out.stdout
+    out = subprocess.run([exe, "--warm", "2", "--iters", "5", "--estimate-tau", str(p)], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert len(re.findall(r"estimate: col_frac = ", out.stdout)) == 15 and re.search(r"estimated: col_frac = \d\.\d\d hot_frac = \d\.\d\d", out.stdout)
     assert "Success! All values match" in out.stdout
     for args in (["0.5", "0.25", str(p)], [str(p)]):
         out = subprocess.run([exe, "--warm", "2", "--iters", "5", *args], capture_output=True, text=True, timeout=120)
