@@ -275,6 +275,23 @@ int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int nnz, const
 int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
                           const void *val_dev, float tau_c, float tau_r, int flags, mx_plan **out);
 
+/* The host's share of laying tiles out on the device, for inspection (no device needed): from the
+ * number of blocks of every chunk alone, the steps of the layout -- a chunk of up to slots / 2 blocks
+ * shares a step with the next such chunk, a larger one takes whole steps of its own -- and its waves,
+ * exactly as mx_plan_layout lays the same chunks out.  stepDesc: 10 ints per step {chunk of half 0,
+ * chunk of half 1 (-1 none, -2 the first goes on), flags, blocks in half 0, blocks in half 1, first
+ * value, first value and blocks in half 0 of the step four further on, first block of half 0 inside
+ * its chunk, 0}; chunkBlock0[nChunks]: first block of every chunk among the stored values; waveDesc: 8
+ * ints per wave.  blockValues: values per block; perMin: fewest steps a wave takes.  No counterpart
+ * in the reference, which walks its fragments in place. */
+typedef struct mx_tile_steps_view {
+    int steps, nWaves;
+    long long totalBlocks;
+    int *stepDesc, *chunkBlock0, *waveDesc;
+} mx_tile_steps_view;
+int mx_tile_steps(const int *chunkBlocks, int nChunks, int slots, int blockValues, int perMin, int nCU, mx_tile_steps_view *out);
+void mx_tile_steps_free(mx_tile_steps_view *v);
+
 /* Every device array of a plan copied to host memory, each with a name ("slices.ecol",
  * "strips.hdr", ...) and its size: for tests that hold two routes of making a plan against each
  * other.  `out` has room for `cap` entries (32 is enough); *n receives their number; the data

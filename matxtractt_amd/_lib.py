@@ -61,6 +61,11 @@ class TauEstimate(C.Structure):
     _fields_ = [("tau_c", C.c_float), ("tau_r", C.c_float), ("saved_us", C.c_double), ("tile_entries", C.c_longlong)]
 
 
+class TileStepsView(C.Structure):
+    _fields_ = [("steps", C.c_int), ("nWaves", C.c_int), ("totalBlocks", C.c_longlong), ("stepDesc", C.c_void_p),
+                ("chunkBlock0", C.c_void_p), ("waveDesc", C.c_void_p)]
+
+
 class PlanArray(C.Structure):
     _fields_ = [("name", C.c_char_p), ("bytes", C.c_size_t), ("data", C.c_void_p)]
 
@@ -131,6 +136,8 @@ SIGNATURES = {
     "mx_plan_create_device_csr": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _i, _pp]),
     "mx_plan_create_device": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, C.c_float, C.c_float, _i, _pp]),
     "mx_estimate_tau": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp]),
+    "mx_tile_steps": (_i, [_vp, _i, _i, _i, _i, _i, _vp]),
+    "mx_tile_steps_free": (None, [_vp]),
     "mx_plan_arrays": (_i, [_vp, _vp, _i, _vp]),
     "mx_plan_arrays_free": (None, [_vp, _i]),
     "mx_plan_destroy": (None, [_vp]),

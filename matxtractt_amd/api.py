@@ -15,7 +15,7 @@ from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLA
                    MX_PLAN_KEEP_TILES, MX_PLAN_NO_TILES, MxError, check)
 
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "split_device", "tiles_device", "cdspmv",
-           "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "estimate_tau", "MxError",
+           "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "estimate_tau", "tile_steps", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
            "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "plan_layout"]
 
@@ -344,6 +344,21 @@ def plan_layout(part, flags=MX_PLAN_DEFAULT, nCU=256):
     finally:
         _lib.load().mx_plan_layout_free(C.byref(v))
     return out
+
+
+def tile_steps(chunk_blocks, slots, block_values, per_min, nCU):
+    """The steps and waves of a tile layout from the block counts of its chunks (mx_tile_steps, no GPU
+    needed): dict with stepDesc [steps, 10], chunkBlock0, waveDesc [nWaves, 8], totalBlocks."""
+    cb = np.ascontiguousarray(chunk_blocks, dtype=np.int32)
+    v = _lib.TileStepsView()
+    check(_lib.load().mx_tile_steps(_p(cb), cb.size, int(slots), int(block_values), int(per_min), int(nCU), C.byref(v)))
+    try:
+        return {"steps": int(v.steps), "nWaves": int(v.nWaves), "totalBlocks": int(v.totalBlocks),
+                "stepDesc": _view(v.stepDesc, v.steps * 10, np.int32).reshape(-1, 10).copy(),
+                "chunkBlock0": _view(v.chunkBlock0, cb.size, np.int32).copy(),
+                "waveDesc": _view(v.waveDesc, v.nWaves * 8, np.int32).reshape(-1, 8).copy()}
+    finally:
+        _lib.load().mx_tile_steps_free(C.byref(v))
 
 
 def tune_tau(A, levels=5, flags=MX_PLAN_DEFAULT, warm=20, iters=200):

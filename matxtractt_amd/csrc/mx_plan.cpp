@@ -2291,6 +2291,51 @@ static int plan_tile_steps(const std::vector<int> &chunkBlocks, int SF, int BS, 
     return MX_OK;
 }
 
+// plan_tile_steps for inspection (tests hold it against the layouts build_tiles makes, without a GPU)
+extern "C" void mx_tile_steps_free(mx_tile_steps_view *v)
+{
+    if (!v) return;
+    free(v->stepDesc);
+    free(v->chunkBlock0);
+    free(v->waveDesc);
+    std::memset(v, 0, sizeof(*v));
+}
+extern "C" int mx_tile_steps(const int *chunkBlocks, int nChunks, int slots, int blockValues, int perMin, int nCU, mx_tile_steps_view *out)
+{
+    if (!out || nChunks < 0 || (nChunks > 0 && !chunkBlocks) || slots < 2 || (slots & 1) || blockValues < 1 || perMin < 1 || nCU < 1) {
+        set_error("mx_tile_steps: bad argument");
+        return MX_ERR_ARG;
+    }
+    std::memset(out, 0, sizeof(*out));
+    try {
+        std::vector<int> blocks(chunkBlocks, chunkBlocks + nChunks), stepDesc, chunkBlock0, waveDesc;
+        long long total = 0;
+        const int rc = plan_tile_steps(blocks, slots, blockValues, perMin, nCU, 10, stepDesc, chunkBlock0, waveDesc, &total);
+        if (rc) return rc;
+        auto give = [](const std::vector<int> &v) {
+            int *q = (int *)malloc(std::max<size_t>(v.size(), 1) * sizeof(int));
+            if (q && !v.empty()) std::memcpy(q, v.data(), v.size() * sizeof(int));
+            return q;
+        };
+        out->steps = (int)(stepDesc.size() / 10);
+        out->nWaves = (int)(waveDesc.size() / 8);
+        out->totalBlocks = total;
+        out->stepDesc = give(stepDesc);
+        out->chunkBlock0 = give(chunkBlock0);
+        out->waveDesc = give(waveDesc);
+        if (!out->stepDesc || !out->chunkBlock0 || !out->waveDesc) {
+            mx_tile_steps_free(out);
+            set_error("mx_tile_steps: out of memory");
+            return MX_ERR_ALLOC;
+        }
+    } catch (const std::bad_alloc &) {
+        mx_tile_steps_free(out);
+        set_error("mx_tile_steps: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    return MX_OK;
+}
+
 // A hybrid plan from a CSR matrix in device memory and the two extraction fractions: the
 // extraction, the plan's decisions, the CSR part with its layout and the strips' layout are all
 // made on the device (mx_hybrid.hip, mx_layout.hip); what a decision needs comes to the host as

@@ -728,6 +728,71 @@ def test_plan_layout_walk(mx, ora, case):
 
 
 
+def _chunks_of_steps(hdr):
+    """The block counts of a tile layout's chunks, read back from its step headers: a step whose
+    halves are different chunks (flag 2) holds two (or one, waiting for a partner that never came), a
+    chunk larger than half a step runs over steps without that flag up to one with flag 1."""
+    chunks, run = [], 0
+    for h in hdr:
+        flags, n0, n1 = int(h[16]), int(h[17]), int(h[18])
+        if flags & 2:
+            chunks.append(n0)
+            if n1 > 0:
+                chunks.append(n1)
+        else:
+            run += n0 + n1
+            if flags & 1:
+                chunks.append(run)
+                run = 0
+    assert run == 0
+    return chunks
+
+
+@pytest.mark.parametrize("case", ["block_f64", "mixed_f16", "strips_f16", "blocks_f16", "twice_f64"])
+def test_tile_steps_from_block_counts_alone(mx, case):
+    """mx_tile_steps -- the host's share of laying tiles out on the device: steps and waves from the
+    chunks' block counts -- gives the steps, value offsets, look-ahead fields and waves that
+    mx_plan_layout gives the same chunks (general tiles, binary16 strips, binary64 blocks)."""
+    rng = np.random.default_rng(sum(map(ord, case)))
+    if case == "strips_f16":
+        A = _strip_matrix(mx, rng)
+    elif case == "blocks_f16":
+        A = _block_rows_matrix(mx, rng)
+    elif case == "twice_f64":
+        lens = rng.integers(0, 50, 300)
+        rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        A = mx.Csr(300, 80, rp, rng.integers(0, 80, rp[-1]).astype(np.int32), rng.integers(-3, 4, rp[-1]).astype(np.float64))
+    else:
+        cfg, scale = {"block_f64": (2, 1 / 64), "mixed_f16": (5, 1 / 512)}[case]
+        A, _ = mx.gen_config(cfg, scale=scale)
+    seen = 0
+    for tau in ((1.0, 1.0), (0.75, 0.5)):
+        P = mx.Partition(A, *tau)
+        for flags in (mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_ALL_TILES):
+            for nCU in (1, 4):
+                L = mx.plan_layout(P, flags, nCU=nCU)
+                f64 = A.dtype == mx.MX_F64
+                for t, T in enumerate(L["tiles"]):
+                    if T["steps"] == 0:
+                        continue
+                    # the plan's own chunks are made of blocks of 8 columns, four to a half, in both precisions
+                    slots, values, per_min = (8, 64, 1 if f64 else 2) if t == 1 else (L["slots"], 8 * L["fragK"], 2)
+                    chunks = _chunks_of_steps(T["hdr"])
+                    S = mx.tile_steps(chunks, slots, values, per_min, nCU)
+                    assert S["steps"] == T["steps"] and S["nWaves"] == T["nWaves"], (case, tau, flags, t)
+                    assert np.array_equal(S["stepDesc"][:, 2:5], T["hdr"][:, 16:19])          # flags, blocks per half
+                    assert np.array_equal(S["stepDesc"][:, 5], T["valOffset"])
+                    assert np.array_equal(S["stepDesc"][:, 6:8], T["hdr"][:, 19:21])          # the step four further on
+                    assert np.array_equal(S["waveDesc"], T["waveDesc"])
+                    assert S["totalBlocks"] * values == T["val"].size
+                    assert len(chunks) == T["chunks"]
+                    seen += 1
+        P.close()
+    assert seen > 0, case
+    with pytest.raises(mx.MxError):
+        mx.tile_steps([0, 3], 8, 64, 2, 4)
+
+
 def test_host_code_under_sanitizers(tmp_path):
     """The library's host code (generators, partition, slice layout, the host half of a plan) built
     with -fsanitize=address,undefined and run on the five workloads at small scale: no report."""
