@@ -236,6 +236,13 @@ double mx_algorithmic_bytes(mx_dtype dtype, int rows, int cols, int nnz);
                                  the CSR part when they do not (the reference gates its tile kernel on matrix
                                  size and fill, test/test_autotc_spmv.cpp:1507,1518) */
 
+#define MX_PLAN_NO_FUSE 32   /* CSR part in slice form: always two launches (csr_slice_kernel, then slice_combine_kernel).
+                                 Without this flag a plan whose CSR part is the whole product takes the one-launch
+                                 form (mx_plan_info.csr_fused) where the matrix suits it -- no row with more than eight
+                                 virtual rows, at most 160 rows per workgroup (beyond that the form only ties) -- and
+                                 the device deals its workgroups round-robin to eight XCDs, which plan creation checks */
+#define MX_PLAN_FUSE 64      /* the one-launch form wherever the matrix suits it, whatever its size */
+
 /* Uploads a partition once and keeps it on the device: the persistent counterpart of the
  * per-call cudaMalloc/cudaMemcpy blocks in cdspmv (src/spmv_kernel/cdSpMV.cu:407-418) and
  * du_tcspmv_fp64 (src/spmv_kernel/du_tcSpMV_fp64.cu:271-300), plus the x_d/x_s/x_CD
@@ -329,6 +336,15 @@ int mx_spmv(mx_plan *plan, const void *x_dev, void *y_dev, void *stream);
  * start at zero: every sum the second kernel reads is written by the first in the same call. */
 int mx_spmv_static(mx_plan *plan, const void *x_dev, void *y_dev, void *stream);
 int mx_static_scratch_bytes(void);
+
+/* For tests of the one-launch form's way out (no counterpart in the reference).  A one-launch product
+ * relies on the device dealing the workgroups of a launch round-robin to its eight XCDs (a workgroup takes
+ * its share of the work by the XCD it runs on and its number / 8); every launch checks that no share is taken
+ * twice, and a workgroup that finds its share taken sets a word in host memory.  The next product of any
+ * one-launch plan then returns MX_ERR_DEVICE once (the products since the previous call may be wrong) and every
+ * plan of the process takes the two-launch form from there on.  mx_debug_fused_misplaced(1) sets that word from
+ * the host, as such a workgroup would; (0) clears it and lets new plans take the one-launch form again. */
+int mx_debug_fused_misplaced(int set);
 
 /* n back-to-back SpMVs y = A*x on `stream`, queued from C without returning to the caller in
  * between: the reference's timed loops (src/spmv_kernel/cdSpMV.cu:464-469) as an entry point,
@@ -443,6 +459,10 @@ typedef struct mx_plan_info {
     int ext_dCols, ext_dRows, ext_nnzRowD, ext_frags; /* what the extraction behind the plan selected (columns, rows,
                             entries of A_dd) and the fragments of its tile encoding -- cols_ratio and TC_nnz_ratio of
                             the reference's driver follow from them; 0 for plans without an extraction */
+    int csr_fused;       /* 1: the CSR part in slice form runs as ONE launch (the reference's residual kernel is one
+                            launch too, src/spmv_kernel/cdSpMV.cu:459): the workgroups that hold sums of the same rows
+                            sit on one XCD, count themselves off on a counter in that XCD's L2, and the one that
+                            completes the count adds the sums up and writes y; nobody waits.  0: two launches */
 } mx_plan_info;
 int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
 
@@ -470,8 +490,22 @@ typedef struct mx_slice_layout_view {
     int nDict;            /* > 0: the value dictionary form exists beside the values (at most 255 distinct values) */
     unsigned char *ecode; /* [nEcol] one byte per entry, at the place of its column offset; 255 = the padding's zero */
     unsigned char *dict;  /* [256] values (binary64 or binary16), zeros beyond nDict */
+    /* the one-launch form (mx_slice_layout_fused; all zero otherwise): rows in groups of groupRows, virtual rows
+     * ordered by (slice, group, length), workgroup b (of nWG = nCU, in the numbering of wgDesc) belongs to XCD
+     * b * 8 / nWG and bumps the counters of groups wgGroups[b] = {first, count}; groupNeed[g] = how many
+     * workgroups bump group g; fusedTarget[64 * chunk + lane] = where that virtual row puts its sum: the k-th
+     * virtual row of row r at ((r / groupRows) * placesPerRow + k) * groupRows + r % groupRows (padding lanes
+     * at nGroups * placesPerRow * groupRows + lane); rowVrows[r] = virtual rows of row r */
+    int fused, groupRows, nGroups, placesPerRow;
+    int *wgGroups, *groupNeed, *fusedTarget;
+    unsigned char *rowVrows;
 } mx_slice_layout_view;
 int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *sel, mx_slice_layout_view *out);
+/* The layout of the one-launch form for the whole matrix (out->fused = 1), or the ordinary one
+ * (out->fused = 0) when the matrix does not suit it: a row with more than eight virtual rows, more
+ * slices with entries in an XCD's rows than the XCD has workgroups, or more chunks in a workgroup
+ * than it can keep the targets of in LDS. */
+int mx_slice_layout_fused(const mx_csr *A, int nCU, mx_slice_layout_view *out);
 /* The same view by the route plans take for a whole matrix: A goes up, the layout is built on the
  * device from the device arrays (sorts, running sums and placement kernels; only the assignment of
  * chunks to workgroups and waves, a few values per thousand entries, is decided on the host, by the

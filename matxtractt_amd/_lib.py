@@ -13,7 +13,7 @@ CSRC = os.path.join(_HERE, "csrc")
 MX_OK, MX_ERR_ARG, MX_ERR_ALLOC, MX_ERR_DEVICE, MX_ERR_IO = 0, 1, 2, 3, 4
 MX_F64, MX_F16 = 0, 1
 MX_PLAN_DEFAULT, MX_PLAN_NO_TILES, MX_PLAN_ALL_TILES = 0, 1, 2
-MX_PLAN_CSR_ROWS, MX_PLAN_CSR_SLICES, MX_PLAN_KEEP_TILES = 4, 8, 16
+MX_PLAN_CSR_ROWS, MX_PLAN_CSR_SLICES, MX_PLAN_KEEP_TILES, MX_PLAN_NO_FUSE, MX_PLAN_FUSE = 4, 8, 16, 32, 64
 
 
 class MxError(RuntimeError):
@@ -54,7 +54,7 @@ class PlanInfo(C.Structure):
                 ("csr_main_kernel", C.c_int), ("csr_main_nnz", C.c_int), ("tile_variant", C.c_int), ("tile_strip_nnz", C.c_int),
                 ("csr_value_dict", C.c_int), ("est_rows_us", C.c_double), ("est_slices_us", C.c_double),
                 ("prep_route", C.c_int), ("ext_dCols", C.c_int), ("ext_dRows", C.c_int), ("ext_nnzRowD", C.c_int),
-                ("ext_frags", C.c_int)]
+                ("ext_frags", C.c_int), ("csr_fused", C.c_int)]
 
 
 class TauEstimate(C.Structure):
@@ -76,7 +76,9 @@ class SliceLayoutView(C.Structure):
                [("nEcol", C.c_longlong)] + \
                [(n, C.c_void_p) for n in ("wgDesc", "waveDesc", "chunkEnd", "segPtr", "segIdx", "rowInfo", "lightInfo",
                                         "heavyInfo", "ecol", "eval")] + \
-               [("nDict", C.c_int), ("ecode", C.c_void_p), ("dict", C.c_void_p)]
+               [("nDict", C.c_int), ("ecode", C.c_void_p), ("dict", C.c_void_p)] + \
+               [(n, C.c_int) for n in ("fused", "groupRows", "nGroups", "placesPerRow")] + \
+               [(n, C.c_void_p) for n in ("wgGroups", "groupNeed", "fusedTarget", "rowVrows")]
 
 
 class TileLayoutView(C.Structure):
@@ -154,6 +156,8 @@ SIGNATURES = {
                          C.POINTER(TauPoint), _i, _pi]),
     "mx_slice_layout": (_i, [C.POINTER(CsrStruct), _i, _vp, C.POINTER(SliceLayoutView)]),
     "mx_slice_layout_device": (_i, [C.POINTER(CsrStruct), _i, C.POINTER(SliceLayoutView)]),
+    "mx_slice_layout_fused": (_i, [C.POINTER(CsrStruct), _i, C.POINTER(SliceLayoutView)]),
+    "mx_debug_fused_misplaced": (_i, [_i]),
     "mx_slice_layout_free": (None, [C.POINTER(SliceLayoutView)]),
     "mx_plan_layout": (_i, [_vp, _i, _i, C.POINTER(PlanLayoutView)]),
     "mx_plan_layout_free": (None, [C.POINTER(PlanLayoutView)]),

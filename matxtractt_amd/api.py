@@ -12,12 +12,12 @@ import numpy as np
 
 from . import _lib
 from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLAN_CSR_ROWS, MX_PLAN_DEFAULT,
-                   MX_PLAN_KEEP_TILES, MX_PLAN_NO_TILES, MxError, check)
+                   MX_PLAN_FUSE, MX_PLAN_KEEP_TILES, MX_PLAN_NO_FUSE, MX_PLAN_NO_TILES, MxError, check)
 
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "split_device", "tiles_device", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "estimate_tau", "tile_steps", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
-           "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "plan_layout"]
+           "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "MX_PLAN_NO_FUSE", "MX_PLAN_FUSE", "plan_layout", "debug_fused_misplaced"]
 
 
 def _p(a):
@@ -278,11 +278,17 @@ class Partition:
             pass
 
 
-def slice_layout(A, nCU=256, sel=None, device=False):
+def debug_fused_misplaced(on):
+    """Sets (or clears) the word a misplaced workgroup of a one-launch product sets (mx_debug_fused_misplaced)."""
+    check(_lib.load().mx_debug_fused_misplaced(1 if on else 0))
+
+
+def slice_layout(A, nCU=256, sel=None, device=False, fused=False):
     """The layout of the column-slice kernel for matrix A as a dict of numpy arrays and sizes (see
     mx_slice_layout in include/matxtract_hip.h), built on the host, or with device=True on the GPU
     (mx_slice_layout_device: the same arrays).  `sel`: optional mask of the rows to include (host
-    route only)."""
+    route only).  fused=True: the layout of the one-launch form (mx_slice_layout_fused; out["fused"]
+    tells whether the matrix suited it)."""
     v = _lib.SliceLayoutView()
     st = A.struct()
     selp = None
@@ -290,7 +296,10 @@ def slice_layout(A, nCU=256, sel=None, device=False):
         sel = np.ascontiguousarray(sel, dtype=np.uint8)
         assert sel.shape == (A.rows,) and not device
         selp = sel.ctypes.data
-    if device:
+    if fused:
+        assert sel is None and not device
+        check(_lib.load().mx_slice_layout_fused(C.byref(st), int(nCU), C.byref(v)))
+    elif device:
         check(_lib.load().mx_slice_layout_device(C.byref(st), int(nCU), C.byref(v)))
     else:
         check(_lib.load().mx_slice_layout(C.byref(st), int(nCU), selp, C.byref(v)))
@@ -311,6 +320,14 @@ def slice_layout(A, nCU=256, sel=None, device=False):
         out["nDict"] = int(v.nDict)
         out["ecode"] = _view(v.ecode, v.nEcol if v.nDict else 0, np.uint8).copy()
         out["dict"] = _view(v.dict, 256 if v.nDict else 0, vt).copy()
+        out["fused"] = int(v.fused)
+        if v.fused:
+            for n in ("groupRows", "nGroups", "placesPerRow"):
+                out[n] = int(getattr(v, n))
+            out["wgGroups"] = _view(v.wgGroups, v.nWG * 2, np.int32).reshape(-1, 2).copy()
+            out["groupNeed"] = _view(v.groupNeed, v.nGroups, np.int32).copy()
+            out["fusedTarget"] = _view(v.fusedTarget, v.chunks * 64, np.int32).copy()
+            out["rowVrows"] = _view(v.rowVrows, v.nGroups * v.groupRows, np.uint8).copy()
     finally:
         _lib.load().mx_slice_layout_free(C.byref(v))
     return out

@@ -126,7 +126,34 @@ struct DeviceSlices {
     int lightQuads = 2;               // 1 when no light row has more than four virtual rows
     int *heavyInfo = nullptr;         // [nHeavy][4]
     int nLight = 0, nHeavy = 0;
+    // The one-launch form (csr_slice_kernel<.., FUSED>), when the layout was made for it: the rows are cut
+    // into groups of kFusedGroupRows, the groups into one contiguous range per XCD, and the virtual rows
+    // of a slice are ordered by group before length, so that a workgroup's chunks cover a contiguous run
+    // of groups.  Logical workgroups [k * nWG / 8, (k + 1) * nWG / 8) belong to XCD k, and a workgroup of
+    // the launch that runs on XCD k takes one of those (which one: blockIdx / 8), so all workgroups that
+    // hold sums of a group share an L2: they store their sums with plain stores, which meet there,
+    // count themselves off on the group's counter with an atomic that executes there, and the one that
+    // completes the count adds the sums of the group's rows up and writes y.  Nobody waits.  The sums do
+    // not go to `partial` in this form but to fusedSums, laid out for the one who adds: the k-th
+    // virtual row of row r at [((r / G) * placesPerRow + k) * G + r % G], G = kFusedGroupRows, so that a
+    // wave that adds 64 consecutive rows reads 64 consecutive sums per place and needs no index list;
+    // fusedTarget names that place for every virtual row (a workgroup keeps its chunks' part of it in
+    // LDS, which bounds the chunks a workgroup may have), rowVrows[r] says how many places of row r hold
+    // a sum.  The arrays above stay valid for the two-launch form, which a plan falls back to.
+    bool fused = false;
+    int nGroups = 0, maxWgGroups = 0;
+    int placesPerRow = 0;             // 4 or 8: most virtual rows of a row
+    int *wgGroups = nullptr;          // [nWG][2] {first group, groups} whose counters the workgroup bumps
+    int *groupNeed = nullptr;         // [nGroups] workgroups that bump the group's counter
+    int *groupCount = nullptr;        // [nGroups] the counters; zero between launches (the last arriver clears its own)
+    int *fusedTarget = nullptr;       // [chunks * 64] where virtual row 64 * chunk + lane puts its sum (a spare place for padding lanes)
+    unsigned char *rowVrows = nullptr;// [nGroups * G] virtual rows of every row
+    void *fusedSums = nullptr;        // [nGroups * placesPerRow * G + 64] accumulators
+    unsigned *claim = nullptr;        // [nWG] launches in which each logical workgroup's work was taken (once each)
 };
+constexpr int kFusedGroupRows = 256;  // rows whose sums one arriver adds up at a time
+constexpr int kFusedXcds = 8;         // L2 domains of the device the one-launch form is laid out for
+constexpr int kFusedWgChunks = 96;    // most chunks of a workgroup in that form (their targets, 256 bytes each, share the LDS with x)
 constexpr int kSliceBytes = 131072;   // the slice of x a workgroup keeps in LDS
 constexpr int kSliceLdsMax = 163840;  // LDS of a CU
 constexpr int kSliceWgChunks = 4096;  // most chunks a workgroup may have
@@ -161,6 +188,9 @@ struct SlicePlan {
     std::vector<int> wgDesc, waveDesc, chunkEnd;
     std::vector<int> chunkSlice, chunkFirst, chunkN, chunkSteps;
     std::vector<long long> chunkStep0;
+    // one-launch form only
+    int nGroups = 0, maxWgGroups = 0;
+    std::vector<int> wgGroups, groupNeed;
 };
 int plan_slice_chunks(mx_dtype dtype, int budget, int S, const std::vector<std::vector<SliceChunk>> &sliceChunks, SlicePlan &P);
 constexpr int kSlicePadSteps = 16;  // spare zero steps after the last of the streams
@@ -239,6 +269,18 @@ struct HybridDevice {
 // row which gets sums from both parts is rounded to the value type once.
 hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
                          int what = 0, const DeviceTiles *strips = nullptr, void *ywide = nullptr);
+// The one-launch form of the same product (P.fused).  `misplaced`: a word in host memory that the
+// device can write (one per process); a workgroup that finds itself on another XCD than the layout
+// assumes sets it, and the product of that launch cannot be trusted.
+// `seq`: how many one-launch products of this layout were queued before this one (the kernel holds
+// the claims of its logical workgroups against it).
+hipError_t launch_fused(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
+                        void *ywide, unsigned *misplaced, unsigned seq);
+// Whether the workgroups of a launch of `nWG` workgroups shaped like the one-launch form's take every
+// logical workgroup (XCC_ID, blockIdx / 8) exactly once on the current device (asked once per device
+// and grid size, by launching a probe that reads the XCC_ID register); *ok = 0 when not -- a device
+// without eight XCDs, or a dispatcher that does not deal workgroups round-robin.
+hipError_t fused_placement_ok(int nWG, int *ok);
 bool strips_can_ride(mx_dtype dtype, const DeviceTiles &T, const void *x);
 hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y, int accumulate, hipStream_t s,
                       void *ywide = nullptr);

@@ -15,9 +15,11 @@
 // same stream and adds its rows on top with a plain read-modify-write.
 #include <hip/hip_runtime.h>
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include "mx_device.h"
 
@@ -540,9 +542,63 @@ static_assert(mx::kSliceBatchEntries == 8, "SliceBatch holds 8 entries per lane"
 // every consumed batch is reloaded with the batch one ring length ahead.
 constexpr int kSliceRing = 6;
 
+// What the one-launch form hands the kernel beyond the arguments of the slice kernel.
+struct FusedArgs {
+    void *y = nullptr;               // [rows] of the value type
+    void *ywide = nullptr;           // optional accumulators, one per row
+    const int *wgGroups = nullptr;   // [workgroups][2]
+    const int *groupNeed = nullptr;  // [groups]
+    int *groupCount = nullptr;       // [groups]
+    const int *target = nullptr;     // [chunks * 64] where every virtual row puts its sum
+    const unsigned char *rowVrows = nullptr;  // [rows rounded up to whole groups] virtual rows of every row
+    void *sums = nullptr;            // the sums, laid out for the one who adds
+    unsigned *misplaced = nullptr;   // host memory: set when two workgroups of a launch took the same work
+    unsigned *claim = nullptr;       // [workgroups] how often each logical workgroup's work has been taken
+    unsigned seq = 0;                // launches of this layout before this one
+    int rows = 0, placesPerRow = 4, accumulate = 0;
+    int debugSkip = 0;               // measurements only: end the kernel early (bits 1, 2, 4: after the stream, the drain, the counters)
+};
+
+// The XCD this wave runs on (XCC_ID, bits 3:0 of hardware register 20).
+__device__ __forceinline__ int xcc_id() { return (int)(__builtin_amdgcn_s_getreg(20 | (3 << 11)) & 15u); }
+
+// The largest v of the wave's 64 lanes, in every lane (as a scalar).
+__device__ __forceinline__ int wave_max(int v)
+{
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_ds_swizzle(v, 0x401F));
+    return max(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 32));
+}
+
+// A load that is served by the L2 and never by this CU's L1 (sc0): what another workgroup on the
+// same XCD stored before it counted itself off is in that L2.
+template <typename T>
+__device__ __forceinline__ T load_from_l2(const T *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
 // DICT: `eval` points at one byte per entry (same places as the column offsets) and `dictG` at the
 // 256 values they name; a workgroup keeps those in LDS behind the chunk ends.
-template <typename VT, bool DICT = false>
+// FUSED: the one-launch form.  The layout gives every XCD the same number of logical workgroups
+// and puts all of them that hold sums of a group of kFusedGroupRows rows on one XCD (DeviceSlices).
+// A workgroup takes its work by where it runs: logical workgroup (XCC_ID, blockIdx / 8) -- the
+// dispatcher deals consecutive workgroups round-robin to the XCDs, from a starting XCD that depends
+// on what ran before, so the workgroups that land on one XCD have distinct blockIdx / 8 and every
+// logical workgroup is taken once.  That one assumption is checked in every launch: each logical
+// workgroup's `claim` is counted up by whoever takes it, and a count that is not the launch's
+// number means that two took the same; the launch's y cannot be trusted then and the host is told.
+// The sums are stored where the one who adds finds them without an index list (DeviceSlices::fusedSums;
+// a workgroup keeps the places of its own virtual rows in LDS).  After its stream a workgroup waits until its own
+// stores have reached the L2 (s_waitcnt vmcnt(0): a store counts as done when the L2 has it),
+// adds one to the counter of each of its groups with an atomic that executes in that L2, and for
+// every group whose count it completes adds the sums of the group's rows up -- in the order of the
+// row's places, whoever does it, so y does not depend on who came last -- and writes y.  It clears
+// the counter for the next launch.  No workgroup ever waits for another.
+template <typename VT, bool DICT = false, bool FUSED = false>
 __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__restrict__ wgDesc,
                                                                   const int4 *__restrict__ waveDesc,
                                                                   const int *__restrict__ chunkEnd,
@@ -550,7 +606,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
                                                                   const VT *__restrict__ eval, const VT *__restrict__ x,
                                                                   typename Acc<VT>::type *__restrict__ partial, int cols,
                                                                   int sliceCols, const VT *__restrict__ dictG,
-                                                                  int maxWgChunks)
+                                                                  int maxWgChunks, FusedArgs fa)
 {
     typedef typename Acc<VT>::type AT;
     typedef typename std::conditional<DICT, SliceBatchDict<VT>, SliceBatch<VT>>::type Batch;
@@ -562,17 +618,28 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     VT *xs = (VT *)smem;                                           // [sliceCols]
     int *endsL = (int *)(smem + (size_t)sliceCols * sizeof(VT));   // [chunks of the workgroup]
     AT *dictL = (AT *)(endsL + ((maxWgChunks + 3) & ~3));            // [256] with DICT
+    int *targetL = (int *)(dictL + (DICT ? 256 : 0));                // [chunks of the workgroup][64] with FUSED
     if constexpr (DICT) {
         if (threadIdx.x < 256) dictL[threadIdx.x] = (AT)dictG[threadIdx.x];  // visible after the barrier below
     }
 
     // the workgroups of a slice are numbered consecutively: with every XCD on one contiguous range
     // of them a slice of x is fetched into one L2, not into all eight
-    const int b = xcd_contiguous_block(blockIdx.x, gridDim.x), tid = threadIdx.x, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int b = FUSED ? min(xcc_id(), mx::kFusedXcds - 1) * ((int)gridDim.x / mx::kFusedXcds) + (int)blockIdx.x / mx::kFusedXcds
+                        : xcd_contiguous_block(blockIdx.x, gridDim.x);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int4 gd = wgDesc[b];
     const int4 d = waveDesc[b * kSliceWaves + wave];
     const int slice = gd.x, wgChunk0 = gd.y, wgChunks = gd.z;
+    int group0 = 0, nGroupsMine = 0;
+    unsigned claimed = 0;
+    if constexpr (FUSED) {
+        group0 = fa.wgGroups[2 * b];
+        nGroupsMine = fa.wgGroups[2 * b + 1];
+        // (looked at when the work is done: the answer is not waited for here)
+        if (tid == 0) claimed = __hip_atomic_fetch_add(fa.claim + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     const int batch0 = __builtin_amdgcn_readfirstlane(d.x), nb = __builtin_amdgcn_readfirstlane(d.y);
     const int chunk0 = __builtin_amdgcn_readfirstlane(d.z), nChunks = __builtin_amdgcn_readfirstlane(d.w);
     // Every load below is unconditional -- indices are clamped instead, and what a clamped load
@@ -583,7 +650,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     // chunk ends of the workgroup, and the slice (all of it at once, one 16-byte vector per
     // lane and round).  The last vector of x may be partial: it is read whole (an aligned 16-byte
     // read cannot leave the page its first byte is on) and the elements beyond x are zeroed.
-    const int ce = chunkEnd[wgChunk0 + min(tid, wgChunks - 1)];
+    const int ce = chunkEnd[wgChunk0 + max(min(tid, wgChunks - 1), 0)];
     constexpr int CB = kSliceBytes / 16 / kSliceThreads;  // rounds of a full slice
     const int lastVec = (cols + EPV - 1) / EPV - 1;
     v4i32 xv[CB];
@@ -598,7 +665,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     const int lastBatch = batch0 + max(nb - 1, 0);
 #pragma unroll
     for (int k = 0; k < NB; ++k) buf[k].load(ecol, estream, (size_t)min(batch0 + k, lastBatch), lane);
-    endsL[min(tid, wgChunks - 1)] = ce;
+    endsL[max(min(tid, wgChunks - 1), 0)] = ce;
     if ((slice + 1) * sliceCols <= cols) {  // the whole slice lies inside x
 #pragma unroll
         for (int q = 0; q < CB; ++q) *(v4i32 *)(xs + (tid + q * kSliceThreads) * EPV) = xv[q];
@@ -617,13 +684,17 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         }
     }
     for (int i = kSliceThreads + tid; i < wgChunks; i += kSliceThreads) endsL[i] = chunkEnd[wgChunk0 + i];
+    if constexpr (FUSED) {
+        for (int i = tid; i < wgChunks * 64; i += kSliceThreads) targetL[i] = fa.target[(size_t)wgChunk0 * 64 + i];
+    }
     __syncthreads();
     // (the chunk ends are the same for all lanes of the wave: kept in scalar registers)
     int ci = 0, nextEnd = nChunks > 0 ? __builtin_amdgcn_readfirstlane(endsL[chunk0]) : -1;
     AT acc = 0;
     AT *out = partial + (size_t)(wgChunk0 + chunk0) * 64 + lane;
     auto flush = [&]() {
-        out[(size_t)ci * 64] = acc;
+        if constexpr (FUSED) ((AT *)fa.sums)[targetL[(chunk0 + ci) * 64 + lane]] = acc;
+        else out[(size_t)ci * 64] = acc;
         acc = 0;
         ++ci;
         nextEnd = ci < nChunks ? __builtin_amdgcn_readfirstlane(endsL[chunk0 + ci]) : -1;
@@ -640,27 +711,121 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 #pragma unroll
         for (int k = 0; k < NB; ++k)
             if (k < nb) consume(buf[k], k);
-        return;
-    }
-    int t = 0;
-    // while a whole ring beyond the one in flight remains: consume and reload
-    for (; t + 2 * NB <= nb; t += NB) {
+    } else {
+        int t = 0;
+        // while a whole ring beyond the one in flight remains: consume and reload
+        for (; t + 2 * NB <= nb; t += NB) {
+#pragma unroll
+            for (int k = 0; k < NB; ++k) {
+                consume(buf[k], t + k);
+                buf[k].load(ecol, estream, (size_t)(batch0 + t + NB + k), lane);
+            }
+        }
+        // one ring in flight and less than one more to come: consume and reload while batches
+        // remain (the last one again after that), then those
 #pragma unroll
         for (int k = 0; k < NB; ++k) {
             consume(buf[k], t + k);
-            buf[k].load(ecol, estream, (size_t)(batch0 + t + NB + k), lane);
+            buf[k].load(ecol, estream, (size_t)min(batch0 + t + NB + k, lastBatch), lane);
+        }
+#pragma unroll
+        for (int k = 0; k < NB; ++k)
+            if (t + NB + k < nb) consume(buf[k], t + NB + k);
+    }
+    if constexpr (FUSED) {
+        constexpr int GR = mx::kFusedGroupRows, R = 8;           // R rows per lane and pass
+        constexpr int GP = R * kSliceThreads / GR;                 // groups per pass
+        static_assert(kSliceThreads % GR == 0 && GR == 256, "a lane keeps its place inside the group from pass to pass");
+        if (tid == 0 && (claimed != fa.seq || xcc_id() >= mx::kFusedXcds))
+            __hip_atomic_store(fa.misplaced, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        if (fa.debugSkip & 1) return;
+        const bool wide8 = fa.placesPerRow == 8;
+        const AT *sums = (const AT *)fa.sums;
+        VT *y = (VT *)fa.y;
+        AT *ywide = (AT *)fa.ywide;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's sums are in the L2
+        __syncthreads();                                    // ... and so are the other waves'
+        if (fa.debugSkip & 2) return;
+        // (the chunk ends are done with) listL[0] = how many groups fall to this workgroup, then which
+        int *listL = endsL;
+        if (tid == 0) listL[0] = 0;
+        __syncthreads();
+        for (int i = tid; i < nGroupsMine; i += kSliceThreads) {
+            const int g = group0 + i;
+            const int old = __hip_atomic_fetch_add(fa.groupCount + g, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (old + 1 == fa.groupNeed[g]) {
+                __hip_atomic_store(fa.groupCount + g, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                listL[1 + atomicAdd(&listL[0], 1)] = g;
+            }
+        }
+        __syncthreads();
+        if (fa.debugSkip & 4) return;
+        // A pass: R groups per half of the workgroup, a row per lane and group.  A wave's 64 rows are
+        // consecutive, so every load is one contiguous stretch; the places a row does not use hold
+        // nothing that counts (rowVrows says how many do).
+        const int nl = listL[0], half = tid >> 8, rl = tid & (GR - 1);
+        for (int j0 = 0; j0 < nl; j0 += GP) {
+            int nv[R];
+            AT old[R];
+            bool live[R], take[R];  // take: the slot holds a group (the same for the whole wave)
+            size_t base[R];
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                const int li = j0 + half + (kSliceThreads / GR) * i;
+                const int g = listL[1 + min(li, nl - 1)];
+                const int r = g * GR + rl;
+                take[i] = __builtin_amdgcn_readfirstlane((int)(li < nl)) != 0;
+                live[i] = take[i] && r < fa.rows;
+                nv[i] = fa.rowVrows[r];
+                base[i] = (size_t)g * (wide8 ? 8 : 4) * GR + rl;
+                old[i] = fa.accumulate && live[i] ? (AT)y[r] : (AT)0;
+            }
+            if (wide8) {
+                AT v[R][8];
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) v[i][k] = 0;
+                    if (take[i]) {
+                        // (places beyond the most any of the wave's 64 rows uses are not asked for)
+                        const int most = wave_max(nv[i]);
+#pragma unroll
+                        for (int k = 0; k < 8; ++k)
+                            if (k < most) v[i][k] = load_from_l2(sums + base[i] + (size_t)k * GR);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    AT sum = old[i];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) sum += k < nv[i] ? v[i][k] : (AT)0;  // (in the order of the places: y does not depend on who adds)
+                    const int r = listL[1 + min(j0 + half + (kSliceThreads / GR) * i, nl - 1)] * GR + rl;
+                    if (live[i]) y[r] = (VT)sum;
+                    if (live[i] && ywide) ywide[r] = sum;
+                }
+            } else {
+                AT v[R][4];
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) v[i][k] = 0;
+                    if (take[i]) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) v[i][k] = load_from_l2(sums + base[i] + (size_t)k * GR);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    AT sum = old[i];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) sum += k < nv[i] ? v[i][k] : (AT)0;
+                    const int r = listL[1 + min(j0 + half + (kSliceThreads / GR) * i, nl - 1)] * GR + rl;
+                    if (live[i]) y[r] = (VT)sum;
+                    if (live[i] && ywide) ywide[r] = sum;
+                }
+            }
         }
     }
-    // one ring in flight and less than one more to come: consume and reload while batches
-    // remain (the last one again after that), then those
-#pragma unroll
-    for (int k = 0; k < NB; ++k) {
-        consume(buf[k], t + k);
-        buf[k].load(ecol, estream, (size_t)min(batch0 + t + NB + k, lastBatch), lane);
-    }
-#pragma unroll
-    for (int k = 0; k < NB; ++k)
-        if (t + NB + k < nb) consume(buf[k], t + NB + k);
 }
 
 // ---- tile part --------------------------------------------------------------------------
@@ -1152,6 +1317,19 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
     }
 }
 
+// Which logical workgroup each workgroup of a launch shaped like the one-launch form's would take
+// (XCC_ID, blockIdx / 8): every one of them exactly once when the dispatcher deals the workgroups
+// round-robin to eight XCDs.
+__global__ __launch_bounds__(kSliceThreads) void xcc_probe_kernel(unsigned *taken, int rep)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    if (threadIdx.x == 0) {
+        smem[0] = (unsigned char)rep;  // (the LDS is asked for so that one workgroup fills a CU, as in the real launch)
+        const int xcc = xcc_id();
+        if (xcc < mx::kFusedXcds) atomicAdd(taken + xcc * ((int)gridDim.x / mx::kFusedXcds) + (int)blockIdx.x / mx::kFusedXcds, 1u);
+    }
+}
+
 // MFMA probes: one wave, operands and accumulators exchanged lane by lane (raw register
 // contents), so a host test can check the operand layout the tile kernels rely on.
 __global__ void probe_mfma_f64_kernel(const double *A /*[64]*/, const double *B /*[64]*/, double *D /*[64][4]*/)
@@ -1247,6 +1425,29 @@ hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y
     return hipGetLastError();
 }
 
+// The slice kernels take more dynamic LDS than the default limit: raised once per device (a function
+// attribute belongs to the device that is current when it is set).
+template <typename VT>
+static hipError_t slice_kernel_attributes()
+{
+    static std::mutex attrLock;
+    static bool attrSet[kMaxDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> hold(attrLock);
+    if (attrSet[dev]) return hipSuccess;
+    const void *fn[4] = {(const void *)mxk::csr_slice_kernel<VT, false, false>, (const void *)mxk::csr_slice_kernel<VT, true, false>,
+                         (const void *)mxk::csr_slice_kernel<VT, false, true>, (const void *)mxk::csr_slice_kernel<VT, true, true>};
+    for (const void *f : fn) {
+        e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
+        if (e != hipSuccess) return e;
+    }
+    attrSet[dev] = true;
+    return hipSuccess;
+}
+
 template <typename VT>
 static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, int what,
                                   const DeviceTiles *strips, void *ywide)
@@ -1254,24 +1455,9 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     typedef typename mxk::Acc<VT>::type AT;
     const bool dict = P.useDict && P.ecode && P.dict;
     const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)((P.maxWgChunks + 3) & ~3) * 4 + 64 + (dict ? 256 * sizeof(AT) : 0);
-    // (a function attribute belongs to the device that is current when it is set: once per device)
     {
-        static std::mutex attrLock;
-        static bool attrSet[kMaxDevices] = {};
-        int dev = 0;
-        hipError_t e = hipGetDevice(&dev);
+        const hipError_t e = slice_kernel_attributes<VT>();
         if (e != hipSuccess) return e;
-        if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
-        std::lock_guard<std::mutex> hold(attrLock);
-        if (!attrSet[dev]) {
-            e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT, false>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
-            if (e == hipSuccess)
-                e = hipFuncSetAttribute((const void *)mxk::csr_slice_kernel<VT, true>,
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
-            if (e != hipSuccess) return e;
-            attrSet[dev] = true;
-        }
     }
     if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16))
         return hipErrorInvalidValue;
@@ -1279,11 +1465,11 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
         if (dict)
             hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, true>), dim3(P.nWG), dim3(kSliceThreads), lds, s,
                                (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.ecode,
-                               (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols, (const VT *)P.dict, P.maxWgChunks);
+                               (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols, (const VT *)P.dict, P.maxWgChunks, mxk::FusedArgs());
         else
             hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, false>), dim3(P.nWG), dim3(kSliceThreads), lds, s,
                                (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.eval,
-                               (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols, (const VT *)nullptr, P.maxWgChunks);
+                               (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols, (const VT *)nullptr, P.maxWgChunks, mxk::FusedArgs());
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || what == 1) return e;
@@ -1317,6 +1503,105 @@ hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, v
 bool strips_can_ride(mx_dtype dtype, const DeviceTiles &T, const void *x)
 {
     return dtype == MX_F16 && T.nWaves > 0 && T.dense && T.ownedRows && !((uintptr_t)x & 15);
+}
+
+template <typename VT>
+static hipError_t launch_fused_t(const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, void *ywide,
+                                 unsigned *misplaced, unsigned seq)
+{
+    typedef typename mxk::Acc<VT>::type AT;
+    const bool dict = P.useDict && P.ecode && P.dict;
+    // (the list of the groups that fall to a workgroup takes the place of its chunk ends; behind them the places of
+    // the sums of the workgroup's chunks)
+    const int ldsInts = std::max(P.maxWgChunks, P.maxWgGroups + 1);
+    const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)((ldsInts + 3) & ~3) * 4 + 64 + (dict ? 256 * sizeof(AT) : 0) +
+                       (size_t)P.maxWgChunks * 256;
+    const hipError_t e = slice_kernel_attributes<VT>();
+    if (e != hipSuccess) return e;
+    if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16) || !P.fused || !P.wgGroups ||
+        !P.groupNeed || !P.groupCount || !P.fusedTarget || !P.rowVrows || !P.fusedSums || !P.claim || !misplaced || (P.placesPerRow != 4 && P.placesPerRow != 8) ||
+        P.nWG <= 0 || P.nWG % mx::kFusedXcds)
+        return hipErrorInvalidValue;
+    mxk::FusedArgs fa;
+    fa.y = y;
+    fa.ywide = ywide;
+    fa.wgGroups = P.wgGroups;
+    fa.groupNeed = P.groupNeed;
+    fa.groupCount = P.groupCount;
+    fa.target = P.fusedTarget;
+    fa.rowVrows = P.rowVrows;
+    fa.sums = P.fusedSums;
+    fa.misplaced = misplaced;
+    fa.claim = P.claim;
+    fa.seq = seq;
+    fa.rows = P.rows;
+    fa.placesPerRow = P.placesPerRow;
+    fa.accumulate = accumulate;
+    {
+        // (for measurements: 1, 2, 4 end the kernel after the stream, the drain, the counters)
+        static const int skip = std::getenv("MX_FUSED_SKIP") ? std::atoi(std::getenv("MX_FUSED_SKIP")) : 0;
+        fa.debugSkip = skip;
+    }
+    if (dict)
+        hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, true, true>), dim3(P.nWG), dim3(kSliceThreads), lds, s, (const int4 *)P.wgDesc,
+                           (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.ecode, (const VT *)x, (AT *)P.partial, P.cols,
+                           P.sliceCols, (const VT *)P.dict, ldsInts, fa);
+    else
+        hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, false, true>), dim3(P.nWG), dim3(kSliceThreads), lds, s, (const int4 *)P.wgDesc,
+                           (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.eval, (const VT *)x, (AT *)P.partial, P.cols,
+                           P.sliceCols, (const VT *)nullptr, ldsInts, fa);
+    return hipGetLastError();
+}
+hipError_t launch_fused(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, void *ywide,
+                        unsigned *misplaced, unsigned seq)
+{
+    if (P.rows <= 0) return hipSuccess;
+    if (dtype == MX_F64) return launch_fused_t<double>(P, x, y, accumulate, s, ywide, misplaced, seq);
+    return launch_fused_t<_Float16>(P, x, y, accumulate, s, ywide, misplaced, seq);
+}
+
+hipError_t fused_placement_ok(int nWG, int *ok)
+{
+    static std::mutex lock;
+    static int known[kMaxDevices] = {}, knownGrid[kMaxDevices] = {};  // 1 = holds, 2 = does not
+    *ok = 0;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices || nWG < 8) return hipSuccess;
+    std::lock_guard<std::mutex> hold(lock);
+    if (known[dev] && knownGrid[dev] == nWG) {
+        *ok = known[dev] == 1;
+        return hipSuccess;
+    }
+    e = hipFuncSetAttribute((const void *)mxk::xcc_probe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
+    if (e != hipSuccess) return e;
+    unsigned *taken = nullptr;
+    e = hipMalloc((void **)&taken, (size_t)nWG * 4);
+    if (e != hipSuccess) return e;
+    std::vector<unsigned> h((size_t)nWG);
+    bool holds = nWG % mx::kFusedXcds == 0;
+    e = hipMemset(taken, 0, (size_t)nWG * 4);
+    // (a few launches in a row, the way products follow each other, with a launch of another size between them)
+    const int reps = 4;
+    for (int rep = 0; rep < reps && e == hipSuccess && holds; ++rep) {
+        hipLaunchKernelGGL(mxk::xcc_probe_kernel, dim3(nWG), dim3(kSliceThreads), mx::kSliceBytes + 2048, nullptr, taken, rep);
+        e = hipGetLastError();
+        if (e == hipSuccess) e = hipMemsetAsync(taken + nWG - 1, 0, 0, nullptr);
+    }
+    if (e == hipSuccess) e = hipMemcpy(h.data(), taken, (size_t)nWG * 4, hipMemcpyDeviceToHost);
+    (void)hipFree(taken);
+    if (e != hipSuccess) return e;
+    for (int b = 0; b < nWG; ++b) holds = holds && h[b] == (unsigned)reps;
+    if (std::getenv("MX_FUSED_DEBUG")) {
+        fprintf(stderr, "fused_placement_ok: nWG %d holds %d; first slots:", nWG, (int)holds);
+        for (int b = 0; b < std::min(nWG, 24); ++b) fprintf(stderr, " %u", h[b]);
+        fprintf(stderr, "\n");
+    }
+    known[dev] = holds ? 1 : 2;
+    knownGrid[dev] = nWG;
+    *ok = holds;
+    return hipSuccess;
 }
 
 hipError_t launch_tiles(mx_dtype dtype, const DeviceTiles &T, const void *x, void *y, int accumulate, hipStream_t s,

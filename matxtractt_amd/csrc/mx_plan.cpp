@@ -1,6 +1,8 @@
 // Device plans: persistent device copies of a partition and the launch sequence of one
 // hybrid SpMV; plus the reference's one-shot host-pointer entry points built on top.
 #include <algorithm>
+#include <mutex>
+#include <atomic>
 #include <chrono>
 #include <climits>
 #include <cstdlib>
@@ -114,6 +116,13 @@ void free_slices(mx::DeviceSlices &P)
     (void)hipFree(P.lightIdx);
     (void)hipFree(P.heavyInfo);
     (void)hipFree(P.segIdx);
+    (void)hipFree(P.wgGroups);
+    (void)hipFree(P.groupNeed);
+    (void)hipFree(P.groupCount);
+    (void)hipFree(P.fusedTarget);
+    (void)hipFree(P.rowVrows);
+    (void)hipFree(P.fusedSums);
+    (void)hipFree(P.claim);
     P = mx::DeviceSlices();
 }
 
@@ -182,14 +191,292 @@ struct HostSlices {
     std::vector<unsigned char> eval;
     std::vector<unsigned char> ecode, dict;  // value dictionary form (empty when the rows hold more than 256 values)
     int nDict = 0;
+    // one-launch form (see DeviceSlices): set when it was asked for and the matrix suits it
+    bool fused = false;
+    int nGroups = 0, maxWgGroups = 0, placesPerRow = 0;
+    std::vector<int> wgGroups, groupNeed, fusedTarget;
+    std::vector<unsigned char> rowVrows;
 };
+
+// A workgroup of the slice layout on its way into the descriptors: its slice and, per wave, the
+// chunks (indices into the slice's list) in the order the wave streams them.
+struct SliceWg {
+    int slice = 0;
+    std::vector<int> chunk[mx::kSliceWaves];
+    int waveSteps[mx::kSliceWaves] = {};
+    long long steps = 0;  // stored steps (every wave's stream rounded up to whole batches)
+    int chunks = 0;
+};
+
+// `mine` (chunks of slice q, in the order they are to be dealt) to the waves of `w`: each to the wave
+// with the fewest steps so far.
+void deal_to_waves(SliceWg &w, int q, const std::vector<int> &mine, const std::vector<mx::SliceChunk> &ch, int SPB)
+{
+    const int W = mx::kSliceWaves;
+    w.slice = q;
+    w.steps = 0;
+    for (int k = 0; k < W; ++k) {
+        w.waveSteps[k] = 0;
+        w.chunk[k].clear();
+    }
+    for (int c : mine) {
+        int best = 0;
+        for (int k = 1; k < W; ++k)
+            if (w.waveSteps[k] < w.waveSteps[best]) best = k;
+        w.chunk[best].push_back(c);
+        w.waveSteps[best] += ch[c].steps;
+    }
+    w.chunks = (int)mine.size();
+    for (int k = 0; k < W; ++k) w.steps += (w.waveSteps[k] + SPB - 1) / SPB * SPB;
+}
+
+// The descriptors the kernels read and the place of every chunk in the streams, from the workgroups
+// and their waves' chunks.
+int emit_slice_plan(const std::vector<SliceWg> &wgs, const std::vector<std::vector<mx::SliceChunk>> &sliceChunks, int SPB, int E,
+                           mx::SlicePlan &P)
+{
+    const int W = mx::kSliceWaves;
+    const int nWG = (int)wgs.size();
+    long long totalSteps = 0, totalChunks = 0;
+    std::vector<long long> wgStep((size_t)nWG + 1, 0), wgChunk((size_t)nWG + 1, 0);
+    int maxWgChunks = 0;
+    for (int b = 0; b < nWG; ++b) {
+        wgStep[b] = totalSteps;
+        wgChunk[b] = totalChunks;
+        totalSteps += wgs[b].steps;
+        totalChunks += wgs[b].chunks;
+        maxWgChunks = std::max(maxWgChunks, wgs[b].chunks);
+    }
+    if (totalSteps * 64 * E > 2000000000LL || totalChunks * 64 > 2000000000LL) {
+        set_error("slice layout: too many entries for 32-bit offsets");
+        return MX_ERR_ARG;
+    }
+    P.nWG = nWG;
+    P.maxWgChunks = maxWgChunks;
+    P.totalSteps = totalSteps;
+    P.totalChunks = totalChunks;
+    P.wgDesc.assign((size_t)nWG * 4 + 4, 0);
+    P.waveDesc.assign((size_t)nWG * W * 4 + 4, 0);
+    P.chunkEnd.assign((size_t)totalChunks + 64, 0);
+    P.chunkSlice.assign((size_t)totalChunks, 0);
+    P.chunkFirst.assign((size_t)totalChunks, 0);
+    P.chunkN.assign((size_t)totalChunks, 0);
+    P.chunkSteps.assign((size_t)totalChunks, 0);
+    P.chunkStep0.assign((size_t)totalChunks, 0);
+    for (int b = 0; b < nWG; ++b) {
+        const SliceWg &G = wgs[b];
+        const int q = G.slice;
+        const auto &ch = sliceChunks[q];
+        long long step = wgStep[b], chunk = wgChunk[b];
+        P.wgDesc[(size_t)b * 4 + 0] = q;
+        P.wgDesc[(size_t)b * 4 + 1] = (int)chunk;
+        P.wgDesc[(size_t)b * 4 + 2] = G.chunks;
+        for (int w = 0; w < W; ++w) {
+            int *d = &P.waveDesc[((size_t)b * W + w) * 4];
+            d[0] = (int)(step / SPB);                   // first batch
+            d[1] = (G.waveSteps[w] + SPB - 1) / SPB;    // batches
+            d[2] = (int)(chunk - wgChunk[b]);           // first chunk, counted inside the workgroup
+            d[3] = (int)G.chunk[w].size();
+            int rel = 0;
+            for (int c : G.chunk[w]) {
+                P.chunkSlice[chunk] = q;
+                P.chunkFirst[chunk] = ch[c].first;
+                P.chunkN[chunk] = ch[c].n;
+                P.chunkSteps[chunk] = ch[c].steps;
+                P.chunkStep0[chunk] = step;
+                step += ch[c].steps;
+                rel += ch[c].steps;
+                P.chunkEnd[chunk++] = rel;
+            }
+            step = (step + SPB - 1) / SPB * SPB;
+        }
+    }
+    return MX_OK;
+}
+
+// A virtual row on its way into the slice layout.
+struct VRow {
+    int start, len, slice;  // start: into the entries in (row, column) order
+    int kind;               // of its row: 0 = this is its only virtual row, 1 = light, 2 = heavy
+};
+
+// The decisions of the one-launch form (see DeviceSlices).  Every XCD gets a contiguous range of whole
+// groups of rows with an eighth of the entries, and budget / 8 logical workgroups; a slice with
+// entries in those rows gets workgroups in proportion to its entries there, and each of them a
+// contiguous run of the slice's virtual rows (in row order) with an even share of the entries.  A
+// workgroup's virtual rows are then ordered by length and cut into chunks of 64, which go to its waves
+// longest first.  The groups a workgroup counts off are those of its rows, stretched so that the
+// workgroups of one (XCD, slice) cover all groups of the XCD between them: every group is counted off by
+// at least one workgroup, also one whose rows have no entries.  Fills `sorted`, `sliceChunks` and SP and
+// returns true; false (nothing filled) when the matrix does not suit the form: a budget that is not a
+// multiple of eight, fewer workgroups per XCD than slices with entries in its rows, an XCD without
+// entries.  (SP.nWG = -1: an error, which is set.)
+static bool plan_fused(mx_dtype dtype, int budget, int S, int rows, int nGroups, int cap, const std::vector<int> &rowStart,
+                       const std::vector<int> &segPtr, const std::vector<VRow> &vr, std::vector<int> &sorted,
+                       std::vector<std::vector<mx::SliceChunk>> &sliceChunks, mx::SlicePlan &SP)
+{
+    const int E = mx::slice_step_entries(dtype), SPB = mx::kSliceBatchEntries / E, X = mx::kFusedXcds, GR = mx::kFusedGroupRows;
+    const int nV = (int)vr.size(), nk = budget / X;
+    const long long nnz = rowStart[rows];
+    if (budget < X || budget % X || nGroups < X || nnz == 0) return false;
+    // the groups of every XCD
+    std::vector<int> xg((size_t)X + 1, 0);
+    {
+        int g = 0;
+        for (int k = 1; k < X; ++k) {
+            const long long target = nnz * k / X;
+            while (g < nGroups && (long long)rowStart[std::min(rows, g * GR)] < target) ++g;
+            xg[k] = std::min(std::max(g, xg[k - 1] + 1), nGroups - (X - k));
+            g = xg[k];
+        }
+        xg[X] = nGroups;
+    }
+    std::vector<int> xcdOfGroup((size_t)nGroups);
+    for (int k = 0; k < X; ++k)
+        for (int g = xg[k]; g < xg[k + 1]; ++g) xcdOfGroup[g] = k;
+    std::vector<int> rowOf((size_t)nV);
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; ++r)
+        for (int t = segPtr[r]; t < segPtr[r + 1]; ++t) rowOf[t] = r;
+    // entries and virtual rows of every (XCD, slice)
+    std::vector<long long> partEntries((size_t)X * S, 0);
+    std::vector<int> partVrows((size_t)X * S, 0);
+    for (int t = 0; t < nV; ++t) {
+        const size_t p = (size_t)xcdOfGroup[rowOf[t] / GR] * S + vr[t].slice;
+        partEntries[p] += vr[t].len;
+        ++partVrows[p];
+    }
+    // workgroups of every part, and the first logical workgroup of each
+    std::vector<int> partWgs((size_t)X * S, 0), partBase((size_t)X * S, 0);
+    for (int k = 0; k < X; ++k) {
+        long long xcdEntries = 0;
+        int busy = 0;
+        for (int q = 0; q < S; ++q) {
+            xcdEntries += partEntries[(size_t)k * S + q];
+            busy += partVrows[(size_t)k * S + q] > 0;
+        }
+        if (busy == 0 || busy > nk) return false;
+        std::vector<double> want((size_t)S, 0.0);
+        int used = 0;
+        for (int q = 0; q < S; ++q) {
+            const size_t p = (size_t)k * S + q;
+            if (partVrows[p] == 0) continue;
+            want[q] = (double)partEntries[p] * nk / (double)xcdEntries;
+            partWgs[p] = std::min(std::max(1, (int)want[q]), partVrows[p]);
+            used += partWgs[p];
+        }
+        while (used > nk) {  // rounding small parts up took more than there is: from the part furthest above its share
+            int best = -1;
+            for (int q = 0; q < S; ++q) {
+                const size_t p = (size_t)k * S + q;
+                if (partWgs[p] > 1 && (best < 0 || partWgs[p] - want[q] > partWgs[(size_t)k * S + best] - want[best])) best = q;
+            }
+            if (best < 0) return false;
+            --partWgs[(size_t)k * S + best];
+            --used;
+        }
+        while (used < nk) {  // what rounding down left over goes where most is missing
+            int best = -1;
+            for (int q = 0; q < S; ++q) {
+                const size_t p = (size_t)k * S + q;
+                if (partVrows[p] > partWgs[p] && (best < 0 || want[q] - partWgs[p] > want[best] - partWgs[(size_t)k * S + best])) best = q;
+            }
+            if (best < 0) break;  // fewer virtual rows than workgroups: the rest stay empty
+            ++partWgs[(size_t)k * S + best];
+            ++used;
+        }
+        int b = k * nk;
+        for (int q = 0; q < S; ++q) {
+            partBase[(size_t)k * S + q] = b;
+            b += partWgs[(size_t)k * S + q];
+        }
+    }
+    // every virtual row to its workgroup: inside a part in row order, cut where the running entries pass
+    // the next share
+    std::vector<int> wgOf((size_t)nV), wgCount((size_t)budget + 1, 0), rowLo((size_t)budget, INT_MAX), rowHi((size_t)budget, -1);
+    {
+        std::vector<long long> run((size_t)X * S, 0);
+        std::vector<int> seen((size_t)X * S, 0);
+        for (int t = 0; t < nV; ++t) {
+            const size_t p = (size_t)xcdOfGroup[rowOf[t] / GR] * S + vr[t].slice;
+            const int w = partWgs[p];
+            // (at least one virtual row per workgroup: the j-th workgroup starts no later than at the part's
+            // (vrows - w + j)-th virtual row and no earlier than at its j-th)
+            int j = partEntries[p] > 0 ? (int)(((run[p] + vr[t].len / 2) * w) / partEntries[p]) : 0;
+            j = std::min(std::min(j, w - 1), seen[p]);
+            j = std::max(j, w - (partVrows[p] - seen[p]));
+            run[p] += vr[t].len;
+            ++seen[p];
+            const int b = partBase[p] + j;
+            wgOf[t] = b;
+            ++wgCount[b + 1];
+            rowLo[b] = std::min(rowLo[b], rowOf[t]);
+            rowHi[b] = std::max(rowHi[b], rowOf[t]);
+        }
+    }
+    // (wgOf rises with t inside a part, so j never skips a workgroup downwards; a skipped one upwards stays empty)
+    for (int b = 0; b < budget; ++b) wgCount[b + 1] += wgCount[b];
+    // virtual rows by (workgroup, length descending), row order kept among equals: two counting sorts
+    {
+        std::vector<int> byLen((size_t)nV), at((size_t)cap + 2, 0);
+        for (int t = 0; t < nV; ++t) at[(size_t)(cap - vr[t].len) + 1]++;
+        for (int k = 0; k <= cap; ++k) at[k + 1] += at[k];
+        for (int t = 0; t < nV; ++t) byLen[at[cap - vr[t].len]++] = t;
+        std::vector<int> cur(wgCount.begin(), wgCount.end() - 1);
+        for (int i = 0; i < nV; ++i) sorted[cur[wgOf[byLen[i]]]++] = byLen[i];
+    }
+    // chunks, waves, groups
+    std::vector<SliceWg> wgs((size_t)budget);
+    SP.wgGroups.assign((size_t)budget * 2 + 2, 0);
+    SP.groupNeed.assign((size_t)nGroups + 1, 0);
+    SP.nGroups = nGroups;
+    SP.maxWgGroups = 0;
+    for (int k = 0; k < X; ++k)
+        for (int q = 0; q < S; ++q) {
+            const size_t p = (size_t)k * S + q;
+            const int w = partWgs[p];
+            // the workgroups of the part that hold anything, in order
+            std::vector<int> live;
+            for (int j = 0; j < w; ++j)
+                if (wgCount[partBase[p] + j + 1] > wgCount[partBase[p] + j]) live.push_back(partBase[p] + j);
+            for (size_t i = 0; i < live.size(); ++i) {
+                const int b = live[i];
+                if ((wgCount[b + 1] - wgCount[b] + 63) / 64 > mx::kFusedWgChunks) return false;  // (its targets would not fit the LDS)
+                std::vector<int> mine;
+                for (int f = wgCount[b]; f < wgCount[b + 1]; f += 64) {
+                    mine.push_back((int)sliceChunks[q].size());
+                    sliceChunks[q].push_back({f, std::min(64, wgCount[b + 1] - f), (vr[sorted[f]].len + E - 1) / E});
+                }
+                deal_to_waves(wgs[b], q, mine, sliceChunks[q], SPB);
+                const int ga = i == 0 ? xg[k] : rowLo[b] / GR;
+                const int gb = i + 1 == live.size() ? xg[k + 1] - 1 : std::max(rowHi[b] / GR, rowLo[live[i + 1]] / GR - 1);
+                SP.wgGroups[(size_t)b * 2] = ga;
+                SP.wgGroups[(size_t)b * 2 + 1] = gb - ga + 1;
+                SP.maxWgGroups = std::max(SP.maxWgGroups, gb - ga + 1);
+                for (int g = ga; g <= gb; ++g) ++SP.groupNeed[g];
+            }
+        }
+    for (int b = 0; b < budget; ++b)
+        if (wgs[b].chunks == 0) {  // a workgroup without virtual rows: nothing to stream, no group to count off
+            int q = 0;
+            while (q < S - 1 && partVrows[(size_t)(b / nk) * S + q] == 0) ++q;
+            deal_to_waves(wgs[b], q, std::vector<int>(), sliceChunks[q], SPB);
+            SP.wgGroups[(size_t)b * 2] = xg[b / nk];
+        }
+    if (emit_slice_plan(wgs, sliceChunks, SPB, E, SP)) SP.nWG = -1;
+    return true;
+}
 
 // `elsewhere` (optional) marks rows whose result another kernel writes: 1 = the strips of a binary16
 // plan (the row has nothing here), 2 = the 8 x 8 blocks of a binary64 plan, whose waves fetch the sums
 // of the row's virtual rows themselves.  Such rows get rowInfo -2 and appear in no list, so that the
 // combine kernel's own kinds neither zero them nor add to them.
+// `fused`: lay the virtual rows out for the one-launch form (ordered by group of rows before length,
+// workgroups dealt per XCD); D.fused tells whether the matrix suited it -- when it does not (a row
+// with more than eight virtual rows, more slices than workgroups in an XCD's rows, row subsets or
+// rows written elsewhere) the ordinary layout is made.
 int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
-                 const char *sel, HostSlices &D, const char *elsewhere = nullptr)
+                 const char *sel, HostSlices &D, const char *elsewhere = nullptr, bool fused = false)
 {
     const int es = mx::elem_size(dtype), E = mx::slice_step_entries(dtype);
     const int BE = mx::kSliceBatchEntries;
@@ -231,10 +518,6 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     }
     for (int r = 0; r < rows; ++r) segPtr[r + 1] += segPtr[r];
     const int nV = segPtr[rows];
-    struct VRow {
-        int start, len, slice;  // start: into ord
-        int kind;               // of its row: 0 = this is its only virtual row, 1 = light, 2 = heavy
-    };
     std::vector<VRow> vr((size_t)nV);
 #pragma omp parallel for schedule(dynamic, 1024)
     for (int r = 0; r < rows; ++r) {
@@ -250,27 +533,44 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
             k = e;
         }
     }
-    // virtual rows by (slice, length descending, kind of row), row order kept among equals: a
-    // counting sort.  The kind keeps the sums that one workgroup of the combine kernel gathers
-    // close together: consecutive heavy rows have virtual rows of the same slice and length more
-    // often than a heavy row and its neighbours of other kinds do.
-    const size_t perSlice = (size_t)(cap + 1) * 3, nKeys = (size_t)S * perSlice;
-    std::vector<int> keyStart(nKeys + 1, 0), sorted((size_t)nV);
-    auto key_of = [&](const VRow &v) { return (size_t)v.slice * perSlice + (size_t)(cap - v.len) * 3 + (size_t)v.kind; };
-    for (int t = 0; t < nV; ++t) keyStart[key_of(vr[t]) + 1]++;
-    for (size_t k = 0; k < nKeys; ++k) keyStart[k + 1] += keyStart[k];
-    {
-        std::vector<int> cur(keyStart.begin(), keyStart.end() - 1);
-        for (int t = 0; t < nV; ++t) sorted[cur[key_of(vr[t])]++] = t;
+    // the one-launch form needs every row's sums in at most eight places
+    const int GR = mx::kFusedGroupRows, nGroups = (rows + GR - 1) / GR;
+    if (fused) {
+        int most = 0;
+        for (int r = 0; r < rows; ++r) most = std::max(most, segPtr[r + 1] - segPtr[r]);
+        if (sel || elsewhere || most > mx::kSliceLightSegs || (long long)nGroups * mx::kSliceLightSegs * GR > 2000000000LL) fused = false;
     }
-    // chunks of every slice: 64 virtual rows of the sorted order each, as long as their first member
+    std::vector<int> keyStart, sorted((size_t)nV);
     std::vector<std::vector<mx::SliceChunk>> sliceChunks(S);
-    for (int q = 0; q < S; ++q) {
-        const int a = keyStart[(size_t)q * perSlice], b = keyStart[(size_t)(q + 1) * perSlice];
-        for (int f = a; f < b; f += 64) sliceChunks[q].push_back({f, std::min(64, b - f), (vr[sorted[f]].len + E - 1) / E});
-    }
     mx::SlicePlan SP;
-    {
+    const size_t perSlice = (size_t)(cap + 1) * 3;
+    if (fused) {
+        fused = plan_fused(dtype, budget, S, rows, nGroups, cap, selPtr, segPtr, vr, sorted, sliceChunks, SP);
+        if (SP.nWG < 0) return MX_ERR_ARG;  // (the error is set)
+        if (!fused) {  // the matrix does not suit the form: the ordinary layout, from a clean slate
+            for (auto &v : sliceChunks) v.clear();
+            SP = mx::SlicePlan();
+        }
+    }
+    if (!fused) {
+        // virtual rows by (slice, length descending, kind of row), row order kept among equals: a
+        // counting sort.  The kind keeps the sums that one workgroup of the combine kernel gathers
+        // close together: consecutive heavy rows have virtual rows of the same slice and length more
+        // often than a heavy row and its neighbours of other kinds do.
+        const size_t nKeys = (size_t)S * perSlice;
+        keyStart.assign(nKeys + 1, 0);
+        auto key_of = [&](const VRow &v) { return (size_t)v.slice * perSlice + (size_t)(cap - v.len) * 3 + (size_t)v.kind; };
+        for (int t = 0; t < nV; ++t) keyStart[key_of(vr[t]) + 1]++;
+        for (size_t k = 0; k < nKeys; ++k) keyStart[k + 1] += keyStart[k];
+        {
+            std::vector<int> cur(keyStart.begin(), keyStart.end() - 1);
+            for (int t = 0; t < nV; ++t) sorted[cur[key_of(vr[t])]++] = t;
+        }
+        // chunks of every slice: 64 virtual rows of the sorted order each, as long as their first member
+        for (int q = 0; q < S; ++q) {
+            const int a = keyStart[(size_t)q * perSlice], b = keyStart[(size_t)(q + 1) * perSlice];
+            for (int f = a; f < b; f += 64) sliceChunks[q].push_back({f, std::min(64, b - f), (vr[sorted[f]].len + E - 1) / E});
+        }
         const int rc = mx::plan_slice_chunks(dtype, budget, S, sliceChunks, SP);
         if (rc) return rc;
     }
@@ -365,18 +665,43 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
         D.dict.swap(dictv);
         D.nDict = nDict;
     }
+    D.fused = fused;
+    if (fused) {
+        int most = 0;
+        for (int r = 0; r < rows; ++r) most = std::max(most, D.segPtr[r + 1] - D.segPtr[r]);
+        const int places = most <= 4 ? 4 : mx::kSliceLightSegs;
+        D.placesPerRow = places;
+        D.nGroups = SP.nGroups;
+        D.maxWgGroups = SP.maxWgGroups;
+        D.wgGroups.swap(SP.wgGroups);
+        D.groupNeed.swap(SP.groupNeed);
+        // where every virtual row puts its sum: the k-th of row r at ((r / GR) * places + k) * GR + r % GR; the
+        // padding lanes of a chunk at the spare places behind the last group
+        const size_t spare = (size_t)nGroups * places * GR;
+        D.fusedTarget.assign((size_t)totalChunks * 64, 0);
+        for (size_t v = 0; v < D.fusedTarget.size(); ++v) D.fusedTarget[v] = (int)(spare + (v & 63));
+        D.rowVrows.assign((size_t)nGroups * GR, 0);
+#pragma omp parallel for schedule(static)
+        for (int r = 0; r < rows; ++r) {
+            D.rowVrows[r] = (unsigned char)(D.segPtr[r + 1] - D.segPtr[r]);
+            for (int t = D.segPtr[r]; t < D.segPtr[r + 1]; ++t)
+                D.fusedTarget[D.segIdx[t]] = (int)(((size_t)(r / GR) * places + (t - D.segPtr[r])) * GR + r % GR);
+        }
+    }
     return MX_OK;
 }
 
 // `segOut` (optional): receives segPtr and segIdx (the virtual rows of every matrix row).
+// `fused`: the layout of the one-launch form where the matrix suits it (D.fused says whether it did);
+// made on the host.
 int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
                   const char *sel, mx::DeviceSlices &D, const char *elsewhere = nullptr,
-                  std::pair<std::vector<int>, std::vector<int>> *segOut = nullptr)
+                  std::pair<std::vector<int>, std::vector<int>> *segOut = nullptr, bool fused = false)
 {
     // The whole matrix: the layout is made on the device (the same arrays, in a fraction of the
     // time for a large matrix); MX_LAYOUT=host keeps the host route, which also serves row subsets.
     const char *lay = std::getenv("MX_LAYOUT");
-    if (!sel && !(lay && !std::strcmp(lay, "host"))) {
+    if (!sel && !fused && !(lay && !std::strcmp(lay, "host"))) {
         const size_t es = (size_t)mx::elem_size(dtype);
         const int nnz = rowPtr[rows];
         int *dRowPtr = nullptr, *dCol = nullptr;
@@ -395,7 +720,7 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
         return rc;
     }
     HostSlices H;
-    int rc = build_slices(dtype, rows, cols, rowPtr, col, val, nCU, S, sel, H, elsewhere);
+    int rc = build_slices(dtype, rows, cols, rowPtr, col, val, nCU, S, sel, H, elsewhere, fused);
     if (rc) return rc;
     if (segOut) {
         segOut->first = H.segPtr;
@@ -446,6 +771,20 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
         if ((rc = upload(&D.lightIdx, li.data(), li.size(), 8))) return rc;
     }
     if ((rc = upload(&D.heavyInfo, H.heavyInfo.data(), H.heavyInfo.size(), 4))) return rc;
+    if (H.fused) {
+        D.nGroups = H.nGroups;
+        D.maxWgGroups = H.maxWgGroups;
+        D.placesPerRow = H.placesPerRow;
+        if ((rc = upload(&D.wgGroups, H.wgGroups.data(), H.wgGroups.size()))) return rc;
+        if ((rc = upload(&D.groupNeed, H.groupNeed.data(), H.groupNeed.size()))) return rc;
+        if ((rc = upload(&D.groupCount, (const int *)nullptr, 0, (size_t)H.nGroups + 1))) return rc;
+        if ((rc = upload(&D.fusedTarget, H.fusedTarget.data(), H.fusedTarget.size(), 64))) return rc;
+        if ((rc = upload(&D.rowVrows, H.rowVrows.data(), H.rowVrows.size(), 64))) return rc;
+        if ((rc = upload_bytes(&D.fusedSums, nullptr, 0, ((size_t)H.nGroups * H.placesPerRow * mx::kFusedGroupRows + 64) * (dtype == MX_F64 ? 8 : 4))))
+            return rc;
+        if ((rc = upload(&D.claim, (const unsigned *)nullptr, 0, (size_t)H.nWG + 1))) return rc;
+        D.fused = true;
+    }
     return MX_OK;
 }
 
@@ -835,7 +1174,7 @@ int upload_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, c
 int mx::plan_slice_chunks(mx_dtype dtype, int budget, int S, const std::vector<std::vector<mx::SliceChunk>> &sliceChunks,
                           mx::SlicePlan &P)
 {
-    const int E = mx::slice_step_entries(dtype), SPB = mx::kSliceBatchEntries / E, W = mx::kSliceWaves;
+    const int E = mx::slice_step_entries(dtype), SPB = mx::kSliceBatchEntries / E;
     // the slice's share of the workgroups (in proportion to its steps, largest remainders, at
     // least one when it holds anything)
     std::vector<long long> sliceSteps(S, 0);
@@ -872,14 +1211,7 @@ int mx::plan_slice_chunks(mx_dtype dtype, int budget, int S, const std::vector<s
     }
     // workgroups: a slice's chunks, longest first, each to the workgroup of the slice with the
     // fewest steps so far; then the same inside the workgroup for its waves
-    struct Wg {
-        int slice;
-        std::vector<int> chunk[mx::kSliceWaves];  // per wave: indices into sliceChunks[slice]
-        int waveSteps[mx::kSliceWaves];
-        long long steps = 0;   // stored steps (every wave's stream rounded up to whole batches)
-        int chunks = 0;
-    };
-    std::vector<Wg> wgs;
+    std::vector<SliceWg> wgs;
     for (int q = 0; q < S; ++q) {
         const int g0 = (int)wgs.size(), G = Gq[q];
         if (G == 0) continue;
@@ -896,80 +1228,21 @@ int mx::plan_slice_chunks(mx_dtype dtype, int budget, int S, const std::vector<s
             top.first += ch[c].steps;
             if ((int)mine[top.second].size() < mx::kSliceWgChunks) heap.push(top);
         }
-        for (int g = 0; g < G; ++g) {
-            Wg &w = wgs[g0 + g];
-            w.slice = q;
-            for (int k = 0; k < W; ++k) w.waveSteps[k] = 0;
-            for (int c : mine[g]) {
-                int best = 0;
-                for (int k = 1; k < W; ++k)
-                    if (w.waveSteps[k] < w.waveSteps[best]) best = k;
-                w.chunk[best].push_back(c);
-                w.waveSteps[best] += ch[c].steps;
-            }
-            w.chunks = (int)mine[g].size();
-            for (int k = 0; k < W; ++k) w.steps += (w.waveSteps[k] + SPB - 1) / SPB * SPB;
-        }
+        for (int g = 0; g < G; ++g) deal_to_waves(wgs[g0 + g], q, mine[g], ch, SPB);
     }
-    const int nWG = (int)wgs.size();
-    long long totalSteps = 0, totalChunks = 0;
-    std::vector<long long> wgStep((size_t)nWG + 1, 0), wgChunk((size_t)nWG + 1, 0);
-    int maxWgChunks = 0;
-    for (int b = 0; b < nWG; ++b) {
-        wgStep[b] = totalSteps;
-        wgChunk[b] = totalChunks;
-        totalSteps += wgs[b].steps;
-        totalChunks += wgs[b].chunks;
-        maxWgChunks = std::max(maxWgChunks, wgs[b].chunks);
-    }
-    if (totalSteps * 64 * E > 2000000000LL || totalChunks * 64 > 2000000000LL) {
-        set_error("slice layout: too many entries for 32-bit offsets");
-        return MX_ERR_ARG;
-    }
-    P.nWG = nWG;
-    P.maxWgChunks = maxWgChunks;
-    P.totalSteps = totalSteps;
-    P.totalChunks = totalChunks;
-    P.wgDesc.assign((size_t)nWG * 4 + 4, 0);
-    P.waveDesc.assign((size_t)nWG * W * 4 + 4, 0);
-    P.chunkEnd.assign((size_t)totalChunks + 64, 0);
-    P.chunkSlice.assign((size_t)totalChunks, 0);
-    P.chunkFirst.assign((size_t)totalChunks, 0);
-    P.chunkN.assign((size_t)totalChunks, 0);
-    P.chunkSteps.assign((size_t)totalChunks, 0);
-    P.chunkStep0.assign((size_t)totalChunks, 0);
-    for (int b = 0; b < nWG; ++b) {
-        const Wg &G = wgs[b];
-        const int q = G.slice;
-        const auto &ch = sliceChunks[q];
-        long long step = wgStep[b], chunk = wgChunk[b];
-        P.wgDesc[(size_t)b * 4 + 0] = q;
-        P.wgDesc[(size_t)b * 4 + 1] = (int)chunk;
-        P.wgDesc[(size_t)b * 4 + 2] = G.chunks;
-        for (int w = 0; w < W; ++w) {
-            int *d = &P.waveDesc[((size_t)b * W + w) * 4];
-            d[0] = (int)(step / SPB);                   // first batch
-            d[1] = (G.waveSteps[w] + SPB - 1) / SPB;    // batches
-            d[2] = (int)(chunk - wgChunk[b]);           // first chunk, counted inside the workgroup
-            d[3] = (int)G.chunk[w].size();
-            int rel = 0;
-            for (int c : G.chunk[w]) {
-                P.chunkSlice[chunk] = q;
-                P.chunkFirst[chunk] = ch[c].first;
-                P.chunkN[chunk] = ch[c].n;
-                P.chunkSteps[chunk] = ch[c].steps;
-                P.chunkStep0[chunk] = step;
-                step += ch[c].steps;
-                rel += ch[c].steps;
-                P.chunkEnd[chunk++] = rel;
-            }
-            step = (step + SPB - 1) / SPB * SPB;
-        }
-    }
-    return MX_OK;
+    return emit_slice_plan(wgs, sliceChunks, SPB, E, P);
 }
 
+static int slice_layout_view(const mx_csr *A, int nCU, const unsigned char *sel, bool fused, mx_slice_layout_view *out);
 extern "C" int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *sel, mx_slice_layout_view *out)
+{
+    return slice_layout_view(A, nCU, sel, false, out);
+}
+extern "C" int mx_slice_layout_fused(const mx_csr *A, int nCU, mx_slice_layout_view *out)
+{
+    return slice_layout_view(A, nCU, nullptr, true, out);
+}
+static int slice_layout_view(const mx_csr *A, int nCU, const unsigned char *sel, bool fused, mx_slice_layout_view *out)
 {
     if (!A || !out || nCU < 1 || A->rows < 0 || A->cols < 1 || !A->rowPtr || (A->nnz > 0 && (!A->colInd || !A->val))) {
         set_error("mx_slice_layout: bad argument");
@@ -993,7 +1266,7 @@ extern "C" int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *se
     const int S = (A->cols + mx::slice_cols(A->dtype) - 1) / mx::slice_cols(A->dtype);
     HostSlices H;
     try {
-        int rc = build_slices(A->dtype, A->rows, A->cols, A->rowPtr, A->colInd, A->val, nCU, S, (const char *)sel, H);
+        int rc = build_slices(A->dtype, A->rows, A->cols, A->rowPtr, A->colInd, A->val, nCU, S, (const char *)sel, H, nullptr, fused);
         if (rc) return rc;
     } catch (const std::bad_alloc &) {
         set_error("mx_slice_layout: out of memory");
@@ -1032,6 +1305,21 @@ extern "C" int mx_slice_layout(const mx_csr *A, int nCU, const unsigned char *se
     out->nDict = H.ecode.empty() ? 0 : H.nDict;
     out->ecode = give(H.ecode);
     out->dict = give(H.dict);
+    out->fused = H.fused ? 1 : 0;
+    if (H.fused) {
+        out->groupRows = mx::kFusedGroupRows;
+        out->nGroups = H.nGroups;
+        out->placesPerRow = H.placesPerRow;
+        out->wgGroups = give(H.wgGroups);
+        out->groupNeed = give(H.groupNeed);
+        out->fusedTarget = give(H.fusedTarget);
+        out->rowVrows = give(H.rowVrows);
+        if (!out->wgGroups || !out->groupNeed || !out->fusedTarget || !out->rowVrows) {
+            mx_slice_layout_free(out);
+            set_error("mx_slice_layout: out of memory");
+            return MX_ERR_ALLOC;
+        }
+    }
     if (!out->wgDesc || !out->waveDesc || !out->chunkEnd || !out->segPtr || !out->segIdx || !out->rowInfo || !out->lightInfo ||
         !out->heavyInfo || !out->ecol || !out->ecode || !out->dict ||
         !out->eval) {
@@ -1057,6 +1345,10 @@ extern "C" void mx_slice_layout_free(mx_slice_layout_view *v)
     free(v->eval);
     free(v->ecode);
     free(v->dict);
+    free(v->wgGroups);
+    free(v->groupNeed);
+    free(v->fusedTarget);
+    free(v->rowVrows);
     std::memset(v, 0, sizeof(*v));
 }
 
@@ -1181,6 +1473,8 @@ struct mx_plan {
     mx::DeviceCsr csr;        // CSR part (or its short rows), row-tile form (csr_rows_kernel)
     mx::DeviceSlices slices;  // CSR part (or its long rows), x-resident-in-LDS form (csr_slice_kernel)
     int csr_variant = 0;      // 0 = row tiles, 1 = slices, 2 = row tiles for the short rows, then slices for the long ones
+    bool fused = false;       // slices in the one-launch form (slices.fused), until a misplaced workgroup is reported
+    unsigned fused_seq = 0;   // one-launch products queued so far
     int csr_nnz = 0;
     double est_rows_us = 0, est_slices_us = 0;  // what the choice of the form was made from (0: no choice was made)
     mx::DeviceTiles tiles;    // tile part, general form (tile_kernel)
@@ -1242,6 +1536,34 @@ static int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
     return MX_OK;
 }
 
+// The word in host memory that the one-launch kernels write when a workgroup is misplaced: one per
+// process, pinned and mapped, allocated at the first use (null when that fails).
+static std::atomic<bool> g_fused_off{false};
+static unsigned *misplaced_word()
+{
+    static std::once_flag once;
+    static unsigned *word = nullptr;
+    std::call_once(once, []() {
+        void *p = nullptr;
+        if (hipHostMalloc(&p, 64, hipHostMallocMapped) == hipSuccess && p) {
+            std::memset(p, 0, 64);
+            word = (unsigned *)p;
+        } else {
+            (void)hipGetLastError();
+        }
+    });
+    return word;
+}
+
+extern "C" int mx_debug_fused_misplaced(int set)
+{
+    unsigned *word = misplaced_word();
+    if (!word) return MX_ERR_DEVICE;
+    *(volatile unsigned *)word = set ? 1u : 0u;
+    if (!set) g_fused_off.store(false);
+    return MX_OK;
+}
+
 // `partial` (optional): where the slice kernel puts the sums of the virtual rows, in place of the
 // plan's own buffer.
 static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate, hipStream_t s,
@@ -1252,6 +1574,35 @@ static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate
         return MX_ERR_ARG;
     }
     if (plan->csr_variant != 1) MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s, ywide));
+    if (plan->csr_variant == 1 && plan->fused && !strips) {
+        // one launch.  A workgroup that found its share of the work taken already has said so in the
+        // host-visible word: the products since the last look cannot be trusted, and from here on every
+        // plan takes the two launches.
+        unsigned *word = misplaced_word();
+        // (a one-launch product carries the number of its launch: under stream capture, where the same
+        // arguments would be replayed, the two launches are recorded)
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
+            (void)hipGetLastError();
+            cap = hipStreamCaptureStatusNone;
+        }
+        if (cap != hipStreamCaptureStatusNone) {
+            // fall through to the two launches below
+        } else if (!word || g_fused_off.load()) {
+            plan->fused = false;
+        } else if (*(volatile unsigned *)word) {
+            g_fused_off.store(true);
+            plan->fused = false;
+            set_error("mx_spmv: two workgroups of an earlier one-launch product took the same share of the work; "
+                      "products since the previous call may be wrong; plans use the two-launch form from now on");
+            return MX_ERR_DEVICE;
+        } else {
+            mx::DeviceSlices L = plan->slices;  // a view: same arrays, maybe other sums
+            if (partial) L.partial = partial;
+            MX_HIP(mx::launch_fused(plan->dtype, L, x, y, accumulate, s, ywide, word, plan->fused_seq++));
+            return MX_OK;
+        }
+    }
     if (plan->csr_variant != 0) {
         if (partial) {
             mx::DeviceSlices L = plan->slices;  // a view: same arrays, other sums
@@ -1285,6 +1636,7 @@ struct CsrStats {
     double linesPerGather = 0;  // mean number of distinct 64-byte lines of x that 64 consecutive entries name
     double vrows = 0;           // virtual rows the slice layout would have (distinct slices per row, long ones cut)
     bool fewValues = false;     // at most 255 distinct values: the one-byte-per-value forms exist
+    int mostVrows = 0;          // most virtual rows of any row
 };
 
 static CsrStats csr_stats(mx_dtype dtype, int rows, const int *rowPtr, const int *col, const void *val, int nCU)
@@ -1310,7 +1662,8 @@ static CsrStats csr_stats(mx_dtype dtype, int rows, const int *rowPtr, const int
     const int BE = mx::kSliceBatchEntries;
     const int cap = (int)std::min<long long>(512, std::max<long long>(16, (fair + BE - 1) / BE * BE));
     double vrows = 0;
-#pragma omp parallel for schedule(dynamic, 4096) reduction(+ : vrows)
+    int mostVrows = 0;
+#pragma omp parallel for schedule(dynamic, 4096) reduction(+ : vrows) reduction(max : mostVrows)
     for (int r = 0; r < rows; ++r) {
         const int a = rowPtr[r], b = rowPtr[r + 1];
         if (b <= a) continue;
@@ -1349,8 +1702,10 @@ static CsrStats csr_stats(mx_dtype dtype, int rows, const int *rowPtr, const int
             }
         }
         vrows += n;
+        mostVrows = std::max(mostVrows, n);
     }
     st.vrows = vrows;
+    st.mostVrows = mostVrows;
     const char *ed = std::getenv("MX_CSR_DICT");
     if (nnz >= 65536 && !(ed && !std::atoi(ed))) {
         std::vector<unsigned char> codes, dict;
@@ -1390,14 +1745,35 @@ struct CsrChoice {
     bool want[3] = {true, true, false};
     double usRows = 0, usSlices = 0;  // the estimates, when they decided
     bool fewValues = false;
+    int mostVrows = -1;  // most virtual rows of a row (-1: not counted)
 };
 static bool plan_autotune()
 {
     static const bool on = std::getenv("MX_PLAN_AUTOTUNE") && std::atoi(std::getenv("MX_PLAN_AUTOTUNE"));
     return on;
 }
+// Whether a plan asks for the one-launch form of the slices.  Never with MX_PLAN_NO_FUSE or
+// MX_CSR_FUSED=0, after a misplaced workgroup was reported, or for a matrix with a row of more than
+// eight virtual rows (mostVrows < 0: not counted, the layout will see).  Otherwise where it pays:
+// the workgroup that comes last to a group of rows adds that group up alone, and the slowest
+// workgroup comes last to all of its groups, so the form wins while a workgroup's rows are few --
+// measured on the block-clustered workload at 256 workgroups: 9.5 against 11.3 us at 32 768 rows, a
+// tie at 49 152 and at 65 536 -- and is taken up to 160 rows per workgroup.  MX_PLAN_FUSE (or
+// MX_CSR_FUSED=1) takes it wherever the matrix suits it.
+static bool fused_wanted(int flags, int rows, int mostVrows, int nCU)
+{
+    static const char *env = std::getenv("MX_CSR_FUSED");
+    if ((flags & MX_PLAN_NO_FUSE) || (env && !std::atoi(env)) || g_fused_off.load()) return false;
+    if (mostVrows > mx::kSliceLightSegs || nCU % mx::kFusedXcds) return false;
+    if ((flags & MX_PLAN_FUSE) || (env && std::atoi(env))) return true;
+    return (long long)rows <= 160LL * nCU;
+}
+// What the one-launch form saves of the slice form's estimate where it is taken (microseconds): the second
+// launch and its wait, less the adding at the end of the first.
+constexpr double kFusedSavesUs = 1.8;
+
 static CsrChoice choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val,
-                                 int flags, int nCU, int S)
+                                 int flags, int nCU, int S, bool mayFuse = false)
 {
     CsrChoice c;
     const char *env = std::getenv("MX_CSR_KERNEL");
@@ -1411,6 +1787,10 @@ static CsrChoice choose_csr_form(mx_dtype dtype, int rows, int cols, const int *
         const CsrStats st = csr_stats(dtype, rows, rowPtr, col, val, nCU);
         csr_estimates(dtype, cols, rowPtr[rows], st, &c.usRows, &c.usSlices);
         c.fewValues = st.fewValues;
+        c.mostVrows = st.mostVrows;
+        // (the one-launch form of the slices, where the plan would take it: the device's placement is looked at
+        // later, and a plan whose strips ride in the second launch keeps both launches)
+        if (mayFuse && fused_wanted(flags, rows, st.mostVrows, nCU)) c.usSlices -= kFusedSavesUs;
         c.want[c.usSlices < c.usRows ? 0 : 1] = false;
     }
     return c;
@@ -1443,7 +1823,7 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
     MX_HIP(hipGetDeviceProperties(&prop, dev));
     const int nCU = std::max(1, prop.multiProcessorCount);
     const int S = slice_count(plan->dtype, rows, cols, nnz, nCU);
-    CsrChoice pick = choose_csr_form(plan->dtype, rows, cols, rowPtr, col, val, flags, nCU, S);
+    CsrChoice pick = choose_csr_form(plan->dtype, rows, cols, rowPtr, col, val, flags, nCU, S, stripRows == nullptr);
     bool(&want)[3] = pick.want;
     plan->est_rows_us = pick.usRows;
     plan->est_slices_us = pick.usSlices;
@@ -1476,9 +1856,17 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
         }
         return e;
     };
+    // the one-launch form of the slices, for a CSR part that is the whole product on a device whose
+    // workgroups land where the layout assumes
+    bool wantFused = want[1] && fused_wanted(flags, rows, pick.mostVrows, nCU) && !stripRows;
+    if (wantFused) {
+        int ok = 0;
+        MX_HIP(mx::fused_placement_ok(nCU, &ok));
+        wantFused = ok != 0;
+    }
     auto build = [&](int v, mx::DeviceCsr &C, mx::DeviceSlices &L) -> int {
         if (v == 0) return upload_csr(plan->dtype, rows, cols, nnz, rowPtr, col, val, C, nullptr);
-        if (v == 1) return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, nullptr, L, stripRows, segOut);
+        if (v == 1) return upload_slices(plan->dtype, rows, cols, rowPtr, col, val, nCU, S, nullptr, L, stripRows, segOut, wantFused);
         // the short rows as a CSR matrix of their own (the long rows empty), the long ones as slices
         std::vector<int> rp((size_t)rows + 1, 0);
         for (int r = 0; r < rows; ++r) rp[r + 1] = rp[r] + (longRow[r] ? 0 : rowPtr[r + 1] - rowPtr[r]);
@@ -1545,6 +1933,7 @@ static int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, cons
             std::swap(plan->csr, C);
             std::swap(plan->slices, L);
             plan->csr_variant = v;
+            plan->fused = v == 1 && plan->slices.fused;
             best = ms;
             have = true;
         }
@@ -2136,10 +2525,42 @@ static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, 
         st.fewValues = plan->slices.ecode != nullptr;
         if ((rc = mx::lines_per_gather_device(dtype, nnz, colInd_dev, nullptr, &st.linesPerGather))) return rc;
         csr_estimates(dtype, cols, nnz, st, &plan->est_rows_us, &plan->est_slices_us);
+        if (!elsewhere_dev && plan->slices.nHeavy == 0 && fused_wanted(flags, rows, -1, nCU)) plan->est_slices_us -= kFusedSavesUs;
         want[plan->est_slices_us < plan->est_rows_us ? 0 : 1] = false;
     }
     if (want[1]) {
         plan->csr_variant = 1;
+        // The one-launch form where the host route would take it (no row with more than eight virtual rows: the
+        // layout just made has no heavy rows).  Its layout is made on the host, from a copy of the part: the
+        // matrices it is taken for are small (160 rows per workgroup at most, unless it is forced).
+        bool wantFused = !elsewhere_dev && plan->slices.nHeavy == 0 && fused_wanted(flags, rows, -1, nCU);
+        if (wantFused) {
+            int ok = 0;
+            MX_HIP(mx::fused_placement_ok(nCU, &ok));
+            wantFused = ok != 0;
+        }
+        if (wantFused) {
+            const size_t es = (size_t)mx::elem_size(dtype);
+            std::vector<int> rp((size_t)rows + 1), ci((size_t)std::max(nnz, 1));
+            std::vector<unsigned char> va(std::max<size_t>((size_t)nnz * es, 1));
+            MX_HIP(hipMemcpy(rp.data(), rowPtr_dev, ((size_t)rows + 1) * 4, hipMemcpyDeviceToHost));
+            if (nnz) MX_HIP(hipMemcpy(ci.data(), colInd_dev, (size_t)nnz * 4, hipMemcpyDeviceToHost));
+            if (nnz) MX_HIP(hipMemcpy(va.data(), val_dev, (size_t)nnz * es, hipMemcpyDeviceToHost));
+            mx::DeviceSlices L;
+            rc = upload_slices(dtype, rows, cols, rp.data(), ci.data(), va.data(), nCU, S, nullptr, L, nullptr, segOut, true);
+            if (rc) {
+                free_slices(L);
+                return rc;
+            }
+            if (L.fused) {
+                free_slices(plan->slices);
+                plan->slices = L;
+                if (plan->slices.ecode) plan->slices.useDict = true;
+                plan->fused = true;
+            } else {
+                free_slices(L);
+            }
+        }
         return MX_OK;
     }
     free_slices(plan->slices);
@@ -2609,6 +3030,12 @@ extern "C" int mx_plan_arrays(const mx_plan *plan, mx_plan_array *out, int cap, 
         add("slices.lightRow", D.lightRow, (size_t)D.nLight * 4);
         add("slices.lightIdx", D.lightIdx, (size_t)D.nLight * 4 * D.lightQuads * 4);
         add("slices.heavyInfo", D.heavyInfo, ((size_t)D.nHeavy * 4 + 4) * 4);
+        if (D.fused) {
+            add("slices.wgGroups", D.wgGroups, ((size_t)D.nWG * 2 + 2) * 4);
+            add("slices.groupNeed", D.groupNeed, ((size_t)D.nGroups + 1) * 4);
+            add("slices.fusedTarget", D.fusedTarget, (size_t)D.chunks * 64 * 4);
+            add("slices.rowVrows", D.rowVrows, (size_t)D.nGroups * mx::kFusedGroupRows);
+        }
     }
     const mx::DeviceTiles *two[2] = {&plan->tiles, &plan->strips};
     static const char *const names[2][5] = {{"tiles.waveDesc", "tiles.hdr", "tiles.atox", "tiles.tcVal", "tiles.vidx"},
@@ -2700,7 +3127,7 @@ extern "C" int mx_plan_layout(const mx_partition *P, int flags, int nCU, mx_plan
             const int *ci = P->extracted ? H.col.data() : P->cdColInd.data();
             const void *va = P->extracted ? (const void *)H.val.data() : P->cdVal.data();
             const int S = slice_count(P->dtype, P->rows, P->cols, rp[P->rows], nCU);
-            const CsrChoice pick = choose_csr_form(P->dtype, P->rows, P->cols, rp, ci, va, flags, nCU, S);
+            const CsrChoice pick = choose_csr_form(P->dtype, P->rows, P->cols, rp, ci, va, flags, nCU, S, H.stripRows.empty());
             out->csr_variant = pick.want[2] ? 2 : pick.want[0] && pick.want[1] ? -1 : pick.want[1] ? 1 : 0;
             out->est_rows_us = pick.usRows;
             out->est_slices_us = pick.usSlices;
@@ -2783,6 +3210,7 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     info->ext_dRows = plan->ext_dRows;
     info->ext_nnzRowD = plan->ext_nnzRowD;
     info->ext_frags = plan->ext_frags;
+    info->csr_fused = plan->csr_variant == 1 && plan->fused ? 1 : 0;
     return MX_OK;
 }
 
@@ -2883,6 +3311,8 @@ extern "C" int mx_time_csr_main(mx_plan *plan, const void *x_dev, void *y_dev, i
     hipStream_t s = plan->stream;
     int rc = time_loop(plan, warm, iters, [&]() -> int {
         // the kernel that holds most of the entries
+        if (plan->csr_variant == 1 && plan->fused)
+            return launch_csr_part(plan, x_dev, y_dev, 0, s);
         if (plan->csr_variant == 1 || (plan->csr_variant == 2 && plan->slices.nnz > plan->csr.nnz))
             MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x_dev, y_dev, 0, s, 1));
         else
@@ -2982,7 +3412,12 @@ extern "C" int mx_time_kernels(mx_plan *plan, const void *x_dev, void *y_dev, in
             });
         xCounted = true;
     }
-    if (plan->csr_variant != 0) {
+    if (plan->csr_variant == 1 && plan->fused && !ride) {
+        // the one-launch form: one kernel multiplies, adds up and writes y
+        add(std::string("csr_slice_kernel<") + vt + (plan->slices.useDict ? ",dict,fused>" : ",fused>"),
+            (double)plan->slices.nnz * (es + 4) + xBytes + yBytes, plan->slices.nnz,
+            [&]() -> int { return launch_csr_part(plan, x_dev, y_dev, 0, s, nullptr, nullptr, wide); });
+    } else if (plan->csr_variant != 0) {
         add(std::string("csr_slice_kernel<") + vt + (plan->slices.useDict ? ",dict>" : ">"),
             (double)plan->slices.nnz * (es + 4) + (xCounted ? 0.0 : xBytes), plan->slices.nnz, [&]() -> int {
                 MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x_dev, y_dev, 0, s, 1));

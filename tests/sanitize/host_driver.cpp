@@ -21,6 +21,12 @@ int main()
         mx_slice_layout_view sv;
         if (mx_slice_layout(&A, 8, nullptr, &sv)) { printf("slice layout: %s\n", mx_last_error()); return 1; }
         mx_slice_layout_free(&sv);
+        // the layout of the one-launch form (refused for the power-law workloads, whose rows reach many slices)
+        for (int nCU : {8, 32, 256}) {
+            if (mx_slice_layout_fused(&A, nCU, &sv)) { printf("fused slice layout: %s\n", mx_last_error()); return 1; }
+            printf("  fused layout on %d workgroups: %d\n", nCU, sv.fused);
+            mx_slice_layout_free(&sv);
+        }
         for (auto &t : taus) {
             mx_partition *P = nullptr;
             if (mx_partition_create(&A, t[0], t[1], &P)) { printf("partition: %s\n", mx_last_error()); return 1; }

@@ -836,6 +836,127 @@ def test_spmv_in_a_hip_graph(mx, ora):
     P.close()
 
 
+def test_one_launch_form_of_the_slices(mx, ora):
+    """The CSR part in slice form as ONE launch (the reference's residual kernel is one launch,
+    src/spmv_kernel/cdSpMV.cu:459): y equals the two-launch form's bit for bit and the oracle's within the
+    bar, on binary64 and binary16, with four and with eight places per row, on rows without entries,
+    on the plan made from device arrays, product after product (the counters clear themselves), with y
+    accumulated; a default plan takes the form only while a workgroup's rows are few; under stream capture
+    the two launches are recorded."""
+    import torch
+    rng = np.random.default_rng(31)
+    cases = []
+    A, x = mx.gen_config(2, scale=0.5)           # 32 768 rows: the default plan takes the form
+    cases.append(("block-clustered, half size", A, x, True))
+    A, x = mx.gen_config(2, scale=1.0)           # 65 536 rows: only when asked
+    cases.append(("block-clustered, full size", A, x, False))
+    A, x = mx.gen_config(3, scale=0.05)          # stencil, one byte per value
+    cases.append(("stencil", A, x, None))
+    rows, cols = 20000, 3 * 65536 + 5             # binary16, rows in any order, stretches of empty rows
+    lens = rng.integers(0, 40, rows)
+    lens[3000:5200] = 0
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = rng.integers(0, cols, rp[-1]).astype(np.int32)
+    cases.append(("binary16", mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, rp[-1]).astype(np.float16)),
+                  rng.uniform(-1, 1, cols).astype(np.float16), None))
+    for name, A, x, default_takes_it in cases:
+        print("one-launch form:", name, A.rows, A.nnz, flush=True)
+        ref = oracle_y(ora, mx, A, x)
+        tol = F64_TOL if A.dtype == mx.MX_F64 else F16_TOL
+        P = mx.Partition(A, 0.0, 0.0)
+        two = mx.Plan(P, mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_NO_FUSE)
+        one = mx.Plan(P, mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_FUSE)
+        assert two.info["csr_variant"] == 1 and two.info["csr_fused"] == 0
+        assert one.info["csr_variant"] == 1 and one.info["csr_fused"] == 1, name
+        xd = torch.from_numpy(x).cuda()
+        y2 = two.spmv(xd).cpu().numpy()
+        y1 = torch.full((A.rows,), 7.0, dtype=xd.dtype, device="cuda")
+        for rep in range(3):                      # the counters of a product are back at zero for the next
+            y1.fill_(7.0)
+            one.spmv(xd, y1)
+        torch.cuda.synchronize()
+        got = y1.cpu().numpy()
+        assert np.array_equal(got.view(np.uint8), y2.view(np.uint8)), name
+        assert rel_l2(got, ref) <= tol
+        # another x, many products back to back, then the first x again
+        xn = torch.from_numpy(rng.uniform(-1, 1, A.cols).astype(x.dtype)).cuda()
+        one.spmv_repeat(xn, y1, 50)
+        one.spmv(xd, y1)
+        torch.cuda.synchronize()
+        assert np.array_equal(y1.cpu().numpy().view(np.uint8), y2.view(np.uint8)), name
+        # the plan made from device arrays takes the same form and gives the same y
+        D = mx.Plan.from_device_csr(torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda(),
+                                    A.cols, mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_FUSE)
+        assert D.info["csr_fused"] == 1
+        assert D.arrays() == one.arrays()
+        assert np.array_equal(D.spmv(xd).cpu().numpy().view(np.uint8), y2.view(np.uint8)), name
+        D.close()
+        if default_takes_it is not None:
+            d = mx.Plan(P, mx.MX_PLAN_CSR_SLICES)
+            assert d.info["csr_fused"] == (1 if default_takes_it else 0), (name, d.info)
+            d.close()
+        # under stream capture the two launches are recorded, and the replays give the same y
+        g = torch.cuda.CUDAGraph()
+        yg = torch.zeros_like(y1)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            one.spmv(xd, yg)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g):
+            one.spmv(xd, yg)
+        for rep in range(3):
+            yg.fill_(3.0)
+            g.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(yg.cpu().numpy().view(np.uint8), y2.view(np.uint8)), (name, rep)
+            one.spmv(xd, y1)                      # eager one-launch products between the replays
+            torch.cuda.synchronize()
+        assert one.info["csr_fused"] == 1
+        one.close()
+        two.close()
+        P.close()
+
+
+def test_one_launch_form_reports_a_share_taken_twice(mx, ora):
+    """The way out of the one-launch form, forced from the host (the word a workgroup sets when it finds its
+    share of the work taken already): the next product returns MX_ERR_DEVICE once, the plan goes on in the
+    two-launch form with the same y, and new plans do not take the one-launch form until the word is cleared."""
+    import torch
+    A, x = mx.gen_config(2, scale=0.25)
+    ref = oracle_y(ora, mx, A, x)
+    P = mx.Partition(A, 0.0, 0.0)
+    plan = mx.Plan(P, mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_FUSE)
+    assert plan.info["csr_fused"] == 1
+    xd = torch.from_numpy(x).cuda()
+    y = plan.spmv(xd)
+    torch.cuda.synchronize()
+    good = y.cpu().numpy()
+    assert rel_l2(good, ref) <= F64_TOL
+    try:
+        mx.debug_fused_misplaced(True)
+        with pytest.raises(mx.MxError) as e:
+            plan.spmv(xd, y)
+        assert e.value.code == 3 and "two-launch" in str(e.value)
+        y.fill_(5.0)
+        plan.spmv(xd, y)                          # two launches from here on
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy(), good)
+        other = mx.Plan(P, mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_FUSE)
+        assert other.info["csr_fused"] == 0
+        assert np.array_equal(other.spmv(xd).cpu().numpy(), good)
+        other.close()
+    finally:
+        mx.debug_fused_misplaced(False)
+    again = mx.Plan(P, mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_FUSE)
+    assert again.info["csr_fused"] == 1
+    assert np.array_equal(again.spmv(xd).cpu().numpy(), good)
+    again.close()
+    plan.close()
+    P.close()
+
+
 def test_tau_tuner(mx, ora):
     """mx_tune_tau walks the grid with tau_c >= tau_r, reports every candidate, returns the fastest;
     candidates without tiles share one timing and are reported as (0, 0)."""
@@ -1285,7 +1406,7 @@ def test_plan_from_a_matrix_in_device_memory(mx, ora):
             print("device csr plan: case %d rows=%d nnz=%d flags=%d" % (i, A.rows, A.nnz, flags), flush=True)
             H = mx.Plan(part, flags)
             D = mx.Plan.from_device_csr(rp, ci, va, A.cols, flags)
-            for k in ("csr_variant", "csr_value_dict", "csr_nnz", "csr_blocks", "tile_nnz"):
+            for k in ("csr_variant", "csr_value_dict", "csr_nnz", "csr_blocks", "tile_nnz", "csr_fused"):
                 assert H.info[k] == D.info[k], (i, flags, k, H.info[k], D.info[k])
             if flags == mx.MX_PLAN_DEFAULT and H.info["est_rows_us"] > 0:
                 assert abs(H.info["est_rows_us"] - D.info["est_rows_us"]) < 1e-9 and abs(H.info["est_slices_us"] - D.info["est_slices_us"]) < 1e-9

@@ -293,7 +293,7 @@ def _walk_slice_layout(L, x, f64, subset=False):
     seen_chunks = 0
     for b in range(L["nWG"]):
         q, wgChunk0, wgChunks, _ = L["wgDesc"][b]
-        assert 0 <= q < L["S"] and wgChunk0 == seen_chunks and 0 < wgChunks <= 4096
+        assert 0 <= q < L["S"] and wgChunk0 == seen_chunks and (0 if L.get("fused") else 1) <= wgChunks <= 4096
         xs = np.zeros(SW)
         n = max(0, min(SW, len(x) - q * SW))
         xs[:n] = x[q * SW:q * SW + n]
@@ -423,6 +423,117 @@ def test_slice_layout_walk(mx, ora, case):
     nv = np.diff(L["segPtr"])
     assert np.all(nv[~keep] == 0) and np.all(nv[keep & (lens > 0)] >= 1) and np.all(nv[lens == 0] == 0)
     assert np.all(nv <= -(-lens // 1) ) and L["cap"] % L["batchEntries"] == 0
+
+
+def _xcd_of_logical_workgroup(b, nWG):
+    """Logical workgroups [k * nWG / 8, (k + 1) * nWG / 8) are taken by workgroups that run on XCD k."""
+    assert nWG % 8 == 0
+    return b // (nWG // 8)
+
+
+@pytest.mark.parametrize("case", ["block", "stencil", "wide_f64", "unsorted_f16", "empty_rows"])
+def test_fused_slice_layout_walk(mx, case):
+    """The layout of the one-launch form, walked on the CPU: the streams give the same sums as ever; every
+    workgroup's sums belong to rows of the groups it counts off; all workgroups that count a group off
+    sit on one XCD and are as many as the group expects; every group is counted off by someone; and the
+    places of a row name exactly its virtual rows, so that adding them up gives A x."""
+    rng = np.random.default_rng(9)
+    nCU = 16
+    if case == "block":
+        A, x = mx.gen_config(2, scale=1 / 8)
+        nCU = 64
+    elif case == "stencil":
+        A, x = mx.gen_config(3, scale=0.03)
+        nCU = 32
+    elif case == "wide_f64":
+        nCU = 64
+        rows, cols = 5000, 4 * 16384 + 77
+        lens = rng.integers(0, 40, rows)
+        rp = np.zeros(rows + 1, np.int32)
+        rp[1:] = np.cumsum(lens)
+        ci = np.concatenate([np.sort(rng.choice(cols, n, replace=False)) for n in lens]).astype(np.int32)
+        A = mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, len(ci)))
+        x = rng.uniform(-1, 1, cols)
+    elif case == "unsorted_f16":
+        nCU = 40
+        rows, cols = 4100, 3 * 65536 + 5
+        lens = rng.integers(0, 30, rows)
+        rp = np.zeros(rows + 1, np.int32)
+        rp[1:] = np.cumsum(lens)
+        ci = rng.integers(0, cols, rp[-1]).astype(np.int32)
+        A = mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, len(ci)).astype(np.float16))
+        x = rng.uniform(-1, 1, cols).astype(np.float16)
+    else:   # long stretches of rows without entries: their groups must still be counted off and written as zero
+        nCU = 32
+        rows, cols = 6000, 40000
+        lens = rng.integers(1, 50, rows)
+        lens[300:1700] = 0
+        lens[4000:4600] = 0
+        rp = np.zeros(rows + 1, np.int32)
+        rp[1:] = np.cumsum(lens)
+        ci = np.concatenate([np.sort(rng.choice(cols, n, replace=False)) for n in lens]).astype(np.int32)
+        A = mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, len(ci)))
+        x = rng.uniform(-1, 1, cols)
+    f64 = A.dtype == mx.MX_F64
+    L = mx.slice_layout(A, nCU=nCU, fused=True)
+    assert L["fused"] == 1 and L["nWG"] == nCU and L["groupRows"] == 256 and L["nGroups"] == -(-A.rows // 256)
+    xf = np.asarray(x, np.float64)
+    y2, partial = _walk_slice_layout(L, xf, f64)          # the arrays of the two-launch form stay valid
+    GR, P = L["groupRows"], L["placesPerRow"]
+    segPtr, segIdx = L["segPtr"], L["segIdx"]
+    rowOfV = np.full(L["chunks"] * 64, -1)
+    rowOfV[segIdx] = np.repeat(np.arange(A.rows), np.diff(segPtr))
+    need = np.zeros(L["nGroups"], np.int64)
+    xcdOfGroup = np.full(L["nGroups"], -1)
+    for b in range(L["nWG"]):
+        g0, ng = L["wgGroups"][b]
+        _, c0, nc, _ = L["wgDesc"][b]
+        k = _xcd_of_logical_workgroup(b, L["nWG"])
+        assert 0 <= g0 and g0 + ng <= L["nGroups"] and (ng > 0 or nc == 0)
+        need[g0:g0 + ng] += 1
+        assert np.all((xcdOfGroup[g0:g0 + ng] == -1) | (xcdOfGroup[g0:g0 + ng] == k)), "a group is counted off from two XCDs"
+        xcdOfGroup[g0:g0 + ng] = k
+        mine = rowOfV[c0 * 64:(c0 + nc) * 64]
+        mine = mine[mine >= 0]
+        assert mine.size == 0 or (mine.min() // GR >= g0 and mine.max() // GR < g0 + ng), "sums outside the workgroup's groups"
+    assert np.array_equal(need, L["groupNeed"]) and need.min() >= 1
+    # the sums as the one-launch kernel stores them: virtual row v at fusedTarget[v]; the k-th virtual row of
+    # row r sits at ((r // GR) * P + k) * GR + r % GR, padding lanes at the spare places behind the last group
+    nv = np.diff(segPtr)
+    assert nv.max() <= P and P in (4, 8) and np.array_equal(L["rowVrows"][:A.rows], nv) and np.all(L["rowVrows"][A.rows:] == 0)
+    tgt = L["fusedTarget"]
+    spare = L["nGroups"] * P * GR
+    assert tgt.shape == (L["chunks"] * 64,)
+    pad = rowOfV < 0
+    assert np.array_equal(tgt[pad], spare + (np.nonzero(pad)[0] & 63))
+    real = tgt[~pad]
+    assert len(np.unique(real)) == len(real) and real.max() < spare
+    sums = np.zeros(spare + 64)
+    sums[tgt] = partial
+    y = np.zeros(A.rows)
+    rows = np.arange(A.rows)
+    for k in range(P):
+        has = nv > k
+        at = ((rows // GR) * P + k) * GR + rows % GR
+        assert np.array_equal(at[has], tgt[segIdx[segPtr[:-1][has] + k]])
+        y[has] += sums[at[has]]
+    assert L["wgDesc"][:, 2].max() <= 96     # the targets of a workgroup's chunks fit the LDS beside x
+    ref = np.zeros(A.rows)
+    np.add.at(ref, np.repeat(np.arange(A.rows), np.diff(A.rowPtr)), A.val.astype(np.float64) * xf[A.colInd])
+    assert np.allclose(y, ref, rtol=1e-12, atol=1e-12 * max(1.0, np.abs(ref).max()))
+    assert np.allclose(y2, ref, rtol=1e-12, atol=1e-12 * max(1.0, np.abs(ref).max()))
+
+
+def test_fused_slice_layout_is_refused_where_it_does_not_fit(mx):
+    """A row with more than eight virtual rows, or fewer workgroups per XCD than slices: the ordinary layout."""
+    A, _ = mx.gen_config(4, scale=1 / 32)     # power-law rows reach every slice
+    L = mx.slice_layout(A, nCU=64, fused=True)
+    assert np.diff(L["segPtr"]).max() > 8 and L["fused"] == 0
+    plain = mx.slice_layout(A, nCU=64)
+    for k in ("wgDesc", "waveDesc", "chunkEnd", "segIdx", "ecol", "eval", "rowInfo"):
+        assert np.array_equal(L[k], plain[k]), k
+    B, _ = mx.gen_config(2, scale=1 / 2)      # two slices everywhere, one workgroup per XCD
+    assert mx.slice_layout(B, nCU=8, fused=True)["fused"] == 0
 
 
 def test_slice_layout_rejects_bad_matrices(mx):
