@@ -10,14 +10,26 @@ tau_c >= tau_r), and workloads 2 (FP64 block-clustered, same sweep), 3 (FP64 ste
 (FP16 power-law) follow under "others", each with its own roofline record, parity figure and
 cold-cache time.
 
-Prints ONE JSON line.  `value` = 2*nnz/t of the headline workload (GFLOP/s).  `roofline` prices
-the WHOLE product: the reference's algorithmic bytes of the matrix (nnz*(sizeof(valT)+4) +
-(rows+1)*4 + cols*sizeof(valT) + rows*sizeof(valT), test/test_cdspmv.cpp:214) over the time of
-one product -- HIP events on the plan's own stream around K back-to-back products -- against
-8 TB/s.  `roofline.kernels` lists every kernel launch of the product timed alone, each with its
-share of those bytes (the shares add up to the whole) and, where profiles/ holds a rocprofv3
-counter run of that kernel on that workload and plan, its measured HBM traffic.  `cpu_baseline`
-is the oracle's single-thread CSR loop on the same matrix, on this box's host cores.
+Prints ONE JSON line.  `value` = 2*nnz/t of the headline workload (GFLOP/s), timed on the plan a
+caller gets with default flags at the best point of the sweep (the sweep itself keeps every
+hybrid's tiles, so that its table shows each one as it is).  `roofline` prices the WHOLE product:
+the reference's algorithmic bytes of the matrix (nnz*(sizeof(valT)+4) + (rows+1)*4 +
+cols*sizeof(valT) + rows*sizeof(valT), test/test_cdspmv.cpp:214) over the time of one product
+against 8 TB/s.  Three times are measured, each the median of five repetitions of the
+reference's protocol (200 warm-ups, then at least 1000 timed launches between HIP events on the
+plan's own stream, src/spmv_kernel/cdSpMV.cu:454-479): `warm` (one plan, back to back: a matrix
+of up to 256 MB stays in the memory-side cache), `rotating` (a train that takes several copies
+of the plan in turn, three times the memory-side cache in all: every array comes from HBM, the
+steady state of a solver whose matrix does not fit that cache) and `cold` (single products after
+a 1 GiB sweep).  `roofline.frac` is the warm figure for a plan that fits the memory-side cache
+and the rotating one for a plan that does not (`frac_basis` says which; all three are there),
+and `frac_traffic` prices the same time with the bytes the counters saw instead of the
+algorithmic ones.  `roofline.kernels` lists every kernel launch of the product timed alone, each
+with its share of the algorithmic bytes (the shares add up to the whole) and, where profiles/
+holds a rocprofv3 counter run of that kernel on that workload and plan, its measured HBM
+traffic.  `cpu_baseline` is the oracle's single-thread CSR loop on the same matrix, on this
+box's host cores.  Workloads 2 and 5 are also run with their dense structure off the grid of
+eight columns (`others.workload_N_unaligned`: CSR-only against the best hybrid).
 """
 import argparse
 import glob
@@ -32,6 +44,8 @@ sys.path.insert(0, ROOT)
 
 METRIC = "SpMV GFLOP/s (2·nnz/t) + % of HBM roofline, FP64 and FP16, 1 GPU"
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
+MALL_BYTES = 256 << 20  # the memory-side cache
+REPS = 5  # repetitions of every timed train; the median is quoted
 GRID = (0.0, 0.25, 0.5, 0.75, 1.0)
 WORKLOADS = {
     1: "configs[0]: FP64 random 4096x4096, 16 nnz/row",
@@ -120,24 +134,33 @@ def cpu_baseline(mx, ora, A, x):
     return base, allc
 
 
-def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=None, keep=None):
-    """mode: 'sweep' (the 5x5 grid), 'points' (CSR-only and two hybrid points) or 'csr' ((0,0) only)."""
+def median_time(fn, reps=REPS):
+    import numpy as np
+    return float(np.median([fn() for _ in range(reps)]))
+
+
+def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=None, keep=None, unaligned=False, brief=False):
+    """mode: 'sweep' (the 5x5 grid), 'points' (CSR-only and two hybrid points) or 'csr' ((0,0) only).
+    brief: no routes, no cold or rotating trains (the records of the unaligned variants)."""
     import numpy as np
     keep = mx.MX_PLAN_KEEP_TILES if keep is None else keep
     t0 = time.time()
-    A, x = mx.gen_config(cfg)
-    log("workload %d: rows=%d nnz=%d generated in %.1fs" % (cfg, A.rows, A.nnz, time.time() - t0))
+    A, x = mx.gen_config(cfg, unaligned=unaligned)
+    log("workload %d%s: rows=%d nnz=%d generated in %.1fs" % (cfg, " (off the grid)" if unaligned else "", A.rows, A.nnz, time.time() - t0))
     dev = torch.device("cuda:0")
     xd = torch.from_numpy(x).to(dev)
     yd = torch.empty(A.rows, dtype=xd.dtype, device=dev)
     B = A.algorithmic_bytes
     dtype = "f64" if A.dtype == mx.MX_F64 else "f16"
+    n_ev = max(steps, 1000)
+    on_device = A.nnz >= (1 << 21)
 
     # ---- which (tau_c, tau_r): every candidate is partitioned (on the device for large matrices),
     # planned and timed by mx_tune_tau with short loops; candidates that send nothing to the tile
     # kernels are one and the same CSR-only plan and are timed once.  MX_PLAN_KEEP_TILES: every
     # candidate runs the hybrid its fragments give, also where the plan's own estimate would send
-    # everything through the CSR part (what that estimate says is recorded below).
+    # everything through the CSR part.  The three fastest candidates and the CSR-only plan are then
+    # timed again with the full protocol, and the point is chosen from those.
     t0 = time.time()
     if only_tau is not None:
         points = [tuple(only_tau)]
@@ -153,32 +176,48 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
         table = [{"tau_c": c, "tau_r": r, "ms_total": ms, "tile_nnz": tn} for c, r, ms, tn in tt]
     else:
         for tau in points:
-            part = mx.Partition(A, *tau, device=A.nnz >= (1 << 21) and tau != (0.0, 0.0))
+            part = mx.Partition(A, *tau, device=on_device and tau != (0.0, 0.0))
             plan = mx.Plan(part, keep)
             ms = plan.time(xd, yd, warm=10, iters=100, parts=False)[0]
             table.append({"tau_c": tau[0], "tau_r": tau[1], "ms_total": ms, "tile_nnz": plan.info["tile_nnz"]})
             plan.close()
             part.close()
+    csr_rec = next((r for r in table if r["tile_nnz"] == 0), None)
+    again = sorted((r for r in table if r["tile_nnz"] > 0), key=lambda r: r["ms_total"])[:3]
+    if csr_rec is not None:
+        again.append(csr_rec)
+    for r in again:
+        part = mx.Partition(A, r["tau_c"], r["tau_r"], device=on_device and r["tile_nnz"] > 0)
+        plan = mx.Plan(part, keep)
+        r["ms_short_loop"] = r["ms_total"]
+        r["ms_total"] = median_time(lambda: plan.time(xd, yd, warm=200, iters=1000, parts=False)[0], 3)
+        r["timed"] = "median of 3 x (200 + 1000)"
+        plan.close()
+        part.close()
     for r in table:
-        log("  tau=(%.2f,%.2f) %.2f us tile_nnz=%d" % (r["tau_c"], r["tau_r"], r["ms_total"] * 1e3, r["tile_nnz"]))
+        log("  tau=(%.2f,%.2f) %.2f us tile_nnz=%d%s" % (r["tau_c"], r["tau_r"], r["ms_total"] * 1e3, r["tile_nnz"],
+                                                         "  (timed again)" if "timed" in r else ""))
     sweep_s = time.time() - t0
-    csr_only = next((r for r in table if r["tile_nnz"] == 0), None)
-    hybrid = [r for r in table if r["tile_nnz"] > 0]
+    csr_only = csr_rec
+    hybrid = [r for r in table if r["tile_nnz"] > 0 and "timed" in r]
     best_hybrid = min(hybrid, key=lambda r: r["ms_total"]) if hybrid else None
-    best = min(table, key=lambda r: r["ms_total"])
-    # a hybrid point is taken when it beats the CSR-only plan by more than the noise of the short timing
-    # loops (2 %); every point without tiles is the CSR-only plan: call it (0, 0)
+    best = min((r for r in table if "timed" in r), key=lambda r: r["ms_total"])
+    # a hybrid point is taken when it beats the CSR-only plan by more than 2 %; every point without tiles is
+    # the CSR-only plan: call it (0, 0)
     if csr_only is not None and (best["tile_nnz"] == 0 or best["ms_total"] > 0.98 * csr_only["ms_total"]):
         best = dict(csr_only, tau_c=0.0, tau_r=0.0)
     tau = (best["tau_c"], best["tau_r"])
 
-    # ---- the plan of the best point, from the matrix to the first y: host route and device route
+    # ---- the plan of the best point as a caller with default flags gets it, from the matrix to the first y:
+    # host route and device route
+    FLAGS = mx.MX_PLAN_DEFAULT if keep == mx.MX_PLAN_KEEP_TILES else keep
+
     def first_y(device):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         part = mx.Partition(A, *tau, device=device)
         t1 = time.perf_counter()
-        plan = mx.Plan(part, keep)
+        plan = mx.Plan(part, FLAGS)
         t2 = time.perf_counter()
         plan.spmv(xd, yd)
         torch.cuda.synchronize()
@@ -187,30 +226,31 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
                             "first_spmv_ms": (t3 - t2) * 1e3, "total_ms": (t3 - t0) * 1e3}
     part, plan, host_route = first_y(False)
     route = {"host": host_route}
-    # the device route: the matrix goes up as it is; extraction, decisions and layouts are made on the device from
-    # the device arrays (mx_plan_create_device: the same plan, so the same y bit for bit); a caller whose matrix
-    # already lives in HBM skips the upload
-    if not getattr(run_workload, "_device_route_used", False):
-        A1 = mx.gen_config(1)[0]  # first use of the device code, not timed
-        mx.Plan.from_device(*(torch.from_numpy(a).to(dev) for a in (A1.rowPtr, A1.colInd, A1.val)), A1.cols, 0.5, 0.5).close()
-        run_workload._device_route_used = True
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    drp, dci, dva = (torch.from_numpy(a).to(dev) for a in (A.rowPtr, A.colInd, A.val))
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    q2 = mx.Plan.from_device(drp, dci, dva, A.cols, tau[0], tau[1], keep)
-    t2 = time.perf_counter()
-    y2 = torch.empty_like(yd)
-    q2.spmv(xd, y2)
-    torch.cuda.synchronize()
-    t3 = time.perf_counter()
-    route["device"] = {"upload_ms": (t1 - t0) * 1e3, "plan_create_ms": (t2 - t1) * 1e3, "first_spmv_ms": (t3 - t2) * 1e3,
-                       "total_ms": (t3 - t0) * 1e3, "prep_route": q2.info["prep_route"]}
-    route["same_y"] = bool(torch.equal(y2, yd))
-    q2.close()
-    del drp, dci, dva, y2
     info = plan.info
+    if not brief:
+        # the device route: the matrix goes up as it is; extraction, decisions and layouts are made on the device from
+        # the device arrays (mx_plan_create_device: the same plan, so the same y bit for bit); a caller whose matrix
+        # already lives in HBM skips the upload
+        if not getattr(run_workload, "_device_route_used", False):
+            A1 = mx.gen_config(1)[0]  # first use of the device code, not timed
+            mx.Plan.from_device(*(torch.from_numpy(a).to(dev) for a in (A1.rowPtr, A1.colInd, A1.val)), A1.cols, 0.5, 0.5).close()
+            run_workload._device_route_used = True
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        drp, dci, dva = (torch.from_numpy(a).to(dev) for a in (A.rowPtr, A.colInd, A.val))
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        q2 = mx.Plan.from_device(drp, dci, dva, A.cols, tau[0], tau[1], FLAGS)
+        t2 = time.perf_counter()
+        y2 = torch.empty_like(yd)
+        q2.spmv(xd, y2)
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        route["device"] = {"upload_ms": (t1 - t0) * 1e3, "plan_create_ms": (t2 - t1) * 1e3, "first_spmv_ms": (t3 - t2) * 1e3,
+                           "total_ms": (t3 - t0) * 1e3, "prep_route": q2.info["prep_route"]}
+        route["same_y"] = bool(torch.equal(y2, yd))
+        q2.close()
+        del drp, dci, dva, y2
 
     # ---- the timed run: W warm-up products, then exactly K products between synchronisations
     plan.spmv_repeat(xd, yd, warmup)
@@ -219,9 +259,9 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
     plan.spmv_repeat(xd, yd, steps)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    # the same by HIP events on the plan's own stream, over enough launches to average the launch jitter
-    n_ev = max(steps, 1000)
-    ev_total = plan.time(xd, yd, warm=max(warmup, 100), iters=n_ev, parts=False)[0]
+    # the reference's protocol: warm-ups, then a train of launches between HIP events on the plan's own stream;
+    # the median of REPS such trains
+    ev_total = median_time(lambda: plan.time(xd, yd, warm=max(warmup, 200), iters=n_ev, parts=False)[0])
     kernels = plan.time_kernels(xd, yd, warm=max(warmup, 100), iters=n_ev)
     y = yd.cpu().numpy().astype(np.float64)
 
@@ -232,20 +272,41 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
         ref = ora.spmv_f16_f32acc(A.val, A.rowPtr, A.colInd, x)[0].astype(np.float64)
     rel_l2 = float(np.linalg.norm(y - ref) / np.linalg.norm(ref))
 
-    # ---- cold caches: a 1 GiB buffer is swept between launches, so neither the L2s (8 x 4 MB) nor
-    # the 256 MB memory-side cache hold the matrix when the product starts
-    flush = torch.empty(1 << 28, dtype=torch.float32, device=dev)
-    cold = []
-    for _ in range(15):
-        flush.add_(1.0)
-        torch.cuda.synchronize()
-        cold.append(plan.time(xd, yd, warm=0, iters=1, parts=False)[0])
-    del flush
-    cold_ms = float(np.median(cold))
+    plan_bytes = info["tile_bytes"] + info["csr_bytes"]
+    cold_ms = rot = None
+    if not brief:
+        # ---- cold caches: a 1 GiB buffer is swept between launches, so neither the L2s (8 x 4 MB) nor
+        # the 256 MB memory-side cache hold the matrix when the product starts
+        flush = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+        cold = []
+        for _ in range(15):
+            flush.add_(1.0)
+            torch.cuda.synchronize()
+            cold.append(plan.time(xd, yd, warm=0, iters=1, parts=False)[0])
+        del flush
+        cold_ms = float(np.median(cold))
+        # ---- every array from HBM, in a steady train: copies of the plan (and of x and y), three times the
+        # memory-side cache in all, taken in turn
+        copies = int(min(24, max(2, -(-3 * MALL_BYTES // max(int(plan_bytes), 1)))))
+        plans, xs, ys = [plan], [xd], [yd]
+        for _ in range(copies - 1):
+            plans.append(mx.Plan(part, FLAGS))
+            xs.append(xd.clone())
+            ys.append(torch.empty_like(yd))
+        rot_ms = median_time(lambda: mx.time_rotate(plans, xs, ys, warm=max(200, 4 * copies), iters=max(n_ev, 20 * copies)))
+        same = all(bool(torch.equal(ys[i], yd)) for i in range(1, copies))
+        for p in plans[1:]:
+            p.close()
+        del plans, xs, ys
+        rot = {"copies": copies, "bytes_in_rotation": copies * plan_bytes, "ms_per_step": rot_ms,
+               "gflops": 2.0 * A.nnz / (rot_ms * 1e-3) / 1e9, "hbm_frac_whole_spmv": B / (rot_ms * 1e-3) / HBM_PEAK,
+               "every_copy_gives_the_same_y": same,
+               "how": "median of %d trains of >= %d products that take %d copies of the plan (each with its own x and y) in "
+                      "turn, HIP events on one stream" % (REPS, max(n_ev, 20 * copies), copies)}
 
     # ---- what the plan's own estimate decides at the best hybrid point (default flags)
     if best_hybrid:
-        p2 = mx.Partition(A, best_hybrid["tau_c"], best_hybrid["tau_r"], device=A.nnz >= (1 << 21))
+        p2 = mx.Partition(A, best_hybrid["tau_c"], best_hybrid["tau_r"], device=on_device)
         q2 = mx.Plan(p2)
         best_hybrid = dict(best_hybrid, default_plan_keeps_tiles=q2.info["tile_nnz"] > 0)
         q2.close()
@@ -254,7 +315,7 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
     plan_kind = "hybrid" if info["tile_nnz"] > 0 else "csr_only"
     krecs, tr_sum, tr_all = [], 0, True
     for k in kernels:
-        t = traffic.get((cfg, plan_kind, k["name"]))
+        t = traffic.get((cfg, plan_kind, k["name"])) if not unaligned else None
         if t is None:
             tr_all = False
         else:
@@ -265,40 +326,53 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
                       "frac": k["algorithmic_bytes"] / (k["ms"] * 1e-3) / HBM_PEAK,
                       "traffic": (t["read"] + t["written"]) if t else None,
                       "traffic_from": t["file"] if t else None})
-    achieved = B / (ev_total * 1e-3)
+    # the time the fraction is priced on: the warm train for a plan that fits the memory-side cache (a solver
+    # that iterates on it finds it there), the rotating train for one that does not
+    in_mall = plan_bytes <= MALL_BYTES or rot is None
+    basis_ms = ev_total if in_mall else rot["ms_per_step"]
+    achieved = B / (basis_ms * 1e-3)
+    traffic_total = tr_sum if (tr_all and krecs) else None
     roofline = {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": achieved / HBM_PEAK,
-                "traffic": tr_sum if (tr_all and krecs) else None,
-                "what": "the whole product (%s): algorithmic bytes of the matrix over the mean time of one product in a "
-                        "train of %d back-to-back products, HIP events on the plan's stream" %
-                        (" + ".join(k["kernel"] for k in krecs), n_ev),
-                "bytes_per_launch": B, "ms_per_launch": ev_total, "kernels": krecs}
+                "frac_basis": ("warm: the plan's %.0f MB stay in the 256 MB memory-side cache between products" % (plan_bytes / 1e6)) if in_mall
+                else ("rotating: the plan's %.0f MB do not fit the 256 MB memory-side cache, every product reads them from HBM" % (plan_bytes / 1e6)),
+                "frac_warm": B / (ev_total * 1e-3) / HBM_PEAK,
+                "frac_rotating": rot and rot["hbm_frac_whole_spmv"],
+                "frac_cold": cold_ms and B / (cold_ms * 1e-3) / HBM_PEAK,
+                "traffic": traffic_total,
+                "frac_traffic": traffic_total and traffic_total / (basis_ms * 1e-3) / HBM_PEAK,
+                "what": "the whole product (%s): algorithmic bytes of the matrix over the median, over %d trains, of the mean time "
+                        "of one product in a train of %d products after 200 warm-ups, HIP events on the plan's stream" %
+                        (" + ".join(k["kernel"] for k in krecs), REPS, n_ev),
+                "bytes_per_launch": B, "ms_per_launch": basis_ms, "kernels": krecs}
     if info["csr_value_dict"]:
         roofline["note"] = ("the matrix has %d distinct values and the main kernel reads one byte per entry for them: the "
-                            "algorithmic bytes still count sizeof(valT) per entry, so frac can exceed what the traffic "
-                            "would give; `traffic` is what the kernels really move" % info["csr_value_dict"])
+                            "algorithmic bytes still count sizeof(valT) per entry, so frac can exceed 1; frac_traffic prices "
+                            "the same time with the bytes the kernels really move" % info["csr_value_dict"])
     rec = {
-        "workload": WORKLOADS[cfg], "dtype": dtype, "rows": A.rows, "nnz": A.nnz,
-        "tau_c": tau[0], "tau_r": tau[1], "plan": plan_kind, "csr_variant": ("rows", "slices", "split")[info["csr_variant"]],
+        "workload": WORKLOADS[cfg] + (", dense structure off the grid of eight columns" if unaligned else ""),
+        "dtype": dtype, "rows": A.rows, "nnz": A.nnz,
+        "tau_c": tau[0], "tau_r": tau[1], "plan": plan_kind, "plan_flags": "MX_PLAN_DEFAULT" if FLAGS == mx.MX_PLAN_DEFAULT else int(FLAGS),
+        "csr_variant": ("rows", "slices", "split")[info["csr_variant"]], "csr_one_launch": bool(info["csr_fused"]),
         "tile_nnz": info["tile_nnz"], "csr_nnz": info["csr_nnz"],
         "ms_per_step": wall_ms, "ms_per_step_events": ev_total,
         "gflops": 2.0 * A.nnz / (wall_ms * 1e-3) / 1e9,
-        "algorithmic_bytes": B,
+        "algorithmic_bytes": B, "plan_bytes_per_product": plan_bytes,
         "hbm_frac_whole_spmv": B / (wall_ms * 1e-3) / HBM_PEAK,
-        "cold_cache": {"ms_per_step": cold_ms, "gflops": 2.0 * A.nnz / (cold_ms * 1e-3) / 1e9,
-                       "hbm_frac_whole_spmv": B / (cold_ms * 1e-3) / HBM_PEAK,
-                       "how": "median of 15 single products, each after a 1 GiB buffer sweep and a sync; the quoted value "
-                              "is the back-to-back (warm) one"},
+        "cold_cache": cold_ms and {"ms_per_step": cold_ms, "gflops": 2.0 * A.nnz / (cold_ms * 1e-3) / 1e9,
+                                   "hbm_frac_whole_spmv": B / (cold_ms * 1e-3) / HBM_PEAK,
+                                   "how": "median of 15 single products, each after a 1 GiB buffer sweep and a sync"},
+        "rotating": rot,
         "rel_l2_vs_oracle": rel_l2,
         # mx_plan_create from a partition in host memory; mx_plan_create_device from the matrix in device memory,
         # extraction included (matrix_to_first_y has both routes whole)
         "plan_create_ms": host_route["plan_create_ms"],
-        "plan_create_device_ms": route["device"]["plan_create_ms"],
+        "plan_create_device_ms": route.get("device", {}).get("plan_create_ms"),
         "matrix_to_first_y": route,
         "plan_estimates_us": {"rows": info["est_rows_us"], "slices": info["est_slices_us"]},
         "csr_only_ms": csr_only and csr_only["ms_total"],
         "best_hybrid": best_hybrid,
         "roofline": roofline,
-        "sweep": table, "sweep_seconds": sweep_s,
+        "sweep": table, "sweep_flags": "MX_PLAN_KEEP_TILES" if keep == mx.MX_PLAN_KEEP_TILES else int(keep), "sweep_seconds": sweep_s,
     }
     plan.close()
     part.close()
@@ -316,6 +390,7 @@ def main():
     ap.add_argument("--tau", type=float, nargs=2, metavar=("TAU_C", "TAU_R"), default=None,
                     help="no sweep: run this point (a profile of a fixed plan)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline (profile runs)")
+    ap.add_argument("--no-unaligned", action="store_true", help="skip the variants of workloads 2 and 5 with structure off the grid")
     ap.add_argument("--all-tiles", action="store_true",
                     help="plans with MX_PLAN_ALL_TILES: every extracted chunk through the general MFMA tile kernel (profile runs)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
@@ -358,9 +433,9 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"], out["cpu_all_cores"] = cpu_baseline(mx, ora, A, x)
     del A, x
-    for k in ("hbm_frac_whole_spmv", "cold_cache", "rel_l2_vs_oracle", "plan_create_ms", "plan_create_device_ms", "matrix_to_first_y",
-              "plan_estimates_us", "csr_only_ms", "best_hybrid", "tile_nnz", "csr_nnz", "ms_per_step_events",
-              "algorithmic_bytes", "sweep", "sweep_seconds"):
+    for k in ("hbm_frac_whole_spmv", "cold_cache", "rotating", "rel_l2_vs_oracle", "plan_create_ms", "plan_create_device_ms",
+              "matrix_to_first_y", "plan_estimates_us", "csr_only_ms", "best_hybrid", "tile_nnz", "csr_nnz", "ms_per_step_events",
+              "algorithmic_bytes", "plan_bytes_per_product", "plan_flags", "csr_one_launch", "sweep", "sweep_flags", "sweep_seconds"):
         out[k] = main_rec[k]
 
     # what a plain device copy reaches on this GPU, next to the 8 TB/s the roofline is priced at:
@@ -394,6 +469,12 @@ def main():
     for cfg in cfgs[1:]:
         r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, mode_of(cfg), traffic, None, keep)
         others["workload_%d" % cfg] = r
+    # the dense structure of workloads 2 and 5 off the grid of eight columns: CSR-only against the best hybrid
+    if not args.no_sweep and args.tau is None and not args.no_unaligned:
+        for cfg in cfgs:
+            if cfg in SWEPT:
+                r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, "sweep", traffic, None, keep, unaligned=True, brief=True)
+                others["workload_%d_unaligned" % cfg] = r
     if others:
         out["others"] = others
     out["bench_seconds"] = time.time() - t_start

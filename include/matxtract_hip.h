@@ -215,6 +215,13 @@ float mx_f16_to_f32(uint16_t h);
  * the input vector x.  The reference has no generators; these define the benchmark. */
 int mx_gen_config(int config_id, uint64_t seed, double scale, int *rows, int *cols, int *nnz,
                   mx_dtype *dtype, int **rowPtr, int **colInd, void **val, void **x);
+/* The same with variants of the recipes.  MX_GEN_UNALIGNED: the dense structure of workloads 2 and 5 off
+ * the grid of eight columns -- a block of workload 2 starts at any column of its band, a strip of workload 5
+ * at a column that is not a multiple of eight (the benchmark quotes the aligned form and reports this one
+ * beside it).  gen_flags = 0 is mx_gen_config. */
+#define MX_GEN_UNALIGNED 1
+int mx_gen_config_ex(int config_id, uint64_t seed, double scale, int gen_flags, int *rows, int *cols, int *nnz,
+                     mx_dtype *dtype, int **rowPtr, int **colInd, void **val, void **x);
 
 /* Algorithmic bytes of one SpMV: nnz*(sizeof(valT)+4) + (rows+1)*4 + cols*sizeof(valT) +
  * rows*sizeof(valT) (`data_origin1`, test/test_cdspmv.cpp:214). */
@@ -260,7 +267,10 @@ void mx_plan_destroy(mx_plan *plan);
  * (slice form) cross to the host.  The form is chosen as in mx_plan_create, from the same counts taken
  * on the device: the plan, and with it every y, equals the one mx_plan_create makes from a partition
  * of the same matrix with tau = (0, 0).  rowPtr_dev and colInd_dev are checked on the device before
- * they are used as addresses (MX_ERR_ARG).  flags: MX_PLAN_CSR_ROWS, MX_PLAN_CSR_SLICES or 0. */
+ * they are used as addresses (MX_ERR_ARG).  flags: MX_PLAN_CSR_ROWS, MX_PLAN_CSR_SLICES, MX_PLAN_NO_FUSE,
+ * MX_PLAN_FUSE or 0.  Three forms of the CSR part are laid out on the host, from a copy of the part that is
+ * brought down for it: the one-launch form of the slices (small matrices, unless it is forced), and the split
+ * form and the timed choice that MX_CSR_KERNEL=split and MX_PLAN_AUTOTUNE=1 ask for. */
 int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
                               const void *val_dev, int flags, mx_plan **out);
 
@@ -313,7 +323,8 @@ void mx_plan_arrays_free(mx_plan_array *a, int n);
 
 /* y = A*x on the device.  x [cols] and y [rows] are DEVICE pointers of the plan's value
  * type, x 16-byte aligned (the kernels copy it in 16-byte vectors; a plan whose CSR part keeps
- * x in LDS returns MX_ERR_ARG otherwise, and reads the last 16-byte block of x whole when cols is
+ * x in LDS, or whose binary64 8 x 8 blocks read x in aligned pieces, returns MX_ERR_ARG otherwise,
+ * before anything is launched, and reads the last 16-byte block of x whole when cols is
  * not a multiple of the vector -- the bytes past x[cols-1] in that block are read, never used);
  * `stream` is a hipStream_t (NULL = default stream).
  * Asynchronous.  The hybrid sequence of test/test_autotc_spmv.cpp:1507-1559 (tile part, scatter
@@ -358,10 +369,21 @@ int mx_spmv_host(mx_plan *plan, const void *x_host, void *y_host);
 /* The reference's timing protocol (200 warm-ups + 4000 timed back-to-back launches,
  * src/spmv_kernel/cdSpMV.cu:454-479, du_tcSpMV_fp64.cu:311-333) on the plan's own stream.
  * ms_total: mean per SpMV of the whole sequence (hipEvents around the loop);
- * ms_tile / ms_csr: mean per launch of each kernel timed on its own (the two numbers the
- * reference adds up, test/test_autotc_spmv.cpp:1561-1572); any may be NULL. */
+ * ms_tile / ms_csr: the tile part and the CSR part timed on their own (the two numbers the reference adds
+ * up, test/test_autotc_spmv.cpp:1561-1572).  Where strips or 8 x 8 blocks ride in the combine kernel's launch
+ * there is no tile launch to time: ms_csr is then the CSR part's launches as the product runs them, riders
+ * included, and ms_tile what the riders add (the same launches without them taken off); binary64 blocks in a
+ * launch of their own are priced the same way, as the pair less the CSR part, so that y never grows.  Any
+ * may be NULL.  MX_ERR_ARG for an x the plan cannot take (see mx_spmv), before anything is launched. */
 int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, int iters,
             double *ms_total, double *ms_tile, double *ms_csr);
+
+/* The protocol of mx_time on a train of products that takes the `n` plans in turn (product k runs
+ * plans[k % n] on x_dev[k % n] into y_dev[k % n], all on the first plan's stream): with n copies of one
+ * plan whose arrays add up to several times the 256 MB memory-side cache, no product finds any of its
+ * arrays in a cache, which is what a solver sees whose matrix is larger than that cache -- the
+ * reference's loops (src/spmv_kernel/cdSpMV.cu:464-469) always re-run one matrix.  ms = mean per product. */
+int mx_time_rotate(mx_plan *const *plans, const void *const *x_dev, void *const *y_dev, int n, int warm, int iters, double *ms);
 
 /* Mean ms per launch of the CSR part's main kernel alone (csr_rows_kernel, or csr_slice_kernel
  * without its combine kernel), same protocol as mx_time: the figure a roofline is priced on. */
@@ -433,8 +455,10 @@ typedef struct mx_plan_info {
                             0 = csr_rows_kernel, 1 = csr_slice_kernel */
     int csr_main_nnz;    /* entries that kernel holds */
     int tile_variant;    /* 1 when part of the tiles runs through tile_dense_kernel: binary16 rows whose columns
-                            fill at most 8 aligned blocks of 8 columns at least half (a row of a dense strip in
-                            the simplest case), with nothing in the residual and no column named twice; the plan
+                            fill at most 8 blocks of 8 consecutive columns at least half (a row of a dense strip in
+                            the simplest case; the blocks start at multiples of eight or, where that takes fewer
+                            blocks, at the row's own first column plus multiples of eight, so a strip may start at
+                            any column), with nothing in the residual and no column named twice; the plan
                             groups rows with the same blocks, 8 at a time, into chunks of its own (at least 4
                             rows each) and takes them out of the reference's fragments.  MX_NO_STRIPS=1 in the
                             environment switches this off; with an x that is not 16-byte aligned these chunks

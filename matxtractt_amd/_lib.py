@@ -133,6 +133,7 @@ SIGNATURES = {
     "mx_f32_to_f16": (C.c_uint16, [C.c_float]),
     "mx_f16_to_f32": (C.c_float, [C.c_uint16]),
     "mx_gen_config": (_i, [_i, C.c_uint64, _d, _pi, _pi, _pi, _pi, _pp, _pp, _pp, _pp]),
+    "mx_gen_config_ex": (_i, [_i, C.c_uint64, _d, _i, _pi, _pi, _pi, _pi, _pp, _pp, _pp, _pp]),
     "mx_algorithmic_bytes": (_d, [_i, _i, _i, _i]),
     "mx_plan_create": (_i, [_vp, _i, _pp]),
     "mx_plan_create_device_csr": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _i, _pp]),
@@ -149,6 +150,7 @@ SIGNATURES = {
     "mx_spmv_repeat": (_i, [_vp, _vp, _vp, _i, _vp]),
     "mx_spmv_host": (_i, [_vp, _vp, _vp]),
     "mx_time": (_i, [_vp, _vp, _vp, _i, _i, _pd, _pd, _pd]),
+    "mx_time_rotate": (_i, [_vp, _vp, _vp, _i, _i, _i, _pd]),
     "mx_time_kernels": (_i, [_vp, _vp, _vp, _i, _i, C.POINTER(KernelTime), _i, _pi]),
     "mx_time_csr_main": (_i, [_vp, _vp, _vp, _i, _i, _pd]),
     "mx_plan_get_info": (_i, [_vp, C.POINTER(PlanInfo)]),

@@ -17,7 +17,7 @@ from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLA
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "split_device", "tiles_device", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "estimate_tau", "tile_steps", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
-           "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "MX_PLAN_NO_FUSE", "MX_PLAN_FUSE", "plan_layout", "debug_fused_misplaced"]
+           "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "MX_PLAN_NO_FUSE", "MX_PLAN_FUSE", "time_rotate", "plan_layout", "debug_fused_misplaced"]
 
 
 def _p(a):
@@ -78,13 +78,14 @@ class Csr:
         return algorithmic_bytes(self.dtype, self.rows, self.cols, self.nnz)
 
 
-def gen_config(config_id, seed=0, scale=1.0):
-    """Synthetic workload 1..5 -> (Csr, x)."""
+def gen_config(config_id, seed=0, scale=1.0, unaligned=False):
+    """Synthetic workload 1..5 -> (Csr, x).  unaligned=True: the dense blocks of workload 2 and the strips of
+    workload 5 start off the grid of eight columns (mx_gen_config_ex, MX_GEN_UNALIGNED)."""
     L = _lib.load()
     rows, cols, nnz, dt = C.c_int(), C.c_int(), C.c_int(), C.c_int()
     rp, ci, va, xv = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
-    check(L.mx_gen_config(config_id, seed, scale, C.byref(rows), C.byref(cols), C.byref(nnz), C.byref(dt),
-                          C.byref(rp), C.byref(ci), C.byref(va), C.byref(xv)))
+    check(L.mx_gen_config_ex(config_id, seed, scale, 1 if unaligned else 0, C.byref(rows), C.byref(cols), C.byref(nnz), C.byref(dt),
+                             C.byref(rp), C.byref(ci), C.byref(va), C.byref(xv)))
     vt = _np_dtype(dt.value)
     A = Csr(rows.value, cols.value, _take(rp.value, rows.value + 1, np.int32),
             _take(ci.value, nnz.value, np.int32), _take(va.value, nnz.value, vt))
@@ -281,6 +282,22 @@ class Partition:
 def debug_fused_misplaced(on):
     """Sets (or clears) the word a misplaced workgroup of a one-launch product sets (mx_debug_fused_misplaced)."""
     check(_lib.load().mx_debug_fused_misplaced(1 if on else 0))
+
+
+def time_rotate(plans, xs, ys, warm=200, iters=4000):
+    """Mean ms per product of a train that takes the plans in turn (mx_time_rotate); xs, ys: one device
+    tensor per plan."""
+    n = len(plans)
+    assert n >= 1 and len(xs) == n and len(ys) == n
+    for p, x, y in zip(plans, xs, ys):
+        p._check_vec(x, p.cols, "x")
+        p._check_vec(y, p.rows, "y")
+    hp = (C.c_void_p * n)(*[p._h.value for p in plans])
+    xp = (C.c_void_p * n)(*[x.data_ptr() for x in xs])
+    yp = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
+    ms = C.c_double()
+    check(_lib.load().mx_time_rotate(hp, xp, yp, n, int(warm), int(iters), C.byref(ms)))
+    return ms.value
 
 
 def slice_layout(A, nCU=256, sel=None, device=False, fused=False):

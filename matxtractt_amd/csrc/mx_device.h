@@ -60,7 +60,7 @@ struct DeviceTiles {
     long long stored = 0;      // values stored (zeros included)
     int steps = 0, nWaves = 0;
     bool dense = false;        // binary16 chunks the plan formed from rows of dense strips: every block's eight
-                               // columns are consecutive from a multiple of eight and every chunk fits one step
+                               // columns are consecutive and every chunk fits one step
                                // (two share a step when both fit a half): tile_dense_kernel can run it
     bool ownedRows = false;    // set by the plan: no row of these tiles gets anything from the CSR part
     // binary64 `dense` layouts (blocks of 8 x 8 on rows that the CSR part shares) when they ride in the

@@ -25,6 +25,12 @@
 //                       at 8*(block + off), off uniform in [-32,32] per strip (clipped) -- a
 //                       dense 8x32 block sliding along the diagonal.  All other rows are
 //                       power-law rows as in 4. f16.
+//
+// MX_GEN_UNALIGNED (mx_gen_config_ex) takes the dense structure of workloads 2 and 5 off the grid of
+// eight columns: a block of workload 2 starts at any column of the band [r - 1024, r + 1024 - 8]
+// (its eight rows still start at a multiple of eight; blocks of one block row do not overlap), and a
+// strip of workload 5 starts at 8*(block + off) + shift with shift uniform in [1, 7] per strip.
+// Everything else is drawn as before.
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
@@ -146,29 +152,37 @@ void gen_random(Rng &g, int n, int per_row, Builder &B)
     }
 }
 
-void gen_block_clustered(Rng &g, int n, Builder &B)
+void gen_block_clustered(Rng &g, int n, Builder &B, bool unaligned)
 {
     const int per_row = std::min(64, n), nb = n / 8;
     const int max_blocks_per_row = per_row / 8;
     int want = (int)std::floor(0.4 * (double)n * per_row / 64.0);
-    std::vector<std::vector<int>> blocks(nb);  // block columns of each block row
+    std::vector<std::vector<int>> blocks(nb);  // first column of every block of each block row
     int placed = 0;
     for (long long attempts = 0; placed < want && attempts < 64LL * want + 1024; ++attempts) {
         int br = g.below(nb);
-        int bc = br - 128 + g.below(256);
-        bc = std::min(std::max(bc, 0), nb - 1);
+        int c0;
+        if (unaligned) {
+            c0 = 8 * br - 1024 + g.below(2048 - 8 + 1);
+            c0 = std::min(std::max(c0, 0), n - 8);
+        } else {
+            int bc = br - 128 + g.below(256);
+            c0 = 8 * std::min(std::max(bc, 0), nb - 1);
+        }
         auto &v = blocks[br];
         if ((int)v.size() >= max_blocks_per_row) continue;
-        if (std::find(v.begin(), v.end(), bc) != v.end()) continue;
-        v.push_back(bc);
+        bool overlaps = false;
+        for (int o : v) overlaps = overlaps || std::abs(o - c0) < 8;
+        if (overlaps) continue;
+        v.push_back(c0);
         ++placed;
     }
     std::vector<int> cols;
     for (int r = 0; r < n; ++r) {
         cols.clear();
         if (r / 8 < nb)
-            for (int bc : blocks[r / 8])
-                for (int j = 0; j < 8; ++j) cols.push_back(8 * bc + j);
+            for (int c0 : blocks[r / 8])
+                for (int j = 0; j < 8; ++j) cols.push_back(c0 + j);
         while ((int)cols.size() < per_row) {
             int c = g.below(n);
             if (std::find(cols.begin(), cols.end(), c) == cols.end()) cols.push_back(c);
@@ -195,7 +209,7 @@ void gen_stencil27(int g3, Builder &B)
             }
 }
 
-void gen_mixed(Rng &g, int n, Builder &B)
+void gen_mixed(Rng &g, int n, Builder &B, bool unaligned)
 {
     PowerLaw pl(n);
     const int run = 128;
@@ -203,10 +217,11 @@ void gen_mixed(Rng &g, int n, Builder &B)
         int r1 = std::min(r0 + run, n);
         bool strip = g.u01() < 0.2 && n >= 64;
         int off = g.below(65) - 32;
+        const int shift = unaligned ? 1 + g.below(7) : 0;
         for (int r = r0; r < r1; ++r) {
             if (strip) {
-                int c0 = 8 * (r / 8 + off);
-                c0 = std::min(std::max(c0, 0), n - 32);
+                int c0 = 8 * (r / 8 + off) + shift;
+                c0 = std::min(std::max(c0, shift), n - 32 - (8 - shift) % 8);
                 for (int j = 0; j < 32; ++j) B.push(c0 + j, g.sym());
                 B.end_row();
             } else {
@@ -229,11 +244,18 @@ T *dup(const std::vector<T> &v)
 extern "C" int mx_gen_config(int config_id, uint64_t seed, double scale, int *rows, int *cols, int *nnz,
                              mx_dtype *dtype, int **rowPtr, int **colInd, void **val, void **x)
 {
+    return mx_gen_config_ex(config_id, seed, scale, 0, rows, cols, nnz, dtype, rowPtr, colInd, val, x);
+}
+
+extern "C" int mx_gen_config_ex(int config_id, uint64_t seed, double scale, int gen_flags, int *rows, int *cols, int *nnz,
+                                mx_dtype *dtype, int **rowPtr, int **colInd, void **val, void **x)
+{
     if (config_id < 1 || config_id > 5 || !(scale > 0.0 && scale <= 1.0) || !rows || !cols || !nnz || !dtype ||
-        !rowPtr || !colInd || !val || !x) {
+        !rowPtr || !colInd || !val || !x || (gen_flags & ~MX_GEN_UNALIGNED)) {
         mx::set_error("mx_gen_config: bad argument (config 1..5, scale in (0,1])");
         return MX_ERR_ARG;
     }
+    const bool unaligned = (gen_flags & MX_GEN_UNALIGNED) != 0;
     if (seed == 0) seed = 0x9E3779B97F4A7C15ull ^ (uint64_t)config_id;
     Rng g(seed);
     Builder B;
@@ -248,7 +270,7 @@ extern "C" int mx_gen_config(int config_id, uint64_t seed, double scale, int *ro
             break;
         case 2:
             n = std::max(64, (int)std::llround(65536.0 * scale) / 8 * 8);
-            gen_block_clustered(g, n, B);
+            gen_block_clustered(g, n, B, unaligned);
             break;
         case 3: {
             int g3 = std::max(3, (int)std::llround(100.0 * std::cbrt(scale)));
@@ -265,7 +287,7 @@ extern "C" int mx_gen_config(int config_id, uint64_t seed, double scale, int *ro
         }
         case 5:
             n = std::max(256, (int)std::llround(4194304.0 * scale) / 128 * 128);
-            gen_mixed(g, n, B);
+            gen_mixed(g, n, B, unaligned);
             break;
         }
     } catch (const std::bad_alloc &) {

@@ -92,43 +92,65 @@ __global__ __launch_bounds__(kBlock) void iota_kernel(int *__restrict__ v, int n
     if (k < n) v[k] = k;
 }
 
-// The aligned blocks of eight columns (caller's numbering) that row i of A_dd touches, ascending.
-// false when the row does not qualify as a row of a strip chunk: fewer than 4 or more than 64
-// entries, something in the residual, a column named twice, a block that would reach past the
-// end of x, more than eight blocks, or blocks less than half full.
+// The blocks of eight consecutive columns (caller's numbering) that row i of A_dd touches: the first
+// column of each, ascending.  The blocks start at multiples of eight, or, where that takes fewer
+// blocks, at the row's own lowest column plus multiples of eight.  false when the row does not qualify
+// as a row of a strip chunk: fewer than 4 or more than 64 entries, something in the residual, a column
+// named twice, a block that would reach past the end of x, more than eight blocks, or blocks less than
+// half full.
 struct RowBlocks {
     int nb;
     int b[8];
 };
+// (0 = fine, 1 = too many blocks or one past the end of x, 2 = a column named twice)
+__device__ int row_blocks_at(const int *__restrict__ ddCol, const int *__restrict__ descColId, int p0, int n, int cols, int shift,
+                             RowBlocks &R)
+{
+    R.nb = 0;
+    unsigned m[8];
+    for (int k = 0; k < n; ++k) {
+        const int c = descColId[ddCol[p0 + k]];
+        const int first = ((c - shift) >> 3) * 8 + shift;
+        const unsigned bit = 1u << (c - first);
+        if (first + 8 > cols) return 1;
+        int j = 0;
+        while (j < R.nb && R.b[j] < first) ++j;
+        if (j < R.nb && R.b[j] == first) {
+            if (m[j] & bit) return 2;
+            m[j] |= bit;
+        } else {
+            if (R.nb == 8) return 1;
+            for (int t = R.nb; t > j; --t) {
+                R.b[t] = R.b[t - 1];
+                m[t] = m[t - 1];
+            }
+            R.b[j] = first;
+            m[j] = bit;
+            ++R.nb;
+        }
+    }
+    return 0;
+}
 __device__ bool row_blocks(const int *__restrict__ ddRowPtr, const int *__restrict__ ddCol, const int *__restrict__ descColId,
                            const int *__restrict__ rId, const int *__restrict__ cdRowPtr, int i, int cols, RowBlocks &R)
 {
     const int p0 = ddRowPtr[i], n = ddRowPtr[i + 1] - p0, r = rId[i];
     R.nb = 0;
     if (n < 4 || n > 64 || cdRowPtr[r + 1] != cdRowPtr[r]) return false;
-    unsigned m[8];
-    for (int k = 0; k < n; ++k) {
-        const int c = descColId[ddCol[p0 + k]];
-        const int blk = c >> 3;
-        const unsigned bit = 1u << (c & 7);
-        if (blk + 1 > cols / 8) return false;
-        int j = 0;
-        while (j < R.nb && R.b[j] < blk) ++j;
-        if (j < R.nb && R.b[j] == blk) {
-            if (m[j] & bit) return false;
-            m[j] |= bit;
-        } else {
-            if (R.nb == 8) return false;
-            for (int t = R.nb; t > j; --t) {
-                R.b[t] = R.b[t - 1];
-                m[t] = m[t - 1];
-            }
-            R.b[j] = blk;
-            m[j] = bit;
-            ++R.nb;
+    const int on = row_blocks_at(ddCol, descColId, p0, n, cols, 0, R);
+    if (on == 2) return false;
+    int lowest = descColId[ddCol[p0]];
+    for (int k = 1; k < n; ++k) lowest = min(lowest, descColId[ddCol[p0 + k]]);
+    const int shift = lowest & 7;
+    bool ok = on == 0;
+    if (shift) {
+        RowBlocks own;
+        if (row_blocks_at(ddCol, descColId, p0, n, cols, shift, own) == 0 && (!ok || own.nb < R.nb)) {
+            R = own;
+            ok = true;
         }
     }
-    return 2 * n >= R.nb * 8;
+    return ok && 2 * n >= R.nb * 8;
 }
 
 __global__ __launch_bounds__(kBlock) void strip_candidates_kernel(const int *__restrict__ ddRowPtr, const int *__restrict__ ddCol,
@@ -141,7 +163,7 @@ __global__ __launch_bounds__(kBlock) void strip_candidates_kernel(const int *__r
     RowBlocks R;
     isCand[i] = row_blocks(ddRowPtr, ddCol, descColId, rId, cdRowPtr, i, cols, R) ? 1 : 0;
 }
-// candidates in row order: their row of A_dd, their blocks (-1 = none) and how many
+// candidates in row order: their row of A_dd, the first columns of their blocks (-1 = none) and how many
 __global__ __launch_bounds__(kBlock) void candidate_keys_kernel(const int *__restrict__ ddRowPtr, const int *__restrict__ ddCol,
                                                                 const int *__restrict__ descColId, const int *__restrict__ rId,
                                                                 const int *__restrict__ cdRowPtr, const int *__restrict__ isCand,
@@ -373,9 +395,9 @@ __global__ __launch_bounds__(64) void strip_steps_kernel(const int *__restrict__
     const int A = d[0], B = d[1], n0 = d[3], n1 = d[4];
     auto first_col = [&](int slot) {  // first column of the block in a slot, -1 = none
         const int half = slot >> 2, i = slot & 3;
-        if (half == 0) return i < n0 ? chunkKey[(size_t)A * 8 + i] * 8 : -1;
+        if (half == 0) return i < n0 ? chunkKey[(size_t)A * 8 + i] : -1;
         if (i >= n1) return -1;
-        return (B >= 0 ? chunkKey[(size_t)B * 8 + i] : chunkKey[(size_t)A * 8 + 4 + i]) * 8;
+        return B >= 0 ? chunkKey[(size_t)B * 8 + i] : chunkKey[(size_t)A * 8 + 4 + i];
     };
     if (l < mx::kTileHdr) {
         int v = 0;
@@ -409,10 +431,10 @@ __global__ __launch_bounds__(kBlock) void strip_values_kernel(const int *__restr
     const int *b = chunkKey + (size_t)chunk * 8;
     const size_t base = (size_t)chunkBlock0[chunk] * 64;
     for (int p = ddRowPtr[i]; p < ddRowPtr[i + 1]; ++p) {
-        const int c = descColId[ddCol[p]], blk = c >> 3;
+        const int c = descColId[ddCol[p]];
         int k = 0;
-        while (k < nb - 1 && b[k] < blk) ++k;
-        tcVal[base + (size_t)k * 64 + jj * 8 + (c & 7)] = ddVal[p];
+        while (k < nb - 1 && b[k] + 8 <= c) ++k;
+        tcVal[base + (size_t)k * 64 + jj * 8 + (c - b[k])] = ddVal[p];
     }
 }
 
@@ -914,7 +936,7 @@ int HybridDevice::analyse(mx_dtype dtype, int rows, int cols, int nnz, const int
             // by (block 0, .., block 7, row): eight stable passes, the last block first
             Buf permB, keyA, keyB, sortTmp;
             unsigned bits = 1;
-            while (bits < 32 && (1ull << bits) < (unsigned long long)(cols / 8) + 2ull) ++bits;
+            while (bits < 32 && (1ull << bits) < (unsigned long long)cols + 2ull) ++bits;  // (the keys are first columns + 1)
             size_t sortBytes = 0;
             MXH_TRY(rocprim::radix_sort_pairs(nullptr, sortBytes, (const unsigned *)nullptr, (unsigned *)nullptr, (const int *)nullptr,
                                               (int *)nullptr, nc, 0u, bits, s));

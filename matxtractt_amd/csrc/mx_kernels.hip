@@ -31,6 +31,7 @@ typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
 typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef double v2f64 __attribute__((ext_vector_type(2)));
 typedef int v2i32 __attribute__((ext_vector_type(2)));
+typedef v4i32 v4i32u __attribute__((aligned(2)));  // 16 bytes at the alignment of a binary16 element
 
 constexpr int kBlock = 256;  // 4 wave64 per workgroup
 using mx::kSliceBytes;
@@ -1004,11 +1005,13 @@ __global__ __launch_bounds__(kBlock) void tile_kernel(const int4 *__restrict__ w
     }
 }
 
-// The binary16 tile kernel for blocks whose eight columns are consecutive and start at a multiple
-// of eight (dense strips), for chunks of at most one step whose rows receive nothing from the CSR
-// part.  A lane's B operand -- the eight x of one block -- is
-// then one aligned 16-byte read of x, so the column ids, the gather, the trip through LDS and the
-// old y all fall away: per step a header, the blocks and 16 bytes of x per block.  The results
+// The binary16 tile kernel for blocks whose eight columns are consecutive (dense strips), for
+// chunks of at most one step whose rows receive nothing from the CSR part.  A lane's B operand --
+// the eight x of one block -- is then one 16-byte read of x (at a multiple of 16 bytes when the
+// block starts at a multiple of eight columns; a strip that starts elsewhere has blocks that start
+// there, and the read is an unaligned one, which global memory serves), so the column ids, the
+// gather, the trip through LDS and the old y all fall away: per step a header, the blocks and 16
+// bytes of x per block.  The results
 // leave from the four lanes that hold them.  Same step stream, headers and wave ranges as
 // tile_kernel; the header carries the first column of every block slot in dwords 21..28.
 struct DenseStep {
@@ -1033,7 +1036,7 @@ __device__ __forceinline__ void tile_dense_wave(const int4 *__restrict__ waveDes
     // rows 8g..8g+7 = slot 4m+g; the other lanes read what lane m&1 of their group reads
     auto fetch = [&](DenseStep &R) {
         const int base = __shfl(R.hdr, 21 + 4 * (m & 1) + g);
-        R.b = *(const v4i32 *)(x + max(base, 0));
+        R.b = *(const v4i32u *)(x + max(base, 0));
     };
     auto step = [&](int s, DenseStep &Ra, DenseStep &Rg, DenseStep &Ri) {
         issue(Ri, min(s + 4, last), __builtin_amdgcn_readlane(Ra.hdr, 19), __builtin_amdgcn_readlane(Ra.hdr, 20));

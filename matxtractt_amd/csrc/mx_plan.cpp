@@ -2038,13 +2038,15 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
         }
     }
     // binary16 rows of A_dd whose columns, in the caller's numbering, fall into at most a
-    // step's worth of aligned blocks of fragK columns (multiples of fragK) and fill them at
-    // least half -- a row of a dense strip in the simplest case -- with nothing in the
-    // residual and no column named twice: rows with the same set of blocks are put together,
-    // fragM at a time, into chunks of the plan's own (the canonical chunks follow the row
-    // order, where rows of other shapes fall between them and one chunk straddles two
-    // strips).  A chunk of at least fragM/2 rows goes to tile_dense_kernel; its rows leave the
-    // fragments.
+    // step's worth of blocks of fragK consecutive columns and fill them at least half -- a row
+    // of a dense strip in the simplest case -- with nothing in the residual and no column
+    // named twice.  The blocks of a row start at multiples of fragK, or, where that takes fewer
+    // blocks, at the row's own first column plus multiples of fragK (a strip that starts off
+    // the grid of eight is four blocks then, not five: two chunks share a step again).  Rows
+    // with the same set of blocks are put together, fragM at a time, into chunks of the plan's
+    // own (the canonical chunks follow the row order, where rows of other shapes fall between
+    // them and one chunk straddles two strips).  A chunk of at least fragM/2 rows goes to
+    // tile_dense_kernel; its rows leave the fragments.
     std::vector<char> &taken = H.taken;
     std::vector<StripChunk> &stripChunks = H.stripChunks;
     taken.clear();
@@ -2053,7 +2055,7 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
         !(std::getenv("MX_NO_STRIPS") && std::atoi(std::getenv("MX_NO_STRIPS")))) {
         constexpr int kMaxBlocks = 8;  // block slots of a binary16 step
         struct Cand {
-            int nb, b[kMaxBlocks], n, i;  // blocks (column / fragK, ascending), entries, row of A_dd
+            int nb, b[kMaxBlocks], n, i;  // first column of every block (ascending), entries, row of A_dd
         };
         std::vector<Cand> cand;
         const int nThreads = std::max(1, omp_get_max_threads());
@@ -2062,6 +2064,20 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
         {
             std::vector<Cand> &mine = found[(size_t)omp_get_thread_num()];
             std::vector<int> cols;
+            // the blocks of the sorted columns for blocks that start at shift + multiples of fragK; false
+            // when they are too many or one would reach past the end of x
+            auto blocks_at = [&](int shift, Cand &c) {
+                c.nb = 0;
+                for (int col : cols) {
+                    const int first = (col - shift) / fragK * fragK + shift;
+                    if (first + fragK > P->cols) return false;
+                    if (c.nb == 0 || c.b[c.nb - 1] != first) {
+                        if (c.nb == kMaxBlocks) return false;
+                        c.b[c.nb++] = first;
+                    }
+                }
+                return true;
+            };
 #pragma omp for schedule(static)
             for (int i = 0; i < P->dRows; ++i) {
                 const int p0 = P->ddRowPtr[i], n = P->ddRowPtr[i + 1] - p0, r = P->rId[i];
@@ -2069,19 +2085,17 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
                 cols.resize((size_t)n);
                 for (int k = 0; k < n; ++k) cols[k] = P->descColId[P->ddColInd[p0 + k]];
                 std::sort(cols.begin(), cols.end());
-                Cand c;
-                c.nb = 0;
-                c.n = n;
-                c.i = i;
-                bool ok = true;
-                for (int k = 0; k < n && ok; ++k) {
-                    if (k && cols[k] == cols[k - 1]) ok = false;  // named twice: stays with the fragments, where the last counts
-                    const int blk = cols[k] / fragK;
-                    if ((blk + 1) * fragK > P->cols) ok = false;  // the block would reach past the end of x
-                    if (c.nb == 0 || c.b[c.nb - 1] != blk) {
-                        if (c.nb == kMaxBlocks) ok = false;
-                        else c.b[c.nb++] = blk;
-                    }
+                bool twice = false;
+                for (int k = 1; k < n; ++k) twice = twice || cols[k] == cols[k - 1];
+                if (twice) continue;  // named twice: stays with the fragments, where the last counts
+                Cand c, own;
+                c.n = own.n = n;
+                c.i = own.i = i;
+                bool ok = blocks_at(0, c);
+                const int shift = cols[0] % fragK;
+                if (shift && blocks_at(shift, own) && (!ok || own.nb < c.nb)) {
+                    c = own;
+                    ok = true;
                 }
                 if (!ok || 2 * n < c.nb * fragK) continue;
                 for (int k = c.nb; k < kMaxBlocks; ++k) c.b[k] = -1;
@@ -2132,7 +2146,7 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
                 C.blocks.resize(nb);
                 for (int k = 0; k < nb; ++k) {
                     C.blocks[k].vals.assign((size_t)fragM * fragK * es, 0);
-                    for (int c = 0; c < fragK; ++c) C.blocks[k].cols[c] = cand[a].b[k] * fragK + c;
+                    for (int c = 0; c < fragK; ++c) C.blocks[k].cols[c] = cand[a].b[k] + c;
                 }
                 for (int j = 0; j < 8; ++j) C.rows[j] = -1;
                 for (int j = 0; j < nr; ++j) {
@@ -2142,8 +2156,8 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
                     C.nnz += cand[g + j].n;
                     for (int p = P->ddRowPtr[i]; p < P->ddRowPtr[i + 1]; ++p) {
                         const int c = P->descColId[P->ddColInd[p]];
-                        const int k = (int)(std::lower_bound(cand[a].b, cand[a].b + nb, c / fragK) - cand[a].b);
-                        ((uint16_t *)C.blocks[k].vals.data())[j * fragK + c % fragK] = ddv16[p];
+                        const int k = (int)(std::upper_bound(cand[a].b, cand[a].b + nb, c) - cand[a].b) - 1;
+                        ((uint16_t *)C.blocks[k].vals.data())[j * fragK + (c - cand[a].b[k])] = ddv16[p];
                     }
                 }
             }
@@ -2507,6 +2521,22 @@ static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, 
     const int S = rows > 0 ? slice_count(dtype, rows, cols, nnz, nCU) : 0;
     bool want[2] = {true, S > 0};
     const char *env = std::getenv("MX_CSR_KERNEL");
+    if ((env && !std::strcmp(env, "split")) || plan_autotune()) {
+        // The split form and the timed choice exist on the host route only: the part comes down and takes that
+        // route, so that the plan is the one mx_plan_create makes under the same settings.
+        const size_t es = (size_t)mx::elem_size(dtype);
+        std::vector<int> rp((size_t)rows + 1), ci((size_t)std::max(nnz, 1));
+        std::vector<unsigned char> va(std::max<size_t>((size_t)nnz * es, 1));
+        std::vector<char> marks;
+        MX_HIP(hipMemcpy(rp.data(), rowPtr_dev, ((size_t)rows + 1) * 4, hipMemcpyDeviceToHost));
+        if (nnz) MX_HIP(hipMemcpy(ci.data(), colInd_dev, (size_t)nnz * 4, hipMemcpyDeviceToHost));
+        if (nnz) MX_HIP(hipMemcpy(va.data(), val_dev, (size_t)nnz * es, hipMemcpyDeviceToHost));
+        if (elsewhere_dev) {
+            marks.resize((size_t)rows);
+            MX_HIP(hipMemcpy(marks.data(), elsewhere_dev, (size_t)rows, hipMemcpyDeviceToHost));
+        }
+        return setup_csr_part(plan, rp.data(), ci.data(), va.data(), flags, elsewhere_dev ? marks.data() : nullptr, segOut);
+    }
     if (flags & MX_PLAN_CSR_ROWS) want[1] = false;
     if ((flags & MX_PLAN_CSR_SLICES) && S > 0) want[0] = false;
     if (env && !std::strcmp(env, "rows")) want[0] = true, want[1] = false;
@@ -2787,6 +2817,23 @@ static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const
     int rc = need_device();
     if (rc) return rc;
     if ((rc = mx::check_csr_device(rows, cols, nnz, rowPtr_dev, colInd_dev, nullptr, who))) return rc;
+    // (what a failure has to release, also one that arrives as an exception)
+    mx_plan *plan = nullptr;
+    int *partPtr = nullptr, *partCol = nullptr;
+    void *partVal = nullptr;
+    char *stripRows = nullptr;
+    auto fail = [&](int code) {
+        (void)hipFree(partPtr);
+        (void)hipFree(partCol);
+        (void)hipFree(partVal);
+        (void)hipFree(stripRows);
+        partPtr = partCol = nullptr;
+        partVal = nullptr;
+        stripRows = nullptr;
+        mx_plan_destroy(plan);
+        plan = nullptr;
+        return code;
+    };
     try {
         hipDeviceProp_t prop;
         int dev = 0;
@@ -2821,7 +2868,7 @@ static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const
         const bool keepStrips = worth >= 1 && !cnt.blocks64 && cnt.stripBlocks > 0;
         const bool keepGeneral = worth == 2 && cnt.generalFrags > 0;
 
-        mx_plan *plan = new (std::nothrow) mx_plan();
+        plan = new (std::nothrow) mx_plan();
         if (!plan) {
             set_error(std::string(who) + ": out of memory");
             return MX_ERR_ALLOC;
@@ -2835,17 +2882,6 @@ static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const
         plan->ext_dRows = cnt.dRows;
         plan->ext_nnzRowD = cnt.nnzRowD;
         plan->ext_frags = cnt.frags;
-        int *partPtr = nullptr, *partCol = nullptr;
-        void *partVal = nullptr;
-        char *stripRows = nullptr;
-        auto fail = [&](int code) {
-            (void)hipFree(partPtr);
-            (void)hipFree(partCol);
-            (void)hipFree(partVal);
-            (void)hipFree(stripRows);
-            mx_plan_destroy(plan);
-            return code;
-        };
         if (hipStreamCreate(&plan->stream) != hipSuccess || hipEventCreate(&plan->ev0) != hipSuccess ||
             hipEventCreate(&plan->ev1) != hipSuccess) {
             set_error(std::string(who) + ": could not create stream/events");
@@ -2962,7 +2998,7 @@ static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const
         return MX_OK;
     } catch (const std::bad_alloc &) {
         set_error(std::string(who) + ": out of memory");
-        return MX_ERR_ALLOC;
+        return fail(MX_ERR_ALLOC);
     }
 }
 
@@ -3214,8 +3250,26 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     return MX_OK;
 }
 
+// What a plan asks of x before anything is launched: 16-byte alignment where a kernel copies x in 16-byte
+// vectors (the slice forms of the CSR part) or reads it in aligned 16-byte pieces with no other way to run
+// (the binary64 8 x 8 blocks; the binary16 strips read at any alignment).
+static int check_x(const mx_plan *plan, const void *x, const char *who)
+{
+    if (!((uintptr_t)x & 15)) return MX_OK;
+    if (plan->csr_variant != 0) {
+        set_error(std::string(who) + ": x must be 16-byte aligned for this plan (its CSR part keeps x in LDS)");
+        return MX_ERR_ARG;
+    }
+    if (plan->dtype == MX_F64 && plan->strips.dense && plan->strips.nWaves > 0) {
+        set_error(std::string(who) + ": x must be 16-byte aligned for this plan (its 8 x 8 blocks read x in aligned 16-byte pieces)");
+        return MX_ERR_ARG;
+    }
+    return MX_OK;
+}
+
 static int spmv_on(mx_plan *plan, const void *x, void *y, hipStream_t s, void *partial = nullptr)
 {
+    if (int bad = check_x(plan, x, "mx_spmv")) return bad;
     // the strips ride in the launch of the combine kernel when the CSR part has one (MX_STRIPS_APART=1:
     // a launch of their own, as with the row-tile form of the CSR part)
     static const bool apart = std::getenv("MX_STRIPS_APART") && std::atoi(std::getenv("MX_STRIPS_APART"));
@@ -3309,6 +3363,7 @@ extern "C" int mx_time_csr_main(mx_plan *plan, const void *x_dev, void *y_dev, i
         return MX_ERR_ARG;
     }
     hipStream_t s = plan->stream;
+    if (int bad = check_x(plan, x_dev, "mx_time_csr_main")) return bad;
     int rc = time_loop(plan, warm, iters, [&]() -> int {
         // the kernel that holds most of the entries
         if (plan->csr_variant == 1 && plan->fused)
@@ -3336,28 +3391,57 @@ extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, 
     hipStream_t s = plan->stream;
     int rc;
     double t = 0.0;
+    if ((rc = check_x(plan, x_dev, "mx_time"))) return rc;
     if (ms_total) {
         rc = time_loop(plan, warm, iters, [&]() { return spmv_on(plan, x_dev, y_dev, s); }, &t);
         if (rc) return rc;
         *ms_total = t;
     }
-    if (ms_csr) {
-        rc = time_loop(plan, warm, iters, [&]() { return launch_csr_part(plan, x_dev, y_dev, 0, s); }, &t);
+    // The reference adds up two numbers, tile part and residual part, each timed alone
+    // (test/test_autotc_spmv.cpp:1561-1572).  A plan whose strips or blocks ride in the combine kernel's
+    // launch has no tile kernel of its own: ms_csr is then the CSR part as the product runs it, riders
+    // included, and ms_tile what they add to that launch (the same launches without them taken off).
+    static const bool apart = std::getenv("MX_STRIPS_APART") && std::atoi(std::getenv("MX_STRIPS_APART"));
+    const bool ride = plan->dtype == MX_F64 ? (plan->csr_variant == 1 && plan->strips.vidx != nullptr)
+                                            : (!apart && plan->csr_variant == 1 && mx::strips_can_ride(plan->dtype, plan->strips, x_dev));
+    void *wide = plan->tiles.nWaves > 0 ? plan->ywide : nullptr;
+    const bool blocksApart = !ride && plan->dtype == MX_F64 && plan->strips.nWaves > 0;  // binary64 blocks in a launch of their own
+    double tBare = 0.0;
+    if (ms_csr || (ms_tile && (ride || blocksApart))) {
+        rc = time_loop(plan, warm, iters, [&]() { return launch_csr_part(plan, x_dev, y_dev, 0, s, ride ? &plan->strips : nullptr, nullptr, wide); }, &t);
         if (rc) return rc;
-        *ms_csr = t;
+        if (ms_csr) *ms_csr = t;
+        if (ms_tile && ride) {
+            // (the rows of riders are left alone by the bare launch: nothing is added to them, y stays bounded)
+            rc = time_loop(plan, warm, iters, [&]() { return launch_csr_part(plan, x_dev, y_dev, 0, s, nullptr, nullptr, wide); }, &tBare);
+            if (rc) return rc;
+        }
     }
     if (ms_tile) {
-        *ms_tile = 0.0;
-        if (plan->tiles.chunkNum + plan->strips.chunkNum > 0) {
+        *ms_tile = ride ? std::max(0.0, t - tBare) : 0.0;
+        if (plan->tiles.chunkNum > 0 || (!ride && !blocksApart && plan->strips.chunkNum > 0)) {
             // overwrite mode: the timed loop must not grow y without bound
+            double tt = 0.0;
             rc = time_loop(plan, warm, iters, [&]() -> int {
                 MX_HIP(mx::launch_tiles(plan->dtype, plan->tiles, x_dev, y_dev, 0, s));
-                // (binary64 blocks always add to y: a few thousand additions stay far from overflow)
-                MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x_dev, y_dev, plan->dtype == MX_F64 ? 1 : 0, s));
+                if (!ride && !blocksApart) MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x_dev, y_dev, 0, s));
                 return MX_OK;
-            }, &t);
+            }, &tt);
             if (rc) return rc;
-            *ms_tile = t;
+            *ms_tile += tt;
+        }
+        if (blocksApart) {
+            // the block kernel adds to y, so it is priced as the pair (CSR part, blocks) less the CSR part: the
+            // CSR part rewrites y before every launch of the blocks
+            double pair = 0.0;
+            rc = time_loop(plan, warm, iters, [&]() -> int {
+                int r = launch_csr_part(plan, x_dev, y_dev, 0, s, nullptr, nullptr, wide);
+                if (r) return r;
+                MX_HIP(mx::launch_tiles(plan->dtype, plan->strips, x_dev, y_dev, 1, s));
+                return MX_OK;
+            }, &pair);
+            if (rc) return rc;
+            *ms_tile += std::max(0.0, pair - t);
         }
     }
     // leave y holding the product
@@ -3365,6 +3449,27 @@ extern "C" int mx_time(mx_plan *plan, const void *x_dev, void *y_dev, int warm, 
     if (rc) return rc;
     MX_HIP(hipStreamSynchronize(s));
     return MX_OK;
+}
+
+extern "C" int mx_time_rotate(mx_plan *const *plans, const void *const *x_dev, void *const *y_dev, int n, int warm, int iters, double *ms)
+{
+    if (!plans || !x_dev || !y_dev || n < 1 || warm < 0 || iters <= 0 || !ms) {
+        set_error("mx_time_rotate: bad argument");
+        return MX_ERR_ARG;
+    }
+    for (int i = 0; i < n; ++i)
+        if (!plans[i] || !x_dev[i] || !y_dev[i]) {
+            set_error("mx_time_rotate: null plan or vector");
+            return MX_ERR_ARG;
+        }
+    mx_plan *first = plans[0];
+    hipStream_t s = first->stream;
+    int turn = 0;
+    return time_loop(first, warm, iters, [&]() -> int {
+        const int i = turn;
+        turn = (turn + 1) % n;
+        return spmv_on(plans[i], x_dev[i], y_dev[i], s);
+    }, ms);
 }
 
 // One record per kernel launch of a product, in launch order: its mean time alone (same protocol as
@@ -3398,10 +3503,7 @@ extern "C" int mx_time_kernels(mx_plan *plan, const void *x_dev, void *y_dev, in
         rc = time_loop(plan, warm, iters, body, &K.ms);
         ++n;
     };
-    if (plan->csr_variant != 0 && ((uintptr_t)x_dev & 15)) {
-        set_error("mx_time_kernels: x must be 16-byte aligned for this plan");
-        return MX_ERR_ARG;
-    }
+    if ((rc = check_x(plan, x_dev, "mx_time_kernels"))) return rc;
     bool xCounted = false;
     if (plan->csr_variant != 1 && plan->csr.nBlocks > 0) {
         const bool last = plan->csr_variant == 0;  // writes y for good

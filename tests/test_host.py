@@ -50,6 +50,25 @@ def test_partition_bit_exact_on_synthetic_workloads(mx, ora, cfg, scale):
         P.close()
 
 
+@pytest.mark.parametrize("cfg,taus", [(3, [(0.75, 0.5), (1.0, 1.0)]), (4, [(0.5, 0.25), (1.0, 1.0)]),
+                                      (5, [(1.0, 1.0), (0.5, 0.25), (0.37, 0.11)])])
+def test_partition_bit_exact_at_full_size(mx, ora, cfg, taus):
+    """The partition at the sizes the benchmark runs, array for array against the oracle: above 2^24 entries
+    (workloads 3 and 5) the reference's `int dColsNnz = nnzA * colProp` is a binary32 product that rounds
+    (test/test_autotc_spmv.cpp:1131, :1249), and at tau = 1 on workload 5 the rounded target lies beyond the
+    matrix, where every line with an entry is taken (63.3 M entries in tiles)."""
+    A, _ = mx.gen_config(cfg)
+    for tau in taus:
+        P = mx.Partition(A, *tau)
+        O = ora.partition(A.rowPtr, A.colInd, A.val, A.cols, *tau)
+        assert_same_partition(P, O)
+        assert P.nnzRowD + P.nnzCD == A.nnz
+        if tau == (1.0, 1.0):
+            assert P.nnzRowD == A.nnz and P.nnzCD == 0
+        P.close()
+        del O
+
+
 @pytest.mark.parametrize("seed", range(8))
 @pytest.mark.parametrize("dtype", [np.float64, np.float16])
 def test_partition_bit_exact_on_hostile_inputs(mx, ora, seed, dtype):
@@ -154,6 +173,44 @@ def test_generator_shapes(mx):
     strip = [r for r in range(0, A.rows, 8) if np.all(lens[r:r + 8] == 32) and
              np.all(np.diff(A.colInd[A.rowPtr[r]:A.rowPtr[r + 1]]) == 1)]
     assert 0.12 <= 8 * len(strip) / A.rows <= 0.28
+
+
+def test_generators_with_structure_off_the_grid(mx, ora):
+    """MX_GEN_UNALIGNED: the 8 x 8 blocks of workload 2 start at any column of their band and the strips of workload
+    5 at a column that is not a multiple of eight; everything else about the matrices stays as it was (sizes, row
+    lengths, sorted distinct columns), and the partition of such a matrix equals the oracle's."""
+    for cfg, scale in ((2, 1 / 8), (5, 1 / 64)):
+        A, _ = mx.gen_config(cfg, scale=scale)
+        U, x = mx.gen_config(cfg, scale=scale, unaligned=True)
+        assert U.rows == A.rows and U.cols == A.cols and U.dtype == A.dtype
+        assert U.colInd.min() >= 0 and U.colInd.max() < U.cols
+        rowOf = np.repeat(np.arange(U.rows), np.diff(U.rowPtr))
+        assert np.all((np.diff(U.colInd) > 0) | (np.diff(rowOf) != 0))
+        # runs of at least eight consecutive columns, and where they start
+        brk = np.ones(U.nnz, bool)
+        brk[1:] = (np.diff(U.colInd) != 1) | (np.diff(rowOf) != 0)
+        starts = np.nonzero(brk)[0]
+        big = np.diff(np.append(starts, U.nnz)) >= 8
+        off = np.bincount(U.colInd[starts[big]] % 8, minlength=8) / big.sum()
+        if cfg == 2:
+            assert np.all(np.diff(U.rowPtr) == 64) and U.nnz == A.nnz
+            assert off.min() > 0.08                    # every offset about as often as any other
+            # the dense blocks are still there: eight rows from a multiple of eight share the run
+            r = int(rowOf[starts[big][len(starts[big]) // 2]]) // 8 * 8
+            c0 = int(U.colInd[starts[big][len(starts[big]) // 2]])
+            for rr in range(r, r + 8):
+                assert np.isin(np.arange(c0, c0 + 8), U.colInd[U.rowPtr[rr]:U.rowPtr[rr + 1]]).all()
+        else:
+            lens = np.diff(U.rowPtr)
+            strip = [r for r in range(0, U.rows, 8) if np.all(lens[r:r + 8] == 32) and
+                     np.all(np.diff(U.colInd[U.rowPtr[r]:U.rowPtr[r + 1]]) == 1)]
+            assert 0.12 <= 8 * len(strip) / U.rows <= 0.28
+            at = np.array([U.colInd[U.rowPtr[r]] % 8 for r in strip])
+            assert (at == 0).mean() < 0.05              # (a strip pushed back from the last columns may land on the grid)
+        for tau in ((1.0, 1.0), (0.5, 0.25)):
+            P = mx.Partition(U, *tau)
+            assert_same_partition(P, ora.partition(U.rowPtr, U.colInd, U.val, U.cols, *tau))
+            P.close()
 
 
 # ---------------------------------------------------------------- Matrix-Market ingest
