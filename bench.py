@@ -224,7 +224,9 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
         t3 = time.perf_counter()
         return part, plan, {"partition_ms": (t1 - t0) * 1e3, "plan_create_ms": (t2 - t1) * 1e3,
                             "first_spmv_ms": (t3 - t2) * 1e3, "total_ms": (t3 - t0) * 1e3}
-    part, plan, host_route = first_y(False)
+    # "host": what a caller of the reference's surface gets (matxtract_preprocess + mx_plan_create, host arrays in):
+    # the extraction on the GPU for a matrix of two million entries or more, the plan from the partition's device arrays
+    part, plan, host_route = first_y(None)
     route = {"host": host_route}
     info = plan.info
     if not brief:

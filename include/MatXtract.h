@@ -212,11 +212,13 @@ inline void exclusive_scan(indT *input, int length)
  * column pass with colProp (global_col), row pass with rowProp (local_row), tile format,
  * residual.  Returns NULL after printing the reason when the arguments are rejected
  * (colProp < rowProp, as at :1064-1069).  Inspect with mx_partition_get(); release with
- * mx_partition_destroy().  onDevice: the extraction runs on the GPU (mx_partition_create_device); the
- * partition is the same. */
+ * mx_partition_destroy().  onDevice: 1 = the extraction runs on the GPU (mx_partition_create_device: the
+ * same partition, whose arrays come to the host when they are asked for), 0 = on the host, -1 (default) = on the
+ * GPU for a matrix of two million entries or more when there is one, on the host otherwise. */
 inline mx_partition *matxtract_preprocess(valT *csrVal, indT *csrRowPtr, indT *csrColInd, int rowA, int colA, indT nnzA,
-                                          float colProp, float rowProp, bool onDevice = false)
+                                          float colProp, float rowProp, int onDevice = -1)
 {
+    if (onDevice < 0) onDevice = nnzA >= (1 << 21) && (colProp != 0.0f || rowProp != 0.0f) && mx_device_count() > 0;
     mx_csr A;
     A.rows = rowA;
     A.cols = colA;

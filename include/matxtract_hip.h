@@ -189,12 +189,21 @@ int mx_tiles_device(mx_dtype dtype, int dRows, int dCols, int nnzRowD, const int
                     const void *ddVal_dev, mx_device_tiles *out, void *stream);
 void mx_tiles_device_free(mx_device_tiles *t);
 
-/* mx_partition_create by the device route: A (host arrays, as there) is uploaded, the three
- * steps above run on the device and the arrays are copied back into the same kind of handle --
- * every array, count and the checksum (mx_partition_hash) equal mx_partition_create's, so plans,
- * files and callers cannot tell the routes apart.  tau = (0, 0) extracts nothing and is handed to
- * the host routine.  MX_ERR_DEVICE without a HIP device: there is no silent fallback. */
+/* mx_partition_create by the device route: A (host arrays, as there) is uploaded and the three
+ * steps above run on the device; the handle is the same kind of handle -- every array, count and
+ * the checksum (mx_partition_hash) equal mx_partition_create's, so plans, files and callers cannot
+ * tell the routes apart.  The arrays stay in device memory, held by the handle, until somebody asks
+ * for them: mx_partition_get, mx_partition_hash and mx_partition_save copy them to the host first
+ * (once); mx_plan_create makes its plan from them where they are and never asks, which is what
+ * takes a caller of the reference's surface from the matrix to the first y in tens of milliseconds
+ * instead of a second on the largest workload; mx_partition_counts gives the counts without the
+ * arrays.  tau = (0, 0) extracts nothing and is handed to the host routine.  MX_ERR_DEVICE without a
+ * HIP device: there is no silent fallback. */
 int mx_partition_create_device(const mx_csr *A, float tau_c, float tau_r, mx_partition **out);
+/* The counts of a partition (every field of the view that is not a pointer: the sizes, cols_ratio,
+ * tc_nnz_ratio, the thresholds) without asking for its arrays; the pointers are filled in as well when the
+ * arrays are in host memory already and are NULL otherwise. */
+int mx_partition_counts(const mx_partition *p, mx_partition_view *view);
 
 /* mmio_allinone (utilities/mmio.cpp:1547-1713): Matrix-Market coordinate file -> CSR with
  * entries kept in file order inside each row, symmetric/hermitian files expanded,
@@ -337,12 +346,13 @@ int mx_spmv(mx_plan *plan, const void *x_dev, void *y_dev, void *stream);
  * compute calls allocate on every call (src/spmv_kernel/cdSpMV.cu:407-418).  Same arguments,
  * same kernels and bit-for-bit the same y as mx_spmv; the one buffer the kernels need beyond
  * the plan's arrays, x and y -- the sums of the virtual rows that csr_slice_kernel hands to
- * slice_combine_kernel -- lives in a fixed array of mx_static_scratch_bytes() (16 MiB) that is
+ * slice_combine_kernel -- lives in a fixed array of mx_static_scratch_bytes() (32 MiB) that is
  * part of the library's code object on every GPU it runs on (held until the process ends) and
  * is addressed through hipGetSymbolAddress once per device.  The call itself allocates
  * nothing, frees nothing and calls no allocating routine.  A plan whose sums need more than
- * the array holds is refused with MX_ERR_ARG and a message that says so (the mixed workload at
- * full size: 27 MB).  Every call on one GPU shares that GPU's array: calls that overlap in time
+ * the array holds is refused with MX_ERR_ARG and a message that says so (the largest benchmark
+ * workload, the mixed one at full size, needs 27 MB and fits).  A plan in the one-launch form runs
+ * its two-launch form here, whose sums are the ones that go to the array.  Every call on one GPU shares that GPU's array: calls that overlap in time
  * on one GPU -- also through different plans or streams -- race.  Nothing in the array has to
  * start at zero: every sum the second kernel reads is written by the first in the same call. */
 int mx_spmv_static(mx_plan *plan, const void *x_dev, void *y_dev, void *stream);

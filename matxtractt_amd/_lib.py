@@ -118,6 +118,7 @@ SIGNATURES = {
     "mx_partition_create_device": (_i, [C.POINTER(CsrStruct), C.c_float, C.c_float, _pp]),
     "mx_partition_destroy": (None, [_vp]),
     "mx_partition_get": (_i, [_vp, C.POINTER(PartitionView)]),
+    "mx_partition_counts": (_i, [_vp, C.POINTER(PartitionView)]),
     "mx_partition_hash": (C.c_uint64, [_vp]),
     "mx_partition_save": (_i, [_vp, C.c_char_p]),
     "mx_partition_load": (_i, [C.c_char_p, _i, _pp]),

@@ -216,10 +216,14 @@ class Partition:
               "sparse_AToX_index", "fragPtr", "fragBit", "tcVal", "cdRowPtr", "cdColInd", "cdVal")
 
     def __init__(self, A, tau_c, tau_r, device=False):
-        """device=True: the extraction runs on the GPU (mx_partition_create_device); same result."""
+        """device=True: the extraction runs on the GPU (mx_partition_create_device); same result.  device=None:
+        what the reference's surface does (matxtract_preprocess, the CLI): the GPU for a matrix of two million
+        entries or more when there is one, the host otherwise."""
         self._h = C.c_void_p()
         self._A = A  # keep the input arrays alive during the call
         st = A.struct()
+        if device is None:
+            device = A.nnz >= (1 << 21) and (tau_c != 0 or tau_r != 0) and _lib.load().mx_device_count() > 0
         create = _lib.load().mx_partition_create_device if device else _lib.load().mx_partition_create
         check(create(C.byref(st), float(tau_c), float(tau_r), C.byref(self._h)))
         self._bind()
@@ -239,11 +243,20 @@ class Partition:
         check(_lib.load().mx_partition_save(self._h, os.fsencode(path)))
 
     def _bind(self):
+        """The counts now; the arrays when one of them is asked for (a partition made on the device keeps them
+        there until then, and a plan made from it never asks)."""
         v = _lib.PartitionView()
-        check(_lib.load().mx_partition_get(self._h, C.byref(v)))
+        check(_lib.load().mx_partition_counts(self._h, C.byref(v)))
         for name, _ in _lib.PartitionView._fields_:
             if name not in self.ARRAYS:
                 setattr(self, name, getattr(v, name))
+        self.tau_c, self.tau_r = float(v.tau_c), float(v.tau_r)
+
+    def __getattr__(self, name):
+        if name not in Partition.ARRAYS or "_h" not in self.__dict__:
+            raise AttributeError(name)
+        v = _lib.PartitionView()
+        check(_lib.load().mx_partition_get(self._h, C.byref(v)))
         vt = _np_dtype(v.dtype)
         bt = np.uint32 if v.dtype == MX_F64 else np.uint64
         self.descColId = _view(v.descColId, v.cols if v.descColId else 0, np.int32)
@@ -261,7 +274,7 @@ class Partition:
         self.cdRowPtr = _view(v.cdRowPtr, v.rows + 1, np.int32)
         self.cdColInd = _view(v.cdColInd, v.nnzCD, np.int32)
         self.cdVal = _view(v.cdVal, v.nnzCD, vt)
-        self.tau_c, self.tau_r = float(v.tau_c), float(v.tau_r)
+        return self.__dict__[name]
 
     @property
     def hash(self):

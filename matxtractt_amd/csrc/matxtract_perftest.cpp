@@ -9,8 +9,8 @@
 // (default 200 / 4000), --no-tiles / --all-tiles (plan flags), --json (one JSON record on the
 // last line), --tune (pick the two fractions from the 5x5 grid by timing each on the device,
 // then run with them), --estimate-tau (pick them from counts over the same grid, nothing timed), --partition-cache FILE (read the partition from FILE when it was made for a
-// matrix of this shape with these fractions, otherwise compute it and write FILE), --device-prep (the extraction runs on the GPU instead of the
-// host cores; same partition), --device-plan (the matrix is uploaded as it is and everything after
+// matrix of this shape with these fractions, otherwise compute it and write FILE), --device-prep / --host-prep (the extraction runs on the GPU /
+// on the host cores; same partition; without either the GPU takes matrices of two million entries or more), --device-plan (the matrix is uploaded as it is and everything after
 // that -- extraction, the plan's decisions, its layouts -- happens on the GPU: mx_plan_create_device;
 // same plan, no partition on the host, so no --partition-cache and no checksum in the JSON record).
 // Precision is the build's: -Dfp64 -> FP64 binary, otherwise FP16.
@@ -97,7 +97,8 @@ int main(int argc, char **argv)
     int config = 0, warm = 200, iters = 4000, planFlags = MX_PLAN_DEFAULT;
     double scale = 1.0;
     unsigned long long seed = 0;
-    bool keepValues = false, json = false, tune = false, estimate = false, devicePrep = false, devicePlan = false;
+    bool keepValues = false, json = false, tune = false, estimate = false, devicePlan = false;
+    int devicePrep = -1;  // -1: the GPU for a matrix of two million entries or more, the host otherwise
     std::string cachePath;
     for (int i = 1; i < argc; ++i) {
         std::string a = argv[i];
@@ -121,7 +122,8 @@ int main(int argc, char **argv)
         else if (a == "--partition-cache") cachePath = next("--partition-cache");
         else if (a == "--tune") tune = true;
         else if (a == "--estimate-tau") estimate = true;
-        else if (a == "--device-prep") devicePrep = true;
+        else if (a == "--device-prep") devicePrep = 1;
+        else if (a == "--host-prep") devicePrep = 0;
         else if (a == "--device-plan") devicePlan = true;
         else pos.push_back(a);
     }
@@ -225,6 +227,7 @@ int main(int argc, char **argv)
         std::cout << "---------------------------------------------------------" << std::endl;
         std::cout << "---------------------Compression Info--------------------" << std::endl;
     }
+    if (devicePrep < 0) devicePrep = nnzA >= (1 << 21) && extracting && mx_device_count() > 0;
     if (devicePrep || devicePlan) (void)hipFree(nullptr);  // the first use of the device is not part of the preprocessing time
     auto t0 = std::chrono::steady_clock::now();
     mx_partition *part = nullptr;
@@ -281,7 +284,7 @@ int main(int argc, char **argv)
             else printf("partition written to %s\n", cachePath.c_str());
         }
         preprocess_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
-        mx_partition_get(part, &pv);
+        mx_partition_counts(part, &pv);  // (the arrays of a partition made on the device stay there: the plan is made from them)
     }
     if (extracting) {
         printf("cols_ratio = %f \n", pv.cols_ratio);

@@ -167,7 +167,7 @@ constexpr int kSliceLightSegs = 8;     // rows with at most this many virtual ro
 // The sums of the virtual rows (DeviceSlices::partial) of mx_spmv_static live in a fixed array
 // in device memory instead of the plan's own buffer: static_scratch gives the address of the
 // current device's copy (looked up once per device, no allocation).
-constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;  // the largest benchmark workload needs 27 MB
 hipError_t static_scratch(void **ptr);
 
 }  // namespace mx
@@ -216,6 +216,19 @@ int upload_csr_device(mx_dtype dtype, int rows, int cols, int nnz, const int *ro
 // caller's numbering, in new device arrays that pass to the caller; strip_layout() lays the
 // binary16 strip chunks out as steps (the caller plans the steps from the chunks' block counts,
 // as the host route does).  All arrays equal the host route's byte for byte.
+// The device arrays of a partition that was made on the device (mx_partition::twin): the two orders, A_dd and
+// the residual, the tile encoding.  HybridDevice::adopt plans from them without any copy.
+struct PartitionTwin {
+    mx_dtype dtype = MX_F64;
+    int rows = 0, cols = 0, nnz = 0, dRows = 0, dCols = 0, nDD = 0, nCD = 0;
+    void *order = nullptr;  // descColId [cols], descRowId [rows] (its first dRows are rId)
+    int *dc = nullptr, *dr = nullptr;
+    void *split = nullptr;  // ddRowPtr, ddColInd, ddVal, cdRowPtr, cdColInd, cdVal
+    int *ddp = nullptr, *ddc = nullptr, *cdp = nullptr, *cdc = nullptr;
+    void *ddv = nullptr, *cdv = nullptr;
+    mx_device_tiles T{};
+};
+
 struct HybridCounts {
     long long generalFrags = 0, generalEntries = 0;  // fragments that pass the fill gate (after the strips took their rows)
     long long stripEntries = 0, stripBlocks = 0;     // binary16 strip chunks, or binary64 8 x 8 blocks (blocks64)
@@ -233,6 +246,9 @@ struct HybridDevice {
     // minVals: entries a fragment needs to pass the gate; want*: which forms the flags allow
     int analyse(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, const void *val_dev, float tau_c,
                 float tau_r, int minVals, bool wantGeneral, bool wantStrips, bool wantBlocks, HybridCounts *counts, hipStream_t s);
+    // the same counts for an extraction that is there already: the arrays of `twin` are used where they are and
+    // stay the twin's
+    int adopt(const PartitionTwin &twin, int minVals, bool wantGeneral, bool wantStrips, bool wantBlocks, HybridCounts *counts, hipStream_t s);
     // stripRows_dev: marks of the rows the strips write (null when keepStrips is false or there are none).
     // keepGeneral: the fragments that pass the gate go to the general tile form -- tile_chunks and tile_layout
     // come first then, and the values of that layout are filled here.

@@ -817,8 +817,19 @@ struct HybridDevice::Impl {
     int nBlk = 0, nBlkChunks = 0;
     Buf blkKey, blkPay, blkBr, blkBc, entryBlock, blkChunkIdIncl, blkChunkStart, blkChunkBr;
     void *tileVal = nullptr;  // the values of the general tile layout (owned by the caller's DeviceTiles): csr_part fills them
-    ~Impl() { mx_tiles_device_free(&T); }
+    bool borrowed = false;    // the extraction's arrays belong to a partition's twin: not released here
+    ~Impl()
+    {
+        if (borrowed) {
+            (void)order.take();
+            (void)split.take();
+        } else {
+            mx_tiles_device_free(&T);
+        }
+    }
 };
+
+static int analyse_tail(HybridDevice::Impl &I, bool wantGeneral, bool wantStrips, bool wantBlocks, HybridCounts *counts);
 
 HybridDevice::~HybridDevice() { delete impl; }
 
@@ -868,7 +879,49 @@ int HybridDevice::analyse(mx_dtype dtype, int rows, int cols, int nnz, const int
     if (rc != MX_OK) return rc;
     rc = mx_tiles_device(dtype, I.dRows, I.dCols, I.nDD, I.ddp, I.ddc, I.ddv, &I.T, s);
     if (rc != MX_OK) return rc;
+    return analyse_tail(I, wantGeneral, wantStrips, wantBlocks, counts);
+}
 
+int HybridDevice::adopt(const PartitionTwin &W, int minVals, bool wantGeneral, bool wantStrips, bool wantBlocks, HybridCounts *counts,
+                        hipStream_t s)
+{
+    delete impl;
+    impl = new Impl();
+    Impl &I = *impl;
+    I.dtype = W.dtype;
+    I.rows = W.rows;
+    I.cols = W.cols;
+    I.nnz = W.nnz;
+    I.s = s;
+    I.minVals = minVals;
+    I.dRows = W.dRows;
+    I.dCols = W.dCols;
+    I.nDD = W.nDD;
+    I.nCD = W.nCD;
+    I.borrowed = true;
+    I.order.p = W.order;
+    I.dc = W.dc;
+    I.dr = W.dr;
+    I.split.p = W.split;
+    I.ddp = W.ddp;
+    I.ddc = W.ddc;
+    I.ddv = W.ddv;
+    I.cdp = W.cdp;
+    I.cdc = W.cdc;
+    I.cdv = W.cdv;
+    I.T = W.T;
+    *counts = HybridCounts();
+    return analyse_tail(I, wantGeneral, wantStrips, wantBlocks, counts);
+}
+
+// What follows the extraction, whoever made it: the maps back to the caller's numbering, the strip rows, the
+// blocks, the fill gate, and the counts the plan decides from.
+static int analyse_tail(HybridDevice::Impl &I, bool wantGeneral, bool wantStrips, bool wantBlocks, HybridCounts *counts)
+{
+    using namespace mxh;
+    const mx_dtype dtype = I.dtype;
+    const int rows = I.rows, cols = I.cols, minVals = I.minVals;
+    hipStream_t s = I.s;
     // columns of the residual's numbering -> the caller's; the row of A_dd of every row
     {
         Buf flag, notSel, pos, tmp;

@@ -61,10 +61,27 @@ struct mx_partition {
     int nnzCD = 0;
     std::vector<int> cdRowPtr, cdColInd;
     mx::ValBuf cdVal;
+    // A partition made on the device (mx_partition_create_device) keeps its arrays there: `twin` owns them and is
+    // released with the partition.  The vectors above are filled from them when somebody asks for the arrays
+    // (mx::partition_host); until then only the counts are set and host_ready is false.  A plan made from such a
+    // partition works on the device arrays and never asks.
+    bool host_ready = true;
+    void *twin = nullptr;
+    int (*twin_download)(mx_partition *) = nullptr;
+    void (*twin_free)(void *) = nullptr;
+    mx_partition() = default;
+    mx_partition(const mx_partition &) = delete;
+    mx_partition &operator=(const mx_partition &) = delete;
+    ~mx_partition()
+    {
+        if (twin && twin_free) twin_free(twin);
+    }
 };
 
 namespace mx {
 // The argument checks of mx_partition_create (null pointers, shape, tau range and order, rowPtr
 // monotone over [0, nnz], column range); *out is cleared.
 int check_partition_args(const mx_csr *A, float tau_c, float tau_r, mx_partition **out);
+// The arrays of `p` in host memory: copies them down first when they still live on the device only.
+int partition_host(const mx_partition *p);
 }  // namespace mx

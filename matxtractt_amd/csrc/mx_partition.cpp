@@ -12,6 +12,7 @@
 //   * tiles are built per 8-row chunk from those sorted rows (:502-585, :718-978).
 // Rows are independent, so steps run under OpenMP.
 #include <algorithm>
+#include <mutex>
 #include <cstdio>
 #include <cstring>
 #include <numeric>
@@ -380,12 +381,40 @@ extern "C" int mx_partition_create(const mx_csr *A, float tau_c, float tau_r, mx
 
 extern "C" void mx_partition_destroy(mx_partition *p) { delete p; }
 
+int mx::partition_host(const mx_partition *p)
+{
+    static std::mutex lock;
+    std::lock_guard<std::mutex> hold(lock);
+    if (p->host_ready) return MX_OK;
+    if (!p->twin || !p->twin_download) {
+        set_error("partition: its arrays are nowhere");
+        return MX_ERR_ARG;
+    }
+    return p->twin_download(const_cast<mx_partition *>(p));
+}
+
+static int partition_view(const mx_partition *p, mx_partition_view *v, bool arrays);
 extern "C" int mx_partition_get(const mx_partition *p, mx_partition_view *v)
 {
     if (!p || !v) {
         set_error("mx_partition_get: null argument");
         return MX_ERR_ARG;
     }
+    const int rc = mx::partition_host(p);
+    if (rc) return rc;
+    return partition_view(p, v, true);
+}
+extern "C" int mx_partition_counts(const mx_partition *p, mx_partition_view *v)
+{
+    if (!p || !v) {
+        set_error("mx_partition_counts: null argument");
+        return MX_ERR_ARG;
+    }
+    return partition_view(p, v, p->host_ready);
+}
+static int partition_view(const mx_partition *p, mx_partition_view *v, bool arrays)
+{
+    std::memset(v, 0, sizeof(*v));
     v->dtype = p->dtype;
     v->rows = p->rows;
     v->cols = p->cols;
@@ -423,12 +452,17 @@ extern "C" int mx_partition_get(const mx_partition *p, mx_partition_view *v)
     v->cdVal = p->cdVal.data();
     v->tau_c = p->tau_c;
     v->tau_r = p->tau_r;
+    if (!arrays) {  // the counts alone: the arrays are still on the device
+        v->descColId = v->newArray = v->rId = v->newArray_ = v->ddRowPtr = v->ddColInd = nullptr;
+        v->chunkPtr = v->sparse_AToX_index = v->fragPtr = v->cdRowPtr = v->cdColInd = nullptr;
+        v->ddVal = v->fragBit = v->tcVal = v->cdVal = nullptr;
+    }
     return MX_OK;
 }
 
 extern "C" uint64_t mx_partition_hash(const mx_partition *p)
 {
-    if (!p) return 0;
+    if (!p || mx::partition_host(p) != MX_OK) return 0;
     uint64_t h = 14695981039346656037ull;
     const int es = mx::elem_size(p->dtype);
     h = fnv(&p->dCols, 4, h);
@@ -513,6 +547,7 @@ extern "C" int mx_partition_save(const mx_partition *p, const char *path)
         set_error("mx_partition_save: null argument");
         return MX_ERR_ARG;
     }
+    if (int rc = mx::partition_host(p)) return rc;
     FILE *f = fopen(path, "wb");
     if (!f) {
         set_error(std::string("mx_partition_save: cannot open ") + path);

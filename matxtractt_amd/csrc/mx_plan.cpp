@@ -1574,7 +1574,7 @@ static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate
         return MX_ERR_ARG;
     }
     if (plan->csr_variant != 1) MX_HIP(mx::launch_csr(plan->dtype, plan->csr, x, y, accumulate, s, ywide));
-    if (plan->csr_variant == 1 && plan->fused && !strips) {
+    if (plan->csr_variant == 1 && plan->fused && !strips && !partial) {  // (sums in a caller's buffer: the two launches)
         // one launch.  A workgroup that found its share of the work taken already has said so in the
         // host-visible word: the products since the last look cannot be trusted, and from here on every
         // plan takes the two launches.
@@ -1597,9 +1597,7 @@ static int launch_csr_part(mx_plan *plan, const void *x, void *y, int accumulate
                       "products since the previous call may be wrong; plans use the two-launch form from now on");
             return MX_ERR_DEVICE;
         } else {
-            mx::DeviceSlices L = plan->slices;  // a view: same arrays, maybe other sums
-            if (partial) L.partial = partial;
-            MX_HIP(mx::launch_fused(plan->dtype, L, x, y, accumulate, s, ywide, word, plan->fused_seq++));
+            MX_HIP(mx::launch_fused(plan->dtype, plan->slices, x, y, accumulate, s, ywide, word, plan->fused_seq++));
             return MX_OK;
         }
     }
@@ -2372,8 +2370,23 @@ static int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, P
 }
 
 static int create_plan(const mx_partition *P, int flags, mx_plan **out, bool noBlocks);
+static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev, const void *val_dev,
+                              float tau_c, float tau_r, int flags, mx_plan **out, bool noBlocks, const mx::PartitionTwin *twin);
 extern "C" int mx_plan_create(const mx_partition *P, int flags, mx_plan **out)
 {
+    // A partition that was made on the device still has its arrays there: the plan is made from them where they
+    // are -- the same plan, array for array, as from the host arrays (MX_LAYOUT=host, MX_CSR_KERNEL=split and
+    // MX_PLAN_AUTOTUNE=1 keep the host route, which brings the arrays down first).
+    if (P && out && P->twin && P->extracted) {
+        const char *lay = std::getenv("MX_LAYOUT"), *ker = std::getenv("MX_CSR_KERNEL");
+        if (!(lay && !std::strcmp(lay, "host")) && !(ker && !std::strcmp(ker, "split")) && !plan_autotune())
+            return create_plan_device(P->dtype, P->rows, P->cols, P->nnz, nullptr, nullptr, nullptr, P->tau_c, P->tau_r, flags, out, false,
+                                      (const mx::PartitionTwin *)P->twin);
+    }
+    if (P) {
+        const int rc = mx::partition_host(P);
+        if (rc) return rc;
+    }
     return create_plan(P, flags, out, false);
 }
 
@@ -2793,7 +2806,7 @@ extern "C" int mx_tile_steps(const int *chunkBlocks, int nChunks, int slots, int
 // counts.  The plan equals the one mx_plan_create makes from mx_partition_create(_device) of the
 // same matrix, whatever tile forms it keeps.
 static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev, const void *val_dev,
-                              float tau_c, float tau_r, int flags, mx_plan **out, bool noBlocks);
+                              float tau_c, float tau_r, int flags, mx_plan **out, bool noBlocks, const mx::PartitionTwin *twin = nullptr);
 extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
                                      const void *val_dev, float tau_c, float tau_r, int flags, mx_plan **out)
 {
@@ -2802,21 +2815,28 @@ extern "C" int mx_plan_create_device(mx_dtype dtype, int rows, int cols, int nnz
 
 // `noBlocks`: a binary64 plan without the 8 x 8 block form (the second attempt, when a row of a block
 // chunk turned out to have more virtual rows than the block layout has places for).
+// `twin`: the extraction is there already, in the device arrays of a partition that was made on the
+// device (mx_plan_create hands it in; the matrix arguments are not looked at then).
 static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev, const void *val_dev,
-                              float tau_c, float tau_r, int flags, mx_plan **out, bool noBlocks)
+                              float tau_c, float tau_r, int flags, mx_plan **out, bool noBlocks, const mx::PartitionTwin *twin)
 {
-    static const char who[] = "mx_plan_create_device";
-    if (!out || (dtype != MX_F64 && dtype != MX_F16) || rows < 1 || cols < 1 || nnz < 0 || !rowPtr_dev ||
-        (nnz > 0 && (!colInd_dev || !val_dev)) || !(tau_c >= 0.0f && tau_c <= 1.0f) || !(tau_r >= 0.0f && tau_r <= 1.0f)) {
-        set_error(std::string(who) + ": bad argument");
-        return MX_ERR_ARG;
+    const char *who = twin ? "mx_plan_create" : "mx_plan_create_device";
+    int rc;
+    if (!twin) {
+        if (!out || (dtype != MX_F64 && dtype != MX_F16) || rows < 1 || cols < 1 || nnz < 0 || !rowPtr_dev ||
+            (nnz > 0 && (!colInd_dev || !val_dev)) || !(tau_c >= 0.0f && tau_c <= 1.0f) || !(tau_r >= 0.0f && tau_r <= 1.0f)) {
+            set_error(std::string(who) + ": bad argument");
+            return MX_ERR_ARG;
+        }
+        *out = nullptr;
+        if (tau_c == 0.0f && tau_r == 0.0f)  // nothing to extract
+            return mx_plan_create_device_csr(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, flags, out);
+        if ((rc = need_device())) return rc;
+        if ((rc = mx::check_csr_device(rows, cols, nnz, rowPtr_dev, colInd_dev, nullptr, who))) return rc;
+    } else {
+        *out = nullptr;
+        if ((rc = need_device())) return rc;
     }
-    *out = nullptr;
-    if (tau_c == 0.0f && tau_r == 0.0f)  // nothing to extract
-        return mx_plan_create_device_csr(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, flags, out);
-    int rc = need_device();
-    if (rc) return rc;
-    if ((rc = mx::check_csr_device(rows, cols, nnz, rowPtr_dev, colInd_dev, nullptr, who))) return rc;
     // (what a failure has to release, also one that arrives as an exception)
     mx_plan *plan = nullptr;
     int *partPtr = nullptr, *partCol = nullptr;
@@ -2854,10 +2874,12 @@ static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const
         mx::HybridDevice H;
         mx::HybridCounts cnt;
         PhaseLog phase;
-        rc = H.analyse(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, tau_c, tau_r, minVals, !noTiles, wantStrips, wantBlocks, &cnt,
-                       nullptr);
+        if (twin) rc = H.adopt(*twin, minVals, !noTiles, wantStrips, wantBlocks, &cnt, nullptr);
+        else
+            rc = H.analyse(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, tau_c, tau_r, minVals, !noTiles, wantStrips, wantBlocks, &cnt,
+                           nullptr);
         if (rc) return rc;
-        phase("extraction, gate, strip rows (device)");
+        phase(twin ? "gate, strip rows (device, on the partition's device arrays)" : "extraction, gate, strip rows (device)");
         if (cnt.blocks64) cnt.generalFrags = cnt.generalEntries = 0;  // the general tiles are not used beside blocks
         int worth = 2;
         if (noTiles) worth = 0;
@@ -2965,7 +2987,7 @@ static int create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const
             }
             if (!fits) {
                 fail(MX_OK);
-                return create_plan_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, tau_c, tau_r, flags, out, true);
+                return create_plan_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, tau_c, tau_r, flags, out, true, twin);
             }
             if ((rc = upload(&plan->strips.vidx, vidx.data(), vidx.size(), 128))) return fail(rc);
         }
@@ -3116,6 +3138,7 @@ extern "C" int mx_plan_layout(const mx_partition *P, int flags, int nCU, mx_plan
         return MX_ERR_ARG;
     }
     std::memset(out, 0, sizeof(*out));
+    if (int rc = mx::partition_host(P)) return rc;
     const int es = mx::elem_size(P->dtype);
     auto give = [](const auto *p, size_t n) {
         typedef typename std::remove_cv<typename std::remove_pointer<decltype(p)>::type>::type T;

@@ -27,6 +27,7 @@
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_scan.hpp>
 
+#include "mx_device.h"
 #include "mx_internal.h"
 
 namespace mxp {
@@ -829,6 +830,80 @@ extern "C" int mx_tiles_device(mx_dtype dtype, int dRows, int dCols, int nnzRowD
 // split and encoded there (mx_select_device, mx_split_device, mx_tiles_device) and the arrays come
 // back into the same host structure, so that everything downstream (plans, files, the checksum)
 // cannot tell the two routes apart.
+// The device arrays of a partition made here (mx_partition::twin) and their way down.
+namespace {
+void twin_free(void *w)
+{
+    mx::PartitionTwin *W = (mx::PartitionTwin *)w;
+    if (!W) return;
+    (void)hipFree(W->order);
+    (void)hipFree(W->split);
+    mx_tiles_device_free(&W->T);
+    delete W;
+}
+// fills the host vectors of P from its twin
+int twin_download(mx_partition *P)
+{
+    using namespace mxp;
+    static const char who[] = "mx_partition_create_device (arrays to the host)";
+    const mx::PartitionTwin &W = *(const mx::PartitionTwin *)P->twin;
+    const int rows = W.rows, cols = W.cols, nDD = W.nDD, nCD = W.nCD, dRows = W.dRows, dCols = W.dCols;
+    const size_t es = (size_t)mx::elem_size(W.dtype);
+    const mx_device_tiles &T = W.T;
+    try {
+        P->descColId.resize(cols);
+        P->rId.resize(dRows);
+        P->ddRowPtr.resize((size_t)dRows + 1);
+        P->ddColInd.resize(nDD);
+        P->ddVal.resize(nDD, (int)es);
+        P->cdRowPtr.resize((size_t)rows + 1);
+        P->cdColInd.resize(nCD);
+        P->cdVal.resize(nCD, (int)es);
+        P->chunkPtr.resize((size_t)T.chunkNum + 1);
+        P->sparse_AToX_index.resize((size_t)T.totalTcFrags * T.fragK);
+        P->fragPtr.resize((size_t)T.totalTcFrags + 1);
+        if (W.dtype == MX_F64) P->fragBit32.resize(T.totalTcFrags);
+        else P->fragBit64.resize(T.totalTcFrags);
+        P->tcVal.resize(T.tcValCount, (int)es);
+    } catch (const std::bad_alloc &) {
+        mx::set_error("mx_partition_create_device: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    auto down = [](void *dst, const void *src, size_t bytes) {
+        return bytes ? hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost) : hipSuccess;
+    };
+    MXP_TRY(down(P->descColId.data(), W.dc, (size_t)cols * 4));
+    MXP_TRY(down(P->rId.data(), W.dr, (size_t)dRows * 4));
+    MXP_TRY(down(P->ddRowPtr.data(), W.ddp, ((size_t)dRows + 1) * 4));
+    MXP_TRY(down(P->ddColInd.data(), W.ddc, (size_t)nDD * 4));
+    MXP_TRY(down(P->ddVal.data(), W.ddv, (size_t)nDD * es));
+    MXP_TRY(down(P->cdRowPtr.data(), W.cdp, ((size_t)rows + 1) * 4));
+    MXP_TRY(down(P->cdColInd.data(), W.cdc, (size_t)nCD * 4));
+    MXP_TRY(down(P->cdVal.data(), W.cdv, (size_t)nCD * es));
+    MXP_TRY(down(P->chunkPtr.data(), T.chunkPtr, ((size_t)T.chunkNum + 1) * 4));
+    MXP_TRY(down(P->sparse_AToX_index.data(), T.sparse_AToX_index, (size_t)T.totalTcFrags * T.fragK * 4));
+    MXP_TRY(down(P->fragPtr.data(), T.fragPtr, ((size_t)T.totalTcFrags + 1) * 4));
+    if (W.dtype == MX_F64) MXP_TRY(down(P->fragBit32.data(), T.fragBit, (size_t)T.totalTcFrags * 4));
+    else MXP_TRY(down(P->fragBit64.data(), T.fragBit, (size_t)T.totalTcFrags * 8));
+    MXP_TRY(down(P->tcVal.data(), T.tcVal, (size_t)T.tcValCount * es));
+    // the lists of what was not selected, ascending (test/test_autotc_spmv.cpp:1143-1160, :1261-1277)
+    std::vector<unsigned char> taken((size_t)std::max(rows, cols), 0);
+    for (int i = 0; i < dCols; ++i) taken[P->descColId[i]] = 1;
+    P->newArray.clear();
+    P->newArray.reserve(P->sCols);
+    for (int c = 0; c < cols; ++c)
+        if (!taken[c]) P->newArray.push_back(c);
+    std::fill(taken.begin(), taken.end(), 0);
+    for (int i = 0; i < dRows; ++i) taken[P->rId[i]] = 1;
+    P->newArray_.clear();
+    P->newArray_.reserve(P->sRows);
+    for (int r = 0; r < rows; ++r)
+        if (!taken[r]) P->newArray_.push_back(r);
+    P->host_ready = true;
+    return MX_OK;
+}
+}  // namespace
+
 extern "C" int mx_partition_create_device(const mx_csr *A, float tau_c, float tau_r, mx_partition **out)
 {
     static const char who[] = "mx_partition_create_device";
@@ -841,18 +916,35 @@ extern "C" int mx_partition_create_device(const mx_csr *A, float tau_c, float ta
         mx::set_error("mx_partition_create_device: no HIP device");
         return MX_ERR_DEVICE;
     }
+    (void)who;
     const int rows = A->rows, cols = A->cols, nnz = A->nnz;
     const size_t es = (size_t)mx::elem_size(A->dtype);
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
-    // the matrix and the two orders
+    mx::PartitionTwin *W = new (std::nothrow) mx::PartitionTwin();
+    if (!W) {
+        mx::set_error("mx_partition_create_device: out of memory");
+        return MX_ERR_ALLOC;
+    }
+    struct TwinGuard {
+        mx::PartitionTwin *w;
+        ~TwinGuard() { twin_free(w); }
+    } wg{W};
+    W->dtype = A->dtype;
+    W->rows = rows;
+    W->cols = cols;
+    W->nnz = nnz;
+    // the matrix (released when the extraction is done) and the two orders (kept)
     const size_t rpB = al(((size_t)rows + 1) * 4), ciB = al((size_t)nnz * 4 + 4), vaB = al((size_t)nnz * es + 8),
                  dcB = al((size_t)cols * 4 + 4), drB = al((size_t)rows * 4 + 4);
     Scratch in;
-    MXP_TRY(hipMalloc(&in.p, rpB + ciB + vaB + dcB + drB));
+    MXP_TRY(hipMalloc(&in.p, rpB + ciB + vaB));
     unsigned char *b = (unsigned char *)in.p;
     int *rp = (int *)b, *ci = (int *)(b + rpB);
     void *va = b + rpB + ciB;
-    int *dc = (int *)(b + rpB + ciB + vaB), *dr = (int *)(b + rpB + ciB + vaB + dcB);
+    MXP_TRY(hipMalloc(&W->order, dcB + drB));
+    W->dc = (int *)W->order;
+    W->dr = (int *)((unsigned char *)W->order + dcB);
+    int *dc = W->dc, *dr = W->dr;
     MXP_TRY(hipMemcpy(rp, A->rowPtr, ((size_t)rows + 1) * 4, hipMemcpyHostToDevice));
     if (nnz > 0) {
         MXP_TRY(hipMemcpy(ci, A->colInd, (size_t)nnz * 4, hipMemcpyHostToDevice));
@@ -864,103 +956,58 @@ extern "C" int mx_partition_create_device(const mx_csr *A, float tau_c, float ta
     const int nDD = sel.nnzRowD, nCD = nnz - nDD;
     const size_t ddpB = al(((size_t)sel.dRows + 1) * 4), ddcB = al((size_t)nDD * 4 + 4), ddvB = al((size_t)nDD * es + 8),
                  cdpB = al(((size_t)rows + 1) * 4), cdcB = al((size_t)nCD * 4 + 4), cdvB = al((size_t)nCD * es + 8);
-    Scratch mid;
-    MXP_TRY(hipMalloc(&mid.p, ddpB + ddcB + ddvB + cdpB + cdcB + cdvB));
-    b = (unsigned char *)mid.p;
-    int *ddp = (int *)b, *ddc = (int *)(b + ddpB);
-    void *ddv = b + ddpB + ddcB;
-    int *cdp = (int *)(b + ddpB + ddcB + ddvB), *cdc = (int *)(b + ddpB + ddcB + ddvB + cdpB);
-    void *cdv = b + ddpB + ddcB + ddvB + cdpB + cdcB;
-    rc = mx_split_device(A->dtype, rows, cols, nnz, rp, ci, va, &sel, dc, dr, ddp, ddc, ddv, cdp, cdc, cdv, nullptr);
+    MXP_TRY(hipMalloc(&W->split, ddpB + ddcB + ddvB + cdpB + cdcB + cdvB));
+    b = (unsigned char *)W->split;
+    W->ddp = (int *)b;
+    W->ddc = (int *)(b + ddpB);
+    W->ddv = b + ddpB + ddcB;
+    W->cdp = (int *)(b + ddpB + ddcB + ddvB);
+    W->cdc = (int *)(b + ddpB + ddcB + ddvB + cdpB);
+    W->cdv = b + ddpB + ddcB + ddvB + cdpB + cdcB;
+    rc = mx_split_device(A->dtype, rows, cols, nnz, rp, ci, va, &sel, dc, dr, W->ddp, W->ddc, W->ddv, W->cdp, W->cdc, W->cdv, nullptr);
     if (rc != MX_OK) return rc;
-    mx_device_tiles T{};
-    rc = mx_tiles_device(A->dtype, sel.dRows, sel.dCols, nDD, ddp, ddc, ddv, &T, nullptr);
+    rc = mx_tiles_device(A->dtype, sel.dRows, sel.dCols, nDD, W->ddp, W->ddc, W->ddv, &W->T, nullptr);
     if (rc != MX_OK) return rc;
-    struct TilesGuard {
-        mx_device_tiles *t;
-        ~TilesGuard() { mx_tiles_device_free(t); }
-    } guard{&T};
+    W->dRows = sel.dRows;
+    W->dCols = sel.dCols;
+    W->nDD = nDD;
+    W->nCD = nCD;
+    const mx_device_tiles &T = W->T;
 
     mx_partition *P = new (std::nothrow) mx_partition();
     if (!P) {
         mx::set_error("mx_partition_create_device: out of memory");
         return MX_ERR_ALLOC;
     }
-    struct PartGuard {
-        mx_partition *p;
-        ~PartGuard() { delete p; }
-    } pg{P};
-    try {
-        P->dtype = A->dtype;
-        P->rows = rows;
-        P->cols = cols;
-        P->nnz = nnz;
-        P->fragM = mx::kFragM;
-        P->fragK = mx::frag_k(A->dtype);
-        P->tau_c = tau_c;
-        P->tau_r = tau_r;
-        P->extracted = true;
-        P->dCols = sel.dCols;
-        P->sCols = cols - sel.dCols;
-        P->nnzColD = sel.nnzColD;
-        P->nnzColS = nnz - sel.nnzColD;
-        P->cols_ratio = (float)sel.dCols / (float)cols;
-        P->dRows = sel.dRows;
-        P->sRows = rows - sel.dRows;
-        P->nnzRowD = nDD;
-        P->nnzRowS = sel.nnzColD - nDD;
-        P->nnzCD = nCD;
-        P->descColId.resize(cols);
-        P->rId.resize(sel.dRows);
-        P->ddRowPtr.resize((size_t)sel.dRows + 1);
-        P->ddColInd.resize(nDD);
-        P->ddVal.resize(nDD, (int)es);
-        P->cdRowPtr.resize((size_t)rows + 1);
-        P->cdColInd.resize(nCD);
-        P->cdVal.resize(nCD, (int)es);
-        P->chunkNum = T.chunkNum;
-        P->totalTcFrags = T.totalTcFrags;
-        P->tcValCount = T.tcValCount;
-        P->tc_nnz_ratio = (double)nDD / ((double)T.totalTcFrags * mx::kFragM * P->fragK);
-        P->chunkPtr.resize((size_t)T.chunkNum + 1);
-        P->sparse_AToX_index.resize((size_t)T.totalTcFrags * T.fragK);
-        P->fragPtr.resize((size_t)T.totalTcFrags + 1);
-        if (A->dtype == MX_F64) P->fragBit32.resize(T.totalTcFrags);
-        else P->fragBit64.resize(T.totalTcFrags);
-        P->tcVal.resize(T.tcValCount, (int)es);
-    } catch (const std::bad_alloc &) {
-        mx::set_error("mx_partition_create_device: out of memory");
-        return MX_ERR_ALLOC;
-    }
-    auto down = [](void *dst, const void *src, size_t bytes) {
-        return bytes ? hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost) : hipSuccess;
-    };
-    MXP_TRY(down(P->descColId.data(), dc, (size_t)cols * 4));
-    MXP_TRY(down(P->rId.data(), dr, (size_t)sel.dRows * 4));
-    MXP_TRY(down(P->ddRowPtr.data(), ddp, ((size_t)sel.dRows + 1) * 4));
-    MXP_TRY(down(P->ddColInd.data(), ddc, (size_t)nDD * 4));
-    MXP_TRY(down(P->ddVal.data(), ddv, (size_t)nDD * es));
-    MXP_TRY(down(P->cdRowPtr.data(), cdp, ((size_t)rows + 1) * 4));
-    MXP_TRY(down(P->cdColInd.data(), cdc, (size_t)nCD * 4));
-    MXP_TRY(down(P->cdVal.data(), cdv, (size_t)nCD * es));
-    MXP_TRY(down(P->chunkPtr.data(), T.chunkPtr, ((size_t)T.chunkNum + 1) * 4));
-    MXP_TRY(down(P->sparse_AToX_index.data(), T.sparse_AToX_index, (size_t)T.totalTcFrags * T.fragK * 4));
-    MXP_TRY(down(P->fragPtr.data(), T.fragPtr, ((size_t)T.totalTcFrags + 1) * 4));
-    if (A->dtype == MX_F64) MXP_TRY(down(P->fragBit32.data(), T.fragBit, (size_t)T.totalTcFrags * 4));
-    else MXP_TRY(down(P->fragBit64.data(), T.fragBit, (size_t)T.totalTcFrags * 8));
-    MXP_TRY(down(P->tcVal.data(), T.tcVal, (size_t)T.tcValCount * es));
-    // the lists of what was not selected, ascending (test/test_autotc_spmv.cpp:1143-1160, :1261-1277)
-    std::vector<unsigned char> taken((size_t)std::max(rows, cols), 0);
-    for (int i = 0; i < sel.dCols; ++i) taken[P->descColId[i]] = 1;
-    P->newArray.reserve(P->sCols);
-    for (int c = 0; c < cols; ++c)
-        if (!taken[c]) P->newArray.push_back(c);
-    std::fill(taken.begin(), taken.end(), 0);
-    for (int i = 0; i < sel.dRows; ++i) taken[P->rId[i]] = 1;
-    P->newArray_.reserve(P->sRows);
-    for (int r = 0; r < rows; ++r)
-        if (!taken[r]) P->newArray_.push_back(r);
-    pg.p = nullptr;
+    // the counts; the arrays stay on the device until somebody asks for them (mx::partition_host)
+    P->dtype = A->dtype;
+    P->rows = rows;
+    P->cols = cols;
+    P->nnz = nnz;
+    P->fragM = mx::kFragM;
+    P->fragK = mx::frag_k(A->dtype);
+    P->tau_c = tau_c;
+    P->tau_r = tau_r;
+    P->extracted = true;
+    P->dCols = sel.dCols;
+    P->sCols = cols - sel.dCols;
+    P->nnzColD = sel.nnzColD;
+    P->nnzColS = nnz - sel.nnzColD;
+    P->cols_ratio = (float)sel.dCols / (float)cols;
+    P->dRows = sel.dRows;
+    P->sRows = rows - sel.dRows;
+    P->nnzRowD = nDD;
+    P->nnzRowS = sel.nnzColD - nDD;
+    P->nnzCD = nCD;
+    P->chunkNum = T.chunkNum;
+    P->totalTcFrags = T.totalTcFrags;
+    P->tcValCount = T.tcValCount;
+    P->tc_nnz_ratio = (double)nDD / ((double)T.totalTcFrags * mx::kFragM * P->fragK);
+    P->host_ready = false;
+    P->twin = W;
+    P->twin_download = twin_download;
+    P->twin_free = twin_free;
+    wg.w = nullptr;  // the partition owns the twin now
     *out = P;
     return MX_OK;
 }

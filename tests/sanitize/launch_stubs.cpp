@@ -18,6 +18,7 @@ struct HybridDevice::Impl {};
 HybridDevice::~HybridDevice() { delete impl; }
 int HybridDevice::analyse(mx_dtype, int, int, int, const int *, const int *, const void *, float, float, int, bool, bool, bool, HybridCounts *,
                           hipStream_t) { return MX_ERR_DEVICE; }
+int HybridDevice::adopt(const PartitionTwin &, int, bool, bool, bool, HybridCounts *, hipStream_t) { return MX_ERR_DEVICE; }
 int HybridDevice::csr_part(bool, bool, bool, int **, int **, void **, int *, char **) { return MX_ERR_DEVICE; }
 int HybridDevice::block_chunks(std::vector<int> &, std::vector<int> &) { return MX_ERR_DEVICE; }
 int HybridDevice::block_layout(const std::vector<int> &, const std::vector<int> &, const std::vector<int> &, long long, DeviceTiles &)

@@ -310,6 +310,42 @@ def test_spmv_host_and_argument_checks(mx, ora):
         plan.spmv(torch.zeros(A.cols, dtype=torch.float32, device="cuda"))
 
 
+def test_x_is_checked_before_anything_is_launched(mx, ora):
+    """An x that a plan cannot take is refused with MX_ERR_ARG and nothing is written to y: a plan whose CSR part
+    keeps x in LDS, and a binary64 plan with 8 x 8 blocks over the row-tile form of the CSR part (the blocks read x
+    in aligned 16-byte pieces and have no other form)."""
+    import torch
+    A, x = mx.gen_config(2, scale=1 / 8)
+    P = mx.Partition(A, 1.0, 1.0)
+    xd = torch.zeros(A.cols + 1, dtype=torch.float64, device="cuda")
+    xd[1:] = torch.from_numpy(x).cuda()
+    off = xd[1:]                                   # 8 bytes past a 16-byte boundary
+    assert off.data_ptr() % 16 == 8
+    ref = oracle_y(ora, mx, A, x)
+    for flags in (mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_ROWS, mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_SLICES, mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_NO_TILES):
+        plan = mx.Plan(P, flags)
+        if flags & mx.MX_PLAN_KEEP_TILES:
+            assert plan.info["tile_variant"] == 2 and plan.info["tile_nnz"] > 0
+        y = torch.full((A.rows,), 7.0, dtype=torch.float64, device="cuda")
+        with pytest.raises(mx.MxError) as e:
+            plan.spmv(off, y)
+        assert e.value.code == 1 and "16-byte aligned" in str(e.value)
+        with pytest.raises(mx.MxError):
+            plan.time(off, y, 1, 2)
+        with pytest.raises(mx.MxError):
+            plan.time_kernels(off, y, 1, 2)
+        torch.cuda.synchronize()
+        assert bool((y == 7.0).all()), "y was touched before x was refused"
+        good = torch.from_numpy(x).cuda()
+        assert rel_l2(plan.spmv(good).cpu().numpy(), ref) <= F64_TOL
+        plan.close()
+    # the row-tile form alone gathers x element by element: any alignment
+    plan = mx.Plan(P, mx.MX_PLAN_NO_TILES | mx.MX_PLAN_CSR_ROWS)
+    assert rel_l2(plan.spmv(off).cpu().numpy(), ref) <= F64_TOL
+    plan.close()
+    P.close()
+
+
 def test_ragged_and_degenerate_shapes(mx, ora):
     import torch
     rng = np.random.default_rng(77)
@@ -1392,6 +1428,46 @@ def test_partition_by_the_device_route_is_the_same_partition(mx, ora):
     assert rel_l2(y.cpu().numpy().astype(np.float64), oracle_y(ora, mx, A, x)) <= F16_TOL
     plan.close()
     D.close()
+
+
+@pytest.mark.gpu
+def test_partition_made_on_the_device_keeps_its_arrays_there(mx, ora, monkeypatch):
+    """mx_partition_create_device leaves the arrays on the device until they are asked for, and mx_plan_create makes
+    its plan from them where they are: the same plan, array for array, as the host route makes from the arrays of a
+    host partition, and the same y; the counts are there at once, the arrays and the checksum when asked for, equal
+    to the host partition's; a second plan from the same handle works as well."""
+    import torch
+    for cfg, scale, tau, flags in ((5, 1 / 32, (1.0, 1.0), mx.MX_PLAN_DEFAULT), (2, 0.5, (0.75, 0.5), mx.MX_PLAN_KEEP_TILES),
+                                   (4, 1 / 16, (0.5, 0.25), mx.MX_PLAN_ALL_TILES), (3, 0.05, (1.0, 0.5), mx.MX_PLAN_DEFAULT)):
+        A, x = mx.gen_config(cfg, scale=scale)
+        xd = torch.from_numpy(x).cuda()
+        H = mx.Partition(A, *tau)
+        D = mx.Partition(A, *tau, device=True)
+        for k in ("dCols", "dRows", "nnzRowD", "nnzCD", "chunkNum", "totalTcFrags", "tcValCount", "cols_ratio", "tc_nnz_ratio"):
+            assert getattr(D, k) == getattr(H, k) or (k == "tc_nnz_ratio" and np.isnan(D.tc_nnz_ratio) and np.isnan(H.tc_nnz_ratio)), k
+        assert "cdColInd" not in D.__dict__          # nothing has come down yet
+        pd = mx.Plan(D, flags)                       # from the device arrays
+        assert "cdColInd" not in D.__dict__
+        monkeypatch.setenv("MX_LAYOUT", "host")
+        ph = mx.Plan(H, flags)                       # the host route from the host arrays
+        monkeypatch.delenv("MX_LAYOUT")
+        assert pd.arrays() == ph.arrays(), (cfg, tau, flags)
+        for k in ("csr_variant", "csr_nnz", "tile_nnz", "tile_variant", "tile_strip_nnz", "csr_fused", "csr_value_dict"):
+            assert pd.info[k] == ph.info[k], (cfg, k)
+        yd, yh = pd.spmv(xd), ph.spmv(xd)
+        torch.cuda.synchronize()
+        assert torch.equal(yd, yh)
+        assert rel_l2(yd.cpu().numpy(), oracle_y(ora, mx, A, x)) <= (F64_TOL if A.dtype == mx.MX_F64 else F16_TOL)
+        # the arrays when asked for, and the checksum
+        assert D.hash == H.hash
+        for name in mx.Partition.ARRAYS:
+            assert np.array_equal(np.asarray(getattr(D, name)).view(np.uint8), np.asarray(getattr(H, name)).view(np.uint8)), name
+        p2 = mx.Plan(D, flags)                       # and again, after the arrays came down
+        assert p2.arrays() == ph.arrays()
+        for p in (pd, ph, p2):
+            p.close()
+        D.close()
+        H.close()
 
 
 @pytest.mark.gpu

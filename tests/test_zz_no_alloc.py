@@ -20,8 +20,16 @@ def _both(mx, torch, A, x, tau, flags):
     y_ref = plan.spmv(xd)
     torch.cuda.synchronize()
     y = torch.full_like(y_ref, float("nan"))
-    plan.spmv_static(xd, y)
+    plan.spmv_static(xd, y)                  # (the first call on a device looks the array's address up)
     torch.cuda.synchronize()
+    # the property the entry point exists for: the device's free memory is the same before and after a call
+    y.fill_(float("nan"))
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    plan.spmv_static(xd, y)
+    free1 = torch.cuda.mem_get_info()[0]
+    torch.cuda.synchronize()
+    assert free1 == free0 == torch.cuda.mem_get_info()[0], (free0, free1)
     info = dict(plan.info)
     plan.close()
     part.close()
@@ -31,10 +39,11 @@ def _both(mx, torch, A, x, tau, flags):
 def test_static_entry_point_equals_mx_spmv(mx, ora):
     import torch
     lib = mx._lib.load()
-    assert lib.mx_static_scratch_bytes() == 16 << 20
+    assert lib.mx_static_scratch_bytes() == 32 << 20
     calls = [
         # (workload, scale, tau, flags): larger first, then smaller
         (2, 1.0, (0.0, 0.0), mx.MX_PLAN_CSR_SLICES),
+        (2, 0.5, (0.0, 0.0), mx.MX_PLAN_CSR_SLICES),   # a plan in the one-launch form: its two launches run here
         (2, 1 / 16, (0.0, 0.0), mx.MX_PLAN_CSR_SLICES),
         (4, 1.0, (0.0, 0.0), mx.MX_PLAN_CSR_SLICES),
         (5, 1 / 64, (1.0, 1.0), mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_KEEP_TILES),
@@ -61,10 +70,29 @@ def test_static_entry_point_equals_mx_spmv(mx, ora):
     assert used.count(1) >= 4, used
 
 
+def test_static_entry_point_holds_the_largest_workload(mx, ora):
+    """The mixed workload at full size (27 MB of sums) fits the array: the hybrid plan of the benchmark's point,
+    made on the device, through both entry points."""
+    import torch
+    A, x = mx.gen_config(5)
+    plan = mx.Plan.from_device(torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda(),
+                               A.cols, 1.0, 1.0)
+    assert plan.info["csr_variant"] == 1 and plan.info["tile_strip_nnz"] > 0
+    xd = torch.from_numpy(x).cuda()
+    y_ref = plan.spmv(xd)
+    y = torch.full_like(y_ref, float("nan"))
+    plan.spmv_static(xd, y)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_ref)
+    ref = ora.spmv_f16_f32acc(A.val, A.rowPtr, A.colInd, x)[0].astype(np.float64)
+    assert np.linalg.norm(y.cpu().numpy().astype(np.float64) - ref) / np.linalg.norm(ref) <= 1e-2
+    plan.close()
+
+
 def test_static_entry_point_refuses_what_does_not_fit(mx):
     import torch
-    # 2.2 M rows of one entry each: one virtual row per row, 8 bytes of sum each -> more than 16 MiB
-    rows = 2200000
+    # 4.4 M rows of one entry each: one virtual row per row, 8 bytes of sum each -> more than 32 MiB
+    rows = 4400000
     cols = 65536
     rng = np.random.default_rng(5)
     A = mx.Csr(rows, cols, np.arange(rows + 1, dtype=np.int32), rng.integers(0, cols, rows).astype(np.int32),
