@@ -497,7 +497,23 @@ typedef struct mx_plan_info {
                             launch too, src/spmv_kernel/cdSpMV.cu:459): the workgroups that hold sums of the same rows
                             sit on one XCD, count themselves off on a counter in that XCD's L2, and the one that
                             completes the count adds the sums up and writes y; nobody waits.  0: two launches */
+    int opt_flags;       /* MX_OPT_* bits: the switches of the environment that were set when the plan was made.  The
+                            library reads the environment when a plan or layout is created and never while a plan
+                            runs; a plan made under one setting keeps it whatever the environment says later */
+    double opt_tile_gate;/* the fill a fragment needed for the tile kernels when the plan was made (MX_TILE_GATE;
+                            one half unless set) */
 } mx_plan_info;
+/* mx_plan_info.opt_flags */
+#define MX_OPT_NO_STRIPS 1     /* MX_NO_STRIPS=1: no binary16 strip chunks */
+#define MX_OPT_NO_BLOCKS 2     /* MX_NO_BLOCKS=1: no binary64 8 x 8 blocks */
+#define MX_OPT_NO_DICT 4       /* MX_CSR_DICT=0: values as they are, also where at most 255 distinct ones exist */
+#define MX_OPT_STRIPS_APART 8  /* MX_STRIPS_APART=1: binary16 strips in a launch of their own */
+#define MX_OPT_CSR_KERNEL 16   /* MX_CSR_KERNEL=rows|slices|split named the form of the CSR part */
+#define MX_OPT_CSR_FUSED 32    /* MX_CSR_FUSED=0|1 decided about the one-launch form */
+#define MX_OPT_AUTOTUNE 64     /* MX_PLAN_AUTOTUNE=1: forms were timed, not estimated (the plan may differ run to run) */
+#define MX_OPT_LAYOUT_HOST 128 /* MX_LAYOUT=host: layouts made on the host where the device route exists (same arrays) */
+#define MX_OPT_TUNING 256      /* one of the tuning knobs was set: MX_SLICE_CAP, MX_SPLIT_LEN, MX_CSR_NPT, MX_TILE_PER,
+                                  MX_CSR_REDUCE, MX_CSR_COL16 */
 int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);
 
 /* The layout csr_slice_kernel runs on, built on the host for a machine with `nCU` compute units,

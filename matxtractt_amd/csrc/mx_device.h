@@ -285,6 +285,9 @@ struct HybridDevice {
 // row which gets sums from both parts is rounded to the value type once.
 hipError_t launch_slices(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s,
                          int what = 0, const DeviceTiles *strips = nullptr, void *ywide = nullptr);
+// Raises the dynamic-LDS limit of the slice kernels on the current device (idempotent).  Every route that makes
+// a DeviceSlices calls it before handing the layout out; launch_slices and launch_fused rely on that.
+hipError_t prepare_slice_kernels(mx_dtype dtype);
 // The one-launch form of the same product (P.fused).  `misplaced`: a word in host memory that the
 // device can write (one per process); a workgroup that finds itself on another XCD than the layout
 // assumes sets it, and the product of that launch cannot be trusted.

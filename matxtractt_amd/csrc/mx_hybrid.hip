@@ -7,9 +7,8 @@
 // the host (a few bytes each), never an entry of the matrix.  The reference does all of this on
 // the host (test/test_autotc_spmv.cpp:1099-1421).
 //
-// The general tile form is laid out here as well (tile_chunks, tile_layout).  The binary64 block
-// form is only counted, so that the caller can decide exactly as the host route does and, when the
-// blocks are to be kept, take the host route for that matrix.
+// The general tile form is laid out here as well (tile_chunks, tile_layout), and so is the binary64
+// block form (block_chunks, block_layout): no form of the tile part sends a matrix to the host.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>

@@ -15,6 +15,30 @@ constexpr int kFragM = 8;
 
 void set_error(const std::string &msg);
 
+// Every switch the library takes from the environment, read in one place (refresh_options, which the
+// entry points that make plans and layouts call first) and looked at through opt() from there on; a plan
+// keeps the ones that change what it computes or how (mx_plan_info.opt_flags, opt_tile_gate).
+struct Options {
+    double tile_gate = -1.0;  // MX_TILE_GATE=<fraction>: fill a fragment needs for the tile kernels; -1 = the default (one half)
+    int csr_dict = 1;         // MX_CSR_DICT: 0 = never one byte per value; 1 = wherever at most 255 values exist; 2 = also against a timed choice
+    bool no_strips = false;   // MX_NO_STRIPS=1: no binary16 strip chunks
+    bool no_blocks = false;   // MX_NO_BLOCKS=1: no binary64 8 x 8 blocks
+    bool strips_apart = false;// MX_STRIPS_APART=1: strips in a launch of their own instead of the combine kernel's
+    int csr_kernel = 0;       // MX_CSR_KERNEL=rows|slices|split: 1 | 2 | 3; 0 = the plan decides
+    int csr_fused = -1;       // MX_CSR_FUSED: 0 = never the one-launch form, 1 = wherever the matrix suits it; -1 = the plan decides
+    bool autotune = false;    // MX_PLAN_AUTOTUNE=1: the forms of the CSR part are timed on the spot instead of estimated
+    bool layout_host = false; // MX_LAYOUT=host: layouts on the host also where the device route exists
+    int slice_cap = 0;        // MX_SLICE_CAP=<entries>: longest virtual row (tuning runs); 0 = a lane's fair share
+    int split_len = 0;        // MX_SPLIT_LEN=<entries>: shortest row the split form sends to the slices; 0 = 32
+    int csr_npt = 0;          // MX_CSR_NPT: entries per lane and tile of the row kernel; 0 = the default
+    int tile_per = 0;         // MX_TILE_PER: steps per wave of the tile kernels; 0 = by the size
+    int csr_reduce = 0;       // MX_CSR_REDUCE=rows|scan: 1 | 2; 0 = by the spread of the row lengths
+    bool csr_col16 = true;    // MX_CSR_COL16=0: never 16-bit column offsets in the row kernel
+    bool plan_log = false;    // MX_PLAN_LOG=1: phase times of plan creation on stderr
+};
+const Options &opt();
+void refresh_options();
+
 // `int dColsNnz = nnzA * colProp;` (test/test_autotc_spmv.cpp:1131, :1249): int * float is a float
 // product, truncated.
 inline int threshold(int nnz, float frac)

@@ -557,7 +557,6 @@ struct FusedArgs {
     unsigned *claim = nullptr;       // [workgroups] how often each logical workgroup's work has been taken
     unsigned seq = 0;                // launches of this layout before this one
     int rows = 0, placesPerRow = 4, accumulate = 0;
-    int debugSkip = 0;               // measurements only: end the kernel early (bits 1, 2, 4: after the stream, the drain, the counters)
 };
 
 // The XCD this wave runs on (XCC_ID, bits 3:0 of hardware register 20).
@@ -739,14 +738,12 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         static_assert(kSliceThreads % GR == 0 && GR == 256, "a lane keeps its place inside the group from pass to pass");
         if (tid == 0 && (claimed != fa.seq || xcc_id() >= mx::kFusedXcds))
             __hip_atomic_store(fa.misplaced, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        if (fa.debugSkip & 1) return;
         const bool wide8 = fa.placesPerRow == 8;
         const AT *sums = (const AT *)fa.sums;
         VT *y = (VT *)fa.y;
         AT *ywide = (AT *)fa.ywide;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's sums are in the L2
         __syncthreads();                                    // ... and so are the other waves'
-        if (fa.debugSkip & 2) return;
         // (the chunk ends are done with) listL[0] = how many groups fall to this workgroup, then which
         int *listL = endsL;
         if (tid == 0) listL[0] = 0;
@@ -760,7 +757,6 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
             }
         }
         __syncthreads();
-        if (fa.debugSkip & 4) return;
         // A pass: R groups per half of the workgroup, a row per lane and group.  A wave's 64 rows are
         // consecutive, so every load is one contiguous stretch; the places a row does not use hold
         // nothing that counts (rowVrows says how many do).
@@ -1357,7 +1353,7 @@ __global__ void probe_mfma_f16_kernel(const _Float16 *A /*[64][8]*/, const _Floa
 
 }  // namespace mxk
 
-// ---- launchers (called from mx_plan.cpp; plain functions so that file needs no HIP syntax)
+// ---- launchers (called from mx_run.cpp and the plan files; plain functions so that those need no HIP syntax)
 namespace mx {
 
 constexpr int kMaxDevices = 64;
@@ -1428,27 +1424,34 @@ hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y
     return hipGetLastError();
 }
 
-// The slice kernels take more dynamic LDS than the default limit: raised once per device (a function
-// attribute belongs to the device that is current when it is set).
+// The slice kernels take more dynamic LDS than the default limit.  The limit is a function attribute and
+// belongs to the device that is current when it is set: whoever makes a slice layout (a plan, on its device)
+// calls this once it exists; the launchers take no lock and ask nothing about the device.
 template <typename VT>
 static hipError_t slice_kernel_attributes()
 {
+    const void *fn[4] = {(const void *)mxk::csr_slice_kernel<VT, false, false>, (const void *)mxk::csr_slice_kernel<VT, true, false>,
+                         (const void *)mxk::csr_slice_kernel<VT, false, true>, (const void *)mxk::csr_slice_kernel<VT, true, true>};
+    for (const void *f : fn) {
+        const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+hipError_t prepare_slice_kernels(mx_dtype dtype)
+{
     static std::mutex attrLock;
-    static bool attrSet[kMaxDevices] = {};
+    static bool attrSet[kMaxDevices][2] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    const int t = dtype == MX_F64 ? 0 : 1;
     std::lock_guard<std::mutex> hold(attrLock);
-    if (attrSet[dev]) return hipSuccess;
-    const void *fn[4] = {(const void *)mxk::csr_slice_kernel<VT, false, false>, (const void *)mxk::csr_slice_kernel<VT, true, false>,
-                         (const void *)mxk::csr_slice_kernel<VT, false, true>, (const void *)mxk::csr_slice_kernel<VT, true, true>};
-    for (const void *f : fn) {
-        e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
-        if (e != hipSuccess) return e;
-    }
-    attrSet[dev] = true;
-    return hipSuccess;
+    if (attrSet[dev][t]) return hipSuccess;
+    e = dtype == MX_F64 ? slice_kernel_attributes<double>() : slice_kernel_attributes<_Float16>();
+    if (e == hipSuccess) attrSet[dev][t] = true;
+    return e;
 }
 
 template <typename VT>
@@ -1458,10 +1461,6 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     typedef typename mxk::Acc<VT>::type AT;
     const bool dict = P.useDict && P.ecode && P.dict;
     const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)((P.maxWgChunks + 3) & ~3) * 4 + 64 + (dict ? 256 * sizeof(AT) : 0);
-    {
-        const hipError_t e = slice_kernel_attributes<VT>();
-        if (e != hipSuccess) return e;
-    }
     if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16))
         return hipErrorInvalidValue;
     if (what != 2 && P.nWG > 0) {
@@ -1519,8 +1518,6 @@ static hipError_t launch_fused_t(const DeviceSlices &P, const void *x, void *y, 
     const int ldsInts = std::max(P.maxWgChunks, P.maxWgGroups + 1);
     const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)((ldsInts + 3) & ~3) * 4 + 64 + (dict ? 256 * sizeof(AT) : 0) +
                        (size_t)P.maxWgChunks * 256;
-    const hipError_t e = slice_kernel_attributes<VT>();
-    if (e != hipSuccess) return e;
     if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16) || !P.fused || !P.wgGroups ||
         !P.groupNeed || !P.groupCount || !P.fusedTarget || !P.rowVrows || !P.fusedSums || !P.claim || !misplaced || (P.placesPerRow != 4 && P.placesPerRow != 8) ||
         P.nWG <= 0 || P.nWG % mx::kFusedXcds)
@@ -1540,11 +1537,6 @@ static hipError_t launch_fused_t(const DeviceSlices &P, const void *x, void *y, 
     fa.rows = P.rows;
     fa.placesPerRow = P.placesPerRow;
     fa.accumulate = accumulate;
-    {
-        // (for measurements: 1, 2, 4 end the kernel after the stream, the drain, the counters)
-        static const int skip = std::getenv("MX_FUSED_SKIP") ? std::atoi(std::getenv("MX_FUSED_SKIP")) : 0;
-        fa.debugSkip = skip;
-    }
     if (dict)
         hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, true, true>), dim3(P.nWG), dim3(kSliceThreads), lds, s, (const int4 *)P.wgDesc,
                            (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.ecode, (const VT *)x, (AT *)P.partial, P.cols,
@@ -1585,22 +1577,16 @@ hipError_t fused_placement_ok(int nWG, int *ok)
     std::vector<unsigned> h((size_t)nWG);
     bool holds = nWG % mx::kFusedXcds == 0;
     e = hipMemset(taken, 0, (size_t)nWG * 4);
-    // (a few launches in a row, the way products follow each other, with a launch of another size between them)
+    // (a few launches in a row, the way products follow each other)
     const int reps = 4;
     for (int rep = 0; rep < reps && e == hipSuccess && holds; ++rep) {
         hipLaunchKernelGGL(mxk::xcc_probe_kernel, dim3(nWG), dim3(kSliceThreads), mx::kSliceBytes + 2048, nullptr, taken, rep);
         e = hipGetLastError();
-        if (e == hipSuccess) e = hipMemsetAsync(taken + nWG - 1, 0, 0, nullptr);
     }
     if (e == hipSuccess) e = hipMemcpy(h.data(), taken, (size_t)nWG * 4, hipMemcpyDeviceToHost);
     (void)hipFree(taken);
     if (e != hipSuccess) return e;
     for (int b = 0; b < nWG; ++b) holds = holds && h[b] == (unsigned)reps;
-    if (std::getenv("MX_FUSED_DEBUG")) {
-        fprintf(stderr, "fused_placement_ok: nWG %d holds %d; first slots:", nWG, (int)holds);
-        for (int b = 0; b < std::min(nWG, 24); ++b) fprintf(stderr, " %u", h[b]);
-        fprintf(stderr, "\n");
-    }
     known[dev] = holds ? 1 : 2;
     knownGrid[dev] = nWG;
     *ok = holds;

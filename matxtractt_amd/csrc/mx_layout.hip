@@ -1,6 +1,6 @@
 // The slice layout of the CSR part (see DeviceSlices) built on the device from a CSR matrix that
 // lives in device memory: the same arrays, byte for byte, as the host route (build_slices in
-// mx_plan.cpp), for matrices that are already in HBM and for plans of large matrices, whose
+// mx_host_layout.cpp), for matrices that are already in HBM and for plans of large matrices, whose
 // layout the host cores take a second to make.  The reference has no counterpart: its CSR
 // kernel reads the CSR arrays as they are (src/spmv_kernel/cdSpMV.cu:407-418).
 //
@@ -490,10 +490,8 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
     const int budget = std::max(nCU, 1);
     const long long fair = (long long)nnz / ((long long)budget * W * 64);
     int cap = (int)std::min<long long>(512, std::max<long long>(16, (fair + BE - 1) / BE * BE));
-    if (const char *e = std::getenv("MX_SLICE_CAP")) {
-        const int v = std::atoi(e);
+    if (const int v = mx::opt().slice_cap)
         if (v >= BE && v <= 4096) cap = v / BE * BE;
-    }
     D = DeviceSlices();
     D.S = S;
     D.rows = rows;
@@ -675,8 +673,7 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
     std::vector<unsigned char> dict;
     int nDict = 0;
     {
-        const char *ed = std::getenv("MX_CSR_DICT");
-        if (nnz >= 65536 && !(ed && !std::atoi(ed))) {
+        if (nnz >= 65536 && mx::opt().csr_dict != 0) {
             if ((rc = device_value_dict<V>(val, nnz, codes, dict, &nDict, s))) return rc;
         }
         if (nDict > 0) {
@@ -824,8 +821,7 @@ int upload_csr_device(mx_dtype dtype, int rows, int cols, int nnz, const int *ro
     if (nnz) MXL_TRY(hipMemcpyAsync(A.val, val_dev, (size_t)nnz * es, hipMemcpyDeviceToDevice, s));
     MXL_TRY(hipMalloc((void **)&A.blockDesc, std::max<size_t>(desc.size(), 4) * 4));
     if (!desc.empty()) MXL_TRY(hipMemcpyAsync(A.blockDesc, desc.data(), desc.size() * 4, hipMemcpyHostToDevice, s));
-    const char *env16 = std::getenv("MX_CSR_COL16");
-    bool narrow = !(env16 && std::atoi(env16) == 0) && nnz > 0;
+    bool narrow = mx::opt().csr_col16 && nnz > 0;
     Buf lo, wide;
     if (narrow) {
         MXL_TRY(hipMalloc(&lo.p, std::max<size_t>((size_t)A.nBlocks, 1) * 4));
@@ -846,8 +842,7 @@ int upload_csr_device(mx_dtype dtype, int rows, int cols, int nnz, const int *ro
                            (const int *)lo.p, A.nBlocks, A.col16);
         MXL_TRY(hipGetLastError());
         A.colBase = (int *)lo.take();
-        const char *ed = std::getenv("MX_CSR_DICT");
-        if (nnz >= 65536 && !(ed && !std::atoi(ed))) {
+        if (nnz >= 65536 && mx::opt().csr_dict != 0) {
             Buf codes;
             std::vector<unsigned char> dict;
             int nd = 0, rc;
@@ -879,6 +874,7 @@ int build_slices_device(mx_dtype dtype, int rows, int cols, int nnz, const int *
         set_error("slice layout on the device: bad argument");
         return MX_ERR_ARG;
     }
+    MXL_TRY(prepare_slice_kernels(dtype));
     if (dtype == MX_F64)
         return build_slices_device_t<double>(dtype, rows, cols, nnz, rowPtr_dev, col_dev, (const double *)val_dev, nCU, S, elsewhere_dev, D,
                                              s, segPtrOut, segIdxOut);

@@ -1,5 +1,7 @@
 // Error text and binary16 conversions shared by the host code.
+#include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "mx_internal.h"
 
@@ -8,6 +10,50 @@ namespace mx {
 static thread_local std::string g_error;
 
 void set_error(const std::string &msg) { g_error = msg; }
+
+// One set for the process (the planners read it from OpenMP workers too).  It is rewritten only when the
+// environment reads differently from the last time, so threads that make plans side by side under one
+// environment never write it.
+static Options g_options;
+static std::mutex g_options_mu;
+const Options &opt() { return g_options; }
+static bool same(const Options &a, const Options &b)
+{
+    return a.tile_gate == b.tile_gate && a.csr_dict == b.csr_dict && a.no_strips == b.no_strips && a.no_blocks == b.no_blocks &&
+           a.strips_apart == b.strips_apart && a.csr_kernel == b.csr_kernel && a.csr_fused == b.csr_fused && a.autotune == b.autotune &&
+           a.layout_host == b.layout_host && a.slice_cap == b.slice_cap && a.split_len == b.split_len && a.csr_npt == b.csr_npt &&
+           a.tile_per == b.tile_per && a.csr_reduce == b.csr_reduce && a.csr_col16 == b.csr_col16 && a.plan_log == b.plan_log;
+}
+void refresh_options()
+{
+    Options o;
+    auto text = [](const char *name) { return std::getenv(name); };
+    auto number = [&](const char *name, int unset) {
+        const char *e = text(name);
+        return e ? std::atoi(e) : unset;
+    };
+    if (const char *e = text("MX_TILE_GATE")) {
+        const double v = std::atof(e);
+        if (v >= 0.0 && v <= 1.0) o.tile_gate = v;
+    }
+    o.csr_dict = number("MX_CSR_DICT", 1);
+    o.no_strips = number("MX_NO_STRIPS", 0) != 0;
+    o.no_blocks = number("MX_NO_BLOCKS", 0) != 0;
+    o.strips_apart = number("MX_STRIPS_APART", 0) != 0;
+    if (const char *e = text("MX_CSR_KERNEL")) o.csr_kernel = !std::strcmp(e, "rows") ? 1 : !std::strcmp(e, "slices") ? 2 : !std::strcmp(e, "split") ? 3 : 0;
+    if (const char *e = text("MX_CSR_FUSED")) o.csr_fused = std::atoi(e) ? 1 : 0;
+    o.autotune = number("MX_PLAN_AUTOTUNE", 0) != 0;
+    if (const char *e = text("MX_LAYOUT")) o.layout_host = !std::strcmp(e, "host");
+    o.slice_cap = number("MX_SLICE_CAP", 0);
+    o.split_len = number("MX_SPLIT_LEN", 0);
+    o.csr_npt = number("MX_CSR_NPT", 0);
+    o.tile_per = number("MX_TILE_PER", 0);
+    if (const char *e = text("MX_CSR_REDUCE")) o.csr_reduce = !std::strcmp(e, "rows") ? 1 : !std::strcmp(e, "scan") ? 2 : 0;
+    o.csr_col16 = number("MX_CSR_COL16", 1) != 0;
+    o.plan_log = number("MX_PLAN_LOG", 0) != 0;
+    std::lock_guard<std::mutex> lock(g_options_mu);
+    if (!same(g_options, o)) g_options = o;
+}
 
 uint16_t f64_to_f16_bits(double v)
 {

@@ -7,6 +7,7 @@ hipError_t launch_csr(mx_dtype, const DeviceCsr &, const void *, void *, int, hi
 hipError_t launch_slices(mx_dtype, const DeviceSlices &, const void *, void *, int, hipStream_t, int, const DeviceTiles *, void *) { return hipErrorUnknown; }
 hipError_t launch_fused(mx_dtype, const DeviceSlices &, const void *, void *, int, hipStream_t, void *, unsigned *, unsigned) { return hipErrorUnknown; }
 hipError_t fused_placement_ok(int, int *ok) { *ok = 0; return hipErrorUnknown; }
+hipError_t prepare_slice_kernels(mx_dtype) { return hipErrorUnknown; }
 hipError_t static_scratch(void **p) { *p = nullptr; return hipErrorUnknown; }
 int build_slices_device(mx_dtype, int, int, int, const int *, const int *, const void *, int, int, const char *, DeviceSlices &, hipStream_t,
                         std::vector<int> *, std::vector<int> *) { return MX_ERR_DEVICE; }

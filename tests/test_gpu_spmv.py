@@ -136,6 +136,45 @@ def test_structure_off_the_grid_matches_oracle(mx, ora, cfg, scale):
         part.close()
 
 
+def test_environment_is_read_when_a_plan_is_made_and_kept(mx, ora, monkeypatch):
+    """The switches of the environment are read when a plan is created, kept with it and reported
+    (mx_plan_info.opt_flags, opt_tile_gate); a plan runs as it was made whatever the environment says later."""
+    import torch
+    A, x = mx.gen_config(5, scale=0.125)
+    ref = oracle_y(ora, mx, A, x)
+    xd = torch.from_numpy(x).cuda()
+    part = mx.Partition(A, 1.0, 1.0)
+    for name in ("MX_NO_STRIPS", "MX_STRIPS_APART", "MX_TILE_GATE", "MX_CSR_DICT"):
+        monkeypatch.delenv(name, raising=False)
+    plain = mx.Plan(part, mx.MX_PLAN_KEEP_TILES)
+    assert plain.info["opt_flags"] == 0 and plain.info["opt_tile_gate"] == 0.5, plain.info
+    assert plain.info["tile_variant"] == 1 and plain.info["tile_strip_nnz"] > 0
+    y_plain = plain.spmv(xd).clone()
+    monkeypatch.setenv("MX_NO_STRIPS", "1")
+    monkeypatch.setenv("MX_TILE_GATE", "0.75")
+    bare = mx.Plan(part, mx.MX_PLAN_KEEP_TILES)
+    assert bare.info["opt_flags"] == mx.MX_OPT_NO_STRIPS and bare.info["opt_tile_gate"] == 0.75, bare.info
+    assert bare.info["tile_strip_nnz"] == 0
+    assert plain.info["opt_flags"] == 0 and plain.info["tile_strip_nnz"] > 0       # the older plan is what it was
+    assert torch.equal(plain.spmv(xd), y_plain)
+    monkeypatch.delenv("MX_NO_STRIPS")
+    monkeypatch.delenv("MX_TILE_GATE")
+    monkeypatch.setenv("MX_STRIPS_APART", "1")
+    apart = mx.Plan(part, mx.MX_PLAN_KEEP_TILES)
+    assert apart.info["opt_flags"] == mx.MX_OPT_STRIPS_APART, apart.info
+    monkeypatch.delenv("MX_STRIPS_APART")
+    kinds = {}
+    for name, plan in (("plain", plain), ("bare", bare), ("apart", apart)):
+        y = plan.spmv(xd)
+        torch.cuda.synchronize()
+        assert rel_l2(y.cpu().numpy(), ref) <= F16_TOL, name
+        kinds[name] = [r["name"] for r in plan.time_kernels(xd, y, 2, 5)]
+        plan.close()
+    assert any("tile_dense_kernel" in k for k in kinds["apart"]), kinds      # its own launch, also after the switch is gone
+    assert not any("tile_dense_kernel" in k for k in kinds["plain"]), kinds
+    part.close()
+
+
 # ---------------------------------------------------------------- full benchmark sizes
 FULL = [
     # (workload, taus)

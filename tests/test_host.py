@@ -974,7 +974,9 @@ def test_host_code_under_sanitizers(tmp_path):
            "-fno-sanitize-recover=undefined", "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(ROOT, "include"), "-I" + src,
            "-I/opt/rocm/include", os.path.join(ROOT, "tests", "sanitize", "host_driver.cpp"),
            os.path.join(ROOT, "tests", "sanitize", "launch_stubs.cpp")] + \
-          [os.path.join(src, f) for f in ("mx_util.cpp", "mx_partition.cpp", "mx_gen.cpp", "mx_mmio.cpp", "mx_plan.cpp")] + \
+          [os.path.join(src, f) for f in ("mx_util.cpp", "mx_partition.cpp", "mx_gen.cpp", "mx_mmio.cpp", "mx_host_layout.cpp",
+                                          "mx_plan.cpp", "mx_plan_device.cpp", "mx_plan_view.cpp", "mx_run.cpp", "mx_tune.cpp",
+                                          "mx_oneshot.cpp")] + \
           ["-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib", "-o", exe]
     b = subprocess.run(cmd, capture_output=True, text=True)
     if b.returncode != 0 and ("asan" in b.stderr or "ubsan" in b.stderr) and "cannot find" in b.stderr:
