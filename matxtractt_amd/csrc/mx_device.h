@@ -138,8 +138,9 @@ struct DeviceSlices {
     // virtual row of row r at [((r / G) * placesPerRow + k) * G + r % G], G = kFusedGroupRows, so that a
     // wave that adds 64 consecutive rows reads 64 consecutive sums per place and needs no index list;
     // fusedTarget names that place for every virtual row (a workgroup keeps its chunks' part of it in
-    // LDS, which bounds the chunks a workgroup may have), rowVrows[r] says how many places of row r hold
-    // a sum.  The arrays above stay valid for the two-launch form, which a plan falls back to.
+    // LDS, which bounds the chunks a workgroup may have).  A place that no virtual row owns keeps the zero
+    // it was allocated with, so the one who adds takes all placesPerRow places of a row without asking how
+    // many count.  The arrays above stay valid for the two-launch form, which a plan falls back to.
     bool fused = false;
     int nGroups = 0, maxWgGroups = 0;
     int placesPerRow = 0;             // 4 or 8: most virtual rows of a row
@@ -147,13 +148,13 @@ struct DeviceSlices {
     int *groupNeed = nullptr;         // [nGroups] workgroups that bump the group's counter
     int *groupCount = nullptr;        // [nGroups] the counters; zero between launches (the last arriver clears its own)
     int *fusedTarget = nullptr;       // [chunks * 64] where virtual row 64 * chunk + lane puts its sum (a spare place for padding lanes)
-    unsigned char *rowVrows = nullptr;// [nGroups * G] virtual rows of every row
-    void *fusedSums = nullptr;        // [nGroups * placesPerRow * G + 64] accumulators
+    void *fusedSums = nullptr;        // [nGroups * placesPerRow * G + 64] accumulators; zero where no virtual row writes
     unsigned *claim = nullptr;        // [nWG] launches in which each logical workgroup's work was taken (once each)
 };
 constexpr int kFusedGroupRows = 256;  // rows whose sums one arriver adds up at a time
 constexpr int kFusedXcds = 8;         // L2 domains of the device the one-launch form is laid out for
 constexpr int kFusedWgChunks = 96;    // most chunks of a workgroup in that form (their targets, 256 bytes each, share the LDS with x)
+constexpr int kFusedWgGroups = 255;  // most groups a workgroup may hold sums of
 constexpr int kSliceBytes = 131072;   // the slice of x a workgroup keeps in LDS
 constexpr int kSliceLdsMax = 163840;  // LDS of a CU
 constexpr int kSliceWgChunks = 4096;  // most chunks a workgroup may have

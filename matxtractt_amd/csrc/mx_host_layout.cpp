@@ -100,7 +100,6 @@ void free_slices(mx::DeviceSlices &P)
     (void)hipFree(P.groupNeed);
     (void)hipFree(P.groupCount);
     (void)hipFree(P.fusedTarget);
-    (void)hipFree(P.rowVrows);
     (void)hipFree(P.fusedSums);
     (void)hipFree(P.claim);
     P = mx::DeviceSlices();
@@ -415,6 +414,7 @@ static bool plan_fused(mx_dtype dtype, int budget, int S, int rows, int nGroups,
                 const int gb = i + 1 == live.size() ? xg[k + 1] - 1 : std::max(rowHi[b] / GR, rowLo[live[i + 1]] / GR - 1);
                 SP.wgGroups[(size_t)b * 2] = ga;
                 SP.wgGroups[(size_t)b * 2 + 1] = gb - ga + 1;
+                if (gb - ga + 1 > mx::kFusedWgGroups) return false;  // (a lane per group counts it off)
                 SP.maxWgGroups = std::max(SP.maxWgGroups, gb - ga + 1);
                 for (int g = ga; g <= gb; ++g) ++SP.groupNeed[g];
             }
@@ -739,7 +739,6 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
         if ((rc = upload(&D.groupNeed, H.groupNeed.data(), H.groupNeed.size()))) return rc;
         if ((rc = upload(&D.groupCount, (const int *)nullptr, 0, (size_t)H.nGroups + 1))) return rc;
         if ((rc = upload(&D.fusedTarget, H.fusedTarget.data(), H.fusedTarget.size(), 64))) return rc;
-        if ((rc = upload(&D.rowVrows, H.rowVrows.data(), H.rowVrows.size(), 64))) return rc;
         if ((rc = upload_bytes(&D.fusedSums, nullptr, 0, ((size_t)H.nGroups * H.placesPerRow * mx::kFusedGroupRows + 64) * (dtype == MX_F64 ? 8 : 4))))
             return rc;
         if ((rc = upload(&D.claim, (const unsigned *)nullptr, 0, (size_t)H.nWG + 1))) return rc;

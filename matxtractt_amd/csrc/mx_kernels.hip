@@ -493,12 +493,15 @@ struct SliceBatch<double> {
         for (int j = 0; j < 4; ++j)
             v[j] = __builtin_nontemporal_load((const v2f64 *)(eval + batch * 512 + j * 128 + lane * 2));
     }
-    // value * x of entry k of the batch
-    __device__ __forceinline__ double term(const double *xs, int k) const
+    // what entry k of the batch multiplies with: its x (a lane asks for all of a batch's before it uses
+    // the first, so the LDS answers them in one go) ...
+    __device__ __forceinline__ double gather(const double *xs, int k) const
     {
         const unsigned w = (unsigned)c[k >> 1];
-        return (k & 1) ? v[k >> 1].y * xs[w >> 16] : v[k >> 1].x * xs[w & 0xffffu];
+        return (k & 1) ? xs[w >> 16] : xs[w & 0xffffu];
     }
+    // ... and value * x
+    __device__ __forceinline__ double term(int k, double xk) const { return ((k & 1) ? v[k >> 1].y : v[k >> 1].x) * xk; }
 };
 template <>
 struct SliceBatch<_Float16> {
@@ -508,11 +511,16 @@ struct SliceBatch<_Float16> {
         c = __builtin_nontemporal_load((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
         v = __builtin_nontemporal_load((const v4i32 *)(eval + (batch * 64 + lane) * 8));
     }
-    __device__ __forceinline__ float term(const _Float16 *xs, int k) const
+    __device__ __forceinline__ _Float16 gather(const _Float16 *xs, int k) const
     {
-        const unsigned cw = (unsigned)c[k >> 1], vw = (unsigned)v[k >> 1];
-        const unsigned ci = (k & 1) ? cw >> 16 : cw & 0xffffu, vi = (k & 1) ? vw >> 16 : vw & 0xffffu;
-        return (float)__builtin_bit_cast(_Float16, (unsigned short)vi) * (float)xs[ci];
+        const unsigned cw = (unsigned)c[k >> 1];
+        return xs[(k & 1) ? cw >> 16 : cw & 0xffffu];
+    }
+    __device__ __forceinline__ float term(int k, _Float16 xk) const
+    {
+        const unsigned vw = (unsigned)v[k >> 1];
+        const unsigned vi = (k & 1) ? vw >> 16 : vw & 0xffffu;
+        return (float)__builtin_bit_cast(_Float16, (unsigned short)vi) * (float)xk;
     }
 };
 // The same with a value dictionary: a byte per entry that names one of at most 256 distinct
@@ -527,13 +535,12 @@ struct SliceBatchDict {
         c = __builtin_nontemporal_load((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
         k = __builtin_nontemporal_load((const v2i32 *)(ecode + (batch * 64 + lane) * 8));
     }
-    __device__ __forceinline__ AT term(const VT *xs, int j, const AT *dict) const
+    __device__ __forceinline__ VT gather(const VT *xs, int j) const
     {
         const unsigned cw = (unsigned)c[j >> 1];
-        const unsigned ci = (j & 1) ? cw >> 16 : cw & 0xffffu;
-        const unsigned code = ((unsigned)k[j >> 2] >> (8 * (j & 3))) & 255u;
-        return dict[code] * (AT)xs[ci];
+        return xs[(j & 1) ? cw >> 16 : cw & 0xffffu];
     }
+    __device__ __forceinline__ AT value(const AT *dict, int j) const { return dict[((unsigned)k[j >> 2] >> (8 * (j & 3))) & 255u]; }
 };
 static_assert(mx::kSliceBatchEntries == 8, "SliceBatch holds 8 entries per lane");
 
@@ -551,7 +558,6 @@ struct FusedArgs {
     const int *groupNeed = nullptr;  // [groups]
     int *groupCount = nullptr;       // [groups]
     const int *target = nullptr;     // [chunks * 64] where every virtual row puts its sum
-    const unsigned char *rowVrows = nullptr;  // [rows rounded up to whole groups] virtual rows of every row
     void *sums = nullptr;            // the sums, laid out for the one who adds
     unsigned *misplaced = nullptr;   // host memory: set when two workgroups of a launch took the same work
     unsigned *claim = nullptr;       // [workgroups] how often each logical workgroup's work has been taken
@@ -581,6 +587,57 @@ __device__ __forceinline__ T load_from_l2(const T *p)
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
+// The last step of the one-launch form: the rows of the `nl` groups in `list` added up by one workgroup.
+// A lane takes R rows at a time, one from each of R groups (2 groups side by side in a workgroup of
+// 512), and asks for everything it needs -- every place of every row, used or not: a place that no
+// virtual row owns holds the zero it was made with -- before it uses any of it: one trip for the lot,
+// and nothing is read that this launch did not write.  The 64 rows of a wave are consecutive, so every
+// load is one contiguous stretch.  Sums in the order of the places, whoever adds: y does not depend on
+// who came last.
+template <typename VT, int P, int R>
+__device__ __forceinline__ void fused_add(const FusedArgs &fa, const int *list, int nl, int tid)
+{
+    typedef typename Acc<VT>::type AT;
+    constexpr int GR = mx::kFusedGroupRows, SIDE = kSliceThreads / GR;  // groups side by side
+    static_assert(kSliceThreads % GR == 0 && GR == 256, "a lane keeps its place inside the group from slot to slot");
+    const AT *sums = (const AT *)fa.sums;
+    VT *y = (VT *)fa.y;
+    AT *ywide = (AT *)fa.ywide;
+    const int half = __builtin_amdgcn_readfirstlane(tid / GR), rl = tid % GR;
+    for (int j0 = 0; j0 < nl; j0 += SIDE * R) {
+        int row[R];
+        AT v[R][P], old[R];
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            // (whether a slot holds a group is the same for all lanes of a wave: a branch, not a mask, so
+            // that an empty slot costs no traffic; nothing is waited for between the slots)
+            const int li = j0 + half + SIDE * i;
+            row[i] = -1;
+            old[i] = 0;
+#pragma unroll
+            for (int k = 0; k < P; ++k) v[i][k] = 0;
+            if (li < nl) {
+                const int g = list[li];
+                if (g * GR + rl < fa.rows) row[i] = g * GR + rl;
+                const AT *p = sums + (size_t)g * P * GR + rl;
+#pragma unroll
+                for (int k = 0; k < P; ++k) v[i][k] = load_from_l2(p + (size_t)k * GR);
+                if (fa.accumulate) old[i] = (AT)y[max(row[i], 0)];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            AT sum = old[i];
+#pragma unroll
+            for (int k = 0; k < P; ++k) sum += v[i][k];
+            if (row[i] >= 0) {
+                y[row[i]] = (VT)sum;
+                if (ywide) ywide[row[i]] = sum;
+            }
+        }
+    }
+}
+
 // DICT: `eval` points at one byte per entry (same places as the column offsets) and `dictG` at the
 // 256 values they name; a workgroup keeps those in LDS behind the chunk ends.
 // FUSED: the one-launch form.  The layout gives every XCD the same number of logical workgroups
@@ -589,8 +646,9 @@ __device__ __forceinline__ T load_from_l2(const T *p)
 // dispatcher deals consecutive workgroups round-robin to the XCDs, from a starting XCD that depends
 // on what ran before, so the workgroups that land on one XCD have distinct blockIdx / 8 and every
 // logical workgroup is taken once.  That one assumption is checked in every launch: each logical
-// workgroup's `claim` is counted up by whoever takes it, and a count that is not the launch's
-// number means that two took the same; the launch's y cannot be trusted then and the host is told.
+// workgroup's `claim` is counted up by whoever takes it (together with the group counters, at the end),
+// and a count that is not the launch's number means that two took the same; the launch's y cannot be
+// trusted then and the host is told.
 // The sums are stored where the one who adds finds them without an index list (DeviceSlices::fusedSums;
 // a workgroup keeps the places of its own virtual rows in LDS).  After its stream a workgroup waits until its own
 // stores have reached the L2 (s_waitcnt vmcnt(0): a store counts as done when the L2 has it),
@@ -612,7 +670,8 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     typedef typename std::conditional<DICT, SliceBatchDict<VT>, SliceBatch<VT>>::type Batch;
     typedef typename std::conditional<DICT, unsigned char, VT>::type StreamT;
     const StreamT *estream = (const StreamT *)eval;
-    constexpr int SPB = mx::kSliceBatchEntries, NB = kSliceRing;  // a step is one entry per lane
+    // (a step is one entry per lane; binary64 values as they are leave registers for a ring of five)
+    constexpr int SPB = mx::kSliceBatchEntries, NB = (sizeof(VT) == 8 && !DICT) ? kSliceRing - 1 : kSliceRing;
     constexpr int EPV = 16 / (int)sizeof(VT);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     VT *xs = (VT *)smem;                                           // [sliceCols]
@@ -632,13 +691,12 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     const int4 gd = wgDesc[b];
     const int4 d = waveDesc[b * kSliceWaves + wave];
     const int slice = gd.x, wgChunk0 = gd.y, wgChunks = gd.z;
-    int group0 = 0, nGroupsMine = 0;
-    unsigned claimed = 0;
+    int group0 = 0, nGroupsMine = 0, need = 0;
     if constexpr (FUSED) {
         group0 = fa.wgGroups[2 * b];
         nGroupsMine = fa.wgGroups[2 * b + 1];
-        // (looked at when the work is done: the answer is not waited for here)
-        if (tid == 0) claimed = __hip_atomic_fetch_add(fa.claim + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        // (asked for now, looked at when the stream is done; a workgroup has fewer groups than lanes)
+        need = fa.groupNeed[group0 + min(tid, max(nGroupsMine - 1, 0))];
     }
     const int batch0 = __builtin_amdgcn_readfirstlane(d.x), nb = __builtin_amdgcn_readfirstlane(d.y);
     const int chunk0 = __builtin_amdgcn_readfirstlane(d.z), nChunks = __builtin_amdgcn_readfirstlane(d.w);
@@ -700,11 +758,29 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         nextEnd = ci < nChunks ? __builtin_amdgcn_readfirstlane(endsL[chunk0 + ci]) : -1;
     };
     auto consume = [&](const Batch &B, int t) {  // t = number of the batch in the wave's stream
+        // what the batch needs from LDS is asked for before the first product: with a request and its wait per
+        // entry the wave would sit out one LDS round trip after the other
+        VT xk[SPB];
+        AT vk[DICT ? SPB : 1];
 #pragma unroll
-        for (int j = 0; j < SPB; ++j) {
-            if constexpr (DICT) acc += B.term(xs, j, dictL);
-            else acc += B.term(xs, j);
-            if (t * SPB + j + 1 == nextEnd) flush();
+        for (int j = 0; j < SPB; ++j) xk[j] = B.gather(xs, j);
+        if constexpr (DICT) {
+#pragma unroll
+            for (int j = 0; j < SPB; ++j) vk[j] = B.value(dictL, j);
+        }
+        auto add = [&](int j) {
+            if constexpr (DICT) acc += vk[j] * (AT)xk[j];
+            else acc += B.term(j, xk[j]);
+        };
+        if (nextEnd < 0 || nextEnd > (t + 1) * SPB) {  // no chunk ends inside the batch
+#pragma unroll
+            for (int j = 0; j < SPB; ++j) add(j);
+        } else {
+#pragma unroll
+            for (int j = 0; j < SPB; ++j) {
+                add(j);
+                if (t * SPB + j + 1 == nextEnd) flush();
+            }
         }
     };
     if (nb <= NB) {  // everything is in the ring already
@@ -733,95 +809,30 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
             if (t + NB + k < nb) consume(buf[k], t + NB + k);
     }
     if constexpr (FUSED) {
-        constexpr int GR = mx::kFusedGroupRows, R = 8;           // R rows per lane and pass
-        constexpr int GP = R * kSliceThreads / GR;                 // groups per pass
-        static_assert(kSliceThreads % GR == 0 && GR == 256, "a lane keeps its place inside the group from pass to pass");
-        if (tid == 0 && (claimed != fa.seq || xcc_id() >= mx::kFusedXcds))
-            __hip_atomic_store(fa.misplaced, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        const bool wide8 = fa.placesPerRow == 8;
-        const AT *sums = (const AT *)fa.sums;
-        VT *y = (VT *)fa.y;
-        AT *ywide = (AT *)fa.ywide;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's sums are in the L2
         __syncthreads();                                    // ... and so are the other waves'
         // (the chunk ends are done with) listL[0] = how many groups fall to this workgroup, then which
         int *listL = endsL;
         if (tid == 0) listL[0] = 0;
         __syncthreads();
-        for (int i = tid; i < nGroupsMine; i += kSliceThreads) {
-            const int g = group0 + i;
+        // a lane per group, and one lane more: it takes the workgroup's claim in the same trip
+        if (tid == nGroupsMine) {
+            const unsigned claimed = __hip_atomic_fetch_add(fa.claim + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (claimed != fa.seq || xcc_id() >= mx::kFusedXcds)
+                __hip_atomic_store(fa.misplaced, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        } else if (tid < nGroupsMine) {
+            const int g = group0 + tid;
             const int old = __hip_atomic_fetch_add(fa.groupCount + g, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            if (old + 1 == fa.groupNeed[g]) {
+            if (old + 1 == need) {
                 __hip_atomic_store(fa.groupCount + g, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 listL[1 + atomicAdd(&listL[0], 1)] = g;
             }
         }
         __syncthreads();
-        // A pass: R groups per half of the workgroup, a row per lane and group.  A wave's 64 rows are
-        // consecutive, so every load is one contiguous stretch; the places a row does not use hold
-        // nothing that counts (rowVrows says how many do).
-        const int nl = listL[0], half = tid >> 8, rl = tid & (GR - 1);
-        for (int j0 = 0; j0 < nl; j0 += GP) {
-            int nv[R];
-            AT old[R];
-            bool live[R], take[R];  // take: the slot holds a group (the same for the whole wave)
-            size_t base[R];
-#pragma unroll
-            for (int i = 0; i < R; ++i) {
-                const int li = j0 + half + (kSliceThreads / GR) * i;
-                const int g = listL[1 + min(li, nl - 1)];
-                const int r = g * GR + rl;
-                take[i] = __builtin_amdgcn_readfirstlane((int)(li < nl)) != 0;
-                live[i] = take[i] && r < fa.rows;
-                nv[i] = fa.rowVrows[r];
-                base[i] = (size_t)g * (wide8 ? 8 : 4) * GR + rl;
-                old[i] = fa.accumulate && live[i] ? (AT)y[r] : (AT)0;
-            }
-            if (wide8) {
-                AT v[R][8];
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) v[i][k] = 0;
-                    if (take[i]) {
-                        // (places beyond the most any of the wave's 64 rows uses are not asked for)
-                        const int most = wave_max(nv[i]);
-#pragma unroll
-                        for (int k = 0; k < 8; ++k)
-                            if (k < most) v[i][k] = load_from_l2(sums + base[i] + (size_t)k * GR);
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    AT sum = old[i];
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) sum += k < nv[i] ? v[i][k] : (AT)0;  // (in the order of the places: y does not depend on who adds)
-                    const int r = listL[1 + min(j0 + half + (kSliceThreads / GR) * i, nl - 1)] * GR + rl;
-                    if (live[i]) y[r] = (VT)sum;
-                    if (live[i] && ywide) ywide[r] = sum;
-                }
-            } else {
-                AT v[R][4];
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) v[i][k] = 0;
-                    if (take[i]) {
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) v[i][k] = load_from_l2(sums + base[i] + (size_t)k * GR);
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    AT sum = old[i];
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) sum += k < nv[i] ? v[i][k] : (AT)0;
-                    const int r = listL[1 + min(j0 + half + (kSliceThreads / GR) * i, nl - 1)] * GR + rl;
-                    if (live[i]) y[r] = (VT)sum;
-                    if (live[i] && ywide) ywide[r] = sum;
-                }
-            }
-        }
+        const int nl = listL[0];
+        if (nl == 0) return;
+        if (fa.placesPerRow == 8) fused_add<VT, 8, 4>(fa, listL + 1, nl, tid);
+        else fused_add<VT, 4, 8>(fa, listL + 1, nl, tid);
     }
 }
 
@@ -1519,7 +1530,7 @@ static hipError_t launch_fused_t(const DeviceSlices &P, const void *x, void *y, 
     const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)((ldsInts + 3) & ~3) * 4 + 64 + (dict ? 256 * sizeof(AT) : 0) +
                        (size_t)P.maxWgChunks * 256;
     if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16) || !P.fused || !P.wgGroups ||
-        !P.groupNeed || !P.groupCount || !P.fusedTarget || !P.rowVrows || !P.fusedSums || !P.claim || !misplaced || (P.placesPerRow != 4 && P.placesPerRow != 8) ||
+        !P.groupNeed || !P.groupCount || !P.fusedTarget || !P.fusedSums || !P.claim || !misplaced || (P.placesPerRow != 4 && P.placesPerRow != 8) ||
         P.nWG <= 0 || P.nWG % mx::kFusedXcds)
         return hipErrorInvalidValue;
     mxk::FusedArgs fa;
@@ -1529,7 +1540,6 @@ static hipError_t launch_fused_t(const DeviceSlices &P, const void *x, void *y, 
     fa.groupNeed = P.groupNeed;
     fa.groupCount = P.groupCount;
     fa.target = P.fusedTarget;
-    fa.rowVrows = P.rowVrows;
     fa.sums = P.fusedSums;
     fa.misplaced = misplaced;
     fa.claim = P.claim;

@@ -86,7 +86,6 @@ extern "C" int mx_plan_arrays(const mx_plan *plan, mx_plan_array *out, int cap, 
             add("slices.wgGroups", D.wgGroups, ((size_t)D.nWG * 2 + 2) * 4);
             add("slices.groupNeed", D.groupNeed, ((size_t)D.nGroups + 1) * 4);
             add("slices.fusedTarget", D.fusedTarget, (size_t)D.chunks * 64 * 4);
-            add("slices.rowVrows", D.rowVrows, (size_t)D.nGroups * mx::kFusedGroupRows);
         }
     }
     const mx::DeviceTiles *two[2] = {&plan->tiles, &plan->strips};
