@@ -747,7 +747,11 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     }
     __syncthreads();
     // (the chunk ends are the same for all lanes of the wave: kept in scalar registers)
-    int ci = 0, nextEnd = nChunks > 0 ? __builtin_amdgcn_readfirstlane(endsL[chunk0]) : -1;
+    // and 64 at a time, lane i holding the end of the wave's chunk 64 * (ci / 64) + i, so that the next end is
+    // there without a trip to the LDS when a chunk is done (chunks of a few entries end every few steps)
+    auto ends64 = [&](int c0) { return endsL[chunk0 + min(c0 + lane, max(nChunks - 1, 0))]; };
+    int endsV = ends64(0);
+    int ci = 0, nextEnd = nChunks > 0 ? __builtin_amdgcn_readlane(endsV, 0) : -1;
     AT acc = 0;
     AT *out = partial + (size_t)(wgChunk0 + chunk0) * 64 + lane;
     auto flush = [&]() {
@@ -755,7 +759,8 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         else out[(size_t)ci * 64] = acc;
         acc = 0;
         ++ci;
-        nextEnd = ci < nChunks ? __builtin_amdgcn_readfirstlane(endsL[chunk0 + ci]) : -1;
+        if ((ci & 63) == 0) endsV = ends64(ci);
+        nextEnd = ci < nChunks ? __builtin_amdgcn_readlane(endsV, ci & 63) : -1;
     };
     auto consume = [&](const Batch &B, int t) {  // t = number of the batch in the wave's stream
         // what the batch needs from LDS is asked for before the first product: with a request and its wait per
