@@ -381,6 +381,45 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
     return rec, (A, x)
 
 
+def tau_family(mx, torch, scales):
+    """mx_estimate_tau held against mx_tune_tau on matrices neither was calibrated on: the families around
+    workloads 5 (5 to 40 % of the row runs in strips) and 2 (10 to 70 % of the entries in 8x8 blocks), on and off
+    the grid of eight columns.  Per case: the estimated and the timed fractions, the time of a default plan at
+    each (median of 3 trains of 200 + 1000 products) and the regret of the estimate."""
+    dev = torch.device("cuda:0")
+
+    def timed(A, xd, tau):
+        part = mx.Partition(A, tau[0], tau[1])
+        plan = mx.Plan(part, mx.MX_PLAN_DEFAULT)
+        y = torch.zeros(A.rows, dtype=xd.dtype, device=dev)
+        ms = median_time(lambda: plan.time(xd, y, 200, 1000, parts=False)[0], 3)
+        tiles = plan.info["tile_nnz"]
+        plan.close()
+        part.close()
+        return ms, tiles
+    rows = []
+    for scale in scales:
+        for unaligned in (False, True):
+            for cfg, shares in ((5, (0.05, 0.1, 0.2, 0.4)), (2, (0.1, 0.25, 0.4, 0.7))):
+                for share in shares:
+                    A, x = mx.gen_config(cfg, scale=scale, unaligned=unaligned, dense_share=share)
+                    xd = torch.from_numpy(x).to(dev)
+                    ec, er, _ = mx.estimate_tau(A, 5)
+                    tc, tr, _ = mx.tune_tau(A, 5, mx.MX_PLAN_DEFAULT, 50, 300)
+                    ms_e, tiles_e = timed(A, xd, (ec, er))
+                    same = (ec, er) == (tc, tr)
+                    ms_t, tiles_t = (ms_e, tiles_e) if same else timed(A, xd, (tc, tr))
+                    rows.append({"workload": cfg, "scale": scale, "unaligned": unaligned, "dense_share": share, "rows": A.rows, "nnz": A.nnz,
+                                 "estimated": [ec, er], "estimated_us": ms_e * 1e3, "estimated_tile_nnz": tiles_e,
+                                 "tuned": [tc, tr], "tuned_us": ms_t * 1e3, "tuned_tile_nnz": tiles_t,
+                                 "regret": ms_e / ms_t - 1.0})
+                    log("tau family: workload %d scale %g %s share %.2f: estimate (%.2f, %.2f) %.2f us, tuned (%.2f, %.2f) %.2f us, regret %+.1f %%" % (
+                        cfg, scale, "off the grid" if unaligned else "aligned", share, ec, er, ms_e * 1e3, tc, tr, ms_t * 1e3, (ms_e / ms_t - 1) * 100))
+                    del A, x, xd
+    return {"cases": rows, "worst_regret": max(r["regret"] for r in rows),
+            "how": "regret = time of the default plan at mx_estimate_tau's fractions over that at mx_tune_tau's timed best, minus one"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -395,6 +434,9 @@ def main():
     ap.add_argument("--no-unaligned", action="store_true", help="skip the variants of workloads 2 and 5 with structure off the grid")
     ap.add_argument("--all-tiles", action="store_true",
                     help="plans with MX_PLAN_ALL_TILES: every extracted chunk through the general MFMA tile kernel (profile runs)")
+    ap.add_argument("--tau-family", choices=("none", "quarter", "full"), default="quarter",
+                    help="check mx_estimate_tau against mx_tune_tau over the families around workloads 2 and 5: at a quarter of "
+                         "the benchmark's size (default, about half a minute), at a quarter and at full size, or not at all")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also launch one elementwise kernel that reads and writes MIB MiB (a known size to "
                          "scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -477,6 +519,8 @@ def main():
             if cfg in SWEPT:
                 r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, "sweep", traffic, None, keep, unaligned=True, brief=True)
                 others["workload_%d_unaligned" % cfg] = r
+    if args.tau_family != "none" and not args.no_sweep and args.tau is None and not args.all_tiles and args.workload is None:
+        out["tau_estimate_family"] = tau_family(mx, torch, (0.25,) if args.tau_family == "quarter" else (0.25, 1.0))
     if others:
         out["others"] = others
     out["bench_seconds"] = time.time() - t_start

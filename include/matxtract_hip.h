@@ -231,6 +231,12 @@ int mx_gen_config(int config_id, uint64_t seed, double scale, int *rows, int *co
 #define MX_GEN_UNALIGNED 1
 int mx_gen_config_ex(int config_id, uint64_t seed, double scale, int gen_flags, int *rows, int *cols, int *nnz,
                      mx_dtype *dtype, int **rowPtr, int **colInd, void **val, void **x);
+/* Members of the families around workloads 2 and 5, for checking decisions away from the benchmark's own
+ * matrices: dense_share is the share of the entries that sit in dense 8x8 blocks (workload 2; 0.4 in the
+ * benchmark, up to 1) or the probability that a run of 128 rows is a strip (workload 5; 0.2 in the benchmark).
+ * A negative share means the benchmark's; other workloads take no share. */
+int mx_gen_config_family(int config_id, uint64_t seed, double scale, int gen_flags, double dense_share, int *rows, int *cols,
+                         int *nnz, mx_dtype *dtype, int **rowPtr, int **colInd, void **val, void **x);
 
 /* Algorithmic bytes of one SpMV: nnz*(sizeof(valT)+4) + (rows+1)*4 + cols*sizeof(valT) +
  * rows*sizeof(valT) (`data_origin1`, test/test_cdspmv.cpp:214). */

@@ -138,6 +138,7 @@ SIGNATURES = {
     "mx_f16_to_f32": (C.c_float, [C.c_uint16]),
     "mx_gen_config": (_i, [_i, C.c_uint64, _d, _pi, _pi, _pi, _pi, _pp, _pp, _pp, _pp]),
     "mx_gen_config_ex": (_i, [_i, C.c_uint64, _d, _i, _pi, _pi, _pi, _pi, _pp, _pp, _pp, _pp]),
+    "mx_gen_config_family": (_i, [_i, C.c_uint64, _d, _i, _d, _pi, _pi, _pi, _pi, _pp, _pp, _pp, _pp]),
     "mx_algorithmic_bytes": (_d, [_i, _i, _i, _i]),
     "mx_plan_create": (_i, [_vp, _i, _pp]),
     "mx_plan_create_device_csr": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _i, _pp]),

@@ -82,14 +82,17 @@ class Csr:
         return algorithmic_bytes(self.dtype, self.rows, self.cols, self.nnz)
 
 
-def gen_config(config_id, seed=0, scale=1.0, unaligned=False):
+def gen_config(config_id, seed=0, scale=1.0, unaligned=False, dense_share=None):
     """Synthetic workload 1..5 -> (Csr, x).  unaligned=True: the dense blocks of workload 2 and the strips of
-    workload 5 start off the grid of eight columns (mx_gen_config_ex, MX_GEN_UNALIGNED)."""
+    workload 5 start off the grid of eight columns (MX_GEN_UNALIGNED).  dense_share: how much of workload 2
+    (share of the entries in 8x8 blocks, 0.4 in the benchmark) or 5 (probability that a run of 128 rows is a
+    strip, 0.2) is dense structure (mx_gen_config_family)."""
     L = _lib.load()
     rows, cols, nnz, dt = C.c_int(), C.c_int(), C.c_int(), C.c_int()
     rp, ci, va, xv = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
-    check(L.mx_gen_config_ex(config_id, seed, scale, 1 if unaligned else 0, C.byref(rows), C.byref(cols), C.byref(nnz), C.byref(dt),
-                             C.byref(rp), C.byref(ci), C.byref(va), C.byref(xv)))
+    check(L.mx_gen_config_family(config_id, seed, scale, 1 if unaligned else 0, -1.0 if dense_share is None else float(dense_share),
+                                 C.byref(rows), C.byref(cols), C.byref(nnz), C.byref(dt), C.byref(rp), C.byref(ci), C.byref(va),
+                                 C.byref(xv)))
     vt = _np_dtype(dt.value)
     A = Csr(rows.value, cols.value, _take(rp.value, rows.value + 1, np.int32),
             _take(ci.value, nnz.value, np.int32), _take(va.value, nnz.value, vt))

@@ -31,6 +31,10 @@
 // (its eight rows still start at a multiple of eight; blocks of one block row do not overlap), and a
 // strip of workload 5 starts at 8*(block + off) + shift with shift uniform in [1, 7] per strip.
 // Everything else is drawn as before.
+//
+// mx_gen_config_family varies how much of the matrix is dense structure: the share of the entries that
+// sit in 8x8 blocks (workload 2, 0.4 in the benchmark) or the probability that a run of 128 rows is a
+// strip (workload 5, 0.2 in the benchmark).
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
@@ -152,11 +156,11 @@ void gen_random(Rng &g, int n, int per_row, Builder &B)
     }
 }
 
-void gen_block_clustered(Rng &g, int n, Builder &B, bool unaligned)
+void gen_block_clustered(Rng &g, int n, Builder &B, bool unaligned, double share)
 {
     const int per_row = std::min(64, n), nb = n / 8;
     const int max_blocks_per_row = per_row / 8;
-    int want = (int)std::floor(0.4 * (double)n * per_row / 64.0);
+    int want = (int)std::floor(share * (double)n * per_row / 64.0);
     std::vector<std::vector<int>> blocks(nb);  // first column of every block of each block row
     int placed = 0;
     for (long long attempts = 0; placed < want && attempts < 64LL * want + 1024; ++attempts) {
@@ -209,13 +213,13 @@ void gen_stencil27(int g3, Builder &B)
             }
 }
 
-void gen_mixed(Rng &g, int n, Builder &B, bool unaligned)
+void gen_mixed(Rng &g, int n, Builder &B, bool unaligned, double share)
 {
     PowerLaw pl(n);
     const int run = 128;
     for (int r0 = 0; r0 < n; r0 += run) {
         int r1 = std::min(r0 + run, n);
-        bool strip = g.u01() < 0.2 && n >= 64;
+        bool strip = g.u01() < share && n >= 64;
         int off = g.below(65) - 32;
         const int shift = unaligned ? 1 + g.below(7) : 0;
         for (int r = r0; r < r1; ++r) {
@@ -250,8 +254,15 @@ extern "C" int mx_gen_config(int config_id, uint64_t seed, double scale, int *ro
 extern "C" int mx_gen_config_ex(int config_id, uint64_t seed, double scale, int gen_flags, int *rows, int *cols, int *nnz,
                                 mx_dtype *dtype, int **rowPtr, int **colInd, void **val, void **x)
 {
+    return mx_gen_config_family(config_id, seed, scale, gen_flags, -1.0, rows, cols, nnz, dtype, rowPtr, colInd, val, x);
+}
+
+extern "C" int mx_gen_config_family(int config_id, uint64_t seed, double scale, int gen_flags, double dense_share, int *rows, int *cols,
+                                    int *nnz, mx_dtype *dtype, int **rowPtr, int **colInd, void **val, void **x)
+{
     if (config_id < 1 || config_id > 5 || !(scale > 0.0 && scale <= 1.0) || !rows || !cols || !nnz || !dtype ||
-        !rowPtr || !colInd || !val || !x || (gen_flags & ~MX_GEN_UNALIGNED)) {
+        !rowPtr || !colInd || !val || !x || (gen_flags & ~MX_GEN_UNALIGNED) || dense_share > 1.0 ||
+        (dense_share >= 0.0 && config_id != 2 && config_id != 5)) {
         mx::set_error("mx_gen_config: bad argument (config 1..5, scale in (0,1])");
         return MX_ERR_ARG;
     }
@@ -270,7 +281,7 @@ extern "C" int mx_gen_config_ex(int config_id, uint64_t seed, double scale, int 
             break;
         case 2:
             n = std::max(64, (int)std::llround(65536.0 * scale) / 8 * 8);
-            gen_block_clustered(g, n, B, unaligned);
+            gen_block_clustered(g, n, B, unaligned, dense_share >= 0.0 ? dense_share : 0.4);
             break;
         case 3: {
             int g3 = std::max(3, (int)std::llround(100.0 * std::cbrt(scale)));
@@ -287,7 +298,7 @@ extern "C" int mx_gen_config_ex(int config_id, uint64_t seed, double scale, int 
         }
         case 5:
             n = std::max(256, (int)std::llround(4194304.0 * scale) / 128 * 128);
-            gen_mixed(g, n, B, unaligned);
+            gen_mixed(g, n, B, unaligned, dense_share >= 0.0 ? dense_share : 0.2);
             break;
         }
     } catch (const std::bad_alloc &) {

@@ -359,12 +359,16 @@ double mxp::tile_gate(mx_dtype)
 // Do the tiles pay for their launch?  (The reference gates its tile kernel on the size of the
 // matrix and its fill, test/test_autotc_spmv.cpp:1507,1518.)  What they take off the CSR part
 // saves es + 2 bytes per entry of its stream; what they cost is one more dependent launch and
-// their own stream.  Rates as measured on MI355X: the CSR part and the strip form of the tile
-// kernel move about 5000 bytes per ns (5 TB/s), the general tile kernel, bound by instruction
-// issue, about 2200; a further launch in the sequence costs about 5 us with its ramp and tail
-// (the strips of the mixed workload break even at about 15 M entries when launched apart);
-// strips usually ride in the launch of the combine kernel, where they came out ahead at every
-// size tried (1.7 M entries and up): they are charged little.
+// their own stream.  Rates as measured on MI355X: the CSR part and the binary16 strips move about
+// 5000 bytes per ns (5 TB/s), the general tile kernel, bound by instruction issue, about 2200; a
+// further launch in the sequence costs about 5 us with its ramp and tail.  The strips ride in the
+// launch of the combine kernel and are charged 3 us for it: over the family of the mixed workload
+// (5 to 40 % of the rows in strips, a quarter of the size and the full size, on and off the grid of
+// eight columns) that is where they stop paying -- 3.3 and 6.5 M entries at a quarter of the size lose
+// 0.3 to 1.3 us, 13 M there and everything from 7 M at full size wins.  The binary64 8 x 8 blocks
+// ride the same way but stream at the general kernel's rate: with 10, 25, 40 and 70 % of the
+// block-clustered workload's entries in blocks they never came out ahead of the CSR part (a tie at
+// 40 %, 17.6 against 12.7 us at 70 %), which is what this price says.
 // general*: the reference's fragments that pass the fill gate; strip*: the chunks of the plan's
 // own (binary16 strips, or binary64 8 x 8 blocks with `blocks64`).
 // 0 = nothing pays, 1 = only the plan's own chunks do, 2 = keep both.
@@ -376,10 +380,10 @@ int mxp::tiles_worth(mx_dtype dtype, int fragM, int fragK, bool blocks64, double
     const double blockBytes = (double)fragM * (blocks64 ? 8 : fragK) * es, slots = mx::tile_slots(dtype);
     const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
     const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
-    const double launchNs = 5000.0, stripLaunchNs = 1000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
+    const double launchNs = 5000.0, stripLaunchNs = 3000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
     const double savedNs = (generalEntries + stripEntries) * (es + 2) / fastRate;
     const double generalCost = generalFrags > 0 ? launchNs + generalBytes / generalRate : 0.0;
-    const double stripCost = stripBlocks > 0 ? stripLaunchNs + stripBytes / fastRate : 0.0;
+    const double stripCost = stripBlocks > 0 ? stripLaunchNs + stripBytes / (blocks64 ? generalRate : fastRate) : 0.0;
     if (netNs) *netNs = 0.0;
     if (savedNs <= generalCost + stripCost) return 0;
     if (generalFrags > 0 && generalEntries * (es + 2) / fastRate <= generalCost) {

@@ -175,6 +175,40 @@ def test_environment_is_read_when_a_plan_is_made_and_kept(mx, ora, monkeypatch):
     part.close()
 
 
+@pytest.mark.parametrize("cfg,scale,unaligned,share", [
+    (5, 0.25, False, 0.1), (5, 0.25, True, 0.2), (5, 0.25, False, 0.4), (2, 1.0, False, 0.7), (2, 0.25, True, 0.25)])
+def test_estimated_fractions_hold_off_the_matrices_they_were_calibrated_on(mx, cfg, scale, unaligned, share):
+    """mx_estimate_tau (counts only) against mx_tune_tau (every grid point timed) on members of the families
+    around workloads 2 and 5 with other shares of dense structure than the benchmark's, other sizes, and the
+    structure off the grid of eight columns: the default plan at the estimated fractions is at most 5 % slower
+    than at the timed best (both timed again the same way: median of three trains; the same fractions are the
+    same plan and need no timing).  The role of the reference's trained model (ML/bayes_opt.py:22-84 on the
+    features of ML/extract_features.cpp:31-95), which is not in this build."""
+    import torch
+    A, x = mx.gen_config(cfg, scale=scale, unaligned=unaligned, dense_share=share)
+    xd = torch.from_numpy(x).cuda()
+    ec, er, _ = mx.estimate_tau(A, 5)
+    tc, tr, _ = mx.tune_tau(A, 5, mx.MX_PLAN_DEFAULT, 50, 300)
+    print("family member: workload %d scale %g unaligned %s share %g: estimated (%g, %g), tuned (%g, %g)" % (
+        cfg, scale, unaligned, share, ec, er, tc, tr), flush=True)
+    if (ec, er) == (tc, tr):
+        return
+
+    def timed(tau):
+        part = mx.Partition(A, *tau)
+        plan = mx.Plan(part, mx.MX_PLAN_DEFAULT)
+        y = torch.zeros(A.rows, dtype=xd.dtype, device="cuda")
+        ts = sorted(plan.time(xd, y, 200, 1000, parts=False)[0] for _ in range(3))
+        tiles = plan.info["tile_nnz"]
+        plan.close()
+        part.close()
+        return ts[1], tiles
+    (te, tiles_e), (tt, tiles_t) = timed((ec, er)), timed((tc, tr))
+    if tiles_e == 0 and tiles_t == 0:
+        return      # both plans run everything through the CSR part: one plan under two names
+    assert te <= 1.05 * tt, (ec, er, te, tc, tr, tt)
+
+
 # ---------------------------------------------------------------- full benchmark sizes
 FULL = [
     # (workload, taus)
@@ -1112,10 +1146,11 @@ def test_tau_tuner(mx, ora):
 def test_tau_from_counts_alone(mx, ora):
     """mx_estimate_tau: the grid of mx_tune_tau walked without planning or timing anything -- per
     point the extraction on the device and the plan's own estimate of what its tiles save.  On the
-    mixed workload it names a point whose default plan keeps exactly the strip entries it counted
+    mixed workload (at a quarter of its size with twice its share of strips: at that size the benchmark's
+    own share does not pay) it names a point whose default plan keeps exactly the strip entries it counted
     and multiplies to the oracle's y; on the others, where no default plan keeps tiles, (0, 0)."""
     import torch
-    A, x = mx.gen_config(5, scale=1 / 4)
+    A, x = mx.gen_config(5, scale=1 / 4, dense_share=0.4)
     tc, tr, table = mx.estimate_tau(A, levels=3)
     assert [(c, r) for c, r, _, _ in table] == [(0.0, 0.0), (0.5, 0.0), (0.5, 0.5), (1.0, 0.0), (1.0, 0.5), (1.0, 1.0)]
     best = max(table, key=lambda t: t[2])
