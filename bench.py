@@ -139,13 +139,13 @@ def median_time(fn, reps=REPS):
     return float(np.median([fn() for _ in range(reps)]))
 
 
-def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=None, keep=None, unaligned=False, brief=False):
+def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=None, keep=None, unaligned=False, brief=False, scale=1.0):
     """mode: 'sweep' (the 5x5 grid), 'points' (CSR-only and two hybrid points) or 'csr' ((0,0) only).
     brief: no routes, no cold or rotating trains (the records of the unaligned variants)."""
     import numpy as np
     keep = mx.MX_PLAN_KEEP_TILES if keep is None else keep
     t0 = time.time()
-    A, x = mx.gen_config(cfg, unaligned=unaligned)
+    A, x = mx.gen_config(cfg, scale=scale, unaligned=unaligned)
     log("workload %d%s: rows=%d nnz=%d generated in %.1fs" % (cfg, " (off the grid)" if unaligned else "", A.rows, A.nnz, time.time() - t0))
     dev = torch.device("cuda:0")
     xd = torch.from_numpy(x).to(dev)
@@ -335,7 +335,8 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
     achieved = B / (basis_ms * 1e-3)
     traffic_total = tr_sum if (tr_all and krecs) else None
     roofline = {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": achieved / HBM_PEAK,
-                "frac_basis": ("warm: the plan's %.0f MB stay in the 256 MB memory-side cache between products" % (plan_bytes / 1e6)) if in_mall
+                "frac_basis": ("warm: the plan's %.0f MB stay in the 256 MB memory-side cache between products" % (plan_bytes / 1e6)) if plan_bytes <= MALL_BYTES
+                else ("warm: one plan back to back (no rotating train was run for this variant; its %.0f MB do not fit the memory-side cache)" % (plan_bytes / 1e6)) if rot is None
                 else ("rotating: the plan's %.0f MB do not fit the 256 MB memory-side cache, every product reads them from HBM" % (plan_bytes / 1e6)),
                 "frac_warm": B / (ev_total * 1e-3) / HBM_PEAK,
                 "frac_rotating": rot and rot["hbm_frac_whole_spmv"],
@@ -351,7 +352,8 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
                             "algorithmic bytes still count sizeof(valT) per entry, so frac can exceed 1; frac_traffic prices "
                             "the same time with the bytes the kernels really move" % info["csr_value_dict"])
     rec = {
-        "workload": WORKLOADS[cfg] + (", dense structure off the grid of eight columns" if unaligned else ""),
+        "workload": WORKLOADS[cfg] + (", dense structure off the grid of eight columns" if unaligned else "") +
+        ("" if scale == 1.0 else ", at %g of the benchmark's rows" % scale),
         "dtype": dtype, "rows": A.rows, "nnz": A.nnz,
         "tau_c": tau[0], "tau_r": tau[1], "plan": plan_kind, "plan_flags": "MX_PLAN_DEFAULT" if FLAGS == mx.MX_PLAN_DEFAULT else int(FLAGS),
         "csr_variant": ("rows", "slices", "split")[info["csr_variant"]], "csr_one_launch": bool(info["csr_fused"]),
@@ -434,6 +436,9 @@ def main():
     ap.add_argument("--no-unaligned", action="store_true", help="skip the variants of workloads 2 and 5 with structure off the grid")
     ap.add_argument("--all-tiles", action="store_true",
                     help="plans with MX_PLAN_ALL_TILES: every extracted chunk through the general MFMA tile kernel (profile runs)")
+    ap.add_argument("--scale", type=float, default=1.0,
+                    help="rows of the workloads as a fraction of the benchmark's (profile runs of plans that small matrices get, "
+                         "such as the one-launch form of the CSR part; the record says so and is no benchmark figure)")
     ap.add_argument("--tau-family", choices=("none", "quarter", "full"), default="quarter",
                     help="check mx_estimate_tau against mx_tune_tau over the families around workloads 2 and 5: at a quarter of "
                          "the benchmark's size (default, about half a minute), at a quarter and at full size, or not at all")
@@ -461,7 +466,7 @@ def main():
             return "csr"
         return "sweep" if cfg in SWEPT else "points"
     keep = mx.MX_PLAN_ALL_TILES if args.all_tiles else None
-    main_rec, (A, x) = run_workload(mx, torch, ora, cfgs[0], args.steps, args.warmup, mode_of(cfgs[0]), traffic, args.tau, keep)
+    main_rec, (A, x) = run_workload(mx, torch, ora, cfgs[0], args.steps, args.warmup, mode_of(cfgs[0]), traffic, args.tau, keep, scale=args.scale)
     out = {
         "metric": METRIC, "value": main_rec["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_rec["ms_per_step"],
@@ -511,15 +516,15 @@ def main():
         del src, dst
     others = {}
     for cfg in cfgs[1:]:
-        r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, mode_of(cfg), traffic, None, keep)
+        r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, mode_of(cfg), traffic, None, keep, scale=args.scale)
         others["workload_%d" % cfg] = r
     # the dense structure of workloads 2 and 5 off the grid of eight columns: CSR-only against the best hybrid
     if not args.no_sweep and args.tau is None and not args.no_unaligned:
         for cfg in cfgs:
             if cfg in SWEPT:
-                r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, "sweep", traffic, None, keep, unaligned=True, brief=True)
+                r, _ = run_workload(mx, torch, ora, cfg, args.steps, args.warmup, "sweep", traffic, None, keep, unaligned=True, brief=True, scale=args.scale)
                 others["workload_%d_unaligned" % cfg] = r
-    if args.tau_family != "none" and not args.no_sweep and args.tau is None and not args.all_tiles and args.workload is None:
+    if args.tau_family != "none" and not args.no_sweep and args.tau is None and not args.all_tiles and args.workload is None and args.scale == 1.0:
         out["tau_estimate_family"] = tau_family(mx, torch, (0.25,) if args.tau_family == "quarter" else (0.25, 1.0))
     if others:
         out["others"] = others

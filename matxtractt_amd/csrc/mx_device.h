@@ -162,6 +162,7 @@ constexpr int kSliceWaves = 8;        // waves per workgroup; one workgroup per 
 constexpr int kSliceThreads = 64 * kSliceWaves;
 inline int slice_cols(mx_dtype d) { return kSliceBytes / (d == MX_F64 ? 8 : 2); }
 constexpr int kSliceBatchEntries = 8;  // entries a lane loads at a time
+constexpr int kSliceChunkCost = 2;     // what ending a chunk costs a wave, in steps of its stream (for dealing chunks out evenly)
 inline int slice_step_entries(mx_dtype) { return 1; }  // entries a lane takes per step; chunks end between steps
 constexpr int kSliceLightSegs = 8;     // rows with at most this many virtual rows are summed by one lane
 

@@ -166,6 +166,7 @@ struct SliceWg {
     int slice = 0;
     std::vector<int> chunk[mx::kSliceWaves];
     int waveSteps[mx::kSliceWaves] = {};
+    int waveCost[mx::kSliceWaves] = {};  // steps plus what the chunk ends cost: what the dealing evens out
     long long steps = 0;  // stored steps (every wave's stream rounded up to whole batches)
     int chunks = 0;
 };
@@ -178,15 +179,18 @@ void deal_to_waves(SliceWg &w, int q, const std::vector<int> &mine, const std::v
     w.slice = q;
     w.steps = 0;
     for (int k = 0; k < W; ++k) {
-        w.waveSteps[k] = 0;
+        w.waveSteps[k] = w.waveCost[k] = 0;
         w.chunk[k].clear();
     }
+    // (a wave that ends a chunk stores 64 sums and starts over: measured, that costs it as much as about two
+    // steps of its stream, and thirty short chunks take a wave far longer than one long chunk of as many steps)
     for (int c : mine) {
         int best = 0;
         for (int k = 1; k < W; ++k)
-            if (w.waveSteps[k] < w.waveSteps[best]) best = k;
+            if (w.waveCost[k] < w.waveCost[best]) best = k;
         w.chunk[best].push_back(c);
         w.waveSteps[best] += ch[c].steps;
+        w.waveCost[best] += ch[c].steps + mx::kSliceChunkCost;
     }
     w.chunks = (int)mine.size();
     for (int k = 0; k < W; ++k) w.steps += (w.waveSteps[k] + SPB - 1) / SPB * SPB;
@@ -1110,7 +1114,7 @@ int mx::plan_slice_chunks(mx_dtype dtype, int budget, int S, const std::vector<s
     long long allSteps = 0;
     int busy = 0;
     for (int q = 0; q < S; ++q) {
-        for (const mx::SliceChunk &c : sliceChunks[q]) sliceSteps[q] += c.steps;
+        for (const mx::SliceChunk &c : sliceChunks[q]) sliceSteps[q] += c.steps + mx::kSliceChunkCost;
         allSteps += sliceSteps[q];
         busy += !sliceChunks[q].empty();
     }
@@ -1154,7 +1158,7 @@ int mx::plan_slice_chunks(mx_dtype dtype, int budget, int S, const std::vector<s
             Load top = heap.top();
             heap.pop();
             mine[top.second].push_back(c);
-            top.first += ch[c].steps;
+            top.first += ch[c].steps + mx::kSliceChunkCost;
             if ((int)mine[top.second].size() < mx::kSliceWgChunks) heap.push(top);
         }
         for (int g = 0; g < G; ++g) deal_to_waves(wgs[g0 + g], q, mine[g], ch, SPB);

@@ -162,18 +162,20 @@ bool mxp::plan_autotune()
 // Whether a plan asks for the one-launch form of the slices.  Never with MX_PLAN_NO_FUSE or
 // MX_CSR_FUSED=0, after a misplaced workgroup was reported, or for a matrix with a row of more than
 // eight virtual rows (mostVrows < 0: not counted, the layout will see).  Otherwise where it pays:
-// the workgroup that comes last to a group of rows adds that group up alone, and the slowest
+// the workgroup that comes last to a group of rows adds that group up alone, the sums it needs have
+// left the L2 by then (what a CU takes in from beyond it is 13 bytes a cycle), and the slowest
 // workgroup comes last to all of its groups, so the form wins while a workgroup's rows are few --
-// measured on the block-clustered workload at 256 workgroups: 9.5 against 11.3 us at 32 768 rows, a
-// tie at 49 152 and at 65 536 -- and is taken up to 160 rows per workgroup.  MX_PLAN_FUSE (or
-// MX_CSR_FUSED=1) takes it wherever the matrix suits it.
+// measured on the block-clustered workload at 256 workgroups, one launch against two: 9.3 against
+// 10.5 us at 32 768 rows, 10.5 against 11.2 at 40 960, 11.1 against 11.6 at 49 152, 12.9 against
+// 12.6 at 57 344, 13.8 against 13.2 at 65 536 -- and is taken up to 200 rows per workgroup.
+// MX_PLAN_FUSE (or MX_CSR_FUSED=1) takes it wherever the matrix suits it.
 bool mxp::fused_wanted(int flags, int rows, int mostVrows, int nCU)
 {
     const int env = mx::opt().csr_fused;
     if ((flags & MX_PLAN_NO_FUSE) || env == 0 || g_fused_off.load()) return false;
     if (mostVrows > mx::kSliceLightSegs || nCU % mx::kFusedXcds) return false;
     if ((flags & MX_PLAN_FUSE) || env == 1) return true;
-    return (long long)rows <= 160LL * nCU;
+    return (long long)rows <= 200LL * nCU;
 }
 
 CsrChoice mxp::choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int flags,
