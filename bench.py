@@ -139,7 +139,7 @@ def median_time(fn, reps=REPS):
     return float(np.median([fn() for _ in range(reps)]))
 
 
-def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=None, keep=None, unaligned=False, brief=False, scale=1.0):
+def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=None, keep=None, unaligned=False, brief=False, scale=1.0, timed_flags=None):
     """mode: 'sweep' (the 5x5 grid), 'points' (CSR-only and two hybrid points) or 'csr' ((0,0) only).
     brief: no routes, no cold or rotating trains (the records of the unaligned variants)."""
     import numpy as np
@@ -210,7 +210,7 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
 
     # ---- the plan of the best point as a caller with default flags gets it, from the matrix to the first y:
     # host route and device route
-    FLAGS = mx.MX_PLAN_DEFAULT if keep == mx.MX_PLAN_KEEP_TILES else keep
+    FLAGS = timed_flags if timed_flags is not None else mx.MX_PLAN_DEFAULT if keep == mx.MX_PLAN_KEEP_TILES else keep
 
     def first_y(device):
         torch.cuda.synchronize()
@@ -355,7 +355,7 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
         "workload": WORKLOADS[cfg] + (", dense structure off the grid of eight columns" if unaligned else "") +
         ("" if scale == 1.0 else ", at %g of the benchmark's rows" % scale),
         "dtype": dtype, "rows": A.rows, "nnz": A.nnz,
-        "tau_c": tau[0], "tau_r": tau[1], "plan": plan_kind, "plan_flags": "MX_PLAN_DEFAULT" if FLAGS == mx.MX_PLAN_DEFAULT else int(FLAGS),
+        "tau_c": tau[0], "tau_r": tau[1], "plan": plan_kind, "plan_flags": "MX_PLAN_DEFAULT" if FLAGS == mx.MX_PLAN_DEFAULT else "MX_PLAN_KEEP_TILES" if FLAGS == mx.MX_PLAN_KEEP_TILES else int(FLAGS),
         "csr_variant": ("rows", "slices", "split")[info["csr_variant"]], "csr_one_launch": bool(info["csr_fused"]),
         "tile_nnz": info["tile_nnz"], "csr_nnz": info["csr_nnz"],
         "ms_per_step": wall_ms, "ms_per_step_events": ev_total,
@@ -436,6 +436,9 @@ def main():
     ap.add_argument("--no-unaligned", action="store_true", help="skip the variants of workloads 2 and 5 with structure off the grid")
     ap.add_argument("--all-tiles", action="store_true",
                     help="plans with MX_PLAN_ALL_TILES: every extracted chunk through the general MFMA tile kernel (profile runs)")
+    ap.add_argument("--keep-tiles", action="store_true",
+                    help="time the plan with MX_PLAN_KEEP_TILES instead of the default flags (profile runs of a tile form on a "
+                         "matrix where a default plan drops it)")
     ap.add_argument("--scale", type=float, default=1.0,
                     help="rows of the workloads as a fraction of the benchmark's (profile runs of plans that small matrices get, "
                          "such as the one-launch form of the CSR part; the record says so and is no benchmark figure)")
@@ -466,7 +469,8 @@ def main():
             return "csr"
         return "sweep" if cfg in SWEPT else "points"
     keep = mx.MX_PLAN_ALL_TILES if args.all_tiles else None
-    main_rec, (A, x) = run_workload(mx, torch, ora, cfgs[0], args.steps, args.warmup, mode_of(cfgs[0]), traffic, args.tau, keep, scale=args.scale)
+    main_rec, (A, x) = run_workload(mx, torch, ora, cfgs[0], args.steps, args.warmup, mode_of(cfgs[0]), traffic, args.tau, keep, scale=args.scale,
+                                    timed_flags=mx.MX_PLAN_KEEP_TILES if args.keep_tiles else None)
     out = {
         "metric": METRIC, "value": main_rec["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_rec["ms_per_step"],
