@@ -175,6 +175,35 @@ def test_generator_shapes(mx):
     assert 0.12 <= 8 * len(strip) / A.rows <= 0.28
 
 
+def test_generator_families(mx):
+    """mx_gen_config_family: the share of dense structure of workloads 2 and 5 as a parameter.  The benchmark's own
+    share gives the benchmark's matrix; more share gives more dense structure, everything else as before; other
+    workloads take no share."""
+    for cfg, scale, default in ((2, 1 / 8, 0.4), (5, 1 / 64, 0.2)):
+        A, x = mx.gen_config(cfg, scale=scale)
+        B, xb = mx.gen_config(cfg, scale=scale, dense_share=default)
+        assert np.array_equal(A.rowPtr, B.rowPtr) and np.array_equal(A.colInd, B.colInd) and np.array_equal(A.val, B.val)
+        assert np.array_equal(x, xb)
+        dense = []
+        for share in (0.1, 0.4, 0.7) if cfg == 2 else (0.05, 0.2, 0.4):
+            F, _ = mx.gen_config(cfg, scale=scale, dense_share=share)
+            assert F.rows == A.rows and F.cols == A.cols
+            rowOf = np.repeat(np.arange(F.rows), np.diff(F.rowPtr))
+            assert np.all((np.diff(F.colInd) > 0) | (np.diff(rowOf) != 0))
+            brk = np.ones(F.nnz, bool)
+            brk[1:] = (np.diff(F.colInd) != 1) | (np.diff(rowOf) != 0)
+            runs = np.diff(np.append(np.nonzero(brk)[0], F.nnz))
+            dense.append(runs[runs >= 8].sum() / F.nnz)      # entries in runs of eight consecutive columns or more
+            if cfg == 2:
+                assert np.all(np.diff(F.rowPtr) == 64)
+                assert abs(dense[-1] - share) < 0.05, (share, dense[-1])
+        assert dense[0] < dense[1] < dense[2], dense
+    with pytest.raises(mx.MxError):
+        mx.gen_config(3, scale=1 / 64, dense_share=0.3)
+    with pytest.raises(mx.MxError):
+        mx.gen_config(2, scale=1 / 64, dense_share=1.5)
+
+
 def test_generators_with_structure_off_the_grid(mx, ora):
     """MX_GEN_UNALIGNED: the 8 x 8 blocks of workload 2 start at any column of their band and the strips of workload
     5 at a column that is not a multiple of eight; everything else about the matrices stays as it was (sizes, row
