@@ -367,7 +367,9 @@ double mxp::tile_gate(mx_dtype)
 // launch of the combine kernel and are charged 3 us for it: over the family of the mixed workload
 // (5 to 40 % of the rows in strips, a quarter of the size and the full size, on and off the grid of
 // eight columns) that is where they stop paying -- 3.3 and 6.5 M entries at a quarter of the size lose
-// 0.3 to 1.3 us, 13 M there and everything from 7 M at full size wins.  The binary64 8 x 8 blocks
+// 0.3 to 1.3 us, 13 M there and everything from 7 M at full size wins.  At a quarter of the size the
+// matrix stays in the memory-side cache and everything streams at 7 instead of 5 bytes per ns, which is
+// what decides the 13 M entries off the grid there (five blocks to a row instead of four: they lose).  The binary64 8 x 8 blocks
 // ride the same way but stream at the general kernel's rate: with 10, 25, 40 and 70 % of the
 // block-clustered workload's entries in blocks they never came out ahead of the CSR part (a tie at
 // 40 %, 17.6 against 12.7 us at 70 %), which is what this price says.
@@ -376,13 +378,16 @@ double mxp::tile_gate(mx_dtype)
 // 0 = nothing pays, 1 = only the plan's own chunks do, 2 = keep both.
 // `netNs` (optional): what the forms that are kept save per product by this estimate, in ns.
 int mxp::tiles_worth(mx_dtype dtype, int fragM, int fragK, bool blocks64, double generalEntries, double generalFrags,
-                     double stripEntries, double stripBlocks, double *netNs)
+                     double stripEntries, double stripBlocks, double allEntries, double *netNs)
 {
     const int es = mx::elem_size(dtype);
     const double blockBytes = (double)fragM * (blocks64 ? 8 : fragK) * es, slots = mx::tile_slots(dtype);
     const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
     const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
-    const double launchNs = 5000.0, stripLaunchNs = 3000.0, fastRate = 5000.0, generalRate = 2200.0;  // bytes per ns
+    // (a matrix whose entries stay in the memory-side cache between products streams faster, tiles or not:
+    // what the strips take off the CSR part is then worth less time, and so is what they stream themselves)
+    const bool resident = allEntries * (es + 2) <= 128e6;
+    const double launchNs = 5000.0, stripLaunchNs = 3000.0, fastRate = resident ? 7000.0 : 5000.0, generalRate = 2200.0;  // bytes per ns
     const double savedNs = (generalEntries + stripEntries) * (es + 2) / fastRate;
     const double generalCost = generalFrags > 0 ? launchNs + generalBytes / generalRate : 0.0;
     const double stripCost = stripBlocks > 0 ? stripLaunchNs + stripBytes / (blocks64 ? generalRate : fastRate) : 0.0;
@@ -664,7 +669,8 @@ int mxp::plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, Pha
             stripEntries += C.nnz;
             stripBlocks += (double)C.blocks.size();
         }
-        const int worth = tiles_worth(P->dtype, fragM, fragK, !inBlock.empty(), generalEntries, generalFrags, stripEntries, stripBlocks);
+        const int worth = tiles_worth(P->dtype, fragM, fragK, !inBlock.empty(), generalEntries, generalFrags, stripEntries, stripBlocks,
+                                      (double)P->nnz);
         if (worth == 0) {
             std::fill(sel.begin(), sel.end(), 0);
             stripChunks.clear();
