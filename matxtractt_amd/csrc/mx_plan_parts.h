@@ -19,11 +19,10 @@
     do {                                                                                              \
         hipError_t e_ = (call);                                                                       \
         if (e_ != hipSuccess) {                                                                       \
-            mx::set_error(std::string(#call) + ": " + hipGetErrorString(e_));                             \
+            mx::set_error(std::string(#call) + ": " + hipGetErrorString(e_));                         \
             return MX_ERR_DEVICE;                                                                     \
         }                                                                                             \
     } while (0)
-
 
 namespace mxp {
 
@@ -53,8 +52,7 @@ int slice_count(mx_dtype dtype, int rows, int cols, int nnz, int nCU);
 bool make_value_dict(int es, const void *val, int nnz, std::vector<unsigned char> &codes, std::vector<unsigned char> &dict,
                      int *nDict, int most = 256);
 
-// Re-lays the rows `sel` marks (all rows when null) of a CSR matrix for csr_slice_kernel (see
-// DeviceSlices).
+// The layout csr_slice_kernel runs on (see DeviceSlices), in host memory.
 struct HostSlices {
     int nWG = 0, S = 0, rows = 0, cols = 0, sliceCols = 0, maxWgChunks = 0, nnz = 0, vrows = 0, cap = 0;
     long long steps = 0, chunks = 0;
@@ -70,35 +68,31 @@ struct HostSlices {
     std::vector<int> wgGroups, groupNeed, fusedTarget;
     std::vector<unsigned char> rowVrows;
 };
+// Re-lays the rows `sel` marks (all rows when null) of a CSR matrix for csr_slice_kernel; `elsewhere` marks
+// rows that the tile forms write (1: alone, 2: together with the CSR part); `fused`: the one-launch form is
+// wanted (D.fused says whether the matrix got it).  upload_slices does the same and puts the layout on the
+// device -- built there when nothing asks for the host (a whole matrix, not fused, MX_LAYOUT unset).
 int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
                  const char *sel, HostSlices &D, const char *elsewhere = nullptr, bool fused = false);
 int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
                   const char *sel, mx::DeviceSlices &D, const char *elsewhere = nullptr,
                   std::pair<std::vector<int>, std::vector<int>> *segOut = nullptr, bool fused = false);
 
-// Puts tiles on the device for the tile kernels (see DeviceTiles): the fragments named by
-// `selFrag` (all when null), expanded to full blocks.  Column ids go through `colMap` and
-// output rows through `rowMap` when given.
 // One block of the tile kernels: fragM x fragK values, row-major, zeros included, and the column
 // of each of its fragK positions (-1 = unused).
 struct TileBlock {
     std::vector<unsigned char> vals;
     int cols[8];
 };
-// A chunk the plan forms itself for tile_dense_kernel: up to fragM rows (caller's numbering, -1 =
-// none) with one and the same set of columns -- whole runs of fragK from a multiple of fragK --
-// and that set as blocks.
+// A chunk the plan forms itself (binary16 strips, binary64 8 x 8 blocks): up to fragM rows (caller's
+// numbering, -1 = none) with one and the same set of blocks of eight consecutive columns, and those blocks.
 struct StripChunk {
     int rows[8];
     std::vector<TileBlock> blocks;
     int nnz;
 };
 
-// `rowTaken` (optional, per row of A_dd) marks rows whose entries the plan has put into strip
-// chunks: they are left out of the fragments here.  With `stripChunks` the canonical chunks are
-// not used at all: the given chunks are laid out, for tile_dense_kernel.
-// (The layout is made on the host alone -- build_tiles; `nCU` only sizes the waves -- and
-// upload_tiles puts it on the device.)
+// The layout the tile kernels run on (see DeviceTiles), in host memory.
 struct HostTiles {
     int chunkNum = 0, frags = 0, vals = 0, steps = 0, nWaves = 0;
     long long stored = 0;
@@ -106,6 +100,11 @@ struct HostTiles {
     std::vector<int> waveDesc, hdr, atox, valOffset;  // valOffset: first value of every step (the kernels get it from the headers)
     std::vector<unsigned char> val;
 };
+// The fragments named by `selFrag` (all when null), expanded to full blocks and grouped into steps.  Column ids
+// go through `colMap` and output rows through `rowMap` when given.  `rowTaken` (optional, per row of A_dd) marks
+// rows whose entries the plan has put into chunks of its own: they are left out of the fragments here.  With
+// `stripChunks` the canonical chunks are not used at all: the given chunks are laid out.  `nCU` only sizes the
+// waves.  upload_tiles does the same and puts the layout on the device.
 int build_tiles(mx_dtype dtype, int chunkNum, const char *selFrag, int dRows, const int *chunkPtr, const int *fragPtr,
                 const void *fragBit, const void *tcVal, const int *atox, const int *colMap, const int *rowMap, int nCU,
                 HostTiles &T, const char *rowTaken = nullptr, const std::vector<StripChunk> *stripChunks = nullptr);
@@ -129,7 +128,6 @@ inline int plan_opt_flags()
 }
 
 }  // namespace mxp
-
 
 struct mx_plan {
     mx_dtype dtype = MX_F64;
@@ -157,7 +155,6 @@ struct mx_plan {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 };
 
-
 namespace mxp {
 
 // Mean milliseconds per iteration of `body` over `iters` back-to-back runs after `warm`
@@ -182,7 +179,6 @@ int time_loop(mx_plan *plan, int warm, int iters, F body, double *ms)
     *ms = (double)t / (double)std::max(iters, 1);
     return MX_OK;
 }
-
 
 // ---- mx_plan.cpp: what a plan is decided from -----------------------------------------------------------
 // What the choice between the forms of the CSR part looks at: all of it is counted from the
