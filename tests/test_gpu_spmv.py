@@ -599,6 +599,32 @@ def test_slice_kernel_with_a_value_dictionary(mx, ora, dtype, monkeypatch):
     part.close()
 
 
+@pytest.mark.parametrize("dtype", [np.float64, np.float16])
+def test_slice_kernel_with_more_chunks_than_a_register_holds(mx, ora, dtype):
+    """A wave of the slice kernel keeps the ends of its next 64 chunks in a register and fetches the next 64
+    when those are used up: nine and a half million rows of one entry (some of three, some of none) in one
+    slice give every wave about seventy chunks of one to three steps.  y exact on integer data."""
+    import torch
+    rng = np.random.default_rng(5)
+    rows, cols = 9_500_000, 5000 if dtype == np.float16 else 3000
+    lens = np.ones(rows, np.int64)
+    lens[rng.integers(0, rows, rows // 50)] = 3
+    lens[rng.integers(0, rows, rows // 100)] = 0
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    A = mx.Csr(rows, cols, rp, rng.integers(0, cols, rp[-1]).astype(np.int32), rng.integers(-3, 4, rp[-1]).astype(dtype))
+    x = rng.integers(-2, 3, cols).astype(dtype)
+    ref = ora.spmv_f64(A.val.astype(np.float64), A.rowPtr, A.colInd, x.astype(np.float64))
+    P = mx.Partition(A, 0.0, 0.0)
+    plan = mx.Plan(P, mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_NO_FUSE)
+    assert plan.info["csr_variant"] == 1
+    waves = np.frombuffer(plan.arrays()["slices.waveDesc"], np.int32).reshape(-1, 4)
+    assert waves[:, 3].max() > 64, waves[:, 3].max()
+    y = plan.spmv(torch.from_numpy(x).cuda()).cpu().numpy().astype(np.float64)
+    assert np.array_equal(y, ref)
+    plan.close()
+    P.close()
+
+
 def test_slice_kernel_layouts(mx, ora):
     """The column-slice kernel on shapes that stress its layout: a ragged end of x (columns not a
     multiple of a 16-byte vector), one slice only, several slices of which one is empty, row
