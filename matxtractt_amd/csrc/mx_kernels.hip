@@ -1280,9 +1280,12 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
             const int4 d = r0 < rows ? ((const int4 *)rowInfo)[r0 >> 2] : int4{-2, -2, -2, -2};  // padded with -2
             dd[4 * q] = d.x, dd[4 * q + 1] = d.y, dd[4 * q + 2] = d.z, dd[4 * q + 3] = d.w;
         }
+        // (asked for whether the row has a sum or not: see the light rows below)
         AT sum[kCombineRows];
 #pragma unroll
-        for (int j = 0; j < kCombineRows; ++j) sum[j] = dd[j] >= 0 ? partial[dd[j]] : (AT)0;
+        for (int j = 0; j < kCombineRows; ++j) sum[j] = partial[max(dd[j], 0)];
+#pragma unroll
+        for (int j = 0; j < kCombineRows; ++j) sum[j] = dd[j] >= 0 ? sum[j] : (AT)0;
 #pragma unroll
         for (int j = 0; j < kCombineRows; ++j) {
             const int r = 4 * ((b * (kCombineRows / 4) + j / 4) * kBlock + tid) + j % 4;
@@ -1303,10 +1306,22 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
         const int4 none = {-1, -1, -1, -1};
         const int4 i0 = lightQuads == 1 ? lightIdx[i] : lightIdx[2 * i], i1 = lightQuads == 1 ? none : lightIdx[2 * i + 1];
         const int id[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
+        // (every sum is asked for whether the place is used or not -- an unused one names sum 0 and is not
+        // added: behind a conditional load the compiler waits before it issues the next, and a row's sums
+        // would arrive one trip after the other)
+        AT v[8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = partial[max(id[k], 0)];
+        if (lightQuads != 1) {
+#pragma unroll
+            for (int k = 4; k < 8; ++k) v[k] = partial[max(id[k], 0)];
+        } else {
+#pragma unroll
+            for (int k = 4; k < 8; ++k) v[k] = 0;
+        }
         AT sum = accumulate ? (AT)y[r] : (AT)0;
 #pragma unroll
-        for (int k = 0; k < 8; ++k)
-            if (id[k] >= 0) sum += partial[id[k]];
+        for (int k = 0; k < 8; ++k) sum += id[k] >= 0 ? v[k] : (AT)0;
         y[r] = (VT)sum;
         if (ywide) ywide[r] = sum;
         return;
@@ -1317,12 +1332,16 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
     const int4 h = live ? heavyInfo[g] : int4{0, 0, 0, 0};
     AT sum = 0;
     for (int k = sub; k < h.z; k += 64) {
+        // (four places of the row's list per lane and round, the row's last place again beyond its end, all
+        // of them asked for before the first is used)
         int id[4];
+        AT v[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) id[j] = k + 16 * j < h.z ? segIdx[h.y + k + 16 * j] : -1;
+        for (int j = 0; j < 4; ++j) id[j] = segIdx[h.y + min(k + 16 * j, h.z - 1)];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (id[j] >= 0) sum += partial[id[j]];
+        for (int j = 0; j < 4; ++j) v[j] = partial[id[j]];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sum += k + 16 * j < h.z ? v[j] : (AT)0;
     }
     sum = group_sum<16>(sum);
     if (live && sub == 0) {
