@@ -234,6 +234,7 @@ struct PartitionTwin {
 struct HybridCounts {
     long long generalFrags = 0, generalEntries = 0;  // fragments that pass the fill gate (after the strips took their rows)
     long long stripEntries = 0, stripBlocks = 0;     // binary16 strip chunks, or binary64 8 x 8 blocks (blocks64)
+    long long stripBlocksOff = 0;                    // of stripBlocks: blocks of chunks that start off the grid of eight columns
     bool blocks64 = false;
     int dRows = 0, dCols = 0, nnzRowD = 0, frags = 0;  // what the extraction selected; fragments of the tile encoding
     std::vector<int> stripChunkBlocks, stripChunkEntries;  // per strip chunk, in layout order

@@ -1048,13 +1048,15 @@ static int analyse_tail(HybridDevice::Impl &I, bool wantGeneral, bool wantStrips
                                    I.taken.as<unsigned char>(), I.memberChunk.as<int>(), I.chunkRows.as<int>(), I.chunkKey.as<int>(),
                                    I.chunkNb.as<int>(), I.chunkNnz.as<int>());
                 MXH_TRY(hipGetLastError());
-                std::vector<int> nb(nk), ne(nk);
+                std::vector<int> nb(nk), ne(nk), key(nk * 8);
                 MXH_TRY(hipMemcpyAsync(nb.data(), I.chunkNb.p, nk * 4, hipMemcpyDeviceToHost, s));
                 MXH_TRY(hipMemcpyAsync(ne.data(), I.chunkNnz.p, nk * 4, hipMemcpyDeviceToHost, s));
+                MXH_TRY(hipMemcpyAsync(key.data(), I.chunkKey.p, nk * 8 * 4, hipMemcpyDeviceToHost, s));
                 MXH_TRY(hipStreamSynchronize(s));
                 for (size_t k = 0; k < nk; ++k) {
                     counts->stripBlocks += nb[k];
                     counts->stripEntries += ne[k];
+                    if (key[k * 8] & 7) counts->stripBlocksOff += nb[k];  // (a chunk's blocks share their offset from the grid)
                 }
                 counts->stripChunkBlocks.swap(nb);
                 counts->stripChunkEntries.swap(ne);

@@ -369,7 +369,9 @@ double mxp::tile_gate(mx_dtype)
 // eight columns) that is where they stop paying -- 3.3 and 6.5 M entries at a quarter of the size lose
 // 0.3 to 1.3 us, 13 M there and everything from 7 M at full size wins.  At a quarter of the size the
 // matrix stays in the memory-side cache and everything streams at 7 instead of 5 bytes per ns, which is
-// what decides the 13 M entries off the grid there (five blocks to a row instead of four: they lose).  The binary64 8 x 8 blocks
+// what decides the 13 M entries off the grid there together with the price of their alignment (a block that
+// starts off the grid of eight columns is charged a quarter more: they win by 0.5 us on the grid and lose
+// about 1 us off it).  The binary64 8 x 8 blocks
 // ride the same way but stream at the general kernel's rate: with 10, 25, 40 and 70 % of the
 // block-clustered workload's entries in blocks they never came out ahead of the CSR part (a tie at
 // 40 %, 17.6 against 12.7 us at 70 %), which is what this price says.
@@ -378,12 +380,13 @@ double mxp::tile_gate(mx_dtype)
 // 0 = nothing pays, 1 = only the plan's own chunks do, 2 = keep both.
 // `netNs` (optional): what the forms that are kept save per product by this estimate, in ns.
 int mxp::tiles_worth(mx_dtype dtype, int fragM, int fragK, bool blocks64, double generalEntries, double generalFrags,
-                     double stripEntries, double stripBlocks, double allEntries, double *netNs)
+                     double stripEntries, double stripBlocks, double stripBlocksOff, double allEntries, double *netNs)
 {
     const int es = mx::elem_size(dtype);
     const double blockBytes = (double)fragM * (blocks64 ? 8 : fragK) * es, slots = mx::tile_slots(dtype);
     const double generalBytes = generalFrags * blockBytes + generalFrags / slots * (mx::kTileHdr * 4.0 + 256.0);
-    const double stripBytes = stripBlocks * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
+    // (a block that starts off the grid of eight columns reads x across 16-byte boundaries: measured, a quarter more)
+    const double stripBytes = (stripBlocks + 0.25 * stripBlocksOff) * blockBytes + stripBlocks / slots * (mx::kTileHdr * 4.0);
     // (a matrix whose entries stay in the memory-side cache between products streams faster, tiles or not:
     // what the strips take off the CSR part is then worth less time, and so is what they stream themselves)
     const bool resident = allEntries * (es + 2) <= 128e6;
@@ -650,7 +653,7 @@ int mxp::plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, Pha
     }
     // do the tiles pay for their launch (tiles_worth)?  MX_PLAN_KEEP_TILES skips the question.
     if (!(flags & (MX_PLAN_NO_TILES | MX_PLAN_ALL_TILES | MX_PLAN_KEEP_TILES))) {
-        double generalEntries = 0, generalFrags = 0, stripEntries = 0, stripBlocks = 0;
+        double generalEntries = 0, generalFrags = 0, stripEntries = 0, stripBlocks = 0, stripBlocksOff = 0;
         for (int w = 0; w < chunkNum; ++w) {
             uint64_t rowsLeft = ~0ull;
             if (!taken.empty())
@@ -668,9 +671,10 @@ int mxp::plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, Pha
         for (const StripChunk &C : stripChunks) {
             stripEntries += C.nnz;
             stripBlocks += (double)C.blocks.size();
+            if (!C.blocks.empty() && (C.blocks[0].cols[0] & 7)) stripBlocksOff += (double)C.blocks.size();
         }
         const int worth = tiles_worth(P->dtype, fragM, fragK, !inBlock.empty(), generalEntries, generalFrags, stripEntries, stripBlocks,
-                                      (double)P->nnz);
+                                      stripBlocksOff, (double)P->nnz);
         if (worth == 0) {
             std::fill(sel.begin(), sel.end(), 0);
             stripChunks.clear();

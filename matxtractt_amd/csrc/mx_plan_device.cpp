@@ -386,7 +386,7 @@ int mxp::create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const i
         if (noTiles) worth = 0;
         else if (!(flags & (MX_PLAN_KEEP_TILES | MX_PLAN_ALL_TILES)))
             worth = tiles_worth(dtype, fragM, fragK, cnt.blocks64, (double)cnt.generalEntries, (double)cnt.generalFrags,
-                                (double)cnt.stripEntries, (double)cnt.stripBlocks, (double)nnz);
+                                (double)cnt.stripEntries, (double)cnt.stripBlocks, (double)cnt.stripBlocksOff, (double)nnz);
         const bool keepBlocks = worth >= 1 && cnt.blocks64 && cnt.stripBlocks > 0;
         const bool keepStrips = worth >= 1 && !cnt.blocks64 && cnt.stripBlocks > 0;
         const bool keepGeneral = worth == 2 && cnt.generalFrags > 0;

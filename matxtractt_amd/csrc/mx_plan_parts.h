@@ -237,7 +237,7 @@ CsrChoice choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr,
 int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags, const char *stripRows = nullptr,
                    std::pair<std::vector<int>, std::vector<int>> *segOut = nullptr);
 int tiles_worth(mx_dtype dtype, int fragM, int fragK, bool blocks64, double generalEntries, double generalFrags, double stripEntries,
-                double stripBlocks, double allEntries, double *netNs = nullptr);
+                double stripBlocks, double stripBlocksOff, double allEntries, double *netNs = nullptr);
 int plan_host_parts(const mx_partition *P, int flags, HostPlanParts &H, PhaseLog &phase, bool noBlocks = false);
 
 // ---- mx_plan_device.cpp -------------------------------------------------------------------------------

@@ -170,7 +170,8 @@ extern "C" int mx_estimate_tau(const mx_csr *A, int levels, float *tau_c, float 
                     if (cnt.blocks64) cnt.generalFrags = cnt.generalEntries = 0;
                     double netNs = 0.0;
                     const int worth = tiles_worth(A->dtype, fragM, fragK, cnt.blocks64, (double)cnt.generalEntries, (double)cnt.generalFrags,
-                                                  (double)cnt.stripEntries, (double)cnt.stripBlocks, (double)A->nnz, &netNs);
+                                                  (double)cnt.stripEntries, (double)cnt.stripBlocks, (double)cnt.stripBlocksOff, (double)A->nnz,
+                                                  &netNs);
                     e.saved_us = netNs * 1e-3;
                     e.tile_entries = worth == 0 ? 0 : (worth == 2 ? cnt.generalEntries : 0) + cnt.stripEntries;
                 }
