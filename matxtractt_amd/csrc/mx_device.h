@@ -155,6 +155,8 @@ constexpr int kFusedGroupRows = 256;  // rows whose sums one arriver adds up at 
 constexpr int kFusedXcds = 8;         // L2 domains of the device the one-launch form is laid out for
 constexpr int kFusedWgChunks = 96;    // most chunks of a workgroup in that form (their targets, 256 bytes each, share the LDS with x)
 constexpr int kFusedWgGroups = 255;  // most groups a workgroup may hold sums of
+constexpr int kFusedFewGroups = 6;    // most groups to a workgroup for which the form is taken unasked (each costs the last
+                                      // workgroup of the launch about 0.3 us of adding)
 constexpr int kSliceBytes = 131072;   // the slice of x a workgroup keeps in LDS
 constexpr int kSliceLdsMax = 163840;  // LDS of a CU
 constexpr int kSliceWgChunks = 4096;  // most chunks a workgroup may have

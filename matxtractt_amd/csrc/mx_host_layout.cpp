@@ -443,7 +443,7 @@ static bool plan_fused(mx_dtype dtype, int budget, int S, int rows, int nGroups,
 // with more than eight virtual rows, more slices than workgroups in an XCD's rows, row subsets or
 // rows written elsewhere) the ordinary layout is made.
 int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
-                 const char *sel, HostSlices &D, const char *elsewhere, bool fused)
+                 const char *sel, HostSlices &D, const char *elsewhere, int fused)
 {
     const int es = mx::elem_size(dtype), E = mx::slice_step_entries(dtype);
     const int BE = mx::kSliceBatchEntries;
@@ -510,7 +510,10 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     mx::SlicePlan SP;
     const size_t perSlice = (size_t)(cap + 1) * 3;
     if (fused) {
-        fused = plan_fused(dtype, budget, S, rows, nGroups, cap, selPtr, segPtr, vr, sorted, sliceChunks, SP);
+        const bool suits = plan_fused(dtype, budget, S, rows, nGroups, cap, selPtr, segPtr, vr, sorted, sliceChunks, SP);
+        // the slowest workgroup adds the sums of every group it covers after its last chunk: with many groups
+        // to a workgroup that tail outweighs the launch saved, and the form is left unless it was asked for
+        fused = suits && (fused == 1 || SP.maxWgGroups <= mx::kFusedFewGroups) ? fused : 0;
         if (SP.nWG < 0) return MX_ERR_ARG;  // (the error is set)
         if (!fused) {  // the matrix does not suit the form: the ordinary layout, from a clean slate
             for (auto &v : sliceChunks) v.clear();
@@ -629,7 +632,7 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
         D.dict.swap(dictv);
         D.nDict = nDict;
     }
-    D.fused = fused;
+    D.fused = fused != 0;
     if (fused) {
         int most = 0;
         for (int r = 0; r < rows; ++r) most = std::max(most, D.segPtr[r + 1] - D.segPtr[r]);
@@ -660,7 +663,7 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
 // made on the host.
 int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
                   const char *sel, mx::DeviceSlices &D, const char *elsewhere,
-                  std::pair<std::vector<int>, std::vector<int>> *segOut, bool fused)
+                  std::pair<std::vector<int>, std::vector<int>> *segOut, int fused)
 {
     // The whole matrix: the layout is made on the device (the same arrays, in a fraction of the
     // time for a large matrix); MX_LAYOUT=host keeps the host route, which also serves row subsets.

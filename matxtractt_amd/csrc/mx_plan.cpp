@@ -167,15 +167,18 @@ bool mxp::plan_autotune()
 // workgroup comes last to all of its groups, so the form wins while a workgroup's rows are few --
 // measured on the block-clustered workload at 256 workgroups, one launch against two: 9.3 against
 // 10.5 us at 32 768 rows, 10.5 against 11.2 at 40 960, 11.1 against 11.6 at 49 152, 12.9 against
-// 12.6 at 57 344, 13.8 against 13.2 at 65 536 -- and is taken up to 200 rows per workgroup.
-// MX_PLAN_FUSE (or MX_CSR_FUSED=1) takes it wherever the matrix suits it.
-bool mxp::fused_wanted(int flags, int rows, int mostVrows, int nCU)
+// 12.6 at 57 344, 13.8 against 13.2 at 65 536 -- and is taken up to 200 rows per workgroup (return
+// value 2: and only where the layout, once made, has no workgroup with more than kFusedFewGroups
+// groups to add, which a matrix of few rows and many slices can have -- at the sizes above the
+// largest count was 3, 6, 6, 11 and 9).
+// MX_PLAN_FUSE (or MX_CSR_FUSED=1) takes it wherever the matrix suits it (return value 1).
+int mxp::fused_wanted(int flags, int rows, int mostVrows, int nCU)
 {
     const int env = mx::opt().csr_fused;
-    if ((flags & MX_PLAN_NO_FUSE) || env == 0 || g_fused_off.load()) return false;
-    if (mostVrows > mx::kSliceLightSegs || nCU % mx::kFusedXcds) return false;
-    if ((flags & MX_PLAN_FUSE) || env == 1) return true;
-    return (long long)rows <= 200LL * nCU;
+    if ((flags & MX_PLAN_NO_FUSE) || env == 0 || g_fused_off.load()) return 0;
+    if (mostVrows > mx::kSliceLightSegs || nCU % mx::kFusedXcds) return 0;
+    if ((flags & MX_PLAN_FUSE) || env == 1) return 1;
+    return (long long)rows <= 200LL * nCU ? 2 : 0;
 }
 
 CsrChoice mxp::choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int flags,
@@ -263,11 +266,11 @@ int mxp::setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const 
     };
     // the one-launch form of the slices, for a CSR part that is the whole product on a device whose
     // workgroups land where the layout assumes
-    bool wantFused = want[1] && fused_wanted(flags, rows, pick.mostVrows, nCU) && !stripRows;
+    int wantFused = want[1] && !stripRows ? fused_wanted(flags, rows, pick.mostVrows, nCU) : 0;
     if (wantFused) {
         int ok = 0;
         MX_HIP(mx::fused_placement_ok(nCU, &ok));
-        wantFused = ok != 0;
+        if (!ok) wantFused = 0;
     }
     auto build = [&](int v, mx::DeviceCsr &C, mx::DeviceSlices &L) -> int {
         if (v == 0) return upload_csr(plan->dtype, rows, cols, nnz, rowPtr, col, val, C, nullptr);

@@ -78,12 +78,12 @@ static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, 
         plan->csr_variant = 1;
         // The one-launch form where the host route would take it (no row with more than eight virtual rows: the
         // layout just made has no heavy rows).  Its layout is made on the host, from a copy of the part: the
-        // matrices it is taken for are small (160 rows per workgroup at most, unless it is forced).
-        bool wantFused = !elsewhere_dev && plan->slices.nHeavy == 0 && fused_wanted(flags, rows, -1, nCU);
+        // matrices it is taken for are small (200 rows per workgroup at most, unless it is forced).
+        int wantFused = !elsewhere_dev && plan->slices.nHeavy == 0 ? fused_wanted(flags, rows, -1, nCU) : 0;
         if (wantFused) {
             int ok = 0;
             MX_HIP(mx::fused_placement_ok(nCU, &ok));
-            wantFused = ok != 0;
+            if (!ok) wantFused = 0;
         }
         if (wantFused) {
             const size_t es = (size_t)mx::elem_size(dtype);
@@ -93,7 +93,7 @@ static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, 
             if (nnz) MX_HIP(hipMemcpy(ci.data(), colInd_dev, (size_t)nnz * 4, hipMemcpyDeviceToHost));
             if (nnz) MX_HIP(hipMemcpy(va.data(), val_dev, (size_t)nnz * es, hipMemcpyDeviceToHost));
             mx::DeviceSlices L;
-            rc = upload_slices(dtype, rows, cols, rp.data(), ci.data(), va.data(), nCU, S, nullptr, L, nullptr, segOut, true);
+            rc = upload_slices(dtype, rows, cols, rp.data(), ci.data(), va.data(), nCU, S, nullptr, L, nullptr, segOut, wantFused);
             if (rc) {
                 free_slices(L);
                 return rc;

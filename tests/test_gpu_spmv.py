@@ -1019,7 +1019,8 @@ def test_one_launch_form_of_the_slices(mx, ora):
     src/spmv_kernel/cdSpMV.cu:459): y equals the two-launch form's bit for bit and the oracle's within the
     bar, on binary64 and binary16, with four and with eight places per row, on rows without entries,
     on the plan made from device arrays, product after product (the counters clear themselves), with y
-    accumulated; a default plan takes the form only while a workgroup's rows are few; under stream capture
+    accumulated; a default plan takes the form only while a workgroup's rows, and the groups of rows under
+    it, are few; under stream capture
     the two launches are recorded."""
     import torch
     rng = np.random.default_rng(31)
@@ -1030,6 +1031,11 @@ def test_one_launch_form_of_the_slices(mx, ora):
     cases.append(("block-clustered, full size", A, x, False))
     A, x = mx.gen_config(3, scale=0.05)          # stencil, one byte per value
     cases.append(("stencil", A, x, None))
+    rows, cols = 16384, 32 * 16384                # few rows, 32 slices, a row in four of them: each of an XCD's 32
+    rp = (np.arange(rows + 1) * 24).astype(np.int32)   # workgroups has a slice to itself and would add all 8 groups of rows
+    ci = (rng.integers(0, 29, rows)[:, None] + rng.integers(0, 4, (rows, 24))) * 16384 + rng.integers(0, 16384, (rows, 24))
+    ci = np.sort(ci, axis=1).astype(np.int32).reshape(-1)
+    cases.append(("few rows, many slices", mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, rp[-1])), rng.uniform(-1, 1, cols), False))
     rows, cols = 20000, 3 * 65536 + 5             # binary16, rows in any order, stretches of empty rows
     lens = rng.integers(0, 40, rows)
     lens[3000:5200] = 0
