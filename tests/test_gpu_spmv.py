@@ -1890,3 +1890,90 @@ def test_device_route_on_random_small_matrices(mx):
                 D.close()
             part.close()
     assert compared >= 400, compared
+
+
+def _mixed_matrix(mx, rng, rows, cols, dt):
+    """Rows of power-law length around a centre column (some matrices with many rows empty), over them runs
+    of 128 rows holding 32 consecutive columns along the diagonal (on or off the grid of eight columns, full
+    or with holes) and/or 8x8 blocks anywhere; small integer values; every third matrix with its rows in any
+    order and columns named twice."""
+    L = np.minimum((1.5 * rng.random(rows) ** (-1 / 0.8)).astype(np.int64), min(cols, int(rng.choice([50, 600, 5000]))))
+    L[rng.random(rows) < rng.choice([0.0, 0.3])] = 0
+    r = np.repeat(np.arange(rows), L)
+    centre = rng.integers(0, cols, rows)
+    near = np.clip(centre[r] + rng.integers(-512, 513, r.size), 0, cols - 1)
+    R, C = [r], [np.where(rng.random(r.size) < 0.7, near, rng.integers(0, cols, r.size))]
+    kind = int(rng.integers(0, 4))
+    if kind in (1, 3) and cols > 128:
+        for r0 in range(0, rows - 128, 128):
+            if rng.random() < 0.25:
+                shift = int(rng.integers(0, 8)) if rng.random() < 0.5 else 0
+                rr = np.arange(r0, r0 + 128)
+                c0 = np.clip((rr // 8 * 8) % max(cols - 64, 1) + shift, 0, cols - 33)
+                keep = rng.random(128 * 32) < rng.choice([1.0, 0.93])
+                R.append(np.repeat(rr, 32)[keep])
+                C.append((c0[:, None] + np.arange(32)[None, :]).reshape(-1)[keep])
+    if kind in (2, 3) and cols > 128:
+        nb = rows // 8 * int(rng.integers(1, 4))
+        br = rng.integers(0, max(rows // 8, 1), nb) * 8
+        bc = rng.integers(0, max((cols - 8) // 8, 1), nb) * 8 + (int(rng.integers(0, 8)) if rng.random() < 0.3 else 0)
+        rr = (br[:, None, None] + np.arange(8)[None, :, None] + np.zeros((1, 1, 8), np.int64)).reshape(-1)
+        cc = (bc[:, None, None] + np.zeros((1, 8, 1), np.int64) + np.arange(8)[None, None, :]).reshape(-1)
+        ok = (rr < rows) & (cc < cols)
+        R.append(rr[ok])
+        C.append(cc[ok])
+    R, C = np.concatenate(R), np.concatenate(C)
+    V = rng.integers(-3, 4, R.size)
+    if rng.random() < 0.3:
+        order = np.lexsort((rng.random(R.size), R))
+    else:
+        order = np.lexsort((C, R))
+        first = np.ones(R.size, bool)
+        first[1:] = (R[order][1:] != R[order][:-1]) | (C[order][1:] != C[order][:-1])
+        order = order[first]
+    rp = np.zeros(rows + 1, np.int64)
+    np.add.at(rp, R[order] + 1, 1)
+    return mx.Csr(rows, cols, np.cumsum(rp).astype(np.int32), C[order].astype(np.int32), V[order].astype(dt))
+
+
+def test_mid_sized_matrices_of_mixed_structure_give_the_exact_product(mx, ora):
+    """Seeded matrices of a thousand to half a million rows with power-law rows, strips, blocks, empty rows
+    and repeated columns, integer values and x (every sum is an integer both precisions hold, so y must equal
+    the oracle's bit for bit whatever the order of the additions), at two pairs of fractions, under eight sets
+    of plan flags, for the plan made from the host partition and the one made from device arrays, into a
+    fresh y and over an old one."""
+    import torch
+    flag_sets = [mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_ALL_TILES, mx.MX_PLAN_NO_TILES | mx.MX_PLAN_CSR_ROWS,
+                 mx.MX_PLAN_NO_TILES | mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_FUSE, mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_SLICES,
+                 mx.MX_PLAN_NO_TILES | mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_NO_FUSE, mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_ROWS]
+    taus = [(0.25, 0.0), (0.5, 0.25), (0.75, 0.0), (0.75, 0.5), (1.0, 0.5)]
+    done = 0
+    for case in range(12):
+        rng = np.random.default_rng(7000 + case)
+        dt = np.float64 if case % 2 else np.float16
+        rows = int(rng.choice([1000, 20000, 70000, 200000, 500000]))
+        cols = int(rng.choice([300, 20000, 66000, 200000, 700000, 3000000]))
+        A = _mixed_matrix(mx, rng, rows, cols, dt)
+        if A.nnz == 0:
+            continue
+        x = rng.integers(-2, 3, cols).astype(dt)
+        want = oracle_y(ora, mx, A, x)
+        xd = torch.from_numpy(x).cuda()
+        d = [torch.from_numpy(a).cuda() for a in (A.rowPtr, A.colInd, A.val)]
+        for tc, tr in ((1.0, 1.0), taus[int(rng.integers(0, 5))]):
+            part = mx.Partition(A, tc, tr)
+            for fl in flag_sets:
+                for device in (False, True):
+                    print("case %d %s rows=%d cols=%d nnz=%d tau=(%g, %g) flags=%d device=%d" % (case, dt.__name__, rows, cols, A.nnz, tc, tr,
+                                                                                             fl, device), flush=True)
+                    P = mx.Plan.from_device(d[0], d[1], d[2], cols, tc, tr, fl) if device else mx.Plan(part, fl)
+                    y = P.spmv(xd)
+                    y2 = torch.full_like(y, 9)
+                    P.spmv(xd, y2)
+                    torch.cuda.synchronize()
+                    assert np.array_equal(y.cpu().numpy(), want), (case, tc, tr, fl, device, P.info)
+                    assert np.array_equal(y2.cpu().numpy(), want), (case, tc, tr, fl, device, P.info)
+                    P.close()
+                    done += 1
+            part.close()
+    assert done >= 300, done
