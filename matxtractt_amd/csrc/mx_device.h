@@ -143,7 +143,7 @@ struct DeviceSlices {
     // many count.  The arrays above stay valid for the two-launch form, which a plan falls back to.
     bool fused = false;
     int nGroups = 0, maxWgGroups = 0;
-    int placesPerRow = 0;             // 4 or 8: most virtual rows of a row
+    int placesPerRow = 0;             // most virtual rows of a row (1 .. 8)
     int *wgGroups = nullptr;          // [nWG][2] {first group, groups} whose counters the workgroup bumps
     int *groupNeed = nullptr;         // [nGroups] workgroups that bump the group's counter
     int *groupCount = nullptr;        // [nGroups] the counters; zero between launches (the last arriver clears its own)

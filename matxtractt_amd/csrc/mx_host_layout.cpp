@@ -636,7 +636,8 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     if (fused) {
         int most = 0;
         for (int r = 0; r < rows; ++r) most = std::max(most, D.segPtr[r + 1] - D.segPtr[r]);
-        const int places = most <= 4 ? 4 : mx::kSliceLightSegs;
+        // (as many places as the longest list of virtual rows has: the one who adds reads every place of a row)
+        const int places = std::max(most, 1);
         D.placesPerRow = places;
         D.nGroups = SP.nGroups;
         D.maxWgGroups = SP.maxWgGroups;

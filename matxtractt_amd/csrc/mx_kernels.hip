@@ -591,7 +591,8 @@ __device__ __forceinline__ T load_from_l2(const T *p)
 // A lane takes R rows at a time, one from each of R groups (2 groups side by side in a workgroup of
 // 512), and asks for everything it needs -- every place of every row, used or not: a place that no
 // virtual row owns holds the zero it was made with -- before it uses any of it: one trip for the lot,
-// and nothing is read that this launch did not write.  The 64 rows of a wave are consecutive, so every
+// and nothing is read that this launch did not write.  A row has fa.placesPerRow places, at most P
+// (what is read per group is places x 2 KB or 1 KB, and reading is what the adding costs).  The 64 rows of a wave are consecutive, so every
 // load is one contiguous stretch.  Sums in the order of the places, whoever adds: y does not depend on
 // who came last.
 template <typename VT, int P, int R>
@@ -604,6 +605,7 @@ __device__ __forceinline__ void fused_add(const FusedArgs &fa, const int *list, 
     VT *y = (VT *)fa.y;
     AT *ywide = (AT *)fa.ywide;
     const int half = __builtin_amdgcn_readfirstlane(tid / GR), rl = tid % GR;
+    const int places = fa.placesPerRow;
     for (int j0 = 0; j0 < nl; j0 += SIDE * R) {
         int row[R];
         AT v[R][P], old[R];
@@ -619,9 +621,10 @@ __device__ __forceinline__ void fused_add(const FusedArgs &fa, const int *list, 
             if (li < nl) {
                 const int g = list[li];
                 if (g * GR + rl < fa.rows) row[i] = g * GR + rl;
-                const AT *p = sums + (size_t)g * P * GR + rl;
+                const AT *p = sums + (size_t)g * places * GR + rl;
 #pragma unroll
-                for (int k = 0; k < P; ++k) v[i][k] = load_from_l2(p + (size_t)k * GR);
+                for (int k = 0; k < P; ++k)
+                    if (k < places) v[i][k] = load_from_l2(p + (size_t)k * GR);
                 if (fa.accumulate) old[i] = (AT)y[max(row[i], 0)];
             }
         }
@@ -836,7 +839,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         __syncthreads();
         const int nl = listL[0];
         if (nl == 0) return;
-        if (fa.placesPerRow == 8) fused_add<VT, 8, 4>(fa, listL + 1, nl, tid);
+        if (fa.placesPerRow > 4) fused_add<VT, 8, 4>(fa, listL + 1, nl, tid);
         else fused_add<VT, 4, 8>(fa, listL + 1, nl, tid);
     }
 }
@@ -1554,7 +1557,7 @@ static hipError_t launch_fused_t(const DeviceSlices &P, const void *x, void *y, 
     const size_t lds = (size_t)P.sliceCols * sizeof(VT) + (size_t)((ldsInts + 3) & ~3) * 4 + 64 + (dict ? 256 * sizeof(AT) : 0) +
                        (size_t)P.maxWgChunks * 256;
     if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16) || !P.fused || !P.wgGroups ||
-        !P.groupNeed || !P.groupCount || !P.fusedTarget || !P.fusedSums || !P.claim || !misplaced || (P.placesPerRow != 4 && P.placesPerRow != 8) ||
+        !P.groupNeed || !P.groupCount || !P.fusedTarget || !P.fusedSums || !P.claim || !misplaced || P.placesPerRow < 1 || P.placesPerRow > mx::kSliceLightSegs ||
         P.nWG <= 0 || P.nWG % mx::kFusedXcds)
         return hipErrorInvalidValue;
     mxk::FusedArgs fa;

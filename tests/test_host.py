@@ -586,7 +586,7 @@ def test_fused_slice_layout_walk(mx, case):
     # the sums as the one-launch kernel stores them: virtual row v at fusedTarget[v]; the k-th virtual row of
     # row r sits at ((r // GR) * P + k) * GR + r % GR, padding lanes at the spare places behind the last group
     nv = np.diff(segPtr)
-    assert nv.max() <= P and P in (4, 8) and np.array_equal(L["rowVrows"][:A.rows], nv) and np.all(L["rowVrows"][A.rows:] == 0)
+    assert nv.max() == P and 1 <= P <= 8 and np.array_equal(L["rowVrows"][:A.rows], nv) and np.all(L["rowVrows"][A.rows:] == 0)
     tgt = L["fusedTarget"]
     spare = L["nGroups"] * P * GR
     assert tgt.shape == (L["chunks"] * 64,)
