@@ -563,6 +563,7 @@ struct FusedArgs {
     unsigned *claim = nullptr;       // [workgroups] how often each logical workgroup's work has been taken
     unsigned seq = 0;                // launches of this layout before this one
     int rows = 0, placesPerRow = 4, accumulate = 0;
+    int ldsCount = 0;                // where in LDS the workgroup counts the groups that fall to it (bytes)
 };
 
 // The XCD this wave runs on (XCC_ID, bits 3:0 of hardware register 20).
@@ -727,6 +728,9 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 #pragma unroll
     for (int k = 0; k < NB; ++k) buf[k].load(ecol, estream, (size_t)min(batch0 + k, lastBatch), lane);
     endsL[max(min(tid, wgChunks - 1), 0)] = ce;
+    if constexpr (FUSED) {
+        if (tid == 0) *(int *)(smem + fa.ldsCount) = 0;  // (read after the stream, behind two barriers)
+    }
     if ((slice + 1) * sliceCols <= cols) {  // the whole slice lies inside x
 #pragma unroll
         for (int q = 0; q < CB; ++q) *(v4i32 *)(xs + (tid + q * kSliceThreads) * EPV) = xv[q];
@@ -819,28 +823,29 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     if constexpr (FUSED) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's sums are in the L2
         __syncthreads();                                    // ... and so are the other waves'
-        // (the chunk ends are done with) listL[0] = how many groups fall to this workgroup, then which
+        // (the chunk ends are done with: the groups that fall to this workgroup are listed in their place; how many,
+        // in a word of its own that was cleared before the stream began)
         int *listL = endsL;
-        if (tid == 0) listL[0] = 0;
-        __syncthreads();
-        // a lane per group, and one lane more: it takes the workgroup's claim in the same trip
-        if (tid == nGroupsMine) {
-            const unsigned claimed = __hip_atomic_fetch_add(fa.claim + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            if (claimed != fa.seq || xcc_id() >= mx::kFusedXcds)
-                __hip_atomic_store(fa.misplaced, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        } else if (tid < nGroupsMine) {
+        int *countL = (int *)(smem + fa.ldsCount);
+        // a lane per group, and one lane more for the workgroup's claim: one atomic each, all in one trip
+        if (tid <= nGroupsMine) {
+            const bool forClaim = tid == nGroupsMine;
             const int g = group0 + tid;
-            const int old = __hip_atomic_fetch_add(fa.groupCount + g, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            if (old + 1 == need) {
-                __hip_atomic_store(fa.groupCount + g, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                listL[1 + atomicAdd(&listL[0], 1)] = g;
+            unsigned *counter = forClaim ? fa.claim + b : (unsigned *)fa.groupCount + g;
+            const unsigned old = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (forClaim) {
+                if (old != fa.seq || xcc_id() >= mx::kFusedXcds)
+                    __hip_atomic_store(fa.misplaced, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            } else if ((int)old + 1 == need) {
+                __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                listL[atomicAdd(countL, 1)] = g;
             }
         }
         __syncthreads();
-        const int nl = listL[0];
+        const int nl = *countL;
         if (nl == 0) return;
-        if (fa.placesPerRow > 4) fused_add<VT, 8, 4>(fa, listL + 1, nl, tid);
-        else fused_add<VT, 4, 8>(fa, listL + 1, nl, tid);
+        if (fa.placesPerRow > 4) fused_add<VT, 8, 4>(fa, listL, nl, tid);
+        else fused_add<VT, 4, 8>(fa, listL, nl, tid);
     }
 }
 
@@ -1574,6 +1579,7 @@ static hipError_t launch_fused_t(const DeviceSlices &P, const void *x, void *y, 
     fa.rows = P.rows;
     fa.placesPerRow = P.placesPerRow;
     fa.accumulate = accumulate;
+    fa.ldsCount = (int)lds - 16;  // (in the 64 spare bytes at the end)
     if (dict)
         hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, true, true>), dim3(P.nWG), dim3(kSliceThreads), lds, s, (const int4 *)P.wgDesc,
                            (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.ecode, (const VT *)x, (AT *)P.partial, P.cols,
