@@ -155,8 +155,11 @@ constexpr int kFusedGroupRows = 256;  // rows whose sums one arriver adds up at 
 constexpr int kFusedXcds = 8;         // L2 domains of the device the one-launch form is laid out for
 constexpr int kFusedWgChunks = 96;    // most chunks of a workgroup in that form (their targets, 256 bytes each, share the LDS with x)
 constexpr int kFusedWgGroups = 255;  // most groups a workgroup may hold sums of
-constexpr int kFusedFewGroups = 6;    // most groups to a workgroup for which the form is taken unasked (each costs the last
-                                      // workgroup of the launch about 0.3 us of adding)
+constexpr int kFusedAddBytes = 100 * 1024;  // most bytes of sums under one workgroup (groups x places x a group's rows) for which
+                                            // the form is taken unasked: the slowest workgroup of a launch reads that much after its last
+                                            // chunk (about 70 ns per 2 KB), and beyond this a second launch is the faster way
+constexpr int kFusedSlicesMost = 8;          // ... and most slices: every XCD copies every slice of x in this form (a slice's workgroups are
+                                            // spread over all eight), 64 ns a slice more than when one XCD has a slice to itself
 constexpr int kSliceBytes = 131072;   // the slice of x a workgroup keeps in LDS
 constexpr int kSliceLdsMax = 163840;  // LDS of a CU
 constexpr int kSliceWgChunks = 4096;  // most chunks a workgroup may have

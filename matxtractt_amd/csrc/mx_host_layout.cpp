@@ -500,8 +500,8 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     }
     // the one-launch form needs every row's sums in at most eight places
     const int GR = mx::kFusedGroupRows, nGroups = (rows + GR - 1) / GR;
+    int most = 0;
     if (fused) {
-        int most = 0;
         for (int r = 0; r < rows; ++r) most = std::max(most, segPtr[r + 1] - segPtr[r]);
         if (sel || elsewhere || most > mx::kSliceLightSegs || (long long)nGroups * mx::kSliceLightSegs * GR > 2000000000LL) fused = false;
     }
@@ -511,9 +511,10 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
     const size_t perSlice = (size_t)(cap + 1) * 3;
     if (fused) {
         const bool suits = plan_fused(dtype, budget, S, rows, nGroups, cap, selPtr, segPtr, vr, sorted, sliceChunks, SP);
-        // the slowest workgroup adds the sums of every group it covers after its last chunk: with many groups
-        // to a workgroup that tail outweighs the launch saved, and the form is left unless it was asked for
-        fused = suits && (fused == 1 || SP.maxWgGroups <= mx::kFusedFewGroups) ? fused : 0;
+        // the slowest workgroup reads the sums of every group it covers after its last chunk: beyond kFusedAddBytes
+        // of them that tail outweighs the launch saved, and the form is left unless it was asked for
+        const long long addBytes = (long long)SP.maxWgGroups * std::max(most, 1) * GR * (dtype == MX_F64 ? 8 : 4);
+        fused = suits && (fused == 1 || addBytes <= mx::kFusedAddBytes) ? fused : 0;
         if (SP.nWG < 0) return MX_ERR_ARG;  // (the error is set)
         if (!fused) {  // the matrix does not suit the form: the ordinary layout, from a clean slate
             for (auto &v : sliceChunks) v.clear();

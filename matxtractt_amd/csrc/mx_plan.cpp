@@ -161,24 +161,29 @@ bool mxp::plan_autotune()
 }
 // Whether a plan asks for the one-launch form of the slices.  Never with MX_PLAN_NO_FUSE or
 // MX_CSR_FUSED=0, after a misplaced workgroup was reported, or for a matrix with a row of more than
-// eight virtual rows (mostVrows < 0: not counted, the layout will see).  Otherwise where it pays:
-// the workgroup that comes last to a group of rows adds that group up alone, the sums it needs have
-// left the L2 by then (what a CU takes in from beyond it is 13 bytes a cycle), and the slowest
-// workgroup comes last to all of its groups, so the form wins while a workgroup's rows are few --
-// measured on the block-clustered workload at 256 workgroups, one launch against two: 9.3 against
-// 10.5 us at 32 768 rows, 10.5 against 11.2 at 40 960, 11.1 against 11.6 at 49 152, 12.9 against
-// 12.6 at 57 344, 13.8 against 13.2 at 65 536 -- and is taken up to 200 rows per workgroup (return
-// value 2: and only where the layout, once made, has no workgroup with more than kFusedFewGroups
-// groups to add, which a matrix of few rows and many slices can have -- at the sizes above the
-// largest count was 3, 6, 6, 11 and 9).
-// MX_PLAN_FUSE (or MX_CSR_FUSED=1) takes it wherever the matrix suits it (return value 1).
-int mxp::fused_wanted(int flags, int rows, int mostVrows, int nCU)
+// eight virtual rows (mostVrows < 0: not counted, the layout will see).  MX_PLAN_FUSE (or
+// MX_CSR_FUSED=1) takes it wherever the matrix suits it (return value 1).  Otherwise where it pays
+// (return value 2): the workgroup that comes last to a group of rows adds that group up alone --
+// a round of atomics, then one of loads, 2 KB (1 KB in binary16) per place of the group's rows at
+// about 30 bytes a cycle, about 70 ns with the additions and the stores -- and the slowest
+// workgroup comes last to all of its groups.  Against that stands the second launch with its wait,
+// about 5 us.  Measured, one launch against two (us): block-clustered workload, 45 places under the
+// busiest workgroup, 12.5 / 13.1 (7.8 / 9.3 at half size); 400 000 rows of 8 entries in two
+// slices, 30 places, 13.9 / 15.6; 200 000 rows of 16 in four slices, 72 places, 15.7 / 14.6;
+// 130 000 rows of 32 in eight slices, 144 places, 20.9 / 17.3.  So the form is taken while the
+// busiest workgroup has at most kFusedAddBytes of sums under it, which only the layout knows
+// (build_slices); here the average stands in for it, so that no layout is made in vain for a
+// matrix that is far off.  And while the slices are few: the workgroups of a slice are spread over
+// all XCDs in this form, so each XCD fetches every slice of x (16 384 rows in 32 slices, 32 places:
+// 10.6 / 8.1).
+int mxp::fused_wanted(int flags, mx_dtype dtype, int rows, int S, int mostVrows, int nCU)
 {
     const int env = mx::opt().csr_fused;
     if ((flags & MX_PLAN_NO_FUSE) || env == 0 || g_fused_off.load()) return 0;
     if (mostVrows > mx::kSliceLightSegs || nCU % mx::kFusedXcds) return 0;
     if ((flags & MX_PLAN_FUSE) || env == 1) return 1;
-    return (long long)rows <= 200LL * nCU ? 2 : 0;
+    const double average = (double)rows * std::max(S, 1) * std::max(mostVrows, 1) * (dtype == MX_F64 ? 8 : 4) / std::max(nCU, 1);
+    return average <= (double)mx::kFusedAddBytes && S <= mx::kFusedSlicesMost ? 2 : 0;
 }
 
 CsrChoice mxp::choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int flags,
@@ -199,7 +204,7 @@ CsrChoice mxp::choose_csr_form(mx_dtype dtype, int rows, int cols, const int *ro
         c.mostVrows = st.mostVrows;
         // (the one-launch form of the slices, where the plan would take it: the device's placement is looked at
         // later, and a plan whose strips ride in the second launch keeps both launches)
-        if (mayFuse && fused_wanted(flags, rows, st.mostVrows, nCU)) c.usSlices -= kFusedSavesUs;
+        if (mayFuse && fused_wanted(flags, dtype, rows, S, st.mostVrows, nCU)) c.usSlices -= kFusedSavesUs;
         c.want[c.usSlices < c.usRows ? 0 : 1] = false;
     }
     return c;
@@ -266,7 +271,7 @@ int mxp::setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const 
     };
     // the one-launch form of the slices, for a CSR part that is the whole product on a device whose
     // workgroups land where the layout assumes
-    int wantFused = want[1] && !stripRows ? fused_wanted(flags, rows, pick.mostVrows, nCU) : 0;
+    int wantFused = want[1] && !stripRows ? fused_wanted(flags, plan->dtype, rows, S, pick.mostVrows, nCU) : 0;
     if (wantFused) {
         int ok = 0;
         MX_HIP(mx::fused_placement_ok(nCU, &ok));

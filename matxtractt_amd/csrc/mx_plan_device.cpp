@@ -71,15 +71,15 @@ static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, 
         st.fewValues = plan->slices.ecode != nullptr;
         if ((rc = mx::lines_per_gather_device(dtype, nnz, colInd_dev, nullptr, &st.linesPerGather))) return rc;
         csr_estimates(dtype, cols, nnz, st, &plan->est_rows_us, &plan->est_slices_us);
-        if (!elsewhere_dev && plan->slices.nHeavy == 0 && fused_wanted(flags, rows, -1, nCU)) plan->est_slices_us -= kFusedSavesUs;
+        if (!elsewhere_dev && plan->slices.nHeavy == 0 && fused_wanted(flags, dtype, rows, S, -1, nCU)) plan->est_slices_us -= kFusedSavesUs;
         want[plan->est_slices_us < plan->est_rows_us ? 0 : 1] = false;
     }
     if (want[1]) {
         plan->csr_variant = 1;
         // The one-launch form where the host route would take it (no row with more than eight virtual rows: the
         // layout just made has no heavy rows).  Its layout is made on the host, from a copy of the part: the
-        // matrices it is taken for are small (200 rows per workgroup at most, unless it is forced).
-        int wantFused = !elsewhere_dev && plan->slices.nHeavy == 0 ? fused_wanted(flags, rows, -1, nCU) : 0;
+        // matrices it is taken for have few sums per workgroup (fused_wanted), unless it is forced.
+        int wantFused = !elsewhere_dev && plan->slices.nHeavy == 0 ? fused_wanted(flags, dtype, rows, S, -1, nCU) : 0;
         if (wantFused) {
             int ok = 0;
             MX_HIP(mx::fused_placement_ok(nCU, &ok));

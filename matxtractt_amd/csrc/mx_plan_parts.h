@@ -70,8 +70,8 @@ struct HostSlices {
 };
 // Re-lays the rows `sel` marks (all rows when null) of a CSR matrix for csr_slice_kernel; `elsewhere` marks
 // rows that the tile forms write (1: alone, 2: together with the CSR part); `fused`: the one-launch form is
-// wanted -- 1: wherever the matrix suits it, 2: only where no workgroup covers more than kFusedFewGroups
-// groups of rows (D.fused says whether the matrix got it).  upload_slices does the same and puts the layout on the
+// wanted -- 1: wherever the matrix suits it, 2: only where no workgroup has more than kFusedAddBytes of
+// sums under it (D.fused says whether the matrix got it).  upload_slices does the same and puts the layout on the
 // device -- built there when nothing asks for the host (a whole matrix, not fused, MX_LAYOUT unset).
 int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
                  const char *sel, HostSlices &D, const char *elsewhere = nullptr, int fused = 0);
@@ -233,7 +233,7 @@ bool plan_autotune();
 double tile_gate(mx_dtype dtype);
 void csr_estimates(mx_dtype dtype, int cols, int nnz, const CsrStats &st, double *usRows, double *usSlices);
 // 0: not wanted; 1: asked for (flag or environment); 2: by the default rule (the `fused` of build_slices)
-int fused_wanted(int flags, int rows, int mostVrows, int nCU);
+int fused_wanted(int flags, mx_dtype dtype, int rows, int S, int mostVrows, int nCU);
 CsrChoice choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int flags, int nCU,
                           int S, bool mayFuse = false);
 int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags, const char *stripRows = nullptr,

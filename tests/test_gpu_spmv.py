@@ -1019,23 +1019,27 @@ def test_one_launch_form_of_the_slices(mx, ora):
     src/spmv_kernel/cdSpMV.cu:459): y equals the two-launch form's bit for bit and the oracle's within the
     bar, on binary64 and binary16, with four and with eight places per row, on rows without entries,
     on the plan made from device arrays, product after product (the counters clear themselves), with y
-    accumulated; a default plan takes the form only while a workgroup's rows, and the groups of rows under
-    it, are few; under stream capture
+    accumulated; a default plan takes the form only while the sums under a workgroup, and the slices, are
+    few; under stream capture
     the two launches are recorded."""
     import torch
     rng = np.random.default_rng(31)
     cases = []
     A, x = mx.gen_config(2, scale=0.5)           # 32 768 rows: the default plan takes the form
     cases.append(("block-clustered, half size", A, x, True))
-    A, x = mx.gen_config(2, scale=1.0)           # 65 536 rows: only when asked
-    cases.append(("block-clustered, full size", A, x, False))
+    A, x = mx.gen_config(2, scale=1.0)           # 65 536 rows, 90 KB of sums under the busiest workgroup: still taken
+    cases.append(("block-clustered, full size", A, x, True))
     A, x = mx.gen_config(3, scale=0.05)          # stencil, one byte per value
     cases.append(("stencil", A, x, None))
-    rows, cols = 16384, 32 * 16384                # few rows, 32 slices, a row in four of them: each of an XCD's 32
-    rp = (np.arange(rows + 1) * 24).astype(np.int32)   # workgroups has a slice to itself and would add all 8 groups of rows
+    rows, cols = 16384, 32 * 16384                # 32 slices, a row in four of them: every XCD would fetch all of x,
+    rp = (np.arange(rows + 1) * 24).astype(np.int32)   # so the form is taken only when asked for
     ci = (rng.integers(0, 29, rows)[:, None] + rng.integers(0, 4, (rows, 24))) * 16384 + rng.integers(0, 16384, (rows, 24))
     ci = np.sort(ci, axis=1).astype(np.int32).reshape(-1)
     cases.append(("few rows, many slices", mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, rp[-1])), rng.uniform(-1, 1, cols), False))
+    rows, cols = 200000, 60000                    # four slices, 144 KB of sums under the busiest workgroup: only when asked
+    rp = (np.arange(rows + 1) * 16).astype(np.int32)
+    ci = np.sort(rng.integers(0, cols, (rows, 16)), axis=1).astype(np.int32).reshape(-1)
+    cases.append(("many sums under a workgroup", mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, rp[-1])), rng.uniform(-1, 1, cols), False))
     rows, cols = 20000, 3 * 65536 + 5             # binary16, rows in any order, stretches of empty rows
     lens = rng.integers(0, 40, rows)
     lens[3000:5200] = 0
