@@ -261,7 +261,7 @@ double mx_algorithmic_bytes(mx_dtype dtype, int rows, int cols, int nnz);
 #define MX_PLAN_NO_FUSE 32   /* CSR part in slice form: always two launches (csr_slice_kernel, then slice_combine_kernel).
                                  Without this flag a plan whose CSR part is the whole product takes the one-launch
                                  form (mx_plan_info.csr_fused) where the matrix suits it -- no row with more than eight
-                                 virtual rows, at most 200 rows per workgroup and six groups of 256 rows under any one workgroup
+                                 virtual rows, at most 100 KB of sums under the busiest workgroup and at most eight slices of x
                                  (beyond that two launches are as fast or faster) -- and
                                  the device deals its workgroups round-robin to eight XCDs, which plan creation checks */
 #define MX_PLAN_FUSE 64      /* the one-launch form wherever the matrix suits it, whatever its size */
