@@ -721,6 +721,15 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
         const int gi = slice * (sliceCols / EPV) + tid + q * kSliceThreads;
         xv[q] = ((const v4i32 *)x)[min(gi, lastVec)];
     }
+    // (one-launch form: where the sums of the workgroup's first chunks go -- asked for before the ring, so that
+    // putting them into LDS waits for them and for x, and not for the ring behind them)
+    constexpr int TR = FUSED ? 4 : 1;
+    int tg[TR];
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int q = 0; q < TR; ++q)
+            tg[q] = fa.target[(size_t)wgChunk0 * 64 + max(min(tid + q * kSliceThreads, wgChunks * 64 - 1), 0)];
+    }
     // the ring: the first batches of the wave's stream (the last one again and again when the
     // stream is shorter than the ring)
     Batch buf[NB];
@@ -730,6 +739,9 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     endsL[max(min(tid, wgChunks - 1), 0)] = ce;
     if constexpr (FUSED) {
         if (tid == 0) *(int *)(smem + fa.ldsCount) = 0;  // (read after the stream, behind two barriers)
+#pragma unroll
+        for (int q = 0; q < TR; ++q)
+            if (tid + q * kSliceThreads < wgChunks * 64) targetL[tid + q * kSliceThreads] = tg[q];
     }
     if ((slice + 1) * sliceCols <= cols) {  // the whole slice lies inside x
 #pragma unroll
@@ -750,7 +762,8 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     }
     for (int i = kSliceThreads + tid; i < wgChunks; i += kSliceThreads) endsL[i] = chunkEnd[wgChunk0 + i];
     if constexpr (FUSED) {
-        for (int i = tid; i < wgChunks * 64; i += kSliceThreads) targetL[i] = fa.target[(size_t)wgChunk0 * 64 + i];
+        // (a workgroup with more than 32 chunks: the rest, behind the ring)
+        for (int i = TR * kSliceThreads + tid; i < wgChunks * 64; i += kSliceThreads) targetL[i] = fa.target[(size_t)wgChunk0 * 64 + i];
     }
     __syncthreads();
     // (the chunk ends are the same for all lanes of the wave: kept in scalar registers)

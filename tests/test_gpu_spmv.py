@@ -1047,6 +1047,11 @@ def test_one_launch_form_of_the_slices(mx, ora):
     ci = rng.integers(0, cols, rp[-1]).astype(np.int32)
     cases.append(("binary16", mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, rp[-1]).astype(np.float16)),
                   rng.uniform(-1, 1, cols).astype(np.float16), None))
+    rows, cols = 600000, 60000                    # binary16, one slice, one place per row, 37 chunks per workgroup (the
+    rp = (np.arange(rows + 1) * 6).astype(np.int32)    # places of the first 32 are asked for ahead of the rest): taken
+    ci = np.sort(rng.integers(0, cols, (rows, 6)), axis=1).astype(np.int32).reshape(-1)
+    cases.append(("many chunks per workgroup", mx.Csr(rows, cols, rp, ci, rng.uniform(-1, 1, rp[-1]).astype(np.float16)),
+                  rng.uniform(-1, 1, cols).astype(np.float16), True))
     for name, A, x, default_takes_it in cases:
         print("one-launch form:", name, A.rows, A.nnz, flush=True)
         ref = oracle_y(ora, mx, A, x)
