@@ -126,6 +126,7 @@ struct DeviceSlices {
     int lightQuads = 2;               // 1 when no light row has more than four virtual rows
     int *heavyInfo = nullptr;         // [nHeavy][4]
     int nLight = 0, nHeavy = 0;
+    int mostVrows = 0;                // most virtual rows of any row
     // The one-launch form (csr_slice_kernel<.., FUSED>), when the layout was made for it: the rows are cut
     // into groups of kFusedGroupRows, the groups into one contiguous range per XCD, and the virtual rows
     // of a slice are ordered by group before length, so that a workgroup's chunks cover a contiguous run
@@ -200,14 +201,27 @@ struct SlicePlan {
     std::vector<int> wgGroups, groupNeed;
 };
 int plan_slice_chunks(mx_dtype dtype, int budget, int S, const std::vector<std::vector<SliceChunk>> &sliceChunks, SlicePlan &P);
+// The plan of the one-launch form from the records of the virtual rows (in the order of the rows, ascending
+// columns inside a row: the numbering both layout routes use): `sorted` receives the order in which the
+// virtual rows are laid out and P the workgroups, waves, chunks and groups.  `mode` 1: wherever the matrix
+// suits the form; 2: only while the busiest workgroup has at most kFusedAddBytes of sums under it.  Returns 1
+// when the form is taken (*places = places per row), 0 when it is not (nothing filled), a negative error code
+// when the plan cannot be made (the error is set).
+int plan_fused_records(mx_dtype dtype, int budget, int S, int rows, int cap, const int *rowPtr, const int *segPtr, const int *vSlice,
+                       const int *vLen, int nV, int mode, std::vector<int> &sorted, SlicePlan &P, int *places);
+// Where the virtual rows of the one-launch form put their sums (DeviceSlices::fusedTarget), from the places the
+// layout gave them.
+void fused_targets(int rows, int nGroups, int places, long long totalChunks, const int *segPtr, const int *segIdx, std::vector<int> &target);
 constexpr int kSlicePadSteps = 16;  // spare zero steps after the last of the streams
 // The slice layout built on the device from a CSR matrix in device memory (mx_layout.hip): the
 // arrays of `D` equal those of the host route byte for byte.  `elsewhere_dev`: optional marks per
 // row (device memory) as in the host route.  segPtrOut / segIdxOut (optional): host copies of the
-// virtual rows of every row.
+// virtual rows of every row.  `fused` (1 or 2, as in plan_fused_records): the one-launch form where the matrix
+// suits it (D.fused says whether it did) -- the records of the virtual rows come down, the plan goes up, the
+// entries never leave the device.
 int build_slices_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, const void *val_dev,
                         int nCU, int S, const char *elsewhere_dev, DeviceSlices &D, hipStream_t s, std::vector<int> *segPtrOut = nullptr,
-                        std::vector<int> *segIdxOut = nullptr);
+                        std::vector<int> *segIdxOut = nullptr, int fused = 0);
 
 // For plans made from a matrix that lives in device memory: the caller's arrays looked at before
 // they are used as addresses; the mean number of distinct lines of x per wave-wide gather (sampled

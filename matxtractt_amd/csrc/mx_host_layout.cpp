@@ -434,6 +434,52 @@ static bool plan_fused(mx_dtype dtype, int budget, int S, int rows, int nGroups,
     return true;
 }
 
+}  // namespace mxp
+
+int mx::plan_fused_records(mx_dtype dtype, int budget, int S, int rows, int cap, const int *rowPtr, const int *segPtrIn, const int *vSlice,
+                           const int *vLen, int nV, int mode, std::vector<int> &sorted, SlicePlan &SP, int *places)
+{
+    const int GR = mx::kFusedGroupRows, nGroups = (rows + GR - 1) / GR;
+    int most = 0;
+    for (int r = 0; r < rows; ++r) most = std::max(most, segPtrIn[r + 1] - segPtrIn[r]);
+    // the form needs every row's sums in at most eight places
+    if (most > mx::kSliceLightSegs || (long long)nGroups * mx::kSliceLightSegs * GR > 2000000000LL) return 0;
+    std::vector<mxp::VRow> vr((size_t)nV);
+    for (int t = 0; t < nV; ++t) vr[t] = {0, vLen[t], vSlice[t], 0};
+    const std::vector<int> rowStart(rowPtr, rowPtr + rows + 1), segPtr(segPtrIn, segPtrIn + rows + 1);
+    std::vector<std::vector<mx::SliceChunk>> sliceChunks((size_t)S);
+    sorted.assign((size_t)nV, 0);
+    SP = mx::SlicePlan();
+    const bool suits = mxp::plan_fused(dtype, budget, S, rows, nGroups, cap, rowStart, segPtr, vr, sorted, sliceChunks, SP);
+    if (SP.nWG < 0) return MX_ERR_ARG;  // (the error is set)
+    // the slowest workgroup reads the sums of every group it covers after its last chunk: beyond kFusedAddBytes
+    // of them that tail outweighs the launch saved, and the form is left unless it was asked for
+    const long long addBytes = (long long)SP.maxWgGroups * std::max(most, 1) * GR * (dtype == MX_F64 ? 8 : 4);
+    if (!suits || (mode != 1 && addBytes > mx::kFusedAddBytes)) {
+        SP = mx::SlicePlan();
+        sorted.clear();
+        return 0;
+    }
+    // (as many places as the longest list of virtual rows has: the one who adds reads every place of a row)
+    *places = std::max(most, 1);
+    return 1;
+}
+
+void mx::fused_targets(int rows, int nGroups, int places, long long totalChunks, const int *segPtr, const int *segIdx, std::vector<int> &target)
+{
+    // the k-th virtual row of row r at ((r / GR) * places + k) * GR + r % GR; the padding lanes of a chunk at the
+    // spare places behind the last group
+    const int GR = mx::kFusedGroupRows;
+    const size_t spare = (size_t)nGroups * places * GR;
+    target.assign((size_t)totalChunks * 64, 0);
+    for (size_t v = 0; v < target.size(); ++v) target[v] = (int)(spare + (v & 63));
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; ++r)
+        for (int t = segPtr[r]; t < segPtr[r + 1]; ++t) target[segIdx[t]] = (int)(((size_t)(r / GR) * places + (t - segPtr[r])) * GR + r % GR);
+}
+
+namespace mxp {
+
 // `elsewhere` (optional) marks rows whose result another kernel writes: 1 = the strips of a binary16
 // plan (the row has nothing here), 2 = the 8 x 8 blocks of a binary64 plan, whose waves fetch the sums
 // of the row's virtual rows themselves.  Such rows get rowInfo -2 and appear in no list, so that the
@@ -644,32 +690,22 @@ int build_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const in
         D.maxWgGroups = SP.maxWgGroups;
         D.wgGroups.swap(SP.wgGroups);
         D.groupNeed.swap(SP.groupNeed);
-        // where every virtual row puts its sum: the k-th of row r at ((r / GR) * places + k) * GR + r % GR; the
-        // padding lanes of a chunk at the spare places behind the last group
-        const size_t spare = (size_t)nGroups * places * GR;
-        D.fusedTarget.assign((size_t)totalChunks * 64, 0);
-        for (size_t v = 0; v < D.fusedTarget.size(); ++v) D.fusedTarget[v] = (int)(spare + (v & 63));
+        mx::fused_targets(rows, nGroups, places, totalChunks, D.segPtr.data(), D.segIdx.data(), D.fusedTarget);
         D.rowVrows.assign((size_t)nGroups * GR, 0);
-#pragma omp parallel for schedule(static)
-        for (int r = 0; r < rows; ++r) {
-            D.rowVrows[r] = (unsigned char)(D.segPtr[r + 1] - D.segPtr[r]);
-            for (int t = D.segPtr[r]; t < D.segPtr[r + 1]; ++t)
-                D.fusedTarget[D.segIdx[t]] = (int)(((size_t)(r / GR) * places + (t - D.segPtr[r])) * GR + r % GR);
-        }
+        for (int r = 0; r < rows; ++r) D.rowVrows[r] = (unsigned char)(D.segPtr[r + 1] - D.segPtr[r]);
     }
     return MX_OK;
 }
 
 // `segOut` (optional): receives segPtr and segIdx (the virtual rows of every matrix row).
-// `fused`: the layout of the one-launch form where the matrix suits it (D.fused says whether it did);
-// made on the host.
+// `fused`: the layout of the one-launch form where the matrix suits it (D.fused says whether it did).
 int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int nCU, int S,
                   const char *sel, mx::DeviceSlices &D, const char *elsewhere,
                   std::pair<std::vector<int>, std::vector<int>> *segOut, int fused)
 {
     // The whole matrix: the layout is made on the device (the same arrays, in a fraction of the
     // time for a large matrix); MX_LAYOUT=host keeps the host route, which also serves row subsets.
-    if (!sel && !fused && !mx::opt().layout_host) {
+    if (!sel && !mx::opt().layout_host) {
         const size_t es = (size_t)mx::elem_size(dtype);
         const int nnz = rowPtr[rows];
         int *dRowPtr = nullptr, *dCol = nullptr;
@@ -680,7 +716,7 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
         if (!rc && elsewhere) rc = upload_bytes(&dElse, elsewhere, (size_t)rows);
         if (!rc)
             rc = mx::build_slices_device(dtype, rows, cols, nnz, dRowPtr, dCol, dVal, nCU, S, (const char *)dElse, D, nullptr,
-                                         segOut ? &segOut->first : nullptr, segOut ? &segOut->second : nullptr);
+                                         segOut ? &segOut->first : nullptr, segOut ? &segOut->second : nullptr, fused);
         (void)hipFree(dRowPtr);
         (void)hipFree(dCol);
         (void)hipFree(dVal);
@@ -708,6 +744,7 @@ int upload_slices(mx_dtype dtype, int rows, int cols, const int *rowPtr, const i
     D.subset = H.subset;
     D.nLight = (int)H.lightInfo.size() / 4;
     D.nHeavy = (int)H.heavyInfo.size() / 4;
+    for (int r = 0; r < rows; ++r) D.mostVrows = std::max(D.mostVrows, H.segPtr[r + 1] - H.segPtr[r]);
     if ((rc = upload(&D.wgDesc, H.wgDesc.data(), H.wgDesc.size()))) return rc;
     if ((rc = upload(&D.waveDesc, H.waveDesc.data(), H.waveDesc.size()))) return rc;
     if ((rc = upload(&D.chunkEnd, H.chunkEnd.data(), H.chunkEnd.size()))) return rc;

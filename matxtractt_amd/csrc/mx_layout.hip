@@ -229,22 +229,27 @@ __global__ __launch_bounds__(kBlock) void pad_columns_kernel(const int *__restri
 __global__ __launch_bounds__(kBlock) void row_info_kernel(const int *__restrict__ segPtr, const int *__restrict__ segIdx,
                                                           const char *__restrict__ elsewhere, int rows, int lightSegs,
                                                           int *__restrict__ rowInfo, int *__restrict__ isLight, int *__restrict__ isHeavy,
-                                                          int *__restrict__ over4)
+                                                          int *__restrict__ over4, int *__restrict__ most)
 {
     const int r = blockIdx.x * kBlock + threadIdx.x;
-    if (r > rows) return;
-    if (r == rows) {  // the scans run over rows + 1 elements
+    int n = 0;
+    if (r < rows) {
+        const int a = segPtr[r];
+        n = segPtr[r + 1] - a;
+        const int e = elsewhere ? elsewhere[r] : 0;
+        const bool fetched = e == 2;
+        rowInfo[r] = fetched ? -2 : n == 0 ? (e ? -2 : -1) : n == 1 ? segIdx[a] : -2;
+        const bool listed = n > 1 && !fetched;
+        isLight[r] = listed && n <= lightSegs;
+        isHeavy[r] = listed && n > lightSegs;
+        if (listed && n <= lightSegs && n > 4) atomicOr(over4, 1);
+    } else if (r == rows) {  // the scans run over rows + 1 elements
         isLight[r] = isHeavy[r] = 0;
-        return;
     }
-    const int a = segPtr[r], n = segPtr[r + 1] - a;
-    const int e = elsewhere ? elsewhere[r] : 0;
-    const bool fetched = e == 2;
-    rowInfo[r] = fetched ? -2 : n == 0 ? (e ? -2 : -1) : n == 1 ? segIdx[a] : -2;
-    const bool listed = n > 1 && !fetched;
-    isLight[r] = listed && n <= lightSegs;
-    isHeavy[r] = listed && n > lightSegs;
-    if (listed && n <= lightSegs && n > 4) atomicOr(over4, 1);
+    // the most virtual rows of any row: one atomic per wave
+    int m = n;
+    for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off));
+    if ((threadIdx.x & 63) == 0 && m > 1) atomicMax(most, m);
 }
 
 __global__ __launch_bounds__(kBlock) void row_lists_kernel(const int *__restrict__ segPtr, const int *__restrict__ segIdx,
@@ -483,7 +488,7 @@ static int device_value_dict(const V *val, int nnz, mxl::Buf &codes, std::vector
 template <typename V>
 static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr, const int *col, const V *val, int nCU,
                                  int S, const char *elsewhere, DeviceSlices &D, hipStream_t s, std::vector<int> *segPtrOut,
-                                 std::vector<int> *segIdxOut)
+                                 std::vector<int> *segIdxOut, int fused)
 {
     using namespace mxl;
     const int E = slice_step_entries(dtype), BE = kSliceBatchEntries, SW = slice_cols(dtype), W = kSliceWaves;
@@ -594,6 +599,31 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
         hipLaunchKernelGGL(vrow_keys_kernel, grid(nV), dim3(kBlock), 0, s, (const int *)vStart.p, (const int *)vRow.p, (const int *)vSlice.p,
                            (const int *)segPtr.p, nV, nnz, cap, kSliceLightSegs, key.as<unsigned>(), pay.as<int>(), vLen.as<int>());
         MXL_TRY(hipGetLastError());
+    }
+    // ---- the one-launch form, where it is wanted and the matrix suits it: the records of the virtual rows come
+    // down, the host plans (plan_fused_records: the same plan as the host route's), the order goes up
+    SlicePlan SP;
+    int fusedPlaces = 0;
+    bool fusedTaken = false;
+    std::vector<int> hSegPtr;
+    if (fused && nV > 0 && !elsewhere) {
+        std::vector<int> hRowPtr((size_t)rows + 1), hSlice((size_t)nV), hLen((size_t)nV), hSorted;
+        hSegPtr.resize((size_t)rows + 1);
+        MXL_TRY(hipMemcpyAsync(hRowPtr.data(), rowPtr, ((size_t)rows + 1) * 4, hipMemcpyDeviceToHost, s));
+        MXL_TRY(hipMemcpyAsync(hSegPtr.data(), segPtr.p, ((size_t)rows + 1) * 4, hipMemcpyDeviceToHost, s));
+        MXL_TRY(hipMemcpyAsync(hSlice.data(), vSlice.p, (size_t)nV * 4, hipMemcpyDeviceToHost, s));
+        MXL_TRY(hipMemcpyAsync(hLen.data(), vLen.p, (size_t)nV * 4, hipMemcpyDeviceToHost, s));
+        MXL_TRY(hipStreamSynchronize(s));
+        const int rc = plan_fused_records(dtype, budget, S, rows, cap, hRowPtr.data(), hSegPtr.data(), hSlice.data(), hLen.data(), nV, fused,
+                                          hSorted, SP, &fusedPlaces);
+        if (rc < 0) return rc;
+        fusedTaken = rc == 1;
+        if (fusedTaken) {
+            MXL_TRY(hipMemcpyAsync(sorted.p, hSorted.data(), (size_t)nV * 4, hipMemcpyHostToDevice, s));
+            MXL_TRY(hipStreamSynchronize(s));  // `hSorted` leaves scope
+        }
+    }
+    if (nV > 0 && !fusedTaken) {
         unsigned keyBits = 1;
         while (keyBits < 32 && (1ull << keyBits) < (unsigned long long)S * (unsigned long long)(cap + 1) * 3ull) ++keyBits;
         size_t sortBytes = 0;
@@ -614,7 +644,7 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
     // ---- chunks: their lengths come down, the plan of the streams goes up
     std::vector<std::vector<SliceChunk>> sliceChunks((size_t)S);
     std::vector<int> firstIdx;
-    {
+    if (!fusedTaken) {
         int at = 0;
         for (int q = 0; q < S; ++q) {
             for (int f = at; f < at + sliceCnt[q]; f += 64) {
@@ -625,7 +655,7 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
         }
     }
     const int nChunk = (int)firstIdx.size();
-    if (nChunk > 0) {
+    if (nChunk > 0 && !fusedTaken) {
         Buf dFirst, dLen;
         std::vector<int> len((size_t)nChunk);
         MXL_TRY(hipMalloc(&dFirst.p, (size_t)nChunk * 4));
@@ -640,8 +670,7 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
         for (int q = 0; q < S; ++q)
             for (SliceChunk &c : sliceChunks[q]) c.steps = (len[i++] + E - 1) / E;
     }
-    SlicePlan SP;
-    {
+    if (!fusedTaken) {
         const int rc = plan_slice_chunks(dtype, budget, S, sliceChunks, SP);
         if (rc) return rc;
     }
@@ -717,17 +746,19 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
     MXL_TRY(hipMalloc(&lightPos.p, r1 * 4));
     MXL_TRY(hipMalloc(&heavyPos.p, r1 * 4));
     hipLaunchKernelGGL(row_info_kernel, grid((long long)rows + 1), dim3(kBlock), 0, s, (const int *)segPtr.p, (const int *)D.segIdx, elsewhere,
-                       rows, kSliceLightSegs, D.rowInfo, isLight.as<int>(), isHeavy.as<int>(), over4);
+                       rows, kSliceLightSegs, D.rowInfo, isLight.as<int>(), isHeavy.as<int>(), over4, over4 + 1);
     MXL_TRY(hipGetLastError());
     MXL_TRY(rocprim::exclusive_scan(tmp.p, scanBytes, (const int *)isLight.p, lightPos.as<int>(), 0, r1, rocprim::plus<int>(), s));
     MXL_TRY(rocprim::exclusive_scan(tmp.p, scanBytes, (const int *)isHeavy.p, heavyPos.as<int>(), 0, r1, rocprim::plus<int>(), s));
-    int nLight = 0, nHeavy = 0, anyOver4 = 0;
+    int nLight = 0, nHeavy = 0, anyOver4 = 0, mostVrows = 0;
+    MXL_TRY(hipMemcpyAsync(&mostVrows, over4 + 1, 4, hipMemcpyDeviceToHost, s));
     MXL_TRY(hipMemcpyAsync(&nLight, lightPos.as<int>() + rows, 4, hipMemcpyDeviceToHost, s));
     MXL_TRY(hipMemcpyAsync(&nHeavy, heavyPos.as<int>() + rows, 4, hipMemcpyDeviceToHost, s));
     MXL_TRY(hipMemcpyAsync(&anyOver4, over4, 4, hipMemcpyDeviceToHost, s));
     MXL_TRY(hipStreamSynchronize(s));
     D.nLight = nLight;
     D.nHeavy = nHeavy;
+    D.mostVrows = std::max(mostVrows, nV > 0 ? 1 : 0);
     const int places = anyOver4 ? kSliceLightSegs : 4;
     D.lightQuads = places / 4;
     MXL_TRY(hipMalloc((void **)&D.lightRow, ((size_t)nLight + 1) * 4));
@@ -744,6 +775,32 @@ static int build_slices_device_t(mx_dtype dtype, int rows, int cols, int nnz, co
     const size_t accBytes = dtype == MX_F64 ? 8 : 4;
     MXL_TRY(hipMalloc(&D.partial, ((size_t)SP.totalChunks * 64 + 64) * accBytes));
     MXL_TRY(hipMemsetAsync(D.partial, 0, ((size_t)SP.totalChunks * 64 + 64) * accBytes, s));
+    if (fusedTaken) {
+        // what the one-launch kernel needs beyond the two-launch arrays (which stay valid: the plan falls back on them)
+        std::vector<int> hSegIdx(nv1, 0), target;
+        MXL_TRY(hipMemcpyAsync(hSegIdx.data(), D.segIdx, nv1 * 4, hipMemcpyDeviceToHost, s));
+        MXL_TRY(hipStreamSynchronize(s));
+        fused_targets(rows, SP.nGroups, fusedPlaces, SP.totalChunks, hSegPtr.data(), hSegIdx.data(), target);
+        D.nGroups = SP.nGroups;
+        D.maxWgGroups = SP.maxWgGroups;
+        D.placesPerRow = fusedPlaces;
+        if ((rc = up((void **)&D.wgGroups, SP.wgGroups.data(), SP.wgGroups.size() * 4))) return rc;
+        if ((rc = up((void **)&D.groupNeed, SP.groupNeed.data(), SP.groupNeed.size() * 4))) return rc;
+        const size_t nTarget = target.size() + 64;  // (64 spare entries, zero)
+        MXL_TRY(hipMalloc((void **)&D.fusedTarget, nTarget * 4));
+        MXL_TRY(hipMemsetAsync(D.fusedTarget, 0, nTarget * 4, s));
+        MXL_TRY(hipMemcpyAsync(D.fusedTarget, target.data(), target.size() * 4, hipMemcpyHostToDevice, s));
+        const size_t nCount = (size_t)SP.nGroups + 1, nClaim = (size_t)SP.nWG + 1;
+        const size_t sumBytes = ((size_t)SP.nGroups * fusedPlaces * kFusedGroupRows + 64) * accBytes;
+        MXL_TRY(hipMalloc((void **)&D.groupCount, nCount * 4));
+        MXL_TRY(hipMemsetAsync(D.groupCount, 0, nCount * 4, s));
+        MXL_TRY(hipMalloc((void **)&D.claim, nClaim * 4));
+        MXL_TRY(hipMemsetAsync(D.claim, 0, nClaim * 4, s));
+        MXL_TRY(hipMalloc(&D.fusedSums, sumBytes));
+        MXL_TRY(hipMemsetAsync(D.fusedSums, 0, sumBytes, s));
+        MXL_TRY(hipStreamSynchronize(s));  // `target` leaves scope
+        D.fused = true;
+    }
     if (segPtrOut) {
         segPtrOut->assign((size_t)rows + 1, 0);
         MXL_TRY(hipMemcpyAsync(segPtrOut->data(), segPtr.p, ((size_t)rows + 1) * 4, hipMemcpyDeviceToHost, s));
@@ -868,7 +925,7 @@ int upload_csr_device(mx_dtype dtype, int rows, int cols, int nnz, const int *ro
 
 int build_slices_device(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *col_dev, const void *val_dev,
                         int nCU, int S, const char *elsewhere_dev, DeviceSlices &D, hipStream_t s, std::vector<int> *segPtrOut,
-                        std::vector<int> *segIdxOut)
+                        std::vector<int> *segIdxOut, int fused)
 {
     if (rows < 1 || cols < 1 || nnz < 0 || S < 1 || !rowPtr_dev || (nnz > 0 && (!col_dev || !val_dev))) {
         set_error("slice layout on the device: bad argument");
@@ -877,9 +934,9 @@ int build_slices_device(mx_dtype dtype, int rows, int cols, int nnz, const int *
     MXL_TRY(prepare_slice_kernels(dtype));
     if (dtype == MX_F64)
         return build_slices_device_t<double>(dtype, rows, cols, nnz, rowPtr_dev, col_dev, (const double *)val_dev, nCU, S, elsewhere_dev, D,
-                                             s, segPtrOut, segIdxOut);
+                                             s, segPtrOut, segIdxOut, fused);
     return build_slices_device_t<_Float16>(dtype, rows, cols, nnz, rowPtr_dev, col_dev, (const _Float16 *)val_dev, nCU, S, elsewhere_dev,
-                                           D, s, segPtrOut, segIdxOut);
+                                           D, s, segPtrOut, segIdxOut, fused);
 }
 
 }  // namespace mx

@@ -58,8 +58,17 @@ static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, 
     if (env == 1) want[0] = true, want[1] = false;
     if (env == 2 && S > 0) want[1] = true, want[0] = false;
     if (want[1]) {
+        // (the one-launch form where the matrix suits it and the device deals its workgroups as the form assumes:
+        // the layout is made for it in the same pass -- the records of the virtual rows go to the host, its plan
+        // comes back, the entries stay)
+        int wantFused = !elsewhere_dev ? fused_wanted(flags, dtype, rows, S, -1, nCU) : 0;
+        if (wantFused) {
+            int ok = 0;
+            MX_HIP(mx::fused_placement_ok(nCU, &ok));
+            if (!ok) wantFused = 0;
+        }
         rc = mx::build_slices_device(dtype, rows, cols, nnz, rowPtr_dev, colInd_dev, val_dev, nCU, S, elsewhere_dev, plan->slices, nullptr,
-                                     segOut ? &segOut->first : nullptr, segOut ? &segOut->second : nullptr);
+                                     segOut ? &segOut->first : nullptr, segOut ? &segOut->second : nullptr, wantFused);
         if (rc) return rc;
         if (plan->slices.ecode) plan->slices.useDict = true;
     }
@@ -71,42 +80,13 @@ static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, 
         st.fewValues = plan->slices.ecode != nullptr;
         if ((rc = mx::lines_per_gather_device(dtype, nnz, colInd_dev, nullptr, &st.linesPerGather))) return rc;
         csr_estimates(dtype, cols, nnz, st, &plan->est_rows_us, &plan->est_slices_us);
-        if (!elsewhere_dev && plan->slices.nHeavy == 0 && fused_wanted(flags, dtype, rows, S, -1, nCU)) plan->est_slices_us -= kFusedSavesUs;
+        // (as the host route, which estimates before it has a layout: by the average of the sums under a workgroup)
+        if (!elsewhere_dev && fused_wanted(flags, dtype, rows, S, plan->slices.mostVrows, nCU)) plan->est_slices_us -= kFusedSavesUs;
         want[plan->est_slices_us < plan->est_rows_us ? 0 : 1] = false;
     }
     if (want[1]) {
         plan->csr_variant = 1;
-        // The one-launch form where the host route would take it (no row with more than eight virtual rows: the
-        // layout just made has no heavy rows).  Its layout is made on the host, from a copy of the part: the
-        // matrices it is taken for have few sums per workgroup (fused_wanted), unless it is forced.
-        int wantFused = !elsewhere_dev && plan->slices.nHeavy == 0 ? fused_wanted(flags, dtype, rows, S, -1, nCU) : 0;
-        if (wantFused) {
-            int ok = 0;
-            MX_HIP(mx::fused_placement_ok(nCU, &ok));
-            if (!ok) wantFused = 0;
-        }
-        if (wantFused) {
-            const size_t es = (size_t)mx::elem_size(dtype);
-            std::vector<int> rp((size_t)rows + 1), ci((size_t)std::max(nnz, 1));
-            std::vector<unsigned char> va(std::max<size_t>((size_t)nnz * es, 1));
-            MX_HIP(hipMemcpy(rp.data(), rowPtr_dev, ((size_t)rows + 1) * 4, hipMemcpyDeviceToHost));
-            if (nnz) MX_HIP(hipMemcpy(ci.data(), colInd_dev, (size_t)nnz * 4, hipMemcpyDeviceToHost));
-            if (nnz) MX_HIP(hipMemcpy(va.data(), val_dev, (size_t)nnz * es, hipMemcpyDeviceToHost));
-            mx::DeviceSlices L;
-            rc = upload_slices(dtype, rows, cols, rp.data(), ci.data(), va.data(), nCU, S, nullptr, L, nullptr, segOut, wantFused);
-            if (rc) {
-                free_slices(L);
-                return rc;
-            }
-            if (L.fused) {
-                free_slices(plan->slices);
-                plan->slices = L;
-                if (plan->slices.ecode) plan->slices.useDict = true;
-                plan->fused = true;
-            } else {
-                free_slices(L);
-            }
-        }
+        plan->fused = plan->slices.fused;
         return MX_OK;
     }
     free_slices(plan->slices);

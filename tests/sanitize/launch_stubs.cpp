@@ -10,7 +10,7 @@ hipError_t fused_placement_ok(int, int *ok) { *ok = 0; return hipErrorUnknown; }
 hipError_t prepare_slice_kernels(mx_dtype) { return hipErrorUnknown; }
 hipError_t static_scratch(void **p) { *p = nullptr; return hipErrorUnknown; }
 int build_slices_device(mx_dtype, int, int, int, const int *, const int *, const void *, int, int, const char *, DeviceSlices &, hipStream_t,
-                        std::vector<int> *, std::vector<int> *) { return MX_ERR_DEVICE; }
+                        std::vector<int> *, std::vector<int> *, int) { return MX_ERR_DEVICE; }
 int check_csr_device(int, int, int, const int *, const int *, hipStream_t, const char *) { return MX_ERR_DEVICE; }
 int lines_per_gather_device(mx_dtype, int, const int *, hipStream_t, double *) { return MX_ERR_DEVICE; }
 int upload_csr_device(mx_dtype, int, int, int, const int *, const int *, const void *, const std::vector<int> &, bool, DeviceCsr &, hipStream_t) { return MX_ERR_DEVICE; }

@@ -1014,11 +1014,12 @@ def test_spmv_in_a_hip_graph(mx, ora):
     P.close()
 
 
-def test_one_launch_form_of_the_slices(mx, ora):
+def test_one_launch_form_of_the_slices(mx, ora, monkeypatch):
     """The CSR part in slice form as ONE launch (the reference's residual kernel is one launch,
     src/spmv_kernel/cdSpMV.cu:459): y equals the two-launch form's bit for bit and the oracle's within the
     bar, on binary64 and binary16, with four and with eight places per row, on rows without entries,
-    on the plan made from device arrays, product after product (the counters clear themselves), with y
+    on the plan made from device arrays and on the one whose layout the host makes (all three the same arrays),
+    product after product (the counters clear themselves), with y
     accumulated; a default plan takes the form only while the sums under a workgroup, and the slices, are
     few; under stream capture
     the two launches are recorded."""
@@ -1084,6 +1085,14 @@ def test_one_launch_form_of_the_slices(mx, ora):
         assert D.arrays() == one.arrays()
         assert np.array_equal(D.spmv(xd).cpu().numpy().view(np.uint8), y2.view(np.uint8)), name
         D.close()
+        # the layout made on the host (the entries re-laid there) is the one the device makes from the host's plan
+        monkeypatch.setenv("MX_LAYOUT", "host")
+        H = mx.Plan(P, mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_FUSE)
+        monkeypatch.delenv("MX_LAYOUT")
+        assert H.info["csr_fused"] == 1
+        assert H.arrays() == one.arrays(), name
+        assert np.array_equal(H.spmv(xd).cpu().numpy().view(np.uint8), y2.view(np.uint8)), name
+        H.close()
         if default_takes_it is not None:
             d = mx.Plan(P, mx.MX_PLAN_CSR_SLICES)
             assert d.info["csr_fused"] == (1 if default_takes_it else 0), (name, d.info)
