@@ -357,6 +357,7 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
         "dtype": dtype, "rows": A.rows, "nnz": A.nnz,
         "tau_c": tau[0], "tau_r": tau[1], "plan": plan_kind, "plan_flags": "MX_PLAN_DEFAULT" if FLAGS == mx.MX_PLAN_DEFAULT else "MX_PLAN_KEEP_TILES" if FLAGS == mx.MX_PLAN_KEEP_TILES else int(FLAGS),
         "csr_variant": ("rows", "slices", "split")[info["csr_variant"]], "csr_one_launch": bool(info["csr_fused"]),
+        "csr_entries_kept_in_cache": bool(info["csr_keep"]),
         "tile_nnz": info["tile_nnz"], "csr_nnz": info["csr_nnz"],
         "ms_per_step": wall_ms, "ms_per_step_events": ev_total,
         "gflops": 2.0 * A.nnz / (wall_ms * 1e-3) / 1e9,
@@ -488,7 +489,7 @@ def main():
     del A, x
     for k in ("hbm_frac_whole_spmv", "cold_cache", "rotating", "rel_l2_vs_oracle", "plan_create_ms", "plan_create_device_ms",
               "matrix_to_first_y", "plan_estimates_us", "csr_only_ms", "best_hybrid", "tile_nnz", "csr_nnz", "ms_per_step_events",
-              "algorithmic_bytes", "plan_bytes_per_product", "plan_flags", "csr_one_launch", "sweep", "sweep_flags", "sweep_seconds"):
+              "algorithmic_bytes", "plan_bytes_per_product", "plan_flags", "csr_one_launch", "csr_entries_kept_in_cache", "sweep", "sweep_flags", "sweep_seconds"):
         out[k] = main_rec[k]
 
     # what a plain device copy reaches on this GPU, next to the 8 TB/s the roofline is priced at:

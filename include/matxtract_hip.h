@@ -265,6 +265,13 @@ double mx_algorithmic_bytes(mx_dtype dtype, int rows, int cols, int nnz);
                                  (beyond that two launches are as fast or faster) -- and
                                  the device deals its workgroups round-robin to eight XCDs, which plan creation checks */
 #define MX_PLAN_FUSE 64      /* the one-launch form wherever the matrix suits it, whatever its size */
+#define MX_PLAN_KEEP 128     /* CSR part in slice form: read the entries with plain loads, so that a matrix that fits the L2s or the
+                                 memory-side cache stays there from one product to the next (a solver that multiplies with the same
+                                 matrix again and again).  Without this flag and MX_PLAN_STREAM the plan decides by size
+                                 (mx_plan_info.csr_keep): plain loads where the entries fit the L2s, or fit the memory-side cache
+                                 and the second launch moves enough to push streamed entries out of it */
+#define MX_PLAN_STREAM 256   /* ... read them with streaming (non-temporal) loads whatever the size: 10-25 % faster when a
+                                 product finds the caches cold, slower when the matrix could have stayed in them */
 
 /* Uploads a partition once and keeps it on the device: the persistent counterpart of the
  * per-call cudaMalloc/cudaMemcpy blocks in cdspmv (src/spmv_kernel/cdSpMV.cu:407-418) and
@@ -509,6 +516,9 @@ typedef struct mx_plan_info {
                             runs; a plan made under one setting keeps it whatever the environment says later */
     double opt_tile_gate;/* the fill a fragment needed for the tile kernels when the plan was made (MX_TILE_GATE;
                             one half unless set) */
+    int csr_keep;        /* 1: the slice kernel reads the entries with plain loads (they may stay in the caches between
+                            products), 0: it streams them (MX_PLAN_KEEP / MX_PLAN_STREAM, MX_CSR_KEEP, or the plan's own
+                            choice by size) */
 } mx_plan_info;
 /* mx_plan_info.opt_flags */
 #define MX_OPT_NO_STRIPS 1     /* MX_NO_STRIPS=1: no binary16 strip chunks */
@@ -519,6 +529,7 @@ typedef struct mx_plan_info {
 #define MX_OPT_CSR_FUSED 32    /* MX_CSR_FUSED=0|1 decided about the one-launch form */
 #define MX_OPT_AUTOTUNE 64     /* MX_PLAN_AUTOTUNE=1: forms were timed, not estimated (the plan may differ run to run) */
 #define MX_OPT_LAYOUT_HOST 128 /* MX_LAYOUT=host: layouts made on the host where the device route exists (same arrays) */
+#define MX_OPT_CSR_KEEP 512    /* MX_CSR_KEEP=0|1 decided how the slice kernel reads its entries */
 #define MX_OPT_TUNING 256      /* one of the tuning knobs was set: MX_SLICE_CAP, MX_SPLIT_LEN, MX_CSR_NPT, MX_TILE_PER,
                                   MX_CSR_REDUCE, MX_CSR_COL16 */
 int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info);

@@ -14,6 +14,8 @@ MX_OK, MX_ERR_ARG, MX_ERR_ALLOC, MX_ERR_DEVICE, MX_ERR_IO = 0, 1, 2, 3, 4
 MX_F64, MX_F16 = 0, 1
 MX_PLAN_DEFAULT, MX_PLAN_NO_TILES, MX_PLAN_ALL_TILES = 0, 1, 2
 MX_PLAN_CSR_ROWS, MX_PLAN_CSR_SLICES, MX_PLAN_KEEP_TILES, MX_PLAN_NO_FUSE, MX_PLAN_FUSE = 4, 8, 16, 32, 64
+MX_PLAN_KEEP, MX_PLAN_STREAM = 128, 256
+MX_OPT_CSR_KEEP = 512
 # mx_plan_info.opt_flags: the switches of the environment a plan was made under
 MX_OPT_NO_STRIPS, MX_OPT_NO_BLOCKS, MX_OPT_NO_DICT, MX_OPT_STRIPS_APART, MX_OPT_CSR_KERNEL = 1, 2, 4, 8, 16
 MX_OPT_CSR_FUSED, MX_OPT_AUTOTUNE, MX_OPT_LAYOUT_HOST, MX_OPT_TUNING = 32, 64, 128, 256
@@ -57,7 +59,7 @@ class PlanInfo(C.Structure):
                 ("csr_main_kernel", C.c_int), ("csr_main_nnz", C.c_int), ("tile_variant", C.c_int), ("tile_strip_nnz", C.c_int),
                 ("csr_value_dict", C.c_int), ("est_rows_us", C.c_double), ("est_slices_us", C.c_double),
                 ("prep_route", C.c_int), ("ext_dCols", C.c_int), ("ext_dRows", C.c_int), ("ext_nnzRowD", C.c_int),
-                ("ext_frags", C.c_int), ("csr_fused", C.c_int), ("opt_flags", C.c_int), ("opt_tile_gate", C.c_double)]
+                ("ext_frags", C.c_int), ("csr_fused", C.c_int), ("opt_flags", C.c_int), ("opt_tile_gate", C.c_double), ("csr_keep", C.c_int)]
 
 
 class TauEstimate(C.Structure):

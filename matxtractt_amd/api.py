@@ -12,14 +12,14 @@ import numpy as np
 
 from . import _lib
 from ._lib import (MX_F16, MX_F64, MX_PLAN_ALL_TILES, MX_PLAN_CSR_SLICES, MX_PLAN_CSR_ROWS, MX_PLAN_DEFAULT,
-                   MX_PLAN_FUSE, MX_PLAN_KEEP_TILES, MX_PLAN_NO_FUSE, MX_PLAN_NO_TILES, MX_OPT_NO_STRIPS, MX_OPT_NO_BLOCKS,
+                   MX_PLAN_FUSE, MX_PLAN_KEEP, MX_PLAN_STREAM, MX_OPT_CSR_KEEP, MX_PLAN_KEEP_TILES, MX_PLAN_NO_FUSE, MX_PLAN_NO_TILES, MX_OPT_NO_STRIPS, MX_OPT_NO_BLOCKS,
                    MX_OPT_NO_DICT, MX_OPT_STRIPS_APART, MX_OPT_CSR_KERNEL, MX_OPT_CSR_FUSED, MX_OPT_AUTOTUNE,
                    MX_OPT_LAYOUT_HOST, MX_OPT_TUNING, MxError, check)
 
 __all__ = ["Csr", "Partition", "Plan", "gen_config", "mmio_read", "transpose", "transpose_device", "select_device", "split_device", "tiles_device", "cdspmv",
            "du_tcspmv", "algorithmic_bytes", "device_count", "init_vec", "slice_layout", "tune_tau", "estimate_tau", "tile_steps", "MxError",
            "MX_F64", "MX_F16", "MX_PLAN_DEFAULT", "MX_PLAN_NO_TILES", "MX_PLAN_ALL_TILES", "MX_PLAN_CSR_ROWS",
-           "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "MX_PLAN_NO_FUSE", "MX_PLAN_FUSE", "time_rotate", "plan_layout", "debug_fused_misplaced",
+           "MX_PLAN_CSR_SLICES", "MX_PLAN_KEEP_TILES", "MX_PLAN_NO_FUSE", "MX_PLAN_FUSE", "MX_PLAN_KEEP", "MX_PLAN_STREAM", "MX_OPT_CSR_KEEP", "time_rotate", "plan_layout", "debug_fused_misplaced",
            "MX_OPT_NO_STRIPS", "MX_OPT_NO_BLOCKS", "MX_OPT_NO_DICT", "MX_OPT_STRIPS_APART", "MX_OPT_CSR_KERNEL",
            "MX_OPT_CSR_FUSED", "MX_OPT_AUTOTUNE", "MX_OPT_LAYOUT_HOST", "MX_OPT_TUNING"]
 

@@ -127,6 +127,7 @@ struct DeviceSlices {
     int *heavyInfo = nullptr;         // [nHeavy][4]
     int nLight = 0, nHeavy = 0;
     int mostVrows = 0;                // most virtual rows of any row
+    bool keep = false;                // the entries are read with plain loads (they may stay in the caches), not streamed
     // The one-launch form (csr_slice_kernel<.., FUSED>), when the layout was made for it: the rows are cut
     // into groups of kFusedGroupRows, the groups into one contiguous range per XCD, and the virtual rows
     // of a slice are ordered by group before length, so that a workgroup's chunks cover a contiguous run
@@ -161,6 +162,10 @@ constexpr int kFusedAddBytes = 100 * 1024;  // most bytes of sums under one work
                                             // chunk (about 70 ns per 2 KB), and beyond this a second launch is the faster way
 constexpr int kFusedSlicesMost = 8;          // ... and most slices: every XCD copies every slice of x in this form (a slice's workgroups are
                                             // spread over all eight), 64 ns a slice more than when one XCD has a slice to itself
+constexpr long long kKeepL2Bytes = 24LL << 20;      // entries of a slice layout up to this size fit the eight L2s beside x and the sums
+constexpr long long kKeepCacheBytes = 192LL << 20;  // ... and up to this size the memory-side cache beside everything else a product touches
+constexpr long long kKeepHandoffBytes = 10LL << 20;  // what the second launch must move per product (sums, row tables, y) to push streamed
+                                                    // entries out of the memory-side cache fast enough for plain loads to pay
 constexpr int kSliceBytes = 131072;   // the slice of x a workgroup keeps in LDS
 constexpr int kSliceLdsMax = 163840;  // LDS of a CU
 constexpr int kSliceWgChunks = 4096;  // most chunks a workgroup may have

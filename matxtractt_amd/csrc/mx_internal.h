@@ -26,6 +26,7 @@ struct Options {
     bool strips_apart = false;// MX_STRIPS_APART=1: strips in a launch of their own instead of the combine kernel's
     int csr_kernel = 0;       // MX_CSR_KERNEL=rows|slices|split: 1 | 2 | 3; 0 = the plan decides
     int csr_fused = -1;       // MX_CSR_FUSED: 0 = never the one-launch form, 1 = wherever the matrix suits it; -1 = the plan decides
+    int csr_keep = -1;        // MX_CSR_KEEP: 0 = the slice kernel streams its entries, 1 = it reads them with plain loads; -1 = the plan decides
     bool autotune = false;    // MX_PLAN_AUTOTUNE=1: the forms of the CSR part are timed on the spot instead of estimated
     bool layout_host = false; // MX_LAYOUT=host: layouts on the host also where the device route exists
     int slice_cap = 0;        // MX_SLICE_CAP=<entries>: longest virtual row (tuning runs); 0 = a lane's fair share

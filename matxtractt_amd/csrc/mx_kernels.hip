@@ -480,18 +480,29 @@ __global__ __launch_bounds__(kBlock) void csr_rows_kernel(const int *__restrict_
 // traffic at all, and at the end of a chunk of 64 virtual rows every lane stores one sum,
 // the wave 64 consecutive ones.  A second kernel adds up the virtual rows of every matrix row.
 // No atomics anywhere: every sum and every y has one owner.
+// How the slice kernel reads its entries.  Streaming (non-temporal) loads leave the caches to x and the sums,
+// and what they bring does not stay in the memory-side cache once other traffic asks for room there: right for a
+// matrix that fits no cache, and for a product that finds the caches cold.  Plain loads let a matrix that fits
+// the L2s or the memory-side cache live there from product to product.  The kind of load is a property of the
+// instruction, so it is a kernel variant, chosen per plan (DeviceSlices::keep).
+template <bool KEEP, typename T>
+__device__ __forceinline__ T stream_load(const T *p)
+{
+    if constexpr (KEEP) return *p;
+    else return __builtin_nontemporal_load(p);
+}
 template <typename VT>
 struct SliceBatch;  // what one lane reads per batch: 8 column offsets, 8 values
 template <>
 struct SliceBatch<double> {
     v4i32 c;
     v2f64 v[4];
+    template <bool KEEP>
     __device__ __forceinline__ void load(const unsigned short *ecol, const double *eval, size_t batch, int lane)
     {
-        c = __builtin_nontemporal_load((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
+        c = stream_load<KEEP>((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            v[j] = __builtin_nontemporal_load((const v2f64 *)(eval + batch * 512 + j * 128 + lane * 2));
+        for (int j = 0; j < 4; ++j) v[j] = stream_load<KEEP>((const v2f64 *)(eval + batch * 512 + j * 128 + lane * 2));
     }
     // what entry k of the batch multiplies with: its x (a lane asks for all of a batch's before it uses
     // the first, so the LDS answers them in one go) ...
@@ -506,10 +517,11 @@ struct SliceBatch<double> {
 template <>
 struct SliceBatch<_Float16> {
     v4i32 c, v;
+    template <bool KEEP>
     __device__ __forceinline__ void load(const unsigned short *ecol, const _Float16 *eval, size_t batch, int lane)
     {
-        c = __builtin_nontemporal_load((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
-        v = __builtin_nontemporal_load((const v4i32 *)(eval + (batch * 64 + lane) * 8));
+        c = stream_load<KEEP>((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
+        v = stream_load<KEEP>((const v4i32 *)(eval + (batch * 64 + lane) * 8));
     }
     __device__ __forceinline__ _Float16 gather(const _Float16 *xs, int k) const
     {
@@ -530,10 +542,11 @@ struct SliceBatchDict {
     typedef typename Acc<VT>::type AT;
     v4i32 c;
     v2i32 k;
+    template <bool KEEP>
     __device__ __forceinline__ void load(const unsigned short *ecol, const unsigned char *ecode, size_t batch, int lane)
     {
-        c = __builtin_nontemporal_load((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
-        k = __builtin_nontemporal_load((const v2i32 *)(ecode + (batch * 64 + lane) * 8));
+        c = stream_load<KEEP>((const v4i32 *)(ecol + (batch * 64 + lane) * 8));
+        k = stream_load<KEEP>((const v2i32 *)(ecode + (batch * 64 + lane) * 8));
     }
     __device__ __forceinline__ VT gather(const VT *xs, int j) const
     {
@@ -660,7 +673,7 @@ __device__ __forceinline__ void fused_add(const FusedArgs &fa, const int *list, 
 // every group whose count it completes adds the sums of the group's rows up -- in the order of the
 // row's places, whoever does it, so y does not depend on who came last -- and writes y.  It clears
 // the counter for the next launch.  No workgroup ever waits for another.
-template <typename VT, bool DICT = false, bool FUSED = false>
+template <typename VT, bool DICT = false, bool FUSED = false, bool KEEP = false>
 __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__restrict__ wgDesc,
                                                                   const int4 *__restrict__ waveDesc,
                                                                   const int *__restrict__ chunkEnd,
@@ -735,7 +748,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
     Batch buf[NB];
     const int lastBatch = batch0 + max(nb - 1, 0);
 #pragma unroll
-    for (int k = 0; k < NB; ++k) buf[k].load(ecol, estream, (size_t)min(batch0 + k, lastBatch), lane);
+    for (int k = 0; k < NB; ++k) buf[k].template load<KEEP>(ecol, estream, (size_t)min(batch0 + k, lastBatch), lane);
     endsL[max(min(tid, wgChunks - 1), 0)] = ce;
     if constexpr (FUSED) {
         if (tid == 0) *(int *)(smem + fa.ldsCount) = 0;  // (read after the stream, behind two barriers)
@@ -819,7 +832,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 #pragma unroll
             for (int k = 0; k < NB; ++k) {
                 consume(buf[k], t + k);
-                buf[k].load(ecol, estream, (size_t)(batch0 + t + NB + k), lane);
+                buf[k].template load<KEEP>(ecol, estream, (size_t)(batch0 + t + NB + k), lane);
             }
         }
         // one ring in flight and less than one more to come: consume and reload while batches
@@ -827,7 +840,7 @@ __global__ __launch_bounds__(kSliceThreads) void csr_slice_kernel(const int4 *__
 #pragma unroll
         for (int k = 0; k < NB; ++k) {
             consume(buf[k], t + k);
-            buf[k].load(ecol, estream, (size_t)min(batch0 + t + NB + k, lastBatch), lane);
+            buf[k].template load<KEEP>(ecol, estream, (size_t)min(batch0 + t + NB + k, lastBatch), lane);
         }
 #pragma unroll
         for (int k = 0; k < NB; ++k)
@@ -1486,8 +1499,10 @@ hipError_t launch_csr(mx_dtype dtype, const DeviceCsr &A, const void *x, void *y
 template <typename VT>
 static hipError_t slice_kernel_attributes()
 {
-    const void *fn[4] = {(const void *)mxk::csr_slice_kernel<VT, false, false>, (const void *)mxk::csr_slice_kernel<VT, true, false>,
-                         (const void *)mxk::csr_slice_kernel<VT, false, true>, (const void *)mxk::csr_slice_kernel<VT, true, true>};
+    const void *fn[8] = {(const void *)mxk::csr_slice_kernel<VT, false, false>,       (const void *)mxk::csr_slice_kernel<VT, true, false>,
+                         (const void *)mxk::csr_slice_kernel<VT, false, true>,        (const void *)mxk::csr_slice_kernel<VT, true, true>,
+                         (const void *)mxk::csr_slice_kernel<VT, false, false, true>, (const void *)mxk::csr_slice_kernel<VT, true, false, true>,
+                         (const void *)mxk::csr_slice_kernel<VT, false, true, true>,  (const void *)mxk::csr_slice_kernel<VT, true, true, true>};
     for (const void *f : fn) {
         const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, mx::kSliceLdsMax);
         if (e != hipSuccess) return e;
@@ -1520,14 +1535,15 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     if (lds > (size_t)mx::kSliceLdsMax || P.sliceCols != mx::slice_cols(sizeof(VT) == 8 ? MX_F64 : MX_F16))
         return hipErrorInvalidValue;
     if (what != 2 && P.nWG > 0) {
-        if (dict)
-            hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, true>), dim3(P.nWG), dim3(kSliceThreads), lds, s,
-                               (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.ecode,
-                               (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols, (const VT *)P.dict, P.maxWgChunks, mxk::FusedArgs());
-        else
-            hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, false>), dim3(P.nWG), dim3(kSliceThreads), lds, s,
-                               (const int4 *)P.wgDesc, (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.eval,
-                               (const VT *)x, (AT *)P.partial, P.cols, P.sliceCols, (const VT *)nullptr, P.maxWgChunks, mxk::FusedArgs());
+#define MX_LAUNCH_SLICES(DICT, KEEP, VALUES, TABLE)                                                                                  \
+    hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, DICT, false, KEEP>), dim3(P.nWG), dim3(kSliceThreads), lds, s, (const int4 *)P.wgDesc, \
+                       (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)(VALUES), (const VT *)x, (AT *)P.partial, P.cols,        \
+                       P.sliceCols, (const VT *)(TABLE), P.maxWgChunks, mxk::FusedArgs())
+        if (dict && P.keep) MX_LAUNCH_SLICES(true, true, P.ecode, P.dict);
+        else if (dict) MX_LAUNCH_SLICES(true, false, P.ecode, P.dict);
+        else if (P.keep) MX_LAUNCH_SLICES(false, true, P.eval, nullptr);
+        else MX_LAUNCH_SLICES(false, false, P.eval, nullptr);
+#undef MX_LAUNCH_SLICES
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || what == 1) return e;
@@ -1593,14 +1609,15 @@ static hipError_t launch_fused_t(const DeviceSlices &P, const void *x, void *y, 
     fa.placesPerRow = P.placesPerRow;
     fa.accumulate = accumulate;
     fa.ldsCount = (int)lds - 16;  // (in the 64 spare bytes at the end)
-    if (dict)
-        hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, true, true>), dim3(P.nWG), dim3(kSliceThreads), lds, s, (const int4 *)P.wgDesc,
-                           (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.ecode, (const VT *)x, (AT *)P.partial, P.cols,
-                           P.sliceCols, (const VT *)P.dict, ldsInts, fa);
-    else
-        hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, false, true>), dim3(P.nWG), dim3(kSliceThreads), lds, s, (const int4 *)P.wgDesc,
-                           (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)P.eval, (const VT *)x, (AT *)P.partial, P.cols,
-                           P.sliceCols, (const VT *)nullptr, ldsInts, fa);
+#define MX_LAUNCH_FUSED(DICT, KEEP, VALUES, TABLE)                                                                                  \
+    hipLaunchKernelGGL((mxk::csr_slice_kernel<VT, DICT, true, KEEP>), dim3(P.nWG), dim3(kSliceThreads), lds, s, (const int4 *)P.wgDesc, \
+                       (const int4 *)P.waveDesc, P.chunkEnd, P.ecol, (const VT *)(VALUES), (const VT *)x, (AT *)P.partial, P.cols,       \
+                       P.sliceCols, (const VT *)(TABLE), ldsInts, fa)
+    if (dict && P.keep) MX_LAUNCH_FUSED(true, true, P.ecode, P.dict);
+    else if (dict) MX_LAUNCH_FUSED(true, false, P.ecode, P.dict);
+    else if (P.keep) MX_LAUNCH_FUSED(false, true, P.eval, nullptr);
+    else MX_LAUNCH_FUSED(false, false, P.eval, nullptr);
+#undef MX_LAUNCH_FUSED
     return hipGetLastError();
 }
 hipError_t launch_fused(mx_dtype dtype, const DeviceSlices &P, const void *x, void *y, int accumulate, hipStream_t s, void *ywide,

@@ -186,6 +186,36 @@ int mxp::fused_wanted(int flags, mx_dtype dtype, int rows, int S, int mostVrows,
     return average <= (double)mx::kFusedAddBytes && S <= mx::kFusedSlicesMost ? 2 : 0;
 }
 
+// How the slice kernel of a plan reads its entries (DeviceSlices::keep).  Streaming loads are the faster way to
+// read a matrix once: they leave the caches to x and the sums, and what they bring is the first to leave the
+// memory-side cache when other traffic asks for room.  That is also their price: the second launch of a product
+// asks for room every time (the sums it is handed, its row tables, y), so a streamed matrix that would fit the
+// cache comes from HBM again in every product -- workload 4, 76 MB: 20.2 us streamed, the same in a rotation of
+// copies as back to back, 18.2 us with plain loads (and 0.42 instead of 0.47 of the roofline in the rotation,
+// 0.28 instead of 0.35 on cold caches: what plain loads cost when nothing can stay).  Plain loads where staying
+// pays: the entries fit the L2s (workload 2 at half size, 22 MB: 7.2 against 8.6 us), or they fit the memory-side
+// cache and the second launch moves enough to push them out (workload 3: 28.6 against 31.5 us; workload 2 at
+// full size in two launches, 44 MB of entries and 7 MB for the second launch, is the case it does not pay: 14.4 against 13.2 -- workload 4 hands 21 MB over).
+// The one-launch form has no second launch: only the first rule applies to it.
+void mxp::decide_keep(mx_plan *plan, int flags)
+{
+    mx::DeviceSlices &L = plan->slices;
+    L.keep = false;
+    if (plan->csr_variant == 0) return;
+    const int env = mx::opt().csr_keep;
+    if ((flags & MX_PLAN_STREAM) || env == 0) return;
+    if ((flags & MX_PLAN_KEEP) || env == 1) {
+        L.keep = true;
+        return;
+    }
+    const long long es = mx::elem_size(plan->dtype), E = mx::slice_step_entries(plan->dtype);
+    const long long entryBytes = (L.steps + mx::kSlicePadSteps) * 64 * E * (2 + (L.useDict ? 1 : es));
+    const long long handoff = (long long)partial_bytes(plan) + (long long)plan->rows * (4 + es) + (long long)L.nLight * (4 + 16 * L.lightQuads) +
+                              (long long)L.vrows * 4;
+    if (entryBytes <= mx::kKeepL2Bytes) L.keep = true;
+    else if (!plan->fused && entryBytes <= mx::kKeepCacheBytes && handoff >= mx::kKeepHandoffBytes) L.keep = true;
+}
+
 CsrChoice mxp::choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int flags,
                                 int nCU, int S, bool mayFuse)
 {
@@ -353,6 +383,7 @@ int mxp::setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const 
     }
     (void)hipFree(tx);
     (void)hipFree(ty);
+    if (!rc) decide_keep(plan, flags);
     return rc;
 }
 

@@ -87,6 +87,7 @@ static int setup_csr_part_device(mx_plan *plan, int nnz, const int *rowPtr_dev, 
     if (want[1]) {
         plan->csr_variant = 1;
         plan->fused = plan->slices.fused;
+        decide_keep(plan, flags);
         return MX_OK;
     }
     free_slices(plan->slices);

@@ -123,7 +123,7 @@ inline int plan_opt_flags()
 {
     const mx::Options &o = mx::opt();
     return (o.no_strips ? MX_OPT_NO_STRIPS : 0) | (o.no_blocks ? MX_OPT_NO_BLOCKS : 0) | (o.csr_dict == 0 ? MX_OPT_NO_DICT : 0) |
-           (o.strips_apart ? MX_OPT_STRIPS_APART : 0) | (o.csr_kernel ? MX_OPT_CSR_KERNEL : 0) | (o.csr_fused >= 0 ? MX_OPT_CSR_FUSED : 0) |
+           (o.strips_apart ? MX_OPT_STRIPS_APART : 0) | (o.csr_kernel ? MX_OPT_CSR_KERNEL : 0) | (o.csr_fused >= 0 ? MX_OPT_CSR_FUSED : 0) | (o.csr_keep >= 0 ? MX_OPT_CSR_KEEP : 0) |
            (o.autotune ? MX_OPT_AUTOTUNE : 0) | (o.layout_host ? MX_OPT_LAYOUT_HOST : 0) |
            (o.slice_cap || o.split_len || o.csr_npt || o.tile_per || o.csr_reduce || !o.csr_col16 ? MX_OPT_TUNING : 0);
 }
@@ -234,6 +234,8 @@ double tile_gate(mx_dtype dtype);
 void csr_estimates(mx_dtype dtype, int cols, int nnz, const CsrStats &st, double *usRows, double *usSlices);
 // 0: not wanted; 1: asked for (flag or environment); 2: by the default rule (the `fused` of build_slices)
 int fused_wanted(int flags, mx_dtype dtype, int rows, int S, int mostVrows, int nCU);
+// Sets plan->slices.keep for a plan whose CSR part is in slice form: how the slice kernel reads its entries.
+void decide_keep(mx_plan *plan, int flags);
 CsrChoice choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int flags, int nCU,
                           int S, bool mayFuse = false);
 int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags, const char *stripRows = nullptr,

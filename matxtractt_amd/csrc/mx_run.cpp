@@ -360,11 +360,11 @@ extern "C" int mx_time_kernels(mx_plan *plan, const void *x_dev, void *y_dev, in
     }
     if (plan->csr_variant == 1 && plan->fused && !ride) {
         // the one-launch form: one kernel multiplies, adds up and writes y
-        add(std::string("csr_slice_kernel<") + vt + (plan->slices.useDict ? ",dict,fused>" : ",fused>"),
+        add(std::string("csr_slice_kernel<") + vt + (plan->slices.useDict ? ",dict" : "") + ",fused" + (plan->slices.keep ? ",keep>" : ">"),
             (double)plan->slices.nnz * (es + 4) + xBytes + yBytes, plan->slices.nnz,
             [&]() -> int { return launch_csr_part(plan, x_dev, y_dev, 0, s, nullptr, nullptr, wide); });
     } else if (plan->csr_variant != 0) {
-        add(std::string("csr_slice_kernel<") + vt + (plan->slices.useDict ? ",dict>" : ">"),
+        add(std::string("csr_slice_kernel<") + vt + (plan->slices.useDict ? ",dict" : "") + (plan->slices.keep ? ",keep>" : ">"),
             (double)plan->slices.nnz * (es + 4) + (xCounted ? 0.0 : xBytes), plan->slices.nnz, [&]() -> int {
                 MX_HIP(mx::launch_slices(plan->dtype, plan->slices, x_dev, y_dev, 0, s, 1));
                 return MX_OK;

@@ -20,7 +20,7 @@ const Options &opt() { return g_options; }
 static bool same(const Options &a, const Options &b)
 {
     return a.tile_gate == b.tile_gate && a.csr_dict == b.csr_dict && a.no_strips == b.no_strips && a.no_blocks == b.no_blocks &&
-           a.strips_apart == b.strips_apart && a.csr_kernel == b.csr_kernel && a.csr_fused == b.csr_fused && a.autotune == b.autotune &&
+           a.strips_apart == b.strips_apart && a.csr_kernel == b.csr_kernel && a.csr_fused == b.csr_fused && a.csr_keep == b.csr_keep && a.autotune == b.autotune &&
            a.layout_host == b.layout_host && a.slice_cap == b.slice_cap && a.split_len == b.split_len && a.csr_npt == b.csr_npt &&
            a.tile_per == b.tile_per && a.csr_reduce == b.csr_reduce && a.csr_col16 == b.csr_col16 && a.plan_log == b.plan_log;
 }
@@ -42,6 +42,7 @@ void refresh_options()
     o.strips_apart = number("MX_STRIPS_APART", 0) != 0;
     if (const char *e = text("MX_CSR_KERNEL")) o.csr_kernel = !std::strcmp(e, "rows") ? 1 : !std::strcmp(e, "slices") ? 2 : !std::strcmp(e, "split") ? 3 : 0;
     if (const char *e = text("MX_CSR_FUSED")) o.csr_fused = std::atoi(e) ? 1 : 0;
+    if (const char *e = text("MX_CSR_KEEP")) o.csr_keep = std::atoi(e) ? 1 : 0;
     o.autotune = number("MX_PLAN_AUTOTUNE", 0) != 0;
     if (const char *e = text("MX_LAYOUT")) o.layout_host = !std::strcmp(e, "host");
     o.slice_cap = number("MX_SLICE_CAP", 0);

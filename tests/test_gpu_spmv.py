@@ -1121,6 +1121,50 @@ def test_one_launch_form_of_the_slices(mx, ora, monkeypatch):
         P.close()
 
 
+def test_entries_kept_in_the_caches_or_streamed(mx, ora, monkeypatch):
+    """How the slice kernel reads its entries is a plan's choice (mx_plan_info.csr_keep): plain loads where the
+    entries fit the L2s, or fit the memory-side cache while the second launch moves enough to push streamed
+    entries out; streaming loads otherwise; MX_PLAN_KEEP / MX_PLAN_STREAM and MX_CSR_KEEP decide it for the plan.
+    The two kernels give the same y bit for bit, in two launches and in one, with and without a value dictionary."""
+    import torch
+    cases = [("power-law, quarter size", mx.gen_config(4, scale=0.25), mx.MX_PLAN_CSR_SLICES, 1),      # 11 MB of entries: the L2s
+             ("power-law", mx.gen_config(4), mx.MX_PLAN_DEFAULT, 1),                                   # 42 MB, 21 MB for the second launch
+             ("stencil, fifth size", mx.gen_config(3, scale=0.2), mx.MX_PLAN_CSR_SLICES, 1),           # a value dictionary
+             ("block-clustered, two launches", mx.gen_config(2), mx.MX_PLAN_NO_FUSE, 0),               # 44 MB, 7 MB for the second launch
+             ("block-clustered", mx.gen_config(2), mx.MX_PLAN_DEFAULT, 0),                             # one launch, beyond the L2s
+             ("block-clustered, half size", mx.gen_config(2, scale=0.5), mx.MX_PLAN_CSR_SLICES, 1)]    # one launch, inside the L2s
+    for name, (A, x), flags, kept in cases:
+        print("kept or streamed:", name, A.rows, A.nnz, flush=True)
+        ref = oracle_y(ora, mx, A, x)
+        tol = F64_TOL if A.dtype == mx.MX_F64 else F16_TOL
+        P = mx.Partition(A, 0.0, 0.0)
+        xd = torch.from_numpy(x).cuda()
+        d = mx.Plan(P, flags)
+        assert d.info["csr_variant"] == 1 and d.info["csr_keep"] == kept, (name, d.info)
+        assert not d.info["opt_flags"] & mx.MX_OPT_CSR_KEEP
+        k = mx.Plan(P, flags | mx.MX_PLAN_KEEP)
+        t = mx.Plan(P, flags | mx.MX_PLAN_STREAM)
+        assert k.info["csr_keep"] == 1 and t.info["csr_keep"] == 0 and k.info["csr_fused"] == t.info["csr_fused"] == d.info["csr_fused"]
+        yk, yt, yd = k.spmv(xd).cpu().numpy(), t.spmv(xd).cpu().numpy(), d.spmv(xd).cpu().numpy()
+        assert np.array_equal(yk.view(np.uint8), yt.view(np.uint8)) and np.array_equal(yd.view(np.uint8), yt.view(np.uint8)), name
+        assert rel_l2(yk, ref) <= tol
+        names = [kk["name"] for kk in k.time_kernels(xd, torch.zeros_like(k.spmv(xd)), 2, 5)]
+        assert any(n.startswith("csr_slice_kernel") and n.endswith(",keep>") for n in names), names
+        # the environment decides for plans made under it, and the plan says so
+        monkeypatch.setenv("MX_CSR_KEEP", "0" if kept else "1")
+        e = mx.Plan(P, flags)
+        monkeypatch.delenv("MX_CSR_KEEP")
+        assert e.info["csr_keep"] == 1 - kept and e.info["opt_flags"] & mx.MX_OPT_CSR_KEEP
+        assert np.array_equal(e.spmv(xd).cpu().numpy().view(np.uint8), yt.view(np.uint8))
+        # ... and the plan made from device arrays decides as the one made from the host's
+        D = mx.Plan.from_device_csr(torch.from_numpy(A.rowPtr).cuda(), torch.from_numpy(A.colInd).cuda(), torch.from_numpy(A.val).cuda(),
+                                    A.cols, flags)
+        assert D.info["csr_keep"] == kept and D.info["csr_fused"] == d.info["csr_fused"]
+        for pl in (d, k, t, e, D):
+            pl.close()
+        P.close()
+
+
 def test_one_launch_form_reports_a_share_taken_twice(mx, ora):
     """The way out of the one-launch form, forced from the host (the word a workgroup sets when it finds its
     share of the work taken already): the next product returns MX_ERR_DEVICE once, the plan goes on in the
