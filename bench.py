@@ -22,7 +22,8 @@ of up to 256 MB stays in the memory-side cache), `rotating` (a train that takes 
 of the plan in turn, three times the memory-side cache in all: every array comes from HBM, the
 steady state of a solver whose matrix does not fit that cache) and `cold` (single products after
 a 1 GiB sweep).  `roofline.frac` is the warm figure for a plan that fits the memory-side cache
-and the rotating one for a plan that does not (`frac_basis` says which; all three are there),
+(by the bytes a product touches as the plan stores them, `plan_bytes_per_product`) and the
+rotating one for a plan that does not (`frac_basis` says which; all three are there),
 and `frac_traffic` prices the same time with the bytes the counters saw instead of the
 algorithmic ones.  `roofline.kernels` lists every kernel launch of the product timed alone, each
 with its share of the algorithmic bytes (the shares add up to the whole) and, where profiles/
@@ -274,7 +275,9 @@ def run_workload(mx, torch, ora, cfg, steps, warmup, mode, traffic, only_tau=Non
         ref = ora.spmv_f16_f32acc(A.val, A.rowPtr, A.colInd, x)[0].astype(np.float64)
     rel_l2 = float(np.linalg.norm(y - ref) / np.linalg.norm(ref))
 
-    plan_bytes = info["tile_bytes"] + info["csr_bytes"]
+    # what one product touches as the plan stores it (a value dictionary stores a byte where the algorithmic count has the
+    # value): that, not the algorithmic count, is what has to fit the memory-side cache
+    plan_bytes = info["touched_bytes"]
     cold_ms = rot = None
     if not brief:
         # ---- cold caches: a 1 GiB buffer is swept between launches, so neither the L2s (8 x 4 MB) nor

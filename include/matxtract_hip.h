@@ -519,6 +519,9 @@ typedef struct mx_plan_info {
     int csr_keep;        /* 1: the slice kernel reads the entries with plain loads (they may stay in the caches between
                             products), 0: it streams them (MX_PLAN_KEEP / MX_PLAN_STREAM, MX_CSR_KEEP, or the plan's own
                             choice by size) */
+    double touched_bytes;/* what one product touches in device memory as the plan stores it (entries in their stored form,
+                            sums, row tables, tile part, x, y): what has to fit a cache for the matrix to stay in it.  The
+                            algorithmic bytes of the matrix count a value and a 4-byte column per entry whatever is stored */
 } mx_plan_info;
 /* mx_plan_info.opt_flags */
 #define MX_OPT_NO_STRIPS 1     /* MX_NO_STRIPS=1: no binary16 strip chunks */

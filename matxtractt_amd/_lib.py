@@ -59,7 +59,7 @@ class PlanInfo(C.Structure):
                 ("csr_main_kernel", C.c_int), ("csr_main_nnz", C.c_int), ("tile_variant", C.c_int), ("tile_strip_nnz", C.c_int),
                 ("csr_value_dict", C.c_int), ("est_rows_us", C.c_double), ("est_slices_us", C.c_double),
                 ("prep_route", C.c_int), ("ext_dCols", C.c_int), ("ext_dRows", C.c_int), ("ext_nnzRowD", C.c_int),
-                ("ext_frags", C.c_int), ("csr_fused", C.c_int), ("opt_flags", C.c_int), ("opt_tile_gate", C.c_double), ("csr_keep", C.c_int)]
+                ("ext_frags", C.c_int), ("csr_fused", C.c_int), ("opt_flags", C.c_int), ("opt_tile_gate", C.c_double), ("csr_keep", C.c_int), ("touched_bytes", C.c_double)]
 
 
 class TauEstimate(C.Structure):

@@ -186,6 +186,35 @@ int mxp::fused_wanted(int flags, mx_dtype dtype, int rows, int S, int mostVrows,
     return average <= (double)mx::kFusedAddBytes && S <= mx::kFusedSlicesMost ? 2 : 0;
 }
 
+// Bytes of the entries of a plan's slice layout as they are stored (column offsets and values or value codes, with
+// the padding), and what its second launch moves per product: the sums it is handed, the row tables, y.
+static long long slice_entry_bytes(const mx_plan *plan)
+{
+    const mx::DeviceSlices &L = plan->slices;
+    const long long es = mx::elem_size(plan->dtype), E = mx::slice_step_entries(plan->dtype);
+    return (L.steps + mx::kSlicePadSteps) * 64 * E * (2 + (L.useDict ? 1 : es));
+}
+static long long slice_handoff_bytes(const mx_plan *plan)
+{
+    const mx::DeviceSlices &L = plan->slices;
+    const long long es = mx::elem_size(plan->dtype);
+    return (long long)mxp::partial_bytes(plan) + (long long)plan->rows * (4 + es) + (long long)L.nLight * (4 + 16 * L.lightQuads) + (long long)L.vrows * 4;
+}
+// What one product touches in device memory, as the plan stores it (mx_plan_info.touched_bytes): the CSR part in
+// its form, the tile part, x and y.  (The algorithmic bytes of the matrix, which the roofline is priced on, count a
+// value and a 4-byte column per entry whatever the plan stores.)
+double mxp::touched_bytes(const mx_plan *plan)
+{
+    const double es = mx::elem_size(plan->dtype);
+    double b = (double)plan->cols * es + (double)plan->rows * es;
+    if (plan->csr_variant != 1) b += (double)plan->csr.nnz * ((plan->csr.useDict ? 1.0 : es) + 4.0) + ((double)plan->rows + 1) * 4;
+    if (plan->csr_variant != 0) b += (double)slice_entry_bytes(plan) + (double)slice_handoff_bytes(plan) - (double)plan->rows * es;
+    if (plan->tiles.steps)
+        b += (double)plan->tiles.steps * (mx::kTileHdr * 4.0 + 64 * 4.0) + (double)plan->tiles.stored * es;
+    if (plan->strips.steps) b += (double)plan->strips.steps * (mx::kTileHdr * 4.0) + (double)plan->strips.stored * es;
+    return b;
+}
+
 // How the slice kernel of a plan reads its entries (DeviceSlices::keep).  Streaming loads are the faster way to
 // read a matrix once: they leave the caches to x and the sums, and what they bring is the first to leave the
 // memory-side cache when other traffic asks for room.  That is also their price: the second launch of a product
@@ -208,12 +237,13 @@ void mxp::decide_keep(mx_plan *plan, int flags)
         L.keep = true;
         return;
     }
-    const long long es = mx::elem_size(plan->dtype), E = mx::slice_step_entries(plan->dtype);
-    const long long entryBytes = (L.steps + mx::kSlicePadSteps) * 64 * E * (2 + (L.useDict ? 1 : es));
-    const long long handoff = (long long)partial_bytes(plan) + (long long)plan->rows * (4 + es) + (long long)L.nLight * (4 + 16 * L.lightQuads) +
-                              (long long)L.vrows * 4;
+    const long long es = mx::elem_size(plan->dtype);
+    const long long entryBytes = slice_entry_bytes(plan), handoff = slice_handoff_bytes(plan);
+    // (everything a product touches has to fit beside the entries: the tile part rides in the second launch)
+    const long long product = (long long)touched_bytes(plan);
+    (void)es;
     if (entryBytes <= mx::kKeepL2Bytes) L.keep = true;
-    else if (!plan->fused && entryBytes <= mx::kKeepCacheBytes && handoff >= mx::kKeepHandoffBytes) L.keep = true;
+    else if (!plan->fused && product <= mx::kKeepCacheBytes && handoff >= mx::kKeepHandoffBytes) L.keep = true;
 }
 
 CsrChoice mxp::choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int flags,

@@ -236,6 +236,7 @@ void csr_estimates(mx_dtype dtype, int cols, int nnz, const CsrStats &st, double
 int fused_wanted(int flags, mx_dtype dtype, int rows, int S, int mostVrows, int nCU);
 // Sets plan->slices.keep for a plan whose CSR part is in slice form: how the slice kernel reads its entries.
 void decide_keep(mx_plan *plan, int flags);
+double touched_bytes(const mx_plan *plan);
 CsrChoice choose_csr_form(mx_dtype dtype, int rows, int cols, const int *rowPtr, const int *col, const void *val, int flags, int nCU,
                           int S, bool mayFuse = false);
 int setup_csr_part(mx_plan *plan, const int *rowPtr, const int *col, const void *val, int flags, const char *stripRows = nullptr,

@@ -267,6 +267,7 @@ extern "C" int mx_plan_get_info(const mx_plan *plan, mx_plan_info *info)
     info->opt_flags = plan->opt_flags;
     info->opt_tile_gate = plan->opt_tile_gate;
     info->csr_keep = plan->csr_variant != 0 && plan->slices.keep ? 1 : 0;
+    info->touched_bytes = mxp::touched_bytes(plan);
     return MX_OK;
 }
 
