@@ -237,11 +237,9 @@ void mxp::decide_keep(mx_plan *plan, int flags)
         L.keep = true;
         return;
     }
-    const long long es = mx::elem_size(plan->dtype);
     const long long entryBytes = slice_entry_bytes(plan), handoff = slice_handoff_bytes(plan);
     // (everything a product touches has to fit beside the entries: the tile part rides in the second launch)
     const long long product = (long long)touched_bytes(plan);
-    (void)es;
     if (entryBytes <= mx::kKeepL2Bytes) L.keep = true;
     else if (!plan->fused && product <= mx::kKeepCacheBytes && handoff >= mx::kKeepHandoffBytes) L.keep = true;
 }
