@@ -1064,7 +1064,9 @@ struct DenseStep {
     int hdr;      // header dword lane%32
     v4i32 v, b;   // A operand (one block row), B operand (the eight x of the lane's block)
 };
-// One wave's range of steps (wave `gw` of the layout).
+// One wave's range of steps (wave `gw` of the layout).  KEEP: the values are read with plain loads (a plan whose
+// product fits the memory-side cache keeps them there, as it keeps the entries of its slices), streamed otherwise.
+template <bool KEEP = false>
 __device__ __forceinline__ void tile_dense_wave(const int4 *__restrict__ waveDesc, const int *__restrict__ hdr,
                                                 const _Float16 *__restrict__ tcVal, const _Float16 *__restrict__ x,
                                                 _Float16 *__restrict__ y, int gw, int lane)
@@ -1076,7 +1078,7 @@ __device__ __forceinline__ void tile_dense_wave(const int4 *__restrict__ waveDes
     const int m = lane & 15, g = lane >> 4, h = m >> 3;
     auto issue = [&](DenseStep &R, int step, int vo, int na) {
         R.hdr = hdr[(size_t)step * kTileHdr + (lane & 31)];
-        R.v = __builtin_nontemporal_load((const v4i32 *)(tcVal + vo + ((h ? na : 0) + g) * 64 + (m & 7) * 8));
+        R.v = stream_load<KEEP>((const v4i32 *)(tcVal + vo + ((h ? na : 0) + g) * 64 + (m & 7) * 8));
     };
     // the x of the lane's block, once the header is there: B column m (0 = half 0, 1 = half 1),
     // rows 8g..8g+7 = slot 4m+g; the other lanes read what lane m&1 of their group reads
@@ -1261,7 +1263,7 @@ __global__ __launch_bounds__(kBlock) void tile_block_kernel(const int4 *__restri
 //    two arrays, so nothing the lane loads depends on another load but the sums themselves;
 //  * the rest take the rows with more, sixteen lanes each.
 constexpr int kCombineRows = 16;  // rows a lane of the first kind takes
-template <typename VT, bool STRIPS>  // STRIPS: an instance of its own, so that the plain one keeps its few registers
+template <typename VT, bool STRIPS, bool KEEP = false>  // STRIPS: an instance of its own, so that the plain one keeps its few registers
 __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Acc<VT>::type *__restrict__ partial,
                                                               const int *__restrict__ rowInfo, int rows, int nRowWG,
                                                               const int *__restrict__ lightRow,
@@ -1286,7 +1288,7 @@ __global__ __launch_bounds__(kBlock) void slice_combine_kernel(const typename Ac
     if (STRIPS && (int)blockIdx.x < nStripWG) {
         if constexpr (STRIPS && sizeof(VT) == 2) {
             const int gw = xcd_contiguous_block(blockIdx.x, nStripWG) * (kBlock / 64) + (tid >> 6);
-            if (gw < nStripWaves) tile_dense_wave(stripWaveDesc, stripHdr, stripVal, x, y, gw, tid & 63);
+            if (gw < nStripWaves) tile_dense_wave<KEEP>(stripWaveDesc, stripHdr, stripVal, x, y, gw, tid & 63);
         }
         // binary64: the 8 x 8 blocks, whose waves also fetch the sums of their rows' virtual rows
         // (those rows are marked -2 in rowInfo and appear in none of the lists below)
@@ -1555,15 +1557,16 @@ static hipError_t launch_slices_t(const DeviceSlices &P, const void *x, void *y,
     const bool ride = strips && strips->nWaves > 0 && (sizeof(VT) == 2 || strips->vidx);
     const int nStripWG = ride ? (strips->nWaves + 3) / 4 : 0;
     if (nStripWG + nRowWG + nLightWG + nHeavyWG == 0) return hipSuccess;
-#define MX_LAUNCH_COMBINE(STRIPS)                                                                                          \
-    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT, STRIPS>), dim3(nStripWG + nRowWG + nLightWG + nHeavyWG),                 \
+#define MX_LAUNCH_COMBINE(STRIPS, KEEP)                                                                                    \
+    hipLaunchKernelGGL((mxk::slice_combine_kernel<VT, STRIPS, KEEP>), dim3(nStripWG + nRowWG + nLightWG + nHeavyWG),           \
                        dim3(mxk::kBlock), 0, s, (const AT *)P.partial, P.rowInfo, P.rows, nRowWG, P.lightRow,                    \
                        (const int4 *)P.lightIdx, P.nLight, nLightWG, (const int4 *)P.heavyInfo, P.nHeavy, P.segIdx, (VT *)y,    \
                        (accumulate || P.subset) ? 1 : 0, P.subset ? 1 : 0, (AT *)ywide, ride ? (const int4 *)strips->waveDesc : nullptr,   \
                        ride ? strips->hdr : nullptr, ride ? (const VT *)strips->tcVal : nullptr, (const VT *)x,              \
                        ride ? strips->nWaves : 0, nStripWG, nHeavyWG, P.lightQuads, ride ? strips->vidx : nullptr)
-    if (ride) MX_LAUNCH_COMBINE(true);
-    else MX_LAUNCH_COMBINE(false);
+    if (ride && P.keep && sizeof(VT) == 2) MX_LAUNCH_COMBINE(true, true);  // (the strips' values stay where the slices' entries stay)
+    else if (ride) MX_LAUNCH_COMBINE(true, false);
+    else MX_LAUNCH_COMBINE(false, false);
 #undef MX_LAUNCH_COMBINE
     return hipGetLastError();
 }

@@ -966,6 +966,7 @@ static int create_plan(const mx_partition *P, int flags, mx_plan **out, bool noB
         set_error("mx_plan_create: out of memory");
         return fail(MX_ERR_ALLOC);
     }
+    decide_keep(plan, flags);  // (again, now that the tile part is known: it counts towards what a product touches)
     *out = plan;
     return MX_OK;
 }

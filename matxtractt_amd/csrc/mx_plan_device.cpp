@@ -498,6 +498,7 @@ int mxp::create_plan_device(mx_dtype dtype, int rows, int cols, int nnz, const i
         (void)hipFree(partCol);
         (void)hipFree(partVal);
         (void)hipFree(stripRows);
+        decide_keep(plan, flags);  // (again, now that the tile part is known: it counts towards what a product touches)
         *out = plan;
         return MX_OK;
     } catch (const std::bad_alloc &) {
