@@ -25,7 +25,9 @@ a 1 GiB sweep).  `roofline.frac` is the warm figure for a plan that fits the mem
 (by the bytes a product touches as the plan stores them, `plan_bytes_per_product`) and the
 rotating one for a plan that does not (`frac_basis` says which; all three are there),
 and `frac_traffic` prices the same time with the bytes the counters saw instead of the
-algorithmic ones.  `roofline.kernels` lists every kernel launch of the product timed alone, each
+algorithmic ones.  `csr_entries_kept_in_cache` says how the plan reads the entries of its slices
+(plain loads, so that a matrix that fits the L2s or the memory-side cache stays there between
+products, or streaming loads: the plan's own choice by size, mx_plan_info.csr_keep).  `roofline.kernels` lists every kernel launch of the product timed alone, each
 with its share of the algorithmic bytes (the shares add up to the whole) and, where profiles/
 holds a rocprofv3 counter run of that kernel on that workload and plan, its measured HBM
 traffic.  `cpu_baseline` is the oracle's single-thread CSR loop on the same matrix, on this
