@@ -291,9 +291,10 @@ void mx_plan_destroy(mx_plan *plan);
  * on the device: the plan, and with it every y, equals the one mx_plan_create makes from a partition
  * of the same matrix with tau = (0, 0).  rowPtr_dev and colInd_dev are checked on the device before
  * they are used as addresses (MX_ERR_ARG).  flags: MX_PLAN_CSR_ROWS, MX_PLAN_CSR_SLICES, MX_PLAN_NO_FUSE,
- * MX_PLAN_FUSE or 0.  Three forms of the CSR part are laid out on the host, from a copy of the part that is
- * brought down for it: the one-launch form of the slices (small matrices, unless it is forced), and the split
- * form and the timed choice that MX_CSR_KERNEL=split and MX_PLAN_AUTOTUNE=1 ask for. */
+ * MX_PLAN_FUSE, MX_PLAN_KEEP, MX_PLAN_STREAM or 0.  For the one-launch form of the slices the records of the
+ * virtual rows (slice and length of each) cross to the host as well, and its plan comes back; the entries stay.
+ * Two things are laid out on the host, from a copy of the part that is brought down for it: the split form and
+ * the timed choice that MX_CSR_KERNEL=split and MX_PLAN_AUTOTUNE=1 ask for. */
 int mx_plan_create_device_csr(mx_dtype dtype, int rows, int cols, int nnz, const int *rowPtr_dev, const int *colInd_dev,
                               const void *val_dev, int flags, mx_plan **out);
 
