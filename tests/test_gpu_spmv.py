@@ -2001,13 +2001,14 @@ def _mixed_matrix(mx, rng, rows, cols, dt):
 def test_mid_sized_matrices_of_mixed_structure_give_the_exact_product(mx, ora):
     """Seeded matrices of a thousand to half a million rows with power-law rows, strips, blocks, empty rows
     and repeated columns, integer values and x (every sum is an integer both precisions hold, so y must equal
-    the oracle's bit for bit whatever the order of the additions), at two pairs of fractions, under eight sets
+    the oracle's bit for bit whatever the order of the additions), at two pairs of fractions, under ten sets
     of plan flags, for the plan made from the host partition and the one made from device arrays, into a
     fresh y and over an old one."""
     import torch
     flag_sets = [mx.MX_PLAN_DEFAULT, mx.MX_PLAN_KEEP_TILES, mx.MX_PLAN_ALL_TILES, mx.MX_PLAN_NO_TILES | mx.MX_PLAN_CSR_ROWS,
                  mx.MX_PLAN_NO_TILES | mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_FUSE, mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_SLICES,
-                 mx.MX_PLAN_NO_TILES | mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_NO_FUSE, mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_ROWS]
+                 mx.MX_PLAN_NO_TILES | mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_NO_FUSE, mx.MX_PLAN_ALL_TILES | mx.MX_PLAN_CSR_ROWS,
+                 mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_STREAM | mx.MX_PLAN_FUSE, mx.MX_PLAN_KEEP_TILES | mx.MX_PLAN_CSR_SLICES | mx.MX_PLAN_KEEP]
     taus = [(0.25, 0.0), (0.5, 0.25), (0.75, 0.0), (0.75, 0.5), (1.0, 0.5)]
     done = 0
     for case in range(12):
@@ -2038,4 +2039,4 @@ def test_mid_sized_matrices_of_mixed_structure_give_the_exact_product(mx, ora):
                     P.close()
                     done += 1
             part.close()
-    assert done >= 300, done
+    assert done >= 380, done
